@@ -1,0 +1,198 @@
+/*
+ * libtango_hip — C ABI of the MI355X (gfx950) quantized-GNN primitive layer.
+ *
+ * Each entry point replaces one binding of the reference's pybind11 module
+ * `cuda_kernels` (cuda/src/cuda.cpp:182-204).  All pointers are DEVICE
+ * pointers unless stated otherwise; scales stay device-resident end to end.
+ * No entry point allocates, frees or synchronises; every launch goes to the
+ * stream the caller passes (a hipStream_t cast to void*; NULL = default
+ * stream).  Return value: TANGO_OK or a negative tango_status; the library
+ * never aborts the process (the reference calls exit() on any native error,
+ * cuda/src/utils.h:4-35).
+ *
+ * Tensors are dense row-major.  "ld*" arguments are row strides in elements.
+ * Index arrays are int64, as in the reference's API; node and edge counts
+ * must stay below 2^31.
+ */
+#ifndef TANGO_HIP_H
+#define TANGO_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef void* tango_stream_t;
+
+enum tango_status {
+    TANGO_OK = 0,
+    TANGO_ERR_INVALID_ARG = -1, /* null pointer, negative size, misaligned operand */
+    TANGO_ERR_UNSUPPORTED = -2, /* unknown op / rounding mode / shape outside the kernels' range */
+    TANGO_ERR_LAUNCH = -3,      /* HIP refused the launch */
+    TANGO_ERR_WORKSPACE = -4    /* workspace missing or too small */
+};
+
+enum tango_round_mode {
+    TANGO_ROUND_RNE = 0,       /* half-to-even + clamp: cuda/src/quantization.cu:6-15 */
+    TANGO_ROUND_TRUNC = 1,     /* toward zero: cuda/src/iterator.h:161 (GEMM fused quantize) */
+    TANGO_ROUND_STOCHASTIC = 2 /* floor(x/s + u), u in [0,1): no counterpart in the reference */
+};
+
+enum tango_sddmm_op { TANGO_OP_ADD = 0, TANGO_OP_SUB = 1, TANGO_OP_MUL = 2, TANGO_OP_DIV = 3 };
+
+const char* tango_status_string(int status);
+/* ABI version; bumped when a signature changes. */
+int tango_abi_version(void);
+
+/* ------------------------------------------------------------ quantization */
+
+/* get_scale (cuda/src/cuda.cpp:24-25 -> get_scale_impl, quantization.cu:79-93):
+   scale_out[0] = max|x| / 127 over n contiguous floats.  scale_out need not be
+   initialised.  Unlike the reference every element is covered when n % 4 != 0. */
+int tango_absmax_f32(const float* x, int64_t n, float* scale_out, tango_stream_t stream);
+
+/* Per-row scales (no counterpart in the reference): scale_out[r] = max_c |x[r,c]| / 127. */
+int tango_absmax_rows_f32(const float* x, int64_t rows, int64_t cols, int64_t ldx,
+                          float* scale_out, tango_stream_t stream);
+
+/* quantize (cuda/src/cuda.cpp:19-23 -> quantize_impl, quantization.cu:17-43):
+   q[i] = clamp(round(x[i] * (1 / scale[0])), -127, 127).  round_mode selects the
+   rounding.  For TANGO_ROUND_STOCHASTIC, `noise` (n floats in [0,1), same
+   indexing as x) is used when non-null; otherwise Philox4x32-10 keyed by `seed`
+   with counter (offset + i) >> 2, word (offset + i) & 3, u = (word >> 8) * 2^-24. */
+int tango_quantize_f32_i8(const float* x, int64_t n, const float* scale, int8_t* q,
+                          int round_mode, const float* noise, uint64_t seed, uint64_t offset,
+                          tango_stream_t stream);
+
+/* Row-strided quantize with an optionally padded output (no counterpart in the
+   reference; lets the SpMM gather aligned rows when cols is odd, e.g. 41):
+   q[r, c] for c < cols as above with scale[per_row ? r : 0]; q[r, cols..ldq) = 0.
+   Noise / Philox indexing uses the dense index r * cols + c. */
+int tango_quantize_rows_f32_i8(const float* x, int64_t rows, int64_t cols, int64_t ldx,
+                               const float* scale, int per_row, int8_t* q, int64_t ldq,
+                               int round_mode, const float* noise, uint64_t seed,
+                               uint64_t offset, tango_stream_t stream);
+
+/* transpose_quant (cuda/src/cuda.cpp:27-33 -> transpose_quant_impl,
+   quantization.cu:95-167): x[nrow, ncol] fp32 -> out[ncol, nrow] int8,
+   half-to-even, clamped to +-127. */
+int tango_transpose_quant_f32_i8(const float* x, int64_t nrow, int64_t ncol, const float* scale,
+                                 int8_t* out, tango_stream_t stream);
+
+/* -------------------------------------------------------------------- GEMM */
+
+/* QGEMM_forward (cuda/src/cuda.cpp:11-17 -> QGEMM_forward_impl,
+   QGEMM_forward.cu:125-157): quantizes X[M,K] and W[N,K] with scaleX / scaleW
+   (round_mode; the reference truncates), stores the int8 copies to Xq[M,K] and
+   Wq[N,K] (dense, row stride K), and writes
+   Y[m,n] = (scaleX*scaleW) * float(sum_k Xq[m,k]*Wq[n,k]) (+ bias[n]).
+   bias may be NULL.  scaleY may be NULL; otherwise scaleY[0] = max|Y| / 127
+   (the fused reduction of cuda/src/epilogue.h:105-626); it need not be
+   initialised.  K is arbitrary (the reference requires K % 4 == 0).
+   workspace: tango_qgemm_fwd_workspace(M,N,K) bytes, may be NULL when that is 0. */
+size_t tango_qgemm_fwd_workspace(int64_t M, int64_t N, int64_t K);
+int tango_qgemm_fwd(float* Y, int64_t ldy, const float* X, int64_t ldx, int8_t* Xq,
+                    const float* W, int64_t ldw, int8_t* Wq, const float* bias, float* scaleY,
+                    const float* scaleX, const float* scaleW, int64_t M, int64_t N, int64_t K,
+                    int round_mode, void* workspace, size_t workspace_bytes,
+                    tango_stream_t stream);
+
+/* Integer GEMM on operands that are already int8 (the cached-operand forward
+   used when quantization was done by tango_quantize_*; same epilogue as above):
+   Y[m,n] = (sA*sB) * float(sum_k A[m,k]*B[n,k]) (+ bias[n]), optional scaleY. */
+int tango_qgemm_i8_nt(float* Y, int64_t ldy, const int8_t* A, int64_t lda, const int8_t* B,
+                      int64_t ldb, const float* bias, float* scaleY, const float* sA,
+                      const float* sB, int64_t M, int64_t N, int64_t K, tango_stream_t stream);
+
+/* QGEMM_backward_gradX (cuda/src/cuda.cpp:90-98 -> QGEMM_backward.cu:21-48):
+   dX[M,K] = (s_dY*s_W) * float(sum_n dYq[m,n] * Wq[n,k]). */
+int tango_qgemm_bwd_dx(float* dX, int64_t lddx, const int8_t* dYq, int64_t lddy,
+                       const int8_t* Wq, int64_t ldw, const float* s_dY, const float* s_W,
+                       int64_t M, int64_t N, int64_t K, tango_stream_t stream);
+
+/* QGEMM_backward_gradW (cuda/src/cuda.cpp:100-108 -> QGEMM_backward.cu:50-113):
+   dW[N,K] = (s_dY*s_X) * float(sum_m dYq[m,n] * Xq[m,k]), int32 accumulation.
+   The reduction over M is split over workgroups whose int32 partials are summed
+   exactly, so the result does not depend on the split.  workspace holds those
+   partials: tango_qgemm_bwd_dw_workspace(M,N,K) bytes. */
+size_t tango_qgemm_bwd_dw_workspace(int64_t M, int64_t N, int64_t K);
+int tango_qgemm_bwd_dw(float* dW, int64_t lddw, const int8_t* dYq, int64_t lddy,
+                       const int8_t* Xq, int64_t ldx, const float* s_dY, const float* s_X,
+                       int64_t M, int64_t N, int64_t K, void* workspace, size_t workspace_bytes,
+                       tango_stream_t stream);
+
+/* QgemmNT / QgemmNN / QgemmTN (cuda/src/cuda.cpp:75-88 -> Qgemm_impl.cu:6-125):
+   quantize fp32 A and B (absmax scale, half-to-even), int8 GEMM, dequantize.
+   A is [m,k] (or [k,m] when trans_a), B is [k,n] (or [n,k] when trans_b),
+   C is [m,n].  workspace: tango_qgemm_legacy_workspace(m,n,k) bytes. */
+size_t tango_qgemm_legacy_workspace(int64_t m, int64_t n, int64_t k);
+int tango_qgemm_legacy(float* C, const float* A, const float* B, int64_t m, int64_t n, int64_t k,
+                       int trans_a, int trans_b, void* workspace, size_t workspace_bytes,
+                       tango_stream_t stream);
+
+/* -------------------------------------------------------------------- SpMM */
+
+/* csr_SPMM (cuda/src/cuda.cpp:110-117 -> cusp_SPMM_csr_impl, SPMM.cu:23-68):
+   out[r, f] = scale[0] * float(sum_{p in [indptr[r], indptr[r+1])} feat[indices[p], f])
+   for r < rows, f < F.  feat has num_src rows of stride ldf bytes (ldf >= F);
+   out is [rows, F] dense; nnz = indptr[rows].  int32 accumulation. */
+int tango_spmm_csr_copy_u(float* out, const int64_t* indptr, const int64_t* indices,
+                          const int8_t* feat, int64_t ldf, const float* scale, int64_t rows,
+                          int64_t num_src, int64_t nnz, int64_t F, tango_stream_t stream);
+
+/* multi_cusparse_SPMM (cuda/src/cuda.cpp:119-158 -> SPMM.cu:70-194):
+   out[r,h,f] = scale[0] * float(sum_p evals[h, d, e(p)] * feat[indices[p], h, f]),
+   d = 0 when D == 1 (broadcast edge value) else d = f (D == F, element-wise).
+   feat is [num_src, H, F] int8, evals is [H, D, nnz] int8, out is [rows, H, F].
+   e(p) = p when edge_ids is NULL (evals already in CSR slot order, as after the
+   index_select of cuda/kernels.py:133-135), else edge_ids[p] (that gather fused). */
+int tango_spmm_csr_u_mul_e(float* out, const int64_t* indptr, const int64_t* indices,
+                           const int64_t* edge_ids, const int8_t* feat, const int8_t* evals,
+                           const float* scale, int64_t rows, int64_t num_src, int64_t H,
+                           int64_t F, int64_t D, int64_t nnz, tango_stream_t stream);
+
+/* incidence_SPMM (cuda/src/cuda.cpp:160-167 -> incidence_SPMM_impl, SPMM.cu:259-303):
+   out[v, f] = scale[0] * float(sum_{i: node_ids[i] == v} E[edge_ids[i], f]).
+   (node_ids, edge_ids) are the COO rows of the incidence matrix and must be
+   sorted by node id, which cuda/util.py:6-7 (coalesce) guarantees. */
+int tango_spmm_incidence(float* out, const int64_t* node_ids, const int64_t* edge_ids,
+                         const int8_t* E, const float* scale, int64_t num_nodes, int64_t nnz,
+                         int64_t num_edges, int64_t F, tango_stream_t stream);
+
+/* ------------------------------------------------------------------- SDDMM */
+
+/* mySDDMM_int8 with op "dot" (cuda/src/cuda.cpp:41-47 -> SDDMM.cu:8-47,124-150):
+   out[e,h] = (sU*sV) * float(sum_d U[src[e],h,d] * V[dst[e],h,d]).
+   U, V are [*, H, D] int8.  scale_out may be NULL; otherwise
+   scale_out[0] = max|out| / 127 (need not be initialised). */
+int tango_sddmm_dot_i8(float* out, float* scale_out, const int64_t* src, const int64_t* dst,
+                       const int8_t* U, const int8_t* V, const float* sU, const float* sV,
+                       int64_t num_edges, int64_t H, int64_t D, tango_stream_t stream);
+
+/* mySDDMM_int8 with op add/sub/mul/div (SDDMM.cu:49-100,152-175):
+   out[e,t] = OP(float(U[src[e],t]) * sU, float(V[dst[e],t]) * sV), t < T. */
+int tango_sddmm_ewise_i8(int op, float* out, float* scale_out, const int64_t* src,
+                         const int64_t* dst, const int8_t* U, const int8_t* V, const float* sU,
+                         const float* sV, int64_t num_edges, int64_t T, tango_stream_t stream);
+
+/* ------------------------------------------------------------ edge softmax */
+
+/* LeakyReLU(slope) followed by softmax over the in-edges of every destination
+   node (dgl.ops.edge_softmax as called at evaluation/test_gat.py:144-146; DGL
+   is not part of the reference tree).  e and a are [num_edges, H] in edge-id
+   order; indptr/edge_ids describe the destination-major CSR (adj_csc);
+   edge_ids may be NULL for the identity.  slope = 1 gives the plain softmax. */
+int tango_edge_softmax_fwd(float* a, const float* e, const int64_t* indptr,
+                           const int64_t* edge_ids, int64_t rows, int64_t H, float slope,
+                           tango_stream_t stream);
+/* de = dLeaky(e) * a * (da - sum_{same dst} a*da). */
+int tango_edge_softmax_bwd(float* de, const float* a, const float* da, const float* e,
+                           const int64_t* indptr, const int64_t* edge_ids, int64_t rows,
+                           int64_t H, float slope, tango_stream_t stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* TANGO_HIP_H */

@@ -1,0 +1,85 @@
+// Shared device/host helpers for the gfx950 kernels of libtango_hip.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/tango_hip.h"
+
+namespace tango {
+
+constexpr int kWave = 64;
+
+// Native vector types (the nontemporal builtins and MFMA operands need these,
+// not HIP's float4/int4 structs).
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef int i32x4 __attribute__((ext_vector_type(4)));
+typedef int i32x16 __attribute__((ext_vector_type(16)));
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
+
+inline hipStream_t as_stream(tango_stream_t s) { return reinterpret_cast<hipStream_t>(s); }
+
+// Status of the launch just issued (configuration errors surface here; kernel
+// faults surface at the caller's next synchronisation, as with any HIP code).
+inline int launch_status() {
+    return hipGetLastError() == hipSuccess ? TANGO_OK : TANGO_ERR_LAUNCH;
+}
+
+inline int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
+
+// Number of workgroups for a grid-stride kernel: enough to give every one of
+// the 256 CUs several resident groups, never more than the work needs.
+inline int grid_for(int64_t work_items, int threads, int groups_per_cu = 8) {
+    int64_t need = ceil_div(work_items, threads);
+    int64_t cap = 256LL * groups_per_cu;
+    if (need < 1) need = 1;
+    return static_cast<int>(need < cap ? need : cap);
+}
+
+__device__ __forceinline__ int lane_id() { return threadIdx.x & (kWave - 1); }
+
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+    for (int off = kWave / 2; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, kWave));
+    return v;
+}
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+    for (int off = kWave / 2; off > 0; off >>= 1) v += __shfl_xor(v, off, kWave);
+    return v;
+}
+
+// Workgroup-wide maximum of non-negative floats followed by one integer
+// atomicMax on the float's bit pattern (order-preserving for values >= 0).
+// *out must hold 0 (or an earlier partial maximum) before the first arrival.
+// Every thread of the workgroup must call this.
+__device__ __forceinline__ void block_absmax_to_global(float v, float* out) {
+    __shared__ float part[16];
+    v = wave_max(v);
+    const int nw = (blockDim.x * blockDim.y + kWave - 1) / kWave;
+    const int tid = threadIdx.y * blockDim.x + threadIdx.x;
+    const int w = tid / kWave;
+    if ((tid & (kWave - 1)) == 0) part[w] = v;
+    __syncthreads();
+    if (w == 0) {
+        float m = (tid < nw) ? part[tid] : 0.0f;
+        m = wave_max(m);
+        if (tid == 0) atomicMax(reinterpret_cast<int*>(out), __float_as_int(m));
+    }
+}
+
+// 1/s with the convention that an all-zero tensor (s == 0) quantizes to zeros.
+__device__ __forceinline__ float rscale_of(float s) { return s > 0.0f ? 1.0f / s : 0.0f; }
+
+// Sets a handful of 32-bit words.  Used instead of hipMemsetAsync so that a
+// caller may capture any entry point into a HIP graph.
+static __global__ void fill_u32_kernel(uint32_t* p, uint32_t v, int n) {
+    if (static_cast<int>(threadIdx.x) < n) p[threadIdx.x] = v;
+}
+
+inline void fill_u32(void* p, uint32_t v, int n, hipStream_t s) {
+    hipLaunchKernelGGL(fill_u32_kernel, dim3(1), dim3(64), 0, s, static_cast<uint32_t*>(p), v, n);
+}
+
+}  // namespace tango

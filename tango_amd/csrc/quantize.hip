@@ -1,0 +1,372 @@
+// Absmax scales and fp32 -> int8 quantization for gfx950.
+//
+// All three kernels are HBM-streaming: 4 B/element read for absmax, 5 B/element
+// for quantize.  Each lane moves 16-byte vectors, a wavefront therefore covers
+// 1 KiB per load instruction, and the grid is sized to keep every CU busy with
+// several resident workgroups (the reference launches a fixed 960x128 grid,
+// cuda/src/quantization.cu:39,87).
+#include <type_traits>
+
+#include "common.hpp"
+
+namespace tango {
+
+// ------------------------------------------------------------------ Philox
+// Philox4x32-10, counter-based (Salmon et al., SC'11).  One call yields the
+// noise of four consecutive elements.
+struct Philox4 {
+    uint32_t v[4];
+};
+
+__device__ __forceinline__ Philox4 philox4x32_10(uint32_t c0, uint32_t c1, uint32_t c2,
+                                                 uint32_t c3, uint32_t k0, uint32_t k1) {
+#pragma unroll
+    for (int r = 0; r < 10; ++r) {
+        const uint32_t hi0 = __umulhi(0xD2511F53u, c0), lo0 = 0xD2511F53u * c0;
+        const uint32_t hi1 = __umulhi(0xCD9E8D57u, c2), lo1 = 0xCD9E8D57u * c2;
+        const uint32_t n0 = hi1 ^ c1 ^ k0;
+        const uint32_t n2 = hi0 ^ c3 ^ k1;
+        c0 = n0;
+        c1 = lo1;
+        c2 = n2;
+        c3 = lo0;
+        k0 += 0x9E3779B9u;
+        k1 += 0xBB67AE85u;
+    }
+    return Philox4{{c0, c1, c2, c3}};
+}
+
+__device__ __forceinline__ float u01(uint32_t w) { return static_cast<float>(w >> 8) * 0x1.0p-24f; }
+
+__device__ __forceinline__ float philox_uniform(uint64_t seed, uint64_t g) {
+    const uint64_t blk = g >> 2;
+    Philox4 r = philox4x32_10(static_cast<uint32_t>(blk), static_cast<uint32_t>(blk >> 32), 0u, 0u,
+                              static_cast<uint32_t>(seed), static_cast<uint32_t>(seed >> 32));
+    return u01(r.v[g & 3]);
+}
+
+// ---------------------------------------------------------------- rounding
+template <int MODE>
+__device__ __forceinline__ int quant_one(float x, float r, float u) {
+    const float p = x * r;
+    float v;
+    if (MODE == TANGO_ROUND_RNE)
+        v = rintf(p);
+    else if (MODE == TANGO_ROUND_TRUNC)
+        v = truncf(p);
+    else
+        v = floorf(p + u);
+    // fmaxf/fminf drop a NaN operand, so a NaN input lands on a bound; map it to 0
+    v = (v == v) ? fminf(fmaxf(v, -127.0f), 127.0f) : 0.0f;
+    return static_cast<int>(v);
+}
+
+__device__ __forceinline__ uint32_t pack4(int a, int b, int c, int d) {
+    return (static_cast<uint32_t>(a) & 0xffu) | ((static_cast<uint32_t>(b) & 0xffu) << 8) |
+           ((static_cast<uint32_t>(c) & 0xffu) << 16) | (static_cast<uint32_t>(d) << 24);
+}
+
+// ------------------------------------------------------------------ absmax
+__global__ __launch_bounds__(256) void absmax_kernel(const float* __restrict__ x, int64_t n,
+                                                     int64_t head, float* __restrict__ out) {
+    // [0, head) scalar, then n4 float4 vectors from an aligned base, then the tail
+    const int64_t tid = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    const int64_t nthr = static_cast<int64_t>(gridDim.x) * blockDim.x;
+    float m = 0.0f;
+    const int64_t n4 = (n - head) >> 2;
+    const f32x4* x4 = reinterpret_cast<const f32x4*>(x + head);
+    int64_t i = tid;
+    for (; i + 3 * nthr < n4; i += 4 * nthr) {
+        const f32x4 a = __builtin_nontemporal_load(x4 + i);
+        const f32x4 b = __builtin_nontemporal_load(x4 + i + nthr);
+        const f32x4 c = __builtin_nontemporal_load(x4 + i + 2 * nthr);
+        const f32x4 d = __builtin_nontemporal_load(x4 + i + 3 * nthr);
+        m = fmaxf(m, fmaxf(fmaxf(fabsf(a.x), fabsf(a.y)), fmaxf(fabsf(a.z), fabsf(a.w))));
+        m = fmaxf(m, fmaxf(fmaxf(fabsf(b.x), fabsf(b.y)), fmaxf(fabsf(b.z), fabsf(b.w))));
+        m = fmaxf(m, fmaxf(fmaxf(fabsf(c.x), fabsf(c.y)), fmaxf(fabsf(c.z), fabsf(c.w))));
+        m = fmaxf(m, fmaxf(fmaxf(fabsf(d.x), fabsf(d.y)), fmaxf(fabsf(d.z), fabsf(d.w))));
+    }
+    for (; i < n4; i += nthr) {
+        const f32x4 a = __builtin_nontemporal_load(x4 + i);
+        m = fmaxf(m, fmaxf(fmaxf(fabsf(a.x), fabsf(a.y)), fmaxf(fabsf(a.z), fabsf(a.w))));
+    }
+    if (tid < head) m = fmaxf(m, fabsf(x[tid]));
+    const int64_t tail0 = head + (n4 << 2);
+    if (tail0 + tid < n) m = fmaxf(m, fabsf(x[tail0 + tid]));
+    block_absmax_to_global(m / 127.0f, out);
+}
+
+// One workgroup, direct store: small tensors need no atomic and no pre-zeroing.
+__global__ __launch_bounds__(1024) void absmax_small_kernel(const float* __restrict__ x, int64_t n,
+                                                            float* __restrict__ out) {
+    __shared__ float part[16];
+    float m = 0.0f;
+    for (int64_t i = threadIdx.x; i < n; i += blockDim.x) m = fmaxf(m, fabsf(x[i]));
+    m = wave_max(m);
+    if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = m;
+    __syncthreads();
+    if (threadIdx.x < 64) {
+        float v = (threadIdx.x < (blockDim.x >> 6)) ? part[threadIdx.x] : 0.0f;
+        v = wave_max(v);
+        if (threadIdx.x == 0) out[0] = v / 127.0f;
+    }
+}
+
+// One wavefront per row.
+__global__ __launch_bounds__(256) void absmax_rows_kernel(const float* __restrict__ x,
+                                                          int64_t rows, int64_t cols, int64_t ldx,
+                                                          float* __restrict__ out) {
+    const int64_t row = static_cast<int64_t>(blockIdx.x) * (blockDim.x / kWave) + threadIdx.x / kWave;
+    if (row >= rows) return;
+    const float* xr = x + row * ldx;
+    float m = 0.0f;
+    for (int64_t c = lane_id(); c < cols; c += kWave) m = fmaxf(m, fabsf(xr[c]));
+    m = wave_max(m);
+    if (lane_id() == 0) out[row] = m / 127.0f;
+}
+
+// ---------------------------------------------------------------- quantize
+// Vector body: x is 16-byte aligned, q 4-byte aligned, n4 = n / 4 vectors.
+template <int MODE>
+__global__ __launch_bounds__(256) void quantize_vec_kernel(
+    const float* __restrict__ x, int64_t n, const float* __restrict__ scale,
+    int8_t* __restrict__ q, const float* __restrict__ noise, uint64_t seed, uint64_t offset) {
+    const int64_t tid = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    const int64_t nthr = static_cast<int64_t>(gridDim.x) * blockDim.x;
+    const float r = rscale_of(scale[0]);
+    const int64_t n4 = n >> 2;
+    const f32x4* x4 = reinterpret_cast<const f32x4*>(x);
+    uint32_t* q4 = reinterpret_cast<uint32_t*>(q);
+    const bool shared_block = (offset & 3) == 0;  // the 4 elements share one Philox block
+    for (int64_t i = tid; i < n4; i += nthr) {
+        const f32x4 v = __builtin_nontemporal_load(x4 + i);
+        float u0 = 0.f, u1 = 0.f, u2 = 0.f, u3 = 0.f;
+        if (MODE == TANGO_ROUND_STOCHASTIC) {
+            if (noise) {
+                // noise shares x's element index but not necessarily its alignment
+                u0 = noise[4 * i];
+                u1 = noise[4 * i + 1];
+                u2 = noise[4 * i + 2];
+                u3 = noise[4 * i + 3];
+            } else if (shared_block) {
+                const uint64_t blk = (offset + 4 * static_cast<uint64_t>(i)) >> 2;
+                Philox4 p = philox4x32_10(static_cast<uint32_t>(blk), static_cast<uint32_t>(blk >> 32),
+                                          0u, 0u, static_cast<uint32_t>(seed),
+                                          static_cast<uint32_t>(seed >> 32));
+                u0 = u01(p.v[0]);
+                u1 = u01(p.v[1]);
+                u2 = u01(p.v[2]);
+                u3 = u01(p.v[3]);
+            } else {
+                const uint64_t g = offset + 4 * static_cast<uint64_t>(i);
+                u0 = philox_uniform(seed, g);
+                u1 = philox_uniform(seed, g + 1);
+                u2 = philox_uniform(seed, g + 2);
+                u3 = philox_uniform(seed, g + 3);
+            }
+        }
+        const uint32_t w = pack4(quant_one<MODE>(v.x, r, u0), quant_one<MODE>(v.y, r, u1),
+                                 quant_one<MODE>(v.z, r, u2), quant_one<MODE>(v.w, r, u3));
+        __builtin_nontemporal_store(w, q4 + i);
+    }
+    const int64_t t = (n4 << 2) + tid;  // tail: at most 3 elements
+    if (t < n) {
+        float u = 0.f;
+        if (MODE == TANGO_ROUND_STOCHASTIC) u = noise ? noise[t] : philox_uniform(seed, offset + t);
+        q[t] = static_cast<int8_t>(quant_one<MODE>(x[t], r, u));
+    }
+}
+
+// Scalar fallback for misaligned views.
+template <int MODE>
+__global__ __launch_bounds__(256) void quantize_scalar_kernel(
+    const float* __restrict__ x, int64_t n, const float* __restrict__ scale,
+    int8_t* __restrict__ q, const float* __restrict__ noise, uint64_t seed, uint64_t offset) {
+    const int64_t tid = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    const int64_t nthr = static_cast<int64_t>(gridDim.x) * blockDim.x;
+    const float r = rscale_of(scale[0]);
+    for (int64_t i = tid; i < n; i += nthr) {
+        float u = 0.f;
+        if (MODE == TANGO_ROUND_STOCHASTIC) u = noise ? noise[i] : philox_uniform(seed, offset + i);
+        q[i] = static_cast<int8_t>(quant_one<MODE>(x[i], r, u));
+    }
+}
+
+// Row-strided: one thread per output dword (4 columns of one row, padding included).
+template <int MODE>
+__global__ __launch_bounds__(256) void quantize_rows_kernel(
+    const float* __restrict__ x, int64_t rows, int64_t cols, int64_t ldx,
+    const float* __restrict__ scale, int per_row, int8_t* __restrict__ q, int64_t ldq,
+    const float* __restrict__ noise, uint64_t seed, uint64_t offset) {
+    const int64_t groups = (ldq + 3) >> 2;  // dword groups per row
+    const int64_t total = rows * groups;
+    const int64_t nthr = static_cast<int64_t>(gridDim.x) * blockDim.x;
+    const bool dword_ok = (ldq & 3) == 0 && (reinterpret_cast<uintptr_t>(q) & 3) == 0;
+    for (int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < total;
+         i += nthr) {
+        const int64_t row = i / groups;
+        const int64_t c0 = (i - row * groups) << 2;
+        const float r = rscale_of(scale[per_row ? row : 0]);
+        int v[4];
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            const int64_t c = c0 + k;
+            v[k] = 0;
+            if (c < cols) {
+                float u = 0.f;
+                const int64_t lin = row * cols + c;
+                if (MODE == TANGO_ROUND_STOCHASTIC)
+                    u = noise ? noise[lin] : philox_uniform(seed, offset + lin);
+                v[k] = quant_one<MODE>(x[row * ldx + c], r, u);
+            }
+        }
+        int8_t* qr = q + row * ldq + c0;
+        if (dword_ok) {
+            *reinterpret_cast<uint32_t*>(qr) = pack4(v[0], v[1], v[2], v[3]);
+        } else {
+#pragma unroll
+            for (int k = 0; k < 4; ++k)
+                if (c0 + k < ldq) qr[k] = static_cast<int8_t>(v[k]);
+        }
+    }
+}
+
+// --------------------------------------------------------- transpose_quant
+// x[nrow, ncol] fp32 -> out[ncol, nrow] int8.  One thread owns four
+// consecutive rows, so for every column the wavefront stores 256 contiguous
+// bytes; the reads of a wavefront cover one contiguous 1 KiB * ncol span.
+__global__ __launch_bounds__(256) void transpose_quant_kernel(const float* __restrict__ x,
+                                                              int64_t nrow, int64_t ncol,
+                                                              const float* __restrict__ scale,
+                                                              int8_t* __restrict__ out) {
+    const float r = rscale_of(scale[0]);
+    const int64_t groups = (nrow + 3) >> 2;
+    const int64_t nthr = static_cast<int64_t>(gridDim.x) * blockDim.x;
+    const bool dword_ok = (nrow & 3) == 0 && (reinterpret_cast<uintptr_t>(out) & 3) == 0;
+    for (int64_t g = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; g < groups;
+         g += nthr) {
+        const int64_t r0 = g << 2;
+        for (int64_t c = 0; c < ncol; ++c) {
+            int v[4];
+#pragma unroll
+            for (int k = 0; k < 4; ++k)
+                v[k] = (r0 + k < nrow) ? quant_one<TANGO_ROUND_RNE>(x[(r0 + k) * ncol + c], r, 0.f) : 0;
+            int8_t* o = out + c * nrow + r0;
+            if (dword_ok) {
+                *reinterpret_cast<uint32_t*>(o) = pack4(v[0], v[1], v[2], v[3]);
+            } else {
+#pragma unroll
+                for (int k = 0; k < 4; ++k)
+                    if (r0 + k < nrow) o[k] = static_cast<int8_t>(v[k]);
+            }
+        }
+    }
+}
+
+template <typename F>
+static int dispatch_mode(int mode, F&& f) {
+    switch (mode) {
+        case TANGO_ROUND_RNE: f(std::integral_constant<int, TANGO_ROUND_RNE>{}); return TANGO_OK;
+        case TANGO_ROUND_TRUNC: f(std::integral_constant<int, TANGO_ROUND_TRUNC>{}); return TANGO_OK;
+        case TANGO_ROUND_STOCHASTIC:
+            f(std::integral_constant<int, TANGO_ROUND_STOCHASTIC>{});
+            return TANGO_OK;
+        default: return TANGO_ERR_UNSUPPORTED;
+    }
+}
+
+}  // namespace tango
+
+using namespace tango;
+
+extern "C" {
+
+const char* tango_status_string(int status) {
+    switch (status) {
+        case TANGO_OK: return "ok";
+        case TANGO_ERR_INVALID_ARG: return "invalid argument";
+        case TANGO_ERR_UNSUPPORTED: return "unsupported op, mode or shape";
+        case TANGO_ERR_LAUNCH: return "kernel launch failed";
+        case TANGO_ERR_WORKSPACE: return "workspace missing or too small";
+        default: return "unknown status";
+    }
+}
+
+int tango_abi_version(void) { return 1; }
+
+int tango_absmax_f32(const float* x, int64_t n, float* scale_out, tango_stream_t stream) {
+    if (!scale_out || n < 0 || (n > 0 && !x)) return TANGO_ERR_INVALID_ARG;
+    if ((reinterpret_cast<uintptr_t>(x) & 3) != 0) return TANGO_ERR_INVALID_ARG;
+    hipStream_t s = as_stream(stream);
+    if (n <= (1 << 16)) {
+        hipLaunchKernelGGL(absmax_small_kernel, dim3(1), dim3(1024), 0, s, x, n, scale_out);
+        return launch_status();
+    }
+    fill_u32(scale_out, 0u, 1, s);
+    const int64_t head = ((16 - (reinterpret_cast<uintptr_t>(x) & 15)) & 15) >> 2;
+    const int grid = grid_for(n / 16, 256);
+    hipLaunchKernelGGL(absmax_kernel, dim3(grid), dim3(256), 0, s, x, n, head, scale_out);
+    return launch_status();
+}
+
+int tango_absmax_rows_f32(const float* x, int64_t rows, int64_t cols, int64_t ldx,
+                          float* scale_out, tango_stream_t stream) {
+    if (rows < 0 || cols < 0 || ldx < cols || (rows > 0 && (!x || !scale_out)))
+        return TANGO_ERR_INVALID_ARG;
+    if (rows == 0) return TANGO_OK;
+    const int64_t blocks = ceil_div(rows, 4);
+    if (blocks > INT32_MAX) return TANGO_ERR_UNSUPPORTED;
+    hipLaunchKernelGGL(absmax_rows_kernel, dim3(static_cast<unsigned>(blocks)), dim3(256), 0,
+                       as_stream(stream), x, rows, cols, ldx, scale_out);
+    return launch_status();
+}
+
+int tango_quantize_f32_i8(const float* x, int64_t n, const float* scale, int8_t* q,
+                          int round_mode, const float* noise, uint64_t seed, uint64_t offset,
+                          tango_stream_t stream) {
+    if (n < 0 || !scale || (n > 0 && (!x || !q))) return TANGO_ERR_INVALID_ARG;
+    if (n == 0) return (round_mode >= 0 && round_mode <= 2) ? TANGO_OK : TANGO_ERR_UNSUPPORTED;
+    hipStream_t s = as_stream(stream);
+    const bool vec = (reinterpret_cast<uintptr_t>(x) & 15) == 0 && (reinterpret_cast<uintptr_t>(q) & 3) == 0;
+    int rc = dispatch_mode(round_mode, [&](auto mode) {
+        constexpr int M = decltype(mode)::value;
+        if (vec) {
+            hipLaunchKernelGGL(quantize_vec_kernel<M>, dim3(grid_for(ceil_div(n, 4), 256)), dim3(256),
+                               0, s, x, n, scale, q, noise, seed, offset);
+        } else {
+            hipLaunchKernelGGL(quantize_scalar_kernel<M>, dim3(grid_for(n, 256)), dim3(256), 0, s, x,
+                               n, scale, q, noise, seed, offset);
+        }
+    });
+    return rc != TANGO_OK ? rc : launch_status();
+}
+
+int tango_quantize_rows_f32_i8(const float* x, int64_t rows, int64_t cols, int64_t ldx,
+                               const float* scale, int per_row, int8_t* q, int64_t ldq,
+                               int round_mode, const float* noise, uint64_t seed,
+                               uint64_t offset, tango_stream_t stream) {
+    if (rows < 0 || cols < 0 || ldx < cols || ldq < cols || !scale ||
+        (rows * cols > 0 && (!x || !q)))
+        return TANGO_ERR_INVALID_ARG;
+    if (rows == 0 || ldq == 0) return (round_mode >= 0 && round_mode <= 2) ? TANGO_OK : TANGO_ERR_UNSUPPORTED;
+    hipStream_t s = as_stream(stream);
+    const int64_t total = rows * ((ldq + 3) >> 2);
+    int rc = dispatch_mode(round_mode, [&](auto mode) {
+        constexpr int M = decltype(mode)::value;
+        hipLaunchKernelGGL(quantize_rows_kernel<M>, dim3(grid_for(total, 256)), dim3(256), 0, s, x,
+                           rows, cols, ldx, scale, per_row, q, ldq, noise, seed, offset);
+    });
+    return rc != TANGO_OK ? rc : launch_status();
+}
+
+int tango_transpose_quant_f32_i8(const float* x, int64_t nrow, int64_t ncol, const float* scale,
+                                 int8_t* out, tango_stream_t stream) {
+    if (nrow < 0 || ncol < 0 || !scale || (nrow * ncol > 0 && (!x || !out)))
+        return TANGO_ERR_INVALID_ARG;
+    if (nrow * ncol == 0) return TANGO_OK;
+    hipLaunchKernelGGL(transpose_quant_kernel, dim3(grid_for(ceil_div(nrow, 4), 256)), dim3(256), 0,
+                       as_stream(stream), x, nrow, ncol, scale, out);
+    return launch_status();
+}
+
+}  // extern "C"

@@ -1,0 +1,166 @@
+// Quantized SDDMM for gfx950: per-edge dot products and element-wise ops on
+// int8 node features gathered by (src, dst).
+//
+// Edge-parallel and memory-bound (two gathered rows + 16 index bytes in, H or
+// T floats out per edge); no MFMA.  One lane owns one (edge, head) pair of the
+// dot product, so the lanes of an edge read consecutive D-byte chunks of the
+// two rows and write consecutive floats; the reduction over D runs inside the
+// lane with v_dot4 on 16-, 4- or 1-byte loads and needs no cross-lane step
+// (the reference spends a 32-lane shuffle tree per head on byte loads,
+// cuda/src/SDDMM.cu:25-34).
+#include "common.hpp"
+
+namespace tango {
+
+template <int VEC, bool REDUCE>
+__global__ __launch_bounds__(256) void sddmm_dot_kernel(
+    float* __restrict__ out, float* __restrict__ scale_out, const int64_t* __restrict__ src,
+    const int64_t* __restrict__ dst, const int8_t* __restrict__ U, const int8_t* __restrict__ V,
+    const float* __restrict__ sU, const float* __restrict__ sV, int64_t E, int H, int D) {
+    const float s = sU[0] * sV[0];
+    const int64_t total = E * H;
+    const int64_t nthr = static_cast<int64_t>(gridDim.x) * blockDim.x;
+    float m = 0.0f;
+    for (int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < total; i += nthr) {
+        const int64_t e = i / H;
+        const int h = static_cast<int>(i - e * H);
+        const int8_t* u = U + (src[e] * H + h) * D;
+        const int8_t* v = V + (dst[e] * H + h) * D;
+        int acc = 0;
+        if (VEC == 16) {
+            for (int d = 0; d < D; d += 16) {
+                const u32x4 a = *reinterpret_cast<const u32x4*>(u + d);
+                const u32x4 b = *reinterpret_cast<const u32x4*>(v + d);
+                acc = __builtin_amdgcn_sdot4(a.x, b.x, acc, false);
+                acc = __builtin_amdgcn_sdot4(a.y, b.y, acc, false);
+                acc = __builtin_amdgcn_sdot4(a.z, b.z, acc, false);
+                acc = __builtin_amdgcn_sdot4(a.w, b.w, acc, false);
+            }
+        } else if (VEC == 4) {
+            for (int d = 0; d < D; d += 4)
+                acc = __builtin_amdgcn_sdot4(*reinterpret_cast<const int*>(u + d),
+                                             *reinterpret_cast<const int*>(v + d), acc, false);
+        } else {
+            for (int d = 0; d < D; ++d) acc += static_cast<int>(u[d]) * static_cast<int>(v[d]);
+        }
+        const float y = static_cast<float>(acc) * s;
+        __builtin_nontemporal_store(y, out + i);
+        if (REDUCE) m = fmaxf(m, fabsf(y));
+    }
+    if (REDUCE) block_absmax_to_global(m / 127.0f, scale_out);
+}
+
+template <int OP>
+__device__ __forceinline__ float apply_op(float a, float b) {
+    if (OP == TANGO_OP_ADD) return a + b;
+    if (OP == TANGO_OP_SUB) return a - b;
+    if (OP == TANGO_OP_MUL) return a * b;
+    return a / b;
+}
+
+// One lane owns VEC consecutive outputs of one edge.
+template <int OP, int VEC, bool REDUCE>
+__global__ __launch_bounds__(256) void sddmm_ewise_kernel(
+    float* __restrict__ out, float* __restrict__ scale_out, const int64_t* __restrict__ src,
+    const int64_t* __restrict__ dst, const int8_t* __restrict__ U, const int8_t* __restrict__ V,
+    const float* __restrict__ sU, const float* __restrict__ sV, int64_t E, int64_t T) {
+    const float su = sU[0], sv = sV[0];
+    const int64_t per = T / VEC;  // VEC divides T
+    const int64_t total = E * per;
+    const int64_t nthr = static_cast<int64_t>(gridDim.x) * blockDim.x;
+    float m = 0.0f;
+    for (int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < total; i += nthr) {
+        const int64_t e = i / per;
+        const int64_t t = (i - e * per) * VEC;
+        const int8_t* u = U + src[e] * T + t;
+        const int8_t* v = V + dst[e] * T + t;
+        if (VEC == 4) {
+            const int a = *reinterpret_cast<const int*>(u);
+            const int b = *reinterpret_cast<const int*>(v);
+            f32x4 y;
+            y.x = apply_op<OP>(static_cast<float>(static_cast<int8_t>(a)) * su,
+                               static_cast<float>(static_cast<int8_t>(b)) * sv);
+            y.y = apply_op<OP>(static_cast<float>(static_cast<int8_t>(a >> 8)) * su,
+                               static_cast<float>(static_cast<int8_t>(b >> 8)) * sv);
+            y.z = apply_op<OP>(static_cast<float>(static_cast<int8_t>(a >> 16)) * su,
+                               static_cast<float>(static_cast<int8_t>(b >> 16)) * sv);
+            y.w = apply_op<OP>(static_cast<float>(a >> 24) * su, static_cast<float>(b >> 24) * sv);
+            __builtin_nontemporal_store(y, reinterpret_cast<f32x4*>(out + e * T + t));
+            if (REDUCE) m = fmaxf(m, fmaxf(fmaxf(fabsf(y.x), fabsf(y.y)), fmaxf(fabsf(y.z), fabsf(y.w))));
+        } else {
+            const float y = apply_op<OP>(static_cast<float>(u[0]) * su, static_cast<float>(v[0]) * sv);
+            out[e * T + t] = y;
+            if (REDUCE) m = fmaxf(m, fabsf(y));
+        }
+    }
+    if (REDUCE) block_absmax_to_global(m / 127.0f, scale_out);
+}
+
+}  // namespace tango
+
+using namespace tango;
+
+extern "C" {
+
+int tango_sddmm_dot_i8(float* out, float* scale_out, const int64_t* src, const int64_t* dst,
+                       const int8_t* U, const int8_t* V, const float* sU, const float* sV,
+                       int64_t num_edges, int64_t H, int64_t D, tango_stream_t stream) {
+    if (num_edges < 0 || H < 0 || D < 0 || !sU || !sV ||
+        (num_edges * H > 0 && (!out || !src || !dst || !U || !V)))
+        return TANGO_ERR_INVALID_ARG;
+    if (H >= (1LL << 31) || D >= (1LL << 31)) return TANGO_ERR_UNSUPPORTED;
+    hipStream_t s = as_stream(stream);
+    if (scale_out) fill_u32(scale_out, 0u, 1, s);
+    const int64_t total = num_edges * H;
+    if (total == 0) return launch_status();
+    const uintptr_t al = reinterpret_cast<uintptr_t>(U) | reinterpret_cast<uintptr_t>(V);
+    const int vec = ((D & 15) == 0 && (al & 15) == 0) ? 16 : ((D & 3) == 0 && (al & 3) == 0) ? 4 : 1;
+    const dim3 grid(grid_for(total, 256, 16)), block(256);
+#define TANGO_DOT(V_, R_)                                                                         \
+    hipLaunchKernelGGL((sddmm_dot_kernel<V_, R_>), grid, block, 0, s, out, scale_out, src, dst, U, \
+                       V, sU, sV, num_edges, static_cast<int>(H), static_cast<int>(D))
+    if (scale_out) {
+        if (vec == 16) TANGO_DOT(16, true); else if (vec == 4) TANGO_DOT(4, true); else TANGO_DOT(1, true);
+    } else {
+        if (vec == 16) TANGO_DOT(16, false); else if (vec == 4) TANGO_DOT(4, false); else TANGO_DOT(1, false);
+    }
+#undef TANGO_DOT
+    return launch_status();
+}
+
+int tango_sddmm_ewise_i8(int op, float* out, float* scale_out, const int64_t* src,
+                         const int64_t* dst, const int8_t* U, const int8_t* V, const float* sU,
+                         const float* sV, int64_t num_edges, int64_t T, tango_stream_t stream) {
+    if (op < TANGO_OP_ADD || op > TANGO_OP_DIV) return TANGO_ERR_UNSUPPORTED;
+    if (num_edges < 0 || T < 0 || !sU || !sV ||
+        (num_edges * T > 0 && (!out || !src || !dst || !U || !V)))
+        return TANGO_ERR_INVALID_ARG;
+    hipStream_t s = as_stream(stream);
+    if (scale_out) fill_u32(scale_out, 0u, 1, s);
+    if (num_edges * T == 0) return launch_status();
+    const uintptr_t al = reinterpret_cast<uintptr_t>(U) | reinterpret_cast<uintptr_t>(V);
+    const bool v4 = (T & 3) == 0 && (al & 3) == 0 && (reinterpret_cast<uintptr_t>(out) & 15) == 0;
+    const dim3 grid(grid_for(num_edges * (v4 ? T / 4 : T), 256, 16)), block(256);
+#define TANGO_EW(OP_, V_, R_)                                                                    \
+    hipLaunchKernelGGL((sddmm_ewise_kernel<OP_, V_, R_>), grid, block, 0, s, out, scale_out, src, \
+                       dst, U, V, sU, sV, num_edges, T)
+#define TANGO_EW_OP(OP_)                                                  \
+    do {                                                                  \
+        if (scale_out) {                                                  \
+            if (v4) TANGO_EW(OP_, 4, true); else TANGO_EW(OP_, 1, true);  \
+        } else {                                                          \
+            if (v4) TANGO_EW(OP_, 4, false); else TANGO_EW(OP_, 1, false);\
+        }                                                                 \
+    } while (0)
+    switch (op) {
+        case TANGO_OP_ADD: TANGO_EW_OP(TANGO_OP_ADD); break;
+        case TANGO_OP_SUB: TANGO_EW_OP(TANGO_OP_SUB); break;
+        case TANGO_OP_MUL: TANGO_EW_OP(TANGO_OP_MUL); break;
+        default: TANGO_EW_OP(TANGO_OP_DIV); break;
+    }
+#undef TANGO_EW_OP
+#undef TANGO_EW
+    return launch_status();
+}
+
+}  // extern "C"

@@ -1,0 +1,321 @@
+// Quantized SpMM family for gfx950: copy_u (CSR), u_mul_e (CSR, int8 edge
+// values, optional fused edge-id permutation) and copy_e (sorted incidence COO).
+//
+// These are gather kernels bound by the memory system, not by arithmetic, so
+// no MFMA is used.  Layout of the work:
+//   * a wavefront (or a 4-wave workgroup for high-degree graphs) owns one
+//     output row and walks that row's CSR slots 64 at a time;
+//   * the 64 column indices of a step are fetched with ONE coalesced 512-byte
+//     load (lane i holds slot i) and handed to the lanes that need them with
+//     ds_bpermute, so index traffic is read exactly once;
+//   * a group of `lpe` lanes (power of two) covers one gathered int8 feature
+//     row with 16-, 4- or 1-byte loads per lane, so one load instruction of
+//     the wavefront pulls 64/lpe neighbour rows (F = 256 -> 4 rows of 256 B,
+//     F = 16 -> 64 rows);
+//   * bytes are added into int32 lane accumulators with v_dot4 against a
+//     one-hot (copy_u) or weight-carrying (u_mul_e) byte mask: one VALU op per
+//     byte, exact integer arithmetic, order-independent;
+//   * the lane groups are folded with ds_bpermute shuffles, the waves of a
+//     workgroup through LDS, and the row leaves as fp32 = scale * float(sum).
+#include "common.hpp"
+
+namespace tango {
+
+struct SpmmParams {
+    float* out;
+    const int64_t* indptr;    // CSR kinds: [rows + 1]
+    const int64_t* node_ids;  // COO kind: [nnz], sorted
+    const int64_t* indices;   // gathered row per slot (COO kind: the edge ids)
+    const int64_t* edge_ids;  // weighted kind: slot -> position in evals, or null
+    const int8_t* feat;
+    const int8_t* evals;
+    const float* scale;
+    int64_t rows;
+    int64_t ldf;  // bytes between gathered rows
+    int64_t W;    // bytes summed per gathered row (H * F)
+    int64_t F;    // bytes per head
+    int64_t D;    // edge-value width (1 or F)
+    int64_t nnz;
+    int lpe_log2;  // log2(lanes per gathered row)
+    int out_vec;   // out rows may be stored as 16-byte vectors
+};
+
+enum { KIND_COPY = 0, KIND_WEIGHTED = 1, KIND_COO = 2 };
+
+template <int VEC>
+struct Gather;
+template <>
+struct Gather<16> {
+    using T = u32x4;
+    static __device__ __forceinline__ T load(const int8_t* p) { return *reinterpret_cast<const T*>(p); }
+    static __device__ __forceinline__ T zero() { return T{0u, 0u, 0u, 0u}; }
+};
+template <>
+struct Gather<4> {
+    using T = uint32_t;
+    static __device__ __forceinline__ T load(const int8_t* p) { return *reinterpret_cast<const T*>(p); }
+    static __device__ __forceinline__ T zero() { return 0u; }
+};
+template <>
+struct Gather<1> {
+    using T = int;
+    static __device__ __forceinline__ T load(const int8_t* p) { return static_cast<int>(*p); }
+    static __device__ __forceinline__ T zero() { return 0; }
+};
+
+__device__ __forceinline__ void acc_dword(int* acc, uint32_t d, uint32_t m0) {
+    // m0 holds the multiplier (1 for copy_u, the int8 edge value otherwise) in byte 0
+    acc[0] = __builtin_amdgcn_sdot4(static_cast<int>(d), static_cast<int>(m0), acc[0], false);
+    acc[1] = __builtin_amdgcn_sdot4(static_cast<int>(d), static_cast<int>(m0 << 8), acc[1], false);
+    acc[2] = __builtin_amdgcn_sdot4(static_cast<int>(d), static_cast<int>(m0 << 16), acc[2], false);
+    acc[3] = __builtin_amdgcn_sdot4(static_cast<int>(d), static_cast<int>(m0 << 24), acc[3], false);
+}
+
+template <int VEC>
+__device__ __forceinline__ void accumulate(int* acc, typename Gather<VEC>::T d, int w);
+template <>
+__device__ __forceinline__ void accumulate<16>(int* acc, u32x4 d, int w) {
+    const uint32_t m0 = static_cast<uint32_t>(w) & 0xffu;
+    acc_dword(acc + 0, d.x, m0);
+    acc_dword(acc + 4, d.y, m0);
+    acc_dword(acc + 8, d.z, m0);
+    acc_dword(acc + 12, d.w, m0);
+}
+template <>
+__device__ __forceinline__ void accumulate<4>(int* acc, uint32_t d, int w) {
+    acc_dword(acc, d, static_cast<uint32_t>(w) & 0xffu);
+}
+template <>
+__device__ __forceinline__ void accumulate<1>(int* acc, int d, int w) {
+    acc[0] += d * w;
+}
+
+__device__ __forceinline__ int64_t lower_bound_i64(const int64_t* a, int64_t n, int64_t key) {
+    int64_t lo = 0, hi = n;
+    while (lo < hi) {
+        const int64_t mid = (lo + hi) >> 1;
+        if (a[mid] < key) lo = mid + 1; else hi = mid;
+    }
+    return lo;
+}
+
+// blockDim.x = 256.  WPR = waves that share one output row (1 or 4).
+// gridDim.y tiles the columns in chunks of 64 * VEC bytes.
+template <int VEC, int WPR, int KIND>
+__global__ __launch_bounds__(256) void spmm_kernel(const SpmmParams p) {
+    constexpr int U = 4;  // gather loads in flight per lane
+    const int lane = lane_id();
+    const int wave = __builtin_amdgcn_readfirstlane(static_cast<int>(threadIdx.x) >> 6);
+    const int64_t row = (WPR == 4) ? static_cast<int64_t>(blockIdx.x)
+                                   : static_cast<int64_t>(blockIdx.x) * 4 + wave;
+    __shared__ int part[(WPR == 4) ? 3 * 64 * VEC : 1];
+    if (WPR == 1 && row >= p.rows) return;  // whole wave leaves; no barrier follows for WPR == 1
+
+    const int lpe = 1 << p.lpe_log2;
+    const int epi = kWave >> p.lpe_log2;
+    const int grp = lane >> p.lpe_log2;
+    const int sub = lane & (lpe - 1);
+    const int64_t col = static_cast<int64_t>(blockIdx.y) * (kWave * VEC) + static_cast<int64_t>(sub) * VEC;
+    const bool col_ok = col < p.W;
+
+    int64_t start, end;
+    if (KIND == KIND_COO) {
+        start = lower_bound_i64(p.node_ids, p.nnz, row);
+        end = lower_bound_i64(p.node_ids, p.nnz, row + 1);
+    } else {
+        start = p.indptr[row];
+        end = p.indptr[row + 1];
+    }
+    if (WPR == 4) {
+        const int64_t per = (end - start + 3) >> 2;
+        const int64_t s = start + per * wave;
+        const int64_t e = s + per;
+        start = s < end ? s : end;
+        end = e < end ? e : end;
+    }
+
+    const int8_t* wbase = nullptr;
+    if (KIND == KIND_WEIGHTED && col_ok) {
+        const int64_t h = col / p.F;
+        const int64_t d = (p.D == 1) ? 0 : (col - h * p.F);
+        wbase = p.evals + (h * p.D + d) * p.nnz;
+    }
+
+    int acc[VEC];
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) acc[i] = 0;
+
+    const int8_t* fcol = p.feat + col;
+    int64_t base = start;
+    int my = (base + lane < end) ? static_cast<int>(p.indices[base + lane]) : -1;
+    int my_e = 0;
+    if (KIND == KIND_WEIGHTED && p.edge_ids)
+        my_e = (base + lane < end) ? static_cast<int>(p.edge_ids[base + lane]) : 0;
+
+    while (base < end) {
+        const int64_t nbase = base + kWave;
+        // prefetch the next step's indices while this step's rows are gathered
+        const int nxt = (nbase + lane < end) ? static_cast<int>(p.indices[nbase + lane]) : -1;
+        int nxt_e = 0;
+        if (KIND == KIND_WEIGHTED && p.edge_ids)
+            nxt_e = (nbase + lane < end) ? static_cast<int>(p.edge_ids[nbase + lane]) : 0;
+        const int cnt = static_cast<int>((end - base) < kWave ? (end - base) : kWave);
+        const int steps = (cnt + epi - 1) >> (6 - p.lpe_log2);
+        for (int t = 0; t < steps; t += U) {
+            typename Gather<VEC>::T d[U];
+            int w[U];
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                const int slot = ((t + u) << (6 - p.lpe_log2)) + grp;  // may exceed 63 past the end
+                const int j = __shfl(my, slot & 63, kWave);
+                const bool ok = (t + u) < steps && j >= 0 && col_ok;
+                d[u] = ok ? Gather<VEC>::load(fcol + static_cast<int64_t>(j) * p.ldf) : Gather<VEC>::zero();
+                w[u] = 1;
+                if (KIND == KIND_WEIGHTED) {
+                    int64_t e = base + slot;
+                    if (p.edge_ids) e = __shfl(my_e, slot & 63, kWave);
+                    w[u] = ok ? static_cast<int>(wbase[e]) : 0;
+                }
+            }
+#pragma unroll
+            for (int u = 0; u < U; ++u) accumulate<VEC>(acc, d[u], w[u]);
+        }
+        my = nxt;
+        my_e = nxt_e;
+        base = nbase;
+    }
+
+    // fold the lane groups: afterwards lanes [0, lpe) hold the wave's column sums
+    for (int off = lpe; off < kWave; off <<= 1) {
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) acc[i] += __shfl_xor(acc[i], off, kWave);
+    }
+
+    if (WPR == 4) {
+        if (wave > 0 && grp == 0) {
+#pragma unroll
+            for (int i = 0; i < VEC; ++i) part[(wave - 1) * 64 * VEC + i * 64 + sub] = acc[i];
+        }
+        __syncthreads();
+        if (wave > 0) return;
+        if (grp == 0) {
+#pragma unroll
+            for (int i = 0; i < VEC; ++i)
+                acc[i] += part[i * 64 + sub] + part[64 * VEC + i * 64 + sub] + part[2 * 64 * VEC + i * 64 + sub];
+        }
+    }
+
+    if (grp == 0 && col_ok) {
+        const float s = p.scale[0];
+        float* o = p.out + row * p.W + col;
+        if (VEC == 16 && p.out_vec && col + 16 <= p.W) {
+            f32x4* o4 = reinterpret_cast<f32x4*>(o);
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+                o4[i] = f32x4{s * static_cast<float>(acc[4 * i]), s * static_cast<float>(acc[4 * i + 1]),
+                              s * static_cast<float>(acc[4 * i + 2]), s * static_cast<float>(acc[4 * i + 3])};
+        } else {
+#pragma unroll
+            for (int i = 0; i < VEC; ++i)
+                if (col + i < p.W) o[i] = s * static_cast<float>(acc[i]);
+        }
+    }
+}
+
+static int ilog2_ceil(int64_t v) {
+    int l = 0;
+    while ((1LL << l) < v) ++l;
+    return l;
+}
+
+template <int KIND>
+static int launch_spmm(SpmmParams p, int vec, hipStream_t s) {
+    if (p.rows == 0 || p.W == 0) return TANGO_OK;
+    const int64_t lanes = ceil_div(p.W, vec);
+    p.lpe_log2 = lanes >= 64 ? 6 : ilog2_ceil(lanes);
+    p.out_vec = (reinterpret_cast<uintptr_t>(p.out) & 15) == 0 && (p.W & 3) == 0;
+    const int64_t ychunks = ceil_div(p.W, 64 * vec);
+    if (ychunks > 65535) return TANGO_ERR_UNSUPPORTED;
+    // high mean degree: four waves split each row; otherwise one wave per row
+    const bool wide = p.nnz >= 128 * p.rows;
+    const int64_t gx = wide ? p.rows : ceil_div(p.rows, 4);
+    if (gx > INT32_MAX) return TANGO_ERR_UNSUPPORTED;
+    const dim3 grid(static_cast<unsigned>(gx), static_cast<unsigned>(ychunks));
+#define TANGO_SPMM_LAUNCH(V, WPR) \
+    hipLaunchKernelGGL((spmm_kernel<V, WPR, KIND>), grid, dim3(256), 0, s, p)
+    if (vec == 16) {
+        if (wide) TANGO_SPMM_LAUNCH(16, 4); else TANGO_SPMM_LAUNCH(16, 1);
+    } else if (vec == 4) {
+        if (wide) TANGO_SPMM_LAUNCH(4, 4); else TANGO_SPMM_LAUNCH(4, 1);
+    } else {
+        if (wide) TANGO_SPMM_LAUNCH(1, 4); else TANGO_SPMM_LAUNCH(1, 1);
+    }
+#undef TANGO_SPMM_LAUNCH
+    return launch_status();
+}
+
+// Widest per-lane load such that every load of a gathered row is aligned and
+// stays inside the row's ldf bytes.
+static int pick_vec(const int8_t* feat, int64_t ldf, int64_t W) {
+    const uintptr_t a = reinterpret_cast<uintptr_t>(feat);
+    if ((a & 15) == 0 && (ldf & 15) == 0 && ((W + 15) & ~15LL) <= ldf) return 16;
+    if ((a & 3) == 0 && (ldf & 3) == 0 && ((W + 3) & ~3LL) <= ldf) return 4;
+    return 1;
+}
+
+}  // namespace tango
+
+using namespace tango;
+
+extern "C" {
+
+int tango_spmm_csr_copy_u(float* out, const int64_t* indptr, const int64_t* indices,
+                          const int8_t* feat, int64_t ldf, const float* scale, int64_t rows,
+                          int64_t num_src, int64_t nnz, int64_t F, tango_stream_t stream) {
+    if (rows < 0 || F < 0 || nnz < 0 || num_src < 0 || ldf < F || !scale || !indptr ||
+        (rows * F > 0 && !out) || (nnz > 0 && (!indices || !feat)))
+        return TANGO_ERR_INVALID_ARG;
+    if (num_src >= (1LL << 31) || nnz >= (1LL << 31)) return TANGO_ERR_UNSUPPORTED;
+    SpmmParams p{};
+    p.out = out; p.indptr = indptr; p.indices = indices; p.feat = feat; p.scale = scale;
+    p.rows = rows; p.ldf = ldf; p.W = F; p.F = F; p.D = 1; p.nnz = nnz;
+    return launch_spmm<KIND_COPY>(p, pick_vec(feat, ldf, F), as_stream(stream));
+}
+
+int tango_spmm_csr_u_mul_e(float* out, const int64_t* indptr, const int64_t* indices,
+                           const int64_t* edge_ids, const int8_t* feat, const int8_t* evals,
+                           const float* scale, int64_t rows, int64_t num_src, int64_t H,
+                           int64_t F, int64_t D, int64_t nnz, tango_stream_t stream) {
+    if (rows < 0 || H < 0 || F < 0 || nnz < 0 || num_src < 0 || !scale || !indptr ||
+        (rows * H * F > 0 && !out) || (nnz > 0 && (!indices || !feat || !evals)))
+        return TANGO_ERR_INVALID_ARG;
+    if (D != 1 && D != F) return TANGO_ERR_UNSUPPORTED;
+    if (num_src >= (1LL << 31) || nnz >= (1LL << 31)) return TANGO_ERR_UNSUPPORTED;
+    SpmmParams p{};
+    p.out = out; p.indptr = indptr; p.indices = indices; p.edge_ids = edge_ids; p.feat = feat;
+    p.evals = evals; p.scale = scale; p.rows = rows; p.ldf = H * F; p.W = H * F; p.F = F; p.D = D;
+    p.nnz = nnz;
+    // a lane's bytes must share one edge value: vector loads only when they stay inside a head
+    int vec = 1;
+    if (D == 1 && F > 0) {
+        const uintptr_t a = reinterpret_cast<uintptr_t>(feat);
+        if ((F & 15) == 0 && (a & 15) == 0) vec = 16;
+        else if ((F & 3) == 0 && (a & 3) == 0) vec = 4;
+    }
+    return launch_spmm<KIND_WEIGHTED>(p, vec, as_stream(stream));
+}
+
+int tango_spmm_incidence(float* out, const int64_t* node_ids, const int64_t* edge_ids,
+                         const int8_t* E, const float* scale, int64_t num_nodes, int64_t nnz,
+                         int64_t num_edges, int64_t F, tango_stream_t stream) {
+    if (num_nodes < 0 || nnz < 0 || num_edges < 0 || F < 0 || !scale ||
+        (num_nodes * F > 0 && !out) || (nnz > 0 && (!node_ids || !edge_ids || !E)))
+        return TANGO_ERR_INVALID_ARG;
+    if (num_edges >= (1LL << 31) || nnz >= (1LL << 31)) return TANGO_ERR_UNSUPPORTED;
+    SpmmParams p{};
+    p.out = out; p.node_ids = node_ids; p.indices = edge_ids; p.feat = E; p.scale = scale;
+    p.rows = num_nodes; p.ldf = F; p.W = F; p.F = F; p.D = 1; p.nnz = nnz;
+    return launch_spmm<KIND_COO>(p, pick_vec(E, F, F), as_stream(stream));
+}
+
+}  // extern "C"

@@ -1,0 +1,151 @@
+"""A DGL-free graph object carrying exactly what the primitive layer reads.
+
+The reference's wrappers touch five cached attributes of a DGL graph plus
+``num_nodes()`` (cuda/kernels.py:35-37,128-130,142-148,156-160); the model
+code additionally reads degrees and uses ``local_scope`` and the feature
+dictionaries.  ``Graph`` offers that surface on torch tensors, and
+``chung_lu`` generates the seeded synthetic power-law graphs the benchmarks
+run on (the reference's datasets are fetched from the network).
+"""
+import contextlib
+
+import torch
+
+
+def _compress(rows, cols, num_nodes):
+    """COO -> (indptr, indices, edge_ids) with rows sorted stably (edge-id order within a row)."""
+    order = torch.sort(rows, stable=True).indices
+    counts = torch.bincount(rows, minlength=num_nodes)
+    indptr = torch.zeros(num_nodes + 1, dtype=torch.int64, device=rows.device)
+    torch.cumsum(counts, 0, out=indptr[1:])
+    return indptr, cols[order].contiguous(), order.contiguous()
+
+
+class Graph:
+    """Homogeneous directed multigraph on ``num_nodes`` nodes; edge e is (src[e], dst[e])."""
+
+    is_block = False
+
+    def __init__(self, src, dst, num_nodes):
+        self._src = src.to(torch.int64).contiguous()
+        self._dst = dst.to(torch.int64).contiguous()
+        self._n = int(num_nodes)
+        self.ndata, self.edata = {}, {}
+        self.srcdata = self.dstdata = self.ndata
+        self._csr = self._csc = None
+
+    # -- the DGL calls of cuda/util.py:5-11 ---------------------------------
+    @property
+    def device(self):
+        return self._src.device
+
+    def to(self, device):
+        g = Graph(self._src.to(device), self._dst.to(device), self._n)
+        return g
+
+    def num_nodes(self):
+        return self._n
+
+    number_of_nodes = num_nodes
+    number_of_dst_nodes = num_nodes
+
+    def num_edges(self):
+        return self._src.numel()
+
+    number_of_edges = num_edges
+
+    def edges(self):
+        return self._src, self._dst
+
+    def adj_sparse(self, fmt):
+        """'csr': rows = source nodes; 'csc': rows = destination nodes."""
+        if fmt == "csr":
+            if self._csr is None:
+                self._csr = _compress(self._src, self._dst, self._n)
+            return self._csr
+        if fmt == "csc":
+            if self._csc is None:
+                self._csc = _compress(self._dst, self._src, self._n)
+            return self._csc
+        raise ValueError("format must be 'csr' or 'csc'")
+
+    def incidence(self, typ):
+        """[2, E] (node, edge) pairs sorted by node then edge: what
+        ``g.inc(typ).coalesce().indices()`` yields in the reference."""
+        if typ == "in":
+            _, _, eid = self.adj_sparse("csc")
+            return torch.stack([self._dst[eid], eid])
+        if typ == "out":
+            _, _, eid = self.adj_sparse("csr")
+            return torch.stack([self._src[eid], eid])
+        raise ValueError("typ must be 'in' or 'out'")
+
+    def in_degrees(self):
+        return torch.bincount(self._dst, minlength=self._n)
+
+    def out_degrees(self):
+        return torch.bincount(self._src, minlength=self._n)
+
+    @contextlib.contextmanager
+    def local_scope(self):
+        yield self
+
+
+def remove_self_loop(src, dst):
+    keep = src != dst
+    return src[keep], dst[keep]
+
+
+def add_self_loop(src, dst, num_nodes):
+    loops = torch.arange(num_nodes, dtype=src.dtype, device=src.device)
+    return torch.cat([src, loops]), torch.cat([dst, loops])
+
+
+def chung_lu(num_nodes, num_edges, gamma, seed, max_degree=None, symmetric=False,
+             self_loops=True, device="cpu"):
+    """Seeded Chung-Lu power-law graph.
+
+    Expected degree of node i is proportional to (i + i0)^(-1/(gamma - 1)),
+    optionally clipped at ``max_degree``.  Endpoints are drawn by inverse-CDF
+    sampling, duplicate edges dropped, the graph optionally symmetrised, and
+    self loops normalised the way the reference's loader does it
+    (evaluation/util.py:28: remove_self_loop then add_self_loop).
+    ``num_edges`` is the target number of directed edges before self loops.
+    """
+    gen = torch.Generator(device=device)
+    gen.manual_seed(int(seed))
+    i = torch.arange(num_nodes, dtype=torch.float64, device=device)
+    w = (i + 1.0).pow(-1.0 / (gamma - 1.0))
+    draws = num_edges // 2 if symmetric else num_edges
+    if max_degree is not None:
+        # scale, clip, rescale a few times so that the clipped weights still sum to the target
+        for _ in range(8):
+            w = w * (draws / w.sum())
+            w = w.clamp(max=float(max_degree) / (2.0 if symmetric else 1.0))
+    cdf = torch.cumsum(w / w.sum(), 0)
+    cdf[-1] = 1.0
+    keys = torch.empty(0, dtype=torch.int64, device=device)
+    need = draws
+    for _ in range(6):  # top up what duplicate removal took away
+        m = int(need * 1.15) + 16
+        u = torch.rand(2, m, generator=gen, device=device, dtype=torch.float64)
+        s = torch.searchsorted(cdf, u[0]).clamp_(max=num_nodes - 1)
+        d = torch.searchsorted(cdf, u[1]).clamp_(max=num_nodes - 1)
+        if symmetric:
+            s, d = torch.minimum(s, d), torch.maximum(s, d)
+        k = s * num_nodes + d
+        k = k[s != d]
+        keys = torch.unique(torch.cat([keys, k]))
+        need = draws - keys.numel()
+        if need <= 0:
+            break
+    if keys.numel() > draws:
+        perm = torch.randperm(keys.numel(), generator=gen, device=device)[:draws]
+        keys = keys[perm.sort().values]
+    src = keys // num_nodes
+    dst = keys - src * num_nodes
+    if symmetric:
+        src, dst = torch.cat([src, dst]), torch.cat([dst, src])
+    if self_loops:
+        src, dst = add_self_loop(src, dst, num_nodes)
+    return Graph(src, dst, num_nodes)

@@ -1,0 +1,499 @@
+"""Functional layer over libtango_hip: mirrors cuda/kernels.py of the reference.
+
+``cuda_kernels`` exposes the fourteen callables of the reference's pybind11
+module (cuda/src/cuda.cpp:182-204) with the same names, arity and argument
+meaning; the module-level functions are the reference's Python wrappers
+(cuda/kernels.py:19-178).  torch supplies device memory and the current
+stream; all arithmetic runs in the HIP library.  Keyword arguments that the
+reference does not have (``round_mode``, ``noise``, ``seed``, ``offset``,
+``edge_ids``) default to the reference's behaviour.
+"""
+import os
+
+import torch
+
+from . import _lib
+from ._lib import ROUND_MODES, ROUND_RNE, ROUND_STOCHASTIC, ROUND_TRUNC, SDDMM_OPS, check
+
+_L = _lib.lib()  # fails here, loudly, if the library is not built
+
+
+def _stream():
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _ptr(t):
+    return None if t is None or t.numel() == 0 else t.data_ptr()
+
+
+def _need(t, dtype, name, contiguous=True):
+    if not isinstance(t, torch.Tensor):
+        raise TypeError("%s must be a tensor" % name)
+    if t.dtype != dtype:
+        raise RuntimeError("%s: expected %s but got %s" % (name, dtype, t.dtype))
+    if not t.is_cuda:
+        raise RuntimeError("%s must be on GPU" % name)
+    if contiguous and not t.is_contiguous():
+        raise RuntimeError("%s must be contiguous" % name)
+    return t
+
+
+def _rows_view(t, name):
+    """2-D row-major view with unit column stride; returns (tensor, row stride)."""
+    if t.dim() != 2 or (t.size(1) > 1 and t.stride(1) != 1):
+        raise RuntimeError("%s must be 2-D with contiguous rows" % name)
+    return t.stride(0) if t.size(0) > 1 else max(t.size(1), t.stride(0))
+
+
+def _mode(round_mode):
+    if isinstance(round_mode, str):
+        return ROUND_MODES[round_mode]
+    return int(round_mode)
+
+
+def default_forward_round_mode():
+    """Rounding of the GEMM's fused quantize.  The reference truncates
+    (cuda/src/iterator.h:161); TANGO_ROUND_MODE=rne selects half-to-even."""
+    return ROUND_MODES[os.environ.get("TANGO_ROUND_MODE", "trunc")]
+
+
+def infer_broadcast_shape(op, shp1, shp2):
+    """Restates dgl.sparse.infer_broadcast_shape (imported at cuda/kernels.py:3):
+    left-pad to equal rank, dims must match or be 1, result is the element-wise
+    maximum; for 'dot' the last dims must match and the result's becomes 1."""
+    shp1, shp2 = tuple(shp1), tuple(shp2)
+    pad = max(len(shp1), len(shp2))
+    a = (1,) * (pad - len(shp1)) + shp1
+    b = (1,) * (pad - len(shp2)) + shp2
+    for d1, d2 in zip(a, b):
+        if d1 != d2 and d1 != 1 and d2 != 1:
+            raise ValueError("Feature shapes %s and %s are not broadcastable" % (shp1, shp2))
+    out = tuple(max(d1, d2) for d1, d2 in zip(a, b))
+    if op == "dot":
+        if a[-1] != b[-1]:
+            raise ValueError("dot needs equal last dimensions")
+        out = out[:-1] + (1,)
+    return out
+
+
+class cuda_kernels:
+    """Namespace with the reference extension's bindings (cuda/src/cuda.cpp:182-204)."""
+
+    # ---------------------------------------------------------- quantization
+    @staticmethod
+    def get_scale(inp):
+        _need(inp, torch.float32, "in")
+        scale = torch.empty(1, dtype=torch.float32, device=inp.device)
+        check(_L.tango_absmax_f32(_ptr(inp), inp.numel(), scale.data_ptr(), _stream()), "get_scale")
+        return scale
+
+    @staticmethod
+    def get_scale_rows(inp):
+        """Per-row scales of a 2-D tensor (not in the reference)."""
+        _need(inp, torch.float32, "in", contiguous=False)
+        ld = _rows_view(inp, "in")
+        scale = torch.empty(inp.size(0), dtype=torch.float32, device=inp.device)
+        check(_L.tango_absmax_rows_f32(_ptr(inp), inp.size(0), inp.size(1), ld, _ptr(scale), _stream()),
+              "get_scale_rows")
+        return scale
+
+    @staticmethod
+    def quantize(out, inp, scale, round_mode=ROUND_RNE, noise=None, seed=0, offset=0):
+        _need(out, torch.int8, "out")
+        _need(inp, torch.float32, "in")
+        _need(scale, torch.float32, "scale")
+        if out.numel() != inp.numel():
+            raise RuntimeError("quantize: out and in differ in size")
+        if noise is not None:
+            _need(noise, torch.float32, "noise")
+            if noise.numel() != inp.numel():
+                raise RuntimeError("quantize: noise and in differ in size")
+        check(_L.tango_quantize_f32_i8(_ptr(inp), inp.numel(), scale.data_ptr(), _ptr(out),
+                                       _mode(round_mode), _ptr(noise), int(seed), int(offset),
+                                       _stream()), "quantize")
+
+    @staticmethod
+    def quantize_rows(out, inp, scale, per_row=False, round_mode=ROUND_RNE, noise=None, seed=0,
+                      offset=0):
+        """Row-strided quantize into a possibly wider (zero-padded) int8 matrix (not in the reference)."""
+        _need(out, torch.int8, "out", contiguous=False)
+        _need(inp, torch.float32, "in", contiguous=False)
+        _need(scale, torch.float32, "scale")
+        ldx, ldq = _rows_view(inp, "in"), _rows_view(out, "out")
+        if out.size(0) != inp.size(0) or out.size(1) < inp.size(1):
+            raise RuntimeError("quantize_rows: out must have in's rows and at least its columns")
+        ldq_pad = out.size(1)
+        if out.size(0) > 1 and ldq != ldq_pad:
+            raise RuntimeError("quantize_rows: out must be dense")
+        if noise is not None:
+            _need(noise, torch.float32, "noise")
+        check(_L.tango_quantize_rows_f32_i8(_ptr(inp), inp.size(0), inp.size(1), ldx, scale.data_ptr(),
+                                            int(bool(per_row)), _ptr(out), ldq_pad, _mode(round_mode),
+                                            _ptr(noise), int(seed), int(offset), _stream()),
+              "quantize_rows")
+
+    @staticmethod
+    def transpose_quant(inp, scale, nrow, ncol):
+        _need(inp, torch.float32, "in")
+        _need(scale, torch.float32, "scale")
+        if inp.numel() != nrow * ncol:
+            raise RuntimeError("transpose_quant: in has %d elements, expected %d" % (inp.numel(), nrow * ncol))
+        out = torch.empty((ncol, nrow), dtype=torch.int8, device=inp.device)
+        check(_L.tango_transpose_quant_f32_i8(_ptr(inp), nrow, ncol, scale.data_ptr(), _ptr(out),
+                                              _stream()), "transpose_quant")
+        return out
+
+    # ------------------------------------------------------------------ GEMM
+    @staticmethod
+    def QGEMM_forward(Y, X, X_q, W, W_q, bias, scaleY, scaleX, scaleW, round_mode=None):
+        for t, dt, nm in ((Y, torch.float32, "Y"), (X, torch.float32, "X"), (W, torch.float32, "W")):
+            _need(t, dt, nm, contiguous=False)
+        _need(X_q, torch.int8, "X_q")
+        _need(W_q, torch.int8, "W_q")
+        _need(scaleX, torch.float32, "scaleX")
+        _need(scaleW, torch.float32, "scaleW")
+        M, K = X.shape
+        N = W.size(0)
+        if W.size(1) != K or tuple(Y.shape) != (M, N) or X_q.numel() != M * K or W_q.numel() != N * K:
+            raise RuntimeError("QGEMM_forward: shape mismatch")
+        if bias is not None and bias.numel():
+            _need(bias, torch.float32, "bias")
+            if bias.numel() != N:
+                raise RuntimeError("QGEMM_forward: bias must have N elements")
+        if scaleY is not None and scaleY.numel():
+            _need(scaleY, torch.float32, "scaleY")
+        mode = default_forward_round_mode() if round_mode is None else _mode(round_mode)
+        ws_bytes = _L.tango_qgemm_fwd_workspace(M, N, K)
+        ws = torch.empty(ws_bytes, dtype=torch.uint8, device=X.device) if ws_bytes else None
+        check(_L.tango_qgemm_fwd(_ptr(Y), _rows_view(Y, "Y"), _ptr(X), _rows_view(X, "X"), _ptr(X_q),
+                                 _ptr(W), _rows_view(W, "W"), _ptr(W_q), _ptr(bias), _ptr(scaleY),
+                                 scaleX.data_ptr(), scaleW.data_ptr(), M, N, K, mode, _ptr(ws),
+                                 ws_bytes, _stream()), "QGEMM_forward")
+
+    @staticmethod
+    def QGEMM_i8(Y, A, B, bias, scaleY, scaleA, scaleB):
+        """Y = dequant(A[M,K] . B[N,K]^T) on int8 operands (not in the reference)."""
+        _need(Y, torch.float32, "Y", contiguous=False)
+        _need(A, torch.int8, "A", contiguous=False)
+        _need(B, torch.int8, "B", contiguous=False)
+        M, K = A.shape
+        N = B.size(0)
+        if B.size(1) != K or tuple(Y.shape) != (M, N):
+            raise RuntimeError("QGEMM_i8: shape mismatch")
+        check(_L.tango_qgemm_i8_nt(_ptr(Y), _rows_view(Y, "Y"), _ptr(A), _rows_view(A, "A"), _ptr(B),
+                                   _rows_view(B, "B"), _ptr(bias), _ptr(scaleY), scaleA.data_ptr(),
+                                   scaleB.data_ptr(), M, N, K, _stream()), "QGEMM_i8")
+
+    @staticmethod
+    def QGEMM_backward_gradX(dX, dY, W, scaledY, scaleW):
+        _need(dX, torch.float32, "dX", contiguous=False)
+        _need(dY, torch.int8, "dY", contiguous=False)
+        _need(W, torch.int8, "W", contiguous=False)
+        _need(scaledY, torch.float32, "scaledY")
+        _need(scaleW, torch.float32, "scaleW")
+        M, K = dX.shape
+        N = dY.size(1)
+        if dY.size(0) != M or tuple(W.shape) != (N, K):
+            raise RuntimeError("QGEMM_backward_gradX: shape mismatch")
+        check(_L.tango_qgemm_bwd_dx(_ptr(dX), _rows_view(dX, "dX"), _ptr(dY), _rows_view(dY, "dY"),
+                                    _ptr(W), _rows_view(W, "W"), scaledY.data_ptr(), scaleW.data_ptr(),
+                                    M, N, K, _stream()), "QGEMM_backward_gradX")
+
+    @staticmethod
+    def QGEMM_backward_gradW(dW, dY, X, scaledY, scaleX):
+        _need(dW, torch.float32, "dW", contiguous=False)
+        _need(dY, torch.int8, "dY", contiguous=False)
+        _need(X, torch.int8, "X", contiguous=False)
+        _need(scaledY, torch.float32, "scaledY")
+        _need(scaleX, torch.float32, "scaleX")
+        N, K = dW.shape
+        M = dY.size(0)
+        if dY.size(1) != N or tuple(X.shape) != (M, K):
+            raise RuntimeError("QGEMM_backward_gradW: shape mismatch")
+        ws_bytes = _L.tango_qgemm_bwd_dw_workspace(M, N, K)
+        ws = torch.empty(ws_bytes, dtype=torch.uint8, device=X.device) if ws_bytes else None
+        check(_L.tango_qgemm_bwd_dw(_ptr(dW), _rows_view(dW, "dW"), _ptr(dY), _rows_view(dY, "dY"),
+                                    _ptr(X), _rows_view(X, "X"), scaledY.data_ptr(), scaleX.data_ptr(),
+                                    M, N, K, _ptr(ws), ws_bytes, _stream()), "QGEMM_backward_gradW")
+
+    @staticmethod
+    def _legacy(A, B, trans_a, trans_b):
+        _need(A, torch.float32, "A")
+        _need(B, torch.float32, "B")
+        m = A.size(1) if trans_a else A.size(0)
+        k = A.size(0) if trans_a else A.size(1)
+        n = B.size(0) if trans_b else B.size(1)
+        if (B.size(1) if trans_b else B.size(0)) != k:
+            raise RuntimeError("Qgemm: inner dimensions differ")
+        out = torch.empty((m, n), dtype=torch.float32, device=A.device)
+        ws_bytes = _L.tango_qgemm_legacy_workspace(m, n, k)
+        ws = torch.empty(ws_bytes, dtype=torch.uint8, device=A.device) if ws_bytes else None
+        check(_L.tango_qgemm_legacy(_ptr(out), _ptr(A), _ptr(B), m, n, k, int(trans_a), int(trans_b),
+                                    _ptr(ws), ws_bytes, _stream()), "Qgemm")
+        return out
+
+    @staticmethod
+    def QgemmNT(A, B):
+        return cuda_kernels._legacy(A, B, False, True)
+
+    @staticmethod
+    def QgemmTN(A, B):
+        return cuda_kernels._legacy(A, B, True, False)
+
+    @staticmethod
+    def QgemmNN(A, B):
+        return cuda_kernels._legacy(A, B, False, False)
+
+    # ------------------------------------------------------------------ SpMM
+    @staticmethod
+    def csr_SPMM(out, indptr, indices, U, scaleU, ldf=None, F=None):
+        _need(out, torch.float32, "out")
+        _need(indptr, torch.int64, "indptr")
+        _need(indices, torch.int64, "indices")
+        _need(U, torch.int8, "U")
+        _need(scaleU, torch.float32, "scaleU")
+        rows = indptr.numel() - 1
+        width = U.numel() // max(U.size(0), 1)
+        ldf = width if ldf is None else ldf
+        F = width if F is None else F
+        if out.numel() != rows * F:
+            raise RuntimeError("csr_SPMM: out must be [%d, %d]" % (rows, F))
+        check(_L.tango_spmm_csr_copy_u(_ptr(out), indptr.data_ptr(), _ptr(indices), _ptr(U), ldf,
+                                       scaleU.data_ptr(), rows, U.size(0), indices.numel(), F,
+                                       _stream()), "csr_SPMM")
+
+    @staticmethod
+    def multi_cusparse_SPMM(indptr, indices, N, E_T, scale, edge_ids=None):
+        """E_T is [H, D, nnz] in CSR slot order, or in edge-id order when the
+        slot->edge permutation ``edge_ids`` is passed (gather fused in-kernel)."""
+        _need(indptr, torch.int64, "indptr")
+        _need(indices, torch.int64, "indices")
+        _need(N, torch.int8, "N")
+        _need(E_T, torch.int8, "E_T")
+        _need(scale, torch.float32, "scale")
+        if N.dim() != 3 or E_T.dim() != 3:
+            raise RuntimeError("E and N must be 3D tensors")
+        k, H, F = N.shape
+        D, nnz = E_T.size(1), E_T.size(2)
+        if E_T.size(0) != H or nnz != indices.numel() or D not in (1, F):
+            raise RuntimeError("multi_cusparse_SPMM: E_T must be [H, 1|F, nnz]")
+        if edge_ids is not None:
+            _need(edge_ids, torch.int64, "edge_ids")
+        rows = indptr.numel() - 1
+        out = torch.empty((rows, H, F), dtype=torch.float32, device=N.device)
+        check(_L.tango_spmm_csr_u_mul_e(_ptr(out), indptr.data_ptr(), _ptr(indices), _ptr(edge_ids),
+                                        _ptr(N), _ptr(E_T), scale.data_ptr(), rows, k, H, F, D, nnz,
+                                        _stream()), "multi_cusparse_SPMM")
+        return out
+
+    # The reference's SpMV binding returns uninitialised memory (cuda/src/SPMM.cu:196-257)
+    # and its Python wrapper calls the SpMM instead (cuda/kernels.py:168-178).
+    multi_cusparse_SPMV = multi_cusparse_SPMM
+
+    @staticmethod
+    def incidence_SPMM(out, src, dst, E, scale):
+        """src = node ids (sorted), dst = edge ids: rows 0 and 1 of g.inc_in / g.inc_out."""
+        _need(out, torch.float32, "out")
+        _need(src, torch.int64, "src")
+        _need(dst, torch.int64, "dst")
+        _need(E, torch.int8, "E")
+        _need(scale, torch.float32, "scale")
+        F = E.numel() // max(E.size(0), 1)
+        if out.dim() != 2 or out.size(1) != F:
+            raise RuntimeError("incidence_SPMM: out must be [num_nodes, %d]" % F)
+        check(_L.tango_spmm_incidence(_ptr(out), _ptr(src), _ptr(dst), _ptr(E), scale.data_ptr(),
+                                      out.size(0), src.numel(), E.size(0), F, _stream()),
+              "incidence_SPMM")
+
+    # ----------------------------------------------------------------- SDDMM
+    @staticmethod
+    def mySDDMM_int8(op, out, scaleOut, src, dst, U, V, scaleU, scaleV):
+        _need(out, torch.float32, "out")
+        _need(src, torch.int64, "src")
+        _need(dst, torch.int64, "dst")
+        _need(U, torch.int8, "U")
+        _need(V, torch.int8, "V")
+        _need(scaleU, torch.float32, "scaleU")
+        _need(scaleV, torch.float32, "scaleV")
+        if scaleOut is not None and scaleOut.numel():
+            _need(scaleOut, torch.float32, "scaleOut")
+        E = src.numel()
+        if dst.numel() != E:
+            raise RuntimeError("mySDDMM_int8: src and dst differ in length")
+        if U.shape[1:] != V.shape[1:]:
+            raise RuntimeError("mySDDMM_int8: U and V must have equal feature shapes")
+        if op == "dot":
+            D = U.size(-1)
+            H = U.numel() // max(U.size(0), 1) // max(D, 1)
+            if out.numel() != E * H:
+                raise RuntimeError("mySDDMM_int8: out must be [E, %d, 1]" % H)
+            check(_L.tango_sddmm_dot_i8(_ptr(out), _ptr(scaleOut), _ptr(src), _ptr(dst), _ptr(U), _ptr(V),
+                                        scaleU.data_ptr(), scaleV.data_ptr(), E, H, D, _stream()),
+                  "mySDDMM_int8(dot)")
+        elif op in SDDMM_OPS:
+            T = U.numel() // max(U.size(0), 1)
+            if out.numel() != E * T:
+                raise RuntimeError("mySDDMM_int8: out must be [E, %d]" % T)
+            check(_L.tango_sddmm_ewise_i8(SDDMM_OPS[op], _ptr(out), _ptr(scaleOut), _ptr(src), _ptr(dst),
+                                          _ptr(U), _ptr(V), scaleU.data_ptr(), scaleV.data_ptr(), E, T,
+                                          _stream()), "mySDDMM_int8(%s)" % op)
+        else:
+            # the reference only prints "op not supported" (cuda/src/SDDMM.cu:175)
+            raise ValueError("%s op not supported" % op)
+
+    # ---------------------------------------------------------- edge softmax
+    @staticmethod
+    def edge_softmax_forward(e, indptr, edge_ids, slope=1.0):
+        _need(e, torch.float32, "e")
+        _need(indptr, torch.int64, "indptr")
+        H = e.numel() // max(e.size(0), 1)
+        a = torch.empty_like(e)
+        check(_L.tango_edge_softmax_fwd(_ptr(a), _ptr(e), indptr.data_ptr(), _ptr(edge_ids),
+                                        indptr.numel() - 1, H, float(slope), _stream()), "edge_softmax")
+        return a
+
+    @staticmethod
+    def edge_softmax_backward(a, da, e, indptr, edge_ids, slope=1.0):
+        _need(a, torch.float32, "a")
+        _need(da, torch.float32, "da")
+        _need(e, torch.float32, "e")
+        H = e.numel() // max(e.size(0), 1)
+        de = torch.empty_like(e)
+        check(_L.tango_edge_softmax_bwd(_ptr(de), _ptr(a), _ptr(da), _ptr(e), indptr.data_ptr(),
+                                        _ptr(edge_ids), indptr.numel() - 1, H, float(slope), _stream()),
+              "edge_softmax_backward")
+        return de
+
+
+# ------------------------------------------------------------------ wrappers
+def quantize(t, scale=None, round_mode=ROUND_RNE, noise=None, seed=0, offset=0):
+    """Quantize to int8; returns (int8 tensor, scale).  cuda/kernels.py:19-30."""
+    assert t.is_cuda, "tensor must be on GPU"
+    if scale is None:
+        scale = cuda_kernels.get_scale(t)
+    out = torch.empty(t.shape, dtype=torch.int8, device=t.device)
+    cuda_kernels.quantize(out, t, scale, round_mode=round_mode, noise=noise, seed=seed, offset=offset)
+    return out, scale
+
+
+def mySDDMM_int8(g, op, U, V, scaleU, scaleV, isReduce, reverse=False):
+    """cuda/kernels.py:33-59."""
+    if reverse:
+        dst, src = g.coo
+    else:
+        src, dst = g.coo
+    assert src.is_cuda, "src must be on GPU"
+    assert dst.is_cuda, "dst must be on GPU"
+    assert U.is_cuda, "U must be on GPU"
+    assert V.is_cuda, "V must be on GPU"
+    assert scaleU.is_cuda, "scaleU must be on GPU"
+    assert scaleV.is_cuda, "scaleV must be on GPU"
+    UV_unsqueezed = False
+    if len(U.shape) == 2 and len(V.shape) == 2:
+        U = U.unsqueeze(1)
+        V = V.unsqueeze(1)
+        UV_unsqueezed = True
+    out_shape = (src.size(0),) + infer_broadcast_shape(op, U.shape[1:], V.shape[1:])
+    out = torch.empty(out_shape, dtype=torch.float32, device=src.device)
+    if isReduce:
+        scale = torch.zeros((1,), dtype=torch.float32, device=src.device)
+    else:
+        scale = torch.Tensor()
+    cuda_kernels.mySDDMM_int8(op, out, scale, src, dst, U, V, scaleU, scaleV)
+    if UV_unsqueezed:
+        out = out.squeeze(1)
+    return out, scale
+
+
+def QGEMM_forward(x, x_, scaleX, w, w_, scaleW, bias=None, isReduce=False, round_mode=None):
+    """cuda/kernels.py:79-95."""
+    assert x.is_cuda, "x must be on GPU"
+    assert w.is_cuda, "w must be on GPU"
+    assert bias is None or bias.is_cuda, "bias must be on GPU"
+    assert x.size(1) == w.size(1), "x and w must have the same number of columns"
+    out_fp = torch.empty((x.size(0), w.size(0)), dtype=torch.float32, device=x.device)
+    scale_out = torch.empty_like(scaleX) if isReduce else torch.Tensor()
+    bias = torch.Tensor() if bias is None else bias
+    cuda_kernels.QGEMM_forward(out_fp, x, x_, w, w_, bias, scale_out, scaleX, scaleW,
+                               round_mode=round_mode)
+    if isReduce:
+        return out_fp, scale_out
+    return out_fp
+
+
+def QGEMM_backward(dY, X, W, scaledY, scaleX, scaleW, X_need=True, W_need=True):
+    """cuda/kernels.py:97-111."""
+    assert scaledY.is_cuda, "scaledY must be on GPU"
+    assert dY.is_cuda, "dY must be on GPU"
+    dX, dW = None, None
+    if X_need:
+        assert W.is_cuda, "W must be on GPU"
+        assert scaleW.is_cuda, "scaleW must be on GPU"
+        dX = torch.empty(X.shape, dtype=torch.float32, device=X.device)
+        cuda_kernels.QGEMM_backward_gradX(dX, dY, W, scaledY, scaleW)
+    if W_need:
+        assert X.is_cuda, "X must be on GPU"
+        assert scaleX.is_cuda, "scaleX must be on GPU"
+        dW = torch.empty(W.shape, dtype=torch.float32, device=X.device)
+        cuda_kernels.QGEMM_backward_gradW(dW, dY, X, scaledY, scaleX)
+    return dX, dW
+
+
+def transpose_quant(data, scale):
+    """[nnz, H, D] fp32 -> int8 [H, D, nnz].  cuda/kernels.py:114-119."""
+    assert data.ndim == 3
+    nrow = data.size(0)
+    ncol = data.numel() // max(nrow, 1)
+    data_ = cuda_kernels.transpose_quant(data, scale, nrow, ncol)
+    return data_.reshape((data.size(1), data.size(2), nrow))
+
+
+def multi_cusparse_SPMM(g, N, E_T, scale, reverse=False):
+    """E_T is [H, D, nnz] in edge-id order.  cuda/kernels.py:122-136; the
+    index_select by edge_ids of the reference happens inside the kernel."""
+    assert E_T.ndim == 3 and N.ndim == 3, "E and N must be 3D tensors"
+    assert E_T.size(1) == 1, "Cannot broadcast E"
+    if reverse:
+        indptr, indices, edge_ids = g.adj_csr
+    else:
+        indptr, indices, edge_ids = g.adj_csc
+    if edge_ids is not None and edge_ids.numel() == 0:
+        edge_ids = None
+    return cuda_kernels.multi_cusparse_SPMM(indptr, indices, N, E_T, scale, edge_ids=edge_ids)
+
+
+def incidence_SPMM(g, E, scaleE, reverse=False):
+    """cuda/kernels.py:139-152."""
+    assert E.is_cuda and scaleE.is_cuda
+    coo = g.inc_out if reverse else g.inc_in
+    src = coo[0]
+    dst = coo[1]
+    out_shape = (g.num_nodes(),) + E.shape[1:]
+    dim = E.numel() // max(E.size(0), 1)
+    out = torch.empty((g.num_nodes(), dim), dtype=torch.float32, device=E.device)
+    cuda_kernels.incidence_SPMM(out, src, dst, E, scaleE)
+    return out.view(out_shape)
+
+
+def csr_SPMM(g, N, scaleN, reverse=False):
+    """cuda/kernels.py:154-165."""
+    if reverse:
+        indptr, indices, _ = g.adj_csr
+    else:
+        indptr, indices, _ = g.adj_csc
+    feat_shape = N.shape[1:]
+    out_shape = (g.num_nodes(),) + feat_shape
+    dim = N.numel() // max(N.size(0), 1)
+    out = torch.empty((g.num_nodes(), dim), dtype=torch.float32, device=N.device)
+    cuda_kernels.csr_SPMM(out, indptr, indices, N, scaleN)
+    return out.view(out_shape)
+
+
+def multi_cusparse_SPMV(g, N_T, E_T, scale, reverse=False):
+    """cuda/kernels.py:168-178 (which itself calls the SpMM binding)."""
+    assert E_T.ndim == 3 and N_T.ndim == 3, "E and N must be 3D tensors"
+    if reverse:
+        indptr, indices, edge_ids = g.adj_csr
+    else:
+        indptr, indices, edge_ids = g.adj_csc
+    return cuda_kernels.multi_cusparse_SPMM(indptr, indices, N_T, E_T, scale, edge_ids=edge_ids)

@@ -1,0 +1,56 @@
+"""CPU-side checks of the drop-in boundary: the library loads without a GPU
+and exports every symbol that include/tango_hip.h declares."""
+import ctypes
+import os
+import re
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def declared_symbols():
+    text = open(os.path.join(ROOT, "include", "tango_hip.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(tango_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_header_symbols_are_exported_and_bound():
+    from tango_amd import _lib
+    handle = ctypes.CDLL(_lib.LIB_PATH)
+    names = declared_symbols()
+    assert len(names) >= 20
+    for n in names:
+        assert hasattr(handle, n), "library lacks %s" % n
+        assert n in _lib.SIGNATURES, "ctypes binding lacks %s" % n
+    assert set(_lib.SIGNATURES) == set(names)
+
+
+def test_status_strings_and_version():
+    from tango_amd import _lib
+    L = _lib.lib()
+    assert L.tango_abi_version() >= 1
+    assert L.tango_status_string(0) == b"ok"
+    for code in (-1, -2, -3, -4):
+        assert L.tango_status_string(code) not in (b"ok", b"unknown status")
+    assert L.tango_status_string(-99) == b"unknown status"
+
+
+def test_argument_validation_needs_no_gpu():
+    # every entry point validates on the host before touching the device
+    from tango_amd import _lib
+    L = _lib.lib()
+    assert L.tango_absmax_f32(None, 10, None, None) == -1
+    assert L.tango_quantize_f32_i8(None, -1, None, None, 0, None, 0, 0, None) == -1
+    assert L.tango_spmm_csr_u_mul_e(1, 1, 1, None, 1, 1, 1, 4, 4, 2, 8, 3, 10, None) == -2  # D not in {1, F}
+    assert L.tango_sddmm_ewise_i8(7, 1, None, 1, 1, 1, 1, 1, 1, 4, 4, None) == -2  # unknown op
+    assert L.tango_spmm_csr_copy_u(1, 1, 1, 1, 8, 1, 4, 1 << 31, 10, 8, None) == -2  # node ids must fit 31 bits
+
+
+def test_infer_broadcast_shape():
+    from tango_amd.kernels import infer_broadcast_shape as ibs
+    assert ibs("add", (8, 1), (8, 1)) == (8, 1)
+    assert ibs("mul", (4, 16), (4, 1)) == (4, 16)
+    assert ibs("dot", (8, 16), (8, 16)) == (8, 1)
+    assert ibs("add", (3,), (2, 3)) == (2, 3)
+    import pytest
+    with pytest.raises(ValueError):
+        ibs("add", (3,), (4,))

@@ -1,0 +1,115 @@
+"""GPU parity: absmax / quantize / transpose_quant kernels vs the CPU oracle (bit-exact)."""
+import numpy as np
+import pytest
+import torch
+
+from gpu_util import dev, host, sc
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def K():
+    from tango_amd import kernels
+    return kernels
+
+
+@pytest.mark.parametrize("n", [1, 3, 4, 5, 1023, 65536, 65537, 1000003, 4 * 1048576 + 2])
+def test_get_scale(K, orc, n):
+    rng = np.random.default_rng(n)
+    x = rng.standard_normal(n).astype(np.float32)
+    x[-1] = 9.5 if n % 2 else -9.5  # maximum in the tail element
+    assert host(K.cuda_kernels.get_scale(dev(x)))[0] == orc.absmax_scale(x)
+
+
+def test_get_scale_misaligned_view_and_zero(K, orc):
+    rng = np.random.default_rng(0)
+    x = rng.standard_normal(300001).astype(np.float32)
+    t = dev(x)
+    for off in (1, 2, 3):
+        assert host(K.cuda_kernels.get_scale(t[off:]))[0] == orc.absmax_scale(x[off:])
+    assert host(K.cuda_kernels.get_scale(torch.zeros(100000, device="cuda")))[0] == 0.0
+    # stale contents of the output slot must not leak: call twice on shrinking data
+    big = K.cuda_kernels.get_scale(dev(x * 100))
+    small = K.cuda_kernels.get_scale(dev(x))
+    assert host(small)[0] == orc.absmax_scale(x) and host(big)[0] > host(small)[0]
+
+
+def test_get_scale_rows(K, orc):
+    rng = np.random.default_rng(1)
+    x = rng.standard_normal((1000, 41)).astype(np.float32)
+    assert np.array_equal(host(K.cuda_kernels.get_scale_rows(dev(x))), orc.absmax_rows(x))
+    wide = rng.standard_normal((50, 700)).astype(np.float32)
+    view = dev(wide)[:, :602]
+    assert np.array_equal(host(K.cuda_kernels.get_scale_rows(view)), orc.absmax_rows(wide[:, :602]))
+
+
+@pytest.mark.parametrize("mode", ["rne", "trunc"])
+@pytest.mark.parametrize("n", [1, 2, 3, 7, 4096, 100003, 232965 * 41])
+def test_quantize_deterministic(K, orc, mode, n):
+    rng = np.random.default_rng(n + 5)
+    x = rng.standard_normal(n).astype(np.float32)
+    s = orc.absmax_scale(x)
+    q, s_dev = K.quantize(dev(x), round_mode=mode)
+    assert host(s_dev)[0] == s
+    assert np.array_equal(host(q), orc.quantize(x, s, orc.RNE if mode == "rne" else orc.TRUNC))
+
+
+def test_quantize_ties_clamp_and_zero_scale(K, orc):
+    x = np.array([0.5, 1.5, 2.5, -0.5, -1.5, -2.5, 126.5, 127.5, 300.0, -300.0, 0.0, 0.49999997,
+                  np.inf, -np.inf, np.nan, 1e-30], np.float32)
+    for mode, om in (("rne", orc.RNE), ("trunc", orc.TRUNC)):
+        q, _ = K.quantize(dev(x), sc(1.0), round_mode=mode)
+        assert np.array_equal(host(q), orc.quantize(x, 1.0, om))
+    q, _ = K.quantize(torch.zeros(37, device="cuda"))
+    assert not host(q).any()
+    # misaligned views take the scalar kernel
+    y = np.random.default_rng(3).standard_normal(5003).astype(np.float32)
+    q, s = K.quantize(dev(y)[1:])
+    assert np.array_equal(host(q), orc.quantize(y[1:], host(s)[0]))
+
+
+@pytest.mark.parametrize("n,offset", [(5, 0), (100003, 0), (100003, 4096), (100003, 3), (1 << 20, (1 << 34) + 1)])
+def test_quantize_stochastic(K, orc, n, offset):
+    rng = np.random.default_rng(n)
+    x = rng.standard_normal(n).astype(np.float32)
+    s = orc.absmax_scale(x)
+    u = rng.random(n, dtype=np.float32)
+    q, _ = K.quantize(dev(x), sc(s), round_mode="stochastic", noise=dev(u))
+    assert np.array_equal(host(q), orc.quantize(x, s, orc.STOCHASTIC, noise=u))
+    q, _ = K.quantize(dev(x), sc(s), round_mode="stochastic", seed=0xDEADBEEFCAFE, offset=offset)
+    assert np.array_equal(host(q), orc.quantize(x, s, orc.STOCHASTIC, seed=0xDEADBEEFCAFE, offset=offset))
+
+
+def test_stochastic_unbiased_native_rng(K):
+    x = torch.randn(1 << 22, device="cuda", generator=torch.Generator("cuda").manual_seed(1))
+    q, s = K.quantize(x, round_mode="stochastic", seed=99)
+    err = (q.double() * s.double() - x.double()).mean().item()
+    assert abs(err) < 1e-3
+    q2, _ = K.quantize(x, round_mode="stochastic", seed=100)
+    assert not torch.equal(q, q2)
+
+
+def test_quantize_rows_padded(K, orc):
+    rng = np.random.default_rng(4)
+    for rows, cols, ld in ((1000, 41, 48), (333, 41, 41), (64, 602, 608), (17, 3, 16)):
+        x = rng.standard_normal((rows, cols)).astype(np.float32)
+        s = orc.absmax_scale(x)
+        out = torch.full((rows, ld), 77, dtype=torch.int8, device="cuda")
+        K.cuda_kernels.quantize_rows(out, dev(x), sc(s))
+        assert np.array_equal(host(out), orc.quantize_rows(x, s, False, ldq=ld))
+        sr = orc.absmax_rows(x)
+        K.cuda_kernels.quantize_rows(out, dev(x), dev(sr), per_row=True, round_mode="trunc")
+        assert np.array_equal(host(out), orc.quantize_rows(x, sr, True, ldq=ld, mode=orc.TRUNC))
+        K.cuda_kernels.quantize_rows(out, dev(x), sc(s), round_mode="stochastic", seed=5, offset=8)
+        assert np.array_equal(host(out), orc.quantize_rows(x, s, False, ldq=ld, mode=orc.STOCHASTIC, seed=5, offset=8))
+
+
+@pytest.mark.parametrize("shape", [(1335586, 8, 1), (1001, 4, 1), (77, 2, 3), (4096, 1, 1), (5, 64, 4)])
+def test_transpose_quant(K, orc, shape):
+    rng = np.random.default_rng(6)
+    e = rng.random(shape, dtype=np.float32)
+    s = orc.absmax_scale(e)
+    got = K.transpose_quant(dev(e), sc(s))
+    assert tuple(got.shape) == (shape[1], shape[2], shape[0])
+    assert np.array_equal(host(got).reshape(shape[1] * shape[2], shape[0]), orc.transpose_quant(e, s))
