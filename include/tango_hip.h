@@ -83,34 +83,43 @@ int tango_transpose_quant_f32_i8(const float* x, int64_t nrow, int64_t ncol, con
 
 /* -------------------------------------------------------------------- GEMM */
 
+/* All GEMM entry points take a caller-provided workspace (device memory,
+   16-byte aligned) whose size the matching *_workspace() query returns; the
+   library uses it to re-pack the small operand into aligned, zero-padded rows. */
+
 /* QGEMM_forward (cuda/src/cuda.cpp:11-17 -> QGEMM_forward_impl,
    QGEMM_forward.cu:125-157): quantizes X[M,K] and W[N,K] with scaleX / scaleW
-   (round_mode; the reference truncates), stores the int8 copies to Xq[M,K] and
-   Wq[N,K] (dense, row stride K), and writes
+   (round_mode; the reference truncates, cuda/src/iterator.h:161), stores the
+   int8 copies to Xq[M,K] (row stride ldxq >= K; bytes K..ldxq of each row are
+   zeroed) and Wq[N,K] (dense), and writes
    Y[m,n] = (scaleX*scaleW) * float(sum_k Xq[m,k]*Wq[n,k]) (+ bias[n]).
    bias may be NULL.  scaleY may be NULL; otherwise scaleY[0] = max|Y| / 127
    (the fused reduction of cuda/src/epilogue.h:105-626); it need not be
-   initialised.  K is arbitrary (the reference requires K % 4 == 0).
-   workspace: tango_qgemm_fwd_workspace(M,N,K) bytes, may be NULL when that is 0. */
+   initialised.  K is arbitrary (the reference requires K % 4 == 0); rows of Xq
+   padded to a multiple of 16 bytes take the fast path. */
 size_t tango_qgemm_fwd_workspace(int64_t M, int64_t N, int64_t K);
-int tango_qgemm_fwd(float* Y, int64_t ldy, const float* X, int64_t ldx, int8_t* Xq,
+int tango_qgemm_fwd(float* Y, int64_t ldy, const float* X, int64_t ldx, int8_t* Xq, int64_t ldxq,
                     const float* W, int64_t ldw, int8_t* Wq, const float* bias, float* scaleY,
                     const float* scaleX, const float* scaleW, int64_t M, int64_t N, int64_t K,
                     int round_mode, void* workspace, size_t workspace_bytes,
                     tango_stream_t stream);
 
-/* Integer GEMM on operands that are already int8 (the cached-operand forward
-   used when quantization was done by tango_quantize_*; same epilogue as above):
+/* Integer GEMM on operands that are already int8 (no counterpart in the
+   reference, whose forward always re-quantizes; same epilogue as above):
    Y[m,n] = (sA*sB) * float(sum_k A[m,k]*B[n,k]) (+ bias[n]), optional scaleY. */
+size_t tango_qgemm_i8_nt_workspace(int64_t M, int64_t N, int64_t K);
 int tango_qgemm_i8_nt(float* Y, int64_t ldy, const int8_t* A, int64_t lda, const int8_t* B,
                       int64_t ldb, const float* bias, float* scaleY, const float* sA,
-                      const float* sB, int64_t M, int64_t N, int64_t K, tango_stream_t stream);
+                      const float* sB, int64_t M, int64_t N, int64_t K, void* workspace,
+                      size_t workspace_bytes, tango_stream_t stream);
 
 /* QGEMM_backward_gradX (cuda/src/cuda.cpp:90-98 -> QGEMM_backward.cu:21-48):
    dX[M,K] = (s_dY*s_W) * float(sum_n dYq[m,n] * Wq[n,k]). */
+size_t tango_qgemm_bwd_dx_workspace(int64_t M, int64_t N, int64_t K);
 int tango_qgemm_bwd_dx(float* dX, int64_t lddx, const int8_t* dYq, int64_t lddy,
                        const int8_t* Wq, int64_t ldw, const float* s_dY, const float* s_W,
-                       int64_t M, int64_t N, int64_t K, tango_stream_t stream);
+                       int64_t M, int64_t N, int64_t K, void* workspace, size_t workspace_bytes,
+                       tango_stream_t stream);
 
 /* QGEMM_backward_gradW (cuda/src/cuda.cpp:100-108 -> QGEMM_backward.cu:50-113):
    dW[N,K] = (s_dY*s_X) * float(sum_m dYq[m,n] * Xq[m,k]), int32 accumulation.

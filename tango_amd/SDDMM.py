@@ -1,0 +1,74 @@
+"""Quantized per-edge ops: mirrors cuda/SDDMM.py of the reference, plus the
+``sddmm_u_dot_v`` op that the reference's drivers call but its tree does not
+define (evaluation/test_HGT.py:58, evaluation/link_pred_gcn.py:145)."""
+import torch
+from torch.autograd.function import Function, once_differentiable
+
+from . import config
+from .kernels import incidence_SPMM, multi_cusparse_SPMM, mySDDMM_int8, quantize, transpose_quant
+
+
+def _quantize_grad(t):
+    t = t if t.is_contiguous() else t.contiguous()
+    if config.grad_round_mode == "stochastic":
+        return quantize(t, round_mode="stochastic", seed=config.seed, offset=config.next_offset())
+    return quantize(t, round_mode=config.grad_round_mode)
+
+
+class sddmm_u_add_v(Function):
+    """out[e] = U[src[e]] + V[dst[e]] on int8-quantized U, V (cuda/SDDMM.py:10-32)."""
+
+    @staticmethod
+    def forward(ctx, g, U, V, scaleU_=None, scaleV_=None):
+        U_, scaleU = quantize(U if U.is_contiguous() else U.contiguous(), scaleU_)
+        if id(U) == id(V):
+            V_, scaleV = U_, scaleU
+        else:
+            V_, scaleV = quantize(V if V.is_contiguous() else V.contiguous(), scaleV_)
+        out, _ = mySDDMM_int8(g, "add", U_, V_, scaleU, scaleV, False)
+        ctx.backward_cache = g
+        return out
+
+    @staticmethod
+    @once_differentiable
+    def backward(ctx, dZ):
+        g = ctx.backward_cache
+        dZ_, scaledZ = _quantize_grad(dZ)
+        dU = dV = None
+        if ctx.needs_input_grad[2]:
+            dV = incidence_SPMM(g, dZ_, scaledZ)
+        if ctx.needs_input_grad[1]:
+            dU = incidence_SPMM(g, dZ_, scaledZ, True)
+        return None, dU, dV, None, None
+
+
+class sddmm_u_dot_v(Function):
+    """out[e, h, 0] = <U[src[e], h, :], V[dst[e], h, :]>.  Built by symmetry with
+    spmm_u_mul_e: the backward is two u_mul_e aggregations with dZ as the edge value."""
+
+    @staticmethod
+    def forward(ctx, g, U, V):
+        U_, scaleU = quantize(U if U.is_contiguous() else U.contiguous())
+        V_, scaleV = quantize(V if V.is_contiguous() else V.contiguous())
+        out, _ = mySDDMM_int8(g, "dot", U_, V_, scaleU, scaleV, False)
+        ctx.backward_cache = g, U_, scaleU, V_, scaleV
+        return out
+
+    @staticmethod
+    @once_differentiable
+    def backward(ctx, dZ):
+        g, U_, scaleU, V_, scaleV = ctx.backward_cache
+        dZ = dZ if dZ.is_contiguous() else dZ.contiguous()
+        squeeze = dZ.dim() == 2
+        dZ3 = dZ.unsqueeze(1) if squeeze else dZ  # [E, H, 1]
+        U3 = U_.unsqueeze(1) if U_.dim() == 2 else U_
+        V3 = V_.unsqueeze(1) if V_.dim() == 2 else V_
+        from .kernels import cuda_kernels
+        scaledZ = cuda_kernels.get_scale(dZ3)
+        dZ_T = transpose_quant(dZ3, scaledZ)  # [H, 1, E], half-to-even
+        dU = dV = None
+        if ctx.needs_input_grad[1]:
+            dU = multi_cusparse_SPMM(g, V3, dZ_T, scaledZ * scaleV, True).reshape(U_.shape)
+        if ctx.needs_input_grad[2]:
+            dV = multi_cusparse_SPMM(g, U3, dZ_T, scaledZ * scaleU).reshape(V_.shape)
+        return None, dU, dV

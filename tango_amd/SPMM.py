@@ -1,0 +1,87 @@
+"""Quantized aggregation ops: mirrors cuda/SPMM.py of the reference."""
+import torch
+from torch.autograd.function import Function, once_differentiable
+
+from . import config
+from .kernels import (cuda_kernels, csr_SPMM, multi_cusparse_SPMM, mySDDMM_int8, quantize,
+                      quantize_padded, transpose_quant)
+
+
+def _quantize_grad(t, padded):
+    t = t if t.is_contiguous() else t.contiguous()
+    kw = {"round_mode": config.grad_round_mode}
+    if config.grad_round_mode == "stochastic":
+        kw.update(seed=config.seed, offset=config.next_offset())
+    if padded and t.dim() == 2:
+        return quantize_padded(t, **kw)
+    return quantize(t, **kw)
+
+
+class spmm_copy_u(Function):
+    """copy_u-sum aggregation (cuda/SPMM.py:8-24).  ``scaleN`` may come from the
+    preceding GEMM's epilogue, in which case no absmax pass runs here."""
+
+    @staticmethod
+    def forward(ctx, g, N, scaleN=None):
+        N = N if N.is_contiguous() else N.contiguous()
+        if N.dim() == 2:
+            N_, scaleN = quantize_padded(N, scaleN)
+        else:
+            N_, scaleN = quantize(N, scaleN)
+        out = csr_SPMM(g, N_, scaleN)
+        ctx.backward_cache = g
+        return out
+
+    @staticmethod
+    @once_differentiable
+    def backward(ctx, dZ):
+        g = ctx.backward_cache
+        dN = None
+        if ctx.needs_input_grad[1]:
+            dZ_, scaledZ = _quantize_grad(dZ, True)
+            dN = csr_SPMM(g, dZ_, scaledZ, True)
+        return None, dN, None
+
+
+def _need_reduce_last_dim(ufeat, efeat):
+    """cuda/SPMM.py:26-34: whether dE reduces the last dimension (dot instead of mul)."""
+    if ufeat is None or efeat is None:
+        return False
+    ushp = ufeat.shape
+    eshp = efeat.shape
+    return ushp[1:-1] == eshp[1:-1] and eshp[-1] == 1 and ushp[-1] > 1
+
+
+class spmm_u_mul_e(Function):
+    """u_mul_e-sum aggregation with int8 node features and int8 edge values
+    (cuda/SPMM.py:36-62).  N is [n, H, F], E is [nnz, H, 1] in edge-id order."""
+
+    @staticmethod
+    def forward(ctx, g, N, E):
+        N = N if N.is_contiguous() else N.contiguous()
+        E = E if E.is_contiguous() else E.contiguous()
+        scaleE = cuda_kernels.get_scale(E)
+        E_T_ = transpose_quant(E, scaleE)
+        N_, scaleN = quantize(N)  # one absmax pass (the reference runs two, cuda/SPMM.py:39,43)
+        scale = scaleN * scaleE
+        out = multi_cusparse_SPMM(g, N_, E_T_, scale)
+        reduce_last = _need_reduce_last_dim(N, E)
+        ctx.backward_cache = g, N_, scaleN, E_T_, scaleE, scale, reduce_last, E.shape
+        return out
+
+    @staticmethod
+    @once_differentiable
+    def backward(ctx, dZ):
+        g, N_, scaleN, E_T_, scaleE, scale, reduce_last, eshape = ctx.backward_cache
+        dZ_, scaledZ = _quantize_grad(dZ, False)
+        dN = dE = None
+        if ctx.needs_input_grad[1]:
+            # dN = A^T (E * dZ): the dequantization scale is s_dZ * s_E.  The reference passes
+            # the forward scale s_N * s_E here (cuda/SPMM.py:56); ref_compat reproduces that.
+            bscale = scale if config.ref_compat else scaledZ * scaleE
+            dN = multi_cusparse_SPMM(g, dZ_, E_T_, bscale, True)
+        if ctx.needs_input_grad[2]:
+            op = "dot" if reduce_last else "mul"
+            dE, _ = mySDDMM_int8(g, op, N_, dZ_, scaleN, scaledZ, False)
+            dE = dE.reshape(eshape)
+        return None, dN, dE

@@ -26,9 +26,11 @@ SIGNATURES = {
     "tango_quantize_rows_f32_i8": (I, [P, I64, I64, I64, P, I, P, I64, I, P, U64, U64, P]),
     "tango_transpose_quant_f32_i8": (I, [P, I64, I64, P, P, P]),
     "tango_qgemm_fwd_workspace": (SZ, [I64, I64, I64]),
-    "tango_qgemm_fwd": (I, [P, I64, P, I64, P, P, I64, P, P, P, P, P, I64, I64, I64, I, P, SZ, P]),
-    "tango_qgemm_i8_nt": (I, [P, I64, P, I64, P, I64, P, P, P, P, I64, I64, I64, P]),
-    "tango_qgemm_bwd_dx": (I, [P, I64, P, I64, P, I64, P, P, I64, I64, I64, P]),
+    "tango_qgemm_fwd": (I, [P, I64, P, I64, P, I64, P, I64, P, P, P, P, P, I64, I64, I64, I, P, SZ, P]),
+    "tango_qgemm_i8_nt_workspace": (SZ, [I64, I64, I64]),
+    "tango_qgemm_i8_nt": (I, [P, I64, P, I64, P, I64, P, P, P, P, I64, I64, I64, P, SZ, P]),
+    "tango_qgemm_bwd_dx_workspace": (SZ, [I64, I64, I64]),
+    "tango_qgemm_bwd_dx": (I, [P, I64, P, I64, P, I64, P, P, I64, I64, I64, P, SZ, P]),
     "tango_qgemm_bwd_dw_workspace": (SZ, [I64, I64, I64]),
     "tango_qgemm_bwd_dw": (I, [P, I64, P, I64, P, I64, P, P, I64, I64, I64, P, SZ, P]),
     "tango_qgemm_legacy_workspace": (SZ, [I64, I64, I64]),

@@ -1,11 +1,599 @@
+// int8 x int8 -> int32 GEMMs on the CDNA4 matrix cores (v_mfma_i32_16x16x64_i8)
+// with the dequant (+bias) (+absmax) epilogue fused, for gfx950.
+//
+// Shapes here are tall and skinny (M ~ 2e5 rows, N and K <= a few hundred), so
+// every GEMM streams one big operand from HBM exactly once and keeps the small
+// one on chip:
+//   * NT kernel (forward, gradX): a wavefront owns 32 rows of the tall operand
+//     and loads them from global memory straight into MFMA fragment layout
+//     (16 bytes per lane, a 4-deep register ring keeps several k-steps in
+//     flight); the small operand is staged through LDS, shared by the
+//     workgroup's four wavefronts, double-buffered, bank-swizzled.
+//   * TN kernel (gradW): both operands are tall and reduction-strided.  Tiles
+//     are staged through LDS in their natural layout and transposed in
+//     registers (v_perm 4x4 byte blocks) on the way into the fragments; the
+//     reduction over rows is split across workgroups and combined with int32
+//     atomics, which is exact and order-independent.
 #include "common.hpp"
-extern "C" {
-size_t tango_qgemm_fwd_workspace(int64_t, int64_t, int64_t) { return 0; }
-int tango_qgemm_fwd(float*, int64_t, const float*, int64_t, int8_t*, const float*, int64_t, int8_t*, const float*, float*, const float*, const float*, int64_t, int64_t, int64_t, int, void*, size_t, tango_stream_t) { return TANGO_ERR_UNSUPPORTED; }
-int tango_qgemm_i8_nt(float*, int64_t, const int8_t*, int64_t, const int8_t*, int64_t, const float*, float*, const float*, const float*, int64_t, int64_t, int64_t, tango_stream_t) { return TANGO_ERR_UNSUPPORTED; }
-int tango_qgemm_bwd_dx(float*, int64_t, const int8_t*, int64_t, const int8_t*, int64_t, const float*, const float*, int64_t, int64_t, int64_t, tango_stream_t) { return TANGO_ERR_UNSUPPORTED; }
-size_t tango_qgemm_bwd_dw_workspace(int64_t, int64_t, int64_t) { return 0; }
-int tango_qgemm_bwd_dw(float*, int64_t, const int8_t*, int64_t, const int8_t*, int64_t, const float*, const float*, int64_t, int64_t, int64_t, void*, size_t, tango_stream_t) { return TANGO_ERR_UNSUPPORTED; }
-size_t tango_qgemm_legacy_workspace(int64_t, int64_t, int64_t) { return 0; }
-int tango_qgemm_legacy(float*, const float*, const float*, int64_t, int64_t, int64_t, int, int, void*, size_t, tango_stream_t) { return TANGO_ERR_UNSUPPORTED; }
+
+namespace tango {
+
+// ----------------------------------------------------------------- helpers
+__device__ __forceinline__ i32x4 mfma_16x16x64(i32x4 a, i32x4 b, i32x4 c) {
+    return __builtin_amdgcn_mfma_i32_16x16x64_i8(a, b, c, 0, 0, 0);
 }
+
+// 16 bytes of one int8 row starting at p; `avail` = bytes that may be read
+// (<= 0: none).  VEC is the widest aligned access the row layout allows.
+template <int VEC>
+__device__ __forceinline__ i32x4 load16(const int8_t* p, int64_t avail) {
+    i32x4 v = {0, 0, 0, 0};
+    if (avail <= 0) return v;
+    if (VEC == 16) {
+        v = *reinterpret_cast<const i32x4*>(p);  // caller guarantees 16 readable bytes
+    } else if (VEC == 4) {
+        const int* q = reinterpret_cast<const int*>(p);
+        if (avail > 0) v.x = q[0];
+        if (avail > 4) v.y = q[1];
+        if (avail > 8) v.z = q[2];
+        if (avail > 12) v.w = q[3];
+    } else {
+        uint32_t w[4] = {0u, 0u, 0u, 0u};
+#pragma unroll
+        for (int b = 0; b < 16; ++b)
+            if (b < avail) w[b >> 2] |= static_cast<uint32_t>(static_cast<uint8_t>(p[b])) << (8 * (b & 3));
+        v = i32x4{static_cast<int>(w[0]), static_cast<int>(w[1]), static_cast<int>(w[2]), static_cast<int>(w[3])};
+    }
+    return v;
+}
+
+struct NtParams {
+    float* C;            // [M, N] fp32, row stride ldc
+    const int8_t* A;     // [M, Kr] int8, row stride lda: the tall operand
+    const int8_t* B;     // [N, Kp] int8 packed: 16-byte aligned rows of stride ldb, zero-filled to Kp
+    const float* bias;   // [N] or null
+    float* absmax_out;   // null, or receives max|C| / 127 (pre-zeroed)
+    const float* sA;
+    const float* sB;
+    int64_t M, N, Kr;    // Kr = reduction length
+    int64_t lda, ldb, ldc;
+    int64_t a_row_bytes; // bytes that may be read from each row of A (>= Kr)
+};
+
+// Workgroup = 4 waves = 128 rows x (16 * NT) columns.  gridDim = (ceil(M/128), ceil(N/(16 NT))).
+template <int NT, int VEC>
+__global__ __launch_bounds__(256, 2) void gemm_nt_kernel(const NtParams p) {
+    constexpr int PF = 4;                 // A fragments in flight (k-steps)
+    constexpr int BROWS = NT * 16;        // rows of B per tile
+    __shared__ i32x4 ldsB[2][BROWS * 4];  // [buffer][row][16-byte chunk], chunk index swizzled
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int g = lane >> 4;    // k-chunk of the fragment this lane holds
+    const int r16 = lane & 15;  // row (A) / column (B, C) within a 16x16 tile
+    const int64_t row0 = static_cast<int64_t>(blockIdx.x) * 128 + wave * 32;
+    const int64_t n0 = static_cast<int64_t>(blockIdx.y) * BROWS;
+    const int ksteps = static_cast<int>((p.Kr + 63) >> 6);
+
+    const int64_t ra0 = row0 + r16, ra1 = row0 + 16 + r16;
+    const int8_t* pa0 = p.A + ra0 * p.lda + g * 16;
+    const int8_t* pa1 = p.A + ra1 * p.lda + g * 16;
+    const bool ok0 = ra0 < p.M, ok1 = ra1 < p.M;
+
+    auto load_a = [&](i32x4* dst, int step) {
+        const int64_t kc = static_cast<int64_t>(step) * 64 + g * 16;
+        const int64_t avail = (step < ksteps && kc < p.Kr) ? (p.a_row_bytes - kc) : 0;
+        dst[0] = load16<VEC>(pa0 + static_cast<int64_t>(step) * 64, ok0 ? avail : 0);
+        dst[1] = load16<VEC>(pa1 + static_cast<int64_t>(step) * 64, ok1 ? avail : 0);
+    };
+
+    // B tile: BROWS rows x 4 chunks; thread handles chunks tid, tid + 256, ...
+    constexpr int BCH = (BROWS * 4 + 255) / 256;
+    auto load_b = [&](i32x4* dst, int step) {
+#pragma unroll
+        for (int c = 0; c < BCH; ++c) {
+            const int idx = tid + c * 256;
+            const int n = idx >> 2, kc = idx & 3;
+            dst[c] = i32x4{0, 0, 0, 0};
+            if (idx < BROWS * 4 && n0 + n < p.N && step < ksteps)
+                dst[c] = *reinterpret_cast<const i32x4*>(p.B + (n0 + n) * p.ldb + static_cast<int64_t>(step) * 64 + kc * 16);
+        }
+    };
+    auto store_b = [&](const i32x4* src, int buf) {
+#pragma unroll
+        for (int c = 0; c < BCH; ++c) {
+            const int idx = tid + c * 256;
+            const int n = idx >> 2, kc = idx & 3;
+            if (idx < BROWS * 4) ldsB[buf][n * 4 + (kc ^ ((n >> 1) & 3))] = src[c];
+        }
+    };
+
+    i32x4 acc[2][NT];
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < NT; ++j) acc[i][j] = i32x4{0, 0, 0, 0};
+
+    i32x4 a[PF][2];
+#pragma unroll
+    for (int s = 0; s < PF; ++s) load_a(a[s], s);
+    i32x4 breg[BCH];
+    load_b(breg, 0);
+    store_b(breg, 0);
+    __syncthreads();
+
+    for (int t = 0; t < ksteps; t += PF) {
+#pragma unroll
+        for (int s = 0; s < PF; ++s) {
+            const int step = t + s;
+            if (step < ksteps) {  // uniform across the workgroup
+                const int buf = step & 1;
+                load_b(breg, step + 1);
+#pragma unroll
+                for (int j = 0; j < NT; ++j) {
+                    const int n = j * 16 + r16;
+                    const i32x4 b = ldsB[buf][n * 4 + (g ^ ((n >> 1) & 3))];
+                    acc[0][j] = mfma_16x16x64(a[s][0], b, acc[0][j]);
+                    acc[1][j] = mfma_16x16x64(a[s][1], b, acc[1][j]);
+                }
+                load_a(a[s], step + PF);
+                store_b(breg, buf ^ 1);
+                __syncthreads();
+            }
+        }
+    }
+
+    // epilogue: lane holds C[row0 + 16 i + 4 g + v][n0 + 16 j + r16]
+    const float s = p.sA[0] * p.sB[0];
+    float m = 0.0f;
+#pragma unroll
+    for (int j = 0; j < NT; ++j) {
+        const int64_t col = n0 + j * 16 + r16;
+        if (col < p.N) {
+            const float bv = p.bias ? p.bias[col] : 0.0f;
+#pragma unroll
+            for (int i = 0; i < 2; ++i) {
+#pragma unroll
+                for (int v = 0; v < 4; ++v) {
+                    const int64_t row = row0 + i * 16 + g * 4 + v;
+                    if (row < p.M) {
+                        float y = s * static_cast<float>(acc[i][j][v]);
+                        if (p.bias) y = bv + y;
+                        p.C[row * p.ldc + col] = y;
+                        m = fmaxf(m, fabsf(y));
+                    }
+                }
+            }
+        }
+    }
+    if (p.absmax_out) block_absmax_to_global(m / 127.0f, p.absmax_out);
+}
+
+// ------------------------------------------------------- operand packing
+// dst[r, 0..ldd) = src[r, 0..cols) zero-filled, for r < rows (src row stride lds).
+__global__ __launch_bounds__(256) void pack_rows_i8_kernel(int8_t* __restrict__ dst, int64_t ldd,
+                                                           const int8_t* __restrict__ src, int64_t lds,
+                                                           int64_t rows, int64_t cols) {
+    const int64_t total = rows * ldd;
+    const int64_t nthr = static_cast<int64_t>(gridDim.x) * blockDim.x;
+    for (int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < total; i += nthr) {
+        const int64_t r = i / ldd, c = i - r * ldd;
+        dst[i] = c < cols ? src[r * lds + c] : static_cast<int8_t>(0);
+    }
+}
+
+// dst[c, 0..ldd) = src[0..rows, c] zero-filled, for c < cols: dst is [cols, ldd].
+__global__ __launch_bounds__(256) void transpose_pack_i8_kernel(int8_t* __restrict__ dst, int64_t ldd,
+                                                                const int8_t* __restrict__ src,
+                                                                int64_t lds, int64_t rows, int64_t cols) {
+    const int64_t total = cols * ldd;
+    const int64_t nthr = static_cast<int64_t>(gridDim.x) * blockDim.x;
+    for (int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < total; i += nthr) {
+        const int64_t c = i / ldd, r = i - c * ldd;
+        dst[i] = r < rows ? src[r * lds + c] : static_cast<int8_t>(0);
+    }
+}
+
+// ------------------------------------------------------------- TN kernel
+struct TnParams {
+    int* acc;          // [N, K] int32 partial sums, pre-zeroed
+    const int8_t* A;   // dY [M, N] int8, row stride lda
+    const int8_t* B;   // X  [M, K] int8, row stride ldb
+    int64_t M, N, K;
+    int64_t lda, ldb;
+    int64_t a_row_bytes, b_row_bytes;  // readable bytes per row
+    int64_t chunk;     // rows of M per split (multiple of 64)
+    int tiles_n, tiles_k, splits;
+};
+
+__device__ __forceinline__ void transpose4x4(uint32_t r0, uint32_t r1, uint32_t r2, uint32_t r3,
+                                             uint32_t* c) {
+    const uint32_t t0 = __builtin_amdgcn_perm(r1, r0, 0x05010400u);
+    const uint32_t t1 = __builtin_amdgcn_perm(r1, r0, 0x07030602u);
+    const uint32_t t2 = __builtin_amdgcn_perm(r3, r2, 0x05010400u);
+    const uint32_t t3 = __builtin_amdgcn_perm(r3, r2, 0x07030602u);
+    c[0] = __builtin_amdgcn_perm(t2, t0, 0x05040100u);
+    c[1] = __builtin_amdgcn_perm(t2, t0, 0x07060302u);
+    c[2] = __builtin_amdgcn_perm(t3, t1, 0x05040100u);
+    c[3] = __builtin_amdgcn_perm(t3, t1, 0x07060302u);
+}
+
+// Workgroup tile: 128 (n) x 128 (k), reduction in steps of 64 rows of M.
+// Waves 2 x 2, each 64 x 64.  Fragment row r16 of sub-tile j maps to column
+// 4 * r16 + j of the wave's 64-wide range (the order the register transpose
+// produces); the output indexing below undoes it.
+template <int VEC>
+__global__ __launch_bounds__(256, 2) void gemm_tn_kernel(const TnParams p) {
+    constexpr int PITCH = 33;  // dwords per LDS row: 128 bytes + 4, odd so that row groups spread over banks
+    __shared__ uint32_t ldsA[64 * PITCH];
+    __shared__ uint32_t ldsB[64 * PITCH];
+
+    // consecutive launch ids land on different XCDs; give each XCD a contiguous range of tiles
+    // so that the tiles sharing one M-chunk run on the same L2
+    const int nblk = gridDim.x;
+    int bid = blockIdx.x;
+    if ((nblk & 7) == 0) bid = (bid & 7) * (nblk >> 3) + (bid >> 3);
+    const int tiles = p.tiles_n * p.tiles_k;
+    const int split = bid / tiles;
+    const int tile = bid - split * tiles;
+    const int tn = tile / p.tiles_k, tk = tile - tn * p.tiles_k;
+    const int64_t n0 = static_cast<int64_t>(tn) * 128, k0 = static_cast<int64_t>(tk) * 128;
+    const int64_t m_begin = static_cast<int64_t>(split) * p.chunk;
+    const int64_t m_end = (m_begin + p.chunk < p.M) ? m_begin + p.chunk : p.M;
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wn = wave >> 1, wk = wave & 1;
+    const int g = lane >> 4, r16 = lane & 15;
+
+    // staging: a tile is 64 rows x 8 chunks of 16 bytes = 512 chunks, 2 per thread per operand
+    const int srow = tid >> 3, scol = tid & 7;  // rows srow and srow + 32, chunk scol
+
+    i32x4 acc[4][4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[i][j] = i32x4{0, 0, 0, 0};
+
+    auto fetch = [&](i32x4* ra, i32x4* rb, int64_t m0) {
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            const int64_t m = m0 + srow + 32 * h;
+            const bool mok = m < m_end;
+            const int64_t ca = n0 + scol * 16, cb = k0 + scol * 16;
+            ra[h] = load16<VEC>(p.A + m * p.lda + ca, (mok && ca < p.N) ? p.a_row_bytes - ca : 0);
+            rb[h] = load16<VEC>(p.B + m * p.ldb + cb, (mok && cb < p.K) ? p.b_row_bytes - cb : 0);
+        }
+    };
+    auto stage = [&](const i32x4* ra, const i32x4* rb) {
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            uint32_t* da = ldsA + (srow + 32 * h) * PITCH + scol * 4;
+            uint32_t* db = ldsB + (srow + 32 * h) * PITCH + scol * 4;
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                da[q] = static_cast<uint32_t>(ra[h][q]);
+                db[q] = static_cast<uint32_t>(rb[h][q]);
+            }
+        }
+    };
+    // four fragments (sub-tiles j = 0..3) of the wave's 64 columns starting at dword column c0
+    auto frags = [&](const uint32_t* lds, int c0, i32x4* out) {
+        uint32_t col[4][4];  // [m-block][j]
+#pragma unroll
+        for (int mb = 0; mb < 4; ++mb) {
+            const uint32_t* base = lds + (g * 16 + mb * 4) * PITCH + c0 + r16;
+            transpose4x4(base[0], base[PITCH], base[2 * PITCH], base[3 * PITCH], col[mb]);
+        }
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+            out[j] = i32x4{static_cast<int>(col[0][j]), static_cast<int>(col[1][j]),
+                           static_cast<int>(col[2][j]), static_cast<int>(col[3][j])};
+    };
+
+    i32x4 ra[2], rb[2];
+    fetch(ra, rb, m_begin);
+    for (int64_t m0 = m_begin; m0 < m_end; m0 += 64) {
+        __syncthreads();  // previous step's fragments are consumed
+        stage(ra, rb);
+        __syncthreads();
+        fetch(ra, rb, m0 + 64);  // rows beyond m_end come back as zeros
+        i32x4 fa[4], fb[4];
+        frags(ldsA, wn * 16, fa);
+        frags(ldsB, wk * 16, fb);
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+#pragma unroll
+            for (int j = 0; j < 4; ++j) acc[i][j] = mfma_16x16x64(fa[i], fb[j], acc[i][j]);
+    }
+
+    // acc[i][j][v] at lane (g, r16): n = n0 + 64 wn + 4 (4 g + v) + i, k = k0 + 64 wk + 4 r16 + j
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int v = 0; v < 4; ++v) {
+            const int64_t n = n0 + wn * 64 + 4 * (4 * g + v) + i;
+            if (n < p.N) {
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const int64_t k = k0 + wk * 64 + 4 * r16 + j;
+                    if (k < p.K) atomicAdd(p.acc + n * p.K + k, acc[i][j][v]);
+                }
+            }
+        }
+}
+
+__global__ __launch_bounds__(256) void zero_i32_kernel(int* __restrict__ p, int64_t n) {
+    const int64_t nthr = static_cast<int64_t>(gridDim.x) * blockDim.x;
+    for (int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < n; i += nthr) p[i] = 0;
+}
+
+// out[r, c] = (sA * sB) * float(acc[r, c])
+__global__ __launch_bounds__(256) void dequant_i32_kernel(float* __restrict__ out, int64_t ldo,
+                                                          const int* __restrict__ acc, int64_t rows,
+                                                          int64_t cols, const float* __restrict__ sA,
+                                                          const float* __restrict__ sB) {
+    const float s = sA[0] * sB[0];
+    const int64_t total = rows * cols;
+    const int64_t nthr = static_cast<int64_t>(gridDim.x) * blockDim.x;
+    for (int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < total; i += nthr) {
+        const int64_t r = i / cols, c = i - r * cols;
+        out[r * ldo + c] = s * static_cast<float>(acc[i]);
+    }
+}
+
+// ------------------------------------------------------------- host side
+static int64_t round_up(int64_t v, int64_t m) { return (v + m - 1) / m * m; }
+
+// widest aligned access for 16-byte row pieces of an int8 matrix; `cols` bytes are meaningful
+static int row_vec(const int8_t* p, int64_t ld, int64_t cols, int64_t* readable) {
+    const uintptr_t a = reinterpret_cast<uintptr_t>(p);
+    if ((a & 15) == 0 && (ld & 15) == 0 && round_up(cols, 16) <= ld) {
+        *readable = round_up(cols, 16);
+        return 16;
+    }
+    if ((a & 3) == 0 && (ld & 3) == 0 && round_up(cols, 4) <= ld) {
+        *readable = round_up(cols, 4);
+        return 4;
+    }
+    *readable = cols;
+    return 1;
+}
+
+template <int VEC>
+static void launch_nt_vec(const NtParams& p, hipStream_t s) {
+    const int64_t n16 = ceil_div(p.N, 16);
+    const unsigned gx = static_cast<unsigned>(ceil_div(p.M, 128));
+#define TANGO_NT(NT_)                                                                             \
+    hipLaunchKernelGGL((gemm_nt_kernel<NT_, VEC>), dim3(gx, static_cast<unsigned>(ceil_div(n16, NT_))), \
+                       dim3(256), 0, s, p)
+    if (n16 <= 1) TANGO_NT(1);
+    else if (n16 <= 2) TANGO_NT(2);
+    else if (n16 <= 3) TANGO_NT(3);
+    else if (n16 <= 4) TANGO_NT(4);
+    else if (n16 <= 8) TANGO_NT(8);
+    else TANGO_NT(16);
+#undef TANGO_NT
+}
+
+// B must already be packed (16-byte aligned rows, zero-filled to a multiple of 64 columns).
+static int launch_nt(NtParams p, hipStream_t s) {
+    if (p.M == 0 || p.N == 0) return TANGO_OK;
+    if (ceil_div(p.M, 128) > INT32_MAX) return TANGO_ERR_UNSUPPORTED;
+    if (p.absmax_out) fill_u32(p.absmax_out, 0u, 1, s);
+    int64_t readable = 0;
+    const int vec = row_vec(p.A, p.lda, p.Kr, &readable);
+    p.a_row_bytes = readable;
+    if (vec == 16) launch_nt_vec<16>(p, s);
+    else if (vec == 4) launch_nt_vec<4>(p, s);
+    else launch_nt_vec<1>(p, s);
+    return launch_status();
+}
+
+}  // namespace tango
+
+using namespace tango;
+
+// declared in quantize.hip
+extern "C" int tango_quantize_rows_f32_i8(const float*, int64_t, int64_t, int64_t, const float*, int,
+                                          int8_t*, int64_t, int, const float*, uint64_t, uint64_t,
+                                          tango_stream_t);
+extern "C" int tango_absmax_f32(const float*, int64_t, float*, tango_stream_t);
+
+extern "C" {
+
+size_t tango_qgemm_fwd_workspace(int64_t M, int64_t N, int64_t K) {
+    (void)M;
+    if (N <= 0 || K <= 0) return 0;
+    return static_cast<size_t>(N * round_up(K, 64));
+}
+
+int tango_qgemm_fwd(float* Y, int64_t ldy, const float* X, int64_t ldx, int8_t* Xq, int64_t ldxq,
+                    const float* W, int64_t ldw, int8_t* Wq, const float* bias, float* scaleY,
+                    const float* scaleX, const float* scaleW, int64_t M, int64_t N, int64_t K,
+                    int round_mode, void* workspace, size_t workspace_bytes,
+                    tango_stream_t stream) {
+    if (M < 0 || N < 0 || K < 0 || !scaleX || !scaleW || ldy < N || ldx < K || ldw < K || ldxq < K)
+        return TANGO_ERR_INVALID_ARG;
+    if (M * N > 0 && !Y) return TANGO_ERR_INVALID_ARG;
+    if (M * K > 0 && (!X || !Xq)) return TANGO_ERR_INVALID_ARG;
+    if (N * K > 0 && (!W || !Wq)) return TANGO_ERR_INVALID_ARG;
+    if (round_mode < 0 || round_mode > 2) return TANGO_ERR_UNSUPPORTED;
+    const size_t need = tango_qgemm_fwd_workspace(M, N, K);
+    if (need > 0 && (!workspace || workspace_bytes < need)) return TANGO_ERR_WORKSPACE;
+    if ((reinterpret_cast<uintptr_t>(workspace) & 15) != 0) return TANGO_ERR_INVALID_ARG;
+    hipStream_t s = as_stream(stream);
+    int rc = tango_quantize_rows_f32_i8(X, M, K, ldx, scaleX, 0, Xq, ldxq, round_mode, nullptr, 0, 0, stream);
+    if (rc != TANGO_OK) return rc;
+    rc = tango_quantize_rows_f32_i8(W, N, K, ldw, scaleW, 0, Wq, K, round_mode, nullptr, 0, 0, stream);
+    if (rc != TANGO_OK) return rc;
+    if (M == 0 || N == 0) return TANGO_OK;
+    int8_t* Bp = static_cast<int8_t*>(workspace);
+    const int64_t ldb = round_up(K, 64);
+    if (K > 0)
+        hipLaunchKernelGGL(pack_rows_i8_kernel, dim3(grid_for(N * ldb, 256)), dim3(256), 0, s, Bp, ldb,
+                           Wq, K, N, K);
+    NtParams p{};
+    p.C = Y; p.A = Xq; p.B = Bp; p.bias = bias; p.absmax_out = scaleY; p.sA = scaleX; p.sB = scaleW;
+    p.M = M; p.N = N; p.Kr = K; p.lda = ldxq; p.ldb = ldb; p.ldc = ldy;
+    return launch_nt(p, s);
+}
+
+size_t tango_qgemm_i8_nt_workspace(int64_t M, int64_t N, int64_t K) {
+    return tango_qgemm_fwd_workspace(M, N, K);
+}
+
+int tango_qgemm_i8_nt(float* Y, int64_t ldy, const int8_t* A, int64_t lda, const int8_t* B,
+                      int64_t ldb, const float* bias, float* scaleY, const float* sA,
+                      const float* sB, int64_t M, int64_t N, int64_t K, void* workspace,
+                      size_t workspace_bytes, tango_stream_t stream) {
+    if (M < 0 || N < 0 || K < 0 || !sA || !sB || ldy < N || lda < K || ldb < K)
+        return TANGO_ERR_INVALID_ARG;
+    if ((M * N > 0 && !Y) || (M * K > 0 && !A) || (N * K > 0 && !B)) return TANGO_ERR_INVALID_ARG;
+    if (M == 0 || N == 0) return TANGO_OK;
+    hipStream_t s = as_stream(stream);
+    NtParams p{};
+    p.C = Y; p.A = A; p.bias = bias; p.absmax_out = scaleY; p.sA = sA; p.sB = sB;
+    p.M = M; p.N = N; p.Kr = K; p.lda = lda; p.ldc = ldy;
+    const size_t need = tango_qgemm_fwd_workspace(M, N, K);
+    if (need > 0 && (!workspace || workspace_bytes < need)) return TANGO_ERR_WORKSPACE;
+    if ((reinterpret_cast<uintptr_t>(workspace) & 15) != 0) return TANGO_ERR_INVALID_ARG;
+    int8_t* Bp = static_cast<int8_t*>(workspace);
+    const int64_t ldp = round_up(K, 64);
+    if (K > 0)
+        hipLaunchKernelGGL(pack_rows_i8_kernel, dim3(grid_for(N * ldp, 256)), dim3(256), 0, s, Bp, ldp,
+                           B, ldb, N, K);
+    p.B = Bp; p.ldb = ldp;
+    return launch_nt(p, s);
+}
+
+size_t tango_qgemm_bwd_dx_workspace(int64_t M, int64_t N, int64_t K) {
+    (void)M;
+    if (N <= 0 || K <= 0) return 0;
+    return static_cast<size_t>(K * round_up(N, 64));
+}
+
+int tango_qgemm_bwd_dx(float* dX, int64_t lddx, const int8_t* dYq, int64_t lddy,
+                       const int8_t* Wq, int64_t ldw, const float* s_dY, const float* s_W,
+                       int64_t M, int64_t N, int64_t K, void* workspace, size_t workspace_bytes,
+                       tango_stream_t stream) {
+    if (M < 0 || N < 0 || K < 0 || !s_dY || !s_W || lddx < K || lddy < N || ldw < K)
+        return TANGO_ERR_INVALID_ARG;
+    if ((M * K > 0 && !dX) || (M * N > 0 && !dYq) || (N * K > 0 && !Wq)) return TANGO_ERR_INVALID_ARG;
+    if (M == 0 || K == 0) return TANGO_OK;
+    const size_t need = tango_qgemm_bwd_dx_workspace(M, N, K);
+    if (need > 0 && (!workspace || workspace_bytes < need)) return TANGO_ERR_WORKSPACE;
+    if ((reinterpret_cast<uintptr_t>(workspace) & 15) != 0) return TANGO_ERR_INVALID_ARG;
+    hipStream_t s = as_stream(stream);
+    // W^T packed as [K, N padded to 64]: the small operand of an NT product with reduction N
+    int8_t* Wt = static_cast<int8_t*>(workspace);
+    const int64_t ldt = round_up(N, 64);
+    if (N > 0)
+        hipLaunchKernelGGL(transpose_pack_i8_kernel, dim3(grid_for(K * ldt, 256)), dim3(256), 0, s, Wt,
+                           ldt, Wq, ldw, N, K);
+    NtParams p{};
+    p.C = dX; p.A = dYq; p.B = Wt; p.sA = s_dY; p.sB = s_W;
+    p.M = M; p.N = K; p.Kr = N; p.lda = lddy; p.ldb = ldt; p.ldc = lddx;
+    return launch_nt(p, s);
+}
+
+size_t tango_qgemm_bwd_dw_workspace(int64_t M, int64_t N, int64_t K) {
+    (void)M;
+    if (N <= 0 || K <= 0) return 0;
+    return static_cast<size_t>(N * K) * sizeof(int);
+}
+
+int tango_qgemm_bwd_dw(float* dW, int64_t lddw, const int8_t* dYq, int64_t lddy,
+                       const int8_t* Xq, int64_t ldx, const float* s_dY, const float* s_X,
+                       int64_t M, int64_t N, int64_t K, void* workspace, size_t workspace_bytes,
+                       tango_stream_t stream) {
+    if (M < 0 || N < 0 || K < 0 || !s_dY || !s_X || lddw < K || lddy < N || ldx < K)
+        return TANGO_ERR_INVALID_ARG;
+    if ((N * K > 0 && !dW) || (M * N > 0 && !dYq) || (M * K > 0 && !Xq)) return TANGO_ERR_INVALID_ARG;
+    if (N == 0 || K == 0) return TANGO_OK;
+    const size_t need = tango_qgemm_bwd_dw_workspace(M, N, K);
+    if (!workspace || workspace_bytes < need) return TANGO_ERR_WORKSPACE;
+    if ((reinterpret_cast<uintptr_t>(workspace) & 3) != 0) return TANGO_ERR_INVALID_ARG;
+    hipStream_t s = as_stream(stream);
+    int* acc = static_cast<int*>(workspace);
+    hipLaunchKernelGGL(zero_i32_kernel, dim3(grid_for(N * K, 256)), dim3(256), 0, s, acc, N * K);
+    if (M > 0) {
+        TnParams p{};
+        p.acc = acc; p.A = dYq; p.B = Xq; p.M = M; p.N = N; p.K = K; p.lda = lddy; p.ldb = ldx;
+        p.tiles_n = static_cast<int>(ceil_div(N, 128));
+        p.tiles_k = static_cast<int>(ceil_div(K, 128));
+        const int64_t tiles = static_cast<int64_t>(p.tiles_n) * p.tiles_k;
+        // enough workgroups for ~3 per CU, each with at least 4 reduction steps
+        int64_t splits = ceil_div(768, tiles);
+        const int64_t max_splits = ceil_div(M, 256);
+        if (splits > max_splits) splits = max_splits;
+        if (splits < 1) splits = 1;
+        p.chunk = round_up(ceil_div(M, splits), 64);
+        splits = ceil_div(M, p.chunk);
+        p.splits = static_cast<int>(splits);
+        if (tiles * splits > INT32_MAX) return TANGO_ERR_UNSUPPORTED;
+        int64_t ra = 0, rb = 0;
+        const int va = row_vec(dYq, lddy, N, &ra), vb = row_vec(Xq, ldx, K, &rb);
+        const int vec = va < vb ? va : vb;
+        p.a_row_bytes = (vec == 16) ? round_up(N, 16) : (vec == 4 ? round_up(N, 4) : N);
+        p.b_row_bytes = (vec == 16) ? round_up(K, 16) : (vec == 4 ? round_up(K, 4) : K);
+        const dim3 grid(static_cast<unsigned>(tiles * splits));
+        if (vec == 16) hipLaunchKernelGGL(gemm_tn_kernel<16>, grid, dim3(256), 0, s, p);
+        else if (vec == 4) hipLaunchKernelGGL(gemm_tn_kernel<4>, grid, dim3(256), 0, s, p);
+        else hipLaunchKernelGGL(gemm_tn_kernel<1>, grid, dim3(256), 0, s, p);
+    }
+    hipLaunchKernelGGL(dequant_i32_kernel, dim3(grid_for(N * K, 256)), dim3(256), 0, s, dW, lddw, acc,
+                       N, K, s_dY, s_X);
+    return launch_status();
+}
+
+// Workspace layout of the legacy path: two scales (16 bytes), Aq packed [m, k64], Bq packed [n, k64],
+// and a dense staging copy of the larger quantized operand before packing / transposing.
+size_t tango_qgemm_legacy_workspace(int64_t m, int64_t n, int64_t k) {
+    if (m <= 0 || n <= 0 || k <= 0) return 16;
+    const int64_t k64 = round_up(k, 64);
+    const int64_t big = (m > n ? m : n) * k;
+    return static_cast<size_t>(16 + round_up(m * k64, 16) + round_up(n * k64, 16) + round_up(big, 16));
+}
+
+int tango_qgemm_legacy(float* C, const float* A, const float* B, int64_t m, int64_t n, int64_t k,
+                       int trans_a, int trans_b, void* workspace, size_t workspace_bytes,
+                       tango_stream_t stream) {
+    if (m < 0 || n < 0 || k < 0) return TANGO_ERR_INVALID_ARG;
+    if (m * n == 0) return TANGO_OK;
+    if (!C || (k > 0 && (!A || !B))) return TANGO_ERR_INVALID_ARG;
+    const size_t need = tango_qgemm_legacy_workspace(m, n, k);
+    if (!workspace || workspace_bytes < need) return TANGO_ERR_WORKSPACE;
+    if ((reinterpret_cast<uintptr_t>(workspace) & 15) != 0) return TANGO_ERR_INVALID_ARG;
+    hipStream_t s = as_stream(stream);
+    const int64_t k64 = round_up(k, 64);
+    int8_t* base = static_cast<int8_t*>(workspace);
+    float* scales = reinterpret_cast<float*>(base);
+    int8_t* Ap = base + 16;
+    int8_t* Bp = Ap + round_up(m * k64, 16);
+    int8_t* tmp = Bp + round_up(n * k64, 16);
+    int rc;
+    if ((rc = tango_absmax_f32(A, m * k, scales, stream)) != TANGO_OK) return rc;
+    if ((rc = tango_absmax_f32(B, n * k, scales + 1, stream)) != TANGO_OK) return rc;
+    // A as stored is [m,k] (or [k,m]); quantize densely, then pack (or transpose-pack) to [m, k64]
+    rc = tango_quantize_rows_f32_i8(A, 1, m * k, m * k, scales, 0, tmp, m * k, TANGO_ROUND_RNE, nullptr, 0, 0, stream);
+    if (rc != TANGO_OK) return rc;
+    if (trans_a)
+        hipLaunchKernelGGL(transpose_pack_i8_kernel, dim3(grid_for(m * k64, 256)), dim3(256), 0, s, Ap, k64, tmp, m, k, m);
+    else
+        hipLaunchKernelGGL(pack_rows_i8_kernel, dim3(grid_for(m * k64, 256)), dim3(256), 0, s, Ap, k64, tmp, k, m, k);
+    rc = tango_quantize_rows_f32_i8(B, 1, n * k, n * k, scales + 1, 0, tmp, n * k, TANGO_ROUND_RNE, nullptr, 0, 0, stream);
+    if (rc != TANGO_OK) return rc;
+    if (trans_b)  // stored [n,k]
+        hipLaunchKernelGGL(pack_rows_i8_kernel, dim3(grid_for(n * k64, 256)), dim3(256), 0, s, Bp, k64, tmp, k, n, k);
+    else  // stored [k,n]
+        hipLaunchKernelGGL(transpose_pack_i8_kernel, dim3(grid_for(n * k64, 256)), dim3(256), 0, s, Bp, k64, tmp, n, k, n);
+    NtParams p{};
+    p.C = C; p.A = Ap; p.B = Bp; p.sA = scales; p.sB = scales + 1;
+    p.M = m; p.N = n; p.Kr = k; p.lda = k64; p.ldb = k64; p.ldc = n;
+    return launch_nt(p, s);
+}
+
+}  // extern "C"

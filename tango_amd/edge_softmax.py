@@ -1,0 +1,29 @@
+"""Edge softmax over the in-edges of each destination node, optionally with the
+LeakyReLU that precedes it in GAT fused in (evaluation/test_gat.py:144-146;
+the reference calls DGL's fp32 edge_softmax, which is not part of its tree)."""
+from torch.autograd.function import Function, once_differentiable
+
+from .kernels import cuda_kernels
+
+
+class _EdgeSoftmax(Function):
+    @staticmethod
+    def forward(ctx, g, e, slope):
+        e = e if e.is_contiguous() else e.contiguous()
+        indptr, _, eids = g.adj_csc
+        a = cuda_kernels.edge_softmax_forward(e, indptr, eids, slope)
+        ctx.backward_cache = g, e, a, slope
+        return a
+
+    @staticmethod
+    @once_differentiable
+    def backward(ctx, da):
+        g, e, a, slope = ctx.backward_cache
+        indptr, _, eids = g.adj_csc
+        da = da if da.is_contiguous() else da.contiguous()
+        return None, cuda_kernels.edge_softmax_backward(a, da, e, indptr, eids, slope), None
+
+
+def edge_softmax(g, e, negative_slope=None):
+    """softmax_dst(e) if ``negative_slope`` is None, else softmax_dst(leaky_relu(e))."""
+    return _EdgeSoftmax.apply(g, e, 1.0 if negative_slope is None else float(negative_slope))

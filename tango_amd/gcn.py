@@ -1,0 +1,63 @@
+"""Quantized GCN layers: the layer math of evaluation/test_gcn.py:26-169,
+restated on the DGL-free graph object so that the benchmark's training epoch
+exercises the primitives the way the reference's driver does."""
+import torch
+import torch.nn as nn
+
+from .QLinear import Qlinear_func, Qlinear_func_reduce
+from .SPMM import spmm_copy_u
+
+
+class QGraphConv(nn.Module):
+    """GraphConv(norm='both') with int8 GEMM and int8 aggregation
+    (evaluation/test_gcn.py:26-139)."""
+
+    def __init__(self, in_feats, out_feats, bias=True, activation=None):
+        super().__init__()
+        self._in_feats, self._out_feats = in_feats, out_feats
+        self.weight = nn.Parameter(torch.empty(out_feats, in_feats))
+        self.bias = nn.Parameter(torch.empty(out_feats)) if bias else None
+        self._activation = activation
+        nn.init.xavier_uniform_(self.weight)
+        if self.bias is not None:
+            nn.init.zeros_(self.bias)
+
+    def forward(self, graph, feat):
+        norm_src = graph.out_degrees().float().clamp(min=1).pow(-0.5).unsqueeze(1)
+        feat_src = feat * norm_src
+        if self._in_feats > self._out_feats:
+            # multiply by W first, hand the GEMM epilogue's scale to the aggregation
+            feat_src, scale_feat = Qlinear_func_reduce.apply(feat_src, self.weight)
+            rst = spmm_copy_u.apply(graph, feat_src, scale_feat)
+        else:
+            rst = spmm_copy_u.apply(graph, feat_src)
+            rst = Qlinear_func.apply(rst, self.weight)
+        norm_dst = graph.in_degrees().float().clamp(min=1).pow(-0.5).unsqueeze(1)
+        rst = rst * norm_dst
+        if self.bias is not None:
+            rst = rst + self.bias
+        if self._activation is not None:
+            rst = self._activation(rst)
+        return rst
+
+
+class GCN(nn.Module):
+    """evaluation/test_gcn.py:140-169 with n_layers hidden layers after the input layer."""
+
+    def __init__(self, g, in_feats, n_hidden, n_classes, n_layers, activation, dropout):
+        super().__init__()
+        self.g = g
+        self.layers = nn.ModuleList()
+        self.layers.append(QGraphConv(in_feats, n_hidden, activation=activation))
+        for _ in range(n_layers - 1):
+            self.layers.append(QGraphConv(n_hidden, n_hidden, activation=activation))
+        self.layers.append(QGraphConv(n_hidden, n_classes))
+        self.dropout = nn.Dropout(p=dropout)
+
+    def forward(self, features):
+        h = features
+        for i, layer in enumerate(self.layers):
+            if i != 0:
+                h = self.dropout(h)
+            h = layer(self.g, h)
+        return h

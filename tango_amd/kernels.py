@@ -45,6 +45,11 @@ def _rows_view(t, name):
     return t.stride(0) if t.size(0) > 1 else max(t.size(1), t.stride(0))
 
 
+def _workspace(nbytes, device):
+    """Scratch for one call, from torch's caching allocator (no hipMalloc on the hot path)."""
+    return torch.empty(nbytes, dtype=torch.uint8, device=device) if nbytes else None
+
+
 def _mode(round_mode):
     if isinstance(round_mode, str):
         return ROUND_MODES[round_mode]
@@ -148,13 +153,14 @@ class cuda_kernels:
     def QGEMM_forward(Y, X, X_q, W, W_q, bias, scaleY, scaleX, scaleW, round_mode=None):
         for t, dt, nm in ((Y, torch.float32, "Y"), (X, torch.float32, "X"), (W, torch.float32, "W")):
             _need(t, dt, nm, contiguous=False)
-        _need(X_q, torch.int8, "X_q")
+        _need(X_q, torch.int8, "X_q", contiguous=False)
         _need(W_q, torch.int8, "W_q")
         _need(scaleX, torch.float32, "scaleX")
         _need(scaleW, torch.float32, "scaleW")
         M, K = X.shape
         N = W.size(0)
-        if W.size(1) != K or tuple(Y.shape) != (M, N) or X_q.numel() != M * K or W_q.numel() != N * K:
+        if (W.size(1) != K or tuple(Y.shape) != (M, N) or tuple(X_q.shape) != (M, K)
+                or W_q.numel() != N * K):
             raise RuntimeError("QGEMM_forward: shape mismatch")
         if bias is not None and bias.numel():
             _need(bias, torch.float32, "bias")
@@ -164,9 +170,10 @@ class cuda_kernels:
             _need(scaleY, torch.float32, "scaleY")
         mode = default_forward_round_mode() if round_mode is None else _mode(round_mode)
         ws_bytes = _L.tango_qgemm_fwd_workspace(M, N, K)
-        ws = torch.empty(ws_bytes, dtype=torch.uint8, device=X.device) if ws_bytes else None
+        ws = _workspace(ws_bytes, X.device)
         check(_L.tango_qgemm_fwd(_ptr(Y), _rows_view(Y, "Y"), _ptr(X), _rows_view(X, "X"), _ptr(X_q),
-                                 _ptr(W), _rows_view(W, "W"), _ptr(W_q), _ptr(bias), _ptr(scaleY),
+                                 _rows_view(X_q, "X_q"), _ptr(W), _rows_view(W, "W"), _ptr(W_q),
+                                 _ptr(bias), _ptr(scaleY),
                                  scaleX.data_ptr(), scaleW.data_ptr(), M, N, K, mode, _ptr(ws),
                                  ws_bytes, _stream()), "QGEMM_forward")
 
@@ -180,9 +187,11 @@ class cuda_kernels:
         N = B.size(0)
         if B.size(1) != K or tuple(Y.shape) != (M, N):
             raise RuntimeError("QGEMM_i8: shape mismatch")
+        ws_bytes = _L.tango_qgemm_i8_nt_workspace(M, N, K)
+        ws = _workspace(ws_bytes, A.device)
         check(_L.tango_qgemm_i8_nt(_ptr(Y), _rows_view(Y, "Y"), _ptr(A), _rows_view(A, "A"), _ptr(B),
                                    _rows_view(B, "B"), _ptr(bias), _ptr(scaleY), scaleA.data_ptr(),
-                                   scaleB.data_ptr(), M, N, K, _stream()), "QGEMM_i8")
+                                   scaleB.data_ptr(), M, N, K, _ptr(ws), ws_bytes, _stream()), "QGEMM_i8")
 
     @staticmethod
     def QGEMM_backward_gradX(dX, dY, W, scaledY, scaleW):
@@ -195,9 +204,11 @@ class cuda_kernels:
         N = dY.size(1)
         if dY.size(0) != M or tuple(W.shape) != (N, K):
             raise RuntimeError("QGEMM_backward_gradX: shape mismatch")
+        ws_bytes = _L.tango_qgemm_bwd_dx_workspace(M, N, K)
+        ws = _workspace(ws_bytes, dY.device)
         check(_L.tango_qgemm_bwd_dx(_ptr(dX), _rows_view(dX, "dX"), _ptr(dY), _rows_view(dY, "dY"),
                                     _ptr(W), _rows_view(W, "W"), scaledY.data_ptr(), scaleW.data_ptr(),
-                                    M, N, K, _stream()), "QGEMM_backward_gradX")
+                                    M, N, K, _ptr(ws), ws_bytes, _stream()), "QGEMM_backward_gradX")
 
     @staticmethod
     def QGEMM_backward_gradW(dW, dY, X, scaledY, scaleX):
@@ -211,7 +222,7 @@ class cuda_kernels:
         if dY.size(1) != N or tuple(X.shape) != (M, K):
             raise RuntimeError("QGEMM_backward_gradW: shape mismatch")
         ws_bytes = _L.tango_qgemm_bwd_dw_workspace(M, N, K)
-        ws = torch.empty(ws_bytes, dtype=torch.uint8, device=X.device) if ws_bytes else None
+        ws = _workspace(ws_bytes, X.device)
         check(_L.tango_qgemm_bwd_dw(_ptr(dW), _rows_view(dW, "dW"), _ptr(dY), _rows_view(dY, "dY"),
                                     _ptr(X), _rows_view(X, "X"), scaledY.data_ptr(), scaleX.data_ptr(),
                                     M, N, K, _ptr(ws), ws_bytes, _stream()), "QGEMM_backward_gradW")
@@ -227,7 +238,7 @@ class cuda_kernels:
             raise RuntimeError("Qgemm: inner dimensions differ")
         out = torch.empty((m, n), dtype=torch.float32, device=A.device)
         ws_bytes = _L.tango_qgemm_legacy_workspace(m, n, k)
-        ws = torch.empty(ws_bytes, dtype=torch.uint8, device=A.device) if ws_bytes else None
+        ws = _workspace(ws_bytes, A.device)
         check(_L.tango_qgemm_legacy(_ptr(out), _ptr(A), _ptr(B), m, n, k, int(trans_a), int(trans_b),
                                     _ptr(ws), ws_bytes, _stream()), "Qgemm")
         return out
@@ -376,6 +387,21 @@ def quantize(t, scale=None, round_mode=ROUND_RNE, noise=None, seed=0, offset=0):
     return out, scale
 
 
+def quantize_padded(t, scale=None, round_mode=ROUND_RNE, noise=None, seed=0, offset=0, align=16):
+    """Like ``quantize`` for a 2-D tensor, but the int8 rows are padded with
+    zeros to a multiple of ``align`` bytes so that the SpMM gather and the GEMM
+    fragment loads stay 16-byte aligned for odd widths (41, 602, ...).  Returns a
+    [rows, cols] view of the padded buffer and the scale."""
+    assert t.is_cuda and t.dim() == 2, "2-D GPU tensor expected"
+    if scale is None:
+        scale = cuda_kernels.get_scale(t) if t.is_contiguous() else cuda_kernels.get_scale(t.contiguous())
+    rows, cols = t.shape
+    ld = (cols + align - 1) // align * align
+    buf = torch.empty((rows, ld), dtype=torch.int8, device=t.device)
+    cuda_kernels.quantize_rows(buf, t, scale, round_mode=round_mode, noise=noise, seed=seed, offset=offset)
+    return buf[:, :cols], scale
+
+
 def mySDDMM_int8(g, op, U, V, scaleU, scaleV, isReduce, reverse=False):
     """cuda/kernels.py:33-59."""
     if reverse:
@@ -476,7 +502,7 @@ def incidence_SPMM(g, E, scaleE, reverse=False):
 
 
 def csr_SPMM(g, N, scaleN, reverse=False):
-    """cuda/kernels.py:154-165."""
+    """cuda/kernels.py:154-165.  N may be a 2-D view of a row-padded buffer."""
     if reverse:
         indptr, indices, _ = g.adj_csr
     else:
@@ -485,7 +511,12 @@ def csr_SPMM(g, N, scaleN, reverse=False):
     out_shape = (g.num_nodes(),) + feat_shape
     dim = N.numel() // max(N.size(0), 1)
     out = torch.empty((g.num_nodes(), dim), dtype=torch.float32, device=N.device)
-    cuda_kernels.csr_SPMM(out, indptr, indices, N, scaleN)
+    if N.dim() == 2 and not N.is_contiguous():
+        ld = _rows_view(N, "N")
+        base = N.as_strided((N.size(0), ld), (ld, 1))
+        cuda_kernels.csr_SPMM(out, indptr, indices, base, scaleN, ldf=ld, F=dim)
+    else:
+        cuda_kernels.csr_SPMM(out, indptr, indices, N, scaleN)
     return out.view(out_shape)
 
 

@@ -1,0 +1,238 @@
+"""GPU tests of the autograd layer (QLinear / spmm / sddmm ops): operand caching,
+GEMM -> SpMM scale hand-off, gradient formulas.  Each op's pieces are checked
+against the oracle; gradients are additionally checked against fp32 autograd
+of the dequantized math within quantization error."""
+import numpy as np
+import pytest
+import torch
+
+from gpu_util import dev, host, rand_graph, sc
+
+pytestmark = pytest.mark.gpu
+
+
+def make_graph(src, dst, n):
+    from tango_amd.graph import Graph
+    from tango_amd.util import graph_preprocess
+    return graph_preprocess(Graph(dev(src), dev(dst), n))
+
+
+def rel_err(a, b):
+    return (a - b).norm().item() / max(b.norm().item(), 1e-30)
+
+
+def test_qlinear_forward_backward_matches_oracle(orc):
+    from tango_amd.QLinear import QLinear
+    rng = np.random.default_rng(0)
+    M, Kd, N = 500, 602, 41
+    X = rng.standard_normal((M, Kd)).astype(np.float32)
+    lin = QLinear(Kd, N).cuda()
+    W, b = host(lin.weight), host(lin.bias)
+    x = dev(X).requires_grad_(True)
+    y = lin(x)
+    Y, Xq, Wq, sX, sW, _ = orc.qgemm_fwd(X, W, bias=b)
+    assert np.array_equal(host(y), Y)
+    dY = rng.standard_normal((M, N)).astype(np.float32)
+    y.backward(dev(dY))
+    s_dY = orc.absmax_scale(dY)
+    dYq = orc.quantize(dY, s_dY)
+    assert np.array_equal(host(x.grad), orc.qgemm_bwd_dx(dYq, Wq, s_dY, sW))
+    assert np.array_equal(host(lin.weight.grad), orc.qgemm_bwd_dw(dYq, Xq, s_dY, sX))
+    assert np.allclose(host(lin.bias.grad), dY.sum(0), rtol=1e-5, atol=1e-4)
+    # and the whole thing approximates the fp32 layer
+    assert rel_err(y.detach(), torch.nn.functional.linear(dev(X), lin.weight, lin.bias).detach()) < 0.02
+
+
+def test_qlinear_reduce_and_3d_input(orc):
+    from tango_amd.QLinear import QLinear
+    lin = QLinear(64, 32, bias=False).cuda()
+    lin.enable_reduce()
+    x = torch.randn(10, 7, 64, device="cuda")
+    y, s = lin(x)
+    assert tuple(y.shape) == (10, 7, 32)
+    assert host(s)[0] == orc.absmax_scale(host(y))
+
+
+def test_gemm_to_spmm_scale_handoff(orc):
+    # Qlinear_func_reduce -> spmm_copy_u(scale) equals the unfused path bit for bit
+    from tango_amd.QLinear import Qlinear_func_reduce, Qlinear_func
+    from tango_amd.SPMM import spmm_copy_u
+    rng = np.random.default_rng(1)
+    n, e = 300, 4000
+    src, dst = rand_graph(rng, n, e)
+    g = make_graph(src, dst, n)
+    X = dev(rng.standard_normal((n, 100)).astype(np.float32))
+    W = dev(rng.standard_normal((41, 100)).astype(np.float32) * 0.1)
+    y, sy = Qlinear_func_reduce.apply(X, W)
+    fused = spmm_copy_u.apply(g, y, sy)
+    unfused = spmm_copy_u.apply(g, Qlinear_func.apply(X, W))
+    assert torch.equal(fused, unfused)
+    o = orc.graph_formats(src, dst, n)
+    Y = host(y)
+    s = orc.absmax_scale(Y)
+    want = orc.spmm_csr_copy_u(o["adj_csc"][0], o["adj_csc"][1], orc.quantize(Y, s), s)
+    assert np.array_equal(host(fused), want)
+
+
+def test_spmm_copy_u_backward(orc):
+    from tango_amd.SPMM import spmm_copy_u
+    rng = np.random.default_rng(2)
+    n, e = 200, 3000
+    src, dst = rand_graph(rng, n, e)
+    g = make_graph(src, dst, n)
+    o = orc.graph_formats(src, dst, n)
+    x = dev(rng.standard_normal((n, 41)).astype(np.float32)).requires_grad_(True)
+    out = spmm_copy_u.apply(g, x)
+    dZ = rng.standard_normal((n, 41)).astype(np.float32)
+    out.backward(dev(dZ))
+    s = orc.absmax_scale(dZ)
+    want = orc.spmm_csr_copy_u(o["adj_csr"][0], o["adj_csr"][1], orc.quantize(dZ, s), s)
+    assert np.array_equal(host(x.grad), want)
+
+
+def test_spmm_u_mul_e_forward_backward(orc):
+    from tango_amd import config
+    from tango_amd.SPMM import spmm_u_mul_e
+    rng = np.random.default_rng(3)
+    n, e, H, F = 150, 2500, 8, 16
+    src, dst = rand_graph(rng, n, e)
+    g = make_graph(src, dst, n)
+    o = orc.graph_formats(src, dst, n)
+    Nf = rng.standard_normal((n, H, F)).astype(np.float32)
+    Ef = rng.random((e, H, 1)).astype(np.float32)
+    N = dev(Nf).requires_grad_(True)
+    E = dev(Ef).requires_grad_(True)
+    out = spmm_u_mul_e.apply(g, N, E)
+    sN, sE = orc.absmax_scale(Nf), orc.absmax_scale(Ef)
+    Nq, ET = orc.quantize(Nf, sN), orc.transpose_quant(Ef, sE).reshape(H, 1, e)
+    want = orc.spmm_csr_u_mul_e(*o["adj_csc"], Nq, ET, np.float32(sN) * np.float32(sE))
+    assert np.array_equal(host(out), want)
+    dZf = rng.standard_normal((n, H, F)).astype(np.float32)
+    out.backward(dev(dZf))
+    sdZ = orc.absmax_scale(dZf)
+    dZq = orc.quantize(dZf, sdZ)
+    want_dN = orc.spmm_csr_u_mul_e(*o["adj_csr"], dZq, ET, np.float32(sdZ) * np.float32(sE))
+    assert np.array_equal(host(N.grad), want_dN)
+    want_dE, _ = orc.sddmm_dot(src, dst, Nq, dZq, sN, sdZ)
+    assert np.array_equal(host(E.grad).reshape(e, H), want_dE)
+    # fp32 autograd of the same op, within quantization error
+    Nr, Er = dev(Nf).requires_grad_(True), dev(Ef).requires_grad_(True)
+    msg = Nr[dev(src)] * Er
+    ref = torch.zeros(n, H, F, device="cuda").index_add(0, dev(dst), msg)
+    ref.backward(dev(dZf))
+    assert rel_err(out.detach(), ref.detach()) < 0.03
+    assert rel_err(N.grad, Nr.grad) < 0.03 and rel_err(E.grad, Er.grad) < 0.03
+    # reference-compat switch reproduces the forward-scale quirk of cuda/SPMM.py:56
+    config.ref_compat = True
+    try:
+        N2 = dev(Nf).requires_grad_(True)
+        spmm_u_mul_e.apply(g, N2, dev(Ef)).backward(dev(dZf))
+        quirk = orc.spmm_csr_u_mul_e(*o["adj_csr"], dZq, ET, np.float32(sN) * np.float32(sE))
+        assert np.array_equal(host(N2.grad), quirk)
+    finally:
+        config.ref_compat = False
+
+
+def test_sddmm_u_add_v_and_dot_backward(orc):
+    from tango_amd.SDDMM import sddmm_u_add_v, sddmm_u_dot_v
+    rng = np.random.default_rng(4)
+    n, e, H = 120, 2000, 8
+    src, dst = rand_graph(rng, n, e)
+    g = make_graph(src, dst, n)
+    o = orc.graph_formats(src, dst, n)
+    el = rng.standard_normal((n, H, 1)).astype(np.float32)
+    er = rng.standard_normal((n, H, 1)).astype(np.float32)
+    U, V = dev(el).requires_grad_(True), dev(er).requires_grad_(True)
+    out = sddmm_u_add_v.apply(g, U, V)
+    sU, sV = orc.absmax_scale(el), orc.absmax_scale(er)
+    want, _ = orc.sddmm_ewise("add", src, dst, orc.quantize(el, sU).reshape(n, H), orc.quantize(er, sV).reshape(n, H), sU, sV)
+    assert np.array_equal(host(out).reshape(e, H), want)
+    dZ = rng.standard_normal((e, H, 1)).astype(np.float32)
+    out.backward(dev(dZ))
+    s = orc.absmax_scale(dZ)
+    dZq = orc.quantize(dZ, s).reshape(e, H)
+    assert np.array_equal(host(V.grad).reshape(n, H), orc.spmm_incidence(o["inc_in"][0], o["inc_in"][1], dZq, s, n))
+    assert np.array_equal(host(U.grad).reshape(n, H), orc.spmm_incidence(o["inc_out"][0], o["inc_out"][1], dZq, s, n))
+    # shared operand is quantized once
+    same = dev(el).requires_grad_(True)
+    out2 = sddmm_u_add_v.apply(g, same, same)
+    want2, _ = orc.sddmm_ewise("add", src, dst, orc.quantize(el, sU).reshape(n, H), orc.quantize(el, sU).reshape(n, H), sU, sU)
+    assert np.array_equal(host(out2).reshape(e, H), want2)
+    # the op the reference's drivers call but do not define
+    D = 16
+    Qf = rng.standard_normal((n, H, D)).astype(np.float32)
+    Kf = rng.standard_normal((n, H, D)).astype(np.float32)
+    Q, Kt = dev(Qf).requires_grad_(True), dev(Kf).requires_grad_(True)
+    sc_ = sddmm_u_dot_v.apply(g, Q, Kt)
+    assert tuple(sc_.shape) == (e, H, 1)
+    Qr, Kr = dev(Qf).requires_grad_(True), dev(Kf).requires_grad_(True)
+    ref = (Qr[dev(src)] * Kr[dev(dst)]).sum(-1, keepdim=True)
+    g_out = dev(rng.standard_normal((e, H, 1)).astype(np.float32))
+    sc_.backward(g_out)
+    ref.backward(g_out)
+    assert rel_err(sc_.detach(), ref.detach()) < 0.03
+    assert rel_err(Q.grad, Qr.grad) < 0.04 and rel_err(Kt.grad, Kr.grad) < 0.04
+
+
+def test_edge_softmax_autograd():
+    from tango_amd.edge_softmax import edge_softmax
+    rng = np.random.default_rng(5)
+    n, e, H = 100, 1500, 8
+    src, dst = rand_graph(rng, n, e)
+    g = make_graph(src, dst, n)
+    x = dev(rng.standard_normal((e, H, 1)).astype(np.float32)).requires_grad_(True)
+    a = edge_softmax(g, x, negative_slope=0.2)
+    xr = x.detach().clone().requires_grad_(True)
+    z = torch.nn.functional.leaky_relu(xr, 0.2)
+    d = dev(dst)
+    mx = torch.full((n, H, 1), -1e30, device="cuda").scatter_reduce(0, d.view(-1, 1, 1).expand(-1, H, 1), z, "amax")
+    ex = torch.exp(z - mx[d])
+    ref = ex / torch.zeros(n, H, 1, device="cuda").index_add(0, d, ex)[d]
+    w = dev(rng.standard_normal((e, H, 1)).astype(np.float32))
+    a.backward(w)
+    ref.backward(w)
+    assert torch.allclose(a, ref, rtol=1e-5, atol=1e-6)
+    assert torch.allclose(x.grad, xr.grad, rtol=1e-4, atol=1e-6)
+
+
+def test_stochastic_gradient_rounding_switch():
+    from tango_amd import config
+    from tango_amd.QLinear import QLinear
+    lin = QLinear(64, 32).cuda()
+    x = torch.randn(4096, 64, device="cuda")
+    dY = torch.randn(4096, 32, device="cuda")
+    grads = []
+    for mode in ("rne", "stochastic", "stochastic"):
+        config.grad_round_mode = mode
+        try:
+            lin.zero_grad()
+            lin(x).backward(dY)
+            grads.append(lin.weight.grad.clone())
+        finally:
+            config.grad_round_mode = "rne"
+    ref = dY.t() @ x
+    for gq in grads:
+        assert rel_err(gq, ref) < 0.03
+    assert not torch.equal(grads[0], grads[1]) and not torch.equal(grads[1], grads[2])
+
+
+def test_gcn_layer_trains():
+    from tango_amd.gcn import GCN
+    from tango_amd.graph import chung_lu
+    from tango_amd.util import graph_preprocess
+    g = graph_preprocess(chung_lu(2000, 20000, 2.1, seed=1, symmetric=True, device="cuda"))
+    assert (g.in_degrees() > 0).all()
+    torch.manual_seed(0)
+    model = GCN(g, 100, 32, 5, 1, torch.relu, 0.0).cuda()
+    x = torch.randn(2000, 100, device="cuda")
+    # labels that depend on the features so that the loss can go down
+    labels = (x[:, :5]).argmax(1)
+    opt = torch.optim.Adam(model.parameters(), lr=1e-2)
+    losses = []
+    for _ in range(30):
+        loss = torch.nn.functional.cross_entropy(model(x), labels)
+        opt.zero_grad()
+        loss.backward()
+        opt.step()
+        losses.append(loss.item())
+    assert losses[-1] < losses[0] * 0.9

@@ -1,0 +1,161 @@
+"""GPU parity: int8 MFMA GEMMs vs the CPU oracle.
+
+Quantized operands and int32 accumulators are bit-exact; the fp32 outputs are
+the same two IEEE roundings on both sides, so they are compared bit-exactly as
+well (the allowed tolerance is 1e-5 relative / 1e-6 absolute)."""
+import numpy as np
+import pytest
+import torch
+
+from gpu_util import dev, host, sc
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def K():
+    from tango_amd import kernels
+    return kernels
+
+
+def glorot(rng, n, k):
+    a = np.sqrt(6.0 / (n + k))
+    return ((rng.random((n, k), dtype=np.float32) * 2 - 1) * a).astype(np.float32)
+
+
+def lcg_matrix(rows, cols, seed):
+    # cuda/src/QGEMM_forward.cu:162-181 (column-major fill)
+    off = np.arange(rows * cols, dtype=np.int64)
+    return ((off + seed) * 16807 % 16 - 8).astype(np.float32).reshape(cols, rows).T.copy()
+
+
+def run_fwd(K, X, W, bias, reduce, padded, round_mode=None):
+    M, k = X.shape
+    N = W.shape[0]
+    Xd, Wd = dev(X), dev(W)
+    sX, sW = K.cuda_kernels.get_scale(Xd), K.cuda_kernels.get_scale(Wd)
+    if padded:
+        ld = (k + 15) // 16 * 16
+        Xq = torch.full((M, ld), 99, dtype=torch.int8, device="cuda")[:, :k]
+    else:
+        Xq = torch.empty((M, k), dtype=torch.int8, device="cuda")
+    Wq = torch.empty((N, k), dtype=torch.int8, device="cuda")
+    res = K.QGEMM_forward(Xd, Xq, sX, Wd, Wq, sW, None if bias is None else dev(bias), reduce,
+                          round_mode=round_mode)
+    return res, Xq, Wq, sX, sW
+
+
+@pytest.mark.parametrize("M,N,Kd", [(300, 16, 128), (1000, 41, 256), (513, 128, 602), (257, 256, 602),
+                                     (129, 300, 64), (64, 7, 20), (1, 1, 1), (4100, 256, 128)])
+@pytest.mark.parametrize("padded", [True, False])
+def test_forward(K, orc, M, N, Kd, padded):
+    rng = np.random.default_rng(M + N + Kd)
+    X = rng.standard_normal((M, Kd)).astype(np.float32)
+    W = glorot(rng, N, Kd)
+    b = rng.standard_normal(N).astype(np.float32)
+    for bias, reduce in ((None, False), (b, True)):
+        res, Xq, Wq, sX, sW = run_fwd(K, X, W, bias, reduce, padded)
+        Y, oXq, oWq, osX, osW, osY = orc.qgemm_fwd(X, W, bias=bias, reduce=reduce)
+        assert host(sX)[0] == osX and host(sW)[0] == osW
+        assert np.array_equal(host(Xq), oXq) and np.array_equal(host(Wq), oWq)
+        out = res[0] if reduce else res
+        assert np.array_equal(host(out), Y)
+        if reduce:
+            assert host(res[1])[0] == osY
+    assert orc.overflow_count() == 0
+
+
+def test_forward_rne_mode_and_lcg_pattern(K, orc):
+    rng = np.random.default_rng(0)
+    X = rng.standard_normal((200, 72)).astype(np.float32)
+    W = glorot(rng, 24, 72)
+    res, Xq, Wq, sX, sW = run_fwd(K, X, W, None, False, True, round_mode="rne")
+    Y, oXq, oWq, *_ = orc.qgemm_fwd(X, W, mode=orc.RNE)
+    assert np.array_equal(host(Xq), oXq) and np.array_equal(host(res), Y)
+    # the reference's TEST pattern: small integers, scales 0.5 -> exact product
+    A, B = lcg_matrix(96, 64, 41), lcg_matrix(40, 64, 17)
+    Xq = torch.empty((96, 64), dtype=torch.int8, device="cuda")
+    Wq = torch.empty((40, 64), dtype=torch.int8, device="cuda")
+    out = K.QGEMM_forward(dev(A), Xq, sc(0.5), dev(B), Wq, sc(0.5))
+    assert np.array_equal(host(out), (A.astype(np.float64) @ B.astype(np.float64).T).astype(np.float32))
+
+
+def test_forward_strided_input_and_output(K, orc):
+    rng = np.random.default_rng(1)
+    big = rng.standard_normal((150, 700)).astype(np.float32)
+    X = big[:, 10:612]  # row stride 700, offset 10 floats
+    W = glorot(rng, 41, 602)
+    Xd = dev(big)[:, 10:612]
+    sX = K.cuda_kernels.get_scale(Xd.contiguous())
+    Wd = dev(W)
+    sW = K.cuda_kernels.get_scale(Wd)
+    Xq = torch.empty((150, 602), dtype=torch.int8, device="cuda")
+    Wq = torch.empty((41, 602), dtype=torch.int8, device="cuda")
+    Ybuf = torch.zeros((150, 64), dtype=torch.float32, device="cuda")
+    K.cuda_kernels.QGEMM_forward(Ybuf[:, :41], Xd, Xq, Wd, Wq, torch.Tensor(), torch.Tensor(), sX, sW)
+    Y, *_ = orc.qgemm_fwd(np.ascontiguousarray(X), W)
+    assert np.array_equal(host(Ybuf)[:, :41], Y) and not host(Ybuf)[:, 41:].any()
+
+
+@pytest.mark.parametrize("M,N,Kd", [(300, 16, 128), (1000, 41, 256), (513, 128, 602), (2049, 256, 602), (65, 3, 5)])
+@pytest.mark.parametrize("padded", [True, False])
+def test_backward(K, orc, M, N, Kd, padded):
+    rng = np.random.default_rng(M * 3 + N + Kd)
+    dY = rng.integers(-127, 128, (M, N)).astype(np.int8)
+    X = rng.integers(-127, 128, (M, Kd)).astype(np.int8)
+    W = rng.integers(-127, 128, (N, Kd)).astype(np.int8)
+    s1, s2, s3 = np.float32(0.013), np.float32(0.27), np.float32(0.0051)
+
+    def put(a):
+        if not padded:
+            return dev(a)
+        ld = (a.shape[1] + 15) // 16 * 16
+        buf = torch.full((a.shape[0], ld), 77, dtype=torch.int8, device="cuda")
+        buf[:, :a.shape[1]] = dev(a)
+        return buf[:, :a.shape[1]]
+
+    dX, dW = K.QGEMM_backward(put(dY), put(X), dev(W), sc(s1), sc(s2), sc(s3))
+    assert np.array_equal(host(dX), orc.qgemm_bwd_dx(dY, W, s1, s3))
+    assert np.array_equal(host(dW), orc.qgemm_bwd_dw(dY, X, s1, s2))
+    assert orc.overflow_count() == 0
+    dX2, dW2 = K.QGEMM_backward(put(dY), put(X), dev(W), sc(s1), sc(s2), sc(s3), X_need=False)
+    assert dX2 is None and torch.equal(dW, dW2)
+
+
+def test_gradw_independent_of_split(K, orc):
+    # the same reduction seen as one long M and as two stacked halves must agree exactly
+    rng = np.random.default_rng(7)
+    M, N, Kd = 40000, 41, 256
+    dY = rng.integers(-127, 128, (M, N)).astype(np.int8)
+    X = rng.integers(-127, 128, (M, Kd)).astype(np.int8)
+    _, dW = K.QGEMM_backward(dev(dY), dev(X), dev(np.zeros((N, Kd), np.int8)), sc(1), sc(1), sc(1), X_need=False)
+    _, a = K.QGEMM_backward(dev(dY[:17000]), dev(X[:17000]), dev(np.zeros((N, Kd), np.int8)), sc(1), sc(1), sc(1), X_need=False)
+    _, b = K.QGEMM_backward(dev(dY[17000:]), dev(X[17000:]), dev(np.zeros((N, Kd), np.int8)), sc(1), sc(1), sc(1), X_need=False)
+    want = dY.astype(np.int64).T @ X.astype(np.int64)
+    assert np.array_equal(host(dW), want.astype(np.float32))
+    # scales are 1, so each part is an exactly representable integer below 2^24 in magnitude
+    assert np.abs(want).max() < 2 ** 24
+    assert np.array_equal(host(a).astype(np.int64) + host(b).astype(np.int64), want)
+
+@pytest.mark.parametrize("m,n,k", [(33, 20, 48), (128, 64, 602), (5, 3, 7)])
+def test_legacy_qgemm(K, orc, m, n, k):
+    rng = np.random.default_rng(m + n + k)
+    A = rng.standard_normal((m, k)).astype(np.float32)
+    B = rng.standard_normal((n, k)).astype(np.float32)
+    assert np.array_equal(host(K.cuda_kernels.QgemmNT(dev(A), dev(B))), orc.qgemm_legacy(A, B, False, True))
+    Bt = np.ascontiguousarray(B.T)
+    assert np.array_equal(host(K.cuda_kernels.QgemmNN(dev(A), dev(Bt))), orc.qgemm_legacy(A, Bt, False, False))
+    At = np.ascontiguousarray(A.T)
+    assert np.array_equal(host(K.cuda_kernels.QgemmTN(dev(At), dev(Bt))), orc.qgemm_legacy(At, Bt, True, False))
+
+
+def test_qgemm_i8(K, orc):
+    rng = np.random.default_rng(3)
+    M, N, Kd = 777, 41, 100
+    A = rng.integers(-127, 128, (M, Kd)).astype(np.int8)
+    B = rng.integers(-127, 128, (N, Kd)).astype(np.int8)
+    Y = torch.empty((M, N), dtype=torch.float32, device="cuda")
+    sY = torch.empty(1, dtype=torch.float32, device="cuda")
+    K.cuda_kernels.QGEMM_i8(Y, dev(A), dev(B), None, sY, sc(0.5), sc(0.25))
+    want = np.float32(0.125) * (A.astype(np.int64) @ B.astype(np.int64).T).astype(np.float32)
+    assert np.array_equal(host(Y), want) and host(sY)[0] == orc.absmax_scale(want)
