@@ -40,7 +40,7 @@ def test_qlinear_forward_backward_matches_oracle(orc):
     assert np.array_equal(host(lin.weight.grad), orc.qgemm_bwd_dw(dYq, Xq, s_dY, sX))
     assert np.allclose(host(lin.bias.grad), dY.sum(0), rtol=1e-5, atol=1e-4)
     # and the whole thing approximates the fp32 layer
-    assert rel_err(y.detach(), torch.nn.functional.linear(dev(X), lin.weight, lin.bias).detach()) < 0.02
+    assert rel_err(y.detach(), torch.nn.functional.linear(dev(X), lin.weight, lin.bias).detach()) < 0.05
 
 
 def test_qlinear_reduce_and_3d_input(orc):
