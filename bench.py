@@ -1,0 +1,318 @@
+#!/usr/bin/env python3
+"""Benchmark of the quantized-GNN primitive layer on one MI355X.
+
+A "step" is one training epoch (forward + loss + backward + Adam step) of the
+quantized 2-layer GCN 602 -> 256 -> 41 on the synthetic 232,965-node /
+~114.6M-edge power-law graph: int8 GEMMs with cached quantized operands, the
+GEMM epilogue's scale handed to the int8 aggregation, stochastic rounding on
+gradients.  Inputs are resident in HBM before the timed region.  Prints one
+JSON line.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBPS = 8000.0
+
+
+def parse():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=10)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--nodes", type=int, default=232965)
+    ap.add_argument("--edges", type=int, default=114_600_000)
+    ap.add_argument("--cpu-fraction", type=float, default=1.0 / 8, help="share of rows the CPU baseline runs")
+    ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--no-primitives", action="store_true")
+    return ap.parse_args()
+
+
+class KernelTimer:
+    """HIP-event timing of selected launches on torch's current stream (the stream the library launches on)."""
+
+    def __init__(self):
+        self.spans = {}
+
+    def wrap(self, fn, key_of):
+        import torch
+
+        def timed(*a, **kw):
+            key = key_of(*a, **kw)
+            if key is None:
+                return fn(*a, **kw)
+            s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            s.record()
+            r = fn(*a, **kw)
+            e.record()
+            self.spans.setdefault(key, []).append((s, e))
+            return r
+        return timed
+
+    def mean_ms(self, key):
+        v = [s.elapsed_time(e) for s, e in self.spans.get(key, [])]
+        return sum(v) / len(v) if v else None
+
+    def clear(self):
+        self.spans = {}
+
+
+def time_op(fn, iters=20, warm=3):
+    import torch
+    for _ in range(warm):
+        fn()
+    s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    torch.cuda.synchronize()
+    s.record()
+    for _ in range(iters):
+        fn()
+    e.record()
+    torch.cuda.synchronize()
+    return s.elapsed_time(e) / iters
+
+
+def spmm_bytes(nnz, rows, F, idx=8):
+    return nnz * (F + idx) + rows * (4 * F + 8)
+
+
+def primitives(g, K, torch):
+    """Per-primitive throughput at the sizes the metric quotes (outside the timed epoch)."""
+    out = {}
+    n, nnz = g.num_nodes(), g.num_edges()
+    one = torch.ones(1, device="cuda") * 0.01
+    for F in (16, 64, 128, 256):
+        feat = torch.randint(-127, 128, (n, F), dtype=torch.int8, device="cuda")
+        ms = time_op(lambda: K.csr_SPMM(g, feat, one), iters=10)
+        b = spmm_bytes(nnz, n, F)
+        out["spmm_copy_u_F%d" % F] = {"ms": round(ms, 4), "GBps": round(b / ms / 1e6, 1),
+                                      "frac_hbm": round(b / ms / 1e6 / HBM_PEAK_GBPS, 4)}
+        del feat
+    # u_mul_e, broadcast edge value: H=4, F=64 (cuda/../evaluation/SPMM_broadcast.py sizes are (2|4, 128|256))
+    H, F = 2, 128
+    feat = torch.randint(-127, 128, (n, H, F), dtype=torch.int8, device="cuda")
+    ev = torch.randint(-127, 128, (H, 1, nnz), dtype=torch.int8, device="cuda")
+    ms = time_op(lambda: K.multi_cusparse_SPMM(g, feat, ev, one), iters=5)
+    b = nnz * (H * F + H + 16) + n * (4 * H * F + 8)
+    out["spmm_u_mul_e_H2_F128"] = {"ms": round(ms, 4), "GBps": round(b / ms / 1e6, 1),
+                                   "frac_hbm": round(b / ms / 1e6 / HBM_PEAK_GBPS, 4)}
+    del feat, ev
+    # QLinear forward / backward at (M, K, N) = (232965, 602, 256) and (232965, 256, 41)
+    for (M, Kd, N) in ((n, 602, 256), (n, 256, 41), (n, 128, 16)):
+        X = torch.randn(M, Kd, device="cuda")
+        W = torch.randn(N, Kd, device="cuda") * 0.05
+        sX, sW = K.cuda_kernels.get_scale(X), K.cuda_kernels.get_scale(W)
+        ld = (Kd + 15) // 16 * 16
+        Xq = torch.empty((M, ld), dtype=torch.int8, device="cuda")[:, :Kd]
+        Wq = torch.empty((N, Kd), dtype=torch.int8, device="cuda")
+        ms = time_op(lambda: K.QGEMM_forward(X, Xq, sX, W, Wq, sW, None, True), iters=10)
+        ops = 2.0 * M * N * Kd
+        byt = 5 * (M * Kd + N * Kd) + 4 * M * N
+        tag = "qlinear_fwd_%dx%dx%d" % (M, Kd, N)
+        out[tag] = {"ms": round(ms, 4), "TOPS": round(ops / ms / 1e9, 2), "GBps": round(byt / ms / 1e6, 1),
+                    "frac_hbm": round(byt / ms / 1e6 / HBM_PEAK_GBPS, 4),
+                    "frac_i8_mfma": round(ops / ms / 1e9 / 5000.0, 4)}
+        dY, s_dY = K.quantize_padded(torch.randn(M, N, device="cuda"))
+        ms = time_op(lambda: K.QGEMM_backward(dY, Xq, Wq, s_dY, sX, sW, True, False), iters=10)
+        byt = M * N + N * Kd + 4 * M * Kd
+        out[tag.replace("fwd", "gradX")] = {"ms": round(ms, 4), "TOPS": round(ops / ms / 1e9, 2),
+                                            "GBps": round(byt / ms / 1e6, 1)}
+        ms = time_op(lambda: K.QGEMM_backward(dY, Xq, Wq, s_dY, sX, sW, False, True), iters=10)
+        byt = M * (N + Kd) + 4 * N * Kd
+        out[tag.replace("fwd", "gradW")] = {"ms": round(ms, 4), "TOPS": round(ops / ms / 1e9, 2),
+                                            "GBps": round(byt / ms / 1e6, 1)}
+        del X, W, Xq, dY
+    # quantize / absmax streaming
+    X = torch.randn(n, 602, device="cuda")
+    ms = time_op(lambda: K.cuda_kernels.get_scale(X))
+    out["absmax_140M"] = {"ms": round(ms, 4), "GBps": round(4 * X.numel() / ms / 1e6, 1)}
+    s = K.cuda_kernels.get_scale(X)
+    q = torch.empty(X.shape, dtype=torch.int8, device="cuda")
+    ms = time_op(lambda: K.cuda_kernels.quantize(q, X, s))
+    out["quantize_140M"] = {"ms": round(ms, 4), "GBps": round(5 * X.numel() / ms / 1e6, 1)}
+    del X, q
+    return out
+
+
+def sddmm_primitives(K, torch):
+    """GAT-shaped SDDMM on the 169,343-node / 1.17M-edge graph (8 heads x 16)."""
+    from tango_amd.graph import chung_lu
+    from tango_amd.util import graph_preprocess
+    g = graph_preprocess(chung_lu(169343, 1166243, 2.2, seed=4, device="cuda"))
+    n, E, H, D = g.num_nodes(), g.num_edges(), 8, 16
+    U = torch.randint(-127, 128, (n, H, D), dtype=torch.int8, device="cuda")
+    V = torch.randint(-127, 128, (n, H, D), dtype=torch.int8, device="cuda")
+    one = torch.ones(1, device="cuda") * 0.01
+    out = {"graph": {"nodes": n, "edges": E}}
+    ms = time_op(lambda: K.mySDDMM_int8(g, "dot", U, V, one, one, False))
+    b = E * (16 + 2 * H * D + 4 * H)
+    out["sddmm_dot_H8_D16"] = {"ms": round(ms, 4), "GBps": round(b / ms / 1e6, 1),
+                               "frac_hbm": round(b / ms / 1e6 / HBM_PEAK_GBPS, 4)}
+    el = torch.randint(-127, 128, (n, H, 1), dtype=torch.int8, device="cuda")
+    ms = time_op(lambda: K.mySDDMM_int8(g, "add", el, el, one, one, False))
+    b = E * (16 + 2 * H + 4 * H)
+    out["sddmm_add_H8"] = {"ms": round(ms, 4), "GBps": round(b / ms / 1e6, 1)}
+    e = torch.randn(E, H, 1, device="cuda")
+    ip, _, eid = g.adj_csc
+    ms = time_op(lambda: K.cuda_kernels.edge_softmax_forward(e, ip, eid, 0.2))
+    out["edge_softmax_H8"] = {"ms": round(ms, 4), "GBps": round(E * (8 * H + 8) / ms / 1e6, 1)}
+    return out
+
+
+def cpu_baseline(g, X, W1, W2, frac):
+    """The CPU oracle (a port of the reference's semantics, OpenMP over the host
+    cores) on every k-th destination row / node of the same workload:
+    forward GEMM+aggregation of both layers and the backward aggregations and
+    GEMMs, i.e. the primitives of one epoch.  Returns (epoch-equivalent ms, note)."""
+    import numpy as np
+    from oracle import oracle as orc
+    n = g.num_nodes()
+    stride = max(1, int(round(1.0 / frac)))
+    rows = np.arange(0, n, stride)
+    threads = len(os.sched_getaffinity(0))
+    orc.set_num_threads(threads)
+
+    def sub_csr(fmt):
+        ip, ix, _ = fmt
+        ip, ix = ip.cpu().numpy(), ix.cpu().numpy()
+        starts, ends = ip[rows], ip[rows + 1]
+        lens = ends - starts
+        sip = np.zeros(rows.size + 1, np.int64)
+        np.cumsum(lens, out=sip[1:])
+        take = np.repeat(starts - sip[:-1], lens) + np.arange(sip[-1])
+        return sip, ix[take]
+
+    csc, csr = sub_csr(g.adj_csc), sub_csr(g.adj_csr)
+    Xs = X[rows].cpu().numpy()
+    W1n, W2n = W1.cpu().numpy(), W2.cpu().numpy()
+    rng = np.random.default_rng(0)
+    f1 = rng.integers(-127, 128, (n, 256)).astype(np.int8)  # full-width int8 node features to gather from
+    f2 = rng.integers(-127, 128, (n, 41)).astype(np.int8)
+    t0 = time.perf_counter()
+    # layer 1 forward: GEMM (quantize fused) then aggregation of 256-wide rows
+    Y1, Xq, W1q, sX, sW1, sY1 = orc.qgemm_fwd(Xs, W1n, reduce=True)
+    orc.quantize(Y1, sY1)
+    orc.spmm_csr_copy_u(csc[0], csc[1], f1, 0.01)
+    # layer 2 forward
+    H1 = np.maximum(Y1, 0)
+    Y2, Hq, W2q, sH, sW2, sY2 = orc.qgemm_fwd(H1, W2n, reduce=True)
+    orc.quantize(Y2, sY2)
+    orc.spmm_csr_copy_u(csc[0], csc[1], f2, 0.01)
+    # backward: aggregation of dZ on the reverse graph, then gradX / gradW, both layers
+    orc.spmm_csr_copy_u(csr[0], csr[1], f2, 0.01)
+    dY2 = rng.standard_normal(Y2.shape).astype(np.float32)
+    s2 = orc.absmax_scale(dY2)
+    dY2q = orc.quantize(dY2, s2)
+    orc.qgemm_bwd_dx(dY2q, W2q, s2, sW2)
+    orc.qgemm_bwd_dw(dY2q, Hq, s2, sH)
+    orc.spmm_csr_copy_u(csr[0], csr[1], f1, 0.01)
+    dY1 = rng.standard_normal(Y1.shape).astype(np.float32)
+    s1 = orc.absmax_scale(dY1)
+    dY1q = orc.quantize(dY1, s1)
+    orc.qgemm_bwd_dw(dY1q, Xq, s1, sX)
+    dt = time.perf_counter() - t0
+    note = ("oracle port, OpenMP x%d, primitives of one epoch on every %dth node/destination row "
+            "(%d rows, %d edges), %.1f s measured, scaled by %d" % (threads, stride, rows.size,
+                                                                   int(csc[0][-1]), dt, stride))
+    return dt * 1000.0 * stride, threads, note
+
+
+def main():
+    args = parse()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py: this build runs on one GPU only (no collectives, no sharding); use --gpus 1",
+              file=sys.stderr)
+        sys.exit(2)
+    import torch
+    from tango_amd import config, kernels as K
+    from tango_amd.gcn import GCN
+    from tango_amd.graph import chung_lu
+    from tango_amd.util import graph_preprocess
+
+    torch.cuda.set_device(0)
+    t0 = time.perf_counter()
+    g = graph_preprocess(chung_lu(args.nodes, args.edges, 2.0, seed=3, max_degree=21000, symmetric=True,
+                                  device="cuda"))
+    torch.cuda.synchronize()
+    n, nnz = g.num_nodes(), g.num_edges()
+    max_deg = int(g.in_degrees().max().item())
+    sys.stderr.write("graph: %d nodes, %d directed edges, max in-degree %d (%.1f s)\n"
+                     % (n, nnz, max_deg, time.perf_counter() - t0))
+
+    gen = torch.Generator().manual_seed(5)
+    X = torch.randn(n, 602, generator=gen).cuda()
+    labels = torch.randint(0, 41, (n,), generator=gen).cuda()
+    torch.manual_seed(5)
+    model = GCN(g, 602, 256, 41, 1, torch.relu, 0.0).cuda()
+    opt = torch.optim.Adam(model.parameters(), lr=1e-2, weight_decay=5e-4)
+    config.grad_round_mode = "stochastic"
+
+    timer = KernelTimer()
+    raw_spmm = K.cuda_kernels.csr_SPMM
+    K.cuda_kernels.csr_SPMM = staticmethod(timer.wrap(
+        raw_spmm, lambda out, ip, ix, U, s, ldf=None, F=None: "spmm_F%d" % (out.size(1))))
+
+    def step():
+        loss = torch.nn.functional.cross_entropy(model(X), labels)
+        opt.zero_grad(set_to_none=True)
+        loss.backward()
+        opt.step()
+        return loss
+
+    for _ in range(args.warmup):
+        step()
+    timer.clear()
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    for _ in range(args.steps):
+        loss = step()
+    torch.cuda.synchronize()
+    ms_per_step = (time.perf_counter() - t1) * 1000.0 / args.steps
+    K.cuda_kernels.csr_SPMM = staticmethod(raw_spmm)
+
+    # dominant kernel: the 256-wide copy_u aggregation (forward and reverse launches of the same kernel)
+    k_ms = timer.mean_ms("spmm_F256")
+    alg = spmm_bytes(nnz, n, 256)
+    achieved = alg / k_ms / 1e6
+    roofline = {"kernel": "spmm_kernel<16,4,copy_u> F=256", "bound": "hbm", "achieved": round(achieved, 1),
+                "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4),
+                "traffic": None, "avg_launch_ms": round(k_ms, 4), "algorithmic_bytes": alg,
+                "launches_timed": len(timer.spans.get("spmm_F256", []))}
+
+    result = {
+        "metric": "quant GCN epoch ms @233K nodes/114.6M edges; SpMM/SDDMM GB/s; QLinear TOPS",
+        "value": round(ms_per_step, 3), "unit": "ms/epoch", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": round(ms_per_step, 3), "higher_is_better": False,
+        "scaling": "weak", "vs_baseline": None, "dtype": "int8 x int8 -> int32 (fp32 dequant)",
+        "data": "synthetic",
+        "config": {"workload": "2-layer quantized GCN 602->256->41 training epoch (fwd+loss+bwd+Adam), "
+                               "Chung-Lu graph gamma=2.0 seed=3 symmetric + self loops",
+                   "nodes": n, "edges": nnz, "max_in_degree": max_deg, "grad_rounding": "stochastic",
+                   "loss": round(float(loss.item()), 4)},
+        "roofline": roofline,
+    }
+    result["spmm_F41_ms"] = timer.mean_ms("spmm_F41")
+
+    if not args.no_primitives:
+        prims = primitives(g, K, torch)
+        prims.update(sddmm_primitives(K, torch))
+        result["primitives"] = prims
+        result["spmm_GBps"] = prims["spmm_copy_u_F256"]["GBps"]
+        result["sddmm_GBps"] = prims["sddmm_dot_H8_D16"]["GBps"]
+        result["qlinear_TOPS"] = prims["qlinear_fwd_%dx602x256" % n]["TOPS"]
+
+    if not args.no_cpu:
+        W1 = model.layers[0].weight.detach()
+        W2 = model.layers[1].weight.detach()
+        ms, cores, note = cpu_baseline(g, X, W1, W2, args.cpu_fraction)
+        result["cpu_baseline"] = {"value": round(ms, 1), "unit": "ms/epoch", "cores": cores, "kind": "port",
+                                  "sample": note}
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

@@ -33,6 +33,7 @@ class Graph:
         self.ndata, self.edata = {}, {}
         self.srcdata = self.dstdata = self.ndata
         self._csr = self._csc = None
+        self._in_deg = self._out_deg = None
 
     # -- the DGL calls of cuda/util.py:5-11 ---------------------------------
     @property
@@ -81,10 +82,18 @@ class Graph:
         raise ValueError("typ must be 'in' or 'out'")
 
     def in_degrees(self):
-        return torch.bincount(self._dst, minlength=self._n)
+        """Cached (DGL keeps degrees with the graph; a bincount over 1e8 edges per call would
+        dominate an epoch)."""
+        if self._in_deg is None:
+            indptr = self.adj_sparse("csc")[0]
+            self._in_deg = indptr[1:] - indptr[:-1]
+        return self._in_deg
 
     def out_degrees(self):
-        return torch.bincount(self._src, minlength=self._n)
+        if self._out_deg is None:
+            indptr = self.adj_sparse("csr")[0]
+            self._out_deg = indptr[1:] - indptr[:-1]
+        return self._out_deg
 
     @contextlib.contextmanager
     def local_scope(self):
