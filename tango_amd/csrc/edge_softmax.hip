@@ -1,10 +1,11 @@
 // LeakyReLU + per-destination edge softmax (forward and backward) for gfx950.
 //
 // fp32, memory-bound: e is read, a written, both [E, H] in edge-id order and
-// reached through the destination-major CSR's edge-id permutation.  A group of
-// lanes (one lane per head) owns one destination row, so the H values of an
-// edge are one contiguous read.  The forward pass keeps a running (max, sum)
+// reached through the destination-major CSR's edge-id permutation.  A wavefront
+// owns one destination row; its lanes are (edge slot, head) pairs, so the H values
+// of an edge are one contiguous read.  The forward pass keeps a running (max, sum)
 // pair per lane (online softmax): two sweeps over the row instead of three.
+// For H > 64 a thread-per-(row, head) fallback is used.
 #include "common.hpp"
 
 namespace tango {
@@ -20,21 +21,22 @@ __global__ __launch_bounds__(256) void edge_softmax_fwd_kernel(
         const int64_t r = i / H;
         const int h = static_cast<int>(i - r * H);
         const int64_t p0 = indptr[r], p1 = indptr[r + 1];
-        float mx = -INFINITY, sum = 0.0f;
+        float mx = -INFINITY;
+        double sum = 0.0;  // long rows: keep the running sum's rounding error out of the result
         for (int64_t p = p0; p < p1; ++p) {
             const int64_t id = eids ? eids[p] : p;
             const float v = leaky(e[id * H + h], slope);
             if (v > mx) {
-                sum = sum * __expf(mx - v) + 1.0f;
+                sum = sum * static_cast<double>(expf(mx - v)) + 1.0;
                 mx = v;
             } else {
-                sum += __expf(v - mx);
+                sum += static_cast<double>(expf(v - mx));
             }
         }
-        const float inv = 1.0f / sum;
+        const float inv = static_cast<float>(1.0 / sum);
         for (int64_t p = p0; p < p1; ++p) {
             const int64_t id = eids ? eids[p] : p;
-            a[id * H + h] = __expf(leaky(e[id * H + h], slope) - mx) * inv;
+            a[id * H + h] = expf(leaky(e[id * H + h], slope) - mx) * inv;
         }
     }
 }
@@ -49,12 +51,91 @@ __global__ __launch_bounds__(256) void edge_softmax_bwd_kernel(
         const int64_t r = i / H;
         const int h = static_cast<int>(i - r * H);
         const int64_t p0 = indptr[r], p1 = indptr[r + 1];
-        float dot = 0.0f;
+        double dsum = 0.0;
         for (int64_t p = p0; p < p1; ++p) {
             const int64_t id = eids ? eids[p] : p;
-            dot += a[id * H + h] * da[id * H + h];
+            dsum += static_cast<double>(a[id * H + h]) * static_cast<double>(da[id * H + h]);
         }
+        const float dot = static_cast<float>(dsum);
         for (int64_t p = p0; p < p1; ++p) {
+            const int64_t id = eids ? eids[p] : p;
+            float g = a[id * H + h] * (da[id * H + h] - dot);
+            if (!(e[id * H + h] > 0.0f)) g *= slope;
+            de[id * H + h] = g;
+        }
+    }
+}
+
+// Wave-per-row kernels: lane = (edge slot es, head h) with Hp = H rounded up to a
+// power of two, so one step of the wavefront covers 64 / Hp edges of the row and
+// the per-head reduction is an xor-shuffle over the slot bits.  Used for H <= 64;
+// a high-degree destination is walked by 64 lanes instead of one.
+__device__ __forceinline__ void softmax_merge(float& m, double& s, float m2, double s2) {
+    const float mx = fmaxf(m, m2);
+    // exp(-inf - -inf) would be NaN: a side with no elements contributes nothing
+    const double a = (m == -INFINITY) ? 0.0 : s * static_cast<double>(expf(m - mx));
+    const double b = (m2 == -INFINITY) ? 0.0 : s2 * static_cast<double>(expf(m2 - mx));
+    m = mx;
+    s = a + b;
+}
+
+__global__ __launch_bounds__(256) void edge_softmax_fwd_wave_kernel(
+    float* __restrict__ a, const float* __restrict__ e, const int64_t* __restrict__ indptr,
+    const int64_t* __restrict__ eids, int64_t rows, int H, int hp_log2, float slope) {
+    const int64_t row = static_cast<int64_t>(blockIdx.x) * 4 + (threadIdx.x >> 6);
+    if (row >= rows) return;
+    const int lane = lane_id();
+    const int h = lane & ((1 << hp_log2) - 1);
+    const int es = lane >> hp_log2;
+    const int nes = kWave >> hp_log2;
+    const int64_t p0 = indptr[row], p1 = indptr[row + 1];
+    const bool hok = h < H;
+    float mx = -INFINITY;
+    double sum = 0.0;
+    for (int64_t p = p0 + es; p < p1; p += nes) {
+        if (hok) {
+            const int64_t id = eids ? eids[p] : p;
+            const float v = leaky(e[id * H + h], slope);
+            softmax_merge(mx, sum, v, 1.0);
+        }
+    }
+    for (int off = 1 << hp_log2; off < kWave; off <<= 1) {
+        const float m2 = __shfl_xor(mx, off, kWave);
+        const double s2 = __shfl_xor(sum, off, kWave);
+        softmax_merge(mx, sum, m2, s2);
+    }
+    const float inv = static_cast<float>(1.0 / sum);
+    for (int64_t p = p0 + es; p < p1; p += nes) {
+        if (hok) {
+            const int64_t id = eids ? eids[p] : p;
+            a[id * H + h] = expf(leaky(e[id * H + h], slope) - mx) * inv;
+        }
+    }
+}
+
+__global__ __launch_bounds__(256) void edge_softmax_bwd_wave_kernel(
+    float* __restrict__ de, const float* __restrict__ a, const float* __restrict__ da,
+    const float* __restrict__ e, const int64_t* __restrict__ indptr,
+    const int64_t* __restrict__ eids, int64_t rows, int H, int hp_log2, float slope) {
+    const int64_t row = static_cast<int64_t>(blockIdx.x) * 4 + (threadIdx.x >> 6);
+    if (row >= rows) return;
+    const int lane = lane_id();
+    const int h = lane & ((1 << hp_log2) - 1);
+    const int es = lane >> hp_log2;
+    const int nes = kWave >> hp_log2;
+    const int64_t p0 = indptr[row], p1 = indptr[row + 1];
+    const bool hok = h < H;
+    double dsum = 0.0;
+    for (int64_t p = p0 + es; p < p1; p += nes) {
+        if (hok) {
+            const int64_t id = eids ? eids[p] : p;
+            dsum += static_cast<double>(a[id * H + h]) * static_cast<double>(da[id * H + h]);
+        }
+    }
+    for (int off = 1 << hp_log2; off < kWave; off <<= 1) dsum += __shfl_xor(dsum, off, kWave);
+    const float dot = static_cast<float>(dsum);
+    for (int64_t p = p0 + es; p < p1; p += nes) {
+        if (hok) {
             const int64_t id = eids ? eids[p] : p;
             float g = a[id * H + h] * (da[id * H + h] - dot);
             if (!(e[id * H + h] > 0.0f)) g *= slope;
@@ -75,6 +156,14 @@ int tango_edge_softmax_fwd(float* a, const float* e, const int64_t* indptr,
     if (rows < 0 || H < 0 || (rows > 0 && !indptr) || H >= (1LL << 31)) return TANGO_ERR_INVALID_ARG;
     if (rows * H == 0) return TANGO_OK;
     if (!a || !e) return TANGO_ERR_INVALID_ARG;
+    if (H <= 64 && ceil_div(rows, 4) <= INT32_MAX) {
+        int hp = 0;
+        while ((1 << hp) < H) ++hp;
+        hipLaunchKernelGGL(edge_softmax_fwd_wave_kernel, dim3(static_cast<unsigned>(ceil_div(rows, 4))),
+                           dim3(256), 0, as_stream(stream), a, e, indptr, edge_ids, rows,
+                           static_cast<int>(H), hp, slope);
+        return launch_status();
+    }
     hipLaunchKernelGGL(edge_softmax_fwd_kernel, dim3(grid_for(rows * H, 256, 16)), dim3(256), 0,
                        as_stream(stream), a, e, indptr, edge_ids, rows, static_cast<int>(H), slope);
     return launch_status();
@@ -86,6 +175,14 @@ int tango_edge_softmax_bwd(float* de, const float* a, const float* da, const flo
     if (rows < 0 || H < 0 || (rows > 0 && !indptr) || H >= (1LL << 31)) return TANGO_ERR_INVALID_ARG;
     if (rows * H == 0) return TANGO_OK;
     if (!de || !a || !da || !e) return TANGO_ERR_INVALID_ARG;
+    if (H <= 64 && ceil_div(rows, 4) <= INT32_MAX) {
+        int hp = 0;
+        while ((1 << hp) < H) ++hp;
+        hipLaunchKernelGGL(edge_softmax_bwd_wave_kernel, dim3(static_cast<unsigned>(ceil_div(rows, 4))),
+                           dim3(256), 0, as_stream(stream), de, a, da, e, indptr, edge_ids, rows,
+                           static_cast<int>(H), hp, slope);
+        return launch_status();
+    }
     hipLaunchKernelGGL(edge_softmax_bwd_kernel, dim3(grid_for(rows * H, 256, 16)), dim3(256), 0,
                        as_stream(stream), de, a, da, e, indptr, edge_ids, rows, static_cast<int>(H),
                        slope);

@@ -3,11 +3,12 @@
 //
 // These are gather kernels bound by the memory system, not by arithmetic, so
 // no MFMA is used.  Layout of the work:
-//   * a wavefront (or a 4-wave workgroup for high-degree graphs) owns one
-//     output row and walks that row's CSR slots 64 at a time;
-//   * the 64 column indices of a step are fetched with ONE coalesced 512-byte
-//     load (lane i holds slot i) and handed to the lanes that need them with
-//     ds_bpermute, so index traffic is read exactly once;
+//   * a wavefront (or a 4-wave workgroup for long, wide rows) owns one
+//     output row and walks that row's CSR slots;
+//   * column indices are fetched 256 slots at a time with four independent
+//     coalesced 512-byte loads (lane i of load r holds slot 64 r + i) and handed
+//     to the lanes that need them with ds_bpermute, so index traffic is read
+//     exactly once and one HBM round trip is paid per 256 edges;
 //   * a group of `lpe` lanes (power of two) covers one gathered int8 feature
 //     row with 16-, 4- or 1-byte loads per lane, so one load instruction of
 //     the wavefront pulls 64/lpe neighbour rows (F = 256 -> 4 rows of 256 B,
@@ -134,7 +135,7 @@ __global__ __launch_bounds__(256) void spmm_kernel(const SpmmParams p) {
         end = e < end ? e : end;
     }
 
-    const int8_t* wbase = nullptr;
+    const int8_t* wbase = p.evals;
     if (KIND == KIND_WEIGHTED && col_ok) {
         const int64_t h = col / p.F;
         const int64_t d = (p.D == 1) ? 0 : (col - h * p.F);
@@ -145,44 +146,66 @@ __global__ __launch_bounds__(256) void spmm_kernel(const SpmmParams p) {
 #pragma unroll
     for (int i = 0; i < VEC; ++i) acc[i] = 0;
 
-    const int8_t* fcol = p.feat + col;
-    int64_t base = start;
-    int my = (base + lane < end) ? static_cast<int>(p.indices[base + lane]) : -1;
-    int my_e = 0;
-    if (KIND == KIND_WEIGHTED && p.edge_ids)
-        my_e = (base + lane < end) ? static_cast<int>(p.edge_ids[base + lane]) : 0;
+    // Lanes past the row's width read column 0 (a valid address) and never store, and the
+    // fold below only mixes lanes of equal `sub`, so they need no masking.
+    const int8_t* fcol = p.feat + (col_ok ? col : 0);
+    const int sh = 6 - p.lpe_log2;
 
-    while (base < end) {
-        const int64_t nbase = base + kWave;
-        // prefetch the next step's indices while this step's rows are gathered
-        const int nxt = (nbase + lane < end) ? static_cast<int>(p.indices[nbase + lane]) : -1;
-        int nxt_e = 0;
-        if (KIND == KIND_WEIGHTED && p.edge_ids)
-            nxt_e = (nbase + lane < end) ? static_cast<int>(p.edge_ids[nbase + lane]) : 0;
-        const int cnt = static_cast<int>((end - base) < kWave ? (end - base) : kWave);
-        const int steps = (cnt + epi - 1) >> (6 - p.lpe_log2);
-        for (int t = 0; t < steps; t += U) {
-            typename Gather<VEC>::T d[U];
-            int w[U];
+    // Indices are fetched 256 slots at a time with four independent coalesced loads
+    // (lane i of load r holds slot 64 r + i), so one HBM round trip is paid per 256 edges.
+    for (int64_t base = start; base < end; base += 4 * kWave) {
+        int my[4], my_e[4];
 #pragma unroll
-            for (int u = 0; u < U; ++u) {
-                const int slot = ((t + u) << (6 - p.lpe_log2)) + grp;  // may exceed 63 past the end
-                const int j = __shfl(my, slot & 63, kWave);
-                const bool ok = (t + u) < steps && j >= 0 && col_ok;
-                d[u] = ok ? Gather<VEC>::load(fcol + static_cast<int64_t>(j) * p.ldf) : Gather<VEC>::zero();
-                w[u] = 1;
-                if (KIND == KIND_WEIGHTED) {
-                    int64_t e = base + slot;
-                    if (p.edge_ids) e = __shfl(my_e, slot & 63, kWave);
-                    w[u] = ok ? static_cast<int>(wbase[e]) : 0;
+        for (int r = 0; r < 4; ++r) {
+            const int64_t q = base + r * kWave + lane;
+            const int64_t qc = q < end ? q : end - 1;  // clamped: the load is unconditional
+            // streamed once: keep the index array from evicting feature rows out of L2
+            const int v = static_cast<int>(__builtin_nontemporal_load(p.indices + qc));
+            my[r] = q < end ? v : -1;
+            my_e[r] = 0;
+            if (KIND == KIND_WEIGHTED && p.edge_ids)
+                my_e[r] = static_cast<int>(__builtin_nontemporal_load(p.edge_ids + qc));
+        }
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const int64_t cbase = base + r * kWave;
+            if (cbase < end) {  // uniform
+                const int cnt = static_cast<int>((end - cbase) < kWave ? (end - cbase) : kWave);
+                const int steps = (cnt + epi - 1) >> sh;
+                for (int t = 0; t < steps; t += U) {
+                    int j[U];
+                    int slot[U];
+#pragma unroll
+                    for (int u = 0; u < U; ++u) {
+                        slot[u] = ((t + u) << sh) + grp;  // wraps past the chunk for t + u >= steps: masked below
+                        j[u] = __shfl(my[r], slot[u] & 63, kWave);
+                    }
+                    typename Gather<VEC>::T d[U];
+                    int w[U];
+                    bool ok[U];
+#pragma unroll
+                    for (int u = 0; u < U; ++u) {
+                        ok[u] = (t + u) < steps && j[u] >= 0;
+                        // invalid slots read row 0 and are zeroed afterwards: no branch around the load
+                        d[u] = Gather<VEC>::load(fcol + static_cast<int64_t>(ok[u] ? j[u] : 0) * p.ldf);
+                        w[u] = 1;
+                        if (KIND == KIND_WEIGHTED) {
+                            int64_t e = cbase + (slot[u] & 63);
+                            if (p.edge_ids) e = __shfl(my_e[r], slot[u] & 63, kWave);
+                            w[u] = static_cast<int>(wbase[ok[u] ? e : 0]);
+                        }
+                    }
+#pragma unroll
+                    for (int u = 0; u < U; ++u) {
+                        if (KIND == KIND_WEIGHTED) {
+                            accumulate<VEC>(acc, d[u], ok[u] ? w[u] : 0);
+                        } else {
+                            accumulate<VEC>(acc, ok[u] ? d[u] : Gather<VEC>::zero(), 1);
+                        }
+                    }
                 }
             }
-#pragma unroll
-            for (int u = 0; u < U; ++u) accumulate<VEC>(acc, d[u], w[u]);
         }
-        my = nxt;
-        my_e = nxt_e;
-        base = nbase;
     }
 
     // fold the lane groups: afterwards lanes [0, lpe) hold the wave's column sums
@@ -212,8 +235,10 @@ __global__ __launch_bounds__(256) void spmm_kernel(const SpmmParams p) {
             f32x4* o4 = reinterpret_cast<f32x4*>(o);
 #pragma unroll
             for (int i = 0; i < 4; ++i)
-                o4[i] = f32x4{s * static_cast<float>(acc[4 * i]), s * static_cast<float>(acc[4 * i + 1]),
-                              s * static_cast<float>(acc[4 * i + 2]), s * static_cast<float>(acc[4 * i + 3])};
+                __builtin_nontemporal_store(
+                    f32x4{s * static_cast<float>(acc[4 * i]), s * static_cast<float>(acc[4 * i + 1]),
+                          s * static_cast<float>(acc[4 * i + 2]), s * static_cast<float>(acc[4 * i + 3])},
+                    o4 + i);
         } else {
 #pragma unroll
             for (int i = 0; i < VEC; ++i)
@@ -236,8 +261,9 @@ static int launch_spmm(SpmmParams p, int vec, hipStream_t s) {
     p.out_vec = (reinterpret_cast<uintptr_t>(p.out) & 15) == 0 && (p.W & 3) == 0;
     const int64_t ychunks = ceil_div(p.W, 64 * vec);
     if (ychunks > 65535) return TANGO_ERR_UNSUPPORTED;
-    // high mean degree: four waves split each row; otherwise one wave per row
-    const bool wide = p.nnz >= 128 * p.rows;
+    // four waves split each row when rows are long AND wide (few neighbours per load instruction);
+    // otherwise one wave per row, which amortises the per-row latencies over more edges
+    const bool wide = p.nnz >= 128 * p.rows && p.lpe_log2 >= 4;
     const int64_t gx = wide ? p.rows : ceil_div(p.rows, 4);
     if (gx > INT32_MAX) return TANGO_ERR_UNSUPPORTED;
     const dim3 grid(static_cast<unsigned>(gx), static_cast<unsigned>(ychunks));

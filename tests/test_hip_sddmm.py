@@ -84,7 +84,7 @@ def test_unknown_op_raises(K):
         K.mySDDMM_int8(g, "add", z.float(), z, sc(1), sc(1), False)
 
 
-@pytest.mark.parametrize("H", [1, 4, 8])
+@pytest.mark.parametrize("H", [1, 3, 8, 70])
 @pytest.mark.parametrize("slope", [1.0, 0.2])
 def test_edge_softmax(K, orc, H, slope):
     rng = np.random.default_rng(H)
