@@ -18,6 +18,10 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBPS = 8000.0
+# Bytes that cross the L2 <-> fabric boundary per launch of the F=256 copy_u kernel on the default
+# benchmark graph: two rocprofv3 --pmc passes (FETCH_SIZE, then WRITE_SIZE, KiB per dispatch), each
+# scaled by what the same counter reads for a 1 GiB device copy (2.000 and 1.000).
+MEASURED_TRAFFIC_SPMM_F256 = 1.770e10
 
 
 def parse():
@@ -30,6 +34,9 @@ def parse():
     ap.add_argument("--cpu-fraction", type=float, default=1.0 / 8, help="share of rows the CPU baseline runs")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--no-primitives", action="store_true")
+    ap.add_argument("--profile-mode", choices=["spmm", "copy"], default=None,
+                    help="run only the dominant kernel (spmm: copy_u F=256 on the benchmark graph) or a "
+                         "1 GiB device copy (counter calibration), for rocprofv3 --pmc passes")
     return ap.parse_args()
 
 
@@ -234,6 +241,14 @@ def main():
     from tango_amd.util import graph_preprocess
 
     torch.cuda.set_device(0)
+    if args.profile_mode == "copy":
+        src = torch.empty(1 << 28, dtype=torch.float32, device="cuda").normal_()
+        dst = torch.empty_like(src)
+        for _ in range(5):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        print(json.dumps({"profile_mode": "copy", "bytes_read": src.numel() * 4, "bytes_written": src.numel() * 4}))
+        return
     t0 = time.perf_counter()
     g = graph_preprocess(chung_lu(args.nodes, args.edges, 2.0, seed=3, max_degree=21000, symmetric=True,
                                   device="cuda"))
@@ -242,6 +257,14 @@ def main():
     max_deg = int(g.in_degrees().max().item())
     sys.stderr.write("graph: %d nodes, %d directed edges, max in-degree %d (%.1f s)\n"
                      % (n, nnz, max_deg, time.perf_counter() - t0))
+
+    if args.profile_mode == "spmm":
+        feat = torch.randint(-127, 128, (n, 256), dtype=torch.int8, device="cuda")
+        one = torch.full((1,), 0.01, device="cuda")
+        ms = time_op(lambda: K.csr_SPMM(g, feat, one), iters=args.steps, warm=args.warmup)
+        print(json.dumps({"profile_mode": "spmm", "F": 256, "nodes": n, "edges": nnz, "avg_ms": round(ms, 4),
+                          "algorithmic_bytes": spmm_bytes(nnz, n, 256)}))
+        return
 
     gen = torch.Generator().manual_seed(5)
     X = torch.randn(n, 602, generator=gen).cuda()
@@ -280,7 +303,8 @@ def main():
     achieved = alg / k_ms / 1e6
     roofline = {"kernel": "spmm_kernel<16,4,copy_u> F=256", "bound": "hbm", "achieved": round(achieved, 1),
                 "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4),
-                "traffic": None, "avg_launch_ms": round(k_ms, 4), "algorithmic_bytes": alg,
+                "traffic": MEASURED_TRAFFIC_SPMM_F256 if (args.nodes, args.edges) == (232965, 114_600_000) else None,
+                "avg_launch_ms": round(k_ms, 4), "algorithmic_bytes": alg,
                 "launches_timed": len(timer.spans.get("spmm_F256", []))}
 
     result = {
