@@ -166,43 +166,45 @@ __global__ __launch_bounds__(256) void spmm_kernel(const SpmmParams p) {
             if (KIND == KIND_WEIGHTED && p.edge_ids)
                 my_e[r] = static_cast<int>(__builtin_nontemporal_load(p.edge_ids + qc));
         }
+        // The 256 slots are walked as one flat sequence of steps (64 / lpe slots each), always
+        // U steps per batch, so narrow rows (one step per 64 slots) keep U gathers in flight too.
+        const int cnt = static_cast<int>((end - base) < 4 * kWave ? (end - base) : 4 * kWave);
+        const int total = (cnt + epi - 1) >> sh;
+        for (int t = 0; t < total; t += U) {
+            int j[U], sl[U];
 #pragma unroll
-        for (int r = 0; r < 4; ++r) {
-            const int64_t cbase = base + r * kWave;
-            if (cbase < end) {  // uniform
-                const int cnt = static_cast<int>((end - cbase) < kWave ? (end - cbase) : kWave);
-                const int steps = (cnt + epi - 1) >> sh;
-                for (int t = 0; t < steps; t += U) {
-                    int j[U];
-                    int slot[U];
+            for (int u = 0; u < U; ++u) {
+                const int tt = t + u;
+                const int r = (tt >> p.lpe_log2) & 3;  // which of the four index registers (wave-uniform)
+                sl[u] = ((tt & (lpe - 1)) << sh) + grp;
+                const int reg = r == 0 ? my[0] : r == 1 ? my[1] : r == 2 ? my[2] : my[3];
+                j[u] = __shfl(reg, sl[u], kWave);
+                if (KIND == KIND_WEIGHTED) {
+                    const int rege = r == 0 ? my_e[0] : r == 1 ? my_e[1] : r == 2 ? my_e[2] : my_e[3];
+                    // position of this slot's edge value: permuted id, or the CSR slot itself
+                    sl[u] = p.edge_ids ? __shfl(rege, sl[u], kWave) : static_cast<int>(base - start) + r * kWave + sl[u];
+                }
+            }
+            typename Gather<VEC>::T d[U];
+            int w[U];
+            bool ok[U];
 #pragma unroll
-                    for (int u = 0; u < U; ++u) {
-                        slot[u] = ((t + u) << sh) + grp;  // wraps past the chunk for t + u >= steps: masked below
-                        j[u] = __shfl(my[r], slot[u] & 63, kWave);
-                    }
-                    typename Gather<VEC>::T d[U];
-                    int w[U];
-                    bool ok[U];
+            for (int u = 0; u < U; ++u) {
+                ok[u] = (t + u) < total && j[u] >= 0;
+                // invalid slots read row 0 and are zeroed afterwards: no branch around the load
+                d[u] = Gather<VEC>::load(fcol + static_cast<int64_t>(ok[u] ? j[u] : 0) * p.ldf);
+                w[u] = 1;
+                if (KIND == KIND_WEIGHTED) {
+                    const int64_t e = p.edge_ids ? static_cast<int64_t>(sl[u]) : start + sl[u];
+                    w[u] = static_cast<int>(wbase[ok[u] ? e : 0]);
+                }
+            }
 #pragma unroll
-                    for (int u = 0; u < U; ++u) {
-                        ok[u] = (t + u) < steps && j[u] >= 0;
-                        // invalid slots read row 0 and are zeroed afterwards: no branch around the load
-                        d[u] = Gather<VEC>::load(fcol + static_cast<int64_t>(ok[u] ? j[u] : 0) * p.ldf);
-                        w[u] = 1;
-                        if (KIND == KIND_WEIGHTED) {
-                            int64_t e = cbase + (slot[u] & 63);
-                            if (p.edge_ids) e = __shfl(my_e[r], slot[u] & 63, kWave);
-                            w[u] = static_cast<int>(wbase[ok[u] ? e : 0]);
-                        }
-                    }
-#pragma unroll
-                    for (int u = 0; u < U; ++u) {
-                        if (KIND == KIND_WEIGHTED) {
-                            accumulate<VEC>(acc, d[u], ok[u] ? w[u] : 0);
-                        } else {
-                            accumulate<VEC>(acc, ok[u] ? d[u] : Gather<VEC>::zero(), 1);
-                        }
-                    }
+            for (int u = 0; u < U; ++u) {
+                if (KIND == KIND_WEIGHTED) {
+                    accumulate<VEC>(acc, d[u], ok[u] ? w[u] : 0);
+                } else {
+                    accumulate<VEC>(acc, ok[u] ? d[u] : Gather<VEC>::zero(), 1);
                 }
             }
         }
