@@ -72,6 +72,27 @@ __device__ __forceinline__ void block_absmax_to_global(float v, float* out) {
 // 1/s with the convention that an all-zero tensor (s == 0) quantizes to zeros.
 __device__ __forceinline__ float rscale_of(float s) { return s > 0.0f ? 1.0f / s : 0.0f; }
 
+// fp32 -> int8 rounding shared by the quantize kernels and the GEMM's fused quantize.
+template <int MODE>
+__device__ __forceinline__ int quant_one(float x, float r, float u) {
+    const float p = x * r;
+    float v;
+    if (MODE == TANGO_ROUND_RNE)
+        v = rintf(p);
+    else if (MODE == TANGO_ROUND_TRUNC)
+        v = truncf(p);
+    else
+        v = floorf(p + u);
+    // fmaxf/fminf drop a NaN operand, so a NaN input lands on a bound; map it to 0
+    v = (v == v) ? fminf(fmaxf(v, -127.0f), 127.0f) : 0.0f;
+    return static_cast<int>(v);
+}
+
+__device__ __forceinline__ uint32_t pack4(int a, int b, int c, int d) {
+    return (static_cast<uint32_t>(a) & 0xffu) | ((static_cast<uint32_t>(b) & 0xffu) << 8) |
+           ((static_cast<uint32_t>(c) & 0xffu) << 16) | (static_cast<uint32_t>(d) << 24);
+}
+
 // Sets a handful of 32-bit words.  Used instead of hipMemsetAsync so that a
 // caller may capture any entry point into a HIP graph.
 static __global__ void fill_u32_kernel(uint32_t* p, uint32_t v, int n) {

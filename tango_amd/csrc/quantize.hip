@@ -45,27 +45,6 @@ __device__ __forceinline__ float philox_uniform(uint64_t seed, uint64_t g) {
     return u01(r.v[g & 3]);
 }
 
-// ---------------------------------------------------------------- rounding
-template <int MODE>
-__device__ __forceinline__ int quant_one(float x, float r, float u) {
-    const float p = x * r;
-    float v;
-    if (MODE == TANGO_ROUND_RNE)
-        v = rintf(p);
-    else if (MODE == TANGO_ROUND_TRUNC)
-        v = truncf(p);
-    else
-        v = floorf(p + u);
-    // fmaxf/fminf drop a NaN operand, so a NaN input lands on a bound; map it to 0
-    v = (v == v) ? fminf(fmaxf(v, -127.0f), 127.0f) : 0.0f;
-    return static_cast<int>(v);
-}
-
-__device__ __forceinline__ uint32_t pack4(int a, int b, int c, int d) {
-    return (static_cast<uint32_t>(a) & 0xffu) | ((static_cast<uint32_t>(b) & 0xffu) << 8) |
-           ((static_cast<uint32_t>(c) & 0xffu) << 16) | (static_cast<uint32_t>(d) << 24);
-}
-
 // ------------------------------------------------------------------ absmax
 __global__ __launch_bounds__(256) void absmax_kernel(const float* __restrict__ x, int64_t n,
                                                      int64_t head, float* __restrict__ out) {
@@ -192,41 +171,73 @@ __global__ __launch_bounds__(256) void quantize_scalar_kernel(
     }
 }
 
-// Row-strided: one thread per output dword (4 columns of one row, padding included).
-template <int MODE>
+// Row-strided: blockDim = (64, 4); each wavefront walks one row at a time, one lane per
+// output dword (4 columns, padding included), so no per-thread index division is needed and
+// a wavefront's loads and stores are contiguous.  XV = floats per aligned load (4, 2 or 1).
+template <int MODE, int XV>
 __global__ __launch_bounds__(256) void quantize_rows_kernel(
     const float* __restrict__ x, int64_t rows, int64_t cols, int64_t ldx,
     const float* __restrict__ scale, int per_row, int8_t* __restrict__ q, int64_t ldq,
     const float* __restrict__ noise, uint64_t seed, uint64_t offset) {
     const int64_t groups = (ldq + 3) >> 2;  // dword groups per row
-    const int64_t total = rows * groups;
-    const int64_t nthr = static_cast<int64_t>(gridDim.x) * blockDim.x;
     const bool dword_ok = (ldq & 3) == 0 && (reinterpret_cast<uintptr_t>(q) & 3) == 0;
-    for (int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < total;
-         i += nthr) {
-        const int64_t row = i / groups;
-        const int64_t c0 = (i - row * groups) << 2;
+    const int64_t row_step = static_cast<int64_t>(gridDim.x) * blockDim.y;
+    for (int64_t row = static_cast<int64_t>(blockIdx.x) * blockDim.y + threadIdx.y; row < rows;
+         row += row_step) {
         const float r = rscale_of(scale[per_row ? row : 0]);
-        int v[4];
+        const float* xr = x + row * ldx;
+        int8_t* qr = q + row * ldq;
+        for (int64_t gi = threadIdx.x; gi < groups; gi += blockDim.x) {
+            const int64_t c0 = gi << 2;
+            float f[4] = {0.f, 0.f, 0.f, 0.f};
+            if (XV == 4 && c0 + 4 <= cols) {
+                const f32x4 v = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(xr + c0));
+                f[0] = v.x; f[1] = v.y; f[2] = v.z; f[3] = v.w;
+            } else if (XV == 2 && c0 + 4 <= cols) {
+                typedef float f32x2 __attribute__((ext_vector_type(2)));
+                const f32x2 v0 = __builtin_nontemporal_load(reinterpret_cast<const f32x2*>(xr + c0));
+                const f32x2 v1 = __builtin_nontemporal_load(reinterpret_cast<const f32x2*>(xr + c0 + 2));
+                f[0] = v0.x; f[1] = v0.y; f[2] = v1.x; f[3] = v1.y;
+            } else {
 #pragma unroll
-        for (int k = 0; k < 4; ++k) {
-            const int64_t c = c0 + k;
-            v[k] = 0;
-            if (c < cols) {
-                float u = 0.f;
-                const int64_t lin = row * cols + c;
-                if (MODE == TANGO_ROUND_STOCHASTIC)
-                    u = noise ? noise[lin] : philox_uniform(seed, offset + lin);
-                v[k] = quant_one<MODE>(x[row * ldx + c], r, u);
+                for (int k = 0; k < 4; ++k)
+                    if (c0 + k < cols) f[k] = xr[c0 + k];
             }
-        }
-        int8_t* qr = q + row * ldq + c0;
-        if (dword_ok) {
-            *reinterpret_cast<uint32_t*>(qr) = pack4(v[0], v[1], v[2], v[3]);
-        } else {
+            int v[4];
+            const uint64_t lin = static_cast<uint64_t>(row) * cols + c0;
+            float u[4] = {0.f, 0.f, 0.f, 0.f};
+            if (MODE == TANGO_ROUND_STOCHASTIC) {
+                if (noise) {
 #pragma unroll
-            for (int k = 0; k < 4; ++k)
-                if (c0 + k < ldq) qr[k] = static_cast<int8_t>(v[k]);
+                    for (int k = 0; k < 4; ++k)
+                        if (c0 + k < cols) u[k] = noise[lin + k];
+                } else {
+                    // the four elements touch at most two Philox blocks
+                    const uint64_t g0 = offset + lin;
+                    const uint64_t b0 = g0 >> 2;
+                    const Philox4 p0 = philox4x32_10(static_cast<uint32_t>(b0), static_cast<uint32_t>(b0 >> 32), 0u, 0u,
+                                                     static_cast<uint32_t>(seed), static_cast<uint32_t>(seed >> 32));
+                    Philox4 p1 = p0;
+                    if (g0 & 3)
+                        p1 = philox4x32_10(static_cast<uint32_t>(b0 + 1), static_cast<uint32_t>((b0 + 1) >> 32), 0u, 0u,
+                                           static_cast<uint32_t>(seed), static_cast<uint32_t>(seed >> 32));
+#pragma unroll
+                    for (int k = 0; k < 4; ++k) {
+                        const uint64_t gk = g0 + k;
+                        const Philox4& pk = ((gk >> 2) == b0) ? p0 : p1;
+                        u[k] = u01(pk.v[gk & 3]);
+                    }
+                }
+            }
+#pragma unroll
+            for (int k = 0; k < 4; ++k) v[k] = (c0 + k < cols) ? quant_one<MODE>(f[k], r, u[k]) : 0;
+            if (dword_ok) {
+                __builtin_nontemporal_store(pack4(v[0], v[1], v[2], v[3]), reinterpret_cast<uint32_t*>(qr + c0));
+            } else {
+#pragma unroll
+                for (int k = 0; k < 4; ++k)
+                    if (c0 + k < ldq) qr[c0 + k] = static_cast<int8_t>(v[k]);
+            }
         }
     }
 }
@@ -350,11 +361,21 @@ int tango_quantize_rows_f32_i8(const float* x, int64_t rows, int64_t cols, int64
         return TANGO_ERR_INVALID_ARG;
     if (rows == 0 || ldq == 0) return (round_mode >= 0 && round_mode <= 2) ? TANGO_OK : TANGO_ERR_UNSUPPORTED;
     hipStream_t s = as_stream(stream);
-    const int64_t total = rows * ((ldq + 3) >> 2);
+    const int64_t blocks = ceil_div(rows, 4);
+    const dim3 grid(static_cast<unsigned>(blocks < 256 * 16 ? blocks : 256 * 16)), block(64, 4);
+    const uintptr_t xa = reinterpret_cast<uintptr_t>(x);
+    const int xv = ((xa & 15) == 0 && (ldx & 3) == 0) ? 4 : ((xa & 7) == 0 && (ldx & 1) == 0) ? 2 : 1;
     int rc = dispatch_mode(round_mode, [&](auto mode) {
         constexpr int M = decltype(mode)::value;
-        hipLaunchKernelGGL(quantize_rows_kernel<M>, dim3(grid_for(total, 256)), dim3(256), 0, s, x,
-                           rows, cols, ldx, scale, per_row, q, ldq, noise, seed, offset);
+        if (xv == 4)
+            hipLaunchKernelGGL((quantize_rows_kernel<M, 4>), grid, block, 0, s, x, rows, cols, ldx, scale,
+                               per_row, q, ldq, noise, seed, offset);
+        else if (xv == 2)
+            hipLaunchKernelGGL((quantize_rows_kernel<M, 2>), grid, block, 0, s, x, rows, cols, ldx, scale,
+                               per_row, q, ldq, noise, seed, offset);
+        else
+            hipLaunchKernelGGL((quantize_rows_kernel<M, 1>), grid, block, 0, s, x, rows, cols, ldx, scale,
+                               per_row, q, ldq, noise, seed, offset);
     });
     return rc != TANGO_OK ? rc : launch_status();
 }
