@@ -134,8 +134,10 @@ __global__ __launch_bounds__(256, 2) void gemm_nt_kernel(const NtParams p) {
                 for (int j = 0; j < NT; ++j) {
                     const int n = j * 16 + r16;
                     const i32x4 b = ldsB[buf][n * 4 + (g ^ ((n >> 1) & 3))];
-                    acc[0][j] = mfma_16x16x64(a[s][0], b, acc[0][j]);
-                    acc[1][j] = mfma_16x16x64(a[s][1], b, acc[1][j]);
+                    // operands swapped (C^T = B A^T): the lane then holds four CONSECUTIVE columns
+                    // of one output row, which makes the epilogue's stores 16 bytes wide
+                    acc[0][j] = mfma_16x16x64(b, a[s][0], acc[0][j]);
+                    acc[1][j] = mfma_16x16x64(b, a[s][1], acc[1][j]);
                 }
                 load_a(a[s], step + PF);
                 store_b(breg, buf ^ 1);
@@ -144,25 +146,37 @@ __global__ __launch_bounds__(256, 2) void gemm_nt_kernel(const NtParams p) {
         }
     }
 
-    // epilogue: lane holds C[row0 + 16 i + 4 g + v][n0 + 16 j + r16]
+    // epilogue: lane holds C[row0 + 16 i + r16][n0 + 16 j + 4 g + v], v = 0..3
     const float s = p.sA[0] * p.sB[0];
     float m = 0.0f;
+    const uintptr_t ca = reinterpret_cast<uintptr_t>(p.C);
+    const int wide = ((ca & 15) == 0 && (p.ldc & 3) == 0) ? 4 : ((ca & 7) == 0 && (p.ldc & 1) == 0) ? 2 : 1;
 #pragma unroll
-    for (int j = 0; j < NT; ++j) {
-        const int64_t col = n0 + j * 16 + r16;
-        if (col < p.N) {
-            const float bv = p.bias ? p.bias[col] : 0.0f;
+    for (int i = 0; i < 2; ++i) {
+        const int64_t row = row0 + i * 16 + r16;
+        if (row < p.M) {
+            float* crow = p.C + row * p.ldc;
 #pragma unroll
-            for (int i = 0; i < 2; ++i) {
+            for (int j = 0; j < NT; ++j) {
+                const int64_t col = n0 + j * 16 + g * 4;
+                float y[4];
 #pragma unroll
                 for (int v = 0; v < 4; ++v) {
-                    const int64_t row = row0 + i * 16 + g * 4 + v;
-                    if (row < p.M) {
-                        float y = s * static_cast<float>(acc[i][j][v]);
-                        if (p.bias) y = bv + y;
-                        p.C[row * p.ldc + col] = y;
-                        m = fmaxf(m, fabsf(y));
-                    }
+                    y[v] = s * static_cast<float>(acc[i][j][v]);
+                    if (p.bias && col + v < p.N) y[v] = p.bias[col + v] + y[v];
+                    if (col + v < p.N) m = fmaxf(m, fabsf(y[v]));
+                }
+                if (col + 4 <= p.N && wide == 4) {
+                    __builtin_nontemporal_store(f32x4{y[0], y[1], y[2], y[3]}, reinterpret_cast<f32x4*>(crow + col));
+                } else if (col + 4 <= p.N && wide == 2) {
+                    typedef float f32x2 __attribute__((ext_vector_type(2)));
+                    // plain stores: these half-aligned pieces rely on L2 to merge them into full lines
+                    *reinterpret_cast<f32x2*>(crow + col) = f32x2{y[0], y[1]};
+                    *reinterpret_cast<f32x2*>(crow + col + 2) = f32x2{y[2], y[3]};
+                } else {
+#pragma unroll
+                    for (int v = 0; v < 4; ++v)
+                        if (col + v < p.N) crow[col + v] = y[v];
                 }
             }
         }
