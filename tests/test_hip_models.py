@@ -1,0 +1,87 @@
+"""GPU tests of the GAT / HGT layer harness: forward and gradients track an fp32
+torch implementation of the same math within int8 quantization error."""
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+
+def rel_err(a, b):
+    return (a - b).norm().item() / max(b.norm().item(), 1e-30)
+
+
+def softmax_dst(e, dst, n):
+    mx = torch.full((n,) + e.shape[1:], -1e30, device=e.device).scatter_reduce(
+        0, dst.view(-1, *([1] * (e.dim() - 1))).expand_as(e), e, "amax")
+    ex = torch.exp(e - mx[dst])
+    return ex / torch.zeros((n,) + e.shape[1:], device=e.device).index_add(0, dst, ex)[dst]
+
+
+@pytest.fixture(scope="module")
+def graph():
+    from tango_amd.graph import chung_lu
+    from tango_amd.util import graph_preprocess
+    return graph_preprocess(chung_lu(3000, 30000, 2.2, seed=4, device="cuda"))
+
+
+def test_gat_layer_tracks_fp32(graph):
+    from tango_amd.gat import QGATConv
+    g = graph
+    n, H, D = g.num_nodes(), 8, 16
+    torch.manual_seed(0)
+    layer = QGATConv(96, D, H, residual=True, activation=None).cuda()
+    x = torch.randn(n, 96, device="cuda", requires_grad=True)
+    out, attn = layer(g, x, get_attention=True)
+    assert tuple(out.shape) == (n, H, D) and tuple(attn.shape) == (g.num_edges(), H, 1)
+    src, dst = g.coo
+    sums = torch.zeros(n, H, 1, device="cuda").index_add(0, dst, attn)
+    assert torch.allclose(sums, torch.ones_like(sums), atol=1e-5)
+    # fp32 reference of the same layer
+    xr = x.detach().clone().requires_grad_(True)
+    fs = torch.nn.functional.linear(xr, layer.fc.weight).view(n, H, D)
+    el = (fs * layer.attn_l).sum(-1, keepdim=True)
+    er = (fs * layer.attn_r).sum(-1, keepdim=True)
+    a = softmax_dst(torch.nn.functional.leaky_relu(el[src] + er[dst], 0.2), dst, n)
+    ref = torch.zeros(n, H, D, device="cuda").index_add(0, dst, fs[src] * a)
+    ref = ref + torch.nn.functional.linear(xr, layer.res_fc.weight).view(n, H, D) + layer.bias.view(1, H, D)
+    assert rel_err(out.detach(), ref.detach()) < 0.06
+    w = torch.randn_like(out)
+    out.backward(w)
+    gq = [p.grad.clone() for p in layer.parameters()] + [x.grad.clone()]
+    layer.zero_grad()
+    ref.backward(w)
+    gr = [p.grad.clone() for p in layer.parameters()] + [xr.grad]
+    names = [k for k, _ in layer.named_parameters()] + ["x"]
+    # gradients that pass through the int8-quantized attention logits (attn_l / attn_r) carry the
+    # per-tensor quantization noise of a heavy-tailed tensor; direction must agree, magnitude roughly
+    cos = {k: round(torch.nn.functional.cosine_similarity(a_.flatten(), b_.flatten(), dim=0).item(), 4)
+           for k, a_, b_ in zip(names, gq, gr)}
+    errs = {k: round(rel_err(a_, b_), 4) for k, a_, b_ in zip(names, gq, gr)}
+    assert all(v > 0.93 for v in cos.values()), (cos, errs)
+    assert all(errs[k] < 0.2 for k in ("fc.weight", "res_fc.weight", "bias", "x")), errs
+
+
+def test_hgt_layer_runs_and_tracks_fp32(graph):
+    from tango_amd.gat import HGTLayer
+    g = graph
+    n = g.num_nodes()
+    torch.manual_seed(1)
+    layer = HGTLayer(64, 64, 4).cuda()
+    x = torch.randn(n, 64, device="cuda", requires_grad=True)
+    out = layer(g, x)
+    assert tuple(out.shape) == (n, 64) and torch.isfinite(out).all()
+    src, dst = g.coo
+    lin = torch.nn.functional.linear
+    xr = x.detach().clone().requires_grad_(True)
+    k = lin(lin(xr, layer.k_linear.weight, layer.k_linear.bias), layer.attn_linear.weight, layer.attn_linear.bias).view(n, 4, 16)
+    v = lin(lin(xr, layer.v_linear.weight, layer.v_linear.bias), layer.msg_linear.weight, layer.msg_linear.bias).view(n, 4, 16)
+    q = lin(xr, layer.q_linear.weight, layer.q_linear.bias).view(n, 4, 16)
+    t = (k[src] * q[dst]).sum(-1, keepdim=True) / 4.0
+    a = softmax_dst(t, dst, n)
+    ref = lin(torch.zeros(n, 4, 16, device="cuda").index_add(0, dst, v[src] * a).reshape(n, 64),
+              layer.a_linear.weight, layer.a_linear.bias)
+    assert rel_err(out.detach(), ref.detach()) < 0.1
+    out.sum().backward()
+    assert all(p.grad is not None and torch.isfinite(p.grad).all() for p in layer.parameters())
+    assert torch.isfinite(x.grad).all()
