@@ -75,6 +75,25 @@ int tango_quantize_rows_f32_i8(const float* x, int64_t rows, int64_t cols, int64
                                int round_mode, const float* noise, uint64_t seed,
                                uint64_t offset, tango_stream_t stream);
 
+/* Fused forms of the two calls above for a layer's glue (no counterpart in the
+   reference, whose drivers run these steps as separate torch passes,
+   evaluation/test_gcn.py:86-94,123-137): every element is first multiplied by
+   row_mul[r] (when non-null; one fp32 rounding) and replaced by zero where
+   mask[r, c] (row stride ldm) is not positive (when non-null).
+   tango_absmax_ex_f32 writes scale_out[0] = max|x*row_mul| / 127 over unmasked
+   elements and, when colsum_out is non-null, colsum_out[c] = sum_r of the
+   unmasked x[r, c] (not multiplied), reduced in a fixed order.  cols <= 1024.
+   workspace: tango_absmax_ex_workspace(rows, cols, colsum_out != NULL) bytes. */
+size_t tango_absmax_ex_workspace(int64_t rows, int64_t cols, int want_colsum);
+int tango_absmax_ex_f32(const float* x, int64_t rows, int64_t cols, int64_t ldx, const float* row_mul,
+                        const float* mask, int64_t ldm, float* scale_out, float* colsum_out,
+                        void* workspace, size_t workspace_bytes, tango_stream_t stream);
+int tango_quantize_rows_ex_f32_i8(const float* x, int64_t rows, int64_t cols, int64_t ldx,
+                                  const float* row_mul, const float* mask, int64_t ldm,
+                                  const float* scale, int per_row, int8_t* q, int64_t ldq,
+                                  int round_mode, const float* noise, uint64_t seed,
+                                  uint64_t offset, tango_stream_t stream);
+
 /* transpose_quant (cuda/src/cuda.cpp:27-33 -> transpose_quant_impl,
    quantization.cu:95-167): x[nrow, ncol] fp32 -> out[ncol, nrow] int8,
    half-to-even, clamped to +-127. */
@@ -104,6 +123,15 @@ int tango_qgemm_fwd(float* Y, int64_t ldy, const float* X, int64_t ldx, int8_t* 
                     int round_mode, void* workspace, size_t workspace_bytes,
                     tango_stream_t stream);
 
+/* As tango_qgemm_fwd, with row m of X multiplied by x_row_mul[m] before it is
+   quantized (the "feat * out_deg^-1/2" of evaluation/test_gcn.py:86-94 folded
+   into the quantize pass; scaleX must then be the scale of the multiplied X). */
+int tango_qgemm_fwd_ex(float* Y, int64_t ldy, const float* X, int64_t ldx, const float* x_row_mul,
+                       int8_t* Xq, int64_t ldxq, const float* W, int64_t ldw, int8_t* Wq,
+                       const float* bias, float* scaleY, const float* scaleX, const float* scaleW,
+                       int64_t M, int64_t N, int64_t K, int round_mode, void* workspace,
+                       size_t workspace_bytes, tango_stream_t stream);
+
 /* Integer GEMM on operands that are already int8 (no counterpart in the
    reference, whose forward always re-quantizes; same epilogue as above):
    Y[m,n] = (sA*sB) * float(sum_k A[m,k]*B[n,k]) (+ bias[n]), optional scaleY. */
@@ -120,6 +148,13 @@ int tango_qgemm_bwd_dx(float* dX, int64_t lddx, const int8_t* dYq, int64_t lddy,
                        const int8_t* Wq, int64_t ldw, const float* s_dY, const float* s_W,
                        int64_t M, int64_t N, int64_t K, void* workspace, size_t workspace_bytes,
                        tango_stream_t stream);
+
+/* As tango_qgemm_bwd_dx, with row m of the result multiplied by row_scale[m]
+   (the backward of the folded row multiplier above). */
+int tango_qgemm_bwd_dx_ex(float* dX, int64_t lddx, const int8_t* dYq, int64_t lddy,
+                          const int8_t* Wq, int64_t ldw, const float* s_dY, const float* s_W,
+                          const float* row_scale, int64_t M, int64_t N, int64_t K, void* workspace,
+                          size_t workspace_bytes, tango_stream_t stream);
 
 /* QGEMM_backward_gradW (cuda/src/cuda.cpp:100-108 -> QGEMM_backward.cu:50-113):
    dW[N,K] = (s_dY*s_X) * float(sum_m dYq[m,n] * Xq[m,k]), int32 accumulation.
@@ -150,6 +185,15 @@ int tango_qgemm_legacy(float* C, const float* A, const float* B, int64_t m, int6
 int tango_spmm_csr_copy_u(float* out, const int64_t* indptr, const int64_t* indices,
                           const int8_t* feat, int64_t ldf, const float* scale, int64_t rows,
                           int64_t num_src, int64_t nnz, int64_t F, tango_stream_t stream);
+
+/* As tango_spmm_csr_copy_u with the layer glue that follows the aggregation in
+   evaluation/test_gcn.py:123-137 folded into the epilogue, in this order and with
+   one fp32 rounding each: y = scale * float(sum); y *= row_scale[r] (if non-null);
+   y += bias[f] (if non-null); y = max(y, 0) (if relu). */
+int tango_spmm_csr_copy_u_ex(float* out, const int64_t* indptr, const int64_t* indices,
+                             const int8_t* feat, int64_t ldf, const float* scale,
+                             const float* row_scale, const float* bias, int relu, int64_t rows,
+                             int64_t num_src, int64_t nnz, int64_t F, tango_stream_t stream);
 
 /* multi_cusparse_SPMM (cuda/src/cuda.cpp:119-158 -> SPMM.cu:70-194):
    out[r,h,f] = scale[0] * float(sum_p evals[h, d, e(p)] * feat[indices[p], h, f]),

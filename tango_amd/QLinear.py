@@ -48,33 +48,40 @@ class QgemmNT_func(Function):
         return grad_A, grad_B
 
 
-def _forward(ctx, X, W, b, reduce):
-    scaleX = kernels.cuda_kernels.get_scale(X if X.is_contiguous() else X.contiguous())
+def _forward(ctx, X, W, b, reduce, row_scale=None):
+    X = X if X.is_contiguous() else X.contiguous()
+    if row_scale is not None:
+        # the layer's "X * row_scale[:, None]" is folded into the quantize pass (no fp32 copy of X)
+        scaleX, _ = kernels.cuda_kernels.absmax_ex(X, row_mul=row_scale)
+    else:
+        scaleX = kernels.cuda_kernels.get_scale(X)
     scaleW = kernels.cuda_kernels.get_scale(W if W.is_contiguous() else W.contiguous())
     X_ = _padded_i8(X.size(0), X.size(1), X.device)
     W_ = torch.empty(W.shape, dtype=torch.int8, device=X.device)
-    res = kernels.QGEMM_forward(X, X_, scaleX, W, W_, scaleW, b, reduce)
-    ctx.backward_cache = X_, scaleX, W_, scaleW, b
+    res = kernels.QGEMM_forward(X, X_, scaleX, W, W_, scaleW, b, reduce, x_row_mul=row_scale)
+    ctx.backward_cache = X_, scaleX, W_, scaleW, b, row_scale
     return res
 
 
 def _backward(ctx, grad_output):
-    X_, scaleX, W_, scaleW, b = ctx.backward_cache
+    X_, scaleX, W_, scaleW, b, row_scale = ctx.backward_cache
     grad_bias = None
     dY_, scaledY = _quantize_grad(grad_output)
     grad_input, grad_weight = kernels.QGEMM_backward(
-        dY_, X_, W_, scaledY, scaleX, scaleW, ctx.needs_input_grad[0], ctx.needs_input_grad[1])
+        dY_, X_, W_, scaledY, scaleX, scaleW, ctx.needs_input_grad[0], ctx.needs_input_grad[1],
+        x_row_scale=row_scale)
     if b is not None and ctx.needs_input_grad[2]:
         grad_bias = grad_output.sum(0)
-    return grad_input, grad_weight, grad_bias
+    return grad_input, grad_weight, grad_bias, None
 
 
 class Qlinear_func(Function):
-    """cuda/QLinear.py:26-47."""
+    """cuda/QLinear.py:26-47.  ``row_scale`` (optional, [M]) multiplies the rows of X before
+    quantization, fused into the quantize pass and, in backward, into gradX's epilogue."""
 
     @staticmethod
-    def forward(ctx, X, W, b=None):
-        return _forward(ctx, X, W, b, False)
+    def forward(ctx, X, W, b=None, row_scale=None):
+        return _forward(ctx, X, W, b, False, row_scale)
 
     @staticmethod
     @once_differentiable
@@ -86,8 +93,8 @@ class Qlinear_func_reduce(Function):
     """cuda/QLinear.py:50-71: also returns the output's quantization scale."""
 
     @staticmethod
-    def forward(ctx, X, W, b=None):
-        out, scaleO = _forward(ctx, X, W, b, True)
+    def forward(ctx, X, W, b=None, row_scale=None):
+        out, scaleO = _forward(ctx, X, W, b, True, row_scale)
         ctx.mark_non_differentiable(scaleO)
         return out, scaleO
 

@@ -19,28 +19,48 @@ def _quantize_grad(t, padded):
 
 class spmm_copy_u(Function):
     """copy_u-sum aggregation (cuda/SPMM.py:8-24).  ``scaleN`` may come from the
-    preceding GEMM's epilogue, in which case no absmax pass runs here."""
+    preceding GEMM's epilogue, in which case no absmax pass runs here.
+
+    ``row_scale`` [n], ``bias`` [F] and ``relu`` fold the glue that follows the
+    aggregation in a GCN layer (evaluation/test_gcn.py:123-137: ``* in_deg^-1/2``,
+    ``+ bias``, activation) into the kernel's epilogue; the backward then masks,
+    sums the bias gradient, scales rows and quantizes in two reads of dOut."""
 
     @staticmethod
-    def forward(ctx, g, N, scaleN=None):
+    def forward(ctx, g, N, scaleN=None, row_scale=None, bias=None, relu=False):
         N = N if N.is_contiguous() else N.contiguous()
+        fused = row_scale is not None or bias is not None or relu
+        if fused and N.dim() != 2:
+            raise RuntimeError("spmm_copy_u: the fused epilogue needs 2-D features")
         if N.dim() == 2:
             N_, scaleN = quantize_padded(N, scaleN)
         else:
             N_, scaleN = quantize(N, scaleN)
-        out = csr_SPMM(g, N_, scaleN)
-        ctx.backward_cache = g
+        out = csr_SPMM(g, N_, scaleN, row_scale=row_scale, bias=bias, relu=relu)
+        ctx.backward_cache = g, row_scale, bias is not None, (out if relu else None)
         return out
 
     @staticmethod
     @once_differentiable
-    def backward(ctx, dZ):
-        g = ctx.backward_cache
-        dN = None
+    def backward(ctx, dOut):
+        g, row_scale, has_bias, mask = ctx.backward_cache
+        dN = dbias = None
+        if row_scale is None and not has_bias and mask is None:
+            if ctx.needs_input_grad[1]:
+                dZ_, scaledZ = _quantize_grad(dOut, True)
+                dN = csr_SPMM(g, dZ_, scaledZ, True)
+            return None, dN, None, None, None, None
+        dOut = dOut if dOut.is_contiguous() else dOut.contiguous()
+        want_bias = has_bias and ctx.needs_input_grad[4]
+        # dZ = (dOut where out > 0) * row_scale; its scale and the bias gradient come from one pass
+        scaledZ, dbias = cuda_kernels.absmax_ex(dOut, row_mul=row_scale, mask=mask, want_colsum=want_bias)
         if ctx.needs_input_grad[1]:
-            dZ_, scaledZ = _quantize_grad(dZ, True)
+            kw = {"round_mode": config.grad_round_mode}
+            if config.grad_round_mode == "stochastic":
+                kw.update(seed=config.seed, offset=config.next_offset())
+            dZ_, _ = quantize_padded(dOut, scaledZ, row_mul=row_scale, mask=mask, **kw)
             dN = csr_SPMM(g, dZ_, scaledZ, True)
-        return None, dN, None
+        return None, dN, None, None, dbias, None
 
 
 def _need_reduce_last_dim(ufeat, efeat):

@@ -24,18 +24,24 @@ SIGNATURES = {
     "tango_absmax_rows_f32": (I, [P, I64, I64, I64, P, P]),
     "tango_quantize_f32_i8": (I, [P, I64, P, P, I, P, U64, U64, P]),
     "tango_quantize_rows_f32_i8": (I, [P, I64, I64, I64, P, I, P, I64, I, P, U64, U64, P]),
+    "tango_absmax_ex_workspace": (SZ, [I64, I64, I]),
+    "tango_absmax_ex_f32": (I, [P, I64, I64, I64, P, P, I64, P, P, P, SZ, P]),
+    "tango_quantize_rows_ex_f32_i8": (I, [P, I64, I64, I64, P, P, I64, P, I, P, I64, I, P, U64, U64, P]),
     "tango_transpose_quant_f32_i8": (I, [P, I64, I64, P, P, P]),
     "tango_qgemm_fwd_workspace": (SZ, [I64, I64, I64]),
     "tango_qgemm_fwd": (I, [P, I64, P, I64, P, I64, P, I64, P, P, P, P, P, I64, I64, I64, I, P, SZ, P]),
+    "tango_qgemm_fwd_ex": (I, [P, I64, P, I64, P, P, I64, P, I64, P, P, P, P, P, I64, I64, I64, I, P, SZ, P]),
     "tango_qgemm_i8_nt_workspace": (SZ, [I64, I64, I64]),
     "tango_qgemm_i8_nt": (I, [P, I64, P, I64, P, I64, P, P, P, P, I64, I64, I64, P, SZ, P]),
     "tango_qgemm_bwd_dx_workspace": (SZ, [I64, I64, I64]),
     "tango_qgemm_bwd_dx": (I, [P, I64, P, I64, P, I64, P, P, I64, I64, I64, P, SZ, P]),
+    "tango_qgemm_bwd_dx_ex": (I, [P, I64, P, I64, P, I64, P, P, P, I64, I64, I64, P, SZ, P]),
     "tango_qgemm_bwd_dw_workspace": (SZ, [I64, I64, I64]),
     "tango_qgemm_bwd_dw": (I, [P, I64, P, I64, P, I64, P, P, I64, I64, I64, P, SZ, P]),
     "tango_qgemm_legacy_workspace": (SZ, [I64, I64, I64]),
     "tango_qgemm_legacy": (I, [P, P, P, I64, I64, I64, I, I, P, SZ, P]),
     "tango_spmm_csr_copy_u": (I, [P, P, P, P, I64, P, I64, I64, I64, I64, P]),
+    "tango_spmm_csr_copy_u_ex": (I, [P, P, P, P, I64, P, P, P, I, I64, I64, I64, I64, P]),
     "tango_spmm_csr_u_mul_e": (I, [P, P, P, P, P, P, P, I64, I64, I64, I64, I64, I64, P]),
     "tango_spmm_incidence": (I, [P, P, P, P, P, I64, I64, I64, I64, P]),
     "tango_sddmm_dot_i8": (I, [P, P, P, P, P, P, P, P, I64, I64, I64, P]),

@@ -52,6 +52,7 @@ struct NtParams {
     const int8_t* A;     // [M, Kr] int8, row stride lda: the tall operand
     const int8_t* B;     // [N, Kp] int8 packed: 16-byte aligned rows of stride ldb, zero-filled to Kp
     const float* bias;   // [N] or null
+    const float* row_scale;  // [M] or null: row m of the dequantized product is multiplied by it
     float* absmax_out;   // null, or receives max|C| / 127 (pre-zeroed)
     const float* sA;
     const float* sB;
@@ -156,6 +157,7 @@ __global__ __launch_bounds__(256, 2) void gemm_nt_kernel(const NtParams p) {
         const int64_t row = row0 + i * 16 + r16;
         if (row < p.M) {
             float* crow = p.C + row * p.ldc;
+            const float rsc = p.row_scale ? p.row_scale[row] : 1.0f;
 #pragma unroll
             for (int j = 0; j < NT; ++j) {
                 const int64_t col = n0 + j * 16 + g * 4;
@@ -163,6 +165,7 @@ __global__ __launch_bounds__(256, 2) void gemm_nt_kernel(const NtParams p) {
 #pragma unroll
                 for (int v = 0; v < 4; ++v) {
                     y[v] = s * static_cast<float>(acc[i][j][v]);
+                    if (p.row_scale) y[v] = y[v] * rsc;
                     if (p.bias && col + v < p.N) y[v] = p.bias[col + v] + y[v];
                     if (col + v < p.N) m = fmaxf(m, fabsf(y[v]));
                 }
@@ -414,6 +417,9 @@ using namespace tango;
 extern "C" int tango_quantize_rows_f32_i8(const float*, int64_t, int64_t, int64_t, const float*, int,
                                           int8_t*, int64_t, int, const float*, uint64_t, uint64_t,
                                           tango_stream_t);
+extern "C" int tango_quantize_rows_ex_f32_i8(const float*, int64_t, int64_t, int64_t, const float*,
+                                             const float*, int64_t, const float*, int, int8_t*, int64_t,
+                                             int, const float*, uint64_t, uint64_t, tango_stream_t);
 extern "C" int tango_absmax_f32(const float*, int64_t, float*, tango_stream_t);
 extern "C" int tango_quantize_f32_i8(const float*, int64_t, const float*, int8_t*, int, const float*, uint64_t,
                                      uint64_t, tango_stream_t);
@@ -426,7 +432,7 @@ size_t tango_qgemm_fwd_workspace(int64_t M, int64_t N, int64_t K) {
     return static_cast<size_t>(N * round_up(K, 64));
 }
 
-int tango_qgemm_fwd(float* Y, int64_t ldy, const float* X, int64_t ldx, int8_t* Xq, int64_t ldxq,
+int tango_qgemm_fwd_ex(float* Y, int64_t ldy, const float* X, int64_t ldx, const float* x_row_mul, int8_t* Xq, int64_t ldxq,
                     const float* W, int64_t ldw, int8_t* Wq, const float* bias, float* scaleY,
                     const float* scaleX, const float* scaleW, int64_t M, int64_t N, int64_t K,
                     int round_mode, void* workspace, size_t workspace_bytes,
@@ -441,7 +447,8 @@ int tango_qgemm_fwd(float* Y, int64_t ldy, const float* X, int64_t ldx, int8_t* 
     if (need > 0 && (!workspace || workspace_bytes < need)) return TANGO_ERR_WORKSPACE;
     if ((reinterpret_cast<uintptr_t>(workspace) & 15) != 0) return TANGO_ERR_INVALID_ARG;
     hipStream_t s = as_stream(stream);
-    int rc = tango_quantize_rows_f32_i8(X, M, K, ldx, scaleX, 0, Xq, ldxq, round_mode, nullptr, 0, 0, stream);
+    int rc = tango_quantize_rows_ex_f32_i8(X, M, K, ldx, x_row_mul, nullptr, 0, scaleX, 0, Xq, ldxq, round_mode,
+                                           nullptr, 0, 0, stream);
     if (rc != TANGO_OK) return rc;
     rc = tango_quantize_rows_f32_i8(W, N, K, ldw, scaleW, 0, Wq, K, round_mode, nullptr, 0, 0, stream);
     if (rc != TANGO_OK) return rc;
@@ -455,6 +462,15 @@ int tango_qgemm_fwd(float* Y, int64_t ldy, const float* X, int64_t ldx, int8_t* 
     p.C = Y; p.A = Xq; p.B = Bp; p.bias = bias; p.absmax_out = scaleY; p.sA = scaleX; p.sB = scaleW;
     p.M = M; p.N = N; p.Kr = K; p.lda = ldxq; p.ldb = ldb; p.ldc = ldy;
     return launch_nt(p, s);
+}
+
+int tango_qgemm_fwd(float* Y, int64_t ldy, const float* X, int64_t ldx, int8_t* Xq, int64_t ldxq,
+                    const float* W, int64_t ldw, int8_t* Wq, const float* bias, float* scaleY,
+                    const float* scaleX, const float* scaleW, int64_t M, int64_t N, int64_t K,
+                    int round_mode, void* workspace, size_t workspace_bytes,
+                    tango_stream_t stream) {
+    return tango_qgemm_fwd_ex(Y, ldy, X, ldx, nullptr, Xq, ldxq, W, ldw, Wq, bias, scaleY, scaleX, scaleW, M, N,
+                              K, round_mode, workspace, workspace_bytes, stream);
 }
 
 size_t tango_qgemm_i8_nt_workspace(int64_t M, int64_t N, int64_t K) {
@@ -491,8 +507,9 @@ size_t tango_qgemm_bwd_dx_workspace(int64_t M, int64_t N, int64_t K) {
     return static_cast<size_t>(K * round_up(N, 64));
 }
 
-int tango_qgemm_bwd_dx(float* dX, int64_t lddx, const int8_t* dYq, int64_t lddy,
-                       const int8_t* Wq, int64_t ldw, const float* s_dY, const float* s_W,
+int tango_qgemm_bwd_dx_ex(float* dX, int64_t lddx, const int8_t* dYq, int64_t lddy,
+                          const int8_t* Wq, int64_t ldw, const float* s_dY, const float* s_W,
+                          const float* row_scale,
                        int64_t M, int64_t N, int64_t K, void* workspace, size_t workspace_bytes,
                        tango_stream_t stream) {
     if (M < 0 || N < 0 || K < 0 || !s_dY || !s_W || lddx < K || lddy < N || ldw < K)
@@ -510,9 +527,17 @@ int tango_qgemm_bwd_dx(float* dX, int64_t lddx, const int8_t* dYq, int64_t lddy,
         hipLaunchKernelGGL(transpose_pack_i8_kernel, dim3(grid_for(K * ldt, 256)), dim3(256), 0, s, Wt,
                            ldt, Wq, ldw, N, K);
     NtParams p{};
-    p.C = dX; p.A = dYq; p.B = Wt; p.sA = s_dY; p.sB = s_W;
+    p.C = dX; p.A = dYq; p.B = Wt; p.sA = s_dY; p.sB = s_W; p.row_scale = row_scale;
     p.M = M; p.N = K; p.Kr = N; p.lda = lddy; p.ldb = ldt; p.ldc = lddx;
     return launch_nt(p, s);
+}
+
+int tango_qgemm_bwd_dx(float* dX, int64_t lddx, const int8_t* dYq, int64_t lddy,
+                       const int8_t* Wq, int64_t ldw, const float* s_dY, const float* s_W,
+                       int64_t M, int64_t N, int64_t K, void* workspace, size_t workspace_bytes,
+                       tango_stream_t stream) {
+    return tango_qgemm_bwd_dx_ex(dX, lddx, dYq, lddy, Wq, ldw, s_dY, s_W, nullptr, M, N, K, workspace,
+                                 workspace_bytes, stream);
 }
 
 size_t tango_qgemm_bwd_dw_workspace(int64_t M, int64_t N, int64_t K) {

@@ -178,7 +178,8 @@ template <int MODE, int XV>
 __global__ __launch_bounds__(256) void quantize_rows_kernel(
     const float* __restrict__ x, int64_t rows, int64_t cols, int64_t ldx,
     const float* __restrict__ scale, int per_row, int8_t* __restrict__ q, int64_t ldq,
-    const float* __restrict__ noise, uint64_t seed, uint64_t offset) {
+    const float* __restrict__ noise, uint64_t seed, uint64_t offset,
+    const float* __restrict__ row_mul, const float* __restrict__ mask, int64_t ldm) {
     const int64_t groups = (ldq + 3) >> 2;  // dword groups per row
     const bool dword_ok = (ldq & 3) == 0 && (reinterpret_cast<uintptr_t>(q) & 3) == 0;
     const int64_t row_step = static_cast<int64_t>(gridDim.x) * blockDim.y;
@@ -202,6 +203,16 @@ __global__ __launch_bounds__(256) void quantize_rows_kernel(
 #pragma unroll
                 for (int k = 0; k < 4; ++k)
                     if (c0 + k < cols) f[k] = xr[c0 + k];
+            }
+            if (row_mul) {  // x * row_mul[row], one rounding, before quantization
+                const float rm = row_mul[row];
+#pragma unroll
+                for (int k = 0; k < 4; ++k) f[k] = f[k] * rm;
+            }
+            if (mask) {  // elements whose mask value is not positive quantize to zero
+#pragma unroll
+                for (int k = 0; k < 4; ++k)
+                    if (c0 + k < cols && !(mask[row * ldm + c0 + k] > 0.0f)) f[k] = 0.0f;
             }
             int v[4];
             const uint64_t lin = static_cast<uint64_t>(row) * cols + c0;
@@ -274,6 +285,64 @@ __global__ __launch_bounds__(256) void transpose_quant_kernel(const float* __res
     }
 }
 
+// max |x[r,c] * row_mul[r]| over unmasked elements, and optionally the column sums of the
+// unmasked x (not multiplied): the two reductions of a fused "mask, sum for the bias gradient,
+// scale rows, quantize" backward step in one read of x.  blockDim = (64, 4), a wavefront walks
+// rows; lane l owns columns 4 l .. 4 l + 3 (+ 256 t).  Column sums are written as one partial
+// row per wavefront and reduced in a fixed order afterwards, so they are deterministic.
+template <int T>
+__global__ __launch_bounds__(256) void absmax_ex_kernel(
+    const float* __restrict__ x, int64_t rows, int64_t cols, int64_t ldx,
+    const float* __restrict__ row_mul, const float* __restrict__ mask, int64_t ldm,
+    float* __restrict__ scale_out, float* __restrict__ partial /* [gridDim.x * 4, cols] or null */) {
+    float m = 0.0f;
+    float cs[T][4];
+#pragma unroll
+    for (int t = 0; t < T; ++t)
+#pragma unroll
+        for (int k = 0; k < 4; ++k) cs[t][k] = 0.0f;
+    const int64_t row_step = static_cast<int64_t>(gridDim.x) * blockDim.y;
+    for (int64_t row = static_cast<int64_t>(blockIdx.x) * blockDim.y + threadIdx.y; row < rows;
+         row += row_step) {
+        const float rm = row_mul ? row_mul[row] : 1.0f;
+        const float* xr = x + row * ldx;
+#pragma unroll
+        for (int t = 0; t < T; ++t) {
+            const int64_t c0 = (static_cast<int64_t>(threadIdx.x) + 64 * t) << 2;
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+                if (c0 + k < cols) {
+                    float v = xr[c0 + k];
+                    if (mask && !(mask[row * ldm + c0 + k] > 0.0f)) v = 0.0f;
+                    cs[t][k] += v;
+                    m = fmaxf(m, fabsf(row_mul ? v * rm : v));
+                }
+            }
+        }
+    }
+    if (partial) {
+        float* prow = partial + (static_cast<int64_t>(blockIdx.x) * blockDim.y + threadIdx.y) * cols;
+#pragma unroll
+        for (int t = 0; t < T; ++t) {
+            const int64_t c0 = (static_cast<int64_t>(threadIdx.x) + 64 * t) << 2;
+#pragma unroll
+            for (int k = 0; k < 4; ++k)
+                if (c0 + k < cols) prow[c0 + k] = cs[t][k];
+        }
+    }
+    block_absmax_to_global(m / 127.0f, scale_out);
+}
+
+__global__ __launch_bounds__(256) void colsum_finish_kernel(const float* __restrict__ partial,
+                                                            int64_t nrows, int64_t cols,
+                                                            float* __restrict__ out) {
+    const int64_t c = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (c >= cols) return;
+    float s = 0.0f;
+    for (int64_t r = 0; r < nrows; ++r) s += partial[r * cols + c];
+    out[c] = s;
+}
+
 template <typename F>
 static int dispatch_mode(int mode, F&& f) {
     switch (mode) {
@@ -332,6 +401,45 @@ int tango_absmax_rows_f32(const float* x, int64_t rows, int64_t cols, int64_t ld
     return launch_status();
 }
 
+static int absmax_ex_grid(int64_t rows) {
+    const int64_t blocks = ceil_div(rows, 4);
+    return static_cast<int>(blocks < 1024 ? (blocks < 1 ? 1 : blocks) : 1024);
+}
+
+size_t tango_absmax_ex_workspace(int64_t rows, int64_t cols, int want_colsum) {
+    if (!want_colsum || rows <= 0 || cols <= 0) return 0;
+    return static_cast<size_t>(absmax_ex_grid(rows)) * 4 * static_cast<size_t>(cols) * sizeof(float);
+}
+
+int tango_absmax_ex_f32(const float* x, int64_t rows, int64_t cols, int64_t ldx, const float* row_mul,
+                        const float* mask, int64_t ldm, float* scale_out, float* colsum_out,
+                        void* workspace, size_t workspace_bytes, tango_stream_t stream) {
+    if (rows < 0 || cols < 0 || ldx < cols || !scale_out || (rows * cols > 0 && !x) || (mask && ldm < cols))
+        return TANGO_ERR_INVALID_ARG;
+    if (cols > 1024) return TANGO_ERR_UNSUPPORTED;
+    hipStream_t s = as_stream(stream);
+    fill_u32(scale_out, 0u, 1, s);
+    const int grid = absmax_ex_grid(rows);
+    float* partial = nullptr;
+    if (colsum_out) {
+        const size_t need = tango_absmax_ex_workspace(rows > 0 ? rows : 1, cols, 1);
+        if (cols > 0 && (!workspace || workspace_bytes < need)) return TANGO_ERR_WORKSPACE;
+        partial = static_cast<float*>(workspace);
+    }
+    if (cols == 0) return launch_status();
+    const dim3 block(64, 4);
+    const int T = static_cast<int>(ceil_div(cols, 256));
+#define TANGO_AEX(T_)                                                                              \
+    hipLaunchKernelGGL((absmax_ex_kernel<T_>), dim3(grid), block, 0, s, x, rows, cols, ldx, row_mul, \
+                       mask, ldm, scale_out, partial)
+    if (T <= 1) TANGO_AEX(1); else if (T == 2) TANGO_AEX(2); else if (T == 3) TANGO_AEX(3); else TANGO_AEX(4);
+#undef TANGO_AEX
+    if (colsum_out)
+        hipLaunchKernelGGL(colsum_finish_kernel, dim3(static_cast<unsigned>(ceil_div(cols, 256))), dim3(256), 0,
+                           s, partial, static_cast<int64_t>(grid) * 4, cols, colsum_out);
+    return launch_status();
+}
+
 int tango_quantize_f32_i8(const float* x, int64_t n, const float* scale, int8_t* q,
                           int round_mode, const float* noise, uint64_t seed, uint64_t offset,
                           tango_stream_t stream) {
@@ -356,6 +464,16 @@ int tango_quantize_rows_f32_i8(const float* x, int64_t rows, int64_t cols, int64
                                const float* scale, int per_row, int8_t* q, int64_t ldq,
                                int round_mode, const float* noise, uint64_t seed,
                                uint64_t offset, tango_stream_t stream) {
+    return tango_quantize_rows_ex_f32_i8(x, rows, cols, ldx, nullptr, nullptr, 0, scale, per_row, q, ldq,
+                                         round_mode, noise, seed, offset, stream);
+}
+
+int tango_quantize_rows_ex_f32_i8(const float* x, int64_t rows, int64_t cols, int64_t ldx,
+                                  const float* row_mul, const float* mask, int64_t ldm,
+                                  const float* scale, int per_row, int8_t* q, int64_t ldq,
+                                  int round_mode, const float* noise, uint64_t seed,
+                                  uint64_t offset, tango_stream_t stream) {
+    if (mask && ldm < cols) return TANGO_ERR_INVALID_ARG;
     if (rows < 0 || cols < 0 || ldx < cols || ldq < cols || !scale ||
         (rows * cols > 0 && (!x || !q)))
         return TANGO_ERR_INVALID_ARG;
@@ -369,13 +487,13 @@ int tango_quantize_rows_f32_i8(const float* x, int64_t rows, int64_t cols, int64
         constexpr int M = decltype(mode)::value;
         if (xv == 4)
             hipLaunchKernelGGL((quantize_rows_kernel<M, 4>), grid, block, 0, s, x, rows, cols, ldx, scale,
-                               per_row, q, ldq, noise, seed, offset);
+                               per_row, q, ldq, noise, seed, offset, row_mul, mask, ldm);
         else if (xv == 2)
             hipLaunchKernelGGL((quantize_rows_kernel<M, 2>), grid, block, 0, s, x, rows, cols, ldx, scale,
-                               per_row, q, ldq, noise, seed, offset);
+                               per_row, q, ldq, noise, seed, offset, row_mul, mask, ldm);
         else
             hipLaunchKernelGGL((quantize_rows_kernel<M, 1>), grid, block, 0, s, x, rows, cols, ldx, scale,
-                               per_row, q, ldq, noise, seed, offset);
+                               per_row, q, ldq, noise, seed, offset, row_mul, mask, ldm);
     });
     return rc != TANGO_OK ? rc : launch_status();
 }

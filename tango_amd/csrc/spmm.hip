@@ -31,6 +31,9 @@ struct SpmmParams {
     const int8_t* feat;
     const int8_t* evals;
     const float* scale;
+    const float* row_scale;  // optional: out row r is multiplied by row_scale[r] after dequantization
+    const float* bias;       // optional: bias[c] added after the row scale
+    int relu;                // clamp at zero last
     int64_t rows;
     int64_t ldf;  // bytes between gathered rows
     int64_t W;    // bytes summed per gathered row (H * F)
@@ -232,19 +235,26 @@ __global__ __launch_bounds__(256) void spmm_kernel(const SpmmParams p) {
 
     if (grp == 0 && col_ok) {
         const float s = p.scale[0];
+        const float rs = p.row_scale ? p.row_scale[row] : 1.0f;
         float* o = p.out + row * p.W + col;
+        float y[VEC];
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) {
+            // same sequence of roundings as dequantize, then "* norm", "+ bias", relu as separate passes
+            y[i] = s * static_cast<float>(acc[i]);
+            if (p.row_scale) y[i] = y[i] * rs;
+            if (p.bias && col + i < p.W) y[i] = y[i] + p.bias[col + i];
+            if (p.relu) y[i] = fmaxf(y[i], 0.0f);
+        }
         if (VEC == 16 && p.out_vec && col + 16 <= p.W) {
             f32x4* o4 = reinterpret_cast<f32x4*>(o);
 #pragma unroll
             for (int i = 0; i < 4; ++i)
-                __builtin_nontemporal_store(
-                    f32x4{s * static_cast<float>(acc[4 * i]), s * static_cast<float>(acc[4 * i + 1]),
-                          s * static_cast<float>(acc[4 * i + 2]), s * static_cast<float>(acc[4 * i + 3])},
-                    o4 + i);
+                __builtin_nontemporal_store(f32x4{y[4 * i], y[4 * i + 1], y[4 * i + 2], y[4 * i + 3]}, o4 + i);
         } else {
 #pragma unroll
             for (int i = 0; i < VEC; ++i)
-                if (col + i < p.W) o[i] = s * static_cast<float>(acc[i]);
+                if (col + i < p.W) o[i] = y[i];
         }
     }
 }
@@ -306,6 +316,21 @@ int tango_spmm_csr_copy_u(float* out, const int64_t* indptr, const int64_t* indi
     if (num_src >= (1LL << 31) || nnz >= (1LL << 31)) return TANGO_ERR_UNSUPPORTED;
     SpmmParams p{};
     p.out = out; p.indptr = indptr; p.indices = indices; p.feat = feat; p.scale = scale;
+    p.rows = rows; p.ldf = ldf; p.W = F; p.F = F; p.D = 1; p.nnz = nnz;
+    return launch_spmm<KIND_COPY>(p, pick_vec(feat, ldf, F), as_stream(stream));
+}
+
+int tango_spmm_csr_copy_u_ex(float* out, const int64_t* indptr, const int64_t* indices,
+                             const int8_t* feat, int64_t ldf, const float* scale,
+                             const float* row_scale, const float* bias, int relu, int64_t rows,
+                             int64_t num_src, int64_t nnz, int64_t F, tango_stream_t stream) {
+    if (rows < 0 || F < 0 || nnz < 0 || num_src < 0 || ldf < F || !scale || !indptr ||
+        (rows * F > 0 && !out) || (nnz > 0 && (!indices || !feat)))
+        return TANGO_ERR_INVALID_ARG;
+    if (num_src >= (1LL << 31) || nnz >= (1LL << 31)) return TANGO_ERR_UNSUPPORTED;
+    SpmmParams p{};
+    p.out = out; p.indptr = indptr; p.indices = indices; p.feat = feat; p.scale = scale;
+    p.row_scale = row_scale; p.bias = bias; p.relu = relu ? 1 : 0;
     p.rows = rows; p.ldf = ldf; p.W = F; p.F = F; p.D = 1; p.nnz = nnz;
     return launch_spmm<KIND_COPY>(p, pick_vec(feat, ldf, F), as_stream(stream));
 }

@@ -12,8 +12,9 @@ class QGraphConv(nn.Module):
     """GraphConv(norm='both') with int8 GEMM and int8 aggregation
     (evaluation/test_gcn.py:26-139)."""
 
-    def __init__(self, in_feats, out_feats, bias=True, activation=None):
+    def __init__(self, in_feats, out_feats, bias=True, activation=None, fused=True):
         super().__init__()
+        self.fused = fused
         self._in_feats, self._out_feats = in_feats, out_feats
         self.weight = nn.Parameter(torch.empty(out_feats, in_feats))
         self.bias = nn.Parameter(torch.empty(out_feats)) if bias else None
@@ -23,17 +24,31 @@ class QGraphConv(nn.Module):
             nn.init.zeros_(self.bias)
 
     def forward(self, graph, feat):
-        norm_src = graph.out_degrees().float().clamp(min=1).pow(-0.5).unsqueeze(1)
-        feat_src = feat * norm_src
-        if self._in_feats > self._out_feats:
-            # multiply by W first, hand the GEMM epilogue's scale to the aggregation
-            feat_src, scale_feat = Qlinear_func_reduce.apply(feat_src, self.weight)
-            rst = spmm_copy_u.apply(graph, feat_src, scale_feat)
+        norm_src = graph.out_degrees().float().clamp(min=1).pow(-0.5)
+        norm_dst = graph.in_degrees().float().clamp(min=1).pow(-0.5)
+        relu = self._activation is torch.relu
+        if self.fused:
+            # same arithmetic as below, with every elementwise pass folded into a kernel:
+            # "* norm_src" into the quantize of the GEMM / aggregation input, "* norm_dst, + bias,
+            # relu" into the aggregation's epilogue (or "* norm_dst" into nothing when the GEMM is last)
+            if self._in_feats > self._out_feats:
+                y, sy = Qlinear_func_reduce.apply(feat, self.weight, None, norm_src)
+                rst = spmm_copy_u.apply(graph, y, sy, norm_dst, self.bias, relu)
+                if self._activation is not None and not relu:
+                    rst = self._activation(rst)
+                return rst
+            rst = spmm_copy_u.apply(graph, feat * norm_src.unsqueeze(1))
+            rst = Qlinear_func.apply(rst, self.weight) * norm_dst.unsqueeze(1)
         else:
-            rst = spmm_copy_u.apply(graph, feat_src)
-            rst = Qlinear_func.apply(rst, self.weight)
-        norm_dst = graph.in_degrees().float().clamp(min=1).pow(-0.5).unsqueeze(1)
-        rst = rst * norm_dst
+            feat_src = feat * norm_src.unsqueeze(1)
+            if self._in_feats > self._out_feats:
+                # multiply by W first, hand the GEMM epilogue's scale to the aggregation
+                feat_src, scale_feat = Qlinear_func_reduce.apply(feat_src, self.weight)
+                rst = spmm_copy_u.apply(graph, feat_src, scale_feat)
+            else:
+                rst = spmm_copy_u.apply(graph, feat_src)
+                rst = Qlinear_func.apply(rst, self.weight)
+            rst = rst * norm_dst.unsqueeze(1)
         if self.bias is not None:
             rst = rst + self.bias
         if self._activation is not None:
@@ -44,14 +59,14 @@ class QGraphConv(nn.Module):
 class GCN(nn.Module):
     """evaluation/test_gcn.py:140-169 with n_layers hidden layers after the input layer."""
 
-    def __init__(self, g, in_feats, n_hidden, n_classes, n_layers, activation, dropout):
+    def __init__(self, g, in_feats, n_hidden, n_classes, n_layers, activation, dropout, fused=True):
         super().__init__()
         self.g = g
         self.layers = nn.ModuleList()
-        self.layers.append(QGraphConv(in_feats, n_hidden, activation=activation))
+        self.layers.append(QGraphConv(in_feats, n_hidden, activation=activation, fused=fused))
         for _ in range(n_layers - 1):
-            self.layers.append(QGraphConv(n_hidden, n_hidden, activation=activation))
-        self.layers.append(QGraphConv(n_hidden, n_classes))
+            self.layers.append(QGraphConv(n_hidden, n_hidden, activation=activation, fused=fused))
+        self.layers.append(QGraphConv(n_hidden, n_classes, fused=fused))
         self.dropout = nn.Dropout(p=dropout)
 
     def forward(self, features):

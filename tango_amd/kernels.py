@@ -119,8 +119,9 @@ class cuda_kernels:
 
     @staticmethod
     def quantize_rows(out, inp, scale, per_row=False, round_mode=ROUND_RNE, noise=None, seed=0,
-                      offset=0):
-        """Row-strided quantize into a possibly wider (zero-padded) int8 matrix (not in the reference)."""
+                      offset=0, row_mul=None, mask=None):
+        """Row-strided quantize into a possibly wider (zero-padded) int8 matrix (not in the reference).
+        ``row_mul`` [rows] multiplies each row first; elements where ``mask`` <= 0 become zero."""
         _need(out, torch.int8, "out", contiguous=False)
         _need(inp, torch.float32, "in", contiguous=False)
         _need(scale, torch.float32, "scale")
@@ -132,10 +133,42 @@ class cuda_kernels:
             raise RuntimeError("quantize_rows: out must be dense")
         if noise is not None:
             _need(noise, torch.float32, "noise")
-        check(_L.tango_quantize_rows_f32_i8(_ptr(inp), inp.size(0), inp.size(1), ldx, scale.data_ptr(),
-                                            int(bool(per_row)), _ptr(out), ldq_pad, _mode(round_mode),
-                                            _ptr(noise), int(seed), int(offset), _stream()),
-              "quantize_rows")
+        ldm = 0
+        if row_mul is not None:
+            _need(row_mul, torch.float32, "row_mul")
+            if row_mul.numel() != inp.size(0):
+                raise RuntimeError("quantize_rows: row_mul must have one entry per row")
+        if mask is not None:
+            _need(mask, torch.float32, "mask", contiguous=False)
+            if tuple(mask.shape) != tuple(inp.shape):
+                raise RuntimeError("quantize_rows: mask must have in's shape")
+            ldm = _rows_view(mask, "mask")
+        check(_L.tango_quantize_rows_ex_f32_i8(_ptr(inp), inp.size(0), inp.size(1), ldx, _ptr(row_mul),
+                                               _ptr(mask), ldm, scale.data_ptr(), int(bool(per_row)),
+                                               _ptr(out), ldq_pad, _mode(round_mode), _ptr(noise),
+                                               int(seed), int(offset), _stream()), "quantize_rows")
+
+    @staticmethod
+    def absmax_ex(inp, row_mul=None, mask=None, want_colsum=False):
+        """(max|inp * row_mul| / 127 over elements with mask > 0, column sums of the unmasked inp or None)
+        in one read of a 2-D tensor (not in the reference)."""
+        _need(inp, torch.float32, "in", contiguous=False)
+        ldx = _rows_view(inp, "in")
+        rows, cols = inp.shape
+        ldm = 0
+        if row_mul is not None:
+            _need(row_mul, torch.float32, "row_mul")
+        if mask is not None:
+            _need(mask, torch.float32, "mask", contiguous=False)
+            ldm = _rows_view(mask, "mask")
+        scale = torch.empty(1, dtype=torch.float32, device=inp.device)
+        colsum = torch.empty(cols, dtype=torch.float32, device=inp.device) if want_colsum else None
+        ws_bytes = _L.tango_absmax_ex_workspace(rows, cols, int(want_colsum))
+        ws = _workspace(ws_bytes, inp.device)
+        check(_L.tango_absmax_ex_f32(_ptr(inp), rows, cols, ldx, _ptr(row_mul), _ptr(mask), ldm,
+                                     scale.data_ptr(), _ptr(colsum), _ptr(ws), ws_bytes, _stream()),
+              "absmax_ex")
+        return scale, colsum
 
     @staticmethod
     def transpose_quant(inp, scale, nrow, ncol):
@@ -150,7 +183,7 @@ class cuda_kernels:
 
     # ------------------------------------------------------------------ GEMM
     @staticmethod
-    def QGEMM_forward(Y, X, X_q, W, W_q, bias, scaleY, scaleX, scaleW, round_mode=None):
+    def QGEMM_forward(Y, X, X_q, W, W_q, bias, scaleY, scaleX, scaleW, round_mode=None, x_row_mul=None):
         for t, dt, nm in ((Y, torch.float32, "Y"), (X, torch.float32, "X"), (W, torch.float32, "W")):
             _need(t, dt, nm, contiguous=False)
         _need(X_q, torch.int8, "X_q", contiguous=False)
@@ -171,9 +204,13 @@ class cuda_kernels:
         mode = default_forward_round_mode() if round_mode is None else _mode(round_mode)
         ws_bytes = _L.tango_qgemm_fwd_workspace(M, N, K)
         ws = _workspace(ws_bytes, X.device)
-        check(_L.tango_qgemm_fwd(_ptr(Y), _rows_view(Y, "Y"), _ptr(X), _rows_view(X, "X"), _ptr(X_q),
-                                 _rows_view(X_q, "X_q"), _ptr(W), _rows_view(W, "W"), _ptr(W_q),
-                                 _ptr(bias), _ptr(scaleY),
+        if x_row_mul is not None:
+            _need(x_row_mul, torch.float32, "x_row_mul")
+            if x_row_mul.numel() != M:
+                raise RuntimeError("QGEMM_forward: x_row_mul must have M entries")
+        check(_L.tango_qgemm_fwd_ex(_ptr(Y), _rows_view(Y, "Y"), _ptr(X), _rows_view(X, "X"), _ptr(x_row_mul),
+                                    _ptr(X_q), _rows_view(X_q, "X_q"), _ptr(W), _rows_view(W, "W"), _ptr(W_q),
+                                    _ptr(bias), _ptr(scaleY),
                                  scaleX.data_ptr(), scaleW.data_ptr(), M, N, K, mode, _ptr(ws),
                                  ws_bytes, _stream()), "QGEMM_forward")
 
@@ -194,7 +231,7 @@ class cuda_kernels:
                                    scaleB.data_ptr(), M, N, K, _ptr(ws), ws_bytes, _stream()), "QGEMM_i8")
 
     @staticmethod
-    def QGEMM_backward_gradX(dX, dY, W, scaledY, scaleW):
+    def QGEMM_backward_gradX(dX, dY, W, scaledY, scaleW, row_scale=None):
         _need(dX, torch.float32, "dX", contiguous=False)
         _need(dY, torch.int8, "dY", contiguous=False)
         _need(W, torch.int8, "W", contiguous=False)
@@ -206,9 +243,12 @@ class cuda_kernels:
             raise RuntimeError("QGEMM_backward_gradX: shape mismatch")
         ws_bytes = _L.tango_qgemm_bwd_dx_workspace(M, N, K)
         ws = _workspace(ws_bytes, dY.device)
-        check(_L.tango_qgemm_bwd_dx(_ptr(dX), _rows_view(dX, "dX"), _ptr(dY), _rows_view(dY, "dY"),
-                                    _ptr(W), _rows_view(W, "W"), scaledY.data_ptr(), scaleW.data_ptr(),
-                                    M, N, K, _ptr(ws), ws_bytes, _stream()), "QGEMM_backward_gradX")
+        if row_scale is not None:
+            _need(row_scale, torch.float32, "row_scale")
+        check(_L.tango_qgemm_bwd_dx_ex(_ptr(dX), _rows_view(dX, "dX"), _ptr(dY), _rows_view(dY, "dY"),
+                                       _ptr(W), _rows_view(W, "W"), scaledY.data_ptr(), scaleW.data_ptr(),
+                                       _ptr(row_scale), M, N, K, _ptr(ws), ws_bytes, _stream()),
+              "QGEMM_backward_gradX")
 
     @staticmethod
     def QGEMM_backward_gradW(dW, dY, X, scaledY, scaleX):
@@ -257,7 +297,7 @@ class cuda_kernels:
 
     # ------------------------------------------------------------------ SpMM
     @staticmethod
-    def csr_SPMM(out, indptr, indices, U, scaleU, ldf=None, F=None):
+    def csr_SPMM(out, indptr, indices, U, scaleU, ldf=None, F=None, row_scale=None, bias=None, relu=False):
         _need(out, torch.float32, "out")
         _need(indptr, torch.int64, "indptr")
         _need(indices, torch.int64, "indices")
@@ -269,9 +309,22 @@ class cuda_kernels:
         F = width if F is None else F
         if out.numel() != rows * F:
             raise RuntimeError("csr_SPMM: out must be [%d, %d]" % (rows, F))
-        check(_L.tango_spmm_csr_copy_u(_ptr(out), indptr.data_ptr(), _ptr(indices), _ptr(U), ldf,
-                                       scaleU.data_ptr(), rows, U.size(0), indices.numel(), F,
-                                       _stream()), "csr_SPMM")
+        if row_scale is None and bias is None and not relu:
+            check(_L.tango_spmm_csr_copy_u(_ptr(out), indptr.data_ptr(), _ptr(indices), _ptr(U), ldf,
+                                           scaleU.data_ptr(), rows, U.size(0), indices.numel(), F,
+                                           _stream()), "csr_SPMM")
+            return
+        if row_scale is not None:
+            _need(row_scale, torch.float32, "row_scale")
+            if row_scale.numel() != rows:
+                raise RuntimeError("csr_SPMM: row_scale must have one entry per output row")
+        if bias is not None:
+            _need(bias, torch.float32, "bias")
+            if bias.numel() != F:
+                raise RuntimeError("csr_SPMM: bias must have F entries")
+        check(_L.tango_spmm_csr_copy_u_ex(_ptr(out), indptr.data_ptr(), _ptr(indices), _ptr(U), ldf,
+                                          scaleU.data_ptr(), _ptr(row_scale), _ptr(bias), int(bool(relu)),
+                                          rows, U.size(0), indices.numel(), F, _stream()), "csr_SPMM")
 
     @staticmethod
     def multi_cusparse_SPMM(indptr, indices, N, E_T, scale, edge_ids=None):
@@ -387,18 +440,23 @@ def quantize(t, scale=None, round_mode=ROUND_RNE, noise=None, seed=0, offset=0):
     return out, scale
 
 
-def quantize_padded(t, scale=None, round_mode=ROUND_RNE, noise=None, seed=0, offset=0, align=16):
+def quantize_padded(t, scale=None, round_mode=ROUND_RNE, noise=None, seed=0, offset=0, align=16,
+                    row_mul=None, mask=None):
     """Like ``quantize`` for a 2-D tensor, but the int8 rows are padded with
     zeros to a multiple of ``align`` bytes so that the SpMM gather and the GEMM
     fragment loads stay 16-byte aligned for odd widths (41, 602, ...).  Returns a
     [rows, cols] view of the padded buffer and the scale."""
     assert t.is_cuda and t.dim() == 2, "2-D GPU tensor expected"
     if scale is None:
-        scale = cuda_kernels.get_scale(t) if t.is_contiguous() else cuda_kernels.get_scale(t.contiguous())
+        if row_mul is not None or mask is not None:
+            scale, _ = cuda_kernels.absmax_ex(t, row_mul=row_mul, mask=mask)
+        else:
+            scale = cuda_kernels.get_scale(t) if t.is_contiguous() else cuda_kernels.get_scale(t.contiguous())
     rows, cols = t.shape
     ld = (cols + align - 1) // align * align
     buf = torch.empty((rows, ld), dtype=torch.int8, device=t.device)
-    cuda_kernels.quantize_rows(buf, t, scale, round_mode=round_mode, noise=noise, seed=seed, offset=offset)
+    cuda_kernels.quantize_rows(buf, t, scale, round_mode=round_mode, noise=noise, seed=seed, offset=offset,
+                               row_mul=row_mul, mask=mask)
     return buf[:, :cols], scale
 
 
@@ -431,7 +489,7 @@ def mySDDMM_int8(g, op, U, V, scaleU, scaleV, isReduce, reverse=False):
     return out, scale
 
 
-def QGEMM_forward(x, x_, scaleX, w, w_, scaleW, bias=None, isReduce=False, round_mode=None):
+def QGEMM_forward(x, x_, scaleX, w, w_, scaleW, bias=None, isReduce=False, round_mode=None, x_row_mul=None):
     """cuda/kernels.py:79-95."""
     assert x.is_cuda, "x must be on GPU"
     assert w.is_cuda, "w must be on GPU"
@@ -441,13 +499,13 @@ def QGEMM_forward(x, x_, scaleX, w, w_, scaleW, bias=None, isReduce=False, round
     scale_out = torch.empty_like(scaleX) if isReduce else torch.Tensor()
     bias = torch.Tensor() if bias is None else bias
     cuda_kernels.QGEMM_forward(out_fp, x, x_, w, w_, bias, scale_out, scaleX, scaleW,
-                               round_mode=round_mode)
+                               round_mode=round_mode, x_row_mul=x_row_mul)
     if isReduce:
         return out_fp, scale_out
     return out_fp
 
 
-def QGEMM_backward(dY, X, W, scaledY, scaleX, scaleW, X_need=True, W_need=True):
+def QGEMM_backward(dY, X, W, scaledY, scaleX, scaleW, X_need=True, W_need=True, x_row_scale=None):
     """cuda/kernels.py:97-111."""
     assert scaledY.is_cuda, "scaledY must be on GPU"
     assert dY.is_cuda, "dY must be on GPU"
@@ -456,7 +514,7 @@ def QGEMM_backward(dY, X, W, scaledY, scaleX, scaleW, X_need=True, W_need=True):
         assert W.is_cuda, "W must be on GPU"
         assert scaleW.is_cuda, "scaleW must be on GPU"
         dX = torch.empty(X.shape, dtype=torch.float32, device=X.device)
-        cuda_kernels.QGEMM_backward_gradX(dX, dY, W, scaledY, scaleW)
+        cuda_kernels.QGEMM_backward_gradX(dX, dY, W, scaledY, scaleW, row_scale=x_row_scale)
     if W_need:
         assert X.is_cuda, "X must be on GPU"
         assert scaleX.is_cuda, "scaleX must be on GPU"
@@ -501,8 +559,9 @@ def incidence_SPMM(g, E, scaleE, reverse=False):
     return out.view(out_shape)
 
 
-def csr_SPMM(g, N, scaleN, reverse=False):
-    """cuda/kernels.py:154-165.  N may be a 2-D view of a row-padded buffer."""
+def csr_SPMM(g, N, scaleN, reverse=False, row_scale=None, bias=None, relu=False):
+    """cuda/kernels.py:154-165.  N may be a 2-D view of a row-padded buffer.  ``row_scale`` / ``bias`` /
+    ``relu`` fold "* norm, + bias, activation" (evaluation/test_gcn.py:123-137) into the kernel's epilogue."""
     if reverse:
         indptr, indices, _ = g.adj_csr
     else:
@@ -514,9 +573,10 @@ def csr_SPMM(g, N, scaleN, reverse=False):
     if N.dim() == 2 and not N.is_contiguous():
         ld = _rows_view(N, "N")
         base = N.as_strided((N.size(0), ld), (ld, 1))
-        cuda_kernels.csr_SPMM(out, indptr, indices, base, scaleN, ldf=ld, F=dim)
+        cuda_kernels.csr_SPMM(out, indptr, indices, base, scaleN, ldf=ld, F=dim, row_scale=row_scale, bias=bias,
+                              relu=relu)
     else:
-        cuda_kernels.csr_SPMM(out, indptr, indices, N, scaleN)
+        cuda_kernels.csr_SPMM(out, indptr, indices, N, scaleN, row_scale=row_scale, bias=bias, relu=relu)
     return out.view(out_shape)
 
 

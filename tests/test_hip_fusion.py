@@ -1,0 +1,115 @@
+"""GPU tests of the layer-glue fusion: the fused prologue / epilogue entry points
+perform the same sequence of fp32 roundings as the separate passes they replace,
+so results must be bit-identical (bias gradient: summation order differs, tolerance)."""
+import numpy as np
+import pytest
+import torch
+
+from gpu_util import dev, host, rand_graph, sc
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def K():
+    from tango_amd import kernels
+    return kernels
+
+
+def make_graph(src, dst, n):
+    from tango_amd.graph import Graph
+    from tango_amd.util import graph_preprocess
+    return graph_preprocess(Graph(dev(src), dev(dst), n))
+
+
+def test_absmax_ex_and_quantize_ex(K, orc):
+    rng = np.random.default_rng(0)
+    for rows, cols in ((1000, 256), (777, 41), (300, 602), (5, 1024)):
+        x = rng.standard_normal((rows, cols)).astype(np.float32)
+        rm = rng.random(rows, dtype=np.float32) + 0.1
+        mask = rng.standard_normal((rows, cols)).astype(np.float32)
+        masked = np.where(mask > 0, x, 0).astype(np.float32)
+        scaled = (masked * rm[:, None]).astype(np.float32)
+        s, cs = K.cuda_kernels.absmax_ex(dev(x), row_mul=dev(rm), mask=dev(mask), want_colsum=True)
+        assert host(s)[0] == orc.absmax_scale(scaled)
+        assert np.allclose(host(cs), masked.astype(np.float64).sum(0), rtol=1e-5, atol=1e-3)
+        s2, none = K.cuda_kernels.absmax_ex(dev(x))
+        assert none is None and host(s2)[0] == orc.absmax_scale(x)
+        q, s3 = K.quantize_padded(dev(x), row_mul=dev(rm), mask=dev(mask))
+        assert host(s3)[0] == host(s)[0]
+        assert np.array_equal(host(q), orc.quantize(scaled, host(s)[0]))
+        q2, _ = K.quantize_padded(dev(x), s, row_mul=dev(rm), mask=dev(mask), round_mode="stochastic", seed=3, offset=64)
+        assert np.array_equal(host(q2), orc.quantize(scaled, host(s)[0], orc.STOCHASTIC, seed=3, offset=64))
+    # colsum is deterministic run to run
+    x = dev(rng.standard_normal((50000, 256)).astype(np.float32))
+    a = K.cuda_kernels.absmax_ex(x, want_colsum=True)[1]
+    b = K.cuda_kernels.absmax_ex(x, want_colsum=True)[1]
+    assert torch.equal(a, b)
+
+
+@pytest.mark.parametrize("F", [16, 41, 256])
+def test_spmm_fused_epilogue_equals_separate_passes(K, F):
+    rng = np.random.default_rng(F)
+    n, e = 600, 40000
+    src, dst = rand_graph(rng, n, e)
+    g = make_graph(src, dst, n)
+    feat = dev(rng.integers(-127, 128, (n, F)).astype(np.int8))
+    rs = dev(rng.random(n, dtype=np.float32) + 0.05)
+    bias = dev(rng.standard_normal(F).astype(np.float32))
+    s = sc(0.0173)
+    base = K.csr_SPMM(g, feat, s)
+    assert torch.equal(K.csr_SPMM(g, feat, s, row_scale=rs), base * rs.unsqueeze(1))
+    assert torch.equal(K.csr_SPMM(g, feat, s, bias=bias), base + bias)
+    assert torch.equal(K.csr_SPMM(g, feat, s, relu=True), torch.relu(base))
+    assert torch.equal(K.csr_SPMM(g, feat, s, row_scale=rs, bias=bias, relu=True),
+                       torch.relu(base * rs.unsqueeze(1) + bias))
+
+
+def test_gemm_row_scale_prologue_and_gradx_epilogue(K, orc):
+    rng = np.random.default_rng(1)
+    M, Kd, N = 700, 602, 41
+    X = rng.standard_normal((M, Kd)).astype(np.float32)
+    W = (rng.random((N, Kd), dtype=np.float32) - 0.5) * 0.2
+    rm = rng.random(M, dtype=np.float32) + 0.1
+    Xs = (X * rm[:, None]).astype(np.float32)
+    sX, _ = K.cuda_kernels.absmax_ex(dev(X), row_mul=dev(rm))
+    sW = K.cuda_kernels.get_scale(dev(W))
+    Xq = torch.empty((M, 608), dtype=torch.int8, device="cuda")[:, :Kd]
+    Wq = torch.empty((N, Kd), dtype=torch.int8, device="cuda")
+    Y, sY = K.QGEMM_forward(dev(X), Xq, sX, dev(W), Wq, sW, None, True, x_row_mul=dev(rm))
+    Yo, Xqo, _, osX, _, osY = orc.qgemm_fwd(Xs, W, reduce=True)
+    assert host(sX)[0] == osX and np.array_equal(host(Xq), Xqo) and np.array_equal(host(Y), Yo) and host(sY)[0] == osY
+    dY = rng.integers(-127, 128, (M, N)).astype(np.int8)
+    dX, _ = K.QGEMM_backward(dev(dY), Xq, Wq, sc(0.01), sX, sW, True, False, x_row_scale=dev(rm))
+    want = (orc.qgemm_bwd_dx(dY, host(Wq), 0.01, host(sW)[0]) * rm[:, None]).astype(np.float32)
+    assert np.array_equal(host(dX), want)
+
+
+@pytest.mark.parametrize("dims", [(100, 32, 7), (64, 16, 16)])
+def test_fused_gcn_matches_unfused(dims):
+    from tango_amd.gcn import GCN
+    from tango_amd.graph import chung_lu
+    from tango_amd.util import graph_preprocess
+    g = graph_preprocess(chung_lu(2500, 30000, 2.1, seed=2, symmetric=True, device="cuda"))
+    fin, hid, ncls = dims
+    torch.manual_seed(0)
+    a = GCN(g, fin, hid, ncls, 1, torch.relu, 0.0, fused=True).cuda()
+    b = GCN(g, fin, hid, ncls, 1, torch.relu, 0.0, fused=False).cuda()
+    b.load_state_dict(a.state_dict())
+    for m in (a, b):
+        for layer in m.layers:
+            torch.nn.init.normal_(layer.bias, std=0.1)
+    b.load_state_dict(a.state_dict())
+    x = torch.randn(2500, fin, device="cuda")
+    xa, xb = x.clone().requires_grad_(True), x.clone().requires_grad_(True)
+    ya, yb = a(xa), b(xb)
+    assert torch.equal(ya, yb)
+    w = torch.randn_like(ya)
+    ya.backward(w)
+    yb.backward(w)
+    assert torch.equal(xa.grad, xb.grad)
+    for (name, pa), (_, pb) in zip(a.named_parameters(), b.named_parameters()):
+        if name.endswith("bias"):
+            assert torch.allclose(pa.grad, pb.grad, rtol=1e-4, atol=1e-4), name
+        else:
+            assert torch.equal(pa.grad, pb.grad), name
