@@ -171,6 +171,26 @@ __global__ __launch_bounds__(256) void quantize_scalar_kernel(
     }
 }
 
+// Four consecutive floats of a row starting at column c0 (zero beyond `cols`), with the widest
+// aligned access the row layout allows: XV = 4 (16-byte rows), 2 (8-byte) or 1.
+template <int XV>
+__device__ __forceinline__ void load4(float* f, const float* __restrict__ row, int64_t c0, int64_t cols) {
+    f[0] = f[1] = f[2] = f[3] = 0.0f;
+    if (XV == 4 && c0 + 4 <= cols) {
+        const f32x4 v = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(row + c0));
+        f[0] = v.x; f[1] = v.y; f[2] = v.z; f[3] = v.w;
+    } else if (XV == 2 && c0 + 4 <= cols) {
+        typedef float f32x2 __attribute__((ext_vector_type(2)));
+        const f32x2 v0 = __builtin_nontemporal_load(reinterpret_cast<const f32x2*>(row + c0));
+        const f32x2 v1 = __builtin_nontemporal_load(reinterpret_cast<const f32x2*>(row + c0 + 2));
+        f[0] = v0.x; f[1] = v0.y; f[2] = v1.x; f[3] = v1.y;
+    } else {
+#pragma unroll
+        for (int k = 0; k < 4; ++k)
+            if (c0 + k < cols) f[k] = row[c0 + k];
+    }
+}
+
 // Row-strided: blockDim = (64, 4); each wavefront walks one row at a time, one lane per
 // output dword (4 columns, padding included), so no per-thread index division is needed and
 // a wavefront's loads and stores are contiguous.  XV = floats per aligned load (4, 2 or 1).
@@ -180,6 +200,9 @@ __global__ __launch_bounds__(256) void quantize_rows_kernel(
     const float* __restrict__ scale, int per_row, int8_t* __restrict__ q, int64_t ldq,
     const float* __restrict__ noise, uint64_t seed, uint64_t offset,
     const float* __restrict__ row_mul, const float* __restrict__ mask, int64_t ldm) {
+    // the mask may use x's vector width when its rows are laid out and aligned like x's
+    const bool mask_vec = mask && ldm == ldx &&
+                          ((reinterpret_cast<uintptr_t>(mask) ^ reinterpret_cast<uintptr_t>(x)) & 15) == 0;
     const int64_t groups = (ldq + 3) >> 2;  // dword groups per row
     const bool dword_ok = (ldq & 3) == 0 && (reinterpret_cast<uintptr_t>(q) & 3) == 0;
     const int64_t row_step = static_cast<int64_t>(gridDim.x) * blockDim.y;
@@ -190,29 +213,19 @@ __global__ __launch_bounds__(256) void quantize_rows_kernel(
         int8_t* qr = q + row * ldq;
         for (int64_t gi = threadIdx.x; gi < groups; gi += blockDim.x) {
             const int64_t c0 = gi << 2;
-            float f[4] = {0.f, 0.f, 0.f, 0.f};
-            if (XV == 4 && c0 + 4 <= cols) {
-                const f32x4 v = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(xr + c0));
-                f[0] = v.x; f[1] = v.y; f[2] = v.z; f[3] = v.w;
-            } else if (XV == 2 && c0 + 4 <= cols) {
-                typedef float f32x2 __attribute__((ext_vector_type(2)));
-                const f32x2 v0 = __builtin_nontemporal_load(reinterpret_cast<const f32x2*>(xr + c0));
-                const f32x2 v1 = __builtin_nontemporal_load(reinterpret_cast<const f32x2*>(xr + c0 + 2));
-                f[0] = v0.x; f[1] = v0.y; f[2] = v1.x; f[3] = v1.y;
-            } else {
-#pragma unroll
-                for (int k = 0; k < 4; ++k)
-                    if (c0 + k < cols) f[k] = xr[c0 + k];
-            }
+            float f[4];
+            load4<XV>(f, xr, c0, cols);
             if (row_mul) {  // x * row_mul[row], one rounding, before quantization
                 const float rm = row_mul[row];
 #pragma unroll
                 for (int k = 0; k < 4; ++k) f[k] = f[k] * rm;
             }
             if (mask) {  // elements whose mask value is not positive quantize to zero
+                float mk[4];
+                if (mask_vec) load4<XV>(mk, mask + row * ldm, c0, cols); else load4<1>(mk, mask + row * ldm, c0, cols);
 #pragma unroll
                 for (int k = 0; k < 4; ++k)
-                    if (c0 + k < cols && !(mask[row * ldm + c0 + k] > 0.0f)) f[k] = 0.0f;
+                    if (!(mk[k] > 0.0f)) f[k] = 0.0f;
             }
             int v[4];
             const uint64_t lin = static_cast<uint64_t>(row) * cols + c0;
@@ -290,11 +303,14 @@ __global__ __launch_bounds__(256) void transpose_quant_kernel(const float* __res
 // scale rows, quantize" backward step in one read of x.  blockDim = (64, 4), a wavefront walks
 // rows; lane l owns columns 4 l .. 4 l + 3 (+ 256 t).  Column sums are written as one partial
 // row per wavefront and reduced in a fixed order afterwards, so they are deterministic.
-template <int T>
+template <int T, int XV>
 __global__ __launch_bounds__(256) void absmax_ex_kernel(
     const float* __restrict__ x, int64_t rows, int64_t cols, int64_t ldx,
     const float* __restrict__ row_mul, const float* __restrict__ mask, int64_t ldm,
-    float* __restrict__ scale_out, float* __restrict__ partial /* [gridDim.x * 4, cols] or null */) {
+    float* __restrict__ scale_out, float* __restrict__ partial /* [gridDim.x, cols] or null */) {
+    __shared__ float red[3][T * 256];
+    const bool mask_vec = mask && ldm == ldx &&
+                          ((reinterpret_cast<uintptr_t>(mask) ^ reinterpret_cast<uintptr_t>(x)) & 15) == 0;
     float m = 0.0f;
     float cs[T][4];
 #pragma unroll
@@ -309,38 +325,63 @@ __global__ __launch_bounds__(256) void absmax_ex_kernel(
 #pragma unroll
         for (int t = 0; t < T; ++t) {
             const int64_t c0 = (static_cast<int64_t>(threadIdx.x) + 64 * t) << 2;
+            if (c0 < cols) {
+                float v[4];
+                load4<XV>(v, xr, c0, cols);
+                if (mask) {
+                    float mk[4];
+                    if (mask_vec) load4<XV>(mk, mask + row * ldm, c0, cols); else load4<1>(mk, mask + row * ldm, c0, cols);
 #pragma unroll
-            for (int k = 0; k < 4; ++k) {
-                if (c0 + k < cols) {
-                    float v = xr[c0 + k];
-                    if (mask && !(mask[row * ldm + c0 + k] > 0.0f)) v = 0.0f;
-                    cs[t][k] += v;
-                    m = fmaxf(m, fabsf(row_mul ? v * rm : v));
+                    for (int k = 0; k < 4; ++k)
+                        if (!(mk[k] > 0.0f)) v[k] = 0.0f;
+                }
+#pragma unroll
+                for (int k = 0; k < 4; ++k) {
+                    cs[t][k] += v[k];
+                    m = fmaxf(m, fabsf(row_mul ? v[k] * rm : v[k]));
                 }
             }
         }
     }
-    if (partial) {
-        float* prow = partial + (static_cast<int64_t>(blockIdx.x) * blockDim.y + threadIdx.y) * cols;
+    if (partial) {  // fold the block's four wavefronts in a fixed order, one partial row per block
+        if (threadIdx.y > 0) {
 #pragma unroll
-        for (int t = 0; t < T; ++t) {
-            const int64_t c0 = (static_cast<int64_t>(threadIdx.x) + 64 * t) << 2;
+            for (int t = 0; t < T; ++t)
 #pragma unroll
-            for (int k = 0; k < 4; ++k)
-                if (c0 + k < cols) prow[c0 + k] = cs[t][k];
+                for (int k = 0; k < 4; ++k) red[threadIdx.y - 1][(t * 4 + k) * 64 + threadIdx.x] = cs[t][k];
+        }
+        __syncthreads();
+        if (threadIdx.y == 0) {
+            float* prow = partial + static_cast<int64_t>(blockIdx.x) * cols;
+#pragma unroll
+            for (int t = 0; t < T; ++t) {
+                const int64_t c0 = (static_cast<int64_t>(threadIdx.x) + 64 * t) << 2;
+#pragma unroll
+                for (int k = 0; k < 4; ++k) {
+                    const int i = (t * 4 + k) * 64 + threadIdx.x;
+                    const float v = ((cs[t][k] + red[0][i]) + red[1][i]) + red[2][i];
+                    if (c0 + k < cols) prow[c0 + k] = v;
+                }
+            }
         }
     }
     block_absmax_to_global(m / 127.0f, scale_out);
 }
 
+// blockDim = (64, 4): 64 columns per block; thread (x, y) sums partial rows y, y + 4, ...;
+// the four sums of a column are then added in a fixed order.
 __global__ __launch_bounds__(256) void colsum_finish_kernel(const float* __restrict__ partial,
                                                             int64_t nrows, int64_t cols,
                                                             float* __restrict__ out) {
-    const int64_t c = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
-    if (c >= cols) return;
+    __shared__ float red[4][64];
+    const int64_t c = static_cast<int64_t>(blockIdx.x) * 64 + threadIdx.x;
     float s = 0.0f;
-    for (int64_t r = 0; r < nrows; ++r) s += partial[r * cols + c];
-    out[c] = s;
+    if (c < cols)
+        for (int64_t r = threadIdx.y; r < nrows; r += 4) s += partial[r * cols + c];
+    red[threadIdx.y][threadIdx.x] = s;
+    __syncthreads();
+    if (threadIdx.y == 0 && c < cols)
+        out[c] = ((red[0][threadIdx.x] + red[1][threadIdx.x]) + red[2][threadIdx.x]) + red[3][threadIdx.x];
 }
 
 template <typename F>
@@ -408,7 +449,7 @@ static int absmax_ex_grid(int64_t rows) {
 
 size_t tango_absmax_ex_workspace(int64_t rows, int64_t cols, int want_colsum) {
     if (!want_colsum || rows <= 0 || cols <= 0) return 0;
-    return static_cast<size_t>(absmax_ex_grid(rows)) * 4 * static_cast<size_t>(cols) * sizeof(float);
+    return static_cast<size_t>(absmax_ex_grid(rows)) * static_cast<size_t>(cols) * sizeof(float);
 }
 
 int tango_absmax_ex_f32(const float* x, int64_t rows, int64_t cols, int64_t ldx, const float* row_mul,
@@ -429,14 +470,21 @@ int tango_absmax_ex_f32(const float* x, int64_t rows, int64_t cols, int64_t ldx,
     if (cols == 0) return launch_status();
     const dim3 block(64, 4);
     const int T = static_cast<int>(ceil_div(cols, 256));
-#define TANGO_AEX(T_)                                                                              \
-    hipLaunchKernelGGL((absmax_ex_kernel<T_>), dim3(grid), block, 0, s, x, rows, cols, ldx, row_mul, \
+    const uintptr_t xa = reinterpret_cast<uintptr_t>(x);
+    const int xv = ((xa & 15) == 0 && (ldx & 3) == 0) ? 4 : ((xa & 7) == 0 && (ldx & 1) == 0) ? 2 : 1;
+#define TANGO_AEX(T_, V_)                                                                              \
+    hipLaunchKernelGGL((absmax_ex_kernel<T_, V_>), dim3(grid), block, 0, s, x, rows, cols, ldx, row_mul, \
                        mask, ldm, scale_out, partial)
-    if (T <= 1) TANGO_AEX(1); else if (T == 2) TANGO_AEX(2); else if (T == 3) TANGO_AEX(3); else TANGO_AEX(4);
+#define TANGO_AEX_T(T_)                                                              \
+    do {                                                                             \
+        if (xv == 4) TANGO_AEX(T_, 4); else if (xv == 2) TANGO_AEX(T_, 2); else TANGO_AEX(T_, 1); \
+    } while (0)
+    if (T <= 1) TANGO_AEX_T(1); else if (T == 2) TANGO_AEX_T(2); else if (T == 3) TANGO_AEX_T(3); else TANGO_AEX_T(4);
+#undef TANGO_AEX_T
 #undef TANGO_AEX
     if (colsum_out)
-        hipLaunchKernelGGL(colsum_finish_kernel, dim3(static_cast<unsigned>(ceil_div(cols, 256))), dim3(256), 0,
-                           s, partial, static_cast<int64_t>(grid) * 4, cols, colsum_out);
+        hipLaunchKernelGGL(colsum_finish_kernel, dim3(static_cast<unsigned>(ceil_div(cols, 64))), dim3(64, 4), 0,
+                           s, partial, static_cast<int64_t>(grid), cols, colsum_out);
     return launch_status();
 }
 
