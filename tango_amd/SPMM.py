@@ -7,13 +7,22 @@ from .kernels import (cuda_kernels, csr_SPMM, multi_cusparse_SPMM, mySDDMM_int8,
                       quantize_padded, transpose_quant)
 
 
+def _gather_align(width):
+    """Row pitch for int8 rows that will be gathered: rows narrower than a 128-byte cache line are
+    padded to a power of two so that no row straddles two lines; wider rows to whole lines."""
+    for a in (16, 32, 64, 128):
+        if width <= a:
+            return a
+    return 128
+
+
 def _quantize_grad(t, padded):
     t = t if t.is_contiguous() else t.contiguous()
     kw = {"round_mode": config.grad_round_mode}
     if config.grad_round_mode == "stochastic":
         kw.update(seed=config.seed, offset=config.next_offset())
     if padded and t.dim() == 2:
-        return quantize_padded(t, **kw)
+        return quantize_padded(t, align=_gather_align(t.size(1)), **kw)
     return quantize(t, **kw)
 
 
@@ -33,7 +42,7 @@ class spmm_copy_u(Function):
         if fused and N.dim() != 2:
             raise RuntimeError("spmm_copy_u: the fused epilogue needs 2-D features")
         if N.dim() == 2:
-            N_, scaleN = quantize_padded(N, scaleN)
+            N_, scaleN = quantize_padded(N, scaleN, align=_gather_align(N.size(1)))
         else:
             N_, scaleN = quantize(N, scaleN)
         out = csr_SPMM(g, N_, scaleN, row_scale=row_scale, bias=bias, relu=relu)
@@ -58,7 +67,8 @@ class spmm_copy_u(Function):
             kw = {"round_mode": config.grad_round_mode}
             if config.grad_round_mode == "stochastic":
                 kw.update(seed=config.seed, offset=config.next_offset())
-            dZ_, _ = quantize_padded(dOut, scaledZ, row_mul=row_scale, mask=mask, **kw)
+            dZ_, _ = quantize_padded(dOut, scaledZ, row_mul=row_scale, mask=mask,
+                                     align=_gather_align(dOut.size(1)), **kw)
             dN = csr_SPMM(g, dZ_, scaledZ, True)
         return None, dN, None, None, dbias, None
 

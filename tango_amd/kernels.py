@@ -8,6 +8,7 @@ stream; all arithmetic runs in the HIP library.  Keyword arguments that the
 reference does not have (``round_mode``, ``noise``, ``seed``, ``offset``,
 ``edge_ids``) default to the reference's behaviour.
 """
+import math
 import os
 
 import torch
@@ -304,7 +305,7 @@ class cuda_kernels:
         _need(U, torch.int8, "U")
         _need(scaleU, torch.float32, "scaleU")
         rows = indptr.numel() - 1
-        width = U.numel() // max(U.size(0), 1)
+        width = math.prod(U.shape[1:])
         ldf = width if ldf is None else ldf
         F = width if F is None else F
         if out.numel() != rows * F:
@@ -362,7 +363,7 @@ class cuda_kernels:
         _need(dst, torch.int64, "dst")
         _need(E, torch.int8, "E")
         _need(scale, torch.float32, "scale")
-        F = E.numel() // max(E.size(0), 1)
+        F = math.prod(E.shape[1:])
         if out.dim() != 2 or out.size(1) != F:
             raise RuntimeError("incidence_SPMM: out must be [num_nodes, %d]" % F)
         check(_L.tango_spmm_incidence(_ptr(out), _ptr(src), _ptr(dst), _ptr(E), scale.data_ptr(),
@@ -388,14 +389,14 @@ class cuda_kernels:
             raise RuntimeError("mySDDMM_int8: U and V must have equal feature shapes")
         if op == "dot":
             D = U.size(-1)
-            H = U.numel() // max(U.size(0), 1) // max(D, 1)
+            H = math.prod(U.shape[1:-1])
             if out.numel() != E * H:
                 raise RuntimeError("mySDDMM_int8: out must be [E, %d, 1]" % H)
             check(_L.tango_sddmm_dot_i8(_ptr(out), _ptr(scaleOut), _ptr(src), _ptr(dst), _ptr(U), _ptr(V),
                                         scaleU.data_ptr(), scaleV.data_ptr(), E, H, D, _stream()),
                   "mySDDMM_int8(dot)")
         elif op in SDDMM_OPS:
-            T = U.numel() // max(U.size(0), 1)
+            T = math.prod(U.shape[1:])
             if out.numel() != E * T:
                 raise RuntimeError("mySDDMM_int8: out must be [E, %d]" % T)
             check(_L.tango_sddmm_ewise_i8(SDDMM_OPS[op], _ptr(out), _ptr(scaleOut), _ptr(src), _ptr(dst),
@@ -553,7 +554,7 @@ def incidence_SPMM(g, E, scaleE, reverse=False):
     src = coo[0]
     dst = coo[1]
     out_shape = (g.num_nodes(),) + E.shape[1:]
-    dim = E.numel() // max(E.size(0), 1)
+    dim = math.prod(E.shape[1:])
     out = torch.empty((g.num_nodes(), dim), dtype=torch.float32, device=E.device)
     cuda_kernels.incidence_SPMM(out, src, dst, E, scaleE)
     return out.view(out_shape)
@@ -568,7 +569,7 @@ def csr_SPMM(g, N, scaleN, reverse=False, row_scale=None, bias=None, relu=False)
         indptr, indices, _ = g.adj_csc
     feat_shape = N.shape[1:]
     out_shape = (g.num_nodes(),) + feat_shape
-    dim = N.numel() // max(N.size(0), 1)
+    dim = math.prod(N.shape[1:])
     out = torch.empty((g.num_nodes(), dim), dtype=torch.float32, device=N.device)
     if N.dim() == 2 and not N.is_contiguous():
         ld = _rows_view(N, "N")
