@@ -187,6 +187,203 @@ __global__ __launch_bounds__(256, 2) void gemm_nt_kernel(const NtParams p) {
     if (p.absmax_out) block_absmax_to_global(m / 127.0f, p.absmax_out);
 }
 
+// ------------------------------------ forward GEMM with the quantize fused in
+// Workgroup = 4 waves = 64 rows of X.  Phase A: the waves stream their rows of the
+// fp32 X from HBM (each lane 4 consecutive floats per step, a wavefront 1 KiB of one
+// row), quantize in registers and write the int8 bytes twice: to Xq (the cache the
+// backward pass reads) and to an LDS copy of the whole 64 x K block.  Phase B: every
+// wave takes a quarter of the output columns, reads A fragments from that LDS block
+// and B fragments straight from the packed small operand (L2-resident), and runs the
+// MFMA k-loop without any further barrier.  X is read once, Xq written once, Y once.
+struct FqParams {
+    float* C;
+    const float* X;
+    int8_t* Xq;
+    const int8_t* B;      // packed [N, Kp]
+    const float* bias;
+    const float* x_row_mul;  // optional per-row multiplier applied before quantization
+    float* absmax_out;
+    const float* sA;
+    const float* sB;
+    int64_t M, N, K;
+    int64_t ldx, ldxq, ldb, ldc;
+    int kp;               // K rounded up to 64
+};
+
+// TPW = 16-column tiles per wave (the workgroup covers 64 * TPW columns), XV = floats per load,
+// RT = 16-row tiles per workgroup (BM = 16 * RT rows).
+template <int TPW, int XV, int MODE, int RT>
+__global__ __launch_bounds__(256, 2) void gemm_fq_kernel(const FqParams p) {
+    extern __shared__ __attribute__((aligned(16))) int8_t a_lds[];  // [BM][kp + 16]
+    constexpr int BM = 16 * RT;
+    const int pitch = p.kp + 16;
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int64_t row_base = static_cast<int64_t>(blockIdx.x) * BM;
+    const float rs = rscale_of(p.sA[0]);
+    const bool store_q = blockIdx.y == 0;
+
+    // ---- phase A: rows wave, wave + 4, ... ; lane owns columns 4 * (lane + 64 it) .. + 3
+    const float* __restrict__ Xp = p.X;
+    int8_t* __restrict__ Xqp = p.Xq;
+    const int iters = (p.kp + 255) >> 8;  // <= 3: kp <= 768 is checked by the host
+    auto fetch = [&](float (*f)[3][4], int rr) {
+#pragma unroll
+        for (int b = 0; b < 4; ++b) {
+            const int64_t row = row_base + wave + 4 * (rr + b);
+            const float* xr = Xp + row * p.ldx;
+#pragma unroll
+            for (int it = 0; it < 3; ++it) {
+                const int64_t c0 = (static_cast<int64_t>(lane) + 64 * it) << 2;
+                f[b][it][0] = f[b][it][1] = f[b][it][2] = f[b][it][3] = 0.0f;
+                if (it < iters && row < p.M && c0 < p.K) {
+                    if (XV == 4 && c0 + 4 <= p.K) {
+                        const f32x4 v = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(xr + c0));
+                        f[b][it][0] = v.x; f[b][it][1] = v.y; f[b][it][2] = v.z; f[b][it][3] = v.w;
+                    } else if (XV == 2 && c0 + 4 <= p.K) {
+                        typedef float f32x2 __attribute__((ext_vector_type(2)));
+                        const f32x2 v0 = __builtin_nontemporal_load(reinterpret_cast<const f32x2*>(xr + c0));
+                        const f32x2 v1 = __builtin_nontemporal_load(reinterpret_cast<const f32x2*>(xr + c0 + 2));
+                        f[b][it][0] = v0.x; f[b][it][1] = v0.y; f[b][it][2] = v1.x; f[b][it][3] = v1.y;
+                    } else {
+#pragma unroll
+                        for (int k = 0; k < 4; ++k)
+                            if (c0 + k < p.K) f[b][it][k] = xr[c0 + k];
+                    }
+                }
+            }
+        }
+    };
+    auto emit = [&](float (*f)[3][4], int rr) {
+#pragma unroll
+        for (int b = 0; b < 4; ++b) {
+            const int lr = wave + 4 * (rr + b);
+            const int64_t row = row_base + lr;
+            const float rm = (p.x_row_mul && row < p.M) ? p.x_row_mul[row] : 1.0f;
+#pragma unroll
+            for (int it = 0; it < 3; ++it) {
+                const int64_t c0 = (static_cast<int64_t>(lane) + 64 * it) << 2;
+                if (it < iters && c0 < p.kp) {
+                    float x0 = f[b][it][0], x1 = f[b][it][1], x2 = f[b][it][2], x3 = f[b][it][3];
+                    if (p.x_row_mul) { x0 = x0 * rm; x1 = x1 * rm; x2 = x2 * rm; x3 = x3 * rm; }
+                    const uint32_t q = pack4(quant_one<MODE>(x0, rs, 0.f), quant_one<MODE>(x1, rs, 0.f),
+                                             quant_one<MODE>(x2, rs, 0.f), quant_one<MODE>(x3, rs, 0.f));
+                    *reinterpret_cast<uint32_t*>(a_lds + lr * pitch + c0) = q;
+                    if (store_q && row < p.M && c0 < p.ldxq)
+                        __builtin_nontemporal_store(q, reinterpret_cast<uint32_t*>(Xqp + row * p.ldxq + c0));
+                }
+            }
+        }
+    };
+    {
+        // two register buffers: the loads of the next four rows are in flight while these are quantized
+        float fa[4][3][4], fb[4][3][4];
+        fetch(fa, 0);
+        fetch(fb, 4);
+        emit(fa, 0);
+        if (RT == 4) fetch(fa, 8);
+        emit(fb, 4);
+        if (RT == 4) {
+            fetch(fb, 12);
+            emit(fa, 8);
+            emit(fb, 12);
+        }
+    }
+    __syncthreads();
+
+    // ---- phase B
+    const int g = lane >> 4, r16 = lane & 15;
+    const int64_t n0 = static_cast<int64_t>(blockIdx.y) * (64 * TPW) + static_cast<int64_t>(wave) * (16 * TPW);
+    const int ksteps = p.kp >> 6;
+    i32x4 acc[RT][TPW];
+#pragma unroll
+    for (int i = 0; i < RT; ++i)
+#pragma unroll
+        for (int j = 0; j < TPW; ++j) acc[i][j] = i32x4{0, 0, 0, 0};
+
+    if (n0 < p.N) {  // wave-uniform: waves whose columns lie beyond N only take part in phase A
+        const int8_t* pb[TPW];
+        bool bok[TPW];
+#pragma unroll
+        for (int j = 0; j < TPW; ++j) {
+            const int64_t n = n0 + j * 16 + r16;
+            bok[j] = n < p.N;
+            pb[j] = p.B + (bok[j] ? n : 0) * p.ldb + g * 16;
+        }
+        // B fragments run two k-steps ahead of the MFMAs that consume them
+        i32x4 b0[TPW], b1[TPW], b2[TPW];
+        auto load_bfrag = [&](i32x4* dst, int step) {
+            const int sc = step < ksteps ? step : ksteps - 1;
+#pragma unroll
+            for (int j = 0; j < TPW; ++j) dst[j] = *reinterpret_cast<const i32x4*>(pb[j] + static_cast<int64_t>(sc) * 64);
+        };
+        auto mma_step = [&](const i32x4* bf, int step) {
+#pragma unroll
+            for (int i = 0; i < RT; ++i) {
+                const i32x4 a = *reinterpret_cast<const i32x4*>(a_lds + (i * 16 + r16) * pitch + step * 64 + g * 16);
+#pragma unroll
+                for (int j = 0; j < TPW; ++j) {
+                    const i32x4 b = bok[j] ? bf[j] : i32x4{0, 0, 0, 0};
+                    acc[i][j] = mfma_16x16x64(b, a, acc[i][j]);
+                }
+            }
+        };
+        load_bfrag(b0, 0);
+        load_bfrag(b1, 1);
+        for (int step = 0; step < ksteps; step += 3) {
+            load_bfrag(b2, step + 2);
+            mma_step(b0, step);
+            if (step + 1 < ksteps) {
+                load_bfrag(b0, step + 3);
+                mma_step(b1, step + 1);
+            }
+            if (step + 2 < ksteps) {
+                load_bfrag(b1, step + 4);
+                mma_step(b2, step + 2);
+            }
+        }
+    }
+
+    // ---- epilogue: lane holds C[row_base + 16 i + r16][n0 + 16 j + 4 g + v]
+    const float s = p.sA[0] * p.sB[0];
+    float m = 0.0f;
+    const uintptr_t ca = reinterpret_cast<uintptr_t>(p.C);
+    const int wide = ((ca & 15) == 0 && (p.ldc & 3) == 0) ? 4 : ((ca & 7) == 0 && (p.ldc & 1) == 0) ? 2 : 1;
+    if (n0 < p.N) {
+#pragma unroll
+        for (int i = 0; i < RT; ++i) {
+            const int64_t row = row_base + i * 16 + r16;
+            if (row < p.M) {
+                float* crow = p.C + row * p.ldc;
+#pragma unroll
+                for (int j = 0; j < TPW; ++j) {
+                    const int64_t col = n0 + j * 16 + g * 4;
+                    float y[4];
+#pragma unroll
+                    for (int v = 0; v < 4; ++v) {
+                        y[v] = s * static_cast<float>(acc[i][j][v]);
+                        if (p.bias && col + v < p.N) y[v] = p.bias[col + v] + y[v];
+                        if (col + v < p.N) m = fmaxf(m, fabsf(y[v]));
+                    }
+                    if (col + 4 <= p.N && wide == 4) {
+                        __builtin_nontemporal_store(f32x4{y[0], y[1], y[2], y[3]}, reinterpret_cast<f32x4*>(crow + col));
+                    } else if (col + 4 <= p.N && wide == 2) {
+                        typedef float f32x2 __attribute__((ext_vector_type(2)));
+                        *reinterpret_cast<f32x2*>(crow + col) = f32x2{y[0], y[1]};
+                        *reinterpret_cast<f32x2*>(crow + col + 2) = f32x2{y[2], y[3]};
+                    } else {
+#pragma unroll
+                        for (int v = 0; v < 4; ++v)
+                            if (col + v < p.N) crow[col + v] = y[v];
+                    }
+                }
+            }
+        }
+    }
+    if (p.absmax_out) block_absmax_to_global(m / 127.0f, p.absmax_out);
+}
+
 // ------------------------------------------------------- operand packing
 // dst[r, 0..ldd) = src[r, 0..cols) zero-filled, for r < rows (src row stride lds).
 __global__ __launch_bounds__(256) void pack_rows_i8_kernel(int8_t* __restrict__ dst, int64_t ldd,
@@ -409,6 +606,44 @@ static int launch_nt(NtParams p, hipStream_t s) {
     return launch_status();
 }
 
+// The fused forward needs: a deterministic rounding mode, K <= 768 (the 64 x K int8 block and
+// the per-lane staging registers are sized for it), Xq rows that are 16-byte aligned and cover
+// round_up(K, 16) bytes, and X rows that are at least 8-byte aligned.
+static bool fq_applicable(const float* X, int64_t ldx, const int8_t* Xq, int64_t ldxq, int64_t K,
+                          int round_mode) {
+    if (round_mode != TANGO_ROUND_RNE && round_mode != TANGO_ROUND_TRUNC) return false;
+    if (K < 1 || K > 768) return false;
+    if ((reinterpret_cast<uintptr_t>(Xq) & 15) != 0 || (ldxq & 15) != 0 || ldxq < round_up(K, 16)) return false;
+    if ((reinterpret_cast<uintptr_t>(X) & 7) != 0 || (ldx & 1) != 0) return false;
+    return true;
+}
+
+template <int XV, int MODE>
+static void launch_fq_mode(const FqParams& p, hipStream_t s) {
+    constexpr int RT = 4;  // 64 rows per workgroup measured faster than 32 at every benchmark shape
+    const size_t lds = static_cast<size_t>(16 * RT) * (p.kp + 16);
+    const unsigned gx = static_cast<unsigned>(ceil_div(p.M, 16 * RT));
+#define TANGO_FQ(TPW_)                                                                           \
+    hipLaunchKernelGGL((gemm_fq_kernel<TPW_, XV, MODE, RT>),                                     \
+                       dim3(gx, static_cast<unsigned>(ceil_div(p.N, 64 * TPW_))), dim3(256), lds, s, p)
+    if (p.N <= 64) TANGO_FQ(1);
+    else if (p.N <= 128) TANGO_FQ(2);
+    else TANGO_FQ(4);
+#undef TANGO_FQ
+}
+
+static int launch_fq(const FqParams& p, int round_mode, hipStream_t s) {
+    if (ceil_div(p.M, 64) > INT32_MAX || ceil_div(p.N, 64) > 65535) return TANGO_ERR_UNSUPPORTED;
+    if (p.absmax_out) fill_u32(p.absmax_out, 0u, 1, s);
+    const bool v4 = (reinterpret_cast<uintptr_t>(p.X) & 15) == 0 && (p.ldx & 3) == 0;
+    if (round_mode == TANGO_ROUND_RNE) {
+        if (v4) launch_fq_mode<4, TANGO_ROUND_RNE>(p, s); else launch_fq_mode<2, TANGO_ROUND_RNE>(p, s);
+    } else {
+        if (v4) launch_fq_mode<4, TANGO_ROUND_TRUNC>(p, s); else launch_fq_mode<2, TANGO_ROUND_TRUNC>(p, s);
+    }
+    return launch_status();
+}
+
 }  // namespace tango
 
 using namespace tango;
@@ -447,9 +682,13 @@ int tango_qgemm_fwd_ex(float* Y, int64_t ldy, const float* X, int64_t ldx, const
     if (need > 0 && (!workspace || workspace_bytes < need)) return TANGO_ERR_WORKSPACE;
     if ((reinterpret_cast<uintptr_t>(workspace) & 15) != 0) return TANGO_ERR_INVALID_ARG;
     hipStream_t s = as_stream(stream);
-    int rc = tango_quantize_rows_ex_f32_i8(X, M, K, ldx, x_row_mul, nullptr, 0, scaleX, 0, Xq, ldxq, round_mode,
+    const bool fused = M > 0 && N > 0 && fq_applicable(X, ldx, Xq, ldxq, K, round_mode);
+    int rc = TANGO_OK;
+    if (!fused) {
+        rc = tango_quantize_rows_ex_f32_i8(X, M, K, ldx, x_row_mul, nullptr, 0, scaleX, 0, Xq, ldxq, round_mode,
                                            nullptr, 0, 0, stream);
-    if (rc != TANGO_OK) return rc;
+        if (rc != TANGO_OK) return rc;
+    }
     rc = tango_quantize_rows_f32_i8(W, N, K, ldw, scaleW, 0, Wq, K, round_mode, nullptr, 0, 0, stream);
     if (rc != TANGO_OK) return rc;
     if (M == 0 || N == 0) return TANGO_OK;
@@ -458,6 +697,13 @@ int tango_qgemm_fwd_ex(float* Y, int64_t ldy, const float* X, int64_t ldx, const
     if (K > 0)
         hipLaunchKernelGGL(pack_rows_i8_kernel, dim3(grid_for(N * ldb, 256)), dim3(256), 0, s, Bp, ldb,
                            Wq, K, N, K);
+    if (fused) {
+        FqParams q{};
+        q.C = Y; q.X = X; q.Xq = Xq; q.B = Bp; q.bias = bias; q.x_row_mul = x_row_mul; q.absmax_out = scaleY;
+        q.sA = scaleX; q.sB = scaleW; q.M = M; q.N = N; q.K = K; q.ldx = ldx; q.ldxq = ldxq; q.ldb = ldb;
+        q.ldc = ldy; q.kp = static_cast<int>(ldb);
+        return launch_fq(q, round_mode, s);
+    }
     NtParams p{};
     p.C = Y; p.A = Xq; p.B = Bp; p.bias = bias; p.absmax_out = scaleY; p.sA = scaleX; p.sB = scaleW;
     p.M = M; p.N = N; p.Kr = K; p.lda = ldxq; p.ldb = ldb; p.ldc = ldy;
