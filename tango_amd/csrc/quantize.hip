@@ -22,8 +22,11 @@ __device__ __forceinline__ Philox4 philox4x32_10(uint32_t c0, uint32_t c1, uint3
                                                  uint32_t c3, uint32_t k0, uint32_t k1) {
 #pragma unroll
     for (int r = 0; r < 10; ++r) {
-        const uint32_t hi0 = __umulhi(0xD2511F53u, c0), lo0 = 0xD2511F53u * c0;
-        const uint32_t hi1 = __umulhi(0xCD9E8D57u, c2), lo1 = 0xCD9E8D57u * c2;
+        // one 32x32->64 multiply (v_mad_u64_u32) yields both halves; integer multiplies are quarter rate
+        const uint64_t p0 = static_cast<uint64_t>(0xD2511F53u) * c0;
+        const uint64_t p1 = static_cast<uint64_t>(0xCD9E8D57u) * c2;
+        const uint32_t hi0 = static_cast<uint32_t>(p0 >> 32), lo0 = static_cast<uint32_t>(p0);
+        const uint32_t hi1 = static_cast<uint32_t>(p1 >> 32), lo1 = static_cast<uint32_t>(p1);
         const uint32_t n0 = hi1 ^ c1 ^ k0;
         const uint32_t n2 = hi0 ^ c3 ^ k1;
         c0 = n0;
@@ -199,19 +202,23 @@ __global__ __launch_bounds__(256) void quantize_rows_kernel(
     const float* __restrict__ x, int64_t rows, int64_t cols, int64_t ldx,
     const float* __restrict__ scale, int per_row, int8_t* __restrict__ q, int64_t ldq,
     const float* __restrict__ noise, uint64_t seed, uint64_t offset,
-    const float* __restrict__ row_mul, const float* __restrict__ mask, int64_t ldm) {
+    const float* __restrict__ row_mul, const float* __restrict__ mask, int64_t ldm, int gpr_log2) {
     // the mask may use x's vector width when its rows are laid out and aligned like x's
     const bool mask_vec = mask && ldm == ldx &&
                           ((reinterpret_cast<uintptr_t>(mask) ^ reinterpret_cast<uintptr_t>(x)) & 15) == 0;
     const int64_t groups = (ldq + 3) >> 2;  // dword groups per row
     const bool dword_ok = (ldq & 3) == 0 && (reinterpret_cast<uintptr_t>(q) & 3) == 0;
-    const int64_t row_step = static_cast<int64_t>(gridDim.x) * blockDim.y;
-    for (int64_t row = static_cast<int64_t>(blockIdx.x) * blockDim.y + threadIdx.y; row < rows;
+    // narrow rows: a wavefront takes 64 / gpr rows at once (gpr = groups rounded up to a power of two)
+    const int gpr = 1 << gpr_log2;
+    const int rpw = kWave >> gpr_log2;
+    const int sub = static_cast<int>(threadIdx.x) >> gpr_log2;
+    const int64_t row_step = static_cast<int64_t>(gridDim.x) * blockDim.y * rpw;
+    for (int64_t row = (static_cast<int64_t>(blockIdx.x) * blockDim.y + threadIdx.y) * rpw + sub; row < rows;
          row += row_step) {
         const float r = rscale_of(scale[per_row ? row : 0]);
         const float* xr = x + row * ldx;
         int8_t* qr = q + row * ldq;
-        for (int64_t gi = threadIdx.x; gi < groups; gi += blockDim.x) {
+        for (int64_t gi = threadIdx.x & (gpr - 1); gi < groups; gi += gpr) {
             const int64_t c0 = gi << 2;
             float f[4];
             load4<XV>(f, xr, c0, cols);
@@ -307,7 +314,8 @@ template <int T, int XV>
 __global__ __launch_bounds__(256) void absmax_ex_kernel(
     const float* __restrict__ x, int64_t rows, int64_t cols, int64_t ldx,
     const float* __restrict__ row_mul, const float* __restrict__ mask, int64_t ldm,
-    float* __restrict__ scale_out, float* __restrict__ partial /* [gridDim.x, cols] or null */) {
+    float* __restrict__ scale_out, float* __restrict__ partial /* [gridDim.x, cols] or null */,
+    int gpr_log2) {
     __shared__ float red[3][T * 256];
     const bool mask_vec = mask && ldm == ldx &&
                           ((reinterpret_cast<uintptr_t>(mask) ^ reinterpret_cast<uintptr_t>(x)) & 15) == 0;
@@ -317,14 +325,19 @@ __global__ __launch_bounds__(256) void absmax_ex_kernel(
     for (int t = 0; t < T; ++t)
 #pragma unroll
         for (int k = 0; k < 4; ++k) cs[t][k] = 0.0f;
-    const int64_t row_step = static_cast<int64_t>(gridDim.x) * blockDim.y;
-    for (int64_t row = static_cast<int64_t>(blockIdx.x) * blockDim.y + threadIdx.y; row < rows;
+    // narrow rows (T == 1): a wavefront takes 64 / gpr rows at once, lane = (row in wave, column group)
+    const int gpr = 1 << gpr_log2;
+    const int rpw = kWave >> gpr_log2;
+    const int sub = static_cast<int>(threadIdx.x) >> gpr_log2;
+    const int gl = static_cast<int>(threadIdx.x) & (gpr - 1);
+    const int64_t row_step = static_cast<int64_t>(gridDim.x) * blockDim.y * rpw;
+    for (int64_t row = (static_cast<int64_t>(blockIdx.x) * blockDim.y + threadIdx.y) * rpw + sub; row < rows;
          row += row_step) {
         const float rm = row_mul ? row_mul[row] : 1.0f;
         const float* xr = x + row * ldx;
 #pragma unroll
         for (int t = 0; t < T; ++t) {
-            const int64_t c0 = (static_cast<int64_t>(threadIdx.x) + 64 * t) << 2;
+            const int64_t c0 = (static_cast<int64_t>(gl) + 64 * t) << 2;
             if (c0 < cols) {
                 float v[4];
                 load4<XV>(v, xr, c0, cols);
@@ -344,6 +357,13 @@ __global__ __launch_bounds__(256) void absmax_ex_kernel(
         }
     }
     if (partial) {  // fold the block's four wavefronts in a fixed order, one partial row per block
+        // first the rows a wavefront handled side by side (lanes that differ only in `sub`)
+        for (int off = gpr; off < kWave; off <<= 1) {
+#pragma unroll
+            for (int t = 0; t < T; ++t)
+#pragma unroll
+                for (int k = 0; k < 4; ++k) cs[t][k] += __shfl_xor(cs[t][k], off, kWave);
+        }
         if (threadIdx.y > 0) {
 #pragma unroll
             for (int t = 0; t < T; ++t)
@@ -470,11 +490,14 @@ int tango_absmax_ex_f32(const float* x, int64_t rows, int64_t cols, int64_t ldx,
     if (cols == 0) return launch_status();
     const dim3 block(64, 4);
     const int T = static_cast<int>(ceil_div(cols, 256));
+    int gpr_log2 = 6;
+    const int64_t cgroups = ceil_div(cols, 4);
+    while (gpr_log2 > 0 && (1LL << (gpr_log2 - 1)) >= cgroups) --gpr_log2;
     const uintptr_t xa = reinterpret_cast<uintptr_t>(x);
     const int xv = ((xa & 15) == 0 && (ldx & 3) == 0) ? 4 : ((xa & 7) == 0 && (ldx & 1) == 0) ? 2 : 1;
 #define TANGO_AEX(T_, V_)                                                                              \
     hipLaunchKernelGGL((absmax_ex_kernel<T_, V_>), dim3(grid), block, 0, s, x, rows, cols, ldx, row_mul, \
-                       mask, ldm, scale_out, partial)
+                       mask, ldm, scale_out, partial, gpr_log2)
 #define TANGO_AEX_T(T_)                                                              \
     do {                                                                             \
         if (xv == 4) TANGO_AEX(T_, 4); else if (xv == 2) TANGO_AEX(T_, 2); else TANGO_AEX(T_, 1); \
@@ -527,21 +550,24 @@ int tango_quantize_rows_ex_f32_i8(const float* x, int64_t rows, int64_t cols, in
         return TANGO_ERR_INVALID_ARG;
     if (rows == 0 || ldq == 0) return (round_mode >= 0 && round_mode <= 2) ? TANGO_OK : TANGO_ERR_UNSUPPORTED;
     hipStream_t s = as_stream(stream);
-    const int64_t blocks = ceil_div(rows, 4);
-    const dim3 grid(static_cast<unsigned>(blocks < 256 * 16 ? blocks : 256 * 16)), block(64, 4);
+    const int64_t groups = (ldq + 3) >> 2;
+    int gpr_log2 = 6;
+    while (gpr_log2 > 0 && (1LL << (gpr_log2 - 1)) >= groups) --gpr_log2;
+    const int64_t blocks = ceil_div(rows, 4 * (64 >> gpr_log2));
+    const dim3 grid(static_cast<unsigned>(blocks < 256 * 16 ? (blocks < 1 ? 1 : blocks) : 256 * 16)), block(64, 4);
     const uintptr_t xa = reinterpret_cast<uintptr_t>(x);
     const int xv = ((xa & 15) == 0 && (ldx & 3) == 0) ? 4 : ((xa & 7) == 0 && (ldx & 1) == 0) ? 2 : 1;
     int rc = dispatch_mode(round_mode, [&](auto mode) {
         constexpr int M = decltype(mode)::value;
         if (xv == 4)
             hipLaunchKernelGGL((quantize_rows_kernel<M, 4>), grid, block, 0, s, x, rows, cols, ldx, scale,
-                               per_row, q, ldq, noise, seed, offset, row_mul, mask, ldm);
+                               per_row, q, ldq, noise, seed, offset, row_mul, mask, ldm, gpr_log2);
         else if (xv == 2)
             hipLaunchKernelGGL((quantize_rows_kernel<M, 2>), grid, block, 0, s, x, rows, cols, ldx, scale,
-                               per_row, q, ldq, noise, seed, offset, row_mul, mask, ldm);
+                               per_row, q, ldq, noise, seed, offset, row_mul, mask, ldm, gpr_log2);
         else
             hipLaunchKernelGGL((quantize_rows_kernel<M, 1>), grid, block, 0, s, x, rows, cols, ldx, scale,
-                               per_row, q, ldq, noise, seed, offset, row_mul, mask, ldm);
+                               per_row, q, ldq, noise, seed, offset, row_mul, mask, ldm, gpr_log2);
     });
     return rc != TANGO_OK ? rc : launch_status();
 }

@@ -162,6 +162,17 @@ class cuda_kernels:
         if mask is not None:
             _need(mask, torch.float32, "mask", contiguous=False)
             ldm = _rows_view(mask, "mask")
+        if cols > 1024:
+            # the kernel keeps a row's column sums in registers, 1024 columns at most: walk column slices
+            scale, sums = None, []
+            for c0 in range(0, cols, 1024):
+                sl = slice(c0, min(cols, c0 + 1024))
+                s_i, cs_i = cuda_kernels.absmax_ex(inp[:, sl], row_mul=row_mul,
+                                                   mask=None if mask is None else mask[:, sl],
+                                                   want_colsum=want_colsum)
+                scale = s_i if scale is None else torch.maximum(scale, s_i)
+                sums.append(cs_i)
+            return scale, (torch.cat(sums) if want_colsum else None)
         scale = torch.empty(1, dtype=torch.float32, device=inp.device)
         colsum = torch.empty(cols, dtype=torch.float32, device=inp.device) if want_colsum else None
         ws_bytes = _L.tango_absmax_ex_workspace(rows, cols, int(want_colsum))

@@ -24,7 +24,7 @@ def make_graph(src, dst, n):
 
 def test_absmax_ex_and_quantize_ex(K, orc):
     rng = np.random.default_rng(0)
-    for rows, cols in ((1000, 256), (777, 41), (300, 602), (5, 1024)):
+    for rows, cols in ((1000, 256), (777, 41), (300, 602), (5, 1024), (64, 1500), (3, 7)):
         x = rng.standard_normal((rows, cols)).astype(np.float32)
         rm = rng.random(rows, dtype=np.float32) + 0.1
         mask = rng.standard_normal((rows, cols)).astype(np.float32)
