@@ -93,6 +93,19 @@ __device__ __forceinline__ uint32_t pack4(int a, int b, int c, int d) {
            ((static_cast<uint32_t>(c) & 0xffu) << 16) | (static_cast<uint32_t>(d) << 24);
 }
 
+// 4x4 byte transpose with v_perm_b32: rows r0..r3 (one dword each) -> c[j] = bytes (r0[j], r1[j], r2[j], r3[j]).
+__device__ __forceinline__ void transpose4x4(uint32_t r0, uint32_t r1, uint32_t r2, uint32_t r3,
+                                             uint32_t* c) {
+    const uint32_t t0 = __builtin_amdgcn_perm(r1, r0, 0x05010400u);
+    const uint32_t t1 = __builtin_amdgcn_perm(r1, r0, 0x07030602u);
+    const uint32_t t2 = __builtin_amdgcn_perm(r3, r2, 0x05010400u);
+    const uint32_t t3 = __builtin_amdgcn_perm(r3, r2, 0x07030602u);
+    c[0] = __builtin_amdgcn_perm(t2, t0, 0x05040100u);
+    c[1] = __builtin_amdgcn_perm(t2, t0, 0x07060302u);
+    c[2] = __builtin_amdgcn_perm(t3, t1, 0x05040100u);
+    c[3] = __builtin_amdgcn_perm(t3, t1, 0x07060302u);
+}
+
 // Sets a handful of 32-bit words.  Used instead of hipMemsetAsync so that a
 // caller may capture any entry point into a HIP graph.
 static __global__ void fill_u32_kernel(uint32_t* p, uint32_t v, int n) {

@@ -421,18 +421,6 @@ struct TnParams {
     int tiles_n, tiles_k, splits;
 };
 
-__device__ __forceinline__ void transpose4x4(uint32_t r0, uint32_t r1, uint32_t r2, uint32_t r3,
-                                             uint32_t* c) {
-    const uint32_t t0 = __builtin_amdgcn_perm(r1, r0, 0x05010400u);
-    const uint32_t t1 = __builtin_amdgcn_perm(r1, r0, 0x07030602u);
-    const uint32_t t2 = __builtin_amdgcn_perm(r3, r2, 0x05010400u);
-    const uint32_t t3 = __builtin_amdgcn_perm(r3, r2, 0x07030602u);
-    c[0] = __builtin_amdgcn_perm(t2, t0, 0x05040100u);
-    c[1] = __builtin_amdgcn_perm(t2, t0, 0x07060302u);
-    c[2] = __builtin_amdgcn_perm(t3, t1, 0x05040100u);
-    c[3] = __builtin_amdgcn_perm(t3, t1, 0x07060302u);
-}
-
 // Workgroup tile: 128 (n) x 128 (k), reduction in steps of 64 rows of M.
 // Waves 2 x 2, each 64 x 64.  Fragment row r16 of sub-tile j maps to column
 // 4 * r16 + j of the wave's 64-wide range (the order the register transpose

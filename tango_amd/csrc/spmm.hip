@@ -13,9 +13,12 @@
 //     row with 16-, 4- or 1-byte loads per lane, so one load instruction of
 //     the wavefront pulls 64/lpe neighbour rows (F = 256 -> 4 rows of 256 B,
 //     F = 16 -> 64 rows);
-//   * bytes are added into int32 lane accumulators with v_dot4 against a
-//     one-hot (copy_u) or weight-carrying (u_mul_e) byte mask: one VALU op per
-//     byte, exact integer arithmetic, order-independent;
+//   * a lane always has four gathers (four neighbours, same columns) in flight;
+//     their dwords are byte-transposed with v_perm and added into int32 lane
+//     accumulators four neighbours at a time with one v_dot4 against a byte
+//     vector of multipliers (1 for copy_u, the int8 edge values for u_mul_e,
+//     0 for slots past the row's end): 0.75 VALU ops per gathered byte, exact
+//     integer arithmetic, order-independent;
 //   * the lane groups are folded with ds_bpermute shuffles, the waves of a
 //     workgroup through LDS, and the row leaves as fp32 = scale * float(sum).
 #include "common.hpp"
@@ -35,16 +38,27 @@ struct SpmmParams {
     const float* bias;       // optional: bias[c] added after the row scale
     int relu;                // clamp at zero last
     int64_t rows;
+    int64_t num_src;  // rows of the gathered matrix
     int64_t ldf;  // bytes between gathered rows
     int64_t W;    // bytes summed per gathered row (H * F)
     int64_t F;    // bytes per head
     int64_t D;    // edge-value width (1 or F)
     int64_t nnz;
     int lpe_log2;  // log2(lanes per gathered row)
+    int ldf_shift; // log2(ldf) when ldf is a power of two and all byte offsets fit 31 bits, else -1
     int out_vec;   // out rows may be stored as 16-byte vectors
 };
 
 enum { KIND_COPY = 0, KIND_WEIGHTED = 1, KIND_COO = 2 };
+
+struct SpmmParams;
+__device__ __forceinline__ int64_t row_offset(int j, const SpmmParams& p);
+
+// Byte offset of gathered row j: a shift when the row pitch allows (64-bit multiplies are quarter rate).
+__device__ __forceinline__ int64_t row_offset(int j, const SpmmParams& p) {
+    return p.ldf_shift >= 0 ? static_cast<int64_t>(static_cast<uint32_t>(j) << p.ldf_shift)
+                            : static_cast<int64_t>(j) * p.ldf;
+}
 
 template <int VEC>
 struct Gather;
@@ -67,31 +81,37 @@ struct Gather<1> {
     static __device__ __forceinline__ T zero() { return 0; }
 };
 
-__device__ __forceinline__ void acc_dword(int* acc, uint32_t d, uint32_t m0) {
-    // m0 holds the multiplier (1 for copy_u, the int8 edge value otherwise) in byte 0
-    acc[0] = __builtin_amdgcn_sdot4(static_cast<int>(d), static_cast<int>(m0), acc[0], false);
-    acc[1] = __builtin_amdgcn_sdot4(static_cast<int>(d), static_cast<int>(m0 << 8), acc[1], false);
-    acc[2] = __builtin_amdgcn_sdot4(static_cast<int>(d), static_cast<int>(m0 << 16), acc[2], false);
-    acc[3] = __builtin_amdgcn_sdot4(static_cast<int>(d), static_cast<int>(m0 << 24), acc[3], false);
-}
-
+// Accumulates the four gathered pieces d[0..3] (same columns, four different neighbours) into the
+// lane's int32 column sums.  Each group of four dwords is transposed with v_perm so that one dword
+// holds ONE column of FOUR neighbours, and a single v_dot4 against `m` adds all four: byte u of `m`
+// is neighbour u's multiplier (1, 0 for an invalid slot, or the int8 edge value of u_mul_e).
+// 8 v_perm + 4 v_dot4 per 16 gathered bytes, instead of 16 v_dot4 with one-hot masks.
 template <int VEC>
-__device__ __forceinline__ void accumulate(int* acc, typename Gather<VEC>::T d, int w);
+__device__ __forceinline__ void accumulate4(int* acc, const typename Gather<VEC>::T* d, uint32_t m);
 template <>
-__device__ __forceinline__ void accumulate<16>(int* acc, u32x4 d, int w) {
-    const uint32_t m0 = static_cast<uint32_t>(w) & 0xffu;
-    acc_dword(acc + 0, d.x, m0);
-    acc_dword(acc + 4, d.y, m0);
-    acc_dword(acc + 8, d.z, m0);
-    acc_dword(acc + 12, d.w, m0);
+__device__ __forceinline__ void accumulate4<16>(int* acc, const u32x4* d, uint32_t m) {
+#pragma unroll
+    for (int w = 0; w < 4; ++w) {
+        uint32_t c[4];
+        transpose4x4(d[0][w], d[1][w], d[2][w], d[3][w], c);
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+            acc[4 * w + j] = __builtin_amdgcn_sdot4(static_cast<int>(c[j]), static_cast<int>(m), acc[4 * w + j], false);
+    }
 }
 template <>
-__device__ __forceinline__ void accumulate<4>(int* acc, uint32_t d, int w) {
-    acc_dword(acc, d, static_cast<uint32_t>(w) & 0xffu);
+__device__ __forceinline__ void accumulate4<4>(int* acc, const uint32_t* d, uint32_t m) {
+    uint32_t c[4];
+    transpose4x4(d[0], d[1], d[2], d[3], c);
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+        acc[j] = __builtin_amdgcn_sdot4(static_cast<int>(c[j]), static_cast<int>(m), acc[j], false);
 }
 template <>
-__device__ __forceinline__ void accumulate<1>(int* acc, int d, int w) {
-    acc[0] += d * w;
+__device__ __forceinline__ void accumulate4<1>(int* acc, const int* d, uint32_t m) {
+#pragma unroll
+    for (int u = 0; u < 4; ++u)
+        acc[0] += d[u] * static_cast<int>(static_cast<int8_t>(m >> (8 * u)));
 }
 
 __device__ __forceinline__ int64_t lower_bound_i64(const int64_t* a, int64_t n, int64_t key) {
@@ -189,27 +209,20 @@ __global__ __launch_bounds__(256) void spmm_kernel(const SpmmParams p) {
                 }
             }
             typename Gather<VEC>::T d[U];
-            int w[U];
-            bool ok[U];
+            uint32_t m = 0u;  // byte u: multiplier of neighbour u (0 = slot not valid)
 #pragma unroll
             for (int u = 0; u < U; ++u) {
-                ok[u] = (t + u) < total && j[u] >= 0;
-                // invalid slots read row 0 and are zeroed afterwards: no branch around the load
-                d[u] = Gather<VEC>::load(fcol + static_cast<int64_t>(ok[u] ? j[u] : 0) * p.ldf);
-                w[u] = 1;
+                const bool ok = (t + u) < total && j[u] >= 0;
+                // invalid slots read row 0 with multiplier 0: no branch around the load
+                d[u] = Gather<VEC>::load(fcol + row_offset(ok ? j[u] : 0, p));
+                uint32_t w = 1u;
                 if (KIND == KIND_WEIGHTED) {
                     const int64_t e = p.edge_ids ? static_cast<int64_t>(sl[u]) : start + sl[u];
-                    w[u] = static_cast<int>(wbase[ok[u] ? e : 0]);
+                    w = static_cast<uint32_t>(static_cast<uint8_t>(wbase[ok ? e : 0]));
                 }
+                m |= (ok ? w : 0u) << (8 * u);
             }
-#pragma unroll
-            for (int u = 0; u < U; ++u) {
-                if (KIND == KIND_WEIGHTED) {
-                    accumulate<VEC>(acc, d[u], ok[u] ? w[u] : 0);
-                } else {
-                    accumulate<VEC>(acc, ok[u] ? d[u] : Gather<VEC>::zero(), 1);
-                }
-            }
+            accumulate4<VEC>(acc, d, m);
         }
     }
 
@@ -271,6 +284,11 @@ static int launch_spmm(SpmmParams p, int vec, hipStream_t s) {
     const int64_t lanes = ceil_div(p.W, vec);
     p.lpe_log2 = lanes >= 64 ? 6 : ilog2_ceil(lanes);
     p.out_vec = (reinterpret_cast<uintptr_t>(p.out) & 15) == 0 && (p.W & 3) == 0;
+    p.ldf_shift = -1;
+    if (p.ldf > 0 && (p.ldf & (p.ldf - 1)) == 0 && p.num_src * p.ldf < (1LL << 31)) {
+        p.ldf_shift = 0;
+        while ((1LL << p.ldf_shift) < p.ldf) ++p.ldf_shift;
+    }
     const int64_t ychunks = ceil_div(p.W, 64 * vec);
     if (ychunks > 65535) return TANGO_ERR_UNSUPPORTED;
     // four waves split each row when rows are long AND wide (few neighbours per load instruction);
@@ -316,7 +334,7 @@ int tango_spmm_csr_copy_u(float* out, const int64_t* indptr, const int64_t* indi
     if (num_src >= (1LL << 31) || nnz >= (1LL << 31)) return TANGO_ERR_UNSUPPORTED;
     SpmmParams p{};
     p.out = out; p.indptr = indptr; p.indices = indices; p.feat = feat; p.scale = scale;
-    p.rows = rows; p.ldf = ldf; p.W = F; p.F = F; p.D = 1; p.nnz = nnz;
+    p.rows = rows; p.num_src = num_src; p.ldf = ldf; p.W = F; p.F = F; p.D = 1; p.nnz = nnz;
     return launch_spmm<KIND_COPY>(p, pick_vec(feat, ldf, F), as_stream(stream));
 }
 
@@ -331,7 +349,7 @@ int tango_spmm_csr_copy_u_ex(float* out, const int64_t* indptr, const int64_t* i
     SpmmParams p{};
     p.out = out; p.indptr = indptr; p.indices = indices; p.feat = feat; p.scale = scale;
     p.row_scale = row_scale; p.bias = bias; p.relu = relu ? 1 : 0;
-    p.rows = rows; p.ldf = ldf; p.W = F; p.F = F; p.D = 1; p.nnz = nnz;
+    p.rows = rows; p.num_src = num_src; p.ldf = ldf; p.W = F; p.F = F; p.D = 1; p.nnz = nnz;
     return launch_spmm<KIND_COPY>(p, pick_vec(feat, ldf, F), as_stream(stream));
 }
 
@@ -346,7 +364,7 @@ int tango_spmm_csr_u_mul_e(float* out, const int64_t* indptr, const int64_t* ind
     if (num_src >= (1LL << 31) || nnz >= (1LL << 31)) return TANGO_ERR_UNSUPPORTED;
     SpmmParams p{};
     p.out = out; p.indptr = indptr; p.indices = indices; p.edge_ids = edge_ids; p.feat = feat;
-    p.evals = evals; p.scale = scale; p.rows = rows; p.ldf = H * F; p.W = H * F; p.F = F; p.D = D;
+    p.evals = evals; p.scale = scale; p.rows = rows; p.num_src = num_src; p.ldf = H * F; p.W = H * F; p.F = F; p.D = D;
     p.nnz = nnz;
     // a lane's bytes must share one edge value: vector loads only when they stay inside a head
     int vec = 1;
@@ -367,7 +385,7 @@ int tango_spmm_incidence(float* out, const int64_t* node_ids, const int64_t* edg
     if (num_edges >= (1LL << 31) || nnz >= (1LL << 31)) return TANGO_ERR_UNSUPPORTED;
     SpmmParams p{};
     p.out = out; p.node_ids = node_ids; p.indices = edge_ids; p.feat = E; p.scale = scale;
-    p.rows = num_nodes; p.ldf = F; p.W = F; p.F = F; p.D = 1; p.nnz = nnz;
+    p.rows = num_nodes; p.num_src = num_edges; p.ldf = F; p.W = F; p.F = F; p.D = 1; p.nnz = nnz;
     return launch_spmm<KIND_COO>(p, pick_vec(E, F, F), as_stream(stream));
 }
 
