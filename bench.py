@@ -273,6 +273,7 @@ def main():
     from tango_amd import config, kernels as K
     from tango_amd.gcn import GCN
     from tango_amd.graph import chung_lu
+    from tango_amd.loss import cross_entropy
     from tango_amd.util import graph_preprocess
 
     torch.cuda.set_device(0)
@@ -315,7 +316,7 @@ def main():
         raw_spmm, lambda out, *a, **kw: "spmm_F%d" % (out.size(1))))
 
     def step():
-        loss = torch.nn.functional.cross_entropy(model(X), labels)
+        loss = cross_entropy(model(X), labels)
         opt.zero_grad(set_to_none=True)
         loss.backward()
         opt.step()

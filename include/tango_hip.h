@@ -245,6 +245,19 @@ int tango_edge_softmax_bwd(float* de, const float* a, const float* da, const flo
                            const int64_t* indptr, const int64_t* edge_ids, int64_t rows,
                            int64_t H, float slope, tango_stream_t stream);
 
+/* -------------------------------------------------------------------- loss */
+
+/* Softmax cross-entropy with mean reduction and its gradient in one pass (no
+   counterpart in the reference's native code: its drivers call torch's
+   F.cross_entropy, evaluation/test_gcn.py:256).  logits [rows, classes] fp32 (row
+   stride ld), labels int64 [rows]; loss_out[0] = mean_r(-log softmax(logits[r])[labels[r]]),
+   grad_out[r, c] = (softmax(logits[r])[c] - (c == labels[r])) / rows.  classes <= 256.
+   The loss is reduced in a fixed order.  workspace: tango_softmax_xent_workspace(rows) bytes. */
+size_t tango_softmax_xent_workspace(int64_t rows);
+int tango_softmax_xent_f32(const float* logits, int64_t ld, const int64_t* labels, int64_t rows,
+                           int64_t classes, float* loss_out, float* grad_out, int64_t ldg,
+                           void* workspace, size_t workspace_bytes, tango_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -113,3 +113,20 @@ def test_fused_gcn_matches_unfused(dims):
             assert torch.allclose(pa.grad, pb.grad, rtol=1e-4, atol=1e-4), name
         else:
             assert torch.equal(pa.grad, pb.grad), name
+
+
+@pytest.mark.parametrize("rows,classes", [(1000, 41), (4097, 7), (300, 256), (17, 3), (5, 1)])
+def test_cross_entropy_matches_torch(rows, classes):
+    from tango_amd.loss import cross_entropy
+    torch.manual_seed(rows)
+    x = (torch.randn(rows, classes, device="cuda") * 3).requires_grad_(True)
+    y = torch.randint(0, classes, (rows,), device="cuda")
+    loss = cross_entropy(x, y)
+    xr = x.detach().clone().requires_grad_(True)
+    ref = torch.nn.functional.cross_entropy(xr, y)
+    assert torch.allclose(loss, ref, rtol=1e-5, atol=1e-6)
+    (loss * 2.5).backward()
+    (ref * 2.5).backward()
+    assert torch.allclose(x.grad, xr.grad, rtol=1e-5, atol=1e-8)
+    # deterministic
+    assert cross_entropy(x.detach(), y).item() == cross_entropy(x.detach(), y).item()
