@@ -206,6 +206,16 @@ int tango_spmm_csr_u_mul_e(float* out, const int64_t* indptr, const int64_t* ind
                            const float* scale, int64_t rows, int64_t num_src, int64_t H,
                            int64_t F, int64_t D, int64_t nnz, tango_stream_t stream);
 
+/* As tango_spmm_csr_u_mul_e with a choice of layout for the edge values (no
+   counterpart in the reference): edge_major != 0 means evals is [nnz, H, D] (what
+   quantizing the [nnz, H, D] fp32 edge tensor in place yields, no transpose pass).
+   With the slot->edge permutation fused, the H * D bytes of a gathered edge then
+   come from one cache sector instead of H * D scattered ones. */
+int tango_spmm_csr_u_mul_e_ex(float* out, const int64_t* indptr, const int64_t* indices,
+                              const int64_t* edge_ids, const int8_t* feat, const int8_t* evals,
+                              int edge_major, const float* scale, int64_t rows, int64_t num_src,
+                              int64_t H, int64_t F, int64_t D, int64_t nnz, tango_stream_t stream);
+
 /* incidence_SPMM (cuda/src/cuda.cpp:160-167 -> incidence_SPMM_impl, SPMM.cu:259-303):
    out[v, f] = scale[0] * float(sum_{i: node_ids[i] == v} E[edge_ids[i], f]).
    (node_ids, edge_ids) are the COO rows of the incidence matrix and must be

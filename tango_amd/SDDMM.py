@@ -63,12 +63,10 @@ class sddmm_u_dot_v(Function):
         dZ3 = dZ.unsqueeze(1) if squeeze else dZ  # [E, H, 1]
         U3 = U_.unsqueeze(1) if U_.dim() == 2 else U_
         V3 = V_.unsqueeze(1) if V_.dim() == 2 else V_
-        from .kernels import cuda_kernels
-        scaledZ = cuda_kernels.get_scale(dZ3)
-        dZ_T = transpose_quant(dZ3, scaledZ)  # [H, 1, E], half-to-even
+        dZ_, scaledZ = _quantize_grad(dZ3)  # [E, H, 1], edge-major edge values
         dU = dV = None
         if ctx.needs_input_grad[1]:
-            dU = multi_cusparse_SPMM(g, V3, dZ_T, scaledZ * scaleV, True).reshape(U_.shape)
+            dU = multi_cusparse_SPMM(g, V3, dZ_, scaledZ * scaleV, True, edge_major=True).reshape(U_.shape)
         if ctx.needs_input_grad[2]:
-            dV = multi_cusparse_SPMM(g, U3, dZ_T, scaledZ * scaleU).reshape(V_.shape)
+            dV = multi_cusparse_SPMM(g, U3, dZ_, scaledZ * scaleU, edge_major=True).reshape(V_.shape)
         return None, dU, dV

@@ -90,11 +90,13 @@ class spmm_u_mul_e(Function):
     def forward(ctx, g, N, E):
         N = N if N.is_contiguous() else N.contiguous()
         E = E if E.is_contiguous() else E.contiguous()
-        scaleE = cuda_kernels.get_scale(E)
-        E_T_ = transpose_quant(E, scaleE)
+        # Edge values stay edge-major ([nnz, H, 1], plain quantize): the reference transposes them to
+        # [H, 1, nnz] (cuda/SPMM.py:41) and then permutes that with index_select; with the permutation
+        # fused into the gather, edge-major keeps the H bytes of an edge in one cache sector.
+        E_T_, scaleE = quantize(E)
         N_, scaleN = quantize(N)  # one absmax pass (the reference runs two, cuda/SPMM.py:39,43)
         scale = scaleN * scaleE
-        out = multi_cusparse_SPMM(g, N_, E_T_, scale)
+        out = multi_cusparse_SPMM(g, N_, E_T_, scale, edge_major=True)
         reduce_last = _need_reduce_last_dim(N, E)
         ctx.backward_cache = g, N_, scaleN, E_T_, scaleE, scale, reduce_last, E.shape
         return out
@@ -109,7 +111,7 @@ class spmm_u_mul_e(Function):
             # dN = A^T (E * dZ): the dequantization scale is s_dZ * s_E.  The reference passes
             # the forward scale s_N * s_E here (cuda/SPMM.py:56); ref_compat reproduces that.
             bscale = scale if config.ref_compat else scaledZ * scaleE
-            dN = multi_cusparse_SPMM(g, dZ_, E_T_, bscale, True)
+            dN = multi_cusparse_SPMM(g, dZ_, E_T_, bscale, True, edge_major=True)
         if ctx.needs_input_grad[2]:
             op = "dot" if reduce_last else "mul"
             dE, _ = mySDDMM_int8(g, op, N_, dZ_, scaleN, scaledZ, False)

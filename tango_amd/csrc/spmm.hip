@@ -43,6 +43,7 @@ struct SpmmParams {
     int64_t W;    // bytes summed per gathered row (H * F)
     int64_t F;    // bytes per head
     int64_t D;    // edge-value width (1 or F)
+    int64_t ev_sh, ev_sd, ev_se;  // strides (bytes) of evals over head, value column, edge
     int64_t nnz;
     int lpe_log2;  // log2(lanes per gathered row)
     int ldf_shift; // log2(ldf) when ldf is a power of two and all byte offsets fit 31 bits, else -1
@@ -162,7 +163,7 @@ __global__ __launch_bounds__(256) void spmm_kernel(const SpmmParams p) {
     if (KIND == KIND_WEIGHTED && col_ok) {
         const int64_t h = col / p.F;
         const int64_t d = (p.D == 1) ? 0 : (col - h * p.F);
-        wbase = p.evals + (h * p.D + d) * p.nnz;
+        wbase = p.evals + h * p.ev_sh + d * p.ev_sd;
     }
 
     int acc[VEC];
@@ -218,7 +219,7 @@ __global__ __launch_bounds__(256) void spmm_kernel(const SpmmParams p) {
                 uint32_t w = 1u;
                 if (KIND == KIND_WEIGHTED) {
                     const int64_t e = p.edge_ids ? static_cast<int64_t>(sl[u]) : start + sl[u];
-                    w = static_cast<uint32_t>(static_cast<uint8_t>(wbase[ok ? e : 0]));
+                    w = static_cast<uint32_t>(static_cast<uint8_t>(wbase[(ok ? e : 0) * p.ev_se]));
                 }
                 m |= (ok ? w : 0u) << (8 * u);
             }
@@ -353,10 +354,10 @@ int tango_spmm_csr_copy_u_ex(float* out, const int64_t* indptr, const int64_t* i
     return launch_spmm<KIND_COPY>(p, pick_vec(feat, ldf, F), as_stream(stream));
 }
 
-int tango_spmm_csr_u_mul_e(float* out, const int64_t* indptr, const int64_t* indices,
-                           const int64_t* edge_ids, const int8_t* feat, const int8_t* evals,
-                           const float* scale, int64_t rows, int64_t num_src, int64_t H,
-                           int64_t F, int64_t D, int64_t nnz, tango_stream_t stream) {
+int tango_spmm_csr_u_mul_e_ex(float* out, const int64_t* indptr, const int64_t* indices,
+                              const int64_t* edge_ids, const int8_t* feat, const int8_t* evals,
+                              int edge_major, const float* scale, int64_t rows, int64_t num_src,
+                              int64_t H, int64_t F, int64_t D, int64_t nnz, tango_stream_t stream) {
     if (rows < 0 || H < 0 || F < 0 || nnz < 0 || num_src < 0 || !scale || !indptr ||
         (rows * H * F > 0 && !out) || (nnz > 0 && (!indices || !feat || !evals)))
         return TANGO_ERR_INVALID_ARG;
@@ -366,6 +367,11 @@ int tango_spmm_csr_u_mul_e(float* out, const int64_t* indptr, const int64_t* ind
     p.out = out; p.indptr = indptr; p.indices = indices; p.edge_ids = edge_ids; p.feat = feat;
     p.evals = evals; p.scale = scale; p.rows = rows; p.num_src = num_src; p.ldf = H * F; p.W = H * F; p.F = F; p.D = D;
     p.nnz = nnz;
+    if (edge_major) {  // evals[nnz, H, D]: the H * D bytes of one edge share a cache sector
+        p.ev_se = H * D; p.ev_sh = D; p.ev_sd = 1;
+    } else {           // evals[H, D, nnz], the reference's transposed layout
+        p.ev_se = 1; p.ev_sh = D * nnz; p.ev_sd = nnz;
+    }
     // a lane's bytes must share one edge value: vector loads only when they stay inside a head
     int vec = 1;
     if (D == 1 && F > 0) {
@@ -374,6 +380,14 @@ int tango_spmm_csr_u_mul_e(float* out, const int64_t* indptr, const int64_t* ind
         else if ((F & 3) == 0 && (a & 3) == 0) vec = 4;
     }
     return launch_spmm<KIND_WEIGHTED>(p, vec, as_stream(stream));
+}
+
+int tango_spmm_csr_u_mul_e(float* out, const int64_t* indptr, const int64_t* indices,
+                           const int64_t* edge_ids, const int8_t* feat, const int8_t* evals,
+                           const float* scale, int64_t rows, int64_t num_src, int64_t H,
+                           int64_t F, int64_t D, int64_t nnz, tango_stream_t stream) {
+    return tango_spmm_csr_u_mul_e_ex(out, indptr, indices, edge_ids, feat, evals, 0, scale, rows, num_src, H, F,
+                                     D, nnz, stream);
 }
 
 int tango_spmm_incidence(float* out, const int64_t* node_ids, const int64_t* edge_ids,

@@ -339,9 +339,10 @@ class cuda_kernels:
                                           rows, U.size(0), indices.numel(), F, _stream()), "csr_SPMM")
 
     @staticmethod
-    def multi_cusparse_SPMM(indptr, indices, N, E_T, scale, edge_ids=None):
+    def multi_cusparse_SPMM(indptr, indices, N, E_T, scale, edge_ids=None, edge_major=False):
         """E_T is [H, D, nnz] in CSR slot order, or in edge-id order when the
-        slot->edge permutation ``edge_ids`` is passed (gather fused in-kernel)."""
+        slot->edge permutation ``edge_ids`` is passed (gather fused in-kernel).
+        With ``edge_major`` the edge values are [nnz, H, D] instead (no transpose pass)."""
         _need(indptr, torch.int64, "indptr")
         _need(indices, torch.int64, "indices")
         _need(N, torch.int8, "N")
@@ -350,16 +351,21 @@ class cuda_kernels:
         if N.dim() != 3 or E_T.dim() != 3:
             raise RuntimeError("E and N must be 3D tensors")
         k, H, F = N.shape
-        D, nnz = E_T.size(1), E_T.size(2)
-        if E_T.size(0) != H or nnz != indices.numel() or D not in (1, F):
-            raise RuntimeError("multi_cusparse_SPMM: E_T must be [H, 1|F, nnz]")
+        if edge_major:
+            nnz, D = E_T.size(0), E_T.size(2)
+            if E_T.size(1) != H or nnz != indices.numel() or D not in (1, F):
+                raise RuntimeError("multi_cusparse_SPMM: edge-major E must be [nnz, H, 1|F]")
+        else:
+            D, nnz = E_T.size(1), E_T.size(2)
+            if E_T.size(0) != H or nnz != indices.numel() or D not in (1, F):
+                raise RuntimeError("multi_cusparse_SPMM: E_T must be [H, 1|F, nnz]")
         if edge_ids is not None:
             _need(edge_ids, torch.int64, "edge_ids")
         rows = indptr.numel() - 1
         out = torch.empty((rows, H, F), dtype=torch.float32, device=N.device)
-        check(_L.tango_spmm_csr_u_mul_e(_ptr(out), indptr.data_ptr(), _ptr(indices), _ptr(edge_ids),
-                                        _ptr(N), _ptr(E_T), scale.data_ptr(), rows, k, H, F, D, nnz,
-                                        _stream()), "multi_cusparse_SPMM")
+        check(_L.tango_spmm_csr_u_mul_e_ex(_ptr(out), indptr.data_ptr(), _ptr(indices), _ptr(edge_ids),
+                                           _ptr(N), _ptr(E_T), int(bool(edge_major)), scale.data_ptr(), rows,
+                                           k, H, F, D, nnz, _stream()), "multi_cusparse_SPMM")
         return out
 
     # The reference's SpMV binding returns uninitialised memory (cuda/src/SPMM.cu:196-257)
@@ -544,18 +550,20 @@ def transpose_quant(data, scale):
     return data_.reshape((data.size(1), data.size(2), nrow))
 
 
-def multi_cusparse_SPMM(g, N, E_T, scale, reverse=False):
+def multi_cusparse_SPMM(g, N, E_T, scale, reverse=False, edge_major=False):
     """E_T is [H, D, nnz] in edge-id order.  cuda/kernels.py:122-136; the
-    index_select by edge_ids of the reference happens inside the kernel."""
+    index_select by edge_ids of the reference happens inside the kernel.
+    ``edge_major``: E_T is the quantized edge tensor as it is, [nnz, H, 1]."""
     assert E_T.ndim == 3 and N.ndim == 3, "E and N must be 3D tensors"
-    assert E_T.size(1) == 1, "Cannot broadcast E"
+    assert E_T.size(2 if edge_major else 1) == 1, "Cannot broadcast E"
     if reverse:
         indptr, indices, edge_ids = g.adj_csr
     else:
         indptr, indices, edge_ids = g.adj_csc
     if edge_ids is not None and edge_ids.numel() == 0:
         edge_ids = None
-    return cuda_kernels.multi_cusparse_SPMM(indptr, indices, N, E_T, scale, edge_ids=edge_ids)
+    return cuda_kernels.multi_cusparse_SPMM(indptr, indices, N, E_T, scale, edge_ids=edge_ids,
+                                            edge_major=edge_major)
 
 
 def incidence_SPMM(g, E, scaleE, reverse=False):

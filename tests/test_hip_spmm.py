@@ -96,7 +96,12 @@ def test_u_mul_e_broadcast(K, orc, kind, n, e, H, F):
     for reverse, fmt in ((False, "adj_csc"), (True, "adj_csr")):
         got = K.multi_cusparse_SPMM(g, dev(feat), dev(ev), sc(s), reverse=reverse)
         ip, ix, eid = o[fmt]
-        assert np.array_equal(host(got), orc.spmm_csr_u_mul_e(ip, ix, eid, feat, ev, s))
+        want = orc.spmm_csr_u_mul_e(ip, ix, eid, feat, ev, s)
+        assert np.array_equal(host(got), want)
+        # the same edge values laid out [nnz, H, 1] (no transpose pass before the SpMM)
+        ev_major = dev(np.ascontiguousarray(ev.transpose(2, 0, 1)))
+        got_major = K.multi_cusparse_SPMM(g, dev(feat), ev_major, sc(s), reverse=reverse, edge_major=True)
+        assert np.array_equal(host(got_major), want)
     # binding-level call with edge values already in CSR slot order (the reference's calling convention)
     ip, ix, eid = g.adj_csc
     ev_sorted = dev(ev[:, :, o["adj_csc"][2]])
@@ -115,7 +120,11 @@ def test_u_mul_e_elementwise(K, orc):
     ev = rng.integers(-127, 128, (H, F, e)).astype(np.int8)
     ip, ix, eid = g.adj_csc
     got = K.cuda_kernels.multi_cusparse_SPMM(ip, ix, dev(feat), dev(ev), sc(0.01), edge_ids=eid)
-    assert np.array_equal(host(got), orc.spmm_csr_u_mul_e(*o["adj_csc"], feat, ev, 0.01))
+    want = orc.spmm_csr_u_mul_e(*o["adj_csc"], feat, ev, 0.01)
+    assert np.array_equal(host(got), want)
+    ev_major = dev(np.ascontiguousarray(ev.transpose(2, 0, 1)))  # [nnz, H, F]
+    got = K.cuda_kernels.multi_cusparse_SPMM(ip, ix, dev(feat), ev_major, sc(0.01), edge_ids=eid, edge_major=True)
+    assert np.array_equal(host(got), want)
 
 
 @pytest.mark.parametrize("F", [1, 8, 16, 20, 64])
