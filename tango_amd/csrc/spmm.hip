@@ -48,6 +48,7 @@ struct SpmmParams {
     int lpe_log2;  // log2(lanes per gathered row)
     int ldf_shift; // log2(ldf) when ldf is a power of two and all byte offsets fit 31 bits, else -1
     int out_vec;   // out rows may be stored as 16-byte vectors
+    int64_t long_row;  // rows with more slots than this go to the sixteen-wave kernel
 };
 
 enum { KIND_COPY = 0, KIND_WEIGHTED = 1, KIND_COO = 2 };
@@ -124,56 +125,47 @@ __device__ __forceinline__ int64_t lower_bound_i64(const int64_t* a, int64_t n, 
     return lo;
 }
 
-// blockDim.x = 256.  WPR = waves that share one output row (1 or 4).
-// gridDim.y tiles the columns in chunks of 64 * VEC bytes.
-template <int VEC, int WPR, int KIND>
-__global__ __launch_bounds__(256) void spmm_kernel(const SpmmParams p) {
+// Per-lane view of the column tile a lane works on.
+struct LaneCols {
+    int lpe, epi, grp, sub, sh;
+    int64_t col;
+    bool col_ok;
+    const int8_t* fcol;   // feat + col (column 0 for lanes past the row's width)
+    const int8_t* wbase;  // weighted kind: evals + this lane's head / value-column offset
+};
+
+template <int VEC, int KIND>
+__device__ __forceinline__ LaneCols lane_cols(const SpmmParams& p, int lane) {
+    LaneCols c;
+    c.lpe = 1 << p.lpe_log2;
+    c.epi = kWave >> p.lpe_log2;
+    c.grp = lane >> p.lpe_log2;
+    c.sub = lane & (c.lpe - 1);
+    c.sh = 6 - p.lpe_log2;
+    c.col = static_cast<int64_t>(blockIdx.y) * (kWave * VEC) + static_cast<int64_t>(c.sub) * VEC;
+    c.col_ok = c.col < p.W;
+    // Lanes past the row's width read column 0 (a valid address) and never store, and the
+    // group fold only mixes lanes of equal `sub`, so they need no masking.
+    c.fcol = p.feat + (c.col_ok ? c.col : 0);
+    c.wbase = p.evals;
+    if (KIND == KIND_WEIGHTED && c.col_ok) {
+        const int64_t h = c.col / p.F;
+        const int64_t d = (p.D == 1) ? 0 : (c.col - h * p.F);
+        c.wbase = p.evals + h * p.ev_sh + d * p.ev_sd;
+    }
+    return c;
+}
+
+// One wavefront sums the gathered rows of CSR slots [start, end) (row_start is the row's first
+// slot: edge values in slot order are addressed relative to the whole array).  On return lanes
+// [0, lpe) hold the column sums of the lane's VEC columns.
+template <int VEC, int KIND>
+__device__ __forceinline__ void wave_row_sum(const SpmmParams& p, const LaneCols& c, int lane, int64_t start,
+                                             int64_t end, int* acc) {
     constexpr int U = 4;  // gather loads in flight per lane
-    const int lane = lane_id();
-    const int wave = __builtin_amdgcn_readfirstlane(static_cast<int>(threadIdx.x) >> 6);
-    const int64_t row = (WPR == 4) ? static_cast<int64_t>(blockIdx.x)
-                                   : static_cast<int64_t>(blockIdx.x) * 4 + wave;
-    __shared__ int part[(WPR == 4) ? 3 * 64 * VEC : 1];
-    if (WPR == 1 && row >= p.rows) return;  // whole wave leaves; no barrier follows for WPR == 1
-
-    const int lpe = 1 << p.lpe_log2;
-    const int epi = kWave >> p.lpe_log2;
-    const int grp = lane >> p.lpe_log2;
-    const int sub = lane & (lpe - 1);
-    const int64_t col = static_cast<int64_t>(blockIdx.y) * (kWave * VEC) + static_cast<int64_t>(sub) * VEC;
-    const bool col_ok = col < p.W;
-
-    int64_t start, end;
-    if (KIND == KIND_COO) {
-        start = lower_bound_i64(p.node_ids, p.nnz, row);
-        end = lower_bound_i64(p.node_ids, p.nnz, row + 1);
-    } else {
-        start = p.indptr[row];
-        end = p.indptr[row + 1];
-    }
-    if (WPR == 4) {
-        const int64_t per = (end - start + 3) >> 2;
-        const int64_t s = start + per * wave;
-        const int64_t e = s + per;
-        start = s < end ? s : end;
-        end = e < end ? e : end;
-    }
-
-    const int8_t* wbase = p.evals;
-    if (KIND == KIND_WEIGHTED && col_ok) {
-        const int64_t h = col / p.F;
-        const int64_t d = (p.D == 1) ? 0 : (col - h * p.F);
-        wbase = p.evals + h * p.ev_sh + d * p.ev_sd;
-    }
-
-    int acc[VEC];
+    const int lpe = c.lpe, epi = c.epi, grp = c.grp, sh = c.sh;
 #pragma unroll
     for (int i = 0; i < VEC; ++i) acc[i] = 0;
-
-    // Lanes past the row's width read column 0 (a valid address) and never store, and the
-    // fold below only mixes lanes of equal `sub`, so they need no masking.
-    const int8_t* fcol = p.feat + (col_ok ? col : 0);
-    const int sh = 6 - p.lpe_log2;
 
     // Indices are fetched 256 slots at a time with four independent coalesced loads
     // (lane i of load r holds slot 64 r + i), so one HBM round trip is paid per 256 edges.
@@ -195,18 +187,20 @@ __global__ __launch_bounds__(256) void spmm_kernel(const SpmmParams p) {
         const int cnt = static_cast<int>((end - base) < 4 * kWave ? (end - base) : 4 * kWave);
         const int total = (cnt + epi - 1) >> sh;
         for (int t = 0; t < total; t += U) {
-            int j[U], sl[U];
+            int j[U];
+            int64_t sl[U];
 #pragma unroll
             for (int u = 0; u < U; ++u) {
                 const int tt = t + u;
                 const int r = (tt >> p.lpe_log2) & 3;  // which of the four index registers (wave-uniform)
-                sl[u] = ((tt & (lpe - 1)) << sh) + grp;
+                const int slot = ((tt & (lpe - 1)) << sh) + grp;
                 const int reg = r == 0 ? my[0] : r == 1 ? my[1] : r == 2 ? my[2] : my[3];
-                j[u] = __shfl(reg, sl[u], kWave);
+                j[u] = __shfl(reg, slot, kWave);
+                sl[u] = 0;
                 if (KIND == KIND_WEIGHTED) {
                     const int rege = r == 0 ? my_e[0] : r == 1 ? my_e[1] : r == 2 ? my_e[2] : my_e[3];
                     // position of this slot's edge value: permuted id, or the CSR slot itself
-                    sl[u] = p.edge_ids ? __shfl(rege, sl[u], kWave) : static_cast<int>(base - start) + r * kWave + sl[u];
+                    sl[u] = p.edge_ids ? static_cast<int64_t>(__shfl(rege, slot, kWave)) : base + r * kWave + slot;
                 }
             }
             typename Gather<VEC>::T d[U];
@@ -215,12 +209,10 @@ __global__ __launch_bounds__(256) void spmm_kernel(const SpmmParams p) {
             for (int u = 0; u < U; ++u) {
                 const bool ok = (t + u) < total && j[u] >= 0;
                 // invalid slots read row 0 with multiplier 0: no branch around the load
-                d[u] = Gather<VEC>::load(fcol + row_offset(ok ? j[u] : 0, p));
+                d[u] = Gather<VEC>::load(c.fcol + row_offset(ok ? j[u] : 0, p));
                 uint32_t w = 1u;
-                if (KIND == KIND_WEIGHTED) {
-                    const int64_t e = p.edge_ids ? static_cast<int64_t>(sl[u]) : start + sl[u];
-                    w = static_cast<uint32_t>(static_cast<uint8_t>(wbase[(ok ? e : 0) * p.ev_se]));
-                }
+                if (KIND == KIND_WEIGHTED)
+                    w = static_cast<uint32_t>(static_cast<uint8_t>(c.wbase[(ok ? sl[u] : 0) * p.ev_se]));
                 m |= (ok ? w : 0u) << (8 * u);
             }
             accumulate4<VEC>(acc, d, m);
@@ -232,44 +224,166 @@ __global__ __launch_bounds__(256) void spmm_kernel(const SpmmParams p) {
 #pragma unroll
         for (int i = 0; i < VEC; ++i) acc[i] += __shfl_xor(acc[i], off, kWave);
     }
+}
+
+// Dequantize and store one output row's tile; called by the lanes with grp == 0.
+template <int VEC>
+__device__ __forceinline__ void store_row(const SpmmParams& p, const LaneCols& c, int64_t row, const int* acc) {
+    if (!c.col_ok) return;
+    const float s = p.scale[0];
+    const float rs = p.row_scale ? p.row_scale[row] : 1.0f;
+    float* o = p.out + row * p.W + c.col;
+    float y[VEC];
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) {
+        // same sequence of roundings as dequantize, then "* norm", "+ bias", relu as separate passes
+        y[i] = s * static_cast<float>(acc[i]);
+        if (p.row_scale) y[i] = y[i] * rs;
+        if (p.bias && c.col + i < p.W) y[i] = y[i] + p.bias[c.col + i];
+        if (p.relu) y[i] = fmaxf(y[i], 0.0f);
+    }
+    if (VEC == 16 && p.out_vec && c.col + 16 <= p.W) {
+        f32x4* o4 = reinterpret_cast<f32x4*>(o);
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+            __builtin_nontemporal_store(f32x4{y[4 * i], y[4 * i + 1], y[4 * i + 2], y[4 * i + 3]}, o4 + i);
+    } else {
+#pragma unroll
+        for (int i = 0; i < VEC; ++i)
+            if (c.col + i < p.W) o[i] = y[i];
+    }
+}
+
+template <int KIND>
+__device__ __forceinline__ void row_range(const SpmmParams& p, int64_t row, int64_t& start, int64_t& end) {
+    if (KIND == KIND_COO) {
+        start = lower_bound_i64(p.node_ids, p.nnz, row);
+        end = lower_bound_i64(p.node_ids, p.nnz, row + 1);
+    } else {
+        start = p.indptr[row];
+        end = p.indptr[row + 1];
+    }
+}
+
+// lower_bound by all 64 lanes of a converged wavefront: 64 probes per round, so
+// at most six dependent loads for 2^31 entries instead of 31.
+__device__ __forceinline__ int64_t lower_bound_wave(const int64_t* a, int64_t n, int64_t key, int lane) {
+    int64_t lo = 0, hi = n;  // the answer lies in [lo, hi]
+    while (lo < hi) {
+        const int64_t step = (hi - lo + kWave - 1) >> 6;
+        const int64_t idx = lo + (lane + 1) * step - 1;
+        const bool below = idx < hi && a[idx] < key;
+        const int cnt = __popcll(__ballot(below));  // probes are sorted: the first cnt are below the key
+        const int64_t nlo = lo + cnt * step;
+        const int64_t nhi = lo + (cnt + 1) * step - 1;
+        lo = nlo;
+        hi = nhi < hi ? nhi : hi;
+    }
+    return lo;
+}
+
+// blockDim.x = 256.  WPR = waves that share one output row (1 or 4).
+// gridDim.y tiles the columns in chunks of 64 * VEC bytes.
+// Rows with more than p.long_row slots are left to spmm_long_kernel.
+template <int VEC, int WPR, int KIND>
+__global__ __launch_bounds__(256) void spmm_kernel(const SpmmParams p) {
+    const int lane = lane_id();
+    const int wave = __builtin_amdgcn_readfirstlane(static_cast<int>(threadIdx.x) >> 6);
+    const int64_t row = (WPR == 4) ? static_cast<int64_t>(blockIdx.x)
+                                   : static_cast<int64_t>(blockIdx.x) * 4 + wave;
+    __shared__ int part[(WPR == 4) ? 3 * 64 * VEC : 1];
+    if (WPR == 1 && row >= p.rows) return;  // whole wave leaves; no barrier follows for WPR == 1
+
+    int64_t start, end;
+    if (KIND == KIND_COO) {
+        start = lower_bound_wave(p.node_ids, p.nnz, row, lane);
+        end = lower_bound_wave(p.node_ids, p.nnz, row + 1, lane);
+    } else {
+        row_range<KIND>(p, row, start, end);
+    }
+    if (end - start > p.long_row) return;  // uniform over the workgroup
+    if (WPR == 4) {
+        const int64_t per = (end - start + 3) >> 2;
+        const int64_t s = start + per * wave;
+        const int64_t e = s + per;
+        start = s < end ? s : end;
+        end = e < end ? e : end;
+    }
+
+    const LaneCols c = lane_cols<VEC, KIND>(p, lane);
+    int acc[VEC];
+    wave_row_sum<VEC, KIND>(p, c, lane, start, end, acc);
 
     if (WPR == 4) {
-        if (wave > 0 && grp == 0) {
+        if (wave > 0 && c.grp == 0) {
 #pragma unroll
-            for (int i = 0; i < VEC; ++i) part[(wave - 1) * 64 * VEC + i * 64 + sub] = acc[i];
+            for (int i = 0; i < VEC; ++i) part[(wave - 1) * 64 * VEC + i * 64 + c.sub] = acc[i];
         }
         __syncthreads();
         if (wave > 0) return;
-        if (grp == 0) {
+        if (c.grp == 0) {
 #pragma unroll
             for (int i = 0; i < VEC; ++i)
-                acc[i] += part[i * 64 + sub] + part[64 * VEC + i * 64 + sub] + part[2 * 64 * VEC + i * 64 + sub];
+                acc[i] += part[i * 64 + c.sub] + part[64 * VEC + i * 64 + c.sub] + part[2 * 64 * VEC + i * 64 + c.sub];
         }
     }
+    if (c.grp == 0) store_row<VEC>(p, c, row, acc);
+}
 
-    if (grp == 0 && col_ok) {
-        const float s = p.scale[0];
-        const float rs = p.row_scale ? p.row_scale[row] : 1.0f;
-        float* o = p.out + row * p.W + col;
-        float y[VEC];
-#pragma unroll
-        for (int i = 0; i < VEC; ++i) {
-            // same sequence of roundings as dequantize, then "* norm", "+ bias", relu as separate passes
-            y[i] = s * static_cast<float>(acc[i]);
-            if (p.row_scale) y[i] = y[i] * rs;
-            if (p.bias && col + i < p.W) y[i] = y[i] + p.bias[col + i];
-            if (p.relu) y[i] = fmaxf(y[i], 0.0f);
+// Rows with more than p.long_row slots, sixteen wavefronts per row.  blockDim.x = 1024;
+// workgroup b looks at the 64 rows b, b + G, b + 2G, ... (G = gridDim.x: hub rows with
+// neighbouring ids land in different workgroups), keeps the long ones and sums each with
+// all of its waves; the waves' partial sums meet in LDS through integer atomics, which
+// are exact in any order.
+template <int VEC, int KIND>
+__global__ __launch_bounds__(1024) void spmm_long_kernel(const SpmmParams p) {
+    constexpr int WAVES = 16;
+    __shared__ int part[64 * VEC];
+    __shared__ int64_t list[kWave];
+    __shared__ int nlist;
+    const int lane = lane_id();
+    const int wave = __builtin_amdgcn_readfirstlane(static_cast<int>(threadIdx.x) >> 6);
+    if (wave == 0) {
+        const int64_t r = static_cast<int64_t>(blockIdx.x) + static_cast<int64_t>(lane) * gridDim.x;
+        bool is_long = false;
+        if (r < p.rows) {
+            int64_t s, e;
+            row_range<KIND>(p, r, s, e);
+            is_long = e - s > p.long_row;
         }
-        if (VEC == 16 && p.out_vec && col + 16 <= p.W) {
-            f32x4* o4 = reinterpret_cast<f32x4*>(o);
+        const uint64_t mask = __ballot(is_long);
+        if (is_long) list[__popcll(mask & ((1ull << lane) - 1ull))] = r;
+        if (lane == 0) nlist = __popcll(mask);
+    }
+    for (int i = threadIdx.x; i < 64 * VEC; i += blockDim.x) part[i] = 0;
+    __syncthreads();
+    const int n = nlist;
+    if (n == 0) return;
+
+    const LaneCols c = lane_cols<VEC, KIND>(p, lane);
+    for (int k = 0; k < n; ++k) {
+        const int64_t row = list[k];
+        int64_t start, end;
+        row_range<KIND>(p, row, start, end);
+        const int64_t per = (end - start + WAVES - 1) / WAVES;
+        const int64_t s = start + per * wave;
+        const int64_t e = s + per;
+        int acc[VEC];
+        wave_row_sum<VEC, KIND>(p, c, lane, s < end ? s : end, e < end ? e : end, acc);
+        if (c.grp == 0) {
 #pragma unroll
-            for (int i = 0; i < 4; ++i)
-                __builtin_nontemporal_store(f32x4{y[4 * i], y[4 * i + 1], y[4 * i + 2], y[4 * i + 3]}, o4 + i);
-        } else {
-#pragma unroll
-            for (int i = 0; i < VEC; ++i)
-                if (col + i < p.W) o[i] = y[i];
+            for (int i = 0; i < VEC; ++i) atomicAdd(&part[i * 64 + c.sub], acc[i]);
         }
+        __syncthreads();
+        if (wave == 0 && c.grp == 0) {
+#pragma unroll
+            for (int i = 0; i < VEC; ++i) {
+                acc[i] = part[i * 64 + c.sub];
+                part[i * 64 + c.sub] = 0;
+            }
+            store_row<VEC>(p, c, row, acc);
+        }
+        __syncthreads();
     }
 }
 
@@ -298,6 +412,15 @@ static int launch_spmm(SpmmParams p, int vec, hipStream_t s) {
     const int64_t gx = wide ? p.rows : ceil_div(p.rows, 4);
     if (gx > INT32_MAX) return TANGO_ERR_UNSUPPORTED;
     const dim3 grid(static_cast<unsigned>(gx), static_cast<unsigned>(ychunks));
+    // A row much longer than one wavefront's share of the whole job would finish long after
+    // everything else (hub rows of a small power-law graph): such rows get sixteen waves each.
+    p.long_row = (p.nnz >> 11) > 1024 ? (p.nnz >> 11) : 1024;
+    const dim3 lgrid(static_cast<unsigned>(ceil_div(p.rows, 64)), static_cast<unsigned>(ychunks));
+    if (p.nnz > p.long_row) {
+        if (vec == 16) hipLaunchKernelGGL((spmm_long_kernel<16, KIND>), lgrid, dim3(1024), 0, s, p);
+        else if (vec == 4) hipLaunchKernelGGL((spmm_long_kernel<4, KIND>), lgrid, dim3(1024), 0, s, p);
+        else hipLaunchKernelGGL((spmm_long_kernel<1, KIND>), lgrid, dim3(1024), 0, s, p);
+    }
 #define TANGO_SPMM_LAUNCH(V, WPR) \
     hipLaunchKernelGGL((spmm_kernel<V, WPR, KIND>), grid, dim3(256), 0, s, p)
     if (vec == 16) {

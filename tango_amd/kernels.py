@@ -567,15 +567,15 @@ def multi_cusparse_SPMM(g, N, E_T, scale, reverse=False, edge_major=False):
 
 
 def incidence_SPMM(g, E, scaleE, reverse=False):
-    """cuda/kernels.py:139-152."""
+    """cuda/kernels.py:139-152.  The incidence matrix in CSR form is (indptr, edge_ids) of the
+    adjacency (the equivalence evaluation/test_incidence.py:14-22 relies on), which the graph
+    already holds, so the row bounds come from indptr instead of a search in the COO node ids."""
     assert E.is_cuda and scaleE.is_cuda
-    coo = g.inc_out if reverse else g.inc_in
-    src = coo[0]
-    dst = coo[1]
+    indptr, _, edge_ids = g.adj_csr if reverse else g.adj_csc
     out_shape = (g.num_nodes(),) + E.shape[1:]
     dim = math.prod(E.shape[1:])
     out = torch.empty((g.num_nodes(), dim), dtype=torch.float32, device=E.device)
-    cuda_kernels.incidence_SPMM(out, src, dst, E, scaleE)
+    cuda_kernels.csr_SPMM(out, indptr, edge_ids, E.reshape(E.size(0), dim), scaleE)
     return out.view(out_shape)
 
 

@@ -36,14 +36,15 @@ def test_graph_formats_match_oracle(orc):
 
 
 # degree regimes: sparse (one wave per row) and dense/skewed (four waves per row)
-GRAPHS = [("sparse", 500, 4000), ("dense", 300, 60000), ("skewed", 2000, 400000)]
+# "hubs": low average degree with a few rows far beyond the long-row threshold (sixteen waves per row)
+GRAPHS = [("sparse", 500, 4000), ("dense", 300, 60000), ("skewed", 2000, 400000), ("hubs", 20000, 300000)]
 
 
 @pytest.mark.parametrize("F", [1, 3, 4, 16, 41, 48, 64, 100, 128, 256, 1040])
 @pytest.mark.parametrize("kind,n,e", GRAPHS)
 def test_csr_spmm_copy_u(K, orc, kind, n, e, F):
     rng = np.random.default_rng(F * 7 + n)
-    src, dst = powerlaw_graph(rng, n, e) if kind == "skewed" else rand_graph(rng, n, e)
+    src, dst = powerlaw_graph(rng, n, e) if kind in ("skewed", "hubs") else rand_graph(rng, n, e)
     g = make_graph(src, dst, n)
     feat = rng.integers(-127, 128, (n, F)).astype(np.int8)
     s = np.float32(0.0173)
@@ -87,7 +88,7 @@ def test_csr_spmm_empty_rows_and_all_ones(K, orc):
 @pytest.mark.parametrize("kind,n,e", GRAPHS)
 def test_u_mul_e_broadcast(K, orc, kind, n, e, H, F):
     rng = np.random.default_rng(H * 31 + F + n)
-    src, dst = powerlaw_graph(rng, n, e) if kind == "skewed" else rand_graph(rng, n, e)
+    src, dst = powerlaw_graph(rng, n, e) if kind in ("skewed", "hubs") else rand_graph(rng, n, e)
     g = make_graph(src, dst, n)
     o = orc.graph_formats(src, dst, n)
     feat = rng.integers(-127, 128, (n, H, F)).astype(np.int8)
@@ -131,14 +132,20 @@ def test_u_mul_e_elementwise(K, orc):
 @pytest.mark.parametrize("kind,n,e", GRAPHS)
 def test_incidence_spmm(K, orc, kind, n, e, F):
     rng = np.random.default_rng(F + n)
-    src, dst = powerlaw_graph(rng, n, e) if kind == "skewed" else rand_graph(rng, n, e)
+    src, dst = powerlaw_graph(rng, n, e) if kind in ("skewed", "hubs") else rand_graph(rng, n, e)
     g = make_graph(src, dst, n)
     o = orc.graph_formats(src, dst, n)
     E = rng.integers(-127, 128, (e, F)).astype(np.int8)
     s = np.float32(0.02)
     for reverse, inc in ((False, "inc_in"), (True, "inc_out")):
+        want = orc.spmm_incidence(o[inc][0], o[inc][1], E, s, n)
         got = K.incidence_SPMM(g, dev(E), sc(s), reverse=reverse)
-        assert np.array_equal(host(got), orc.spmm_incidence(o[inc][0], o[inc][1], E, s, n))
+        assert np.array_equal(host(got), want)
+        # the binding with the reference's arguments: sorted (node, edge) pairs
+        coo = g.inc_out if reverse else g.inc_in
+        got = torch.empty((n, F), dtype=torch.float32, device="cuda")
+        K.cuda_kernels.incidence_SPMM(got, coo[0], coo[1], dev(E), sc(s))
+        assert np.array_equal(host(got), want)
     # the equivalence the reference relies on: incidence SpMM == CSR SpMM over (indptr, edge_ids)
     ip, _, eid = g.adj_csc
     out = torch.empty((n, F), dtype=torch.float32, device="cuda")
