@@ -1,10 +1,11 @@
 // LeakyReLU + per-destination edge softmax (forward and backward) for gfx950.
 //
 // fp32, memory-bound: e is read, a written, both [E, H] in edge-id order and
-// reached through the destination-major CSR's edge-id permutation.  A wavefront
-// owns one destination row; its lanes are (edge slot, head) pairs, so the H values
-// of an edge are one contiguous read.  The forward pass keeps a running (max, sum)
-// pair per lane (online softmax): two sweeps over the row instead of three.
+// reached through the destination-major CSR's edge-id permutation.  Threads are
+// (edge slot, head) pairs, so the H values of an edge are one contiguous read, and
+// a destination is owned by a thread group sized to its in-degree (see the tiers
+// below).  The forward pass keeps a running (max, sum) pair per thread (online
+// softmax): two sweeps over a row instead of three, one for rows held in registers.
 // For H > 64 a thread-per-(row, head) fallback is used.
 #include "common.hpp"
 
@@ -66,13 +67,19 @@ __global__ __launch_bounds__(256) void edge_softmax_bwd_kernel(
     }
 }
 
-// Wave-per-row kernels: lane = (edge slot es, head h) with Hp = H rounded up to a
-// power of two, so one step of the wavefront covers 64 / Hp edges of the row and
-// the per-head reduction is an xor-shuffle over the slot bits.  Used for H <= 64;
-// a high-degree destination is walked by 64 lanes instead of one.
-// Destinations with more in-edges than this are walked by a 1024-thread workgroup, not one wavefront.
-constexpr int64_t kLongRow = 512;
-constexpr int64_t kRowsPerLongBlock = 16;  // rows each long-row workgroup inspects
+// Three tiers by in-degree, for H <= 64 (Hp = H rounded up to a power of two):
+//   short  (<= kShortRow edges): a thread owns one (row, head) and keeps the row's values in
+//          registers, one sweep over memory; a wavefront covers 64 / H rows, which is what
+//          keeps enough bytes in flight when most destinations have a handful of in-edges;
+//   medium (<= kMediumValues / Hp edges): a wavefront owns the row, lane = (edge slot, head),
+//          four edges per lane in flight, reduction by xor-shuffles over the slot bits;
+//   long   : a 1024-thread workgroup owns the row (a hub destination must not be walked by one
+//          wavefront while the rest of the chip idles).
+// The medium and long kernels find their rows themselves: a wavefront / workgroup inspects a
+// strided set of rows at once (hubs with neighbouring ids spread out over the launch) and walks
+// the ones of its tier; no list of rows is built in global memory.
+constexpr int kShortRow = 16;
+constexpr int kMediumValues = 2048;
 
 __device__ __forceinline__ void softmax_merge(float& m, double& s, float m2, double s2) {
     const float mx = fmaxf(m, m2);
@@ -83,238 +90,329 @@ __device__ __forceinline__ void softmax_merge(float& m, double& s, float m2, dou
     s = a + b;
 }
 
-__global__ __launch_bounds__(256) void edge_softmax_fwd_wave_kernel(
+// 0 = short, 1 = medium, 2 = long
+__device__ __forceinline__ int row_tier(int64_t deg, int hp_log2) {
+    if (deg <= kShortRow) return 0;
+    return deg <= (kMediumValues >> hp_log2) ? 1 : 2;
+}
+
+__global__ __launch_bounds__(256) void edge_softmax_fwd_short_kernel(
     float* __restrict__ a, const float* __restrict__ e, const int64_t* __restrict__ indptr,
-    const int64_t* __restrict__ eids, int64_t rows, int H, int hp_log2, float slope) {
-    const int64_t row = static_cast<int64_t>(blockIdx.x) * 4 + (threadIdx.x >> 6);
-    if (row >= rows) return;
-    const int lane = lane_id();
-    const int h = lane & ((1 << hp_log2) - 1);
-    const int es = lane >> hp_log2;
-    const int nes = kWave >> hp_log2;
-    const int64_t p0 = indptr[row], p1 = indptr[row + 1];
-    if (p1 - p0 > kLongRow) return;  // left to the workgroup-per-row kernel
-    const bool hok = h < H;
-    float mx = -INFINITY;
-    double sum = 0.0;
-    for (int64_t p = p0 + es; p < p1; p += 4 * nes) {  // four independent edges in flight per lane
-        float v[4];
+    const int64_t* __restrict__ eids, int64_t rows, int H, float slope) {
+    const int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (i >= rows * H) return;
+    const int64_t r = i / H;
+    const int h = static_cast<int>(i - r * H);
+    const int64_t p0 = indptr[r];
+    const int64_t deg = indptr[r + 1] - p0;
+    if (deg > kShortRow || deg == 0) return;
+    int64_t id[kShortRow];
+    float v[kShortRow];
 #pragma unroll
-        for (int u = 0; u < 4; ++u) {
-            const int64_t q = p + u * nes;
-            v[u] = -INFINITY;
-            if (hok && q < p1) v[u] = leaky(e[(eids ? eids[q] : q) * H + h], slope);
+    for (int u = 0; u < kShortRow; ++u) {
+        v[u] = -INFINITY;
+        id[u] = 0;
+        if (u < deg) {
+            id[u] = (eids ? eids[p0 + u] : p0 + u) * H + h;
+            v[u] = leaky(e[id[u]], slope);
         }
-#pragma unroll
-        for (int u = 0; u < 4; ++u)
-            if (v[u] != -INFINITY) softmax_merge(mx, sum, v[u], 1.0);
     }
-    for (int off = 1 << hp_log2; off < kWave; off <<= 1) {
-        const float m2 = __shfl_xor(mx, off, kWave);
-        const double s2 = __shfl_xor(sum, off, kWave);
-        softmax_merge(mx, sum, m2, s2);
+    float mx = v[0];
+#pragma unroll
+    for (int u = 1; u < kShortRow; ++u) mx = fmaxf(mx, v[u]);
+    double sum = 0.0;
+#pragma unroll
+    for (int u = 0; u < kShortRow; ++u) {
+        v[u] = u < deg ? expf(v[u] - mx) : 0.0f;
+        sum += static_cast<double>(v[u]);
     }
     const float inv = static_cast<float>(1.0 / sum);
-    for (int64_t p = p0 + es; p < p1; p += 4 * nes) {
-        int64_t id[4];
-        float v[4];
 #pragma unroll
-        for (int u = 0; u < 4; ++u) {
-            const int64_t q = p + u * nes;
-            id[u] = -1;
-            if (hok && q < p1) {
-                id[u] = eids ? eids[q] : q;
-                v[u] = e[id[u] * H + h];
-            }
-        }
-#pragma unroll
-        for (int u = 0; u < 4; ++u)
-            if (id[u] >= 0) a[id[u] * H + h] = expf(leaky(v[u], slope) - mx) * inv;
-    }
+    for (int u = 0; u < kShortRow; ++u)
+        if (u < deg) a[id[u]] = v[u] * inv;
 }
 
-__global__ __launch_bounds__(256) void edge_softmax_bwd_wave_kernel(
+__global__ __launch_bounds__(256) void edge_softmax_bwd_short_kernel(
     float* __restrict__ de, const float* __restrict__ a, const float* __restrict__ da,
     const float* __restrict__ e, const int64_t* __restrict__ indptr,
-    const int64_t* __restrict__ eids, int64_t rows, int H, int hp_log2, float slope) {
-    const int64_t row = static_cast<int64_t>(blockIdx.x) * 4 + (threadIdx.x >> 6);
-    if (row >= rows) return;
-    const int lane = lane_id();
-    const int h = lane & ((1 << hp_log2) - 1);
-    const int es = lane >> hp_log2;
-    const int nes = kWave >> hp_log2;
-    const int64_t p0 = indptr[row], p1 = indptr[row + 1];
-    if (p1 - p0 > kLongRow) return;  // left to the workgroup-per-row kernel
-    const bool hok = h < H;
+    const int64_t* __restrict__ eids, int64_t rows, int H, float slope) {
+    const int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (i >= rows * H) return;
+    const int64_t r = i / H;
+    const int h = static_cast<int>(i - r * H);
+    const int64_t p0 = indptr[r];
+    const int64_t deg = indptr[r + 1] - p0;
+    if (deg > kShortRow || deg == 0) return;
+    int64_t id[kShortRow];
+    float x[kShortRow], y[kShortRow], z[kShortRow];
     double dsum = 0.0;
-    for (int64_t p = p0 + es; p < p1; p += 4 * nes) {
-        float x[4], y[4];
 #pragma unroll
-        for (int u = 0; u < 4; ++u) {
-            const int64_t q = p + u * nes;
-            x[u] = y[u] = 0.0f;
-            if (hok && q < p1) {
-                const int64_t id = eids ? eids[q] : q;
-                x[u] = a[id * H + h];
-                y[u] = da[id * H + h];
-            }
+    for (int u = 0; u < kShortRow; ++u) {
+        x[u] = y[u] = z[u] = 0.0f;
+        id[u] = 0;
+        if (u < deg) {
+            id[u] = (eids ? eids[p0 + u] : p0 + u) * H + h;
+            x[u] = a[id[u]];
+            y[u] = da[id[u]];
+            z[u] = e[id[u]];
         }
-#pragma unroll
-        for (int u = 0; u < 4; ++u) dsum += static_cast<double>(x[u]) * static_cast<double>(y[u]);
     }
-    for (int off = 1 << hp_log2; off < kWave; off <<= 1) dsum += __shfl_xor(dsum, off, kWave);
+#pragma unroll
+    for (int u = 0; u < kShortRow; ++u) dsum += static_cast<double>(x[u]) * static_cast<double>(y[u]);
     const float dot = static_cast<float>(dsum);
-    for (int64_t p = p0 + es; p < p1; p += 4 * nes) {
-        int64_t id[4];
-        float x[4], y[4], z[4];
 #pragma unroll
-        for (int u = 0; u < 4; ++u) {
-            const int64_t q = p + u * nes;
-            id[u] = -1;
-            if (hok && q < p1) {
-                id[u] = eids ? eids[q] : q;
-                x[u] = a[id[u] * H + h];
-                y[u] = da[id[u] * H + h];
-                z[u] = e[id[u] * H + h];
-            }
+    for (int u = 0; u < kShortRow; ++u)
+        if (u < deg) {
+            float g = x[u] * (y[u] - dot);
+            if (!(z[u] > 0.0f)) g *= slope;
+            de[id[u]] = g;
         }
-#pragma unroll
-        for (int u = 0; u < 4; ++u)
-            if (id[u] >= 0) {
-                float g = x[u] * (y[u] - dot);
-                if (!(z[u] > 0.0f)) g *= slope;
-                de[id[u] * H + h] = g;
-            }
-    }
 }
 
-// Workgroup-per-row kernels for hub destinations (in-degree > kLongRow): 1024 threads, thread =
-// (edge slot, head), four independent edges per thread in flight, reduction through LDS.
-// Each workgroup inspects every gridDim-th row and walks the long ones among them.
-__global__ __launch_bounds__(1024) void edge_softmax_fwd_long_kernel(
-    float* __restrict__ a, const float* __restrict__ e, const int64_t* __restrict__ indptr,
-    const int64_t* __restrict__ eids, int64_t rows, int H, int hp_log2, float slope) {
-    __shared__ float mred[1024];
-    __shared__ double sred[1024];
-    // strided assignment: neighbouring hub rows go to different workgroups
-    for (int64_t row = blockIdx.x; row < rows; row += gridDim.x) {
-    const int64_t p0 = indptr[row], p1 = indptr[row + 1];
-    if (p1 - p0 <= kLongRow) continue;  // uniform for the workgroup
-    __syncthreads();                    // the previous long row's LDS values are consumed
-    const int t = threadIdx.x;
-    const int hp = 1 << hp_log2;
-    const int h = t & (hp - 1);
-    const int64_t es = t >> hp_log2, nes = 1024 >> hp_log2;
+// `nthreads` threads (a wavefront or a workgroup) walk slots [p0, p1) of one row: thread t is
+// (edge slot t >> hp_log2, head t & (Hp - 1)).  Returns this thread's running (max, sum).
+template <int U>
+__device__ __forceinline__ void fwd_partial(const float* __restrict__ e, const int64_t* __restrict__ eids,
+                                            int64_t p0, int64_t p1, int t, int nthreads, int H, int hp_log2,
+                                            float slope, float& mx, double& sum) {
+    const int h = t & ((1 << hp_log2) - 1);
+    const int64_t es = t >> hp_log2, nes = nthreads >> hp_log2;
     const bool hok = h < H;
-    float mx = -INFINITY;
-    double sum = 0.0;
-    for (int64_t p = p0 + es; p < p1; p += 4 * nes) {
-        float v[4];
+    mx = -INFINITY;
+    sum = 0.0;
+    for (int64_t p = p0 + es; p < p1; p += U * nes) {  // U independent edges in flight per thread
+        float v[U];
 #pragma unroll
-        for (int u = 0; u < 4; ++u) {
+        for (int u = 0; u < U; ++u) {
             const int64_t q = p + u * nes;
             v[u] = -INFINITY;
             if (hok && q < p1) v[u] = leaky(e[(eids ? eids[q] : q) * H + h], slope);
         }
 #pragma unroll
-        for (int u = 0; u < 4; ++u)
-            if (v[u] != -INFINITY) softmax_merge(mx, sum, v[u], 1.0);
-    }
-    mred[t] = mx;
-    sred[t] = sum;
-    __syncthreads();
-    for (int off = 512; off >= hp; off >>= 1) {
-        if (t < off) {
-            float m1 = mred[t];
-            double s1 = sred[t];
-            softmax_merge(m1, s1, mred[t + off], sred[t + off]);
-            mred[t] = m1;
-            sred[t] = s1;
-        }
-        __syncthreads();
-    }
-    mx = mred[h];
-    const float inv = static_cast<float>(1.0 / sred[h]);
-    for (int64_t p = p0 + es; p < p1; p += 4 * nes) {
-        int64_t id[4];
-        float v[4];
-#pragma unroll
-        for (int u = 0; u < 4; ++u) {
-            const int64_t q = p + u * nes;
-            id[u] = -1;
-            if (hok && q < p1) {
-                id[u] = eids ? eids[q] : q;
-                v[u] = e[id[u] * H + h];
+        for (int u = 0; u < U; ++u) {
+            if (v[u] == -INFINITY) continue;
+            if (v[u] > mx) {  // one exp per element either way
+                sum = sum * static_cast<double>(expf(mx - v[u])) + 1.0;  // exp(-inf) = 0 for the first element
+                mx = v[u];
+            } else {
+                sum += static_cast<double>(expf(v[u] - mx));
             }
         }
-#pragma unroll
-        for (int u = 0; u < 4; ++u)
-            if (id[u] >= 0) a[id[u] * H + h] = expf(leaky(v[u], slope) - mx) * inv;
-    }
     }
 }
 
-__global__ __launch_bounds__(1024) void edge_softmax_bwd_long_kernel(
-    float* __restrict__ de, const float* __restrict__ a, const float* __restrict__ da,
-    const float* __restrict__ e, const int64_t* __restrict__ indptr,
-    const int64_t* __restrict__ eids, int64_t rows, int H, int hp_log2, float slope) {
-    __shared__ double sred[1024];
-    // strided assignment: neighbouring hub rows go to different workgroups
-    for (int64_t row = blockIdx.x; row < rows; row += gridDim.x) {
-    const int64_t p0 = indptr[row], p1 = indptr[row + 1];
-    if (p1 - p0 <= kLongRow) continue;
-    __syncthreads();
-    const int t = threadIdx.x;
-    const int hp = 1 << hp_log2;
-    const int h = t & (hp - 1);
-    const int64_t es = t >> hp_log2, nes = 1024 >> hp_log2;
+template <int U>
+__device__ __forceinline__ void fwd_write(float* __restrict__ a, const float* __restrict__ e,
+                                          const int64_t* __restrict__ eids, int64_t p0, int64_t p1, int t,
+                                          int nthreads, int H, int hp_log2, float slope, float mx, float inv) {
+    const int h = t & ((1 << hp_log2) - 1);
+    const int64_t es = t >> hp_log2, nes = nthreads >> hp_log2;
     const bool hok = h < H;
-    double dsum = 0.0;
-    for (int64_t p = p0 + es; p < p1; p += 4 * nes) {
-        float x[4], y[4];
+    for (int64_t p = p0 + es; p < p1; p += U * nes) {
+        int64_t id[U];
+        float v[U];
 #pragma unroll
-        for (int u = 0; u < 4; ++u) {
-            const int64_t q = p + u * nes;
-            x[u] = y[u] = 0.0f;
-            if (hok && q < p1) {
-                const int64_t id = eids ? eids[q] : q;
-                x[u] = a[id * H + h];
-                y[u] = da[id * H + h];
-            }
-        }
-#pragma unroll
-        for (int u = 0; u < 4; ++u) dsum += static_cast<double>(x[u]) * static_cast<double>(y[u]);
-    }
-    sred[t] = dsum;
-    __syncthreads();
-    for (int off = 512; off >= hp; off >>= 1) {
-        if (t < off) sred[t] += sred[t + off];
-        __syncthreads();
-    }
-    const float dot = static_cast<float>(sred[h]);
-    for (int64_t p = p0 + es; p < p1; p += 4 * nes) {
-        int64_t id[4];
-        float x[4], y[4], z[4];
-#pragma unroll
-        for (int u = 0; u < 4; ++u) {
+        for (int u = 0; u < U; ++u) {
             const int64_t q = p + u * nes;
             id[u] = -1;
             if (hok && q < p1) {
-                id[u] = eids ? eids[q] : q;
-                x[u] = a[id[u] * H + h];
-                y[u] = da[id[u] * H + h];
-                z[u] = e[id[u] * H + h];
+                id[u] = (eids ? eids[q] : q) * H + h;
+                v[u] = e[id[u]];
             }
         }
 #pragma unroll
-        for (int u = 0; u < 4; ++u)
+        for (int u = 0; u < U; ++u)
+            if (id[u] >= 0) a[id[u]] = expf(leaky(v[u], slope) - mx) * inv;
+    }
+}
+
+template <int U>
+__device__ __forceinline__ double bwd_partial(const float* __restrict__ a, const float* __restrict__ da,
+                                              const int64_t* __restrict__ eids, int64_t p0, int64_t p1, int t,
+                                              int nthreads, int H, int hp_log2) {
+    const int h = t & ((1 << hp_log2) - 1);
+    const int64_t es = t >> hp_log2, nes = nthreads >> hp_log2;
+    const bool hok = h < H;
+    double dsum = 0.0;
+    for (int64_t p = p0 + es; p < p1; p += U * nes) {
+        float x[U], y[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const int64_t q = p + u * nes;
+            x[u] = y[u] = 0.0f;
+            if (hok && q < p1) {
+                const int64_t id = (eids ? eids[q] : q) * H + h;
+                x[u] = a[id];
+                y[u] = da[id];
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u) dsum += static_cast<double>(x[u]) * static_cast<double>(y[u]);
+    }
+    return dsum;
+}
+
+template <int U>
+__device__ __forceinline__ void bwd_write(float* __restrict__ de, const float* __restrict__ a,
+                                          const float* __restrict__ da, const float* __restrict__ e,
+                                          const int64_t* __restrict__ eids, int64_t p0, int64_t p1, int t,
+                                          int nthreads, int H, int hp_log2, float slope, float dot) {
+    const int h = t & ((1 << hp_log2) - 1);
+    const int64_t es = t >> hp_log2, nes = nthreads >> hp_log2;
+    const bool hok = h < H;
+    for (int64_t p = p0 + es; p < p1; p += U * nes) {
+        int64_t id[U];
+        float x[U], y[U], z[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const int64_t q = p + u * nes;
+            id[u] = -1;
+            if (hok && q < p1) {
+                id[u] = (eids ? eids[q] : q) * H + h;
+                x[u] = a[id[u]];
+                y[u] = da[id[u]];
+                z[u] = e[id[u]];
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u)
             if (id[u] >= 0) {
                 float g = x[u] * (y[u] - dot);
                 if (!(z[u] > 0.0f)) g *= slope;
-                de[id[u] * H + h] = g;
+                de[id[u]] = g;
             }
     }
+}
+
+// Medium rows.  Wavefront w of the launch inspects rows w, w + W, w + 2W, ... (kRowsPerWave of
+// them, W = number of wavefronts launched) and walks the medium ones in turn.
+constexpr int kRowsPerWave = 8;
+template <bool FWD>
+__global__ __launch_bounds__(256) void edge_softmax_medium_kernel(
+    float* __restrict__ out, const float* __restrict__ a, const float* __restrict__ da,
+    const float* __restrict__ e, const int64_t* __restrict__ indptr, const int64_t* __restrict__ eids,
+    int64_t rows, int H, int hp_log2, float slope) {
+    const int lane = lane_id();
+    const int64_t nwaves = static_cast<int64_t>(gridDim.x) * 4;
+    const int64_t w = static_cast<int64_t>(blockIdx.x) * 4 + (threadIdx.x >> 6);
+    const int64_t mine = w + static_cast<int64_t>(lane) * nwaves;
+    int64_t q0 = 0, q1 = 0;
+    if (lane < kRowsPerWave && mine < rows) {
+        q0 = indptr[mine];
+        q1 = indptr[mine + 1];
     }
+    uint64_t todo = __ballot(row_tier(q1 - q0, hp_log2) == 1);
+    while (todo) {
+        const int l = __builtin_ctzll(todo);
+        todo &= todo - 1;
+        const int64_t p0 = __shfl(q0, l, kWave), p1 = __shfl(q1, l, kWave);
+        if (FWD) {
+            float mx;
+            double sum;
+            fwd_partial<8>(e, eids, p0, p1, lane, kWave, H, hp_log2, slope, mx, sum);
+            for (int off = 1 << hp_log2; off < kWave; off <<= 1) {
+                const float m2 = __shfl_xor(mx, off, kWave);
+                const double s2 = __shfl_xor(sum, off, kWave);
+                softmax_merge(mx, sum, m2, s2);
+            }
+            fwd_write<8>(out, e, eids, p0, p1, lane, kWave, H, hp_log2, slope, mx, static_cast<float>(1.0 / sum));
+        } else {
+            double dsum = bwd_partial<8>(a, da, eids, p0, p1, lane, kWave, H, hp_log2);
+            for (int off = 1 << hp_log2; off < kWave; off <<= 1) dsum += __shfl_xor(dsum, off, kWave);
+            bwd_write<8>(out, a, da, e, eids, p0, p1, lane, kWave, H, hp_log2, slope, static_cast<float>(dsum));
+        }
+    }
+}
+
+// Long rows.  A fixed number of 1024-thread workgroups (G = gridDim.x) share the rows: thread t
+// of workgroup b inspects row b + G * t (then b + G * (1024 + t), ...), the long ones are
+// collected in LDS and walked in turn by all sixteen wavefronts: shuffles inside a wavefront,
+// then one exchange of the sixteen partial results through LDS.
+constexpr int kLongGrid = 512;
+
+template <bool FWD>
+__global__ __launch_bounds__(1024) void edge_softmax_long_kernel(
+    float* __restrict__ out, const float* __restrict__ a, const float* __restrict__ da,
+    const float* __restrict__ e, const int64_t* __restrict__ indptr, const int64_t* __restrict__ eids,
+    int64_t rows, int H, int hp_log2, float slope) {
+    __shared__ float mred[16][64];
+    __shared__ double sred[16][64];
+    __shared__ int64_t lp0[1024], lp1[1024];
+    __shared__ int nlist;
+    const int t = threadIdx.x;
+    const int lane = lane_id();
+    const int wave = t >> 6;
+    const int hp = 1 << hp_log2;
+    const int h = t & (hp - 1);
+    const int64_t G = gridDim.x;
+    for (int64_t first = blockIdx.x; first < rows; first += 1024 * G) {  // uniform trip count
+        if (t == 0) nlist = 0;
+        __syncthreads();
+        const int64_t mine = first + G * t;
+        if (mine < rows) {
+            const int64_t q0 = indptr[mine], q1 = indptr[mine + 1];
+            if (row_tier(q1 - q0, hp_log2) == 2) {
+                const int k = atomicAdd(&nlist, 1);  // any order: rows are independent
+                lp0[k] = q0;
+                lp1[k] = q1;
+            }
+        }
+        __syncthreads();
+        const int n = nlist;
+        for (int k = 0; k < n; ++k) {
+            const int64_t p0 = lp0[k], p1 = lp1[k];
+            if (FWD) {
+                float mx;
+                double sum;
+                fwd_partial<8>(e, eids, p0, p1, t, 1024, H, hp_log2, slope, mx, sum);
+                for (int off = hp; off < kWave; off <<= 1) {
+                    const float m2 = __shfl_xor(mx, off, kWave);
+                    const double s2 = __shfl_xor(sum, off, kWave);
+                    softmax_merge(mx, sum, m2, s2);
+                }
+                if (lane < hp) {
+                    mred[wave][lane] = mx;
+                    sred[wave][lane] = sum;
+                }
+                __syncthreads();
+                mx = mred[0][h];
+                sum = sred[0][h];
+#pragma unroll
+                for (int w = 1; w < 16; ++w) softmax_merge(mx, sum, mred[w][h], sred[w][h]);
+                fwd_write<8>(out, e, eids, p0, p1, t, 1024, H, hp_log2, slope, mx, static_cast<float>(1.0 / sum));
+            } else {
+                double dsum = bwd_partial<8>(a, da, eids, p0, p1, t, 1024, H, hp_log2);
+                for (int off = hp; off < kWave; off <<= 1) dsum += __shfl_xor(dsum, off, kWave);
+                if (lane < hp) sred[wave][lane] = dsum;
+                __syncthreads();
+                dsum = 0.0;
+#pragma unroll
+                for (int w = 0; w < 16; ++w) dsum += sred[w][h];
+                bwd_write<8>(out, a, da, e, eids, p0, p1, t, 1024, H, hp_log2, slope, static_cast<float>(dsum));
+            }
+            __syncthreads();  // the partial results are consumed before the next row overwrites them
+        }
+    }
+}
+
+// Launches the three tiers.  FWD: out = a; otherwise out = de.
+template <bool FWD>
+static void launch_tiers(float* out, const float* a, const float* da, const float* e, const int64_t* indptr,
+                         const int64_t* eids, int64_t rows, int H, float slope, hipStream_t s) {
+    int hp = 0;
+    while ((1 << hp) < H) ++hp;
+    const unsigned sgrid = static_cast<unsigned>(ceil_div(rows * H, 256));
+    if (FWD)
+        hipLaunchKernelGGL(edge_softmax_fwd_short_kernel, dim3(sgrid), dim3(256), 0, s, out, e, indptr, eids, rows, H,
+                           slope);
+    else
+        hipLaunchKernelGGL(edge_softmax_bwd_short_kernel, dim3(sgrid), dim3(256), 0, s, out, a, da, e, indptr, eids,
+                           rows, H, slope);
+    hipLaunchKernelGGL(edge_softmax_medium_kernel<FWD>, dim3(static_cast<unsigned>(ceil_div(rows, 4 * kRowsPerWave))),
+                       dim3(256), 0, s, out, a, da, e, indptr, eids, rows, H, hp, slope);
+    hipLaunchKernelGGL(edge_softmax_long_kernel<FWD>,
+                       dim3(static_cast<unsigned>(rows < kLongGrid ? rows : kLongGrid)), dim3(1024), 0,
+                       s, out, a, da, e, indptr, eids, rows, H, hp, slope);
 }
 
 }  // namespace tango
@@ -329,14 +427,9 @@ int tango_edge_softmax_fwd(float* a, const float* e, const int64_t* indptr,
     if (rows < 0 || H < 0 || (rows > 0 && !indptr) || H >= (1LL << 31)) return TANGO_ERR_INVALID_ARG;
     if (rows * H == 0) return TANGO_OK;
     if (!a || !e) return TANGO_ERR_INVALID_ARG;
-    if (H <= 64 && rows <= INT32_MAX) {
-        int hp = 0;
-        while ((1 << hp) < H) ++hp;
-        hipLaunchKernelGGL(edge_softmax_fwd_wave_kernel, dim3(static_cast<unsigned>(ceil_div(rows, 4))),
-                           dim3(256), 0, as_stream(stream), a, e, indptr, edge_ids, rows,
-                           static_cast<int>(H), hp, slope);
-        hipLaunchKernelGGL(edge_softmax_fwd_long_kernel, dim3(static_cast<unsigned>(ceil_div(rows, kRowsPerLongBlock))),
-                           dim3(1024), 0, as_stream(stream), a, e, indptr, edge_ids, rows, static_cast<int>(H), hp, slope);
+    if (H <= 64 && rows * H <= 256LL * INT32_MAX) {
+        launch_tiers<true>(a, nullptr, nullptr, e, indptr, edge_ids, rows, static_cast<int>(H), slope,
+                           as_stream(stream));
         return launch_status();
     }
     hipLaunchKernelGGL(edge_softmax_fwd_kernel, dim3(grid_for(rows * H, 256, 16)), dim3(256), 0,
@@ -350,14 +443,8 @@ int tango_edge_softmax_bwd(float* de, const float* a, const float* da, const flo
     if (rows < 0 || H < 0 || (rows > 0 && !indptr) || H >= (1LL << 31)) return TANGO_ERR_INVALID_ARG;
     if (rows * H == 0) return TANGO_OK;
     if (!de || !a || !da || !e) return TANGO_ERR_INVALID_ARG;
-    if (H <= 64 && rows <= INT32_MAX) {
-        int hp = 0;
-        while ((1 << hp) < H) ++hp;
-        hipLaunchKernelGGL(edge_softmax_bwd_wave_kernel, dim3(static_cast<unsigned>(ceil_div(rows, 4))),
-                           dim3(256), 0, as_stream(stream), de, a, da, e, indptr, edge_ids, rows,
-                           static_cast<int>(H), hp, slope);
-        hipLaunchKernelGGL(edge_softmax_bwd_long_kernel, dim3(static_cast<unsigned>(ceil_div(rows, kRowsPerLongBlock))),
-                           dim3(1024), 0, as_stream(stream), de, a, da, e, indptr, edge_ids, rows, static_cast<int>(H), hp, slope);
+    if (H <= 64 && rows * H <= 256LL * INT32_MAX) {
+        launch_tiers<false>(de, a, da, e, indptr, edge_ids, rows, static_cast<int>(H), slope, as_stream(stream));
         return launch_status();
     }
     hipLaunchKernelGGL(edge_softmax_bwd_kernel, dim3(grid_for(rows * H, 256, 16)), dim3(256), 0,

@@ -49,6 +49,7 @@ struct SpmmParams {
     int ldf_shift; // log2(ldf) when ldf is a power of two and all byte offsets fit 31 bits, else -1
     int out_vec;   // out rows may be stored as 16-byte vectors
     int64_t long_row;  // rows with more slots than this go to the sixteen-wave kernel
+    int64_t group_row; // sparse graphs: rows with at most this many slots are owned by a lane group
 };
 
 enum { KIND_COPY = 0, KIND_WEIGHTED = 1, KIND_COO = 2 };
@@ -330,60 +331,132 @@ __global__ __launch_bounds__(256) void spmm_kernel(const SpmmParams p) {
     if (c.grp == 0) store_row<VEC>(p, c, row, acc);
 }
 
-// Rows with more than p.long_row slots, sixteen wavefronts per row.  blockDim.x = 1024;
-// workgroup b looks at the 64 rows b, b + G, b + 2G, ... (G = gridDim.x: hub rows with
-// neighbouring ids land in different workgroups), keeps the long ones and sums each with
-// all of its waves; the waves' partial sums meet in LDS through integer atomics, which
-// are exact in any order.
+// Sparse graphs (a handful of neighbours per row): a wavefront that owns one row would leave most
+// of its gather slots empty and the launch would be bound by per-wave latency chains.  Here every
+// group of `lpe` lanes owns a row of its own (64 / lpe rows per wavefront) and walks it four
+// neighbours at a time; rows with more than p.group_row slots are left to spmm_medium_kernel.
+template <int VEC, int KIND>
+__global__ __launch_bounds__(256) void spmm_group_kernel(const SpmmParams p) {
+    constexpr int U = 4;
+    const int lane = lane_id();
+    const int wave = __builtin_amdgcn_readfirstlane(static_cast<int>(threadIdx.x) >> 6);
+    const LaneCols c = lane_cols<VEC, KIND>(p, lane);
+    const int64_t row = ((static_cast<int64_t>(blockIdx.x) * 4 + wave) << c.sh) + c.grp;
+    int64_t start = 0, end = 0;
+    if (row < p.rows) {
+        start = p.indptr[row];
+        end = p.indptr[row + 1];
+    }
+    const bool mine = row < p.rows && end - start <= p.group_row;
+    if (!mine) end = start;
+    int acc[VEC];
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) acc[i] = 0;
+    for (int64_t q = start; q < end; q += U) {  // trip counts differ between the groups of a wave
+        typename Gather<VEC>::T d[U];
+        uint32_t m = 0u;
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const bool ok = q + u < end;
+            const int64_t qc = ok ? q + u : start;  // a valid slot: start < end inside the loop
+            const int j = static_cast<int>(p.indices[qc]);
+            d[u] = Gather<VEC>::load(c.fcol + row_offset(j, p));
+            uint32_t w = 1u;
+            if (KIND == KIND_WEIGHTED) {
+                const int64_t pos = p.edge_ids ? p.edge_ids[qc] : qc;
+                w = static_cast<uint32_t>(static_cast<uint8_t>(c.wbase[pos * p.ev_se]));
+            }
+            m |= (ok ? w : 0u) << (8 * u);
+        }
+        accumulate4<VEC>(acc, d, m);
+    }
+    if (mine) store_row<VEC>(p, c, row, acc);
+}
+
+// Rows with more than p.group_row and at most p.long_row slots of a sparse graph, one wavefront
+// per row.  Wavefront w of the launch inspects rows w, w + W, ... (kRowsPerWave of them, W =
+// wavefronts launched) and walks the ones of this tier in turn.
+constexpr int kRowsPerWave = 8;
+
+template <int VEC, int KIND>
+__global__ __launch_bounds__(256) void spmm_medium_kernel(const SpmmParams p) {
+    const int lane = lane_id();
+    const int wave = __builtin_amdgcn_readfirstlane(static_cast<int>(threadIdx.x) >> 6);
+    const int64_t nwaves = static_cast<int64_t>(gridDim.x) * 4;
+    const int64_t w = static_cast<int64_t>(blockIdx.x) * 4 + wave;
+    const int64_t mine = w + static_cast<int64_t>(lane) * nwaves;
+    int64_t q0 = 0, q1 = 0;
+    if (lane < kRowsPerWave && mine < p.rows) {
+        q0 = p.indptr[mine];
+        q1 = p.indptr[mine + 1];
+    }
+    uint64_t todo = __ballot(q1 - q0 > p.group_row && q1 - q0 <= p.long_row);
+    if (!todo) return;
+    const LaneCols c = lane_cols<VEC, KIND>(p, lane);
+    while (todo) {
+        const int l = __builtin_ctzll(todo);
+        todo &= todo - 1;
+        const int64_t start = __shfl(q0, l, kWave), end = __shfl(q1, l, kWave);
+        int acc[VEC];
+        wave_row_sum<VEC, KIND>(p, c, lane, start, end, acc);
+        if (c.grp == 0) store_row<VEC>(p, c, w + static_cast<int64_t>(l) * nwaves, acc);
+    }
+}
+
+// Rows with more than p.long_row slots, sixteen wavefronts per row.  blockDim.x = 1024, a
+// fixed number of workgroups (G = gridDim.x): thread t of workgroup b inspects row b + G * t
+// (then b + G * (1024 + t), ...; hub rows with neighbouring ids land in different workgroups),
+// the long ones are collected in LDS and each is summed by all waves; the waves' partial sums
+// meet in LDS through integer atomics, which are exact in any order.
+constexpr int kLongGrid = 512;
+
 template <int VEC, int KIND>
 __global__ __launch_bounds__(1024) void spmm_long_kernel(const SpmmParams p) {
     constexpr int WAVES = 16;
     __shared__ int part[64 * VEC];
-    __shared__ int64_t list[kWave];
+    __shared__ int64_t list[1024];
     __shared__ int nlist;
+    const int t = threadIdx.x;
     const int lane = lane_id();
-    const int wave = __builtin_amdgcn_readfirstlane(static_cast<int>(threadIdx.x) >> 6);
-    if (wave == 0) {
-        const int64_t r = static_cast<int64_t>(blockIdx.x) + static_cast<int64_t>(lane) * gridDim.x;
-        bool is_long = false;
-        if (r < p.rows) {
-            int64_t s, e;
-            row_range<KIND>(p, r, s, e);
-            is_long = e - s > p.long_row;
-        }
-        const uint64_t mask = __ballot(is_long);
-        if (is_long) list[__popcll(mask & ((1ull << lane) - 1ull))] = r;
-        if (lane == 0) nlist = __popcll(mask);
-    }
-    for (int i = threadIdx.x; i < 64 * VEC; i += blockDim.x) part[i] = 0;
-    __syncthreads();
-    const int n = nlist;
-    if (n == 0) return;
-
+    const int wave = __builtin_amdgcn_readfirstlane(t >> 6);
     const LaneCols c = lane_cols<VEC, KIND>(p, lane);
-    for (int k = 0; k < n; ++k) {
-        const int64_t row = list[k];
-        int64_t start, end;
-        row_range<KIND>(p, row, start, end);
-        const int64_t per = (end - start + WAVES - 1) / WAVES;
-        const int64_t s = start + per * wave;
-        const int64_t e = s + per;
-        int acc[VEC];
-        wave_row_sum<VEC, KIND>(p, c, lane, s < end ? s : end, e < end ? e : end, acc);
-        if (c.grp == 0) {
-#pragma unroll
-            for (int i = 0; i < VEC; ++i) atomicAdd(&part[i * 64 + c.sub], acc[i]);
+    const int64_t G = gridDim.x;
+    for (int i = t; i < 64 * VEC; i += 1024) part[i] = 0;
+    for (int64_t first = blockIdx.x; first < p.rows; first += 1024 * G) {  // uniform trip count
+        if (t == 0) nlist = 0;
+        __syncthreads();
+        const int64_t mine = first + G * t;
+        if (mine < p.rows) {
+            int64_t s, e;
+            row_range<KIND>(p, mine, s, e);
+            if (e - s > p.long_row) list[atomicAdd(&nlist, 1)] = mine;  // any order: rows are independent
         }
         __syncthreads();
-        if (wave == 0 && c.grp == 0) {
+        const int n = nlist;
+        for (int k = 0; k < n; ++k) {
+            const int64_t row = list[k];
+            int64_t start, end;
+            row_range<KIND>(p, row, start, end);
+            const int64_t per = (end - start + WAVES - 1) / WAVES;
+            const int64_t s = start + per * wave;
+            const int64_t e = s + per;
+            int acc[VEC];
+            wave_row_sum<VEC, KIND>(p, c, lane, s < end ? s : end, e < end ? e : end, acc);
+            if (c.grp == 0) {
 #pragma unroll
-            for (int i = 0; i < VEC; ++i) {
-                acc[i] = part[i * 64 + c.sub];
-                part[i * 64 + c.sub] = 0;
+                for (int i = 0; i < VEC; ++i) atomicAdd(&part[i * 64 + c.sub], acc[i]);
             }
-            store_row<VEC>(p, c, row, acc);
+            __syncthreads();
+            if (wave == 0 && c.grp == 0) {
+#pragma unroll
+                for (int i = 0; i < VEC; ++i) {
+                    acc[i] = part[i * 64 + c.sub];
+                    part[i * 64 + c.sub] = 0;
+                }
+                store_row<VEC>(p, c, row, acc);
+            }
+            __syncthreads();
         }
-        __syncthreads();
     }
 }
 
@@ -415,11 +488,28 @@ static int launch_spmm(SpmmParams p, int vec, hipStream_t s) {
     // A row much longer than one wavefront's share of the whole job would finish long after
     // everything else (hub rows of a small power-law graph): such rows get sixteen waves each.
     p.long_row = (p.nnz >> 11) > 1024 ? (p.nnz >> 11) : 1024;
-    const dim3 lgrid(static_cast<unsigned>(ceil_div(p.rows, 64)), static_cast<unsigned>(ychunks));
+    const dim3 lgrid(static_cast<unsigned>(p.rows < kLongGrid ? p.rows : kLongGrid), static_cast<unsigned>(ychunks));
     if (p.nnz > p.long_row) {
         if (vec == 16) hipLaunchKernelGGL((spmm_long_kernel<16, KIND>), lgrid, dim3(1024), 0, s, p);
         else if (vec == 4) hipLaunchKernelGGL((spmm_long_kernel<4, KIND>), lgrid, dim3(1024), 0, s, p);
         else hipLaunchKernelGGL((spmm_long_kernel<1, KIND>), lgrid, dim3(1024), 0, s, p);
+    }
+    // Sparse graph: lane groups own the short rows, single waves the rest up to long_row.
+    if (KIND != KIND_COO && p.nnz < 64 * p.rows && p.lpe_log2 < 6) {
+        p.group_row = 32;
+        const int64_t rows_per_block = 4LL << (6 - p.lpe_log2);
+        const dim3 ggrid(static_cast<unsigned>(ceil_div(p.rows, rows_per_block)), static_cast<unsigned>(ychunks));
+        const dim3 mgrid(static_cast<unsigned>(ceil_div(p.rows, 4 * kRowsPerWave)), static_cast<unsigned>(ychunks));
+#define TANGO_SPMM_TIERS(V)                                                                     \
+    do {                                                                                        \
+        hipLaunchKernelGGL((spmm_group_kernel<V, KIND>), ggrid, dim3(256), 0, s, p);            \
+        hipLaunchKernelGGL((spmm_medium_kernel<V, KIND>), mgrid, dim3(256), 0, s, p);           \
+    } while (0)
+        if (vec == 16) TANGO_SPMM_TIERS(16);
+        else if (vec == 4) TANGO_SPMM_TIERS(4);
+        else TANGO_SPMM_TIERS(1);
+#undef TANGO_SPMM_TIERS
+        return launch_status();
     }
 #define TANGO_SPMM_LAUNCH(V, WPR) \
     hipLaunchKernelGGL((spmm_kernel<V, WPR, KIND>), grid, dim3(256), 0, s, p)
