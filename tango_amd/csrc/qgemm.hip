@@ -411,7 +411,8 @@ __global__ __launch_bounds__(256) void transpose_pack_i8_kernel(int8_t* __restri
 
 // ------------------------------------------------------------- TN kernel
 struct TnParams {
-    int* acc;          // [N, K] int32 partial sums, pre-zeroed
+    int* acc;          // [splits, N, Kp] int32 partial sums, one slab per split of M (Kp = K rounded up to 4)
+    int64_t Kp;
     const int8_t* A;   // dY [M, N] int8, row stride lda
     const int8_t* B;   // X  [M, K] int8, row stride ldb
     int64_t M, N, K;
@@ -511,38 +512,56 @@ __global__ __launch_bounds__(256, 2) void gemm_tn_kernel(const TnParams p) {
             for (int j = 0; j < 4; ++j) acc[i][j] = mfma_16x16x64(fa[i], fb[j], acc[i][j]);
     }
 
-    // acc[i][j][v] at lane (g, r16): n = n0 + 64 wn + 4 (4 g + v) + i, k = k0 + 64 wk + 4 r16 + j
+    // acc[i][j][v] at lane (g, r16): n = n0 + 64 wn + 4 (4 g + v) + i, k = k0 + 64 wk + 4 r16 + j.
+    // Every (split, n, k) belongs to exactly one workgroup, so the slab is written with plain
+    // 16-byte stores (j = 0..3 are adjacent columns) and needs no zero fill.
+    int* slab = p.acc + static_cast<int64_t>(split) * p.N * p.Kp;
 #pragma unroll
     for (int i = 0; i < 4; ++i)
 #pragma unroll
         for (int v = 0; v < 4; ++v) {
             const int64_t n = n0 + wn * 64 + 4 * (4 * g + v) + i;
-            if (n < p.N) {
-#pragma unroll
-                for (int j = 0; j < 4; ++j) {
-                    const int64_t k = k0 + wk * 64 + 4 * r16 + j;
-                    if (k < p.K) atomicAdd(p.acc + n * p.K + k, acc[i][j][v]);
-                }
-            }
+            const int64_t k = k0 + wk * 64 + 4 * r16;
+            if (n < p.N && k < p.Kp)
+                *reinterpret_cast<i32x4*>(slab + n * p.Kp + k) =
+                    i32x4{acc[i][0][v], acc[i][1][v], acc[i][2][v], acc[i][3][v]};
         }
 }
 
-__global__ __launch_bounds__(256) void zero_i32_kernel(int* __restrict__ p, int64_t n) {
-    const int64_t nthr = static_cast<int64_t>(gridDim.x) * blockDim.x;
-    for (int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < n; i += nthr) p[i] = 0;
-}
-
-// out[r, c] = (sA * sB) * float(acc[r, c])
-__global__ __launch_bounds__(256) void dequant_i32_kernel(float* __restrict__ out, int64_t ldo,
-                                                          const int* __restrict__ acc, int64_t rows,
-                                                          int64_t cols, const float* __restrict__ sA,
-                                                          const float* __restrict__ sB) {
-    const float s = sA[0] * sB[0];
-    const int64_t total = rows * cols;
-    const int64_t nthr = static_cast<int64_t>(gridDim.x) * blockDim.x;
-    for (int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < total; i += nthr) {
-        const int64_t r = i / cols, c = i - r * cols;
-        out[r * ldo + c] = s * static_cast<float>(acc[i]);
+// dW[n, k] = (sA * sB) * float(sum over splits of part[split][n][k]).  A workgroup is 16 column
+// quads x 16 split lanes: the split lanes add every 16th slab, LDS adds the sixteen.
+__global__ __launch_bounds__(256) void tn_reduce_kernel(float* __restrict__ out, int64_t ldo,
+                                                        const int* __restrict__ part, int64_t N, int64_t K,
+                                                        int64_t Kp, int splits, const float* __restrict__ sA,
+                                                        const float* __restrict__ sB) {
+    __shared__ int red[16][16][4];
+    const int vq = threadIdx.x & 15, sl = threadIdx.x >> 4;
+    const int64_t quads = N * Kp / 4;
+    const int64_t q = static_cast<int64_t>(blockIdx.x) * 16 + vq;
+    i32x4 sum{0, 0, 0, 0};
+    if (q < quads) {
+        const i32x4* src = reinterpret_cast<const i32x4*>(part) + q;
+        int sp = sl;
+        for (; sp + 48 < splits; sp += 64) {  // four slabs in flight
+            const i32x4 a = src[static_cast<int64_t>(sp) * quads], b = src[static_cast<int64_t>(sp + 16) * quads];
+            const i32x4 c = src[static_cast<int64_t>(sp + 32) * quads], d = src[static_cast<int64_t>(sp + 48) * quads];
+            sum += (a + b) + (c + d);
+        }
+        for (; sp < splits; sp += 16) sum += src[static_cast<int64_t>(sp) * quads];
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) red[sl][vq][i] = sum[i];
+    __syncthreads();
+    if (sl == 0 && q < quads) {
+        const float s = sA[0] * sB[0];
+        const int64_t n = (q * 4) / Kp, k = q * 4 - n * Kp;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            int t = 0;
+#pragma unroll
+            for (int w = 0; w < 16; ++w) t += red[w][vq][i];
+            if (k + i < K) out[n * ldo + k + i] = s * static_cast<float>(t);
+        }
     }
 }
 
@@ -774,10 +793,35 @@ int tango_qgemm_bwd_dx(float* dX, int64_t lddx, const int8_t* dYq, int64_t lddy,
                                  workspace_bytes, stream);
 }
 
+// How the reduction over M is cut: `splits` chunks of `chunk` rows (a multiple of 64).
+struct TnPlan {
+    int tiles_n, tiles_k;
+    int64_t splits, chunk, Kp;
+};
+
+static TnPlan tn_plan(int64_t M, int64_t N, int64_t K) {
+    TnPlan t{};
+    t.tiles_n = static_cast<int>(ceil_div(N, 128));
+    t.tiles_k = static_cast<int>(ceil_div(K, 128));
+    t.Kp = round_up(K, 4);
+    const int64_t tiles = static_cast<int64_t>(t.tiles_n) * t.tiles_k;
+    // enough workgroups for ~3 per CU, each with at least 4 reduction steps ...
+    int64_t splits = ceil_div(768, tiles);
+    const int64_t max_splits = ceil_div(M, 256);
+    if (splits > max_splits) splits = max_splits;
+    // ... but the slabs (written once, read once, 4 bytes each way) stay below the operand bytes
+    const int64_t by_traffic = M * (N + K) / (8 * N * t.Kp);
+    if (splits > by_traffic) splits = by_traffic;
+    if (splits < 1) splits = 1;
+    t.chunk = round_up(ceil_div(M, splits), 64);
+    t.splits = M > 0 ? ceil_div(M, t.chunk) : 0;
+    return t;
+}
+
 size_t tango_qgemm_bwd_dw_workspace(int64_t M, int64_t N, int64_t K) {
-    (void)M;
-    if (N <= 0 || K <= 0) return 0;
-    return static_cast<size_t>(N * K) * sizeof(int);
+    if (N <= 0 || K <= 0 || M < 0) return 0;
+    const TnPlan t = tn_plan(M, N, K);
+    return static_cast<size_t>((t.splits > 0 ? t.splits : 1) * N * t.Kp) * sizeof(int);
 }
 
 int tango_qgemm_bwd_dw(float* dW, int64_t lddw, const int8_t* dYq, int64_t lddy,
@@ -790,37 +834,32 @@ int tango_qgemm_bwd_dw(float* dW, int64_t lddw, const int8_t* dYq, int64_t lddy,
     if (N == 0 || K == 0) return TANGO_OK;
     const size_t need = tango_qgemm_bwd_dw_workspace(M, N, K);
     if (!workspace || workspace_bytes < need) return TANGO_ERR_WORKSPACE;
-    if ((reinterpret_cast<uintptr_t>(workspace) & 3) != 0) return TANGO_ERR_INVALID_ARG;
+    if ((reinterpret_cast<uintptr_t>(workspace) & 15) != 0) return TANGO_ERR_INVALID_ARG;
     hipStream_t s = as_stream(stream);
     int* acc = static_cast<int*>(workspace);
-    hipLaunchKernelGGL(zero_i32_kernel, dim3(grid_for(N * K, 256)), dim3(256), 0, s, acc, N * K);
+    const TnPlan t = tn_plan(M, N, K);
     if (M > 0) {
         TnParams p{};
-        p.acc = acc; p.A = dYq; p.B = Xq; p.M = M; p.N = N; p.K = K; p.lda = lddy; p.ldb = ldx;
-        p.tiles_n = static_cast<int>(ceil_div(N, 128));
-        p.tiles_k = static_cast<int>(ceil_div(K, 128));
+        p.acc = acc; p.Kp = t.Kp; p.A = dYq; p.B = Xq; p.M = M; p.N = N; p.K = K; p.lda = lddy; p.ldb = ldx;
+        p.tiles_n = t.tiles_n;
+        p.tiles_k = t.tiles_k;
         const int64_t tiles = static_cast<int64_t>(p.tiles_n) * p.tiles_k;
-        // enough workgroups for ~3 per CU, each with at least 4 reduction steps
-        int64_t splits = ceil_div(768, tiles);
-        const int64_t max_splits = ceil_div(M, 256);
-        if (splits > max_splits) splits = max_splits;
-        if (splits < 1) splits = 1;
-        p.chunk = round_up(ceil_div(M, splits), 64);
-        splits = ceil_div(M, p.chunk);
-        p.splits = static_cast<int>(splits);
-        if (tiles * splits > INT32_MAX) return TANGO_ERR_UNSUPPORTED;
+        p.chunk = t.chunk;
+        p.splits = static_cast<int>(t.splits);
+        if (tiles * t.splits > INT32_MAX) return TANGO_ERR_UNSUPPORTED;
         int64_t ra = 0, rb = 0;
         const int va = row_vec(dYq, lddy, N, &ra), vb = row_vec(Xq, ldx, K, &rb);
         const int vec = va < vb ? va : vb;
         p.a_row_bytes = (vec == 16) ? round_up(N, 16) : (vec == 4 ? round_up(N, 4) : N);
         p.b_row_bytes = (vec == 16) ? round_up(K, 16) : (vec == 4 ? round_up(K, 4) : K);
-        const dim3 grid(static_cast<unsigned>(tiles * splits));
+        const dim3 grid(static_cast<unsigned>(tiles * t.splits));
         if (vec == 16) hipLaunchKernelGGL(gemm_tn_kernel<16>, grid, dim3(256), 0, s, p);
         else if (vec == 4) hipLaunchKernelGGL(gemm_tn_kernel<4>, grid, dim3(256), 0, s, p);
         else hipLaunchKernelGGL(gemm_tn_kernel<1>, grid, dim3(256), 0, s, p);
     }
-    hipLaunchKernelGGL(dequant_i32_kernel, dim3(grid_for(N * K, 256)), dim3(256), 0, s, dW, lddw, acc,
-                       N, K, s_dY, s_X);
+    const int64_t quads = N * t.Kp / 4;
+    hipLaunchKernelGGL(tn_reduce_kernel, dim3(static_cast<unsigned>(ceil_div(quads, 16))), dim3(256), 0, s, dW, lddw,
+                       acc, N, K, t.Kp, static_cast<int>(t.splits), s_dY, s_X);
     return launch_status();
 }
 
