@@ -210,11 +210,13 @@ int tango_spmm_csr_u_mul_e(float* out, const int64_t* indptr, const int64_t* ind
    counterpart in the reference): edge_major != 0 means evals is [nnz, H, D] (what
    quantizing the [nnz, H, D] fp32 edge tensor in place yields, no transpose pass).
    With the slot->edge permutation fused, the H * D bytes of a gathered edge then
-   come from one cache sector instead of H * D scattered ones. */
+   come from one cache sector instead of H * D scattered ones.  bias (H * F floats or
+   NULL) is added after dequantization ("rst + bias", evaluation/test_gat.py:160-162). */
 int tango_spmm_csr_u_mul_e_ex(float* out, const int64_t* indptr, const int64_t* indices,
                               const int64_t* edge_ids, const int8_t* feat, const int8_t* evals,
-                              int edge_major, const float* scale, int64_t rows, int64_t num_src,
-                              int64_t H, int64_t F, int64_t D, int64_t nnz, tango_stream_t stream);
+                              int edge_major, const float* scale, const float* bias, int64_t rows,
+                              int64_t num_src, int64_t H, int64_t F, int64_t D, int64_t nnz,
+                              tango_stream_t stream);
 
 /* incidence_SPMM (cuda/src/cuda.cpp:160-167 -> incidence_SPMM_impl, SPMM.cu:259-303):
    out[v, f] = scale[0] * float(sum_{i: node_ids[i] == v} E[edge_ids[i], f]).
@@ -254,6 +256,24 @@ int tango_edge_softmax_fwd(float* a, const float* e, const int64_t* indptr,
 int tango_edge_softmax_bwd(float* de, const float* a, const float* da, const float* e,
                            const int64_t* indptr, const int64_t* edge_ids, int64_t rows,
                            int64_t H, float slope, tango_stream_t stream);
+
+/* ------------------------------------------------------ GAT attention logits */
+
+/* el[n,h] = sum_d feat[n,h,d] * attn_l[h,d], er likewise with attn_r: the two
+   broadcast-multiply + sum lines of the GAT layer (evaluation/test_gat.py:135-137),
+   torch ops in the reference, in one read of feat.  fp32. */
+int tango_attn_scores_fwd(float* el, float* er, const float* feat, const float* attn_l,
+                          const float* attn_r, int64_t n, int64_t H, int64_t D,
+                          tango_stream_t stream);
+
+/* Backward of the above: dfeat[n,h,d] = del[n,h]*attn_l[h,d] + der[n,h]*attn_r[h,d],
+   dattn_l[h,d] = sum_n del[n,h]*feat[n,h,d], dattn_r likewise; the sums over n are
+   reduced in a fixed order.  H <= 256.  workspace: tango_attn_scores_bwd_workspace bytes. */
+size_t tango_attn_scores_bwd_workspace(int64_t n, int64_t H, int64_t D);
+int tango_attn_scores_bwd(float* dfeat, float* dattn_l, float* dattn_r, const float* del,
+                          const float* der, const float* feat, const float* attn_l,
+                          const float* attn_r, int64_t n, int64_t H, int64_t D, void* workspace,
+                          size_t workspace_bytes, tango_stream_t stream);
 
 /* -------------------------------------------------------------------- loss */
 

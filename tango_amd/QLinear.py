@@ -19,13 +19,19 @@ def _padded_i8(rows, cols, device):
     return torch.empty((rows, ld), dtype=torch.int8, device=device)[:, :cols]
 
 
-def _quantize_grad(dY):
-    """Quantize a gradient (cuda/QLinear.py:42) with the configured rounding."""
+def _quantize_grad(dY, want_colsum=False):
+    """Quantize a gradient (cuda/QLinear.py:42) with the configured rounding.  Returns
+    (int8, scale, column sums or None): the bias gradient dY.sum(0) (cuda/QLinear.py:46)
+    comes out of the same read of dY that finds its scale."""
     dY = dY if dY.is_contiguous() else dY.contiguous()
+    scale = colsum = None
+    if want_colsum:
+        scale, colsum = kernels.cuda_kernels.absmax_ex(dY, want_colsum=True)
+    kw = {"round_mode": config.grad_round_mode}
     if config.grad_round_mode == "stochastic":
-        return kernels.quantize_padded(dY, round_mode="stochastic", seed=config.seed,
-                                       offset=config.next_offset())
-    return kernels.quantize_padded(dY, round_mode=config.grad_round_mode)
+        kw.update(seed=config.seed, offset=config.next_offset())
+    q, scale = kernels.quantize_padded(dY, scale, **kw)
+    return q, scale, colsum
 
 
 class QgemmNT_func(Function):
@@ -48,9 +54,12 @@ class QgemmNT_func(Function):
         return grad_A, grad_B
 
 
-def _forward(ctx, X, W, b, reduce, row_scale=None):
+def _forward(ctx, X, W, b, reduce, row_scale=None, scaleX=None):
     X = X if X.is_contiguous() else X.contiguous()
-    if row_scale is not None:
+    if scaleX is not None:
+        if row_scale is not None:
+            raise RuntimeError("QLinear: a precomputed input scale cannot be combined with row_scale")
+    elif row_scale is not None:
         # the layer's "X * row_scale[:, None]" is folded into the quantize pass (no fp32 copy of X)
         scaleX, _ = kernels.cuda_kernels.absmax_ex(X, row_mul=row_scale)
     else:
@@ -65,43 +74,43 @@ def _forward(ctx, X, W, b, reduce, row_scale=None):
 
 def _backward(ctx, grad_output):
     X_, scaleX, W_, scaleW, b, row_scale = ctx.backward_cache
-    grad_bias = None
-    dY_, scaledY = _quantize_grad(grad_output)
+    want_bias = b is not None and ctx.needs_input_grad[2]
+    dY_, scaledY, grad_bias = _quantize_grad(grad_output, want_bias)
     grad_input, grad_weight = kernels.QGEMM_backward(
         dY_, X_, W_, scaledY, scaleX, scaleW, ctx.needs_input_grad[0], ctx.needs_input_grad[1],
         x_row_scale=row_scale)
-    if b is not None and ctx.needs_input_grad[2]:
-        grad_bias = grad_output.sum(0)
     return grad_input, grad_weight, grad_bias, None
 
 
 class Qlinear_func(Function):
     """cuda/QLinear.py:26-47.  ``row_scale`` (optional, [M]) multiplies the rows of X before
-    quantization, fused into the quantize pass and, in backward, into gradX's epilogue."""
+    quantization, fused into the quantize pass and, in backward, into gradX's epilogue.
+    ``scaleX`` (optional, [1]) is max|X| / 127 when the producer of X already knows it
+    (a preceding Qlinear_func_reduce): no absmax pass over X runs then."""
 
     @staticmethod
-    def forward(ctx, X, W, b=None, row_scale=None):
-        return _forward(ctx, X, W, b, False, row_scale)
+    def forward(ctx, X, W, b=None, row_scale=None, scaleX=None):
+        return _forward(ctx, X, W, b, False, row_scale, scaleX)
 
     @staticmethod
     @once_differentiable
     def backward(ctx, grad_output):
-        return _backward(ctx, grad_output)
+        return _backward(ctx, grad_output) + (None,)
 
 
 class Qlinear_func_reduce(Function):
     """cuda/QLinear.py:50-71: also returns the output's quantization scale."""
 
     @staticmethod
-    def forward(ctx, X, W, b=None, row_scale=None):
-        out, scaleO = _forward(ctx, X, W, b, True, row_scale)
+    def forward(ctx, X, W, b=None, row_scale=None, scaleX=None):
+        out, scaleO = _forward(ctx, X, W, b, True, row_scale, scaleX)
         ctx.mark_non_differentiable(scaleO)
         return out, scaleO
 
     @staticmethod
     @once_differentiable
     def backward(ctx, grad_output, grad_dummy):
-        return _backward(ctx, grad_output)
+        return _backward(ctx, grad_output) + (None,)
 
 
 class QLinear(nn.Linear):
@@ -115,11 +124,13 @@ class QLinear(nn.Linear):
     def enable_reduce(self):
         self.isReduce = True
 
-    def forward(self, input):
+    def forward(self, input, scale=None):
+        """``scale``: max|input| / 127 if the caller has it (the second output of a preceding
+        layer with enable_reduce()); the reference's layer always recomputes it."""
         t = input.reshape(-1, input.size(-1))
         out_shape = input.shape[:-1] + (self.weight.size(0),)
         if self.isReduce:
-            out, scale = Qlinear_func_reduce.apply(t, self.weight, self.bias)
-            return out.reshape(out_shape), scale
-        out = Qlinear_func.apply(t, self.weight, self.bias)
+            out, oscale = Qlinear_func_reduce.apply(t, self.weight, self.bias, None, scale)
+            return out.reshape(out_shape), oscale
+        out = Qlinear_func.apply(t, self.weight, self.bias, None, scale)
         return out.reshape(out_shape)

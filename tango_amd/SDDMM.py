@@ -44,12 +44,13 @@ class sddmm_u_add_v(Function):
 
 class sddmm_u_dot_v(Function):
     """out[e, h, 0] = <U[src[e], h, :], V[dst[e], h, :]>.  Built by symmetry with
-    spmm_u_mul_e: the backward is two u_mul_e aggregations with dZ as the edge value."""
+    spmm_u_mul_e: the backward is two u_mul_e aggregations with dZ as the edge value.
+    ``scaleU_`` / ``scaleV_`` may come from the producers of U and V (as in sddmm_u_add_v)."""
 
     @staticmethod
-    def forward(ctx, g, U, V):
-        U_, scaleU = quantize(U if U.is_contiguous() else U.contiguous())
-        V_, scaleV = quantize(V if V.is_contiguous() else V.contiguous())
+    def forward(ctx, g, U, V, scaleU_=None, scaleV_=None):
+        U_, scaleU = quantize(U if U.is_contiguous() else U.contiguous(), scaleU_)
+        V_, scaleV = quantize(V if V.is_contiguous() else V.contiguous(), scaleV_)
         out, _ = mySDDMM_int8(g, "dot", U_, V_, scaleU, scaleV, False)
         ctx.backward_cache = g, U_, scaleU, V_, scaleV
         return out
@@ -69,4 +70,4 @@ class sddmm_u_dot_v(Function):
             dU = multi_cusparse_SPMM(g, V3, dZ_, scaledZ * scaleV, True, edge_major=True).reshape(U_.shape)
         if ctx.needs_input_grad[2]:
             dV = multi_cusparse_SPMM(g, U3, dZ_, scaledZ * scaleU, edge_major=True).reshape(V_.shape)
-        return None, dU, dV
+        return None, dU, dV, None, None

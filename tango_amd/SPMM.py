@@ -84,28 +84,42 @@ def _need_reduce_last_dim(ufeat, efeat):
 
 class spmm_u_mul_e(Function):
     """u_mul_e-sum aggregation with int8 node features and int8 edge values
-    (cuda/SPMM.py:36-62).  N is [n, H, F], E is [nnz, H, 1] in edge-id order."""
+    (cuda/SPMM.py:36-62).  N is [n, H, F], E is [nnz, H, 1] in edge-id order.
+
+    ``bias`` ([H * F]) folds the "rst + bias" that follows the aggregation in a GAT layer
+    (evaluation/test_gat.py:160-162) into the kernel's epilogue; its gradient then comes
+    out of the pass that finds the scale of dZ.  ``scaleN`` may come from the producer of N."""
 
     @staticmethod
-    def forward(ctx, g, N, E):
+    def forward(ctx, g, N, E, bias=None, scaleN=None):
         N = N if N.is_contiguous() else N.contiguous()
         E = E if E.is_contiguous() else E.contiguous()
         # Edge values stay edge-major ([nnz, H, 1], plain quantize): the reference transposes them to
         # [H, 1, nnz] (cuda/SPMM.py:41) and then permutes that with index_select; with the permutation
         # fused into the gather, edge-major keeps the H bytes of an edge in one cache sector.
         E_T_, scaleE = quantize(E)
-        N_, scaleN = quantize(N)  # one absmax pass (the reference runs two, cuda/SPMM.py:39,43)
+        N_, scaleN = quantize(N, scaleN)  # one absmax pass (the reference runs two, cuda/SPMM.py:39,43)
         scale = scaleN * scaleE
-        out = multi_cusparse_SPMM(g, N_, E_T_, scale, edge_major=True)
+        out = multi_cusparse_SPMM(g, N_, E_T_, scale, edge_major=True, bias=bias)
         reduce_last = _need_reduce_last_dim(N, E)
-        ctx.backward_cache = g, N_, scaleN, E_T_, scaleE, scale, reduce_last, E.shape
+        ctx.backward_cache = g, N_, scaleN, E_T_, scaleE, scale, reduce_last, E.shape, bias is not None
         return out
 
     @staticmethod
     @once_differentiable
     def backward(ctx, dZ):
-        g, N_, scaleN, E_T_, scaleE, scale, reduce_last, eshape = ctx.backward_cache
-        dZ_, scaledZ = _quantize_grad(dZ, False)
+        g, N_, scaleN, E_T_, scaleE, scale, reduce_last, eshape, has_bias = ctx.backward_cache
+        dbias = None
+        if has_bias and ctx.needs_input_grad[3]:
+            # the scale of dZ and the bias gradient (column sums) in one read
+            dZ = dZ if dZ.is_contiguous() else dZ.contiguous()
+            scaledZ, dbias = cuda_kernels.absmax_ex(dZ.view(dZ.size(0), -1), want_colsum=True)
+            kw = {"round_mode": config.grad_round_mode}
+            if config.grad_round_mode == "stochastic":
+                kw.update(seed=config.seed, offset=config.next_offset())
+            dZ_, _ = quantize(dZ, scaledZ, **kw)
+        else:
+            dZ_, scaledZ = _quantize_grad(dZ, False)
         dN = dE = None
         if ctx.needs_input_grad[1]:
             # dN = A^T (E * dZ): the dequantization scale is s_dZ * s_E.  The reference passes
@@ -116,4 +130,4 @@ class spmm_u_mul_e(Function):
             op = "dot" if reduce_last else "mul"
             dE, _ = mySDDMM_int8(g, op, N_, dZ_, scaleN, scaledZ, False)
             dE = dE.reshape(eshape)
-        return None, dN, dE
+        return None, dN, dE, dbias, None

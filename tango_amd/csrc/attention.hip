@@ -1,0 +1,203 @@
+// GAT attention logits per node and head, with their backward.
+//
+//   el[n, h] = sum_d feat[n, h, d] * attn_l[h, d]      er likewise with attn_r
+//
+// Not part of the reference's primitive layer: its GAT driver writes this as
+// broadcast-multiply + sum in torch (evaluation/test_gat.py:135-137), which costs
+// four elementwise/reduction passes forward and, backward, two column reductions
+// over all nodes that torch runs far below memory speed.  fp32, HBM-bound: the
+// forward reads feat once (4 bytes per element), the backward reads feat once and
+// writes d_feat once (8 bytes per element) and reduces the two [H, D] parameter
+// gradients in a fixed order (registers over a thread's rows, LDS over a
+// workgroup's threads, one slab per workgroup, then a finishing kernel), so the
+// result is deterministic.
+#include "common.hpp"
+
+namespace tango {
+
+constexpr int kDChunk = 16;       // columns of one head a backward thread keeps in registers
+constexpr int kBwdGroups = 1024;  // workgroups (slabs) of the backward reduction
+
+__global__ __launch_bounds__(256) void attn_scores_fwd_kernel(
+    float* __restrict__ el, float* __restrict__ er, const float* __restrict__ feat,
+    const float* __restrict__ al, const float* __restrict__ ar, int64_t total, int H, int D, int vec4) {
+    const int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;  // (node, head)
+    if (i >= total) return;
+    const int h = static_cast<int>(i % H);
+    const float* f = feat + i * D;
+    const float* a = al + static_cast<int64_t>(h) * D;
+    const float* b = ar + static_cast<int64_t>(h) * D;
+    float sl = 0.0f, sr = 0.0f;
+    if (vec4) {
+        for (int d = 0; d < D; d += 4) {
+            const f32x4 x = *reinterpret_cast<const f32x4*>(f + d);
+            const f32x4 u = *reinterpret_cast<const f32x4*>(a + d);
+            const f32x4 v = *reinterpret_cast<const f32x4*>(b + d);
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+                sl += x[k] * u[k];
+                sr += x[k] * v[k];
+            }
+        }
+    } else {
+        for (int d = 0; d < D; ++d) {
+            sl += f[d] * a[d];
+            sr += f[d] * b[d];
+        }
+    }
+    el[i] = sl;
+    er[i] = sr;
+}
+
+// blockDim.x = tpb, a multiple of H: thread t is head t % H of row slot t / H.  gridDim.y tiles D
+// in chunks of kDChunk.  part[b][2][H][D]: workgroup b's sums of del * feat and der * feat.
+__global__ __launch_bounds__(256) void attn_scores_bwd_kernel(
+    float* __restrict__ dfeat, float* __restrict__ part, const float* __restrict__ del,
+    const float* __restrict__ der, const float* __restrict__ feat, const float* __restrict__ al,
+    const float* __restrict__ ar, int64_t n, int H, int D, int vec4) {
+    __shared__ float red[256][2 * kDChunk + 1];
+    const int t = threadIdx.x;
+    const int tpb = blockDim.x;
+    const int h = t % H;
+    const int slots = tpb / H;
+    const int d0 = blockIdx.y * kDChunk;
+    const int dn = (D - d0) < kDChunk ? (D - d0) : kDChunk;
+    float wl[kDChunk], wr[kDChunk], accl[kDChunk], accr[kDChunk];
+#pragma unroll
+    for (int k = 0; k < kDChunk; ++k) {
+        wl[k] = k < dn ? al[static_cast<int64_t>(h) * D + d0 + k] : 0.0f;
+        wr[k] = k < dn ? ar[static_cast<int64_t>(h) * D + d0 + k] : 0.0f;
+        accl[k] = accr[k] = 0.0f;
+    }
+    const int64_t step = static_cast<int64_t>(gridDim.x) * slots;
+    for (int64_t r = static_cast<int64_t>(blockIdx.x) * slots + t / H; r < n; r += step) {
+        const int64_t i = r * H + h;
+        const float gl = del[i], gr = der[i];
+        const float* f = feat + i * D + d0;
+        float* o = dfeat + i * D + d0;
+        if (vec4) {  // whole chunks, 16-byte aligned
+#pragma unroll
+            for (int q = 0; q < kDChunk / 4; ++q) {
+                const f32x4 x = *reinterpret_cast<const f32x4*>(f + 4 * q);
+                f32x4 y;
+#pragma unroll
+                for (int k = 0; k < 4; ++k) {
+                    y[k] = gl * wl[4 * q + k] + gr * wr[4 * q + k];
+                    accl[4 * q + k] += gl * x[k];
+                    accr[4 * q + k] += gr * x[k];
+                }
+                *reinterpret_cast<f32x4*>(o + 4 * q) = y;
+            }
+            continue;
+        }
+#pragma unroll
+        for (int k = 0; k < kDChunk; ++k) {
+            if (k < dn) {
+                const float x = f[k];
+                o[k] = gl * wl[k] + gr * wr[k];
+                accl[k] += gl * x;
+                accr[k] += gr * x;
+            }
+        }
+    }
+#pragma unroll
+    for (int k = 0; k < kDChunk; ++k) {
+        red[t][k] = accl[k];
+        red[t][kDChunk + k] = accr[k];
+    }
+    __syncthreads();
+    // (which, head, column) sums over the workgroup's row slots, in slot order
+    for (int idx = t; idx < 2 * H * dn; idx += tpb) {
+        const int which = idx / (H * dn);
+        const int rem = idx - which * H * dn;
+        const int hh = rem / dn, k = rem - hh * dn;
+        float s = 0.0f;
+        for (int sl = 0; sl < slots; ++sl) s += red[sl * H + hh][which * kDChunk + k];
+        part[((static_cast<int64_t>(blockIdx.x) * 2 + which) * H + hh) * D + d0 + k] = s;
+    }
+}
+
+// out[0 .. 2 H D) = sum over slabs, sixteen slab lanes per element, fixed order.
+__global__ __launch_bounds__(256) void attn_scores_finish_kernel(float* __restrict__ dal, float* __restrict__ dar,
+                                                                 const float* __restrict__ part, int slabs,
+                                                                 int64_t hd) {
+    __shared__ float red[16][16];
+    const int e = threadIdx.x & 15, sl = threadIdx.x >> 4;
+    const int64_t idx = static_cast<int64_t>(blockIdx.x) * 16 + e;
+    float s = 0.0f;
+    if (idx < 2 * hd)
+        for (int b = sl; b < slabs; b += 16) s += part[static_cast<int64_t>(b) * 2 * hd + idx];
+    red[sl][e] = s;
+    __syncthreads();
+    if (sl == 0 && idx < 2 * hd) {
+        float tot = 0.0f;
+#pragma unroll
+        for (int w = 0; w < 16; ++w) tot += red[w][e];
+        if (idx < hd) dal[idx] = tot; else dar[idx - hd] = tot;
+    }
+}
+
+static int bwd_groups(int64_t n, int64_t H) {
+    const int64_t slots = (256 / H);
+    const int64_t g = ceil_div(n, slots);
+    return static_cast<int>(g < kBwdGroups ? (g < 1 ? 1 : g) : kBwdGroups);
+}
+
+}  // namespace tango
+
+using namespace tango;
+
+extern "C" {
+
+int tango_attn_scores_fwd(float* el, float* er, const float* feat, const float* attn_l,
+                          const float* attn_r, int64_t n, int64_t H, int64_t D, tango_stream_t stream) {
+    if (n < 0 || H < 0 || D < 0 || H >= (1LL << 31) || D >= (1LL << 31)) return TANGO_ERR_INVALID_ARG;
+    if (n * H == 0) return TANGO_OK;
+    if (!el || !er || (D > 0 && (!feat || !attn_l || !attn_r))) return TANGO_ERR_INVALID_ARG;
+    const int64_t total = n * H;
+    if (ceil_div(total, 256) > INT32_MAX) return TANGO_ERR_UNSUPPORTED;
+    const uintptr_t bits = reinterpret_cast<uintptr_t>(feat) | reinterpret_cast<uintptr_t>(attn_l) |
+                           reinterpret_cast<uintptr_t>(attn_r);
+    const int vec4 = (D % 4 == 0) && (bits & 15) == 0;
+    hipLaunchKernelGGL(attn_scores_fwd_kernel, dim3(static_cast<unsigned>(ceil_div(total, 256))), dim3(256), 0,
+                       as_stream(stream), el, er, feat, attn_l, attn_r, total, static_cast<int>(H),
+                       static_cast<int>(D), vec4);
+    return launch_status();
+}
+
+size_t tango_attn_scores_bwd_workspace(int64_t n, int64_t H, int64_t D) {
+    if (n <= 0 || H <= 0 || D <= 0 || H > 256) return 0;
+    return static_cast<size_t>(bwd_groups(n, H)) * 2 * H * D * sizeof(float);
+}
+
+int tango_attn_scores_bwd(float* dfeat, float* dattn_l, float* dattn_r, const float* del,
+                          const float* der, const float* feat, const float* attn_l,
+                          const float* attn_r, int64_t n, int64_t H, int64_t D, void* workspace,
+                          size_t workspace_bytes, tango_stream_t stream) {
+    if (n < 0 || H < 0 || D < 0) return TANGO_ERR_INVALID_ARG;
+    if (H * D == 0) return TANGO_OK;
+    if (H > 256 || D >= (1LL << 31) || ceil_div(D, kDChunk) > 65535) return TANGO_ERR_UNSUPPORTED;
+    if (!dattn_l || !dattn_r || !attn_l || !attn_r || (n > 0 && (!dfeat || !del || !der || !feat)))
+        return TANGO_ERR_INVALID_ARG;
+    hipStream_t s = as_stream(stream);
+    int groups = 0;
+    float* part = static_cast<float*>(workspace);
+    if (n > 0) {
+        const size_t need = tango_attn_scores_bwd_workspace(n, H, D);
+        if (!workspace || workspace_bytes < need) return TANGO_ERR_WORKSPACE;
+        if ((reinterpret_cast<uintptr_t>(workspace) & 3) != 0) return TANGO_ERR_INVALID_ARG;
+        groups = bwd_groups(n, H);
+        const int tpb = static_cast<int>((256 / H) * H);
+        const uintptr_t bits = reinterpret_cast<uintptr_t>(feat) | reinterpret_cast<uintptr_t>(dfeat);
+        const int vec4 = (D % kDChunk == 0) && (bits & 15) == 0;
+        hipLaunchKernelGGL(attn_scores_bwd_kernel,
+                           dim3(static_cast<unsigned>(groups), static_cast<unsigned>(ceil_div(D, kDChunk))),
+                           dim3(tpb), 0, s, dfeat, part, del, der, feat, attn_l, attn_r, n, static_cast<int>(H),
+                           static_cast<int>(D), vec4);
+    }
+    hipLaunchKernelGGL(attn_scores_finish_kernel, dim3(static_cast<unsigned>(ceil_div(2 * H * D, 16))), dim3(256), 0,
+                       s, dattn_l, dattn_r, part, groups, H * D);
+    return launch_status();
+}
+
+}  // extern "C"

@@ -388,20 +388,32 @@ __global__ __launch_bounds__(256) void absmax_ex_kernel(
     block_absmax_to_global(m / 127.0f, scale_out);
 }
 
-// blockDim = (64, 4): 64 columns per block; thread (x, y) sums partial rows y, y + 4, ...;
-// the four sums of a column are then added in a fixed order.
+// blockDim = (16, 16): 16 columns per block; thread (x, y) sums partial rows y, y + 16, ... with
+// four loads in flight; the sixteen sums of a column are then added in a fixed order.
 __global__ __launch_bounds__(256) void colsum_finish_kernel(const float* __restrict__ partial,
                                                             int64_t nrows, int64_t cols,
                                                             float* __restrict__ out) {
-    __shared__ float red[4][64];
-    const int64_t c = static_cast<int64_t>(blockIdx.x) * 64 + threadIdx.x;
-    float s = 0.0f;
-    if (c < cols)
-        for (int64_t r = threadIdx.y; r < nrows; r += 4) s += partial[r * cols + c];
-    red[threadIdx.y][threadIdx.x] = s;
+    __shared__ float red[16][16];
+    const int64_t c = static_cast<int64_t>(blockIdx.x) * 16 + threadIdx.x;
+    float a0 = 0.0f, a1 = 0.0f, a2 = 0.0f, a3 = 0.0f;
+    if (c < cols) {
+        int64_t r = threadIdx.y;
+        for (; r + 48 < nrows; r += 64) {
+            a0 += partial[r * cols + c];
+            a1 += partial[(r + 16) * cols + c];
+            a2 += partial[(r + 32) * cols + c];
+            a3 += partial[(r + 48) * cols + c];
+        }
+        for (; r < nrows; r += 16) a0 += partial[r * cols + c];
+    }
+    red[threadIdx.y][threadIdx.x] = (a0 + a1) + (a2 + a3);
     __syncthreads();
-    if (threadIdx.y == 0 && c < cols)
-        out[c] = ((red[0][threadIdx.x] + red[1][threadIdx.x]) + red[2][threadIdx.x]) + red[3][threadIdx.x];
+    if (threadIdx.y == 0 && c < cols) {
+        float s = 0.0f;
+#pragma unroll
+        for (int y = 0; y < 16; ++y) s += red[y][threadIdx.x];
+        out[c] = s;
+    }
 }
 
 template <typename F>
@@ -506,7 +518,7 @@ int tango_absmax_ex_f32(const float* x, int64_t rows, int64_t cols, int64_t ldx,
 #undef TANGO_AEX_T
 #undef TANGO_AEX
     if (colsum_out)
-        hipLaunchKernelGGL(colsum_finish_kernel, dim3(static_cast<unsigned>(ceil_div(cols, 64))), dim3(64, 4), 0,
+        hipLaunchKernelGGL(colsum_finish_kernel, dim3(static_cast<unsigned>(ceil_div(cols, 16))), dim3(16, 16), 0,
                            s, partial, static_cast<int64_t>(grid), cols, colsum_out);
     return launch_status();
 }

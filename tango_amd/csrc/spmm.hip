@@ -569,8 +569,9 @@ int tango_spmm_csr_copy_u_ex(float* out, const int64_t* indptr, const int64_t* i
 
 int tango_spmm_csr_u_mul_e_ex(float* out, const int64_t* indptr, const int64_t* indices,
                               const int64_t* edge_ids, const int8_t* feat, const int8_t* evals,
-                              int edge_major, const float* scale, int64_t rows, int64_t num_src,
-                              int64_t H, int64_t F, int64_t D, int64_t nnz, tango_stream_t stream) {
+                              int edge_major, const float* scale, const float* bias, int64_t rows,
+                              int64_t num_src, int64_t H, int64_t F, int64_t D, int64_t nnz,
+                              tango_stream_t stream) {
     if (rows < 0 || H < 0 || F < 0 || nnz < 0 || num_src < 0 || !scale || !indptr ||
         (rows * H * F > 0 && !out) || (nnz > 0 && (!indices || !feat || !evals)))
         return TANGO_ERR_INVALID_ARG;
@@ -578,7 +579,7 @@ int tango_spmm_csr_u_mul_e_ex(float* out, const int64_t* indptr, const int64_t* 
     if (num_src >= (1LL << 31) || nnz >= (1LL << 31)) return TANGO_ERR_UNSUPPORTED;
     SpmmParams p{};
     p.out = out; p.indptr = indptr; p.indices = indices; p.edge_ids = edge_ids; p.feat = feat;
-    p.evals = evals; p.scale = scale; p.rows = rows; p.num_src = num_src; p.ldf = H * F; p.W = H * F; p.F = F; p.D = D;
+    p.evals = evals; p.scale = scale; p.bias = bias; p.rows = rows; p.num_src = num_src; p.ldf = H * F; p.W = H * F; p.F = F; p.D = D;
     p.nnz = nnz;
     if (edge_major) {  // evals[nnz, H, D]: the H * D bytes of one edge share a cache sector
         p.ev_se = H * D; p.ev_sh = D; p.ev_sd = 1;
@@ -599,8 +600,8 @@ int tango_spmm_csr_u_mul_e(float* out, const int64_t* indptr, const int64_t* ind
                            const int64_t* edge_ids, const int8_t* feat, const int8_t* evals,
                            const float* scale, int64_t rows, int64_t num_src, int64_t H,
                            int64_t F, int64_t D, int64_t nnz, tango_stream_t stream) {
-    return tango_spmm_csr_u_mul_e_ex(out, indptr, indices, edge_ids, feat, evals, 0, scale, rows, num_src, H, F,
-                                     D, nnz, stream);
+    return tango_spmm_csr_u_mul_e_ex(out, indptr, indices, edge_ids, feat, evals, 0, scale, nullptr, rows, num_src,
+                                     H, F, D, nnz, stream);
 }
 
 int tango_spmm_incidence(float* out, const int64_t* node_ids, const int64_t* edge_ids,

@@ -339,10 +339,11 @@ class cuda_kernels:
                                           rows, U.size(0), indices.numel(), F, _stream()), "csr_SPMM")
 
     @staticmethod
-    def multi_cusparse_SPMM(indptr, indices, N, E_T, scale, edge_ids=None, edge_major=False):
+    def multi_cusparse_SPMM(indptr, indices, N, E_T, scale, edge_ids=None, edge_major=False, bias=None):
         """E_T is [H, D, nnz] in CSR slot order, or in edge-id order when the
         slot->edge permutation ``edge_ids`` is passed (gather fused in-kernel).
-        With ``edge_major`` the edge values are [nnz, H, D] instead (no transpose pass)."""
+        With ``edge_major`` the edge values are [nnz, H, D] instead (no transpose pass).
+        ``bias`` ([H * F] fp32) is added to every output row after dequantization."""
         _need(indptr, torch.int64, "indptr")
         _need(indices, torch.int64, "indices")
         _need(N, torch.int8, "N")
@@ -361,11 +362,15 @@ class cuda_kernels:
                 raise RuntimeError("multi_cusparse_SPMM: E_T must be [H, 1|F, nnz]")
         if edge_ids is not None:
             _need(edge_ids, torch.int64, "edge_ids")
+        if bias is not None:
+            _need(bias, torch.float32, "bias")
+            if bias.numel() != H * F:
+                raise RuntimeError("multi_cusparse_SPMM: bias must have H * F elements")
         rows = indptr.numel() - 1
         out = torch.empty((rows, H, F), dtype=torch.float32, device=N.device)
         check(_L.tango_spmm_csr_u_mul_e_ex(_ptr(out), indptr.data_ptr(), _ptr(indices), _ptr(edge_ids),
-                                           _ptr(N), _ptr(E_T), int(bool(edge_major)), scale.data_ptr(), rows,
-                                           k, H, F, D, nnz, _stream()), "multi_cusparse_SPMM")
+                                           _ptr(N), _ptr(E_T), int(bool(edge_major)), scale.data_ptr(),
+                                           _ptr(bias), rows, k, H, F, D, nnz, _stream()), "multi_cusparse_SPMM")
         return out
 
     # The reference's SpMV binding returns uninitialised memory (cuda/src/SPMM.cu:196-257)
@@ -445,6 +450,39 @@ class cuda_kernels:
                                         _ptr(edge_ids), indptr.numel() - 1, H, float(slope), _stream()),
               "edge_softmax_backward")
         return de
+
+    # ------------------------------------------------- GAT attention logits
+    @staticmethod
+    def attn_scores_forward(feat, attn_l, attn_r):
+        """el, er [n, H] from feat [n, H, D] and attn_l, attn_r [H, D] (evaluation/test_gat.py:135-137)."""
+        for t, nm in ((feat, "feat"), (attn_l, "attn_l"), (attn_r, "attn_r")):
+            _need(t, torch.float32, nm)
+        n, H, D = feat.shape
+        if attn_l.numel() != H * D or attn_r.numel() != H * D:
+            raise RuntimeError("attn_scores: attn_l / attn_r must have H * D elements")
+        el = torch.empty((n, H), dtype=torch.float32, device=feat.device)
+        er = torch.empty((n, H), dtype=torch.float32, device=feat.device)
+        check(_L.tango_attn_scores_fwd(_ptr(el), _ptr(er), _ptr(feat), _ptr(attn_l), _ptr(attn_r), n, H, D,
+                                       _stream()), "attn_scores_forward")
+        return el, er
+
+    @staticmethod
+    def attn_scores_backward(del_, der, feat, attn_l, attn_r):
+        """(dfeat [n, H, D], dattn_l [H, D], dattn_r [H, D])."""
+        for t, nm in ((del_, "del"), (der, "der"), (feat, "feat"), (attn_l, "attn_l"), (attn_r, "attn_r")):
+            _need(t, torch.float32, nm)
+        n, H, D = feat.shape
+        if del_.numel() != n * H or der.numel() != n * H:
+            raise RuntimeError("attn_scores_backward: del / der must have n * H elements")
+        dfeat = torch.empty_like(feat)
+        dal = torch.empty((H, D), dtype=torch.float32, device=feat.device)
+        dar = torch.empty((H, D), dtype=torch.float32, device=feat.device)
+        ws_bytes = _L.tango_attn_scores_bwd_workspace(n, H, D)
+        ws = _workspace(ws_bytes, feat.device)
+        check(_L.tango_attn_scores_bwd(_ptr(dfeat), _ptr(dal), _ptr(dar), _ptr(del_), _ptr(der), _ptr(feat),
+                                       _ptr(attn_l), _ptr(attn_r), n, H, D, _ptr(ws), ws_bytes, _stream()),
+              "attn_scores_backward")
+        return dfeat, dal, dar
 
 
 # ------------------------------------------------------------------ wrappers
@@ -550,7 +588,7 @@ def transpose_quant(data, scale):
     return data_.reshape((data.size(1), data.size(2), nrow))
 
 
-def multi_cusparse_SPMM(g, N, E_T, scale, reverse=False, edge_major=False):
+def multi_cusparse_SPMM(g, N, E_T, scale, reverse=False, edge_major=False, bias=None):
     """E_T is [H, D, nnz] in edge-id order.  cuda/kernels.py:122-136; the
     index_select by edge_ids of the reference happens inside the kernel.
     ``edge_major``: E_T is the quantized edge tensor as it is, [nnz, H, 1]."""
@@ -563,7 +601,7 @@ def multi_cusparse_SPMM(g, N, E_T, scale, reverse=False, edge_major=False):
     if edge_ids is not None and edge_ids.numel() == 0:
         edge_ids = None
     return cuda_kernels.multi_cusparse_SPMM(indptr, indices, N, E_T, scale, edge_ids=edge_ids,
-                                            edge_major=edge_major)
+                                            edge_major=edge_major, bias=bias)
 
 
 def incidence_SPMM(g, E, scaleE, reverse=False):

@@ -130,3 +130,88 @@ def test_cross_entropy_matches_torch(rows, classes):
     assert torch.allclose(x.grad, xr.grad, rtol=1e-5, atol=1e-8)
     # deterministic
     assert cross_entropy(x.detach(), y).item() == cross_entropy(x.detach(), y).item()
+
+
+@pytest.mark.parametrize("n,H,D", [(1000, 8, 16), (333, 3, 5), (50, 1, 64), (2049, 12, 20), (7, 70, 4)])
+def test_attn_scores_match_torch(K, n, H, D):
+    """fp32 kernel against the torch expression it replaces; only the summation order differs."""
+    g = torch.Generator().manual_seed(n + H)
+    feat = torch.randn(n, H, D, generator=g).cuda()
+    al = torch.randn(1, H, D, generator=g).cuda()
+    ar = torch.randn(1, H, D, generator=g).cuda()
+    el, er = K.cuda_kernels.attn_scores_forward(feat, al.contiguous(), ar.contiguous())
+    assert torch.allclose(el, (feat * al).sum(-1), rtol=1e-5, atol=1e-5)
+    assert torch.allclose(er, (feat * ar).sum(-1), rtol=1e-5, atol=1e-5)
+    dl = torch.randn(n, H, generator=g).cuda()
+    dr = torch.randn(n, H, generator=g).cuda()
+    dfeat, dal, dar = K.cuda_kernels.attn_scores_backward(dl, dr, feat, al.contiguous(), ar.contiguous())
+    want = dl.unsqueeze(-1) * al + dr.unsqueeze(-1) * ar
+    assert torch.equal(dfeat, want)  # two products and one sum per element, same roundings
+    f64 = feat.double()
+    assert torch.allclose(dal.double(), (dl.double().unsqueeze(-1) * f64).sum(0), rtol=1e-5, atol=1e-4)
+    assert torch.allclose(dar.double(), (dr.double().unsqueeze(-1) * f64).sum(0), rtol=1e-5, atol=1e-4)
+
+
+def test_attn_scores_autograd_matches_torch():
+    from tango_amd.gat import attn_scores
+    g = torch.Generator().manual_seed(5)
+    feat = torch.randn(400, 4, 8, generator=g).cuda().requires_grad_()
+    al = torch.randn(1, 4, 8, generator=g).cuda().requires_grad_()
+    ar = torch.randn(1, 4, 8, generator=g).cuda().requires_grad_()
+    w1, w2 = torch.randn(400, 4, 1, generator=g).cuda(), torch.randn(400, 4, 1, generator=g).cuda()
+    el, er = attn_scores.apply(feat, al, ar)
+    ((el * w1).sum() + (er * w2).sum()).backward()
+    got = [t.grad.clone() for t in (feat, al, ar)]
+    for t in (feat, al, ar):
+        t.grad = None
+    el2 = (feat * al).sum(-1).unsqueeze(-1)
+    er2 = (feat * ar).sum(-1).unsqueeze(-1)
+    ((el2 * w1).sum() + (er2 * w2).sum()).backward()
+    for a, b in zip(got, (feat.grad, al.grad, ar.grad)):
+        assert a.shape == b.shape and torch.allclose(a, b, rtol=1e-4, atol=1e-4)
+
+
+def test_u_mul_e_bias_epilogue(K):
+    """bias in the SpMM epilogue == separate add (same roundings); its gradient == column sums of dZ."""
+    from tango_amd.SPMM import spmm_u_mul_e
+    rng = np.random.default_rng(9)
+    n, e, H, F = 700, 9000, 4, 16
+    src, dst = rand_graph(rng, n, e)
+    g = make_graph(src, dst, n)
+    N = dev(rng.standard_normal((n, H, F)).astype(np.float32)).requires_grad_()
+    E = dev(rng.random((e, H, 1)).astype(np.float32)).requires_grad_()
+    bias = dev(rng.standard_normal(H * F).astype(np.float32)).requires_grad_()
+    dZ = dev(rng.standard_normal((n, H, F)).astype(np.float32))
+    out = spmm_u_mul_e.apply(g, N, E, bias)
+    out.backward(dZ)
+    got = [t.grad.clone() for t in (N, E, bias)]
+    for t in (N, E, bias):
+        t.grad = None
+    ref = spmm_u_mul_e.apply(g, N, E) + bias.view(1, H, F)
+    assert torch.equal(out, ref)
+    ref.backward(dZ)
+    assert torch.equal(got[0], N.grad) and torch.equal(got[1], E.grad)
+    assert torch.allclose(got[2], bias.grad, rtol=1e-5, atol=1e-4)
+
+
+def test_scale_hand_off_is_bit_identical(K):
+    """A layer fed the preceding GEMM epilogue's scale computes what it computes when it
+    runs its own absmax pass (the epilogue's max is over the stored fp32 outputs)."""
+    from tango_amd.QLinear import QLinear
+    torch.manual_seed(3)
+    x = torch.randn(3000, 96, device="cuda")
+    l1, l2 = QLinear(96, 128).cuda(), QLinear(128, 64).cuda()
+    ref = l2(l1(x))
+    l1.enable_reduce()
+    y, s = l1(x)
+    assert torch.equal(s, K.cuda_kernels.get_scale(y))
+    got = l2(y, s)
+    assert torch.equal(got, ref)
+    got.sum().backward()
+    g1 = [p.grad.clone() for p in list(l1.parameters()) + list(l2.parameters())]
+    for p in list(l1.parameters()) + list(l2.parameters()):
+        p.grad = None
+    l1.isReduce = False
+    l2(l1(x)).sum().backward()
+    for a, p in zip(g1, list(l1.parameters()) + list(l2.parameters())):
+        assert torch.equal(a, p.grad)
