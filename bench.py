@@ -21,7 +21,7 @@ HBM_PEAK_GBPS = 8000.0
 # Bytes that cross the L2 <-> fabric boundary per launch of the F=256 copy_u kernel on the default
 # benchmark graph: two rocprofv3 --pmc passes (FETCH_SIZE, then WRITE_SIZE, KiB per dispatch), each
 # scaled by what the same counter reads for a 1 GiB device copy (2.000 and 1.000).
-MEASURED_TRAFFIC_SPMM_F256 = 1.747e10
+MEASURED_TRAFFIC_SPMM_F256 = 1.405e10
 
 
 def parse():
@@ -337,7 +337,7 @@ def main():
     k_ms = timer.mean_ms("spmm_F256")
     alg = spmm_bytes(nnz, n, 256)
     achieved = alg / k_ms / 1e6
-    roofline = {"kernel": "spmm_kernel<16,4,copy_u> F=256", "bound": "hbm", "achieved": round(achieved, 1),
+    roofline = {"kernel": "spmm_kernel<16,1,copy_u> F=256 (two 128-column tiles)", "bound": "hbm", "achieved": round(achieved, 1),
                 "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4),
                 "traffic": MEASURED_TRAFFIC_SPMM_F256 if (args.nodes, args.edges) == (232965, 114_600_000) else None,
                 "avg_launch_ms": round(k_ms, 4), "algorithmic_bytes": alg,

@@ -45,7 +45,8 @@ struct SpmmParams {
     int64_t D;    // edge-value width (1 or F)
     int64_t ev_sh, ev_sd, ev_se;  // strides (bytes) of evals over head, value column, edge
     int64_t nnz;
-    int lpe_log2;  // log2(lanes per gathered row)
+    int lpe_log2;  // log2(lanes per gathered row piece)
+    int64_t tile;  // bytes of a gathered row one workgroup column (blockIdx.y) covers: lanes per piece * VEC
     int ldf_shift; // log2(ldf) when ldf is a power of two and all byte offsets fit 31 bits, else -1
     int out_vec;   // out rows may be stored as 16-byte vectors
     int64_t long_row;  // rows with more slots than this go to the sixteen-wave kernel
@@ -143,7 +144,7 @@ __device__ __forceinline__ LaneCols lane_cols(const SpmmParams& p, int lane) {
     c.grp = lane >> p.lpe_log2;
     c.sub = lane & (c.lpe - 1);
     c.sh = 6 - p.lpe_log2;
-    c.col = static_cast<int64_t>(blockIdx.y) * (kWave * VEC) + static_cast<int64_t>(c.sub) * VEC;
+    c.col = static_cast<int64_t>(blockIdx.y) * p.tile + static_cast<int64_t>(c.sub) * VEC;
     c.col_ok = c.col < p.W;
     // Lanes past the row's width read column 0 (a valid address) and never store, and the
     // group fold only mixes lanes of equal `sub`, so they need no masking.
@@ -284,7 +285,7 @@ __device__ __forceinline__ int64_t lower_bound_wave(const int64_t* a, int64_t n,
 }
 
 // blockDim.x = 256.  WPR = waves that share one output row (1 or 4).
-// gridDim.y tiles the columns in chunks of 64 * VEC bytes.
+// gridDim.y tiles the columns in chunks of p.tile bytes.
 // Rows with more than p.long_row slots are left to spmm_long_kernel.
 template <int VEC, int WPR, int KIND>
 __global__ __launch_bounds__(256) void spmm_kernel(const SpmmParams p) {
@@ -471,13 +472,19 @@ static int launch_spmm(SpmmParams p, int vec, hipStream_t s) {
     if (p.rows == 0 || p.W == 0) return TANGO_OK;
     const int64_t lanes = ceil_div(p.W, vec);
     p.lpe_log2 = lanes >= 64 ? 6 : ilog2_ceil(lanes);
+    // A gathered matrix far beyond the L2 (4 MB per XCD) is walked one 128-byte column tile at a
+    // time: gridDim.y orders the launch tile by tile, so at any moment the resident waves gather
+    // the same 128 columns and an L2 holds twice as many distinct rows' pieces as with 256-byte
+    // rows.  The index array is streamed once per tile, which the better hit rate outweighs.
+    if (vec == 16 && p.W >= 256 && p.num_src * p.ldf >= (16LL << 20)) p.lpe_log2 = 3;
+    p.tile = static_cast<int64_t>(vec) << p.lpe_log2;
     p.out_vec = (reinterpret_cast<uintptr_t>(p.out) & 15) == 0 && (p.W & 3) == 0;
     p.ldf_shift = -1;
     if (p.ldf > 0 && (p.ldf & (p.ldf - 1)) == 0 && p.num_src * p.ldf < (1LL << 31)) {
         p.ldf_shift = 0;
         while ((1LL << p.ldf_shift) < p.ldf) ++p.ldf_shift;
     }
-    const int64_t ychunks = ceil_div(p.W, 64 * vec);
+    const int64_t ychunks = ceil_div(p.W, p.tile);
     if (ychunks > 65535) return TANGO_ERR_UNSUPPORTED;
     // four waves split each row when rows are long AND wide (few neighbours per load instruction);
     // otherwise one wave per row, which amortises the per-row latencies over more edges
