@@ -189,8 +189,10 @@ int tango_spmm_csr_copy_u(float* out, const int64_t* indptr, const int64_t* indi
 /* As tango_spmm_csr_copy_u with the layer glue that follows the aggregation in
    evaluation/test_gcn.py:123-137 folded into the epilogue, in this order and with
    one fp32 rounding each: y = scale * float(sum); y *= row_scale[r] (if non-null);
-   y += bias[f] (if non-null); y = max(y, 0) (if relu). */
-int tango_spmm_csr_copy_u_ex(float* out, const int64_t* indptr, const int64_t* indices,
+   y += bias[f] (if non-null); y = max(y, 0) (if relu).
+   idx_bits: 64 (int64 indices, as the reference passes them) or 32 (a one-time int32
+   copy of the column indices made by the caller: half the index traffic). */
+int tango_spmm_csr_copy_u_ex(float* out, const int64_t* indptr, const void* indices, int idx_bits,
                              const int8_t* feat, int64_t ldf, const float* scale,
                              const float* row_scale, const float* bias, int relu, int64_t rows,
                              int64_t num_src, int64_t nnz, int64_t F, tango_stream_t stream);
@@ -211,9 +213,10 @@ int tango_spmm_csr_u_mul_e(float* out, const int64_t* indptr, const int64_t* ind
    quantizing the [nnz, H, D] fp32 edge tensor in place yields, no transpose pass).
    With the slot->edge permutation fused, the H * D bytes of a gathered edge then
    come from one cache sector instead of H * D scattered ones.  bias (H * F floats or
-   NULL) is added after dequantization ("rst + bias", evaluation/test_gat.py:160-162). */
-int tango_spmm_csr_u_mul_e_ex(float* out, const int64_t* indptr, const int64_t* indices,
-                              const int64_t* edge_ids, const int8_t* feat, const int8_t* evals,
+   NULL) is added after dequantization ("rst + bias", evaluation/test_gat.py:160-162).
+   idx_bits: width of the entries of indices and edge_ids, 64 or 32. */
+int tango_spmm_csr_u_mul_e_ex(float* out, const int64_t* indptr, const void* indices,
+                              const void* edge_ids, int idx_bits, const int8_t* feat, const int8_t* evals,
                               int edge_major, const float* scale, const float* bias, int64_t rows,
                               int64_t num_src, int64_t H, int64_t F, int64_t D, int64_t nnz,
                               tango_stream_t stream);

@@ -49,6 +49,7 @@ struct SpmmParams {
     int64_t tile;  // bytes of a gathered row one workgroup column (blockIdx.y) covers: lanes per piece * VEC
     int ldf_shift; // log2(ldf) when ldf is a power of two and all byte offsets fit 31 bits, else -1
     int out_vec;   // out rows may be stored as 16-byte vectors
+    int idx32;     // indices and edge_ids point to int32 arrays (half the index traffic); indptr stays int64
     int64_t long_row;  // rows with more slots than this go to the sixteen-wave kernel
     int64_t group_row; // sparse graphs: rows with at most this many slots are owned by a lane group
 };
@@ -127,6 +128,17 @@ __device__ __forceinline__ int64_t lower_bound_i64(const int64_t* a, int64_t n, 
     return lo;
 }
 
+// Entry i of an index array that is int64, or int32 when p.idx32 is set.  `stream`: the array is read
+// once front to back (nontemporal: it should not evict gathered rows from the L2).
+template <bool STREAM>
+__device__ __forceinline__ int load_index(const SpmmParams& p, const int64_t* a, int64_t i) {
+    if (p.idx32) {
+        const int* a32 = reinterpret_cast<const int*>(a);
+        return STREAM ? __builtin_nontemporal_load(a32 + i) : a32[i];
+    }
+    return static_cast<int>(STREAM ? __builtin_nontemporal_load(a + i) : a[i]);
+}
+
 // Per-lane view of the column tile a lane works on.
 struct LaneCols {
     int lpe, epi, grp, sub, sh;
@@ -178,11 +190,11 @@ __device__ __forceinline__ void wave_row_sum(const SpmmParams& p, const LaneCols
             const int64_t q = base + r * kWave + lane;
             const int64_t qc = q < end ? q : end - 1;  // clamped: the load is unconditional
             // streamed once: keep the index array from evicting feature rows out of L2
-            const int v = static_cast<int>(__builtin_nontemporal_load(p.indices + qc));
+            const int v = load_index<true>(p, p.indices, qc);
             my[r] = q < end ? v : -1;
             my_e[r] = 0;
             if (KIND == KIND_WEIGHTED && p.edge_ids)
-                my_e[r] = static_cast<int>(__builtin_nontemporal_load(p.edge_ids + qc));
+                my_e[r] = load_index<true>(p, p.edge_ids, qc);
         }
         // The 256 slots are walked as one flat sequence of steps (64 / lpe slots each), always
         // U steps per batch, so narrow rows (one step per 64 slots) keep U gathers in flight too.
@@ -360,11 +372,11 @@ __global__ __launch_bounds__(256) void spmm_group_kernel(const SpmmParams p) {
         for (int u = 0; u < U; ++u) {
             const bool ok = q + u < end;
             const int64_t qc = ok ? q + u : start;  // a valid slot: start < end inside the loop
-            const int j = static_cast<int>(p.indices[qc]);
+            const int j = load_index<false>(p, p.indices, qc);
             d[u] = Gather<VEC>::load(c.fcol + row_offset(j, p));
             uint32_t w = 1u;
             if (KIND == KIND_WEIGHTED) {
-                const int64_t pos = p.edge_ids ? p.edge_ids[qc] : qc;
+                const int64_t pos = p.edge_ids ? static_cast<int64_t>(load_index<false>(p, p.edge_ids, qc)) : qc;
                 w = static_cast<uint32_t>(static_cast<uint8_t>(c.wbase[pos * p.ev_se]));
             }
             m |= (ok ? w : 0u) << (8 * u);
@@ -559,33 +571,36 @@ int tango_spmm_csr_copy_u(float* out, const int64_t* indptr, const int64_t* indi
     return launch_spmm<KIND_COPY>(p, pick_vec(feat, ldf, F), as_stream(stream));
 }
 
-int tango_spmm_csr_copy_u_ex(float* out, const int64_t* indptr, const int64_t* indices,
+int tango_spmm_csr_copy_u_ex(float* out, const int64_t* indptr, const void* indices, int idx_bits,
                              const int8_t* feat, int64_t ldf, const float* scale,
                              const float* row_scale, const float* bias, int relu, int64_t rows,
                              int64_t num_src, int64_t nnz, int64_t F, tango_stream_t stream) {
     if (rows < 0 || F < 0 || nnz < 0 || num_src < 0 || ldf < F || !scale || !indptr ||
-        (rows * F > 0 && !out) || (nnz > 0 && (!indices || !feat)))
+        (rows * F > 0 && !out) || (nnz > 0 && (!indices || !feat)) || (idx_bits != 32 && idx_bits != 64))
         return TANGO_ERR_INVALID_ARG;
     if (num_src >= (1LL << 31) || nnz >= (1LL << 31)) return TANGO_ERR_UNSUPPORTED;
     SpmmParams p{};
-    p.out = out; p.indptr = indptr; p.indices = indices; p.feat = feat; p.scale = scale;
+    p.out = out; p.indptr = indptr; p.indices = static_cast<const int64_t*>(indices); p.idx32 = idx_bits == 32;
+    p.feat = feat; p.scale = scale;
     p.row_scale = row_scale; p.bias = bias; p.relu = relu ? 1 : 0;
     p.rows = rows; p.num_src = num_src; p.ldf = ldf; p.W = F; p.F = F; p.D = 1; p.nnz = nnz;
     return launch_spmm<KIND_COPY>(p, pick_vec(feat, ldf, F), as_stream(stream));
 }
 
-int tango_spmm_csr_u_mul_e_ex(float* out, const int64_t* indptr, const int64_t* indices,
-                              const int64_t* edge_ids, const int8_t* feat, const int8_t* evals,
+int tango_spmm_csr_u_mul_e_ex(float* out, const int64_t* indptr, const void* indices,
+                              const void* edge_ids, int idx_bits, const int8_t* feat, const int8_t* evals,
                               int edge_major, const float* scale, const float* bias, int64_t rows,
                               int64_t num_src, int64_t H, int64_t F, int64_t D, int64_t nnz,
                               tango_stream_t stream) {
     if (rows < 0 || H < 0 || F < 0 || nnz < 0 || num_src < 0 || !scale || !indptr ||
-        (rows * H * F > 0 && !out) || (nnz > 0 && (!indices || !feat || !evals)))
+        (rows * H * F > 0 && !out) || (nnz > 0 && (!indices || !feat || !evals)) ||
+        (idx_bits != 32 && idx_bits != 64))
         return TANGO_ERR_INVALID_ARG;
     if (D != 1 && D != F) return TANGO_ERR_UNSUPPORTED;
     if (num_src >= (1LL << 31) || nnz >= (1LL << 31)) return TANGO_ERR_UNSUPPORTED;
     SpmmParams p{};
-    p.out = out; p.indptr = indptr; p.indices = indices; p.edge_ids = edge_ids; p.feat = feat;
+    p.out = out; p.indptr = indptr; p.indices = static_cast<const int64_t*>(indices);
+    p.edge_ids = static_cast<const int64_t*>(edge_ids); p.idx32 = idx_bits == 32; p.feat = feat;
     p.evals = evals; p.scale = scale; p.bias = bias; p.rows = rows; p.num_src = num_src; p.ldf = H * F; p.W = H * F; p.F = F; p.D = D;
     p.nnz = nnz;
     if (edge_major) {  // evals[nnz, H, D]: the H * D bytes of one edge share a cache sector
@@ -607,7 +622,7 @@ int tango_spmm_csr_u_mul_e(float* out, const int64_t* indptr, const int64_t* ind
                            const int64_t* edge_ids, const int8_t* feat, const int8_t* evals,
                            const float* scale, int64_t rows, int64_t num_src, int64_t H,
                            int64_t F, int64_t D, int64_t nnz, tango_stream_t stream) {
-    return tango_spmm_csr_u_mul_e_ex(out, indptr, indices, edge_ids, feat, evals, 0, scale, nullptr, rows, num_src,
+    return tango_spmm_csr_u_mul_e_ex(out, indptr, indices, edge_ids, 64, feat, evals, 0, scale, nullptr, rows, num_src,
                                      H, F, D, nnz, stream);
 }
 

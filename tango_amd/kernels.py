@@ -39,6 +39,19 @@ def _need(t, dtype, name, contiguous=True):
     return t
 
 
+def _need_index(t, name):
+    """An index array: int64 as the reference passes it, or a caller-made int32 copy.  Returns its width."""
+    if not isinstance(t, torch.Tensor):
+        raise TypeError("%s must be a tensor" % name)
+    if t.dtype not in (torch.int64, torch.int32):
+        raise RuntimeError("%s: expected torch.int64 or torch.int32 but got %s" % (name, t.dtype))
+    if not t.is_cuda:
+        raise RuntimeError("%s must be on GPU" % name)
+    if not t.is_contiguous():
+        raise RuntimeError("%s must be contiguous" % name)
+    return 32 if t.dtype == torch.int32 else 64
+
+
 def _rows_view(t, name):
     """2-D row-major view with unit column stride; returns (tensor, row stride)."""
     if t.dim() != 2 or (t.size(1) > 1 and t.stride(1) != 1):
@@ -312,7 +325,7 @@ class cuda_kernels:
     def csr_SPMM(out, indptr, indices, U, scaleU, ldf=None, F=None, row_scale=None, bias=None, relu=False):
         _need(out, torch.float32, "out")
         _need(indptr, torch.int64, "indptr")
-        _need(indices, torch.int64, "indices")
+        idx_bits = _need_index(indices, "indices")
         _need(U, torch.int8, "U")
         _need(scaleU, torch.float32, "scaleU")
         rows = indptr.numel() - 1
@@ -321,7 +334,7 @@ class cuda_kernels:
         F = width if F is None else F
         if out.numel() != rows * F:
             raise RuntimeError("csr_SPMM: out must be [%d, %d]" % (rows, F))
-        if row_scale is None and bias is None and not relu:
+        if row_scale is None and bias is None and not relu and idx_bits == 64:
             check(_L.tango_spmm_csr_copy_u(_ptr(out), indptr.data_ptr(), _ptr(indices), _ptr(U), ldf,
                                            scaleU.data_ptr(), rows, U.size(0), indices.numel(), F,
                                            _stream()), "csr_SPMM")
@@ -334,7 +347,7 @@ class cuda_kernels:
             _need(bias, torch.float32, "bias")
             if bias.numel() != F:
                 raise RuntimeError("csr_SPMM: bias must have F entries")
-        check(_L.tango_spmm_csr_copy_u_ex(_ptr(out), indptr.data_ptr(), _ptr(indices), _ptr(U), ldf,
+        check(_L.tango_spmm_csr_copy_u_ex(_ptr(out), indptr.data_ptr(), _ptr(indices), idx_bits, _ptr(U), ldf,
                                           scaleU.data_ptr(), _ptr(row_scale), _ptr(bias), int(bool(relu)),
                                           rows, U.size(0), indices.numel(), F, _stream()), "csr_SPMM")
 
@@ -345,7 +358,7 @@ class cuda_kernels:
         With ``edge_major`` the edge values are [nnz, H, D] instead (no transpose pass).
         ``bias`` ([H * F] fp32) is added to every output row after dequantization."""
         _need(indptr, torch.int64, "indptr")
-        _need(indices, torch.int64, "indices")
+        idx_bits = _need_index(indices, "indices")
         _need(N, torch.int8, "N")
         _need(E_T, torch.int8, "E_T")
         _need(scale, torch.float32, "scale")
@@ -360,15 +373,15 @@ class cuda_kernels:
             D, nnz = E_T.size(1), E_T.size(2)
             if E_T.size(0) != H or nnz != indices.numel() or D not in (1, F):
                 raise RuntimeError("multi_cusparse_SPMM: E_T must be [H, 1|F, nnz]")
-        if edge_ids is not None:
-            _need(edge_ids, torch.int64, "edge_ids")
+        if edge_ids is not None and _need_index(edge_ids, "edge_ids") != idx_bits:
+            raise RuntimeError("multi_cusparse_SPMM: indices and edge_ids must have the same integer width")
         if bias is not None:
             _need(bias, torch.float32, "bias")
             if bias.numel() != H * F:
                 raise RuntimeError("multi_cusparse_SPMM: bias must have H * F elements")
         rows = indptr.numel() - 1
         out = torch.empty((rows, H, F), dtype=torch.float32, device=N.device)
-        check(_L.tango_spmm_csr_u_mul_e_ex(_ptr(out), indptr.data_ptr(), _ptr(indices), _ptr(edge_ids),
+        check(_L.tango_spmm_csr_u_mul_e_ex(_ptr(out), indptr.data_ptr(), _ptr(indices), _ptr(edge_ids), idx_bits,
                                            _ptr(N), _ptr(E_T), int(bool(edge_major)), scale.data_ptr(),
                                            _ptr(bias), rows, k, H, F, D, nnz, _stream()), "multi_cusparse_SPMM")
         return out
@@ -588,16 +601,23 @@ def transpose_quant(data, scale):
     return data_.reshape((data.size(1), data.size(2), nrow))
 
 
+def _csr_of(g, reverse):
+    """(indptr, indices, edge_ids) of the source-major (reverse) or destination-major CSR, with the
+    32-bit copies of indices / edge_ids when graph_preprocess made them."""
+    indptr, indices, edge_ids = g.adj_csr if reverse else g.adj_csc
+    narrow = getattr(g, "adj_csr32" if reverse else "adj_csc32", None)
+    if narrow is not None:
+        indices, edge_ids = narrow
+    return indptr, indices, edge_ids
+
+
 def multi_cusparse_SPMM(g, N, E_T, scale, reverse=False, edge_major=False, bias=None):
     """E_T is [H, D, nnz] in edge-id order.  cuda/kernels.py:122-136; the
     index_select by edge_ids of the reference happens inside the kernel.
     ``edge_major``: E_T is the quantized edge tensor as it is, [nnz, H, 1]."""
     assert E_T.ndim == 3 and N.ndim == 3, "E and N must be 3D tensors"
     assert E_T.size(2 if edge_major else 1) == 1, "Cannot broadcast E"
-    if reverse:
-        indptr, indices, edge_ids = g.adj_csr
-    else:
-        indptr, indices, edge_ids = g.adj_csc
+    indptr, indices, edge_ids = _csr_of(g, reverse)
     if edge_ids is not None and edge_ids.numel() == 0:
         edge_ids = None
     return cuda_kernels.multi_cusparse_SPMM(indptr, indices, N, E_T, scale, edge_ids=edge_ids,
@@ -609,7 +629,7 @@ def incidence_SPMM(g, E, scaleE, reverse=False):
     adjacency (the equivalence evaluation/test_incidence.py:14-22 relies on), which the graph
     already holds, so the row bounds come from indptr instead of a search in the COO node ids."""
     assert E.is_cuda and scaleE.is_cuda
-    indptr, _, edge_ids = g.adj_csr if reverse else g.adj_csc
+    indptr, _, edge_ids = _csr_of(g, reverse)
     out_shape = (g.num_nodes(),) + E.shape[1:]
     dim = math.prod(E.shape[1:])
     out = torch.empty((g.num_nodes(), dim), dtype=torch.float32, device=E.device)
@@ -620,10 +640,7 @@ def incidence_SPMM(g, E, scaleE, reverse=False):
 def csr_SPMM(g, N, scaleN, reverse=False, row_scale=None, bias=None, relu=False):
     """cuda/kernels.py:154-165.  N may be a 2-D view of a row-padded buffer.  ``row_scale`` / ``bias`` /
     ``relu`` fold "* norm, + bias, activation" (evaluation/test_gcn.py:123-137) into the kernel's epilogue."""
-    if reverse:
-        indptr, indices, _ = g.adj_csr
-    else:
-        indptr, indices, _ = g.adj_csc
+    indptr, indices, _ = _csr_of(g, reverse)
     feat_shape = N.shape[1:]
     out_shape = (g.num_nodes(),) + feat_shape
     dim = math.prod(N.shape[1:])

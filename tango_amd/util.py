@@ -1,4 +1,6 @@
 """Graph preprocessing: mirrors cuda/util.py of the reference."""
+import torch
+
 from .graph import Graph
 
 
@@ -16,4 +18,9 @@ def graph_preprocess(graph):
     graph.adj_csr = graph.adj_sparse("csr")
     graph.adj_csc = graph.adj_sparse("csc")
     graph.coo = graph.edges()
+    # One-time 32-bit copies of the column indices and edge ids (node and edge counts are below
+    # 2^31 wherever the kernels run): the aggregation kernels stream these arrays once per launch,
+    # and at 4 bytes per edge they cost half the traffic of the int64 arrays the reference passes.
+    graph.adj_csr32 = tuple(t.to(torch.int32) for t in graph.adj_csr[1:])
+    graph.adj_csc32 = tuple(t.to(torch.int32) for t in graph.adj_csc[1:])
     return graph
