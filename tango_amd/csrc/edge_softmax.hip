@@ -80,6 +80,24 @@ __global__ __launch_bounds__(256) void edge_softmax_bwd_kernel(
 // the ones of its tier; no list of rows is built in global memory.
 constexpr int kShortRow = 16;
 constexpr int kMediumValues = 2048;
+// A hub: a destination with more than kHubValues / Hp in-edges.  One workgroup walking it alone
+// would outlast the whole rest of the launch, so (when the caller passes a workspace) the long
+// tier only records such rows and two further launches cut each into kHubChunks chunks: partial
+// (max, sum) per chunk and head, then every chunk combines its row's partials and writes its part.
+constexpr int kHubValues = 32768;
+constexpr int kHubChunks = 32;
+constexpr int kMaxHubs = 256;     // hubs beyond this stay with the long tier's single workgroup
+constexpr int kHubGridY = 64;     // workgroup rows of the hub launches; each walks hubs y, y + 64, ...
+
+// Workspace: [0] hub count (int), then kMaxHubs x (p0, p1) int64, then the partials
+// [kMaxHubs][kHubChunks][Hp] of {float max; double sum} (backward: the double only).
+struct HubPartial {
+    double sum;
+    float mx;
+    float pad;
+};
+__host__ __device__ inline size_t hub_list_offset() { return 256; }
+__host__ __device__ inline size_t hub_partial_offset() { return 256 + sizeof(int64_t) * 2 * kMaxHubs; }
 
 __device__ __forceinline__ void softmax_merge(float& m, double& s, float m2, double s2) {
     const float mx = fmaxf(m, m2);
@@ -334,7 +352,7 @@ template <bool FWD>
 __global__ __launch_bounds__(1024) void edge_softmax_long_kernel(
     float* __restrict__ out, const float* __restrict__ a, const float* __restrict__ da,
     const float* __restrict__ e, const int64_t* __restrict__ indptr, const int64_t* __restrict__ eids,
-    int64_t rows, int H, int hp_log2, float slope) {
+    int64_t rows, int H, int hp_log2, float slope, void* __restrict__ hub_ws) {
     __shared__ float mred[16][64];
     __shared__ double sred[16][64];
     __shared__ int64_t lp0[1024], lp1[1024];
@@ -352,9 +370,20 @@ __global__ __launch_bounds__(1024) void edge_softmax_long_kernel(
         if (mine < rows) {
             const int64_t q0 = indptr[mine], q1 = indptr[mine + 1];
             if (row_tier(q1 - q0, hp_log2) == 2) {
-                const int k = atomicAdd(&nlist, 1);  // any order: rows are independent
-                lp0[k] = q0;
-                lp1[k] = q1;
+                int hub = -1;
+                if (hub_ws && (q1 - q0) > (kHubValues >> hp_log2)) {
+                    hub = atomicAdd(static_cast<int*>(hub_ws), 1);  // any order: rows are independent
+                    if (hub < kMaxHubs) {
+                        int64_t* hl = reinterpret_cast<int64_t*>(static_cast<char*>(hub_ws) + hub_list_offset());
+                        hl[2 * hub] = q0;
+                        hl[2 * hub + 1] = q1;
+                    }
+                }
+                if (hub < 0 || hub >= kMaxHubs) {
+                    const int k = atomicAdd(&nlist, 1);
+                    lp0[k] = q0;
+                    lp1[k] = q1;
+                }
             }
         }
         __syncthreads();
@@ -395,13 +424,92 @@ __global__ __launch_bounds__(1024) void edge_softmax_long_kernel(
     }
 }
 
-// Launches the three tiers.  FWD: out = a; otherwise out = de.
+// Hub launches.  blockDim.x = 256, grid = (kHubChunks, kHubGridY).  PHASE 0 writes the chunk's
+// partials, PHASE 1 combines the kHubChunks partials of the row (every chunk does so for itself,
+// in chunk order) and writes the chunk's outputs.
+template <bool FWD, int PHASE>
+__global__ __launch_bounds__(256) void edge_softmax_hub_kernel(
+    float* __restrict__ out, const float* __restrict__ a, const float* __restrict__ da,
+    const float* __restrict__ e, const int64_t* __restrict__ eids, int H, int hp_log2, float slope,
+    void* __restrict__ hub_ws) {
+    __shared__ float mred[4][64];
+    __shared__ double sred[4][64];
+    const int count = *static_cast<const int*>(hub_ws);
+    const int nhubs = count < kMaxHubs ? count : kMaxHubs;
+    const int64_t* hl = reinterpret_cast<const int64_t*>(static_cast<const char*>(hub_ws) + hub_list_offset());
+    HubPartial* part = reinterpret_cast<HubPartial*>(static_cast<char*>(hub_ws) + hub_partial_offset());
+    const int t = threadIdx.x, lane = lane_id(), wave = t >> 6;
+    const int hp = 1 << hp_log2;
+    const int h = t & (hp - 1);
+    const int c = blockIdx.x;
+    for (int hub = blockIdx.y; hub < nhubs; hub += gridDim.y) {
+        const int64_t p0 = hl[2 * hub], p1 = hl[2 * hub + 1];
+        const int64_t len = (p1 - p0 + kHubChunks - 1) / kHubChunks;
+        const int64_t c0 = p0 + len * c < p1 ? p0 + len * c : p1;
+        const int64_t c1 = c0 + len < p1 ? c0 + len : p1;
+        HubPartial* row_part = part + (static_cast<int64_t>(hub) * kHubChunks << hp_log2);
+        if (PHASE == 0) {
+            float mx = -INFINITY;
+            double sum = 0.0;
+            if (FWD) {
+                fwd_partial<8>(e, eids, c0, c1, t, 256, H, hp_log2, slope, mx, sum);
+                for (int off = hp; off < kWave; off <<= 1) {
+                    const float m2 = __shfl_xor(mx, off, kWave);
+                    const double s2 = __shfl_xor(sum, off, kWave);
+                    softmax_merge(mx, sum, m2, s2);
+                }
+            } else {
+                sum = bwd_partial<8>(a, da, eids, c0, c1, t, 256, H, hp_log2);
+                for (int off = hp; off < kWave; off <<= 1) sum += __shfl_xor(sum, off, kWave);
+            }
+            if (lane < hp) {
+                mred[wave][lane] = mx;
+                sred[wave][lane] = sum;
+            }
+            __syncthreads();
+            if (t < hp) {
+                mx = mred[0][t];
+                sum = sred[0][t];
+                for (int w = 1; w < 4; ++w) {
+                    if (FWD) softmax_merge(mx, sum, mred[w][t], sred[w][t]);
+                    else sum += sred[w][t];
+                }
+                row_part[(c << hp_log2) + t] = HubPartial{sum, mx, 0.0f};
+            }
+            __syncthreads();
+        } else {
+            float mx = -INFINITY;
+            double sum = 0.0;
+            for (int k = 0; k < kHubChunks; ++k) {
+                const HubPartial q = row_part[(k << hp_log2) + h];
+                if (FWD) softmax_merge(mx, sum, q.mx, q.sum);
+                else sum += q.sum;
+            }
+            if (FWD) fwd_write<8>(out, e, eids, c0, c1, t, 256, H, hp_log2, slope, mx, static_cast<float>(1.0 / sum));
+            else bwd_write<8>(out, a, da, e, eids, c0, c1, t, 256, H, hp_log2, slope, static_cast<float>(sum));
+        }
+    }
+}
+
+// Launches the tiers.  FWD: out = a; otherwise out = de.  hub_ws may be null.
 template <bool FWD>
 static void launch_tiers(float* out, const float* a, const float* da, const float* e, const int64_t* indptr,
-                         const int64_t* eids, int64_t rows, int H, float slope, hipStream_t s) {
+                         const int64_t* eids, int64_t rows, int H, float slope, void* hub_ws, hipStream_t s) {
     int hp = 0;
     while ((1 << hp) < H) ++hp;
     const unsigned sgrid = static_cast<unsigned>(ceil_div(rows * H, 256));
+    if (hub_ws) fill_u32(hub_ws, 0u, 1, s);  // the hub counter
+    // the long tier first: its workgroups are the last to finish
+    hipLaunchKernelGGL(edge_softmax_long_kernel<FWD>,
+                       dim3(static_cast<unsigned>(rows < kLongGrid ? rows : kLongGrid)), dim3(1024), 0,
+                       s, out, a, da, e, indptr, eids, rows, H, hp, slope, hub_ws);
+    if (hub_ws) {
+        const dim3 hgrid(kHubChunks, kHubGridY);
+        hipLaunchKernelGGL((edge_softmax_hub_kernel<FWD, 0>), hgrid, dim3(256), 0, s, out, a, da, e, eids, H, hp, slope,
+                           hub_ws);
+        hipLaunchKernelGGL((edge_softmax_hub_kernel<FWD, 1>), hgrid, dim3(256), 0, s, out, a, da, e, eids, H, hp, slope,
+                           hub_ws);
+    }
     if (FWD)
         hipLaunchKernelGGL(edge_softmax_fwd_short_kernel, dim3(sgrid), dim3(256), 0, s, out, e, indptr, eids, rows, H,
                            slope);
@@ -410,9 +518,13 @@ static void launch_tiers(float* out, const float* a, const float* da, const floa
                            rows, H, slope);
     hipLaunchKernelGGL(edge_softmax_medium_kernel<FWD>, dim3(static_cast<unsigned>(ceil_div(rows, 4 * kRowsPerWave))),
                        dim3(256), 0, s, out, a, da, e, indptr, eids, rows, H, hp, slope);
-    hipLaunchKernelGGL(edge_softmax_long_kernel<FWD>,
-                       dim3(static_cast<unsigned>(rows < kLongGrid ? rows : kLongGrid)), dim3(1024), 0,
-                       s, out, a, da, e, indptr, eids, rows, H, hp, slope);
+}
+
+static size_t hub_workspace_bytes(int64_t H) {
+    if (H <= 0 || H > 64) return 0;
+    int hp = 0;
+    while ((1 << hp) < H) ++hp;
+    return hub_partial_offset() + (static_cast<size_t>(kMaxHubs) * kHubChunks << hp) * sizeof(HubPartial);
 }
 
 }  // namespace tango
@@ -421,14 +533,18 @@ using namespace tango;
 
 extern "C" {
 
+size_t tango_edge_softmax_workspace(int64_t H) { return hub_workspace_bytes(H); }
+
 int tango_edge_softmax_fwd(float* a, const float* e, const int64_t* indptr,
                            const int64_t* edge_ids, int64_t rows, int64_t H, float slope,
-                           tango_stream_t stream) {
+                           void* workspace, size_t workspace_bytes, tango_stream_t stream) {
     if (rows < 0 || H < 0 || (rows > 0 && !indptr) || H >= (1LL << 31)) return TANGO_ERR_INVALID_ARG;
     if (rows * H == 0) return TANGO_OK;
     if (!a || !e) return TANGO_ERR_INVALID_ARG;
     if (H <= 64 && rows * H <= 256LL * INT32_MAX) {
-        launch_tiers<true>(a, nullptr, nullptr, e, indptr, edge_ids, rows, static_cast<int>(H), slope,
+        if (workspace && (workspace_bytes < hub_workspace_bytes(H) || (reinterpret_cast<uintptr_t>(workspace) & 15)))
+            return TANGO_ERR_WORKSPACE;
+        launch_tiers<true>(a, nullptr, nullptr, e, indptr, edge_ids, rows, static_cast<int>(H), slope, workspace,
                            as_stream(stream));
         return launch_status();
     }
@@ -439,12 +555,16 @@ int tango_edge_softmax_fwd(float* a, const float* e, const int64_t* indptr,
 
 int tango_edge_softmax_bwd(float* de, const float* a, const float* da, const float* e,
                            const int64_t* indptr, const int64_t* edge_ids, int64_t rows,
-                           int64_t H, float slope, tango_stream_t stream) {
+                           int64_t H, float slope, void* workspace, size_t workspace_bytes,
+                           tango_stream_t stream) {
     if (rows < 0 || H < 0 || (rows > 0 && !indptr) || H >= (1LL << 31)) return TANGO_ERR_INVALID_ARG;
     if (rows * H == 0) return TANGO_OK;
     if (!de || !a || !da || !e) return TANGO_ERR_INVALID_ARG;
     if (H <= 64 && rows * H <= 256LL * INT32_MAX) {
-        launch_tiers<false>(de, a, da, e, indptr, edge_ids, rows, static_cast<int>(H), slope, as_stream(stream));
+        if (workspace && (workspace_bytes < hub_workspace_bytes(H) || (reinterpret_cast<uintptr_t>(workspace) & 15)))
+            return TANGO_ERR_WORKSPACE;
+        launch_tiers<false>(de, a, da, e, indptr, edge_ids, rows, static_cast<int>(H), slope, workspace,
+                            as_stream(stream));
         return launch_status();
     }
     hipLaunchKernelGGL(edge_softmax_bwd_kernel, dim3(grid_for(rows * H, 256, 16)), dim3(256), 0,

@@ -85,13 +85,15 @@ def test_unknown_op_raises(K):
 
 
 # (n, e): mostly medium rows, and mostly short rows with some destinations empty; both get hubs
-@pytest.mark.parametrize("n,e", [(900, 40000), (6000, 30000)])
+@pytest.mark.parametrize("n,e", [(900, 40000), (6000, 30000), (500, 90000)])
 @pytest.mark.parametrize("H", [1, 3, 8, 64, 70])
 @pytest.mark.parametrize("slope", [1.0, 0.2])
 def test_edge_softmax(K, orc, H, slope, n, e):
     rng = np.random.default_rng(H)
     src, dst = rand_graph(rng, n, e)
     dst[:5000] = 3  # one high-degree destination
+    if e > 60000:
+        dst[:40000] = 3  # a hub for every H: cut over many workgroups through the workspace
     dst[5000:5300] = 7  # and one between the wavefront and workgroup thresholds for small H
     g = make_graph(src, dst, n)
     o = orc.graph_formats(src, dst, n)
