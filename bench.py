@@ -178,6 +178,45 @@ def sddmm_primitives(K, torch):
     return out
 
 
+def model_steps(K, torch):
+    """The other model configurations, one training step each (forward + loss + backward + Adam):
+    the 3-layer GAT (hidden 16 x 8 heads, evaluation/test_gat.py:170-214) on the 169,343-node graph
+    and two HGT layers (256-d, 4 heads) on the homogenised 3-type / 4-relation graph."""
+    from tango_amd.gat import GAT, HGTStack
+    from tango_amd.graph import chung_lu, hetero_power_law
+    from tango_amd.loss import cross_entropy
+    from tango_amd.util import graph_preprocess
+    out = {}
+    torch.manual_seed(4)
+    g = graph_preprocess(chung_lu(169343, 1166243, 2.2, seed=4, device="cuda"))
+    n = g.num_nodes()
+    model = GAT(g, 3, 128, 16, 40, [8, 8, 1], torch.nn.functional.elu).cuda()
+    x = torch.randn(n, 128, device="cuda")
+    labels = torch.randint(0, 16, (n,), device="cuda")
+    opt = torch.optim.Adam(model.parameters(), lr=1e-3)
+
+    def gat_step():
+        opt.zero_grad(set_to_none=True)
+        cross_entropy(model(x), labels).backward()
+        opt.step()
+    out["gat3_step_169343n_1.34Me_ms"] = round(time_op(gat_step, iters=10, warm=3), 3)
+    del model, opt, x, g
+    g, _, _ = hetero_power_law(device="cuda")
+    g = graph_preprocess(g)
+    n = g.num_nodes()
+    hgt = HGTStack(256, 256, 16, 4, n_layers=2).cuda()
+    xh = torch.randn(n, 256, device="cuda")
+    lh = torch.randint(0, 16, (n,), device="cuda")
+    opth = torch.optim.Adam(hgt.parameters(), lr=1e-3)
+
+    def hgt_step():
+        opth.zero_grad(set_to_none=True)
+        cross_entropy(hgt(g, xh), lh).backward()
+        opth.step()
+    out["hgt2_step_170000n_8.17Me_ms"] = round(time_op(hgt_step, iters=10, warm=3), 3)
+    return out
+
+
 def cpu_baseline(g, X, W1, W2, frac, reps=3):
     """The CPU oracle (a port of the reference's semantics, OpenMP over the host
     cores) on every k-th destination row / node of the same workload:
@@ -365,6 +404,7 @@ def main():
     if not args.no_primitives:
         prims = primitives(g, K, torch)
         prims.update(sddmm_primitives(K, torch))
+        prims.update(model_steps(K, torch))
         result["primitives"] = prims
         result["spmm_GBps"] = prims["spmm_copy_u_F256"]["GBps"]
         result["sddmm_GBps"] = prims["sddmm_dot_H8_D16"]["GBps"]

@@ -51,6 +51,8 @@ struct SpmmParams {
     int out_vec;   // out rows may be stored as 16-byte vectors
     int idx32;     // indices and edge_ids point to int32 arrays (half the index traffic); indptr stays int64
     int64_t long_row;  // rows with more slots than this go to the sixteen-wave kernel
+    int64_t hub_row;   // rows with more slots than this are cut over several workgroups
+    int64_t max_row;   // caller's upper bound of the longest row, 0 if unknown
     int64_t group_row; // sparse graphs: rows with at most this many slots are owned by a lane group
 };
 
@@ -348,9 +350,15 @@ __global__ __launch_bounds__(256) void spmm_kernel(const SpmmParams p) {
 // of its gather slots empty and the launch would be bound by per-wave latency chains.  Here every
 // group of `lpe` lanes owns a row of its own (64 / lpe rows per wavefront) and walks it four
 // neighbours at a time; rows with more than p.group_row slots are left to spmm_medium_kernel.
+constexpr int kGroupRow = 32;  // most slots of a row that a lane group owns
+
 template <int VEC, int KIND>
 __global__ __launch_bounds__(256) void spmm_group_kernel(const SpmmParams p) {
     constexpr int U = 4;
+    // a wave's groups stage their rows' column indices (and edge ids) here, so that the gather loop
+    // holds no dependent index load; used when a wave has at most 16 groups
+    __shared__ int sidx[4][16 * kGroupRow];
+    __shared__ int seid[KIND == KIND_WEIGHTED ? 4 : 1][KIND == KIND_WEIGHTED ? 16 * kGroupRow : 1];
     const int lane = lane_id();
     const int wave = __builtin_amdgcn_readfirstlane(static_cast<int>(threadIdx.x) >> 6);
     const LaneCols c = lane_cols<VEC, KIND>(p, lane);
@@ -360,28 +368,52 @@ __global__ __launch_bounds__(256) void spmm_group_kernel(const SpmmParams p) {
         start = p.indptr[row];
         end = p.indptr[row + 1];
     }
-    const bool mine = row < p.rows && end - start <= p.group_row;
-    if (!mine) end = start;
+    const bool mine = row < p.rows && end - start <= kGroupRow;
+    const int deg = mine ? static_cast<int>(end - start) : 0;
+    const bool staged = p.lpe_log2 >= 2;
+    const bool permuted = KIND == KIND_WEIGHTED && p.edge_ids;
+    if (staged) {
+        for (int k = c.sub; k < deg; k += c.lpe) {
+            sidx[wave][(c.grp << 5) + k] = load_index<false>(p, p.indices, start + k);
+            if (permuted) seid[KIND == KIND_WEIGHTED ? wave : 0][(c.grp << 5) + k] = load_index<false>(p, p.edge_ids, start + k);
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    }
     int acc[VEC];
 #pragma unroll
     for (int i = 0; i < VEC; ++i) acc[i] = 0;
-    for (int64_t q = start; q < end; q += U) {  // trip counts differ between the groups of a wave
-        typename Gather<VEC>::T d[U];
-        uint32_t m = 0u;
+    // four gathers of slots q .. q + 3 (slots past the row's end read its first neighbour with multiplier 0)
+    auto issue = [&](typename Gather<VEC>::T* d, uint32_t& m, int q) {
+        m = 0u;
 #pragma unroll
         for (int u = 0; u < U; ++u) {
-            const bool ok = q + u < end;
-            const int64_t qc = ok ? q + u : start;  // a valid slot: start < end inside the loop
-            const int j = load_index<false>(p, p.indices, qc);
+            const bool ok = q + u < deg;
+            const int slot = ok ? q + u : 0;
+            const int j = staged ? sidx[wave][(c.grp << 5) + slot] : load_index<false>(p, p.indices, start + slot);
             d[u] = Gather<VEC>::load(c.fcol + row_offset(j, p));
             uint32_t w = 1u;
             if (KIND == KIND_WEIGHTED) {
-                const int64_t pos = p.edge_ids ? static_cast<int64_t>(load_index<false>(p, p.edge_ids, qc)) : qc;
+                int64_t pos = start + slot;
+                if (permuted)
+                    pos = staged ? seid[KIND == KIND_WEIGHTED ? wave : 0][(c.grp << 5) + slot]
+                                 : load_index<false>(p, p.edge_ids, start + slot);
                 w = static_cast<uint32_t>(static_cast<uint8_t>(c.wbase[pos * p.ev_se]));
             }
             m |= (ok ? w : 0u) << (8 * u);
         }
-        accumulate4<VEC>(acc, d, m);
+    };
+    // two batches in flight: the next one is issued before the current one is consumed
+    typename Gather<VEC>::T da[U], db[U];
+    uint32_t ma = 0u, mb = 0u;
+    if (deg > 0) issue(da, ma, 0);
+    for (int q = 0; q < deg; q += 2 * U) {  // trip counts differ between the groups of a wave
+        const bool has_b = q + U < deg;
+        if (has_b) issue(db, mb, q + U);
+        accumulate4<VEC>(acc, da, ma);
+        if (q + 2 * U < deg) issue(da, ma, q + 2 * U);
+        if (has_b) accumulate4<VEC>(acc, db, mb);
     }
     if (mine) store_row<VEC>(p, c, row, acc);
 }
@@ -421,9 +453,19 @@ __global__ __launch_bounds__(256) void spmm_medium_kernel(const SpmmParams p) {
 // (then b + G * (1024 + t), ...; hub rows with neighbouring ids land in different workgroups),
 // the long ones are collected in LDS and each is summed by all waves; the waves' partial sums
 // meet in LDS through integer atomics, which are exact in any order.
+//
+// Hub rows (more than p.hub_row slots) would still keep one workgroup busy long after the rest of
+// the launch has drained, so they take three steps, each a launch of this kernel:
+//   LONG      zeroes the hub row's output, viewed as int32 (and sums the ordinary long rows);
+//   HUB_SUM   gridDim.z = kHubChunks workgroups per hub row each sum one chunk of its slots and add
+//             the int32 result into the output row with integer atomics (exact in any order);
+//   HUB_STORE turns the int32 sums into the fp32 result in place.
 constexpr int kLongGrid = 512;
+constexpr int kHubChunks = 16;
+constexpr int kHubGrid = 32;  // scanning workgroups of the hub launches (x kHubChunks): hubs are few
+enum { LONG = 0, HUB_SUM = 1, HUB_STORE = 2 };
 
-template <int VEC, int KIND>
+template <int VEC, int KIND, int MODE>
 __global__ __launch_bounds__(1024) void spmm_long_kernel(const SpmmParams p) {
     constexpr int WAVES = 16;
     __shared__ int part[64 * VEC];
@@ -442,7 +484,8 @@ __global__ __launch_bounds__(1024) void spmm_long_kernel(const SpmmParams p) {
         if (mine < p.rows) {
             int64_t s, e;
             row_range<KIND>(p, mine, s, e);
-            if (e - s > p.long_row) list[atomicAdd(&nlist, 1)] = mine;  // any order: rows are independent
+            const bool take = (MODE == LONG) ? (e - s > p.long_row) : (e - s > p.hub_row);
+            if (take) list[atomicAdd(&nlist, 1)] = mine;  // any order: rows are independent
         }
         __syncthreads();
         const int n = nlist;
@@ -450,6 +493,31 @@ __global__ __launch_bounds__(1024) void spmm_long_kernel(const SpmmParams p) {
             const int64_t row = list[k];
             int64_t start, end;
             row_range<KIND>(p, row, start, end);
+            int* orow = reinterpret_cast<int*>(p.out) + row * p.W + c.col;  // this lane's VEC output columns
+            if (MODE == HUB_STORE || (MODE == LONG && end - start > p.hub_row)) {
+                if (wave == 0 && c.grp == 0 && c.col_ok) {
+                    int acc[VEC];
+#pragma unroll
+                    for (int i = 0; i < VEC; ++i) {
+                        acc[i] = 0;
+                        if (MODE == HUB_STORE && c.col + i < p.W) acc[i] = orow[i];
+                    }
+                    if (MODE == HUB_STORE) {
+                        store_row<VEC>(p, c, row, acc);
+                    } else {
+#pragma unroll
+                        for (int i = 0; i < VEC; ++i)
+                            if (c.col + i < p.W) orow[i] = 0;
+                    }
+                }
+                continue;  // uniform over the workgroup
+            }
+            if (MODE == HUB_SUM) {  // this workgroup's chunk of the row
+                const int64_t len = (end - start + kHubChunks - 1) / kHubChunks;
+                const int64_t cs = start + len * blockIdx.z;
+                start = cs < end ? cs : end;
+                end = cs + len < end ? cs + len : end;
+            }
             const int64_t per = (end - start + WAVES - 1) / WAVES;
             const int64_t s = start + per * wave;
             const int64_t e = s + per;
@@ -466,7 +534,15 @@ __global__ __launch_bounds__(1024) void spmm_long_kernel(const SpmmParams p) {
                     acc[i] = part[i * 64 + c.sub];
                     part[i * 64 + c.sub] = 0;
                 }
-                store_row<VEC>(p, c, row, acc);
+                if (MODE == HUB_SUM) {
+                    if (c.col_ok) {
+#pragma unroll
+                        for (int i = 0; i < VEC; ++i)
+                            if (c.col + i < p.W) atomicAdd(orow + i, acc[i]);
+                    }
+                } else {
+                    store_row<VEC>(p, c, row, acc);
+                }
             }
             __syncthreads();
         }
@@ -488,7 +564,8 @@ static int launch_spmm(SpmmParams p, int vec, hipStream_t s) {
     // time: gridDim.y orders the launch tile by tile, so at any moment the resident waves gather
     // the same 128 columns and an L2 holds twice as many distinct rows' pieces as with 256-byte
     // rows.  The index array is streamed once per tile, which the better hit rate outweighs.
-    if (vec == 16 && p.W >= 256 && p.num_src * p.ldf >= (16LL << 20)) p.lpe_log2 = 3;
+    if (vec == 16 && p.W >= 256 && p.num_src * p.ldf >= (16LL << 20) && (KIND == KIND_COO || p.nnz >= 64 * p.rows))
+        p.lpe_log2 = 3;  // (sparse graphs are bound by per-row latencies, not by the L2: one pass there)
     p.tile = static_cast<int64_t>(vec) << p.lpe_log2;
     p.out_vec = (reinterpret_cast<uintptr_t>(p.out) & 15) == 0 && (p.W & 3) == 0;
     p.ldf_shift = -1;
@@ -506,16 +583,38 @@ static int launch_spmm(SpmmParams p, int vec, hipStream_t s) {
     const dim3 grid(static_cast<unsigned>(gx), static_cast<unsigned>(ychunks));
     // A row much longer than one wavefront's share of the whole job would finish long after
     // everything else (hub rows of a small power-law graph): such rows get sixteen waves each.
-    p.long_row = (p.nnz >> 11) > 1024 ? (p.nnz >> 11) : 1024;
+    // The share is nnz / 8192 (8192 resident waves).  A single wave walks a row 4 * 64 / lpe slots
+    // at a time, and below ~16 such batches the sixteen-wave path is not worth its barriers.  On
+    // very large jobs the main launch runs for milliseconds and hides rows of a few shares (they
+    // sit at the front of the grid), while a separate launch for them would only add its own
+    // tail: there the threshold is four shares (measured on the 114.8 M-edge benchmark graph).
+    const int64_t by_batches = 16LL * 4 * (64 >> p.lpe_log2);
+    const int64_t share = p.nnz >= (64LL << 20) ? (p.nnz >> 11) : (p.nnz >> 13);
+    p.long_row = share > by_batches ? share : by_batches;
+    p.hub_row = 16 * p.long_row;
+    const int64_t longest = p.max_row > 0 ? p.max_row : p.nnz;  // no row has more slots than this
+    const bool hubs = longest > p.hub_row;
+    if (!hubs) p.hub_row = INT64_MAX;
     const dim3 lgrid(static_cast<unsigned>(p.rows < kLongGrid ? p.rows : kLongGrid), static_cast<unsigned>(ychunks));
-    if (p.nnz > p.long_row) {
-        if (vec == 16) hipLaunchKernelGGL((spmm_long_kernel<16, KIND>), lgrid, dim3(1024), 0, s, p);
-        else if (vec == 4) hipLaunchKernelGGL((spmm_long_kernel<4, KIND>), lgrid, dim3(1024), 0, s, p);
-        else hipLaunchKernelGGL((spmm_long_kernel<1, KIND>), lgrid, dim3(1024), 0, s, p);
+    const dim3 hgrid(static_cast<unsigned>(p.rows < kHubGrid ? p.rows : kHubGrid), lgrid.y, kHubChunks);
+    const dim3 sgrid(hgrid.x, lgrid.y);
+#define TANGO_SPMM_LONG(V)                                                                                  \
+    do {                                                                                                    \
+        hipLaunchKernelGGL((spmm_long_kernel<V, KIND, LONG>), lgrid, dim3(1024), 0, s, p);                  \
+        if (hubs) {                                                                                         \
+            hipLaunchKernelGGL((spmm_long_kernel<V, KIND, HUB_SUM>), hgrid, dim3(1024), 0, s, p);           \
+            hipLaunchKernelGGL((spmm_long_kernel<V, KIND, HUB_STORE>), sgrid, dim3(1024), 0, s, p);         \
+        }                                                                                                   \
+    } while (0)
+    if (longest > p.long_row) {
+        if (vec == 16) TANGO_SPMM_LONG(16);
+        else if (vec == 4) TANGO_SPMM_LONG(4);
+        else TANGO_SPMM_LONG(1);
     }
+#undef TANGO_SPMM_LONG
     // Sparse graph: lane groups own the short rows, single waves the rest up to long_row.
     if (KIND != KIND_COO && p.nnz < 64 * p.rows && p.lpe_log2 < 6) {
-        p.group_row = 32;
+        p.group_row = kGroupRow;
         const int64_t rows_per_block = 4LL << (6 - p.lpe_log2);
         const dim3 ggrid(static_cast<unsigned>(ceil_div(p.rows, rows_per_block)), static_cast<unsigned>(ychunks));
         const dim3 mgrid(static_cast<unsigned>(ceil_div(p.rows, 4 * kRowsPerWave)), static_cast<unsigned>(ychunks));
@@ -574,15 +673,16 @@ int tango_spmm_csr_copy_u(float* out, const int64_t* indptr, const int64_t* indi
 int tango_spmm_csr_copy_u_ex(float* out, const int64_t* indptr, const void* indices, int idx_bits,
                              const int8_t* feat, int64_t ldf, const float* scale,
                              const float* row_scale, const float* bias, int relu, int64_t rows,
-                             int64_t num_src, int64_t nnz, int64_t F, tango_stream_t stream) {
-    if (rows < 0 || F < 0 || nnz < 0 || num_src < 0 || ldf < F || !scale || !indptr ||
+                             int64_t num_src, int64_t nnz, int64_t F, int64_t max_row_nnz,
+                             tango_stream_t stream) {
+    if (rows < 0 || F < 0 || nnz < 0 || num_src < 0 || ldf < F || !scale || !indptr || max_row_nnz < 0 ||
         (rows * F > 0 && !out) || (nnz > 0 && (!indices || !feat)) || (idx_bits != 32 && idx_bits != 64))
         return TANGO_ERR_INVALID_ARG;
     if (num_src >= (1LL << 31) || nnz >= (1LL << 31)) return TANGO_ERR_UNSUPPORTED;
     SpmmParams p{};
     p.out = out; p.indptr = indptr; p.indices = static_cast<const int64_t*>(indices); p.idx32 = idx_bits == 32;
     p.feat = feat; p.scale = scale;
-    p.row_scale = row_scale; p.bias = bias; p.relu = relu ? 1 : 0;
+    p.row_scale = row_scale; p.bias = bias; p.relu = relu ? 1 : 0; p.max_row = max_row_nnz;
     p.rows = rows; p.num_src = num_src; p.ldf = ldf; p.W = F; p.F = F; p.D = 1; p.nnz = nnz;
     return launch_spmm<KIND_COPY>(p, pick_vec(feat, ldf, F), as_stream(stream));
 }
@@ -591,8 +691,8 @@ int tango_spmm_csr_u_mul_e_ex(float* out, const int64_t* indptr, const void* ind
                               const void* edge_ids, int idx_bits, const int8_t* feat, const int8_t* evals,
                               int edge_major, const float* scale, const float* bias, int64_t rows,
                               int64_t num_src, int64_t H, int64_t F, int64_t D, int64_t nnz,
-                              tango_stream_t stream) {
-    if (rows < 0 || H < 0 || F < 0 || nnz < 0 || num_src < 0 || !scale || !indptr ||
+                              int64_t max_row_nnz, tango_stream_t stream) {
+    if (rows < 0 || H < 0 || F < 0 || nnz < 0 || num_src < 0 || !scale || !indptr || max_row_nnz < 0 ||
         (rows * H * F > 0 && !out) || (nnz > 0 && (!indices || !feat || !evals)) ||
         (idx_bits != 32 && idx_bits != 64))
         return TANGO_ERR_INVALID_ARG;
@@ -601,6 +701,7 @@ int tango_spmm_csr_u_mul_e_ex(float* out, const int64_t* indptr, const void* ind
     SpmmParams p{};
     p.out = out; p.indptr = indptr; p.indices = static_cast<const int64_t*>(indices);
     p.edge_ids = static_cast<const int64_t*>(edge_ids); p.idx32 = idx_bits == 32; p.feat = feat;
+    p.max_row = max_row_nnz;
     p.evals = evals; p.scale = scale; p.bias = bias; p.rows = rows; p.num_src = num_src; p.ldf = H * F; p.W = H * F; p.F = F; p.D = D;
     p.nnz = nnz;
     if (edge_major) {  // evals[nnz, H, D]: the H * D bytes of one edge share a cache sector
@@ -623,7 +724,7 @@ int tango_spmm_csr_u_mul_e(float* out, const int64_t* indptr, const int64_t* ind
                            const float* scale, int64_t rows, int64_t num_src, int64_t H,
                            int64_t F, int64_t D, int64_t nnz, tango_stream_t stream) {
     return tango_spmm_csr_u_mul_e_ex(out, indptr, indices, edge_ids, 64, feat, evals, 0, scale, nullptr, rows, num_src,
-                                     H, F, D, nnz, stream);
+                                     H, F, D, nnz, 0, stream);
 }
 
 int tango_spmm_incidence(float* out, const int64_t* node_ids, const int64_t* edge_ids,

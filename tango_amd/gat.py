@@ -37,16 +37,20 @@ class attn_scores(Function):
 
 
 class QGATConv(nn.Module):
-    """evaluation/test_gat.py:24-169 for a homogeneous graph (feat is one tensor)."""
+    """evaluation/test_gat.py:24-169 for a homogeneous graph (feat is one tensor); same
+    constructor arguments in the same order."""
 
-    def __init__(self, in_feats, out_feats, num_heads, negative_slope=0.2, residual=False,
-                 activation=None, bias=True):
+    def __init__(self, in_feats, out_feats, num_heads, feat_drop=0., attn_drop=0., negative_slope=0.2,
+                 residual=False, activation=None, allow_zero_in_degree=False, bias=True):
         super().__init__()
         self._num_heads, self._out_feats = num_heads, out_feats
+        self._allow_zero_in_degree = allow_zero_in_degree
         self.fc = QLinear(in_feats, out_feats * num_heads, bias=False)
         self.fc.enable_reduce()  # the GEMM epilogue hands max|feat_src| / 127 to the aggregation
         self.attn_l = nn.Parameter(torch.empty(1, num_heads, out_feats))
         self.attn_r = nn.Parameter(torch.empty(1, num_heads, out_feats))
+        self.feat_drop = nn.Dropout(feat_drop)
+        self.attn_drop = nn.Dropout(attn_drop)
         self.negative_slope = negative_slope
         self.bias = nn.Parameter(torch.zeros(num_heads * out_feats)) if bias else None
         if residual:
@@ -63,13 +67,16 @@ class QGATConv(nn.Module):
             nn.init.xavier_normal_(self.res_fc.weight, gain=gain)
 
     def forward(self, graph, feat, get_attention=False):
+        if not self._allow_zero_in_degree and bool((graph.in_degrees() == 0).any()):
+            raise Exception("There are 0-in-degree nodes in the graph.")  # test_gat.py:93-96
         n = feat.size(0)
-        h = feat.contiguous()
+        h = self.feat_drop(feat).contiguous()
         feat_src, s_feat = self.fc(h)
         feat_src = feat_src.view(n, self._num_heads, self._out_feats)
         el, er = attn_scores.apply(feat_src, self.attn_l, self.attn_r)  # test_gat.py:135-137
         e = sddmm_u_add_v.apply(graph, el, er)                      # :141
         a = edge_softmax(graph, e, negative_slope=self.negative_slope)  # LeakyReLU :144 + softmax :146
+        a = self.attn_drop(a)
         # without a residual branch the bias add (:160-162) rides in the aggregation's epilogue
         fold_bias = self.bias is not None and self.res_fc is None
         rst = spmm_u_mul_e.apply(graph, feat_src, a, self.bias if fold_bias else None, s_feat)  # :151
@@ -82,8 +89,38 @@ class QGATConv(nn.Module):
         return (rst, a) if get_attention else rst
 
 
+class GAT(nn.Module):
+    """evaluation/test_gat.py:170-214: input projection, hidden layers on the concatenated
+    heads, output layer averaged over its heads."""
+
+    def __init__(self, g, num_layers, in_dim, num_hidden, num_classes, heads, activation, feat_drop=0.,
+                 attn_drop=0., negative_slope=0.2, residual=False):
+        super().__init__()
+        self.g, self.num_layers = g, num_layers
+        self.gat_layers = nn.ModuleList()
+        if num_layers > 1:
+            self.gat_layers.append(QGATConv(in_dim, num_hidden, heads[0], feat_drop, attn_drop, negative_slope,
+                                            False, activation))
+            for l in range(1, num_layers - 1):
+                self.gat_layers.append(QGATConv(num_hidden * heads[l - 1], num_hidden, heads[l], feat_drop,
+                                                attn_drop, negative_slope, residual, activation))
+            # as in the reference, the output layer keeps num_hidden columns (num_classes is unused there)
+            self.gat_layers.append(QGATConv(num_hidden * heads[-2], num_hidden, heads[-1], feat_drop, attn_drop,
+                                            negative_slope, residual, None))
+        else:
+            self.gat_layers.append(QGATConv(in_dim, num_hidden, heads[0], feat_drop, attn_drop, negative_slope,
+                                            residual, None))
+
+    def forward(self, inputs):
+        h = inputs
+        for l in range(self.num_layers - 1):
+            h = self.gat_layers[l](self.g, h).flatten(1)
+        return self.gat_layers[-1](self.g, h).mean(1)
+
+
 class HGTLayer(nn.Module):
-    """evaluation/test_HGT.py:21-67 (the reference's HGT has no per-type weights)."""
+    """evaluation/test_HGT.py:27-67, the class the reference calls HGT: one attention layer over a
+    homogenised graph (it has no per-type weights)."""
 
     def __init__(self, in_dim, out_dim, n_heads):
         super().__init__()
@@ -111,3 +148,22 @@ class HGTLayer(nn.Module):
         attn = edge_softmax(g, t)
         t = spmm_u_mul_e.apply(g, v, attn, None, s_v).reshape(-1, self.out_dim)
         return self.a_linear(t)
+
+
+HGT = HGTLayer  # the reference's name (evaluation/test_HGT.py:27)
+
+
+class HGTStack(nn.Module):
+    """Several HGT layers back to back with a linear read-out, the shape of the reference's
+    driver loop (evaluation/test_HGT.py:87-96: model, then ``proj_layer``)."""
+
+    def __init__(self, in_dim, hidden, n_classes, n_heads, n_layers=2):
+        super().__init__()
+        dims = [in_dim] + [hidden] * n_layers
+        self.layers = nn.ModuleList(HGTLayer(dims[i], dims[i + 1], n_heads) for i in range(n_layers))
+        self.proj = nn.Linear(hidden, n_classes)
+
+    def forward(self, g, h):
+        for layer in self.layers:
+            h = layer(g, h)
+        return self.proj(h)

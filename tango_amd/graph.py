@@ -158,3 +158,48 @@ def chung_lu(num_nodes, num_edges, gamma, seed, max_degree=None, symmetric=False
     if self_loops:
         src, dst = add_self_loop(src, dst, num_nodes)
     return Graph(src, dst, num_nodes)
+
+
+def hetero_power_law(type_sizes=(100_000, 50_000, 20_000),
+                     relations=((0, 1), (1, 0), (1, 2), (2, 0)), edges_per_relation=2_000_000,
+                     gamma=2.0, seed0=50, device="cpu"):
+    """Synthetic heterogeneous graph, homogenised the way the reference's HGT driver
+    consumes its graphs (one node id space, evaluation/test_cache_SPMM.py:98): node types
+    occupy consecutive id ranges, relation ``(a, b)`` contributes power-law edges from
+    type ``a`` nodes to type ``b`` nodes (seed ``seed0 + relation index``), and every
+    node gets a self loop.  Returns (Graph, node_type [n], edge_type [num_edges])
+    with self loops carrying edge type ``len(relations)``."""
+    offs = [0]
+    for n in type_sizes:
+        offs.append(offs[-1] + n)
+    srcs, dsts, ets = [], [], []
+    for r, (a, b) in enumerate(relations):
+        gen = torch.Generator(device=device)
+        gen.manual_seed(int(seed0 + r))
+        cdfs = []
+        for n in (type_sizes[a], type_sizes[b]):
+            w = (torch.arange(n, dtype=torch.float64, device=device) + 1.0).pow(-1.0 / (gamma - 1.0))
+            c = torch.cumsum(w / w.sum(), 0)
+            c[-1] = 1.0
+            cdfs.append(c)
+        keys = torch.empty(0, dtype=torch.int64, device=device)
+        need = edges_per_relation
+        for _ in range(12):  # top up what duplicate removal took away
+            u = torch.rand(2, max(int(need * 1.3), 65536), generator=gen, device=device, dtype=torch.float64)
+            s = torch.searchsorted(cdfs[0], u[0]).clamp_(max=type_sizes[a] - 1)
+            d = torch.searchsorted(cdfs[1], u[1]).clamp_(max=type_sizes[b] - 1)
+            keys = torch.unique(torch.cat([keys, s * type_sizes[b] + d]))
+            need = edges_per_relation - keys.numel()
+            if need <= 0:
+                break
+        if keys.numel() > edges_per_relation:
+            perm = torch.randperm(keys.numel(), generator=gen, device=device)[:edges_per_relation]
+            keys = keys[perm.sort().values]
+        srcs.append(keys // type_sizes[b] + offs[a])
+        dsts.append(keys % type_sizes[b] + offs[b])
+        ets.append(torch.full((keys.numel(),), r, dtype=torch.int64, device=device))
+    n = offs[-1]
+    src, dst = add_self_loop(torch.cat(srcs), torch.cat(dsts), n)
+    ets.append(torch.full((n,), len(relations), dtype=torch.int64, device=device))
+    node_type = torch.cat([torch.full((m,), t, dtype=torch.int64, device=device) for t, m in enumerate(type_sizes)])
+    return Graph(src, dst, n), node_type, torch.cat(ets)

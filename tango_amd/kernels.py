@@ -322,7 +322,8 @@ class cuda_kernels:
 
     # ------------------------------------------------------------------ SpMM
     @staticmethod
-    def csr_SPMM(out, indptr, indices, U, scaleU, ldf=None, F=None, row_scale=None, bias=None, relu=False):
+    def csr_SPMM(out, indptr, indices, U, scaleU, ldf=None, F=None, row_scale=None, bias=None, relu=False,
+                 max_row=0):
         _need(out, torch.float32, "out")
         _need(indptr, torch.int64, "indptr")
         idx_bits = _need_index(indices, "indices")
@@ -334,7 +335,7 @@ class cuda_kernels:
         F = width if F is None else F
         if out.numel() != rows * F:
             raise RuntimeError("csr_SPMM: out must be [%d, %d]" % (rows, F))
-        if row_scale is None and bias is None and not relu and idx_bits == 64:
+        if row_scale is None and bias is None and not relu and idx_bits == 64 and not max_row:
             check(_L.tango_spmm_csr_copy_u(_ptr(out), indptr.data_ptr(), _ptr(indices), _ptr(U), ldf,
                                            scaleU.data_ptr(), rows, U.size(0), indices.numel(), F,
                                            _stream()), "csr_SPMM")
@@ -349,14 +350,15 @@ class cuda_kernels:
                 raise RuntimeError("csr_SPMM: bias must have F entries")
         check(_L.tango_spmm_csr_copy_u_ex(_ptr(out), indptr.data_ptr(), _ptr(indices), idx_bits, _ptr(U), ldf,
                                           scaleU.data_ptr(), _ptr(row_scale), _ptr(bias), int(bool(relu)),
-                                          rows, U.size(0), indices.numel(), F, _stream()), "csr_SPMM")
+                                          rows, U.size(0), indices.numel(), F, int(max_row), _stream()), "csr_SPMM")
 
     @staticmethod
-    def multi_cusparse_SPMM(indptr, indices, N, E_T, scale, edge_ids=None, edge_major=False, bias=None):
+    def multi_cusparse_SPMM(indptr, indices, N, E_T, scale, edge_ids=None, edge_major=False, bias=None, max_row=0):
         """E_T is [H, D, nnz] in CSR slot order, or in edge-id order when the
         slot->edge permutation ``edge_ids`` is passed (gather fused in-kernel).
         With ``edge_major`` the edge values are [nnz, H, D] instead (no transpose pass).
-        ``bias`` ([H * F] fp32) is added to every output row after dequantization."""
+        ``bias`` ([H * F] fp32) is added to every output row after dequantization.  ``max_row``: an
+        upper bound of the longest row if known (0 = unknown)."""
         _need(indptr, torch.int64, "indptr")
         idx_bits = _need_index(indices, "indices")
         _need(N, torch.int8, "N")
@@ -383,7 +385,8 @@ class cuda_kernels:
         out = torch.empty((rows, H, F), dtype=torch.float32, device=N.device)
         check(_L.tango_spmm_csr_u_mul_e_ex(_ptr(out), indptr.data_ptr(), _ptr(indices), _ptr(edge_ids), idx_bits,
                                            _ptr(N), _ptr(E_T), int(bool(edge_major)), scale.data_ptr(),
-                                           _ptr(bias), rows, k, H, F, D, nnz, _stream()), "multi_cusparse_SPMM")
+                                           _ptr(bias), rows, k, H, F, D, nnz, int(max_row), _stream()),
+              "multi_cusparse_SPMM")
         return out
 
     # The reference's SpMV binding returns uninitialised memory (cuda/src/SPMM.cu:196-257)
@@ -608,13 +611,14 @@ def transpose_quant(data, scale):
 
 
 def _csr_of(g, reverse):
-    """(indptr, indices, edge_ids) of the source-major (reverse) or destination-major CSR, with the
-    32-bit copies of indices / edge_ids when graph_preprocess made them."""
+    """(indptr, indices, edge_ids, longest row) of the source-major (reverse) or destination-major
+    CSR, with the 32-bit copies of indices / edge_ids and the row-length bound when
+    graph_preprocess made them (0 = unknown)."""
     indptr, indices, edge_ids = g.adj_csr if reverse else g.adj_csc
     narrow = getattr(g, "adj_csr32" if reverse else "adj_csc32", None)
     if narrow is not None:
         indices, edge_ids = narrow
-    return indptr, indices, edge_ids
+    return indptr, indices, edge_ids, getattr(g, "max_out_degree" if reverse else "max_in_degree", 0)
 
 
 def multi_cusparse_SPMM(g, N, E_T, scale, reverse=False, edge_major=False, bias=None):
@@ -623,11 +627,11 @@ def multi_cusparse_SPMM(g, N, E_T, scale, reverse=False, edge_major=False, bias=
     ``edge_major``: E_T is the quantized edge tensor as it is, [nnz, H, 1]."""
     assert E_T.ndim == 3 and N.ndim == 3, "E and N must be 3D tensors"
     assert E_T.size(2 if edge_major else 1) == 1, "Cannot broadcast E"
-    indptr, indices, edge_ids = _csr_of(g, reverse)
+    indptr, indices, edge_ids, longest = _csr_of(g, reverse)
     if edge_ids is not None and edge_ids.numel() == 0:
         edge_ids = None
     return cuda_kernels.multi_cusparse_SPMM(indptr, indices, N, E_T, scale, edge_ids=edge_ids,
-                                            edge_major=edge_major, bias=bias)
+                                            edge_major=edge_major, bias=bias, max_row=longest)
 
 
 def incidence_SPMM(g, E, scaleE, reverse=False):
@@ -635,18 +639,18 @@ def incidence_SPMM(g, E, scaleE, reverse=False):
     adjacency (the equivalence evaluation/test_incidence.py:14-22 relies on), which the graph
     already holds, so the row bounds come from indptr instead of a search in the COO node ids."""
     assert E.is_cuda and scaleE.is_cuda
-    indptr, _, edge_ids = _csr_of(g, reverse)
+    indptr, _, edge_ids, longest = _csr_of(g, reverse)
     out_shape = (g.num_nodes(),) + E.shape[1:]
     dim = math.prod(E.shape[1:])
     out = torch.empty((g.num_nodes(), dim), dtype=torch.float32, device=E.device)
-    cuda_kernels.csr_SPMM(out, indptr, edge_ids, E.reshape(E.size(0), dim), scaleE)
+    cuda_kernels.csr_SPMM(out, indptr, edge_ids, E.reshape(E.size(0), dim), scaleE, max_row=longest)
     return out.view(out_shape)
 
 
 def csr_SPMM(g, N, scaleN, reverse=False, row_scale=None, bias=None, relu=False):
     """cuda/kernels.py:154-165.  N may be a 2-D view of a row-padded buffer.  ``row_scale`` / ``bias`` /
     ``relu`` fold "* norm, + bias, activation" (evaluation/test_gcn.py:123-137) into the kernel's epilogue."""
-    indptr, indices, _ = _csr_of(g, reverse)
+    indptr, indices, _, longest = _csr_of(g, reverse)
     feat_shape = N.shape[1:]
     out_shape = (g.num_nodes(),) + feat_shape
     dim = math.prod(N.shape[1:])
@@ -655,9 +659,10 @@ def csr_SPMM(g, N, scaleN, reverse=False, row_scale=None, bias=None, relu=False)
         ld = _rows_view(N, "N")
         base = N.as_strided((N.size(0), ld), (ld, 1))
         cuda_kernels.csr_SPMM(out, indptr, indices, base, scaleN, ldf=ld, F=dim, row_scale=row_scale, bias=bias,
-                              relu=relu)
+                              relu=relu, max_row=longest)
     else:
-        cuda_kernels.csr_SPMM(out, indptr, indices, N, scaleN, row_scale=row_scale, bias=bias, relu=relu)
+        cuda_kernels.csr_SPMM(out, indptr, indices, N, scaleN, row_scale=row_scale, bias=bias, relu=relu,
+                              max_row=longest)
     return out.view(out_shape)
 
 

@@ -23,4 +23,8 @@ def graph_preprocess(graph):
     # and at 4 bytes per edge they cost half the traffic of the int64 arrays the reference passes.
     graph.adj_csr32 = tuple(t.to(torch.int32) for t in graph.adj_csr[1:])
     graph.adj_csc32 = tuple(t.to(torch.int32) for t in graph.adj_csc[1:])
+    # the longest row of either orientation (one host read per graph): tells the aggregation
+    # kernels whether the launches that exist for hub rows are needed at all
+    graph.max_out_degree = int(torch.diff(graph.adj_csr[0]).max().item()) if graph.adj_csr[0].numel() > 1 else 0
+    graph.max_in_degree = int(torch.diff(graph.adj_csc[0]).max().item()) if graph.adj_csc[0].numel() > 1 else 0
     return graph
