@@ -12,8 +12,9 @@
 //   * TN kernel (gradW): both operands are tall and reduction-strided.  Tiles
 //     are staged through LDS in their natural layout and transposed in
 //     registers (v_perm 4x4 byte blocks) on the way into the fragments; the
-//     reduction over rows is split across workgroups and combined with int32
-//     atomics, which is exact and order-independent.
+//     reduction over rows is split across workgroups, each writing an int32
+//     slab of its own; a second kernel adds the slabs (exact, independent of
+//     the split) and dequantizes.
 #include "common.hpp"
 
 namespace tango {

@@ -3,16 +3,19 @@
 //
 // These are gather kernels bound by the memory system, not by arithmetic, so
 // no MFMA is used.  Layout of the work:
-//   * a wavefront (or a 4-wave workgroup for long, wide rows) owns one
-//     output row and walks that row's CSR slots;
+//   * a wavefront owns one output row and walks that row's CSR slots (4 waves for
+//     long rows of wide pieces, 16 waves for rows far above the average, several
+//     workgroups for hub rows, a lane group per row on sparse graphs: see the
+//     kernels below);
 //   * column indices are fetched 256 slots at a time with four independent
 //     coalesced 512-byte loads (lane i of load r holds slot 64 r + i) and handed
 //     to the lanes that need them with ds_bpermute, so index traffic is read
 //     exactly once and one HBM round trip is paid per 256 edges;
 //   * a group of `lpe` lanes (power of two) covers one gathered int8 feature
 //     row with 16-, 4- or 1-byte loads per lane, so one load instruction of
-//     the wavefront pulls 64/lpe neighbour rows (F = 256 -> 4 rows of 256 B,
-//     F = 16 -> 64 rows);
+//     the wavefront pulls 64/lpe neighbour rows (128-byte pieces -> 8 rows,
+//     F = 16 -> 64 rows); a matrix far beyond the L2 is walked in 128-byte column
+//     tiles, one tile after the other;
 //   * a lane always has four gathers (four neighbours, same columns) in flight;
 //     their dwords are byte-transposed with v_perm and added into int32 lane
 //     accumulators four neighbours at a time with one v_dot4 against a byte
@@ -57,9 +60,6 @@ struct SpmmParams {
 };
 
 enum { KIND_COPY = 0, KIND_WEIGHTED = 1, KIND_COO = 2 };
-
-struct SpmmParams;
-__device__ __forceinline__ int64_t row_offset(int j, const SpmmParams& p);
 
 // Byte offset of gathered row j: a shift when the row pitch allows (64-bit multiplies are quarter rate).
 __device__ __forceinline__ int64_t row_offset(int j, const SpmmParams& p) {
