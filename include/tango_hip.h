@@ -53,6 +53,12 @@ int tango_abi_version(void);
    initialised.  Unlike the reference every element is covered when n % 4 != 0. */
 int tango_absmax_f32(const float* x, int64_t n, float* scale_out, tango_stream_t stream);
 
+/* Accumulating form (no counterpart in the reference): scale_acc[0] = max(scale_acc[0],
+   max|x| / 127).  scale_acc must hold 0 or an earlier partial result (any non-negative
+   float).  A caller that hands out zero-initialised slots saves the fill launch that
+   tango_absmax_f32 spends on its output; several tensors may share one scale. */
+int tango_absmax_acc_f32(const float* x, int64_t n, float* scale_acc, tango_stream_t stream);
+
 /* Per-row scales (no counterpart in the reference): scale_out[r] = max_c |x[r,c]| / 127. */
 int tango_absmax_rows_f32(const float* x, int64_t rows, int64_t cols, int64_t ldx,
                           float* scale_out, tango_stream_t stream);
@@ -83,11 +89,13 @@ int tango_quantize_rows_f32_i8(const float* x, int64_t rows, int64_t cols, int64
    tango_absmax_ex_f32 writes scale_out[0] = max|x*row_mul| / 127 over unmasked
    elements and, when colsum_out is non-null, colsum_out[c] = sum_r of the
    unmasked x[r, c] (not multiplied), reduced in a fixed order.  cols <= 1024.
+   accumulate != 0: scale_out[0] already holds 0 or a partial result and is maxed into
+   (as tango_absmax_acc_f32); otherwise it need not be initialised.
    workspace: tango_absmax_ex_workspace(rows, cols, colsum_out != NULL) bytes. */
 size_t tango_absmax_ex_workspace(int64_t rows, int64_t cols, int want_colsum);
 int tango_absmax_ex_f32(const float* x, int64_t rows, int64_t cols, int64_t ldx, const float* row_mul,
-                        const float* mask, int64_t ldm, float* scale_out, float* colsum_out,
-                        void* workspace, size_t workspace_bytes, tango_stream_t stream);
+                        const float* mask, int64_t ldm, float* scale_out, int accumulate,
+                        float* colsum_out, void* workspace, size_t workspace_bytes, tango_stream_t stream);
 int tango_quantize_rows_ex_f32_i8(const float* x, int64_t rows, int64_t cols, int64_t ldx,
                                   const float* row_mul, const float* mask, int64_t ldm,
                                   const float* scale, int per_row, int8_t* q, int64_t ldq,

@@ -462,6 +462,17 @@ int tango_absmax_f32(const float* x, int64_t n, float* scale_out, tango_stream_t
     return launch_status();
 }
 
+int tango_absmax_acc_f32(const float* x, int64_t n, float* scale_acc, tango_stream_t stream) {
+    if (!scale_acc || n < 0 || (n > 0 && !x)) return TANGO_ERR_INVALID_ARG;
+    if ((reinterpret_cast<uintptr_t>(x) & 3) != 0) return TANGO_ERR_INVALID_ARG;
+    if (n == 0) return TANGO_OK;
+    int64_t head = ((16 - (reinterpret_cast<uintptr_t>(x) & 15)) & 15) >> 2;
+    if (head > n) head = n;
+    const int grid = grid_for(n / 16 + 1, 256);
+    hipLaunchKernelGGL(absmax_kernel, dim3(grid), dim3(256), 0, as_stream(stream), x, n, head, scale_acc);
+    return launch_status();
+}
+
 int tango_absmax_rows_f32(const float* x, int64_t rows, int64_t cols, int64_t ldx,
                           float* scale_out, tango_stream_t stream) {
     if (rows < 0 || cols < 0 || ldx < cols || (rows > 0 && (!x || !scale_out)))
@@ -485,13 +496,13 @@ size_t tango_absmax_ex_workspace(int64_t rows, int64_t cols, int want_colsum) {
 }
 
 int tango_absmax_ex_f32(const float* x, int64_t rows, int64_t cols, int64_t ldx, const float* row_mul,
-                        const float* mask, int64_t ldm, float* scale_out, float* colsum_out,
-                        void* workspace, size_t workspace_bytes, tango_stream_t stream) {
+                        const float* mask, int64_t ldm, float* scale_out, int accumulate,
+                        float* colsum_out, void* workspace, size_t workspace_bytes, tango_stream_t stream) {
     if (rows < 0 || cols < 0 || ldx < cols || !scale_out || (rows * cols > 0 && !x) || (mask && ldm < cols))
         return TANGO_ERR_INVALID_ARG;
     if (cols > 1024) return TANGO_ERR_UNSUPPORTED;
     hipStream_t s = as_stream(stream);
-    fill_u32(scale_out, 0u, 1, s);
+    if (!accumulate) fill_u32(scale_out, 0u, 1, s);
     const int grid = absmax_ex_grid(rows);
     float* partial = nullptr;
     if (colsum_out) {

@@ -64,6 +64,26 @@ def _workspace(nbytes, device):
     return torch.empty(nbytes, dtype=torch.uint8, device=device) if nbytes else None
 
 
+_ZERO_SLOTS = {}   # device -> [pool tensor, next free index]
+_POOL_SIZE = 4096
+
+
+def _zero_slot(device):
+    """A 1-element fp32 tensor that holds 0: a view into a pool that one fill zeroes 4096 slots at a
+    time, so that the absmax kernels (which max into their output with an atomic) need no fill launch
+    of their own per call.  A slot is handed out once and never reused.  Returns None while the
+    current stream is being captured into a graph: a replay would find the slot already used."""
+    if torch.cuda.is_current_stream_capturing():
+        return None
+    key = (device.type, device.index)
+    pool = _ZERO_SLOTS.get(key)
+    if pool is None or pool[1] >= _POOL_SIZE:
+        pool = _ZERO_SLOTS[key] = [torch.zeros(_POOL_SIZE, dtype=torch.float32, device=device), 0]
+    slot = pool[0][pool[1]:pool[1] + 1]
+    pool[1] += 1
+    return slot
+
+
 def _mode(round_mode):
     if isinstance(round_mode, str):
         return ROUND_MODES[round_mode]
@@ -102,6 +122,10 @@ class cuda_kernels:
     @staticmethod
     def get_scale(inp):
         _need(inp, torch.float32, "in")
+        scale = _zero_slot(inp.device) if inp.numel() > (1 << 16) else None  # small tensors: one launch anyway
+        if scale is not None:
+            check(_L.tango_absmax_acc_f32(_ptr(inp), inp.numel(), scale.data_ptr(), _stream()), "get_scale")
+            return scale
         scale = torch.empty(1, dtype=torch.float32, device=inp.device)
         check(_L.tango_absmax_f32(_ptr(inp), inp.numel(), scale.data_ptr(), _stream()), "get_scale")
         return scale
@@ -186,13 +210,16 @@ class cuda_kernels:
                 scale = s_i if scale is None else torch.maximum(scale, s_i)
                 sums.append(cs_i)
             return scale, (torch.cat(sums) if want_colsum else None)
-        scale = torch.empty(1, dtype=torch.float32, device=inp.device)
+        scale = _zero_slot(inp.device)
+        accumulate = scale is not None
+        if not accumulate:
+            scale = torch.empty(1, dtype=torch.float32, device=inp.device)
         colsum = torch.empty(cols, dtype=torch.float32, device=inp.device) if want_colsum else None
         ws_bytes = _L.tango_absmax_ex_workspace(rows, cols, int(want_colsum))
         ws = _workspace(ws_bytes, inp.device)
         check(_L.tango_absmax_ex_f32(_ptr(inp), rows, cols, ldx, _ptr(row_mul), _ptr(mask), ldm,
-                                     scale.data_ptr(), _ptr(colsum), _ptr(ws), ws_bytes, _stream()),
-              "absmax_ex")
+                                     scale.data_ptr(), int(accumulate), _ptr(colsum), _ptr(ws), ws_bytes,
+                                     _stream()), "absmax_ex")
         return scale, colsum
 
     @staticmethod

@@ -113,3 +113,24 @@ def test_transpose_quant(K, orc, shape):
     got = K.transpose_quant(dev(e), sc(s))
     assert tuple(got.shape) == (shape[1], shape[2], shape[0])
     assert np.array_equal(host(got).reshape(shape[1] * shape[2], shape[0]), orc.transpose_quant(e, s))
+
+
+def test_absmax_accumulating_form(K, orc):
+    """tango_absmax_acc_f32 maxes into a slot that holds 0 or a partial result; the Python layer hands it
+    pre-zeroed pool slots, which must never be handed out twice."""
+    from tango_amd._lib import lib, check
+    L = lib()
+    rng = np.random.default_rng(11)
+    a = rng.standard_normal(300001).astype(np.float32)
+    b = (rng.standard_normal(77) * 9).astype(np.float32)
+    slot = torch.zeros(1, device="cuda")
+    st = torch.cuda.current_stream().cuda_stream
+    for t in (dev(a), dev(b), dev(a[:3])):
+        check(L.tango_absmax_acc_f32(t.data_ptr(), t.numel(), slot.data_ptr(), st), "acc")
+    assert host(slot)[0] == max(orc.absmax_scale(a), orc.absmax_scale(b))
+    x = dev(a)
+    s1, s2 = K.cuda_kernels.get_scale(x), K.cuda_kernels.get_scale(x * 2)
+    assert s1.data_ptr() != s2.data_ptr()
+    assert host(s1)[0] == orc.absmax_scale(a) and host(s2)[0] == orc.absmax_scale(a * 2)
+    s3, _ = K.cuda_kernels.absmax_ex(x.view(-1, 1)[:300000].view(3000, 100))
+    assert host(s3)[0] == orc.absmax_scale(a[:300000])
