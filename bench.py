@@ -391,7 +391,7 @@ def main():
         "metric": "quant GCN epoch ms @233K nodes/114.6M edges; SpMM/SDDMM GB/s; QLinear TOPS",
         "value": round(ms_per_step, 3), "unit": "ms/epoch", "n_gpus": 1, "steps": args.steps,
         "warmup": args.warmup, "ms_per_step": round(ms_per_step, 3), "higher_is_better": False,
-        "scaling": "weak", "vs_baseline": None, "dtype": "int8 x int8 -> int32 (fp32 dequant)",
+        "scaling": "weak", "vs_baseline": None, "dtype": "int8",
         "data": "synthetic",
         "config": {"workload": "2-layer quantized GCN 602->256->41 training epoch (fwd+loss+bwd+Adam), "
                                "Chung-Lu graph gamma=2.0 seed=3 symmetric + self loops",

@@ -10,6 +10,7 @@ reference does not have (``round_mode``, ``noise``, ``seed``, ``offset``,
 """
 import math
 import os
+import threading
 
 import torch
 
@@ -65,6 +66,7 @@ def _workspace(nbytes, device):
 
 
 _ZERO_SLOTS = {}   # device -> [pool tensor, next free index]
+_ZERO_SLOTS_LOCK = threading.Lock()  # forward and autograd's backward thread both draw slots
 _POOL_SIZE = 4096
 
 
@@ -76,12 +78,13 @@ def _zero_slot(device):
     if torch.cuda.is_current_stream_capturing():
         return None
     key = (device.type, device.index)
-    pool = _ZERO_SLOTS.get(key)
-    if pool is None or pool[1] >= _POOL_SIZE:
-        pool = _ZERO_SLOTS[key] = [torch.zeros(_POOL_SIZE, dtype=torch.float32, device=device), 0]
-    slot = pool[0][pool[1]:pool[1] + 1]
-    pool[1] += 1
-    return slot
+    with _ZERO_SLOTS_LOCK:
+        pool = _ZERO_SLOTS.get(key)
+        if pool is None or pool[1] >= _POOL_SIZE:
+            pool = _ZERO_SLOTS[key] = [torch.zeros(_POOL_SIZE, dtype=torch.float32, device=device), 0]
+        k = pool[1]
+        pool[1] = k + 1
+    return pool[0][k:k + 1]
 
 
 def _mode(round_mode):
