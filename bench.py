@@ -21,7 +21,7 @@ HBM_PEAK_GBPS = 8000.0
 # Bytes that cross the L2 <-> fabric boundary per launch of the F=256 copy_u kernel on the default
 # benchmark graph: two rocprofv3 --pmc passes (FETCH_SIZE, then WRITE_SIZE, KiB per dispatch), each
 # scaled by what the same counter reads for a 1 GiB device copy (2.000 and 1.000).
-MEASURED_TRAFFIC_SPMM_F256 = 1.405e10
+MEASURED_TRAFFIC_SPMM_F256 = 1.318e10
 
 
 def parse():
