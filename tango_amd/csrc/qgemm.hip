@@ -385,6 +385,183 @@ __global__ __launch_bounds__(256, 2) void gemm_fq_kernel(const FqParams p) {
     if (p.absmax_out) block_absmax_to_global(m / 127.0f, p.absmax_out);
 }
 
+// W-stationary forward for tall X and narrow outputs (N <= 32): one persistent 12-wave workgroup per
+// CU keeps the whole packed W in LDS; the 16-row blocks of X are dealt round-robin over the waves of
+// the launch and a wave owns ALL N columns of its block.  A lane loads floats of X that belong to
+// its row's MFMA A-fragment, quantizes them in registers, the four lanes of a row exchange dwords,
+// the 16 bytes go to Xq (the backward cache) and straight into the MFMAs: X never passes through
+// LDS, there is no barrier after the W load, and the HBM reads run three k-steps ahead, so loads,
+// MFMAs and the Y stores of different waves overlap.  NT = 16-column tiles (N <= 16 NT).
+// (For wide outputs the accumulators of all N columns leave too few registers for the prefetch
+// and gemm_fq_kernel's LDS-staged form is faster: 0.30 ms against 0.49 ms at 232,965 x 602 x 256.)
+template <int NT, int XV, int MODE>
+__global__ __launch_bounds__(768) void gemm_ws_kernel(const FqParams p, int nblocks, int pitch, int kq) {
+    extern __shared__ __attribute__((aligned(16))) int8_t w_lds[];  // [16 NT][pitch]
+    constexpr int RT = 1;
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int g = lane >> 4, r16 = lane & 15;
+
+    // ---- W -> LDS, rows beyond N and chunks beyond kq zero-filled
+    {
+        const int cpr = pitch >> 4;  // 16-byte chunks per LDS row
+        for (int idx = tid; idx < 16 * NT * cpr; idx += 768) {
+            const int n = idx / cpr, c = idx - n * cpr;
+            i32x4 v{0, 0, 0, 0};
+            if (n < p.N && c * 16 < kq) v = *reinterpret_cast<const i32x4*>(p.B + static_cast<int64_t>(n) * p.ldb + c * 16);
+            *reinterpret_cast<i32x4*>(w_lds + n * pitch + c * 16) = v;
+        }
+    }
+    __syncthreads();
+
+    const float rs = rscale_of(p.sA[0]);
+    const float s = p.sA[0] * p.sB[0];
+    const int ksteps = (static_cast<int>(p.K) + 63) >> 6;
+    const uintptr_t ca = reinterpret_cast<uintptr_t>(p.C);
+    const int wide = ((ca & 15) == 0 && (p.ldc & 3) == 0) ? 4 : ((ca & 7) == 0 && (p.ldc & 1) == 0) ? 2 : 1;
+    float m = 0.0f;
+
+    // raw[i][4 w + c] = X[row0 + 16 i + r16][64 step + 16 w + 4 g + c]: in load w the four lanes of a row
+    // (g = 0..3) read 64 contiguous bytes, so a wave-wide load covers 16 rows x 64 B instead of 64
+    // scattered 16-byte pieces; the lanes of a row exchange dwords after quantization (below).
+    auto load_raw = [&](float (*raw)[16], int64_t row0, int step) {
+        const int64_t kbase = static_cast<int64_t>(step) * 64 + g * 4;
+#pragma unroll
+        for (int i = 0; i < RT; ++i) {
+            const int64_t row = row0 + 16 * i + r16;
+            const float* xr = p.X + row * p.ldx + kbase;
+            if (row < p.M && static_cast<int64_t>(step) * 64 + 64 <= p.K) {
+#pragma unroll
+                for (int w = 0; w < 4; ++w) {
+                    if (XV == 4) {
+                        const f32x4 v = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(xr + 16 * w));
+                        raw[i][4 * w] = v.x; raw[i][4 * w + 1] = v.y; raw[i][4 * w + 2] = v.z; raw[i][4 * w + 3] = v.w;
+                    } else {
+                        typedef float f32x2 __attribute__((ext_vector_type(2)));
+                        const f32x2 v0 = __builtin_nontemporal_load(reinterpret_cast<const f32x2*>(xr + 16 * w));
+                        const f32x2 v1 = __builtin_nontemporal_load(reinterpret_cast<const f32x2*>(xr + 16 * w + 2));
+                        raw[i][4 * w] = v0.x; raw[i][4 * w + 1] = v0.y; raw[i][4 * w + 2] = v1.x; raw[i][4 * w + 3] = v1.y;
+                    }
+                }
+            } else {  // the last, partial k-step and rows past M
+#pragma unroll
+                for (int w = 0; w < 4; ++w)
+#pragma unroll
+                    for (int c = 0; c < 4; ++c)
+                        raw[i][4 * w + c] = (row < p.M && kbase + 16 * w + c < p.K) ? xr[16 * w + c] : 0.0f;
+            }
+        }
+    };
+    // quantize raw into the A fragments of this step, store them to Xq, run the step's MFMAs
+    auto step_mma = [&](float (*raw)[16], int64_t row0, int step, i32x4 (*acc)[NT]) {
+        const int64_t k0 = static_cast<int64_t>(step) * 64 + g * 16;
+        const bool chunk_ok = k0 < kq;
+        i32x4 a[RT];
+#pragma unroll
+        for (int i = 0; i < RT; ++i) {
+            const int64_t row = row0 + 16 * i + r16;
+            const float rm = (p.x_row_mul && row < p.M) ? p.x_row_mul[row] : 1.0f;
+            uint32_t q[4];  // q[w]: the bytes of columns 64 step + 16 w + 4 g .. + 3
+#pragma unroll
+            for (int w = 0; w < 4; ++w) {
+                float x0 = raw[i][4 * w], x1 = raw[i][4 * w + 1], x2 = raw[i][4 * w + 2], x3 = raw[i][4 * w + 3];
+                if (p.x_row_mul) { x0 = x0 * rm; x1 = x1 * rm; x2 = x2 * rm; x3 = x3 * rm; }
+                q[w] = pack4(quant_one<MODE>(x0, rs, 0.f), quant_one<MODE>(x1, rs, 0.f),
+                             quant_one<MODE>(x2, rs, 0.f), quant_one<MODE>(x3, rs, 0.f));
+            }
+            // 4 x 4 dword transpose over the four lanes of the row (lanes r16 + 16 g): afterwards this lane holds
+            // columns 64 step + 16 g .. + 15 in order, i.e. its MFMA fragment.  Round k: lane g pulls from lane
+            // (g + k) & 3 the dword that lane holds for w = g, which is that lane's register (its g - k) & 3.
+            uint32_t f[4] = {0u, 0u, 0u, 0u};
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+                const int give = (g - k) & 3;
+                const uint32_t present = give == 0 ? q[0] : give == 1 ? q[1] : give == 2 ? q[2] : q[3];
+                const int from = (g + k) & 3;
+                const uint32_t got = static_cast<uint32_t>(__shfl(static_cast<int>(present), from * 16 + r16, kWave));
+#pragma unroll
+                for (int d = 0; d < 4; ++d)
+                    if (from == d) f[d] = got;
+            }
+            a[i] = i32x4{static_cast<int>(f[0]), static_cast<int>(f[1]), static_cast<int>(f[2]), static_cast<int>(f[3])};
+            if (chunk_ok && row < p.M)
+                __builtin_nontemporal_store(a[i], reinterpret_cast<i32x4*>(p.Xq + row * p.ldxq + k0));
+        }
+        const int kb = chunk_ok ? static_cast<int>(k0) : 0;  // a is all zero for chunks past kq: any in-range B will do
+#pragma unroll
+        for (int j = 0; j < NT; ++j) {
+            const i32x4 b = *reinterpret_cast<const i32x4*>(w_lds + (16 * j + r16) * pitch + kb);
+#pragma unroll
+            for (int i = 0; i < RT; ++i) acc[i][j] = mfma_16x16x64(b, a[i], acc[i][j]);
+        }
+    };
+
+    // blocks are dealt round-robin over all waves of the launch (a shared ticket counter serialises:
+    // one device-scope atomic per block on a single address, ~15 ns each, costs more than the block)
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int waves = static_cast<int>(gridDim.x) * (static_cast<int>(blockDim.x) >> 6);
+    for (int t = static_cast<int>(blockIdx.x) * (static_cast<int>(blockDim.x) >> 6) + wave; t < nblocks; t += waves) {
+        const int64_t row0 = static_cast<int64_t>(t) * (16 * RT);
+        i32x4 acc[RT][NT];
+#pragma unroll
+        for (int i = 0; i < RT; ++i)
+#pragma unroll
+            for (int j = 0; j < NT; ++j) acc[i][j] = i32x4{0, 0, 0, 0};
+        // the X loads run three k-steps ahead of the MFMAs that consume them
+        float r0[RT][16], r1[RT][16], r2[RT][16], r3[RT][16];
+        load_raw(r0, row0, 0);
+        if (1 < ksteps) load_raw(r1, row0, 1);
+        if (2 < ksteps) load_raw(r2, row0, 2);
+        for (int step = 0; step < ksteps; step += 4) {
+            if (step + 3 < ksteps) load_raw(r3, row0, step + 3);
+            step_mma(r0, row0, step, acc);
+            if (step + 1 < ksteps) {
+                if (step + 4 < ksteps) load_raw(r0, row0, step + 4);
+                step_mma(r1, row0, step + 1, acc);
+            }
+            if (step + 2 < ksteps) {
+                if (step + 5 < ksteps) load_raw(r1, row0, step + 5);
+                step_mma(r2, row0, step + 2, acc);
+            }
+            if (step + 3 < ksteps) {
+                if (step + 6 < ksteps) load_raw(r2, row0, step + 6);
+                step_mma(r3, row0, step + 3, acc);
+            }
+        }
+        // lane holds C[row0 + 16 i + r16][16 j + 4 g + v]
+#pragma unroll
+        for (int i = 0; i < RT; ++i) {
+            const int64_t row = row0 + i * 16 + r16;
+            if (row < p.M) {
+                float* crow = p.C + row * p.ldc;
+#pragma unroll
+                for (int j = 0; j < NT; ++j) {
+                    const int64_t col = j * 16 + g * 4;
+                    float y[4];
+#pragma unroll
+                    for (int v = 0; v < 4; ++v) {
+                        y[v] = s * static_cast<float>(acc[i][j][v]);
+                        if (p.bias && col + v < p.N) y[v] = p.bias[col + v] + y[v];
+                        if (col + v < p.N) m = fmaxf(m, fabsf(y[v]));
+                    }
+                    if (col + 4 <= p.N && wide == 4) {
+                        __builtin_nontemporal_store(f32x4{y[0], y[1], y[2], y[3]}, reinterpret_cast<f32x4*>(crow + col));
+                    } else if (col + 4 <= p.N && wide == 2) {
+                        typedef float f32x2 __attribute__((ext_vector_type(2)));
+                        *reinterpret_cast<f32x2*>(crow + col) = f32x2{y[0], y[1]};
+                        *reinterpret_cast<f32x2*>(crow + col + 2) = f32x2{y[2], y[3]};
+                    } else {
+#pragma unroll
+                        for (int v = 0; v < 4; ++v)
+                            if (col + v < p.N) crow[col + v] = y[v];
+                    }
+                }
+            }
+        }
+    }
+    if (p.absmax_out) block_absmax_to_global(m / 127.0f, p.absmax_out);
+}
+
 // ------------------------------------------------------- operand packing
 // dst[r, 0..ldd) = src[r, 0..cols) zero-filled, for r < rows (src row stride lds).
 __global__ __launch_bounds__(256) void pack_rows_i8_kernel(int8_t* __restrict__ dst, int64_t ldd,
@@ -626,9 +803,52 @@ static bool fq_applicable(const float* X, int64_t ldx, const int8_t* Xq, int64_t
     return true;
 }
 
+// Compute units of the current device (queried once; a fixed property of the machine).
+static int compute_units() {
+    static const int n = [] {
+        int dev = 0, cus = 0;
+        if (hipGetDevice(&dev) != hipSuccess ||
+            hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0)
+            cus = 256;
+        return cus;
+    }();
+    return n;
+}
+
+constexpr size_t kLdsBytes = 160 * 1024;
+
+template <int NT, int XV, int MODE>
+static bool launch_ws_nt(const FqParams& p, hipStream_t s) {
+    const int kq = static_cast<int>(round_up(p.K, 16));
+    int pitch = kq + 16;  // the extra chunk spreads the rows of a fragment read over the LDS banks
+    if (static_cast<size_t>(16 * NT) * pitch + 256 > kLdsBytes) pitch = kq;
+    const size_t lds = static_cast<size_t>(16 * NT) * pitch;
+    if (lds + 256 > kLdsBytes) return false;
+    static const bool ok = [] {  // more than 64 KB of dynamic LDS has to be asked for once per kernel
+        return hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_ws_kernel<NT, XV, MODE>),
+                                   hipFuncAttributeMaxDynamicSharedMemorySize,
+                                   static_cast<int>(kLdsBytes - 256)) == hipSuccess;
+    }();
+    if (!ok) return false;
+    const int64_t nblocks = ceil_div(p.M, 16);
+    const int64_t wgs = ceil_div(nblocks, 12) < compute_units() ? ceil_div(nblocks, 12) : compute_units();
+    hipLaunchKernelGGL((gemm_ws_kernel<NT, XV, MODE>), dim3(static_cast<unsigned>(wgs)), dim3(768), lds, s, p,
+                       static_cast<int>(nblocks), pitch, kq);
+    return true;
+}
+
+// W-stationary form when X is tall (at least one 16-row block per wave of the machine) and N <= 32.
+template <int XV, int MODE>
+static bool launch_ws(const FqParams& p, hipStream_t s) {
+    if (p.N > 32 || ceil_div(p.M, 16) < 12LL * compute_units() || ceil_div(p.M, 16) > INT32_MAX) return false;
+    if (p.N <= 16) return launch_ws_nt<1, XV, MODE>(p, s);
+    return launch_ws_nt<2, XV, MODE>(p, s);
+}
+
 template <int XV, int MODE>
 static void launch_fq_mode(const FqParams& p, hipStream_t s) {
     constexpr int RT = 4;  // 64 rows per workgroup measured faster than 32 at every benchmark shape
+    if (launch_ws<XV, MODE>(p, s)) return;
     const size_t lds = static_cast<size_t>(16 * RT) * (p.kp + 16);
     const unsigned gx = static_cast<unsigned>(ceil_div(p.M, 16 * RT));
 #define TANGO_FQ(TPW_)                                                                           \

@@ -215,3 +215,27 @@ def test_scale_hand_off_is_bit_identical(K):
     l2(l1(x)).sum().backward()
     for a, p in zip(g1, list(l1.parameters()) + list(l2.parameters())):
         assert torch.equal(a, p.grad)
+
+
+@pytest.mark.parametrize("Kd,N,mode,bias", [(130, 16, "rne", True), (602, 29, "trunc", False), (64, 7, "trunc", True)])
+def test_forward_gemm_tall_narrow(K, orc, Kd, N, mode, bias):
+    """Tall X with N <= 32 takes the W-stationary kernel (rows dealt over persistent waves, X quantized
+    in registers): row multiplier, bias, both deterministic rounding modes, 8- and 16-byte aligned rows,
+    a partial last k-step and a row count that is no multiple of the 16-row block."""
+    rng = np.random.default_rng(Kd + N)
+    M = 50011
+    X = rng.standard_normal((M, Kd)).astype(np.float32)
+    W = ((rng.random((N, Kd), dtype=np.float32) - 0.5) * 0.3).astype(np.float32)
+    b = rng.standard_normal(N).astype(np.float32) if bias else None
+    rm = (rng.random(M, dtype=np.float32) + 0.1).astype(np.float32)
+    Xs = (X * rm[:, None]).astype(np.float32)
+    sX, _ = K.cuda_kernels.absmax_ex(dev(X), row_mul=dev(rm))
+    sW = K.cuda_kernels.get_scale(dev(W))
+    ld = (Kd + 15) // 16 * 16
+    Xq = torch.empty((M, ld), dtype=torch.int8, device="cuda")[:, :Kd]
+    Wq = torch.empty((N, Kd), dtype=torch.int8, device="cuda")
+    Y, sY = K.QGEMM_forward(dev(X), Xq, sX, dev(W), Wq, sW, None if b is None else dev(b), True,
+                            round_mode=mode, x_row_mul=dev(rm))
+    Yo, Xqo, _, osX, _, osY = orc.qgemm_fwd(Xs, W, b, reduce=True, mode=orc.RNE if mode == "rne" else orc.TRUNC)
+    assert host(sX)[0] == osX and np.array_equal(host(Xq), Xqo)
+    assert np.array_equal(host(Y), Yo) and host(sY)[0] == osY
