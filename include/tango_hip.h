@@ -202,12 +202,17 @@ int tango_spmm_csr_copy_u(float* out, const int64_t* indptr, const int64_t* indi
    copy of the column indices made by the caller: half the index traffic).
    max_row_nnz: an upper bound of the longest row if the caller knows one (a graph
    object usually does), else 0; it only lets the library skip the launches that
-   exist for hub rows when there is none. */
+   exist for hub rows when there is none.
+   workspace (tango_spmm_workspace(nnz) bytes, 16-byte aligned, contents arbitrary) or
+   NULL: with it, hub rows (thousands of slots and far above the average) are cut over
+   many workgroups whose int32 partial sums are added into the output row with integer
+   atomics, so the result is the same either way. */
+size_t tango_spmm_workspace(int64_t nnz);
 int tango_spmm_csr_copy_u_ex(float* out, const int64_t* indptr, const void* indices, int idx_bits,
                              const int8_t* feat, int64_t ldf, const float* scale,
                              const float* row_scale, const float* bias, int relu, int64_t rows,
                              int64_t num_src, int64_t nnz, int64_t F, int64_t max_row_nnz,
-                             tango_stream_t stream);
+                             void* workspace, size_t workspace_bytes, tango_stream_t stream);
 
 /* multi_cusparse_SPMM (cuda/src/cuda.cpp:119-158 -> SPMM.cu:70-194):
    out[r,h,f] = scale[0] * float(sum_p evals[h, d, e(p)] * feat[indices[p], h, f]),
@@ -226,13 +231,14 @@ int tango_spmm_csr_u_mul_e(float* out, const int64_t* indptr, const int64_t* ind
    With the slot->edge permutation fused, the H * D bytes of a gathered edge then
    come from one cache sector instead of H * D scattered ones.  bias (H * F floats or
    NULL) is added after dequantization ("rst + bias", evaluation/test_gat.py:160-162).
-   idx_bits: width of the entries of indices and edge_ids, 64 or 32; max_row_nnz as
-   for tango_spmm_csr_copy_u_ex. */
+   idx_bits: width of the entries of indices and edge_ids, 64 or 32; max_row_nnz and
+   workspace as for tango_spmm_csr_copy_u_ex. */
 int tango_spmm_csr_u_mul_e_ex(float* out, const int64_t* indptr, const void* indices,
                               const void* edge_ids, int idx_bits, const int8_t* feat, const int8_t* evals,
                               int edge_major, const float* scale, const float* bias, int64_t rows,
                               int64_t num_src, int64_t H, int64_t F, int64_t D, int64_t nnz,
-                              int64_t max_row_nnz, tango_stream_t stream);
+                              int64_t max_row_nnz, void* workspace, size_t workspace_bytes,
+                              tango_stream_t stream);
 
 /* incidence_SPMM (cuda/src/cuda.cpp:160-167 -> incidence_SPMM_impl, SPMM.cu:259-303):
    out[v, f] = scale[0] * float(sum_{i: node_ids[i] == v} E[edge_ids[i], f]).

@@ -55,6 +55,7 @@ struct SpmmParams {
     int idx32;     // indices and edge_ids point to int32 arrays (half the index traffic); indptr stays int64
     int64_t long_row;  // rows with more slots than this go to the sixteen-wave kernel
     int64_t hub_row;   // rows with more slots than this are cut over several workgroups
+    void* hub_ws;      // caller's workspace for the hub path, or null (then no row counts as a hub)
     int64_t max_row;   // caller's upper bound of the longest row, 0 if unknown
     int64_t group_row; // sparse graphs: rows with at most this many slots are owned by a lane group
 };
@@ -454,18 +455,22 @@ __global__ __launch_bounds__(256) void spmm_medium_kernel(const SpmmParams p) {
 // the long ones are collected in LDS and each is summed by all waves; the waves' partial sums
 // meet in LDS through integer atomics, which are exact in any order.
 //
-// Hub rows (more than p.hub_row slots) would still keep one workgroup busy long after the rest of
-// the launch has drained, so they take three steps, each a launch of this kernel:
-//   LONG      zeroes the hub row's output, viewed as int32 (and sums the ordinary long rows);
-//   HUB_SUM   gridDim.z = kHubChunks workgroups per hub row each sum one chunk of its slots and add
-//             the int32 result into the output row with integer atomics (exact in any order);
-//   HUB_STORE turns the int32 sums into the fp32 result in place.
+// Hub rows (more than p.hub_row slots; needs the caller's workspace) would still keep one
+// workgroup busy long after the rest of the launch has drained.  This kernel only records them in
+// the workspace's list and zeroes their output rows, viewed as int32; spmm_hub_sum_kernel then
+// cuts every hub row into chunks of kHubChunk slots, deals all chunks over its workgroups, and adds
+// each chunk's int32 sums into the output row with integer atomics (exact in any order), and
+// spmm_hub_store_kernel turns the int32 sums into the fp32 result in place.
 constexpr int kLongGrid = 512;
-constexpr int kHubChunks = 16;
-constexpr int kHubGrid = 32;  // scanning workgroups of the hub launches (x kHubChunks): hubs are few
-enum { LONG = 0, HUB_SUM = 1, HUB_STORE = 2 };
+constexpr int kHubChunk = 2048;      // slots per chunk of a hub row: 128 per wave
+constexpr int64_t kHubRowMin = 4096; // no row shorter than this is ever treated as a hub
+constexpr int kHubSumGrid = 256;
+constexpr int kHubBatch = 2048;      // hub rows whose chunk counts a workgroup scans at a time
 
-template <int VEC, int KIND, int MODE>
+// workspace: word 0 = number of hub rows (zeroed by the library at the start of a call), byte 64.. = row ids
+__device__ __forceinline__ int64_t* hub_list(void* ws) { return reinterpret_cast<int64_t*>(static_cast<char*>(ws) + 64); }
+
+template <int VEC, int KIND>
 __global__ __launch_bounds__(1024) void spmm_long_kernel(const SpmmParams p) {
     constexpr int WAVES = 16;
     __shared__ int part[64 * VEC];
@@ -484,8 +489,7 @@ __global__ __launch_bounds__(1024) void spmm_long_kernel(const SpmmParams p) {
         if (mine < p.rows) {
             int64_t s, e;
             row_range<KIND>(p, mine, s, e);
-            const bool take = (MODE == LONG) ? (e - s > p.long_row) : (e - s > p.hub_row);
-            if (take) list[atomicAdd(&nlist, 1)] = mine;  // any order: rows are independent
+            if (e - s > p.long_row) list[atomicAdd(&nlist, 1)] = mine;  // any order: rows are independent
         }
         __syncthreads();
         const int n = nlist;
@@ -493,30 +497,15 @@ __global__ __launch_bounds__(1024) void spmm_long_kernel(const SpmmParams p) {
             const int64_t row = list[k];
             int64_t start, end;
             row_range<KIND>(p, row, start, end);
-            int* orow = reinterpret_cast<int*>(p.out) + row * p.W + c.col;  // this lane's VEC output columns
-            if (MODE == HUB_STORE || (MODE == LONG && end - start > p.hub_row)) {
+            if (end - start > p.hub_row) {  // uniform over the workgroup
+                if (blockIdx.y == 0 && t == 0) hub_list(p.hub_ws)[atomicAdd(static_cast<int*>(p.hub_ws), 1)] = row;
+                int* orow = reinterpret_cast<int*>(p.out) + row * p.W + c.col;  // this lane's VEC output columns
                 if (wave == 0 && c.grp == 0 && c.col_ok) {
-                    int acc[VEC];
 #pragma unroll
-                    for (int i = 0; i < VEC; ++i) {
-                        acc[i] = 0;
-                        if (MODE == HUB_STORE && c.col + i < p.W) acc[i] = orow[i];
-                    }
-                    if (MODE == HUB_STORE) {
-                        store_row<VEC>(p, c, row, acc);
-                    } else {
-#pragma unroll
-                        for (int i = 0; i < VEC; ++i)
-                            if (c.col + i < p.W) orow[i] = 0;
-                    }
+                    for (int i = 0; i < VEC; ++i)
+                        if (c.col + i < p.W) orow[i] = 0;
                 }
-                continue;  // uniform over the workgroup
-            }
-            if (MODE == HUB_SUM) {  // this workgroup's chunk of the row
-                const int64_t len = (end - start + kHubChunks - 1) / kHubChunks;
-                const int64_t cs = start + len * blockIdx.z;
-                start = cs < end ? cs : end;
-                end = cs + len < end ? cs + len : end;
+                continue;
             }
             const int64_t per = (end - start + WAVES - 1) / WAVES;
             const int64_t s = start + per * wave;
@@ -534,17 +523,113 @@ __global__ __launch_bounds__(1024) void spmm_long_kernel(const SpmmParams p) {
                     acc[i] = part[i * 64 + c.sub];
                     part[i * 64 + c.sub] = 0;
                 }
-                if (MODE == HUB_SUM) {
-                    if (c.col_ok) {
-#pragma unroll
-                        for (int i = 0; i < VEC; ++i)
-                            if (c.col + i < p.W) atomicAdd(orow + i, acc[i]);
-                    }
-                } else {
-                    store_row<VEC>(p, c, row, acc);
-                }
+                store_row<VEC>(p, c, row, acc);
             }
             __syncthreads();
+        }
+    }
+}
+
+// blockDim.x = 1024, grid (kHubSumGrid, column tiles).  All chunks of all hub rows form one
+// sequence (hub 0's chunks, hub 1's, ...); workgroup b takes chunks b, b + G, ...
+template <int VEC, int KIND>
+__global__ __launch_bounds__(1024) void spmm_hub_sum_kernel(const SpmmParams p) {
+    constexpr int WAVES = 16;
+    __shared__ int part[64 * VEC];
+    __shared__ int first_chunk[kHubBatch + 1];  // exclusive prefix sums of the batch's chunk counts
+    __shared__ int wsum[WAVES];
+    const int t = threadIdx.x;
+    const int lane = lane_id();
+    const int wave = __builtin_amdgcn_readfirstlane(t >> 6);
+    const LaneCols c = lane_cols<VEC, KIND>(p, lane);
+    const int nhub = *static_cast<const int*>(p.hub_ws);
+    const int64_t* hubs = hub_list(p.hub_ws);
+    for (int i = t; i < 64 * VEC; i += 1024) part[i] = 0;
+    for (int h0 = 0; h0 < nhub; h0 += kHubBatch) {  // uniform trip count
+        const int nb = nhub - h0 < kHubBatch ? nhub - h0 : kHubBatch;
+        // chunk counts of hubs h0 + 2 t and h0 + 2 t + 1, then a workgroup-wide exclusive scan
+        int cnt[2];
+#pragma unroll
+        for (int u = 0; u < 2; ++u) {
+            cnt[u] = 0;
+            const int h = 2 * t + u;
+            if (h < nb) {
+                int64_t s, e;
+                row_range<KIND>(p, hubs[h0 + h], s, e);
+                cnt[u] = static_cast<int>((e - s + kHubChunk - 1) / kHubChunk);
+            }
+        }
+        int incl = cnt[0] + cnt[1];
+        for (int off = 1; off < kWave; off <<= 1) {
+            const int v = __shfl_up(incl, off, kWave);
+            if (lane >= off) incl += v;
+        }
+        if (lane == kWave - 1) wsum[wave] = incl;
+        __syncthreads();
+        int base = 0;
+        for (int w = 0; w < wave; ++w) base += wsum[w];
+        const int excl = base + incl - cnt[0] - cnt[1];
+        if (2 * t < kHubBatch) first_chunk[2 * t] = excl;
+        if (2 * t + 1 < kHubBatch) first_chunk[2 * t + 1] = excl + cnt[0];
+        if (t == 1023) first_chunk[kHubBatch] = base + incl;
+        __syncthreads();
+        const int total = first_chunk[kHubBatch];
+        for (int gc = blockIdx.x; gc < total; gc += gridDim.x) {
+            // the hub this chunk belongs to: last h with first_chunk[h] <= gc
+            int lo = 0, hi = nb - 1;
+            while (lo < hi) {
+                const int mid = (lo + hi + 1) >> 1;
+                if (first_chunk[mid] <= gc) lo = mid; else hi = mid - 1;
+            }
+            const int64_t row = hubs[h0 + lo];
+            int64_t start, end;
+            row_range<KIND>(p, row, start, end);
+            start += static_cast<int64_t>(gc - first_chunk[lo]) * kHubChunk;
+            if (start + kHubChunk < end) end = start + kHubChunk;
+            const int64_t per = (end - start + WAVES - 1) / WAVES;
+            const int64_t s = start + per * wave;
+            const int64_t e = s + per;
+            int acc[VEC];
+            wave_row_sum<VEC, KIND>(p, c, lane, s < end ? s : end, e < end ? e : end, acc);
+            if (c.grp == 0) {
+#pragma unroll
+                for (int i = 0; i < VEC; ++i) atomicAdd(&part[i * 64 + c.sub], acc[i]);
+            }
+            __syncthreads();
+            if (wave == 0 && c.grp == 0 && c.col_ok) {
+                int* orow = reinterpret_cast<int*>(p.out) + row * p.W + c.col;
+#pragma unroll
+                for (int i = 0; i < VEC; ++i) {
+                    const int v = part[i * 64 + c.sub];
+                    part[i * 64 + c.sub] = 0;
+                    if (c.col + i < p.W) atomicAdd(orow + i, v);
+                }
+            } else if (wave == 0 && c.grp == 0) {
+#pragma unroll
+                for (int i = 0; i < VEC; ++i) part[i * 64 + c.sub] = 0;
+            }
+            __syncthreads();
+        }
+        __syncthreads();  // first_chunk is rebuilt by the next batch
+    }
+}
+
+// One wavefront per hub row: out = epilogue(int32 sum), in place.  blockDim.x = 256.
+template <int VEC, int KIND>
+__global__ __launch_bounds__(256) void spmm_hub_store_kernel(const SpmmParams p) {
+    const int lane = lane_id();
+    const int wave = __builtin_amdgcn_readfirstlane(static_cast<int>(threadIdx.x) >> 6);
+    const LaneCols c = lane_cols<VEC, KIND>(p, lane);
+    const int nhub = *static_cast<const int*>(p.hub_ws);
+    const int64_t* hubs = hub_list(p.hub_ws);
+    for (int h = blockIdx.x * 4 + wave; h < nhub; h += gridDim.x * 4) {
+        const int64_t row = hubs[h];
+        if (c.grp == 0 && c.col_ok) {
+            const int* orow = reinterpret_cast<const int*>(p.out) + row * p.W + c.col;
+            int acc[VEC];
+#pragma unroll
+            for (int i = 0; i < VEC; ++i) acc[i] = (c.col + i < p.W) ? orow[i] : 0;
+            store_row<VEC>(p, c, row, acc);
         }
     }
 }
@@ -591,20 +676,20 @@ static int launch_spmm(SpmmParams p, int vec, hipStream_t s) {
     const int64_t by_batches = 16LL * 4 * (64 >> p.lpe_log2);
     const int64_t share = p.nnz >= (64LL << 20) ? (p.nnz >> 11) : (p.nnz >> 13);
     p.long_row = share > by_batches ? share : by_batches;
-    p.hub_row = 16 * p.long_row;
     const int64_t longest = p.max_row > 0 ? p.max_row : p.nnz;  // no row has more slots than this
-    const bool hubs = longest > p.hub_row;
+    p.hub_row = 4 * p.long_row > kHubRowMin ? 4 * p.long_row : kHubRowMin;
+    const bool hubs = p.hub_ws && longest > p.hub_row;
     if (!hubs) p.hub_row = INT64_MAX;
     const dim3 lgrid(static_cast<unsigned>(p.rows < kLongGrid ? p.rows : kLongGrid), static_cast<unsigned>(ychunks));
-    const dim3 hgrid(static_cast<unsigned>(p.rows < kHubGrid ? p.rows : kHubGrid), lgrid.y, kHubChunks);
-    const dim3 sgrid(hgrid.x, lgrid.y);
-#define TANGO_SPMM_LONG(V)                                                                                  \
-    do {                                                                                                    \
-        hipLaunchKernelGGL((spmm_long_kernel<V, KIND, LONG>), lgrid, dim3(1024), 0, s, p);                  \
-        if (hubs) {                                                                                         \
-            hipLaunchKernelGGL((spmm_long_kernel<V, KIND, HUB_SUM>), hgrid, dim3(1024), 0, s, p);           \
-            hipLaunchKernelGGL((spmm_long_kernel<V, KIND, HUB_STORE>), sgrid, dim3(1024), 0, s, p);         \
-        }                                                                                                   \
+    const dim3 hgrid(kHubSumGrid, lgrid.y), sgrid(64, lgrid.y);
+#define TANGO_SPMM_LONG(V)                                                                          \
+    do {                                                                                            \
+        if (hubs) fill_u32(p.hub_ws, 0u, 1, s);                                                     \
+        hipLaunchKernelGGL((spmm_long_kernel<V, KIND>), lgrid, dim3(1024), 0, s, p);                \
+        if (hubs) {                                                                                 \
+            hipLaunchKernelGGL((spmm_hub_sum_kernel<V, KIND>), hgrid, dim3(1024), 0, s, p);         \
+            hipLaunchKernelGGL((spmm_hub_store_kernel<V, KIND>), sgrid, dim3(256), 0, s, p);        \
+        }                                                                                           \
     } while (0)
     if (longest > p.long_row) {
         if (vec == 16) TANGO_SPMM_LONG(16);
@@ -657,6 +742,11 @@ using namespace tango;
 
 extern "C" {
 
+size_t tango_spmm_workspace(int64_t nnz) {
+    if (nnz < 0) return 0;
+    return 64 + sizeof(int64_t) * static_cast<size_t>(nnz / kHubRowMin + 2);
+}
+
 int tango_spmm_csr_copy_u(float* out, const int64_t* indptr, const int64_t* indices,
                           const int8_t* feat, int64_t ldf, const float* scale, int64_t rows,
                           int64_t num_src, int64_t nnz, int64_t F, tango_stream_t stream) {
@@ -674,15 +764,17 @@ int tango_spmm_csr_copy_u_ex(float* out, const int64_t* indptr, const void* indi
                              const int8_t* feat, int64_t ldf, const float* scale,
                              const float* row_scale, const float* bias, int relu, int64_t rows,
                              int64_t num_src, int64_t nnz, int64_t F, int64_t max_row_nnz,
-                             tango_stream_t stream) {
+                             void* workspace, size_t workspace_bytes, tango_stream_t stream) {
     if (rows < 0 || F < 0 || nnz < 0 || num_src < 0 || ldf < F || !scale || !indptr || max_row_nnz < 0 ||
         (rows * F > 0 && !out) || (nnz > 0 && (!indices || !feat)) || (idx_bits != 32 && idx_bits != 64))
         return TANGO_ERR_INVALID_ARG;
+    if (workspace && (workspace_bytes < tango_spmm_workspace(nnz) || (reinterpret_cast<uintptr_t>(workspace) & 15)))
+        return TANGO_ERR_WORKSPACE;
     if (num_src >= (1LL << 31) || nnz >= (1LL << 31)) return TANGO_ERR_UNSUPPORTED;
     SpmmParams p{};
     p.out = out; p.indptr = indptr; p.indices = static_cast<const int64_t*>(indices); p.idx32 = idx_bits == 32;
     p.feat = feat; p.scale = scale;
-    p.row_scale = row_scale; p.bias = bias; p.relu = relu ? 1 : 0; p.max_row = max_row_nnz;
+    p.row_scale = row_scale; p.bias = bias; p.relu = relu ? 1 : 0; p.max_row = max_row_nnz; p.hub_ws = workspace;
     p.rows = rows; p.num_src = num_src; p.ldf = ldf; p.W = F; p.F = F; p.D = 1; p.nnz = nnz;
     return launch_spmm<KIND_COPY>(p, pick_vec(feat, ldf, F), as_stream(stream));
 }
@@ -691,17 +783,20 @@ int tango_spmm_csr_u_mul_e_ex(float* out, const int64_t* indptr, const void* ind
                               const void* edge_ids, int idx_bits, const int8_t* feat, const int8_t* evals,
                               int edge_major, const float* scale, const float* bias, int64_t rows,
                               int64_t num_src, int64_t H, int64_t F, int64_t D, int64_t nnz,
-                              int64_t max_row_nnz, tango_stream_t stream) {
+                              int64_t max_row_nnz, void* workspace, size_t workspace_bytes,
+                              tango_stream_t stream) {
     if (rows < 0 || H < 0 || F < 0 || nnz < 0 || num_src < 0 || !scale || !indptr || max_row_nnz < 0 ||
         (rows * H * F > 0 && !out) || (nnz > 0 && (!indices || !feat || !evals)) ||
         (idx_bits != 32 && idx_bits != 64))
         return TANGO_ERR_INVALID_ARG;
+    if (workspace && (workspace_bytes < tango_spmm_workspace(nnz) || (reinterpret_cast<uintptr_t>(workspace) & 15)))
+        return TANGO_ERR_WORKSPACE;
     if (D != 1 && D != F) return TANGO_ERR_UNSUPPORTED;
     if (num_src >= (1LL << 31) || nnz >= (1LL << 31)) return TANGO_ERR_UNSUPPORTED;
     SpmmParams p{};
     p.out = out; p.indptr = indptr; p.indices = static_cast<const int64_t*>(indices);
     p.edge_ids = static_cast<const int64_t*>(edge_ids); p.idx32 = idx_bits == 32; p.feat = feat;
-    p.max_row = max_row_nnz;
+    p.max_row = max_row_nnz; p.hub_ws = workspace;
     p.evals = evals; p.scale = scale; p.bias = bias; p.rows = rows; p.num_src = num_src; p.ldf = H * F; p.W = H * F; p.F = F; p.D = D;
     p.nnz = nnz;
     if (edge_major) {  // evals[nnz, H, D]: the H * D bytes of one edge share a cache sector
@@ -724,7 +819,7 @@ int tango_spmm_csr_u_mul_e(float* out, const int64_t* indptr, const int64_t* ind
                            const float* scale, int64_t rows, int64_t num_src, int64_t H,
                            int64_t F, int64_t D, int64_t nnz, tango_stream_t stream) {
     return tango_spmm_csr_u_mul_e_ex(out, indptr, indices, edge_ids, 64, feat, evals, 0, scale, nullptr, rows, num_src,
-                                     H, F, D, nnz, 0, stream);
+                                     H, F, D, nnz, 0, nullptr, 0, stream);
 }
 
 int tango_spmm_incidence(float* out, const int64_t* node_ids, const int64_t* edge_ids,
