@@ -82,6 +82,8 @@ def _zero_slot(device):
         pool = _ZERO_SLOTS.get(key)
         if pool is None or pool[1] >= _POOL_SIZE:
             pool = _ZERO_SLOTS[key] = [torch.zeros(_POOL_SIZE, dtype=torch.float32, device=device), 0]
+            # slots may be used on any stream later: have the one fill finished before the first is handed out
+            torch.cuda.current_stream(device).synchronize()
         k = pool[1]
         pool[1] = k + 1
     return pool[0][k:k + 1]
