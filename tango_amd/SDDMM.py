@@ -1,11 +1,10 @@
 """Quantized per-edge ops: mirrors cuda/SDDMM.py of the reference, plus the
 ``sddmm_u_dot_v`` op that the reference's drivers call but its tree does not
 define (evaluation/test_HGT.py:58, evaluation/link_pred_gcn.py:145)."""
-import torch
 from torch.autograd.function import Function, once_differentiable
 
 from . import config
-from .kernels import incidence_SPMM, multi_cusparse_SPMM, mySDDMM_int8, quantize, transpose_quant
+from .kernels import incidence_SPMM, multi_cusparse_SPMM, mySDDMM_int8, quantize
 
 
 def _quantize_grad(t):

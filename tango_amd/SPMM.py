@@ -1,10 +1,8 @@
 """Quantized aggregation ops: mirrors cuda/SPMM.py of the reference."""
-import torch
 from torch.autograd.function import Function, once_differentiable
 
 from . import config
-from .kernels import (cuda_kernels, csr_SPMM, multi_cusparse_SPMM, mySDDMM_int8, quantize,
-                      quantize_padded, transpose_quant)
+from .kernels import cuda_kernels, csr_SPMM, multi_cusparse_SPMM, mySDDMM_int8, quantize, quantize_padded
 
 
 def _gather_align(width):

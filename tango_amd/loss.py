@@ -4,7 +4,6 @@ call (evaluation/test_gcn.py:256)."""
 import torch
 from torch.autograd.function import Function, once_differentiable
 
-from . import _lib
 from .kernels import _L, _ptr, _stream, _workspace, check
 
 

@@ -6,7 +6,7 @@ import numpy as np
 import pytest
 import torch
 
-from gpu_util import dev, host, rand_graph, sc
+from gpu_util import dev, host, rand_graph
 
 pytestmark = pytest.mark.gpu
 
