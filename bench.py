@@ -193,7 +193,7 @@ def model_steps(K, torch):
     model = GAT(g, 3, 128, 16, 40, [8, 8, 1], torch.nn.functional.elu).cuda()
     x = torch.randn(n, 128, device="cuda")
     labels = torch.randint(0, 16, (n,), device="cuda")
-    opt = torch.optim.Adam(model.parameters(), lr=1e-3)
+    opt = torch.optim.Adam(model.parameters(), lr=1e-3, fused=True)
 
     def gat_step():
         opt.zero_grad(set_to_none=True)
@@ -207,7 +207,7 @@ def model_steps(K, torch):
     hgt = HGTStack(256, 256, 16, 4, n_layers=2).cuda()
     xh = torch.randn(n, 256, device="cuda")
     lh = torch.randint(0, 16, (n,), device="cuda")
-    opth = torch.optim.Adam(hgt.parameters(), lr=1e-3)
+    opth = torch.optim.Adam(hgt.parameters(), lr=1e-3, fused=True)
 
     def hgt_step():
         opth.zero_grad(set_to_none=True)
@@ -351,7 +351,7 @@ def main():
     labels = torch.randint(0, 41, (n,), generator=gen).cuda()
     torch.manual_seed(5)
     model = GCN(g, 602, 256, 41, 1, torch.relu, 0.0).cuda()
-    opt = torch.optim.Adam(model.parameters(), lr=1e-2, weight_decay=5e-4)
+    opt = torch.optim.Adam(model.parameters(), lr=1e-2, weight_decay=5e-4, fused=True)  # one kernel for all parameters
     config.grad_round_mode = "stochastic"
 
     timer = KernelTimer()
