@@ -47,11 +47,16 @@ def test_absmax_ex_and_quantize_ex(K, orc):
     assert torch.equal(a, b)
 
 
+# (n, e): rows of ~66 slots (one wave per row), and a sparse graph with a long row and a hub row (the epilogue
+# also runs in the sixteen-wave kernel and in the hub store pass)
+@pytest.mark.parametrize("n,e", [(600, 40000), (5000, 40000)])
 @pytest.mark.parametrize("F", [16, 41, 256])
-def test_spmm_fused_epilogue_equals_separate_passes(K, F):
+def test_spmm_fused_epilogue_equals_separate_passes(K, F, n, e):
     rng = np.random.default_rng(F)
-    n, e = 600, 40000
     src, dst = rand_graph(rng, n, e)
+    if n == 5000:
+        dst[:9000] = 5
+        dst[9000:10500] = 6
     g = make_graph(src, dst, n)
     feat = dev(rng.integers(-127, 128, (n, F)).astype(np.int8))
     rs = dev(rng.random(n, dtype=np.float32) + 0.05)

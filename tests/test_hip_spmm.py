@@ -111,10 +111,13 @@ def test_u_mul_e_broadcast(K, orc, kind, n, e, H, F):
     assert np.array_equal(host(got2), want)
 
 
-def test_u_mul_e_elementwise(K, orc):
+@pytest.mark.parametrize("n,e,H,F", [(300, 20000, 3, 8), (3000, 9000, 2, 16), (2000, 30000, 1, 5)])
+def test_u_mul_e_elementwise(K, orc, n, e, H, F):
+    """Edge values as wide as the features (D == F): dense rows, lane-group rows of a sparse graph, and a hub."""
     rng = np.random.default_rng(2)
-    n, e, H, F = 300, 20000, 3, 8
     src, dst = rand_graph(rng, n, e)
+    if e == 30000:
+        dst[:6000] = 11
     g = make_graph(src, dst, n)
     o = orc.graph_formats(src, dst, n)
     feat = rng.integers(-127, 128, (n, H, F)).astype(np.int8)
