@@ -37,7 +37,7 @@ def parse():
     ap.add_argument("--no-primitives", action="store_true")
     ap.add_argument("--emit", default=None, metavar="JSON_FILE",
                     help="also store the result under the key 'measured_mi355x' of this JSON file")
-    ap.add_argument("--profile-mode", choices=["spmm", "copy"], default=None,
+    ap.add_argument("--profile-mode", choices=["spmm", "copy", "qlinear", "sddmm", "quantize"], default=None,
                     help="run only the dominant kernel (spmm: copy_u F=256 on the benchmark graph) or a "
                          "1 GiB device copy (counter calibration), for rocprofv3 --pmc passes")
     return ap.parse_args()
@@ -328,6 +328,37 @@ def main():
             dst.copy_(src)
         torch.cuda.synchronize()
         print(json.dumps({"profile_mode": "copy", "bytes_read": src.numel() * 4, "bytes_written": src.numel() * 4}))
+        return
+    if args.profile_mode == "qlinear":  # the forward GEMM of layer 1, fp32 in, Xq cached, fp32 out + scale
+        M, Kd, N = args.nodes, 602, 256
+        X = torch.randn(M, Kd, device="cuda")
+        W = torch.randn(N, Kd, device="cuda") * 0.05
+        sX, sW = K.cuda_kernels.get_scale(X), K.cuda_kernels.get_scale(W)
+        Xq = torch.empty((M, 608), dtype=torch.int8, device="cuda")[:, :Kd]
+        Wq = torch.empty((N, Kd), dtype=torch.int8, device="cuda")
+        ms = time_op(lambda: K.QGEMM_forward(X, Xq, sX, W, Wq, sW, None, True), iters=args.steps, warm=args.warmup)
+        print(json.dumps({"profile_mode": "qlinear", "M": M, "K": Kd, "N": N, "avg_ms": round(ms, 4),
+                          "ops": 2 * M * N * Kd, "algorithmic_bytes": 5 * (M * Kd + N * Kd) + 4 * M * N + 4 * N}))
+        return
+    if args.profile_mode == "quantize":
+        X = torch.randn(args.nodes, 602, device="cuda")
+        s = K.cuda_kernels.get_scale(X)
+        q = torch.empty(X.shape, dtype=torch.int8, device="cuda")
+        ms = time_op(lambda: K.cuda_kernels.quantize(q, X, s), iters=args.steps, warm=args.warmup)
+        ms_a = time_op(lambda: K.cuda_kernels.get_scale(X), iters=args.steps, warm=args.warmup)
+        print(json.dumps({"profile_mode": "quantize", "elements": X.numel(), "quantize_ms": round(ms, 4),
+                          "absmax_ms": round(ms_a, 4), "quantize_bytes": 5 * X.numel(), "absmax_bytes": 4 * X.numel()}))
+        return
+    if args.profile_mode == "sddmm":
+        g4 = graph_preprocess(chung_lu(169343, 1166243, 2.2, seed=4, device="cuda"))
+        n4, E, H, D = g4.num_nodes(), g4.num_edges(), 8, 16
+        U = torch.randint(-127, 128, (n4, H, D), dtype=torch.int8, device="cuda")
+        V = torch.randint(-127, 128, (n4, H, D), dtype=torch.int8, device="cuda")
+        one = torch.full((1,), 0.01, device="cuda")
+        ms = time_op(lambda: K.mySDDMM_int8(g4, "dot", U, V, one, one, False), iters=args.steps, warm=args.warmup)
+        print(json.dumps({"profile_mode": "sddmm", "nodes": n4, "edges": E, "H": H, "D": D, "avg_ms": round(ms, 4),
+                          "algorithmic_bytes": E * (16 + 2 * H * D + 4 * H),
+                          "compulsory_bytes": E * 16 + 2 * n4 * H * D + 4 * E * H}))
         return
     t0 = time.perf_counter()
     g = graph_preprocess(chung_lu(args.nodes, args.edges, 2.0, seed=3, max_degree=21000, symmetric=True,
