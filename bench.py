@@ -37,7 +37,7 @@ def parse():
     ap.add_argument("--no-primitives", action="store_true")
     ap.add_argument("--emit", default=None, metavar="JSON_FILE",
                     help="also store the result under the key 'measured_mi355x' of this JSON file")
-    ap.add_argument("--profile-mode", choices=["spmm", "copy", "qlinear", "sddmm", "quantize"], default=None,
+    ap.add_argument("--profile-mode", choices=["spmm", "copy", "qlinear", "sddmm", "quantize", "gat", "hgt"], default=None,
                     help="run only the dominant kernel (spmm: copy_u F=256 on the benchmark graph) or a "
                          "1 GiB device copy (counter calibration), for rocprofv3 --pmc passes")
     return ap.parse_args()
@@ -178,16 +178,24 @@ def sddmm_primitives(K, torch):
     return out
 
 
-def model_steps(K, torch):
+def model_steps(K, torch, which=("gat", "hgt"), iters=10, warm=3):
     """The other model configurations, one training step each (forward + loss + backward + Adam):
     the 3-layer GAT (hidden 16 x 8 heads, evaluation/test_gat.py:170-214) on the 169,343-node graph
     and two HGT layers (256-d, 4 heads) on the homogenised 3-type / 4-relation graph."""
-    from tango_amd.gat import GAT, HGTStack
-    from tango_amd.graph import chung_lu, hetero_power_law
-    from tango_amd.loss import cross_entropy
-    from tango_amd.util import graph_preprocess
     out = {}
     torch.manual_seed(4)
+    if "gat" in which:
+        out.update(_gat_step(K, torch, iters, warm))
+    if "hgt" in which:
+        out.update(_hgt_step(K, torch, iters, warm))
+    return out
+
+
+def _gat_step(K, torch, iters, warm):
+    from tango_amd.gat import GAT
+    from tango_amd.graph import chung_lu
+    from tango_amd.loss import cross_entropy
+    from tango_amd.util import graph_preprocess
     g = graph_preprocess(chung_lu(169343, 1166243, 2.2, seed=4, device="cuda"))
     n = g.num_nodes()
     model = GAT(g, 3, 128, 16, 40, [8, 8, 1], torch.nn.functional.elu).cuda()
@@ -199,8 +207,14 @@ def model_steps(K, torch):
         opt.zero_grad(set_to_none=True)
         cross_entropy(model(x), labels).backward()
         opt.step()
-    out["gat3_step_169343n_1.34Me_ms"] = round(time_op(gat_step, iters=10, warm=3), 3)
-    del model, opt, x, g
+    return {"gat3_step_169343n_1.34Me_ms": round(time_op(gat_step, iters=iters, warm=warm), 3)}
+
+
+def _hgt_step(K, torch, iters, warm):
+    from tango_amd.gat import HGTStack
+    from tango_amd.graph import hetero_power_law
+    from tango_amd.loss import cross_entropy
+    from tango_amd.util import graph_preprocess
     g, _, _ = hetero_power_law(device="cuda")
     g = graph_preprocess(g)
     n = g.num_nodes()
@@ -213,8 +227,7 @@ def model_steps(K, torch):
         opth.zero_grad(set_to_none=True)
         cross_entropy(hgt(g, xh), lh).backward()
         opth.step()
-    out["hgt2_step_170000n_8.17Me_ms"] = round(time_op(hgt_step, iters=10, warm=3), 3)
-    return out
+    return {"hgt2_step_170000n_8.17Me_ms": round(time_op(hgt_step, iters=iters, warm=warm), 3)}
 
 
 def cpu_baseline(g, X, W1, W2, frac, reps=3):
@@ -328,6 +341,10 @@ def main():
             dst.copy_(src)
         torch.cuda.synchronize()
         print(json.dumps({"profile_mode": "copy", "bytes_read": src.numel() * 4, "bytes_written": src.numel() * 4}))
+        return
+    if args.profile_mode in ("gat", "hgt"):  # one training step of the attention models, for kernel traces
+        out = model_steps(K, torch, which=(args.profile_mode,), iters=args.steps, warm=args.warmup)
+        print(json.dumps(dict(out, profile_mode=args.profile_mode)))
         return
     if args.profile_mode == "qlinear":  # the forward GEMM of layer 1, fp32 in, Xq cached, fp32 out + scale
         M, Kd, N = args.nodes, 602, 256

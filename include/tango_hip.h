@@ -271,19 +271,22 @@ int tango_sddmm_ewise_i8(int op, float* out, float* scale_out, const int64_t* sr
    is not part of the reference tree).  e and a are [num_edges, H] in edge-id
    order; indptr/edge_ids describe the destination-major CSR (adj_csc);
    edge_ids may be NULL for the identity.  slope = 1 gives the plain softmax.
-   workspace (tango_edge_softmax_workspace(H) bytes, 16-byte aligned) lets hub
-   destinations (tens of thousands of in-edges) be cut over many workgroups; with
-   NULL one workgroup walks each of them.  The result is the same either way up to
-   the summation order of the fp64 partial sums. */
-size_t tango_edge_softmax_workspace(int64_t H);
+   num_edges = indptr[rows].  The work is cut by edge slots (256 per wavefront), so hub
+   destinations cost no more per edge than the others; rows cut by a slot boundary
+   are combined through workspace (tango_edge_softmax_workspace(num_edges, H) bytes,
+   16-byte aligned; contents need not be initialised).  With workspace = NULL a thread
+   walks each (destination, head) alone: same results up to the fp32 summation order,
+   slow for hubs. */
+size_t tango_edge_softmax_workspace(int64_t num_edges, int64_t H);
 int tango_edge_softmax_fwd(float* a, const float* e, const int64_t* indptr,
-                           const int64_t* edge_ids, int64_t rows, int64_t H, float slope,
-                           void* workspace, size_t workspace_bytes, tango_stream_t stream);
+                           const int64_t* edge_ids, int64_t rows, int64_t num_edges, int64_t H,
+                           float slope, void* workspace, size_t workspace_bytes,
+                           tango_stream_t stream);
 /* de = dLeaky(e) * a * (da - sum_{same dst} a*da). */
 int tango_edge_softmax_bwd(float* de, const float* a, const float* da, const float* e,
                            const int64_t* indptr, const int64_t* edge_ids, int64_t rows,
-                           int64_t H, float slope, void* workspace, size_t workspace_bytes,
-                           tango_stream_t stream);
+                           int64_t num_edges, int64_t H, float slope, void* workspace,
+                           size_t workspace_bytes, tango_stream_t stream);
 
 /* ------------------------------------------------------ GAT attention logits */
 

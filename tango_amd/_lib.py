@@ -54,9 +54,9 @@ SIGNATURES = {
     "tango_sddmm_ewise_i8": (I, [I, P, P, P, P, P, P, P, P, I64, I64, P]),
     "tango_softmax_xent_workspace": (SZ, [I64]),
     "tango_softmax_xent_f32": (I, [P, I64, P, I64, I64, P, P, I64, P, SZ, P]),
-    "tango_edge_softmax_workspace": (SZ, [I64]),
-    "tango_edge_softmax_fwd": (I, [P, P, P, P, I64, I64, F, P, SZ, P]),
-    "tango_edge_softmax_bwd": (I, [P, P, P, P, P, P, I64, I64, F, P, SZ, P]),
+    "tango_edge_softmax_workspace": (SZ, [I64, I64]),
+    "tango_edge_softmax_fwd": (I, [P, P, P, P, I64, I64, I64, F, P, SZ, P]),
+    "tango_edge_softmax_bwd": (I, [P, P, P, P, P, P, I64, I64, I64, F, P, SZ, P]),
 }
 
 ROUND_RNE, ROUND_TRUNC, ROUND_STOCHASTIC = 0, 1, 2

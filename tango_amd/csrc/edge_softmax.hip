@@ -1,12 +1,14 @@
 // LeakyReLU + per-destination edge softmax (forward and backward) for gfx950.
 //
 // fp32, memory-bound: e is read, a written, both [E, H] in edge-id order and
-// reached through the destination-major CSR's edge-id permutation.  Threads are
-// (edge slot, head) pairs, so the H values of an edge are one contiguous read, and
-// a destination is owned by a thread group sized to its in-degree (see the tiers
-// below).  The forward pass keeps a running (max, sum) pair per thread (online
-// softmax): two sweeps over a row instead of three, one for rows held in registers.
-// For H > 64 a thread-per-(row, head) fallback is used.
+// reached through the destination-major CSR's edge-id permutation.  The work is cut
+// by edge slots, not by rows: a wavefront owns a span of 256 consecutive slots of the
+// destination-major order whatever rows they belong to, so a hub destination and a
+// million destinations with three in-edges cost the same per edge.  Rows that lie
+// inside one span are finished in one sweep (values stay in registers between the
+// reduction and the write); a row cut by a span boundary leaves per-span partial
+// results that a small second launch combines and a third writes out.  Without a
+// workspace a thread-per-(row, head) kernel is used.
 #include "common.hpp"
 
 namespace tango {
@@ -67,464 +69,449 @@ __global__ __launch_bounds__(256) void edge_softmax_bwd_kernel(
     }
 }
 
-// Three tiers by in-degree, for H <= 64 (Hp = H rounded up to a power of two):
-//   short  (<= kShortRow edges): a thread owns one (row, head) and keeps the row's values in
-//          registers, one sweep over memory; a wavefront covers 64 / H rows, which is what
-//          keeps enough bytes in flight when most destinations have a handful of in-edges;
-//   medium (<= kMediumValues / Hp edges): a wavefront owns the row, lane = (edge slot, head),
-//          four edges per lane in flight, reduction by xor-shuffles over the slot bits;
-//   long   : a 1024-thread workgroup owns the row (a hub destination must not be walked by one
-//          wavefront while the rest of the chip idles).
-// The medium and long kernels find their rows themselves: a wavefront / workgroup inspects a
-// strided set of rows at once (hubs with neighbouring ids spread out over the launch) and walks
-// the ones of its tier; no list of rows is built in global memory.
-constexpr int kShortRow = 16;
-constexpr int kMediumValues = 2048;
-// A hub: a destination with more than kHubValues / Hp in-edges.  One workgroup walking it alone
-// would outlast the whole rest of the launch, so (when the caller passes a workspace) the long
-// tier only records such rows and two further launches cut each into kHubChunks chunks: partial
-// (max, sum) per chunk and head, then every chunk combines its row's partials and writes its part.
-constexpr int kHubValues = 32768;
-constexpr int kHubChunks = 32;
-constexpr int kMaxHubs = 256;     // hubs beyond this stay with the long tier's single workgroup
-constexpr int kHubGridY = 64;     // workgroup rows of the hub launches; each walks hubs y, y + 64, ...
+// ---------------------------------------------------------------------------------------------
+// Span kernels.  Wavefront w owns slots [w * kSpan, (w + 1) * kSpan), lane l of step u holds slot
+// base + 64 u + l with HB heads of it (head block blockIdx.y).  Per step, a segmented scan over
+// the lanes (segments = rows) gives every lane its row's (max, sum of exp) within the step; rows
+// running over a step boundary chain through a wave-uniform carry, and the lanes of their earlier
+// steps pick the finished result up from `fin`.  Three kinds of row:
+//   inside : starts and ends within the span -> written by this launch;
+//   head   : started in an earlier span      -> partial result in piece 0 of the span's record;
+//   tail   : runs on into the next span      -> partial result in piece 1.
+// span_fix_kernel merges a row's pieces (the tail of the span it starts in and the heads of the
+// spans that follow) and stores the row's result back into every piece; span_rest_kernel then
+// writes the head and tail slots.  No atomics: results do not depend on scheduling.
+constexpr int kSteps = 4;
+constexpr int kSpan = kWave * kSteps;
+constexpr int kWin = kSpan + kWave;  // row pointers staged per wavefront: 64 empty rows of slack
 
-// Workspace: [0] hub count (int), then kMaxHubs x (p0, p1) int64, then the partials
-// [kMaxHubs][kHubChunks][Hp] of {float max; double sum} (backward: the double only).
-struct HubPartial {
-    double sum;
-    float mx;
-    float pad;
+struct SpanMeta {
+    int64_t head_end;    // slots [base, head_end) belong to a row that started before the span
+    int64_t tail_start;  // slots [tail_start, end) belong to a row that runs on after the span
+    int64_t head_open;   // the head row also runs on after the span (then there is no tail)
 };
-__host__ __device__ inline size_t hub_list_offset() { return 256; }
-__host__ __device__ inline size_t hub_partial_offset() { return 256 + sizeof(int64_t) * 2 * kMaxHubs; }
 
-__device__ __forceinline__ void softmax_merge(float& m, double& s, float m2, double s2) {
-    const float mx = fmaxf(m, m2);
-    // exp(-inf - -inf) would be NaN: a side with no elements contributes nothing
-    const double a = (m == -INFINITY) ? 0.0 : s * static_cast<double>(expf(m - mx));
-    const double b = (m2 == -INFINITY) ? 0.0 : s2 * static_cast<double>(expf(m2 - mx));
-    m = mx;
-    s = a + b;
+__host__ __device__ inline size_t span_vals_offset(int64_t nspans) {
+    return (static_cast<size_t>(nspans) * sizeof(SpanMeta) + 255) & ~static_cast<size_t>(255);
+}
+// vals[span][piece][component][H]: component 0 = max, 1 = sum (backward: only the sum)
+__device__ __forceinline__ float* span_vals(void* ws, int64_t nspans, int64_t w, int piece, int comp, int H) {
+    return reinterpret_cast<float*>(static_cast<char*>(ws) + span_vals_offset(nspans)) +
+           ((w * 2 + piece) * 2 + comp) * static_cast<int64_t>(H);
 }
 
-// 0 = short, 1 = medium, 2 = long
-__device__ __forceinline__ int row_tier(int64_t deg, int hp_log2) {
-    if (deg <= kShortRow) return 0;
-    return deg <= (kMediumValues >> hp_log2) ? 1 : 2;
+__device__ __forceinline__ float rl_f(float v, int l) {
+    return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), l));
 }
 
-__global__ __launch_bounds__(256) void edge_softmax_fwd_short_kernel(
-    float* __restrict__ a, const float* __restrict__ e, const int64_t* __restrict__ indptr,
-    const int64_t* __restrict__ eids, int64_t rows, int H, float slope) {
-    const int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
-    if (i >= rows * H) return;
-    const int64_t r = i / H;
-    const int h = static_cast<int>(i - r * H);
-    const int64_t p0 = indptr[r];
-    const int64_t deg = indptr[r + 1] - p0;
-    if (deg > kShortRow || deg == 0) return;
-    int64_t id[kShortRow];
-    float v[kShortRow];
+// inclusive scans over lanes [lo, lane] (lo = first lane of this lane's segment)
+__device__ __forceinline__ float seg_scan_max(float x, int lane, int lo) {
 #pragma unroll
-    for (int u = 0; u < kShortRow; ++u) {
-        v[u] = -INFINITY;
-        id[u] = 0;
-        if (u < deg) {
-            id[u] = (eids ? eids[p0 + u] : p0 + u) * H + h;
-            v[u] = leaky(e[id[u]], slope);
-        }
+    for (int off = 1; off < kWave; off <<= 1) {
+        const float t = __shfl_up(x, off, kWave);
+        if (lane - off >= lo) x = fmaxf(x, t);
     }
-    float mx = v[0];
+    return x;
+}
+__device__ __forceinline__ float seg_scan_add(float x, int lane, int lo) {
 #pragma unroll
-    for (int u = 1; u < kShortRow; ++u) mx = fmaxf(mx, v[u]);
-    double sum = 0.0;
-#pragma unroll
-    for (int u = 0; u < kShortRow; ++u) {
-        v[u] = u < deg ? expf(v[u] - mx) : 0.0f;
-        sum += static_cast<double>(v[u]);
+    for (int off = 1; off < kWave; off <<= 1) {
+        const float t = __shfl_up(x, off, kWave);
+        if (lane - off >= lo) x += t;
     }
-    const float inv = static_cast<float>(1.0 / sum);
-#pragma unroll
-    for (int u = 0; u < kShortRow; ++u)
-        if (u < deg) a[id[u]] = v[u] * inv;
+    return x;
 }
 
-__global__ __launch_bounds__(256) void edge_softmax_bwd_short_kernel(
-    float* __restrict__ de, const float* __restrict__ a, const float* __restrict__ da,
-    const float* __restrict__ e, const int64_t* __restrict__ indptr,
-    const int64_t* __restrict__ eids, int64_t rows, int H, float slope) {
-    const int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
-    if (i >= rows * H) return;
-    const int64_t r = i / H;
-    const int h = static_cast<int>(i - r * H);
-    const int64_t p0 = indptr[r];
-    const int64_t deg = indptr[r + 1] - p0;
-    if (deg > kShortRow || deg == 0) return;
-    int64_t id[kShortRow];
-    float x[kShortRow], y[kShortRow], z[kShortRow];
-    double dsum = 0.0;
-#pragma unroll
-    for (int u = 0; u < kShortRow; ++u) {
-        x[u] = y[u] = z[u] = 0.0f;
-        id[u] = 0;
-        if (u < deg) {
-            id[u] = (eids ? eids[p0 + u] : p0 + u) * H + h;
-            x[u] = a[id[u]];
-            y[u] = da[id[u]];
-            z[u] = e[id[u]];
-        }
+// largest r in [0, rows) with indptr[r] <= key (indptr[0] = 0 <= key): 64 probes per round
+__device__ __forceinline__ int64_t row_of_slot_wave(const int64_t* __restrict__ indptr, int64_t rows, int64_t key,
+                                                    int lane) {
+    int64_t lo = 0, hi = rows;  // the answer lies in [lo, hi)
+    while (hi - lo > 1) {
+        const int64_t step = (hi - lo + kWave - 1) >> 6;
+        const int64_t probe = lo + lane * step;
+        const bool ok = probe < hi && indptr[probe] <= key;
+        const int cnt = __popcll(__ballot(ok));  // lane 0 always holds
+        lo += (cnt - 1) * step;
+        hi = lo + step < hi ? lo + step : hi;
     }
-#pragma unroll
-    for (int u = 0; u < kShortRow; ++u) dsum += static_cast<double>(x[u]) * static_cast<double>(y[u]);
-    const float dot = static_cast<float>(dsum);
-#pragma unroll
-    for (int u = 0; u < kShortRow; ++u)
-        if (u < deg) {
-            float g = x[u] * (y[u] - dot);
-            if (!(z[u] > 0.0f)) g *= slope;
-            de[id[u]] = g;
-        }
+    return lo;
 }
 
-// `nthreads` threads (a wavefront or a workgroup) walk slots [p0, p1) of one row: thread t is
-// (edge slot t >> hp_log2, head t & (Hp - 1)).  Returns this thread's running (max, sum).
-template <int U>
-__device__ __forceinline__ void fwd_partial(const float* __restrict__ e, const int64_t* __restrict__ eids,
-                                            int64_t p0, int64_t p1, int t, int nthreads, int H, int hp_log2,
-                                            float slope, float& mx, double& sum) {
-    const int h = t & ((1 << hp_log2) - 1);
-    const int64_t es = t >> hp_log2, nes = nthreads >> hp_log2;
-    const bool hok = h < H;
-    mx = -INFINITY;
-    sum = 0.0;
-    for (int64_t p = p0 + es; p < p1; p += U * nes) {  // U independent edges in flight per thread
-        float v[U];
+template <int HB, bool VEC>
+__device__ __forceinline__ void load_heads(float (&v)[HB], const float* __restrict__ p, int nh) {
+    if (VEC && HB == 8) {
+        const float4 x = *reinterpret_cast<const float4*>(p), y = *reinterpret_cast<const float4*>(p + 4);
+        v[0] = x.x; v[1] = x.y; v[2] = x.z; v[3] = x.w;
+        v[4 % HB] = y.x; v[5 % HB] = y.y; v[6 % HB] = y.z; v[7 % HB] = y.w;
+    } else if (VEC && HB == 4) {
+        const float4 x = *reinterpret_cast<const float4*>(p);
+        v[0] = x.x; v[1 % HB] = x.y; v[2 % HB] = x.z; v[3 % HB] = x.w;
+    } else if (VEC && HB == 2) {
+        const float2 x = *reinterpret_cast<const float2*>(p);
+        v[0] = x.x; v[1 % HB] = x.y;
+    } else {
 #pragma unroll
-        for (int u = 0; u < U; ++u) {
-            const int64_t q = p + u * nes;
-            v[u] = -INFINITY;
-            if (hok && q < p1) v[u] = leaky(e[(eids ? eids[q] : q) * H + h], slope);
-        }
-#pragma unroll
-        for (int u = 0; u < U; ++u) {
-            if (v[u] == -INFINITY) continue;
-            if (v[u] > mx) {  // one exp per element either way
-                sum = sum * static_cast<double>(expf(mx - v[u])) + 1.0;  // exp(-inf) = 0 for the first element
-                mx = v[u];
-            } else {
-                sum += static_cast<double>(expf(v[u] - mx));
-            }
-        }
+        for (int i = 0; i < HB; ++i) v[i] = i < nh ? p[i] : 0.0f;
     }
 }
 
-template <int U>
-__device__ __forceinline__ void fwd_write(float* __restrict__ a, const float* __restrict__ e,
-                                          const int64_t* __restrict__ eids, int64_t p0, int64_t p1, int t,
-                                          int nthreads, int H, int hp_log2, float slope, float mx, float inv) {
-    const int h = t & ((1 << hp_log2) - 1);
-    const int64_t es = t >> hp_log2, nes = nthreads >> hp_log2;
-    const bool hok = h < H;
-    for (int64_t p = p0 + es; p < p1; p += U * nes) {
-        int64_t id[U];
-        float v[U];
+template <int HB, bool VEC>
+__device__ __forceinline__ void store_heads(float* __restrict__ p, const float (&v)[HB], int nh) {
+    if (VEC && HB == 8) {
+        *reinterpret_cast<float4*>(p) = make_float4(v[0], v[1 % HB], v[2 % HB], v[3 % HB]);
+        *reinterpret_cast<float4*>(p + 4) = make_float4(v[4 % HB], v[5 % HB], v[6 % HB], v[7 % HB]);
+    } else if (VEC && HB == 4) {
+        *reinterpret_cast<float4*>(p) = make_float4(v[0], v[1 % HB], v[2 % HB], v[3 % HB]);
+    } else if (VEC && HB == 2) {
+        *reinterpret_cast<float2*>(p) = make_float2(v[0], v[1 % HB]);
+    } else {
 #pragma unroll
-        for (int u = 0; u < U; ++u) {
-            const int64_t q = p + u * nes;
-            id[u] = -1;
-            if (hok && q < p1) {
-                id[u] = (eids ? eids[q] : q) * H + h;
-                v[u] = e[id[u]];
-            }
-        }
-#pragma unroll
-        for (int u = 0; u < U; ++u)
-            if (id[u] >= 0) a[id[u]] = expf(leaky(v[u], slope) - mx) * inv;
+        for (int i = 0; i < HB; ++i)
+            if (i < nh) p[i] = v[i];
     }
 }
 
-template <int U>
-__device__ __forceinline__ double bwd_partial(const float* __restrict__ a, const float* __restrict__ da,
-                                              const int64_t* __restrict__ eids, int64_t p0, int64_t p1, int t,
-                                              int nthreads, int H, int hp_log2) {
-    const int h = t & ((1 << hp_log2) - 1);
-    const int64_t es = t >> hp_log2, nes = nthreads >> hp_log2;
-    const bool hok = h < H;
-    double dsum = 0.0;
-    for (int64_t p = p0 + es; p < p1; p += U * nes) {
-        float x[U], y[U];
-#pragma unroll
-        for (int u = 0; u < U; ++u) {
-            const int64_t q = p + u * nes;
-            x[u] = y[u] = 0.0f;
-            if (hok && q < p1) {
-                const int64_t id = (eids ? eids[q] : q) * H + h;
-                x[u] = a[id];
-                y[u] = da[id];
-            }
-        }
-#pragma unroll
-        for (int u = 0; u < U; ++u) dsum += static_cast<double>(x[u]) * static_cast<double>(y[u]);
-    }
-    return dsum;
-}
-
-template <int U>
-__device__ __forceinline__ void bwd_write(float* __restrict__ de, const float* __restrict__ a,
-                                          const float* __restrict__ da, const float* __restrict__ e,
-                                          const int64_t* __restrict__ eids, int64_t p0, int64_t p1, int t,
-                                          int nthreads, int H, int hp_log2, float slope, float dot) {
-    const int h = t & ((1 << hp_log2) - 1);
-    const int64_t es = t >> hp_log2, nes = nthreads >> hp_log2;
-    const bool hok = h < H;
-    for (int64_t p = p0 + es; p < p1; p += U * nes) {
-        int64_t id[U];
-        float x[U], y[U], z[U];
-#pragma unroll
-        for (int u = 0; u < U; ++u) {
-            const int64_t q = p + u * nes;
-            id[u] = -1;
-            if (hok && q < p1) {
-                id[u] = (eids ? eids[q] : q) * H + h;
-                x[u] = a[id[u]];
-                y[u] = da[id[u]];
-                z[u] = e[id[u]];
-            }
-        }
-#pragma unroll
-        for (int u = 0; u < U; ++u)
-            if (id[u] >= 0) {
-                float g = x[u] * (y[u] - dot);
-                if (!(z[u] > 0.0f)) g *= slope;
-                de[id[u]] = g;
-            }
-    }
-}
-
-// Medium rows.  Wavefront w of the launch inspects rows w, w + W, w + 2W, ... (kRowsPerWave of
-// them, W = number of wavefronts launched) and walks the medium ones in turn.
-constexpr int kRowsPerWave = 8;
-template <bool FWD>
-__global__ __launch_bounds__(256) void edge_softmax_medium_kernel(
+// blockDim.x = 256 (four spans per workgroup), grid = (ceil(nspans / 4), ceil(H / HB)).
+// VEC: H is a multiple of HB, so the HB heads of an edge are one aligned vector.
+template <int HB, bool VEC, bool FWD>
+__global__ __launch_bounds__(256) void span_kernel(
     float* __restrict__ out, const float* __restrict__ a, const float* __restrict__ da,
     const float* __restrict__ e, const int64_t* __restrict__ indptr, const int64_t* __restrict__ eids,
-    int64_t rows, int H, int hp_log2, float slope) {
+    int64_t rows, int64_t nnz, int H, float slope, void* __restrict__ ws) {
+    __shared__ int64_t win_all[4][kWin];
     const int lane = lane_id();
-    const int64_t nwaves = static_cast<int64_t>(gridDim.x) * 4;
-    const int64_t w = static_cast<int64_t>(blockIdx.x) * 4 + (threadIdx.x >> 6);
-    const int64_t mine = w + static_cast<int64_t>(lane) * nwaves;
-    int64_t q0 = 0, q1 = 0;
-    if (lane < kRowsPerWave && mine < rows) {
-        q0 = indptr[mine];
-        q1 = indptr[mine + 1];
+    const int wave = static_cast<int>(threadIdx.x) >> 6;
+    const int64_t nspans = (nnz + kSpan - 1) / kSpan;
+    const int64_t w = static_cast<int64_t>(blockIdx.x) * 4 + wave;
+    if (w >= nspans) return;  // the whole wavefront leaves; no workgroup barrier below
+    int64_t* win = win_all[wave];
+    const int h0 = static_cast<int>(blockIdx.y) * HB;
+    const int nh = H - h0 < HB ? H - h0 : HB;
+    const int64_t base = w * kSpan;
+    const int endl = static_cast<int>((nnz - base < kSpan) ? nnz - base : kSpan);  // slots in this span
+    const int64_t end = base + endl;
+
+    // ---- which row does each of my slots belong to
+    const int64_t r0 = row_of_slot_wave(indptr, rows, base, lane);
+#pragma unroll
+    for (int k = 0; k < kWin / kWave; ++k) {
+        const int64_t r = r0 + lane + kWave * k;
+        win[lane + kWave * k] = r <= rows ? indptr[r] : INT64_MAX;
     }
-    uint64_t todo = __ballot(row_tier(q1 - q0, hp_log2) == 1);
-    while (todo) {
-        const int l = __builtin_ctzll(todo);
-        todo &= todo - 1;
-        const int64_t p0 = __shfl(q0, l, kWave), p1 = __shfl(q1, l, kWave);
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    const bool staged = win[kWin - 1] >= end;  // every row of the span has both pointers in the window
+    int rsl[kSteps], rel[kSteps];  // my row's first slot and end slot relative to base: -1 = before, kSpan + 1 = after
+#pragma unroll
+    for (int u = 0; u < kSteps; ++u) {
+        int64_t s = base + kWave * u + lane;
+        s = s < end ? s : end - 1;
+        int64_t rs, re;
+        if (staged) {
+            int pos = 0;
+#pragma unroll
+            for (int step = 256; step > 0; step >>= 1)
+                if (pos + step < kWin && win[pos + step] <= s) pos += step;
+            rs = win[pos];
+            re = win[pos + 1];
+        } else {  // a long run of empty rows inside the span: search the array itself
+            int64_t lo = r0, hi = rows;
+            while (hi - lo > 1) {
+                const int64_t mid = lo + ((hi - lo) >> 1);
+                if (indptr[mid] <= s) lo = mid; else hi = mid;
+            }
+            rs = indptr[lo];
+            re = indptr[lo + 1];
+        }
+        rsl[u] = rs < base ? -1 : static_cast<int>(rs - base);
+        rel[u] = re > end ? kSpan + 1 : static_cast<int>(re - base);
+    }
+
+    // ---- values
+    int64_t id[kSteps];
+    float x[kSteps][HB];   // forward: leaky(e); backward: a
+    float y[kSteps][HB];   // backward: da
+#pragma unroll
+    for (int u = 0; u < kSteps; ++u) {
+        const int64_t s = base + kWave * u + lane;
+        const bool valid = kWave * u + lane < endl;
+        id[u] = -1;
+#pragma unroll
+        for (int i = 0; i < HB; ++i) x[u][i] = FWD ? -INFINITY : 0.0f, y[u][i] = 0.0f;
+        if (valid) {
+            id[u] = (eids ? eids[s] : s) * H + h0;
+            if (FWD) {
+                load_heads<HB, VEC>(x[u], e + id[u], nh);
+#pragma unroll
+                for (int i = 0; i < HB; ++i) x[u][i] = leaky(x[u][i], slope);
+            } else {
+                load_heads<HB, VEC>(x[u], a + id[u], nh);
+                load_heads<HB, VEC>(y[u], da + id[u], nh);
+            }
+        }
+    }
+
+    // ---- per step: my row's result within the span so far
+    float tm[kSteps][HB], ts[kSteps][HB];
+    float fm[kSteps - 1][HB], fs[kSteps - 1][HB];  // wave-uniform: the row crossing the boundary after step b
+    float cm[HB], cs[HB];                          // wave-uniform carry of the row open at the end of the last step
+#pragma unroll
+    for (int i = 0; i < HB; ++i) cm[i] = -INFINITY, cs[i] = 0.0f;
+#pragma unroll
+    for (int b = 0; b < kSteps - 1; ++b)
+#pragma unroll
+        for (int i = 0; i < HB; ++i) fm[b][i] = 0.0f, fs[b][i] = 1.0f;
+#pragma unroll
+    for (int u = 0; u < kSteps; ++u) {
+        const int sbl = kWave * u;
+        const int sel = sbl + kWave < endl ? sbl + kWave : endl;
+        if (sbl >= endl) break;  // uniform
+        const int lo = rsl[u] > sbl ? rsl[u] - sbl : 0;
+        const int hi = (rel[u] < sel ? rel[u] : sel) - 1 - sbl;
+        const bool cont_in = rsl[u] < sbl;  // my row began in an earlier step (or span)
+#pragma unroll
+        for (int i = 0; i < HB; ++i) {
+            if (FWD) {
+                float m = seg_scan_max(x[u][i], lane, lo);
+                m = __shfl(m, hi, kWave);
+                if (cont_in) m = fmaxf(m, cm[i]);
+                const float ex = (kWave * u + lane < endl) ? expf(x[u][i] - m) : 0.0f;
+                float s = seg_scan_add(ex, lane, lo);
+                s = __shfl(s, hi, kWave);
+                if (cont_in) s += cs[i] * expf(cm[i] - m);  // an empty carry is (-inf, 0)
+                tm[u][i] = m;
+                ts[u][i] = s;
+            } else {
+                float s = seg_scan_add(x[u][i] * y[u][i], lane, lo);
+                s = __shfl(s, hi, kWave);
+                if (cont_in) s += cs[i];
+                tm[u][i] = 0.0f;
+                ts[u][i] = s;
+            }
+        }
+        // the row of lane 0 ends in this step and began in an earlier step of this span: its result
+        // goes to the boundaries it crossed
+        const int rs0 = __builtin_amdgcn_readfirstlane(rsl[u]);
+        const int re0 = __builtin_amdgcn_readfirstlane(rel[u]);
+        if (rs0 >= 0 && rs0 < sbl && re0 <= sel) {
+#pragma unroll
+            for (int b = 0; b < kSteps - 1; ++b)
+                if (b < u && b >= (rs0 >> 6)) {
+#pragma unroll
+                    for (int i = 0; i < HB; ++i) fm[b][i] = rl_f(tm[u][i], 0), fs[b][i] = rl_f(ts[u][i], 0);
+                }
+        }
+        // carry: the row of the last lane, if it runs on
+        const bool open = __builtin_amdgcn_readlane(rel[u], kWave - 1) > sel;
+#pragma unroll
+        for (int i = 0; i < HB; ++i) {
+            cm[i] = open ? rl_f(tm[u][i], kWave - 1) : -INFINITY;
+            cs[i] = open ? rl_f(ts[u][i], kWave - 1) : 0.0f;
+        }
+        // partial results of the head row (at its last slot in the span) and of the tail row (at the span's last slot)
+        const int ls = sbl + lane;  // my slot, relative
+        if (ls < endl) {
+            const bool last_of_row = ls == (rel[u] < endl ? rel[u] : endl) - 1;
+            if (last_of_row && rsl[u] < 0) {
+                store_heads<HB, false>(span_vals(ws, nspans, w, 0, 0, H) + h0, tm[u], nh);
+                store_heads<HB, false>(span_vals(ws, nspans, w, 0, 1, H) + h0, ts[u], nh);
+            }
+            if (last_of_row && rsl[u] >= 0 && rel[u] > endl) {
+                store_heads<HB, false>(span_vals(ws, nspans, w, 1, 0, H) + h0, tm[u], nh);
+                store_heads<HB, false>(span_vals(ws, nspans, w, 1, 1, H) + h0, ts[u], nh);
+            }
+            if (blockIdx.y == 0) {
+                SpanMeta* meta = static_cast<SpanMeta*>(ws) + w;
+                if (ls == 0) {
+                    meta->head_end = rsl[u] < 0 ? base + (rel[u] < endl ? rel[u] : endl) : base;
+                    meta->head_open = (rsl[u] < 0 && rel[u] > endl) ? 1 : 0;
+                }
+                if (ls == endl - 1) meta->tail_start = (rsl[u] >= 0 && rel[u] > endl) ? base + rsl[u] : end;
+            }
+        }
+    }
+
+    // ---- rows inside the span: write
+#pragma unroll
+    for (int u = 0; u < kSteps; ++u) {
+        const int sbl = kWave * u;
+        const int sel = sbl + kWave < endl ? sbl + kWave : endl;
+        if (id[u] < 0 || rsl[u] < 0 || rel[u] > endl) continue;
+        const bool later = rel[u] > sel;  // my row ends in a later step
+        float o[HB];
         if (FWD) {
-            float mx;
-            double sum;
-            fwd_partial<8>(e, eids, p0, p1, lane, kWave, H, hp_log2, slope, mx, sum);
-            for (int off = 1 << hp_log2; off < kWave; off <<= 1) {
-                const float m2 = __shfl_xor(mx, off, kWave);
-                const double s2 = __shfl_xor(sum, off, kWave);
-                softmax_merge(mx, sum, m2, s2);
+#pragma unroll
+            for (int i = 0; i < HB; ++i) {
+                const float m = (later && u < kSteps - 1) ? fm[u < kSteps - 1 ? u : 0][i] : tm[u][i];
+                const float s = (later && u < kSteps - 1) ? fs[u < kSteps - 1 ? u : 0][i] : ts[u][i];
+                o[i] = expf(x[u][i] - m) * (1.0f / s);
             }
-            fwd_write<8>(out, e, eids, p0, p1, lane, kWave, H, hp_log2, slope, mx, static_cast<float>(1.0 / sum));
         } else {
-            double dsum = bwd_partial<8>(a, da, eids, p0, p1, lane, kWave, H, hp_log2);
-            for (int off = 1 << hp_log2; off < kWave; off <<= 1) dsum += __shfl_xor(dsum, off, kWave);
-            bwd_write<8>(out, a, da, e, eids, p0, p1, lane, kWave, H, hp_log2, slope, static_cast<float>(dsum));
+            float z[HB];
+            load_heads<HB, VEC>(z, e + id[u], nh);
+#pragma unroll
+            for (int i = 0; i < HB; ++i) {
+                const float dot = (later && u < kSteps - 1) ? fs[u < kSteps - 1 ? u : 0][i] : ts[u][i];
+                float g = x[u][i] * (y[u][i] - dot);
+                if (!(z[i] > 0.0f)) g *= slope;
+                o[i] = g;
+            }
         }
+        store_heads<HB, VEC>(out + id[u], o, nh);
     }
 }
 
-// Long rows.  A fixed number of 1024-thread workgroups (G = gridDim.x) share the rows: thread t
-// of workgroup b inspects row b + G * t (then b + G * (1024 + t), ...), the long ones are
-// collected in LDS and walked in turn by all sixteen wavefronts: shuffles inside a wavefront,
-// then one exchange of the sixteen partial results through LDS.
-constexpr int kLongGrid = 512;
-
+// One wavefront per span that holds the start of a cut row: merges the row's pieces and stores the
+// result into each of them.  blockDim.x = 256, grid = ceil(nspans / 4).
 template <bool FWD>
-__global__ __launch_bounds__(1024) void edge_softmax_long_kernel(
-    float* __restrict__ out, const float* __restrict__ a, const float* __restrict__ da,
-    const float* __restrict__ e, const int64_t* __restrict__ indptr, const int64_t* __restrict__ eids,
-    int64_t rows, int H, int hp_log2, float slope, void* __restrict__ hub_ws) {
-    __shared__ float mred[16][64];
-    __shared__ double sred[16][64];
-    __shared__ int64_t lp0[1024], lp1[1024];
-    __shared__ int nlist;
-    const int t = threadIdx.x;
+__global__ __launch_bounds__(256) void span_fix_kernel(int64_t nnz, int H, void* __restrict__ ws) {
     const int lane = lane_id();
-    const int wave = t >> 6;
-    const int hp = 1 << hp_log2;
-    const int h = t & (hp - 1);
-    const int64_t G = gridDim.x;
-    for (int64_t first = blockIdx.x; first < rows; first += 1024 * G) {  // uniform trip count
-        if (t == 0) nlist = 0;
-        __syncthreads();
-        const int64_t mine = first + G * t;
-        if (mine < rows) {
-            const int64_t q0 = indptr[mine], q1 = indptr[mine + 1];
-            if (row_tier(q1 - q0, hp_log2) == 2) {
-                int hub = -1;
-                if (hub_ws && (q1 - q0) > (kHubValues >> hp_log2)) {
-                    hub = atomicAdd(static_cast<int*>(hub_ws), 1);  // any order: rows are independent
-                    if (hub < kMaxHubs) {
-                        int64_t* hl = reinterpret_cast<int64_t*>(static_cast<char*>(hub_ws) + hub_list_offset());
-                        hl[2 * hub] = q0;
-                        hl[2 * hub + 1] = q1;
-                    }
-                }
-                if (hub < 0 || hub >= kMaxHubs) {
-                    const int k = atomicAdd(&nlist, 1);
-                    lp0[k] = q0;
-                    lp1[k] = q1;
-                }
+    const int64_t nspans = (nnz + kSpan - 1) / kSpan;
+    const int64_t w = static_cast<int64_t>(blockIdx.x) * 4 + (static_cast<int>(threadIdx.x) >> 6);
+    if (w >= nspans) return;
+    const SpanMeta* meta = static_cast<const SpanMeta*>(ws);
+    const int64_t end = (w + 1) * kSpan < nnz ? (w + 1) * kSpan : nnz;
+    if (meta[w].tail_start >= end) return;  // no row starts here and runs on
+    // the pieces: tail of w, then heads of w + 1 .. last, where last is the first span whose head is closed
+    int64_t last = w + 1;
+    for (;; last += kWave) {
+        const int64_t j = last + lane;
+        const bool closed = j >= nspans || meta[j].head_open == 0;
+        const uint64_t m = __ballot(closed);
+        if (m) {
+            last += __builtin_ctzll(m);
+            break;
+        }
+    }
+    if (last >= nspans) last = nspans - 1;
+    for (int h = 0; h < H; ++h) {
+        float m = -INFINITY, s = 0.0f;
+        for (int64_t j = w + 1 + lane; j <= last; j += kWave) {
+            const float s2 = *(span_vals(ws, nspans, j, 0, 1, H) + h);
+            if (FWD) {
+                const float m2 = *(span_vals(ws, nspans, j, 0, 0, H) + h);
+                const float mx = fmaxf(m, m2);
+                s = (m == -INFINITY ? 0.0f : s * expf(m - mx)) + s2 * expf(m2 - mx);
+                m = mx;
+            } else {
+                s += s2;
             }
         }
-        __syncthreads();
-        const int n = nlist;
-        for (int k = 0; k < n; ++k) {
-            const int64_t p0 = lp0[k], p1 = lp1[k];
+        if (lane == 0) {  // the tail piece joins on lane 0
+            const float s2 = *(span_vals(ws, nspans, w, 1, 1, H) + h);
             if (FWD) {
-                float mx;
-                double sum;
-                fwd_partial<8>(e, eids, p0, p1, t, 1024, H, hp_log2, slope, mx, sum);
-                for (int off = hp; off < kWave; off <<= 1) {
-                    const float m2 = __shfl_xor(mx, off, kWave);
-                    const double s2 = __shfl_xor(sum, off, kWave);
-                    softmax_merge(mx, sum, m2, s2);
-                }
-                if (lane < hp) {
-                    mred[wave][lane] = mx;
-                    sred[wave][lane] = sum;
-                }
-                __syncthreads();
-                mx = mred[0][h];
-                sum = sred[0][h];
-#pragma unroll
-                for (int w = 1; w < 16; ++w) softmax_merge(mx, sum, mred[w][h], sred[w][h]);
-                fwd_write<8>(out, e, eids, p0, p1, t, 1024, H, hp_log2, slope, mx, static_cast<float>(1.0 / sum));
+                const float m2 = *(span_vals(ws, nspans, w, 1, 0, H) + h);
+                const float mx = fmaxf(m, m2);
+                s = (m == -INFINITY ? 0.0f : s * expf(m - mx)) + s2 * expf(m2 - mx);
+                m = mx;
             } else {
-                double dsum = bwd_partial<8>(a, da, eids, p0, p1, t, 1024, H, hp_log2);
-                for (int off = hp; off < kWave; off <<= 1) dsum += __shfl_xor(dsum, off, kWave);
-                if (lane < hp) sred[wave][lane] = dsum;
-                __syncthreads();
-                dsum = 0.0;
-#pragma unroll
-                for (int w = 0; w < 16; ++w) dsum += sred[w][h];
-                bwd_write<8>(out, a, da, e, eids, p0, p1, t, 1024, H, hp_log2, slope, static_cast<float>(dsum));
+                s += s2;
             }
-            __syncthreads();  // the partial results are consumed before the next row overwrites them
+        }
+        if (FWD) {
+            const float mx = wave_max(m);
+            s = (m == -INFINITY) ? 0.0f : s * expf(m - mx);
+            m = mx;
+        }
+        s = wave_sum(s);
+        for (int64_t j = w + 1 + lane; j <= last; j += kWave) {
+            *(span_vals(ws, nspans, j, 0, 0, H) + h) = m;
+            *(span_vals(ws, nspans, j, 0, 1, H) + h) = s;
+        }
+        if (lane == 0) {
+            *(span_vals(ws, nspans, w, 1, 0, H) + h) = m;
+            *(span_vals(ws, nspans, w, 1, 1, H) + h) = s;
         }
     }
 }
 
-// Hub launches.  blockDim.x = 256, grid = (kHubChunks, kHubGridY).  PHASE 0 writes the chunk's
-// partials, PHASE 1 combines the kHubChunks partials of the row (every chunk does so for itself,
-// in chunk order) and writes the chunk's outputs.
-template <bool FWD, int PHASE>
-__global__ __launch_bounds__(256) void edge_softmax_hub_kernel(
+// Writes the head and tail slots of every span from the merged results.  Launched like span_kernel.
+template <int HB, bool VEC, bool FWD>
+__global__ __launch_bounds__(256) void span_rest_kernel(
     float* __restrict__ out, const float* __restrict__ a, const float* __restrict__ da,
-    const float* __restrict__ e, const int64_t* __restrict__ eids, int H, int hp_log2, float slope,
-    void* __restrict__ hub_ws) {
-    __shared__ float mred[4][64];
-    __shared__ double sred[4][64];
-    const int count = *static_cast<const int*>(hub_ws);
-    const int nhubs = count < kMaxHubs ? count : kMaxHubs;
-    const int64_t* hl = reinterpret_cast<const int64_t*>(static_cast<const char*>(hub_ws) + hub_list_offset());
-    HubPartial* part = reinterpret_cast<HubPartial*>(static_cast<char*>(hub_ws) + hub_partial_offset());
-    const int t = threadIdx.x, lane = lane_id(), wave = t >> 6;
-    const int hp = 1 << hp_log2;
-    const int h = t & (hp - 1);
-    const int c = blockIdx.x;
-    for (int hub = blockIdx.y; hub < nhubs; hub += gridDim.y) {
-        const int64_t p0 = hl[2 * hub], p1 = hl[2 * hub + 1];
-        const int64_t len = (p1 - p0 + kHubChunks - 1) / kHubChunks;
-        const int64_t c0 = p0 + len * c < p1 ? p0 + len * c : p1;
-        const int64_t c1 = c0 + len < p1 ? c0 + len : p1;
-        HubPartial* row_part = part + (static_cast<int64_t>(hub) * kHubChunks << hp_log2);
-        if (PHASE == 0) {
-            float mx = -INFINITY;
-            double sum = 0.0;
-            if (FWD) {
-                fwd_partial<8>(e, eids, c0, c1, t, 256, H, hp_log2, slope, mx, sum);
-                for (int off = hp; off < kWave; off <<= 1) {
-                    const float m2 = __shfl_xor(mx, off, kWave);
-                    const double s2 = __shfl_xor(sum, off, kWave);
-                    softmax_merge(mx, sum, m2, s2);
-                }
-            } else {
-                sum = bwd_partial<8>(a, da, eids, c0, c1, t, 256, H, hp_log2);
-                for (int off = hp; off < kWave; off <<= 1) sum += __shfl_xor(sum, off, kWave);
-            }
-            if (lane < hp) {
-                mred[wave][lane] = mx;
-                sred[wave][lane] = sum;
-            }
-            __syncthreads();
-            if (t < hp) {
-                mx = mred[0][t];
-                sum = sred[0][t];
-                for (int w = 1; w < 4; ++w) {
-                    if (FWD) softmax_merge(mx, sum, mred[w][t], sred[w][t]);
-                    else sum += sred[w][t];
-                }
-                row_part[(c << hp_log2) + t] = HubPartial{sum, mx, 0.0f};
-            }
-            __syncthreads();
-        } else {
-            float mx = -INFINITY;
-            double sum = 0.0;
-            for (int k = 0; k < kHubChunks; ++k) {
-                const HubPartial q = row_part[(k << hp_log2) + h];
-                if (FWD) softmax_merge(mx, sum, q.mx, q.sum);
-                else sum += q.sum;
-            }
-            if (FWD) fwd_write<8>(out, e, eids, c0, c1, t, 256, H, hp_log2, slope, mx, static_cast<float>(1.0 / sum));
-            else bwd_write<8>(out, a, da, e, eids, c0, c1, t, 256, H, hp_log2, slope, static_cast<float>(sum));
+    const float* __restrict__ e, const int64_t* __restrict__ eids, int64_t nnz, int H, float slope,
+    void* __restrict__ ws) {
+    const int lane = lane_id();
+    const int64_t nspans = (nnz + kSpan - 1) / kSpan;
+    const int64_t w = static_cast<int64_t>(blockIdx.x) * 4 + (static_cast<int>(threadIdx.x) >> 6);
+    if (w >= nspans) return;
+    const SpanMeta mt = static_cast<const SpanMeta*>(ws)[w];
+    const int64_t base = w * kSpan;
+    const int64_t end = base + kSpan < nnz ? base + kSpan : nnz;
+    if (mt.head_end <= base && mt.tail_start >= end) return;
+    const int h0 = static_cast<int>(blockIdx.y) * HB;
+    const int nh = H - h0 < HB ? H - h0 : HB;
+    float rm[2][HB], rs[2][HB];
+#pragma unroll
+    for (int piece = 0; piece < 2; ++piece) {
+        const bool have = piece == 0 ? mt.head_end > base : mt.tail_start < end;
+#pragma unroll
+        for (int i = 0; i < HB; ++i) {
+            rm[piece][i] = (have && i < nh) ? *(span_vals(ws, nspans, w, piece, 0, H) + h0 + i) : 0.0f;
+            rs[piece][i] = (have && i < nh) ? *(span_vals(ws, nspans, w, piece, 1, H) + h0 + i) : 1.0f;
         }
     }
-}
-
-// Launches the tiers.  FWD: out = a; otherwise out = de.  hub_ws may be null.
-template <bool FWD>
-static void launch_tiers(float* out, const float* a, const float* da, const float* e, const int64_t* indptr,
-                         const int64_t* eids, int64_t rows, int H, float slope, void* hub_ws, hipStream_t s) {
-    int hp = 0;
-    while ((1 << hp) < H) ++hp;
-    const unsigned sgrid = static_cast<unsigned>(ceil_div(rows * H, 256));
-    if (hub_ws) fill_u32(hub_ws, 0u, 1, s);  // the hub counter
-    // the long tier first: its workgroups are the last to finish
-    hipLaunchKernelGGL(edge_softmax_long_kernel<FWD>,
-                       dim3(static_cast<unsigned>(rows < kLongGrid ? rows : kLongGrid)), dim3(1024), 0,
-                       s, out, a, da, e, indptr, eids, rows, H, hp, slope, hub_ws);
-    if (hub_ws) {
-        const dim3 hgrid(kHubChunks, kHubGridY);
-        hipLaunchKernelGGL((edge_softmax_hub_kernel<FWD, 0>), hgrid, dim3(256), 0, s, out, a, da, e, eids, H, hp, slope,
-                           hub_ws);
-        hipLaunchKernelGGL((edge_softmax_hub_kernel<FWD, 1>), hgrid, dim3(256), 0, s, out, a, da, e, eids, H, hp, slope,
-                           hub_ws);
+#pragma unroll
+    for (int u = 0; u < kSteps; ++u) {
+        const int64_t s = base + kWave * u + lane;
+        const bool inhead = s < mt.head_end;
+        const bool intail = s >= mt.tail_start && s < end;
+        if (!inhead && !intail) continue;
+        const int piece = inhead ? 0 : 1;
+        const int64_t id = (eids ? eids[s] : s) * H + h0;
+        float o[HB], z[HB];
+        load_heads<HB, VEC>(z, e + id, nh);
+        if (FWD) {
+#pragma unroll
+            for (int i = 0; i < HB; ++i)
+                o[i] = expf(leaky(z[i], slope) - (piece ? rm[1][i] : rm[0][i])) * (1.0f / (piece ? rs[1][i] : rs[0][i]));
+        } else {
+            float x[HB], y[HB];
+            load_heads<HB, VEC>(x, a + id, nh);
+            load_heads<HB, VEC>(y, da + id, nh);
+#pragma unroll
+            for (int i = 0; i < HB; ++i) {
+                float g = x[i] * (y[i] - (piece ? rs[1][i] : rs[0][i]));
+                if (!(z[i] > 0.0f)) g *= slope;
+                o[i] = g;
+            }
+        }
+        store_heads<HB, VEC>(out + id, o, nh);
     }
-    if (FWD)
-        hipLaunchKernelGGL(edge_softmax_fwd_short_kernel, dim3(sgrid), dim3(256), 0, s, out, e, indptr, eids, rows, H,
-                           slope);
-    else
-        hipLaunchKernelGGL(edge_softmax_bwd_short_kernel, dim3(sgrid), dim3(256), 0, s, out, a, da, e, indptr, eids,
-                           rows, H, slope);
-    hipLaunchKernelGGL(edge_softmax_medium_kernel<FWD>, dim3(static_cast<unsigned>(ceil_div(rows, 4 * kRowsPerWave))),
-                       dim3(256), 0, s, out, a, da, e, indptr, eids, rows, H, hp, slope);
 }
 
-static size_t hub_workspace_bytes(int64_t H) {
-    if (H <= 0 || H > 64) return 0;
-    int hp = 0;
-    while ((1 << hp) < H) ++hp;
-    return hub_partial_offset() + (static_cast<size_t>(kMaxHubs) * kHubChunks << hp) * sizeof(HubPartial);
+template <int HB, bool VEC, bool FWD>
+static void launch_spans_hb(float* out, const float* a, const float* da, const float* e, const int64_t* indptr,
+                            const int64_t* eids, int64_t rows, int64_t nnz, int H, float slope, void* ws,
+                            hipStream_t s) {
+    const int64_t nspans = ceil_div(nnz, kSpan);
+    const dim3 grid(static_cast<unsigned>(ceil_div(nspans, 4)), static_cast<unsigned>(ceil_div(H, HB)));
+    hipLaunchKernelGGL((span_kernel<HB, VEC, FWD>), grid, dim3(256), 0, s, out, a, da, e, indptr, eids, rows, nnz, H,
+                       slope, ws);
+    hipLaunchKernelGGL(span_fix_kernel<FWD>, dim3(grid.x), dim3(256), 0, s, nnz, H, ws);
+    hipLaunchKernelGGL((span_rest_kernel<HB, VEC, FWD>), grid, dim3(256), 0, s, out, a, da, e, eids, nnz, H, slope,
+                       ws);
+}
+
+template <bool FWD>
+static void launch_spans(float* out, const float* a, const float* da, const float* e, const int64_t* indptr,
+                         const int64_t* eids, int64_t rows, int64_t nnz, int H, float slope, void* ws,
+                         hipStream_t s) {
+#define TANGO_SPANS(HB, VEC) launch_spans_hb<HB, VEC, FWD>(out, a, da, e, indptr, eids, rows, nnz, H, slope, ws, s)
+    if (H % 8 == 0) TANGO_SPANS(8, true);
+    else if (H % 4 == 0) TANGO_SPANS(4, true);
+    else if (H == 2) TANGO_SPANS(2, true);
+    else if (H == 1) TANGO_SPANS(1, false);
+    else if (H < 4) TANGO_SPANS(4, false);
+    else TANGO_SPANS(8, false);
+#undef TANGO_SPANS
+}
+
+static size_t span_workspace_bytes(int64_t nnz, int64_t H) {
+    if (nnz <= 0 || H <= 0) return 0;
+    const int64_t nspans = ceil_div(nnz, kSpan);
+    return span_vals_offset(nspans) + static_cast<size_t>(nspans) * 4 * static_cast<size_t>(H) * sizeof(float);
 }
 
 }  // namespace tango
@@ -533,19 +520,19 @@ using namespace tango;
 
 extern "C" {
 
-size_t tango_edge_softmax_workspace(int64_t H) { return hub_workspace_bytes(H); }
+size_t tango_edge_softmax_workspace(int64_t nnz, int64_t H) { return span_workspace_bytes(nnz, H); }
 
 int tango_edge_softmax_fwd(float* a, const float* e, const int64_t* indptr,
-                           const int64_t* edge_ids, int64_t rows, int64_t H, float slope,
+                           const int64_t* edge_ids, int64_t rows, int64_t nnz, int64_t H, float slope,
                            void* workspace, size_t workspace_bytes, tango_stream_t stream) {
-    if (rows < 0 || H < 0 || (rows > 0 && !indptr) || H >= (1LL << 31)) return TANGO_ERR_INVALID_ARG;
-    if (rows * H == 0) return TANGO_OK;
+    if (rows < 0 || nnz < 0 || H < 0 || (rows > 0 && !indptr) || H >= (1LL << 31)) return TANGO_ERR_INVALID_ARG;
+    if (rows * H == 0 || nnz == 0) return TANGO_OK;
     if (!a || !e) return TANGO_ERR_INVALID_ARG;
-    if (H <= 64 && rows * H <= 256LL * INT32_MAX) {
-        if (workspace && (workspace_bytes < hub_workspace_bytes(H) || (reinterpret_cast<uintptr_t>(workspace) & 15)))
+    if (workspace && ceil_div(nnz, 4 * kSpan) <= INT32_MAX && ceil_div(H, 8) <= 65535) {
+        if (workspace_bytes < span_workspace_bytes(nnz, H) || (reinterpret_cast<uintptr_t>(workspace) & 15))
             return TANGO_ERR_WORKSPACE;
-        launch_tiers<true>(a, nullptr, nullptr, e, indptr, edge_ids, rows, static_cast<int>(H), slope, workspace,
-                           as_stream(stream));
+        launch_spans<true>(a, nullptr, nullptr, e, indptr, edge_ids, rows, nnz, static_cast<int>(H), slope,
+                           workspace, as_stream(stream));
         return launch_status();
     }
     hipLaunchKernelGGL(edge_softmax_fwd_kernel, dim3(grid_for(rows * H, 256, 16)), dim3(256), 0,
@@ -554,16 +541,16 @@ int tango_edge_softmax_fwd(float* a, const float* e, const int64_t* indptr,
 }
 
 int tango_edge_softmax_bwd(float* de, const float* a, const float* da, const float* e,
-                           const int64_t* indptr, const int64_t* edge_ids, int64_t rows,
+                           const int64_t* indptr, const int64_t* edge_ids, int64_t rows, int64_t nnz,
                            int64_t H, float slope, void* workspace, size_t workspace_bytes,
                            tango_stream_t stream) {
-    if (rows < 0 || H < 0 || (rows > 0 && !indptr) || H >= (1LL << 31)) return TANGO_ERR_INVALID_ARG;
-    if (rows * H == 0) return TANGO_OK;
+    if (rows < 0 || nnz < 0 || H < 0 || (rows > 0 && !indptr) || H >= (1LL << 31)) return TANGO_ERR_INVALID_ARG;
+    if (rows * H == 0 || nnz == 0) return TANGO_OK;
     if (!de || !a || !da || !e) return TANGO_ERR_INVALID_ARG;
-    if (H <= 64 && rows * H <= 256LL * INT32_MAX) {
-        if (workspace && (workspace_bytes < hub_workspace_bytes(H) || (reinterpret_cast<uintptr_t>(workspace) & 15)))
+    if (workspace && ceil_div(nnz, 4 * kSpan) <= INT32_MAX && ceil_div(H, 8) <= 65535) {
+        if (workspace_bytes < span_workspace_bytes(nnz, H) || (reinterpret_cast<uintptr_t>(workspace) & 15))
             return TANGO_ERR_WORKSPACE;
-        launch_tiers<false>(de, a, da, e, indptr, edge_ids, rows, static_cast<int>(H), slope, workspace,
+        launch_spans<false>(de, a, da, e, indptr, edge_ids, rows, nnz, static_cast<int>(H), slope, workspace,
                             as_stream(stream));
         return launch_status();
     }

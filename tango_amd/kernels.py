@@ -488,10 +488,11 @@ class cuda_kernels:
         _need(indptr, torch.int64, "indptr")
         H = e.numel() // max(e.size(0), 1)
         a = torch.empty_like(e)
-        ws_bytes = _L.tango_edge_softmax_workspace(H)
+        ws_bytes = _L.tango_edge_softmax_workspace(e.size(0), H)
         ws = _workspace(ws_bytes, e.device)
         check(_L.tango_edge_softmax_fwd(_ptr(a), _ptr(e), indptr.data_ptr(), _ptr(edge_ids),
-                                        indptr.numel() - 1, H, float(slope), _ptr(ws), ws_bytes, _stream()),
+                                        indptr.numel() - 1, e.size(0), H, float(slope), _ptr(ws), ws_bytes,
+                                        _stream()),
               "edge_softmax")
         return a
 
@@ -502,11 +503,11 @@ class cuda_kernels:
         _need(e, torch.float32, "e")
         H = e.numel() // max(e.size(0), 1)
         de = torch.empty_like(e)
-        ws_bytes = _L.tango_edge_softmax_workspace(H)
+        ws_bytes = _L.tango_edge_softmax_workspace(e.size(0), H)
         ws = _workspace(ws_bytes, e.device)
         check(_L.tango_edge_softmax_bwd(_ptr(de), _ptr(a), _ptr(da), _ptr(e), indptr.data_ptr(),
-                                        _ptr(edge_ids), indptr.numel() - 1, H, float(slope), _ptr(ws), ws_bytes,
-                                        _stream()),
+                                        _ptr(edge_ids), indptr.numel() - 1, e.size(0), H, float(slope), _ptr(ws),
+                                        ws_bytes, _stream()),
               "edge_softmax_backward")
         return de
 

@@ -84,17 +84,18 @@ def test_unknown_op_raises(K):
         K.mySDDMM_int8(g, "add", z.float(), z, sc(1), sc(1), False)
 
 
-# (n, e): mostly medium rows, and mostly short rows with some destinations empty; both get hubs
+# (n, e): rows of some hundred slots, rows of a few slots with some destinations empty, and a
+# graph that is mostly one hub; every graph gets rows that spread over several wavefronts' spans
 @pytest.mark.parametrize("n,e", [(900, 40000), (6000, 30000), (500, 90000)])
-@pytest.mark.parametrize("H", [1, 3, 8, 64, 70])
+@pytest.mark.parametrize("H", [1, 3, 4, 8, 12, 64, 70])
 @pytest.mark.parametrize("slope", [1.0, 0.2])
 def test_edge_softmax(K, orc, H, slope, n, e):
     rng = np.random.default_rng(H)
     src, dst = rand_graph(rng, n, e)
     dst[:5000] = 3  # one high-degree destination
     if e > 60000:
-        dst[:40000] = 3  # a hub for every H: cut over many workgroups through the workspace
-    dst[5000:5300] = 7  # and one between the wavefront and workgroup thresholds for small H
+        dst[:40000] = 3  # a hub: 150 spans of one row
+    dst[5000:5300] = 7  # a row a little longer than one span
     g = make_graph(src, dst, n)
     o = orc.graph_formats(src, dst, n)
     x = (rng.standard_normal((e, H)) * 4).astype(np.float32)
@@ -105,4 +106,49 @@ def test_edge_softmax(K, orc, H, slope, n, e):
     da = rng.standard_normal((e, H)).astype(np.float32)
     de = K.cuda_kernels.edge_softmax_backward(a, dev(da), dev(x), ip, eid, slope)
     want_de = orc.edge_softmax_bwd(want, da, x, o["adj_csc"][0], o["adj_csc"][2], slope)
+    assert np.allclose(host(de), want_de, rtol=1e-4, atol=1e-6)
+
+
+@pytest.mark.parametrize("e", [1, 63, 256, 257, 1000, 20011])
+def test_edge_softmax_empty_runs(K, orc, e):
+    """Destinations only at both ends of the id range: thousands of empty rows in a row inside one
+    span, which the row-pointer window of a wavefront cannot hold."""
+    rng = np.random.default_rng(e)
+    n, H = 9000, 8
+    src = rng.integers(0, n, e).astype(np.int64)
+    dst = np.where(rng.random(e) < 0.5, rng.integers(0, 40, e), rng.integers(n - 40, n, e)).astype(np.int64)
+    g = make_graph(src, dst, n)
+    o = orc.graph_formats(src, dst, n)
+    x = (rng.standard_normal((e, H)) * 3).astype(np.float32)
+    ip, _, eid = g.adj_csc
+    a = K.cuda_kernels.edge_softmax_forward(dev(x), ip, eid, 0.2)
+    want = orc.edge_softmax_fwd(x, o["adj_csc"][0], o["adj_csc"][2], 0.2)
+    assert np.allclose(host(a), want, rtol=1e-5, atol=1e-6)
+    da = rng.standard_normal((e, H)).astype(np.float32)
+    de = K.cuda_kernels.edge_softmax_backward(a, dev(da), dev(x), ip, eid, 0.2)
+    want_de = orc.edge_softmax_bwd(want, da, x, o["adj_csc"][0], o["adj_csc"][2], 0.2)
+    assert np.allclose(host(de), want_de, rtol=1e-4, atol=1e-6)
+
+
+def test_edge_softmax_without_workspace(K, orc):
+    """workspace = NULL: the thread-per-(row, head) path of the C entry points."""
+    from tango_amd import _lib
+    rng = np.random.default_rng(5)
+    n, e, H = 300, 5000, 3
+    src, dst = rand_graph(rng, n, e)
+    g = make_graph(src, dst, n)
+    o = orc.graph_formats(src, dst, n)
+    x = dev((rng.standard_normal((e, H)) * 3).astype(np.float32))
+    ip, _, eid = g.adj_csc
+    a = torch.empty_like(x)
+    st = torch.cuda.current_stream().cuda_stream
+    assert _lib.lib().tango_edge_softmax_fwd(a.data_ptr(), x.data_ptr(), ip.data_ptr(), eid.data_ptr(), n, e, H, 0.2,
+                                             None, 0, st) == 0
+    want = orc.edge_softmax_fwd(host(x), o["adj_csc"][0], o["adj_csc"][2], 0.2)
+    assert np.allclose(host(a), want, rtol=1e-5, atol=1e-6)
+    da = dev(rng.standard_normal((e, H)).astype(np.float32))
+    de = torch.empty_like(x)
+    assert _lib.lib().tango_edge_softmax_bwd(de.data_ptr(), a.data_ptr(), da.data_ptr(), x.data_ptr(), ip.data_ptr(),
+                                             eid.data_ptr(), n, e, H, 0.2, None, 0, st) == 0
+    want_de = orc.edge_softmax_bwd(want, host(da), host(x), o["adj_csc"][0], o["adj_csc"][2], 0.2)
     assert np.allclose(host(de), want_de, rtol=1e-4, atol=1e-6)
