@@ -203,11 +203,15 @@ int tango_spmm_csr_copy_u(float* out, const int64_t* indptr, const int64_t* indi
    max_row_nnz: an upper bound of the longest row if the caller knows one (a graph
    object usually does), else 0; it only lets the library skip the launches that
    exist for hub rows when there is none.
-   workspace (tango_spmm_workspace(nnz) bytes, 16-byte aligned, contents arbitrary) or
-   NULL: with it, hub rows (thousands of slots and far above the average) are cut over
-   many workgroups whose int32 partial sums are added into the output row with integer
-   atomics, so the result is the same either way. */
-size_t tango_spmm_workspace(int64_t nnz);
+   workspace (tango_spmm_workspace(rows, nnz, F) bytes, 16-byte aligned, contents
+   arbitrary) or NULL.  With it, on graphs whose rows average fewer than 64 slots the
+   work is cut by slots (256 per wavefront) instead of rows, rows cut by such a boundary
+   leaving int32 partial rows in the workspace that a second launch adds up; on denser
+   graphs hub rows (thousands of slots and far above the average) are cut over many
+   workgroups whose int32 partial sums are added into the output row with integer
+   atomics.  Integer sums are exact in any order, so the result is the same either way.
+   W in the size query: bytes summed per gathered row (F here, H * F for u_mul_e). */
+size_t tango_spmm_workspace(int64_t rows, int64_t nnz, int64_t W);
 int tango_spmm_csr_copy_u_ex(float* out, const int64_t* indptr, const void* indices, int idx_bits,
                              const int8_t* feat, int64_t ldf, const float* scale,
                              const float* row_scale, const float* bias, int relu, int64_t rows,

@@ -106,6 +106,21 @@ __device__ __forceinline__ void transpose4x4(uint32_t r0, uint32_t r1, uint32_t 
     c[3] = __builtin_amdgcn_perm(t3, t1, 0x07060302u);
 }
 
+// largest r in [0, rows) with indptr[r] <= key (indptr[0] = 0 <= key): 64 probes per round
+__device__ __forceinline__ int64_t row_of_slot_wave(const int64_t* __restrict__ indptr, int64_t rows, int64_t key,
+                                                    int lane) {
+    int64_t lo = 0, hi = rows;  // the answer lies in [lo, hi)
+    while (hi - lo > 1) {
+        const int64_t step = (hi - lo + kWave - 1) >> 6;
+        const int64_t probe = lo + lane * step;
+        const bool ok = probe < hi && indptr[probe] <= key;
+        const int cnt = __popcll(__ballot(ok));  // lane 0 always holds
+        lo += (cnt - 1) * step;
+        hi = lo + step < hi ? lo + step : hi;
+    }
+    return lo;
+}
+
 // Sets a handful of 32-bit words.  Used instead of hipMemsetAsync so that a
 // caller may capture any entry point into a HIP graph.
 static __global__ void fill_u32_kernel(uint32_t* p, uint32_t v, int n) {

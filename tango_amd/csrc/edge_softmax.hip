@@ -122,21 +122,6 @@ __device__ __forceinline__ float seg_scan_add(float x, int lane, int lo) {
     return x;
 }
 
-// largest r in [0, rows) with indptr[r] <= key (indptr[0] = 0 <= key): 64 probes per round
-__device__ __forceinline__ int64_t row_of_slot_wave(const int64_t* __restrict__ indptr, int64_t rows, int64_t key,
-                                                    int lane) {
-    int64_t lo = 0, hi = rows;  // the answer lies in [lo, hi)
-    while (hi - lo > 1) {
-        const int64_t step = (hi - lo + kWave - 1) >> 6;
-        const int64_t probe = lo + lane * step;
-        const bool ok = probe < hi && indptr[probe] <= key;
-        const int cnt = __popcll(__ballot(ok));  // lane 0 always holds
-        lo += (cnt - 1) * step;
-        hi = lo + step < hi ? lo + step : hi;
-    }
-    return lo;
-}
-
 template <int HB, bool VEC>
 __device__ __forceinline__ void load_heads(float (&v)[HB], const float* __restrict__ p, int nh) {
     if (VEC && HB == 8) {

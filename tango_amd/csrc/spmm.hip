@@ -58,6 +58,8 @@ struct SpmmParams {
     void* hub_ws;      // caller's workspace for the hub path, or null (then no row counts as a hub)
     int64_t max_row;   // caller's upper bound of the longest row, 0 if unknown
     int64_t group_row; // sparse graphs: rows with at most this many slots are owned by a lane group
+    void* span_ws;     // sparse graphs: caller's workspace for the slot-span path, or null
+    int64_t span_wp;   // padded row width (int32 entries) of a partial row in span_ws
 };
 
 enum { KIND_COPY = 0, KIND_WEIGHTED = 1, KIND_COO = 2 };
@@ -634,6 +636,323 @@ __global__ __launch_bounds__(256) void spmm_hub_store_kernel(const SpmmParams p)
     }
 }
 
+// ---------------------------------------------------------------------------------------------
+// Sparse graphs, slot spans.  The tiers above need five launches whose tails run one after the
+// other; here the work is cut by CSR slots instead of rows.  Wavefront w owns slots
+// [256 w, 256 w + 256) whatever rows they belong to; lane group g (lpe lanes = one gathered row
+// piece) walks the K = 256 / groups consecutive slots [g K, g K + K) four at a time and keeps the
+// running int32 sums of the row it is in.  Row starts inside the span are bits of a 256-bit mask in
+// LDS, built from the row pointers that follow the span's first row (a 64-ary search finds that
+// row).  A row that starts and ends inside one group's slots is complete when the group reaches
+// its end.  Pieces of rows cut by a group boundary meet in an LDS accumulator (integer atomics,
+// exact in any order) owned by the group the row starts in; pieces of rows cut by the span boundary
+// go to the caller's workspace as int32 partial rows (at most two per span) and
+// spmm_span_fix_kernel adds them up, stores those rows and the rows without any slot.
+constexpr int kSpanSlots = 256;
+constexpr int kSpanWin = kSpanSlots + kWave;  // row pointers staged per span: 64 empty rows of slack
+
+struct SpanRowMeta {
+    int64_t tail_row;   // the row that starts in this span and runs on into the next, or -1
+    int64_t head_open;  // the span lies inside one row that began before it and runs on after it
+};
+__host__ __device__ inline size_t span_parts_offset(int64_t nspans) {
+    return (static_cast<size_t>(nspans) * sizeof(SpanRowMeta) + 255) & ~static_cast<size_t>(255);
+}
+// partial row `piece` (0 = head: began before the span, 1 = tail) of span w
+__device__ __forceinline__ int* span_part(const SpmmParams& p, int64_t nspans, int64_t w, int piece) {
+    return reinterpret_cast<int*>(static_cast<char*>(p.span_ws) + span_parts_offset(nspans)) +
+           (w * 2 + piece) * p.span_wp;
+}
+
+// blockDim.x = 256: four spans per workgroup, grid (ceil(spans / 4), column tiles);
+// dynamic LDS: span_lds_bytes().
+__host__ __device__ inline size_t span_wave_ints(int lpe_log2, int vec) {
+    // groups + 1 accumulator rows of one column tile; while the row structure is built the staged
+    // row pointers (kSpanWin int64) use the same space
+    const size_t acc = ((64 >> lpe_log2) + 1) * (static_cast<size_t>(vec) << lpe_log2);
+    const size_t win = static_cast<size_t>(kSpanWin) * 2;
+    return ((acc > win ? acc : win) + 1) & ~static_cast<size_t>(1);
+}
+static size_t span_lds_bytes(int lpe_log2, int vec) { return sizeof(int) * 4 * span_wave_ints(lpe_log2, vec); }
+
+template <int VEC, int KIND>
+__global__ __launch_bounds__(256) void spmm_span_kernel(const SpmmParams p) {
+    constexpr int U = 4;
+    extern __shared__ __align__(16) int dyn_lds[];
+    __shared__ int sidx_all[4][kSpanSlots];
+    __shared__ int seid_all[KIND == KIND_WEIGHTED ? 4 : 1][KIND == KIND_WEIGHTED ? kSpanSlots : 1];
+    __shared__ int rowof_all[4][kSpanSlots];
+    __shared__ unsigned maskw_all[4][12];
+    const int lane = lane_id();
+    const int wave = __builtin_amdgcn_readfirstlane(static_cast<int>(threadIdx.x) >> 6);
+    const int64_t nspans = (p.nnz + kSpanSlots - 1) / kSpanSlots;
+    const int64_t w = static_cast<int64_t>(blockIdx.x) * 4 + wave;
+    if (w >= nspans) return;  // the whole wavefront leaves; no workgroup barrier below
+    const LaneCols c = lane_cols<VEC, KIND>(p, lane);
+    const int tile_ints = c.lpe * VEC;
+    int* accbuf = dyn_lds + wave * span_wave_ints(p.lpe_log2, VEC);
+    int64_t* win = reinterpret_cast<int64_t*>(accbuf);  // only while the row structure is built
+    int* sidx = sidx_all[wave];
+    int* seid = seid_all[KIND == KIND_WEIGHTED ? wave : 0];
+    int* rowof = rowof_all[wave];
+    unsigned* maskw = maskw_all[wave];
+    const bool permuted = KIND == KIND_WEIGHTED && p.edge_ids;
+    const int64_t base = w * kSpanSlots;
+    const int endl = static_cast<int>(p.nnz - base < kSpanSlots ? p.nnz - base : kSpanSlots);
+    const int64_t end = base + endl;
+
+    // ---- row structure of the span
+    const int64_t r0 = row_of_slot_wave(p.indptr, p.rows, base, lane);
+    if (lane < 12) maskw[lane] = 0u;
+#pragma unroll
+    for (int u = 0; u < kSpanSlots / kWave; ++u) rowof[kWave * u + lane] = 0;
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll
+    for (int k = 0; k < kSpanWin / kWave; ++k) {
+        const int i = lane + kWave * k;
+        const int64_t r = r0 + i;
+        const int64_t pv = r <= p.rows ? p.indptr[r] : INT64_MAX;
+        win[i] = pv;
+        if (pv >= base && pv < end) {  // row r0 + i starts at slot pv; of several (empty rows), the last one owns the slot
+            const int sl = static_cast<int>(pv - base);
+            atomicOr(&maskw[sl >> 5], 1u << (sl & 31));
+            atomicMax(&rowof[sl], i);
+        }
+        if (pv == end) atomicOr(&maskw[8], 1u);  // a row ends exactly at the span's end
+    }
+    // the span's column indices (and edge ids): one coalesced pass
+#pragma unroll
+    for (int u = 0; u < kSpanSlots / kWave; ++u) {
+        const int sl = kWave * u + lane;
+        if (sl < endl) {
+            sidx[sl] = load_index<true>(p, p.indices, base + sl);
+            if (permuted) seid[sl] = load_index<true>(p, p.edge_ids, base + sl);
+        }
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    if (win[kSpanWin - 1] < end) {  // more than 64 empty rows inside the span: search the array per slot
+#pragma unroll
+        for (int u = 0; u < kSpanSlots / kWave; ++u) {
+            const int sl = kWave * u + lane;
+            if (sl < endl) {
+                const int64_t s = base + sl;
+                int64_t lo = r0, hi = p.rows;
+                while (hi - lo > 1) {
+                    const int64_t mid = lo + ((hi - lo) >> 1);
+                    if (p.indptr[mid] <= s) lo = mid; else hi = mid;
+                }
+                if (p.indptr[lo] == s) {
+                    atomicOr(&maskw[sl >> 5], 1u << (sl & 31));
+                    atomicMax(&rowof[sl], static_cast<int>(lo - r0));
+                }
+                if (sl == endl - 1 && p.indptr[lo + 1] == end) atomicOr(&maskw[8], 1u);
+            }
+        }
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    for (int i = lane; i < (c.epi + 1) * tile_ints; i += kWave) accbuf[i] = 0;  // the row pointers are done with
+    const bool last_open = (maskw[8] & 1u) == 0u;  // the row of the last slot runs on into the next span
+    // largest flagged slot < pos, or -1; smallest flagged slot >= pos, or kSpanSlots
+    auto prev_flag = [&](int pos) {
+        for (int wd = (pos - 1) >> 5; wd >= 0 && pos > 0; --wd) {
+            unsigned m = maskw[wd];
+            if (wd == ((pos - 1) >> 5)) m &= (2u << ((pos - 1) & 31)) - 1u;  // 2u << 31 wraps to 0: all bits kept
+            if (m) return wd * 32 + 31 - __builtin_clz(m);
+        }
+        return -1;
+    };
+    auto next_flag = [&](int pos) {
+        for (int wd = pos >> 5; wd < kSpanSlots / 32; ++wd) {
+            unsigned m = maskw[wd];
+            if (wd == (pos >> 5)) m &= ~((1u << (pos & 31)) - 1u);
+            if (m) return wd * 32 + __builtin_ctz(m);
+        }
+        return kSpanSlots;
+    };
+
+    // ---- the walk
+    const int K = kSpanSlots >> c.sh;  // slots per group: 4 * lpe
+    const int gbase = c.grp * K;
+    int acc[VEC];
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) acc[i] = 0;
+    bool have = false, started = false, tail_partial = false;
+    int cur_start = 0, my_last_flag = -1, first_target = -2;
+    // ends the piece the group is in
+    auto flush = [&](bool closed) {
+        if (started && closed) {
+            store_row<VEC>(p, c, r0 + rowof[cur_start], acc);
+        } else {
+            int target = c.grp;
+            if (!started) {
+                if (first_target == -2) {
+                    const int pf = prev_flag(gbase);
+                    first_target = pf < 0 ? c.epi : pf / K;
+                }
+                target = first_target;
+            } else {
+                tail_partial = true;
+            }
+            int* ab = accbuf + target * tile_ints + c.sub * VEC;
+#pragma unroll
+            for (int i = 0; i < VEC; ++i) atomicAdd(&ab[i], acc[i]);
+        }
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) acc[i] = 0;
+        have = false;
+    };
+    auto issue = [&](typename Gather<VEC>::T* d, uint32_t& m, int q) {
+        m = 0u;
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const int slot = gbase + q + u;
+            const bool ok = slot < endl;
+            const int sl = ok ? slot : 0;  // slot 0 exists; its multiplier is 0 here
+            d[u] = Gather<VEC>::load(c.fcol + row_offset(sidx[sl], p));
+            uint32_t wv = 1u;
+            if (KIND == KIND_WEIGHTED) {
+                const int64_t pos = permuted ? static_cast<int64_t>(seid[sl]) : base + sl;
+                wv = static_cast<uint32_t>(static_cast<uint8_t>(c.wbase[pos * p.ev_se]));
+            }
+            m |= (ok ? wv : 0u) << (8 * u);
+        }
+    };
+    auto consume = [&](const typename Gather<VEC>::T* d, uint32_t m, int q) {
+        const int slot0 = gbase + q;
+        if (slot0 >= endl) return;
+        const unsigned bits = (maskw[slot0 >> 5] >> (slot0 & 31)) & 0xFu;
+        int pos = 0;
+        while (pos < 4) {  // one pass per row that has slots in this batch
+            if ((bits >> pos) & 1u) {
+                if (have) flush(true);
+                started = true;
+                cur_start = slot0 + pos;
+                my_last_flag = cur_start;
+            }
+            const unsigned rest = bits >> (pos + 1);
+            const int nxt = rest ? pos + 1 + __builtin_ctz(rest) : 4;
+            const uint32_t upto = nxt == 4 ? 0xFFFFFFFFu : ((1u << (8 * nxt)) - 1u);
+            accumulate4<VEC>(acc, d, m & upto & ~((1u << (8 * pos)) - 1u));
+            if (slot0 + pos < endl) have = true;
+            pos = nxt;
+        }
+    };
+    {
+        typename Gather<VEC>::T da[U], db[U];
+        uint32_t ma = 0u, mb = 0u;
+        issue(da, ma, 0);
+        for (int q = 0; q < K; q += 2 * U) {  // two batches in flight
+            const bool has_b = q + U < K;
+            if (has_b) issue(db, mb, q + U);
+            consume(da, ma, q);
+            if (q + 2 * U < K) issue(da, ma, q + 2 * U);
+            if (has_b) consume(db, mb, q + U);
+        }
+    }
+    if (have) {
+        const int e = gbase + K;
+        flush(e >= endl ? !last_open : ((maskw[e >> 5] >> (e & 31)) & 1u) != 0u);
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+
+    // ---- rows cut by a group boundary: the group a row starts in finishes it
+    if (tail_partial) {
+        const int e = gbase + K;
+        const bool closed = e >= endl ? !last_open : (next_flag(e) < endl || !last_open);
+        const int* ab = accbuf + c.grp * tile_ints + c.sub * VEC;
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) acc[i] = ab[i];
+        if (closed) {
+            store_row<VEC>(p, c, r0 + rowof[my_last_flag], acc);
+        } else {
+            int* part = span_part(p, nspans, w, 1) + c.col;
+#pragma unroll
+            for (int i = 0; i < VEC; ++i) part[i] = acc[i];
+        }
+    }
+    const bool head = (maskw[0] & 1u) == 0u;  // the first slot's row began before the span
+    if (c.grp == 0 && head) {
+        const int* ab = accbuf + c.epi * tile_ints + c.sub * VEC;
+        int* part = span_part(p, nspans, w, 0) + c.col;
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) part[i] = ab[i];
+    }
+    if (lane == 0 && blockIdx.y == 0) {
+        const int lf = prev_flag(kSpanSlots);
+        SpanRowMeta* meta = static_cast<SpanRowMeta*>(p.span_ws) + w;
+        meta->tail_row = (last_open && lf >= 0) ? r0 + rowof[lf] : -1;
+        meta->head_open = (last_open && lf < 0) ? 1 : 0;
+    }
+}
+
+// Adds up the pieces of every row cut by a span boundary (the tail piece of the span it starts in,
+// then the head pieces of the following spans) and stores the row; also stores the rows that have
+// no slot at all.  Launched like spmm_span_kernel, without dynamic LDS.
+template <int VEC>
+__global__ __launch_bounds__(256) void spmm_span_fix_kernel(const SpmmParams p) {
+    const int lane = lane_id();
+    const int wave = __builtin_amdgcn_readfirstlane(static_cast<int>(threadIdx.x) >> 6);
+    const int64_t nspans = (p.nnz + kSpanSlots - 1) / kSpanSlots;
+    const int64_t w = static_cast<int64_t>(blockIdx.x) * 4 + wave;
+    const LaneCols c = lane_cols<VEC, KIND_COPY>(p, lane);
+    const SpanRowMeta* meta = static_cast<const SpanRowMeta*>(p.span_ws);
+    if (w < nspans && meta[w].tail_row >= 0) {
+        int64_t last = w + 1;  // the first following span whose head piece ends its row
+        for (;; last += kWave) {
+            const int64_t j = last + lane;
+            const uint64_t m = __ballot(j >= nspans || meta[j].head_open == 0);
+            if (m) {
+                last += __builtin_ctzll(m);
+                break;
+            }
+        }
+        if (last >= nspans) last = nspans - 1;
+        int acc[VEC];
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) acc[i] = 0;
+        if (c.grp == 0) {
+            const int* part = span_part(p, nspans, w, 1) + c.col;
+#pragma unroll
+            for (int i = 0; i < VEC; ++i) acc[i] = part[i];
+        }
+        for (int64_t j = w + 1 + c.grp; j <= last; j += c.epi) {
+            const int* part = span_part(p, nspans, j, 0) + c.col;
+#pragma unroll
+            for (int i = 0; i < VEC; ++i) acc[i] += part[i];
+        }
+        for (int off = c.lpe; off < kWave; off <<= 1) {
+#pragma unroll
+            for (int i = 0; i < VEC; ++i) acc[i] += __shfl_xor(acc[i], off, kWave);
+        }
+        if (c.grp == 0) store_row<VEC>(p, c, meta[w].tail_row, acc);
+    }
+    // rows without slots: out = epilogue(0)
+    const int64_t nwaves = static_cast<int64_t>(gridDim.x) * 4;
+    for (int64_t rb = (static_cast<int64_t>(blockIdx.x) * 4 + wave) * kWave; rb < p.rows; rb += nwaves * kWave) {
+        const int64_t r = rb + lane;
+        uint64_t m = __ballot(r < p.rows && p.indptr[r] == p.indptr[r + 1]);
+        int zero[VEC];
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) zero[i] = 0;
+        while (m) {
+            const int b = __builtin_ctzll(m);
+            m &= m - 1;
+            if (c.grp == 0) store_row<VEC>(p, c, rb + b, zero);
+        }
+    }
+}
+
+// graphs whose rows average fewer than 64 slots take the slot-span path (given a workspace)
+static bool span_graph(int64_t rows, int64_t nnz) { return nnz < 64 * rows; }
+
 static int ilog2_ceil(int64_t v) {
     int l = 0;
     while ((1LL << l) < v) ++l;
@@ -691,6 +1010,22 @@ static int launch_spmm(SpmmParams p, int vec, hipStream_t s) {
             hipLaunchKernelGGL((spmm_hub_store_kernel<V, KIND>), sgrid, dim3(256), 0, s, p);        \
         }                                                                                           \
     } while (0)
+    if (KIND != KIND_COO && p.span_ws && span_graph(p.rows, p.nnz)) {  // sparse graph: slot spans, two launches
+        const int64_t nspans = ceil_div(p.nnz, kSpanSlots);
+        p.span_wp = ychunks * p.tile;
+        const dim3 spgrid(static_cast<unsigned>(ceil_div(nspans > 0 ? nspans : 1, 4)), static_cast<unsigned>(ychunks));
+        const size_t lds = span_lds_bytes(p.lpe_log2, vec);
+#define TANGO_SPMM_SPANS(V)                                                                      \
+    do {                                                                                         \
+        if (nspans > 0) hipLaunchKernelGGL((spmm_span_kernel<V, KIND>), spgrid, dim3(256), lds, s, p); \
+        hipLaunchKernelGGL(spmm_span_fix_kernel<V>, spgrid, dim3(256), 0, s, p);                 \
+    } while (0)
+        if (vec == 16) TANGO_SPMM_SPANS(16);
+        else if (vec == 4) TANGO_SPMM_SPANS(4);
+        else TANGO_SPMM_SPANS(1);
+#undef TANGO_SPMM_SPANS
+        return launch_status();
+    }
     if (longest > p.long_row) {
         if (vec == 16) TANGO_SPMM_LONG(16);
         else if (vec == 4) TANGO_SPMM_LONG(4);
@@ -742,8 +1077,12 @@ using namespace tango;
 
 extern "C" {
 
-size_t tango_spmm_workspace(int64_t nnz) {
-    if (nnz < 0) return 0;
+size_t tango_spmm_workspace(int64_t rows, int64_t nnz, int64_t W) {
+    if (rows < 0 || nnz < 0 || W < 0) return 0;
+    if (span_graph(rows, nnz)) {  // two int32 partial rows per span; the padded width is at most 2 W + 1024
+        const int64_t nspans = ceil_div(nnz, kSpanSlots);
+        return span_parts_offset(nspans) + sizeof(int) * 2 * static_cast<size_t>(nspans) * static_cast<size_t>(2 * W + 1024);
+    }
     return 64 + sizeof(int64_t) * static_cast<size_t>(nnz / kHubRowMin + 2);
 }
 
@@ -768,13 +1107,14 @@ int tango_spmm_csr_copy_u_ex(float* out, const int64_t* indptr, const void* indi
     if (rows < 0 || F < 0 || nnz < 0 || num_src < 0 || ldf < F || !scale || !indptr || max_row_nnz < 0 ||
         (rows * F > 0 && !out) || (nnz > 0 && (!indices || !feat)) || (idx_bits != 32 && idx_bits != 64))
         return TANGO_ERR_INVALID_ARG;
-    if (workspace && (workspace_bytes < tango_spmm_workspace(nnz) || (reinterpret_cast<uintptr_t>(workspace) & 15)))
+    if (workspace && (workspace_bytes < tango_spmm_workspace(rows, nnz, F) || (reinterpret_cast<uintptr_t>(workspace) & 15)))
         return TANGO_ERR_WORKSPACE;
     if (num_src >= (1LL << 31) || nnz >= (1LL << 31)) return TANGO_ERR_UNSUPPORTED;
     SpmmParams p{};
     p.out = out; p.indptr = indptr; p.indices = static_cast<const int64_t*>(indices); p.idx32 = idx_bits == 32;
     p.feat = feat; p.scale = scale;
     p.row_scale = row_scale; p.bias = bias; p.relu = relu ? 1 : 0; p.max_row = max_row_nnz; p.hub_ws = workspace;
+    p.span_ws = workspace;
     p.rows = rows; p.num_src = num_src; p.ldf = ldf; p.W = F; p.F = F; p.D = 1; p.nnz = nnz;
     return launch_spmm<KIND_COPY>(p, pick_vec(feat, ldf, F), as_stream(stream));
 }
@@ -789,14 +1129,14 @@ int tango_spmm_csr_u_mul_e_ex(float* out, const int64_t* indptr, const void* ind
         (rows * H * F > 0 && !out) || (nnz > 0 && (!indices || !feat || !evals)) ||
         (idx_bits != 32 && idx_bits != 64))
         return TANGO_ERR_INVALID_ARG;
-    if (workspace && (workspace_bytes < tango_spmm_workspace(nnz) || (reinterpret_cast<uintptr_t>(workspace) & 15)))
+    if (workspace && (workspace_bytes < tango_spmm_workspace(rows, nnz, H * F) || (reinterpret_cast<uintptr_t>(workspace) & 15)))
         return TANGO_ERR_WORKSPACE;
     if (D != 1 && D != F) return TANGO_ERR_UNSUPPORTED;
     if (num_src >= (1LL << 31) || nnz >= (1LL << 31)) return TANGO_ERR_UNSUPPORTED;
     SpmmParams p{};
     p.out = out; p.indptr = indptr; p.indices = static_cast<const int64_t*>(indices);
     p.edge_ids = static_cast<const int64_t*>(edge_ids); p.idx32 = idx_bits == 32; p.feat = feat;
-    p.max_row = max_row_nnz; p.hub_ws = workspace;
+    p.max_row = max_row_nnz; p.hub_ws = workspace; p.span_ws = workspace;
     p.evals = evals; p.scale = scale; p.bias = bias; p.rows = rows; p.num_src = num_src; p.ldf = H * F; p.W = H * F; p.F = F; p.D = D;
     p.nnz = nnz;
     if (edge_major) {  // evals[nnz, H, D]: the H * D bytes of one edge share a cache sector

@@ -380,7 +380,7 @@ class cuda_kernels:
             _need(bias, torch.float32, "bias")
             if bias.numel() != F:
                 raise RuntimeError("csr_SPMM: bias must have F entries")
-        ws_bytes = _L.tango_spmm_workspace(indices.numel())
+        ws_bytes = _L.tango_spmm_workspace(rows, indices.numel(), F)
         ws = _workspace(ws_bytes, U.device)
         check(_L.tango_spmm_csr_copy_u_ex(_ptr(out), indptr.data_ptr(), _ptr(indices), idx_bits, _ptr(U), ldf,
                                           scaleU.data_ptr(), _ptr(row_scale), _ptr(bias), int(bool(relu)),
@@ -418,7 +418,7 @@ class cuda_kernels:
                 raise RuntimeError("multi_cusparse_SPMM: bias must have H * F elements")
         rows = indptr.numel() - 1
         out = torch.empty((rows, H, F), dtype=torch.float32, device=N.device)
-        ws_bytes = _L.tango_spmm_workspace(nnz)
+        ws_bytes = _L.tango_spmm_workspace(rows, nnz, H * F)
         ws = _workspace(ws_bytes, N.device)
         check(_L.tango_spmm_csr_u_mul_e_ex(_ptr(out), indptr.data_ptr(), _ptr(indices), _ptr(edge_ids), idx_bits,
                                            _ptr(N), _ptr(E_T), int(bool(edge_major)), scale.data_ptr(),

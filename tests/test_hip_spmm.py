@@ -156,3 +156,47 @@ def test_incidence_spmm(K, orc, kind, n, e, F):
     assert torch.equal(out, K.incidence_SPMM(g, dev(E), sc(s)))
     E3 = dev(E).view(e, F, 1) if F > 1 else dev(E)
     assert tuple(K.incidence_SPMM(g, E3, sc(s)).shape) == (n,) + tuple(E3.shape[1:])
+
+
+@pytest.mark.parametrize("e", [1, 5, 255, 256, 257, 3000, 40011])
+@pytest.mark.parametrize("F", [16, 40, 128])
+def test_spmm_slot_spans_with_empty_row_runs(K, orc, e, F):
+    """Sparse graphs are cut by slots, 256 per wavefront.  Destinations only at both ends of the id
+    range leave thousands of empty rows in a row inside one span (more than the staged row pointers
+    cover), rows without slots before the first and after the last edge, and spans cut mid-row."""
+    rng = np.random.default_rng(e + F)
+    n = 9000
+    src = rng.integers(0, n, e).astype(np.int64)
+    dst = np.where(rng.random(e) < 0.5, rng.integers(5, 40, e), rng.integers(n - 40, n - 3, e)).astype(np.int64)
+    g = make_graph(src, dst, n)
+    o = orc.graph_formats(src, dst, n)
+    feat = rng.integers(-127, 128, (n, F)).astype(np.int8)
+    s = np.float32(0.031)
+    got = K.csr_SPMM(g, dev(feat), sc(s))
+    assert np.array_equal(host(got), orc.spmm_csr_copy_u(o["adj_csc"][0], o["adj_csc"][1], feat, s))
+    H = 4 if F % 4 == 0 else 1
+    f3 = feat.reshape(n, H, F // H)
+    ev = rng.integers(-127, 128, (e, H, 1)).astype(np.int8)
+    got = K.multi_cusparse_SPMM(g, dev(f3), dev(ev), sc(s), edge_major=True)
+    want = orc.spmm_csr_u_mul_e(*o["adj_csc"], f3, np.ascontiguousarray(ev.transpose(1, 2, 0)), s)
+    assert np.array_equal(host(got), want)
+
+
+@pytest.mark.parametrize("kind,n,e", [GRAPHS[0], GRAPHS[3]])
+@pytest.mark.parametrize("F", [16, 100, 256])
+def test_spmm_without_workspace(K, orc, kind, n, e, F):
+    """workspace = NULL through the C entry point: sparse graphs then go by in-degree tiers
+    (lane group, wavefront, sixteen wavefronts per row)."""
+    from tango_amd import _lib
+    rng = np.random.default_rng(F + n)
+    src, dst = powerlaw_graph(rng, n, e) if kind == "hubs" else rand_graph(rng, n, e)
+    g = make_graph(src, dst, n)
+    o = orc.graph_formats(src, dst, n)
+    feat = dev(rng.integers(-127, 128, (n, F)).astype(np.int8))
+    ip, ix, _ = g.adj_csc
+    out = torch.empty((n, F), dtype=torch.float32, device="cuda")
+    s = sc(0.25)
+    st = torch.cuda.current_stream().cuda_stream
+    assert _lib.lib().tango_spmm_csr_copy_u_ex(out.data_ptr(), ip.data_ptr(), ix.data_ptr(), 64, feat.data_ptr(), F,
+                                               s.data_ptr(), None, None, 0, n, n, e, F, 0, None, 0, st) == 0
+    assert np.array_equal(host(out), orc.spmm_csr_copy_u(o["adj_csc"][0], o["adj_csc"][1], host(feat), 0.25))
