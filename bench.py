@@ -196,7 +196,9 @@ def _gat_step(K, torch, iters, warm):
     from tango_amd.graph import chung_lu
     from tango_amd.loss import cross_entropy
     from tango_amd.util import graph_preprocess
-    g = graph_preprocess(chung_lu(169343, 1166243, 2.2, seed=4, device="cuda"))
+    # edges numbered in destination-major order: the [E, H] tensors of the attention layers are then
+    # walked front to back (node outputs do not depend on the numbering)
+    g = graph_preprocess(chung_lu(169343, 1166243, 2.2, seed=4, device="cuda").reorder_edges_by_dst())
     n = g.num_nodes()
     model = GAT(g, 3, 128, 16, 40, [8, 8, 1], torch.nn.functional.elu).cuda()
     x = torch.randn(n, 128, device="cuda")
@@ -216,7 +218,7 @@ def _hgt_step(K, torch, iters, warm):
     from tango_amd.loss import cross_entropy
     from tango_amd.util import graph_preprocess
     g, _, _ = hetero_power_law(device="cuda")
-    g = graph_preprocess(g)
+    g = graph_preprocess(g.reorder_edges_by_dst())
     n = g.num_nodes()
     hgt = HGTStack(256, 256, 16, 4, n_layers=2).cuda()
     xh = torch.randn(n, 256, device="cuda")

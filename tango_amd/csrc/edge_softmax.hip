@@ -70,20 +70,21 @@ __global__ __launch_bounds__(256) void edge_softmax_bwd_kernel(
 }
 
 // ---------------------------------------------------------------------------------------------
-// Span kernels.  Wavefront w owns slots [w * kSpan, (w + 1) * kSpan), lane l of step u holds slot
-// base + 64 u + l with HB heads of it (head block blockIdx.y).  Per step, a segmented scan over
-// the lanes (segments = rows) gives every lane its row's (max, sum of exp) within the step; rows
-// running over a step boundary chain through a wave-uniform carry, and the lanes of their earlier
-// steps pick the finished result up from `fin`.  Three kinds of row:
+// Span kernels.  Wavefront w owns SPAN consecutive slots (64 to 256, by the number of heads a
+// wavefront covers).  The lanes are (group g, head h) pairs, HB heads (head block blockIdx.y) by
+// G = 64 / HB groups, and a lane holds the K consecutive slots [g K, g K + K) of its head in
+// registers: a row's reduction is a serial sweep over the lane's own values, and only one
+// aggregate per lane crosses lanes (a segmented scan over the G groups, then one fetch from the
+// group the row ends in): about 1.5 cross-lane steps per value instead of the 14 a lane-per-slot
+// layout needs.  Row starts are the bits of a mask in LDS, built from the row pointers that
+// follow the span's first row (a 64-ary search finds that row).  Three kinds of row:
 //   inside : starts and ends within the span -> written by this launch;
 //   head   : started in an earlier span      -> partial result in piece 0 of the span's record;
 //   tail   : runs on into the next span      -> partial result in piece 1.
 // span_fix_kernel merges a row's pieces (the tail of the span it starts in and the heads of the
 // spans that follow) and stores the row's result back into every piece; span_rest_kernel then
-// writes the head and tail slots.  No atomics: results do not depend on scheduling.
-constexpr int kSteps = 4;
-constexpr int kSpan = kWave * kSteps;
-constexpr int kWin = kSpan + kWave;  // row pointers staged per wavefront: 64 empty rows of slack
+// writes the head and tail slots.  No atomics on results: they do not depend on scheduling.
+constexpr int kWin = 256 + kWave;  // row pointers inspected per span: 64 empty rows of slack
 
 struct SpanMeta {
     int64_t head_end;    // slots [base, head_end) belong to a row that started before the span
@@ -98,28 +99,6 @@ __host__ __device__ inline size_t span_vals_offset(int64_t nspans) {
 __device__ __forceinline__ float* span_vals(void* ws, int64_t nspans, int64_t w, int piece, int comp, int H) {
     return reinterpret_cast<float*>(static_cast<char*>(ws) + span_vals_offset(nspans)) +
            ((w * 2 + piece) * 2 + comp) * static_cast<int64_t>(H);
-}
-
-__device__ __forceinline__ float rl_f(float v, int l) {
-    return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), l));
-}
-
-// inclusive scans over lanes [lo, lane] (lo = first lane of this lane's segment)
-__device__ __forceinline__ float seg_scan_max(float x, int lane, int lo) {
-#pragma unroll
-    for (int off = 1; off < kWave; off <<= 1) {
-        const float t = __shfl_up(x, off, kWave);
-        if (lane - off >= lo) x = fmaxf(x, t);
-    }
-    return x;
-}
-__device__ __forceinline__ float seg_scan_add(float x, int lane, int lo) {
-#pragma unroll
-    for (int off = 1; off < kWave; off <<= 1) {
-        const float t = __shfl_up(x, off, kWave);
-        if (lane - off >= lo) x += t;
-    }
-    return x;
 }
 
 template <int HB, bool VEC>
@@ -156,207 +135,239 @@ __device__ __forceinline__ void store_heads(float* __restrict__ p, const float (
     }
 }
 
+// Where a row's aggregate comes from, per lane: everything the cross-group step needs.
+struct GroupLinks {
+    int g;        // my group
+    int seg0;     // first group of the run of groups my last segment's row spans so far (scan bound)
+    int next;     // lane (same head) of the next group that holds a row start, or -1
+    int last;     // lane (same head) of the last group with slots of this span
+};
+
+// F = aggregate of my slots before my first row start (all of them if I have none), L = of my slots
+// from my last row start on.  Returns TF = the whole (within the span) of the row that ends at my
+// first row start and X = of the row my last slots belong to.
+template <int HB, bool MAX>
+__device__ __forceinline__ void cross_groups(float F, float L, const GroupLinks& k, float& TF, float& X) {
+    constexpr int G = kWave / HB;
+    float S = L;  // inclusive scan over the groups back to the one my row starts in
+#pragma unroll
+    for (int d = 1; d < G; d <<= 1) {
+        const float t = __shfl_up(S, d * HB, kWave);
+        if (k.g - d >= k.seg0) S = MAX ? fmaxf(S, t) : S + t;
+    }
+    float PF = __shfl_up(S, HB, kWave);
+    if (k.g == 0) PF = MAX ? -INFINITY : 0.0f;
+    TF = MAX ? fmaxf(PF, F) : PF + F;
+    const float xn = __shfl(TF, k.next < 0 ? 0 : k.next, kWave);
+    const float xe = __shfl(S, k.last, kWave);
+    X = k.next < 0 ? xe : xn;
+}
+
+// In-lane pass over the lane's K values: v[] becomes, slot by slot, the aggregate of the slot's
+// row within the span.  `sub` has bit k set when slot k starts a row.
+template <int HB, int K, bool MAX>
+__device__ __forceinline__ void row_aggregates(float (&v)[K], unsigned sub, const GroupLinks& lk, float& TF, float& X) {
+    const float ident = MAX ? -INFINITY : 0.0f;
+    float run = ident, F = ident;
+    bool seen = false;
+#pragma unroll
+    for (int k = 0; k < K; ++k) {
+        if ((sub >> k) & 1u) {
+            if (!seen) F = run;
+            seen = true;
+            run = ident;
+        }
+        run = MAX ? fmaxf(run, v[k]) : run + v[k];
+        v[k] = run;  // prefix within the row's slots of this lane
+    }
+    if (!seen) F = run;
+    cross_groups<HB, MAX>(F, run, lk, TF, X);
+    // backwards: the last slots take X, rows inside the lane their own prefix at their last slot, the first slots TF
+    const int kf = sub ? __builtin_ctz(sub) : K;
+    float cur = X;
+#pragma unroll
+    for (int k = K - 1; k >= 0; --k) {
+        const float prev = k > 0 ? v[k - 1] : ident;
+        v[k] = cur;
+        if ((sub >> k) & 1u) cur = (k == kf) ? TF : prev;
+    }
+}
+
 // blockDim.x = 256 (four spans per workgroup), grid = (ceil(nspans / 4), ceil(H / HB)).
-// VEC: H is a multiple of HB, so the HB heads of an edge are one aligned vector.
-template <int HB, bool VEC, bool FWD>
+template <int HB, int K, bool FWD>
 __global__ __launch_bounds__(256) void span_kernel(
     float* __restrict__ out, const float* __restrict__ a, const float* __restrict__ da,
     const float* __restrict__ e, const int64_t* __restrict__ indptr, const int64_t* __restrict__ eids,
     int64_t rows, int64_t nnz, int H, float slope, void* __restrict__ ws) {
-    __shared__ int64_t win_all[4][kWin];
+    constexpr int G = kWave / HB;
+    constexpr int SPAN = G * K;
+    static_assert(SPAN <= 256 && (32 % K) == 0, "a lane's row-start bits must sit in one mask word");
+    __shared__ unsigned maskw_all[4][12];
     const int lane = lane_id();
     const int wave = static_cast<int>(threadIdx.x) >> 6;
-    const int64_t nspans = (nnz + kSpan - 1) / kSpan;
+    const int64_t nspans = (nnz + SPAN - 1) / SPAN;
     const int64_t w = static_cast<int64_t>(blockIdx.x) * 4 + wave;
     if (w >= nspans) return;  // the whole wavefront leaves; no workgroup barrier below
-    int64_t* win = win_all[wave];
+    unsigned* maskw = maskw_all[wave];
+    const int g = lane / HB, h = lane % HB;
     const int h0 = static_cast<int>(blockIdx.y) * HB;
-    const int nh = H - h0 < HB ? H - h0 : HB;
-    const int64_t base = w * kSpan;
-    const int endl = static_cast<int>((nnz - base < kSpan) ? nnz - base : kSpan);  // slots in this span
+    const bool hok = h0 + h < H;
+    const int64_t base = w * SPAN;
+    const int endl = static_cast<int>((nnz - base < SPAN) ? nnz - base : SPAN);  // slots in this span
     const int64_t end = base + endl;
 
-    // ---- which row does each of my slots belong to
-    const int64_t r0 = row_of_slot_wave(indptr, rows, base, lane);
+    // ---- values first: their loads are in flight while the row structure is worked out
+    int64_t id[K];
+    float x[K], y[K];
 #pragma unroll
-    for (int k = 0; k < kWin / kWave; ++k) {
-        const int64_t r = r0 + lane + kWave * k;
-        win[lane + kWave * k] = r <= rows ? indptr[r] : INT64_MAX;
+    for (int k = 0; k < K; ++k) {
+        const int j = g * K + k;
+        id[k] = -1;
+        x[k] = FWD ? -INFINITY : 0.0f;
+        y[k] = 0.0f;
+        if (j < endl && hok) {
+            id[k] = (eids ? eids[base + j] : base + j) * H + h0 + h;
+            if (FWD) {
+                x[k] = leaky(e[id[k]], slope);
+            } else {
+                x[k] = a[id[k]];
+                y[k] = da[id[k]];
+            }
+        }
     }
+
+    // ---- row starts inside the span
+    const int64_t r0 = row_of_slot_wave(indptr, rows, base, lane);
+    if (lane < 12) maskw[lane] = 0u;
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-    const bool staged = win[kWin - 1] >= end;  // every row of the span has both pointers in the window
-    int rsl[kSteps], rel[kSteps];  // my row's first slot and end slot relative to base: -1 = before, kSpan + 1 = after
+    bool covered = false;  // the inspected row pointers reach the span's end
 #pragma unroll
-    for (int u = 0; u < kSteps; ++u) {
-        int64_t s = base + kWave * u + lane;
-        s = s < end ? s : end - 1;
-        int64_t rs, re;
-        if (staged) {
-            int pos = 0;
-#pragma unroll
-            for (int step = 256; step > 0; step >>= 1)
-                if (pos + step < kWin && win[pos + step] <= s) pos += step;
-            rs = win[pos];
-            re = win[pos + 1];
-        } else {  // a long run of empty rows inside the span: search the array itself
+    for (int k = 0; k < kWin / kWave; ++k) {
+        const int64_t r = r0 + lane + kWave * k;
+        const int64_t pv = r <= rows ? indptr[r] : INT64_MAX;
+        if (pv >= base && pv < end) {
+            const int sl = static_cast<int>(pv - base);
+            atomicOr(&maskw[sl >> 5], 1u << (sl & 31));
+        }
+        if (pv == end) atomicOr(&maskw[8], 1u);  // a row ends exactly at the span's end
+        if (k == kWin / kWave - 1) covered = __builtin_amdgcn_readlane(static_cast<int>(pv >= end), kWave - 1) != 0;
+    }
+    if (!covered) {  // more than 64 empty rows inside the span: search the array per slot
+        for (int sl = lane; sl < endl; sl += kWave) {
+            const int64_t s = base + sl;
             int64_t lo = r0, hi = rows;
             while (hi - lo > 1) {
                 const int64_t mid = lo + ((hi - lo) >> 1);
                 if (indptr[mid] <= s) lo = mid; else hi = mid;
             }
-            rs = indptr[lo];
-            re = indptr[lo + 1];
-        }
-        rsl[u] = rs < base ? -1 : static_cast<int>(rs - base);
-        rel[u] = re > end ? kSpan + 1 : static_cast<int>(re - base);
-    }
-
-    // ---- values
-    int64_t id[kSteps];
-    float x[kSteps][HB];   // forward: leaky(e); backward: a
-    float y[kSteps][HB];   // backward: da
-#pragma unroll
-    for (int u = 0; u < kSteps; ++u) {
-        const int64_t s = base + kWave * u + lane;
-        const bool valid = kWave * u + lane < endl;
-        id[u] = -1;
-#pragma unroll
-        for (int i = 0; i < HB; ++i) x[u][i] = FWD ? -INFINITY : 0.0f, y[u][i] = 0.0f;
-        if (valid) {
-            id[u] = (eids ? eids[s] : s) * H + h0;
-            if (FWD) {
-                load_heads<HB, VEC>(x[u], e + id[u], nh);
-#pragma unroll
-                for (int i = 0; i < HB; ++i) x[u][i] = leaky(x[u][i], slope);
-            } else {
-                load_heads<HB, VEC>(x[u], a + id[u], nh);
-                load_heads<HB, VEC>(y[u], da + id[u], nh);
-            }
+            if (indptr[lo] == s) atomicOr(&maskw[sl >> 5], 1u << (sl & 31));
+            if (sl == endl - 1 && indptr[lo + 1] == end) atomicOr(&maskw[8], 1u);
         }
     }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    const unsigned sub = (maskw[(g * K) >> 5] >> ((g * K) & 31)) & ((1u << K) - 1u);
+    const bool last_open = (maskw[8] & 1u) == 0u;  // the row of the last slot runs on into the next span
+    const bool head = (maskw[0] & 1u) == 0u;       // the row of the first slot began before the span
+    const uint64_t bm = __ballot(sub != 0u);       // lanes of groups that hold a row start
+    GroupLinks lk;
+    lk.g = g;
+    {
+        const uint64_t upto = bm & ((2ull << (g * HB + HB - 1)) - 1ull);  // 2 << 63 wraps to 0: all bits kept
+        lk.seg0 = upto ? (63 - __builtin_clzll(upto)) / HB : 0;
+        const int sh = (g + 1) * HB;
+        const uint64_t after = sh < kWave ? bm >> sh : 0ull;
+        lk.next = after ? (g + 1 + __builtin_ctzll(after) / HB) * HB + h : -1;
+        lk.last = ((endl - 1) / K) * HB + h;
+    }
+    // first and last row start of the span, as slots (wave-uniform)
+    const int kf = sub ? __builtin_ctz(sub) : K;
+    const int kl = sub ? 31 - __builtin_clz(sub) : 0;
+    const int gfirst = bm ? __builtin_ctzll(bm) / HB : 0, glast = bm ? (63 - __builtin_clzll(bm)) / HB : 0;
+    const int ffpos = __shfl(g * K + kf, gfirst * HB, kWave), lfpos = __shfl(g * K + kl, glast * HB, kWave);
+    const int hpos = !head ? 0 : (bm ? ffpos : endl);                // slots before hpos: the head row
+    const int tpos = (last_open && bm) ? lfpos : endl;               // slots from tpos on: the tail row
 
-    // ---- per step: my row's result within the span so far
-    float tm[kSteps][HB], ts[kSteps][HB];
-    float fm[kSteps - 1][HB], fs[kSteps - 1][HB];  // wave-uniform: the row crossing the boundary after step b
-    float cm[HB], cs[HB];                          // wave-uniform carry of the row open at the end of the last step
+    float rm[K], rs[K];  // per slot: the row's max and sum within the span
+    float tfm = 0.0f, xm = 0.0f, tfs, xs;
+    if (FWD) {
 #pragma unroll
-    for (int i = 0; i < HB; ++i) cm[i] = -INFINITY, cs[i] = 0.0f;
+        for (int k = 0; k < K; ++k) rm[k] = x[k];
+        row_aggregates<HB, K, true>(rm, sub, lk, tfm, xm);
 #pragma unroll
-    for (int b = 0; b < kSteps - 1; ++b)
-#pragma unroll
-        for (int i = 0; i < HB; ++i) fm[b][i] = 0.0f, fs[b][i] = 1.0f;
-#pragma unroll
-    for (int u = 0; u < kSteps; ++u) {
-        const int sbl = kWave * u;
-        const int sel = sbl + kWave < endl ? sbl + kWave : endl;
-        if (sbl >= endl) break;  // uniform
-        const int lo = rsl[u] > sbl ? rsl[u] - sbl : 0;
-        const int hi = (rel[u] < sel ? rel[u] : sel) - 1 - sbl;
-        const bool cont_in = rsl[u] < sbl;  // my row began in an earlier step (or span)
-#pragma unroll
-        for (int i = 0; i < HB; ++i) {
-            if (FWD) {
-                float m = seg_scan_max(x[u][i], lane, lo);
-                m = __shfl(m, hi, kWave);
-                if (cont_in) m = fmaxf(m, cm[i]);
-                const float ex = (kWave * u + lane < endl) ? expf(x[u][i] - m) : 0.0f;
-                float s = seg_scan_add(ex, lane, lo);
-                s = __shfl(s, hi, kWave);
-                if (cont_in) s += cs[i] * expf(cm[i] - m);  // an empty carry is (-inf, 0)
-                tm[u][i] = m;
-                ts[u][i] = s;
-            } else {
-                float s = seg_scan_add(x[u][i] * y[u][i], lane, lo);
-                s = __shfl(s, hi, kWave);
-                if (cont_in) s += cs[i];
-                tm[u][i] = 0.0f;
-                ts[u][i] = s;
-            }
+        for (int k = 0; k < K; ++k) {
+            x[k] = id[k] >= 0 ? expf(x[k] - rm[k]) : 0.0f;
+            rs[k] = x[k];
         }
-        // the row of lane 0 ends in this step and began in an earlier step of this span: its result
-        // goes to the boundaries it crossed
-        const int rs0 = __builtin_amdgcn_readfirstlane(rsl[u]);
-        const int re0 = __builtin_amdgcn_readfirstlane(rel[u]);
-        if (rs0 >= 0 && rs0 < sbl && re0 <= sel) {
+    } else {
 #pragma unroll
-            for (int b = 0; b < kSteps - 1; ++b)
-                if (b < u && b >= (rs0 >> 6)) {
-#pragma unroll
-                    for (int i = 0; i < HB; ++i) fm[b][i] = rl_f(tm[u][i], 0), fs[b][i] = rl_f(ts[u][i], 0);
-                }
+        for (int k = 0; k < K; ++k) rs[k] = x[k] * y[k], rm[k] = 0.0f;
+    }
+    row_aggregates<HB, K, false>(rs, sub, lk, tfs, xs);
+
+    // ---- partial results of the head row and of the tail row, the span's record
+    float* vals_hm = span_vals(ws, nspans, w, 0, 0, H) + h0 + h;
+    float* vals_hs = span_vals(ws, nspans, w, 0, 1, H) + h0 + h;
+    if (head && hok) {
+        if (bm && g == gfirst) {
+            *vals_hm = tfm;
+            *vals_hs = tfs;
         }
-        // carry: the row of the last lane, if it runs on
-        const bool open = __builtin_amdgcn_readlane(rel[u], kWave - 1) > sel;
-#pragma unroll
-        for (int i = 0; i < HB; ++i) {
-            cm[i] = open ? rl_f(tm[u][i], kWave - 1) : -INFINITY;
-            cs[i] = open ? rl_f(ts[u][i], kWave - 1) : 0.0f;
+        if (!bm && lane == lk.last) {  // no row starts in the span: it is all head
+            *vals_hm = xm;
+            *vals_hs = xs;
         }
-        // partial results of the head row (at its last slot in the span) and of the tail row (at the span's last slot)
-        const int ls = sbl + lane;  // my slot, relative
-        if (ls < endl) {
-            const bool last_of_row = ls == (rel[u] < endl ? rel[u] : endl) - 1;
-            if (last_of_row && rsl[u] < 0) {
-                store_heads<HB, false>(span_vals(ws, nspans, w, 0, 0, H) + h0, tm[u], nh);
-                store_heads<HB, false>(span_vals(ws, nspans, w, 0, 1, H) + h0, ts[u], nh);
-            }
-            if (last_of_row && rsl[u] >= 0 && rel[u] > endl) {
-                store_heads<HB, false>(span_vals(ws, nspans, w, 1, 0, H) + h0, tm[u], nh);
-                store_heads<HB, false>(span_vals(ws, nspans, w, 1, 1, H) + h0, ts[u], nh);
-            }
-            if (blockIdx.y == 0) {
-                SpanMeta* meta = static_cast<SpanMeta*>(ws) + w;
-                if (ls == 0) {
-                    meta->head_end = rsl[u] < 0 ? base + (rel[u] < endl ? rel[u] : endl) : base;
-                    meta->head_open = (rsl[u] < 0 && rel[u] > endl) ? 1 : 0;
-                }
-                if (ls == endl - 1) meta->tail_start = (rsl[u] >= 0 && rel[u] > endl) ? base + rsl[u] : end;
-            }
-        }
+    }
+    if (last_open && bm && lane == lk.last && hok) {
+        *(span_vals(ws, nspans, w, 1, 0, H) + h0 + h) = xm;
+        *(span_vals(ws, nspans, w, 1, 1, H) + h0 + h) = xs;
+    }
+    if (lane == 0 && blockIdx.y == 0) {
+        SpanMeta* meta = static_cast<SpanMeta*>(ws) + w;
+        meta->head_end = base + hpos;
+        meta->tail_start = base + tpos;
+        meta->head_open = (head && !bm && last_open) ? 1 : 0;
     }
 
     // ---- rows inside the span: write
 #pragma unroll
-    for (int u = 0; u < kSteps; ++u) {
-        const int sbl = kWave * u;
-        const int sel = sbl + kWave < endl ? sbl + kWave : endl;
-        if (id[u] < 0 || rsl[u] < 0 || rel[u] > endl) continue;
-        const bool later = rel[u] > sel;  // my row ends in a later step
-        float o[HB];
+    for (int k = 0; k < K; ++k) {
+        const int j = g * K + k;
+        if (id[k] < 0 || j < hpos || j >= tpos) continue;
         if (FWD) {
-#pragma unroll
-            for (int i = 0; i < HB; ++i) {
-                const float m = (later && u < kSteps - 1) ? fm[u < kSteps - 1 ? u : 0][i] : tm[u][i];
-                const float s = (later && u < kSteps - 1) ? fs[u < kSteps - 1 ? u : 0][i] : ts[u][i];
-                o[i] = expf(x[u][i] - m) * (1.0f / s);
-            }
+            out[id[k]] = x[k] * (1.0f / rs[k]);
         } else {
-            float z[HB];
-            load_heads<HB, VEC>(z, e + id[u], nh);
-#pragma unroll
-            for (int i = 0; i < HB; ++i) {
-                const float dot = (later && u < kSteps - 1) ? fs[u < kSteps - 1 ? u : 0][i] : ts[u][i];
-                float g = x[u][i] * (y[u][i] - dot);
-                if (!(z[i] > 0.0f)) g *= slope;
-                o[i] = g;
-            }
+            float gr = x[k] * (y[k] - rs[k]);
+            if (!(e[id[k]] > 0.0f)) gr *= slope;
+            out[id[k]] = gr;
         }
-        store_heads<HB, VEC>(out + id[u], o, nh);
     }
 }
 
-// One wavefront per span that holds the start of a cut row: merges the row's pieces and stores the
-// result into each of them.  blockDim.x = 256, grid = ceil(nspans / 4).
+__device__ __forceinline__ void merge_max_sum(float& m, float& s, float m2, float s2) {
+    const float mx = fmaxf(m, m2);
+    // exp(-inf - -inf) would be NaN: a side with no elements contributes nothing
+    const float u = (m == -INFINITY) ? 0.0f : s * expf(m - mx);
+    const float v = (m2 == -INFINITY) ? 0.0f : s2 * expf(m2 - mx);
+    m = mx;
+    s = u + v;
+}
+
+// One wavefront per span that holds the start of a cut row: merges the row's pieces (the tail piece
+// of this span, the head pieces of the following ones) and stores the result into each of them.
+// Lanes are (chunk, head) pairs: a lane folds every 64/Hp-th piece of its head, the chunks are
+// folded with xor-shuffles.  blockDim.x = 256, grid = ceil(nspans / 4).
 template <bool FWD>
-__global__ __launch_bounds__(256) void span_fix_kernel(int64_t nnz, int H, void* __restrict__ ws) {
+__global__ __launch_bounds__(256) void span_fix_kernel(int64_t nnz, int span, int H, void* __restrict__ ws) {
     const int lane = lane_id();
-    const int64_t nspans = (nnz + kSpan - 1) / kSpan;
+    const int64_t nspans = (nnz + span - 1) / span;
     const int64_t w = static_cast<int64_t>(blockIdx.x) * 4 + (static_cast<int>(threadIdx.x) >> 6);
     if (w >= nspans) return;
     const SpanMeta* meta = static_cast<const SpanMeta*>(ws);
-    const int64_t end = (w + 1) * kSpan < nnz ? (w + 1) * kSpan : nnz;
+    const int64_t end = (w + 1) * span < nnz ? (w + 1) * span : nnz;
     if (meta[w].tail_start >= end) return;  // no row starts here and runs on
     // the pieces: tail of w, then heads of w + 1 .. last, where last is the first span whose head is closed
     int64_t last = w + 1;
@@ -370,43 +381,39 @@ __global__ __launch_bounds__(256) void span_fix_kernel(int64_t nnz, int H, void*
         }
     }
     if (last >= nspans) last = nspans - 1;
-    for (int h = 0; h < H; ++h) {
+    int hp = 1;
+    while (hp < H && hp < kWave) hp <<= 1;
+    const int chunks = kWave / hp, c = lane / hp;
+    for (int hb = 0; hb < H; hb += hp) {
+        const int h = hb + lane % hp;
+        const bool ok = h < H;
         float m = -INFINITY, s = 0.0f;
-        for (int64_t j = w + 1 + lane; j <= last; j += kWave) {
-            const float s2 = *(span_vals(ws, nspans, j, 0, 1, H) + h);
-            if (FWD) {
-                const float m2 = *(span_vals(ws, nspans, j, 0, 0, H) + h);
-                const float mx = fmaxf(m, m2);
-                s = (m == -INFINITY ? 0.0f : s * expf(m - mx)) + s2 * expf(m2 - mx);
-                m = mx;
-            } else {
-                s += s2;
+        if (ok) {
+            for (int64_t j = w + 1 + c; j <= last; j += chunks) {
+                const float s2 = *(span_vals(ws, nspans, j, 0, 1, H) + h);
+                if (FWD) merge_max_sum(m, s, *(span_vals(ws, nspans, j, 0, 0, H) + h), s2);
+                else s += s2;
+            }
+            if (c == 0) {  // the tail piece joins on chunk 0
+                const float s2 = *(span_vals(ws, nspans, w, 1, 1, H) + h);
+                if (FWD) merge_max_sum(m, s, *(span_vals(ws, nspans, w, 1, 0, H) + h), s2);
+                else s += s2;
             }
         }
-        if (lane == 0) {  // the tail piece joins on lane 0
-            const float s2 = *(span_vals(ws, nspans, w, 1, 1, H) + h);
-            if (FWD) {
-                const float m2 = *(span_vals(ws, nspans, w, 1, 0, H) + h);
-                const float mx = fmaxf(m, m2);
-                s = (m == -INFINITY ? 0.0f : s * expf(m - mx)) + s2 * expf(m2 - mx);
-                m = mx;
-            } else {
-                s += s2;
+        for (int off = hp; off < kWave; off <<= 1) {
+            const float m2 = __shfl_xor(m, off, kWave), s2 = __shfl_xor(s, off, kWave);
+            if (FWD) merge_max_sum(m, s, m2, s2);
+            else s += s2;
+        }
+        if (ok) {
+            for (int64_t j = w + 1 + c; j <= last; j += chunks) {
+                *(span_vals(ws, nspans, j, 0, 0, H) + h) = m;
+                *(span_vals(ws, nspans, j, 0, 1, H) + h) = s;
             }
-        }
-        if (FWD) {
-            const float mx = wave_max(m);
-            s = (m == -INFINITY) ? 0.0f : s * expf(m - mx);
-            m = mx;
-        }
-        s = wave_sum(s);
-        for (int64_t j = w + 1 + lane; j <= last; j += kWave) {
-            *(span_vals(ws, nspans, j, 0, 0, H) + h) = m;
-            *(span_vals(ws, nspans, j, 0, 1, H) + h) = s;
-        }
-        if (lane == 0) {
-            *(span_vals(ws, nspans, w, 1, 0, H) + h) = m;
-            *(span_vals(ws, nspans, w, 1, 1, H) + h) = s;
+            if (c == 0) {
+                *(span_vals(ws, nspans, w, 1, 0, H) + h) = m;
+                *(span_vals(ws, nspans, w, 1, 1, H) + h) = s;
+            }
         }
     }
 }
@@ -415,15 +422,15 @@ __global__ __launch_bounds__(256) void span_fix_kernel(int64_t nnz, int H, void*
 template <int HB, bool VEC, bool FWD>
 __global__ __launch_bounds__(256) void span_rest_kernel(
     float* __restrict__ out, const float* __restrict__ a, const float* __restrict__ da,
-    const float* __restrict__ e, const int64_t* __restrict__ eids, int64_t nnz, int H, float slope,
+    const float* __restrict__ e, const int64_t* __restrict__ eids, int64_t nnz, int span, int H, float slope,
     void* __restrict__ ws) {
     const int lane = lane_id();
-    const int64_t nspans = (nnz + kSpan - 1) / kSpan;
+    const int64_t nspans = (nnz + span - 1) / span;
     const int64_t w = static_cast<int64_t>(blockIdx.x) * 4 + (static_cast<int>(threadIdx.x) >> 6);
     if (w >= nspans) return;
     const SpanMeta mt = static_cast<const SpanMeta*>(ws)[w];
-    const int64_t base = w * kSpan;
-    const int64_t end = base + kSpan < nnz ? base + kSpan : nnz;
+    const int64_t base = static_cast<int64_t>(w) * span;
+    const int64_t end = base + span < nnz ? base + span : nnz;
     if (mt.head_end <= base && mt.tail_start >= end) return;
     const int h0 = static_cast<int>(blockIdx.y) * HB;
     const int nh = H - h0 < HB ? H - h0 : HB;
@@ -437,8 +444,7 @@ __global__ __launch_bounds__(256) void span_rest_kernel(
             rs[piece][i] = (have && i < nh) ? *(span_vals(ws, nspans, w, piece, 1, H) + h0 + i) : 1.0f;
         }
     }
-#pragma unroll
-    for (int u = 0; u < kSteps; ++u) {
+    for (int u = 0; u < span / kWave; ++u) {
         const int64_t s = base + kWave * u + lane;
         const bool inhead = s < mt.head_end;
         const bool intail = s >= mt.tail_start && s < end;
@@ -466,36 +472,40 @@ __global__ __launch_bounds__(256) void span_rest_kernel(
     }
 }
 
-template <int HB, bool VEC, bool FWD>
+// slots per span by head count: lanes are (group, head) pairs, K slots per lane
+static int span_slots(int H) { return H % 8 == 0 || H > 4 ? 128 : 256; }
+
+template <int HB, int K, bool VEC, bool FWD>
 static void launch_spans_hb(float* out, const float* a, const float* da, const float* e, const int64_t* indptr,
                             const int64_t* eids, int64_t rows, int64_t nnz, int H, float slope, void* ws,
                             hipStream_t s) {
-    const int64_t nspans = ceil_div(nnz, kSpan);
+    constexpr int SPAN = (kWave / HB) * K;
+    const int64_t nspans = ceil_div(nnz, SPAN);
     const dim3 grid(static_cast<unsigned>(ceil_div(nspans, 4)), static_cast<unsigned>(ceil_div(H, HB)));
-    hipLaunchKernelGGL((span_kernel<HB, VEC, FWD>), grid, dim3(256), 0, s, out, a, da, e, indptr, eids, rows, nnz, H,
+    hipLaunchKernelGGL((span_kernel<HB, K, FWD>), grid, dim3(256), 0, s, out, a, da, e, indptr, eids, rows, nnz, H,
                        slope, ws);
-    hipLaunchKernelGGL(span_fix_kernel<FWD>, dim3(grid.x), dim3(256), 0, s, nnz, H, ws);
-    hipLaunchKernelGGL((span_rest_kernel<HB, VEC, FWD>), grid, dim3(256), 0, s, out, a, da, e, eids, nnz, H, slope,
-                       ws);
+    hipLaunchKernelGGL(span_fix_kernel<FWD>, dim3(grid.x), dim3(256), 0, s, nnz, SPAN, H, ws);
+    hipLaunchKernelGGL((span_rest_kernel<HB, VEC, FWD>), grid, dim3(256), 0, s, out, a, da, e, eids, nnz, SPAN, H,
+                       slope, ws);
 }
 
 template <bool FWD>
 static void launch_spans(float* out, const float* a, const float* da, const float* e, const int64_t* indptr,
                          const int64_t* eids, int64_t rows, int64_t nnz, int H, float slope, void* ws,
                          hipStream_t s) {
-#define TANGO_SPANS(HB, VEC) launch_spans_hb<HB, VEC, FWD>(out, a, da, e, indptr, eids, rows, nnz, H, slope, ws, s)
-    if (H % 8 == 0) TANGO_SPANS(8, true);
-    else if (H % 4 == 0) TANGO_SPANS(4, true);
-    else if (H == 2) TANGO_SPANS(2, true);
-    else if (H == 1) TANGO_SPANS(1, false);
-    else if (H < 4) TANGO_SPANS(4, false);
-    else TANGO_SPANS(8, false);
+#define TANGO_SPANS(HB, K, VEC) launch_spans_hb<HB, K, VEC, FWD>(out, a, da, e, indptr, eids, rows, nnz, H, slope, ws, s)
+    if (H % 8 == 0) TANGO_SPANS(8, 16, true);
+    else if (H > 4) TANGO_SPANS(8, 16, false);
+    else if (H == 4) TANGO_SPANS(4, 16, true);
+    else if (H == 3) TANGO_SPANS(4, 16, false);
+    else if (H == 2) TANGO_SPANS(2, 8, true);
+    else TANGO_SPANS(1, 4, false);
 #undef TANGO_SPANS
 }
 
 static size_t span_workspace_bytes(int64_t nnz, int64_t H) {
     if (nnz <= 0 || H <= 0) return 0;
-    const int64_t nspans = ceil_div(nnz, kSpan);
+    const int64_t nspans = ceil_div(nnz, span_slots(static_cast<int>(H < 64 ? H : 64)));
     return span_vals_offset(nspans) + static_cast<size_t>(nspans) * 4 * static_cast<size_t>(H) * sizeof(float);
 }
 
@@ -513,7 +523,7 @@ int tango_edge_softmax_fwd(float* a, const float* e, const int64_t* indptr,
     if (rows < 0 || nnz < 0 || H < 0 || (rows > 0 && !indptr) || H >= (1LL << 31)) return TANGO_ERR_INVALID_ARG;
     if (rows * H == 0 || nnz == 0) return TANGO_OK;
     if (!a || !e) return TANGO_ERR_INVALID_ARG;
-    if (workspace && ceil_div(nnz, 4 * kSpan) <= INT32_MAX && ceil_div(H, 8) <= 65535) {
+    if (workspace && ceil_div(nnz, 4 * 128) <= INT32_MAX && ceil_div(H, 8) <= 65535) {
         if (workspace_bytes < span_workspace_bytes(nnz, H) || (reinterpret_cast<uintptr_t>(workspace) & 15))
             return TANGO_ERR_WORKSPACE;
         launch_spans<true>(a, nullptr, nullptr, e, indptr, edge_ids, rows, nnz, static_cast<int>(H), slope,
@@ -532,7 +542,7 @@ int tango_edge_softmax_bwd(float* de, const float* a, const float* da, const flo
     if (rows < 0 || nnz < 0 || H < 0 || (rows > 0 && !indptr) || H >= (1LL << 31)) return TANGO_ERR_INVALID_ARG;
     if (rows * H == 0 || nnz == 0) return TANGO_OK;
     if (!de || !a || !da || !e) return TANGO_ERR_INVALID_ARG;
-    if (workspace && ceil_div(nnz, 4 * kSpan) <= INT32_MAX && ceil_div(H, 8) <= 65535) {
+    if (workspace && ceil_div(nnz, 4 * 128) <= INT32_MAX && ceil_div(H, 8) <= 65535) {
         if (workspace_bytes < span_workspace_bytes(nnz, H) || (reinterpret_cast<uintptr_t>(workspace) & 15))
             return TANGO_ERR_WORKSPACE;
         launch_spans<false>(de, a, da, e, indptr, edge_ids, rows, nnz, static_cast<int>(H), slope, workspace,

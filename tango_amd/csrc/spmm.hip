@@ -701,6 +701,19 @@ __global__ __launch_bounds__(256) void spmm_span_kernel(const SpmmParams p) {
     const int endl = static_cast<int>(p.nnz - base < kSpanSlots ? p.nnz - base : kSpanSlots);
     const int64_t end = base + endl;
 
+    // the span's column indices (and edge ids), one coalesced pass; issued first so that they are in
+    // flight while the row structure is worked out
+    int my_idx[kSpanSlots / kWave], my_eid[kSpanSlots / kWave];
+#pragma unroll
+    for (int u = 0; u < kSpanSlots / kWave; ++u) {
+        const int sl = kWave * u + lane;
+        my_idx[u] = my_eid[u] = 0;
+        if (sl < endl) {
+            my_idx[u] = load_index<true>(p, p.indices, base + sl);
+            if (permuted) my_eid[u] = load_index<true>(p, p.edge_ids, base + sl);
+        }
+    }
+
     // ---- row structure of the span
     const int64_t r0 = row_of_slot_wave(p.indptr, p.rows, base, lane);
     if (lane < 12) maskw[lane] = 0u;
@@ -722,14 +735,10 @@ __global__ __launch_bounds__(256) void spmm_span_kernel(const SpmmParams p) {
         }
         if (pv == end) atomicOr(&maskw[8], 1u);  // a row ends exactly at the span's end
     }
-    // the span's column indices (and edge ids): one coalesced pass
 #pragma unroll
     for (int u = 0; u < kSpanSlots / kWave; ++u) {
-        const int sl = kWave * u + lane;
-        if (sl < endl) {
-            sidx[sl] = load_index<true>(p, p.indices, base + sl);
-            if (permuted) seid[sl] = load_index<true>(p, p.edge_ids, base + sl);
-        }
+        sidx[kWave * u + lane] = my_idx[u];
+        if (permuted) seid[kWave * u + lane] = my_eid[u];
     }
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();

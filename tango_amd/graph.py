@@ -99,6 +99,19 @@ class Graph:
     def local_scope(self):
         yield self
 
+    def reorder_edges_by_dst(self):
+        """The same graph with its edges renumbered in destination-major order (new edge i is old
+        edge ``edge_order[i]``, kept as an attribute of the result).  Edge tensors of the
+        attention layers ([E, H] logits, softmax outputs, their gradients) are reached through the
+        destination-major CSR; when that order is the edge-id order itself they are read and written
+        front to back instead of gathered and scattered 4 H bytes at a time.  Models that take no
+        per-edge input (GAT, HGT) give the same node outputs on either numbering; per-edge inputs
+        must be permuted with ``edge_order`` first."""
+        order = self.adj_sparse("csc")[2]
+        g = Graph(self._src[order], self._dst[order], self._n)
+        g.edge_order = order
+        return g
+
 
 def remove_self_loop(src, dst):
     keep = src != dst

@@ -139,3 +139,30 @@ def test_hgt_stack_on_heterogeneous_graph():
         opt.step()
         losses.append(loss.item())
     assert all(np.isfinite(losses)) and losses[-1] < losses[0], losses
+
+
+def test_edge_renumbering_leaves_node_outputs_unchanged():
+    """Destination-major edge numbering (Graph.reorder_edges_by_dst) is an internal matter of the
+    attention layers: same node outputs and parameter gradients, attention values permuted."""
+    from tango_amd.gat import QGATConv
+    from tango_amd.graph import chung_lu
+    from tango_amd.util import graph_preprocess
+    g0 = chung_lu(3000, 30000, 2.2, seed=4, device="cuda")
+    g1 = g0.reorder_edges_by_dst()
+    assert bool((g1.adj_sparse("csc")[2] == torch.arange(g1.num_edges(), device="cuda")).all())
+    g0, g1 = graph_preprocess(g0), graph_preprocess(g1)
+    torch.manual_seed(9)
+    layer = QGATConv(64, 16, 8).cuda()
+    x = torch.randn(g0.num_nodes(), 64, device="cuda")
+    outs, grads, att = [], [], []
+    for g in (g0, g1):
+        layer.zero_grad()
+        rst, a = layer(g, x, get_attention=True)
+        rst.square().sum().backward()
+        outs.append(rst.detach().clone())
+        att.append(a.detach().clone())
+        grads.append([p.grad.detach().clone() for p in layer.parameters()])
+    assert torch.allclose(outs[0], outs[1], rtol=1e-5, atol=1e-6)
+    assert torch.allclose(att[0][g1.edge_order], att[1], rtol=1e-5, atol=1e-7)
+    for a, b in zip(*grads):
+        assert torch.allclose(a, b, rtol=1e-3, atol=1e-4 * float(a.abs().max()))
