@@ -67,8 +67,14 @@ class QGATConv(nn.Module):
             nn.init.xavier_normal_(self.res_fc.weight, gain=gain)
 
     def forward(self, graph, feat, get_attention=False):
-        if not self._allow_zero_in_degree and bool((graph.in_degrees() == 0).any()):
-            raise Exception("There are 0-in-degree nodes in the graph.")  # test_gat.py:93-96
+        if not self._allow_zero_in_degree:  # test_gat.py:93-96
+            # answered once per graph: the check reads a device tensor back, and a host sync in every
+            # layer's forward would leave the GPU idle while the host issues the next launches
+            zero_in = getattr(graph, "_has_zero_in_degree", None)
+            if zero_in is None:
+                zero_in = graph._has_zero_in_degree = bool((graph.in_degrees() == 0).any())
+            if zero_in:
+                raise Exception("There are 0-in-degree nodes in the graph.")
         n = feat.size(0)
         h = self.feat_drop(feat).contiguous()
         feat_src, s_feat = self.fc(h)

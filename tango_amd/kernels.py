@@ -20,8 +20,13 @@ from ._lib import ROUND_MODES, ROUND_RNE, ROUND_STOCHASTIC, ROUND_TRUNC, SDDMM_O
 _L = _lib.lib()  # fails here, loudly, if the library is not built
 
 
+_raw_stream = torch._C._cuda_getCurrentRawStream  # the handle itself, without building a Stream object
+_current_device = torch._C._cuda_getDevice
+
+
 def _stream():
-    return torch.cuda.current_stream().cuda_stream
+    """The current stream of the current device as a raw hipStream_t (what torch's own ops launch on)."""
+    return _raw_stream(_current_device())
 
 
 def _ptr(t):
