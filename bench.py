@@ -37,6 +37,7 @@ def parse():
     ap.add_argument("--no-primitives", action="store_true")
     ap.add_argument("--emit", default=None, metavar="JSON_FILE",
                     help="also store the result under the key 'measured_mi355x' of this JSON file")
+    ap.add_argument("--feat", type=int, default=256, help="feature width of --profile-mode spmm")
     ap.add_argument("--profile-mode", choices=["spmm", "copy", "qlinear", "sddmm", "quantize", "gat", "hgt"], default=None,
                     help="run only the dominant kernel (spmm: copy_u F=256 on the benchmark graph) or a "
                          "1 GiB device copy (counter calibration), for rocprofv3 --pmc passes")
@@ -389,11 +390,11 @@ def main():
                      % (n, nnz, max_deg, time.perf_counter() - t0))
 
     if args.profile_mode == "spmm":
-        feat = torch.randint(-127, 128, (n, 256), dtype=torch.int8, device="cuda")
+        feat = torch.randint(-127, 128, (n, args.feat), dtype=torch.int8, device="cuda")
         one = torch.full((1,), 0.01, device="cuda")
         ms = time_op(lambda: K.csr_SPMM(g, feat, one), iters=args.steps, warm=args.warmup)
-        print(json.dumps({"profile_mode": "spmm", "F": 256, "nodes": n, "edges": nnz, "avg_ms": round(ms, 4),
-                          "algorithmic_bytes": spmm_bytes(nnz, n, 256)}))
+        print(json.dumps({"profile_mode": "spmm", "F": args.feat, "nodes": n, "edges": nnz, "avg_ms": round(ms, 4),
+                          "algorithmic_bytes": spmm_bytes(nnz, n, args.feat)}))
         return
 
     gen = torch.Generator().manual_seed(5)
