@@ -83,7 +83,25 @@ __global__ __launch_bounds__(1024) void absmax_small_kernel(const float* __restr
                                                             float* __restrict__ out) {
     __shared__ float part[16];
     float m = 0.0f;
-    for (int64_t i = threadIdx.x; i < n; i += blockDim.x) m = fmaxf(m, fabsf(x[i]));
+    if ((reinterpret_cast<uintptr_t>(x) & 15) == 0) {
+        // four independent 16-byte loads in flight per thread: one workgroup is bound by load latency
+        const f32x4* x4 = reinterpret_cast<const f32x4*>(x);
+        const int64_t n4 = n >> 2;
+        for (int64_t i = threadIdx.x; i < n4; i += 4 * blockDim.x) {
+            f32x4 v[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                const int64_t j = i + u * blockDim.x;
+                v[u] = j < n4 ? x4[j] : f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+            }
+#pragma unroll
+            for (int u = 0; u < 4; ++u)
+                m = fmaxf(fmaxf(m, fmaxf(fabsf(v[u][0]), fabsf(v[u][1]))), fmaxf(fabsf(v[u][2]), fabsf(v[u][3])));
+        }
+        for (int64_t i = (n4 << 2) + threadIdx.x; i < n; i += blockDim.x) m = fmaxf(m, fabsf(x[i]));
+    } else {
+        for (int64_t i = threadIdx.x; i < n; i += blockDim.x) m = fmaxf(m, fabsf(x[i]));
+    }
     m = wave_max(m);
     if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = m;
     __syncthreads();

@@ -50,6 +50,46 @@ __global__ __launch_bounds__(256) void sddmm_dot_kernel(
     if (REDUCE) block_absmax_to_global(m / 127.0f, scale_out);
 }
 
+// Heads wider than 16 bytes (D = 16 * LPH, LPH a power of two): LPH consecutive lanes share one
+// (edge, head) pair, each with 16 bytes of it, so the lanes of an edge read its two rows as
+// contiguous runs; the partial dot products meet with xor-shuffles.  (With one lane per head and
+// D = 64, the lanes of a wavefront would read 64 separate 16-byte pieces per load instruction.)
+template <int LPH, bool REDUCE>
+__global__ __launch_bounds__(256) void sddmm_dot_split_kernel(
+    float* __restrict__ out, float* __restrict__ scale_out, const int64_t* __restrict__ src,
+    const int64_t* __restrict__ dst, const int8_t* __restrict__ U, const int8_t* __restrict__ V,
+    const float* __restrict__ sU, const float* __restrict__ sV, int64_t E, int H) {
+    const float s = sU[0] * sV[0];
+    const int64_t per = static_cast<int64_t>(H) * LPH;  // lanes per edge; the row is per * 16 bytes
+    const int64_t total = E * per;
+    const int64_t nthr = static_cast<int64_t>(gridDim.x) * blockDim.x;
+    float m = 0.0f;
+    // every lane of a wavefront takes part in the shuffles: the loop bound is rounded up to whole wavefronts
+    const int64_t total_up = (total + kWave - 1) & ~static_cast<int64_t>(kWave - 1);
+    for (int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < total_up; i += nthr) {
+        int acc = 0;
+        const bool ok = i < total;
+        const int64_t e = ok ? i / per : 0;
+        const int64_t r = ok ? i - e * per : 0;  // 16-byte piece of the row
+        if (ok) {
+            const u32x4 a = *reinterpret_cast<const u32x4*>(U + (src[e] * per + r) * 16);
+            const u32x4 b = *reinterpret_cast<const u32x4*>(V + (dst[e] * per + r) * 16);
+            acc = __builtin_amdgcn_sdot4(a.x, b.x, acc, false);
+            acc = __builtin_amdgcn_sdot4(a.y, b.y, acc, false);
+            acc = __builtin_amdgcn_sdot4(a.z, b.z, acc, false);
+            acc = __builtin_amdgcn_sdot4(a.w, b.w, acc, false);
+        }
+#pragma unroll
+        for (int off = 1; off < LPH; off <<= 1) acc += __shfl_xor(acc, off, kWave);
+        if (ok && (r & (LPH - 1)) == 0) {
+            const float y = static_cast<float>(acc) * s;
+            __builtin_nontemporal_store(y, out + e * H + r / LPH);
+            if (REDUCE) m = fmaxf(m, fabsf(y));
+        }
+    }
+    if (REDUCE) block_absmax_to_global(m / 127.0f, scale_out);
+}
+
 template <int OP>
 __device__ __forceinline__ float apply_op(float a, float b) {
     if (OP == TANGO_OP_ADD) return a + b;
@@ -115,6 +155,25 @@ int tango_sddmm_dot_i8(float* out, float* scale_out, const int64_t* src, const i
     if (total == 0) return launch_status();
     const uintptr_t al = reinterpret_cast<uintptr_t>(U) | reinterpret_cast<uintptr_t>(V);
     const int vec = ((D & 15) == 0 && (al & 15) == 0) ? 16 : ((D & 3) == 0 && (al & 3) == 0) ? 4 : 1;
+    const int64_t lph = D / 16;
+    if (vec == 16 && lph >= 2 && lph <= 16 && (lph & (lph - 1)) == 0) {
+        const dim3 sgrid(grid_for(total * lph, 256, 16)), sblock(256);
+#define TANGO_DOT_SPLIT(L_)                                                                                   \
+    do {                                                                                                      \
+        if (scale_out)                                                                                        \
+            hipLaunchKernelGGL((sddmm_dot_split_kernel<L_, true>), sgrid, sblock, 0, s, out, scale_out, src,  \
+                               dst, U, V, sU, sV, num_edges, static_cast<int>(H));                            \
+        else                                                                                                  \
+            hipLaunchKernelGGL((sddmm_dot_split_kernel<L_, false>), sgrid, sblock, 0, s, out, scale_out, src, \
+                               dst, U, V, sU, sV, num_edges, static_cast<int>(H));                            \
+    } while (0)
+        if (lph == 2) TANGO_DOT_SPLIT(2);
+        else if (lph == 4) TANGO_DOT_SPLIT(4);
+        else if (lph == 8) TANGO_DOT_SPLIT(8);
+        else TANGO_DOT_SPLIT(16);
+#undef TANGO_DOT_SPLIT
+        return launch_status();
+    }
     const dim3 grid(grid_for(total, 256, 16)), block(256);
 #define TANGO_DOT(V_, R_)                                                                         \
     hipLaunchKernelGGL((sddmm_dot_kernel<V_, R_>), grid, block, 0, s, out, scale_out, src, dst, U, \

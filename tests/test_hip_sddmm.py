@@ -36,7 +36,7 @@ def test_reference_test_pattern(K):
             assert np.array_equal(host(out)[e], ((src[e] * dim + j) + (3 * dim - dst[e] * dim - j)).astype(np.float32))
 
 
-@pytest.mark.parametrize("H,D", [(8, 16), (4, 64), (1, 128), (3, 4), (2, 7), (8, 1), (5, 20)])
+@pytest.mark.parametrize("H,D", [(8, 16), (4, 64), (1, 128), (3, 32), (2, 256), (3, 48), (3, 4), (2, 7), (8, 1), (5, 20)])
 @pytest.mark.parametrize("reduce", [False, True])
 def test_dot(K, orc, H, D, reduce):
     rng = np.random.default_rng(H * 100 + D)
