@@ -171,7 +171,7 @@ __global__ __launch_bounds__(256, 2) void gemm_nt_kernel(const NtParams p) {
                     if (col + v < p.N) m = fmaxf(m, fabsf(y[v]));
                 }
                 if (col + 4 <= p.N && wide == 4) {
-                    __builtin_nontemporal_store(f32x4{y[0], y[1], y[2], y[3]}, reinterpret_cast<f32x4*>(crow + col));
+                    *reinterpret_cast<f32x4*>(crow + col) = f32x4{y[0], y[1], y[2], y[3]};
                 } else if (col + 4 <= p.N && wide == 2) {
                     typedef float f32x2 __attribute__((ext_vector_type(2)));
                     // plain stores: these half-aligned pieces rely on L2 to merge them into full lines
@@ -212,8 +212,9 @@ struct FqParams {
 };
 
 // TPW = 16-column tiles per wave (the workgroup covers 64 * TPW columns), XV = floats per load,
-// RT = 16-row tiles per workgroup (BM = 16 * RT rows).
-template <int TPW, int XV, int MODE, int RT>
+// RT = 16-row tiles per workgroup (BM = 16 * RT rows), IT = 256-column chunks of a row a lane
+// loads from (kp <= 256 IT): sizes the prefetch registers.
+template <int TPW, int XV, int MODE, int RT, int IT>
 __global__ __launch_bounds__(256, 2) void gemm_fq_kernel(const FqParams p) {
     extern __shared__ __attribute__((aligned(16))) int8_t a_lds[];  // [BM][kp + 16]
     constexpr int BM = 16 * RT;
@@ -228,14 +229,14 @@ __global__ __launch_bounds__(256, 2) void gemm_fq_kernel(const FqParams p) {
     // ---- phase A: rows wave, wave + 4, ... ; lane owns columns 4 * (lane + 64 it) .. + 3
     const float* __restrict__ Xp = p.X;
     int8_t* __restrict__ Xqp = p.Xq;
-    const int iters = (p.kp + 255) >> 8;  // <= 3: kp <= 768 is checked by the host
-    auto fetch = [&](float (*f)[3][4], int rr) {
+    const int iters = (p.kp + 255) >> 8;  // <= IT (1, 2 or 3 by the host: kp <= 768)
+    auto fetch = [&](float (*f)[IT][4], int rr) {
 #pragma unroll
         for (int b = 0; b < 4; ++b) {
             const int64_t row = row_base + wave + 4 * (rr + b);
             const float* xr = Xp + row * p.ldx;
 #pragma unroll
-            for (int it = 0; it < 3; ++it) {
+            for (int it = 0; it < IT; ++it) {
                 const int64_t c0 = (static_cast<int64_t>(lane) + 64 * it) << 2;
                 f[b][it][0] = f[b][it][1] = f[b][it][2] = f[b][it][3] = 0.0f;
                 if (it < iters && row < p.M && c0 < p.K) {
@@ -256,14 +257,14 @@ __global__ __launch_bounds__(256, 2) void gemm_fq_kernel(const FqParams p) {
             }
         }
     };
-    auto emit = [&](float (*f)[3][4], int rr) {
+    auto emit = [&](float (*f)[IT][4], int rr) {
 #pragma unroll
         for (int b = 0; b < 4; ++b) {
             const int lr = wave + 4 * (rr + b);
             const int64_t row = row_base + lr;
             const float rm = (p.x_row_mul && row < p.M) ? p.x_row_mul[row] : 1.0f;
 #pragma unroll
-            for (int it = 0; it < 3; ++it) {
+            for (int it = 0; it < IT; ++it) {
                 const int64_t c0 = (static_cast<int64_t>(lane) + 64 * it) << 2;
                 if (it < iters && c0 < p.kp) {
                     float x0 = f[b][it][0], x1 = f[b][it][1], x2 = f[b][it][2], x3 = f[b][it][3];
@@ -279,7 +280,7 @@ __global__ __launch_bounds__(256, 2) void gemm_fq_kernel(const FqParams p) {
     };
     {
         // two register buffers: the loads of the next four rows are in flight while these are quantized
-        float fa[4][3][4], fb[4][3][4];
+        float fa[4][IT][4], fb[4][IT][4];
         fetch(fa, 0);
         fetch(fb, 4);
         emit(fa, 0);
@@ -330,18 +331,32 @@ __global__ __launch_bounds__(256, 2) void gemm_fq_kernel(const FqParams p) {
                 }
             }
         };
-        load_bfrag(b0, 0);
-        load_bfrag(b1, 1);
-        for (int step = 0; step < ksteps; step += 3) {
-            load_bfrag(b2, step + 2);
-            mma_step(b0, step);
-            if (step + 1 < ksteps) {
-                load_bfrag(b0, step + 3);
-                mma_step(b1, step + 1);
+        if (TPW >= 4) {
+            // sixteen accumulator tiles per wave: one k-step of B fragments ahead keeps the kernel
+            // under 128 registers (four waves per SIMD instead of three)
+            load_bfrag(b0, 0);
+            for (int step = 0; step < ksteps; step += 2) {
+                load_bfrag(b1, step + 1);
+                mma_step(b0, step);
+                if (step + 1 < ksteps) {
+                    load_bfrag(b0, step + 2);
+                    mma_step(b1, step + 1);
+                }
             }
-            if (step + 2 < ksteps) {
-                load_bfrag(b1, step + 4);
-                mma_step(b2, step + 2);
+        } else {
+            load_bfrag(b0, 0);
+            load_bfrag(b1, 1);
+            for (int step = 0; step < ksteps; step += 3) {
+                load_bfrag(b2, step + 2);
+                mma_step(b0, step);
+                if (step + 1 < ksteps) {
+                    load_bfrag(b0, step + 3);
+                    mma_step(b1, step + 1);
+                }
+                if (step + 2 < ksteps) {
+                    load_bfrag(b1, step + 4);
+                    mma_step(b2, step + 2);
+                }
             }
         }
     }
@@ -368,7 +383,7 @@ __global__ __launch_bounds__(256, 2) void gemm_fq_kernel(const FqParams p) {
                         if (col + v < p.N) m = fmaxf(m, fabsf(y[v]));
                     }
                     if (col + 4 <= p.N && wide == 4) {
-                        __builtin_nontemporal_store(f32x4{y[0], y[1], y[2], y[3]}, reinterpret_cast<f32x4*>(crow + col));
+                        *reinterpret_cast<f32x4*>(crow + col) = f32x4{y[0], y[1], y[2], y[3]};
                     } else if (col + 4 <= p.N && wide == 2) {
                         typedef float f32x2 __attribute__((ext_vector_type(2)));
                         *reinterpret_cast<f32x2*>(crow + col) = f32x2{y[0], y[1]};
@@ -545,7 +560,7 @@ __global__ __launch_bounds__(768) void gemm_ws_kernel(const FqParams p, int nblo
                         if (col + v < p.N) m = fmaxf(m, fabsf(y[v]));
                     }
                     if (col + 4 <= p.N && wide == 4) {
-                        __builtin_nontemporal_store(f32x4{y[0], y[1], y[2], y[3]}, reinterpret_cast<f32x4*>(crow + col));
+                        *reinterpret_cast<f32x4*>(crow + col) = f32x4{y[0], y[1], y[2], y[3]};
                     } else if (col + 4 <= p.N && wide == 2) {
                         typedef float f32x2 __attribute__((ext_vector_type(2)));
                         *reinterpret_cast<f32x2*>(crow + col) = f32x2{y[0], y[1]};
@@ -851,13 +866,19 @@ static void launch_fq_mode(const FqParams& p, hipStream_t s) {
     if (launch_ws<XV, MODE>(p, s)) return;
     const size_t lds = static_cast<size_t>(16 * RT) * (p.kp + 16);
     const unsigned gx = static_cast<unsigned>(ceil_div(p.M, 16 * RT));
-#define TANGO_FQ(TPW_)                                                                           \
-    hipLaunchKernelGGL((gemm_fq_kernel<TPW_, XV, MODE, RT>),                                     \
+#define TANGO_FQ_IT(TPW_, IT_)                                                                   \
+    hipLaunchKernelGGL((gemm_fq_kernel<TPW_, XV, MODE, RT, IT_>),                                \
                        dim3(gx, static_cast<unsigned>(ceil_div(p.N, 64 * TPW_))), dim3(256), lds, s, p)
+#define TANGO_FQ(TPW_)                                                   \
+    do {                                                                 \
+        if (p.kp <= 256) TANGO_FQ_IT(TPW_, 1);                           \
+        else TANGO_FQ_IT(TPW_, 3);                                       \
+    } while (0)
     if (p.N <= 64) TANGO_FQ(1);
     else if (p.N <= 128) TANGO_FQ(2);
     else TANGO_FQ(4);
 #undef TANGO_FQ
+#undef TANGO_FQ_IT
 }
 
 static int launch_fq(const FqParams& p, int round_mode, hipStream_t s) {
