@@ -793,10 +793,39 @@ __global__ __launch_bounds__(256) void spmm_span_kernel(const SpmmParams p) {
     for (int i = 0; i < VEC; ++i) acc[i] = 0;
     bool have = false, started = false, tail_partial = false;
     int cur_start = 0, my_last_flag = -1, first_target = -2;
+    // Rows end at different slots in different groups, so the end-of-row code runs under divergence
+    // many times per wavefront: the scale and the lane's bias values are fetched once, here.
+    const float dq = p.scale[0];
+    float breg[VEC];
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) breg[i] = (p.bias && c.col + i < p.W) ? p.bias[c.col + i] : 0.0f;
+    // same sequence of roundings as store_row
+    auto finish_row = [&](int64_t row, const int* sum) {
+        if (!c.col_ok) return;
+        const float rs = p.row_scale ? p.row_scale[row] : 1.0f;
+        float* o = p.out + row * p.W + c.col;
+        float y[VEC];
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) {
+            y[i] = dq * static_cast<float>(sum[i]);
+            if (p.row_scale) y[i] = y[i] * rs;
+            if (p.bias) y[i] = y[i] + breg[i];
+            if (p.relu) y[i] = fmaxf(y[i], 0.0f);
+        }
+        if (VEC == 16 && p.out_vec && c.col + 16 <= p.W) {
+            f32x4* o4 = reinterpret_cast<f32x4*>(o);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) o4[i] = f32x4{y[4 * i], y[4 * i + 1], y[4 * i + 2], y[4 * i + 3]};
+        } else {
+#pragma unroll
+            for (int i = 0; i < VEC; ++i)
+                if (c.col + i < p.W) o[i] = y[i];
+        }
+    };
     // ends the piece the group is in
     auto flush = [&](bool closed) {
         if (started && closed) {
-            store_row<VEC>(p, c, r0 + rowof[cur_start], acc);
+            finish_row(r0 + rowof[cur_start], acc);
         } else {
             int target = c.grp;
             if (!started) {
@@ -880,7 +909,7 @@ __global__ __launch_bounds__(256) void spmm_span_kernel(const SpmmParams p) {
 #pragma unroll
         for (int i = 0; i < VEC; ++i) acc[i] = ab[i];
         if (closed) {
-            store_row<VEC>(p, c, r0 + rowof[my_last_flag], acc);
+            finish_row(r0 + rowof[my_last_flag], acc);
         } else {
             int* part = span_part(p, nspans, w, 1) + c.col;
 #pragma unroll
