@@ -235,12 +235,14 @@ int tango_spmm_csr_u_mul_e(float* out, const int64_t* indptr, const int64_t* ind
    With the slot->edge permutation fused, the H * D bytes of a gathered edge then
    come from one cache sector instead of H * D scattered ones.  bias (H * F floats or
    NULL) is added after dequantization ("rst + bias", evaluation/test_gat.py:160-162).
+   scale2 (or NULL): the dequantization scale is scale[0] * scale2[0] (the scales of the
+   node features and of the edge values, multiplied by a torch op in cuda/SPMM.py:44).
    idx_bits: width of the entries of indices and edge_ids, 64 or 32; max_row_nnz and
    workspace as for tango_spmm_csr_copy_u_ex. */
 int tango_spmm_csr_u_mul_e_ex(float* out, const int64_t* indptr, const void* indices,
                               const void* edge_ids, int idx_bits, const int8_t* feat, const int8_t* evals,
-                              int edge_major, const float* scale, const float* bias, int64_t rows,
-                              int64_t num_src, int64_t H, int64_t F, int64_t D, int64_t nnz,
+                              int edge_major, const float* scale, const float* scale2, const float* bias,
+                              int64_t rows, int64_t num_src, int64_t H, int64_t F, int64_t D, int64_t nnz,
                               int64_t max_row_nnz, void* workspace, size_t workspace_bytes,
                               tango_stream_t stream);
 

@@ -66,7 +66,7 @@ class sddmm_u_dot_v(Function):
         dZ_, scaledZ = _quantize_grad(dZ3)  # [E, H, 1], edge-major edge values
         dU = dV = None
         if ctx.needs_input_grad[1]:
-            dU = multi_cusparse_SPMM(g, V3, dZ_, scaledZ * scaleV, True, edge_major=True).reshape(U_.shape)
+            dU = multi_cusparse_SPMM(g, V3, dZ_, scaledZ, True, edge_major=True, scale2=scaleV).reshape(U_.shape)
         if ctx.needs_input_grad[2]:
-            dV = multi_cusparse_SPMM(g, U3, dZ_, scaledZ * scaleU, edge_major=True).reshape(V_.shape)
+            dV = multi_cusparse_SPMM(g, U3, dZ_, scaledZ, edge_major=True, scale2=scaleU).reshape(V_.shape)
         return None, dU, dV, None, None

@@ -97,16 +97,16 @@ class spmm_u_mul_e(Function):
         # fused into the gather, edge-major keeps the H bytes of an edge in one cache sector.
         E_T_, scaleE = quantize(E)
         N_, scaleN = quantize(N, scaleN)  # one absmax pass (the reference runs two, cuda/SPMM.py:39,43)
-        scale = scaleN * scaleE
-        out = multi_cusparse_SPMM(g, N_, E_T_, scale, edge_major=True, bias=bias)
+        # dequantized with scaleN * scaleE (cuda/SPMM.py:44); the kernel multiplies the two itself
+        out = multi_cusparse_SPMM(g, N_, E_T_, scaleN, edge_major=True, bias=bias, scale2=scaleE)
         reduce_last = _need_reduce_last_dim(N, E)
-        ctx.backward_cache = g, N_, scaleN, E_T_, scaleE, scale, reduce_last, E.shape, bias is not None
+        ctx.backward_cache = g, N_, scaleN, E_T_, scaleE, reduce_last, E.shape, bias is not None
         return out
 
     @staticmethod
     @once_differentiable
     def backward(ctx, dZ):
-        g, N_, scaleN, E_T_, scaleE, scale, reduce_last, eshape, has_bias = ctx.backward_cache
+        g, N_, scaleN, E_T_, scaleE, reduce_last, eshape, has_bias = ctx.backward_cache
         dbias = None
         if has_bias and ctx.needs_input_grad[3]:
             # the scale of dZ and the bias gradient (column sums) in one read
@@ -122,8 +122,8 @@ class spmm_u_mul_e(Function):
         if ctx.needs_input_grad[1]:
             # dN = A^T (E * dZ): the dequantization scale is s_dZ * s_E.  The reference passes
             # the forward scale s_N * s_E here (cuda/SPMM.py:56); ref_compat reproduces that.
-            bscale = scale if config.ref_compat else scaledZ * scaleE
-            dN = multi_cusparse_SPMM(g, dZ_, E_T_, bscale, True, edge_major=True)
+            first = scaleN if config.ref_compat else scaledZ
+            dN = multi_cusparse_SPMM(g, dZ_, E_T_, first, True, edge_major=True, scale2=scaleE)
         if ctx.needs_input_grad[2]:
             op = "dot" if reduce_last else "mul"
             dE, _ = mySDDMM_int8(g, op, N_, dZ_, scaleN, scaledZ, False)

@@ -590,6 +590,30 @@ __global__ __launch_bounds__(256) void pack_rows_i8_kernel(int8_t* __restrict__ 
     }
 }
 
+// The weight operand of the forward GEMM in one pass: Wq[n, k] = quantize(W[n, k]) (the cache the
+// backward reads) and the same bytes in the packed form the MFMA loop reads, rows of ldp bytes,
+// zero-filled.  Thread 0 also zeroes the slot the GEMM's epilogue maxes the output scale into.
+template <int MODE>
+__global__ __launch_bounds__(256) void quantize_pack_w_kernel(const float* __restrict__ W, int64_t ldw,
+                                                              const float* __restrict__ scale,
+                                                              int8_t* __restrict__ Wq, int8_t* __restrict__ packed,
+                                                              int64_t ldp, int64_t N, int64_t K,
+                                                              float* __restrict__ zero_slot) {
+    if (zero_slot && blockIdx.x == 0 && threadIdx.x == 0) zero_slot[0] = 0.0f;
+    const float r = rscale_of(scale[0]);
+    const int64_t total = N * ldp;
+    const int64_t nthr = static_cast<int64_t>(gridDim.x) * blockDim.x;
+    for (int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < total; i += nthr) {
+        const int64_t n = i / ldp, k = i - n * ldp;
+        int8_t q = 0;
+        if (k < K) {
+            q = static_cast<int8_t>(quant_one<MODE>(W[n * ldw + k], r, 0.0f));
+            Wq[n * K + k] = q;
+        }
+        packed[i] = q;
+    }
+}
+
 // dst[c, 0..ldd) = src[0..rows, c] zero-filled, for c < cols: dst is [cols, ldd].
 __global__ __launch_bounds__(256) void transpose_pack_i8_kernel(int8_t* __restrict__ dst, int64_t ldd,
                                                                 const int8_t* __restrict__ src,
@@ -793,10 +817,11 @@ static void launch_nt_vec(const NtParams& p, hipStream_t s) {
 }
 
 // B must already be packed (16-byte aligned rows, zero-filled to a multiple of 64 columns).
-static int launch_nt(NtParams p, hipStream_t s) {
+// slot_zeroed: the caller has already zeroed absmax_out on this stream
+static int launch_nt(NtParams p, hipStream_t s, bool slot_zeroed = false) {
     if (p.M == 0 || p.N == 0) return TANGO_OK;
     if (ceil_div(p.M, 128) > INT32_MAX) return TANGO_ERR_UNSUPPORTED;
-    if (p.absmax_out) fill_u32(p.absmax_out, 0u, 1, s);
+    if (p.absmax_out && !slot_zeroed) fill_u32(p.absmax_out, 0u, 1, s);
     int64_t readable = 0;
     const int vec = row_vec(p.A, p.lda, p.Kr, &readable);
     p.a_row_bytes = readable;
@@ -881,9 +906,9 @@ static void launch_fq_mode(const FqParams& p, hipStream_t s) {
 #undef TANGO_FQ_IT
 }
 
-static int launch_fq(const FqParams& p, int round_mode, hipStream_t s) {
+static int launch_fq(const FqParams& p, int round_mode, hipStream_t s, bool slot_zeroed = false) {
     if (ceil_div(p.M, 64) > INT32_MAX || ceil_div(p.N, 64) > 65535) return TANGO_ERR_UNSUPPORTED;
-    if (p.absmax_out) fill_u32(p.absmax_out, 0u, 1, s);
+    if (p.absmax_out && !slot_zeroed) fill_u32(p.absmax_out, 0u, 1, s);
     const bool v4 = (reinterpret_cast<uintptr_t>(p.X) & 15) == 0 && (p.ldx & 3) == 0;
     if (round_mode == TANGO_ROUND_RNE) {
         if (v4) launch_fq_mode<4, TANGO_ROUND_RNE>(p, s); else launch_fq_mode<2, TANGO_ROUND_RNE>(p, s);
@@ -938,25 +963,31 @@ int tango_qgemm_fwd_ex(float* Y, int64_t ldy, const float* X, int64_t ldx, const
                                            nullptr, 0, 0, stream);
         if (rc != TANGO_OK) return rc;
     }
-    rc = tango_quantize_rows_f32_i8(W, N, K, ldw, scaleW, 0, Wq, K, round_mode, nullptr, 0, 0, stream);
-    if (rc != TANGO_OK) return rc;
-    if (M == 0 || N == 0) return TANGO_OK;
     int8_t* Bp = static_cast<int8_t*>(workspace);
     const int64_t ldb = round_up(K, 64);
-    if (K > 0)
-        hipLaunchKernelGGL(pack_rows_i8_kernel, dim3(grid_for(N * ldb, 256)), dim3(256), 0, s, Bp, ldb,
-                           Wq, K, N, K);
+    if (N > 0 && K > 0) {  // W -> Wq and its packed copy, and the zeroing of scaleY, in one launch
+        const dim3 wgrid(grid_for(N * ldb, 256));
+        if (round_mode == TANGO_ROUND_RNE)
+            hipLaunchKernelGGL(quantize_pack_w_kernel<TANGO_ROUND_RNE>, wgrid, dim3(256), 0, s, W, ldw, scaleW, Wq, Bp,
+                               ldb, N, K, scaleY);
+        else
+            hipLaunchKernelGGL(quantize_pack_w_kernel<TANGO_ROUND_TRUNC>, wgrid, dim3(256), 0, s, W, ldw, scaleW, Wq, Bp,
+                               ldb, N, K, scaleY);
+    } else if (scaleY) {
+        fill_u32(scaleY, 0u, 1, s);
+    }
+    if (M == 0 || N == 0) return launch_status();
     if (fused) {
         FqParams q{};
         q.C = Y; q.X = X; q.Xq = Xq; q.B = Bp; q.bias = bias; q.x_row_mul = x_row_mul; q.absmax_out = scaleY;
         q.sA = scaleX; q.sB = scaleW; q.M = M; q.N = N; q.K = K; q.ldx = ldx; q.ldxq = ldxq; q.ldb = ldb;
         q.ldc = ldy; q.kp = static_cast<int>(ldb);
-        return launch_fq(q, round_mode, s);
+        return launch_fq(q, round_mode, s, true);
     }
     NtParams p{};
     p.C = Y; p.A = Xq; p.B = Bp; p.bias = bias; p.absmax_out = scaleY; p.sA = scaleX; p.sB = scaleW;
     p.M = M; p.N = N; p.Kr = K; p.lda = ldxq; p.ldb = ldb; p.ldc = ldy;
-    return launch_nt(p, s);
+    return launch_nt(p, s, true);
 }
 
 int tango_qgemm_fwd(float* Y, int64_t ldy, const float* X, int64_t ldx, int8_t* Xq, int64_t ldxq,

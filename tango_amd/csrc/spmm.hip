@@ -37,6 +37,7 @@ struct SpmmParams {
     const int8_t* feat;
     const int8_t* evals;
     const float* scale;
+    const float* scale2;     // optional second factor of the dequantization scale (s = scale[0] * scale2[0])
     const float* row_scale;  // optional: out row r is multiplied by row_scale[r] after dequantization
     const float* bias;       // optional: bias[c] added after the row scale
     int relu;                // clamp at zero last
@@ -249,7 +250,7 @@ __device__ __forceinline__ void wave_row_sum(const SpmmParams& p, const LaneCols
 template <int VEC>
 __device__ __forceinline__ void store_row(const SpmmParams& p, const LaneCols& c, int64_t row, const int* acc) {
     if (!c.col_ok) return;
-    const float s = p.scale[0];
+    const float s = p.scale2 ? p.scale[0] * p.scale2[0] : p.scale[0];
     const float rs = p.row_scale ? p.row_scale[row] : 1.0f;
     float* o = p.out + row * p.W + c.col;
     float y[VEC];
@@ -795,7 +796,7 @@ __global__ __launch_bounds__(256) void spmm_span_kernel(const SpmmParams p) {
     int cur_start = 0, my_last_flag = -1, first_target = -2;
     // Rows end at different slots in different groups, so the end-of-row code runs under divergence
     // many times per wavefront: the scale and the lane's bias values are fetched once, here.
-    const float dq = p.scale[0];
+    const float dq = p.scale2 ? p.scale[0] * p.scale2[0] : p.scale[0];
     float breg[VEC];
 #pragma unroll
     for (int i = 0; i < VEC; ++i) breg[i] = (p.bias && c.col + i < p.W) ? p.bias[c.col + i] : 0.0f;
@@ -1159,7 +1160,8 @@ int tango_spmm_csr_copy_u_ex(float* out, const int64_t* indptr, const void* indi
 
 int tango_spmm_csr_u_mul_e_ex(float* out, const int64_t* indptr, const void* indices,
                               const void* edge_ids, int idx_bits, const int8_t* feat, const int8_t* evals,
-                              int edge_major, const float* scale, const float* bias, int64_t rows,
+                              int edge_major, const float* scale, const float* scale2, const float* bias,
+                              int64_t rows,
                               int64_t num_src, int64_t H, int64_t F, int64_t D, int64_t nnz,
                               int64_t max_row_nnz, void* workspace, size_t workspace_bytes,
                               tango_stream_t stream) {
@@ -1175,7 +1177,7 @@ int tango_spmm_csr_u_mul_e_ex(float* out, const int64_t* indptr, const void* ind
     p.out = out; p.indptr = indptr; p.indices = static_cast<const int64_t*>(indices);
     p.edge_ids = static_cast<const int64_t*>(edge_ids); p.idx32 = idx_bits == 32; p.feat = feat;
     p.max_row = max_row_nnz; p.hub_ws = workspace; p.span_ws = workspace;
-    p.evals = evals; p.scale = scale; p.bias = bias; p.rows = rows; p.num_src = num_src; p.ldf = H * F; p.W = H * F; p.F = F; p.D = D;
+    p.evals = evals; p.scale = scale; p.scale2 = scale2; p.bias = bias; p.rows = rows; p.num_src = num_src; p.ldf = H * F; p.W = H * F; p.F = F; p.D = D;
     p.nnz = nnz;
     if (edge_major) {  // evals[nnz, H, D]: the H * D bytes of one edge share a cache sector
         p.ev_se = H * D; p.ev_sh = D; p.ev_sd = 1;
@@ -1196,7 +1198,7 @@ int tango_spmm_csr_u_mul_e(float* out, const int64_t* indptr, const int64_t* ind
                            const int64_t* edge_ids, const int8_t* feat, const int8_t* evals,
                            const float* scale, int64_t rows, int64_t num_src, int64_t H,
                            int64_t F, int64_t D, int64_t nnz, tango_stream_t stream) {
-    return tango_spmm_csr_u_mul_e_ex(out, indptr, indices, edge_ids, 64, feat, evals, 0, scale, nullptr, rows, num_src,
+    return tango_spmm_csr_u_mul_e_ex(out, indptr, indices, edge_ids, 64, feat, evals, 0, scale, nullptr, nullptr, rows, num_src,
                                      H, F, D, nnz, 0, nullptr, 0, stream);
 }
 

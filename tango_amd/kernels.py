@@ -393,17 +393,21 @@ class cuda_kernels:
                                           _stream()), "csr_SPMM")
 
     @staticmethod
-    def multi_cusparse_SPMM(indptr, indices, N, E_T, scale, edge_ids=None, edge_major=False, bias=None, max_row=0):
+    def multi_cusparse_SPMM(indptr, indices, N, E_T, scale, edge_ids=None, edge_major=False, bias=None, max_row=0,
+                            scale2=None):
         """E_T is [H, D, nnz] in CSR slot order, or in edge-id order when the
         slot->edge permutation ``edge_ids`` is passed (gather fused in-kernel).
         With ``edge_major`` the edge values are [nnz, H, D] instead (no transpose pass).
         ``bias`` ([H * F] fp32) is added to every output row after dequantization.  ``max_row``: an
-        upper bound of the longest row if known (0 = unknown)."""
+        upper bound of the longest row if known (0 = unknown).  ``scale2``: the output is dequantized
+        with scale * scale2 (saves the launch that multiplies two 1-element tensors)."""
         _need(indptr, torch.int64, "indptr")
         idx_bits = _need_index(indices, "indices")
         _need(N, torch.int8, "N")
         _need(E_T, torch.int8, "E_T")
         _need(scale, torch.float32, "scale")
+        if scale2 is not None:
+            _need(scale2, torch.float32, "scale2")
         if N.dim() != 3 or E_T.dim() != 3:
             raise RuntimeError("E and N must be 3D tensors")
         k, H, F = N.shape
@@ -427,7 +431,7 @@ class cuda_kernels:
         ws = _workspace(ws_bytes, N.device)
         check(_L.tango_spmm_csr_u_mul_e_ex(_ptr(out), indptr.data_ptr(), _ptr(indices), _ptr(edge_ids), idx_bits,
                                            _ptr(N), _ptr(E_T), int(bool(edge_major)), scale.data_ptr(),
-                                           _ptr(bias), rows, k, H, F, D, nnz, int(max_row), _ptr(ws), ws_bytes,
+                                           _ptr(scale2), _ptr(bias), rows, k, H, F, D, nnz, int(max_row), _ptr(ws), ws_bytes,
                                            _stream()), "multi_cusparse_SPMM")
         return out
 
@@ -664,7 +668,7 @@ def _csr_of(g, reverse):
     return indptr, indices, edge_ids, getattr(g, "max_out_degree" if reverse else "max_in_degree", 0)
 
 
-def multi_cusparse_SPMM(g, N, E_T, scale, reverse=False, edge_major=False, bias=None):
+def multi_cusparse_SPMM(g, N, E_T, scale, reverse=False, edge_major=False, bias=None, scale2=None):
     """E_T is [H, D, nnz] in edge-id order.  cuda/kernels.py:122-136; the
     index_select by edge_ids of the reference happens inside the kernel.
     ``edge_major``: E_T is the quantized edge tensor as it is, [nnz, H, 1]."""
@@ -674,7 +678,7 @@ def multi_cusparse_SPMM(g, N, E_T, scale, reverse=False, edge_major=False, bias=
     if edge_ids is not None and edge_ids.numel() == 0:
         edge_ids = None
     return cuda_kernels.multi_cusparse_SPMM(indptr, indices, N, E_T, scale, edge_ids=edge_ids,
-                                            edge_major=edge_major, bias=bias, max_row=longest)
+                                            edge_major=edge_major, bias=bias, max_row=longest, scale2=scale2)
 
 
 def incidence_SPMM(g, E, scaleE, reverse=False):
