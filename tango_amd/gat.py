@@ -144,11 +144,12 @@ class HGTLayer(nn.Module):
             lin.enable_reduce()
 
     def forward(self, g, h):
-        k, s_k = self.k_linear(h)
+        s_h = cuda_kernels.get_scale(h if h.is_contiguous() else h.contiguous())  # one absmax pass for the three projections of h
+        k, s_k = self.k_linear(h, s_h)
         k, s_k = self.attn_linear(k, s_k)
-        v, s_v = self.v_linear(h)
+        v, s_v = self.v_linear(h, s_h)
         v, s_v = self.msg_linear(v, s_v)
-        q, s_q = self.q_linear(h)
+        q, s_q = self.q_linear(h, s_h)
         k, v, q = (t.view(-1, self.n_heads, self.d_k) for t in (k, v, q))
         t = sddmm_u_dot_v.apply(g, k, q, s_k, s_q) / self.sqrt_dk
         attn = edge_softmax(g, t)
