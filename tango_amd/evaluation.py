@@ -1,0 +1,130 @@
+"""Drivers in the shape of the reference's evaluation scripts, on synthetic graphs.
+
+The reference's drivers load Reddit / PubMed / ogbn-arxiv / DBLP / Amazon through DGL and OGB
+(evaluation/util.py:10-32) and call a ``load_graph_train`` that its tree does not define
+(evaluation/test_gcn.py:173, test_gat.py:238, test_HGT.py:72).  Neither library nor the datasets
+exist here, so ``load_graph`` / ``load_graph_train`` return seeded Chung-Lu graphs with the named
+dataset's node count, edge count, feature width and class count, random features and labels, and
+the 60/20/20 masks the drivers index with.  The training loops time forward + backward per epoch
+with events the way evaluation/test_gcn.py:241-263 does (the reference records its ``backward``
+event before ``loss.backward()``; here it is recorded after).
+
+    python -m tango_amd.evaluation --model gcn --dataset pubmed --epochs 20
+"""
+import argparse
+import math
+
+import numpy as np
+import torch
+import torch.nn as nn
+import torch.nn.functional as F
+
+from .gat import GAT, HGT
+from .gcn import GCN
+from .graph import chung_lu
+from .util import graph_preprocess
+
+# name: (nodes, directed edges before self loops, degree exponent, largest degree or None,
+#        symmetric as loaded by the reference, feature width, classes, generator seed)
+DATASETS = {
+    "pubmed": (19717, 177302, 2.1, None, True, 500, 3, 1),
+    "ogbn-arxiv": (169343, 1166243, 2.2, None, False, 128, 40, 4),
+    "reddit": (232965, 114600000, 2.0, 21000, True, 602, 41, 3),
+    "dblp": (317080, 2099732, 2.3, None, True, 128, 16, 6),
+    "amazon": (410236, 4878874, 2.3, None, True, 128, 16, 7),
+}
+
+
+def load_graph(name, device="cuda"):
+    """evaluation/util.py:10-32: the graph with self loops removed and re-added, on the device,
+    preprocessed.  Synthetic stand-in of the named dataset's size."""
+    if name not in DATASETS:
+        raise ValueError("Unknown dataset: {}".format(name))
+    n, e, gamma, max_deg, sym, _, _, seed = DATASETS[name]
+    g = chung_lu(n, e, gamma, seed=seed, max_degree=max_deg, symmetric=sym, device=device)
+    return graph_preprocess(g)
+
+
+def load_graph_train(name, device="cuda"):
+    """The graph of ``load_graph`` with ``ndata`` feat / label / train_mask / val_mask / test_mask and
+    ``n_classes``, the attributes the reference's training drivers read."""
+    g = load_graph(name, device)
+    n, (_, _, _, _, _, width, classes, seed) = g.num_nodes(), DATASETS[name]
+    gen = torch.Generator().manual_seed(1000 + seed)
+    g.ndata["feat"] = torch.randn(n, width, generator=gen).to(device)
+    g.ndata["label"] = torch.randint(0, classes, (n,), generator=gen).to(device)
+    r = torch.rand(n, generator=gen).to(device)
+    g.ndata["train_mask"], g.ndata["val_mask"], g.ndata["test_mask"] = r < 0.6, (r >= 0.6) & (r < 0.8), r >= 0.8
+    g.n_classes = classes
+    return g
+
+
+def evaluate(model_fn, labels, mask):
+    """evaluation/test_gcn.py:172-181."""
+    with torch.no_grad():
+        logits = model_fn()[mask]
+        return (logits.argmax(1) == labels[mask]).float().mean().item()
+
+
+def train(model_name, dataset, epochs=20, hidden=None, layers=None, heads=8, lr=1e-2, weight_decay=5e-4,
+          quiet=False):
+    """One of the reference's three training drivers (test_gcn.py:183-275, test_gat.py:236-330,
+    test_HGT.py:70-130).  Returns (mean ms per epoch after the first three, final loss)."""
+    g = load_graph_train(dataset)
+    feats, labels, train_mask = g.ndata["feat"], g.ndata["label"], g.ndata["train_mask"]
+    if model_name == "gcn":
+        hidden, layers = hidden or 256, layers or 1
+        model = GCN(g, feats.size(1), hidden, hidden, layers, torch.relu, 0.0).cuda()
+        fwd = lambda: model(feats)
+    elif model_name == "gat":
+        hidden, layers = hidden or 16, layers or 3
+        model = GAT(g, layers, feats.size(1), hidden, g.n_classes, [heads] * (layers - 1) + [1], F.elu).cuda()
+        fwd = lambda: model(feats)
+    elif model_name == "hgt":
+        hidden = hidden or 256
+        model = HGT(feats.size(1), hidden, heads).cuda()
+        fwd = lambda: model(g, feats)
+    else:
+        raise ValueError("model must be gcn, gat or hgt")
+    proj = nn.Linear(hidden, g.n_classes).cuda()  # "proj to predict" (test_gcn.py:229)
+    opt = torch.optim.Adam(list(model.parameters()) + list(proj.parameters()), lr=lr, weight_decay=weight_decay)
+    dur, loss = [], None
+    for epoch in range(epochs):
+        model.train()
+        start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        start.record()
+        logits = proj(fwd())
+        loss = F.cross_entropy(logits[train_mask], labels[train_mask])
+        opt.zero_grad()
+        loss.backward()
+        stop.record()
+        torch.cuda.synchronize()
+        opt.step()
+        if epoch >= 3:
+            dur.append(start.elapsed_time(stop))
+        if not quiet:
+            acc = evaluate(lambda: proj(fwd()), labels, g.ndata["val_mask"])
+            print("Epoch {:05d} | Time(ms) {:.4f} | Loss {:.4f} | Accuracy {:.4f} | ETputs(KTEPS) {:.2f}".format(
+                epoch, np.mean(dur) if dur else float("nan"), loss.item(), acc,
+                g.num_edges() / np.mean(dur) if dur else float("nan")))
+    return (float(np.mean(dur)) if dur else math.nan), float(loss.item())
+
+
+def main():
+    ap = argparse.ArgumentParser(description="quantized GCN / GAT / HGT training on a synthetic stand-in of a dataset")
+    ap.add_argument("--model", choices=["gcn", "gat", "hgt"], default="gcn")
+    ap.add_argument("--dataset", choices=sorted(DATASETS), default="pubmed")
+    ap.add_argument("--epochs", type=int, default=20)
+    ap.add_argument("--n-hidden", type=int, default=None)
+    ap.add_argument("--n-layers", type=int, default=None)
+    ap.add_argument("--num-heads", type=int, default=8)
+    ap.add_argument("--lr", type=float, default=1e-2)
+    ap.add_argument("--weight-decay", type=float, default=5e-4)
+    args = ap.parse_args()
+    ms, loss = train(args.model, args.dataset, args.epochs, args.n_hidden, args.n_layers, args.num_heads, args.lr,
+                     args.weight_decay)
+    print("mean fwd+bwd {:.3f} ms/epoch, final loss {:.4f}".format(ms, loss))
+
+
+if __name__ == "__main__":
+    main()

@@ -166,3 +166,18 @@ def test_edge_renumbering_leaves_node_outputs_unchanged():
     assert torch.allclose(att[0][g1.edge_order], att[1], rtol=1e-5, atol=1e-7)
     for a, b in zip(*grads):
         assert torch.allclose(a, b, rtol=1e-3, atol=1e-4 * float(a.abs().max()))
+
+
+@pytest.mark.parametrize("model", ["gcn", "gat", "hgt"])
+def test_evaluation_drivers_train_on_the_pubmed_stand_in(model):
+    """tango_amd.evaluation: the reference's three training loops (evaluation/test_gcn.py,
+    test_gat.py, test_HGT.py) on the synthetic graph with PubMed's sizes."""
+    from tango_amd import evaluation
+    torch.manual_seed(11)
+    g = evaluation.load_graph_train("pubmed")
+    assert g.num_nodes() == 19717 and g.ndata["feat"].shape == (19717, 500) and g.n_classes == 3
+    assert int(g.ndata["train_mask"].sum() + g.ndata["val_mask"].sum() + g.ndata["test_mask"].sum()) == 19717
+    first_ms, first_loss = evaluation.train(model, "pubmed", epochs=1, quiet=True)
+    torch.manual_seed(11)
+    ms, loss = evaluation.train(model, "pubmed", epochs=12, quiet=True, lr=5e-3)
+    assert np.isfinite(ms) and ms > 0 and np.isfinite(loss) and loss < first_loss
