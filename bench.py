@@ -117,6 +117,18 @@ def primitives(g, K, torch):
     out["spmm_u_mul_e_H2_F128"] = {"ms": round(ms, 4), "GBps": round(b / ms / 1e6, 1),
                                    "frac_hbm": round(b / ms / 1e6 / HBM_PEAK_GBPS, 4)}
     del feat, ev
+    # u_mul_e without broadcast: every head has one feature column and its own edge value
+    # (evaluation/SPMM_nobroadcast.py:27-29: N [n, H, 1], E [nnz, H, 1]); and the incidence form (copy_e)
+    H = 8
+    feat = torch.randint(-127, 128, (n, H, 1), dtype=torch.int8, device="cuda")
+    ev = torch.randint(-127, 128, (nnz, H, 1), dtype=torch.int8, device="cuda")
+    ms = time_op(lambda: K.multi_cusparse_SPMM(g, feat, ev, one, edge_major=True), iters=5)
+    b = nnz * (H + H + 2 * IDX_BYTES) + n * (4 * H + 8)
+    out["spmm_u_mul_e_nobroadcast_H8"] = {"ms": round(ms, 4), "GBps": round(b / ms / 1e6, 1)}
+    ms = time_op(lambda: K.incidence_SPMM(g, ev.view(nnz, H), one), iters=5)
+    b = nnz * (H + IDX_BYTES) + n * (4 * H + 8)
+    out["spmm_incidence_F8"] = {"ms": round(ms, 4), "GBps": round(b / ms / 1e6, 1)}
+    del feat, ev
     # QLinear forward / backward at (M, K, N) = (232965, 602, 256) and (232965, 256, 41)
     for (M, Kd, N) in ((n, 602, 256), (n, 256, 41), (n, 128, 16)):
         X = torch.randn(M, Kd, device="cuda")
