@@ -61,6 +61,7 @@ struct SpmmParams {
     int64_t group_row; // sparse graphs: rows with at most this many slots are owned by a lane group
     void* span_ws;     // sparse graphs: caller's workspace for the slot-span path, or null
     int64_t span_wp;   // padded row width (int32 entries) of a partial row in span_ws
+    size_t span_ws_bytes;
 };
 
 enum { KIND_COPY = 0, KIND_WEIGHTED = 1, KIND_COO = 2 };
@@ -1049,8 +1050,11 @@ static int launch_spmm(SpmmParams p, int vec, hipStream_t s) {
             hipLaunchKernelGGL((spmm_hub_store_kernel<V, KIND>), sgrid, dim3(256), 0, s, p);        \
         }                                                                                           \
     } while (0)
-    if (KIND != KIND_COO && p.span_ws && span_graph(p.rows, p.nnz)) {  // sparse graph: slot spans, two launches
-        const int64_t nspans = ceil_div(p.nnz, kSpanSlots);
+    const int64_t nspans_all = ceil_div(p.nnz, kSpanSlots);
+    const bool span_fits = span_parts_offset(nspans_all) + sizeof(int) * 2 * static_cast<size_t>(nspans_all) *
+                               static_cast<size_t>(ychunks * p.tile) <= p.span_ws_bytes;
+    if (KIND != KIND_COO && p.span_ws && span_fits && span_graph(p.rows, p.nnz)) {  // sparse graph: slot spans, two launches
+        const int64_t nspans = nspans_all;
         p.span_wp = ychunks * p.tile;
         const dim3 spgrid(static_cast<unsigned>(ceil_div(nspans > 0 ? nspans : 1, 4)), static_cast<unsigned>(ychunks));
         const size_t lds = span_lds_bytes(p.lpe_log2, vec);
@@ -1118,9 +1122,12 @@ extern "C" {
 
 size_t tango_spmm_workspace(int64_t rows, int64_t nnz, int64_t W) {
     if (rows < 0 || nnz < 0 || W < 0) return 0;
-    if (span_graph(rows, nnz)) {  // two int32 partial rows per span; the padded width is at most 2 W + 1024
+    if (span_graph(rows, nnz)) {
+        // two int32 partial rows per span.  Their padded width is column tiles x tile: below 2 W + 16 while the
+        // lanes of a row piece fit a wavefront (tile = vec x the lane count rounded up to a power of two), and
+        // below W + 64 vec < 2 W once they do not
         const int64_t nspans = ceil_div(nnz, kSpanSlots);
-        return span_parts_offset(nspans) + sizeof(int) * 2 * static_cast<size_t>(nspans) * static_cast<size_t>(2 * W + 1024);
+        return span_parts_offset(nspans) + sizeof(int) * 2 * static_cast<size_t>(nspans) * static_cast<size_t>(2 * W + 16);
     }
     return 64 + sizeof(int64_t) * static_cast<size_t>(nnz / kHubRowMin + 2);
 }
@@ -1153,7 +1160,7 @@ int tango_spmm_csr_copy_u_ex(float* out, const int64_t* indptr, const void* indi
     p.out = out; p.indptr = indptr; p.indices = static_cast<const int64_t*>(indices); p.idx32 = idx_bits == 32;
     p.feat = feat; p.scale = scale;
     p.row_scale = row_scale; p.bias = bias; p.relu = relu ? 1 : 0; p.max_row = max_row_nnz; p.hub_ws = workspace;
-    p.span_ws = workspace;
+    p.span_ws = workspace; p.span_ws_bytes = workspace_bytes;
     p.rows = rows; p.num_src = num_src; p.ldf = ldf; p.W = F; p.F = F; p.D = 1; p.nnz = nnz;
     return launch_spmm<KIND_COPY>(p, pick_vec(feat, ldf, F), as_stream(stream));
 }
@@ -1176,7 +1183,7 @@ int tango_spmm_csr_u_mul_e_ex(float* out, const int64_t* indptr, const void* ind
     SpmmParams p{};
     p.out = out; p.indptr = indptr; p.indices = static_cast<const int64_t*>(indices);
     p.edge_ids = static_cast<const int64_t*>(edge_ids); p.idx32 = idx_bits == 32; p.feat = feat;
-    p.max_row = max_row_nnz; p.hub_ws = workspace; p.span_ws = workspace;
+    p.max_row = max_row_nnz; p.hub_ws = workspace; p.span_ws = workspace; p.span_ws_bytes = workspace_bytes;
     p.evals = evals; p.scale = scale; p.scale2 = scale2; p.bias = bias; p.rows = rows; p.num_src = num_src; p.ldf = H * F; p.W = H * F; p.F = F; p.D = D;
     p.nnz = nnz;
     if (edge_major) {  // evals[nnz, H, D]: the H * D bytes of one edge share a cache sector
