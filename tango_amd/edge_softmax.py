@@ -6,11 +6,17 @@ from torch.autograd.function import Function, once_differentiable
 from .kernels import cuda_kernels
 
 
+def _dst_major(g):
+    """(indptr, slot -> edge id or None when the slots are in edge-id order) of the destination-major CSR."""
+    indptr, _, eids = g.adj_csc
+    return indptr, (None if getattr(g, "csc_slots_are_edge_ids", False) else eids)
+
+
 class _EdgeSoftmax(Function):
     @staticmethod
     def forward(ctx, g, e, slope):
         e = e if e.is_contiguous() else e.contiguous()
-        indptr, _, eids = g.adj_csc
+        indptr, eids = _dst_major(g)
         a = cuda_kernels.edge_softmax_forward(e, indptr, eids, slope)
         ctx.backward_cache = g, e, a, slope
         return a
@@ -19,7 +25,7 @@ class _EdgeSoftmax(Function):
     @once_differentiable
     def backward(ctx, da):
         g, e, a, slope = ctx.backward_cache
-        indptr, _, eids = g.adj_csc
+        indptr, eids = _dst_major(g)
         da = da if da.is_contiguous() else da.contiguous()
         return None, cuda_kernels.edge_softmax_backward(a, da, e, indptr, eids, slope), None
 

@@ -665,6 +665,8 @@ def _csr_of(g, reverse):
     narrow = getattr(g, "adj_csr32" if reverse else "adj_csc32", None)
     if narrow is not None:
         indices, edge_ids = narrow
+    if getattr(g, "csr_slots_are_edge_ids" if reverse else "csc_slots_are_edge_ids", False):
+        edge_ids = None  # identity: edge tensors are addressed by the slot itself
     return indptr, indices, edge_ids, getattr(g, "max_out_degree" if reverse else "max_in_degree", 0)
 
 
@@ -687,6 +689,9 @@ def incidence_SPMM(g, E, scaleE, reverse=False):
     already holds, so the row bounds come from indptr instead of a search in the COO node ids."""
     assert E.is_cuda and scaleE.is_cuda
     indptr, _, edge_ids, longest = _csr_of(g, reverse)
+    if edge_ids is None:  # slot order = edge-id order: here the ids are the gather indices, identity or not
+        narrow = getattr(g, "adj_csr32" if reverse else "adj_csc32", None)
+        edge_ids = narrow[1] if narrow is not None else (g.adj_csr if reverse else g.adj_csc)[2]
     out_shape = (g.num_nodes(),) + E.shape[1:]
     dim = math.prod(E.shape[1:])
     out = torch.empty((g.num_nodes(), dim), dtype=torch.float32, device=E.device)

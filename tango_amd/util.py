@@ -23,6 +23,12 @@ def graph_preprocess(graph):
     # and at 4 bytes per edge they cost half the traffic of the int64 arrays the reference passes.
     graph.adj_csr32 = tuple(t.to(torch.int32) for t in graph.adj_csr[1:])
     graph.adj_csc32 = tuple(t.to(torch.int32) for t in graph.adj_csc[1:])
+    # whether a CSR's slot order is the edge-id order itself (edges already sorted by that endpoint, e.g.
+    # after Graph.reorder_edges_by_dst): the kernels then skip the slot -> edge-id indirection altogether
+    ar = torch.arange(graph.adj_csr[2].numel(), device=graph.adj_csr[2].device)
+    graph.csr_slots_are_edge_ids = bool(torch.equal(graph.adj_csr[2], ar))
+    graph.csc_slots_are_edge_ids = bool(torch.equal(graph.adj_csc[2], ar))
+    del ar
     # the longest row of either orientation (one host read per graph): tells the aggregation
     # kernels whether the launches that exist for hub rows are needed at all
     graph.max_out_degree = int(torch.diff(graph.adj_csr[0]).max().item()) if graph.adj_csr[0].numel() > 1 else 0
