@@ -278,7 +278,20 @@ __global__ __launch_bounds__(256, 2) void gemm_fq_kernel(const FqParams p) {
             }
         }
     };
-    {
+    if (IT == 1 && RT == 4 && TPW <= 2) {
+        // rows of at most 256 columns, at most 128 output columns: all sixteen rows of the wave are requested
+        // at once (64 registers), so the phase pays the memory latency once instead of four times
+        // (232,965 x 256 x 41: 0.092 -> 0.085 ms; at 256 output columns it measured 3 % slower)
+        float f0[4][IT][4], f1[4][IT][4], f2[4][IT][4], f3[4][IT][4];
+        fetch(f0, 0);
+        fetch(f1, 4);
+        fetch(f2, 8);
+        fetch(f3, 12);
+        emit(f0, 0);
+        emit(f1, 4);
+        emit(f2, 8);
+        emit(f3, 12);
+    } else {
         // two register buffers: the loads of the next four rows are in flight while these are quantized
         float fa[4][IT][4], fb[4][IT][4];
         fetch(fa, 0);
