@@ -65,9 +65,30 @@ def _rows_view(t, name):
     return t.stride(0) if t.size(0) > 1 else max(t.size(1), t.stride(0))
 
 
+_WS_BUFFERS = {}  # (device index, raw stream) -> uint8 tensor, grown on demand
+_WS_SIZES = {}    # (size query, arguments) -> bytes
+
+
 def _workspace(nbytes, device):
-    """Scratch for one call, from torch's caching allocator (no hipMalloc on the hot path)."""
-    return torch.empty(nbytes, dtype=torch.uint8, device=device) if nbytes else None
+    """Scratch for one call.  One buffer per (device, stream), grown on demand and reused: calls on a
+    stream run in order, so the next call's kernels cannot start before this call's are done with it.
+    (The reference allocates its temporaries from torch's allocator in every call.)"""
+    if not nbytes:
+        return None
+    key = (device.index, _stream())
+    buf = _WS_BUFFERS.get(key)
+    if buf is None or buf.numel() < nbytes:
+        buf = _WS_BUFFERS[key] = torch.empty(max(int(nbytes), 1 << 20), dtype=torch.uint8, device=device)
+    return buf
+
+
+def _ws_bytes(query, *args):
+    """A workspace size query of the library, answered from a table after the first time."""
+    key = (query, args)
+    n = _WS_SIZES.get(key)
+    if n is None:
+        n = _WS_SIZES[key] = getattr(_L, query)(*args)
+    return n
 
 
 _ZERO_SLOTS = {}   # device -> [pool tensor, next free index]
@@ -225,7 +246,7 @@ class cuda_kernels:
         if not accumulate:
             scale = torch.empty(1, dtype=torch.float32, device=inp.device)
         colsum = torch.empty(cols, dtype=torch.float32, device=inp.device) if want_colsum else None
-        ws_bytes = _L.tango_absmax_ex_workspace(rows, cols, int(want_colsum))
+        ws_bytes = _ws_bytes("tango_absmax_ex_workspace", rows, cols, int(want_colsum))
         ws = _workspace(ws_bytes, inp.device)
         check(_L.tango_absmax_ex_f32(_ptr(inp), rows, cols, ldx, _ptr(row_mul), _ptr(mask), ldm,
                                      scale.data_ptr(), int(accumulate), _ptr(colsum), _ptr(ws), ws_bytes,
@@ -264,7 +285,7 @@ class cuda_kernels:
         if scaleY is not None and scaleY.numel():
             _need(scaleY, torch.float32, "scaleY")
         mode = default_forward_round_mode() if round_mode is None else _mode(round_mode)
-        ws_bytes = _L.tango_qgemm_fwd_workspace(M, N, K)
+        ws_bytes = _ws_bytes("tango_qgemm_fwd_workspace", M, N, K)
         ws = _workspace(ws_bytes, X.device)
         if x_row_mul is not None:
             _need(x_row_mul, torch.float32, "x_row_mul")
@@ -286,7 +307,7 @@ class cuda_kernels:
         N = B.size(0)
         if B.size(1) != K or tuple(Y.shape) != (M, N):
             raise RuntimeError("QGEMM_i8: shape mismatch")
-        ws_bytes = _L.tango_qgemm_i8_nt_workspace(M, N, K)
+        ws_bytes = _ws_bytes("tango_qgemm_i8_nt_workspace", M, N, K)
         ws = _workspace(ws_bytes, A.device)
         check(_L.tango_qgemm_i8_nt(_ptr(Y), _rows_view(Y, "Y"), _ptr(A), _rows_view(A, "A"), _ptr(B),
                                    _rows_view(B, "B"), _ptr(bias), _ptr(scaleY), scaleA.data_ptr(),
@@ -303,7 +324,7 @@ class cuda_kernels:
         N = dY.size(1)
         if dY.size(0) != M or tuple(W.shape) != (N, K):
             raise RuntimeError("QGEMM_backward_gradX: shape mismatch")
-        ws_bytes = _L.tango_qgemm_bwd_dx_workspace(M, N, K)
+        ws_bytes = _ws_bytes("tango_qgemm_bwd_dx_workspace", M, N, K)
         ws = _workspace(ws_bytes, dY.device)
         if row_scale is not None:
             _need(row_scale, torch.float32, "row_scale")
@@ -323,7 +344,7 @@ class cuda_kernels:
         M = dY.size(0)
         if dY.size(1) != N or tuple(X.shape) != (M, K):
             raise RuntimeError("QGEMM_backward_gradW: shape mismatch")
-        ws_bytes = _L.tango_qgemm_bwd_dw_workspace(M, N, K)
+        ws_bytes = _ws_bytes("tango_qgemm_bwd_dw_workspace", M, N, K)
         ws = _workspace(ws_bytes, X.device)
         check(_L.tango_qgemm_bwd_dw(_ptr(dW), _rows_view(dW, "dW"), _ptr(dY), _rows_view(dY, "dY"),
                                     _ptr(X), _rows_view(X, "X"), scaledY.data_ptr(), scaleX.data_ptr(),
@@ -339,7 +360,7 @@ class cuda_kernels:
         if (B.size(1) if trans_b else B.size(0)) != k:
             raise RuntimeError("Qgemm: inner dimensions differ")
         out = torch.empty((m, n), dtype=torch.float32, device=A.device)
-        ws_bytes = _L.tango_qgemm_legacy_workspace(m, n, k)
+        ws_bytes = _ws_bytes("tango_qgemm_legacy_workspace", m, n, k)
         ws = _workspace(ws_bytes, A.device)
         check(_L.tango_qgemm_legacy(_ptr(out), _ptr(A), _ptr(B), m, n, k, int(trans_a), int(trans_b),
                                     _ptr(ws), ws_bytes, _stream()), "Qgemm")
@@ -385,7 +406,7 @@ class cuda_kernels:
             _need(bias, torch.float32, "bias")
             if bias.numel() != F:
                 raise RuntimeError("csr_SPMM: bias must have F entries")
-        ws_bytes = _L.tango_spmm_workspace(rows, indices.numel(), F)
+        ws_bytes = _ws_bytes("tango_spmm_workspace", rows, indices.numel(), F)
         ws = _workspace(ws_bytes, U.device)
         check(_L.tango_spmm_csr_copy_u_ex(_ptr(out), indptr.data_ptr(), _ptr(indices), idx_bits, _ptr(U), ldf,
                                           scaleU.data_ptr(), _ptr(row_scale), _ptr(bias), int(bool(relu)),
@@ -427,7 +448,7 @@ class cuda_kernels:
                 raise RuntimeError("multi_cusparse_SPMM: bias must have H * F elements")
         rows = indptr.numel() - 1
         out = torch.empty((rows, H, F), dtype=torch.float32, device=N.device)
-        ws_bytes = _L.tango_spmm_workspace(rows, nnz, H * F)
+        ws_bytes = _ws_bytes("tango_spmm_workspace", rows, nnz, H * F)
         ws = _workspace(ws_bytes, N.device)
         check(_L.tango_spmm_csr_u_mul_e_ex(_ptr(out), indptr.data_ptr(), _ptr(indices), _ptr(edge_ids), idx_bits,
                                            _ptr(N), _ptr(E_T), int(bool(edge_major)), scale.data_ptr(),
@@ -497,7 +518,7 @@ class cuda_kernels:
         _need(indptr, torch.int64, "indptr")
         H = e.numel() // max(e.size(0), 1)
         a = torch.empty_like(e)
-        ws_bytes = _L.tango_edge_softmax_workspace(e.size(0), H)
+        ws_bytes = _ws_bytes("tango_edge_softmax_workspace", e.size(0), H)
         ws = _workspace(ws_bytes, e.device)
         check(_L.tango_edge_softmax_fwd(_ptr(a), _ptr(e), indptr.data_ptr(), _ptr(edge_ids),
                                         indptr.numel() - 1, e.size(0), H, float(slope), _ptr(ws), ws_bytes,
@@ -512,7 +533,7 @@ class cuda_kernels:
         _need(e, torch.float32, "e")
         H = e.numel() // max(e.size(0), 1)
         de = torch.empty_like(e)
-        ws_bytes = _L.tango_edge_softmax_workspace(e.size(0), H)
+        ws_bytes = _ws_bytes("tango_edge_softmax_workspace", e.size(0), H)
         ws = _workspace(ws_bytes, e.device)
         check(_L.tango_edge_softmax_bwd(_ptr(de), _ptr(a), _ptr(da), _ptr(e), indptr.data_ptr(),
                                         _ptr(edge_ids), indptr.numel() - 1, e.size(0), H, float(slope), _ptr(ws),
@@ -546,7 +567,7 @@ class cuda_kernels:
         dfeat = torch.empty_like(feat)
         dal = torch.empty((H, D), dtype=torch.float32, device=feat.device)
         dar = torch.empty((H, D), dtype=torch.float32, device=feat.device)
-        ws_bytes = _L.tango_attn_scores_bwd_workspace(n, H, D)
+        ws_bytes = _ws_bytes("tango_attn_scores_bwd_workspace", n, H, D)
         ws = _workspace(ws_bytes, feat.device)
         check(_L.tango_attn_scores_bwd(_ptr(dfeat), _ptr(dal), _ptr(dar), _ptr(del_), _ptr(der), _ptr(feat),
                                        _ptr(attn_l), _ptr(attn_r), n, H, D, _ptr(ws), ws_bytes, _stream()),
@@ -580,8 +601,12 @@ def quantize_padded(t, scale=None, round_mode=ROUND_RNE, noise=None, seed=0, off
     rows, cols = t.shape
     ld = (cols + align - 1) // align * align
     buf = torch.empty((rows, ld), dtype=torch.int8, device=t.device)
-    cuda_kernels.quantize_rows(buf, t, scale, round_mode=round_mode, noise=noise, seed=seed, offset=offset,
-                               row_mul=row_mul, mask=mask)
+    if ld == cols and row_mul is None and mask is None and t.is_contiguous():
+        # nothing to pad: the flat kernel (16-byte loads front to back, same element -> noise index mapping)
+        cuda_kernels.quantize(buf, t, scale, round_mode=round_mode, noise=noise, seed=seed, offset=offset)
+    else:
+        cuda_kernels.quantize_rows(buf, t, scale, round_mode=round_mode, noise=noise, seed=seed, offset=offset,
+                                   row_mul=row_mul, mask=mask)
     return buf[:, :cols], scale
 
 
