@@ -75,6 +75,9 @@ def _workspace(nbytes, device):
     (The reference allocates its temporaries from torch's allocator in every call.)"""
     if not nbytes:
         return None
+    if torch.cuda.is_current_stream_capturing():
+        # a graph's allocations live in its own pool and must stay with the graph, not in this table
+        return torch.empty(int(nbytes), dtype=torch.uint8, device=device)
     key = (device.index, _stream())
     buf = _WS_BUFFERS.get(key)
     if buf is None or buf.numel() < nbytes:
