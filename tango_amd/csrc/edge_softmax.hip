@@ -338,7 +338,7 @@ __global__ __launch_bounds__(256) void span_kernel(
         const int j = g * K + k;
         if (id[k] < 0 || j < hpos || j >= tpos) continue;
         if (FWD) {
-            out[id[k]] = x[k] * (1.0f / rs[k]);
+            out[id[k]] = x[k] * __builtin_amdgcn_rcpf(rs[k]);  // 1 ulp: an IEEE divide is ten instructions per value
         } else {
             float gr = x[k] * (y[k] - rs[k]);
             if (!(e[id[k]] > 0.0f)) gr *= slope;
@@ -456,7 +456,7 @@ __global__ __launch_bounds__(256) void span_rest_kernel(
         if (FWD) {
 #pragma unroll
             for (int i = 0; i < HB; ++i)
-                o[i] = expf(leaky(z[i], slope) - (piece ? rm[1][i] : rm[0][i])) * (1.0f / (piece ? rs[1][i] : rs[0][i]));
+                o[i] = expf(leaky(z[i], slope) - (piece ? rm[1][i] : rm[0][i])) * __builtin_amdgcn_rcpf(piece ? rs[1][i] : rs[0][i]);
         } else {
             float x[HB], y[HB];
             load_heads<HB, VEC>(x, a + id, nh);
