@@ -83,21 +83,24 @@ int tango_quantize_rows_f32_i8(const float* x, int64_t rows, int64_t cols, int64
 
 /* Fused forms of the two calls above for a layer's glue (no counterpart in the
    reference, whose drivers run these steps as separate torch passes,
-   evaluation/test_gcn.py:86-94,123-137): every element is first multiplied by
-   row_mul[r] (when non-null; one fp32 rounding) and replaced by zero where
-   mask[r, c] (row stride ldm) is not positive (when non-null).
-   tango_absmax_ex_f32 writes scale_out[0] = max|x*row_mul| / 127 over unmasked
-   elements and, when colsum_out is non-null, colsum_out[c] = sum_r of the
-   unmasked x[r, c] (not multiplied), reduced in a fixed order.  cols <= 1024.
+   evaluation/test_gcn.py:86-94,123-137): every
+   element first passes backwards through the activation whose forward output (or any
+   tensor of its sign) is mask[r, c] (row stride ldm; when non-null), then is multiplied
+   by row_mul[r] (when non-null; one fp32 rounding).  mask_mode 0 (ReLU): x becomes zero
+   where mask is not positive.  mask_mode 1 (ELU, mask = the activation's output):
+   x becomes x * (mask + 1) where mask is not positive.
+   tango_absmax_ex_f32 writes scale_out[0] = max|x'*row_mul| / 127 of the elements x' so
+   masked and, when colsum_out is non-null, colsum_out[c] = sum_r x'[r, c]
+   (not multiplied), reduced in a fixed order.  cols <= 1024.
    accumulate != 0: scale_out[0] already holds 0 or a partial result and is maxed into
    (as tango_absmax_acc_f32); otherwise it need not be initialised.
    workspace: tango_absmax_ex_workspace(rows, cols, colsum_out != NULL) bytes. */
 size_t tango_absmax_ex_workspace(int64_t rows, int64_t cols, int want_colsum);
 int tango_absmax_ex_f32(const float* x, int64_t rows, int64_t cols, int64_t ldx, const float* row_mul,
-                        const float* mask, int64_t ldm, float* scale_out, int accumulate,
+                        const float* mask, int64_t ldm, int mask_mode, float* scale_out, int accumulate,
                         float* colsum_out, void* workspace, size_t workspace_bytes, tango_stream_t stream);
 int tango_quantize_rows_ex_f32_i8(const float* x, int64_t rows, int64_t cols, int64_t ldx,
-                                  const float* row_mul, const float* mask, int64_t ldm,
+                                  const float* row_mul, const float* mask, int64_t ldm, int mask_mode,
                                   const float* scale, int per_row, int8_t* q, int64_t ldq,
                                   int round_mode, const float* noise, uint64_t seed,
                                   uint64_t offset, tango_stream_t stream);
@@ -197,7 +200,8 @@ int tango_spmm_csr_copy_u(float* out, const int64_t* indptr, const int64_t* indi
 /* As tango_spmm_csr_copy_u with the layer glue that follows the aggregation in
    evaluation/test_gcn.py:123-137 folded into the epilogue, in this order and with
    one fp32 rounding each: y = scale * float(sum); y *= row_scale[r] (if non-null);
-   y += bias[f] (if non-null); y = max(y, 0) (if relu).
+   y += bias[f] (if non-null); then relu = 1: y = max(y, 0); relu = 2: y = y > 0 ? y : exp(y) - 1
+   (ELU, alpha 1); relu = 0: nothing.
    idx_bits: 64 (int64 indices, as the reference passes them) or 32 (a one-time int32
    copy of the column indices made by the caller: half the index traffic).
    max_row_nnz: an upper bound of the longest row if the caller knows one (a graph
@@ -234,7 +238,9 @@ int tango_spmm_csr_u_mul_e(float* out, const int64_t* indptr, const int64_t* ind
    quantizing the [nnz, H, D] fp32 edge tensor in place yields, no transpose pass).
    With the slot->edge permutation fused, the H * D bytes of a gathered edge then
    come from one cache sector instead of H * D scattered ones.  bias (H * F floats or
-   NULL) is added after dequantization ("rst + bias", evaluation/test_gat.py:160-162).
+   NULL) is added after dequantization ("rst + bias", evaluation/test_gat.py:160-162);
+   act then applies the layer's activation (evaluation/test_gat.py:164-165) with the codes
+   of tango_spmm_csr_copy_u_ex's relu: 0 none, 1 ReLU, 2 ELU.
    scale2 (or NULL): the dequantization scale is scale[0] * scale2[0] (the scales of the
    node features and of the edge values, multiplied by a torch op in cuda/SPMM.py:44).
    idx_bits: width of the entries of indices and edge_ids, 64 or 32; max_row_nnz and
@@ -242,7 +248,7 @@ int tango_spmm_csr_u_mul_e(float* out, const int64_t* indptr, const int64_t* ind
 int tango_spmm_csr_u_mul_e_ex(float* out, const int64_t* indptr, const void* indices,
                               const void* edge_ids, int idx_bits, const int8_t* feat, const int8_t* evals,
                               int edge_major, const float* scale, const float* scale2, const float* bias,
-                              int64_t rows, int64_t num_src, int64_t H, int64_t F, int64_t D, int64_t nnz,
+                              int act, int64_t rows, int64_t num_src, int64_t H, int64_t F, int64_t D, int64_t nnz,
                               int64_t max_row_nnz, void* workspace, size_t workspace_bytes,
                               tango_stream_t stream);
 

@@ -86,10 +86,13 @@ class spmm_u_mul_e(Function):
 
     ``bias`` ([H * F]) folds the "rst + bias" that follows the aggregation in a GAT layer
     (evaluation/test_gat.py:160-162) into the kernel's epilogue; its gradient then comes
-    out of the pass that finds the scale of dZ.  ``scaleN`` may come from the producer of N."""
+    out of the pass that finds the scale of dZ.  ``scaleN`` may come from the producer of N.
+    ``act`` ("relu" or "elu") folds the layer's activation (evaluation/test_gat.py:164-165) in as
+    well: the epilogue applies it, and the backward pass takes dZ back through it inside the two
+    kernels that read dZ anyway (scale / bias gradient, quantize) instead of a separate pass."""
 
     @staticmethod
-    def forward(ctx, g, N, E, bias=None, scaleN=None):
+    def forward(ctx, g, N, E, bias=None, scaleN=None, act=None):
         N = N if N.is_contiguous() else N.contiguous()
         E = E if E.is_contiguous() else E.contiguous()
         # Edge values stay edge-major ([nnz, H, 1], plain quantize): the reference transposes them to
@@ -98,17 +101,29 @@ class spmm_u_mul_e(Function):
         E_T_, scaleE = quantize(E)
         N_, scaleN = quantize(N, scaleN)  # one absmax pass (the reference runs two, cuda/SPMM.py:39,43)
         # dequantized with scaleN * scaleE (cuda/SPMM.py:44); the kernel multiplies the two itself
-        out = multi_cusparse_SPMM(g, N_, E_T_, scaleN, edge_major=True, bias=bias, scale2=scaleE)
+        out = multi_cusparse_SPMM(g, N_, E_T_, scaleN, edge_major=True, bias=bias, scale2=scaleE, act=act)
         reduce_last = _need_reduce_last_dim(N, E)
-        ctx.backward_cache = g, N_, scaleN, E_T_, scaleE, reduce_last, E.shape, bias is not None
+        ctx.backward_cache = (g, N_, scaleN, E_T_, scaleE, reduce_last, E.shape, bias is not None, act,
+                              out if act is not None else None)
         return out
 
     @staticmethod
     @once_differentiable
     def backward(ctx, dZ):
-        g, N_, scaleN, E_T_, scaleE, reduce_last, eshape, has_bias = ctx.backward_cache
+        g, N_, scaleN, E_T_, scaleE, reduce_last, eshape, has_bias, act, out = ctx.backward_cache
         dbias = None
-        if has_bias and ctx.needs_input_grad[3]:
+        if act is not None:
+            # dZ goes back through the activation on its way into the scale, the bias gradient and int8
+            dZ = dZ if dZ.is_contiguous() else dZ.contiguous()
+            dZ2, out2 = dZ.view(dZ.size(0), -1), out.view(out.size(0), -1)
+            scaledZ, dbias = cuda_kernels.absmax_ex(dZ2, mask=out2, mask_mode=act,
+                                                    want_colsum=has_bias and ctx.needs_input_grad[3])
+            kw = {"round_mode": config.grad_round_mode}
+            if config.grad_round_mode == "stochastic":
+                kw.update(seed=config.seed, offset=config.next_offset())
+            dZ_, _ = quantize_padded(dZ2, scaledZ, mask=out2, mask_mode=act, align=1, **kw)
+            dZ_ = dZ_.view(dZ.shape)
+        elif has_bias and ctx.needs_input_grad[3]:
             # the scale of dZ and the bias gradient (column sums) in one read
             dZ = dZ if dZ.is_contiguous() else dZ.contiguous()
             scaledZ, dbias = cuda_kernels.absmax_ex(dZ.view(dZ.size(0), -1), want_colsum=True)
@@ -128,4 +143,4 @@ class spmm_u_mul_e(Function):
             op = "dot" if reduce_last else "mul"
             dE, _ = mySDDMM_int8(g, op, N_, dZ_, scaleN, scaledZ, False)
             dE = dE.reshape(eshape)
-        return None, dN, dE, dbias, None
+        return None, dN, dE, dbias, None, None

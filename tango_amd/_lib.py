@@ -26,8 +26,8 @@ SIGNATURES = {
     "tango_quantize_f32_i8": (I, [P, I64, P, P, I, P, U64, U64, P]),
     "tango_quantize_rows_f32_i8": (I, [P, I64, I64, I64, P, I, P, I64, I, P, U64, U64, P]),
     "tango_absmax_ex_workspace": (SZ, [I64, I64, I]),
-    "tango_absmax_ex_f32": (I, [P, I64, I64, I64, P, P, I64, P, I, P, P, SZ, P]),
-    "tango_quantize_rows_ex_f32_i8": (I, [P, I64, I64, I64, P, P, I64, P, I, P, I64, I, P, U64, U64, P]),
+    "tango_absmax_ex_f32": (I, [P, I64, I64, I64, P, P, I64, I, P, I, P, P, SZ, P]),
+    "tango_quantize_rows_ex_f32_i8": (I, [P, I64, I64, I64, P, P, I64, I, P, I, P, I64, I, P, U64, U64, P]),
     "tango_transpose_quant_f32_i8": (I, [P, I64, I64, P, P, P]),
     "tango_qgemm_fwd_workspace": (SZ, [I64, I64, I64]),
     "tango_qgemm_fwd": (I, [P, I64, P, I64, P, I64, P, I64, P, P, P, P, P, I64, I64, I64, I, P, SZ, P]),
@@ -45,7 +45,7 @@ SIGNATURES = {
     "tango_spmm_workspace": (SZ, [I64, I64, I64]),
     "tango_spmm_csr_copy_u_ex": (I, [P, P, P, I, P, I64, P, P, P, I, I64, I64, I64, I64, I64, P, SZ, P]),
     "tango_spmm_csr_u_mul_e": (I, [P, P, P, P, P, P, P, I64, I64, I64, I64, I64, I64, P]),
-    "tango_spmm_csr_u_mul_e_ex": (I, [P, P, P, P, I, P, P, I, P, P, P, I64, I64, I64, I64, I64, I64, I64, P, SZ, P]),
+    "tango_spmm_csr_u_mul_e_ex": (I, [P, P, P, P, I, P, P, I, P, P, P, I, I64, I64, I64, I64, I64, I64, I64, P, SZ, P]),
     "tango_attn_scores_fwd": (I, [P, P, P, P, P, I64, I64, I64, P]),
     "tango_attn_scores_bwd_workspace": (SZ, [I64, I64, I64]),
     "tango_attn_scores_bwd": (I, [P, P, P, P, P, P, P, P, I64, I64, I64, P, SZ, P]),

@@ -940,7 +940,7 @@ extern "C" int tango_quantize_rows_f32_i8(const float*, int64_t, int64_t, int64_
                                           int8_t*, int64_t, int, const float*, uint64_t, uint64_t,
                                           tango_stream_t);
 extern "C" int tango_quantize_rows_ex_f32_i8(const float*, int64_t, int64_t, int64_t, const float*,
-                                             const float*, int64_t, const float*, int, int8_t*, int64_t,
+                                             const float*, int64_t, int, const float*, int, int8_t*, int64_t,
                                              int, const float*, uint64_t, uint64_t, tango_stream_t);
 extern "C" int tango_absmax_f32(const float*, int64_t, float*, tango_stream_t);
 extern "C" int tango_quantize_f32_i8(const float*, int64_t, const float*, int8_t*, int, const float*, uint64_t,
@@ -972,7 +972,7 @@ int tango_qgemm_fwd_ex(float* Y, int64_t ldy, const float* X, int64_t ldx, const
     const bool fused = M > 0 && N > 0 && fq_applicable(X, ldx, Xq, ldxq, K, round_mode);
     int rc = TANGO_OK;
     if (!fused) {
-        rc = tango_quantize_rows_ex_f32_i8(X, M, K, ldx, x_row_mul, nullptr, 0, scaleX, 0, Xq, ldxq, round_mode,
+        rc = tango_quantize_rows_ex_f32_i8(X, M, K, ldx, x_row_mul, nullptr, 0, 0, scaleX, 0, Xq, ldxq, round_mode,
                                            nullptr, 0, 0, stream);
         if (rc != TANGO_OK) return rc;
     }

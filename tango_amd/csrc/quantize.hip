@@ -212,6 +212,14 @@ __device__ __forceinline__ void load4(float* f, const float* __restrict__ row, i
     }
 }
 
+// x under the mask value mk of a fused activation backward.  Mode 0 (ReLU): x where mk > 0, else 0.
+// Mode 1 (ELU, mk = the activation's output): x where mk > 0, else x * (mk + 1), since
+// d/dz (exp(z) - 1) = exp(z) = elu(z) + 1.
+__device__ __forceinline__ float masked(float x, float mk, int mode) {
+    if (mk > 0.0f) return x;
+    return mode == 1 ? x * (mk + 1.0f) : 0.0f;
+}
+
 // Row-strided: blockDim = (64, 4); each wavefront walks one row at a time, one lane per
 // output dword (4 columns, padding included), so no per-thread index division is needed and
 // a wavefront's loads and stores are contiguous.  XV = floats per aligned load (4, 2 or 1).
@@ -220,7 +228,8 @@ __global__ __launch_bounds__(256) void quantize_rows_kernel(
     const float* __restrict__ x, int64_t rows, int64_t cols, int64_t ldx,
     const float* __restrict__ scale, int per_row, int8_t* __restrict__ q, int64_t ldq,
     const float* __restrict__ noise, uint64_t seed, uint64_t offset,
-    const float* __restrict__ row_mul, const float* __restrict__ mask, int64_t ldm, int gpr_log2) {
+    const float* __restrict__ row_mul, const float* __restrict__ mask, int64_t ldm, int gpr_log2,
+    int mask_mode) {
     // the mask may use x's vector width when its rows are laid out and aligned like x's
     const bool mask_vec = mask && ldm == ldx &&
                           ((reinterpret_cast<uintptr_t>(mask) ^ reinterpret_cast<uintptr_t>(x)) & 15) == 0;
@@ -240,17 +249,16 @@ __global__ __launch_bounds__(256) void quantize_rows_kernel(
             const int64_t c0 = gi << 2;
             float f[4];
             load4<XV>(f, xr, c0, cols);
+            if (mask) {  // the activation's backward first (as the absmax pass does), then the row multiplier
+                float mk[4];
+                if (mask_vec) load4<XV>(mk, mask + row * ldm, c0, cols); else load4<1>(mk, mask + row * ldm, c0, cols);
+#pragma unroll
+                for (int k = 0; k < 4; ++k) f[k] = masked(f[k], mk[k], mask_mode);
+            }
             if (row_mul) {  // x * row_mul[row], one rounding, before quantization
                 const float rm = row_mul[row];
 #pragma unroll
                 for (int k = 0; k < 4; ++k) f[k] = f[k] * rm;
-            }
-            if (mask) {  // elements whose mask value is not positive quantize to zero
-                float mk[4];
-                if (mask_vec) load4<XV>(mk, mask + row * ldm, c0, cols); else load4<1>(mk, mask + row * ldm, c0, cols);
-#pragma unroll
-                for (int k = 0; k < 4; ++k)
-                    if (!(mk[k] > 0.0f)) f[k] = 0.0f;
             }
             int v[4];
             const uint64_t lin = static_cast<uint64_t>(row) * cols + c0;
@@ -333,7 +341,7 @@ __global__ __launch_bounds__(256) void absmax_ex_kernel(
     const float* __restrict__ x, int64_t rows, int64_t cols, int64_t ldx,
     const float* __restrict__ row_mul, const float* __restrict__ mask, int64_t ldm,
     float* __restrict__ scale_out, float* __restrict__ partial /* [gridDim.x, cols] or null */,
-    int gpr_log2) {
+    int gpr_log2, int mask_mode) {
     __shared__ float red[3][T * 256];
     const bool mask_vec = mask && ldm == ldx &&
                           ((reinterpret_cast<uintptr_t>(mask) ^ reinterpret_cast<uintptr_t>(x)) & 15) == 0;
@@ -381,7 +389,7 @@ __global__ __launch_bounds__(256) void absmax_ex_kernel(
             for (int t = 0; t < T; ++t)
 #pragma unroll
                 for (int k = 0; k < 4; ++k) {
-                    const float e = (mk[u][t][k] > 0.0f) ? v[u][t][k] : 0.0f;
+                    const float e = masked(v[u][t][k], mk[u][t][k], mask_mode);
                     cs[t][k] += e;
                     m = fmaxf(m, fabsf(row_mul ? e * rm : e));
                 }
@@ -529,11 +537,11 @@ size_t tango_absmax_ex_workspace(int64_t rows, int64_t cols, int want_colsum) {
 }
 
 int tango_absmax_ex_f32(const float* x, int64_t rows, int64_t cols, int64_t ldx, const float* row_mul,
-                        const float* mask, int64_t ldm, float* scale_out, int accumulate,
+                        const float* mask, int64_t ldm, int mask_mode, float* scale_out, int accumulate,
                         float* colsum_out, void* workspace, size_t workspace_bytes, tango_stream_t stream) {
     if (rows < 0 || cols < 0 || ldx < cols || !scale_out || (rows * cols > 0 && !x) || (mask && ldm < cols))
         return TANGO_ERR_INVALID_ARG;
-    if (cols > 1024) return TANGO_ERR_UNSUPPORTED;
+    if (cols > 1024 || mask_mode < 0 || mask_mode > 1) return TANGO_ERR_UNSUPPORTED;
     hipStream_t s = as_stream(stream);
     if (!accumulate) fill_u32(scale_out, 0u, 1, s);
     const int grid = absmax_ex_grid(rows);
@@ -553,7 +561,7 @@ int tango_absmax_ex_f32(const float* x, int64_t rows, int64_t cols, int64_t ldx,
     const int xv = ((xa & 15) == 0 && (ldx & 3) == 0) ? 4 : ((xa & 7) == 0 && (ldx & 1) == 0) ? 2 : 1;
 #define TANGO_AEX(T_, V_)                                                                              \
     hipLaunchKernelGGL((absmax_ex_kernel<T_, V_>), dim3(grid), block, 0, s, x, rows, cols, ldx, row_mul, \
-                       mask, ldm, scale_out, partial, gpr_log2)
+                       mask, ldm, scale_out, partial, gpr_log2, mask_mode)
 #define TANGO_AEX_T(T_)                                                              \
     do {                                                                             \
         if (xv == 4) TANGO_AEX(T_, 4); else if (xv == 2) TANGO_AEX(T_, 2); else TANGO_AEX(T_, 1); \
@@ -591,16 +599,17 @@ int tango_quantize_rows_f32_i8(const float* x, int64_t rows, int64_t cols, int64
                                const float* scale, int per_row, int8_t* q, int64_t ldq,
                                int round_mode, const float* noise, uint64_t seed,
                                uint64_t offset, tango_stream_t stream) {
-    return tango_quantize_rows_ex_f32_i8(x, rows, cols, ldx, nullptr, nullptr, 0, scale, per_row, q, ldq,
+    return tango_quantize_rows_ex_f32_i8(x, rows, cols, ldx, nullptr, nullptr, 0, 0, scale, per_row, q, ldq,
                                          round_mode, noise, seed, offset, stream);
 }
 
 int tango_quantize_rows_ex_f32_i8(const float* x, int64_t rows, int64_t cols, int64_t ldx,
-                                  const float* row_mul, const float* mask, int64_t ldm,
+                                  const float* row_mul, const float* mask, int64_t ldm, int mask_mode,
                                   const float* scale, int per_row, int8_t* q, int64_t ldq,
                                   int round_mode, const float* noise, uint64_t seed,
                                   uint64_t offset, tango_stream_t stream) {
     if (mask && ldm < cols) return TANGO_ERR_INVALID_ARG;
+    if (mask_mode < 0 || mask_mode > 1) return TANGO_ERR_UNSUPPORTED;
     if (rows < 0 || cols < 0 || ldx < cols || ldq < cols || !scale ||
         (rows * cols > 0 && (!x || !q)))
         return TANGO_ERR_INVALID_ARG;
@@ -617,13 +626,13 @@ int tango_quantize_rows_ex_f32_i8(const float* x, int64_t rows, int64_t cols, in
         constexpr int M = decltype(mode)::value;
         if (xv == 4)
             hipLaunchKernelGGL((quantize_rows_kernel<M, 4>), grid, block, 0, s, x, rows, cols, ldx, scale,
-                               per_row, q, ldq, noise, seed, offset, row_mul, mask, ldm, gpr_log2);
+                               per_row, q, ldq, noise, seed, offset, row_mul, mask, ldm, gpr_log2, mask_mode);
         else if (xv == 2)
             hipLaunchKernelGGL((quantize_rows_kernel<M, 2>), grid, block, 0, s, x, rows, cols, ldx, scale,
-                               per_row, q, ldq, noise, seed, offset, row_mul, mask, ldm, gpr_log2);
+                               per_row, q, ldq, noise, seed, offset, row_mul, mask, ldm, gpr_log2, mask_mode);
         else
             hipLaunchKernelGGL((quantize_rows_kernel<M, 1>), grid, block, 0, s, x, rows, cols, ldx, scale,
-                               per_row, q, ldq, noise, seed, offset, row_mul, mask, ldm, gpr_log2);
+                               per_row, q, ldq, noise, seed, offset, row_mul, mask, ldm, gpr_log2, mask_mode);
     });
     return rc != TANGO_OK ? rc : launch_status();
 }

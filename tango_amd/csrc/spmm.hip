@@ -40,7 +40,7 @@ struct SpmmParams {
     const float* scale2;     // optional second factor of the dequantization scale (s = scale[0] * scale2[0])
     const float* row_scale;  // optional: out row r is multiplied by row_scale[r] after dequantization
     const float* bias;       // optional: bias[c] added after the row scale
-    int relu;                // clamp at zero last
+    int relu;                // activation applied last: 0 none, 1 max(y, 0), 2 ELU (y > 0 ? y : exp(y) - 1)
     int64_t rows;
     int64_t num_src;  // rows of the gathered matrix
     int64_t ldf;  // bytes between gathered rows
@@ -247,6 +247,12 @@ __device__ __forceinline__ void wave_row_sum(const SpmmParams& p, const LaneCols
     }
 }
 
+__device__ __forceinline__ float activate(float y, int act) {
+    if (act == 1) return fmaxf(y, 0.0f);
+    if (act == 2) return y > 0.0f ? y : expm1f(y);
+    return y;
+}
+
 // Dequantize and store one output row's tile; called by the lanes with grp == 0.
 template <int VEC>
 __device__ __forceinline__ void store_row(const SpmmParams& p, const LaneCols& c, int64_t row, const int* acc) {
@@ -261,7 +267,7 @@ __device__ __forceinline__ void store_row(const SpmmParams& p, const LaneCols& c
         y[i] = s * static_cast<float>(acc[i]);
         if (p.row_scale) y[i] = y[i] * rs;
         if (p.bias && c.col + i < p.W) y[i] = y[i] + p.bias[c.col + i];
-        if (p.relu) y[i] = fmaxf(y[i], 0.0f);
+        y[i] = activate(y[i], p.relu);
     }
     if (VEC == 16 && p.out_vec && c.col + 16 <= p.W) {
         f32x4* o4 = reinterpret_cast<f32x4*>(o);
@@ -812,7 +818,7 @@ __global__ __launch_bounds__(256) void spmm_span_kernel(const SpmmParams p) {
             y[i] = dq * static_cast<float>(sum[i]);
             if (p.row_scale) y[i] = y[i] * rs;
             if (p.bias) y[i] = y[i] + breg[i];
-            if (p.relu) y[i] = fmaxf(y[i], 0.0f);
+            y[i] = activate(y[i], p.relu);
         }
         if (VEC == 16 && p.out_vec && c.col + 16 <= p.W) {
             f32x4* o4 = reinterpret_cast<f32x4*>(o);
@@ -1155,11 +1161,11 @@ int tango_spmm_csr_copy_u_ex(float* out, const int64_t* indptr, const void* indi
         return TANGO_ERR_INVALID_ARG;
     if (workspace && (workspace_bytes < tango_spmm_workspace(rows, nnz, F) || (reinterpret_cast<uintptr_t>(workspace) & 15)))
         return TANGO_ERR_WORKSPACE;
-    if (num_src >= (1LL << 31) || nnz >= (1LL << 31)) return TANGO_ERR_UNSUPPORTED;
+    if (num_src >= (1LL << 31) || nnz >= (1LL << 31) || relu < 0 || relu > 2) return TANGO_ERR_UNSUPPORTED;
     SpmmParams p{};
     p.out = out; p.indptr = indptr; p.indices = static_cast<const int64_t*>(indices); p.idx32 = idx_bits == 32;
     p.feat = feat; p.scale = scale;
-    p.row_scale = row_scale; p.bias = bias; p.relu = relu ? 1 : 0; p.max_row = max_row_nnz; p.hub_ws = workspace;
+    p.row_scale = row_scale; p.bias = bias; p.relu = relu; p.max_row = max_row_nnz; p.hub_ws = workspace;
     p.span_ws = workspace; p.span_ws_bytes = workspace_bytes;
     p.rows = rows; p.num_src = num_src; p.ldf = ldf; p.W = F; p.F = F; p.D = 1; p.nnz = nnz;
     return launch_spmm<KIND_COPY>(p, pick_vec(feat, ldf, F), as_stream(stream));
@@ -1168,7 +1174,7 @@ int tango_spmm_csr_copy_u_ex(float* out, const int64_t* indptr, const void* indi
 int tango_spmm_csr_u_mul_e_ex(float* out, const int64_t* indptr, const void* indices,
                               const void* edge_ids, int idx_bits, const int8_t* feat, const int8_t* evals,
                               int edge_major, const float* scale, const float* scale2, const float* bias,
-                              int64_t rows,
+                              int act, int64_t rows,
                               int64_t num_src, int64_t H, int64_t F, int64_t D, int64_t nnz,
                               int64_t max_row_nnz, void* workspace, size_t workspace_bytes,
                               tango_stream_t stream) {
@@ -1179,11 +1185,11 @@ int tango_spmm_csr_u_mul_e_ex(float* out, const int64_t* indptr, const void* ind
     if (workspace && (workspace_bytes < tango_spmm_workspace(rows, nnz, H * F) || (reinterpret_cast<uintptr_t>(workspace) & 15)))
         return TANGO_ERR_WORKSPACE;
     if (D != 1 && D != F) return TANGO_ERR_UNSUPPORTED;
-    if (num_src >= (1LL << 31) || nnz >= (1LL << 31)) return TANGO_ERR_UNSUPPORTED;
+    if (num_src >= (1LL << 31) || nnz >= (1LL << 31) || act < 0 || act > 2) return TANGO_ERR_UNSUPPORTED;
     SpmmParams p{};
     p.out = out; p.indptr = indptr; p.indices = static_cast<const int64_t*>(indices);
     p.edge_ids = static_cast<const int64_t*>(edge_ids); p.idx32 = idx_bits == 32; p.feat = feat;
-    p.max_row = max_row_nnz; p.hub_ws = workspace; p.span_ws = workspace; p.span_ws_bytes = workspace_bytes;
+    p.relu = act; p.max_row = max_row_nnz; p.hub_ws = workspace; p.span_ws = workspace; p.span_ws_bytes = workspace_bytes;
     p.evals = evals; p.scale = scale; p.scale2 = scale2; p.bias = bias; p.rows = rows; p.num_src = num_src; p.ldf = H * F; p.W = H * F; p.F = F; p.D = D;
     p.nnz = nnz;
     if (edge_major) {  // evals[nnz, H, D]: the H * D bytes of one edge share a cache sector
@@ -1205,7 +1211,7 @@ int tango_spmm_csr_u_mul_e(float* out, const int64_t* indptr, const int64_t* ind
                            const int64_t* edge_ids, const int8_t* feat, const int8_t* evals,
                            const float* scale, int64_t rows, int64_t num_src, int64_t H,
                            int64_t F, int64_t D, int64_t nnz, tango_stream_t stream) {
-    return tango_spmm_csr_u_mul_e_ex(out, indptr, indices, edge_ids, 64, feat, evals, 0, scale, nullptr, nullptr, rows, num_src,
+    return tango_spmm_csr_u_mul_e_ex(out, indptr, indices, edge_ids, 64, feat, evals, 0, scale, nullptr, nullptr, 0, rows, num_src,
                                      H, F, D, nnz, 0, nullptr, 0, stream);
 }
 

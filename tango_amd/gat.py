@@ -5,6 +5,7 @@ import math
 
 import torch
 import torch.nn as nn
+import torch.nn.functional as F
 
 from torch.autograd.function import Function, once_differentiable
 
@@ -85,12 +86,16 @@ class QGATConv(nn.Module):
         a = self.attn_drop(a)
         # without a residual branch the bias add (:160-162) rides in the aggregation's epilogue
         fold_bias = self.bias is not None and self.res_fc is None
-        rst = spmm_u_mul_e.apply(graph, feat_src, a, self.bias if fold_bias else None, s_feat)  # :151
+        # and so does the activation (:164-165) when nothing else is added between the two
+        fold_act = None
+        if self.res_fc is None and (fold_bias or self.bias is None):
+            fold_act = "elu" if self.activation is F.elu else "relu" if self.activation in (F.relu, torch.relu) else None
+        rst = spmm_u_mul_e.apply(graph, feat_src, a, self.bias if fold_bias else None, s_feat, fold_act)  # :151
         if self.res_fc is not None:
             rst = rst + self.res_fc(h).view(n, -1, self._out_feats)
         if self.bias is not None and not fold_bias:
             rst = rst + self.bias.view(1, self._num_heads, self._out_feats)
-        if self.activation:
+        if self.activation and fold_act is None:
             rst = self.activation(rst)
         return (rst, a) if get_attention else rst
 

@@ -118,6 +118,10 @@ def _zero_slot(device):
     return pool[0][k:k + 1]
 
 
+_MASK_MODES = {"relu": 0, "elu": 1}
+_ACTIVATIONS = {None: 0, "relu": 1, "elu": 2}
+
+
 def _mode(round_mode):
     if isinstance(round_mode, str):
         return ROUND_MODES[round_mode]
@@ -191,9 +195,11 @@ class cuda_kernels:
 
     @staticmethod
     def quantize_rows(out, inp, scale, per_row=False, round_mode=ROUND_RNE, noise=None, seed=0,
-                      offset=0, row_mul=None, mask=None):
+                      offset=0, row_mul=None, mask=None, mask_mode="relu"):
         """Row-strided quantize into a possibly wider (zero-padded) int8 matrix (not in the reference).
-        ``row_mul`` [rows] multiplies each row first; elements where ``mask`` <= 0 become zero."""
+        ``mask`` (an activation's output) takes each element backwards through that activation first:
+        ``mask_mode`` "relu" zeroes it where mask <= 0, "elu" multiplies it by mask + 1 there.
+        ``row_mul`` [rows] then multiplies each row."""
         _need(out, torch.int8, "out", contiguous=False)
         _need(inp, torch.float32, "in", contiguous=False)
         _need(scale, torch.float32, "scale")
@@ -216,14 +222,16 @@ class cuda_kernels:
                 raise RuntimeError("quantize_rows: mask must have in's shape")
             ldm = _rows_view(mask, "mask")
         check(_L.tango_quantize_rows_ex_f32_i8(_ptr(inp), inp.size(0), inp.size(1), ldx, _ptr(row_mul),
-                                               _ptr(mask), ldm, scale.data_ptr(), int(bool(per_row)),
+                                               _ptr(mask), ldm, _MASK_MODES[mask_mode], scale.data_ptr(),
+                                               int(bool(per_row)),
                                                _ptr(out), ldq_pad, _mode(round_mode), _ptr(noise),
                                                int(seed), int(offset), _stream()), "quantize_rows")
 
     @staticmethod
-    def absmax_ex(inp, row_mul=None, mask=None, want_colsum=False):
-        """(max|inp * row_mul| / 127 over elements with mask > 0, column sums of the unmasked inp or None)
-        in one read of a 2-D tensor (not in the reference)."""
+    def absmax_ex(inp, row_mul=None, mask=None, want_colsum=False, mask_mode="relu"):
+        """(max|inp' * row_mul| / 127, column sums of inp' or None) in one read of a 2-D tensor (not in
+        the reference); inp' = inp passed backwards through the activation whose output is ``mask``
+        (``mask_mode`` as for ``quantize_rows``)."""
         _need(inp, torch.float32, "in", contiguous=False)
         ldx = _rows_view(inp, "in")
         rows, cols = inp.shape
@@ -240,7 +248,7 @@ class cuda_kernels:
                 sl = slice(c0, min(cols, c0 + 1024))
                 s_i, cs_i = cuda_kernels.absmax_ex(inp[:, sl], row_mul=row_mul,
                                                    mask=None if mask is None else mask[:, sl],
-                                                   want_colsum=want_colsum)
+                                                   want_colsum=want_colsum, mask_mode=mask_mode)
                 scale = s_i if scale is None else torch.maximum(scale, s_i)
                 sums.append(cs_i)
             return scale, (torch.cat(sums) if want_colsum else None)
@@ -252,7 +260,7 @@ class cuda_kernels:
         ws_bytes = _ws_bytes("tango_absmax_ex_workspace", rows, cols, int(want_colsum))
         ws = _workspace(ws_bytes, inp.device)
         check(_L.tango_absmax_ex_f32(_ptr(inp), rows, cols, ldx, _ptr(row_mul), _ptr(mask), ldm,
-                                     scale.data_ptr(), int(accumulate), _ptr(colsum), _ptr(ws), ws_bytes,
+                                     _MASK_MODES[mask_mode], scale.data_ptr(), int(accumulate), _ptr(colsum), _ptr(ws), ws_bytes,
                                      _stream()), "absmax_ex")
         return scale, colsum
 
@@ -418,13 +426,14 @@ class cuda_kernels:
 
     @staticmethod
     def multi_cusparse_SPMM(indptr, indices, N, E_T, scale, edge_ids=None, edge_major=False, bias=None, max_row=0,
-                            scale2=None):
+                            scale2=None, act=None):
         """E_T is [H, D, nnz] in CSR slot order, or in edge-id order when the
         slot->edge permutation ``edge_ids`` is passed (gather fused in-kernel).
         With ``edge_major`` the edge values are [nnz, H, D] instead (no transpose pass).
         ``bias`` ([H * F] fp32) is added to every output row after dequantization.  ``max_row``: an
         upper bound of the longest row if known (0 = unknown).  ``scale2``: the output is dequantized
-        with scale * scale2 (saves the launch that multiplies two 1-element tensors)."""
+        with scale * scale2 (saves the launch that multiplies two 1-element tensors).  ``act``: None,
+        "relu" or "elu", applied last."""
         _need(indptr, torch.int64, "indptr")
         idx_bits = _need_index(indices, "indices")
         _need(N, torch.int8, "N")
@@ -455,7 +464,8 @@ class cuda_kernels:
         ws = _workspace(ws_bytes, N.device)
         check(_L.tango_spmm_csr_u_mul_e_ex(_ptr(out), indptr.data_ptr(), _ptr(indices), _ptr(edge_ids), idx_bits,
                                            _ptr(N), _ptr(E_T), int(bool(edge_major)), scale.data_ptr(),
-                                           _ptr(scale2), _ptr(bias), rows, k, H, F, D, nnz, int(max_row), _ptr(ws), ws_bytes,
+                                           _ptr(scale2), _ptr(bias), _ACTIVATIONS[act], rows, k, H, F, D, nnz,
+                                           int(max_row), _ptr(ws), ws_bytes,
                                            _stream()), "multi_cusparse_SPMM")
         return out
 
@@ -590,7 +600,7 @@ def quantize(t, scale=None, round_mode=ROUND_RNE, noise=None, seed=0, offset=0):
 
 
 def quantize_padded(t, scale=None, round_mode=ROUND_RNE, noise=None, seed=0, offset=0, align=16,
-                    row_mul=None, mask=None):
+                    row_mul=None, mask=None, mask_mode="relu"):
     """Like ``quantize`` for a 2-D tensor, but the int8 rows are padded with
     zeros to a multiple of ``align`` bytes so that the SpMM gather and the GEMM
     fragment loads stay 16-byte aligned for odd widths (41, 602, ...).  Returns a
@@ -598,7 +608,7 @@ def quantize_padded(t, scale=None, round_mode=ROUND_RNE, noise=None, seed=0, off
     assert t.is_cuda and t.dim() == 2, "2-D GPU tensor expected"
     if scale is None:
         if row_mul is not None or mask is not None:
-            scale, _ = cuda_kernels.absmax_ex(t, row_mul=row_mul, mask=mask)
+            scale, _ = cuda_kernels.absmax_ex(t, row_mul=row_mul, mask=mask, mask_mode=mask_mode)
         else:
             scale = cuda_kernels.get_scale(t) if t.is_contiguous() else cuda_kernels.get_scale(t.contiguous())
     rows, cols = t.shape
@@ -609,7 +619,7 @@ def quantize_padded(t, scale=None, round_mode=ROUND_RNE, noise=None, seed=0, off
         cuda_kernels.quantize(buf, t, scale, round_mode=round_mode, noise=noise, seed=seed, offset=offset)
     else:
         cuda_kernels.quantize_rows(buf, t, scale, round_mode=round_mode, noise=noise, seed=seed, offset=offset,
-                                   row_mul=row_mul, mask=mask)
+                                   row_mul=row_mul, mask=mask, mask_mode=mask_mode)
     return buf[:, :cols], scale
 
 
@@ -698,7 +708,7 @@ def _csr_of(g, reverse):
     return indptr, indices, edge_ids, getattr(g, "max_out_degree" if reverse else "max_in_degree", 0)
 
 
-def multi_cusparse_SPMM(g, N, E_T, scale, reverse=False, edge_major=False, bias=None, scale2=None):
+def multi_cusparse_SPMM(g, N, E_T, scale, reverse=False, edge_major=False, bias=None, scale2=None, act=None):
     """E_T is [H, D, nnz] in edge-id order.  cuda/kernels.py:122-136; the
     index_select by edge_ids of the reference happens inside the kernel.
     ``edge_major``: E_T is the quantized edge tensor as it is, [nnz, H, 1]."""
@@ -708,7 +718,8 @@ def multi_cusparse_SPMM(g, N, E_T, scale, reverse=False, edge_major=False, bias=
     if edge_ids is not None and edge_ids.numel() == 0:
         edge_ids = None
     return cuda_kernels.multi_cusparse_SPMM(indptr, indices, N, E_T, scale, edge_ids=edge_ids,
-                                            edge_major=edge_major, bias=bias, max_row=longest, scale2=scale2)
+                                            edge_major=edge_major, bias=bias, max_row=longest, scale2=scale2,
+                                            act=act)
 
 
 def incidence_SPMM(g, E, scaleE, reverse=False):

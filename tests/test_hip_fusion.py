@@ -40,6 +40,15 @@ def test_absmax_ex_and_quantize_ex(K, orc):
         assert np.array_equal(host(q), orc.quantize(scaled, host(s)[0]))
         q2, _ = K.quantize_padded(dev(x), s, row_mul=dev(rm), mask=dev(mask), round_mode="stochastic", seed=3, offset=64)
         assert np.array_equal(host(q2), orc.quantize(scaled, host(s)[0], orc.STOCHASTIC, seed=3, offset=64))
+        # ELU backward: elements whose mask (the activation's output) is not positive are multiplied by mask + 1
+        emask = np.where(mask > 0, mask, np.expm1(mask)).astype(np.float32)
+        through = np.where(emask > 0, x, x * (emask + np.float32(1))).astype(np.float32)
+        scaled = (through * rm[:, None]).astype(np.float32)
+        s, cs = K.cuda_kernels.absmax_ex(dev(x), row_mul=dev(rm), mask=dev(emask), want_colsum=True, mask_mode="elu")
+        assert host(s)[0] == orc.absmax_scale(scaled)
+        assert np.allclose(host(cs), through.astype(np.float64).sum(0), rtol=1e-5, atol=1e-3)
+        q, _ = K.quantize_padded(dev(x), s, row_mul=dev(rm), mask=dev(emask), mask_mode="elu")
+        assert np.array_equal(host(q), orc.quantize(scaled, host(s)[0]))
     # colsum is deterministic run to run
     x = dev(rng.standard_normal((50000, 256)).astype(np.float32))
     a = K.cuda_kernels.absmax_ex(x, want_colsum=True)[1]
@@ -197,6 +206,69 @@ def test_u_mul_e_bias_epilogue(K):
     ref.backward(dZ)
     assert torch.equal(got[0], N.grad) and torch.equal(got[1], E.grad)
     assert torch.allclose(got[2], bias.grad, rtol=1e-5, atol=1e-4)
+
+
+@pytest.mark.parametrize("act", ["relu", "elu"])
+@pytest.mark.parametrize("with_bias", [True, False])
+@pytest.mark.parametrize("n,e,H,F", [(700, 9000, 4, 16), (300, 40000, 3, 5)])
+def test_u_mul_e_activation_epilogue(K, act, with_bias, n, e, H, F):
+    """Activation in the SpMM epilogue == a separate pass over its output; in the backward pass the
+    activation's derivative applied inside the scale and quantize kernels == applied to dZ beforehand."""
+    from tango_amd.SPMM import spmm_u_mul_e
+    rng = np.random.default_rng(10)
+    src, dst = rand_graph(rng, n, e)
+    g = make_graph(src, dst, n)
+    N = dev(rng.standard_normal((n, H, F)).astype(np.float32)).requires_grad_()
+    E = dev(rng.random((e, H, 1)).astype(np.float32)).requires_grad_()
+    bias = dev(rng.standard_normal(H * F).astype(np.float32)).requires_grad_() if with_bias else None
+    leaves = [t for t in (N, E, bias) if t is not None]
+    dZ = dev(rng.standard_normal((n, H, F)).astype(np.float32))
+    out = spmm_u_mul_e.apply(g, N, E, bias, None, act)
+    out.backward(dZ)
+    got = [t.grad.clone() for t in leaves]
+    for t in leaves:
+        t.grad = None
+    pre = spmm_u_mul_e.apply(g, N, E, bias)
+    if act == "relu":
+        assert torch.equal(out, torch.relu(pre))
+        back = torch.where(out > 0, dZ, torch.zeros_like(dZ))
+    else:
+        assert torch.allclose(out, torch.nn.functional.elu(pre), rtol=1e-6, atol=1e-7)
+        assert torch.equal(out > 0, pre > 0)
+        back = torch.where(out > 0, dZ, dZ * (out.detach() + 1.0))
+    pre.backward(back)
+    assert torch.equal(got[0], N.grad) and torch.equal(got[1], E.grad)
+    if with_bias:
+        assert torch.allclose(got[2], bias.grad, rtol=1e-5, atol=1e-4)
+
+
+@pytest.mark.parametrize("act", [torch.nn.functional.elu, torch.relu])
+def test_gat_layer_with_folded_activation_tracks_torch_activation(act):
+    """A GAT layer whose activation rides in the aggregation's epilogue against the same layer with the
+    activation as a torch op on the aggregation's output (forward equal, gradients within int8 noise:
+    the torch path quantizes dZ after a separate fp32 pass whose exp differs in the last bits)."""
+    from tango_amd.gat import QGATConv
+    rng = np.random.default_rng(12)
+    n, e = 2000, 24000
+    src, dst = rand_graph(rng, n, e)
+    loops = np.arange(n)
+    g = make_graph(np.concatenate([src, loops]), np.concatenate([dst, loops]), n)
+    torch.manual_seed(3)
+    layer = QGATConv(48, 16, 4, activation=act).cuda()
+    x = dev(rng.standard_normal((n, 48)).astype(np.float32)).requires_grad_()
+    w = dev(rng.standard_normal((n, 4, 16)).astype(np.float32))
+    outs, grads = [], []
+    for fold in (True, False):
+        layer.zero_grad()
+        x.grad = None
+        layer.activation = act if fold else (lambda t: act(t))  # an unknown callable is not folded
+        y = layer(g, x)
+        y.backward(w)
+        outs.append(y.detach().clone())
+        grads.append([p.grad.clone() for p in layer.parameters()] + [x.grad.clone()])
+    assert torch.allclose(outs[0], outs[1], rtol=1e-6, atol=1e-7)
+    for a, b in zip(*grads):
+        assert torch.allclose(a, b, rtol=1e-3, atol=2e-2 * float(b.abs().max()))
 
 
 def test_scale_hand_off_is_bit_identical(K):
