@@ -68,6 +68,7 @@ __global__ __launch_bounds__(256, 2) void gemm_nt_kernel(const NtParams p) {
     constexpr int PF = 4;                 // A fragments in flight (k-steps)
     constexpr int BROWS = NT * 16;        // rows of B per tile
     __shared__ i32x4 ldsB[2][BROWS * 4];  // [buffer][row][16-byte chunk], chunk index swizzled
+    __shared__ __attribute__((aligned(16))) float bias_s[BROWS];  // this tile's bias, zero where there is none
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -122,6 +123,7 @@ __global__ __launch_bounds__(256, 2) void gemm_nt_kernel(const NtParams p) {
     for (int s = 0; s < PF; ++s) load_a(a[s], s);
     i32x4 breg[BCH];
     load_b(breg, 0);
+    for (int n = tid; n < BROWS; n += 256) bias_s[n] = (p.bias && n0 + n < p.N) ? p.bias[n0 + n] : 0.0f;
     store_b(breg, 0);
     __syncthreads();
 
@@ -163,11 +165,12 @@ __global__ __launch_bounds__(256, 2) void gemm_nt_kernel(const NtParams p) {
             for (int j = 0; j < NT; ++j) {
                 const int64_t col = n0 + j * 16 + g * 4;
                 float y[4];
+                const f32x4 bv = *reinterpret_cast<const f32x4*>(bias_s + j * 16 + g * 4);
 #pragma unroll
                 for (int v = 0; v < 4; ++v) {
                     y[v] = s * static_cast<float>(acc[i][j][v]);
                     if (p.row_scale) y[v] = y[v] * rsc;
-                    if (p.bias && col + v < p.N) y[v] = p.bias[col + v] + y[v];
+                    if (p.bias) y[v] = bv[v] + y[v];
                     if (col + v < p.N) m = fmaxf(m, fabsf(y[v]));
                 }
                 if (col + 4 <= p.N && wide == 4) {
@@ -184,6 +187,109 @@ __global__ __launch_bounds__(256, 2) void gemm_nt_kernel(const NtParams p) {
                 }
             }
         }
+    }
+    if (p.absmax_out) block_absmax_to_global(m / 127.0f, p.absmax_out);
+}
+
+// NT kernel with the small operand stationary in LDS, for reductions of at most 256 (four k-steps).
+// A persistent workgroup of WAVES waves first copies its 16 * NT rows of the packed B into LDS (row pitch
+// an odd number of 16-byte units: the sixteen rows of a fragment read start in different bank quads) and
+// then never synchronises again: the 16-row tiles of A are dealt round-robin over all waves of the
+// launch, a wave loads the whole 16 x K tile as its A fragments (and the next tile's while it works on
+// this one), reads the B fragments from LDS, and stores 16 rows x 16 NT columns.  The kernels above pay
+// one L2 round trip per k-step (several microseconds under load) in every workgroup; here the only
+// global loads are the A tiles, requested one tile ahead, so loads, MFMAs and the output stores of the
+// sixteen waves of a CU overlap.
+template <int NT, int VEC, int WAVES>
+__global__ __launch_bounds__(64 * WAVES) void gemm_nts_kernel(const NtParams p, int ntiles, int pitch) {
+    extern __shared__ __attribute__((aligned(16))) int8_t b_lds[];  // [16 NT][pitch]
+    constexpr int KS = 4;
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int g = lane >> 4, r16 = lane & 15;
+    const int64_t n0 = static_cast<int64_t>(blockIdx.y) * (16 * NT);
+    const int ksteps = static_cast<int>((p.Kr + 63) >> 6);  // <= KS (host)
+    {
+        const int cpr = pitch >> 4;
+        const int kchunks = ksteps * 4;  // 16-byte chunks of a packed row that hold data or its zero fill
+        for (int idx = tid; idx < 16 * NT * cpr; idx += 64 * WAVES) {
+            const int n = idx / cpr, c = idx - n * cpr;
+            i32x4 v{0, 0, 0, 0};
+            if (n0 + n < p.N && c < kchunks) v = *reinterpret_cast<const i32x4*>(p.B + (n0 + n) * p.ldb + c * 16);
+            *reinterpret_cast<i32x4*>(b_lds + n * pitch + c * 16) = v;
+        }
+    }
+    float* bias_lds = reinterpret_cast<float*>(b_lds + 16 * NT * pitch);  // [16 NT], zero where there is none
+    for (int n = tid; n < 16 * NT; n += 64 * WAVES) bias_lds[n] = (p.bias && n0 + n < p.N) ? p.bias[n0 + n] : 0.0f;
+    __syncthreads();
+
+    const float s = p.sA[0] * p.sB[0];
+    const uintptr_t ca = reinterpret_cast<uintptr_t>(p.C);
+    const int wide = ((ca & 15) == 0 && (p.ldc & 3) == 0) ? 4 : ((ca & 7) == 0 && (p.ldc & 1) == 0) ? 2 : 1;
+    float m = 0.0f;
+    auto load_tile = [&](i32x4* a, int t) {
+        const int64_t row = static_cast<int64_t>(t) * 16 + r16;
+        const bool ok = t < ntiles && row < p.M;
+        const int8_t* pa = p.A + (ok ? row : 0) * p.lda + g * 16;
+#pragma unroll
+        for (int st = 0; st < KS; ++st) {
+            const int64_t kc = static_cast<int64_t>(st) * 64 + g * 16;
+            const int64_t avail = (ok && st < ksteps && kc < p.Kr) ? p.a_row_bytes - kc : 0;
+            a[st] = load16<VEC>(pa + st * 64, avail);
+        }
+    };
+    const int stride = static_cast<int>(gridDim.x) * WAVES;
+    i32x4 cur[KS], nxt[KS];
+    int t = static_cast<int>(blockIdx.x) * WAVES + wave;
+    load_tile(cur, t);
+    for (; t < ntiles; t += stride) {
+        load_tile(nxt, t + stride);
+        i32x4 acc[NT];
+#pragma unroll
+        for (int j = 0; j < NT; ++j) acc[j] = i32x4{0, 0, 0, 0};
+#pragma unroll
+        for (int st = 0; st < KS; ++st) {
+            if (st < ksteps) {
+#pragma unroll
+                for (int j = 0; j < NT; ++j) {
+                    const i32x4 b = *reinterpret_cast<const i32x4*>(b_lds + (16 * j + r16) * pitch + st * 64 + g * 16);
+                    acc[j] = mfma_16x16x64(b, cur[st], acc[j]);  // operands swapped, see gemm_nt_kernel
+                }
+            }
+        }
+        // lane holds C[16 t + r16][n0 + 16 j + 4 g + v]
+        const int64_t row = static_cast<int64_t>(t) * 16 + r16;
+        if (row < p.M) {
+            float* crow = p.C + row * p.ldc;
+            const float rsc = p.row_scale ? p.row_scale[row] : 1.0f;
+#pragma unroll
+            for (int j = 0; j < NT; ++j) {
+                const int64_t col = n0 + j * 16 + g * 4;
+                float y[4];
+                const f32x4 bv = *reinterpret_cast<const f32x4*>(bias_lds + j * 16 + g * 4);
+#pragma unroll
+                for (int v = 0; v < 4; ++v) {
+                    y[v] = s * static_cast<float>(acc[j][v]);
+                    if (p.row_scale) y[v] = y[v] * rsc;
+                    if (p.bias) y[v] = bv[v] + y[v];
+                    if (col + v < p.N) m = fmaxf(m, fabsf(y[v]));
+                }
+                if (col + 4 <= p.N && wide == 4) {
+                    *reinterpret_cast<f32x4*>(crow + col) = f32x4{y[0], y[1], y[2], y[3]};
+                } else if (col + 4 <= p.N && wide == 2) {
+                    typedef float f32x2 __attribute__((ext_vector_type(2)));
+                    *reinterpret_cast<f32x2*>(crow + col) = f32x2{y[0], y[1]};
+                    *reinterpret_cast<f32x2*>(crow + col + 2) = f32x2{y[2], y[3]};
+                } else {
+#pragma unroll
+                    for (int v = 0; v < 4; ++v)
+                        if (col + v < p.N) crow[col + v] = y[v];
+                }
+            }
+        }
+#pragma unroll
+        for (int st = 0; st < KS; ++st) cur[st] = nxt[st];
     }
     if (p.absmax_out) block_absmax_to_global(m / 127.0f, p.absmax_out);
 }
@@ -209,6 +315,7 @@ struct FqParams {
     int64_t M, N, K;
     int64_t ldx, ldxq, ldb, ldc;
     int kp;               // K rounded up to 64
+    int pitch;            // bytes between rows of the LDS block (fq_pitch)
 };
 
 // TPW = 16-column tiles per wave (the workgroup covers 64 * TPW columns), XV = floats per load,
@@ -216,15 +323,20 @@ struct FqParams {
 // loads from (kp <= 256 IT): sizes the prefetch registers.
 template <int TPW, int XV, int MODE, int RT, int IT>
 __global__ __launch_bounds__(256, 2) void gemm_fq_kernel(const FqParams p) {
-    extern __shared__ __attribute__((aligned(16))) int8_t a_lds[];  // [BM][kp + 16]
+    extern __shared__ __attribute__((aligned(16))) int8_t a_lds[];  // [BM][pitch] + 64, then 64 TPW floats of bias
     constexpr int BM = 16 * RT;
-    const int pitch = p.kp + 16;
+    const int pitch = p.pitch;
+    float* bias_lds = reinterpret_cast<float*>(a_lds + BM * pitch + 64);
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int64_t row_base = static_cast<int64_t>(blockIdx.x) * BM;
     const float rs = rscale_of(p.sA[0]);
     const bool store_q = blockIdx.y == 0;
+    if (threadIdx.x < 64 * TPW) {  // this workgroup's slice of the bias, zero where there is none
+        const int64_t n = static_cast<int64_t>(blockIdx.y) * (64 * TPW) + threadIdx.x;
+        bias_lds[threadIdx.x] = (p.bias && n < p.N) ? p.bias[n] : 0.0f;
+    }
 
     // ---- phase A: rows wave, wave + 4, ... ; lane owns columns 4 * (lane + 64 it) .. + 3
     const float* __restrict__ Xp = p.X;
@@ -271,9 +383,9 @@ __global__ __launch_bounds__(256, 2) void gemm_fq_kernel(const FqParams p) {
                     if (p.x_row_mul) { x0 = x0 * rm; x1 = x1 * rm; x2 = x2 * rm; x3 = x3 * rm; }
                     const uint32_t q = pack4(quant_one<MODE>(x0, rs, 0.f), quant_one<MODE>(x1, rs, 0.f),
                                              quant_one<MODE>(x2, rs, 0.f), quant_one<MODE>(x3, rs, 0.f));
-                    *reinterpret_cast<uint32_t*>(a_lds + lr * pitch + c0) = q;
+                    if (c0 < pitch) *reinterpret_cast<uint32_t*>(a_lds + lr * pitch + c0) = q;
                     if (store_q && row < p.M && c0 < p.ldxq)
-                        __builtin_nontemporal_store(q, reinterpret_cast<uint32_t*>(Xqp + row * p.ldxq + c0));
+                        *reinterpret_cast<uint32_t*>(Xqp + row * p.ldxq + c0) = q;
                 }
             }
         }
@@ -389,10 +501,11 @@ __global__ __launch_bounds__(256, 2) void gemm_fq_kernel(const FqParams p) {
                 for (int j = 0; j < TPW; ++j) {
                     const int64_t col = n0 + j * 16 + g * 4;
                     float y[4];
+                    const f32x4 bv = *reinterpret_cast<const f32x4*>(bias_lds + wave * (16 * TPW) + j * 16 + g * 4);
 #pragma unroll
                     for (int v = 0; v < 4; ++v) {
                         y[v] = s * static_cast<float>(acc[i][j][v]);
-                        if (p.bias && col + v < p.N) y[v] = p.bias[col + v] + y[v];
+                        if (p.bias) y[v] = bv[v] + y[v];
                         if (col + v < p.N) m = fmaxf(m, fabsf(y[v]));
                     }
                     if (col + 4 <= p.N && wide == 4) {
@@ -798,6 +911,18 @@ __global__ __launch_bounds__(256) void tn_reduce_kernel(float* __restrict__ out,
 // ------------------------------------------------------------- host side
 static int64_t round_up(int64_t v, int64_t m) { return (v + m - 1) / m * m; }
 
+// Compute units of the current device (queried once; a fixed property of the machine).
+static int compute_units() {
+    static const int n = [] {
+        int dev = 0, cus = 0;
+        if (hipGetDevice(&dev) != hipSuccess ||
+            hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0)
+            cus = 256;
+        return cus;
+    }();
+    return n;
+}
+
 // widest aligned access for 16-byte row pieces of an int8 matrix; `cols` bytes are meaningful
 static int row_vec(const int8_t* p, int64_t ld, int64_t cols, int64_t* readable) {
     const uintptr_t a = reinterpret_cast<uintptr_t>(p);
@@ -820,6 +945,33 @@ static void launch_nt_vec(const NtParams& p, hipStream_t s) {
 #define TANGO_NT(NT_)                                                                             \
     hipLaunchKernelGGL((gemm_nt_kernel<NT_, VEC>), dim3(gx, static_cast<unsigned>(ceil_div(n16, NT_))), \
                        dim3(256), 0, s, p)
+    if (p.Kr <= 256 && VEC != 1) {  // the small operand fits LDS: the stationary form
+        constexpr int WAVES = 12;
+        const int ny = static_cast<int>(ceil_div(n16, 16));
+        const int nt = static_cast<int>(ceil_div(n16, ny));
+        const int pitch = 16 * ((static_cast<int>(ceil_div(p.Kr, 64)) * 4) | 1);
+        const int ntiles = static_cast<int>(ceil_div(p.M, 16));
+        int gx = compute_units() / ny;
+        if (gx > ceil_div(ntiles, WAVES)) gx = static_cast<int>(ceil_div(ntiles, WAVES));
+        if (gx < 1) gx = 1;
+#define TANGO_NTS(NT_)                                                                                          \
+    do {                                                                                                        \
+        /* more than 64 KB of dynamic LDS has to be asked for once per kernel */                                \
+        static const bool ok = hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_nts_kernel<NT_, VEC, WAVES>), \
+                                                   hipFuncAttributeMaxDynamicSharedMemorySize, 80 * 1024) == hipSuccess; \
+        if (ok) {                                                                                               \
+            hipLaunchKernelGGL((gemm_nts_kernel<NT_, VEC, WAVES>), dim3(gx, ny), dim3(64 * WAVES),               \
+                               static_cast<size_t>(16 * NT_) * (pitch + 4), s, p, ntiles, pitch);               \
+            return;                                                                                             \
+        }                                                                                                       \
+    } while (0)
+        if (nt <= 2) TANGO_NTS(2);
+        else if (nt <= 4) TANGO_NTS(4);
+        else if (nt <= 8) TANGO_NTS(8);
+        else if (nt <= 13) TANGO_NTS(13);
+        else TANGO_NTS(16);
+#undef TANGO_NTS
+    }
     if (n16 <= 1) TANGO_NT(1);
     else if (n16 <= 2) TANGO_NT(2);
     else if (n16 <= 3) TANGO_NT(3);
@@ -856,18 +1008,6 @@ static bool fq_applicable(const float* X, int64_t ldx, const int8_t* Xq, int64_t
     return true;
 }
 
-// Compute units of the current device (queried once; a fixed property of the machine).
-static int compute_units() {
-    static const int n = [] {
-        int dev = 0, cus = 0;
-        if (hipGetDevice(&dev) != hipSuccess ||
-            hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0)
-            cus = 256;
-        return cus;
-    }();
-    return n;
-}
-
 constexpr size_t kLdsBytes = 160 * 1024;
 
 template <int NT, int XV, int MODE>
@@ -898,11 +1038,20 @@ static bool launch_ws(const FqParams& p, hipStream_t s) {
     return launch_ws_nt<2, XV, MODE>(p, s);
 }
 
+// Row pitch of the forward kernel's LDS block: K rounded up to an odd number of 16-byte units, so that the
+// sixteen rows of a fragment read start in sixteen different bank quads.  The last k-step may read past a
+// row's end (into the next row, or the 64 spare bytes after the block): those bytes meet the zero padding of
+// the packed small operand, and any int8 times zero is zero.
+static int fq_pitch(int64_t K) {
+    const int64_t units = ceil_div(K, 16);
+    return static_cast<int>(16 * (units | 1));
+}
+
 template <int XV, int MODE>
 static void launch_fq_mode(const FqParams& p, hipStream_t s) {
     constexpr int RT = 4;  // 64 rows per workgroup measured faster than 32 at every benchmark shape
     if (launch_ws<XV, MODE>(p, s)) return;
-    const size_t lds = static_cast<size_t>(16 * RT) * (p.kp + 16);
+    const size_t lds = static_cast<size_t>(16 * RT) * p.pitch + 64 + 256 * sizeof(float);
     const unsigned gx = static_cast<unsigned>(ceil_div(p.M, 16 * RT));
 #define TANGO_FQ_IT(TPW_, IT_)                                                                   \
     hipLaunchKernelGGL((gemm_fq_kernel<TPW_, XV, MODE, RT, IT_>),                                \
@@ -994,7 +1143,7 @@ int tango_qgemm_fwd_ex(float* Y, int64_t ldy, const float* X, int64_t ldx, const
         FqParams q{};
         q.C = Y; q.X = X; q.Xq = Xq; q.B = Bp; q.bias = bias; q.x_row_mul = x_row_mul; q.absmax_out = scaleY;
         q.sA = scaleX; q.sB = scaleW; q.M = M; q.N = N; q.K = K; q.ldx = ldx; q.ldxq = ldxq; q.ldb = ldb;
-        q.ldc = ldy; q.kp = static_cast<int>(ldb);
+        q.ldc = ldy; q.kp = static_cast<int>(ldb); q.pitch = fq_pitch(K);
         return launch_fq(q, round_mode, s, true);
     }
     NtParams p{};

@@ -249,7 +249,9 @@ __device__ __forceinline__ void wave_row_sum(const SpmmParams& p, const LaneCols
 
 __device__ __forceinline__ float activate(float y, int act) {
     if (act == 1) return fmaxf(y, 0.0f);
-    if (act == 2) return y > 0.0f ? y : expm1f(y);
+    // the hardware exponential: exp(y) - 1 carries an absolute error of about 1e-7 for y <= 0 (the library's
+    // expm1f is some forty instructions, which these epilogues run under divergence, once per finished row)
+    if (act == 2) return y > 0.0f ? y : __expf(y) - 1.0f;
     return y;
 }
 
@@ -267,7 +269,10 @@ __device__ __forceinline__ void store_row(const SpmmParams& p, const LaneCols& c
         y[i] = s * static_cast<float>(acc[i]);
         if (p.row_scale) y[i] = y[i] * rs;
         if (p.bias && c.col + i < p.W) y[i] = y[i] + p.bias[c.col + i];
-        y[i] = activate(y[i], p.relu);
+    }
+    if (p.relu) {  // uniform: rows without an activation skip its instructions altogether
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) y[i] = activate(y[i], p.relu);
     }
     if (VEC == 16 && p.out_vec && c.col + 16 <= p.W) {
         f32x4* o4 = reinterpret_cast<f32x4*>(o);
@@ -818,7 +823,10 @@ __global__ __launch_bounds__(256) void spmm_span_kernel(const SpmmParams p) {
             y[i] = dq * static_cast<float>(sum[i]);
             if (p.row_scale) y[i] = y[i] * rs;
             if (p.bias) y[i] = y[i] + breg[i];
-            y[i] = activate(y[i], p.relu);
+        }
+        if (p.relu) {  // uniform: rows without an activation skip its instructions altogether
+#pragma unroll
+            for (int i = 0; i < VEC; ++i) y[i] = activate(y[i], p.relu);
         }
         if (VEC == 16 && p.out_vec && c.col + 16 <= p.W) {
             f32x4* o4 = reinterpret_cast<f32x4*>(o);

@@ -233,7 +233,8 @@ def test_u_mul_e_activation_epilogue(K, act, with_bias, n, e, H, F):
         assert torch.equal(out, torch.relu(pre))
         back = torch.where(out > 0, dZ, torch.zeros_like(dZ))
     else:
-        assert torch.allclose(out, torch.nn.functional.elu(pre), rtol=1e-6, atol=1e-7)
+        # the epilogue computes exp(y) - 1 with the hardware exponential: absolute error ~1e-7 where y <= 0
+        assert torch.allclose(out, torch.nn.functional.elu(pre), rtol=1e-6, atol=5e-7)
         assert torch.equal(out > 0, pre > 0)
         back = torch.where(out > 0, dZ, dZ * (out.detach() + 1.0))
     pre.backward(back)
@@ -266,7 +267,7 @@ def test_gat_layer_with_folded_activation_tracks_torch_activation(act):
         y.backward(w)
         outs.append(y.detach().clone())
         grads.append([p.grad.clone() for p in layer.parameters()] + [x.grad.clone()])
-    assert torch.allclose(outs[0], outs[1], rtol=1e-6, atol=1e-7)
+    assert torch.allclose(outs[0], outs[1], rtol=1e-6, atol=5e-7)
     for a, b in zip(*grads):
         assert torch.allclose(a, b, rtol=1e-3, atol=2e-2 * float(b.abs().max()))
 

@@ -159,3 +159,23 @@ def test_qgemm_i8(K, orc):
     K.cuda_kernels.QGEMM_i8(Y, dev(A), dev(B), None, sY, sc(0.5), sc(0.25))
     want = np.float32(0.125) * (A.astype(np.int64) @ B.astype(np.int64).T).astype(np.float32)
     assert np.array_equal(host(Y), want) and host(sY)[0] == orc.absmax_scale(want)
+
+
+@pytest.mark.parametrize("M,N,Kd", [(70001, 200, 130), (50000, 602, 256), (4000, 41, 64), (15, 256, 200)])
+def test_qgemm_i8_small_operand_stationary(K, orc, M, N, Kd):
+    """The NT form that keeps the small operand in LDS (reduction <= 256, 4-byte aligned rows): more 16-row
+    tiles than waves in the launch (every wave walks several tiles, the next one prefetched), column
+    blocks of 13 and 16 tiles, a partial last tile, bias and the output scale."""
+    rng = np.random.default_rng(M + N + Kd)
+    A = rng.integers(-127, 128, (M, Kd)).astype(np.int8)
+    B = rng.integers(-127, 128, (N, Kd)).astype(np.int8)
+    bias = rng.standard_normal(N).astype(np.float32)
+    ld = (Kd + 15) // 16 * 16
+    Abuf = torch.full((M, ld), 77, dtype=torch.int8, device="cuda")
+    Abuf[:, :Kd] = dev(A)
+    Y = torch.empty((M, N), dtype=torch.float32, device="cuda")
+    sY = torch.empty(1, dtype=torch.float32, device="cuda")
+    K.cuda_kernels.QGEMM_i8(Y, Abuf[:, :Kd], dev(B), dev(bias), sY, sc(0.5), sc(0.25))
+    acc = (A.astype(np.float64) @ B.astype(np.float64).T)  # exact: |sums| < 2^53
+    want = bias[None, :] + np.float32(0.125) * acc.astype(np.float32)
+    assert np.array_equal(host(Y), want) and host(sY)[0] == orc.absmax_scale(want)
