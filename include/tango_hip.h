@@ -136,7 +136,11 @@ int tango_qgemm_fwd(float* Y, int64_t ldy, const float* X, int64_t ldx, int8_t* 
 
 /* As tango_qgemm_fwd, with row m of X multiplied by x_row_mul[m] before it is
    quantized (the "feat * out_deg^-1/2" of evaluation/test_gcn.py:86-94 folded
-   into the quantize pass; scaleX must then be the scale of the multiplied X). */
+   into the quantize pass; scaleX must then be the scale of the multiplied X).
+   X may be NULL (x_row_mul must then be NULL too): Xq is then an input that already
+   holds X quantized with scaleX, e.g. because several layers consume the same X
+   (the q / k / v projections of evaluation/test_HGT.py:44-50) and one quantize
+   pass serves them all; W is still quantized here. */
 int tango_qgemm_fwd_ex(float* Y, int64_t ldy, const float* X, int64_t ldx, const float* x_row_mul,
                        int8_t* Xq, int64_t ldxq, const float* W, int64_t ldw, int8_t* Wq,
                        const float* bias, float* scaleY, const float* scaleX, const float* scaleW,

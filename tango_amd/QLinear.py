@@ -54,8 +54,26 @@ class QgemmNT_func(Function):
         return grad_A, grad_B
 
 
-def _forward(ctx, X, W, b, reduce, row_scale=None, scaleX=None):
+def quantize_input(X, scaleX=None):
+    """(int8 X, scale) the way the forward GEMM quantizes its input, for layers that share one input:
+    pass both to each ``QLinear.forward`` and X is read and quantized once instead of once per layer."""
+    X = X.reshape(-1, X.size(-1))
     X = X if X.is_contiguous() else X.contiguous()
+    return kernels.quantize_padded(X, scaleX, round_mode=kernels.default_forward_round_mode())
+
+
+def _forward(ctx, X, W, b, reduce, row_scale=None, scaleX=None, Xq=None):
+    X = X if X.is_contiguous() else X.contiguous()
+    if Xq is not None:
+        if scaleX is None or row_scale is not None:
+            raise RuntimeError("QLinear: a quantized input needs its scale and excludes row_scale")
+        if tuple(Xq.shape) != tuple(X.shape) or Xq.dtype != torch.int8:
+            raise RuntimeError("QLinear: the quantized input must be int8 of the input's shape")
+        scaleW = kernels.cuda_kernels.get_scale(W if W.is_contiguous() else W.contiguous())
+        W_ = torch.empty(W.shape, dtype=torch.int8, device=X.device)
+        res = kernels.QGEMM_forward(None, Xq, scaleX, W, W_, scaleW, b, reduce)
+        ctx.backward_cache = Xq, scaleX, W_, scaleW, b, None
+        return res
     if scaleX is not None:
         if row_scale is not None:
             raise RuntimeError("QLinear: a precomputed input scale cannot be combined with row_scale")
@@ -86,31 +104,32 @@ class Qlinear_func(Function):
     """cuda/QLinear.py:26-47.  ``row_scale`` (optional, [M]) multiplies the rows of X before
     quantization, fused into the quantize pass and, in backward, into gradX's epilogue.
     ``scaleX`` (optional, [1]) is max|X| / 127 when the producer of X already knows it
-    (a preceding Qlinear_func_reduce): no absmax pass over X runs then."""
+    (a preceding Qlinear_func_reduce): no absmax pass over X runs then.  ``Xq`` (optional, with
+    ``scaleX``): X already quantized (``quantize_input``), shared by several layers."""
 
     @staticmethod
-    def forward(ctx, X, W, b=None, row_scale=None, scaleX=None):
-        return _forward(ctx, X, W, b, False, row_scale, scaleX)
+    def forward(ctx, X, W, b=None, row_scale=None, scaleX=None, Xq=None):
+        return _forward(ctx, X, W, b, False, row_scale, scaleX, Xq)
 
     @staticmethod
     @once_differentiable
     def backward(ctx, grad_output):
-        return _backward(ctx, grad_output) + (None,)
+        return _backward(ctx, grad_output) + (None, None)
 
 
 class Qlinear_func_reduce(Function):
     """cuda/QLinear.py:50-71: also returns the output's quantization scale."""
 
     @staticmethod
-    def forward(ctx, X, W, b=None, row_scale=None, scaleX=None):
-        out, scaleO = _forward(ctx, X, W, b, True, row_scale, scaleX)
+    def forward(ctx, X, W, b=None, row_scale=None, scaleX=None, Xq=None):
+        out, scaleO = _forward(ctx, X, W, b, True, row_scale, scaleX, Xq)
         ctx.mark_non_differentiable(scaleO)
         return out, scaleO
 
     @staticmethod
     @once_differentiable
     def backward(ctx, grad_output, grad_dummy):
-        return _backward(ctx, grad_output) + (None,)
+        return _backward(ctx, grad_output) + (None, None)
 
 
 class QLinear(nn.Linear):
@@ -124,13 +143,14 @@ class QLinear(nn.Linear):
     def enable_reduce(self):
         self.isReduce = True
 
-    def forward(self, input, scale=None):
+    def forward(self, input, scale=None, input_q=None):
         """``scale``: max|input| / 127 if the caller has it (the second output of a preceding
-        layer with enable_reduce()); the reference's layer always recomputes it."""
+        layer with enable_reduce()); the reference's layer always recomputes it.  ``input_q``
+        (with ``scale``): the input already quantized by ``quantize_input``."""
         t = input.reshape(-1, input.size(-1))
         out_shape = input.shape[:-1] + (self.weight.size(0),)
         if self.isReduce:
-            out, oscale = Qlinear_func_reduce.apply(t, self.weight, self.bias, None, scale)
+            out, oscale = Qlinear_func_reduce.apply(t, self.weight, self.bias, None, scale, input_q)
             return out.reshape(out_shape), oscale
-        out = Qlinear_func.apply(t, self.weight, self.bias, None, scale)
+        out = Qlinear_func.apply(t, self.weight, self.bias, None, scale, input_q)
         return out.reshape(out_shape)

@@ -1108,19 +1108,21 @@ int tango_qgemm_fwd_ex(float* Y, int64_t ldy, const float* X, int64_t ldx, const
                     const float* scaleX, const float* scaleW, int64_t M, int64_t N, int64_t K,
                     int round_mode, void* workspace, size_t workspace_bytes,
                     tango_stream_t stream) {
-    if (M < 0 || N < 0 || K < 0 || !scaleX || !scaleW || ldy < N || ldx < K || ldw < K || ldxq < K)
+    if (M < 0 || N < 0 || K < 0 || !scaleX || !scaleW || ldy < N || (X && ldx < K) || ldw < K || ldxq < K)
         return TANGO_ERR_INVALID_ARG;
     if (M * N > 0 && !Y) return TANGO_ERR_INVALID_ARG;
-    if (M * K > 0 && (!X || !Xq)) return TANGO_ERR_INVALID_ARG;
+    const bool cached = X == nullptr;  // Xq is an input: the caller has quantized X already
+    if (M * K > 0 && !Xq) return TANGO_ERR_INVALID_ARG;
+    if (cached && x_row_mul) return TANGO_ERR_INVALID_ARG;
     if (N * K > 0 && (!W || !Wq)) return TANGO_ERR_INVALID_ARG;
     if (round_mode < 0 || round_mode > 2) return TANGO_ERR_UNSUPPORTED;
     const size_t need = tango_qgemm_fwd_workspace(M, N, K);
     if (need > 0 && (!workspace || workspace_bytes < need)) return TANGO_ERR_WORKSPACE;
     if ((reinterpret_cast<uintptr_t>(workspace) & 15) != 0) return TANGO_ERR_INVALID_ARG;
     hipStream_t s = as_stream(stream);
-    const bool fused = M > 0 && N > 0 && fq_applicable(X, ldx, Xq, ldxq, K, round_mode);
+    const bool fused = !cached && M > 0 && N > 0 && fq_applicable(X, ldx, Xq, ldxq, K, round_mode);
     int rc = TANGO_OK;
-    if (!fused) {
+    if (!fused && !cached) {
         rc = tango_quantize_rows_ex_f32_i8(X, M, K, ldx, x_row_mul, nullptr, 0, 0, scaleX, 0, Xq, ldxq, round_mode,
                                            nullptr, 0, 0, stream);
         if (rc != TANGO_OK) return rc;

@@ -9,7 +9,7 @@ import torch.nn.functional as F
 
 from torch.autograd.function import Function, once_differentiable
 
-from .QLinear import QLinear
+from .QLinear import QLinear, quantize_input
 from .kernels import cuda_kernels
 from .SDDMM import sddmm_u_add_v, sddmm_u_dot_v
 from .SPMM import spmm_u_mul_e
@@ -149,12 +149,12 @@ class HGTLayer(nn.Module):
             lin.enable_reduce()
 
     def forward(self, g, h):
-        s_h = cuda_kernels.get_scale(h if h.is_contiguous() else h.contiguous())  # one absmax pass for the three projections of h
-        k, s_k = self.k_linear(h, s_h)
+        h_q, s_h = quantize_input(h)  # one absmax and one quantize pass for the three projections of h
+        k, s_k = self.k_linear(h, s_h, h_q)
         k, s_k = self.attn_linear(k, s_k)
-        v, s_v = self.v_linear(h, s_h)
+        v, s_v = self.v_linear(h, s_h, h_q)
         v, s_v = self.msg_linear(v, s_v)
-        q, s_q = self.q_linear(h, s_h)
+        q, s_q = self.q_linear(h, s_h, h_q)
         k, v, q = (t.view(-1, self.n_heads, self.d_k) for t in (k, v, q))
         t = sddmm_u_dot_v.apply(g, k, q, s_k, s_q) / self.sqrt_dk
         attn = edge_softmax(g, t)

@@ -278,15 +278,20 @@ class cuda_kernels:
     # ------------------------------------------------------------------ GEMM
     @staticmethod
     def QGEMM_forward(Y, X, X_q, W, W_q, bias, scaleY, scaleX, scaleW, round_mode=None, x_row_mul=None):
+        """``X`` None: ``X_q`` already holds X quantized with ``scaleX`` (one quantize pass shared by
+        several layers that consume the same X)."""
         for t, dt, nm in ((Y, torch.float32, "Y"), (X, torch.float32, "X"), (W, torch.float32, "W")):
-            _need(t, dt, nm, contiguous=False)
+            if t is not None:
+                _need(t, dt, nm, contiguous=False)
         _need(X_q, torch.int8, "X_q", contiguous=False)
         _need(W_q, torch.int8, "W_q")
         _need(scaleX, torch.float32, "scaleX")
         _need(scaleW, torch.float32, "scaleW")
-        M, K = X.shape
+        M, K = X_q.shape
+        if X is None and x_row_mul is not None:
+            raise RuntimeError("QGEMM_forward: x_row_mul needs the fp32 X")
         N = W.size(0)
-        if (W.size(1) != K or tuple(Y.shape) != (M, N) or tuple(X_q.shape) != (M, K)
+        if (W.size(1) != K or tuple(Y.shape) != (M, N) or (X is not None and tuple(X.shape) != (M, K))
                 or W_q.numel() != N * K):
             raise RuntimeError("QGEMM_forward: shape mismatch")
         if bias is not None and bias.numel():
@@ -297,12 +302,12 @@ class cuda_kernels:
             _need(scaleY, torch.float32, "scaleY")
         mode = default_forward_round_mode() if round_mode is None else _mode(round_mode)
         ws_bytes = _ws_bytes("tango_qgemm_fwd_workspace", M, N, K)
-        ws = _workspace(ws_bytes, X.device)
+        ws = _workspace(ws_bytes, X_q.device)
         if x_row_mul is not None:
             _need(x_row_mul, torch.float32, "x_row_mul")
             if x_row_mul.numel() != M:
                 raise RuntimeError("QGEMM_forward: x_row_mul must have M entries")
-        check(_L.tango_qgemm_fwd_ex(_ptr(Y), _rows_view(Y, "Y"), _ptr(X), _rows_view(X, "X"), _ptr(x_row_mul),
+        check(_L.tango_qgemm_fwd_ex(_ptr(Y), _rows_view(Y, "Y"), _ptr(X), 0 if X is None else _rows_view(X, "X"), _ptr(x_row_mul),
                                     _ptr(X_q), _rows_view(X_q, "X_q"), _ptr(W), _rows_view(W, "W"), _ptr(W_q),
                                     _ptr(bias), _ptr(scaleY),
                                  scaleX.data_ptr(), scaleW.data_ptr(), M, N, K, mode, _ptr(ws),
@@ -653,12 +658,12 @@ def mySDDMM_int8(g, op, U, V, scaleU, scaleV, isReduce, reverse=False):
 
 
 def QGEMM_forward(x, x_, scaleX, w, w_, scaleW, bias=None, isReduce=False, round_mode=None, x_row_mul=None):
-    """cuda/kernels.py:79-95."""
-    assert x.is_cuda, "x must be on GPU"
+    """cuda/kernels.py:79-95.  ``x`` None: ``x_`` is an input (x quantized with scaleX by the caller)."""
+    assert x_.is_cuda, "x must be on GPU"
     assert w.is_cuda, "w must be on GPU"
     assert bias is None or bias.is_cuda, "bias must be on GPU"
-    assert x.size(1) == w.size(1), "x and w must have the same number of columns"
-    out_fp = torch.empty((x.size(0), w.size(0)), dtype=torch.float32, device=x.device)
+    assert x_.size(1) == w.size(1), "x and w must have the same number of columns"
+    out_fp = torch.empty((x_.size(0), w.size(0)), dtype=torch.float32, device=x_.device)
     scale_out = torch.empty_like(scaleX) if isReduce else torch.Tensor()
     bias = torch.Tensor() if bias is None else bias
     cuda_kernels.QGEMM_forward(out_fp, x, x_, w, w_, bias, scale_out, scaleX, scaleW,

@@ -317,3 +317,30 @@ def test_forward_gemm_tall_narrow(K, orc, Kd, N, mode, bias):
     Yo, Xqo, _, osX, _, osY = orc.qgemm_fwd(Xs, W, b, reduce=True, mode=orc.RNE if mode == "rne" else orc.TRUNC)
     assert host(sX)[0] == osX and np.array_equal(host(Xq), Xqo)
     assert np.array_equal(host(Y), Yo) and host(sY)[0] == osY
+
+
+@pytest.mark.parametrize("M,Kd,N", [(3000, 256, 256), (1000, 100, 41), (500, 602, 64)])
+def test_linear_layers_sharing_one_quantized_input(M, Kd, N):
+    """QLinear fed the already quantized input (one quantize pass shared by several layers, as the q / k / v
+    projections of the HGT layer use it) == QLinear quantizing the input itself: outputs, output scales and
+    all gradients bit for bit."""
+    from tango_amd.QLinear import QLinear, quantize_input
+    torch.manual_seed(M + N)
+    a, b = QLinear(Kd, N).cuda(), QLinear(Kd, N, bias=False).cuda()
+    a.enable_reduce()
+    x = torch.randn(M, Kd, device="cuda", requires_grad=True)
+    w = torch.randn(M, N, device="cuda")
+    outs, grads = [], []
+    for shared in (False, True):
+        for t in (x, *a.parameters(), *b.parameters()):
+            t.grad = None
+        if shared:
+            xq, sx = quantize_input(x.detach())
+            (ya, sa), yb = a(x, sx, xq), b(x, sx, xq)
+        else:
+            (ya, sa), yb = a(x), b(x)
+        ((ya * w).sum() + (yb * w).sum() * 0.5).backward()
+        outs.append((ya.detach().clone(), sa.clone(), yb.detach().clone()))
+        grads.append([t.grad.clone() for t in (x, *a.parameters(), *b.parameters())])
+    assert all(torch.equal(p, q) for p, q in zip(*outs))
+    assert all(torch.equal(p, q) for p, q in zip(*grads))
