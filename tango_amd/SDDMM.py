@@ -44,14 +44,24 @@ class sddmm_u_add_v(Function):
 class sddmm_u_dot_v(Function):
     """out[e, h, 0] = <U[src[e], h, :], V[dst[e], h, :]>.  Built by symmetry with
     spmm_u_mul_e: the backward is two u_mul_e aggregations with dZ as the edge value.
-    ``scaleU_`` / ``scaleV_`` may come from the producers of U and V (as in sddmm_u_add_v)."""
+    ``scaleU_`` / ``scaleV_`` may come from the producers of U and V (as in sddmm_u_add_v).
+    ``out_scale`` (a Python float) multiplies the result, e.g. the 1 / sqrt(d_k) of an attention
+    score (evaluation/test_HGT.py:58): it is folded into the dequantization scales of the forward
+    and of both backward aggregations, so no pass over the [E, H] tensor runs for it (bit-identical
+    to multiplying afterwards when it is a power of two, else within an ulp or two)."""
 
     @staticmethod
-    def forward(ctx, g, U, V, scaleU_=None, scaleV_=None):
+    def forward(ctx, g, U, V, scaleU_=None, scaleV_=None, out_scale=None):
         U_, scaleU = quantize(U if U.is_contiguous() else U.contiguous(), scaleU_)
         V_, scaleV = quantize(V if V.is_contiguous() else V.contiguous(), scaleV_)
-        out, _ = mySDDMM_int8(g, "dot", U_, V_, scaleU, scaleV, False)
-        ctx.backward_cache = g, U_, scaleU, V_, scaleV
+        if out_scale is not None:
+            # 1-element products: the forward dequantizes with sU * (sV c), the backward passes with
+            # s_dZ * (sV c) and s_dZ * (sU c)
+            scaleU_c, scaleV_c = scaleU * out_scale, scaleV * out_scale
+        else:
+            scaleU_c, scaleV_c = scaleU, scaleV
+        out, _ = mySDDMM_int8(g, "dot", U_, V_, scaleU, scaleV_c, False)
+        ctx.backward_cache = g, U_, scaleU_c, V_, scaleV_c
         return out
 
     @staticmethod
@@ -69,4 +79,4 @@ class sddmm_u_dot_v(Function):
             dU = multi_cusparse_SPMM(g, V3, dZ_, scaledZ, True, edge_major=True, scale2=scaleV).reshape(U_.shape)
         if ctx.needs_input_grad[2]:
             dV = multi_cusparse_SPMM(g, U3, dZ_, scaledZ, edge_major=True, scale2=scaleU).reshape(V_.shape)
-        return None, dU, dV, None, None
+        return None, dU, dV, None, None, None

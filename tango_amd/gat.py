@@ -156,7 +156,7 @@ class HGTLayer(nn.Module):
         v, s_v = self.msg_linear(v, s_v)
         q, s_q = self.q_linear(h, s_h, h_q)
         k, v, q = (t.view(-1, self.n_heads, self.d_k) for t in (k, v, q))
-        t = sddmm_u_dot_v.apply(g, k, q, s_k, s_q) / self.sqrt_dk
+        t = sddmm_u_dot_v.apply(g, k, q, s_k, s_q, 1.0 / self.sqrt_dk)  # "/ sqrt_dk" folded into the scales
         attn = edge_softmax(g, t)
         t = spmm_u_mul_e.apply(g, v, attn, None, s_v).reshape(-1, self.out_dim)
         return self.a_linear(t)

@@ -172,6 +172,17 @@ def test_sddmm_u_add_v_and_dot_backward(orc):
     ref.backward(g_out)
     assert rel_err(sc_.detach(), ref.detach()) < 0.03
     assert rel_err(Q.grad, Qr.grad) < 0.04 and rel_err(Kt.grad, Kr.grad) < 0.04
+    # a result multiplier folded into the scales: a power of two is bit-identical to multiplying the result
+    # afterwards (forward and both gradients), any other factor agrees to rounding
+    for c, exact in ((0.125, True), (1.0 / 3.0, False)):
+        Q2, K2 = dev(Qf).requires_grad_(True), dev(Kf).requires_grad_(True)
+        folded = sddmm_u_dot_v.apply(g, Q2, K2, None, None, c)
+        folded.backward(g_out)
+        Q3, K3 = dev(Qf).requires_grad_(True), dev(Kf).requires_grad_(True)
+        after = sddmm_u_dot_v.apply(g, Q3, K3) * c
+        after.backward(g_out)
+        same = torch.equal if exact else (lambda a, b: torch.allclose(a, b, rtol=1e-6, atol=1e-7))
+        assert same(folded.detach(), after.detach()) and same(Q2.grad, Q3.grad) and same(K2.grad, K3.grad), c
 
 
 def test_edge_softmax_autograd():
