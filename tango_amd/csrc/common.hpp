@@ -65,14 +65,11 @@ __device__ __forceinline__ void block_absmax_to_global(float v, float* out) {
     if (w == 0) {
         float m = (tid < nw) ? part[tid] : 0.0f;
         m = wave_max(m);
-        if (tid == 0) {
-            // Atomics on one address are served one at a time (some 15 ns each): a kernel of thousands of
-            // short workgroups would wait for them.  The stored maximum only grows, so a workgroup whose
-            // value does not exceed what it reads there (device-coherent load) has nothing to add.
-            int* slot = reinterpret_cast<int*>(out);
-            const int mine = __float_as_int(m);
-            if (mine > __hip_atomic_load(slot, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)) atomicMax(slot, mine);
-        }
+        // Fire and forget.  Atomics on one address are served one at a time (some 15 ns each), in the
+        // background of the kernel; reading the slot first to skip the atomic was tried, at the end of a
+        // workgroup and at its start, and either way the coherent load of that hot address stalls the
+        // workgroup for longer than the atomic costs.
+        if (tid == 0) atomicMax(reinterpret_cast<int*>(out), __float_as_int(m));
     }
 }
 

@@ -228,9 +228,10 @@ __global__ __launch_bounds__(64 * WAVES) void gemm_nts_kernel(const NtParams p, 
     const uintptr_t ca = reinterpret_cast<uintptr_t>(p.C);
     const int wide = ((ca & 15) == 0 && (p.ldc & 3) == 0) ? 4 : ((ca & 7) == 0 && (p.ldc & 1) == 0) ? 2 : 1;
     float m = 0.0f;
-    auto load_tile = [&](i32x4* a, int t) {
+    auto load_tile = [&](i32x4* a, float& rsc, int t) {
         const int64_t row = static_cast<int64_t>(t) * 16 + r16;
         const bool ok = t < ntiles && row < p.M;
+        rsc = (p.row_scale && ok) ? p.row_scale[row] : 1.0f;  // requested with the tile, not in the epilogue
         const int8_t* pa = p.A + (ok ? row : 0) * p.lda + g * 16;
 #pragma unroll
         for (int st = 0; st < KS; ++st) {
@@ -241,10 +242,11 @@ __global__ __launch_bounds__(64 * WAVES) void gemm_nts_kernel(const NtParams p, 
     };
     const int stride = static_cast<int>(gridDim.x) * WAVES;
     i32x4 cur[KS], nxt[KS];
+    float rsc, rsc_nxt;
     int t = static_cast<int>(blockIdx.x) * WAVES + wave;
-    load_tile(cur, t);
+    load_tile(cur, rsc, t);
     for (; t < ntiles; t += stride) {
-        load_tile(nxt, t + stride);
+        load_tile(nxt, rsc_nxt, t + stride);
         i32x4 acc[NT];
 #pragma unroll
         for (int j = 0; j < NT; ++j) acc[j] = i32x4{0, 0, 0, 0};
@@ -262,7 +264,6 @@ __global__ __launch_bounds__(64 * WAVES) void gemm_nts_kernel(const NtParams p, 
         const int64_t row = static_cast<int64_t>(t) * 16 + r16;
         if (row < p.M) {
             float* crow = p.C + row * p.ldc;
-            const float rsc = p.row_scale ? p.row_scale[row] : 1.0f;
 #pragma unroll
             for (int j = 0; j < NT; ++j) {
                 const int64_t col = n0 + j * 16 + g * 4;
@@ -290,6 +291,7 @@ __global__ __launch_bounds__(64 * WAVES) void gemm_nts_kernel(const NtParams p, 
         }
 #pragma unroll
         for (int st = 0; st < KS; ++st) cur[st] = nxt[st];
+        rsc = rsc_nxt;
     }
     if (p.absmax_out) block_absmax_to_global(m / 127.0f, p.absmax_out);
 }

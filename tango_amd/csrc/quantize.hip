@@ -78,6 +78,42 @@ __global__ __launch_bounds__(256) void absmax_kernel(const float* __restrict__ x
     block_absmax_to_global(m / 127.0f, out);
 }
 
+// max |x[r, c] * row_mul[r]| / 127 of a dense matrix (no padding between rows) with an even number of columns,
+// walked as a flat array of 16-byte vectors like absmax_kernel: rows whose length is not a multiple of four
+// floats (602 columns) then cost no narrow loads.  A vector starts at an even column, so it lies in one row
+// or has its second half in the next; the (row, column) of a lane's vector advances by a fixed step.
+__global__ __launch_bounds__(256) void absmax_rowmul_dense_kernel(const float* __restrict__ x, int64_t n, int64_t cols,
+                                                                  const float* __restrict__ row_mul,
+                                                                  float* __restrict__ out) {
+    const int64_t tid = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    const int64_t nthr = static_cast<int64_t>(gridDim.x) * blockDim.x;
+    const int64_t n4 = n >> 2;
+    const f32x4* x4 = reinterpret_cast<const f32x4*>(x);
+    int64_t row = (4 * tid) / cols, col = (4 * tid) % cols;
+    const int64_t srow = (4 * nthr) / cols, scol = (4 * nthr) % cols;
+    float m = 0.0f;
+    auto take = [&](const f32x4 v) {
+        const float r0 = row_mul[row];
+        const float r1 = (col + 2 >= cols) ? row_mul[row + 1] : r0;
+        m = fmaxf(m, fmaxf(fmaxf(fabsf(v.x * r0), fabsf(v.y * r0)), fmaxf(fabsf(v.z * r1), fabsf(v.w * r1))));
+        row += srow;
+        col += scol;
+        if (col >= cols) { col -= cols; ++row; }
+    };
+    int64_t i = tid;
+    for (; i + 3 * nthr < n4; i += 4 * nthr) {
+        const f32x4 a = __builtin_nontemporal_load(x4 + i);
+        const f32x4 b = __builtin_nontemporal_load(x4 + i + nthr);
+        const f32x4 c = __builtin_nontemporal_load(x4 + i + 2 * nthr);
+        const f32x4 d = __builtin_nontemporal_load(x4 + i + 3 * nthr);
+        take(a); take(b); take(c); take(d);
+    }
+    for (; i < n4; i += nthr) take(__builtin_nontemporal_load(x4 + i));
+    const int64_t t = (n4 << 2) + tid;  // at most two elements remain, in the last row
+    if (t < n) m = fmaxf(m, fabsf(x[t] * row_mul[t / cols]));
+    block_absmax_to_global(m / 127.0f, out);
+}
+
 // One workgroup, direct store: small tensors need no atomic and no pre-zeroing.
 __global__ __launch_bounds__(1024) void absmax_small_kernel(const float* __restrict__ x, int64_t n,
                                                             float* __restrict__ out) {
@@ -177,6 +213,69 @@ __global__ __launch_bounds__(256) void quantize_vec_kernel(
     }
 }
 
+// x under the mask value mk of a fused activation backward.  Mode 0 (ReLU): x where mk > 0, else 0.
+// Mode 1 (ELU, mk = the activation's output): x where mk > 0, else x * (mk + 1), since
+// d/dz (exp(z) - 1) = exp(z) = elu(z) + 1.
+__device__ __forceinline__ float masked(float x, float mk, int mode) {
+    if (mk > 0.0f) return x;
+    return mode == 1 ? x * (mk + 1.0f) : 0.0f;
+}
+
+// quantize_rows_kernel's job on dense matrices whose rows hold a multiple of four columns (x, q and the
+// mask all [rows, cols] without padding): the flat walk of quantize_vec_kernel, a lane's four elements
+// never straddle a row, and the row index (for row_mul) advances by a fixed step per iteration.
+template <int MODE>
+__global__ __launch_bounds__(256) void quantize_dense_ex_kernel(
+    const float* __restrict__ x, int64_t n4, int64_t cols, const float* __restrict__ scale,
+    int8_t* __restrict__ q, const float* __restrict__ noise, uint64_t seed, uint64_t offset,
+    const float* __restrict__ row_mul, const float* __restrict__ mask, int mask_mode) {
+    const int64_t tid = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    const int64_t nthr = static_cast<int64_t>(gridDim.x) * blockDim.x;
+    const float r = rscale_of(scale[0]);
+    const f32x4* x4 = reinterpret_cast<const f32x4*>(x);
+    const f32x4* m4 = reinterpret_cast<const f32x4*>(mask);
+    uint32_t* q4 = reinterpret_cast<uint32_t*>(q);
+    const bool shared_block = (offset & 3) == 0;
+    int64_t row = (4 * tid) / cols, col = (4 * tid) % cols;
+    const int64_t srow = (4 * nthr) / cols, scol = (4 * nthr) % cols;
+    for (int64_t i = tid; i < n4; i += nthr) {
+        const f32x4 v = __builtin_nontemporal_load(x4 + i);
+        float f[4] = {v.x, v.y, v.z, v.w};
+        if (mask) {
+            const f32x4 mk = __builtin_nontemporal_load(m4 + i);
+            f[0] = masked(f[0], mk.x, mask_mode); f[1] = masked(f[1], mk.y, mask_mode);
+            f[2] = masked(f[2], mk.z, mask_mode); f[3] = masked(f[3], mk.w, mask_mode);
+        }
+        if (row_mul) {
+            const float rm = row_mul[row];
+#pragma unroll
+            for (int k = 0; k < 4; ++k) f[k] = f[k] * rm;
+            row += srow;
+            col += scol;
+            if (col >= cols) { col -= cols; ++row; }
+        }
+        float u[4] = {0.f, 0.f, 0.f, 0.f};
+        if (MODE == TANGO_ROUND_STOCHASTIC) {
+            if (noise) {
+#pragma unroll
+                for (int k = 0; k < 4; ++k) u[k] = noise[4 * i + k];
+            } else if (shared_block) {
+                const uint64_t blk = (offset + 4 * static_cast<uint64_t>(i)) >> 2;
+                const Philox4 p = philox4x32_10(static_cast<uint32_t>(blk), static_cast<uint32_t>(blk >> 32), 0u, 0u,
+                                                static_cast<uint32_t>(seed), static_cast<uint32_t>(seed >> 32));
+#pragma unroll
+                for (int k = 0; k < 4; ++k) u[k] = u01(p.v[k]);
+            } else {
+                const uint64_t g = offset + 4 * static_cast<uint64_t>(i);
+#pragma unroll
+                for (int k = 0; k < 4; ++k) u[k] = philox_uniform(seed, g + k);
+            }
+        }
+        __builtin_nontemporal_store(pack4(quant_one<MODE>(f[0], r, u[0]), quant_one<MODE>(f[1], r, u[1]),
+                                          quant_one<MODE>(f[2], r, u[2]), quant_one<MODE>(f[3], r, u[3])), q4 + i);
+    }
+}
+
 // Scalar fallback for misaligned views.
 template <int MODE>
 __global__ __launch_bounds__(256) void quantize_scalar_kernel(
@@ -212,14 +311,6 @@ __device__ __forceinline__ void load4(float* f, const float* __restrict__ row, i
     }
 }
 
-// x under the mask value mk of a fused activation backward.  Mode 0 (ReLU): x where mk > 0, else 0.
-// Mode 1 (ELU, mk = the activation's output): x where mk > 0, else x * (mk + 1), since
-// d/dz (exp(z) - 1) = exp(z) = elu(z) + 1.
-__device__ __forceinline__ float masked(float x, float mk, int mode) {
-    if (mk > 0.0f) return x;
-    return mode == 1 ? x * (mk + 1.0f) : 0.0f;
-}
-
 // Row-strided: blockDim = (64, 4); each wavefront walks one row at a time, one lane per
 // output dword (4 columns, padding included), so no per-thread index division is needed and
 // a wavefront's loads and stores are contiguous.  XV = floats per aligned load (4, 2 or 1).
@@ -234,6 +325,7 @@ __global__ __launch_bounds__(256) void quantize_rows_kernel(
     const bool mask_vec = mask && ldm == ldx &&
                           ((reinterpret_cast<uintptr_t>(mask) ^ reinterpret_cast<uintptr_t>(x)) & 15) == 0;
     const int64_t groups = (ldq + 3) >> 2;  // dword groups per row
+    const bool quad_aligned = (cols & 3) == 0 && (offset & 3) == 0;  // every lane's quad starts a Philox block
     const bool dword_ok = (ldq & 3) == 0 && (reinterpret_cast<uintptr_t>(q) & 3) == 0;
     // narrow rows: a wavefront takes 64 / gpr rows at once (gpr = groups rounded up to a power of two)
     const int gpr = 1 << gpr_log2;
@@ -269,20 +361,28 @@ __global__ __launch_bounds__(256) void quantize_rows_kernel(
                     for (int k = 0; k < 4; ++k)
                         if (c0 + k < cols) u[k] = noise[lin + k];
                 } else {
-                    // the four elements touch at most two Philox blocks
                     const uint64_t g0 = offset + lin;
                     const uint64_t b0 = g0 >> 2;
                     const Philox4 p0 = philox4x32_10(static_cast<uint32_t>(b0), static_cast<uint32_t>(b0 >> 32), 0u, 0u,
                                                      static_cast<uint32_t>(seed), static_cast<uint32_t>(seed >> 32));
+                    if (quad_aligned) {  // uniform: a lane's four elements are exactly one Philox block
+#pragma unroll
+                        for (int k = 0; k < 4; ++k) u[k] = u01(p0.v[k]);
+                    } else {
+                    // the four elements touch two Philox blocks
                     Philox4 p1 = p0;
                     if (g0 & 3)
                         p1 = philox4x32_10(static_cast<uint32_t>(b0 + 1), static_cast<uint32_t>((b0 + 1) >> 32), 0u, 0u,
                                            static_cast<uint32_t>(seed), static_cast<uint32_t>(seed >> 32));
+                    // words shift .. shift + 3 of the eight, picked with selects (a register array indexed
+                    // by a run-time value would live in scratch memory)
+                    const int shift = static_cast<int>(g0 & 3);
+                    const uint32_t w[8] = {p0.v[0], p0.v[1], p0.v[2], p0.v[3], p1.v[0], p1.v[1], p1.v[2], p1.v[3]};
+                    uint32_t h[6];
 #pragma unroll
-                    for (int k = 0; k < 4; ++k) {
-                        const uint64_t gk = g0 + k;
-                        const Philox4& pk = ((gk >> 2) == b0) ? p0 : p1;
-                        u[k] = u01(pk.v[gk & 3]);
+                    for (int i = 0; i < 6; ++i) h[i] = (shift & 1) ? w[i + 1] : w[i];
+#pragma unroll
+                    for (int k = 0; k < 4; ++k) u[k] = u01((shift & 2) ? h[k + 2] : h[k]);
                     }
                 }
             }
@@ -552,6 +652,14 @@ int tango_absmax_ex_f32(const float* x, int64_t rows, int64_t cols, int64_t ldx,
         partial = static_cast<float*>(workspace);
     }
     if (cols == 0) return launch_status();
+    if (row_mul && !mask && !colsum_out && ldx == cols && (cols & 1) == 0 && (cols & 3) != 0 &&
+        (reinterpret_cast<uintptr_t>(x) & 15) == 0 && rows * cols >= (1 << 16)) {
+        // rows of 8-byte alignment only: the flat walk reads them with 16-byte loads all the same
+        const int64_t n = rows * cols;
+        hipLaunchKernelGGL(absmax_rowmul_dense_kernel, dim3(grid_for(n / 16, 256, 2)), dim3(256), 0, s, x, n, cols,
+                           row_mul, scale_out);
+        return launch_status();
+    }
     const dim3 block(64, 4);
     const int T = static_cast<int>(ceil_div(cols, 256));
     int gpr_log2 = 6;
@@ -615,6 +723,17 @@ int tango_quantize_rows_ex_f32_i8(const float* x, int64_t rows, int64_t cols, in
         return TANGO_ERR_INVALID_ARG;
     if (rows == 0 || ldq == 0) return (round_mode >= 0 && round_mode <= 2) ? TANGO_OK : TANGO_ERR_UNSUPPORTED;
     hipStream_t s = as_stream(stream);
+    if ((row_mul || mask) && !per_row && cols > 0 && (cols & 3) == 0 && ldx == cols && ldq == cols &&
+        (!mask || ldm == cols) && (reinterpret_cast<uintptr_t>(x) & 15) == 0 &&
+        (reinterpret_cast<uintptr_t>(mask) & 15) == 0 && (reinterpret_cast<uintptr_t>(q) & 3) == 0) {
+        const int64_t n4 = rows * (cols >> 2);
+        int rc = dispatch_mode(round_mode, [&](auto mode) {
+            constexpr int M = decltype(mode)::value;
+            hipLaunchKernelGGL(quantize_dense_ex_kernel<M>, dim3(grid_for(n4, 256)), dim3(256), 0, s, x, n4, cols, scale,
+                               q, noise, seed, offset, row_mul, mask, mask_mode);
+        });
+        return rc != TANGO_OK ? rc : launch_status();
+    }
     const int64_t groups = (ldq + 3) >> 2;
     int gpr_log2 = 6;
     while (gpr_log2 > 0 && (1LL << (gpr_log2 - 1)) >= groups) --gpr_log2;

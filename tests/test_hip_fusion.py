@@ -38,8 +38,9 @@ def test_absmax_ex_and_quantize_ex(K, orc):
         q, s3 = K.quantize_padded(dev(x), row_mul=dev(rm), mask=dev(mask))
         assert host(s3)[0] == host(s)[0]
         assert np.array_equal(host(q), orc.quantize(scaled, host(s)[0]))
-        q2, _ = K.quantize_padded(dev(x), s, row_mul=dev(rm), mask=dev(mask), round_mode="stochastic", seed=3, offset=64)
-        assert np.array_equal(host(q2), orc.quantize(scaled, host(s)[0], orc.STOCHASTIC, seed=3, offset=64))
+        for off in (64, 66):  # a lane's four elements inside one block of the random stream / across two
+            q2, _ = K.quantize_padded(dev(x), s, row_mul=dev(rm), mask=dev(mask), round_mode="stochastic", seed=3, offset=off)
+            assert np.array_equal(host(q2), orc.quantize(scaled, host(s)[0], orc.STOCHASTIC, seed=3, offset=off))
         # ELU backward: elements whose mask (the activation's output) is not positive are multiplied by mask + 1
         emask = np.where(mask > 0, mask, np.expm1(mask)).astype(np.float32)
         through = np.where(emask > 0, x, x * (emask + np.float32(1))).astype(np.float32)
@@ -54,6 +55,17 @@ def test_absmax_ex_and_quantize_ex(K, orc):
     a = K.cuda_kernels.absmax_ex(x, want_colsum=True)[1]
     b = K.cuda_kernels.absmax_ex(x, want_colsum=True)[1]
     assert torch.equal(a, b)
+
+
+@pytest.mark.parametrize("rows,cols", [(1001, 602), (333, 602), (2000, 86), (40000, 2)])
+def test_absmax_with_row_multiplier_on_dense_rows_of_even_length(K, orc, rows, cols):
+    """Rows whose length is even but not a multiple of four floats are read as one flat array of 16-byte
+    vectors (a vector may end in the next row); an odd row count leaves a two-element tail."""
+    rng = np.random.default_rng(rows + cols)
+    x = rng.standard_normal((rows, cols)).astype(np.float32)
+    rm = (rng.random(rows, dtype=np.float32) + 0.1) * np.where(rng.random(rows) < 0.01, 50, 1).astype(np.float32)
+    s, cs = K.cuda_kernels.absmax_ex(dev(x), row_mul=dev(rm))
+    assert cs is None and host(s)[0] == orc.absmax_scale((x * rm[:, None]).astype(np.float32))
 
 
 # (n, e): rows of ~66 slots (one wave per row), and a sparse graph with a long row and a hub row (the epilogue
