@@ -154,6 +154,14 @@ def primitives(g, K, torch):
         out[tag.replace("fwd", "gradW")] = {"ms": round(ms, 4), "TOPS": round(ops / ms / 1e9, 2),
                                             "GBps": round(byt / ms / 1e6, 1)}
         del X, W, Xq, dY
+    # the int8 matrix rate the device sustains on register-resident operands (the ceiling of any int8 GEMM here)
+    from tango_amd import _lib
+    sink = torch.zeros(1, dtype=torch.int32, device="cuda")
+    wgs, iters = 256 * 8, 4096
+    stream = torch.cuda.current_stream().cuda_stream
+    ms = time_op(lambda: _lib.check(_lib.lib().tango_probe_mfma_i8(wgs, iters, sink.data_ptr(), stream), "probe"), iters=5)
+    out["mfma_i8_probe"] = {"ms": round(ms, 4), "TOPS": round(wgs * 4 * iters * 8 * 32768.0 / ms / 1e9, 1),
+                            "published_peak_TOPS": 5000.0}
     # quantize / absmax streaming
     X = torch.randn(n, 602, device="cuda")
     ms = time_op(lambda: K.cuda_kernels.get_scale(X))

@@ -147,6 +147,12 @@ int tango_qgemm_fwd_ex(float* Y, int64_t ldy, const float* X, int64_t ldx, const
                        int64_t M, int64_t N, int64_t K, int round_mode, void* workspace,
                        size_t workspace_bytes, tango_stream_t stream);
 
+/* Measurement aid (no counterpart in the reference): launches `workgroups` workgroups of four waves that
+   each issue iters * 8 register-resident v_mfma_i32_16x16x64_i8 (32768 int8 operations per instruction
+   and wave) and nothing else, so that a caller timing the launch learns the int8 matrix rate the device
+   sustains.  sink: one int of device memory (practically never written). */
+int tango_probe_mfma_i8(int64_t workgroups, int64_t iters, int* sink, tango_stream_t stream);
+
 /* Integer GEMM on operands that are already int8 (no counterpart in the
    reference, whose forward always re-quantizes; same epilogue as above):
    Y[m,n] = (sA*sB) * float(sum_k A[m,k]*B[n,k]) (+ bias[n]), optional scaleY. */

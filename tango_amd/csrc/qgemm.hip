@@ -705,6 +705,26 @@ __global__ __launch_bounds__(768) void gemm_ws_kernel(const FqParams p, int nblo
     if (p.absmax_out) block_absmax_to_global(m / 127.0f, p.absmax_out);
 }
 
+// ------------------------------------------------ MFMA rate probe (measurement only)
+// Register-resident v_mfma_i32_16x16x64_i8: eight independent accumulator chains per wave, operands never
+// reloaded.  The sustained rate of this loop is the ceiling any int8 GEMM here can reach; the benchmark
+// prints it beside the published peak.
+__global__ __launch_bounds__(256) void mfma_i8_probe_kernel(int iters, int* __restrict__ sink) {
+    const int lane = threadIdx.x & 63;
+    const i32x4 a{lane, lane + 1, lane + 2, lane + 3}, b{lane * 3, 1, 2, lane};
+    i32x4 acc[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) acc[j] = i32x4{j, 0, 0, 0};
+    for (int it = 0; it < iters; ++it) {
+#pragma unroll
+        for (int j = 0; j < 8; ++j) acc[j] = mfma_16x16x64(a, b, acc[j]);
+    }
+    int v = 0;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) v ^= acc[j].x ^ acc[j].y ^ acc[j].z ^ acc[j].w;
+    if (v == 0x7fffffff) sink[0] = v;  // keeps the loop alive; practically never true
+}
+
 // ------------------------------------------------------- operand packing
 // dst[r, 0..ldd) = src[r, 0..cols) zero-filled, for r < rows (src row stride lds).
 __global__ __launch_bounds__(256) void pack_rows_i8_kernel(int8_t* __restrict__ dst, int64_t ldd,
@@ -1154,6 +1174,13 @@ int tango_qgemm_fwd_ex(float* Y, int64_t ldy, const float* X, int64_t ldx, const
     p.C = Y; p.A = Xq; p.B = Bp; p.bias = bias; p.absmax_out = scaleY; p.sA = scaleX; p.sB = scaleW;
     p.M = M; p.N = N; p.Kr = K; p.lda = ldxq; p.ldb = ldb; p.ldc = ldy;
     return launch_nt(p, s, true);
+}
+
+int tango_probe_mfma_i8(int64_t workgroups, int64_t iters, int* sink, tango_stream_t stream) {
+    if (workgroups <= 0 || workgroups > INT32_MAX || iters < 0 || iters > INT32_MAX || !sink) return TANGO_ERR_INVALID_ARG;
+    hipLaunchKernelGGL(mfma_i8_probe_kernel, dim3(static_cast<unsigned>(workgroups)), dim3(256), 0, as_stream(stream),
+                       static_cast<int>(iters), sink);
+    return launch_status();
 }
 
 int tango_qgemm_fwd(float* Y, int64_t ldy, const float* X, int64_t ldx, int8_t* Xq, int64_t ldxq,

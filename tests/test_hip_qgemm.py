@@ -179,3 +179,13 @@ def test_qgemm_i8_small_operand_stationary(K, orc, M, N, Kd):
     acc = (A.astype(np.float64) @ B.astype(np.float64).T)  # exact: |sums| < 2^53
     want = bias[None, :] + np.float32(0.125) * acc.astype(np.float32)
     assert np.array_equal(host(Y), want) and host(sY)[0] == orc.absmax_scale(want)
+
+
+def test_mfma_rate_probe_runs():
+    """The measurement aid launches, finishes and leaves its sink untouched."""
+    from tango_amd import _lib
+    sink = torch.zeros(1, dtype=torch.int32, device="cuda")
+    _lib.check(_lib.lib().tango_probe_mfma_i8(8, 4, sink.data_ptr(), torch.cuda.current_stream().cuda_stream), "probe")
+    torch.cuda.synchronize()
+    assert int(sink[0]) == 0
+    assert _lib.lib().tango_probe_mfma_i8(0, 4, sink.data_ptr(), 0) != 0
