@@ -88,7 +88,9 @@ int tango_quantize_rows_f32_i8(const float* x, int64_t rows, int64_t cols, int64
    tensor of its sign) is mask[r, c] (row stride ldm; when non-null), then is multiplied
    by row_mul[r] (when non-null; one fp32 rounding).  mask_mode 0 (ReLU): x becomes zero
    where mask is not positive.  mask_mode 1 (ELU, mask = the activation's output):
-   x becomes x * (mask + 1) where mask is not positive.
+   x becomes x * (mask + 1) where mask is not positive.  mask_mode 2: mask points to 16-bit words,
+   ldm words per row, bit c % 16 of word [r, c / 16] set where x is kept, clear where it becomes zero
+   (cols % 16 == 0; written by tango_spmm_csr_copy_u_ex's sign_bits).
    tango_absmax_ex_f32 writes scale_out[0] = max|x'*row_mul| / 127 of the elements x' so
    masked and, when colsum_out is non-null, colsum_out[c] = sum_r x'[r, c]
    (not multiplied), reduced in a fixed order.  cols <= 1024.
@@ -97,10 +99,10 @@ int tango_quantize_rows_f32_i8(const float* x, int64_t rows, int64_t cols, int64
    workspace: tango_absmax_ex_workspace(rows, cols, colsum_out != NULL) bytes. */
 size_t tango_absmax_ex_workspace(int64_t rows, int64_t cols, int want_colsum);
 int tango_absmax_ex_f32(const float* x, int64_t rows, int64_t cols, int64_t ldx, const float* row_mul,
-                        const float* mask, int64_t ldm, int mask_mode, float* scale_out, int accumulate,
+                        const void* mask, int64_t ldm, int mask_mode, float* scale_out, int accumulate,
                         float* colsum_out, void* workspace, size_t workspace_bytes, tango_stream_t stream);
 int tango_quantize_rows_ex_f32_i8(const float* x, int64_t rows, int64_t cols, int64_t ldx,
-                                  const float* row_mul, const float* mask, int64_t ldm, int mask_mode,
+                                  const float* row_mul, const void* mask, int64_t ldm, int mask_mode,
                                   const float* scale, int per_row, int8_t* q, int64_t ldq,
                                   int round_mode, const float* noise, uint64_t seed,
                                   uint64_t offset, tango_stream_t stream);
@@ -224,12 +226,15 @@ int tango_spmm_csr_copy_u(float* out, const int64_t* indptr, const int64_t* indi
    graphs hub rows (thousands of slots and far above the average) are cut over many
    workgroups whose int32 partial sums are added into the output row with integer
    atomics.  Integer sums are exact in any order, so the result is the same either way.
-   W in the size query: bytes summed per gathered row (F here, H * F for u_mul_e). */
+   W in the size query: bytes summed per gathered row (F here, H * F for u_mul_e).
+   sign_bits (or NULL; needs F % 16 == 0 and 16-byte aligned feat rows): [rows, F / 16] 16-bit words that
+   receive bit c % 16 of word [r, c / 16] = (out[r, c] > 0), the mask the backward pass of the ReLU needs,
+   in 1/32 of the bytes of out (mask_mode 2 of tango_absmax_ex_f32 / tango_quantize_rows_ex_f32_i8). */
 size_t tango_spmm_workspace(int64_t rows, int64_t nnz, int64_t W);
 int tango_spmm_csr_copy_u_ex(float* out, const int64_t* indptr, const void* indices, int idx_bits,
                              const int8_t* feat, int64_t ldf, const float* scale,
-                             const float* row_scale, const float* bias, int relu, int64_t rows,
-                             int64_t num_src, int64_t nnz, int64_t F, int64_t max_row_nnz,
+                             const float* row_scale, const float* bias, int relu, uint16_t* sign_bits,
+                             int64_t rows, int64_t num_src, int64_t nnz, int64_t F, int64_t max_row_nnz,
                              void* workspace, size_t workspace_bytes, tango_stream_t stream);
 
 /* multi_cusparse_SPMM (cuda/src/cuda.cpp:119-158 -> SPMM.cu:70-194):

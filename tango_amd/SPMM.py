@@ -1,4 +1,5 @@
 """Quantized aggregation ops: mirrors cuda/SPMM.py of the reference."""
+import torch
 from torch.autograd.function import Function, once_differentiable
 
 from . import config
@@ -43,8 +44,13 @@ class spmm_copy_u(Function):
             N_, scaleN = quantize_padded(N, scaleN, align=_gather_align(N.size(1)))
         else:
             N_, scaleN = quantize(N, scaleN)
-        out = csr_SPMM(g, N_, scaleN, row_scale=row_scale, bias=bias, relu=relu)
-        ctx.backward_cache = g, row_scale, bias is not None, (out if relu else None)
+        # the backward pass needs only the sign of the ReLU's output: sixteen columns per 16-bit word, written
+        # by the epilogue, instead of two more reads of the fp32 output
+        bits = None
+        if relu and N.dim() == 2 and N.size(1) % 16 == 0:
+            bits = torch.empty((g.num_nodes(), N.size(1) // 16), dtype=torch.int16, device=N.device)
+        out = csr_SPMM(g, N_, scaleN, row_scale=row_scale, bias=bias, relu=relu, sign_bits=bits)
+        ctx.backward_cache = g, row_scale, bias is not None, ((bits if bits is not None else out) if relu else None)
         return out
 
     @staticmethod
@@ -60,12 +66,13 @@ class spmm_copy_u(Function):
         dOut = dOut if dOut.is_contiguous() else dOut.contiguous()
         want_bias = has_bias and ctx.needs_input_grad[4]
         # dZ = (dOut where out > 0) * row_scale; its scale and the bias gradient come from one pass
-        scaledZ, dbias = cuda_kernels.absmax_ex(dOut, row_mul=row_scale, mask=mask, want_colsum=want_bias)
+        mode = "bits" if mask is not None and mask.dtype == torch.int16 else "relu"
+        scaledZ, dbias = cuda_kernels.absmax_ex(dOut, row_mul=row_scale, mask=mask, want_colsum=want_bias, mask_mode=mode)
         if ctx.needs_input_grad[1]:
             kw = {"round_mode": config.grad_round_mode}
             if config.grad_round_mode == "stochastic":
                 kw.update(seed=config.seed, offset=config.next_offset())
-            dZ_, _ = quantize_padded(dOut, scaledZ, row_mul=row_scale, mask=mask,
+            dZ_, _ = quantize_padded(dOut, scaledZ, row_mul=row_scale, mask=mask, mask_mode=mode,
                                      align=_gather_align(dOut.size(1)), **kw)
             dN = csr_SPMM(g, dZ_, scaledZ, True)
         return None, dN, None, None, dbias, None

@@ -1111,7 +1111,7 @@ extern "C" int tango_quantize_rows_f32_i8(const float*, int64_t, int64_t, int64_
                                           int8_t*, int64_t, int, const float*, uint64_t, uint64_t,
                                           tango_stream_t);
 extern "C" int tango_quantize_rows_ex_f32_i8(const float*, int64_t, int64_t, int64_t, const float*,
-                                             const float*, int64_t, int, const float*, int, int8_t*, int64_t,
+                                             const void*, int64_t, int, const float*, int, int8_t*, int64_t,
                                              int, const float*, uint64_t, uint64_t, tango_stream_t);
 extern "C" int tango_absmax_f32(const float*, int64_t, float*, tango_stream_t);
 extern "C" int tango_quantize_f32_i8(const float*, int64_t, const float*, int8_t*, int, const float*, uint64_t,

@@ -221,6 +221,15 @@ __device__ __forceinline__ float masked(float x, float mk, int mode) {
     return mode == 1 ? x * (mk + 1.0f) : 0.0f;
 }
 
+// Mode 2: the mask is one sign bit per element, bit c % 16 of the 16-bit word c / 16 of the row (what the
+// aggregation's ReLU epilogue can write beside its output: 1/32 of the bytes of the fp32 output the other
+// modes read).  mk[k] = 1 where the bit of column c0 + k is set, else 0; c0 is a multiple of four.
+__device__ __forceinline__ void mask_bits4(float* mk, const uint16_t* __restrict__ words, int64_t c0) {
+    const unsigned w = static_cast<unsigned>(words[c0 >> 4]) >> (c0 & 15);
+#pragma unroll
+    for (int k = 0; k < 4; ++k) mk[k] = ((w >> k) & 1u) ? 1.0f : 0.0f;
+}
+
 // quantize_rows_kernel's job on dense matrices whose rows hold a multiple of four columns (x, q and the
 // mask all [rows, cols] without padding): the flat walk of quantize_vec_kernel, a lane's four elements
 // never straddle a row, and the row index (for row_mul) advances by a fixed step per iteration.
@@ -241,7 +250,12 @@ __global__ __launch_bounds__(256) void quantize_dense_ex_kernel(
     for (int64_t i = tid; i < n4; i += nthr) {
         const f32x4 v = __builtin_nontemporal_load(x4 + i);
         float f[4] = {v.x, v.y, v.z, v.w};
-        if (mask) {
+        if (mask && mask_mode == 2) {  // dense rows of a multiple of 16 columns: element e lies in word e / 16
+            float mk[4];
+            mask_bits4(mk, reinterpret_cast<const uint16_t*>(mask), 4 * i);
+#pragma unroll
+            for (int k = 0; k < 4; ++k) f[k] = masked(f[k], mk[k], mask_mode);
+        } else if (mask) {
             const f32x4 mk = __builtin_nontemporal_load(m4 + i);
             f[0] = masked(f[0], mk.x, mask_mode); f[1] = masked(f[1], mk.y, mask_mode);
             f[2] = masked(f[2], mk.z, mask_mode); f[3] = masked(f[3], mk.w, mask_mode);
@@ -343,7 +357,9 @@ __global__ __launch_bounds__(256) void quantize_rows_kernel(
             load4<XV>(f, xr, c0, cols);
             if (mask) {  // the activation's backward first (as the absmax pass does), then the row multiplier
                 float mk[4];
-                if (mask_vec) load4<XV>(mk, mask + row * ldm, c0, cols); else load4<1>(mk, mask + row * ldm, c0, cols);
+                if (mask_mode == 2) mask_bits4(mk, reinterpret_cast<const uint16_t*>(mask) + row * ldm, c0);
+                else if (mask_vec) load4<XV>(mk, mask + row * ldm, c0, cols);
+                else load4<1>(mk, mask + row * ldm, c0, cols);
 #pragma unroll
                 for (int k = 0; k < 4; ++k) f[k] = masked(f[k], mk[k], mask_mode);
             }
@@ -475,7 +491,8 @@ __global__ __launch_bounds__(256) void absmax_ex_kernel(
                 if (row < rows && c0 < cols) {
                     load4<XV>(v[u][t], x + row * ldx, c0, cols);
                     if (mask) {
-                        if (mask_vec) load4<XV>(mk[u][t], mask + row * ldm, c0, cols);
+                        if (mask_mode == 2) mask_bits4(mk[u][t], reinterpret_cast<const uint16_t*>(mask) + row * ldm, c0);
+                        else if (mask_vec) load4<XV>(mk[u][t], mask + row * ldm, c0, cols);
                         else load4<1>(mk[u][t], mask + row * ldm, c0, cols);
                     }
                 }
@@ -637,11 +654,14 @@ size_t tango_absmax_ex_workspace(int64_t rows, int64_t cols, int want_colsum) {
 }
 
 int tango_absmax_ex_f32(const float* x, int64_t rows, int64_t cols, int64_t ldx, const float* row_mul,
-                        const float* mask, int64_t ldm, int mask_mode, float* scale_out, int accumulate,
+                        const void* mask_, int64_t ldm, int mask_mode, float* scale_out, int accumulate,
                         float* colsum_out, void* workspace, size_t workspace_bytes, tango_stream_t stream) {
-    if (rows < 0 || cols < 0 || ldx < cols || !scale_out || (rows * cols > 0 && !x) || (mask && ldm < cols))
+    const float* mask = static_cast<const float*>(mask_);  // 16-bit words in mode 2
+    if (rows < 0 || cols < 0 || ldx < cols || !scale_out || (rows * cols > 0 && !x) ||
+        (mask && ldm < (mask_mode == 2 ? cols / 16 : cols)))
         return TANGO_ERR_INVALID_ARG;
-    if (cols > 1024 || mask_mode < 0 || mask_mode > 1) return TANGO_ERR_UNSUPPORTED;
+    if (cols > 1024 || mask_mode < 0 || mask_mode > 2 || (mask && mask_mode == 2 && (cols & 15) != 0))
+        return TANGO_ERR_UNSUPPORTED;
     hipStream_t s = as_stream(stream);
     if (!accumulate) fill_u32(scale_out, 0u, 1, s);
     const int grid = absmax_ex_grid(rows);
@@ -712,20 +732,21 @@ int tango_quantize_rows_f32_i8(const float* x, int64_t rows, int64_t cols, int64
 }
 
 int tango_quantize_rows_ex_f32_i8(const float* x, int64_t rows, int64_t cols, int64_t ldx,
-                                  const float* row_mul, const float* mask, int64_t ldm, int mask_mode,
+                                  const float* row_mul, const void* mask_, int64_t ldm, int mask_mode,
                                   const float* scale, int per_row, int8_t* q, int64_t ldq,
                                   int round_mode, const float* noise, uint64_t seed,
                                   uint64_t offset, tango_stream_t stream) {
-    if (mask && ldm < cols) return TANGO_ERR_INVALID_ARG;
-    if (mask_mode < 0 || mask_mode > 1) return TANGO_ERR_UNSUPPORTED;
+    const float* mask = static_cast<const float*>(mask_);  // 16-bit words in mode 2
+    if (mask && ldm < (mask_mode == 2 ? cols / 16 : cols)) return TANGO_ERR_INVALID_ARG;
+    if (mask_mode < 0 || mask_mode > 2 || (mask && mask_mode == 2 && (cols & 15) != 0)) return TANGO_ERR_UNSUPPORTED;
     if (rows < 0 || cols < 0 || ldx < cols || ldq < cols || !scale ||
         (rows * cols > 0 && (!x || !q)))
         return TANGO_ERR_INVALID_ARG;
     if (rows == 0 || ldq == 0) return (round_mode >= 0 && round_mode <= 2) ? TANGO_OK : TANGO_ERR_UNSUPPORTED;
     hipStream_t s = as_stream(stream);
     if ((row_mul || mask) && !per_row && cols > 0 && (cols & 3) == 0 && ldx == cols && ldq == cols &&
-        (!mask || ldm == cols) && (reinterpret_cast<uintptr_t>(x) & 15) == 0 &&
-        (reinterpret_cast<uintptr_t>(mask) & 15) == 0 && (reinterpret_cast<uintptr_t>(q) & 3) == 0) {
+        (!mask || ldm == (mask_mode == 2 ? cols / 16 : cols)) && (reinterpret_cast<uintptr_t>(x) & 15) == 0 &&
+        (reinterpret_cast<uintptr_t>(mask) & (mask_mode == 2 ? 1 : 15)) == 0 && (reinterpret_cast<uintptr_t>(q) & 3) == 0) {
         const int64_t n4 = rows * (cols >> 2);
         int rc = dispatch_mode(round_mode, [&](auto mode) {
             constexpr int M = decltype(mode)::value;

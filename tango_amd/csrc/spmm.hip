@@ -41,6 +41,7 @@ struct SpmmParams {
     const float* row_scale;  // optional: out row r is multiplied by row_scale[r] after dequantization
     const float* bias;       // optional: bias[c] added after the row scale
     int relu;                // activation applied last: 0 none, 1 max(y, 0), 2 ELU (y > 0 ? y : exp(y) - 1)
+    uint16_t* sign_bits;     // optional, VEC == 16 and W % 16 == 0: bit c % 16 of word [r, c / 16] = (out[r, c] > 0)
     int64_t rows;
     int64_t num_src;  // rows of the gathered matrix
     int64_t ldf;  // bytes between gathered rows
@@ -255,6 +256,16 @@ __device__ __forceinline__ float activate(float y, int act) {
     return y;
 }
 
+// The signs of a lane's sixteen consecutive outputs as one 16-bit word (what a backward pass needs of a ReLU's
+// output: 1/32 of its bytes).
+template <int VEC>
+__device__ __forceinline__ void store_sign_bits(const SpmmParams& p, int64_t row, int64_t col, const float* y) {
+    unsigned b = 0;
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) b |= (y[i] > 0.0f ? 1u : 0u) << (i & 15);
+    p.sign_bits[row * (p.W >> 4) + (col >> 4)] = static_cast<uint16_t>(b);
+}
+
 // Dequantize and store one output row's tile; called by the lanes with grp == 0.
 template <int VEC>
 __device__ __forceinline__ void store_row(const SpmmParams& p, const LaneCols& c, int64_t row, const int* acc) {
@@ -274,6 +285,7 @@ __device__ __forceinline__ void store_row(const SpmmParams& p, const LaneCols& c
 #pragma unroll
         for (int i = 0; i < VEC; ++i) y[i] = activate(y[i], p.relu);
     }
+    if (VEC == 16 && p.sign_bits) store_sign_bits<VEC>(p, row, c.col, y);
     if (VEC == 16 && p.out_vec && c.col + 16 <= p.W) {
         f32x4* o4 = reinterpret_cast<f32x4*>(o);
 #pragma unroll
@@ -828,6 +840,7 @@ __global__ __launch_bounds__(256) void spmm_span_kernel(const SpmmParams p) {
 #pragma unroll
             for (int i = 0; i < VEC; ++i) y[i] = activate(y[i], p.relu);
         }
+        if (VEC == 16 && p.sign_bits) store_sign_bits<VEC>(p, row, c.col, y);
         if (VEC == 16 && p.out_vec && c.col + 16 <= p.W) {
             f32x4* o4 = reinterpret_cast<f32x4*>(o);
 #pragma unroll
@@ -1161,8 +1174,8 @@ int tango_spmm_csr_copy_u(float* out, const int64_t* indptr, const int64_t* indi
 
 int tango_spmm_csr_copy_u_ex(float* out, const int64_t* indptr, const void* indices, int idx_bits,
                              const int8_t* feat, int64_t ldf, const float* scale,
-                             const float* row_scale, const float* bias, int relu, int64_t rows,
-                             int64_t num_src, int64_t nnz, int64_t F, int64_t max_row_nnz,
+                             const float* row_scale, const float* bias, int relu, uint16_t* sign_bits,
+                             int64_t rows, int64_t num_src, int64_t nnz, int64_t F, int64_t max_row_nnz,
                              void* workspace, size_t workspace_bytes, tango_stream_t stream) {
     if (rows < 0 || F < 0 || nnz < 0 || num_src < 0 || ldf < F || !scale || !indptr || max_row_nnz < 0 ||
         (rows * F > 0 && !out) || (nnz > 0 && (!indices || !feat)) || (idx_bits != 32 && idx_bits != 64))
@@ -1173,7 +1186,9 @@ int tango_spmm_csr_copy_u_ex(float* out, const int64_t* indptr, const void* indi
     SpmmParams p{};
     p.out = out; p.indptr = indptr; p.indices = static_cast<const int64_t*>(indices); p.idx32 = idx_bits == 32;
     p.feat = feat; p.scale = scale;
-    p.row_scale = row_scale; p.bias = bias; p.relu = relu; p.max_row = max_row_nnz; p.hub_ws = workspace;
+    const int vec = pick_vec(feat, ldf, F);
+    if (sign_bits && (vec != 16 || (F & 15) != 0)) return TANGO_ERR_UNSUPPORTED;
+    p.row_scale = row_scale; p.bias = bias; p.relu = relu; p.sign_bits = sign_bits; p.max_row = max_row_nnz; p.hub_ws = workspace;
     p.span_ws = workspace; p.span_ws_bytes = workspace_bytes;
     p.rows = rows; p.num_src = num_src; p.ldf = ldf; p.W = F; p.F = F; p.D = 1; p.nnz = nnz;
     return launch_spmm<KIND_COPY>(p, pick_vec(feat, ldf, F), as_stream(stream));

@@ -8,6 +8,12 @@ from .QLinear import Qlinear_func, Qlinear_func_reduce
 from .SPMM import spmm_copy_u
 
 
+def degree_norms(graph):
+    """(out_deg^-1/2, in_deg^-1/2) with degrees clamped to >= 1 (evaluation/test_gcn.py:86-94,123-131)."""
+    return (graph.out_degrees().float().clamp(min=1).pow(-0.5),
+            graph.in_degrees().float().clamp(min=1).pow(-0.5))
+
+
 class QGraphConv(nn.Module):
     """GraphConv(norm='both') with int8 GEMM and int8 aggregation
     (evaluation/test_gcn.py:26-139)."""
@@ -23,9 +29,10 @@ class QGraphConv(nn.Module):
         if self.bias is not None:
             nn.init.zeros_(self.bias)
 
-    def forward(self, graph, feat):
-        norm_src = graph.out_degrees().float().clamp(min=1).pow(-0.5)
-        norm_dst = graph.in_degrees().float().clamp(min=1).pow(-0.5)
+    def forward(self, graph, feat, norms=None):
+        """``norms``: (out_deg^-1/2, in_deg^-1/2) from ``degree_norms`` when the caller computes them once
+        for several layers of one forward pass; the reference's layer computes them itself every time."""
+        norm_src, norm_dst = degree_norms(graph) if norms is None else norms
         relu = self._activation is torch.relu
         if self.fused:
             # same arithmetic as below, with every elementwise pass folded into a kernel:
@@ -71,8 +78,9 @@ class GCN(nn.Module):
 
     def forward(self, features):
         h = features
+        norms = degree_norms(self.g)  # once per forward pass, shared by the layers
         for i, layer in enumerate(self.layers):
             if i != 0:
                 h = self.dropout(h)
-            h = layer(self.g, h)
+            h = layer(self.g, h, norms)
         return h

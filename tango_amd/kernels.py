@@ -118,7 +118,7 @@ def _zero_slot(device):
     return pool[0][k:k + 1]
 
 
-_MASK_MODES = {"relu": 0, "elu": 1}
+_MASK_MODES = {"relu": 0, "elu": 1, "bits": 2}
 _ACTIVATIONS = {None: 0, "relu": 1, "elu": 2}
 
 
@@ -194,11 +194,26 @@ class cuda_kernels:
                                        _stream()), "quantize")
 
     @staticmethod
+    def _mask_ld(mask, mask_mode, inp, what):
+        """Row stride of ``mask`` in its own units: floats of inp's shape, or for "bits" the int16 words
+        [rows, cols / 16] that csr_SPMM's ``sign_bits`` writes."""
+        if mask_mode == "bits":
+            _need(mask, torch.int16, "mask")
+            if inp.size(1) % 16 or tuple(mask.shape) != (inp.size(0), inp.size(1) // 16):
+                raise RuntimeError(what + ": a bit mask must be int16 [rows, cols / 16], cols a multiple of 16")
+            return mask.size(1)
+        _need(mask, torch.float32, "mask", contiguous=False)
+        if tuple(mask.shape) != tuple(inp.shape):
+            raise RuntimeError(what + ": mask must have in's shape")
+        return _rows_view(mask, "mask")
+
+    @staticmethod
     def quantize_rows(out, inp, scale, per_row=False, round_mode=ROUND_RNE, noise=None, seed=0,
                       offset=0, row_mul=None, mask=None, mask_mode="relu"):
         """Row-strided quantize into a possibly wider (zero-padded) int8 matrix (not in the reference).
         ``mask`` (an activation's output) takes each element backwards through that activation first:
-        ``mask_mode`` "relu" zeroes it where mask <= 0, "elu" multiplies it by mask + 1 there.
+        ``mask_mode`` "relu" zeroes it where mask <= 0, "elu" multiplies it by mask + 1 there, "bits":
+        the mask is the int16 [rows, cols / 16] sign words of csr_SPMM (bit clear = zero the element).
         ``row_mul`` [rows] then multiplies each row."""
         _need(out, torch.int8, "out", contiguous=False)
         _need(inp, torch.float32, "in", contiguous=False)
@@ -217,10 +232,7 @@ class cuda_kernels:
             if row_mul.numel() != inp.size(0):
                 raise RuntimeError("quantize_rows: row_mul must have one entry per row")
         if mask is not None:
-            _need(mask, torch.float32, "mask", contiguous=False)
-            if tuple(mask.shape) != tuple(inp.shape):
-                raise RuntimeError("quantize_rows: mask must have in's shape")
-            ldm = _rows_view(mask, "mask")
+            ldm = cuda_kernels._mask_ld(mask, mask_mode, inp, "quantize_rows")
         check(_L.tango_quantize_rows_ex_f32_i8(_ptr(inp), inp.size(0), inp.size(1), ldx, _ptr(row_mul),
                                                _ptr(mask), ldm, _MASK_MODES[mask_mode], scale.data_ptr(),
                                                int(bool(per_row)),
@@ -239,15 +251,16 @@ class cuda_kernels:
         if row_mul is not None:
             _need(row_mul, torch.float32, "row_mul")
         if mask is not None:
-            _need(mask, torch.float32, "mask", contiguous=False)
-            ldm = _rows_view(mask, "mask")
+            ldm = cuda_kernels._mask_ld(mask, mask_mode, inp, "absmax_ex")
         if cols > 1024:
             # the kernel keeps a row's column sums in registers, 1024 columns at most: walk column slices
             scale, sums = None, []
             for c0 in range(0, cols, 1024):
                 sl = slice(c0, min(cols, c0 + 1024))
                 s_i, cs_i = cuda_kernels.absmax_ex(inp[:, sl], row_mul=row_mul,
-                                                   mask=None if mask is None else mask[:, sl],
+                                                   mask=None if mask is None else
+                                                   (mask[:, c0 // 16:(min(cols, c0 + 1024) + 15) // 16].contiguous()
+                                                    if mask_mode == "bits" else mask[:, sl]),
                                                    want_colsum=want_colsum, mask_mode=mask_mode)
                 scale = s_i if scale is None else torch.maximum(scale, s_i)
                 sums.append(cs_i)
@@ -397,7 +410,9 @@ class cuda_kernels:
     # ------------------------------------------------------------------ SpMM
     @staticmethod
     def csr_SPMM(out, indptr, indices, U, scaleU, ldf=None, F=None, row_scale=None, bias=None, relu=False,
-                 max_row=0):
+                 max_row=0, sign_bits=None):
+        """``sign_bits`` (int16 [rows, F / 16], F a multiple of 16): receives one bit per output element,
+        set where it is positive: all a backward pass needs of a ReLU's output."""
         _need(out, torch.float32, "out")
         _need(indptr, torch.int64, "indptr")
         idx_bits = _need_index(indices, "indices")
@@ -409,7 +424,11 @@ class cuda_kernels:
         F = width if F is None else F
         if out.numel() != rows * F:
             raise RuntimeError("csr_SPMM: out must be [%d, %d]" % (rows, F))
-        if row_scale is None and bias is None and not relu and idx_bits == 64 and not max_row:
+        if sign_bits is not None:
+            _need(sign_bits, torch.int16, "sign_bits")
+            if F % 16 or tuple(sign_bits.shape) != (rows, F // 16):
+                raise RuntimeError("csr_SPMM: sign_bits must be int16 [rows, F / 16], F a multiple of 16")
+        if row_scale is None and bias is None and not relu and idx_bits == 64 and not max_row and sign_bits is None:
             check(_L.tango_spmm_csr_copy_u(_ptr(out), indptr.data_ptr(), _ptr(indices), _ptr(U), ldf,
                                            scaleU.data_ptr(), rows, U.size(0), indices.numel(), F,
                                            _stream()), "csr_SPMM")
@@ -426,7 +445,7 @@ class cuda_kernels:
         ws = _workspace(ws_bytes, U.device)
         check(_L.tango_spmm_csr_copy_u_ex(_ptr(out), indptr.data_ptr(), _ptr(indices), idx_bits, _ptr(U), ldf,
                                           scaleU.data_ptr(), _ptr(row_scale), _ptr(bias), int(bool(relu)),
-                                          rows, U.size(0), indices.numel(), F, int(max_row), _ptr(ws), ws_bytes,
+                                          _ptr(sign_bits), rows, U.size(0), indices.numel(), F, int(max_row), _ptr(ws), ws_bytes,
                                           _stream()), "csr_SPMM")
 
     @staticmethod
@@ -743,9 +762,10 @@ def incidence_SPMM(g, E, scaleE, reverse=False):
     return out.view(out_shape)
 
 
-def csr_SPMM(g, N, scaleN, reverse=False, row_scale=None, bias=None, relu=False):
+def csr_SPMM(g, N, scaleN, reverse=False, row_scale=None, bias=None, relu=False, sign_bits=None):
     """cuda/kernels.py:154-165.  N may be a 2-D view of a row-padded buffer.  ``row_scale`` / ``bias`` /
-    ``relu`` fold "* norm, + bias, activation" (evaluation/test_gcn.py:123-137) into the kernel's epilogue."""
+    ``relu`` fold "* norm, + bias, activation" (evaluation/test_gcn.py:123-137) into the kernel's epilogue;
+    ``sign_bits`` (int16 [n, F / 16]) receives the signs of the output."""
     indptr, indices, _, longest = _csr_of(g, reverse)
     feat_shape = N.shape[1:]
     out_shape = (g.num_nodes(),) + feat_shape
@@ -755,10 +775,10 @@ def csr_SPMM(g, N, scaleN, reverse=False, row_scale=None, bias=None, relu=False)
         ld = _rows_view(N, "N")
         base = N.as_strided((N.size(0), ld), (ld, 1))
         cuda_kernels.csr_SPMM(out, indptr, indices, base, scaleN, ldf=ld, F=dim, row_scale=row_scale, bias=bias,
-                              relu=relu, max_row=longest)
+                              relu=relu, max_row=longest, sign_bits=sign_bits)
     else:
         cuda_kernels.csr_SPMM(out, indptr, indices, N, scaleN, row_scale=row_scale, bias=bias, relu=relu,
-                              max_row=longest)
+                              max_row=longest, sign_bits=sign_bits)
     return out.view(out_shape)
 
 

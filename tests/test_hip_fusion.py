@@ -24,7 +24,7 @@ def make_graph(src, dst, n):
 
 def test_absmax_ex_and_quantize_ex(K, orc):
     rng = np.random.default_rng(0)
-    for rows, cols in ((1000, 256), (777, 41), (300, 602), (5, 1024), (64, 1500), (3, 7)):
+    for rows, cols in ((1000, 256), (777, 41), (300, 602), (5, 1024), (64, 1500), (3, 7), (200, 48)):
         x = rng.standard_normal((rows, cols)).astype(np.float32)
         rm = rng.random(rows, dtype=np.float32) + 0.1
         mask = rng.standard_normal((rows, cols)).astype(np.float32)
@@ -50,6 +50,20 @@ def test_absmax_ex_and_quantize_ex(K, orc):
         assert np.allclose(host(cs), through.astype(np.float64).sum(0), rtol=1e-5, atol=1e-3)
         q, _ = K.quantize_padded(dev(x), s, row_mul=dev(rm), mask=dev(emask), mask_mode="elu")
         assert np.array_equal(host(q), orc.quantize(scaled, host(s)[0]))
+        if cols % 16 == 0:
+            # the same ReLU mask as sign bits, sixteen columns per 16-bit word
+            bits = np.packbits((mask > 0).reshape(rows, cols // 16, 16), axis=-1, bitorder="little").view(np.int16)
+            bits = dev(np.ascontiguousarray(bits.reshape(rows, cols // 16)))
+            sb, csb = K.cuda_kernels.absmax_ex(dev(x), row_mul=dev(rm), mask=bits, want_colsum=True, mask_mode="bits")
+            s0, cs0 = K.cuda_kernels.absmax_ex(dev(x), row_mul=dev(rm), mask=dev(mask), want_colsum=True)
+            assert torch.equal(sb, s0) and torch.equal(csb, cs0)
+            for kw in ({}, {"round_mode": "stochastic", "seed": 3, "offset": 64}):
+                qb, _ = K.quantize_padded(dev(x), s0, row_mul=dev(rm), mask=bits, mask_mode="bits", **kw)
+                q0, _ = K.quantize_padded(dev(x), s0, row_mul=dev(rm), mask=dev(mask), **kw)
+                assert torch.equal(qb, q0)
+                qb, _ = K.quantize_padded(dev(x), s0, mask=bits, mask_mode="bits", align=64, **kw)  # row-strided kernel
+                q0, _ = K.quantize_padded(dev(x), s0, mask=dev(mask), align=64, **kw)
+                assert torch.equal(qb, q0)
     # colsum is deterministic run to run
     x = dev(rng.standard_normal((50000, 256)).astype(np.float32))
     a = K.cuda_kernels.absmax_ex(x, want_colsum=True)[1]
@@ -87,8 +101,13 @@ def test_spmm_fused_epilogue_equals_separate_passes(K, F, n, e):
     assert torch.equal(K.csr_SPMM(g, feat, s, row_scale=rs), base * rs.unsqueeze(1))
     assert torch.equal(K.csr_SPMM(g, feat, s, bias=bias), base + bias)
     assert torch.equal(K.csr_SPMM(g, feat, s, relu=True), torch.relu(base))
-    assert torch.equal(K.csr_SPMM(g, feat, s, row_scale=rs, bias=bias, relu=True),
-                       torch.relu(base * rs.unsqueeze(1) + bias))
+    want = torch.relu(base * rs.unsqueeze(1) + bias)
+    assert torch.equal(K.csr_SPMM(g, feat, s, row_scale=rs, bias=bias, relu=True), want)
+    if F % 16 == 0:  # the epilogue also writes the signs of its output, sixteen columns per word
+        bits = torch.full((n, F // 16), -1, dtype=torch.int16, device="cuda")
+        assert torch.equal(K.csr_SPMM(g, feat, s, row_scale=rs, bias=bias, relu=True, sign_bits=bits), want)
+        got = np.unpackbits(host(bits).view(np.uint8).reshape(n, F // 16, 2), axis=-1, bitorder="little").reshape(n, F)
+        assert np.array_equal(got.astype(bool), host(want) > 0)
 
 
 def test_gemm_row_scale_prologue_and_gradx_epilogue(K, orc):
