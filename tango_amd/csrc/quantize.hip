@@ -477,6 +477,7 @@ __global__ __launch_bounds__(256) void absmax_ex_kernel(
     for (int64_t row0 = (static_cast<int64_t>(blockIdx.x) * blockDim.y + threadIdx.y) * rpw + sub; row0 < rows;
          row0 += RU * row_step) {
         float v[RU][T][4], mk[RU][T][4];
+        unsigned wb[RU][T];  // mode 2: the four sign bits of the lane's columns (bit set = keep)
 #pragma unroll
         for (int u = 0; u < RU; ++u) {
             const int64_t row = row0 + u * row_step;
@@ -488,10 +489,12 @@ __global__ __launch_bounds__(256) void absmax_ex_kernel(
                     v[u][t][k] = 0.0f;
                     mk[u][t][k] = 1.0f;
                 }
+                wb[u][t] = 0xFu;
                 if (row < rows && c0 < cols) {
                     load4<XV>(v[u][t], x + row * ldx, c0, cols);
                     if (mask) {
-                        if (mask_mode == 2) mask_bits4(mk[u][t], reinterpret_cast<const uint16_t*>(mask) + row * ldm, c0);
+                        if (mask_mode == 2)
+                            wb[u][t] = static_cast<unsigned>((reinterpret_cast<const uint16_t*>(mask) + row * ldm)[c0 >> 4]) >> (c0 & 15);
                         else if (mask_vec) load4<XV>(mk[u][t], mask + row * ldm, c0, cols);
                         else load4<1>(mk[u][t], mask + row * ldm, c0, cols);
                     }
@@ -506,7 +509,7 @@ __global__ __launch_bounds__(256) void absmax_ex_kernel(
             for (int t = 0; t < T; ++t)
 #pragma unroll
                 for (int k = 0; k < 4; ++k) {
-                    const float e = masked(v[u][t][k], mk[u][t][k], mask_mode);
+                    const float e = ((wb[u][t] >> k) & 1u) ? masked(v[u][t][k], mk[u][t][k], mask_mode) : 0.0f;
                     cs[t][k] += e;
                     m = fmaxf(m, fabsf(row_mul ? e * rm : e));
                 }
