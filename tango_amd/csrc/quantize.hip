@@ -452,7 +452,7 @@ __global__ __launch_bounds__(256) void transpose_quant_kernel(const float* __res
 // scale rows, quantize" backward step in one read of x.  blockDim = (64, 4), a wavefront walks
 // rows; lane l owns columns 4 l .. 4 l + 3 (+ 256 t).  Column sums are written as one partial
 // row per wavefront and reduced in a fixed order afterwards, so they are deterministic.
-template <int T, int XV>
+template <int T, int XV, int MK /* 0 no mask, 1 fp32 mask, 2 sign-bit words */>
 __global__ __launch_bounds__(256) void absmax_ex_kernel(
     const float* __restrict__ x, int64_t rows, int64_t cols, int64_t ldx,
     const float* __restrict__ row_mul, const float* __restrict__ mask, int64_t ldm,
@@ -476,8 +476,9 @@ __global__ __launch_bounds__(256) void absmax_ex_kernel(
     constexpr int RU = 4;  // rows in flight per lane: the loads of four rows are issued before any is used
     for (int64_t row0 = (static_cast<int64_t>(blockIdx.x) * blockDim.y + threadIdx.y) * rpw + sub; row0 < rows;
          row0 += RU * row_step) {
-        float v[RU][T][4], mk[RU][T][4];
-        unsigned wb[RU][T];  // mode 2: the four sign bits of the lane's columns (bit set = keep)
+        float v[RU][T][4];
+        float mk[MK == 1 ? RU : 1][T][4];  // fp32 mask values
+        unsigned wb[MK == 2 ? RU : 1][T];  // the four sign bits of the lane's columns (bit set = keep)
 #pragma unroll
         for (int u = 0; u < RU; ++u) {
             const int64_t row = row0 + u * row_step;
@@ -487,17 +488,15 @@ __global__ __launch_bounds__(256) void absmax_ex_kernel(
 #pragma unroll
                 for (int k = 0; k < 4; ++k) {
                     v[u][t][k] = 0.0f;
-                    mk[u][t][k] = 1.0f;
+                    if (MK == 1) mk[u][t][k] = 1.0f;
                 }
-                wb[u][t] = 0xFu;
+                if (MK == 2) wb[u][t] = 0xFu;
                 if (row < rows && c0 < cols) {
                     load4<XV>(v[u][t], x + row * ldx, c0, cols);
-                    if (mask) {
-                        if (mask_mode == 2)
-                            wb[u][t] = static_cast<unsigned>((reinterpret_cast<const uint16_t*>(mask) + row * ldm)[c0 >> 4]) >> (c0 & 15);
-                        else if (mask_vec) load4<XV>(mk[u][t], mask + row * ldm, c0, cols);
-                        else load4<1>(mk[u][t], mask + row * ldm, c0, cols);
-                    }
+                    if (MK == 2)
+                        wb[u][t] = static_cast<unsigned>((reinterpret_cast<const uint16_t*>(mask) + row * ldm)[c0 >> 4]) >> (c0 & 15);
+                    else if (MK == 1 && mask_vec) load4<XV>(mk[u][t], mask + row * ldm, c0, cols);
+                    else if (MK == 1) load4<1>(mk[u][t], mask + row * ldm, c0, cols);
                 }
             }
         }
@@ -509,7 +508,9 @@ __global__ __launch_bounds__(256) void absmax_ex_kernel(
             for (int t = 0; t < T; ++t)
 #pragma unroll
                 for (int k = 0; k < 4; ++k) {
-                    const float e = ((wb[u][t] >> k) & 1u) ? masked(v[u][t][k], mk[u][t][k], mask_mode) : 0.0f;
+                    float e = v[u][t][k];
+                    if (MK == 1) e = masked(e, mk[u][t][k], mask_mode);
+                    if (MK == 2) e = ((wb[u][t] >> k) & 1u) ? e : 0.0f;
                     cs[t][k] += e;
                     m = fmaxf(m, fabsf(row_mul ? e * rm : e));
                 }
@@ -690,9 +691,14 @@ int tango_absmax_ex_f32(const float* x, int64_t rows, int64_t cols, int64_t ldx,
     while (gpr_log2 > 0 && (1LL << (gpr_log2 - 1)) >= cgroups) --gpr_log2;
     const uintptr_t xa = reinterpret_cast<uintptr_t>(x);
     const int xv = ((xa & 15) == 0 && (ldx & 3) == 0) ? 4 : ((xa & 7) == 0 && (ldx & 1) == 0) ? 2 : 1;
-#define TANGO_AEX(T_, V_)                                                                              \
-    hipLaunchKernelGGL((absmax_ex_kernel<T_, V_>), dim3(grid), block, 0, s, x, rows, cols, ldx, row_mul, \
+#define TANGO_AEX_M(T_, V_, M_)                                                                             \
+    hipLaunchKernelGGL((absmax_ex_kernel<T_, V_, M_>), dim3(grid), block, 0, s, x, rows, cols, ldx, row_mul, \
                        mask, ldm, scale_out, partial, gpr_log2, mask_mode)
+#define TANGO_AEX(T_, V_)                                                                   \
+    do {                                                                                    \
+        if (!mask) TANGO_AEX_M(T_, V_, 0); else if (mask_mode == 2) TANGO_AEX_M(T_, V_, 2); \
+        else TANGO_AEX_M(T_, V_, 1);                                                        \
+    } while (0)
 #define TANGO_AEX_T(T_)                                                              \
     do {                                                                             \
         if (xv == 4) TANGO_AEX(T_, 4); else if (xv == 2) TANGO_AEX(T_, 2); else TANGO_AEX(T_, 1); \
@@ -700,6 +706,7 @@ int tango_absmax_ex_f32(const float* x, int64_t rows, int64_t cols, int64_t ldx,
     if (T <= 1) TANGO_AEX_T(1); else if (T == 2) TANGO_AEX_T(2); else if (T == 3) TANGO_AEX_T(3); else TANGO_AEX_T(4);
 #undef TANGO_AEX_T
 #undef TANGO_AEX
+#undef TANGO_AEX_M
     if (colsum_out)
         hipLaunchKernelGGL(colsum_finish_kernel, dim3(static_cast<unsigned>(ceil_div(cols, 16))), dim3(16, 16), 0,
                            s, partial, static_cast<int64_t>(grid), cols, colsum_out);

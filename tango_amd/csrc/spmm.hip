@@ -285,7 +285,6 @@ __device__ __forceinline__ void store_row(const SpmmParams& p, const LaneCols& c
 #pragma unroll
         for (int i = 0; i < VEC; ++i) y[i] = activate(y[i], p.relu);
     }
-    if (VEC == 16 && p.sign_bits) store_sign_bits<VEC>(p, row, c.col, y);
     if (VEC == 16 && p.out_vec && c.col + 16 <= p.W) {
         f32x4* o4 = reinterpret_cast<f32x4*>(o);
 #pragma unroll
@@ -296,6 +295,8 @@ __device__ __forceinline__ void store_row(const SpmmParams& p, const LaneCols& c
         for (int i = 0; i < VEC; ++i)
             if (c.col + i < p.W) o[i] = y[i];
     }
+    // after the row's own stores, so that the sixteen values need not all be live at once
+    if (VEC == 16 && p.sign_bits) store_sign_bits<VEC>(p, row, c.col, y);
 }
 
 template <int KIND>
@@ -840,7 +841,6 @@ __global__ __launch_bounds__(256) void spmm_span_kernel(const SpmmParams p) {
 #pragma unroll
             for (int i = 0; i < VEC; ++i) y[i] = activate(y[i], p.relu);
         }
-        if (VEC == 16 && p.sign_bits) store_sign_bits<VEC>(p, row, c.col, y);
         if (VEC == 16 && p.out_vec && c.col + 16 <= p.W) {
             f32x4* o4 = reinterpret_cast<f32x4*>(o);
 #pragma unroll
@@ -850,6 +850,7 @@ __global__ __launch_bounds__(256) void spmm_span_kernel(const SpmmParams p) {
             for (int i = 0; i < VEC; ++i)
                 if (c.col + i < p.W) o[i] = y[i];
         }
+        if (KIND == KIND_COPY && VEC == 16 && p.sign_bits) store_sign_bits<VEC>(p, row, c.col, y);
     };
     // ends the piece the group is in
     auto flush = [&](bool closed) {
