@@ -461,6 +461,7 @@ __global__ __launch_bounds__(256) void absmax_ex_kernel(
     __shared__ float red[3][T * 256];
     const bool mask_vec = mask && ldm == ldx &&
                           ((reinterpret_cast<uintptr_t>(mask) ^ reinterpret_cast<uintptr_t>(x)) & 15) == 0;
+    const bool whole_quads = (cols & 3) == 0 && rows > 0;
     float m = 0.0f;
     float cs[T][4];
 #pragma unroll
@@ -479,6 +480,33 @@ __global__ __launch_bounds__(256) void absmax_ex_kernel(
         float v[RU][T][4];
         float mk[MK == 1 ? RU : 1][T][4];  // fp32 mask values
         unsigned wb[MK == 2 ? RU : 1][T];  // the four sign bits of the lane's columns (bit set = keep)
+        if (XV == 4 && whole_quads && (MK != 1 || mask_vec)) {
+            // No lane has a partial quad: every load is issued unconditionally from a clamped address and the
+            // lanes outside the matrix discard theirs.  Without branches between them the loads of all RU rows
+            // are in flight together (with the guarded form below the compiler waits between rows).
+#pragma unroll
+            for (int u = 0; u < RU; ++u) {
+                const int64_t row = row0 + u * row_step;
+#pragma unroll
+                for (int t = 0; t < T; ++t) {
+                    const int64_t c0 = (static_cast<int64_t>(gl) + 64 * t) << 2;
+                    const bool in = row < rows && c0 < cols;
+                    const int64_t rr = in ? row : 0, cc = in ? c0 : 0;
+                    const f32x4 a = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(x + rr * ldx + cc));
+#pragma unroll
+                    for (int k = 0; k < 4; ++k) v[u][t][k] = in ? a[k] : 0.0f;
+                    if (MK == 1) {
+                        const f32x4 b = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(mask + rr * ldm + cc));
+#pragma unroll
+                        for (int k = 0; k < 4; ++k) mk[u][t][k] = in ? b[k] : 1.0f;
+                    }
+                    if (MK == 2) {
+                        const unsigned w = (reinterpret_cast<const uint16_t*>(mask) + rr * ldm)[cc >> 4];
+                        wb[u][t] = in ? (w >> (cc & 15)) : 0xFu;
+                    }
+                }
+            }
+        } else {
 #pragma unroll
         for (int u = 0; u < RU; ++u) {
             const int64_t row = row0 + u * row_step;
@@ -499,6 +527,7 @@ __global__ __launch_bounds__(256) void absmax_ex_kernel(
                     else if (MK == 1) load4<1>(mk[u][t], mask + row * ldm, c0, cols);
                 }
             }
+        }
         }
 #pragma unroll
         for (int u = 0; u < RU; ++u) {  // rows are added in the order a one-row-at-a-time loop would take them
