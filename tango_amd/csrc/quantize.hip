@@ -491,7 +491,8 @@ __global__ __launch_bounds__(256) void absmax_ex_kernel(
                 for (int t = 0; t < T; ++t) {
                     const int64_t c0 = (static_cast<int64_t>(gl) + 64 * t) << 2;
                     const bool in = row < rows && c0 < cols;
-                    const int64_t rr = in ? row : 0, cc = in ? c0 : 0;
+                    // lanes outside re-read a nearby vector (one fixed address for all of them would be a hot spot)
+                    const int64_t rr = row < rows ? row : rows - 1, cc = c0 < cols ? c0 : cols - 4;
                     const f32x4 a = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(x + rr * ldx + cc));
 #pragma unroll
                     for (int k = 0; k < 4; ++k) v[u][t][k] = in ? a[k] : 0.0f;
