@@ -10,6 +10,7 @@ with events the way evaluation/test_gcn.py:241-263 does (the reference records i
 event before ``loss.backward()``; here it is recorded after).
 
     python -m tango_amd.evaluation --model gcn --dataset pubmed --epochs 20
+    python -m tango_amd.evaluation --model linkpred --dataset pubmed --epochs 20   # evaluation/link_pred_gcn.py
 """
 import argparse
 import math
@@ -21,7 +22,8 @@ import torch.nn.functional as F
 
 from .gat import GAT, HGT
 from .gcn import GCN
-from .graph import chung_lu
+from .graph import Graph, add_self_loop, chung_lu, remove_self_loop
+from .SDDMM import sddmm_u_dot_v
 from .util import graph_preprocess
 
 # name: (nodes, directed edges before self loops, degree exponent, largest degree or None,
@@ -110,9 +112,65 @@ def train(model_name, dataset, epochs=20, hidden=None, layers=None, heads=8, lr=
     return (float(np.mean(dur)) if dur else math.nan), float(loss.item())
 
 
+def construct_negative_graph(g, k):
+    """evaluation/link_pred_gcn.py:164-169: k random destinations per source of every edge.  Built and
+    preprocessed (CSR / CSC / incidence, all on the device) once per epoch."""
+    src, _ = g.edges()
+    neg_src = src.repeat_interleave(k)
+    neg_dst = torch.randint(0, g.num_nodes(), (neg_src.numel(),), device=src.device)
+    return graph_preprocess(Graph(neg_src, neg_dst, g.num_nodes()))
+
+
+def train_link_pred(dataset, epochs=20, hidden=256, layers=4, k=8, lr=1e-2, weight_decay=5e-4, dropout=0.5,
+                    edge_fraction=None, quiet=False):
+    """The reference's link prediction driver (evaluation/link_pred_gcn.py:137-153,172-264): a quantized GCN
+    embeds the nodes, sddmm_u_dot_v scores the graph's edges and k sampled non-edges per edge, binary cross
+    entropy separates the two.  The negative graph is rebuilt every epoch outside the timed region, as there.
+    ``edge_fraction``: train on a random subset of the edges (the reference keeps 8 % of Reddit's).
+    Returns (mean forward + backward ms per epoch after the first three, final loss)."""
+    n, e, gamma, max_deg, sym, width, _, seed = DATASETS[dataset]
+    g = chung_lu(n, e, gamma, seed=seed, max_degree=max_deg, symmetric=sym, device="cuda")
+    if edge_fraction is None:
+        edge_fraction = 0.08 if dataset == "reddit" else 1.0
+    src, dst = g.edges()
+    if edge_fraction < 1.0:
+        keep = torch.randperm(src.numel(), device=src.device)[:int(src.numel() * edge_fraction)]
+        src, dst = src[keep], dst[keep]
+    g = graph_preprocess(Graph(*add_self_loop(*remove_self_loop(src, dst), n), n))  # link_pred_gcn.py:213-216
+    width -= width % 4  # "trim features to fit in k%4" (link_pred_gcn.py:206-208)
+    feats = torch.randn(n, width, generator=torch.Generator().manual_seed(1000 + seed)).cuda()
+    model = GCN(g, width, hidden, hidden, layers, torch.relu, dropout).cuda()
+    opt = torch.optim.Adam(model.parameters(), lr=lr, weight_decay=weight_decay)
+    dur, loss = [], None
+    for epoch in range(epochs):
+        model.train()
+        neg = construct_negative_graph(g, k)
+        start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        start.record()
+        h = model(feats).unsqueeze(1)
+        pos_score = sddmm_u_dot_v.apply(g, h, h)
+        neg_score = sddmm_u_dot_v.apply(neg, h, h)
+        score = torch.cat([pos_score, neg_score])
+        label = torch.cat([torch.ones_like(pos_score), torch.zeros_like(neg_score)])
+        loss = F.binary_cross_entropy_with_logits(score, label)
+        opt.zero_grad()
+        loss.backward()
+        stop.record()
+        torch.cuda.synchronize()
+        opt.step()
+        if epoch >= 3:
+            dur.append(start.elapsed_time(stop))
+        if not quiet:
+            print("Epoch {:05d} | Time(ms) {:.4f} | Loss {:.4f} | ETputs(KTEPS) {:.2f}".format(
+                epoch, np.mean(dur) if dur else float("nan"), loss.item(),
+                g.num_edges() / np.mean(dur) if dur else float("nan")))
+    return (float(np.mean(dur)) if dur else math.nan), float(loss.item())
+
+
 def main():
     ap = argparse.ArgumentParser(description="quantized GCN / GAT / HGT training on a synthetic stand-in of a dataset")
-    ap.add_argument("--model", choices=["gcn", "gat", "hgt"], default="gcn")
+    ap.add_argument("--model", choices=["gcn", "gat", "hgt", "linkpred"], default="gcn")
+    ap.add_argument("--k", type=int, default=8, help="negative samples per edge (linkpred)")
     ap.add_argument("--dataset", choices=sorted(DATASETS), default="pubmed")
     ap.add_argument("--epochs", type=int, default=20)
     ap.add_argument("--n-hidden", type=int, default=None)
@@ -121,8 +179,12 @@ def main():
     ap.add_argument("--lr", type=float, default=1e-2)
     ap.add_argument("--weight-decay", type=float, default=5e-4)
     args = ap.parse_args()
-    ms, loss = train(args.model, args.dataset, args.epochs, args.n_hidden, args.n_layers, args.num_heads, args.lr,
-                     args.weight_decay)
+    if args.model == "linkpred":
+        ms, loss = train_link_pred(args.dataset, args.epochs, args.n_hidden or 256, args.n_layers or 4, args.k, args.lr,
+                                   args.weight_decay)
+    else:
+        ms, loss = train(args.model, args.dataset, args.epochs, args.n_hidden, args.n_layers, args.num_heads, args.lr,
+                         args.weight_decay)
     print("mean fwd+bwd {:.3f} ms/epoch, final loss {:.4f}".format(ms, loss))
 
 

@@ -183,6 +183,17 @@ def test_evaluation_drivers_train_on_the_pubmed_stand_in(model):
     assert np.isfinite(ms) and ms > 0 and np.isfinite(loss) and loss < first_loss
 
 
+def test_link_prediction_driver_trains_on_the_pubmed_stand_in():
+    """tango_amd.evaluation.train_link_pred: the reference's evaluation/link_pred_gcn.py loop (GCN embeddings,
+    sddmm_u_dot_v scores of edges and of k sampled non-edges, a negative graph built on the device per epoch)."""
+    from tango_amd import evaluation
+    torch.manual_seed(13)
+    _, first = evaluation.train_link_pred("pubmed", epochs=1, hidden=64, layers=2, k=2, dropout=0.0, quiet=True)
+    torch.manual_seed(13)
+    ms, loss = evaluation.train_link_pred("pubmed", epochs=10, hidden=64, layers=2, k=2, dropout=0.0, lr=5e-3, quiet=True)
+    assert np.isfinite(ms) and ms > 0 and np.isfinite(loss) and loss < first
+
+
 @pytest.mark.parametrize("model_name", ["gcn", "gat"])
 def test_inference_forward_replays_from_a_hip_graph(model_name, graph):
     """The entry points launch kernels only (no memset, no host sync, scratch from the caller), so an
