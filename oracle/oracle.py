@@ -231,7 +231,7 @@ def spmm_incidence(node, edge, E, scale, num_nodes):
     node = _i64(node)
     edge = _i64(edge)
     E = _i8(E)
-    F = E.size // E.shape[0]
+    F = int(np.prod(E.shape[1:], dtype=np.int64)) if E.ndim > 1 else 1  # also for a graph without edges
     out = np.empty((num_nodes, F), dtype=np.float32)
     lib().orc_spmm_incidence(_p(out), _p(node), _p(edge), _p(E), f32(float(scale)),
                              i64(num_nodes), i64(node.size), i64(F))
