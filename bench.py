@@ -38,7 +38,7 @@ def parse():
     ap.add_argument("--emit", default=None, metavar="JSON_FILE",
                     help="also store the result under the key 'measured_mi355x' of this JSON file")
     ap.add_argument("--feat", type=int, default=256, help="feature width of --profile-mode spmm")
-    ap.add_argument("--profile-mode", choices=["spmm", "copy", "qlinear", "sddmm", "quantize", "gat", "hgt"], default=None,
+    ap.add_argument("--profile-mode", choices=["spmm", "copy", "qlinear", "gradx", "sddmm", "quantize", "gat", "hgt"], default=None,
                     help="run only the dominant kernel (spmm: copy_u F=256 on the benchmark graph) or a "
                          "1 GiB device copy (counter calibration), for rocprofv3 --pmc passes")
     return ap.parse_args()
@@ -379,6 +379,16 @@ def main():
         ms = time_op(lambda: K.QGEMM_forward(X, Xq, sX, W, Wq, sW, None, True), iters=args.steps, warm=args.warmup)
         print(json.dumps({"profile_mode": "qlinear", "M": M, "K": Kd, "N": N, "avg_ms": round(ms, 4),
                           "ops": 2 * M * N * Kd, "algorithmic_bytes": 5 * (M * Kd + N * Kd) + 4 * M * N + 4 * N}))
+        return
+    if args.profile_mode == "gradx":  # gradX of the epoch's second layer: int8 dY [M, 41] -> fp32 dX [M, 256]
+        M, Kd, N = args.nodes, 256, 41
+        dY, s_dY = K.quantize_padded(torch.randn(M, N, device="cuda"))
+        Wq, sW = K.quantize(torch.randn(N, Kd, device="cuda") * 0.05)
+        Xq = torch.empty((M, Kd), dtype=torch.int8, device="cuda")
+        sX = torch.ones(1, device="cuda")
+        ms = time_op(lambda: K.QGEMM_backward(dY, Xq, Wq, s_dY, sX, sW, True, False), iters=args.steps, warm=args.warmup)
+        print(json.dumps({"profile_mode": "gradx", "M": M, "K": Kd, "N": N, "avg_ms": round(ms, 4),
+                          "ops": 2 * M * N * Kd, "algorithmic_bytes": M * N + N * Kd + 4 * M * Kd}))
         return
     if args.profile_mode == "quantize":
         X = torch.randn(args.nodes, 602, device="cuda")
