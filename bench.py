@@ -154,6 +154,21 @@ def primitives(g, K, torch):
         out[tag.replace("fwd", "gradW")] = {"ms": round(ms, 4), "TOPS": round(ops / ms / 1e9, 2),
                                             "GBps": round(byt / ms / 1e6, 1)}
         del X, W, Xq, dY
+    # the two call patterns of evaluation/test_cache_GEMM.py and evaluation/test_fuse.py at the first layer's shape:
+    # the forward on an input that was quantized once before (several consumers share it), and the output scale
+    # from the GEMM's epilogue against a separate absmax pass over Y
+    M, Kd, N = n, 256, 256
+    X = torch.randn(M, Kd, device="cuda")
+    W = torch.randn(N, Kd, device="cuda") * 0.05
+    sX, sW = K.cuda_kernels.get_scale(X), K.cuda_kernels.get_scale(W)
+    Xq = torch.empty((M, Kd), dtype=torch.int8, device="cuda")
+    Wq = torch.empty((N, Kd), dtype=torch.int8, device="cuda")
+    t_fused = time_op(lambda: K.QGEMM_forward(X, Xq, sX, W, Wq, sW, None, True), iters=10)
+    t_cached = time_op(lambda: K.QGEMM_forward(None, Xq, sX, W, Wq, sW, None, True), iters=10)
+    t_plain = time_op(lambda: K.cuda_kernels.get_scale(K.QGEMM_forward(X, Xq, sX, W, Wq, sW, None, False)), iters=10)
+    out["qlinear_fwd_%dx%dx%d" % (M, Kd, N)] = {"ms": round(t_fused, 4), "ms_input_already_int8": round(t_cached, 4),
+                                                 "ms_with_separate_output_absmax": round(t_plain, 4)}
+    del X, W, Xq, Wq
     # the int8 matrix rate the device sustains on register-resident operands (the ceiling of any int8 GEMM here)
     from tango_amd import _lib
     sink = torch.zeros(1, dtype=torch.int32, device="cuda")
