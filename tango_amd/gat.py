@@ -9,7 +9,7 @@ import torch.nn.functional as F
 
 from torch.autograd.function import Function, once_differentiable
 
-from .QLinear import QLinear, quantize_input
+from .QLinear import QLinear, Qlinear_func_reduce, quantize_input
 from .kernels import cuda_kernels
 from .SDDMM import sddmm_u_add_v, sddmm_u_dot_v
 from .SPMM import spmm_u_mul_e
@@ -148,8 +148,10 @@ class HGTLayer(nn.Module):
         for lin in (self.q_linear, self.k_linear, self.v_linear, self.msg_linear, self.attn_linear):
             lin.enable_reduce()
 
-    def forward(self, g, h):
-        h_q, s_h = quantize_input(h)  # one absmax and one quantize pass for the three projections of h
+    def forward(self, g, h, s_h=None, return_scale=False):
+        """``s_h``: max|h| / 127 when the producer of h knows it (the previous layer's output GEMM);
+        ``return_scale``: also return this layer's output scale for the next layer."""
+        h_q, s_h = quantize_input(h, s_h)  # one absmax (unless handed in) and one quantize pass for the three projections of h
         k, s_k = self.k_linear(h, s_h, h_q)
         k, s_k = self.attn_linear(k, s_k)
         v, s_v = self.v_linear(h, s_h, h_q)
@@ -159,6 +161,8 @@ class HGTLayer(nn.Module):
         t = sddmm_u_dot_v.apply(g, k, q, s_k, s_q, 1.0 / self.sqrt_dk)  # "/ sqrt_dk" folded into the scales
         attn = edge_softmax(g, t)
         t = spmm_u_mul_e.apply(g, v, attn, None, s_v).reshape(-1, self.out_dim)
+        if return_scale:
+            return Qlinear_func_reduce.apply(t, self.a_linear.weight, self.a_linear.bias)
         return self.a_linear(t)
 
 
@@ -176,6 +180,10 @@ class HGTStack(nn.Module):
         self.proj = nn.Linear(hidden, n_classes)
 
     def forward(self, g, h):
-        for layer in self.layers:
-            h = layer(g, h)
+        s_h = None
+        for i, layer in enumerate(self.layers):
+            if i + 1 < len(self.layers):  # the output GEMM's epilogue hands max|h| / 127 to the next layer
+                h, s_h = layer(g, h, s_h, return_scale=True)
+            else:
+                h = layer(g, h, s_h)
         return self.proj(h)

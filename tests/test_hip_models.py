@@ -141,6 +141,23 @@ def test_hgt_stack_on_heterogeneous_graph():
     assert all(np.isfinite(losses)) and losses[-1] < losses[0], losses
 
 
+def test_hgt_layers_hand_their_output_scale_on(graph):
+    """Between HGT layers the output GEMM's epilogue supplies the next layer's input scale: same bits as the
+    absmax pass the next layer would run itself."""
+    from tango_amd.gat import HGTStack
+    g = graph
+    torch.manual_seed(21)
+    model = HGTStack(64, 64, 5, 4, n_layers=3).cuda()
+    x = torch.randn(g.num_nodes(), 64, device="cuda")
+    with torch.no_grad():
+        got = model(g, x)
+        h = x
+        for layer in model.layers:
+            h = layer(g, h)
+        want = model.proj(h)
+    assert torch.equal(got, want)
+
+
 def test_edge_renumbering_leaves_node_outputs_unchanged():
     """Destination-major edge numbering (Graph.reorder_edges_by_dst) is an internal matter of the
     attention layers: same node outputs and parameter gradients, attention values permuted."""
