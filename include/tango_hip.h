@@ -173,11 +173,13 @@ int tango_qgemm_bwd_dx(float* dX, int64_t lddx, const int8_t* dYq, int64_t lddy,
                        tango_stream_t stream);
 
 /* As tango_qgemm_bwd_dx, with row m of the result multiplied by row_scale[m]
-   (the backward of the folded row multiplier above). */
+   (the backward of the folded row multiplier above).  accumulate != 0: the result is added to
+   what dX holds, for an input that feeds several layers (the sum autograd forms of their input
+   gradients, evaluation/test_HGT.py:51-53, without the separate additions). */
 int tango_qgemm_bwd_dx_ex(float* dX, int64_t lddx, const int8_t* dYq, int64_t lddy,
                           const int8_t* Wq, int64_t ldw, const float* s_dY, const float* s_W,
-                          const float* row_scale, int64_t M, int64_t N, int64_t K, void* workspace,
-                          size_t workspace_bytes, tango_stream_t stream);
+                          const float* row_scale, int accumulate, int64_t M, int64_t N, int64_t K,
+                          void* workspace, size_t workspace_bytes, tango_stream_t stream);
 
 /* QGEMM_backward_gradW (cuda/src/cuda.cpp:100-108 -> QGEMM_backward.cu:50-113):
    dW[N,K] = (s_dY*s_X) * float(sum_m dYq[m,n] * Xq[m,k]), int32 accumulation.

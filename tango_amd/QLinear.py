@@ -132,6 +132,61 @@ class Qlinear_func_reduce(Function):
         return _backward(ctx, grad_output) + (None, None)
 
 
+class Qlinear_shared_func(Function):
+    """Several linear layers over one input (the k / v / q projections of evaluation/test_HGT.py:51-53)
+    as one autograd node: ``apply(X, Xq, scaleX, W_0, b_0, W_1, b_1, ...)`` with (Xq, scaleX) from
+    ``quantize_input(X)`` returns (Y_0, scale_0, Y_1, scale_1, ...), each pair what Qlinear_func_reduce
+    returns.  Backward runs each layer's weight / bias gradient as usual, and the input gradients go into
+    one tensor: the first layer's GEMM writes it, the others add to it in their epilogues, where autograd
+    would run a separate addition per extra layer over three [M, K] fp32 tensors."""
+
+    @staticmethod
+    def forward(ctx, X, Xq, scaleX, *wb):
+        if len(wb) == 0 or len(wb) % 2:
+            raise RuntimeError("Qlinear_shared_func: expects (weight, bias) pairs")
+        if tuple(Xq.shape) != tuple(X.shape) or Xq.dtype != torch.int8 or X.dim() != 2:
+            raise RuntimeError("Qlinear_shared_func: the quantized input must be int8 of the 2-D input's shape")
+        ctx.set_materialize_grads(False)
+        outs, layers = [], []
+        for W, b in zip(wb[0::2], wb[1::2]):
+            scaleW = kernels.cuda_kernels.get_scale(W if W.is_contiguous() else W.contiguous())
+            W_ = torch.empty(W.shape, dtype=torch.int8, device=X.device)
+            out, scaleO = kernels.QGEMM_forward(None, Xq, scaleX, W, W_, scaleW, b, True)
+            ctx.mark_non_differentiable(scaleO)
+            outs += [out, scaleO]
+            layers.append((W_, scaleW, b is not None))
+        ctx.backward_cache = Xq, scaleX, layers
+        return tuple(outs)
+
+    @staticmethod
+    @once_differentiable
+    def backward(ctx, *grads):
+        Xq, scaleX, layers = ctx.backward_cache
+        dX, rest = None, []
+        for i, (W_, scaleW, has_bias) in enumerate(layers):
+            dY = grads[2 * i]
+            if dY is None:
+                rest += [None, None]
+                continue
+            want_bias = has_bias and ctx.needs_input_grad[4 + 2 * i]
+            dY_, scaledY, grad_bias = _quantize_grad(dY, want_bias)
+            dXi, dW = kernels.QGEMM_backward(dY_, Xq, W_, scaledY, scaleX, scaleW, ctx.needs_input_grad[0],
+                                             ctx.needs_input_grad[3 + 2 * i], dX_acc=dX)
+            dX = dXi if dXi is not None else dX
+            rest += [dW, grad_bias]
+        return (dX, None, None) + tuple(rest)
+
+
+def shared_input_linears(X, layers, scaleX=None):
+    """[(Y, scale of Y)] of the QLinear ``layers`` applied to one 2-D input: X is quantized once and the
+    layers run as one autograd node (Qlinear_shared_func)."""
+    Xq, scaleX = quantize_input(X, scaleX)
+    X = X if X.is_contiguous() else X.contiguous()
+    flat = [t for lin in layers for t in (lin.weight, lin.bias)]
+    res = Qlinear_shared_func.apply(X, Xq, scaleX, *flat)
+    return [(res[2 * i], res[2 * i + 1]) for i in range(len(layers))]
+
+
 class QLinear(nn.Linear):
     """cuda/QLinear.py:74-93.  The reference requires in_features % 4 == 0 for
     its 128-bit loads; any width works here."""

@@ -60,6 +60,7 @@ struct NtParams {
     int64_t M, N, Kr;    // Kr = reduction length
     int64_t lda, ldb, ldc;
     int64_t a_row_bytes; // bytes that may be read from each row of A (>= Kr)
+    int accumulate;      // nonzero: the product is added to what C holds (gradients of one tensor from several layers)
 };
 
 // Workgroup = 4 waves = 128 rows x (16 * NT) columns.  gridDim = (ceil(M/128), ceil(N/(16 NT))).
@@ -173,6 +174,17 @@ __global__ __launch_bounds__(256, 2) void gemm_nt_kernel(const NtParams p) {
                     if (p.bias) y[v] = bv[v] + y[v];
                     if (col + v < p.N) m = fmaxf(m, fabsf(y[v]));
                 }
+                if (p.accumulate) {  // uniform; the absmax above is of the product alone and is not asked for with it
+                    if (col + 4 <= p.N && wide == 4) {
+                        const f32x4 o = *reinterpret_cast<const f32x4*>(crow + col);
+                        *reinterpret_cast<f32x4*>(crow + col) = f32x4{o[0] + y[0], o[1] + y[1], o[2] + y[2], o[3] + y[3]};
+                    } else {
+#pragma unroll
+                        for (int v = 0; v < 4; ++v)
+                            if (col + v < p.N) crow[col + v] += y[v];
+                    }
+                    continue;
+                }
                 if (col + 4 <= p.N && wide == 4) {
                     *reinterpret_cast<f32x4*>(crow + col) = f32x4{y[0], y[1], y[2], y[3]};
                 } else if (col + 4 <= p.N && wide == 2) {
@@ -275,6 +287,17 @@ __global__ __launch_bounds__(64 * WAVES) void gemm_nts_kernel(const NtParams p, 
                     if (p.row_scale) y[v] = y[v] * rsc;
                     if (p.bias) y[v] = bv[v] + y[v];
                     if (col + v < p.N) m = fmaxf(m, fabsf(y[v]));
+                }
+                if (p.accumulate) {  // uniform
+                    if (col + 4 <= p.N && wide == 4) {
+                        const f32x4 o = *reinterpret_cast<const f32x4*>(crow + col);
+                        *reinterpret_cast<f32x4*>(crow + col) = f32x4{o[0] + y[0], o[1] + y[1], o[2] + y[2], o[3] + y[3]};
+                    } else {
+#pragma unroll
+                        for (int v = 0; v < 4; ++v)
+                            if (col + v < p.N) crow[col + v] += y[v];
+                    }
+                    continue;
                 }
                 if (col + 4 <= p.N && wide == 4) {
                     *reinterpret_cast<f32x4*>(crow + col) = f32x4{y[0], y[1], y[2], y[3]};
@@ -1228,7 +1251,7 @@ size_t tango_qgemm_bwd_dx_workspace(int64_t M, int64_t N, int64_t K) {
 
 int tango_qgemm_bwd_dx_ex(float* dX, int64_t lddx, const int8_t* dYq, int64_t lddy,
                           const int8_t* Wq, int64_t ldw, const float* s_dY, const float* s_W,
-                          const float* row_scale,
+                          const float* row_scale, int accumulate,
                        int64_t M, int64_t N, int64_t K, void* workspace, size_t workspace_bytes,
                        tango_stream_t stream) {
     if (M < 0 || N < 0 || K < 0 || !s_dY || !s_W || lddx < K || lddy < N || ldw < K)
@@ -1246,7 +1269,7 @@ int tango_qgemm_bwd_dx_ex(float* dX, int64_t lddx, const int8_t* dYq, int64_t ld
         hipLaunchKernelGGL(transpose_pack_i8_kernel, dim3(grid_for(K * ldt, 256)), dim3(256), 0, s, Wt,
                            ldt, Wq, ldw, N, K);
     NtParams p{};
-    p.C = dX; p.A = dYq; p.B = Wt; p.sA = s_dY; p.sB = s_W; p.row_scale = row_scale;
+    p.C = dX; p.A = dYq; p.B = Wt; p.sA = s_dY; p.sB = s_W; p.row_scale = row_scale; p.accumulate = accumulate;
     p.M = M; p.N = K; p.Kr = N; p.lda = lddy; p.ldb = ldt; p.ldc = lddx;
     return launch_nt(p, s);
 }
@@ -1255,7 +1278,7 @@ int tango_qgemm_bwd_dx(float* dX, int64_t lddx, const int8_t* dYq, int64_t lddy,
                        const int8_t* Wq, int64_t ldw, const float* s_dY, const float* s_W,
                        int64_t M, int64_t N, int64_t K, void* workspace, size_t workspace_bytes,
                        tango_stream_t stream) {
-    return tango_qgemm_bwd_dx_ex(dX, lddx, dYq, lddy, Wq, ldw, s_dY, s_W, nullptr, M, N, K, workspace,
+    return tango_qgemm_bwd_dx_ex(dX, lddx, dYq, lddy, Wq, ldw, s_dY, s_W, nullptr, 0, M, N, K, workspace,
                                  workspace_bytes, stream);
 }
 

@@ -9,7 +9,7 @@ import torch.nn.functional as F
 
 from torch.autograd.function import Function, once_differentiable
 
-from .QLinear import QLinear, Qlinear_func_reduce, quantize_input
+from .QLinear import QLinear, Qlinear_func_reduce, shared_input_linears
 from .kernels import cuda_kernels
 from .SDDMM import sddmm_u_add_v, sddmm_u_dot_v
 from .SPMM import spmm_u_mul_e
@@ -151,12 +151,11 @@ class HGTLayer(nn.Module):
     def forward(self, g, h, s_h=None, return_scale=False):
         """``s_h``: max|h| / 127 when the producer of h knows it (the previous layer's output GEMM);
         ``return_scale``: also return this layer's output scale for the next layer."""
-        h_q, s_h = quantize_input(h, s_h)  # one absmax (unless handed in) and one quantize pass for the three projections of h
-        k, s_k = self.k_linear(h, s_h, h_q)
+        # one absmax (unless handed in) and one quantize pass for the three projections of h, and one input
+        # gradient that their backward GEMMs accumulate into
+        (k, s_k), (v, s_v), (q, s_q) = shared_input_linears(h, (self.k_linear, self.v_linear, self.q_linear), s_h)
         k, s_k = self.attn_linear(k, s_k)
-        v, s_v = self.v_linear(h, s_h, h_q)
         v, s_v = self.msg_linear(v, s_v)
-        q, s_q = self.q_linear(h, s_h, h_q)
         k, v, q = (t.view(-1, self.n_heads, self.d_k) for t in (k, v, q))
         t = sddmm_u_dot_v.apply(g, k, q, s_k, s_q, 1.0 / self.sqrt_dk)  # "/ sqrt_dk" folded into the scales
         attn = edge_softmax(g, t)

@@ -343,7 +343,8 @@ class cuda_kernels:
                                    scaleB.data_ptr(), M, N, K, _ptr(ws), ws_bytes, _stream()), "QGEMM_i8")
 
     @staticmethod
-    def QGEMM_backward_gradX(dX, dY, W, scaledY, scaleW, row_scale=None):
+    def QGEMM_backward_gradX(dX, dY, W, scaledY, scaleW, row_scale=None, accumulate=False):
+        """``accumulate``: add the product to what dX holds instead of overwriting it."""
         _need(dX, torch.float32, "dX", contiguous=False)
         _need(dY, torch.int8, "dY", contiguous=False)
         _need(W, torch.int8, "W", contiguous=False)
@@ -359,7 +360,8 @@ class cuda_kernels:
             _need(row_scale, torch.float32, "row_scale")
         check(_L.tango_qgemm_bwd_dx_ex(_ptr(dX), _rows_view(dX, "dX"), _ptr(dY), _rows_view(dY, "dY"),
                                        _ptr(W), _rows_view(W, "W"), scaledY.data_ptr(), scaleW.data_ptr(),
-                                       _ptr(row_scale), M, N, K, _ptr(ws), ws_bytes, _stream()),
+                                       _ptr(row_scale), int(bool(accumulate)), M, N, K, _ptr(ws), ws_bytes,
+                                       _stream()),
               "QGEMM_backward_gradX")
 
     @staticmethod
@@ -692,16 +694,18 @@ def QGEMM_forward(x, x_, scaleX, w, w_, scaleW, bias=None, isReduce=False, round
     return out_fp
 
 
-def QGEMM_backward(dY, X, W, scaledY, scaleX, scaleW, X_need=True, W_need=True, x_row_scale=None):
-    """cuda/kernels.py:97-111."""
+def QGEMM_backward(dY, X, W, scaledY, scaleX, scaleW, X_need=True, W_need=True, x_row_scale=None, dX_acc=None):
+    """cuda/kernels.py:97-111.  ``dX_acc``: a gradient of X from another consumer; the input gradient is
+    added to it in place (and it is returned) instead of going to a new tensor."""
     assert scaledY.is_cuda, "scaledY must be on GPU"
     assert dY.is_cuda, "dY must be on GPU"
     dX, dW = None, None
     if X_need:
         assert W.is_cuda, "W must be on GPU"
         assert scaleW.is_cuda, "scaleW must be on GPU"
-        dX = torch.empty(X.shape, dtype=torch.float32, device=X.device)
-        cuda_kernels.QGEMM_backward_gradX(dX, dY, W, scaledY, scaleW, row_scale=x_row_scale)
+        dX = torch.empty(X.shape, dtype=torch.float32, device=X.device) if dX_acc is None else dX_acc
+        cuda_kernels.QGEMM_backward_gradX(dX, dY, W, scaledY, scaleW, row_scale=x_row_scale,
+                                          accumulate=dX_acc is not None)
     if W_need:
         assert X.is_cuda, "X must be on GPU"
         assert scaleX.is_cuda, "scaleX must be on GPU"

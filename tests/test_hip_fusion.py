@@ -375,3 +375,39 @@ def test_linear_layers_sharing_one_quantized_input(M, Kd, N):
         grads.append([t.grad.clone() for t in (x, *a.parameters(), *b.parameters())])
     assert all(torch.equal(p, q) for p, q in zip(*outs))
     assert all(torch.equal(p, q) for p, q in zip(*grads))
+
+
+@pytest.mark.parametrize("M,Kd,N", [(3000, 256, 256), (1000, 100, 41), (700, 602, 300)])
+def test_shared_input_linears_accumulate_one_input_gradient(M, Kd, N):
+    """Three layers over one input as a single autograd node == the three layers on their own: outputs, output
+    scales, weight and bias gradients bit for bit, and the input gradient equal to the layers' input gradients
+    added in layer order (the node's GEMM epilogues add in that order).  One layer's output is left unused in
+    a second pass: its gradients stay None and the other two still add up."""
+    from tango_amd.QLinear import QLinear, shared_input_linears
+    torch.manual_seed(M + N + 1)
+    lins = [QLinear(Kd, N).cuda(), QLinear(Kd, N, bias=False).cuda(), QLinear(Kd, N).cuda()]
+    for lin in lins:
+        lin.enable_reduce()
+    params = [p for lin in lins for p in lin.parameters()]
+    x = torch.randn(M, Kd, device="cuda", requires_grad=True)
+    ws = [torch.randn(M, N, device="cuda") for _ in lins]
+    for used in ((0, 1, 2), (0, 2)):
+        want_y, want_dx, want_dp = [], None, []
+        for i, lin in enumerate(lins):
+            y, s = lin(x)
+            want_y.append((y.detach().clone(), s.clone()))
+            if i in used:
+                g = torch.autograd.grad((y * ws[i]).sum(), [x] + list(lin.parameters()))
+                want_dx = g[0] if want_dx is None else want_dx + g[0]
+                want_dp += list(g[1:])
+            else:
+                want_dp += [None] * len(list(lin.parameters()))
+        for t in [x] + params:
+            t.grad = None
+        res = shared_input_linears(x, lins)
+        sum((res[i][0] * ws[i]).sum() for i in used).backward()
+        for (y, s), (wy, wsc) in zip(res, want_y):
+            assert torch.equal(y, wy) and torch.equal(s, wsc)
+        assert torch.equal(x.grad, want_dx)
+        for p, w in zip(params, want_dp):
+            assert (p.grad is None and w is None) or torch.equal(p.grad, w)

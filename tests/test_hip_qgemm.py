@@ -181,6 +181,30 @@ def test_qgemm_i8_small_operand_stationary(K, orc, M, N, Kd):
     assert np.array_equal(host(Y), want) and host(sY)[0] == orc.absmax_scale(want)
 
 
+@pytest.mark.parametrize("M,N,Kd,rows", [(5000, 256, 256, False), (3001, 300, 41, True), (777, 64, 130, False)])
+def test_gradx_accumulates_into_its_output(K, M, N, Kd, rows):
+    """gradX added to what dX holds == dX + the gradX written on its own, bit for bit (one fp32 addition per
+    element), through the stationary form (reduction <= 256), the streaming form (reduction 300), odd and
+    even output widths and a row multiplier."""
+    rng = np.random.default_rng(M + N + Kd)
+    dY = rng.integers(-127, 128, (M, N)).astype(np.int8)
+    W = rng.integers(-127, 128, (N, Kd)).astype(np.int8)
+    prior = rng.standard_normal((M, Kd)).astype(np.float32)
+    rs = dev(rng.random(M).astype(np.float32) + 0.5) if rows else None
+    ld = (N + 15) // 16 * 16
+    dYb = torch.full((M, max(ld, 16)), 55, dtype=torch.int8, device="cuda")
+    dYb[:, :N] = dev(dY)
+    alone = torch.empty((M, Kd), dtype=torch.float32, device="cuda")
+    K.cuda_kernels.QGEMM_backward_gradX(alone, dYb[:, :N], dev(W), sc(0.5), sc(0.125), row_scale=rs)
+    acc = (dY.astype(np.float64) @ W.astype(np.float64)).astype(np.float32) * np.float32(0.0625)
+    if rows:
+        acc = acc * host(rs)[:, None]
+    assert np.array_equal(host(alone), acc)
+    out = dev(prior)
+    K.cuda_kernels.QGEMM_backward_gradX(out, dYb[:, :N], dev(W), sc(0.5), sc(0.125), row_scale=rs, accumulate=True)
+    assert np.array_equal(host(out), prior + acc)
+
+
 def test_mfma_rate_probe_runs():
     """The measurement aid launches, finishes and leaves its sink untouched."""
     from tango_amd import _lib
