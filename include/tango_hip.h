@@ -321,9 +321,12 @@ int tango_edge_softmax_bwd(float* de, const float* a, const float* da, const flo
 
 /* el[n,h] = sum_d feat[n,h,d] * attn_l[h,d], er likewise with attn_r: the two
    broadcast-multiply + sum lines of the GAT layer (evaluation/test_gat.py:135-137),
-   torch ops in the reference, in one read of feat.  fp32. */
-int tango_attn_scores_fwd(float* el, float* er, const float* feat, const float* attn_l,
-                          const float* attn_r, int64_t n, int64_t H, int64_t D,
+   torch ops in the reference, in one read of feat.  fp32.  scale_el / scale_er (both or
+   neither): pre-zeroed slots that receive max|el| / 127 and max|er| / 127 (what get_scale
+   computes in a pass of its own, cuda/kernels.py:26-27, when sddmm_u_add_v quantizes the
+   two, cuda/SDDMM.py:13-17). */
+int tango_attn_scores_fwd(float* el, float* er, float* scale_el, float* scale_er, const float* feat,
+                          const float* attn_l, const float* attn_r, int64_t n, int64_t H, int64_t D,
                           tango_stream_t stream);
 
 /* Backward of the above: dfeat[n,h,d] = del[n,h]*attn_l[h,d] + der[n,h]*attn_r[h,d],

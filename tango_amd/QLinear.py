@@ -124,11 +124,14 @@ class Qlinear_func_reduce(Function):
     def forward(ctx, X, W, b=None, row_scale=None, scaleX=None, Xq=None):
         out, scaleO = _forward(ctx, X, W, b, True, row_scale, scaleX, Xq)
         ctx.mark_non_differentiable(scaleO)
+        ctx.set_materialize_grads(False)  # no zero tensor (a fill launch) for the scale's absent gradient
         return out, scaleO
 
     @staticmethod
     @once_differentiable
     def backward(ctx, grad_output, grad_dummy):
+        if grad_output is None:
+            return (None,) * 6
         return _backward(ctx, grad_output) + (None, None)
 
 

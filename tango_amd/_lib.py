@@ -47,7 +47,7 @@ SIGNATURES = {
     "tango_spmm_csr_copy_u_ex": (I, [P, P, P, I, P, I64, P, P, P, I, P, I64, I64, I64, I64, I64, P, SZ, P]),
     "tango_spmm_csr_u_mul_e": (I, [P, P, P, P, P, P, P, I64, I64, I64, I64, I64, I64, P]),
     "tango_spmm_csr_u_mul_e_ex": (I, [P, P, P, P, I, P, P, I, P, P, P, I, I64, I64, I64, I64, I64, I64, I64, P, SZ, P]),
-    "tango_attn_scores_fwd": (I, [P, P, P, P, P, I64, I64, I64, P]),
+    "tango_attn_scores_fwd": (I, [P, P, P, P, P, P, P, I64, I64, I64, P]),
     "tango_attn_scores_bwd_workspace": (SZ, [I64, I64, I64]),
     "tango_attn_scores_bwd": (I, [P, P, P, P, P, P, P, P, I64, I64, I64, P, SZ, P]),
     "tango_spmm_incidence": (I, [P, P, P, P, P, I64, I64, I64, I64, P]),

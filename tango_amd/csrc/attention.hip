@@ -18,35 +18,51 @@ namespace tango {
 constexpr int kDChunk = 16;       // columns of one head a backward thread keeps in registers
 constexpr int kBwdGroups = 1024;  // workgroups (slabs) of the backward reduction
 
-__global__ __launch_bounds__(256) void attn_scores_fwd_kernel(
-    float* __restrict__ el, float* __restrict__ er, const float* __restrict__ feat,
-    const float* __restrict__ al, const float* __restrict__ ar, int64_t total, int H, int D, int vec4) {
-    const int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;  // (node, head)
-    if (i >= total) return;
-    const int h = static_cast<int>(i % H);
-    const float* f = feat + i * D;
-    const float* a = al + static_cast<int64_t>(h) * D;
-    const float* b = ar + static_cast<int64_t>(h) * D;
-    float sl = 0.0f, sr = 0.0f;
-    if (vec4) {
-        for (int d = 0; d < D; d += 4) {
-            const f32x4 x = *reinterpret_cast<const f32x4*>(f + d);
-            const f32x4 u = *reinterpret_cast<const f32x4*>(a + d);
-            const f32x4 v = *reinterpret_cast<const f32x4*>(b + d);
+// One (node, head) item per thread and loop step.  SCALES: the launch is a fixed number of large workgroups
+// walking the items with a grid stride, and each ends with one atomic max per output of max|el| / 127 and
+// max|er| / 127 into pre-zeroed slots, so the quantize passes that follow need no absmax pass of their own.
+template <bool SCALES>
+__global__ __launch_bounds__(SCALES ? 1024 : 256) void attn_scores_fwd_kernel(
+    float* __restrict__ el, float* __restrict__ er, float* __restrict__ scale_el, float* __restrict__ scale_er,
+    const float* __restrict__ feat, const float* __restrict__ al, const float* __restrict__ ar, int64_t total,
+    int H, int D, int vec4) {
+    const int64_t nthr = static_cast<int64_t>(gridDim.x) * blockDim.x;
+    float ml = 0.0f, mr = 0.0f;
+    for (int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < total; i += nthr) {
+        const int h = static_cast<int>(i % H);
+        const float* f = feat + i * D;
+        const float* a = al + static_cast<int64_t>(h) * D;
+        const float* b = ar + static_cast<int64_t>(h) * D;
+        float sl = 0.0f, sr = 0.0f;
+        if (vec4) {
+            for (int d = 0; d < D; d += 4) {
+                const f32x4 x = *reinterpret_cast<const f32x4*>(f + d);
+                const f32x4 u = *reinterpret_cast<const f32x4*>(a + d);
+                const f32x4 v = *reinterpret_cast<const f32x4*>(b + d);
 #pragma unroll
-            for (int k = 0; k < 4; ++k) {
-                sl += x[k] * u[k];
-                sr += x[k] * v[k];
+                for (int k = 0; k < 4; ++k) {
+                    sl += x[k] * u[k];
+                    sr += x[k] * v[k];
+                }
+            }
+        } else {
+            for (int d = 0; d < D; ++d) {
+                sl += f[d] * a[d];
+                sr += f[d] * b[d];
             }
         }
-    } else {
-        for (int d = 0; d < D; ++d) {
-            sl += f[d] * a[d];
-            sr += f[d] * b[d];
+        el[i] = sl;
+        er[i] = sr;
+        if (SCALES) {
+            ml = fmaxf(ml, fabsf(sl));
+            mr = fmaxf(mr, fabsf(sr));
         }
     }
-    el[i] = sl;
-    er[i] = sr;
+    if (SCALES) {
+        block_absmax_to_global(ml / 127.0f, scale_el);
+        __syncthreads();  // the helper's staging array is reused by the second call
+        block_absmax_to_global(mr / 127.0f, scale_er);
+    }
 }
 
 // blockDim.x = tpb, a multiple of H: thread t is head t % H of row slot t / H.  gridDim.y tiles D
@@ -149,9 +165,11 @@ using namespace tango;
 
 extern "C" {
 
-int tango_attn_scores_fwd(float* el, float* er, const float* feat, const float* attn_l,
-                          const float* attn_r, int64_t n, int64_t H, int64_t D, tango_stream_t stream) {
+int tango_attn_scores_fwd(float* el, float* er, float* scale_el, float* scale_er, const float* feat,
+                          const float* attn_l, const float* attn_r, int64_t n, int64_t H, int64_t D,
+                          tango_stream_t stream) {
     if (n < 0 || H < 0 || D < 0 || H >= (1LL << 31) || D >= (1LL << 31)) return TANGO_ERR_INVALID_ARG;
+    if ((scale_el == nullptr) != (scale_er == nullptr)) return TANGO_ERR_INVALID_ARG;
     if (n * H == 0) return TANGO_OK;
     if (!el || !er || (D > 0 && (!feat || !attn_l || !attn_r))) return TANGO_ERR_INVALID_ARG;
     const int64_t total = n * H;
@@ -159,9 +177,18 @@ int tango_attn_scores_fwd(float* el, float* er, const float* feat, const float* 
     const uintptr_t bits = reinterpret_cast<uintptr_t>(feat) | reinterpret_cast<uintptr_t>(attn_l) |
                            reinterpret_cast<uintptr_t>(attn_r);
     const int vec4 = (D % 4 == 0) && (bits & 15) == 0;
-    hipLaunchKernelGGL(attn_scores_fwd_kernel, dim3(static_cast<unsigned>(ceil_div(total, 256))), dim3(256), 0,
-                       as_stream(stream), el, er, feat, attn_l, attn_r, total, static_cast<int>(H),
-                       static_cast<int>(D), vec4);
+    if (scale_el) {
+        // one 16-wave workgroup per compute unit at most: a few hundred atomics per slot in all
+        const int64_t want = ceil_div(total, 1024);
+        const unsigned groups = static_cast<unsigned>(want < 256 ? want : 256);
+        hipLaunchKernelGGL(attn_scores_fwd_kernel<true>, dim3(groups), dim3(1024), 0, as_stream(stream), el, er,
+                           scale_el, scale_er, feat, attn_l, attn_r, total, static_cast<int>(H),
+                           static_cast<int>(D), vec4);
+    } else {
+        hipLaunchKernelGGL(attn_scores_fwd_kernel<false>, dim3(static_cast<unsigned>(ceil_div(total, 256))),
+                           dim3(256), 0, as_stream(stream), el, er, scale_el, scale_er, feat, attn_l, attn_r, total,
+                           static_cast<int>(H), static_cast<int>(D), vec4);
+    }
     return launch_status();
 }
 

@@ -19,20 +19,28 @@ from .edge_softmax import edge_softmax
 class attn_scores(Function):
     """el = (feat * attn_l).sum(-1), er = (feat * attn_r).sum(-1) for feat [n, H, D] and
     attn_l, attn_r [1, H, D] (evaluation/test_gat.py:135-137), forward and backward each in
-    one pass over feat.  Returns el, er as [n, H, 1]."""
+    one pass over feat.  Returns el, er as [n, H, 1] and their quantization scales max|.| / 127
+    (None while a graph is being captured), which the same kernel finds."""
 
     @staticmethod
     def forward(ctx, feat, attn_l, attn_r):
         feat = feat if feat.is_contiguous() else feat.contiguous()
         al, ar = attn_l.contiguous(), attn_r.contiguous()
-        el, er = cuda_kernels.attn_scores_forward(feat, al, ar)
+        el, er, s_el, s_er = cuda_kernels.attn_scores_forward(feat, al, ar, want_scales=True)
         ctx.backward_cache = feat, al, ar, attn_l.shape
-        return el.unsqueeze(-1), er.unsqueeze(-1)
+        ctx.set_materialize_grads(False)  # no zero tensors (a fill launch each) for the scales' absent gradients
+        if s_el is not None:
+            ctx.mark_non_differentiable(s_el, s_er)
+        return el.unsqueeze(-1), er.unsqueeze(-1), s_el, s_er
 
     @staticmethod
     @once_differentiable
-    def backward(ctx, del_, der):
+    def backward(ctx, del_, der, _ds_el=None, _ds_er=None):
         feat, al, ar, shape = ctx.backward_cache
+        if del_ is None and der is None:
+            return None, None, None
+        del_ = torch.zeros_like(der) if del_ is None else del_
+        der = torch.zeros_like(del_) if der is None else der
         dfeat, dal, dar = cuda_kernels.attn_scores_backward(del_.contiguous(), der.contiguous(), feat, al, ar)
         return dfeat, dal.view(shape), dar.view(shape)
 
@@ -80,8 +88,8 @@ class QGATConv(nn.Module):
         h = self.feat_drop(feat).contiguous()
         feat_src, s_feat = self.fc(h)
         feat_src = feat_src.view(n, self._num_heads, self._out_feats)
-        el, er = attn_scores.apply(feat_src, self.attn_l, self.attn_r)  # test_gat.py:135-137
-        e = sddmm_u_add_v.apply(graph, el, er)                      # :141
+        el, er, s_el, s_er = attn_scores.apply(feat_src, self.attn_l, self.attn_r)  # test_gat.py:135-137
+        e = sddmm_u_add_v.apply(graph, el, er, s_el, s_er)          # :141
         a = edge_softmax(graph, e, negative_slope=self.negative_slope)  # LeakyReLU :144 + softmax :146
         a = self.attn_drop(a)
         # without a residual branch the bias add (:160-162) rides in the aggregation's epilogue

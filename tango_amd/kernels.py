@@ -582,8 +582,10 @@ class cuda_kernels:
 
     # ------------------------------------------------- GAT attention logits
     @staticmethod
-    def attn_scores_forward(feat, attn_l, attn_r):
-        """el, er [n, H] from feat [n, H, D] and attn_l, attn_r [H, D] (evaluation/test_gat.py:135-137)."""
+    def attn_scores_forward(feat, attn_l, attn_r, want_scales=False):
+        """el, er [n, H] from feat [n, H, D] and attn_l, attn_r [H, D] (evaluation/test_gat.py:135-137).
+        ``want_scales``: also return max|el| / 127 and max|er| / 127 (1-element tensors, or None while the
+        stream is being captured), found by the same kernel."""
         for t, nm in ((feat, "feat"), (attn_l, "attn_l"), (attn_r, "attn_r")):
             _need(t, torch.float32, nm)
         n, H, D = feat.shape
@@ -591,9 +593,13 @@ class cuda_kernels:
             raise RuntimeError("attn_scores: attn_l / attn_r must have H * D elements")
         el = torch.empty((n, H), dtype=torch.float32, device=feat.device)
         er = torch.empty((n, H), dtype=torch.float32, device=feat.device)
-        check(_L.tango_attn_scores_fwd(_ptr(el), _ptr(er), _ptr(feat), _ptr(attn_l), _ptr(attn_r), n, H, D,
-                                       _stream()), "attn_scores_forward")
-        return el, er
+        s_el = s_er = None
+        if want_scales:
+            s_el = _zero_slot(feat.device)
+            s_er = _zero_slot(feat.device) if s_el is not None else None
+        check(_L.tango_attn_scores_fwd(_ptr(el), _ptr(er), _ptr(s_el), _ptr(s_er), _ptr(feat), _ptr(attn_l),
+                                       _ptr(attn_r), n, H, D, _stream()), "attn_scores_forward")
+        return (el, er, s_el, s_er) if want_scales else (el, er)
 
     @staticmethod
     def attn_scores_backward(del_, der, feat, attn_l, attn_r):
