@@ -293,6 +293,13 @@ int tango_sddmm_ewise_i8(int op, float* out, float* scale_out, const int64_t* sr
                          const int64_t* dst, const int8_t* U, const int8_t* V, const float* sU,
                          const float* sV, int64_t num_edges, int64_t T, tango_stream_t stream);
 
+/* The same with fp32 U, V quantized as they are loaded (round_mode TANGO_ROUND_RNE or
+   TANGO_ROUND_TRUNC, scales sU, sV): what sddmm_u_add_v's two quantize calls followed by
+   mySDDMM_int8 compute (cuda/SDDMM.py:13-18), bit for bit, without the int8 copies. */
+int tango_sddmm_ewise_f32q(int op, float* out, const int64_t* src, const int64_t* dst, const float* U,
+                           const float* V, const float* sU, const float* sV, int64_t num_edges, int64_t T,
+                           int round_mode, tango_stream_t stream);
+
 /* ------------------------------------------------------------ edge softmax */
 
 /* LeakyReLU(slope) followed by softmax over the in-edges of every destination

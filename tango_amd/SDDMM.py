@@ -4,7 +4,8 @@ define (evaluation/test_HGT.py:58, evaluation/link_pred_gcn.py:145)."""
 from torch.autograd.function import Function, once_differentiable
 
 from . import config
-from .kernels import incidence_SPMM, multi_cusparse_SPMM, mySDDMM_int8, quantize
+from .kernels import (cuda_kernels, incidence_SPMM, multi_cusparse_SPMM, mySDDMM_int8, mySDDMM_quantize_on_load,
+                      quantize)
 
 
 def _quantize_grad(t):
@@ -15,16 +16,20 @@ def _quantize_grad(t):
 
 
 class sddmm_u_add_v(Function):
-    """out[e] = U[src[e]] + V[dst[e]] on int8-quantized U, V (cuda/SDDMM.py:10-32)."""
+    """out[e] = U[src[e]] + V[dst[e]] on int8-quantized U, V (cuda/SDDMM.py:10-32).  Nothing else reads the
+    int8 copies of U and V (the backward pass needs only the graph), so they are never stored: the kernel
+    rounds the fp32 values with the two scales as it gathers them, which gives the same result bit for bit."""
 
     @staticmethod
     def forward(ctx, g, U, V, scaleU_=None, scaleV_=None):
-        U_, scaleU = quantize(U if U.is_contiguous() else U.contiguous(), scaleU_)
+        U = U if U.is_contiguous() else U.contiguous()
+        scaleU = cuda_kernels.get_scale(U) if scaleU_ is None else scaleU_
         if id(U) == id(V):
-            V_, scaleV = U_, scaleU
+            V, scaleV = U, scaleU
         else:
-            V_, scaleV = quantize(V if V.is_contiguous() else V.contiguous(), scaleV_)
-        out, _ = mySDDMM_int8(g, "add", U_, V_, scaleU, scaleV, False)
+            V = V if V.is_contiguous() else V.contiguous()
+            scaleV = cuda_kernels.get_scale(V) if scaleV_ is None else scaleV_
+        out = mySDDMM_quantize_on_load(g, "add", U, V, scaleU, scaleV)
         ctx.backward_cache = g
         return out
 

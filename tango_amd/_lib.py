@@ -53,6 +53,7 @@ SIGNATURES = {
     "tango_spmm_incidence": (I, [P, P, P, P, P, I64, I64, I64, I64, P]),
     "tango_sddmm_dot_i8": (I, [P, P, P, P, P, P, P, P, I64, I64, I64, P]),
     "tango_sddmm_ewise_i8": (I, [I, P, P, P, P, P, P, P, P, I64, I64, P]),
+    "tango_sddmm_ewise_f32q": (I, [I, P, P, P, P, P, P, P, I64, I64, I, P]),
     "tango_softmax_xent_workspace": (SZ, [I64]),
     "tango_softmax_xent_f32": (I, [P, I64, P, I64, I64, P, P, I64, P, SZ, P]),
     "tango_edge_softmax_workspace": (SZ, [I64, I64]),

@@ -136,6 +136,40 @@ __global__ __launch_bounds__(256) void sddmm_ewise_kernel(
     if (REDUCE) block_absmax_to_global(m / 127.0f, scale_out);
 }
 
+// As sddmm_ewise_kernel with fp32 operands quantized as they are loaded (round to nearest even or
+// truncation with the given scales): the same int8 values a separate quantize pass would have stored, so
+// the same result, without that pass and its int8 copies.
+template <int OP, int VEC, int MODE>
+__global__ __launch_bounds__(256) void sddmm_ewise_f32q_kernel(
+    float* __restrict__ out, const int64_t* __restrict__ src, const int64_t* __restrict__ dst,
+    const float* __restrict__ U, const float* __restrict__ V, const float* __restrict__ sU,
+    const float* __restrict__ sV, int64_t E, int64_t T) {
+    const float su = sU[0], sv = sV[0];
+    const float ru = rscale_of(su), rv = rscale_of(sv);
+    const int64_t per = T / VEC;  // VEC divides T
+    const int64_t total = E * per;
+    const int64_t nthr = static_cast<int64_t>(gridDim.x) * blockDim.x;
+    for (int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < total; i += nthr) {
+        const int64_t e = i / per;
+        const int64_t t = (i - e * per) * VEC;
+        const float* u = U + src[e] * T + t;
+        const float* v = V + dst[e] * T + t;
+        if (VEC == 4) {
+            const f32x4 a = *reinterpret_cast<const f32x4*>(u);
+            const f32x4 b = *reinterpret_cast<const f32x4*>(v);
+            f32x4 y;
+#pragma unroll
+            for (int k = 0; k < 4; ++k)
+                y[k] = apply_op<OP>(static_cast<float>(quant_one<MODE>(a[k], ru, 0.0f)) * su,
+                                    static_cast<float>(quant_one<MODE>(b[k], rv, 0.0f)) * sv);
+            __builtin_nontemporal_store(y, reinterpret_cast<f32x4*>(out + e * T + t));
+        } else {
+            out[e * T + t] = apply_op<OP>(static_cast<float>(quant_one<MODE>(u[0], ru, 0.0f)) * su,
+                                          static_cast<float>(quant_one<MODE>(v[0], rv, 0.0f)) * sv);
+        }
+    }
+}
+
 }  // namespace tango
 
 using namespace tango;
@@ -219,6 +253,43 @@ int tango_sddmm_ewise_i8(int op, float* out, float* scale_out, const int64_t* sr
     }
 #undef TANGO_EW_OP
 #undef TANGO_EW
+    return launch_status();
+}
+
+int tango_sddmm_ewise_f32q(int op, float* out, const int64_t* src, const int64_t* dst, const float* U,
+                           const float* V, const float* sU, const float* sV, int64_t num_edges, int64_t T,
+                           int round_mode, tango_stream_t stream) {
+    if (op < TANGO_OP_ADD || op > TANGO_OP_DIV) return TANGO_ERR_UNSUPPORTED;
+    if (round_mode != TANGO_ROUND_RNE && round_mode != TANGO_ROUND_TRUNC) return TANGO_ERR_UNSUPPORTED;
+    if (num_edges < 0 || T < 0 || !sU || !sV || (num_edges * T > 0 && (!out || !src || !dst || !U || !V)))
+        return TANGO_ERR_INVALID_ARG;
+    if (num_edges * T == 0) return TANGO_OK;
+    const uintptr_t al = reinterpret_cast<uintptr_t>(U) | reinterpret_cast<uintptr_t>(V) |
+                         reinterpret_cast<uintptr_t>(out);
+    const bool v4 = (T & 3) == 0 && (al & 15) == 0;
+    const dim3 grid(grid_for(num_edges * (v4 ? T / 4 : T), 256, 16)), block(256);
+    hipStream_t s = as_stream(stream);
+#define TANGO_EWQ(OP_, V_, M_)                                                                              \
+    hipLaunchKernelGGL((sddmm_ewise_f32q_kernel<OP_, V_, M_>), grid, block, 0, s, out, src, dst, U, V, sU, \
+                       sV, num_edges, T)
+#define TANGO_EWQ_OP(OP_)                                                      \
+    do {                                                                       \
+        if (round_mode == TANGO_ROUND_RNE) {                                   \
+            if (v4) TANGO_EWQ(OP_, 4, TANGO_ROUND_RNE);                        \
+            else TANGO_EWQ(OP_, 1, TANGO_ROUND_RNE);                           \
+        } else {                                                               \
+            if (v4) TANGO_EWQ(OP_, 4, TANGO_ROUND_TRUNC);                      \
+            else TANGO_EWQ(OP_, 1, TANGO_ROUND_TRUNC);                         \
+        }                                                                      \
+    } while (0)
+    switch (op) {
+        case TANGO_OP_ADD: TANGO_EWQ_OP(TANGO_OP_ADD); break;
+        case TANGO_OP_SUB: TANGO_EWQ_OP(TANGO_OP_SUB); break;
+        case TANGO_OP_MUL: TANGO_EWQ_OP(TANGO_OP_MUL); break;
+        default: TANGO_EWQ_OP(TANGO_OP_DIV); break;
+    }
+#undef TANGO_EWQ_OP
+#undef TANGO_EWQ
     return launch_status();
 }
 

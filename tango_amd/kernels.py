@@ -550,6 +550,23 @@ class cuda_kernels:
             # the reference only prints "op not supported" (cuda/src/SDDMM.cu:175)
             raise ValueError("%s op not supported" % op)
 
+    @staticmethod
+    def mySDDMM_quantize_on_load(op, out, src, dst, U, V, scaleU, scaleV, round_mode=ROUND_RNE):
+        """mySDDMM_int8 for add / sub / mul / div on fp32 U, V that the kernel quantizes as it loads them."""
+        for t, nm in ((out, "out"), (U, "U"), (V, "V"), (scaleU, "scaleU"), (scaleV, "scaleV")):
+            _need(t, torch.float32, nm)
+        _need(src, torch.int64, "src")
+        _need(dst, torch.int64, "dst")
+        if op not in SDDMM_OPS:
+            raise ValueError("%s op not supported" % op)
+        E = src.numel()
+        T = math.prod(U.shape[1:])
+        if dst.numel() != E or U.shape[1:] != V.shape[1:] or out.numel() != E * T:
+            raise RuntimeError("mySDDMM_quantize_on_load: shape mismatch")
+        check(_L.tango_sddmm_ewise_f32q(SDDMM_OPS[op], _ptr(out), _ptr(src), _ptr(dst), _ptr(U), _ptr(V),
+                                        scaleU.data_ptr(), scaleV.data_ptr(), E, T, _mode(round_mode), _stream()),
+              "mySDDMM_quantize_on_load(%s)" % op)
+
     # ---------------------------------------------------------- edge softmax
     @staticmethod
     def edge_softmax_forward(e, indptr, edge_ids, slope=1.0):
@@ -698,6 +715,17 @@ def QGEMM_forward(x, x_, scaleX, w, w_, scaleW, bias=None, isReduce=False, round
     if isReduce:
         return out_fp, scale_out
     return out_fp
+
+
+def mySDDMM_quantize_on_load(g, op, U, V, scaleU, scaleV, round_mode=ROUND_RNE):
+    """``mySDDMM_int8(g, op, quantize(U, scaleU)[0], quantize(V, scaleV)[0], scaleU, scaleV, False)[0]`` for
+    add / sub / mul / div without the two quantize passes: the kernel rounds the fp32 values as it gathers them."""
+    src, dst = g.coo
+    U3, V3 = (U.unsqueeze(1), V.unsqueeze(1)) if U.dim() == 2 and V.dim() == 2 else (U, V)
+    out_shape = (src.size(0),) + infer_broadcast_shape(op, U3.shape[1:], V3.shape[1:])
+    out = torch.empty(out_shape, dtype=torch.float32, device=src.device)
+    cuda_kernels.mySDDMM_quantize_on_load(op, out, src, dst, U3, V3, scaleU, scaleV, round_mode)
+    return out.squeeze(1) if U3 is not U else out
 
 
 def QGEMM_backward(dY, X, W, scaledY, scaleX, scaleW, X_need=True, W_need=True, x_row_scale=None, dX_acc=None):

@@ -75,6 +75,32 @@ def test_elementwise(K, orc, op, shape):
     assert host(so)[0] == wso
 
 
+@pytest.mark.parametrize("mode", ["rne", "trunc"])
+@pytest.mark.parametrize("op", ["add", "sub", "mul", "div"])
+@pytest.mark.parametrize("shape", [(8, 1), (3,), (1, 5), (16,)])
+def test_elementwise_quantizing_on_load(K, orc, op, shape, mode):
+    """fp32 operands rounded by the SDDMM kernel as it gathers them == the oracle's quantize followed by its
+    element-wise SDDMM, bit for bit, including values that clamp (|x| above 127 scale) and an all-zero scale."""
+    rng = np.random.default_rng(len(shape) + sum(shape) + len(op))
+    n, e = 700, 20011
+    src, dst = rand_graph(rng, n, e)
+    g = make_graph(src, dst, n)
+    U = (rng.standard_normal((n,) + shape) * 3).astype(np.float32)
+    V = (np.abs(rng.standard_normal((n,) + shape)) + 0.5).astype(np.float32)  # rounds to >= 10: no zero divisors
+    sU, sV = np.float32(np.abs(U).max() / 127 * 0.8), np.float32(np.abs(V).max() / 127)
+    omode = orc.RNE if mode == "rne" else orc.TRUNC
+    Uq, Vq = orc.quantize(U, sU, omode).reshape(n, -1), orc.quantize(V, sV, omode).reshape(n, -1)
+    assert np.abs(Vq).min() > 0 and np.abs(Uq).max() == 127
+    want, _ = orc.sddmm_ewise(op, src, dst, Uq, Vq, sU, sV)
+    out = K.mySDDMM_quantize_on_load(g, op, dev(U), dev(V), sc(sU), sc(sV), round_mode=mode)
+    assert tuple(out.shape) == (e,) + shape
+    assert np.array_equal(host(out).reshape(e, -1), want)
+    if op == "add":  # a tensor of zeros has scale 0 and quantizes to zeros
+        out0 = K.mySDDMM_quantize_on_load(g, op, dev(np.zeros_like(U)), dev(V), sc(0.0), sc(sV), round_mode=mode)
+        want0, _ = orc.sddmm_ewise(op, src, dst, np.zeros_like(Uq), Vq, np.float32(0), sV)
+        assert np.array_equal(host(out0).reshape(e, -1), want0)
+
+
 def test_unknown_op_raises(K):
     g = make_graph(np.array([0], np.int64), np.array([0], np.int64), 1)
     z = torch.zeros((1, 4), dtype=torch.int8, device="cuda")
