@@ -155,6 +155,19 @@ int tango_qgemm_fwd_ex(float* Y, int64_t ldy, const float* X, int64_t ldx, const
    sustains.  sink: one int of device memory (practically never written). */
 int tango_probe_mfma_i8(int64_t workgroups, int64_t iters, int* sink, tango_stream_t stream);
 
+/* Forward linear whose output is read only by another quantized op (the first of two chained
+   QLinear layers, evaluation/test_HGT.py:51-55): instead of the fp32 Y that cuda/QLinear.py:30-36
+   stores and the next layer's quantize reads back, the int8 Yq = quantize(Y, scaleY) and
+   scaleY[0] = max|Y| / 127 themselves.  The product is formed twice (first for its absmax, then
+   rounded with it); same bits as tango_qgemm_fwd followed by a quantize pass.  Xq is the
+   already quantized input (16-byte aligned rows); K <= 256, round_mode RNE or TRUNC (used for W
+   and for Yq), else TANGO_ERR_UNSUPPORTED before anything is launched.  Workspace as
+   tango_qgemm_fwd. */
+int tango_qgemm_fwd_q8(int8_t* Yq, int64_t ldyq, float* scaleY, const int8_t* Xq, int64_t ldxq,
+                       const float* W, int64_t ldw, int8_t* Wq, const float* bias, const float* scaleX,
+                       const float* scaleW, int64_t M, int64_t N, int64_t K, int round_mode,
+                       void* workspace, size_t workspace_bytes, tango_stream_t stream);
+
 /* Integer GEMM on operands that are already int8 (no counterpart in the
    reference, whose forward always re-quantizes; same epilogue as above):
    Y[m,n] = (sA*sB) * float(sum_k A[m,k]*B[n,k]) (+ bias[n]), optional scaleY. */

@@ -137,27 +137,47 @@ class Qlinear_func_reduce(Function):
 
 class Qlinear_shared_func(Function):
     """Several linear layers over one input (the k / v / q projections of evaluation/test_HGT.py:51-53)
-    as one autograd node: ``apply(X, Xq, scaleX, W_0, b_0, W_1, b_1, ...)`` with (Xq, scaleX) from
-    ``quantize_input(X)`` returns (Y_0, scale_0, Y_1, scale_1, ...), each pair what Qlinear_func_reduce
-    returns.  Backward runs each layer's weight / bias gradient as usual, and the input gradients go into
+    as one autograd node: ``apply(X, Xq, scaleX, n, W_0, b_0, ..., W_n-1, b_n-1, V_0, c_0, ...)`` with
+    (Xq, scaleX) from ``quantize_input(X)`` returns (Y_0, scale_0, Y_1, scale_1, ...), each pair what
+    Qlinear_func_reduce returns; where (V_i, c_i) is not (None, None), Y_i is that second layer applied to the
+    first one's output (evaluation/test_HGT.py:54-55), which is then kept in int8 only.  Backward runs each layer's weight / bias gradient as usual, and the input gradients go into
     one tensor: the first layer's GEMM writes it, the others add to it in their epilogues, where autograd
     would run a separate addition per extra layer over three [M, K] fp32 tensors."""
 
     @staticmethod
-    def forward(ctx, X, Xq, scaleX, *wb):
-        if len(wb) == 0 or len(wb) % 2:
-            raise RuntimeError("Qlinear_shared_func: expects (weight, bias) pairs")
+    def forward(ctx, X, Xq, scaleX, n_first, *wb):
+        """``wb``: (W, b) of the ``n_first`` layers applied to X, then (W2, b2) or (None, None) per layer:
+        a second linear layer applied to that layer's output, which then is the only reader of it."""
+        if n_first < 1 or len(wb) != 4 * n_first:
+            raise RuntimeError("Qlinear_shared_func: expects (weight, bias) of every layer and of its follower")
         if tuple(Xq.shape) != tuple(X.shape) or Xq.dtype != torch.int8 or X.dim() != 2:
             raise RuntimeError("Qlinear_shared_func: the quantized input must be int8 of the 2-D input's shape")
         ctx.set_materialize_grads(False)
         outs, layers = [], []
-        for W, b in zip(wb[0::2], wb[1::2]):
-            scaleW = kernels.cuda_kernels.get_scale(W if W.is_contiguous() else W.contiguous())
+        get_scale = kernels.cuda_kernels.get_scale
+        for i in range(n_first):
+            W, b = wb[2 * i], wb[2 * i + 1]
+            W2, b2 = wb[2 * n_first + 2 * i], wb[2 * n_first + 2 * i + 1]
+            scaleW = get_scale(W if W.is_contiguous() else W.contiguous())
             W_ = torch.empty(W.shape, dtype=torch.int8, device=X.device)
-            out, scaleO = kernels.QGEMM_forward(None, Xq, scaleX, W, W_, scaleW, b, True)
+            second = None
+            if W2 is None:
+                out, scaleO = kernels.QGEMM_forward(None, Xq, scaleX, W, W_, scaleW, b, True)
+            else:
+                # the first layer's output in int8 only (nothing but the second layer reads it), where the
+                # kernel for that applies; else in fp32 and quantized by the second GEMM as usual
+                Yq = _padded_i8(X.size(0), W.size(0), X.device)
+                sY = torch.empty_like(scaleX)
+                Y = None
+                if not kernels.cuda_kernels.QGEMM_forward_q8(Yq, sY, Xq, W, W_, b, scaleX, scaleW):
+                    Y, sY = kernels.QGEMM_forward(None, Xq, scaleX, W, W_, scaleW, b, True)
+                scaleW2 = get_scale(W2 if W2.is_contiguous() else W2.contiguous())
+                W2_ = torch.empty(W2.shape, dtype=torch.int8, device=X.device)
+                out, scaleO = kernels.QGEMM_forward(Y, Yq, sY, W2, W2_, scaleW2, b2, True)
+                second = (Yq, sY, W2_, scaleW2, b2 is not None)
             ctx.mark_non_differentiable(scaleO)
             outs += [out, scaleO]
-            layers.append((W_, scaleW, b is not None))
+            layers.append((W_, scaleW, b is not None, second))
         ctx.backward_cache = Xq, scaleX, layers
         return tuple(outs)
 
@@ -165,28 +185,37 @@ class Qlinear_shared_func(Function):
     @once_differentiable
     def backward(ctx, *grads):
         Xq, scaleX, layers = ctx.backward_cache
-        dX, rest = None, []
-        for i, (W_, scaleW, has_bias) in enumerate(layers):
+        n = len(layers)
+        need = ctx.needs_input_grad
+        dX, first, second = None, [None] * (2 * n), [None] * (2 * n)
+        for i, (W_, scaleW, has_bias, chained) in enumerate(layers):
             dY = grads[2 * i]
             if dY is None:
-                rest += [None, None]
                 continue
-            want_bias = has_bias and ctx.needs_input_grad[4 + 2 * i]
-            dY_, scaledY, grad_bias = _quantize_grad(dY, want_bias)
-            dXi, dW = kernels.QGEMM_backward(dY_, Xq, W_, scaledY, scaleX, scaleW, ctx.needs_input_grad[0],
-                                             ctx.needs_input_grad[3 + 2 * i], dX_acc=dX)
+            if chained is not None:  # back through the second layer to the first layer's output
+                Yq, sY, W2_, scaleW2, has_bias2 = chained
+                dY_, scaledY, second[2 * i + 1] = _quantize_grad(dY, has_bias2 and need[4 + 2 * n + 2 * i + 1])
+                dY, second[2 * i] = kernels.QGEMM_backward(dY_, Yq, W2_, scaledY, sY, scaleW2, True,
+                                                           need[4 + 2 * n + 2 * i])
+            dY_, scaledY, first[2 * i + 1] = _quantize_grad(dY, has_bias and need[4 + 2 * i + 1])
+            dXi, first[2 * i] = kernels.QGEMM_backward(dY_, Xq, W_, scaledY, scaleX, scaleW, need[0], need[4 + 2 * i],
+                                                       dX_acc=dX)
             dX = dXi if dXi is not None else dX
-            rest += [dW, grad_bias]
-        return (dX, None, None) + tuple(rest)
+        return (dX, None, None, None) + tuple(first) + tuple(second)
 
 
-def shared_input_linears(X, layers, scaleX=None):
+def shared_input_linears(X, layers, scaleX=None, then=None):
     """[(Y, scale of Y)] of the QLinear ``layers`` applied to one 2-D input: X is quantized once and the
-    layers run as one autograd node (Qlinear_shared_func)."""
+    layers run as one autograd node (Qlinear_shared_func).  ``then``: per layer, None or a second QLinear
+    applied to that layer's output (``then[i](layers[i](X))``); the pair returned is the second layer's."""
     Xq, scaleX = quantize_input(X, scaleX)
     X = X if X.is_contiguous() else X.contiguous()
+    then = [None] * len(layers) if then is None else list(then)
+    if len(then) != len(layers):
+        raise RuntimeError("shared_input_linears: one entry of `then` per layer")
     flat = [t for lin in layers for t in (lin.weight, lin.bias)]
-    res = Qlinear_shared_func.apply(X, Xq, scaleX, *flat)
+    flat += [t for lin in then for t in ((lin.weight, lin.bias) if lin is not None else (None, None))]
+    res = Qlinear_shared_func.apply(X, Xq, scaleX, len(layers), *flat)
     return [(res[2 * i], res[2 * i + 1]) for i in range(len(layers))]
 
 

@@ -37,6 +37,7 @@ SIGNATURES = {
     "tango_qgemm_i8_nt": (I, [P, I64, P, I64, P, I64, P, P, P, P, I64, I64, I64, P, SZ, P]),
     "tango_qgemm_bwd_dx_workspace": (SZ, [I64, I64, I64]),
     "tango_qgemm_bwd_dx": (I, [P, I64, P, I64, P, I64, P, P, I64, I64, I64, P, SZ, P]),
+    "tango_qgemm_fwd_q8": (I, [P, I64, P, P, I64, P, I64, P, P, P, P, I64, I64, I64, I, P, SZ, P]),
     "tango_qgemm_bwd_dx_ex": (I, [P, I64, P, I64, P, I64, P, P, P, I, I64, I64, I64, P, SZ, P]),
     "tango_qgemm_bwd_dw_workspace": (SZ, [I64, I64, I64]),
     "tango_qgemm_bwd_dw": (I, [P, I64, P, I64, P, I64, P, P, I64, I64, I64, P, SZ, P]),

@@ -61,6 +61,10 @@ struct NtParams {
     int64_t lda, ldb, ldc;
     int64_t a_row_bytes; // bytes that may be read from each row of A (>= Kr)
     int accumulate;      // nonzero: the product is added to what C holds (gradients of one tensor from several layers)
+    int8_t* Cq;          // stationary form with an int8 epilogue: [M, N] int8, row stride ldcq
+    int64_t ldcq;
+    const float* q_scale;  // the scale Cq is rounded with
+    int q_mode;          // TANGO_ROUND_RNE or TANGO_ROUND_TRUNC
 };
 
 // Workgroup = 4 waves = 128 rows x (16 * NT) columns.  gridDim = (ceil(M/128), ceil(N/(16 NT))).
@@ -212,7 +216,10 @@ __global__ __launch_bounds__(256, 2) void gemm_nt_kernel(const NtParams p) {
 // one L2 round trip per k-step (several microseconds under load) in every workgroup; here the only
 // global loads are the A tiles, requested one tile ahead, so loads, MFMAs and the output stores of the
 // sixteen waves of a CU overlap.
-template <int NT, int VEC, int WAVES>
+// EPI 0: the tile goes to C as fp32.  EPI 1: nothing is stored, only max|C| / 127 is found.  EPI 2: the tile
+// is rounded to int8 with the scale q_scale and goes to Cq (the fp32 values are the same in all three, so
+// 1 then 2 store exactly what a quantize pass over the fp32 output of 0 would).
+template <int NT, int VEC, int WAVES, int EPI = 0>
 __global__ __launch_bounds__(64 * WAVES) void gemm_nts_kernel(const NtParams p, int ntiles, int pitch) {
     extern __shared__ __attribute__((aligned(16))) int8_t b_lds[];  // [16 NT][pitch]
     constexpr int KS = 4;
@@ -239,6 +246,8 @@ __global__ __launch_bounds__(64 * WAVES) void gemm_nts_kernel(const NtParams p, 
     const float s = p.sA[0] * p.sB[0];
     const uintptr_t ca = reinterpret_cast<uintptr_t>(p.C);
     const int wide = ((ca & 15) == 0 && (p.ldc & 3) == 0) ? 4 : ((ca & 7) == 0 && (p.ldc & 1) == 0) ? 2 : 1;
+    const float qr = EPI == 2 ? rscale_of(p.q_scale[0]) : 0.0f;
+    const bool qwide = EPI == 2 && (reinterpret_cast<uintptr_t>(p.Cq) & 3) == 0 && (p.ldcq & 3) == 0;
     float m = 0.0f;
     auto load_tile = [&](i32x4* a, float& rsc, int t) {
         const int64_t row = static_cast<int64_t>(t) * 16 + r16;
@@ -287,6 +296,23 @@ __global__ __launch_bounds__(64 * WAVES) void gemm_nts_kernel(const NtParams p, 
                     if (p.row_scale) y[v] = y[v] * rsc;
                     if (p.bias) y[v] = bv[v] + y[v];
                     if (col + v < p.N) m = fmaxf(m, fabsf(y[v]));
+                }
+                if (EPI == 1) continue;
+                if (EPI == 2) {
+                    int q[4];
+#pragma unroll
+                    for (int v = 0; v < 4; ++v)
+                        q[v] = p.q_mode == TANGO_ROUND_TRUNC ? quant_one<TANGO_ROUND_TRUNC>(y[v], qr, 0.0f)
+                                                             : quant_one<TANGO_ROUND_RNE>(y[v], qr, 0.0f);
+                    int8_t* qrow = p.Cq + row * p.ldcq;
+                    if (col + 4 <= p.N && qwide) {
+                        *reinterpret_cast<uint32_t*>(qrow + col) = pack4(q[0], q[1], q[2], q[3]);
+                    } else {
+#pragma unroll
+                        for (int v = 0; v < 4; ++v)
+                            if (col + v < p.N) qrow[col + v] = static_cast<int8_t>(q[v]);
+                    }
+                    continue;
                 }
                 if (p.accumulate) {  // uniform
                     if (col + 4 <= p.N && wide == 4) {
@@ -983,6 +1009,38 @@ static int row_vec(const int8_t* p, int64_t ld, int64_t cols, int64_t* readable)
     return 1;
 }
 
+// The stationary form (reduction <= 256, A rows readable in 4- or 16-byte pieces).  EPI: what the epilogue does
+// with the dequantized tile (see gemm_nts_kernel).  False when the launch could not be set up.
+template <int VEC, int EPI>
+static bool launch_nts(const NtParams& p, hipStream_t s) {
+    constexpr int WAVES = 12;
+    const int64_t n16 = ceil_div(p.N, 16);
+    const int ny = static_cast<int>(ceil_div(n16, 16));
+    const int nt = static_cast<int>(ceil_div(n16, ny));
+    const int pitch = 16 * ((static_cast<int>(ceil_div(p.Kr, 64)) * 4) | 1);
+    const int ntiles = static_cast<int>(ceil_div(p.M, 16));
+    int gx = compute_units() / ny;
+    if (gx > ceil_div(ntiles, WAVES)) gx = static_cast<int>(ceil_div(ntiles, WAVES));
+    if (gx < 1) gx = 1;
+#define TANGO_NTS(NT_)                                                                                          \
+    do {                                                                                                        \
+        /* more than 64 KB of dynamic LDS has to be asked for once per kernel */                                \
+        static const bool ok =                                                                                  \
+            hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_nts_kernel<NT_, VEC, WAVES, EPI>),          \
+                                hipFuncAttributeMaxDynamicSharedMemorySize, 80 * 1024) == hipSuccess;           \
+        if (!ok) return false;                                                                                  \
+        hipLaunchKernelGGL((gemm_nts_kernel<NT_, VEC, WAVES, EPI>), dim3(gx, ny), dim3(64 * WAVES),             \
+                           static_cast<size_t>(16 * NT_) * (pitch + 4), s, p, ntiles, pitch);                   \
+        return true;                                                                                            \
+    } while (0)
+    if (nt <= 2) TANGO_NTS(2);
+    else if (nt <= 4) TANGO_NTS(4);
+    else if (nt <= 8) TANGO_NTS(8);
+    else if (nt <= 13) TANGO_NTS(13);
+    else TANGO_NTS(16);
+#undef TANGO_NTS
+}
+
 template <int VEC>
 static void launch_nt_vec(const NtParams& p, hipStream_t s) {
     const int64_t n16 = ceil_div(p.N, 16);
@@ -991,31 +1049,7 @@ static void launch_nt_vec(const NtParams& p, hipStream_t s) {
     hipLaunchKernelGGL((gemm_nt_kernel<NT_, VEC>), dim3(gx, static_cast<unsigned>(ceil_div(n16, NT_))), \
                        dim3(256), 0, s, p)
     if (p.Kr <= 256 && VEC != 1) {  // the small operand fits LDS: the stationary form
-        constexpr int WAVES = 12;
-        const int ny = static_cast<int>(ceil_div(n16, 16));
-        const int nt = static_cast<int>(ceil_div(n16, ny));
-        const int pitch = 16 * ((static_cast<int>(ceil_div(p.Kr, 64)) * 4) | 1);
-        const int ntiles = static_cast<int>(ceil_div(p.M, 16));
-        int gx = compute_units() / ny;
-        if (gx > ceil_div(ntiles, WAVES)) gx = static_cast<int>(ceil_div(ntiles, WAVES));
-        if (gx < 1) gx = 1;
-#define TANGO_NTS(NT_)                                                                                          \
-    do {                                                                                                        \
-        /* more than 64 KB of dynamic LDS has to be asked for once per kernel */                                \
-        static const bool ok = hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_nts_kernel<NT_, VEC, WAVES>), \
-                                                   hipFuncAttributeMaxDynamicSharedMemorySize, 80 * 1024) == hipSuccess; \
-        if (ok) {                                                                                               \
-            hipLaunchKernelGGL((gemm_nts_kernel<NT_, VEC, WAVES>), dim3(gx, ny), dim3(64 * WAVES),               \
-                               static_cast<size_t>(16 * NT_) * (pitch + 4), s, p, ntiles, pitch);               \
-            return;                                                                                             \
-        }                                                                                                       \
-    } while (0)
-        if (nt <= 2) TANGO_NTS(2);
-        else if (nt <= 4) TANGO_NTS(4);
-        else if (nt <= 8) TANGO_NTS(8);
-        else if (nt <= 13) TANGO_NTS(13);
-        else TANGO_NTS(16);
-#undef TANGO_NTS
+        if (launch_nts<VEC == 1 ? 4 : VEC, 0>(p, s)) return;
     }
     if (n16 <= 1) TANGO_NT(1);
     else if (n16 <= 2) TANGO_NT(2);
@@ -1197,6 +1231,45 @@ int tango_qgemm_fwd_ex(float* Y, int64_t ldy, const float* X, int64_t ldx, const
     p.C = Y; p.A = Xq; p.B = Bp; p.bias = bias; p.absmax_out = scaleY; p.sA = scaleX; p.sB = scaleW;
     p.M = M; p.N = N; p.Kr = K; p.lda = ldxq; p.ldb = ldb; p.ldc = ldy;
     return launch_nt(p, s, true);
+}
+
+int tango_qgemm_fwd_q8(int8_t* Yq, int64_t ldyq, float* scaleY, const int8_t* Xq, int64_t ldxq, const float* W,
+                       int64_t ldw, int8_t* Wq, const float* bias, const float* scaleX, const float* scaleW,
+                       int64_t M, int64_t N, int64_t K, int round_mode, void* workspace, size_t workspace_bytes,
+                       tango_stream_t stream) {
+    if (M < 0 || N < 0 || K < 0 || !scaleX || !scaleW || !scaleY || ldyq < N || ldw < K || ldxq < K)
+        return TANGO_ERR_INVALID_ARG;
+    if ((M * N > 0 && !Yq) || (M * K > 0 && !Xq) || (N * K > 0 && (!W || !Wq))) return TANGO_ERR_INVALID_ARG;
+    if (round_mode != TANGO_ROUND_RNE && round_mode != TANGO_ROUND_TRUNC) return TANGO_ERR_UNSUPPORTED;
+    if (K < 1 || K > 256 || ceil_div(M, 16) > INT32_MAX) return TANGO_ERR_UNSUPPORTED;  // the stationary form only
+    int64_t readable = 0;
+    if (M > 0 && row_vec(Xq, ldxq, K, &readable) != 16) return TANGO_ERR_UNSUPPORTED;
+    const size_t need = tango_qgemm_fwd_workspace(M, N, K);
+    if (need > 0 && (!workspace || workspace_bytes < need)) return TANGO_ERR_WORKSPACE;
+    if ((reinterpret_cast<uintptr_t>(workspace) & 15) != 0) return TANGO_ERR_INVALID_ARG;
+    hipStream_t s = as_stream(stream);
+    int8_t* Bp = static_cast<int8_t*>(workspace);
+    const int64_t ldb = round_up(K, 64);
+    if (N > 0) {  // W -> Wq and its packed copy, and the zeroing of scaleY, in one launch
+        const dim3 wgrid(grid_for(N * ldb, 256));
+        if (round_mode == TANGO_ROUND_RNE)
+            hipLaunchKernelGGL(quantize_pack_w_kernel<TANGO_ROUND_RNE>, wgrid, dim3(256), 0, s, W, ldw, scaleW, Wq, Bp,
+                               ldb, N, K, scaleY);
+        else
+            hipLaunchKernelGGL(quantize_pack_w_kernel<TANGO_ROUND_TRUNC>, wgrid, dim3(256), 0, s, W, ldw, scaleW, Wq, Bp,
+                               ldb, N, K, scaleY);
+    } else {
+        fill_u32(scaleY, 0u, 1, s);
+    }
+    if (M == 0 || N == 0) return launch_status();
+    NtParams p{};
+    p.A = Xq; p.B = Bp; p.bias = bias; p.absmax_out = scaleY; p.sA = scaleX; p.sB = scaleW;
+    p.M = M; p.N = N; p.Kr = K; p.lda = ldxq; p.ldb = ldb; p.a_row_bytes = readable;
+    // the product twice: first only its absmax, then, with the scale known, rounded straight to int8
+    if (!launch_nts<16, 1>(p, s)) return TANGO_ERR_UNSUPPORTED;
+    p.absmax_out = nullptr; p.Cq = Yq; p.ldcq = ldyq; p.q_scale = scaleY; p.q_mode = round_mode;
+    if (!launch_nts<16, 2>(p, s)) return TANGO_ERR_UNSUPPORTED;
+    return launch_status();
 }
 
 int tango_probe_mfma_i8(int64_t workgroups, int64_t iters, int* sink, tango_stream_t stream) {

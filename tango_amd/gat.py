@@ -161,9 +161,10 @@ class HGTLayer(nn.Module):
         ``return_scale``: also return this layer's output scale for the next layer."""
         # one absmax (unless handed in) and one quantize pass for the three projections of h, and one input
         # gradient that their backward GEMMs accumulate into
-        (k, s_k), (v, s_v), (q, s_q) = shared_input_linears(h, (self.k_linear, self.v_linear, self.q_linear), s_h)
-        k, s_k = self.attn_linear(k, s_k)
-        v, s_v = self.msg_linear(v, s_v)
+        # (attn_linear and msg_linear are the only readers of the k and v projections, which therefore exist
+        # in int8 only)
+        (k, s_k), (v, s_v), (q, s_q) = shared_input_linears(
+            h, (self.k_linear, self.v_linear, self.q_linear), s_h, then=(self.attn_linear, self.msg_linear, None))
         k, v, q = (t.view(-1, self.n_heads, self.d_k) for t in (k, v, q))
         t = sddmm_u_dot_v.apply(g, k, q, s_k, s_q, 1.0 / self.sqrt_dk)  # "/ sqrt_dk" folded into the scales
         attn = edge_softmax(g, t)

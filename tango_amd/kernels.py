@@ -327,6 +327,36 @@ class cuda_kernels:
                                  ws_bytes, _stream()), "QGEMM_forward")
 
     @staticmethod
+    def QGEMM_forward_q8(Y_q, scaleY, X_q, W, W_q, bias, scaleX, scaleW, round_mode=None):
+        """int8 Y_q = quantize(X W^T + bias) and scaleY = max|X W^T + bias| / 127 from the already quantized
+        X_q, without the fp32 product in memory.  Returns False (nothing launched) where the kernel does not
+        apply (reduction above 256, rows of X_q not 16-byte aligned, stochastic rounding)."""
+        _need(Y_q, torch.int8, "Y_q", contiguous=False)
+        _need(X_q, torch.int8, "X_q", contiguous=False)
+        _need(W, torch.float32, "W", contiguous=False)
+        _need(W_q, torch.int8, "W_q")
+        for t, nm in ((scaleY, "scaleY"), (scaleX, "scaleX"), (scaleW, "scaleW")):
+            _need(t, torch.float32, nm)
+        M, K = X_q.shape
+        N = W.size(0)
+        if W.size(1) != K or tuple(Y_q.shape) != (M, N) or W_q.numel() != N * K:
+            raise RuntimeError("QGEMM_forward_q8: shape mismatch")
+        if bias is not None:
+            _need(bias, torch.float32, "bias")
+            if bias.numel() != N:
+                raise RuntimeError("QGEMM_forward_q8: bias must have N elements")
+        mode = default_forward_round_mode() if round_mode is None else _mode(round_mode)
+        ws_bytes = _ws_bytes("tango_qgemm_fwd_workspace", M, N, K)
+        ws = _workspace(ws_bytes, X_q.device)
+        rc = _L.tango_qgemm_fwd_q8(_ptr(Y_q), _rows_view(Y_q, "Y_q"), scaleY.data_ptr(), _ptr(X_q),
+                                   _rows_view(X_q, "X_q"), _ptr(W), _rows_view(W, "W"), _ptr(W_q), _ptr(bias),
+                                   scaleX.data_ptr(), scaleW.data_ptr(), M, N, K, mode, _ptr(ws), ws_bytes, _stream())
+        if rc == -2:  # TANGO_ERR_UNSUPPORTED
+            return False
+        check(rc, "QGEMM_forward_q8")
+        return True
+
+    @staticmethod
     def QGEMM_i8(Y, A, B, bias, scaleY, scaleA, scaleB):
         """Y = dequant(A[M,K] . B[N,K]^T) on int8 operands (not in the reference)."""
         _need(Y, torch.float32, "Y", contiguous=False)

@@ -421,3 +421,37 @@ def test_shared_input_linears_accumulate_one_input_gradient(M, Kd, N):
         assert torch.equal(x.grad, want_dx)
         for p, w in zip(params, want_dp):
             assert (p.grad is None and w is None) or torch.equal(p.grad, w)
+
+
+@pytest.mark.parametrize("M,Kd,N,N2", [(3000, 256, 256, 256), (1000, 100, 41, 64), (700, 602, 300, 32), (50, 64, 16, 7)])
+def test_shared_input_linears_with_a_second_layer(M, Kd, N, N2):
+    """then=[second layer or None]: the node == the layers chained one by one (outputs, scales and every
+    gradient bit for bit, the input gradient added in layer order).  The first layer's output exists in int8
+    only where the kernel for that applies (reduction <= 256) and in fp32 otherwise (602)."""
+    from tango_amd.QLinear import QLinear, shared_input_linears
+    torch.manual_seed(M + N2)
+    firsts = [QLinear(Kd, N).cuda(), QLinear(Kd, N, bias=False).cuda(), QLinear(Kd, N).cuda()]
+    seconds = [QLinear(N, N2).cuda(), None, QLinear(N, N2, bias=False).cuda()]
+    for lin in firsts + [s for s in seconds if s is not None]:
+        lin.enable_reduce()
+    params = [p for lin in firsts + [s for s in seconds if s is not None] for p in lin.parameters()]
+    x = torch.randn(M, Kd, device="cuda", requires_grad=True)
+    ws = [torch.randn(M, N2 if s is not None else N, device="cuda") for s in seconds]
+    want_y, want_dx = [], None
+    want_dp = {}
+    for i, (lin, sec) in enumerate(zip(firsts, seconds)):
+        y, s = lin(x)
+        if sec is not None:
+            y, s = sec(y, s)
+        want_y.append((y.detach().clone(), s.clone()))
+        ps = list(lin.parameters()) + (list(sec.parameters()) if sec is not None else [])
+        g = torch.autograd.grad((y * ws[i]).sum(), [x] + ps)
+        want_dx = g[0] if want_dx is None else want_dx + g[0]
+        want_dp.update({id(p): gp for p, gp in zip(ps, g[1:])})
+    res = shared_input_linears(x, firsts, then=seconds)
+    sum((res[i][0] * ws[i]).sum() for i in range(3)).backward()
+    for (y, s), (wy, wsc) in zip(res, want_y):
+        assert torch.equal(y, wy) and torch.equal(s, wsc)
+    assert torch.equal(x.grad, want_dx)
+    for p in params:
+        assert torch.equal(p.grad, want_dp[id(p)])

@@ -205,6 +205,41 @@ def test_gradx_accumulates_into_its_output(K, M, N, Kd, rows):
     assert np.array_equal(host(out), prior + acc)
 
 
+@pytest.mark.parametrize("mode", ["rne", "trunc"])
+@pytest.mark.parametrize("M,N,Kd", [(40000, 256, 256), (3001, 41, 100), (16, 600, 64), (1, 16, 16)])
+def test_forward_gemm_with_int8_output(K, orc, M, N, Kd, mode):
+    """The forward GEMM that stores its output already quantized == the oracle's int8 GEMM, absmax scale and
+    quantize on the fp32 product, bit for bit; a reduction above 256 is declined with nothing launched."""
+    rng = np.random.default_rng(M + N + Kd)
+    Xq = rng.integers(-127, 128, (M, Kd)).astype(np.int8)
+    W = rng.standard_normal((N, Kd)).astype(np.float32)
+    bias = rng.standard_normal(N).astype(np.float32)
+    omode = orc.RNE if mode == "rne" else orc.TRUNC
+    sX, sW = np.float32(0.031), orc.absmax_scale(W)
+    Wq = orc.quantize(W, sW, omode)
+    acc = (Xq.astype(np.float64) @ Wq.astype(np.float64).T).astype(np.float32)
+    Y = bias[None, :] + (sX * sW) * acc
+    sY = orc.absmax_scale(Y)
+    want = orc.quantize(Y, sY, omode)
+    ld = (Kd + 15) // 16 * 16
+    Xb = torch.full((M, ld), 33, dtype=torch.int8, device="cuda")
+    Xb[:, :Kd] = dev(Xq)
+    ldy = (N + 15) // 16 * 16
+    Yb = torch.full((M, ldy), 99, dtype=torch.int8, device="cuda")
+    W_q = torch.empty((N, Kd), dtype=torch.int8, device="cuda")
+    s_out = torch.full((1,), 7.0, device="cuda")
+    assert K.cuda_kernels.QGEMM_forward_q8(Yb[:, :N], s_out, Xb[:, :Kd], dev(W), W_q, dev(bias), sc(sX), sc(sW),
+                                           round_mode=mode)
+    assert host(s_out)[0] == sY and np.array_equal(host(W_q), Wq)
+    assert np.array_equal(host(Yb[:, :N]), want)
+    assert (host(Yb[:, N:]) == 99).all()  # the padding of the output rows is left alone
+    big = torch.zeros((4, 272), dtype=torch.int8, device="cuda")
+    assert not K.cuda_kernels.QGEMM_forward_q8(torch.empty((4, 16), dtype=torch.int8, device="cuda"), s_out, big,
+                                               torch.zeros((16, 272), device="cuda"),
+                                               torch.empty((16, 272), dtype=torch.int8, device="cuda"), None,
+                                               sc(1.0), sc(1.0), round_mode=mode)
+
+
 def test_mfma_rate_probe_runs():
     """The measurement aid launches, finishes and leaves its sink untouched."""
     from tango_amd import _lib
