@@ -229,18 +229,32 @@ __global__ __launch_bounds__(64 * WAVES) void gemm_nts_kernel(const NtParams p, 
     const int g = lane >> 4, r16 = lane & 15;
     const int64_t n0 = static_cast<int64_t>(blockIdx.y) * (16 * NT);
     const int ksteps = static_cast<int>((p.Kr + 63) >> 6);  // <= KS (host)
+    // Which column of the block the LDS row n = 16 j + 4 g + v (column 4 g + v of MFMA tile j) stands for.  A lane
+    // holds columns 4 g .. 4 g + 3 of every tile: four output bytes in the int8 epilogue.  There the tiles of a
+    // group of four are interleaved, so that a lane's four tiles cover sixteen adjacent columns (one 16-byte
+    // store, 64 contiguous bytes per row from the four lanes) instead of four 4-byte pieces.
+    constexpr bool PERM = EPI == 2 && NT % 4 == 0;
+    auto lds_row_column = [](int n) {
+        if (!PERM) return n;
+        const int j = n >> 4, gq = (n >> 2) & 3, v = n & 3;
+        return 64 * (j >> 2) + 16 * gq + 4 * (j & 3) + v;
+    };
     {
         const int cpr = pitch >> 4;
         const int kchunks = ksteps * 4;  // 16-byte chunks of a packed row that hold data or its zero fill
         for (int idx = tid; idx < 16 * NT * cpr; idx += 64 * WAVES) {
             const int n = idx / cpr, c = idx - n * cpr;
             i32x4 v{0, 0, 0, 0};
-            if (n0 + n < p.N && c < kchunks) v = *reinterpret_cast<const i32x4*>(p.B + (n0 + n) * p.ldb + c * 16);
+            const int64_t nb = n0 + lds_row_column(n);
+            if (nb < p.N && c < kchunks) v = *reinterpret_cast<const i32x4*>(p.B + nb * p.ldb + c * 16);
             *reinterpret_cast<i32x4*>(b_lds + n * pitch + c * 16) = v;
         }
     }
     float* bias_lds = reinterpret_cast<float*>(b_lds + 16 * NT * pitch);  // [16 NT], zero where there is none
-    for (int n = tid; n < 16 * NT; n += 64 * WAVES) bias_lds[n] = (p.bias && n0 + n < p.N) ? p.bias[n0 + n] : 0.0f;
+    for (int n = tid; n < 16 * NT; n += 64 * WAVES) {
+        const int64_t nb = n0 + lds_row_column(n);
+        bias_lds[n] = (p.bias && nb < p.N) ? p.bias[nb] : 0.0f;
+    }
     __syncthreads();
 
     const float s = p.sA[0] * p.sB[0];
@@ -248,6 +262,7 @@ __global__ __launch_bounds__(64 * WAVES) void gemm_nts_kernel(const NtParams p, 
     const int wide = ((ca & 15) == 0 && (p.ldc & 3) == 0) ? 4 : ((ca & 7) == 0 && (p.ldc & 1) == 0) ? 2 : 1;
     const float qr = EPI == 2 ? rscale_of(p.q_scale[0]) : 0.0f;
     const bool qwide = EPI == 2 && (reinterpret_cast<uintptr_t>(p.Cq) & 3) == 0 && (p.ldcq & 3) == 0;
+    const bool q16 = EPI == 2 && (reinterpret_cast<uintptr_t>(p.Cq) & 15) == 0 && (p.ldcq & 15) == 0;
     float m = 0.0f;
     auto load_tile = [&](i32x4* a, float& rsc, int t) {
         const int64_t row = static_cast<int64_t>(t) * 16 + r16;
@@ -281,13 +296,14 @@ __global__ __launch_bounds__(64 * WAVES) void gemm_nts_kernel(const NtParams p, 
                 }
             }
         }
-        // lane holds C[16 t + r16][n0 + 16 j + 4 g + v]
+        // lane holds C[16 t + r16][n0 + 16 j + 4 g + v] (PERM: the column lds_row_column gives)
         const int64_t row = static_cast<int64_t>(t) * 16 + r16;
         if (row < p.M) {
             float* crow = p.C + row * p.ldc;
+            uint32_t qw[4];
 #pragma unroll
             for (int j = 0; j < NT; ++j) {
-                const int64_t col = n0 + j * 16 + g * 4;
+                const int64_t col = PERM ? n0 + 64 * (j >> 2) + 16 * g + 4 * (j & 3) : n0 + j * 16 + g * 4;
                 float y[4];
                 const f32x4 bv = *reinterpret_cast<const f32x4*>(bias_lds + j * 16 + g * 4);
 #pragma unroll
@@ -295,16 +311,33 @@ __global__ __launch_bounds__(64 * WAVES) void gemm_nts_kernel(const NtParams p, 
                     y[v] = s * static_cast<float>(acc[j][v]);
                     if (p.row_scale) y[v] = y[v] * rsc;
                     if (p.bias) y[v] = bv[v] + y[v];
-                    if (col + v < p.N) m = fmaxf(m, fabsf(y[v]));
+                    if (EPI != 2 && col + v < p.N) m = fmaxf(m, fabsf(y[v]));
                 }
                 if (EPI == 1) continue;
                 if (EPI == 2) {
                     int q[4];
+                    if (p.q_mode == TANGO_ROUND_TRUNC) {  // uniform
 #pragma unroll
-                    for (int v = 0; v < 4; ++v)
-                        q[v] = p.q_mode == TANGO_ROUND_TRUNC ? quant_one<TANGO_ROUND_TRUNC>(y[v], qr, 0.0f)
-                                                             : quant_one<TANGO_ROUND_RNE>(y[v], qr, 0.0f);
+                        for (int v = 0; v < 4; ++v) q[v] = quant_one<TANGO_ROUND_TRUNC>(y[v], qr, 0.0f);
+                    } else {
+#pragma unroll
+                        for (int v = 0; v < 4; ++v) q[v] = quant_one<TANGO_ROUND_RNE>(y[v], qr, 0.0f);
+                    }
                     int8_t* qrow = p.Cq + row * p.ldcq;
+                    if (PERM) {
+                        qw[j & 3] = pack4(q[0], q[1], q[2], q[3]);
+                        if ((j & 3) != 3) continue;
+                        const int64_t col0 = col - 12;  // n0 + 64 (j / 4) + 16 g
+                        if (col0 + 16 <= p.N && q16) {
+                            typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+                            *reinterpret_cast<u32x4*>(qrow + col0) = u32x4{qw[0], qw[1], qw[2], qw[3]};
+                        } else {
+#pragma unroll
+                            for (int b = 0; b < 16; ++b)
+                                if (col0 + b < p.N) qrow[col0 + b] = static_cast<int8_t>(qw[b >> 2] >> (8 * (b & 3)));
+                        }
+                        continue;
+                    }
                     if (col + 4 <= p.N && qwide) {
                         *reinterpret_cast<uint32_t*>(qrow + col) = pack4(q[0], q[1], q[2], q[3]);
                     } else {

@@ -206,7 +206,8 @@ def test_gradx_accumulates_into_its_output(K, M, N, Kd, rows):
 
 
 @pytest.mark.parametrize("mode", ["rne", "trunc"])
-@pytest.mark.parametrize("M,N,Kd", [(40000, 256, 256), (3001, 41, 100), (16, 600, 64), (1, 16, 16)])
+@pytest.mark.parametrize("M,N,Kd", [(40000, 256, 256), (3001, 41, 100), (16, 600, 64), (1, 16, 16), (500, 128, 192),
+                                    (777, 250, 33)])
 def test_forward_gemm_with_int8_output(K, orc, M, N, Kd, mode):
     """The forward GEMM that stores its output already quantized == the oracle's int8 GEMM, absmax scale and
     quantize on the fp32 product, bit for bit; a reduction above 256 is declined with nothing launched."""
