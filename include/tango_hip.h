@@ -31,7 +31,8 @@ enum tango_status {
     TANGO_ERR_INVALID_ARG = -1, /* null pointer, negative size, misaligned operand */
     TANGO_ERR_UNSUPPORTED = -2, /* unknown op / rounding mode / shape outside the kernels' range */
     TANGO_ERR_LAUNCH = -3,      /* HIP refused the launch */
-    TANGO_ERR_WORKSPACE = -4    /* workspace missing or too small */
+    TANGO_ERR_WORKSPACE = -4,   /* workspace missing or too small */
+    TANGO_ERR_STATIC_LIMIT = -5 /* input beyond the fixed scratch of tango_edge_softmax_fwd_static */
 };
 
 enum tango_round_mode {
@@ -331,6 +332,20 @@ int tango_edge_softmax_fwd(float* a, const float* e, const int64_t* indptr,
                            const int64_t* edge_ids, int64_t rows, int64_t num_edges, int64_t H,
                            float slope, void* workspace, size_t workspace_bytes,
                            tango_stream_t stream);
+/* tango_edge_softmax_fwd for callers that cannot allocate (code under HIP graph capture, tight
+   serving loops, harnesses that forbid hipMalloc).  It has no counterpart in the reference.  Same
+   kernels and same results as tango_edge_softmax_fwd with a workspace, but the per-span records live
+   in a fixed array of TANGO_EDGE_SOFTMAX_STATIC_BYTES inside the library's device image (one copy
+   per GPU, held until the process ends) and no memory is allocated or freed by the call.
+   Inputs with tango_edge_softmax_workspace(num_edges, H) > TANGO_EDGE_SOFTMAX_STATIC_BYTES are
+   rejected with TANGO_ERR_STATIC_LIMIT before anything is launched (at H = 8 the limit is about
+   3.5 million edges).  All calls on one GPU share the array: calls that overlap on one GPU
+   (different streams or threads) race; calls on one stream are ordered and safe. */
+#define TANGO_EDGE_SOFTMAX_STATIC_BYTES (4u << 20)
+int tango_edge_softmax_fwd_static(float* a, const float* e, const int64_t* indptr,
+                                  const int64_t* edge_ids, int64_t rows, int64_t num_edges, int64_t H,
+                                  float slope, tango_stream_t stream);
+
 /* de = dLeaky(e) * a * (da - sum_{same dst} a*da). */
 int tango_edge_softmax_bwd(float* de, const float* a, const float* da, const float* e,
                            const int64_t* indptr, const int64_t* edge_ids, int64_t rows,

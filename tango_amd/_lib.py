@@ -59,6 +59,7 @@ SIGNATURES = {
     "tango_softmax_xent_f32": (I, [P, I64, P, I64, I64, P, P, I64, P, SZ, P]),
     "tango_edge_softmax_workspace": (SZ, [I64, I64]),
     "tango_edge_softmax_fwd": (I, [P, P, P, P, I64, I64, I64, F, P, SZ, P]),
+    "tango_edge_softmax_fwd_static": (I, [P, P, P, P, I64, I64, I64, F, P]),
     "tango_edge_softmax_bwd": (I, [P, P, P, P, P, P, I64, I64, I64, F, P, SZ, P]),
 }
 

@@ -11,7 +11,35 @@
 // workspace a thread-per-(row, head) kernel is used.
 #include "common.hpp"
 
+#include <mutex>
+
 namespace tango {
+
+// Scratch of the entry point that allocates nothing (tango_edge_softmax_fwd_static): the per-span partial
+// (max, sum) records that the span kernels otherwise keep in the caller's workspace.  One copy per device,
+// held until the process ends.  In host code this name is only a handle for hipGetSymbolAddress; kernels
+// receive the device address that call returns.
+static __device__ __align__(256) unsigned char scratch[TANGO_EDGE_SOFTMAX_STATIC_BYTES];
+
+constexpr int kMaxDevices = 64;
+static std::mutex scratch_mutex;
+static void* scratch_address[kMaxDevices];  // device address of `scratch` on each device, once looked up
+
+// Device address of `scratch` on the current device (looked up once per device), or nullptr.
+static void* scratch_of_current_device() {
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return nullptr;
+    std::lock_guard<std::mutex> lock(scratch_mutex);
+    if (!scratch_address[dev]) {
+        void* p = nullptr;
+        if (hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)) != hipSuccess) {
+            (void)hipGetLastError();
+            return nullptr;
+        }
+        scratch_address[dev] = p;
+    }
+    return scratch_address[dev];
+}
 
 __device__ __forceinline__ float leaky(float v, float slope) { return v > 0.0f ? v : v * slope; }
 
@@ -532,6 +560,21 @@ int tango_edge_softmax_fwd(float* a, const float* e, const int64_t* indptr,
     }
     hipLaunchKernelGGL(edge_softmax_fwd_kernel, dim3(grid_for(rows * H, 256, 16)), dim3(256), 0,
                        as_stream(stream), a, e, indptr, edge_ids, rows, static_cast<int>(H), slope);
+    return launch_status();
+}
+
+int tango_edge_softmax_fwd_static(float* a, const float* e, const int64_t* indptr, const int64_t* edge_ids,
+                                  int64_t rows, int64_t nnz, int64_t H, float slope, tango_stream_t stream) {
+    if (rows < 0 || nnz < 0 || H < 0 || (rows > 0 && !indptr) || H >= (1LL << 31)) return TANGO_ERR_INVALID_ARG;
+    if (rows * H == 0 || nnz == 0) return TANGO_OK;
+    if (!a || !e) return TANGO_ERR_INVALID_ARG;
+    if (ceil_div(nnz, 4 * 128) > INT32_MAX || ceil_div(H, 8) > 65535) return TANGO_ERR_UNSUPPORTED;
+    if (span_workspace_bytes(nnz, H) > TANGO_EDGE_SOFTMAX_STATIC_BYTES) return TANGO_ERR_STATIC_LIMIT;
+    void* ws = scratch_of_current_device();
+    if (!ws) return TANGO_ERR_LAUNCH;
+    // The span kernels write every record of the scratch they later read, so nothing has to be cleared.
+    launch_spans<true>(a, nullptr, nullptr, e, indptr, edge_ids, rows, nnz, static_cast<int>(H), slope, ws,
+                       as_stream(stream));
     return launch_status();
 }
 

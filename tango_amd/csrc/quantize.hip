@@ -631,6 +631,7 @@ const char* tango_status_string(int status) {
         case TANGO_ERR_UNSUPPORTED: return "unsupported op, mode or shape";
         case TANGO_ERR_LAUNCH: return "kernel launch failed";
         case TANGO_ERR_WORKSPACE: return "workspace missing or too small";
+        case TANGO_ERR_STATIC_LIMIT: return "input too large for the fixed scratch of the entry point that allocates nothing";
         default: return "unknown status";
     }
 }

@@ -45,6 +45,16 @@ def test_argument_validation_needs_no_gpu():
     assert L.tango_spmm_csr_copy_u(1, 1, 1, 1, 8, 1, 4, 1 << 31, 10, 8, None) == -2  # node ids must fit 31 bits
 
 
+def test_static_scratch_rejects_oversized_input():
+    from tango_amd import _lib
+    L = _lib.lib()
+    E, H = 40_000_000, 8
+    assert L.tango_edge_softmax_workspace(E, H) > (4 << 20)
+    # rejected on the host before any launch: the pointers are never dereferenced
+    assert L.tango_edge_softmax_fwd_static(16, 16, 16, None, 10, E, H, 0.2, None) == -5
+    assert b"scratch" in L.tango_status_string(-5)
+
+
 def test_infer_broadcast_shape():
     from tango_amd.kernels import infer_broadcast_shape as ibs
     assert ibs("add", (8, 1), (8, 1)) == (8, 1)
