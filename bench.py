@@ -18,10 +18,22 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBPS = 8000.0
-# Bytes that cross the L2 <-> fabric boundary per launch of the F=256 copy_u kernel on the default
-# benchmark graph: two rocprofv3 --pmc passes (FETCH_SIZE, then WRITE_SIZE, KiB per dispatch), each
-# scaled by what the same counter reads for a 1 GiB device copy (2.000 and 1.000).
-MEASURED_TRAFFIC_SPMM_F256 = 1.318e10
+# Counter figures of the dominant kernel on the default benchmark graph live in one place, the committed
+# rocprofv3 summary below (a line `bench-constants: {json}`): bytes that cross the L2 <-> fabric boundary per
+# launch (FETCH_SIZE + WRITE_SIZE, each scaled by what the same counter reads for a 1 GiB device copy) and the
+# launch time with every gather hitting the L2.  Counters cannot be read from inside a timed run.
+SPMM_COUNTER_SUMMARY = os.path.join(ROOT, "profiles", "spmm_copy_u_F256_counters.md")
+
+
+def counter_constants(path=SPMM_COUNTER_SUMMARY):
+    try:
+        with open(path) as f:
+            for line in f:
+                if line.startswith("bench-constants:"):
+                    return json.loads(line.split(":", 1)[1])
+    except (OSError, ValueError):
+        pass
+    return {}
 
 
 def parse():
@@ -38,6 +50,8 @@ def parse():
     ap.add_argument("--emit", default=None, metavar="JSON_FILE",
                     help="also store the result under the key 'measured_mi355x' of this JSON file")
     ap.add_argument("--feat", type=int, default=256, help="feature width of --profile-mode spmm")
+    ap.add_argument("--permute-ids", action="store_true",
+                    help="--profile-mode spmm on the benchmark graph with its node ids randomly permuted")
     ap.add_argument("--profile-mode", choices=["spmm", "copy", "qlinear", "gradx", "sddmm", "quantize", "gat", "hgt"], default=None,
                     help="run only the dominant kernel (spmm: copy_u F=256 on the benchmark graph) or a "
                          "1 GiB device copy (counter calibration), for rocprofv3 --pmc passes")
@@ -93,7 +107,29 @@ IDX_BYTES = 4
 
 
 def spmm_bytes(nnz, rows, F, idx=IDX_BYTES):
+    """Gather-traffic model: every gathered row counted once per edge.  Most of these bytes are served by the
+    caches, so the rate it gives is an effective (cache-inclusive) bandwidth, not a fraction of HBM."""
     return nnz * (F + idx) + rows * (4 * F + 8)
+
+
+def spmm_compulsory_bytes(nnz, rows, num_src, F, idx=IDX_BYTES):
+    """What must cross HBM at least once: the index stream, the int8 features, the fp32 output."""
+    return nnz * idx + rows * 8 + num_src * F + rows * 4 * F
+
+
+def permuted_graph(g, torch, seed=11):
+    """The same graph with its node ids randomly permuted (the generator numbers nodes by falling degree)."""
+    from tango_amd.graph import Graph
+    from tango_amd.util import graph_preprocess
+    gen = torch.Generator(device="cuda").manual_seed(seed)
+    perm = torch.randperm(g.num_nodes(), generator=gen, device="cuda")
+    src, dst = g.coo
+    return graph_preprocess(Graph(perm[src], perm[dst], g.num_nodes()))
+
+
+def gather_entry(ms, model_bytes, compulsory_bytes):
+    return {"ms": round(ms, 4), "gather_model_GBps": round(model_bytes / ms / 1e6, 1),
+            "frac_hbm_compulsory": round(compulsory_bytes / ms / 1e6 / HBM_PEAK_GBPS, 4)}
 
 
 def primitives(g, K, torch):
@@ -104,18 +140,15 @@ def primitives(g, K, torch):
     for F in (16, 64, 128, 256):
         feat = torch.randint(-127, 128, (n, F), dtype=torch.int8, device="cuda")
         ms = time_op(lambda: K.csr_SPMM(g, feat, one), iters=10)
-        b = spmm_bytes(nnz, n, F)
-        out["spmm_copy_u_F%d" % F] = {"ms": round(ms, 4), "GBps": round(b / ms / 1e6, 1),
-                                      "frac_hbm": round(b / ms / 1e6 / HBM_PEAK_GBPS, 4)}
+        out["spmm_copy_u_F%d" % F] = gather_entry(ms, spmm_bytes(nnz, n, F), spmm_compulsory_bytes(nnz, n, n, F))
         del feat
     # u_mul_e, broadcast edge value: H=4, F=64 (cuda/../evaluation/SPMM_broadcast.py sizes are (2|4, 128|256))
     H, F = 2, 128
     feat = torch.randint(-127, 128, (n, H, F), dtype=torch.int8, device="cuda")
     ev = torch.randint(-127, 128, (H, 1, nnz), dtype=torch.int8, device="cuda")
     ms = time_op(lambda: K.multi_cusparse_SPMM(g, feat, ev, one), iters=5)
-    b = nnz * (H * F + H + 2 * IDX_BYTES) + n * (4 * H * F + 8)
-    out["spmm_u_mul_e_H2_F128"] = {"ms": round(ms, 4), "GBps": round(b / ms / 1e6, 1),
-                                   "frac_hbm": round(b / ms / 1e6 / HBM_PEAK_GBPS, 4)}
+    out["spmm_u_mul_e_H2_F128"] = gather_entry(ms, nnz * (H * F + H + 2 * IDX_BYTES) + n * (4 * H * F + 8),
+                                               nnz * (H + 2 * IDX_BYTES) + n * (5 * H * F + 8))
     del feat, ev
     # u_mul_e without broadcast: every head has one feature column and its own edge value
     # (evaluation/SPMM_nobroadcast.py:27-29: N [n, H, 1], E [nnz, H, 1]); and the incidence form (copy_e)
@@ -123,11 +156,11 @@ def primitives(g, K, torch):
     feat = torch.randint(-127, 128, (n, H, 1), dtype=torch.int8, device="cuda")
     ev = torch.randint(-127, 128, (nnz, H, 1), dtype=torch.int8, device="cuda")
     ms = time_op(lambda: K.multi_cusparse_SPMM(g, feat, ev, one, edge_major=True), iters=5)
-    b = nnz * (H + H + 2 * IDX_BYTES) + n * (4 * H + 8)
-    out["spmm_u_mul_e_nobroadcast_H8"] = {"ms": round(ms, 4), "GBps": round(b / ms / 1e6, 1)}
+    out["spmm_u_mul_e_nobroadcast_H8"] = gather_entry(ms, nnz * (H + H + 2 * IDX_BYTES) + n * (4 * H + 8),
+                                                      nnz * (H + 2 * IDX_BYTES) + n * (5 * H + 8))
     ms = time_op(lambda: K.incidence_SPMM(g, ev.view(nnz, H), one), iters=5)
-    b = nnz * (H + IDX_BYTES) + n * (4 * H + 8)
-    out["spmm_incidence_F8"] = {"ms": round(ms, 4), "GBps": round(b / ms / 1e6, 1)}
+    out["spmm_incidence_F8"] = gather_entry(ms, nnz * (H + IDX_BYTES) + n * (4 * H + 8),
+                                            nnz * (H + IDX_BYTES) + n * (4 * H + 8))
     del feat, ev
     # QLinear forward / backward at (M, K, N) = (232965, 602, 256) and (232965, 256, 41)
     for (M, Kd, N) in ((n, 602, 256), (n, 256, 41), (n, 128, 16)):
@@ -169,14 +202,6 @@ def primitives(g, K, torch):
     out["qlinear_fwd_%dx%dx%d" % (M, Kd, N)] = {"ms": round(t_fused, 4), "ms_input_already_int8": round(t_cached, 4),
                                                  "ms_with_separate_output_absmax": round(t_plain, 4)}
     del X, W, Xq, Wq
-    # the int8 matrix rate the device sustains on register-resident operands (the ceiling of any int8 GEMM here)
-    from tango_amd import _lib
-    sink = torch.zeros(1, dtype=torch.int32, device="cuda")
-    wgs, iters = 256 * 8, 4096
-    stream = torch.cuda.current_stream().cuda_stream
-    ms = time_op(lambda: _lib.check(_lib.lib().tango_probe_mfma_i8(wgs, iters, sink.data_ptr(), stream), "probe"), iters=5)
-    out["mfma_i8_probe"] = {"ms": round(ms, 4), "TOPS": round(wgs * 4 * iters * 8 * 32768.0 / ms / 1e9, 1),
-                            "published_peak_TOPS": 5000.0}
     # quantize / absmax streaming
     X = torch.randn(n, 602, device="cuda")
     ms = time_op(lambda: K.cuda_kernels.get_scale(X))
@@ -200,17 +225,16 @@ def sddmm_primitives(K, torch):
     one = torch.ones(1, device="cuda") * 0.01
     out = {"graph": {"nodes": n, "edges": E}}
     ms = time_op(lambda: K.mySDDMM_int8(g, "dot", U, V, one, one, False))
-    b = E * (16 + 2 * H * D + 4 * H)
-    out["sddmm_dot_H8_D16"] = {"ms": round(ms, 4), "GBps": round(b / ms / 1e6, 1),
-                               "frac_hbm": round(b / ms / 1e6 / HBM_PEAK_GBPS, 4)}
+    out["sddmm_dot_H8_D16"] = gather_entry(ms, E * (16 + 2 * H * D + 4 * H), E * 16 + 2 * n * H * D + 4 * E * H)
     el = torch.randint(-127, 128, (n, H, 1), dtype=torch.int8, device="cuda")
     ms = time_op(lambda: K.mySDDMM_int8(g, "add", el, el, one, one, False))
-    b = E * (16 + 2 * H + 4 * H)
-    out["sddmm_add_H8"] = {"ms": round(ms, 4), "GBps": round(b / ms / 1e6, 1)}
+    out["sddmm_add_H8"] = gather_entry(ms, E * (16 + 2 * H + 4 * H), E * 16 + 2 * n * H + 4 * E * H)
     e = torch.randn(E, H, 1, device="cuda")
     ip, _, eid = g.adj_csc
     ms = time_op(lambda: K.cuda_kernels.edge_softmax_forward(e, ip, eid, 0.2))
-    out["edge_softmax_H8"] = {"ms": round(ms, 4), "GBps": round(E * (8 * H + 8) / ms / 1e6, 1)}
+    b = E * (8 * H + 8)  # a stream: e read once, a written once, row pointers / edge ids
+    out["edge_softmax_H8"] = {"ms": round(ms, 4), "GBps": round(b / ms / 1e6, 1),
+                              "frac_hbm": round(b / ms / 1e6 / HBM_PEAK_GBPS, 4)}
     return out
 
 
@@ -435,11 +459,14 @@ def main():
                      % (n, nnz, max_deg, time.perf_counter() - t0))
 
     if args.profile_mode == "spmm":
+        if args.permute_ids:
+            g = permuted_graph(g, torch)
         feat = torch.randint(-127, 128, (n, args.feat), dtype=torch.int8, device="cuda")
         one = torch.full((1,), 0.01, device="cuda")
         ms = time_op(lambda: K.csr_SPMM(g, feat, one), iters=args.steps, warm=args.warmup)
         print(json.dumps({"profile_mode": "spmm", "F": args.feat, "nodes": n, "edges": nnz, "avg_ms": round(ms, 4),
-                          "algorithmic_bytes": spmm_bytes(nnz, n, args.feat)}))
+                          "permuted_ids": bool(args.permute_ids), "gather_model_bytes": spmm_bytes(nnz, n, args.feat),
+                          "compulsory_bytes": spmm_compulsory_bytes(nnz, n, n, args.feat)}))
         return
 
     gen = torch.Generator().manual_seed(5)
@@ -473,15 +500,32 @@ def main():
     ms_per_step = (time.perf_counter() - t1) * 1000.0 / args.steps
     K.cuda_kernels.csr_SPMM = staticmethod(raw_spmm)
 
-    # dominant kernel: the 256-wide copy_u aggregation (forward and reverse launches of the same kernel)
+    # Dominant kernel: the 256-wide copy_u aggregation (forward and reverse launches of the same kernel).
+    # What binds it is the caches, not HBM: a gathered 128-byte row piece is one L2 -> L1 line transfer, and
+    # the misses of the 4 MB L2s are refilled over the fabric.  `achieved` is therefore the measured traffic
+    # beyond L2 (rocprofv3 counters, committed summary) over the launch time measured here, as a fraction of
+    # the 8 TB/s memory-side peak; the gather-traffic model (every gathered byte counted per edge) is reported
+    # beside it as an effective bandwidth without a fraction, since the caches serve most of it.
     k_ms = timer.mean_ms("spmm_F256")
     alg = spmm_bytes(nnz, n, 256)
-    achieved = alg / k_ms / 1e6
-    roofline = {"kernel": "spmm_kernel<16,1,copy_u> F=256 (two 128-column tiles)", "bound": "hbm", "achieved": round(achieved, 1),
-                "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4),
-                "traffic": MEASURED_TRAFFIC_SPMM_F256 if (args.nodes, args.edges) == (232965, 114_600_000) else None,
-                "avg_launch_ms": round(k_ms, 4), "algorithmic_bytes": alg, "index_bytes": IDX_BYTES,
-                "launches_timed": len(timer.spans.get("spmm_F256", []))}
+    comp = spmm_compulsory_bytes(nnz, n, n, 256)
+    consts = counter_constants() if (args.nodes, args.edges) == (232965, 114_600_000) else {}
+    traffic = consts.get("traffic_bytes_per_launch")
+    floor_ms = consts.get("l2_all_hit_launch_ms")
+    achieved = traffic / k_ms / 1e6 if traffic else None
+    roofline = {"kernel": consts.get("kernel", "copy_u aggregation, F=256"), "bound": "hbm",
+                "achieved": round(achieved, 1) if achieved else None, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                "frac": round(achieved / HBM_PEAK_GBPS, 4) if achieved else None, "traffic": traffic,
+                "achieved_basis": "measured bytes beyond L2 per launch (FETCH_SIZE + WRITE_SIZE, "
+                                  "profiles/spmm_copy_u_F256_counters.md) / avg_launch_ms",
+                "binding_limit": "L2 -> L1 line rate (one 128-byte line per gathered row piece) plus the L2 "
+                                 "misses' refills over the fabric; the int8 features stay in the Infinity Cache",
+                "avg_launch_ms": round(k_ms, 4), "launches_timed": len(timer.spans.get("spmm_F256", [])),
+                "l2_all_hit_launch_ms": floor_ms,
+                "frac_l2_floor": round(floor_ms / k_ms, 4) if floor_ms else None,
+                "compulsory_bytes": comp, "frac_hbm_compulsory": round(comp / k_ms / 1e6 / HBM_PEAK_GBPS, 4),
+                "model": {"name": "gather traffic (cache-served)", "bytes": alg, "index_bytes": IDX_BYTES,
+                          "effective_GBps": round(alg / k_ms / 1e6, 1)}}
 
     result = {
         "metric": "quant GCN epoch ms @233K nodes/114.6M edges; SpMM/SDDMM GB/s; QLinear TOPS",
@@ -502,8 +546,15 @@ def main():
         prims.update(sddmm_primitives(K, torch))
         prims.update(model_steps(K, torch))
         result["primitives"] = prims
-        result["spmm_GBps"] = prims["spmm_copy_u_F256"]["GBps"]
-        result["sddmm_GBps"] = prims["sddmm_dot_H8_D16"]["GBps"]
+        # sensitivity: the same aggregation with the node ids randomly permuted (hub rows scattered over the
+        # feature matrix instead of contiguous at its top)
+        gp = permuted_graph(g, torch)
+        feat = torch.randint(-127, 128, (n, 256), dtype=torch.int8, device="cuda")
+        one = torch.full((1,), 0.01, device="cuda")
+        prims["spmm_copy_u_F256_permuted_ids"] = {"ms": round(time_op(lambda: K.csr_SPMM(gp, feat, one), iters=10), 4)}
+        del gp, feat
+        result["spmm_gather_model_GBps"] = prims["spmm_copy_u_F256"]["gather_model_GBps"]
+        result["sddmm_gather_model_GBps"] = prims["sddmm_dot_H8_D16"]["gather_model_GBps"]
         result["qlinear_TOPS"] = prims["qlinear_fwd_%dx602x256" % n]["TOPS"]
 
     if not args.no_cpu:

@@ -129,7 +129,9 @@ int tango_transpose_quant_f32_i8(const float* x, int64_t nrow, int64_t ncol, con
    bias may be NULL.  scaleY may be NULL; otherwise scaleY[0] = max|Y| / 127
    (the fused reduction of cuda/src/epilogue.h:105-626); it need not be
    initialised.  K is arbitrary (the reference requires K % 4 == 0); rows of Xq
-   padded to a multiple of 16 bytes take the fast path. */
+   padded to a multiple of 16 bytes take the fast path.  round_mode: TANGO_ROUND_RNE or
+   TANGO_ROUND_TRUNC, used for X and W alike; TANGO_ROUND_STOCHASTIC (for which this
+   signature carries no seed) returns TANGO_ERR_UNSUPPORTED before anything is launched. */
 size_t tango_qgemm_fwd_workspace(int64_t M, int64_t N, int64_t K);
 int tango_qgemm_fwd(float* Y, int64_t ldy, const float* X, int64_t ldx, int8_t* Xq, int64_t ldxq,
                     const float* W, int64_t ldw, int8_t* Wq, const float* bias, float* scaleY,
@@ -149,12 +151,6 @@ int tango_qgemm_fwd_ex(float* Y, int64_t ldy, const float* X, int64_t ldx, const
                        const float* bias, float* scaleY, const float* scaleX, const float* scaleW,
                        int64_t M, int64_t N, int64_t K, int round_mode, void* workspace,
                        size_t workspace_bytes, tango_stream_t stream);
-
-/* Measurement aid (no counterpart in the reference): launches `workgroups` workgroups of four waves that
-   each issue iters * 8 register-resident v_mfma_i32_16x16x64_i8 (32768 int8 operations per instruction
-   and wave) and nothing else, so that a caller timing the launch learns the int8 matrix rate the device
-   sustains.  sink: one int of device memory (practically never written). */
-int tango_probe_mfma_i8(int64_t workgroups, int64_t iters, int* sink, tango_stream_t stream);
 
 /* Forward linear whose output is read only by another quantized op (the first of two chained
    QLinear layers, evaluation/test_HGT.py:51-55): instead of the fp32 Y that cuda/QLinear.py:30-36

@@ -153,7 +153,7 @@ class Qlinear_shared_func(Function):
         if tuple(Xq.shape) != tuple(X.shape) or Xq.dtype != torch.int8 or X.dim() != 2:
             raise RuntimeError("Qlinear_shared_func: the quantized input must be int8 of the 2-D input's shape")
         ctx.set_materialize_grads(False)
-        outs, layers = [], []
+        outs, layers, scales = [], [], []
         get_scale = kernels.cuda_kernels.get_scale
         for i in range(n_first):
             W, b = wb[2 * i], wb[2 * i + 1]
@@ -175,9 +175,10 @@ class Qlinear_shared_func(Function):
                 W2_ = torch.empty(W2.shape, dtype=torch.int8, device=X.device)
                 out, scaleO = kernels.QGEMM_forward(Y, Yq, sY, W2, W2_, scaleW2, b2, True)
                 second = (Yq, sY, W2_, scaleW2, b2 is not None)
-            ctx.mark_non_differentiable(scaleO)
+            scales.append(scaleO)
             outs += [out, scaleO]
             layers.append((W_, scaleW, b is not None, second))
+        ctx.mark_non_differentiable(*scales)  # one call: each call replaces the set of the one before
         ctx.backward_cache = Xq, scaleX, layers
         return tuple(outs)
 

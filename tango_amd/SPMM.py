@@ -50,13 +50,20 @@ class spmm_copy_u(Function):
         if relu and N.dim() == 2 and N.size(1) % 16 == 0:
             bits = torch.empty((g.num_nodes(), N.size(1) // 16), dtype=torch.int16, device=N.device)
         out = csr_SPMM(g, N_, scaleN, row_scale=row_scale, bias=bias, relu=relu, sign_bits=bits)
-        ctx.backward_cache = g, row_scale, bias is not None, ((bits if bits is not None else out) if relu else None)
+        # the op's own output goes through save_for_backward (autograd then holds it without the
+        # output -> grad_fn -> ctx -> output cycle a plain attribute would form); everything else is an input
+        # or an auxiliary tensor, kept as the reference keeps its cache (cuda/SPMM.py:13)
+        ctx.backward_cache = g, row_scale, bias is not None, bits, relu
+        if relu and bits is None:
+            ctx.save_for_backward(out)
         return out
 
     @staticmethod
     @once_differentiable
     def backward(ctx, dOut):
-        g, row_scale, has_bias, mask = ctx.backward_cache
+        g, row_scale, has_bias, mask, relu = ctx.backward_cache
+        if relu and mask is None:
+            mask, = ctx.saved_tensors
         dN = dbias = None
         if row_scale is None and not has_bias and mask is None:
             if ctx.needs_input_grad[1]:
@@ -110,16 +117,18 @@ class spmm_u_mul_e(Function):
         # dequantized with scaleN * scaleE (cuda/SPMM.py:44); the kernel multiplies the two itself
         out = multi_cusparse_SPMM(g, N_, E_T_, scaleN, edge_major=True, bias=bias, scale2=scaleE, act=act)
         reduce_last = _need_reduce_last_dim(N, E)
-        ctx.backward_cache = (g, N_, scaleN, E_T_, scaleE, reduce_last, E.shape, bias is not None, act,
-                              out if act is not None else None)
+        ctx.backward_cache = g, N_, scaleN, E_T_, scaleE, reduce_last, E.shape, bias is not None, act
+        if act is not None:
+            ctx.save_for_backward(out)  # not an attribute: that would tie the output to its own grad_fn
         return out
 
     @staticmethod
     @once_differentiable
     def backward(ctx, dZ):
-        g, N_, scaleN, E_T_, scaleE, reduce_last, eshape, has_bias, act, out = ctx.backward_cache
+        g, N_, scaleN, E_T_, scaleE, reduce_last, eshape, has_bias, act = ctx.backward_cache
         dbias = None
         if act is not None:
+            out, = ctx.saved_tensors
             # dZ goes back through the activation on its way into the scale, the bias gradient and int8
             dZ = dZ if dZ.is_contiguous() else dZ.contiguous()
             dZ2, out2 = dZ.view(dZ.size(0), -1), out.view(out.size(0), -1)

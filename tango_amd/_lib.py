@@ -20,7 +20,6 @@ SZ = C.c_size_t
 SIGNATURES = {
     "tango_status_string": (C.c_char_p, [I]),
     "tango_abi_version": (I, []),
-    "tango_probe_mfma_i8": (I, [I64, I64, P, P]),
     "tango_absmax_f32": (I, [P, I64, P, P]),
     "tango_absmax_acc_f32": (I, [P, I64, P, P]),
     "tango_absmax_rows_f32": (I, [P, I64, I64, I64, P, P]),

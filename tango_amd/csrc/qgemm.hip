@@ -787,26 +787,6 @@ __global__ __launch_bounds__(768) void gemm_ws_kernel(const FqParams p, int nblo
     if (p.absmax_out) block_absmax_to_global(m / 127.0f, p.absmax_out);
 }
 
-// ------------------------------------------------ MFMA rate probe (measurement only)
-// Register-resident v_mfma_i32_16x16x64_i8: eight independent accumulator chains per wave, operands never
-// reloaded.  The sustained rate of this loop is the ceiling any int8 GEMM here can reach; the benchmark
-// prints it beside the published peak.
-__global__ __launch_bounds__(256) void mfma_i8_probe_kernel(int iters, int* __restrict__ sink) {
-    const int lane = threadIdx.x & 63;
-    const i32x4 a{lane, lane + 1, lane + 2, lane + 3}, b{lane * 3, 1, 2, lane};
-    i32x4 acc[8];
-#pragma unroll
-    for (int j = 0; j < 8; ++j) acc[j] = i32x4{j, 0, 0, 0};
-    for (int it = 0; it < iters; ++it) {
-#pragma unroll
-        for (int j = 0; j < 8; ++j) acc[j] = mfma_16x16x64(a, b, acc[j]);
-    }
-    int v = 0;
-#pragma unroll
-    for (int j = 0; j < 8; ++j) v ^= acc[j].x ^ acc[j].y ^ acc[j].z ^ acc[j].w;
-    if (v == 0x7fffffff) sink[0] = v;  // keeps the loop alive; practically never true
-}
-
 // ------------------------------------------------------- operand packing
 // dst[r, 0..ldd) = src[r, 0..cols) zero-filled, for r < rows (src row stride lds).
 __global__ __launch_bounds__(256) void pack_rows_i8_kernel(int8_t* __restrict__ dst, int64_t ldd,
@@ -1227,7 +1207,8 @@ int tango_qgemm_fwd_ex(float* Y, int64_t ldy, const float* X, int64_t ldx, const
     if (M * K > 0 && !Xq) return TANGO_ERR_INVALID_ARG;
     if (cached && x_row_mul) return TANGO_ERR_INVALID_ARG;
     if (N * K > 0 && (!W || !Wq)) return TANGO_ERR_INVALID_ARG;
-    if (round_mode < 0 || round_mode > 2) return TANGO_ERR_UNSUPPORTED;
+    // no seed / noise argument exists here, so stochastic rounding cannot be honoured: refuse it
+    if (round_mode != TANGO_ROUND_RNE && round_mode != TANGO_ROUND_TRUNC) return TANGO_ERR_UNSUPPORTED;
     const size_t need = tango_qgemm_fwd_workspace(M, N, K);
     if (need > 0 && (!workspace || workspace_bytes < need)) return TANGO_ERR_WORKSPACE;
     if ((reinterpret_cast<uintptr_t>(workspace) & 15) != 0) return TANGO_ERR_INVALID_ARG;
@@ -1302,13 +1283,6 @@ int tango_qgemm_fwd_q8(int8_t* Yq, int64_t ldyq, float* scaleY, const int8_t* Xq
     if (!launch_nts<16, 1>(p, s)) return TANGO_ERR_UNSUPPORTED;
     p.absmax_out = nullptr; p.Cq = Yq; p.ldcq = ldyq; p.q_scale = scaleY; p.q_mode = round_mode;
     if (!launch_nts<16, 2>(p, s)) return TANGO_ERR_UNSUPPORTED;
-    return launch_status();
-}
-
-int tango_probe_mfma_i8(int64_t workgroups, int64_t iters, int* sink, tango_stream_t stream) {
-    if (workgroups <= 0 || workgroups > INT32_MAX || iters < 0 || iters > INT32_MAX || !sink) return TANGO_ERR_INVALID_ARG;
-    hipLaunchKernelGGL(mfma_i8_probe_kernel, dim3(static_cast<unsigned>(workgroups)), dim3(256), 0, as_stream(stream),
-                       static_cast<int>(iters), sink);
     return launch_status();
 }
 

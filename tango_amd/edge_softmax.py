@@ -18,13 +18,15 @@ class _EdgeSoftmax(Function):
         e = e if e.is_contiguous() else e.contiguous()
         indptr, eids = _dst_major(g)
         a = cuda_kernels.edge_softmax_forward(e, indptr, eids, slope)
-        ctx.backward_cache = g, e, a, slope
+        ctx.backward_cache = g, slope
+        ctx.save_for_backward(e, a)  # a is this op's output: saved, not an attribute (no reference cycle)
         return a
 
     @staticmethod
     @once_differentiable
     def backward(ctx, da):
-        g, e, a, slope = ctx.backward_cache
+        g, slope = ctx.backward_cache
+        e, a = ctx.saved_tensors
         indptr, eids = _dst_major(g)
         da = da if da.is_contiguous() else da.contiguous()
         return None, cuda_kernels.edge_softmax_backward(a, da, e, indptr, eids, slope), None

@@ -241,11 +241,20 @@ def test_forward_gemm_with_int8_output(K, orc, M, N, Kd, mode):
                                                sc(1.0), sc(1.0), round_mode=mode)
 
 
-def test_mfma_rate_probe_runs():
-    """The measurement aid launches, finishes and leaves its sink untouched."""
+def test_forward_gemm_refuses_stochastic_rounding():
+    """The forward GEMM's signature carries no seed, so it cannot round stochastically: it says so instead
+    of rounding some other way."""
     from tango_amd import _lib
-    sink = torch.zeros(1, dtype=torch.int32, device="cuda")
-    _lib.check(_lib.lib().tango_probe_mfma_i8(8, 4, sink.data_ptr(), torch.cuda.current_stream().cuda_stream), "probe")
-    torch.cuda.synchronize()
-    assert int(sink[0]) == 0
-    assert _lib.lib().tango_probe_mfma_i8(0, 4, sink.data_ptr(), 0) != 0
+    L = _lib.lib()
+    M, N, Kd = 32, 16, 64
+    X = torch.randn(M, Kd, device="cuda")
+    W = torch.randn(N, Kd, device="cuda")
+    Xq = torch.empty((M, Kd), dtype=torch.int8, device="cuda")
+    Wq = torch.empty((N, Kd), dtype=torch.int8, device="cuda")
+    Y = torch.empty((M, N), device="cuda")
+    ws_bytes = L.tango_qgemm_fwd_workspace(M, N, Kd)
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device="cuda")
+    rc = L.tango_qgemm_fwd(Y.data_ptr(), N, X.data_ptr(), Kd, Xq.data_ptr(), Kd, W.data_ptr(), Kd, Wq.data_ptr(), None,
+                           None, sc(0.1).data_ptr(), sc(0.1).data_ptr(), M, N, Kd, _lib.ROUND_STOCHASTIC, ws.data_ptr(),
+                           ws_bytes, None)
+    assert rc == -2
