@@ -319,3 +319,104 @@ def graph_formats(src, dst, num_nodes):
     inc_out = np.stack([src[csr[2]], csr[2]])
     return {"coo": (src, dst), "adj_csr": csr, "adj_csc": csc, "inc_in": inc_in,
             "inc_out": inc_out}
+
+
+# ------------------------------------------------------------- fused forms
+MASK_MODES = {"relu": 0, "elu": 1, "bits": 2}
+
+
+def _mask_args(mask, mask_mode, cols):
+    if mask is None:
+        return None, None, 0, 0
+    mode = MASK_MODES[mask_mode]
+    if mode == 2:
+        m = np.ascontiguousarray(mask).view(np.uint16)
+        return m, _p(m), m.shape[1], mode
+    m = _f32(mask)
+    return m, _p(m), cols, mode
+
+
+def absmax_ex(x, row_mul=None, mask=None, mask_mode="relu", want_colsum=False):
+    """(max|x' * row_mul| / 127, column sums of x' or None); x' = x taken back through the activation."""
+    x = _f32(x)
+    rows, cols = x.shape
+    rm = None if row_mul is None else _f32(row_mul)
+    keep, mp, ldm, mode = _mask_args(mask, mask_mode, cols)
+    s = C.c_float(0.0)
+    cs = np.zeros(cols, dtype=np.float64) if want_colsum else None
+    lib().orc_absmax_ex(_p(x), i64(rows), i64(cols), i64(cols), _p(rm), mp, i64(ldm), C.c_int(mode),
+                        C.byref(s), _p(cs))
+    return np.float32(s.value), cs
+
+
+def quantize_rows_ex(x, scale, row_mul=None, mask=None, mask_mode="relu", ldq=None, mode=RNE, noise=None,
+                     seed=0, offset=0):
+    x = _f32(x)
+    rows, cols = x.shape
+    ldq = cols if ldq is None else ldq
+    rm = None if row_mul is None else _f32(row_mul)
+    keep, mp, ldm, mm = _mask_args(mask, mask_mode, cols)
+    sc = np.array([scale], dtype=np.float32)
+    nz = None if noise is None else _f32(noise)
+    q = np.empty((rows, ldq), dtype=np.int8)
+    lib().orc_quantize_rows_ex(_p(x), i64(rows), i64(cols), i64(cols), _p(rm), mp, i64(ldm), C.c_int(mm),
+                               _p(sc), C.c_int(0), _p(q), i64(ldq), C.c_int(mode), _p(nz), u64(seed), u64(offset))
+    return q
+
+
+def qgemm_i8_nt(A, B, sA, sB, bias=None, reduce=False):
+    """Y = (sA*sB) * float(A . B^T) (+ bias) for int8 A [M,K], B [N,K]; with ``reduce`` also max|Y| / 127."""
+    A, B = _i8(A), _i8(B)
+    M, K = A.shape
+    N = B.shape[0]
+    b = None if bias is None else _f32(bias)
+    Y = np.empty((M, N), dtype=np.float32)
+    sy = C.c_float(0.0)
+    lib().orc_qgemm_i8_nt(_p(Y), i64(N), _p(A), i64(K), _p(B), i64(K), _p(b), C.byref(sy) if reduce else None,
+                          f32(float(sA)), f32(float(sB)), i64(M), i64(N), i64(K))
+    return (Y, np.float32(sy.value)) if reduce else Y
+
+
+def qgemm_bwd_dx_ex(dYq, Wq, s_dY, s_W, row_scale=None, accumulate_into=None):
+    dYq, Wq = _i8(dYq), _i8(Wq)
+    M, N = dYq.shape
+    K = Wq.shape[1]
+    rs = None if row_scale is None else _f32(row_scale)
+    dX = np.empty((M, K), dtype=np.float32) if accumulate_into is None else _f32(accumulate_into).copy()
+    lib().orc_qgemm_bwd_dx_ex(_p(dX), i64(K), _p(dYq), i64(N), _p(Wq), i64(K), f32(float(s_dY)), f32(float(s_W)),
+                              _p(rs), C.c_int(0 if accumulate_into is None else 1), i64(M), i64(N), i64(K))
+    return dX
+
+
+def spmm_csr_copy_u_ex(indptr, indices, feat, scale, row_scale=None, bias=None, act=0, want_bits=False, F=None):
+    """out (and the sign words when ``want_bits``) of the aggregation with the GCN layer's epilogue."""
+    indptr, indices, feat = _i64(indptr), _i64(indices), _i8(feat)
+    rows = indptr.size - 1
+    ld = feat.size // feat.shape[0]
+    F = ld if F is None else F
+    rs = None if row_scale is None else _f32(row_scale)
+    b = None if bias is None else _f32(bias)
+    out = np.empty((rows, F), dtype=np.float32)
+    bits = np.zeros((rows, F // 16), dtype=np.uint16) if want_bits else None
+    lib().orc_spmm_csr_copy_u_ex(_p(out), _p(bits), _p(indptr), _p(indices), _p(feat), i64(ld), f32(float(scale)),
+                                 _p(rs), _p(b), C.c_int(act), i64(rows), i64(F))
+    return (out, bits) if want_bits else out
+
+
+def spmm_csr_u_mul_e_ex(indptr, indices, edge_ids, feat, evals, scale, scale2=None, bias=None, act=0,
+                        edge_major=False):
+    """feat [k,H,F] int8; evals [H,D,nnz] or, edge-major, [nnz,H,D] int8 -> out [rows,H,F] fp32."""
+    indptr, indices, edge_ids, feat, evals = _i64(indptr), _i64(indices), _i64(edge_ids), _i8(feat), _i8(evals)
+    k, H, F = feat.shape
+    if edge_major:
+        nnz, D = evals.shape[0], evals.shape[2]
+    else:
+        D, nnz = evals.shape[1], evals.shape[2]
+    rows = indptr.size - 1
+    s2 = None if scale2 is None else np.array([scale2], dtype=np.float32)
+    b = None if bias is None else _f32(bias)
+    out = np.empty((rows, H, F), dtype=np.float32)
+    lib().orc_spmm_csr_u_mul_e_ex(_p(out), _p(indptr), _p(indices), _p(edge_ids), _p(feat), _p(evals),
+                                  C.c_int(1 if edge_major else 0), f32(float(scale)), _p(s2), _p(b), C.c_int(act),
+                                  i64(rows), i64(H), i64(F), i64(D), i64(nnz))
+    return out

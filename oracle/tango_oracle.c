@@ -518,3 +518,185 @@ void orc_edge_softmax_bwd(float *de, const float *a, const float *da, const floa
             }
         }
 }
+
+/* ------------------------------------------------------------ fused forms -- */
+/* The layer glue of evaluation/test_gcn.py:86-94,123-137 and evaluation/test_gat.py:160-165
+   (separate torch passes in the reference) folded into the primitives.  Every fused step
+   performs the same fp32 operations, each rounded once, in the order the separate passes
+   would: these restate that order. */
+
+/* element of a gradient taken back through an activation whose output (or sign mask) is known:
+   mode 0 (ReLU, mask fp32): x where mask > 0, else 0
+   mode 1 (ELU,  mask fp32 = the activation's output): x where mask > 0, else x * (mask + 1)
+   mode 2 (ReLU, mask = 16-bit words, bit c % 16 of word [r, c / 16]): x where the bit is set, else 0 */
+static inline float masked_elem(float x, const void *mask, int64_t ldm, int mode, int64_t r, int64_t c) {
+    if (!mask) return x;
+    if (mode == 2) {
+        const uint16_t w = ((const uint16_t *)mask)[r * ldm + (c >> 4)];
+        return ((w >> (c & 15)) & 1u) ? x : 0.0f;
+    }
+    const float m = ((const float *)mask)[r * ldm + c];
+    if (m > 0.0f) return x;
+    if (mode == 0) return 0.0f;
+    volatile float t = m + 1.0f;
+    volatile float y = x * t;
+    return y;
+}
+
+/* scale_out = max|x' * row_mul| / 127 over the masked elements x'; colsum_out[c] = sum_r x'[r, c]
+   (not multiplied), accumulated in double here (the shipped kernel adds fp32 partials in a fixed
+   order: compared with a tolerance). */
+void orc_absmax_ex(const float *x, int64_t rows, int64_t cols, int64_t ldx, const float *row_mul,
+                   const void *mask, int64_t ldm, int mask_mode, float *scale_out, double *colsum_out) {
+    float m = 0.0f;
+    if (colsum_out)
+        for (int64_t c = 0; c < cols; ++c) colsum_out[c] = 0.0;
+    for (int64_t r = 0; r < rows; ++r)
+        for (int64_t c = 0; c < cols; ++c) {
+            const float v = masked_elem(x[r * ldx + c], mask, ldm, mask_mode, r, c);
+            if (colsum_out) colsum_out[c] += (double)v;
+            volatile float t = row_mul ? v * row_mul[r] : v;
+            const float a = fabsf(t);
+            if (a > m) m = a;
+        }
+    volatile float s = m / 127.0f;
+    *scale_out = s;
+}
+
+/* q[r, c] = quantize(x'[r, c] * row_mul[r]) with one scale (or one per row); q[r, cols..ldq) = 0.
+   Noise / Philox index r * cols + c, as orc_quantize_rows. */
+void orc_quantize_rows_ex(const float *x, int64_t rows, int64_t cols, int64_t ldx, const float *row_mul,
+                          const void *mask, int64_t ldm, int mask_mode, const float *scales, int per_row,
+                          int8_t *q, int64_t ldq, int mode, const float *noise, uint64_t seed,
+                          uint64_t offset) {
+#pragma omp parallel for schedule(static)
+    for (int64_t r = 0; r < rows; ++r) {
+        const float rs = rscale_of(per_row ? scales[r] : scales[0]);
+        for (int64_t c = 0; c < cols; ++c) {
+            const float v = masked_elem(x[r * ldx + c], mask, ldm, mask_mode, r, c);
+            volatile float t = row_mul ? v * row_mul[r] : v;
+            float u = 0.0f;
+            const int64_t lin = r * cols + c;
+            if (mode == ORC_ROUND_STOCHASTIC)
+                u = noise ? noise[lin] : orc_philox_uniform(seed, offset + (uint64_t)lin);
+            q[r * ldq + c] = quant_one(t, rs, mode, u);
+        }
+        for (int64_t c = cols; c < ldq; ++c) q[r * ldq + c] = 0;
+    }
+}
+
+/* Forward GEMM on operands that are already int8 (the cached-input form of cuda/QLinear.py's
+   forward and the second of two chained layers): Y = (sA*sB) * float(A . B^T) (+ bias), optional
+   scaleY = max|Y| / 127.  Epilogue as orc_qgemm_fwd (cuda/src/epilogue.h:62-100). */
+void orc_qgemm_i8_nt(float *Y, int64_t ldy, const int8_t *A, int64_t lda, const int8_t *B, int64_t ldb,
+                     const float *bias, float *scaleY, float sA, float sB, int64_t M, int64_t N,
+                     int64_t K) {
+    int32_t *acc = (int32_t *)malloc(sizeof(int32_t) * (size_t)(M * N > 0 ? M * N : 1));
+    igemm_nt(A, lda, B, ldb, acc, N, M, N, K);
+    volatile float s = sA * sB;
+    float m = 0.0f;
+    for (int64_t i = 0; i < M; ++i)
+        for (int64_t j = 0; j < N; ++j) {
+            float y = dequant(acc[i * N + j], s);
+            if (bias) {
+                volatile float yb = bias[j] + y;
+                y = yb;
+            }
+            Y[i * ldy + j] = y;
+            const float a = fabsf(y);
+            if (a > m) m = a;
+        }
+    if (scaleY) {
+        volatile float sy = m / 127.0f;
+        *scaleY = sy;
+    }
+    free(acc);
+}
+
+/* gradX with the backward of a folded row multiplier and an optional accumulation into dX:
+   y = (s_dY*s_W) * float(acc); y = y * row_scale[m]; dX = accumulate ? dX + y : y. */
+void orc_qgemm_bwd_dx_ex(float *dX, int64_t lddx, const int8_t *dYq, int64_t lddy, const int8_t *Wq,
+                         int64_t ldw, float s_dY, float s_W, const float *row_scale, int accumulate,
+                         int64_t M, int64_t N, int64_t K) {
+    volatile float s = s_dY * s_W;
+#pragma omp parallel for schedule(static)
+    for (int64_t m = 0; m < M; ++m)
+        for (int64_t k = 0; k < K; ++k) {
+            int64_t acc = 0;
+            for (int64_t n = 0; n < N; ++n)
+                acc += (int32_t)dYq[m * lddy + n] * (int32_t)Wq[n * ldw + k];
+            volatile float y = dequant(narrow_i32(acc), s);
+            if (row_scale) y = y * row_scale[m];
+            if (accumulate) y = dX[m * lddx + k] + y;
+            dX[m * lddx + k] = y;
+        }
+}
+
+/* copy_u aggregation with the epilogue of a GCN layer: y = s * float(sum); y = y * row_scale[r];
+   y = y + bias[f]; act 1: max(y, 0); act 2: ELU (y > 0 ? y : exp(y) - 1, libm here, the hardware
+   exponential in the shipped kernel: compared with a tolerance); sign_bits (optional, F % 16 == 0):
+   bit f % 16 of word [r, f / 16] = (y > 0). */
+void orc_spmm_csr_copy_u_ex(float *out, uint16_t *sign_bits, const int64_t *indptr,
+                            const int64_t *indices, const int8_t *feat, int64_t ldf, float scale,
+                            const float *row_scale, const float *bias, int act, int64_t rows, int64_t F) {
+#pragma omp parallel
+    {
+        int64_t *acc = (int64_t *)malloc(sizeof(int64_t) * (size_t)(F > 0 ? F : 1));
+#pragma omp for schedule(dynamic, 64)
+        for (int64_t r = 0; r < rows; ++r) {
+            for (int64_t f = 0; f < F; ++f) acc[f] = 0;
+            for (int64_t p = indptr[r]; p < indptr[r + 1]; ++p) {
+                const int8_t *u = feat + indices[p] * ldf;
+                for (int64_t f = 0; f < F; ++f) acc[f] += u[f];
+            }
+            if (sign_bits)
+                for (int64_t w = 0; w < F / 16; ++w) sign_bits[r * (F / 16) + w] = 0;
+            for (int64_t f = 0; f < F; ++f) {
+                volatile float y = scale * (float)narrow_i32(acc[f]);
+                if (row_scale) y = y * row_scale[r];
+                if (bias) y = y + bias[f];
+                if (act == 1) y = y > 0.0f ? y : 0.0f;
+                if (act == 2 && !(y > 0.0f)) y = expf(y) - 1.0f;
+                out[r * F + f] = y;
+                if (sign_bits && y > 0.0f) sign_bits[r * (F / 16) + (f >> 4)] |= (uint16_t)(1u << (f & 15));
+            }
+        }
+        free(acc);
+    }
+}
+
+/* u_mul_e aggregation with the epilogue of a GAT layer (evaluation/test_gat.py:160-165):
+   y = (scale * scale2) * float(sum) with the product of the two scales rounded first; + bias[h, f]; act. */
+void orc_spmm_csr_u_mul_e_ex(float *out, const int64_t *indptr, const int64_t *indices,
+                             const int64_t *edge_ids, const int8_t *feat, const int8_t *evals,
+                             int edge_major, float scale, const float *scale2, const float *bias, int act,
+                             int64_t rows, int64_t H, int64_t F, int64_t D, int64_t nnz) {
+    const int64_t HF = H * F;
+    volatile float s = scale2 ? scale * scale2[0] : scale;
+#pragma omp parallel
+    {
+        int64_t *acc = (int64_t *)malloc(sizeof(int64_t) * (size_t)(HF > 0 ? HF : 1));
+#pragma omp for schedule(dynamic, 64)
+        for (int64_t r = 0; r < rows; ++r) {
+            for (int64_t t = 0; t < HF; ++t) acc[t] = 0;
+            for (int64_t p = indptr[r]; p < indptr[r + 1]; ++p) {
+                const int8_t *u = feat + indices[p] * HF;
+                const int64_t e = edge_ids ? edge_ids[p] : p;
+                for (int64_t h = 0; h < H; ++h)
+                    for (int64_t f = 0; f < F; ++f) {
+                        const int64_t d = (D == 1) ? 0 : f;
+                        const int8_t ev = edge_major ? evals[(e * H + h) * D + d] : evals[(h * D + d) * nnz + e];
+                        acc[h * F + f] += (int32_t)ev * (int32_t)u[h * F + f];
+                    }
+            }
+            for (int64_t t = 0; t < HF; ++t) {
+                volatile float y = s * (float)narrow_i32(acc[t]);
+                if (bias) y = y + bias[t];
+                if (act == 1) y = y > 0.0f ? y : 0.0f;
+                if (act == 2 && !(y > 0.0f)) y = expf(y) - 1.0f;
+                out[r * HF + t] = y;
+            }
+        }
+        free(acc);
+    }
+}

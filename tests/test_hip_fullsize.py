@@ -175,6 +175,30 @@ def test_copy_u_F128_full(K, orc, big_graph):
     assert torch.equal(K.csr_SPMM(g, b, sc(1.0)) + K.csr_SPMM(g, c, sc(1.0)), K.csr_SPMM(g, b + c, sc(1.0)))
 
 
+def test_copy_u_F256_fused_epilogue_full(K, orc, big_graph):
+    """The launch the benchmark epoch runs: width 256 (two column tiles), '* norm, + bias, ReLU' and the sign
+    words in the epilogue, on the 114.8 M-edge graph; the oracle's fused form on a row sample."""
+    g = big_graph
+    F = 256
+    gen = torch.Generator("cuda").manual_seed(256)
+    feat = torch.randint(-127, 128, (N_NODES, F), dtype=torch.int8, device="cuda", generator=gen)
+    rs = g.in_degrees().float().clamp(min=1).pow(-0.5)
+    bias = torch.randn(F, device="cuda", generator=gen) * 0.05
+    bits = torch.empty((N_NODES, F // 16), dtype=torch.int16, device="cuda")
+    out = K.csr_SPMM(g, feat, sc(0.0004), row_scale=rs, bias=bias, relu=True, sign_bits=bits)
+    rows, sub_ip, sub_ix, _ = _row_sample_csr(g, 2000, 11)
+    want, wbits = orc.spmm_csr_copy_u_ex(sub_ip, sub_ix, host(feat), np.float32(0.0004), row_scale=host(rs)[rows],
+                                         bias=host(bias), act=1, want_bits=True)
+    assert np.array_equal(host(out)[rows], want)
+    assert np.array_equal(host(bits).view(np.uint16)[rows], wbits)
+    frac = float((out > 0).float().mean())
+    assert 0.2 < frac < 0.8  # the ReLU is exercised on both sides
+    # reverse orientation, no epilogue: the backward launch of the epoch
+    out_r = K.csr_SPMM(g, feat, sc(0.0004), reverse=True)
+    rows, sub_ip, sub_ix, _ = _row_sample_csr(g, 1000, 12, reverse=True)
+    assert np.array_equal(host(out_r)[rows], orc.spmm_csr_copy_u(sub_ip, sub_ix, host(feat), np.float32(0.0004)))
+
+
 @pytest.mark.parametrize("H,F", [(8, 1), (2, 128)])
 def test_u_mul_e_full_real_edge_weights(K, orc, big_graph, H, F):
     """u_mul_e on the 114.8 M-edge graph with the edge weights 1/sqrt(deg_u deg_v) quantized by

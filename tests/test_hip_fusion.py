@@ -84,30 +84,35 @@ def test_absmax_with_row_multiplier_on_dense_rows_of_even_length(K, orc, rows, c
 
 # (n, e): rows of ~66 slots (one wave per row), and a sparse graph with a long row and a hub row (the epilogue
 # also runs in the sixteen-wave kernel and in the hub store pass)
-@pytest.mark.parametrize("n,e", [(600, 40000), (5000, 40000)])
+@pytest.mark.parametrize("n,e", [(600, 40000), (5000, 40000), (3000, 9000)])
 @pytest.mark.parametrize("F", [16, 41, 256])
-def test_spmm_fused_epilogue_equals_separate_passes(K, F, n, e):
+def test_spmm_fused_epilogue_matches_oracle(K, orc, F, n, e):
+    """The aggregation with '* row_scale, + bias, activation, sign bits' in its epilogue against the oracle's
+    fused form, on rows of ~66 slots (one wave per row), on a sparse graph with a long row and a hub row (the
+    epilogue also runs in the sixteen-wave kernel and in the hub store pass) and on a very sparse graph (the
+    slot-span kernels)."""
     rng = np.random.default_rng(F)
     src, dst = rand_graph(rng, n, e)
     if n == 5000:
         dst[:9000] = 5
         dst[9000:10500] = 6
     g = make_graph(src, dst, n)
-    feat = dev(rng.integers(-127, 128, (n, F)).astype(np.int8))
-    rs = dev(rng.random(n, dtype=np.float32) + 0.05)
-    bias = dev(rng.standard_normal(F).astype(np.float32))
-    s = sc(0.0173)
-    base = K.csr_SPMM(g, feat, s)
-    assert torch.equal(K.csr_SPMM(g, feat, s, row_scale=rs), base * rs.unsqueeze(1))
-    assert torch.equal(K.csr_SPMM(g, feat, s, bias=bias), base + bias)
-    assert torch.equal(K.csr_SPMM(g, feat, s, relu=True), torch.relu(base))
-    want = torch.relu(base * rs.unsqueeze(1) + bias)
-    assert torch.equal(K.csr_SPMM(g, feat, s, row_scale=rs, bias=bias, relu=True), want)
+    ip, ix = host(g.adj_csc[0]), host(g.adj_csc[1])
+    feat = rng.integers(-127, 128, (n, F)).astype(np.int8)
+    rs = rng.random(n, dtype=np.float32) + 0.05
+    bias = rng.standard_normal(F).astype(np.float32)
+    s = np.float32(0.0173)
+    for kw in ({}, {"row_scale": rs}, {"bias": bias}, {"act": 1}, {"row_scale": rs, "bias": bias, "act": 1}):
+        want = orc.spmm_csr_copy_u_ex(ip, ix, feat, s, **kw)
+        dkw = {k: dev(v) for k, v in kw.items() if k != "act"}
+        got = K.csr_SPMM(g, dev(feat), sc(s), relu=bool(kw.get("act")), **dkw)
+        assert np.array_equal(host(got), want), sorted(kw)
     if F % 16 == 0:  # the epilogue also writes the signs of its output, sixteen columns per word
+        want, wbits = orc.spmm_csr_copy_u_ex(ip, ix, feat, s, row_scale=rs, bias=bias, act=1, want_bits=True)
         bits = torch.full((n, F // 16), -1, dtype=torch.int16, device="cuda")
-        assert torch.equal(K.csr_SPMM(g, feat, s, row_scale=rs, bias=bias, relu=True, sign_bits=bits), want)
-        got = np.unpackbits(host(bits).view(np.uint8).reshape(n, F // 16, 2), axis=-1, bitorder="little").reshape(n, F)
-        assert np.array_equal(got.astype(bool), host(want) > 0)
+        got = K.csr_SPMM(g, dev(feat), sc(s), row_scale=dev(rs), bias=dev(bias), relu=True, sign_bits=bits)
+        assert np.array_equal(host(got), want)
+        assert np.array_equal(host(bits).view(np.uint16), wbits)
 
 
 def test_gemm_row_scale_prologue_and_gradx_epilogue(K, orc):

@@ -393,3 +393,103 @@ def test_edge_softmax_properties(orc):
         out = out.index_copy(0, m, torch.softmax(z[m], 0))
     out.backward(torch.from_numpy(da).double())
     assert np.allclose(de, xt.grad.float().numpy(), atol=1e-5, rtol=1e-4)
+
+
+# ------------------------------------------------------------ fused forms
+# Each fused oracle function must equal the chain of separate numpy fp32 passes (one IEEE rounding per
+# operation, numpy never contracts) over the unfused oracle function that is pinned above.
+def _csr(rng, n, e):
+    src, dst = rand_graph(rng, n, e)
+    order = np.argsort(dst, kind="stable")
+    indptr = np.zeros(n + 1, np.int64)
+    np.cumsum(np.bincount(dst, minlength=n), out=indptr[1:])
+    return indptr, src[order], order.astype(np.int64)
+
+
+def test_fused_copy_u_epilogue_is_the_chain_of_separate_passes(orc):
+    rng = np.random.default_rng(21)
+    n, F = 300, 48
+    indptr, indices, _ = _csr(rng, n, 5000)
+    feat = rng.integers(-127, 128, (n, F)).astype(np.int8)
+    rs = (rng.random(n) + 0.05).astype(np.float32)
+    bias = rng.standard_normal(F).astype(np.float32)
+    s = np.float32(0.0173)
+    base = orc.spmm_csr_copy_u(indptr, indices, feat, s)
+    assert np.array_equal(orc.spmm_csr_copy_u_ex(indptr, indices, feat, s), base)
+    assert np.array_equal(orc.spmm_csr_copy_u_ex(indptr, indices, feat, s, row_scale=rs), base * rs[:, None])
+    assert np.array_equal(orc.spmm_csr_copy_u_ex(indptr, indices, feat, s, bias=bias), base + bias)
+    chain = base * rs[:, None] + bias
+    out, bits = orc.spmm_csr_copy_u_ex(indptr, indices, feat, s, row_scale=rs, bias=bias, act=1, want_bits=True)
+    assert np.array_equal(out, np.maximum(chain, 0))
+    unpacked = np.unpackbits(bits.view(np.uint8).reshape(n, F // 16, 2), axis=-1, bitorder="little").reshape(n, F)
+    assert np.array_equal(unpacked.astype(bool), chain > 0)
+    # a dropped row scale, a bias added before the row scale or a mask taken before the bias all fail this
+    assert not np.array_equal(out, np.maximum((base + bias) * rs[:, None], 0))
+    elu = orc.spmm_csr_copy_u_ex(indptr, indices, feat, s, row_scale=rs, bias=bias, act=2)
+    want = np.where(chain > 0, chain, np.expm1(chain.astype(np.float64)))
+    np.testing.assert_allclose(elu, want, rtol=1e-6, atol=1e-6)
+
+
+def test_fused_u_mul_e_epilogue(orc):
+    rng = np.random.default_rng(22)
+    n, H, F = 200, 3, 8
+    indptr, indices, eids = _csr(rng, n, 3000)
+    feat = rng.integers(-127, 128, (n, H, F)).astype(np.int8)
+    ev = rng.integers(-127, 128, (3000, H, 1)).astype(np.int8)  # edge-major
+    evT = np.ascontiguousarray(ev.reshape(3000, H).T).reshape(H, 1, 3000)
+    sN, sE = np.float32(0.011), np.float32(0.0007)
+    bias = rng.standard_normal(H * F).astype(np.float32)
+    base = orc.spmm_csr_u_mul_e(indptr, indices, eids, feat, evT, np.float32(sN * sE))
+    got = orc.spmm_csr_u_mul_e_ex(indptr, indices, eids, feat, ev, sN, scale2=sE, edge_major=True)
+    assert np.array_equal(got, base)
+    got = orc.spmm_csr_u_mul_e_ex(indptr, indices, eids, feat, evT, sN, scale2=sE, bias=bias, act=1)
+    assert np.array_equal(got, np.maximum(base + bias.reshape(1, H, F), 0))
+
+
+def test_masked_absmax_and_quantize(orc):
+    rng = np.random.default_rng(23)
+    rows, cols = 257, 48
+    x = rng.standard_normal((rows, cols)).astype(np.float32)
+    act_out = rng.standard_normal((rows, cols)).astype(np.float32)
+    act_out[rng.random((rows, cols)) < 0.1] = 0.0  # exact zeros belong to the masked side
+    rm = (rng.random(rows) + 0.1).astype(np.float32)
+    relu_x = np.where(act_out > 0, x, np.float32(0))
+    elu_x = np.where(act_out > 0, x, x * (act_out + np.float32(1)))
+    packed = np.packbits((act_out > 0).reshape(rows, cols // 16, 16), axis=-1, bitorder="little").view(np.uint16)
+    packed = packed.reshape(rows, cols // 16)
+    for mask, mode, xm in ((act_out, "relu", relu_x), (act_out, "elu", elu_x), (packed, "bits", relu_x), (None, "relu", x)):
+        for row_mul in (None, rm):
+            y = xm if row_mul is None else xm * row_mul[:, None]
+            s, cs = orc.absmax_ex(x, row_mul=row_mul, mask=mask, mask_mode=mode, want_colsum=True)
+            assert s == orc.absmax_scale(y)
+            np.testing.assert_allclose(cs, xm.astype(np.float64).sum(0), rtol=1e-12)
+            for kw in ({"mode": orc.RNE}, {"mode": orc.STOCHASTIC, "seed": 5, "offset": 1 << 40}):
+                q = orc.quantize_rows_ex(x, s, row_mul=row_mul, mask=mask, mask_mode=mode, ldq=64, **kw)
+                assert np.array_equal(q[:, :cols], orc.quantize(y, s, **kw)) and not q[:, cols:].any()
+
+
+def test_int8_input_forward_and_accumulating_gradx(orc):
+    rng = np.random.default_rng(24)
+    M, K, N = 70, 100, 24
+    A = rng.integers(-127, 128, (M, K)).astype(np.int8)
+    B = rng.integers(-127, 128, (N, K)).astype(np.int8)
+    bias = rng.standard_normal(N).astype(np.float32)
+    sA, sB = np.float32(0.013), np.float32(0.0021)
+    acc = A.astype(np.int64) @ B.astype(np.int64).T
+    want = np.float32(sA * sB) * acc.astype(np.float32) + bias
+    Y, sY = orc.qgemm_i8_nt(A, B, sA, sB, bias=bias, reduce=True)
+    assert np.array_equal(Y, want) and sY == orc.absmax_scale(want)
+    # the int8 operands of the fp32-input forward give the same result through this entry
+    X = rng.standard_normal((M, K)).astype(np.float32)
+    W = rng.standard_normal((N, K)).astype(np.float32)
+    Yf, Xq, Wq, sX, sW, _ = orc.qgemm_fwd(X, W, bias=bias, reduce=True)
+    assert np.array_equal(orc.qgemm_i8_nt(Xq, Wq, sX, sW, bias=bias), Yf)
+    # gradX: row scale in the epilogue, then one fp32 add into the running gradient
+    dY = rng.integers(-127, 128, (M, N)).astype(np.int8)
+    rs = (rng.random(M) + 0.2).astype(np.float32)
+    prev = rng.standard_normal((M, K)).astype(np.float32)
+    plain = orc.qgemm_bwd_dx(dY, B, 0.02, sB)
+    assert np.array_equal(orc.qgemm_bwd_dx_ex(dY, B, 0.02, sB), plain)
+    assert np.array_equal(orc.qgemm_bwd_dx_ex(dY, B, 0.02, sB, row_scale=rs), plain * rs[:, None])
+    assert np.array_equal(orc.qgemm_bwd_dx_ex(dY, B, 0.02, sB, row_scale=rs, accumulate_into=prev),
+                          prev + plain * rs[:, None])
