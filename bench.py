@@ -181,11 +181,14 @@ def primitives(g, K, torch):
         ms = time_op(lambda: K.QGEMM_backward(dY, Xq, Wq, s_dY, sX, sW, True, False), iters=10)
         byt = M * N + N * Kd + 4 * M * Kd
         out[tag.replace("fwd", "gradX")] = {"ms": round(ms, 4), "TOPS": round(ops / ms / 1e9, 2),
-                                            "GBps": round(byt / ms / 1e6, 1)}
+                                            "GBps": round(byt / ms / 1e6, 1),
+                                            "frac_hbm": round(byt / ms / 1e6 / HBM_PEAK_GBPS, 4)}
         ms = time_op(lambda: K.QGEMM_backward(dY, Xq, Wq, s_dY, sX, sW, False, True), iters=10)
         byt = M * (N + Kd) + 4 * N * Kd
         out[tag.replace("fwd", "gradW")] = {"ms": round(ms, 4), "TOPS": round(ops / ms / 1e9, 2),
-                                            "GBps": round(byt / ms / 1e6, 1)}
+                                            "GBps": round(byt / ms / 1e6, 1),
+                                            "frac_hbm": round(byt / ms / 1e6 / HBM_PEAK_GBPS, 4),
+                                            "frac_i8_mfma": round(ops / ms / 1e9 / 5000.0, 4)}
         del X, W, Xq, dY
     # the two call patterns of evaluation/test_cache_GEMM.py and evaluation/test_fuse.py at the first layer's shape:
     # the forward on an input that was quantized once before (several consumers share it), and the output scale

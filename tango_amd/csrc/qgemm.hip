@@ -208,8 +208,8 @@ __global__ __launch_bounds__(256, 2) void gemm_nt_kernel(const NtParams p) {
 }
 
 // NT kernel with the small operand stationary in LDS, for reductions of at most 256 (four k-steps).
-// A persistent workgroup of WAVES waves first copies its 16 * NT rows of the packed B into LDS (row pitch
-// an odd number of 16-byte units: the sixteen rows of a fragment read start in different bank quads) and
+// A persistent workgroup of WAVES waves first copies its 16 * NT rows of the packed B into LDS (in fragment
+// order: the 1 KB a wave reads for one MFMA is contiguous, lane after lane) and
 // then never synchronises again: the 16-row tiles of A are dealt round-robin over all waves of the
 // launch, a wave loads the whole 16 x K tile as its A fragments (and the next tile's while it works on
 // this one), reads the B fragments from LDS, and stores 16 rows x 16 NT columns.  The kernels above pay
@@ -219,15 +219,19 @@ __global__ __launch_bounds__(256, 2) void gemm_nt_kernel(const NtParams p) {
 // EPI 0: the tile goes to C as fp32.  EPI 1: nothing is stored, only max|C| / 127 is found.  EPI 2: the tile
 // is rounded to int8 with the scale q_scale and goes to Cq (the fp32 values are the same in all three, so
 // 1 then 2 store exactly what a quantize pass over the fp32 output of 0 would).
-template <int NT, int VEC, int WAVES, int EPI = 0>
-__global__ __launch_bounds__(64 * WAVES) void gemm_nts_kernel(const NtParams p, int ntiles, int pitch) {
-    extern __shared__ __attribute__((aligned(16))) int8_t b_lds[];  // [16 NT][pitch]
+template <int NT, int VEC, int WAVES, int EPI = 0, int PASSES = 1>
+__global__ __launch_bounds__(64 * WAVES) void gemm_nts_kernel(const NtParams p, int ntiles) {
+    // B in fragment order: block (j, st) of 1 KB holds, at 16 lane bytes, the 16 bytes lane `lane` feeds the MFMA
+    // of column tile j at k-step st, so a fragment read is one linear 1 KB sweep (no bank conflicts by construction)
+    extern __shared__ __attribute__((aligned(16))) int8_t b_lds[];  // [PASSES NT][ksteps][64 lanes][16]
     constexpr int KS = 4;
+    constexpr int TT = NT * PASSES;  // column tiles of the block: a wave walks them NT at a time (PASSES rounds over
+                                     // one A tile held in registers), so that the accumulators stay at 4 NT registers
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int g = lane >> 4, r16 = lane & 15;
-    const int64_t n0 = static_cast<int64_t>(blockIdx.y) * (16 * NT);
+    const int64_t n0 = static_cast<int64_t>(blockIdx.y) * (16 * TT);
     const int ksteps = static_cast<int>((p.Kr + 63) >> 6);  // <= KS (host)
     // Which column of the block the LDS row n = 16 j + 4 g + v (column 4 g + v of MFMA tile j) stands for.  A lane
     // holds columns 4 g .. 4 g + 3 of every tile: four output bytes in the int8 epilogue.  There the tiles of a
@@ -240,18 +244,18 @@ __global__ __launch_bounds__(64 * WAVES) void gemm_nts_kernel(const NtParams p, 
         return 64 * (j >> 2) + 16 * gq + 4 * (j & 3) + v;
     };
     {
-        const int cpr = pitch >> 4;
         const int kchunks = ksteps * 4;  // 16-byte chunks of a packed row that hold data or its zero fill
-        for (int idx = tid; idx < 16 * NT * cpr; idx += 64 * WAVES) {
-            const int n = idx / cpr, c = idx - n * cpr;
+        for (int idx = tid; idx < 16 * TT * kchunks; idx += 64 * WAVES) {
+            const int n = idx / kchunks, c = idx - n * kchunks;
             i32x4 v{0, 0, 0, 0};
             const int64_t nb = n0 + lds_row_column(n);
-            if (nb < p.N && c < kchunks) v = *reinterpret_cast<const i32x4*>(p.B + nb * p.ldb + c * 16);
-            *reinterpret_cast<i32x4*>(b_lds + n * pitch + c * 16) = v;
+            if (nb < p.N) v = *reinterpret_cast<const i32x4*>(p.B + nb * p.ldb + c * 16);
+            // row n = 16 j + r16, chunk c = 4 st + g  ->  block (j, st), lane 16 g + r16
+            *reinterpret_cast<i32x4*>(b_lds + ((((n >> 4) * ksteps + (c >> 2)) << 6) + ((c & 3) << 4) + (n & 15)) * 16) = v;
         }
     }
-    float* bias_lds = reinterpret_cast<float*>(b_lds + 16 * NT * pitch);  // [16 NT], zero where there is none
-    for (int n = tid; n < 16 * NT; n += 64 * WAVES) {
+    float* bias_lds = reinterpret_cast<float*>(b_lds + TT * ksteps * 1024);  // [16 TT], zero where there is none
+    for (int n = tid; n < 16 * TT; n += 64 * WAVES) {
         const int64_t nb = n0 + lds_row_column(n);
         bias_lds[n] = (p.bias && nb < p.N) ? p.bias[nb] : 0.0f;
     }
@@ -281,8 +285,20 @@ __global__ __launch_bounds__(64 * WAVES) void gemm_nts_kernel(const NtParams p, 
     float rsc, rsc_nxt;
     int t = static_cast<int>(blockIdx.x) * WAVES + wave;
     load_tile(cur, rsc, t);
+    // fp32 output with nothing but the dequantization (and the optional row scale) in the epilogue: the common case
+    // gets a loop without a branch per tile (the general loop below tests six uniform conditions per column tile)
+    const bool plain = EPI == 0 && !p.bias && !p.accumulate && wide == 4;
+    const bool want_max = EPI == 1 || (EPI == 0 && p.absmax_out != nullptr);
+    // columns of this block, as a 32-bit count: the bounds tests of the epilogue are 32-bit compares
+    const int ncols = static_cast<int>(p.N - n0 < 16 * TT ? p.N - n0 : 16 * TT);
+    // columns that may be written: a row's padding up to its pitch takes the zeros of the zero-filled rows of B
+    const int wcols = EPI == 0 ? static_cast<int>(p.ldc - n0 < 16 * TT ? p.ldc - n0 : 16 * TT) : ncols;
     for (; t < ntiles; t += stride) {
         load_tile(nxt, rsc_nxt, t + stride);
+        const int64_t row = static_cast<int64_t>(t) * 16 + r16;
+        float* crow = p.C + row * p.ldc + n0;
+#pragma unroll
+        for (int ps = 0; ps < PASSES; ++ps) {
         i32x4 acc[NT];
 #pragma unroll
         for (int j = 0; j < NT; ++j) acc[j] = i32x4{0, 0, 0, 0};
@@ -291,27 +307,54 @@ __global__ __launch_bounds__(64 * WAVES) void gemm_nts_kernel(const NtParams p, 
             if (st < ksteps) {
 #pragma unroll
                 for (int j = 0; j < NT; ++j) {
-                    const i32x4 b = *reinterpret_cast<const i32x4*>(b_lds + (16 * j + r16) * pitch + st * 64 + g * 16);
+                    const i32x4 b = *reinterpret_cast<const i32x4*>(b_lds + ((((ps * NT + j) * ksteps + st) << 6) + lane) * 16);
                     acc[j] = mfma_16x16x64(b, cur[st], acc[j]);  // operands swapped, see gemm_nt_kernel
                 }
             }
         }
-        // lane holds C[16 t + r16][n0 + 16 j + 4 g + v] (PERM: the column lds_row_column gives)
-        const int64_t row = static_cast<int64_t>(t) * 16 + r16;
+        // lane holds C[16 t + r16][n0 + 16 (ps NT + j) + 4 g + v] (PERM: the column lds_row_column gives)
         if (row < p.M) {
-            float* crow = p.C + row * p.ldc;
+            const int c0 = ps * 16 * NT;  // first column of this pass inside the block
+            if (plain && c0 + 16 * NT <= wcols) {
+                f32x4* cp = reinterpret_cast<f32x4*>(crow + c0 + 4 * g);
+                if (want_max) {
+#pragma unroll
+                    for (int j = 0; j < NT; ++j) {
+                        const f32x4 y{(s * static_cast<float>(acc[j][0])) * rsc, (s * static_cast<float>(acc[j][1])) * rsc,
+                                      (s * static_cast<float>(acc[j][2])) * rsc, (s * static_cast<float>(acc[j][3])) * rsc};
+                        m = fmaxf(fmaxf(m, fmaxf(fabsf(y[0]), fabsf(y[1]))), fmaxf(fabsf(y[2]), fabsf(y[3])));
+                        cp[4 * j] = y;
+                    }
+                } else {
+#pragma unroll
+                    for (int j = 0; j < NT; ++j)
+                        cp[4 * j] = f32x4{(s * static_cast<float>(acc[j][0])) * rsc, (s * static_cast<float>(acc[j][1])) * rsc,
+                                          (s * static_cast<float>(acc[j][2])) * rsc, (s * static_cast<float>(acc[j][3])) * rsc};
+                }
+                continue;
+            }
             uint32_t qw[4];
 #pragma unroll
             for (int j = 0; j < NT; ++j) {
-                const int64_t col = PERM ? n0 + 64 * (j >> 2) + 16 * g + 4 * (j & 3) : n0 + j * 16 + g * 4;
+                const int cl = c0 + (PERM ? 64 * (j >> 2) + 16 * g + 4 * (j & 3) : j * 16 + g * 4);  // column inside the block
+                const int col = cl;  // relative to crow / qrow, which start at the block's first column
+                const bool full = cl + 4 <= ncols;
                 float y[4];
-                const f32x4 bv = *reinterpret_cast<const f32x4*>(bias_lds + j * 16 + g * 4);
+                const f32x4 bv = *reinterpret_cast<const f32x4*>(bias_lds + c0 + j * 16 + g * 4);
 #pragma unroll
                 for (int v = 0; v < 4; ++v) {
                     y[v] = s * static_cast<float>(acc[j][v]);
                     if (p.row_scale) y[v] = y[v] * rsc;
                     if (p.bias) y[v] = bv[v] + y[v];
-                    if (EPI != 2 && col + v < p.N) m = fmaxf(m, fabsf(y[v]));
+                }
+                if (want_max) {  // uniform
+                    if (full) {
+                        m = fmaxf(fmaxf(m, fmaxf(fabsf(y[0]), fabsf(y[1]))), fmaxf(fabsf(y[2]), fabsf(y[3])));
+                    } else {
+#pragma unroll
+                        for (int v = 0; v < 4; ++v)
+                            if (cl + v < ncols) m = fmaxf(m, fabsf(y[v]));
+                    }
                 }
                 if (EPI == 1) continue;
                 if (EPI == 2) {
@@ -323,54 +366,55 @@ __global__ __launch_bounds__(64 * WAVES) void gemm_nts_kernel(const NtParams p, 
 #pragma unroll
                         for (int v = 0; v < 4; ++v) q[v] = quant_one<TANGO_ROUND_RNE>(y[v], qr, 0.0f);
                     }
-                    int8_t* qrow = p.Cq + row * p.ldcq;
+                    int8_t* qrow = p.Cq + row * p.ldcq + n0;
                     if (PERM) {
                         qw[j & 3] = pack4(q[0], q[1], q[2], q[3]);
                         if ((j & 3) != 3) continue;
-                        const int64_t col0 = col - 12;  // n0 + 64 (j / 4) + 16 g
-                        if (col0 + 16 <= p.N && q16) {
+                        const int col0 = col - 12;  // 64 (j / 4) + 16 g
+                        if (col0 + 16 <= ncols && q16) {
                             typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
                             *reinterpret_cast<u32x4*>(qrow + col0) = u32x4{qw[0], qw[1], qw[2], qw[3]};
                         } else {
 #pragma unroll
                             for (int b = 0; b < 16; ++b)
-                                if (col0 + b < p.N) qrow[col0 + b] = static_cast<int8_t>(qw[b >> 2] >> (8 * (b & 3)));
+                                if (col0 + b < ncols) qrow[col0 + b] = static_cast<int8_t>(qw[b >> 2] >> (8 * (b & 3)));
                         }
                         continue;
                     }
-                    if (col + 4 <= p.N && qwide) {
+                    if (full && qwide) {
                         *reinterpret_cast<uint32_t*>(qrow + col) = pack4(q[0], q[1], q[2], q[3]);
                     } else {
 #pragma unroll
                         for (int v = 0; v < 4; ++v)
-                            if (col + v < p.N) qrow[col + v] = static_cast<int8_t>(q[v]);
+                            if (cl + v < ncols) qrow[col + v] = static_cast<int8_t>(q[v]);
                     }
                     continue;
                 }
                 if (p.accumulate) {  // uniform
-                    if (col + 4 <= p.N && wide == 4) {
+                    if (full && wide == 4) {
                         const f32x4 o = *reinterpret_cast<const f32x4*>(crow + col);
                         *reinterpret_cast<f32x4*>(crow + col) = f32x4{o[0] + y[0], o[1] + y[1], o[2] + y[2], o[3] + y[3]};
                     } else {
 #pragma unroll
                         for (int v = 0; v < 4; ++v)
-                            if (col + v < p.N) crow[col + v] += y[v];
+                            if (cl + v < ncols) crow[col + v] += y[v];
                     }
                     continue;
                 }
-                if (col + 4 <= p.N && wide == 4) {
+                if (full && wide == 4) {
                     *reinterpret_cast<f32x4*>(crow + col) = f32x4{y[0], y[1], y[2], y[3]};
-                } else if (col + 4 <= p.N && wide == 2) {
+                } else if (full && wide == 2) {
                     typedef float f32x2 __attribute__((ext_vector_type(2)));
                     *reinterpret_cast<f32x2*>(crow + col) = f32x2{y[0], y[1]};
                     *reinterpret_cast<f32x2*>(crow + col + 2) = f32x2{y[2], y[3]};
                 } else {
 #pragma unroll
                     for (int v = 0; v < 4; ++v)
-                        if (col + v < p.N) crow[col + v] = y[v];
+                        if (cl + v < ncols) crow[col + v] = y[v];
                 }
             }
         }
+        }  // passes
 #pragma unroll
         for (int st = 0; st < KS; ++st) cur[st] = nxt[st];
         rsc = rsc_nxt;
@@ -619,8 +663,8 @@ __global__ __launch_bounds__(256, 2) void gemm_fq_kernel(const FqParams p) {
 // MFMAs and the Y stores of different waves overlap.  NT = 16-column tiles (N <= 16 NT).
 // (For wide outputs the accumulators of all N columns leave too few registers for the prefetch
 // and gemm_fq_kernel's LDS-staged form is faster: 0.30 ms against 0.49 ms at 232,965 x 602 x 256.)
-template <int NT, int XV, int MODE>
-__global__ __launch_bounds__(768) void gemm_ws_kernel(const FqParams p, int nblocks, int pitch, int kq) {
+template <int NT, int XV, int MODE, int THREADS>
+__global__ __launch_bounds__(THREADS) void gemm_ws_kernel(const FqParams p, int nblocks, int pitch, int kq) {
     extern __shared__ __attribute__((aligned(16))) int8_t w_lds[];  // [16 NT][pitch]
     constexpr int RT = 1;
     const int tid = threadIdx.x;
@@ -630,7 +674,7 @@ __global__ __launch_bounds__(768) void gemm_ws_kernel(const FqParams p, int nblo
     // ---- W -> LDS, rows beyond N and chunks beyond kq zero-filled
     {
         const int cpr = pitch >> 4;  // 16-byte chunks per LDS row
-        for (int idx = tid; idx < 16 * NT * cpr; idx += 768) {
+        for (int idx = tid; idx < 16 * NT * cpr; idx += THREADS) {
             const int n = idx / cpr, c = idx - n * cpr;
             i32x4 v{0, 0, 0, 0};
             if (n < p.N && c * 16 < kq) v = *reinterpret_cast<const i32x4*>(p.B + static_cast<int64_t>(n) * p.ldb + c * 16);
@@ -1022,35 +1066,55 @@ static int row_vec(const int8_t* p, int64_t ld, int64_t cols, int64_t* readable)
     return 1;
 }
 
+constexpr size_t kLdsBytes = 160 * 1024;
+
 // The stationary form (reduction <= 256, A rows readable in 4- or 16-byte pieces).  EPI: what the epilogue does
 // with the dequantized tile (see gemm_nts_kernel).  False when the launch could not be set up.
 template <int VEC, int EPI>
 static bool launch_nts(const NtParams& p, hipStream_t s) {
-    constexpr int WAVES = 12;
     const int64_t n16 = ceil_div(p.N, 16);
-    const int ny = static_cast<int>(ceil_div(n16, 16));
-    const int nt = static_cast<int>(ceil_div(n16, ny));
-    const int pitch = 16 * ((static_cast<int>(ceil_div(p.Kr, 64)) * 4) | 1);
+    const int ksteps = static_cast<int>(ceil_div(p.Kr, 64));
     const int ntiles = static_cast<int>(ceil_div(p.M, 16));
-    int gx = compute_units() / ny;
-    if (gx > ceil_div(ntiles, WAVES)) gx = static_cast<int>(ceil_div(ntiles, WAVES));
-    if (gx < 1) gx = 1;
-#define TANGO_NTS(NT_)                                                                                          \
+    // One column block wherever the whole small operand fits the LDS (up to 38 tiles at four k-steps): a wave
+    // then writes whole output rows, in two rounds of half the tiles over the A tile it holds.  Cutting the
+    // columns over workgroups makes rows arrive in pieces from different compute units at different times, which
+    // a store-only kernel of that shape shows at half the rate (232,960 x 608 fp32: 3.3 TB/s in three blocks of
+    // 13 tiles against 6.6 TB/s for whole rows).  Wider outputs are cut into blocks of sixteen tiles, which meet
+    // on 1 KB boundaries.
+    const bool two_rounds = EPI == 0 && n16 > 16 && n16 <= 38 &&
+                            n16 * (ksteps * 1024 + 64) + 256 <= static_cast<int64_t>(kLdsBytes);
+    int ny = 1;
+    int64_t nt = n16;
+    if (!two_rounds && n16 > 16) {
+        ny = static_cast<int>(ceil_div(n16, 16));
+        nt = 16;
+    }
+#define TANGO_NTS(NT_, PASSES_)                                                                                 \
     do {                                                                                                        \
+        constexpr int WAVES = 12;                                                                               \
+        int gx = compute_units() / ny;                                                                          \
+        if (gx > ceil_div(ntiles, WAVES)) gx = static_cast<int>(ceil_div(ntiles, WAVES));                       \
+        if (gx < 1) gx = 1;                                                                                     \
         /* more than 64 KB of dynamic LDS has to be asked for once per kernel */                                \
         static const bool ok =                                                                                  \
-            hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_nts_kernel<NT_, VEC, WAVES, EPI>),          \
-                                hipFuncAttributeMaxDynamicSharedMemorySize, 80 * 1024) == hipSuccess;           \
+            hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_nts_kernel<NT_, VEC, WAVES, EPI, PASSES_>), \
+                                hipFuncAttributeMaxDynamicSharedMemorySize,                                     \
+                                static_cast<int>(kLdsBytes - 256)) == hipSuccess;                               \
         if (!ok) return false;                                                                                  \
-        hipLaunchKernelGGL((gemm_nts_kernel<NT_, VEC, WAVES, EPI>), dim3(gx, ny), dim3(64 * WAVES),             \
-                           static_cast<size_t>(16 * NT_) * (pitch + 4), s, p, ntiles, pitch);                   \
+        hipLaunchKernelGGL((gemm_nts_kernel<NT_, VEC, WAVES, EPI, PASSES_>), dim3(gx, ny), dim3(64 * WAVES),    \
+                           static_cast<size_t>(NT_ * PASSES_) * (ksteps * 1024 + 64), s, p, ntiles);           \
         return true;                                                                                            \
     } while (0)
-    if (nt <= 2) TANGO_NTS(2);
-    else if (nt <= 4) TANGO_NTS(4);
-    else if (nt <= 8) TANGO_NTS(8);
-    else if (nt <= 13) TANGO_NTS(13);
-    else TANGO_NTS(16);
+    if (two_rounds) {
+        if (nt <= 24) TANGO_NTS(12, (EPI == 0 ? 2 : 1));
+        else if (nt <= 32) TANGO_NTS(16, (EPI == 0 ? 2 : 1));
+        else TANGO_NTS(19, (EPI == 0 ? 2 : 1));
+    }
+    if (nt <= 2) TANGO_NTS(2, 1);
+    else if (nt <= 4) TANGO_NTS(4, 1);
+    else if (nt <= 8) TANGO_NTS(8, 1);
+    else if (nt <= 13) TANGO_NTS(13, 1);
+    else TANGO_NTS(16, 1);
 #undef TANGO_NTS
 }
 
@@ -1100,34 +1164,36 @@ static bool fq_applicable(const float* X, int64_t ldx, const int8_t* Xq, int64_t
     return true;
 }
 
-constexpr size_t kLdsBytes = 160 * 1024;
-
-template <int NT, int XV, int MODE>
+template <int NT, int XV, int MODE, int THREADS>
 static bool launch_ws_nt(const FqParams& p, hipStream_t s) {
     const int kq = static_cast<int>(round_up(p.K, 16));
     int pitch = kq + 16;  // the extra chunk spreads the rows of a fragment read over the LDS banks
-    if (static_cast<size_t>(16 * NT) * pitch + 256 > kLdsBytes) pitch = kq;
+    if ((pitch >> 4) % 2 == 0) pitch += 16;  // an odd number of 16-byte units per row
     const size_t lds = static_cast<size_t>(16 * NT) * pitch;
     if (lds + 256 > kLdsBytes) return false;
     static const bool ok = [] {  // more than 64 KB of dynamic LDS has to be asked for once per kernel
-        return hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_ws_kernel<NT, XV, MODE>),
+        return hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_ws_kernel<NT, XV, MODE, THREADS>),
                                    hipFuncAttributeMaxDynamicSharedMemorySize,
                                    static_cast<int>(kLdsBytes - 256)) == hipSuccess;
     }();
     if (!ok) return false;
+    constexpr int WAVES = THREADS / 64;
     const int64_t nblocks = ceil_div(p.M, 16);
-    const int64_t wgs = ceil_div(nblocks, 12) < compute_units() ? ceil_div(nblocks, 12) : compute_units();
-    hipLaunchKernelGGL((gemm_ws_kernel<NT, XV, MODE>), dim3(static_cast<unsigned>(wgs)), dim3(768), lds, s, p,
+    const int64_t wgs = ceil_div(nblocks, WAVES) < compute_units() ? ceil_div(nblocks, WAVES) : compute_units();
+    hipLaunchKernelGGL((gemm_ws_kernel<NT, XV, MODE, THREADS>), dim3(static_cast<unsigned>(wgs)), dim3(THREADS), lds, s, p,
                        static_cast<int>(nblocks), pitch, kq);
     return true;
 }
 
-// W-stationary form when X is tall (at least one 16-row block per wave of the machine) and N <= 32.
+// W-stationary form when X is tall (at least one 16-row block per wave of the machine) and N <= 32.  (Wider
+// outputs were measured with this kernel too, eight or twelve waves per compute unit and 4 NT accumulator
+// registers per lane: 232,965 x 602 x 256 0.336 ms against 0.29 ms for gemm_fq_kernel, x 256 x 41 0.098 against
+// 0.080 ms.)
 template <int XV, int MODE>
 static bool launch_ws(const FqParams& p, hipStream_t s) {
     if (p.N > 32 || ceil_div(p.M, 16) < 12LL * compute_units() || ceil_div(p.M, 16) > INT32_MAX) return false;
-    if (p.N <= 16) return launch_ws_nt<1, XV, MODE>(p, s);
-    return launch_ws_nt<2, XV, MODE>(p, s);
+    if (p.N <= 16) return launch_ws_nt<1, XV, MODE, 768>(p, s);
+    return launch_ws_nt<2, XV, MODE, 768>(p, s);
 }
 
 // Row pitch of the forward kernel's LDS block: K rounded up to an odd number of 16-byte units, so that the

@@ -767,7 +767,15 @@ def QGEMM_backward(dY, X, W, scaledY, scaleX, scaleW, X_need=True, W_need=True, 
     if X_need:
         assert W.is_cuda, "W must be on GPU"
         assert scaleW.is_cuda, "scaleW must be on GPU"
-        dX = torch.empty(X.shape, dtype=torch.float32, device=X.device) if dX_acc is None else dX_acc
+        if dX_acc is not None:
+            dX = dX_acc
+        elif X.dim() == 2 and X.size(1) % 32 != 0 and X.size(1) > 32:
+            # rows padded to whole 128-byte lines (the [M, K] view is returned): the GEMM's 64-byte output
+            # pieces then never straddle a line, which rows of e.g. 602 floats (2408 bytes) make them do
+            ld = (X.size(1) + 31) // 32 * 32
+            dX = torch.empty((X.size(0), ld), dtype=torch.float32, device=X.device)[:, :X.size(1)]
+        else:
+            dX = torch.empty(X.shape, dtype=torch.float32, device=X.device)
         cuda_kernels.QGEMM_backward_gradX(dX, dY, W, scaledY, scaleW, row_scale=x_row_scale,
                                           accumulate=dX_acc is not None)
     if W_need:
