@@ -272,7 +272,22 @@ def _gat_step(K, torch, iters, warm):
         opt.zero_grad(set_to_none=True)
         cross_entropy(model(x), labels).backward()
         opt.step()
-    return {"gat3_step_169343n_1.34Me_ms": round(time_op(gat_step, iters=iters, warm=warm), 3)}
+    out = {"gat3_step_169343n_1.34Me_ms": round(time_op(gat_step, iters=iters, warm=warm), 3)}
+    # the stack the reference trains on this graph (evaluation/arxiv_gat.py:376-448): a residual projection in
+    # every layer, batch norm between layers, a one-head output layer, the smoothed loss; dropout off
+    from tango_amd.evaluation import arxiv_loss
+    from tango_amd.gat import ArxivGAT
+    del model, opt
+    am = ArxivGAT(128, 40, 16, 3, 8, torch.nn.functional.relu).cuda()
+    al = torch.randint(0, 40, (n,), device="cuda")
+    aopt = torch.optim.RMSprop(am.parameters(), lr=2e-3)
+
+    def arxiv_step():
+        aopt.zero_grad(set_to_none=True)
+        arxiv_loss(am(g, x), al).backward()
+        aopt.step()
+    out["arxiv_gat3_step_169343n_1.34Me_ms"] = round(time_op(arxiv_step, iters=iters, warm=warm), 3)
+    return out
 
 
 def _hgt_step(K, torch, iters, warm):
@@ -292,7 +307,28 @@ def _hgt_step(K, torch, iters, warm):
         opth.zero_grad(set_to_none=True)
         cross_entropy(hgt(g, xh), lh).backward()
         opth.step()
-    return {"hgt2_step_170000n_8.17Me_ms": round(time_op(hgt_step, iters=iters, warm=warm), 3)}
+    out = {"hgt2_step_170000n_8.17Me_ms": round(time_op(hgt_step, iters=iters, warm=warm), 3)}
+    # the same graph as a heterogeneous one: weights per node type and per relation, one SDDMM and one aggregation
+    # per relation, one softmax over all in-edges
+    from tango_amd.gat import HeteroHGTLayer, relation_graphs
+    del hgt, opth
+    sizes, rels = (100_000, 50_000, 20_000), ((0, 1), (1, 0), (1, 2), (2, 0))
+    g2, _, etype = hetero_power_law(type_sizes=sizes, relations=rels, device="cuda")
+    g2 = graph_preprocess(g2)
+    rg = relation_graphs(g2, etype, rels, sizes)
+    layers = torch.nn.ModuleList([HeteroHGTLayer(256, 256, 4, sizes, rg) for _ in range(2)]).cuda()
+    proj = torch.nn.Linear(256, 16).cuda()
+    opt2 = torch.optim.Adam(list(layers.parameters()) + list(proj.parameters()), lr=1e-3, fused=True)
+
+    def hetero_step():
+        opt2.zero_grad(set_to_none=True)
+        h = xh
+        for layer in layers:
+            h = layer(g2, h)
+        cross_entropy(proj(h), lh).backward()
+        opt2.step()
+    out["hetero_hgt2_step_170000n_8.17Me_ms"] = round(time_op(hetero_step, iters=iters, warm=warm), 3)
+    return out
 
 
 def cpu_baseline(g, X, W1, W2, frac, reps=3):

@@ -20,9 +20,9 @@ import torch
 import torch.nn as nn
 import torch.nn.functional as F
 
-from .gat import GAT, HGT
-from .gcn import GCN
-from .graph import Graph, add_self_loop, chung_lu, remove_self_loop
+from .gat import GAT, HGT, ArxivGAT, HeteroHGTLayer, QGATConv, relation_graphs
+from .gcn import GCN, ArxivGCN
+from .graph import Graph, add_self_loop, chung_lu, hetero_power_law, remove_self_loop
 from .SDDMM import sddmm_u_dot_v
 from .util import graph_preprocess
 
@@ -59,6 +59,91 @@ def load_graph_train(name, device="cuda"):
     g.ndata["train_mask"], g.ndata["val_mask"], g.ndata["test_mask"] = r < 0.6, (r >= 0.6) & (r < 0.8), r >= 0.8
     g.n_classes = classes
     return g
+
+
+ARXIV_EPSILON = 1 - math.log(2)  # evaluation/arxiv_gat.py:451
+
+
+def arxiv_loss(x, labels):
+    """The log-smoothed cross entropy of evaluation/arxiv_gat.py:528-531 and arxiv_gcn.py:224-227."""
+    y = F.cross_entropy(x, labels, reduction="none")
+    return torch.mean(torch.log(ARXIV_EPSILON + y) - math.log(ARXIV_EPSILON))
+
+
+def train_arxiv(model_name="gat", epochs=20, n_hidden=None, n_layers=3, n_heads=3, lr=2e-3, dropout=0.75,
+                input_drop=0.1, attn_drop=0.05, use_linear=True, dataset="ogbn-arxiv", quiet=False):
+    """evaluation/arxiv_gat.py:536-560 / arxiv_gcn.py:246-281 (``train``) on the synthetic stand-in of
+    ogbn-arxiv: the GAT or GCN stack of those scripts, the smoothed loss on the training nodes, RMSprop for the
+    GAT (arxiv_gat.py:603) and AdamW for the GCN (arxiv_gcn.py:311).  The scripts' label-reuse trick
+    (``--use-labels``) and their learning-rate warm-up are left to the caller.  Returns (mean ms per epoch
+    after the first three, final loss)."""
+    g = load_graph_train(dataset)
+    feats, labels, train_mask = g.ndata["feat"], g.ndata["label"], g.ndata["train_mask"]
+    if model_name == "gat":
+        model = ArxivGAT(feats.size(1), g.n_classes, n_hidden or 250, n_layers, n_heads, F.relu, dropout=dropout,
+                         input_drop=input_drop, attn_drop=attn_drop).cuda()
+        opt = torch.optim.RMSprop(model.parameters(), lr=lr, weight_decay=0)
+    elif model_name == "gcn":
+        model = ArxivGCN(feats.size(1), n_hidden or 256, g.n_classes, n_layers, F.relu, min(dropout, 0.5),
+                         use_linear).cuda()
+        opt = torch.optim.AdamW(model.parameters(), lr=lr, weight_decay=0)
+    else:
+        raise ValueError("model must be gat or gcn")
+    dur, loss = [], None
+    for epoch in range(epochs):
+        model.train()
+        start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        start.record()
+        pred = model(g, feats)
+        loss = arxiv_loss(pred[train_mask], labels[train_mask])
+        opt.zero_grad()
+        loss.backward()
+        stop.record()
+        torch.cuda.synchronize()
+        opt.step()
+        if epoch >= 3:
+            dur.append(start.elapsed_time(stop))
+        if not quiet:
+            print("Epoch {:05d} | Time(ms) {:.4f} | Loss {:.4f}".format(epoch, np.mean(dur) if dur else float("nan"),
+                                                                        loss.item()))
+    return (float(np.mean(dur)) if dur else math.nan), float(loss.item())
+
+
+def train_hetero_hgt(epochs=10, hidden=256, heads=4, n_classes=16, lr=1e-3, quiet=False, **graph_kw):
+    """Two heterogeneous HGT layers (weights per node type and per relation) with a linear read-out on the
+    synthetic 3-type / 4-relation graph.  Returns (mean forward + backward ms per epoch after the first three,
+    final loss)."""
+    type_sizes = graph_kw.pop("type_sizes", (100_000, 50_000, 20_000))
+    relations = graph_kw.pop("relations", ((0, 1), (1, 0), (1, 2), (2, 0)))
+    g, _, edge_type = hetero_power_law(type_sizes=type_sizes, relations=relations, device="cuda", **graph_kw)
+    g = graph_preprocess(g)
+    rels = relation_graphs(g, edge_type, relations, type_sizes)
+    n = g.num_nodes()
+    layers = nn.ModuleList([HeteroHGTLayer(hidden, hidden, heads, type_sizes, rels) for _ in range(2)]).cuda()
+    proj = nn.Linear(hidden, n_classes).cuda()
+    gen = torch.Generator().manual_seed(77)
+    x = torch.randn(n, hidden, generator=gen).cuda()
+    labels = torch.randint(0, n_classes, (n,), generator=gen).cuda()
+    opt = torch.optim.Adam(list(layers.parameters()) + list(proj.parameters()), lr=lr)
+    dur, loss = [], None
+    for epoch in range(epochs):
+        start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        start.record()
+        h = x
+        for layer in layers:
+            h = layer(g, h)
+        loss = F.cross_entropy(proj(h), labels)
+        opt.zero_grad()
+        loss.backward()
+        stop.record()
+        torch.cuda.synchronize()
+        opt.step()
+        if epoch >= 3:
+            dur.append(start.elapsed_time(stop))
+        if not quiet:
+            print("Epoch {:05d} | Time(ms) {:.4f} | Loss {:.4f}".format(epoch, np.mean(dur) if dur else float("nan"),
+                                                                        loss.item()))
+    return (float(np.mean(dur)) if dur else math.nan), float(loss.item())
 
 
 def evaluate(model_fn, labels, mask):
@@ -121,11 +206,39 @@ def construct_negative_graph(g, k):
     return graph_preprocess(Graph(neg_src, neg_dst, g.num_nodes()))
 
 
+class _LinkPredGAT(nn.Module):
+    """evaluation/link_pred_gat.py:172-221: the GAT stack whose last layer keeps its heads ([n, heads, hidden])
+    as the node embedding that scores the edges."""
+
+    def __init__(self, num_layers, in_dim, num_hidden, heads, activation, feat_drop=0.0, attn_drop=0.0,
+                 negative_slope=0.2, residual=False):
+        super().__init__()
+        self.num_layers = num_layers
+        self.gat_layers = nn.ModuleList()
+        if num_layers > 1:
+            self.gat_layers.append(QGATConv(in_dim, num_hidden, heads[0], feat_drop, attn_drop, negative_slope,
+                                            False, activation))
+            for l in range(1, num_layers - 1):
+                self.gat_layers.append(QGATConv(num_hidden * heads[l - 1], num_hidden, heads[l], feat_drop, attn_drop,
+                                                negative_slope, residual, activation))
+            self.gat_layers.append(QGATConv(num_hidden * heads[-2], num_hidden, heads[-1], feat_drop, attn_drop,
+                                            negative_slope, residual, None))
+        else:
+            self.gat_layers.append(QGATConv(in_dim, num_hidden, heads[0], feat_drop, attn_drop, negative_slope,
+                                            residual, None))
+
+    def forward(self, g, inputs):
+        h = inputs
+        for l in range(self.num_layers - 1):
+            h = self.gat_layers[l](g, h).flatten(1)
+        return self.gat_layers[-1](g, h)  # [n, heads, hidden]
+
+
 def train_link_pred(dataset, epochs=20, hidden=256, layers=4, k=8, lr=1e-2, weight_decay=5e-4, dropout=0.5,
-                    edge_fraction=None, quiet=False):
-    """The reference's link prediction driver (evaluation/link_pred_gcn.py:137-153,172-264): a quantized GCN
-    embeds the nodes, sddmm_u_dot_v scores the graph's edges and k sampled non-edges per edge, binary cross
-    entropy separates the two.  The negative graph is rebuilt every epoch outside the timed region, as there.
+                    edge_fraction=None, quiet=False, model_name="gcn", heads=4):
+    """The reference's link prediction drivers (evaluation/link_pred_gcn.py:137-153,172-264, link_pred_gat.py:
+    172-230, link_pred_hgt.py:27-89): a quantized GCN, GAT or HGT layer embeds the nodes, sddmm_u_dot_v scores the
+    graph's edges and k sampled non-edges per edge, binary cross entropy separates the two.  The negative graph is rebuilt every epoch outside the timed region, as there.
     ``edge_fraction``: train on a random subset of the edges (the reference keeps 8 % of Reddit's).
     Returns (mean forward + backward ms per epoch after the first three, final loss)."""
     n, e, gamma, max_deg, sym, width, _, seed = DATASETS[dataset]
@@ -139,7 +252,17 @@ def train_link_pred(dataset, epochs=20, hidden=256, layers=4, k=8, lr=1e-2, weig
     g = graph_preprocess(Graph(*add_self_loop(*remove_self_loop(src, dst), n), n))  # link_pred_gcn.py:213-216
     width -= width % 4  # "trim features to fit in k%4" (link_pred_gcn.py:206-208)
     feats = torch.randn(n, width, generator=torch.Generator().manual_seed(1000 + seed)).cuda()
-    model = GCN(g, width, hidden, hidden, layers, torch.relu, dropout).cuda()
+    if model_name == "gcn":
+        model = GCN(g, width, hidden, hidden, layers, torch.relu, dropout).cuda()
+        embed = lambda: model(feats).unsqueeze(1)
+    elif model_name == "gat":  # link_pred_gat.py:172-221; heads of the last layer stay separate in the score
+        model = _LinkPredGAT(layers, width, hidden, [heads] * layers, F.elu).cuda()
+        embed = lambda: model(g, feats)
+    elif model_name == "hgt":  # link_pred_hgt.py:27-75: one layer, its output as a one-head embedding
+        model = HGT(width, hidden, heads).cuda()
+        embed = lambda: model(g, feats).unsqueeze(1)
+    else:
+        raise ValueError("model must be gcn, gat or hgt")
     opt = torch.optim.Adam(model.parameters(), lr=lr, weight_decay=weight_decay)
     dur, loss = [], None
     for epoch in range(epochs):
@@ -147,7 +270,7 @@ def train_link_pred(dataset, epochs=20, hidden=256, layers=4, k=8, lr=1e-2, weig
         neg = construct_negative_graph(g, k)
         start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         start.record()
-        h = model(feats).unsqueeze(1)
+        h = embed()
         pos_score = sddmm_u_dot_v.apply(g, h, h)
         neg_score = sddmm_u_dot_v.apply(neg, h, h)
         score = torch.cat([pos_score, neg_score])
@@ -169,7 +292,8 @@ def train_link_pred(dataset, epochs=20, hidden=256, layers=4, k=8, lr=1e-2, weig
 
 def main():
     ap = argparse.ArgumentParser(description="quantized GCN / GAT / HGT training on a synthetic stand-in of a dataset")
-    ap.add_argument("--model", choices=["gcn", "gat", "hgt", "linkpred"], default="gcn")
+    ap.add_argument("--model", choices=["gcn", "gat", "hgt", "linkpred", "linkpred-gat", "linkpred-hgt", "arxiv-gat",
+                                        "arxiv-gcn", "hetero-hgt"], default="gcn")
     ap.add_argument("--k", type=int, default=8, help="negative samples per edge (linkpred)")
     ap.add_argument("--dataset", choices=sorted(DATASETS), default="pubmed")
     ap.add_argument("--epochs", type=int, default=20)
@@ -179,9 +303,15 @@ def main():
     ap.add_argument("--lr", type=float, default=1e-2)
     ap.add_argument("--weight-decay", type=float, default=5e-4)
     args = ap.parse_args()
-    if args.model == "linkpred":
-        ms, loss = train_link_pred(args.dataset, args.epochs, args.n_hidden or 256, args.n_layers or 4, args.k, args.lr,
-                                   args.weight_decay)
+    if args.model.startswith("linkpred"):
+        which = args.model.partition("-")[2] or "gcn"
+        ms, loss = train_link_pred(args.dataset, args.epochs, args.n_hidden or (256 if which != "gat" else 64),
+                                   args.n_layers or (4 if which == "gcn" else 2), args.k, args.lr, args.weight_decay,
+                                   model_name=which, heads=min(args.num_heads, 4))
+    elif args.model.startswith("arxiv"):
+        ms, loss = train_arxiv(args.model.partition("-")[2], args.epochs, args.n_hidden, args.n_layers or 3)
+    elif args.model == "hetero-hgt":
+        ms, loss = train_hetero_hgt(args.epochs, args.n_hidden or 256, min(args.num_heads, 4))
     else:
         ms, loss = train(args.model, args.dataset, args.epochs, args.n_hidden, args.n_layers, args.num_heads, args.lr,
                          args.weight_decay)

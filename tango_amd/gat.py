@@ -177,6 +177,175 @@ class HGTLayer(nn.Module):
 HGT = HGTLayer  # the reference's name (evaluation/test_HGT.py:27)
 
 
+class ArxivGATConv(nn.Module):
+    """The attention layer of evaluation/arxiv_gat.py:63-218 on a homogeneous graph: no bias (the model adds
+    one after its last layer), a quantized residual projection of the layer's input, an optional attention
+    term for the destination (``use_attn_dst``) and the optional symmetric degree normalisation.
+    ``edge_drop`` must be 0: dropping edges needs the ``eids=`` form of the edge softmax
+    (arxiv_gat.py:191-194), which this package does not carry."""
+
+    def __init__(self, in_feats, out_feats, num_heads=1, feat_drop=0.0, attn_drop=0.0, edge_drop=0.0,
+                 negative_slope=0.2, use_attn_dst=True, residual=False, activation=None,
+                 allow_zero_in_degree=False, use_symmetric_norm=False):
+        super().__init__()
+        if edge_drop != 0.0:
+            raise NotImplementedError("ArxivGATConv: edge_drop needs an edge softmax over a subset of the edges")
+        self._num_heads, self._out_feats = num_heads, out_feats
+        self._allow_zero_in_degree, self._use_symmetric_norm = allow_zero_in_degree, use_symmetric_norm
+        self.fc = QLinear(in_feats, out_feats * num_heads, bias=False)
+        self.fc.enable_reduce()
+        self.attn_l = nn.Parameter(torch.empty(1, num_heads, out_feats))
+        self.attn_r = nn.Parameter(torch.empty(1, num_heads, out_feats)) if use_attn_dst else None
+        self.feat_drop, self.attn_drop = nn.Dropout(feat_drop), nn.Dropout(attn_drop)
+        self.negative_slope = negative_slope
+        self.res_fc = QLinear(in_feats, num_heads * out_feats, bias=False) if residual else None
+        self._activation = activation
+        gain = nn.init.calculate_gain("relu")  # arxiv_gat.py:113-124
+        nn.init.xavier_normal_(self.fc.weight, gain=gain)
+        nn.init.xavier_normal_(self.attn_l, gain=gain)
+        if self.attn_r is not None:
+            nn.init.xavier_normal_(self.attn_r, gain=gain)
+        if self.res_fc is not None:
+            nn.init.xavier_normal_(self.res_fc.weight, gain=gain)
+
+    def forward(self, graph, feat):
+        if not self._allow_zero_in_degree:  # arxiv_gat.py:131-133, answered once per graph
+            zero_in = getattr(graph, "_has_zero_in_degree", None)
+            if zero_in is None:
+                zero_in = graph._has_zero_in_degree = bool((graph.in_degrees() == 0).any())
+            assert not zero_in
+        n = feat.size(0)
+        h = self.feat_drop(feat).contiguous()
+        if self._use_symmetric_norm:  # :158-163; the product is a new tensor, so the epilogue's scale does not apply
+            self.fc.isReduce = False
+            feat_src = self.fc(h).view(n, self._num_heads, self._out_feats)
+            self.fc.isReduce = True
+            s_feat = None
+            feat_src = feat_src * graph.out_degrees().float().clamp(min=1).pow(-0.5).view(n, 1, 1)
+        else:
+            feat_src, s_feat = self.fc(h)
+            feat_src = feat_src.view(n, self._num_heads, self._out_feats)
+        if self.attn_r is not None:  # :176-184
+            el, er, s_el, s_er = attn_scores.apply(feat_src, self.attn_l, self.attn_r)
+            e = sddmm_u_add_v.apply(graph, el, er, s_el, s_er)
+        else:  # copy_u of el (:186)
+            e = (feat_src * self.attn_l).sum(-1, keepdim=True)[graph.coo[0]]
+        a = self.attn_drop(edge_softmax(graph, e, negative_slope=self.negative_slope))  # :187, :196
+        rst = spmm_u_mul_e.apply(graph, feat_src, a, None, s_feat)  # :201
+        if self._use_symmetric_norm:  # :203-208
+            rst = rst * graph.in_degrees().float().clamp(min=1).pow(0.5).view(n, 1, 1)
+        if self.res_fc is not None:  # :211-214
+            rst = rst + self.res_fc(h).view(n, -1, self._out_feats)
+        if self._activation is not None:
+            rst = self._activation(rst)
+        return rst
+
+
+class ArxivGAT(nn.Module):
+    """evaluation/arxiv_gat.py:376-448: ``n_layers`` attention layers with a residual projection each, batch
+    normalisation, the activation and dropout between them; the last layer has one head and ``n_classes``
+    columns, is averaged over that head and gets a bias of its own."""
+
+    def __init__(self, in_feats, n_classes, n_hidden, n_layers, n_heads, activation, dropout=0.0, input_drop=0.0,
+                 attn_drop=0.0, edge_drop=0.0, use_attn_dst=True, use_symmetric_norm=False):
+        super().__init__()
+        self.n_layers = n_layers
+        self.convs, self.norms = nn.ModuleList(), nn.ModuleList()
+        for i in range(n_layers):
+            in_hidden = n_heads * n_hidden if i > 0 else in_feats
+            out_hidden = n_hidden if i < n_layers - 1 else n_classes
+            heads = n_heads if i < n_layers - 1 else 1
+            self.convs.append(ArxivGATConv(in_hidden, out_hidden, num_heads=heads, attn_drop=attn_drop,
+                                           edge_drop=edge_drop, use_attn_dst=use_attn_dst,
+                                           use_symmetric_norm=use_symmetric_norm, residual=True))
+            if i < n_layers - 1:
+                self.norms.append(nn.BatchNorm1d(n_heads * out_hidden))
+        self.bias_last = nn.Parameter(torch.zeros(n_classes))  # ElementWiseLinear(weight=False, bias=True), :28-58
+        self.input_drop, self.dropout = nn.Dropout(input_drop), nn.Dropout(dropout)
+        self.activation = activation
+
+    def forward(self, graph, feat):
+        h = self.input_drop(feat)
+        for i in range(self.n_layers):
+            h = self.convs[i](graph, h)
+            if i < self.n_layers - 1:
+                h = self.dropout(self.activation(self.norms[i](h.flatten(1))))
+        return h.mean(1) + self.bias_last
+
+
+class HeteroHGTLayer(nn.Module):
+    """One HGT layer on a heterogeneous graph held in one node id space (node types occupy consecutive id
+    ranges, every edge carries a relation id): the layer of evaluation/test_HGT.py:27-67 with what that file's
+    homogenised form leaves out, weights per node type and per relation.  Projections k / q / v and the output
+    projection are typed by node type; each relation r has its own attention and message layers
+    (``attn_linear[r]``, ``msg_linear[r]``, the homogeneous layer's two, now one pair per relation) and runs its
+    own SDDMM and aggregation over its edges; the softmax runs over all in-edges of a destination, whatever
+    their relation."""
+
+    def __init__(self, in_dim, out_dim, n_heads, type_sizes, relation_graphs):
+        """``type_sizes``: nodes per type, in id order.  ``relation_graphs``: per relation a preprocessed Graph
+        on all nodes holding that relation's edges, its attribute ``eids`` their ids in the full graph, and
+        ``src_type``: the node type its sources belong to."""
+        super().__init__()
+        self.out_dim, self.n_heads, self.d_k = out_dim, n_heads, out_dim // n_heads
+        self.sqrt_dk = math.sqrt(self.d_k)
+        self.bounds = [0]
+        for m in type_sizes:
+            self.bounds.append(self.bounds[-1] + m)
+        self.rels = list(relation_graphs)
+        nt, nr = len(type_sizes), len(self.rels)
+        mk = lambda i, o, k: nn.ModuleList(QLinear(i, o) for _ in range(k))
+        self.k_linear, self.q_linear, self.v_linear = mk(in_dim, out_dim, nt), mk(in_dim, out_dim, nt), mk(in_dim, out_dim, nt)
+        self.a_linear = mk(out_dim, out_dim, nt)
+        self.attn_linear, self.msg_linear = mk(out_dim, out_dim, nr), mk(out_dim, out_dim, nr)
+
+    def _typed(self, layers, h):
+        """Rows of node type t through layers[t]."""
+        return torch.cat([layers[t](h[self.bounds[t]:self.bounds[t + 1]]) for t in range(len(layers))])
+
+    def forward(self, g, h):
+        n, H, dk = h.size(0), self.n_heads, self.d_k
+        k, q, v = self._typed(self.k_linear, h), self._typed(self.q_linear, h), self._typed(self.v_linear, h)
+        q = q.view(n, H, dk)
+        t = h.new_zeros((g.num_edges(), H, 1))
+        vr = []
+        for r, gr in enumerate(self.rels):
+            lo, hi = (0, n) if gr.src_type is None else (self.bounds[gr.src_type], self.bounds[gr.src_type + 1])
+            # relation-specific key and message of the relation's source type; other rows stay zero (no edge of
+            # this relation starts there)
+            kr = torch.zeros_like(k)
+            kr[lo:hi] = self.attn_linear[r](k[lo:hi])
+            vv = torch.zeros_like(v)
+            vv[lo:hi] = self.msg_linear[r](v[lo:hi])
+            vr.append(vv.view(n, H, dk))
+            tr = sddmm_u_dot_v.apply(gr, kr.view(n, H, dk), q, None, None, 1.0 / self.sqrt_dk)
+            t = t.index_copy(0, gr.eids, tr)
+        attn = edge_softmax(g, t)  # over every in-edge of a destination, all relations together
+        out = None
+        for r, gr in enumerate(self.rels):
+            o = spmm_u_mul_e.apply(gr, vr[r], attn[gr.eids])
+            out = o if out is None else out + o
+        return self._typed(self.a_linear, out.reshape(n, self.out_dim))
+
+
+def relation_graphs(g, edge_type, relations, type_sizes):
+    """Per relation id in ``edge_type`` ([E], ids 0 .. len(relations) where the last id marks self loops) a
+    preprocessed Graph over all nodes of ``g`` with that relation's edges, ``eids`` and ``src_type`` attached."""
+    from .graph import Graph
+    from .util import graph_preprocess
+    src, dst = g.edges()
+    out = []
+    for r in range(len(relations) + 1):
+        eids = torch.nonzero(edge_type == r).flatten()
+        if eids.numel() == 0:
+            continue
+        gr = graph_preprocess(Graph(src[eids], dst[eids], g.num_nodes()))
+        gr.eids = eids
+        gr.src_type = relations[r][0] if r < len(relations) else None  # self loops start at every type
+        out.append(gr)
+    return out
+
+
 class HGTStack(nn.Module):
     """Several HGT layers back to back with a linear read-out, the shape of the reference's
     driver loop (evaluation/test_HGT.py:87-96: model, then ``proj_layer``)."""

@@ -84,3 +84,36 @@ class GCN(nn.Module):
                 h = self.dropout(h)
             h = layer(self.g, h, norms)
         return h
+
+
+class ArxivGCN(nn.Module):
+    """evaluation/arxiv_gcn.py:156-209 (QGCN): graph convolutions without bias except the last, an optional
+    quantized linear skip branch per layer, batch normalisation + activation + dropout between layers, and an
+    input dropout of at most 0.1."""
+
+    def __init__(self, in_feats, n_hidden, n_classes, n_layers, activation, dropout, use_linear):
+        super().__init__()
+        from .QLinear import QLinear
+        self.n_layers, self.use_linear = n_layers, use_linear
+        self.convs, self.norms = nn.ModuleList(), nn.ModuleList()
+        self.linear = nn.ModuleList() if use_linear else None
+        for i in range(n_layers):
+            in_hidden = n_hidden if i > 0 else in_feats
+            out_hidden = n_hidden if i < n_layers - 1 else n_classes
+            self.convs.append(QGraphConv(in_hidden, out_hidden, bias=(i == n_layers - 1)))
+            if use_linear:
+                self.linear.append(QLinear(in_hidden, out_hidden, bias=False))
+            if i < n_layers - 1:
+                self.norms.append(nn.BatchNorm1d(out_hidden))
+        self.input_drop, self.dropout = nn.Dropout(min(0.1, dropout)), nn.Dropout(dropout)
+        self.activation = activation
+
+    def forward(self, graph, feat):
+        h = self.input_drop(feat)
+        norms = degree_norms(graph)
+        for i in range(self.n_layers):
+            conv = self.convs[i](graph, h, norms)
+            h = conv + self.linear[i](h) if self.use_linear else conv
+            if i < self.n_layers - 1:
+                h = self.dropout(self.activation(self.norms[i](h)))
+        return h
