@@ -68,10 +68,18 @@ int tango_absmax_rows_f32(const float* x, int64_t rows, int64_t cols, int64_t ld
    q[i] = clamp(round(x[i] * (1 / scale[0])), -127, 127).  round_mode selects the
    rounding.  For TANGO_ROUND_STOCHASTIC, `noise` (n floats in [0,1), same
    indexing as x) is used when non-null; otherwise Philox4x32-10 keyed by `seed`
-   with counter (offset + i) >> 2, word (offset + i) & 3, u = (word >> 8) * 2^-24. */
+   with counter (offset + i) >> 2, word (offset + i) & 3, u = (word >> 8) * 2^-24.
+   offset_dev (or NULL): one 64-bit word of device memory whose value is added to `offset` when
+   the kernel starts.  A caller that keeps its position in the random stream there and advances it
+   with tango_counter_add_u64 draws fresh numbers on every replay of a captured graph, which a
+   host-side offset (a constant of the captured launch) cannot; keep its value a multiple of 4. */
 int tango_quantize_f32_i8(const float* x, int64_t n, const float* scale, int8_t* q,
                           int round_mode, const float* noise, uint64_t seed, uint64_t offset,
-                          tango_stream_t stream);
+                          const uint64_t* offset_dev, tango_stream_t stream);
+
+/* counter[0] += inc by a one-thread kernel on the stream (no counterpart in the reference): the
+   device-side position in the stream of random numbers, see tango_quantize_f32_i8. */
+int tango_counter_add_u64(uint64_t* counter, uint64_t inc, tango_stream_t stream);
 
 /* Row-strided quantize with an optionally padded output (no counterpart in the
    reference; lets the SpMM gather aligned rows when cols is odd, e.g. 41):
@@ -106,7 +114,7 @@ int tango_quantize_rows_ex_f32_i8(const float* x, int64_t rows, int64_t cols, in
                                   const float* row_mul, const void* mask, int64_t ldm, int mask_mode,
                                   const float* scale, int per_row, int8_t* q, int64_t ldq,
                                   int round_mode, const float* noise, uint64_t seed,
-                                  uint64_t offset, tango_stream_t stream);
+                                  uint64_t offset, const uint64_t* offset_dev, tango_stream_t stream);
 
 /* transpose_quant (cuda/src/cuda.cpp:27-33 -> transpose_quant_impl,
    quantization.cu:95-167): x[nrow, ncol] fp32 -> out[ncol, nrow] int8,

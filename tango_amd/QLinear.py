@@ -29,7 +29,7 @@ def _quantize_grad(dY, want_colsum=False):
         scale, colsum = kernels.cuda_kernels.absmax_ex(dY, want_colsum=True)
     kw = {"round_mode": config.grad_round_mode}
     if config.grad_round_mode == "stochastic":
-        kw.update(seed=config.seed, offset=config.next_offset())
+        kw.update(config.stochastic_args(dY.device))
     q, scale = kernels.quantize_padded(dY, scale, **kw)
     return q, scale, colsum
 
@@ -44,6 +44,7 @@ class QgemmNT_func(Function):
 
     @staticmethod
     def backward(ctx, grad_output):
+        kernels.refuse_capture("QgemmNT_func.backward")
         A, B = ctx.saved_tensors
         grad_A = grad_B = None
         grad_output = grad_output.contiguous()
@@ -91,6 +92,7 @@ def _forward(ctx, X, W, b, reduce, row_scale=None, scaleX=None, Xq=None):
 
 
 def _backward(ctx, grad_output):
+    kernels.refuse_capture("QLinear.backward")
     X_, scaleX, W_, scaleW, b, row_scale = ctx.backward_cache
     want_bias = b is not None and ctx.needs_input_grad[2]
     dY_, scaledY, grad_bias = _quantize_grad(grad_output, want_bias)
@@ -185,6 +187,7 @@ class Qlinear_shared_func(Function):
     @staticmethod
     @once_differentiable
     def backward(ctx, *grads):
+        kernels.refuse_capture("Qlinear_shared_func.backward")
         Xq, scaleX, layers = ctx.backward_cache
         n = len(layers)
         need = ctx.needs_input_grad

@@ -5,13 +5,13 @@ from torch.autograd.function import Function, once_differentiable
 
 from . import config
 from .kernels import (cuda_kernels, incidence_SPMM, multi_cusparse_SPMM, mySDDMM_int8, mySDDMM_quantize_on_load,
-                      quantize)
+                      quantize, refuse_capture)
 
 
 def _quantize_grad(t):
     t = t if t.is_contiguous() else t.contiguous()
     if config.grad_round_mode == "stochastic":
-        return quantize(t, round_mode="stochastic", seed=config.seed, offset=config.next_offset())
+        return quantize(t, round_mode="stochastic", **config.stochastic_args(t.device))
     return quantize(t, round_mode=config.grad_round_mode)
 
 
@@ -36,6 +36,7 @@ class sddmm_u_add_v(Function):
     @staticmethod
     @once_differentiable
     def backward(ctx, dZ):
+        refuse_capture("sddmm_u_add_v.backward")
         g = ctx.backward_cache
         dZ_, scaledZ = _quantize_grad(dZ)
         dU = dV = None
@@ -72,6 +73,7 @@ class sddmm_u_dot_v(Function):
     @staticmethod
     @once_differentiable
     def backward(ctx, dZ):
+        refuse_capture("sddmm_u_dot_v.backward")
         g, U_, scaleU, V_, scaleV = ctx.backward_cache
         dZ = dZ if dZ.is_contiguous() else dZ.contiguous()
         squeeze = dZ.dim() == 2

@@ -3,7 +3,8 @@ import torch
 from torch.autograd.function import Function, once_differentiable
 
 from . import config
-from .kernels import cuda_kernels, csr_SPMM, multi_cusparse_SPMM, mySDDMM_int8, quantize, quantize_padded
+from .kernels import (cuda_kernels, csr_SPMM, multi_cusparse_SPMM, mySDDMM_int8, quantize, quantize_padded,
+                      refuse_capture)
 
 
 def _gather_align(width):
@@ -19,7 +20,7 @@ def _quantize_grad(t, padded):
     t = t if t.is_contiguous() else t.contiguous()
     kw = {"round_mode": config.grad_round_mode}
     if config.grad_round_mode == "stochastic":
-        kw.update(seed=config.seed, offset=config.next_offset())
+        kw.update(config.stochastic_args(t.device))
     if padded and t.dim() == 2:
         return quantize_padded(t, align=_gather_align(t.size(1)), **kw)
     return quantize(t, **kw)
@@ -61,6 +62,7 @@ class spmm_copy_u(Function):
     @staticmethod
     @once_differentiable
     def backward(ctx, dOut):
+        refuse_capture("spmm_copy_u.backward")
         g, row_scale, has_bias, mask, relu = ctx.backward_cache
         if relu and mask is None:
             mask, = ctx.saved_tensors
@@ -78,7 +80,7 @@ class spmm_copy_u(Function):
         if ctx.needs_input_grad[1]:
             kw = {"round_mode": config.grad_round_mode}
             if config.grad_round_mode == "stochastic":
-                kw.update(seed=config.seed, offset=config.next_offset())
+                kw.update(config.stochastic_args(dOut.device))
             dZ_, _ = quantize_padded(dOut, scaledZ, row_mul=row_scale, mask=mask, mask_mode=mode,
                                      align=_gather_align(dOut.size(1)), **kw)
             dN = csr_SPMM(g, dZ_, scaledZ, True)
@@ -125,6 +127,7 @@ class spmm_u_mul_e(Function):
     @staticmethod
     @once_differentiable
     def backward(ctx, dZ):
+        refuse_capture("spmm_u_mul_e.backward")
         g, N_, scaleN, E_T_, scaleE, reduce_last, eshape, has_bias, act = ctx.backward_cache
         dbias = None
         if act is not None:
@@ -136,7 +139,7 @@ class spmm_u_mul_e(Function):
                                                     want_colsum=has_bias and ctx.needs_input_grad[3])
             kw = {"round_mode": config.grad_round_mode}
             if config.grad_round_mode == "stochastic":
-                kw.update(seed=config.seed, offset=config.next_offset())
+                kw.update(config.stochastic_args(dZ.device))
             dZ_, _ = quantize_padded(dZ2, scaledZ, mask=out2, mask_mode=act, align=1, **kw)
             dZ_ = dZ_.view(dZ.shape)
         elif has_bias and ctx.needs_input_grad[3]:
@@ -145,7 +148,7 @@ class spmm_u_mul_e(Function):
             scaledZ, dbias = cuda_kernels.absmax_ex(dZ.view(dZ.size(0), -1), want_colsum=True)
             kw = {"round_mode": config.grad_round_mode}
             if config.grad_round_mode == "stochastic":
-                kw.update(seed=config.seed, offset=config.next_offset())
+                kw.update(config.stochastic_args(dZ.device))
             dZ_, _ = quantize(dZ, scaledZ, **kw)
         else:
             dZ_, scaledZ = _quantize_grad(dZ, False)

@@ -23,11 +23,12 @@ SIGNATURES = {
     "tango_absmax_f32": (I, [P, I64, P, P]),
     "tango_absmax_acc_f32": (I, [P, I64, P, P]),
     "tango_absmax_rows_f32": (I, [P, I64, I64, I64, P, P]),
-    "tango_quantize_f32_i8": (I, [P, I64, P, P, I, P, U64, U64, P]),
+    "tango_quantize_f32_i8": (I, [P, I64, P, P, I, P, U64, U64, P, P]),
+    "tango_counter_add_u64": (I, [P, U64, P]),
     "tango_quantize_rows_f32_i8": (I, [P, I64, I64, I64, P, I, P, I64, I, P, U64, U64, P]),
     "tango_absmax_ex_workspace": (SZ, [I64, I64, I]),
     "tango_absmax_ex_f32": (I, [P, I64, I64, I64, P, P, I64, I, P, I, P, P, SZ, P]),
-    "tango_quantize_rows_ex_f32_i8": (I, [P, I64, I64, I64, P, P, I64, I, P, I, P, I64, I, P, U64, U64, P]),
+    "tango_quantize_rows_ex_f32_i8": (I, [P, I64, I64, I64, P, P, I64, I, P, I, P, I64, I, P, U64, U64, P, P]),
     "tango_transpose_quant_f32_i8": (I, [P, I64, I64, P, P, P]),
     "tango_qgemm_fwd_workspace": (SZ, [I64, I64, I64]),
     "tango_qgemm_fwd": (I, [P, I64, P, I64, P, I64, P, I64, P, P, P, P, P, I64, I64, I64, I, P, SZ, P]),

@@ -15,8 +15,39 @@ grad_round_mode = os.environ.get("TANGO_GRAD_ROUND", "rne")
 # Seed of the counter-based RNG for stochastic rounding; every quantize call
 # draws a fresh 2^40-element window of the stream.
 seed = int(os.environ.get("TANGO_SEED", "0"))
+WINDOW = 1 << 40
 _calls = itertools.count()
+_counters = {}
 
 
 def next_offset():
-    return next(_calls) << 40
+    """Host-side position in the stream (a Python counter): for callers that pass ``offset`` as a number."""
+    return next(_calls) * WINDOW
+
+
+def device_offset(device):
+    """The position in the stream as one int64 word in ``device``'s memory.  The quantize kernels add it to their
+    offset when they start and the call that used it advances it by WINDOW with a one-thread kernel on the same
+    stream, so the position moves with the work itself: a captured graph that is replayed draws a fresh window
+    per replay, where a host-side counter would be frozen into the captured launch."""
+    import torch
+    key = torch.device(device)
+    if key.index is None and key.type == "cuda":
+        key = torch.device("cuda", torch.cuda.current_device())
+    c = _counters.get(key)
+    if c is None:
+        c = _counters[key] = torch.zeros(1, dtype=torch.int64, device=key)
+    return c
+
+
+def reset_offsets():
+    """Back to the start of the stream (tests that compare with a host-side replay of the same draws)."""
+    global _calls
+    _calls = itertools.count()
+    for c in _counters.values():
+        c.zero_()
+
+
+def stochastic_args(device):
+    """Keyword arguments of a stochastically rounding quantize call."""
+    return {"seed": seed, "offset": device_offset(device), "advance": WINDOW}

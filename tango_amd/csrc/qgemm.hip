@@ -1248,10 +1248,10 @@ extern "C" int tango_quantize_rows_f32_i8(const float*, int64_t, int64_t, int64_
                                           tango_stream_t);
 extern "C" int tango_quantize_rows_ex_f32_i8(const float*, int64_t, int64_t, int64_t, const float*,
                                              const void*, int64_t, int, const float*, int, int8_t*, int64_t,
-                                             int, const float*, uint64_t, uint64_t, tango_stream_t);
+                                             int, const float*, uint64_t, uint64_t, const uint64_t*, tango_stream_t);
 extern "C" int tango_absmax_f32(const float*, int64_t, float*, tango_stream_t);
 extern "C" int tango_quantize_f32_i8(const float*, int64_t, const float*, int8_t*, int, const float*, uint64_t,
-                                     uint64_t, tango_stream_t);
+                                     uint64_t, const uint64_t*, tango_stream_t);
 
 extern "C" {
 
@@ -1283,7 +1283,7 @@ int tango_qgemm_fwd_ex(float* Y, int64_t ldy, const float* X, int64_t ldx, const
     int rc = TANGO_OK;
     if (!fused && !cached) {
         rc = tango_quantize_rows_ex_f32_i8(X, M, K, ldx, x_row_mul, nullptr, 0, 0, scaleX, 0, Xq, ldxq, round_mode,
-                                           nullptr, 0, 0, stream);
+                                           nullptr, 0, 0, nullptr, stream);
         if (rc != TANGO_OK) return rc;
     }
     int8_t* Bp = static_cast<int8_t*>(workspace);
@@ -1527,13 +1527,13 @@ int tango_qgemm_legacy(float* C, const float* A, const float* B, int64_t m, int6
     if ((rc = tango_absmax_f32(A, m * k, scales, stream)) != TANGO_OK) return rc;
     if ((rc = tango_absmax_f32(B, n * k, scales + 1, stream)) != TANGO_OK) return rc;
     // A as stored is [m,k] (or [k,m]); quantize densely, then pack (or transpose-pack) to [m, k64]
-    rc = tango_quantize_f32_i8(A, m * k, scales, tmp, TANGO_ROUND_RNE, nullptr, 0, 0, stream);
+    rc = tango_quantize_f32_i8(A, m * k, scales, tmp, TANGO_ROUND_RNE, nullptr, 0, 0, nullptr, stream);
     if (rc != TANGO_OK) return rc;
     if (trans_a)
         hipLaunchKernelGGL(transpose_pack_i8_kernel, dim3(grid_for(m * k64, 256)), dim3(256), 0, s, Ap, k64, tmp, m, k, m);
     else
         hipLaunchKernelGGL(pack_rows_i8_kernel, dim3(grid_for(m * k64, 256)), dim3(256), 0, s, Ap, k64, tmp, k, m, k);
-    rc = tango_quantize_f32_i8(B, n * k, scales + 1, tmp, TANGO_ROUND_RNE, nullptr, 0, 0, stream);
+    rc = tango_quantize_f32_i8(B, n * k, scales + 1, tmp, TANGO_ROUND_RNE, nullptr, 0, 0, nullptr, stream);
     if (rc != TANGO_OK) return rc;
     if (trans_b)  // stored [n,k]
         hipLaunchKernelGGL(pack_rows_i8_kernel, dim3(grid_for(n * k64, 256)), dim3(256), 0, s, Bp, k64, tmp, k, n, k);

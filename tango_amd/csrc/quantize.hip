@@ -166,7 +166,9 @@ __global__ __launch_bounds__(256) void absmax_rows_kernel(const float* __restric
 template <int MODE>
 __global__ __launch_bounds__(256) void quantize_vec_kernel(
     const float* __restrict__ x, int64_t n, const float* __restrict__ scale,
-    int8_t* __restrict__ q, const float* __restrict__ noise, uint64_t seed, uint64_t offset) {
+    int8_t* __restrict__ q, const float* __restrict__ noise, uint64_t seed, uint64_t offset_host,
+    const uint64_t* __restrict__ offset_dev) {
+    const uint64_t offset = offset_host + (offset_dev ? offset_dev[0] : 0);
     const int64_t tid = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
     const int64_t nthr = static_cast<int64_t>(gridDim.x) * blockDim.x;
     const float r = rscale_of(scale[0]);
@@ -236,8 +238,10 @@ __device__ __forceinline__ void mask_bits4(float* mk, const uint16_t* __restrict
 template <int MODE>
 __global__ __launch_bounds__(256) void quantize_dense_ex_kernel(
     const float* __restrict__ x, int64_t n4, int64_t cols, const float* __restrict__ scale,
-    int8_t* __restrict__ q, const float* __restrict__ noise, uint64_t seed, uint64_t offset,
+    int8_t* __restrict__ q, const float* __restrict__ noise, uint64_t seed, uint64_t offset_host,
+    const uint64_t* __restrict__ offset_dev,
     const float* __restrict__ row_mul, const float* __restrict__ mask, int mask_mode) {
+    const uint64_t offset = offset_host + (offset_dev ? offset_dev[0] : 0);
     const int64_t tid = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
     const int64_t nthr = static_cast<int64_t>(gridDim.x) * blockDim.x;
     const float r = rscale_of(scale[0]);
@@ -294,7 +298,9 @@ __global__ __launch_bounds__(256) void quantize_dense_ex_kernel(
 template <int MODE>
 __global__ __launch_bounds__(256) void quantize_scalar_kernel(
     const float* __restrict__ x, int64_t n, const float* __restrict__ scale,
-    int8_t* __restrict__ q, const float* __restrict__ noise, uint64_t seed, uint64_t offset) {
+    int8_t* __restrict__ q, const float* __restrict__ noise, uint64_t seed, uint64_t offset_host,
+    const uint64_t* __restrict__ offset_dev) {
+    const uint64_t offset = offset_host + (offset_dev ? offset_dev[0] : 0);
     const int64_t tid = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
     const int64_t nthr = static_cast<int64_t>(gridDim.x) * blockDim.x;
     const float r = rscale_of(scale[0]);
@@ -332,9 +338,10 @@ template <int MODE, int XV>
 __global__ __launch_bounds__(256) void quantize_rows_kernel(
     const float* __restrict__ x, int64_t rows, int64_t cols, int64_t ldx,
     const float* __restrict__ scale, int per_row, int8_t* __restrict__ q, int64_t ldq,
-    const float* __restrict__ noise, uint64_t seed, uint64_t offset,
+    const float* __restrict__ noise, uint64_t seed, uint64_t offset_host, const uint64_t* __restrict__ offset_dev,
     const float* __restrict__ row_mul, const float* __restrict__ mask, int64_t ldm, int gpr_log2,
     int mask_mode) {
+    const uint64_t offset = offset_host + (offset_dev ? offset_dev[0] : 0);
     // the mask may use x's vector width when its rows are laid out and aligned like x's
     const bool mask_vec = mask && ldm == ldx &&
                           ((reinterpret_cast<uintptr_t>(mask) ^ reinterpret_cast<uintptr_t>(x)) & 15) == 0;
@@ -636,7 +643,7 @@ const char* tango_status_string(int status) {
     }
 }
 
-int tango_abi_version(void) { return 1; }
+int tango_abi_version(void) { return 2; }
 
 int tango_absmax_f32(const float* x, int64_t n, float* scale_out, tango_stream_t stream) {
     if (!scale_out || n < 0 || (n > 0 && !x)) return TANGO_ERR_INVALID_ARG;
@@ -744,9 +751,19 @@ int tango_absmax_ex_f32(const float* x, int64_t rows, int64_t cols, int64_t ldx,
     return launch_status();
 }
 
+// counter[0] += inc, one thread (a kernel rather than a host-side update, so that a captured graph advances the
+// stream of random numbers on every replay)
+static __global__ void counter_add_kernel(uint64_t* counter, uint64_t inc) { counter[0] += inc; }
+
+int tango_counter_add_u64(uint64_t* counter, uint64_t inc, tango_stream_t stream) {
+    if (!counter || (reinterpret_cast<uintptr_t>(counter) & 7) != 0) return TANGO_ERR_INVALID_ARG;
+    hipLaunchKernelGGL(counter_add_kernel, dim3(1), dim3(1), 0, as_stream(stream), counter, inc);
+    return launch_status();
+}
+
 int tango_quantize_f32_i8(const float* x, int64_t n, const float* scale, int8_t* q,
                           int round_mode, const float* noise, uint64_t seed, uint64_t offset,
-                          tango_stream_t stream) {
+                          const uint64_t* offset_dev, tango_stream_t stream) {
     if (n < 0 || !scale || (n > 0 && (!x || !q))) return TANGO_ERR_INVALID_ARG;
     if (n == 0) return (round_mode >= 0 && round_mode <= 2) ? TANGO_OK : TANGO_ERR_UNSUPPORTED;
     hipStream_t s = as_stream(stream);
@@ -755,10 +772,10 @@ int tango_quantize_f32_i8(const float* x, int64_t n, const float* scale, int8_t*
         constexpr int M = decltype(mode)::value;
         if (vec) {
             hipLaunchKernelGGL(quantize_vec_kernel<M>, dim3(grid_for(ceil_div(n, 4), 256)), dim3(256),
-                               0, s, x, n, scale, q, noise, seed, offset);
+                               0, s, x, n, scale, q, noise, seed, offset, offset_dev);
         } else {
             hipLaunchKernelGGL(quantize_scalar_kernel<M>, dim3(grid_for(n, 256)), dim3(256), 0, s, x,
-                               n, scale, q, noise, seed, offset);
+                               n, scale, q, noise, seed, offset, offset_dev);
         }
     });
     return rc != TANGO_OK ? rc : launch_status();
@@ -769,14 +786,14 @@ int tango_quantize_rows_f32_i8(const float* x, int64_t rows, int64_t cols, int64
                                int round_mode, const float* noise, uint64_t seed,
                                uint64_t offset, tango_stream_t stream) {
     return tango_quantize_rows_ex_f32_i8(x, rows, cols, ldx, nullptr, nullptr, 0, 0, scale, per_row, q, ldq,
-                                         round_mode, noise, seed, offset, stream);
+                                         round_mode, noise, seed, offset, nullptr, stream);
 }
 
 int tango_quantize_rows_ex_f32_i8(const float* x, int64_t rows, int64_t cols, int64_t ldx,
                                   const float* row_mul, const void* mask_, int64_t ldm, int mask_mode,
                                   const float* scale, int per_row, int8_t* q, int64_t ldq,
                                   int round_mode, const float* noise, uint64_t seed,
-                                  uint64_t offset, tango_stream_t stream) {
+                                  uint64_t offset, const uint64_t* offset_dev, tango_stream_t stream) {
     const float* mask = static_cast<const float*>(mask_);  // 16-bit words in mode 2
     if (mask && ldm < (mask_mode == 2 ? cols / 16 : cols)) return TANGO_ERR_INVALID_ARG;
     if (mask_mode < 0 || mask_mode > 2 || (mask && mask_mode == 2 && (cols & 15) != 0)) return TANGO_ERR_UNSUPPORTED;
@@ -792,7 +809,7 @@ int tango_quantize_rows_ex_f32_i8(const float* x, int64_t rows, int64_t cols, in
         int rc = dispatch_mode(round_mode, [&](auto mode) {
             constexpr int M = decltype(mode)::value;
             hipLaunchKernelGGL(quantize_dense_ex_kernel<M>, dim3(grid_for(n4, 256)), dim3(256), 0, s, x, n4, cols, scale,
-                               q, noise, seed, offset, row_mul, mask, mask_mode);
+                               q, noise, seed, offset, offset_dev, row_mul, mask, mask_mode);
         });
         return rc != TANGO_OK ? rc : launch_status();
     }
@@ -807,13 +824,13 @@ int tango_quantize_rows_ex_f32_i8(const float* x, int64_t rows, int64_t cols, in
         constexpr int M = decltype(mode)::value;
         if (xv == 4)
             hipLaunchKernelGGL((quantize_rows_kernel<M, 4>), grid, block, 0, s, x, rows, cols, ldx, scale,
-                               per_row, q, ldq, noise, seed, offset, row_mul, mask, ldm, gpr_log2, mask_mode);
+                               per_row, q, ldq, noise, seed, offset, offset_dev, row_mul, mask, ldm, gpr_log2, mask_mode);
         else if (xv == 2)
             hipLaunchKernelGGL((quantize_rows_kernel<M, 2>), grid, block, 0, s, x, rows, cols, ldx, scale,
-                               per_row, q, ldq, noise, seed, offset, row_mul, mask, ldm, gpr_log2, mask_mode);
+                               per_row, q, ldq, noise, seed, offset, offset_dev, row_mul, mask, ldm, gpr_log2, mask_mode);
         else
             hipLaunchKernelGGL((quantize_rows_kernel<M, 1>), grid, block, 0, s, x, rows, cols, ldx, scale,
-                               per_row, q, ldq, noise, seed, offset, row_mul, mask, ldm, gpr_log2, mask_mode);
+                               per_row, q, ldq, noise, seed, offset, offset_dev, row_mul, mask, ldm, gpr_log2, mask_mode);
     });
     return rc != TANGO_OK ? rc : launch_status();
 }

@@ -3,7 +3,7 @@ LeakyReLU that precedes it in GAT fused in (evaluation/test_gat.py:144-146;
 the reference calls DGL's fp32 edge_softmax, which is not part of its tree)."""
 from torch.autograd.function import Function, once_differentiable
 
-from .kernels import cuda_kernels
+from .kernels import cuda_kernels, refuse_capture
 
 
 def _dst_major(g):
@@ -25,6 +25,7 @@ class _EdgeSoftmax(Function):
     @staticmethod
     @once_differentiable
     def backward(ctx, da):
+        refuse_capture("edge_softmax.backward")
         g, slope = ctx.backward_cache
         e, a = ctx.saved_tensors
         indptr, eids = _dst_major(g)

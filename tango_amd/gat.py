@@ -10,7 +10,7 @@ import torch.nn.functional as F
 from torch.autograd.function import Function, once_differentiable
 
 from .QLinear import QLinear, Qlinear_func_reduce, shared_input_linears
-from .kernels import cuda_kernels
+from .kernels import cuda_kernels, refuse_capture
 from .SDDMM import sddmm_u_add_v, sddmm_u_dot_v
 from .SPMM import spmm_u_mul_e
 from .edge_softmax import edge_softmax
@@ -36,6 +36,7 @@ class attn_scores(Function):
     @staticmethod
     @once_differentiable
     def backward(ctx, del_, der, _ds_el=None, _ds_er=None):
+        refuse_capture("attn_scores.backward")
         feat, al, ar, shape = ctx.backward_cache
         if del_ is None and der is None:
             return None, None, None

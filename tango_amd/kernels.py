@@ -122,6 +122,32 @@ _MASK_MODES = {"relu": 0, "elu": 1, "bits": 2}
 _ACTIVATIONS = {None: 0, "relu": 1, "elu": 2}
 
 
+def refuse_capture(what):
+    """Raises when the current stream is being captured into a HIP graph.  Called first thing by every backward
+    pass of this package: forward passes capture and replay (they launch kernels only, on the capturing thread),
+    but a backward pass runs on autograd's worker thread, where it draws workspaces and scale slots from torch's
+    allocator and reads pools that the capturing thread owns; capturing a whole training step ended the process
+    with a segmentation fault when it was tried, and stays refused until that is understood."""
+    if torch.cuda.is_initialized() and torch.cuda.is_current_stream_capturing():
+        raise RuntimeError(
+            what + ": backward passes of the quantized operators cannot be captured into a HIP graph "
+            "(capture the forward pass only and run the training step eagerly)")
+
+
+def _split_offset(offset):
+    """(host offset, device counter or None) of an ``offset`` argument that is a number or an int64 device tensor."""
+    if torch.is_tensor(offset):
+        if offset.dtype != torch.int64 or offset.numel() != 1 or not offset.is_cuda:
+            raise RuntimeError("quantize: a device offset must be a 1-element int64 GPU tensor")
+        return 0, offset
+    return int(offset), None
+
+
+def _advance(counter, inc):
+    if counter is not None and inc:
+        check(_L.tango_counter_add_u64(counter.data_ptr(), int(inc), _stream()), "counter_add")
+
+
 def _mode(round_mode):
     if isinstance(round_mode, str):
         return ROUND_MODES[round_mode]
@@ -179,7 +205,9 @@ class cuda_kernels:
         return scale
 
     @staticmethod
-    def quantize(out, inp, scale, round_mode=ROUND_RNE, noise=None, seed=0, offset=0):
+    def quantize(out, inp, scale, round_mode=ROUND_RNE, noise=None, seed=0, offset=0, advance=0):
+        """``offset``: a number, or a 1-element int64 device tensor holding the position in the random stream
+        (then ``advance`` is added to it after the launch, by a kernel on the same stream)."""
         _need(out, torch.int8, "out")
         _need(inp, torch.float32, "in")
         _need(scale, torch.float32, "scale")
@@ -189,9 +217,11 @@ class cuda_kernels:
             _need(noise, torch.float32, "noise")
             if noise.numel() != inp.numel():
                 raise RuntimeError("quantize: noise and in differ in size")
+        offset, offset_dev = _split_offset(offset)
         check(_L.tango_quantize_f32_i8(_ptr(inp), inp.numel(), scale.data_ptr(), _ptr(out),
-                                       _mode(round_mode), _ptr(noise), int(seed), int(offset),
+                                       _mode(round_mode), _ptr(noise), int(seed), offset, _ptr(offset_dev),
                                        _stream()), "quantize")
+        _advance(offset_dev, advance)
 
     @staticmethod
     def _mask_ld(mask, mask_mode, inp, what):
@@ -209,7 +239,7 @@ class cuda_kernels:
 
     @staticmethod
     def quantize_rows(out, inp, scale, per_row=False, round_mode=ROUND_RNE, noise=None, seed=0,
-                      offset=0, row_mul=None, mask=None, mask_mode="relu"):
+                      offset=0, row_mul=None, mask=None, mask_mode="relu", advance=0):
         """Row-strided quantize into a possibly wider (zero-padded) int8 matrix (not in the reference).
         ``mask`` (an activation's output) takes each element backwards through that activation first:
         ``mask_mode`` "relu" zeroes it where mask <= 0, "elu" multiplies it by mask + 1 there, "bits":
@@ -233,11 +263,13 @@ class cuda_kernels:
                 raise RuntimeError("quantize_rows: row_mul must have one entry per row")
         if mask is not None:
             ldm = cuda_kernels._mask_ld(mask, mask_mode, inp, "quantize_rows")
+        offset, offset_dev = _split_offset(offset)
         check(_L.tango_quantize_rows_ex_f32_i8(_ptr(inp), inp.size(0), inp.size(1), ldx, _ptr(row_mul),
                                                _ptr(mask), ldm, _MASK_MODES[mask_mode], scale.data_ptr(),
                                                int(bool(per_row)),
                                                _ptr(out), ldq_pad, _mode(round_mode), _ptr(noise),
-                                               int(seed), int(offset), _stream()), "quantize_rows")
+                                               int(seed), offset, _ptr(offset_dev), _stream()), "quantize_rows")
+        _advance(offset_dev, advance)
 
     @staticmethod
     def absmax_ex(inp, row_mul=None, mask=None, want_colsum=False, mask_mode="relu"):
@@ -668,18 +700,19 @@ class cuda_kernels:
 
 
 # ------------------------------------------------------------------ wrappers
-def quantize(t, scale=None, round_mode=ROUND_RNE, noise=None, seed=0, offset=0):
+def quantize(t, scale=None, round_mode=ROUND_RNE, noise=None, seed=0, offset=0, advance=0):
     """Quantize to int8; returns (int8 tensor, scale).  cuda/kernels.py:19-30."""
     assert t.is_cuda, "tensor must be on GPU"
     if scale is None:
         scale = cuda_kernels.get_scale(t)
     out = torch.empty(t.shape, dtype=torch.int8, device=t.device)
-    cuda_kernels.quantize(out, t, scale, round_mode=round_mode, noise=noise, seed=seed, offset=offset)
+    cuda_kernels.quantize(out, t, scale, round_mode=round_mode, noise=noise, seed=seed, offset=offset,
+                          advance=advance)
     return out, scale
 
 
 def quantize_padded(t, scale=None, round_mode=ROUND_RNE, noise=None, seed=0, offset=0, align=16,
-                    row_mul=None, mask=None, mask_mode="relu"):
+                    row_mul=None, mask=None, mask_mode="relu", advance=0):
     """Like ``quantize`` for a 2-D tensor, but the int8 rows are padded with
     zeros to a multiple of ``align`` bytes so that the SpMM gather and the GEMM
     fragment loads stay 16-byte aligned for odd widths (41, 602, ...).  Returns a
@@ -695,10 +728,11 @@ def quantize_padded(t, scale=None, round_mode=ROUND_RNE, noise=None, seed=0, off
     buf = torch.empty((rows, ld), dtype=torch.int8, device=t.device)
     if ld == cols and row_mul is None and mask is None and t.is_contiguous():
         # nothing to pad: the flat kernel (16-byte loads front to back, same element -> noise index mapping)
-        cuda_kernels.quantize(buf, t, scale, round_mode=round_mode, noise=noise, seed=seed, offset=offset)
+        cuda_kernels.quantize(buf, t, scale, round_mode=round_mode, noise=noise, seed=seed, offset=offset,
+                              advance=advance)
     else:
         cuda_kernels.quantize_rows(buf, t, scale, round_mode=round_mode, noise=noise, seed=seed, offset=offset,
-                                   row_mul=row_mul, mask=mask, mask_mode=mask_mode)
+                                   row_mul=row_mul, mask=mask, mask_mode=mask_mode, advance=advance)
     return buf[:, :cols], scale
 
 

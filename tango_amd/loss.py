@@ -4,7 +4,7 @@ call (evaluation/test_gcn.py:256)."""
 import torch
 from torch.autograd.function import Function, once_differentiable
 
-from .kernels import _L, _ptr, _stream, _workspace, check
+from .kernels import _L, _ptr, _stream, _workspace, check, refuse_capture
 
 
 class _SoftmaxXent(Function):
@@ -30,6 +30,7 @@ class _SoftmaxXent(Function):
     @staticmethod
     @once_differentiable
     def backward(ctx, gout):
+        refuse_capture("cross_entropy.backward")
         return ctx.backward_cache * gout, None
 
 

@@ -39,7 +39,7 @@ def test_argument_validation_needs_no_gpu():
     from tango_amd import _lib
     L = _lib.lib()
     assert L.tango_absmax_f32(None, 10, None, None) == -1
-    assert L.tango_quantize_f32_i8(None, -1, None, None, 0, None, 0, 0, None) == -1
+    assert L.tango_quantize_f32_i8(None, -1, None, None, 0, None, 0, 0, None, None) == -1
     assert L.tango_spmm_csr_u_mul_e(1, 1, 1, None, 1, 1, 1, 4, 4, 2, 8, 3, 10, None) == -2  # D not in {1, F}
     assert L.tango_sddmm_ewise_i8(7, 1, None, 1, 1, 1, 1, 1, 1, 4, 4, None) == -2  # unknown op
     assert L.tango_spmm_csr_copy_u(1, 1, 1, 1, 8, 1, 4, 1 << 31, 10, 8, None) == -2  # node ids must fit 31 bits
@@ -64,3 +64,28 @@ def test_infer_broadcast_shape():
     import pytest
     with pytest.raises(ValueError):
         ibs("add", (3,), (4,))
+
+
+def test_backward_passes_refuse_graph_capture(monkeypatch):
+    """Capturing a whole training step into a HIP graph once ended the process with a segmentation fault whose
+    cause is not established; until it is, every backward pass of the package raises when its stream is being
+    captured.  Checked on the host: the capture state is stubbed, no GPU work is involved (the capture itself is
+    deliberately never attempted on a GPU, not even to see the error)."""
+    import pytest
+    import torch
+    from tango_amd import kernels
+    from tango_amd.QLinear import Qlinear_func, Qlinear_shared_func
+    from tango_amd.SDDMM import sddmm_u_add_v, sddmm_u_dot_v
+    from tango_amd.SPMM import spmm_copy_u, spmm_u_mul_e
+    from tango_amd.edge_softmax import _EdgeSoftmax
+    from tango_amd.gat import attn_scores
+    from tango_amd.loss import _SoftmaxXent
+    kernels.refuse_capture("eager")  # not capturing: passes
+    monkeypatch.setattr(torch.cuda, "is_initialized", lambda: True)
+    monkeypatch.setattr(torch.cuda, "is_current_stream_capturing", lambda: True)
+    with pytest.raises(RuntimeError, match="HIP graph"):
+        kernels.refuse_capture("x")
+    for fn, nargs in ((Qlinear_func, 1), (Qlinear_shared_func, 2), (sddmm_u_add_v, 1), (sddmm_u_dot_v, 1),
+                      (spmm_copy_u, 1), (spmm_u_mul_e, 1), (_EdgeSoftmax, 1), (attn_scores, 2), (_SoftmaxXent, 1)):
+        with pytest.raises(RuntimeError, match="HIP graph"):
+            fn.backward(object(), *([None] * nargs))  # refuses before it looks at its context

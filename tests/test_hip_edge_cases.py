@@ -97,7 +97,7 @@ def test_status_codes_surface_as_exceptions(K):
     L = _lib.lib()
     x = torch.zeros(8, device="cuda")
     q = torch.zeros(8, dtype=torch.int8, device="cuda")
-    assert L.tango_quantize_f32_i8(x.data_ptr(), 8, x.data_ptr(), q.data_ptr(), 9, None, 0, 0, None) == -2
+    assert L.tango_quantize_f32_i8(x.data_ptr(), 8, x.data_ptr(), q.data_ptr(), 9, None, 0, 0, None, None) == -2
     # GEMM without the workspace it asked for
     assert L.tango_qgemm_bwd_dw(x.data_ptr(), 4, q.data_ptr(), 2, q.data_ptr(), 4, x.data_ptr(), x.data_ptr(),
                                 2, 2, 4, None, 0, None) == -4

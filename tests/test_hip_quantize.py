@@ -134,3 +134,47 @@ def test_absmax_accumulating_form(K, orc):
     assert host(s1)[0] == orc.absmax_scale(a) and host(s2)[0] == orc.absmax_scale(a * 2)
     s3, _ = K.cuda_kernels.absmax_ex(x.view(-1, 1)[:300000].view(3000, 100))
     assert host(s3)[0] == orc.absmax_scale(a[:300000])
+
+
+def test_device_resident_stream_position_advances_on_graph_replay(K, orc):
+    """Stochastic rounding whose position in the random stream lives in device memory: the kernel adds the word
+    to its offset and a one-thread kernel advances it afterwards, so every replay of a captured quantize draws
+    the next window (a host-side offset would be frozen into the captured launch).  Each replay equals the oracle
+    with the window the counter stood at."""
+    from tango_amd import config
+    n = 100003
+    x = torch.randn(n, device="cuda")
+    s = K.cuda_kernels.get_scale(x)
+    counter = torch.zeros(1, dtype=torch.int64, device="cuda")
+    out = torch.empty(n, dtype=torch.int8, device="cuda")
+
+    def step():
+        K.cuda_kernels.quantize(out, x, s, round_mode="stochastic", seed=9, offset=counter, advance=config.WINDOW)
+
+    stream = torch.cuda.Stream()
+    stream.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(stream):
+        step()  # warm-up outside capture: the counter now stands at one window
+    torch.cuda.current_stream().wait_stream(stream)
+    assert int(counter) == config.WINDOW
+    assert np.array_equal(host(out), orc.quantize(host(x), host(s)[0], orc.STOCHASTIC, seed=9, offset=0))
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        step()
+    seen = []
+    for k in range(1, 4):
+        x.mul_(1.0)  # eager work between replays
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert int(counter) == (k + 1) * config.WINDOW
+        got = host(out)
+        assert np.array_equal(got, orc.quantize(host(x), host(s)[0], orc.STOCHASTIC, seed=9, offset=k * config.WINDOW))
+        seen.append(got)
+    assert not np.array_equal(seen[0], seen[1]) and not np.array_equal(seen[1], seen[2])
+    # a host offset and the device word add up
+    counter.fill_(8)
+    K.cuda_kernels.quantize(out, x, s, round_mode="stochastic", seed=9, offset=counter)
+    out2 = torch.empty_like(out)
+    K.cuda_kernels.quantize(out2, x, s, round_mode="stochastic", seed=9, offset=8)
+    assert torch.equal(out, out2) and int(counter) == 8
