@@ -287,6 +287,18 @@ int tango_spmm_csr_u_mul_e_ex(float* out, const int64_t* indptr, const void* ind
                               int64_t max_row_nnz, void* workspace, size_t workspace_bytes,
                               tango_stream_t stream);
 
+/* As tango_spmm_csr_u_mul_e_ex with the edge values still in fp32 (no counterpart in the reference, which
+   quantizes them in a pass of its own, cuda/SPMM.py:41-43): each value is rounded to int8 as it is loaded,
+   half to even with the scale scale_e[0] (required; e.g. from tango_edge_softmax_fwd_ex), so the result is
+   what quantizing evals_f32 first and calling tango_spmm_csr_u_mul_e_ex with scale2 = scale_e gives, bit for
+   bit, without that pass and the int8 copy. */
+int tango_spmm_csr_u_mul_e_f32e(float* out, const int64_t* indptr, const void* indices,
+                                const void* edge_ids, int idx_bits, const int8_t* feat, const float* evals_f32,
+                                int edge_major, const float* scale, const float* scale_e, const float* bias,
+                                int act, int64_t rows, int64_t num_src, int64_t H, int64_t F, int64_t D, int64_t nnz,
+                                int64_t max_row_nnz, void* workspace, size_t workspace_bytes,
+                                tango_stream_t stream);
+
 /* incidence_SPMM (cuda/src/cuda.cpp:160-167 -> incidence_SPMM_impl, SPMM.cu:259-303):
    out[v, f] = scale[0] * float(sum_{i: node_ids[i] == v} E[edge_ids[i], f]).
    (node_ids, edge_ids) are the COO rows of the incidence matrix and must be
@@ -350,7 +362,27 @@ int tango_edge_softmax_fwd_static(float* a, const float* e, const int64_t* indpt
                                   const int64_t* edge_ids, int64_t rows, int64_t num_edges, int64_t H,
                                   float slope, tango_stream_t stream);
 
-/* de = dLeaky(e) * a * (da - sum_{same dst} a*da). */
+/* The attention block's forms of the two calls (no counterpart in the reference, where SDDMM, LeakyReLU, DGL's
+   edge softmax, get_scale and quantize are separate passes, evaluation/test_gat.py:141-151, cuda/SPMM.py:39-43).
+   Forward: e may be NULL when el, er [num_src / rows, H] fp32, their scales s_el, s_er and the edge list
+   (src, dst) in edge-id order are given: the logits are then formed on the fly,
+   e[edge, h] = q(el[src, h]) * s_el + q(er[dst, h]) * s_er with q the half-to-even int8 rounding, the values
+   tango_sddmm_ewise_f32q(add) would have written, and never reach memory.  scale_a (or NULL): receives
+   max(a) / 127, what the quantizer of a needs (it need not be initialised).  sign_out (or NULL):
+   [num_edges, ceil(H / 8)] bytes in the destination-major slot order, bit h % 8 of byte [slot, h / 8] = (e > 0),
+   all the backward pass needs of e.  Backward: e or sign_in (those bytes) supplies LeakyReLU's derivative
+   (neither is needed for slope 1); scale_de as scale_a, for max|de| / 127.  Both need the workspace. */
+int tango_edge_softmax_fwd_ex(float* a, float* scale_a, uint8_t* sign_out, const float* e, const float* el,
+                              const float* er, const float* s_el, const float* s_er, const int64_t* src,
+                              const int64_t* dst, const int64_t* indptr, const int64_t* edge_ids, int64_t rows,
+                              int64_t num_edges, int64_t H, float slope, void* workspace, size_t workspace_bytes,
+                              tango_stream_t stream);
+int tango_edge_softmax_bwd_ex(float* de, float* scale_de, const float* a, const float* da, const float* e,
+                              const uint8_t* sign_in, const int64_t* indptr, const int64_t* edge_ids, int64_t rows,
+                              int64_t num_edges, int64_t H, float slope, void* workspace, size_t workspace_bytes,
+                              tango_stream_t stream);
+
+/* de = dLeaky(e) * a * (da - sum_{same dst} a*da).  e may be NULL when slope is 1 (plain softmax: it is not read). */
 int tango_edge_softmax_bwd(float* de, const float* a, const float* da, const float* e,
                            const int64_t* indptr, const int64_t* edge_ids, int64_t rows,
                            int64_t num_edges, int64_t H, float slope, void* workspace,

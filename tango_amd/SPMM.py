@@ -108,13 +108,21 @@ class spmm_u_mul_e(Function):
     kernels that read dZ anyway (scale / bias gradient, quantize) instead of a separate pass."""
 
     @staticmethod
-    def forward(ctx, g, N, E, bias=None, scaleN=None, act=None):
+    def forward(ctx, g, N, E, bias=None, scaleN=None, act=None, scaleE=None):
+        """``scaleE``: max|E| / 127 when the producer of E knows it (the edge softmax's kernel does): E is then
+        neither scanned nor stored in int8, the aggregation rounds the fp32 values as it loads them, here and
+        in the backward pass (same int8 values, so the same results)."""
         N = N if N.is_contiguous() else N.contiguous()
         E = E if E.is_contiguous() else E.contiguous()
         # Edge values stay edge-major ([nnz, H, 1], plain quantize): the reference transposes them to
         # [H, 1, nnz] (cuda/SPMM.py:41) and then permutes that with index_select; with the permutation
         # fused into the gather, edge-major keeps the H bytes of an edge in one cache sector.
-        E_T_, scaleE = quantize(E)
+        if scaleE is not None and config.edge_values_on_load:
+            E_T_ = E  # fp32, quantized on load
+        elif scaleE is not None:
+            E_T_, _ = quantize(E, scaleE)  # no pass that looks for the scale
+        else:
+            E_T_, scaleE = quantize(E)
         N_, scaleN = quantize(N, scaleN)  # one absmax pass (the reference runs two, cuda/SPMM.py:39,43)
         # dequantized with scaleN * scaleE (cuda/SPMM.py:44); the kernel multiplies the two itself
         out = multi_cusparse_SPMM(g, N_, E_T_, scaleN, edge_major=True, bias=bias, scale2=scaleE, act=act)
@@ -162,4 +170,4 @@ class spmm_u_mul_e(Function):
             op = "dot" if reduce_last else "mul"
             dE, _ = mySDDMM_int8(g, op, N_, dZ_, scaleN, scaledZ, False)
             dE = dE.reshape(eshape)
-        return None, dN, dE, dbias, None, None
+        return None, dN, dE, dbias, None, None, None

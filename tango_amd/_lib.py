@@ -48,6 +48,7 @@ SIGNATURES = {
     "tango_spmm_csr_copy_u_ex": (I, [P, P, P, I, P, I64, P, P, P, I, P, I64, I64, I64, I64, I64, P, SZ, P]),
     "tango_spmm_csr_u_mul_e": (I, [P, P, P, P, P, P, P, I64, I64, I64, I64, I64, I64, P]),
     "tango_spmm_csr_u_mul_e_ex": (I, [P, P, P, P, I, P, P, I, P, P, P, I, I64, I64, I64, I64, I64, I64, I64, P, SZ, P]),
+    "tango_spmm_csr_u_mul_e_f32e": (I, [P, P, P, P, I, P, P, I, P, P, P, I, I64, I64, I64, I64, I64, I64, I64, P, SZ, P]),
     "tango_attn_scores_fwd": (I, [P, P, P, P, P, P, P, I64, I64, I64, P]),
     "tango_attn_scores_bwd_workspace": (SZ, [I64, I64, I64]),
     "tango_attn_scores_bwd": (I, [P, P, P, P, P, P, P, P, I64, I64, I64, P, SZ, P]),
@@ -60,6 +61,8 @@ SIGNATURES = {
     "tango_edge_softmax_workspace": (SZ, [I64, I64]),
     "tango_edge_softmax_fwd": (I, [P, P, P, P, I64, I64, I64, F, P, SZ, P]),
     "tango_edge_softmax_fwd_static": (I, [P, P, P, P, I64, I64, I64, F, P]),
+    "tango_edge_softmax_fwd_ex": (I, [P, P, P, P, P, P, P, P, P, P, P, P, I64, I64, I64, F, P, SZ, P]),
+    "tango_edge_softmax_bwd_ex": (I, [P, P, P, P, P, P, P, P, I64, I64, I64, F, P, SZ, P]),
     "tango_edge_softmax_bwd": (I, [P, P, P, P, P, P, I64, I64, I64, F, P, SZ, P]),
 }
 

@@ -12,6 +12,15 @@ ref_compat = os.environ.get("TANGO_REF_COMPAT", "0") == "1"
 # (cuda/QLinear.py:42, cuda/SPMM.py:20,53, cuda/SDDMM.py:26 use half-to-even).
 grad_round_mode = os.environ.get("TANGO_GRAD_ROUND", "rne")
 
+# spmm_u_mul_e with a scale handed in (the edge softmax's kernel finds it): round the fp32 edge values inside the
+# aggregation as they are loaded (no int8 copy, no quantize launch) instead of in a pass of their own.
+edge_values_on_load = os.environ.get("TANGO_EDGE_ON_LOAD", "0") == "1"
+
+# gat_edge_attention: form the logits q(el)[src] + q(er)[dst] inside the softmax kernel instead of storing them with
+# the element-wise SDDMM first.  Same values; measured slower on the benchmark graphs (the two dependent gathers
+# per slot lengthen the softmax kernel's latency chain by more than the stored tensor costs), hence off.
+attention_logits_on_the_fly = os.environ.get("TANGO_ATTN_ON_THE_FLY", "0") == "1"
+
 # Seed of the counter-based RNG for stochastic rounding; every quantize call
 # draws a fresh 2^40-element window of the stream.
 seed = int(os.environ.get("TANGO_SEED", "0"))

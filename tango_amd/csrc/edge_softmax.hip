@@ -91,7 +91,7 @@ __global__ __launch_bounds__(256) void edge_softmax_bwd_kernel(
         for (int64_t p = p0; p < p1; ++p) {
             const int64_t id = eids ? eids[p] : p;
             float g = a[id * H + h] * (da[id * H + h] - dot);
-            if (!(e[id * H + h] > 0.0f)) g *= slope;
+            if (e && !(e[id * H + h] > 0.0f)) g *= slope;  // e may be absent for slope 1
             de[id * H + h] = g;
         }
     }
@@ -114,6 +114,58 @@ __global__ __launch_bounds__(256) void edge_softmax_bwd_kernel(
 // writes the head and tail slots.  No atomics on results: they do not depend on scheduling.
 constexpr int kWin = 256 + kWave;  // row pointers inspected per span: 64 empty rows of slack
 
+// What the neighbours of the softmax in an attention layer fold into these kernels (all optional):
+//   el, er ..: the logits are formed here, e[edge, h] = q(el[src, h]) s_el + q(er[dst, h]) s_er with q the
+//              half-to-even int8 rounding of the two scales (what the quantize-on-load element-wise SDDMM
+//              writes out, same operations in the same order), instead of being read from memory;
+//   sign_out : forward, bit h % 8 of byte [slot, h / 8] = (e > 0), all the backward pass needs of e;
+//   sign_in  : backward, those bytes in place of e;
+//   scale_out: receives max|result| / 127, the scale the next quantizer needs, so that no separate pass over the
+//              result looks for it: every wavefront leaves the maximum of what it wrote in `part` (one word per
+//              wavefront of the two writing launches, plain stores: thousands of atomics on one word would be
+//              served one at a time) and a one-workgroup launch folds those.
+struct AttnFuse {
+    const float* el;
+    const float* er;
+    const float* s_el;
+    const float* s_er;
+    const int64_t* src;  // edge-id order
+    const int64_t* dst;
+    uint8_t* sign_out;
+    const uint8_t* sign_in;
+    float* scale_out;
+    float* part;  // [2][head blocks][spans] in the workspace
+};
+
+__device__ __forceinline__ float fused_logit(const AttnFuse& fz, int64_t edge, int H, int h, float r_el, float r_er,
+                                             float s_el, float s_er) {
+    const float u = static_cast<float>(quant_one<TANGO_ROUND_RNE>(fz.el[fz.src[edge] * H + h], r_el, 0.0f)) * s_el;
+    const float v = static_cast<float>(quant_one<TANGO_ROUND_RNE>(fz.er[fz.dst[edge] * H + h], r_er, 0.0f)) * s_er;
+    return u + v;
+}
+
+// the wavefront's maximum into its word of the partial results
+__device__ __forceinline__ void wave_part_out(float m, float* slot) {
+    m = wave_max(m);
+    if (lane_id() == 0) *slot = m;
+}
+
+// scale_out[0] = max(part[0 .. count)) / 127.  One workgroup of 1024.
+__global__ __launch_bounds__(1024) void scale_reduce_kernel(const float* __restrict__ part, int64_t count,
+                                                            float* __restrict__ scale_out) {
+    __shared__ float wm[16];
+    float m = 0.0f;
+    for (int64_t i = threadIdx.x; i < count; i += 1024) m = fmaxf(m, part[i]);
+    m = wave_max(m);
+    if ((threadIdx.x & 63) == 0) wm[threadIdx.x >> 6] = m;
+    __syncthreads();
+    if (threadIdx.x < 64) {
+        m = threadIdx.x < 16 ? wm[threadIdx.x] : 0.0f;
+        m = wave_max(m);
+        if (threadIdx.x == 0) scale_out[0] = m / 127.0f;
+    }
+}
+
 struct SpanMeta {
     int64_t head_end;    // slots [base, head_end) belong to a row that started before the span
     int64_t tail_start;  // slots [tail_start, end) belong to a row that runs on after the span
@@ -122,6 +174,10 @@ struct SpanMeta {
 
 __host__ __device__ inline size_t span_vals_offset(int64_t nspans) {
     return (static_cast<size_t>(nspans) * sizeof(SpanMeta) + 255) & ~static_cast<size_t>(255);
+}
+// after the records' values: one word per wavefront of the two launches that write results (see AttnFuse::part)
+__host__ __device__ inline size_t span_parts_offset(int64_t nspans, int64_t H) {
+    return span_vals_offset(nspans) + static_cast<size_t>(nspans) * 4 * static_cast<size_t>(H) * sizeof(float);
 }
 // vals[span][piece][component][H]: component 0 = max, 1 = sum (backward: only the sum)
 __device__ __forceinline__ float* span_vals(void* ws, int64_t nspans, int64_t w, int piece, int comp, int H) {
@@ -226,7 +282,7 @@ template <int HB, int K, bool FWD>
 __global__ __launch_bounds__(256) void span_kernel(
     float* __restrict__ out, const float* __restrict__ a, const float* __restrict__ da,
     const float* __restrict__ e, const int64_t* __restrict__ indptr, const int64_t* __restrict__ eids,
-    int64_t rows, int64_t nnz, int H, float slope, void* __restrict__ ws) {
+    int64_t rows, int64_t nnz, int H, float slope, void* __restrict__ ws, const AttnFuse fz) {
     constexpr int G = kWave / HB;
     constexpr int SPAN = G * K;
     static_assert(SPAN <= 256 && (32 % K) == 0, "a lane's row-start bits must sit in one mask word");
@@ -247,6 +303,13 @@ __global__ __launch_bounds__(256) void span_kernel(
     // ---- values first: their loads are in flight while the row structure is worked out
     int64_t id[K];
     float x[K], y[K];
+    unsigned posbits = 0u;  // bit k: the logit of slot k is positive (LeakyReLU's derivative is 1)
+    const int nhb = (H + 7) >> 3;  // sign bytes per slot
+    float s_el = 0.0f, s_er = 0.0f, r_el = 0.0f, r_er = 0.0f;
+    if (FWD && fz.el) {
+        s_el = fz.s_el[0], s_er = fz.s_er[0];
+        r_el = rscale_of(s_el), r_er = rscale_of(s_er);
+    }
 #pragma unroll
     for (int k = 0; k < K; ++k) {
         const int j = g * K + k;
@@ -254,13 +317,31 @@ __global__ __launch_bounds__(256) void span_kernel(
         x[k] = FWD ? -INFINITY : 0.0f;
         y[k] = 0.0f;
         if (j < endl && hok) {
-            id[k] = (eids ? eids[base + j] : base + j) * H + h0 + h;
+            const int64_t edge = eids ? eids[base + j] : base + j;
+            id[k] = edge * H + h0 + h;
             if (FWD) {
-                x[k] = leaky(e[id[k]], slope);
+                const float ev = fz.el ? fused_logit(fz, edge, H, h0 + h, r_el, r_er, s_el, s_er) : e[id[k]];
+                posbits |= (ev > 0.0f ? 1u : 0u) << k;
+                x[k] = leaky(ev, slope);
             } else {
                 x[k] = a[id[k]];
                 y[k] = da[id[k]];
+                bool pos = true;
+                if (fz.sign_in) pos = (fz.sign_in[(base + j) * nhb + ((h0 + h) >> 3)] >> ((h0 + h) & 7)) & 1;
+                else if (e) pos = e[id[k]] > 0.0f;
+                posbits |= (pos ? 1u : 0u) << k;
             }
+        }
+    }
+    if (FWD && fz.sign_out) {
+        // A lane group holds HB <= 8 heads of a slot, and head blocks narrower than eight only occur when they
+        // hold every head (H <= HB), so each sign byte is written whole by one lane.
+#pragma unroll
+        for (int k = 0; k < K; ++k) {
+            const uint64_t bal = __ballot((posbits >> k) & 1u);
+            const int j = g * K + k;
+            if (h == 0 && j < endl)
+                fz.sign_out[(base + j) * nhb + (h0 >> 3)] = static_cast<uint8_t>((bal >> (g * HB)) & ((1u << HB) - 1u));
         }
     }
 
@@ -361,18 +442,22 @@ __global__ __launch_bounds__(256) void span_kernel(
     }
 
     // ---- rows inside the span: write
+    float amax = 0.0f;
 #pragma unroll
     for (int k = 0; k < K; ++k) {
         const int j = g * K + k;
         if (id[k] < 0 || j < hpos || j >= tpos) continue;
+        float o;
         if (FWD) {
-            out[id[k]] = x[k] * __builtin_amdgcn_rcpf(rs[k]);  // 1 ulp: an IEEE divide is ten instructions per value
+            o = x[k] * __builtin_amdgcn_rcpf(rs[k]);  // 1 ulp: an IEEE divide is ten instructions per value
         } else {
-            float gr = x[k] * (y[k] - rs[k]);
-            if (!(e[id[k]] > 0.0f)) gr *= slope;
-            out[id[k]] = gr;
+            o = x[k] * (y[k] - rs[k]);
+            if (!((posbits >> k) & 1u)) o *= slope;
         }
+        out[id[k]] = o;
+        amax = fmaxf(amax, fabsf(o));
     }
+    if (fz.scale_out) wave_part_out(amax, fz.part + static_cast<int64_t>(blockIdx.y) * nspans + w);
 }
 
 __device__ __forceinline__ void merge_max_sum(float& m, float& s, float m2, float s2) {
@@ -451,7 +536,7 @@ template <int HB, bool VEC, bool FWD>
 __global__ __launch_bounds__(256) void span_rest_kernel(
     float* __restrict__ out, const float* __restrict__ a, const float* __restrict__ da,
     const float* __restrict__ e, const int64_t* __restrict__ eids, int64_t nnz, int span, int H, float slope,
-    void* __restrict__ ws) {
+    void* __restrict__ ws, const AttnFuse fz) {
     const int lane = lane_id();
     const int64_t nspans = (nnz + span - 1) / span;
     const int64_t w = static_cast<int64_t>(blockIdx.x) * 4 + (static_cast<int>(threadIdx.x) >> 6);
@@ -459,7 +544,11 @@ __global__ __launch_bounds__(256) void span_rest_kernel(
     const SpanMeta mt = static_cast<const SpanMeta*>(ws)[w];
     const int64_t base = static_cast<int64_t>(w) * span;
     const int64_t end = base + span < nnz ? base + span : nnz;
-    if (mt.head_end <= base && mt.tail_start >= end) return;
+    float* const my_part = fz.part + (static_cast<int64_t>(gridDim.y) + blockIdx.y) * nspans + w;
+    if (mt.head_end <= base && mt.tail_start >= end) {
+        if (fz.scale_out && lane == 0) *my_part = 0.0f;
+        return;
+    }
     const int h0 = static_cast<int>(blockIdx.y) * HB;
     const int nh = H - h0 < HB ? H - h0 : HB;
     float rm[2][HB], rs[2][HB];
@@ -472,15 +561,35 @@ __global__ __launch_bounds__(256) void span_rest_kernel(
             rs[piece][i] = (have && i < nh) ? *(span_vals(ws, nspans, w, piece, 1, H) + h0 + i) : 1.0f;
         }
     }
+    const int nhb = (H + 7) >> 3;
+    float s_el = 0.0f, s_er = 0.0f, r_el = 0.0f, r_er = 0.0f;
+    if (FWD && fz.el) {
+        s_el = fz.s_el[0], s_er = fz.s_er[0];
+        r_el = rscale_of(s_el), r_er = rscale_of(s_er);
+    }
+    float amax = 0.0f;
     for (int u = 0; u < span / kWave; ++u) {
         const int64_t s = base + kWave * u + lane;
         const bool inhead = s < mt.head_end;
         const bool intail = s >= mt.tail_start && s < end;
         if (!inhead && !intail) continue;
         const int piece = inhead ? 0 : 1;
-        const int64_t id = (eids ? eids[s] : s) * H + h0;
+        const int64_t edge = eids ? eids[s] : s;
+        const int64_t id = edge * H + h0;
         float o[HB], z[HB];
-        load_heads<HB, VEC>(z, e + id, nh);
+        if (FWD && fz.el) {
+#pragma unroll
+            for (int i = 0; i < HB; ++i) z[i] = i < nh ? fused_logit(fz, edge, H, h0 + i, r_el, r_er, s_el, s_er) : 0.0f;
+        } else if (!FWD && fz.sign_in) {
+            const unsigned bits = fz.sign_in[s * nhb + (h0 >> 3)] >> (h0 & 7);
+#pragma unroll
+            for (int i = 0; i < HB; ++i) z[i] = ((bits >> i) & 1u) ? 1.0f : -1.0f;
+        } else if (e) {
+            load_heads<HB, VEC>(z, e + id, nh);
+        } else {
+#pragma unroll
+            for (int i = 0; i < HB; ++i) z[i] = 1.0f;
+        }
         if (FWD) {
 #pragma unroll
             for (int i = 0; i < HB; ++i)
@@ -497,7 +606,11 @@ __global__ __launch_bounds__(256) void span_rest_kernel(
             }
         }
         store_heads<HB, VEC>(out + id, o, nh);
+#pragma unroll
+        for (int i = 0; i < HB; ++i)
+            if (i < nh) amax = fmaxf(amax, fabsf(o[i]));
     }
+    if (fz.scale_out) wave_part_out(amax, my_part);
 }
 
 // slots per span by head count: lanes are (group, head) pairs, K slots per lane
@@ -506,22 +619,27 @@ static int span_slots(int H) { return H % 8 == 0 || H > 4 ? 128 : 256; }
 template <int HB, int K, bool VEC, bool FWD>
 static void launch_spans_hb(float* out, const float* a, const float* da, const float* e, const int64_t* indptr,
                             const int64_t* eids, int64_t rows, int64_t nnz, int H, float slope, void* ws,
-                            hipStream_t s) {
+                            hipStream_t s, const AttnFuse& fz_) {
     constexpr int SPAN = (kWave / HB) * K;
     const int64_t nspans = ceil_div(nnz, SPAN);
     const dim3 grid(static_cast<unsigned>(ceil_div(nspans, 4)), static_cast<unsigned>(ceil_div(H, HB)));
+    AttnFuse fz = fz_;
+    fz.part = reinterpret_cast<float*>(static_cast<char*>(ws) + span_parts_offset(nspans, H));
     hipLaunchKernelGGL((span_kernel<HB, K, FWD>), grid, dim3(256), 0, s, out, a, da, e, indptr, eids, rows, nnz, H,
-                       slope, ws);
+                       slope, ws, fz);
     hipLaunchKernelGGL(span_fix_kernel<FWD>, dim3(grid.x), dim3(256), 0, s, nnz, SPAN, H, ws);
     hipLaunchKernelGGL((span_rest_kernel<HB, VEC, FWD>), grid, dim3(256), 0, s, out, a, da, e, eids, nnz, SPAN, H,
-                       slope, ws);
+                       slope, ws, fz);
+    if (fz.scale_out)
+        hipLaunchKernelGGL(scale_reduce_kernel, dim3(1), dim3(1024), 0, s, fz.part, 2 * static_cast<int64_t>(grid.y) * nspans,
+                           fz.scale_out);
 }
 
 template <bool FWD>
 static void launch_spans(float* out, const float* a, const float* da, const float* e, const int64_t* indptr,
                          const int64_t* eids, int64_t rows, int64_t nnz, int H, float slope, void* ws,
-                         hipStream_t s) {
-#define TANGO_SPANS(HB, K, VEC) launch_spans_hb<HB, K, VEC, FWD>(out, a, da, e, indptr, eids, rows, nnz, H, slope, ws, s)
+                         hipStream_t s, const AttnFuse& fz = AttnFuse{}) {
+#define TANGO_SPANS(HB, K, VEC) launch_spans_hb<HB, K, VEC, FWD>(out, a, da, e, indptr, eids, rows, nnz, H, slope, ws, s, fz)
     if (H % 8 == 0) TANGO_SPANS(8, 16, true);
     else if (H > 4) TANGO_SPANS(8, 16, false);
     else if (H == 4) TANGO_SPANS(4, 16, true);
@@ -534,7 +652,9 @@ static void launch_spans(float* out, const float* a, const float* da, const floa
 static size_t span_workspace_bytes(int64_t nnz, int64_t H) {
     if (nnz <= 0 || H <= 0) return 0;
     const int64_t nspans = ceil_div(nnz, span_slots(static_cast<int>(H < 64 ? H : 64)));
-    return span_vals_offset(nspans) + static_cast<size_t>(nspans) * 4 * static_cast<size_t>(H) * sizeof(float);
+    // head blocks are min(H, 8) heads wide: one for H <= 8, else ceil(H / 8)
+    const int64_t blocks = H <= 8 ? 1 : ceil_div(H, 8);
+    return span_parts_offset(nspans, H) + static_cast<size_t>(2 * blocks * nspans) * sizeof(float);
 }
 
 }  // namespace tango
@@ -578,13 +698,55 @@ int tango_edge_softmax_fwd_static(float* a, const float* e, const int64_t* indpt
     return launch_status();
 }
 
+int tango_edge_softmax_fwd_ex(float* a, float* scale_a, uint8_t* sign_out, const float* e, const float* el,
+                              const float* er, const float* s_el, const float* s_er, const int64_t* src,
+                              const int64_t* dst, const int64_t* indptr, const int64_t* edge_ids, int64_t rows,
+                              int64_t nnz, int64_t H, float slope, void* workspace, size_t workspace_bytes,
+                              tango_stream_t stream) {
+    if (rows < 0 || nnz < 0 || H < 0 || (rows > 0 && !indptr) || H >= (1LL << 31)) return TANGO_ERR_INVALID_ARG;
+    if (rows * H == 0 || nnz == 0) return TANGO_OK;
+    if (!a) return TANGO_ERR_INVALID_ARG;
+    const bool fused = el != nullptr;
+    if (fused ? (!er || !s_el || !s_er || !src || !dst) : !e) return TANGO_ERR_INVALID_ARG;
+    if (!workspace) return TANGO_ERR_WORKSPACE;  // only the slot-span kernels carry the fused forms
+    if (ceil_div(nnz, 4 * 128) > INT32_MAX || ceil_div(H, 8) > 65535) return TANGO_ERR_UNSUPPORTED;
+    if (workspace_bytes < span_workspace_bytes(nnz, H) || (reinterpret_cast<uintptr_t>(workspace) & 15))
+        return TANGO_ERR_WORKSPACE;
+    hipStream_t s = as_stream(stream);
+    AttnFuse fz{};
+    fz.el = el; fz.er = er; fz.s_el = s_el; fz.s_er = s_er; fz.src = src; fz.dst = dst;
+    fz.sign_out = sign_out; fz.scale_out = scale_a;
+    launch_spans<true>(a, nullptr, nullptr, e, indptr, edge_ids, rows, nnz, static_cast<int>(H), slope, workspace, s,
+                       fz);
+    return launch_status();
+}
+
+int tango_edge_softmax_bwd_ex(float* de, float* scale_de, const float* a, const float* da, const float* e,
+                              const uint8_t* sign_in, const int64_t* indptr, const int64_t* edge_ids, int64_t rows,
+                              int64_t nnz, int64_t H, float slope, void* workspace, size_t workspace_bytes,
+                              tango_stream_t stream) {
+    if (rows < 0 || nnz < 0 || H < 0 || (rows > 0 && !indptr) || H >= (1LL << 31)) return TANGO_ERR_INVALID_ARG;
+    if (rows * H == 0 || nnz == 0) return TANGO_OK;
+    if (!de || !a || !da) return TANGO_ERR_INVALID_ARG;
+    if (!e && !sign_in && slope != 1.0f) return TANGO_ERR_INVALID_ARG;  // LeakyReLU's derivative needs one of them
+    if (!workspace) return TANGO_ERR_WORKSPACE;
+    if (ceil_div(nnz, 4 * 128) > INT32_MAX || ceil_div(H, 8) > 65535) return TANGO_ERR_UNSUPPORTED;
+    if (workspace_bytes < span_workspace_bytes(nnz, H) || (reinterpret_cast<uintptr_t>(workspace) & 15))
+        return TANGO_ERR_WORKSPACE;
+    AttnFuse fz{};
+    fz.sign_in = sign_in; fz.scale_out = scale_de;
+    launch_spans<false>(de, a, da, e, indptr, edge_ids, rows, nnz, static_cast<int>(H), slope, workspace,
+                        as_stream(stream), fz);
+    return launch_status();
+}
+
 int tango_edge_softmax_bwd(float* de, const float* a, const float* da, const float* e,
                            const int64_t* indptr, const int64_t* edge_ids, int64_t rows, int64_t nnz,
                            int64_t H, float slope, void* workspace, size_t workspace_bytes,
                            tango_stream_t stream) {
     if (rows < 0 || nnz < 0 || H < 0 || (rows > 0 && !indptr) || H >= (1LL << 31)) return TANGO_ERR_INVALID_ARG;
     if (rows * H == 0 || nnz == 0) return TANGO_OK;
-    if (!de || !a || !da || !e) return TANGO_ERR_INVALID_ARG;
+    if (!de || !a || !da || (!e && slope != 1.0f)) return TANGO_ERR_INVALID_ARG;
     if (workspace && ceil_div(nnz, 4 * 128) <= INT32_MAX && ceil_div(H, 8) <= 65535) {
         if (workspace_bytes < span_workspace_bytes(nnz, H) || (reinterpret_cast<uintptr_t>(workspace) & 15))
             return TANGO_ERR_WORKSPACE;

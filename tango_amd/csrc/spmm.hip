@@ -36,6 +36,8 @@ struct SpmmParams {
     const int64_t* edge_ids;  // weighted kind: slot -> position in evals, or null
     const int8_t* feat;
     const int8_t* evals;
+    const float* evals_f32;  // weighted kind, instead of evals: fp32 edge values, rounded to int8 (half to even,
+                             // scale scale2[0]) as they are loaded; same strides, counted in elements
     const float* scale;
     const float* scale2;     // optional second factor of the dequantization scale (s = scale[0] * scale2[0])
     const float* row_scale;  // optional: out row r is multiplied by row_scale[r] after dequantization
@@ -154,7 +156,16 @@ struct LaneCols {
     bool col_ok;
     const int8_t* fcol;   // feat + col (column 0 for lanes past the row's width)
     const int8_t* wbase;  // weighted kind: evals + this lane's head / value-column offset
+    const float* wbase_f;  // the same for fp32 edge values that are quantized on load
+    float ev_r;            // 1 / their scale
 };
+
+// The int8 edge value at position pos (in units of ev_se) as the multiplier byte of a v_dot4.
+__device__ __forceinline__ uint32_t edge_value(const SpmmParams& p, const LaneCols& c, int64_t pos) {
+    if (p.evals_f32)  // uniform
+        return static_cast<uint32_t>(quant_one<TANGO_ROUND_RNE>(c.wbase_f[pos * p.ev_se], c.ev_r, 0.0f)) & 0xffu;
+    return static_cast<uint32_t>(static_cast<uint8_t>(c.wbase[pos * p.ev_se]));
+}
 
 template <int VEC, int KIND>
 __device__ __forceinline__ LaneCols lane_cols(const SpmmParams& p, int lane) {
@@ -170,10 +181,16 @@ __device__ __forceinline__ LaneCols lane_cols(const SpmmParams& p, int lane) {
     // group fold only mixes lanes of equal `sub`, so they need no masking.
     c.fcol = p.feat + (c.col_ok ? c.col : 0);
     c.wbase = p.evals;
+    c.wbase_f = p.evals_f32;
+    c.ev_r = 0.0f;
     if (KIND == KIND_WEIGHTED && c.col_ok) {
         const int64_t h = c.col / p.F;
         const int64_t d = (p.D == 1) ? 0 : (c.col - h * p.F);
         c.wbase = p.evals + h * p.ev_sh + d * p.ev_sd;
+        if (p.evals_f32) {
+            c.wbase_f = p.evals_f32 + h * p.ev_sh + d * p.ev_sd;
+            c.ev_r = rscale_of(p.scale2[0]);
+        }
     }
     return c;
 }
@@ -234,7 +251,7 @@ __device__ __forceinline__ void wave_row_sum(const SpmmParams& p, const LaneCols
                 d[u] = Gather<VEC>::load(c.fcol + row_offset(ok ? j[u] : 0, p));
                 uint32_t w = 1u;
                 if (KIND == KIND_WEIGHTED)
-                    w = static_cast<uint32_t>(static_cast<uint8_t>(c.wbase[(ok ? sl[u] : 0) * p.ev_se]));
+                    w = edge_value(p, c, ok ? sl[u] : 0);
                 m |= (ok ? w : 0u) << (8 * u);
             }
             accumulate4<VEC>(acc, d, m);
@@ -428,7 +445,7 @@ __global__ __launch_bounds__(256) void spmm_group_kernel(const SpmmParams p) {
                 if (permuted)
                     pos = staged ? seid[KIND == KIND_WEIGHTED ? wave : 0][(c.grp << 5) + slot]
                                  : load_index<false>(p, p.edge_ids, start + slot);
-                w = static_cast<uint32_t>(static_cast<uint8_t>(c.wbase[pos * p.ev_se]));
+                w = edge_value(p, c, pos);
             }
             m |= (ok ? w : 0u) << (8 * u);
         }
@@ -886,7 +903,7 @@ __global__ __launch_bounds__(256) void spmm_span_kernel(const SpmmParams p) {
             uint32_t wv = 1u;
             if (KIND == KIND_WEIGHTED) {
                 const int64_t pos = permuted ? static_cast<int64_t>(seid[sl]) : base + sl;
-                wv = static_cast<uint32_t>(static_cast<uint8_t>(c.wbase[pos * p.ev_se]));
+                wv = edge_value(p, c, pos);
             }
             m |= (ok ? wv : 0u) << (8 * u);
         }
@@ -1195,16 +1212,17 @@ int tango_spmm_csr_copy_u_ex(float* out, const int64_t* indptr, const void* indi
     return launch_spmm<KIND_COPY>(p, pick_vec(feat, ldf, F), as_stream(stream));
 }
 
-int tango_spmm_csr_u_mul_e_ex(float* out, const int64_t* indptr, const void* indices,
+static int spmm_u_mul_e_common(float* out, const int64_t* indptr, const void* indices,
                               const void* edge_ids, int idx_bits, const int8_t* feat, const int8_t* evals,
+                              const float* evals_f32,
                               int edge_major, const float* scale, const float* scale2, const float* bias,
                               int act, int64_t rows,
                               int64_t num_src, int64_t H, int64_t F, int64_t D, int64_t nnz,
                               int64_t max_row_nnz, void* workspace, size_t workspace_bytes,
                               tango_stream_t stream) {
     if (rows < 0 || H < 0 || F < 0 || nnz < 0 || num_src < 0 || !scale || !indptr || max_row_nnz < 0 ||
-        (rows * H * F > 0 && !out) || (nnz > 0 && (!indices || !feat || !evals)) ||
-        (idx_bits != 32 && idx_bits != 64))
+        (rows * H * F > 0 && !out) || (nnz > 0 && (!indices || !feat || (!evals && !evals_f32))) ||
+        (idx_bits != 32 && idx_bits != 64) || (evals_f32 && !scale2))
         return TANGO_ERR_INVALID_ARG;
     if (workspace && (workspace_bytes < tango_spmm_workspace(rows, nnz, H * F) || (reinterpret_cast<uintptr_t>(workspace) & 15)))
         return TANGO_ERR_WORKSPACE;
@@ -1214,7 +1232,7 @@ int tango_spmm_csr_u_mul_e_ex(float* out, const int64_t* indptr, const void* ind
     p.out = out; p.indptr = indptr; p.indices = static_cast<const int64_t*>(indices);
     p.edge_ids = static_cast<const int64_t*>(edge_ids); p.idx32 = idx_bits == 32; p.feat = feat;
     p.relu = act; p.max_row = max_row_nnz; p.hub_ws = workspace; p.span_ws = workspace; p.span_ws_bytes = workspace_bytes;
-    p.evals = evals; p.scale = scale; p.scale2 = scale2; p.bias = bias; p.rows = rows; p.num_src = num_src; p.ldf = H * F; p.W = H * F; p.F = F; p.D = D;
+    p.evals = evals; p.evals_f32 = evals_f32; p.scale = scale; p.scale2 = scale2; p.bias = bias; p.rows = rows; p.num_src = num_src; p.ldf = H * F; p.W = H * F; p.F = F; p.D = D;
     p.nnz = nnz;
     if (edge_major) {  // evals[nnz, H, D]: the H * D bytes of one edge share a cache sector
         p.ev_se = H * D; p.ev_sh = D; p.ev_sd = 1;
@@ -1229,6 +1247,29 @@ int tango_spmm_csr_u_mul_e_ex(float* out, const int64_t* indptr, const void* ind
         else if ((F & 3) == 0 && (a & 3) == 0) vec = 4;
     }
     return launch_spmm<KIND_WEIGHTED>(p, vec, as_stream(stream));
+}
+
+int tango_spmm_csr_u_mul_e_ex(float* out, const int64_t* indptr, const void* indices,
+                              const void* edge_ids, int idx_bits, const int8_t* feat, const int8_t* evals,
+                              int edge_major, const float* scale, const float* scale2, const float* bias,
+                              int act, int64_t rows, int64_t num_src, int64_t H, int64_t F, int64_t D, int64_t nnz,
+                              int64_t max_row_nnz, void* workspace, size_t workspace_bytes,
+                              tango_stream_t stream) {
+    return spmm_u_mul_e_common(out, indptr, indices, edge_ids, idx_bits, feat, evals, nullptr, edge_major, scale, scale2,
+                               bias, act, rows, num_src, H, F, D, nnz, max_row_nnz, workspace, workspace_bytes, stream);
+}
+
+int tango_spmm_csr_u_mul_e_f32e(float* out, const int64_t* indptr, const void* indices,
+                                const void* edge_ids, int idx_bits, const int8_t* feat, const float* evals_f32,
+                                int edge_major, const float* scale, const float* scale_e, const float* bias,
+                                int act, int64_t rows, int64_t num_src, int64_t H, int64_t F, int64_t D, int64_t nnz,
+                                int64_t max_row_nnz, void* workspace, size_t workspace_bytes,
+                                tango_stream_t stream) {
+    if (nnz > 0 && !evals_f32) return TANGO_ERR_INVALID_ARG;
+    if ((reinterpret_cast<uintptr_t>(evals_f32) & 3) != 0) return TANGO_ERR_INVALID_ARG;
+    return spmm_u_mul_e_common(out, indptr, indices, edge_ids, idx_bits, feat, nullptr, evals_f32, edge_major, scale,
+                               scale_e, bias, act, rows, num_src, H, F, D, nnz, max_row_nnz, workspace, workspace_bytes,
+                               stream);
 }
 
 int tango_spmm_csr_u_mul_e(float* out, const int64_t* indptr, const int64_t* indices,

@@ -13,7 +13,12 @@ from .QLinear import QLinear, Qlinear_func_reduce, shared_input_linears
 from .kernels import cuda_kernels, refuse_capture
 from .SDDMM import sddmm_u_add_v, sddmm_u_dot_v
 from .SPMM import spmm_u_mul_e
-from .edge_softmax import edge_softmax
+from .edge_softmax import edge_softmax, gat_edge_attention
+
+
+# Whether the GAT layers run u_add_v + LeakyReLU + edge softmax as one op (gat_edge_attention); the separate ops
+# give the same values and remain for stream capture and for comparison.
+fused_attention = True
 
 
 class attn_scores(Function):
@@ -90,16 +95,23 @@ class QGATConv(nn.Module):
         feat_src, s_feat = self.fc(h)
         feat_src = feat_src.view(n, self._num_heads, self._out_feats)
         el, er, s_el, s_er = attn_scores.apply(feat_src, self.attn_l, self.attn_r)  # test_gat.py:135-137
-        e = sddmm_u_add_v.apply(graph, el, er, s_el, s_er)          # :141
-        a = edge_softmax(graph, e, negative_slope=self.negative_slope)  # LeakyReLU :144 + softmax :146
-        a = self.attn_drop(a)
+        s_a = None
+        if s_el is not None and fused_attention:
+            # u_add_v :141, LeakyReLU :144 and the softmax :146 as one op that also hands the aggregation
+            # max(a) / 127; e is never stored
+            a, s_a = gat_edge_attention.apply(graph, el, er, s_el, s_er, self.negative_slope)
+        else:
+            e = sddmm_u_add_v.apply(graph, el, er, s_el, s_er)          # :141
+            a = edge_softmax(graph, e, negative_slope=self.negative_slope)  # LeakyReLU :144 + softmax :146
+        if self.attn_drop.p > 0 and self.training:
+            a, s_a = self.attn_drop(a), None  # the dropped-out tensor has another maximum
         # without a residual branch the bias add (:160-162) rides in the aggregation's epilogue
         fold_bias = self.bias is not None and self.res_fc is None
         # and so does the activation (:164-165) when nothing else is added between the two
         fold_act = None
         if self.res_fc is None and (fold_bias or self.bias is None):
             fold_act = "elu" if self.activation is F.elu else "relu" if self.activation in (F.relu, torch.relu) else None
-        rst = spmm_u_mul_e.apply(graph, feat_src, a, self.bias if fold_bias else None, s_feat, fold_act)  # :151
+        rst = spmm_u_mul_e.apply(graph, feat_src, a, self.bias if fold_bias else None, s_feat, fold_act, s_a)  # :151
         if self.res_fc is not None:
             rst = rst + self.res_fc(h).view(n, -1, self._out_feats)
         if self.bias is not None and not fold_bias:
@@ -168,8 +180,8 @@ class HGTLayer(nn.Module):
             h, (self.k_linear, self.v_linear, self.q_linear), s_h, then=(self.attn_linear, self.msg_linear, None))
         k, v, q = (t.view(-1, self.n_heads, self.d_k) for t in (k, v, q))
         t = sddmm_u_dot_v.apply(g, k, q, s_k, s_q, 1.0 / self.sqrt_dk)  # "/ sqrt_dk" folded into the scales
-        attn = edge_softmax(g, t)
-        t = spmm_u_mul_e.apply(g, v, attn, None, s_v).reshape(-1, self.out_dim)
+        attn, s_attn = edge_softmax(g, t, want_scale=True)  # the softmax kernel also finds the scale of its output
+        t = spmm_u_mul_e.apply(g, v, attn, None, s_v, None, s_attn).reshape(-1, self.out_dim)
         if return_scale:
             return Qlinear_func_reduce.apply(t, self.a_linear.weight, self.a_linear.bias)
         return self.a_linear(t)
@@ -226,13 +238,19 @@ class ArxivGATConv(nn.Module):
         else:
             feat_src, s_feat = self.fc(h)
             feat_src = feat_src.view(n, self._num_heads, self._out_feats)
+        s_a = None
         if self.attn_r is not None:  # :176-184
             el, er, s_el, s_er = attn_scores.apply(feat_src, self.attn_l, self.attn_r)
-            e = sddmm_u_add_v.apply(graph, el, er, s_el, s_er)
+            if s_el is not None and fused_attention:
+                a, s_a = gat_edge_attention.apply(graph, el, er, s_el, s_er, self.negative_slope)  # :184, :187, :196
+            else:
+                a = edge_softmax(graph, sddmm_u_add_v.apply(graph, el, er, s_el, s_er), negative_slope=self.negative_slope)
         else:  # copy_u of el (:186)
             e = (feat_src * self.attn_l).sum(-1, keepdim=True)[graph.coo[0]]
-        a = self.attn_drop(edge_softmax(graph, e, negative_slope=self.negative_slope))  # :187, :196
-        rst = spmm_u_mul_e.apply(graph, feat_src, a, None, s_feat)  # :201
+            a, s_a = edge_softmax(graph, e, negative_slope=self.negative_slope, want_scale=True)  # :187, :196
+        if self.attn_drop.p > 0 and self.training:
+            a, s_a = self.attn_drop(a), None
+        rst = spmm_u_mul_e.apply(graph, feat_src, a, None, s_feat, None, s_a)  # :201
         if self._use_symmetric_norm:  # :203-208
             rst = rst * graph.in_degrees().float().clamp(min=1).pow(0.5).view(n, 1, 1)
         if self.res_fc is not None:  # :211-214

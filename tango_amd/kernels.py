@@ -109,10 +109,14 @@ def _zero_slot(device):
     key = (device.type, device.index)
     with _ZERO_SLOTS_LOCK:
         pool = _ZERO_SLOTS.get(key)
+        stream = torch.cuda.current_stream(device)
         if pool is None or pool[1] >= _POOL_SIZE:
-            pool = _ZERO_SLOTS[key] = [torch.zeros(_POOL_SIZE, dtype=torch.float32, device=device), 0]
-            # slots may be used on any stream later: have the one fill finished before the first is handed out
-            torch.cuda.current_stream(device).synchronize()
+            zeros = torch.zeros(_POOL_SIZE, dtype=torch.float32, device=device)
+            done = torch.cuda.Event()
+            done.record(stream)  # the fill is ordered on this stream; other streams wait for the event below
+            pool = _ZERO_SLOTS[key] = [zeros, 0, stream.cuda_stream, done]
+        elif pool[2] != stream.cuda_stream:
+            stream.wait_event(pool[3])  # a device-side wait (no host synchronisation) on the pool's one fill
         k = pool[1]
         pool[1] = k + 1
     return pool[0][k:k + 1]
@@ -525,10 +529,13 @@ class cuda_kernels:
         _need(indptr, torch.int64, "indptr")
         idx_bits = _need_index(indices, "indices")
         _need(N, torch.int8, "N")
-        _need(E_T, torch.int8, "E_T")
+        on_load = E_T.dtype == torch.float32  # fp32 edge values, rounded with scale2 as the kernel loads them
+        _need(E_T, torch.float32 if on_load else torch.int8, "E_T")
         _need(scale, torch.float32, "scale")
         if scale2 is not None:
             _need(scale2, torch.float32, "scale2")
+        if on_load and scale2 is None:
+            raise RuntimeError("multi_cusparse_SPMM: fp32 edge values need their quantization scale (scale2)")
         if N.dim() != 3 or E_T.dim() != 3:
             raise RuntimeError("E and N must be 3D tensors")
         k, H, F = N.shape
@@ -550,11 +557,12 @@ class cuda_kernels:
         out = torch.empty((rows, H, F), dtype=torch.float32, device=N.device)
         ws_bytes = _ws_bytes("tango_spmm_workspace", rows, nnz, H * F)
         ws = _workspace(ws_bytes, N.device)
-        check(_L.tango_spmm_csr_u_mul_e_ex(_ptr(out), indptr.data_ptr(), _ptr(indices), _ptr(edge_ids), idx_bits,
-                                           _ptr(N), _ptr(E_T), int(bool(edge_major)), scale.data_ptr(),
-                                           _ptr(scale2), _ptr(bias), _ACTIVATIONS[act], rows, k, H, F, D, nnz,
-                                           int(max_row), _ptr(ws), ws_bytes,
-                                           _stream()), "multi_cusparse_SPMM")
+        entry = _L.tango_spmm_csr_u_mul_e_f32e if on_load else _L.tango_spmm_csr_u_mul_e_ex
+        check(entry(_ptr(out), indptr.data_ptr(), _ptr(indices), _ptr(edge_ids), idx_bits,
+                    _ptr(N), _ptr(E_T), int(bool(edge_major)), scale.data_ptr(),
+                    _ptr(scale2), _ptr(bias), _ACTIVATIONS[act], rows, k, H, F, D, nnz,
+                    int(max_row), _ptr(ws), ws_bytes,
+                    _stream()), "multi_cusparse_SPMM")
         return out
 
     # The reference's SpMV binding returns uninitialised memory (cuda/src/SPMM.cu:196-257)
@@ -645,16 +653,70 @@ class cuda_kernels:
         return a
 
     @staticmethod
-    def edge_softmax_backward(a, da, e, indptr, edge_ids, slope=1.0):
+    def edge_softmax_forward_ex(e, indptr, edge_ids, slope=1.0, logits=None, want_sign=False):
+        """The attention block's forward: (a, max(a) / 127, sign bytes or None).  ``logits``: None (``e`` [E, H]
+        is read) or (el, er, s_el, s_er, src, dst): e = q(el[src]) s_el + q(er[dst]) s_er is formed inside the
+        kernel and never stored (then ``e`` is None).  ``want_sign``: also return [E, ceil(H / 8)] uint8 in
+        destination-major slot order, bit h % 8 of byte [slot, h / 8] = (e > 0)."""
+        s_a = torch.empty(1, dtype=torch.float32, device=indptr.device)
+        if logits is None:
+            _need(e, torch.float32, "e")
+            E, H = e.size(0), e.numel() // max(e.size(0), 1)
+            shape, args = e.shape, (_ptr(e), None, None, None, None, None, None)
+        else:
+            el, er, s_el, s_er, src, dst = logits
+            for t, nm in ((el, "el"), (er, "er"), (s_el, "s_el"), (s_er, "s_er")):
+                _need(t, torch.float32, nm)
+            _need(src, torch.int64, "src")
+            _need(dst, torch.int64, "dst")
+            E, H = src.numel(), el.numel() // max(el.size(0), 1)
+            if er.numel() // max(er.size(0), 1) != H or dst.numel() != E:
+                raise RuntimeError("edge_softmax: el, er must have the same heads and src, dst one entry per edge")
+            shape = (E,) + tuple(el.shape[1:])
+            args = (None, _ptr(el), _ptr(er), s_el.data_ptr(), s_er.data_ptr(), src.data_ptr(), dst.data_ptr())
+        _need(indptr, torch.int64, "indptr")
+        a = torch.empty(shape, dtype=torch.float32, device=indptr.device)
+        sign = torch.empty((E, (H + 7) // 8), dtype=torch.uint8, device=indptr.device) if want_sign else None
+        ws_bytes = _ws_bytes("tango_edge_softmax_workspace", E, H)
+        ws = _workspace(ws_bytes, indptr.device)
+        check(_L.tango_edge_softmax_fwd_ex(_ptr(a), s_a.data_ptr(), _ptr(sign), *args, indptr.data_ptr(),
+                                           _ptr(edge_ids), indptr.numel() - 1, E, H, float(slope), _ptr(ws), ws_bytes,
+                                           _stream()), "edge_softmax_ex")
+        return a, s_a, sign
+
+    @staticmethod
+    def edge_softmax_backward_ex(a, da, e, sign, indptr, edge_ids, slope=1.0):
+        """(de, max|de| / 127) of the attention block's backward; ``e`` or ``sign`` (the forward's sign bytes) gives
+        LeakyReLU's derivative (neither is needed for slope 1)."""
+        s_de = torch.empty(1, dtype=torch.float32, device=a.device)
         _need(a, torch.float32, "a")
         _need(da, torch.float32, "da")
-        _need(e, torch.float32, "e")
-        H = e.numel() // max(e.size(0), 1)
-        de = torch.empty_like(e)
-        ws_bytes = _ws_bytes("tango_edge_softmax_workspace", e.size(0), H)
-        ws = _workspace(ws_bytes, e.device)
+        if e is not None:
+            _need(e, torch.float32, "e")
+        E, H = a.size(0), a.numel() // max(a.size(0), 1)
+        de = torch.empty_like(a)
+        ws_bytes = _ws_bytes("tango_edge_softmax_workspace", E, H)
+        ws = _workspace(ws_bytes, a.device)
+        check(_L.tango_edge_softmax_bwd_ex(_ptr(de), s_de.data_ptr(), _ptr(a), _ptr(da), _ptr(e), _ptr(sign),
+                                           indptr.data_ptr(), _ptr(edge_ids), indptr.numel() - 1, E, H, float(slope),
+                                           _ptr(ws), ws_bytes, _stream()), "edge_softmax_backward_ex")
+        return de, s_de
+
+    @staticmethod
+    def edge_softmax_backward(a, da, e, indptr, edge_ids, slope=1.0):
+        """``e`` may be None for slope 1 (the plain softmax's backward does not read it)."""
+        _need(a, torch.float32, "a")
+        _need(da, torch.float32, "da")
+        if e is not None:
+            _need(e, torch.float32, "e")
+        elif float(slope) != 1.0:
+            raise RuntimeError("edge_softmax_backward: e is needed for LeakyReLU's derivative")
+        H = a.numel() // max(a.size(0), 1)
+        de = torch.empty_like(a)
+        ws_bytes = _ws_bytes("tango_edge_softmax_workspace", a.size(0), H)
+        ws = _workspace(ws_bytes, a.device)
         check(_L.tango_edge_softmax_bwd(_ptr(de), _ptr(a), _ptr(da), _ptr(e), indptr.data_ptr(),
-                                        _ptr(edge_ids), indptr.numel() - 1, e.size(0), H, float(slope), _ptr(ws),
+                                        _ptr(edge_ids), indptr.numel() - 1, a.size(0), H, float(slope), _ptr(ws),
                                         ws_bytes, _stream()),
               "edge_softmax_backward")
         return de
@@ -848,6 +910,7 @@ def multi_cusparse_SPMM(g, N, E_T, scale, reverse=False, edge_major=False, bias=
     ``edge_major``: E_T is the quantized edge tensor as it is, [nnz, H, 1]."""
     assert E_T.ndim == 3 and N.ndim == 3, "E and N must be 3D tensors"
     assert E_T.size(2 if edge_major else 1) == 1, "Cannot broadcast E"
+    assert E_T.dtype == torch.int8 or (edge_major and scale2 is not None), "fp32 E: edge-major, with its scale"
     indptr, indices, edge_ids, longest = _csr_of(g, reverse)
     if edge_ids is not None and edge_ids.numel() == 0:
         edge_ids = None

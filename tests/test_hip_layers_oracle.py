@@ -46,8 +46,10 @@ def _small_graph(n, e, seed):
     return graph_preprocess(chung_lu(n, e, 2.2, seed=seed, device="cuda"))
 
 
-def test_arxiv_gat_layer_matches_oracle_stage_by_stage(orc, recorded):
+def test_arxiv_gat_layer_matches_oracle_stage_by_stage(orc, recorded, monkeypatch):
+    import tango_amd.gat as gat_module
     from tango_amd.gat import ArxivGATConv
+    monkeypatch.setattr(gat_module, "fused_attention", False)  # the separate ops, one oracle stage each
     g = _small_graph(3000, 24000, 5)
     n, E, H, D, Fin = g.num_nodes(), g.num_edges(), 3, 16, 64
     torch.manual_seed(3)
@@ -122,9 +124,10 @@ def test_hgt_layer_matches_oracle_stage_by_stage(orc, recorded):
     # "/ sqrt(d_k)" folded into the second scale (1/4 here: a power of two, so exact either way)
     want_t, _ = orc.sddmm_dot(host(g.coo[0]), host(g.coo[1]), kq, qq, s_k, np.float32(s_q * np.float32(0.25)))
     assert np.array_equal(host(t).reshape(E, H), want_t)
-    (args, kw, a), = recorded["edge_softmax"].calls
+    (args, kw, (a, s_attn)), = recorded["edge_softmax"].calls
     ip, ix, eid = (host(x_) for x_ in g.adj_csc)
     np.testing.assert_allclose(host(a).reshape(E, H), orc.edge_softmax_fwd(want_t, ip, eid, 1.0), rtol=1e-5, atol=1e-6)
+    assert host(s_attn)[0] == orc.absmax_scale(host(a))  # found by the softmax kernel itself
     (args, agg), = recorded["spmm_u_mul_e"].calls
     sa = orc.absmax_scale(host(a))
     want_agg = orc.spmm_csr_u_mul_e_ex(ip, ix, eid, orc.quantize(v, s_v).reshape(n, H, dk),
@@ -133,6 +136,115 @@ def test_hgt_layer_matches_oracle_stage_by_stage(orc, recorded):
     Wa, ba = lin(layer.a_linear)
     want_out, *_ = orc.qgemm_fwd(want_agg.reshape(n, H * dk), Wa, bias=ba)
     assert np.array_equal(host(out), want_out)
+
+
+@pytest.mark.parametrize("H,slope,reorder", [(8, 0.2, True), (8, 0.2, False), (3, 0.2, False), (1, 0.5, True),
+                                              (12, 0.2, False), (4, 1.0, True)])
+def test_fused_attention_kernels_match_oracle(orc, H, slope, reorder):
+    """tango_edge_softmax_fwd_ex / _bwd_ex: logits formed on the fly from el, er (never stored), sign bytes for the
+    backward pass, the scales of both results from the same kernels; against the oracle's separate stages."""
+    from tango_amd.graph import Graph
+    from tango_amd.kernels import cuda_kernels as ck
+    from tango_amd.util import graph_preprocess
+    rng = np.random.default_rng(H)
+    n, E = 4000, 60000
+    w = 1.0 / np.arange(1, n + 1) ** 1.2
+    w /= w.sum()
+    src, dst = rng.choice(n, E, p=w), rng.choice(n, E, p=w)  # hubs with thousands of in-edges, rows cut by spans
+    g0 = Graph(torch.from_numpy(src).cuda(), torch.from_numpy(dst).cuda(), n)
+    g = graph_preprocess(g0.reorder_edges_by_dst() if reorder else g0)
+    src, dst = host(g.coo[0]), host(g.coo[1])
+    ip, _, eid = g.adj_csc
+    eids = None if g.csc_slots_are_edge_ids else eid
+    el = rng.standard_normal((n, H)).astype(np.float32)
+    er = rng.standard_normal((n, H)).astype(np.float32)
+    s_el, s_er = orc.absmax_scale(el), orc.absmax_scale(er)
+    dev = lambda x: torch.from_numpy(x).cuda()
+    sc = lambda v: torch.tensor([v], dtype=torch.float32, device="cuda")
+    a, s_a, sign = ck.edge_softmax_forward_ex(None, ip, eids, slope, logits=(dev(el), dev(er), sc(s_el), sc(s_er), g.coo[0], g.coo[1]),
+                                              want_sign=True)
+    want_e, _ = orc.sddmm_ewise("add", src, dst, orc.quantize(el, s_el), orc.quantize(er, s_er), s_el, s_er)
+    want_a = orc.edge_softmax_fwd(want_e, host(ip), host(eid), slope)
+    np.testing.assert_allclose(host(a), want_a, rtol=1e-5, atol=1e-6)
+    assert host(s_a)[0] == orc.absmax_scale(host(a))
+    # the same kernel reading stored logits gives the same bits
+    a2, s_a2, _ = ck.edge_softmax_forward_ex(dev(want_e), ip, eids, slope)
+    assert torch.equal(a2, a) and torch.equal(s_a2, s_a)
+    assert torch.equal(ck.edge_softmax_forward(dev(want_e), ip, eids, slope), a)
+    # sign bytes, in destination-major slot order
+    slot_edge = host(eid)
+    bits = np.unpackbits(host(sign), axis=1, bitorder="little")[:, :H].astype(bool)
+    assert np.array_equal(bits, want_e[slot_edge] > 0)
+    # backward from the sign bytes == backward from the stored logits == oracle
+    da = rng.standard_normal((E, H)).astype(np.float32)
+    de, s_de = ck.edge_softmax_backward_ex(a, dev(da), None, sign, ip, eids, slope)
+    de2 = ck.edge_softmax_backward(a, dev(da), dev(want_e), ip, eids, slope)
+    assert torch.equal(de, de2)
+    np.testing.assert_allclose(host(de), orc.edge_softmax_bwd(host(a), da, want_e, host(ip), host(eid), slope),
+                               rtol=1e-4, atol=1e-6)
+    assert host(s_de)[0] == orc.absmax_scale(host(de))
+
+
+@pytest.mark.parametrize("H,F", [(8, 16), (3, 5), (4, 64)])
+def test_aggregation_quantizes_fp32_edge_values_on_load(orc, H, F):
+    """tango_spmm_csr_u_mul_e_f32e == quantize the edge values first, then tango_spmm_csr_u_mul_e_ex: on a sparse
+    graph (slot-span kernels), a dense one (row kernels) and both orientations."""
+    from tango_amd import kernels as K
+    rng = np.random.default_rng(F)
+    for n, E in ((3000, 20000), (300, 60000)):
+        g = _small_graph(n, E, 11) if n == 3000 else None
+        if g is None:
+            from tango_amd.graph import Graph
+            from tango_amd.util import graph_preprocess
+            g = graph_preprocess(Graph(torch.from_numpy(rng.integers(0, n, E)).cuda(), torch.from_numpy(rng.integers(0, n, E)).cuda(), n))
+        nn, ne = g.num_nodes(), g.num_edges()
+        feat = torch.from_numpy(rng.integers(-127, 128, (nn, H, F)).astype(np.int8)).cuda()
+        a = torch.rand(ne, H, 1, device="cuda")
+        s_a = K.cuda_kernels.get_scale(a)
+        aq, _ = K.quantize(a, s_a)
+        one = torch.tensor([0.013], device="cuda")
+        bias = torch.randn(H * F, device="cuda")
+        for rev in (False, True):
+            want = K.multi_cusparse_SPMM(g, feat, aq, one, rev, edge_major=True, scale2=s_a, bias=bias, act="relu")
+            got = K.multi_cusparse_SPMM(g, feat, a, one, rev, edge_major=True, scale2=s_a, bias=bias, act="relu")
+            assert torch.equal(got, want)
+        ip, ix, eid = (host(t) for t in g.adj_csc)
+        ref = orc.spmm_csr_u_mul_e_ex(ip, ix, eid, host(feat), host(aq), 0.013, scale2=host(s_a)[0], edge_major=True)
+        assert np.array_equal(host(K.multi_cusparse_SPMM(g, feat, a, one, edge_major=True, scale2=s_a)), ref)
+
+
+@pytest.mark.parametrize("on_the_fly,on_load", [(False, False), (True, True)])
+@pytest.mark.parametrize("layer_kind", ["gat", "arxiv"])
+def test_fused_attention_layer_equals_separate_ops(monkeypatch, layer_kind, on_the_fly, on_load):
+    """A GAT layer with u_add_v + LeakyReLU + softmax as one op, the scale of the attention handed on and the
+    aggregation rounding fp32 attention as it loads: the same output and the same gradients, bit for bit, as the
+    layer built from the separate ops (which the stage-by-stage test above ties to the oracle)."""
+    import torch.nn.functional as F
+    import tango_amd.gat as gat_module
+    from tango_amd import config
+    monkeypatch.setattr(config, "attention_logits_on_the_fly", on_the_fly)
+    monkeypatch.setattr(config, "edge_values_on_load", on_load)
+    g = _small_graph(3000, 24000, 5)
+    n = g.num_nodes()
+    torch.manual_seed(3)
+    if layer_kind == "gat":
+        layer = gat_module.QGATConv(64, 16, 4, activation=F.elu).cuda()
+    else:
+        layer = gat_module.ArxivGATConv(64, 16, num_heads=3, residual=True).cuda()
+    x = torch.randn(n, 64, device="cuda")
+    w = torch.randn(n, layer._num_heads, 16, device="cuda")
+    results = []
+    for fused in (True, False):
+        monkeypatch.setattr(gat_module, "fused_attention", fused)
+        xi = x.clone().requires_grad_(True)
+        layer.zero_grad()
+        out = layer(g, xi)
+        out.backward(w)
+        results.append((out.detach().clone(), xi.grad.clone(), [p.grad.clone() for p in layer.parameters()]))
+    (o1, gx1, gp1), (o2, gx2, gp2) = results
+    assert torch.equal(o1, o2) and torch.equal(gx1, gx2)
+    for (name, _), a_, b_ in zip(layer.named_parameters(), gp1, gp2):
+        assert torch.equal(a_, b_), name
 
 
 def _fp32_hetero_hgt(layer, g, h):
