@@ -310,10 +310,11 @@ def _hgt_step(K, torch, iters, warm):
     out = {"hgt2_step_170000n_8.17Me_ms": round(time_op(hgt_step, iters=iters, warm=warm), 3)}
     # the same graph as a heterogeneous one: weights per node type and per relation, one SDDMM and one aggregation
     # per relation, one softmax over all in-edges
-    from tango_amd.gat import HeteroHGTLayer, relation_graphs
+    from tango_amd.gat import HeteroHGTLayer, relation_graphs, relation_major
     del hgt, opth
     sizes, rels = (100_000, 50_000, 20_000), ((0, 1), (1, 0), (1, 2), (2, 0))
     g2, _, etype = hetero_power_law(type_sizes=sizes, relations=rels, device="cuda")
+    g2, etype = relation_major(g2, etype)
     g2 = graph_preprocess(g2)
     rg = relation_graphs(g2, etype, rels, sizes)
     layers = torch.nn.ModuleList([HeteroHGTLayer(256, 256, 4, sizes, rg) for _ in range(2)]).cuda()

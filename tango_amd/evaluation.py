@@ -20,7 +20,7 @@ import torch
 import torch.nn as nn
 import torch.nn.functional as F
 
-from .gat import GAT, HGT, ArxivGAT, HeteroHGTLayer, QGATConv, relation_graphs
+from .gat import GAT, HGT, ArxivGAT, HeteroHGTLayer, QGATConv, relation_graphs, relation_major
 from .gcn import GCN, ArxivGCN
 from .graph import Graph, add_self_loop, chung_lu, hetero_power_law, remove_self_loop
 from .SDDMM import sddmm_u_dot_v
@@ -116,6 +116,7 @@ def train_hetero_hgt(epochs=10, hidden=256, heads=4, n_classes=16, lr=1e-3, quie
     type_sizes = graph_kw.pop("type_sizes", (100_000, 50_000, 20_000))
     relations = graph_kw.pop("relations", ((0, 1), (1, 0), (1, 2), (2, 0)))
     g, _, edge_type = hetero_power_law(type_sizes=type_sizes, relations=relations, device="cuda", **graph_kw)
+    g, edge_type = relation_major(g, edge_type)
     g = graph_preprocess(g)
     rels = relation_graphs(g, edge_type, relations, type_sizes)
     n = g.num_nodes()

@@ -326,8 +326,9 @@ class HeteroHGTLayer(nn.Module):
         n, H, dk = h.size(0), self.n_heads, self.d_k
         k, q, v = self._typed(self.k_linear, h), self._typed(self.q_linear, h), self._typed(self.v_linear, h)
         q = q.view(n, H, dk)
-        t = h.new_zeros((g.num_edges(), H, 1))
-        vr = []
+        contiguous = all(getattr(gr, "edge_range", None) is not None for gr in self.rels)
+        t = None if contiguous else h.new_zeros((g.num_edges(), H, 1))
+        vr, parts = [], []
         for r, gr in enumerate(self.rels):
             lo, hi = (0, n) if gr.src_type is None else (self.bounds[gr.src_type], self.bounds[gr.src_type + 1])
             # relation-specific key and message of the relation's source type; other rows stay zero (no edge of
@@ -338,30 +339,57 @@ class HeteroHGTLayer(nn.Module):
             vv[lo:hi] = self.msg_linear[r](v[lo:hi])
             vr.append(vv.view(n, H, dk))
             tr = sddmm_u_dot_v.apply(gr, kr.view(n, H, dk), q, None, None, 1.0 / self.sqrt_dk)
-            t = t.index_copy(0, gr.eids, tr)
+            if contiguous:
+                parts.append(tr)
+            else:
+                t = t.index_copy(0, gr.eids, tr)
+        if contiguous:  # relations own consecutive edge-id ranges, in order: the scores are their concatenation
+            t = torch.cat(parts)
         attn = edge_softmax(g, t)  # over every in-edge of a destination, all relations together
         out = None
         for r, gr in enumerate(self.rels):
-            o = spmm_u_mul_e.apply(gr, vr[r], attn[gr.eids])
+            ar = attn[gr.edge_range[0]:gr.edge_range[1]] if contiguous else attn[gr.eids]
+            o = spmm_u_mul_e.apply(gr, vr[r], ar)
             out = o if out is None else out + o
         return self._typed(self.a_linear, out.reshape(n, self.out_dim))
 
 
+def relation_major(g, edge_type):
+    """(graph, edge types) with the edges renumbered relation by relation and, inside a relation, by destination:
+    every relation then owns a consecutive range of edge ids (per-relation edge tensors are slices of the full
+    one, no gather or scatter), and its own graph walks its edges front to back."""
+    from .graph import Graph
+    src, dst = g.edges()
+    order = torch.sort(edge_type * g.num_nodes() + dst, stable=True).indices
+    g2 = Graph(src[order], dst[order], g.num_nodes())
+    g2.edge_order = order
+    return g2, edge_type[order]
+
+
 def relation_graphs(g, edge_type, relations, type_sizes):
     """Per relation id in ``edge_type`` ([E], ids 0 .. len(relations) where the last id marks self loops) a
-    preprocessed Graph over all nodes of ``g`` with that relation's edges, ``eids`` and ``src_type`` attached."""
+    preprocessed Graph over all nodes of ``g`` with that relation's edges, ``eids`` (their ids in ``g``),
+    ``edge_range`` ((first, last + 1) when those ids are consecutive and the relations come in order, as after
+    ``relation_major``; else None) and ``src_type`` attached."""
     from .graph import Graph
     from .util import graph_preprocess
     src, dst = g.edges()
-    out = []
+    out, nxt, in_order = [], 0, True
     for r in range(len(relations) + 1):
         eids = torch.nonzero(edge_type == r).flatten()
         if eids.numel() == 0:
             continue
         gr = graph_preprocess(Graph(src[eids], dst[eids], g.num_nodes()))
         gr.eids = eids
+        lo, hi = int(eids[0]), int(eids[-1]) + 1
+        in_order = in_order and lo == nxt and hi - lo == eids.numel()
+        gr.edge_range = (lo, hi)
+        nxt = hi
         gr.src_type = relations[r][0] if r < len(relations) else None  # self loops start at every type
         out.append(gr)
+    if not in_order or nxt != g.num_edges():
+        for gr in out:
+            gr.edge_range = None
     return out
 
 

@@ -274,18 +274,33 @@ def test_hetero_hgt_layer_tracks_fp32_and_trains():
     """Weights per node type and per relation: the quantized layer stays within int8 noise of the same math in
     fp32, every typed and relation-specific parameter receives a gradient, and a relation's weights do not
     influence destinations that relation does not reach."""
-    from tango_amd.gat import HeteroHGTLayer, relation_graphs
+    from tango_amd.gat import HeteroHGTLayer, relation_graphs, relation_major
     from tango_amd.graph import hetero_power_law
     from tango_amd.util import graph_preprocess
     sizes, rels = (3000, 1500, 600), ((0, 1), (1, 0), (1, 2), (2, 0))
-    g, node_type, edge_type = hetero_power_law(type_sizes=sizes, relations=rels, edges_per_relation=30000, device="cuda")
+    g0, node_type, edge_type0 = hetero_power_law(type_sizes=sizes, relations=rels, edges_per_relation=30000, device="cuda")
+    # any edge numbering works (per-relation tensors are gathered and scattered) ...
+    perm = torch.randperm(g0.num_edges(), device="cuda", generator=torch.Generator("cuda").manual_seed(3))
+    from tango_amd.graph import Graph
+    g_any = graph_preprocess(Graph(g0.edges()[0][perm], g0.edges()[1][perm], g0.num_nodes()))
+    rg_any = relation_graphs(g_any, edge_type0[perm], rels, sizes)
+    assert all(r.edge_range is None for r in rg_any)
+    # ... and the relation-major one turns them into slices
+    g, edge_type = relation_major(g0, edge_type0)
     g = graph_preprocess(g)
     rg = relation_graphs(g, edge_type, rels, sizes)
     assert len(rg) == 5 and sum(r.num_edges() for r in rg) == g.num_edges()
+    assert all(r.edge_range is not None and r.csc_slots_are_edge_ids for r in rg)
     torch.manual_seed(9)
     layer = HeteroHGTLayer(64, 64, 4, sizes, rg).cuda()
     h = torch.randn(g.num_nodes(), 64, device="cuda", requires_grad=True)
     out = layer(g, h)
+    layer_any = HeteroHGTLayer(64, 64, 4, sizes, rg_any).cuda()
+    layer_any.load_state_dict(layer.state_dict())
+    # node outputs do not depend on the edge numbering (up to the softmax's fp32 summation order, which can move
+    # an int8 attention value by one step here and there)
+    out_any = layer_any(g_any, h)
+    assert ((out_any - out).norm() / out.norm()).item() < 2e-3
     with torch.no_grad():
         ref = _fp32_hetero_hgt(layer, g, h)
     assert ((out - ref).norm() / ref.norm()).item() < 0.1
