@@ -77,6 +77,9 @@ __device__ __forceinline__ void block_absmax_to_global(float v, float* out) {
 __device__ __forceinline__ float rscale_of(float s) { return s > 0.0f ? 1.0f / s : 0.0f; }
 
 // fp32 -> int8 rounding shared by the quantize kernels and the GEMM's fused quantize.
+// The rounded value goes through v_cvt_i32_f32 (toward zero, saturating, NaN -> 0: what the float-domain clamp and
+// the NaN test before a C cast spelled out in four more instructions) and is clamped as an integer: three VALU
+// instructions per element for truncation, four for half-to-even.
 template <int MODE>
 __device__ __forceinline__ int quant_one(float x, float r, float u) {
     const float p = x * r;
@@ -84,17 +87,19 @@ __device__ __forceinline__ int quant_one(float x, float r, float u) {
     if (MODE == TANGO_ROUND_RNE)
         v = rintf(p);
     else if (MODE == TANGO_ROUND_TRUNC)
-        v = truncf(p);
+        v = p;  // the conversion below truncates
     else
         v = floorf(p + u);
-    // fmaxf/fminf drop a NaN operand, so a NaN input lands on a bound; map it to 0
-    v = (v == v) ? fminf(fmaxf(v, -127.0f), 127.0f) : 0.0f;
-    return static_cast<int>(v);
+    int q;
+    asm("v_cvt_i32_f32 %0, %1" : "=v"(q) : "v"(v));
+    return q < -127 ? -127 : (q > 127 ? 127 : q);
 }
 
+// bytes (a, b, c, d) of four ints in [-128, 127] as one dword, three v_perm_b32
 __device__ __forceinline__ uint32_t pack4(int a, int b, int c, int d) {
-    return (static_cast<uint32_t>(a) & 0xffu) | ((static_cast<uint32_t>(b) & 0xffu) << 8) |
-           ((static_cast<uint32_t>(c) & 0xffu) << 16) | (static_cast<uint32_t>(d) << 24);
+    const uint32_t lo = __builtin_amdgcn_perm(static_cast<uint32_t>(b), static_cast<uint32_t>(a), 0x0c0c0400u);
+    const uint32_t hi = __builtin_amdgcn_perm(static_cast<uint32_t>(d), static_cast<uint32_t>(c), 0x0c0c0400u);
+    return __builtin_amdgcn_perm(hi, lo, 0x05040100u);
 }
 
 // 4x4 byte transpose with v_perm_b32: rows r0..r3 (one dword each) -> c[j] = bytes (r0[j], r1[j], r2[j], r3[j]).
