@@ -52,7 +52,11 @@ def parse():
     ap.add_argument("--feat", type=int, default=256, help="feature width of --profile-mode spmm")
     ap.add_argument("--permute-ids", action="store_true",
                     help="--profile-mode spmm on the benchmark graph with its node ids randomly permuted")
-    ap.add_argument("--profile-mode", choices=["spmm", "copy", "qlinear", "gradx", "sddmm", "quantize", "gat", "hgt"], default=None,
+    ap.add_argument("--gemm-shape", default="256,41", metavar="K,N",
+                    help="layer shape of --profile-mode gradx / gradw (dY [nodes, N] int8, X [nodes, K])")
+    ap.add_argument("--profile-mode", default=None,
+                    choices=["spmm", "copy", "qlinear", "gradx", "gradw", "sddmm", "quantize", "softmax",
+                             "gat", "arxiv", "hgt", "hetero"],
                     help="run only the dominant kernel (spmm: copy_u F=256 on the benchmark graph) or a "
                          "1 GiB device copy (counter calibration), for rocprofv3 --pmc passes")
     return ap.parse_args()
@@ -241,30 +245,33 @@ def sddmm_primitives(K, torch):
     return out
 
 
-def model_steps(K, torch, which=("gat", "hgt"), iters=10, warm=3):
+def model_steps(K, torch, which=("gat", "arxiv", "hgt", "hetero"), iters=10, warm=3):
     """The other model configurations, one training step each (forward + loss + backward + Adam):
     the 3-layer GAT (hidden 16 x 8 heads, evaluation/test_gat.py:170-214) on the 169,343-node graph
     and two HGT layers (256-d, 4 heads) on the homogenised 3-type / 4-relation graph."""
     out = {}
     torch.manual_seed(4)
-    if "gat" in which:
-        out.update(_gat_step(K, torch, iters, warm))
-    if "hgt" in which:
-        out.update(_hgt_step(K, torch, iters, warm))
+    for name, fn in (("gat", _gat_step), ("arxiv", _arxiv_step), ("hgt", _hgt_step), ("hetero", _hetero_step)):
+        if name in which:
+            out.update(fn(K, torch, iters, warm))
     return out
 
 
-def _gat_step(K, torch, iters, warm):
-    from tango_amd.gat import GAT
+def _gat_graph(torch):
     from tango_amd.graph import chung_lu
-    from tango_amd.loss import cross_entropy
     from tango_amd.util import graph_preprocess
     # edges numbered in destination-major order: the [E, H] tensors of the attention layers are then
     # walked front to back (node outputs do not depend on the numbering)
     g = graph_preprocess(chung_lu(169343, 1166243, 2.2, seed=4, device="cuda").reorder_edges_by_dst())
+    return g, torch.randn(g.num_nodes(), 128, device="cuda")
+
+
+def _gat_step(K, torch, iters, warm):
+    from tango_amd.gat import GAT
+    from tango_amd.loss import cross_entropy
+    g, x = _gat_graph(torch)
     n = g.num_nodes()
     model = GAT(g, 3, 128, 16, 40, [8, 8, 1], torch.nn.functional.elu).cuda()
-    x = torch.randn(n, 128, device="cuda")
     labels = torch.randint(0, 16, (n,), device="cuda")
     opt = torch.optim.Adam(model.parameters(), lr=1e-3, fused=True)
 
@@ -272,12 +279,16 @@ def _gat_step(K, torch, iters, warm):
         opt.zero_grad(set_to_none=True)
         cross_entropy(model(x), labels).backward()
         opt.step()
-    out = {"gat3_step_169343n_1.34Me_ms": round(time_op(gat_step, iters=iters, warm=warm), 3)}
+    return {"gat3_step_169343n_1.34Me_ms": round(time_op(gat_step, iters=iters, warm=warm), 3)}
+
+
+def _arxiv_step(K, torch, iters, warm):
     # the stack the reference trains on this graph (evaluation/arxiv_gat.py:376-448): a residual projection in
     # every layer, batch norm between layers, a one-head output layer, the smoothed loss; dropout off
     from tango_amd.evaluation import arxiv_loss
     from tango_amd.gat import ArxivGAT
-    del model, opt
+    g, x = _gat_graph(torch)
+    n = g.num_nodes()
     am = ArxivGAT(128, 40, 16, 3, 8, torch.nn.functional.relu).cuda()
     al = torch.randint(0, 40, (n,), device="cuda")
     aopt = torch.optim.RMSprop(am.parameters(), lr=2e-3)
@@ -286,8 +297,7 @@ def _gat_step(K, torch, iters, warm):
         aopt.zero_grad(set_to_none=True)
         arxiv_loss(am(g, x), al).backward()
         aopt.step()
-    out["arxiv_gat3_step_169343n_1.34Me_ms"] = round(time_op(arxiv_step, iters=iters, warm=warm), 3)
-    return out
+    return {"arxiv_gat3_step_169343n_1.34Me_ms": round(time_op(arxiv_step, iters=iters, warm=warm), 3)}
 
 
 def _hgt_step(K, torch, iters, warm):
@@ -307,16 +317,24 @@ def _hgt_step(K, torch, iters, warm):
         opth.zero_grad(set_to_none=True)
         cross_entropy(hgt(g, xh), lh).backward()
         opth.step()
-    out = {"hgt2_step_170000n_8.17Me_ms": round(time_op(hgt_step, iters=iters, warm=warm), 3)}
+    return {"hgt2_step_170000n_8.17Me_ms": round(time_op(hgt_step, iters=iters, warm=warm), 3)}
+
+
+def _hetero_step(K, torch, iters, warm):
     # the same graph as a heterogeneous one: weights per node type and per relation, one SDDMM and one aggregation
     # per relation, one softmax over all in-edges
     from tango_amd.gat import HeteroHGTLayer, relation_graphs, relation_major
-    del hgt, opth
+    from tango_amd.graph import hetero_power_law
+    from tango_amd.loss import cross_entropy
+    from tango_amd.util import graph_preprocess
     sizes, rels = (100_000, 50_000, 20_000), ((0, 1), (1, 0), (1, 2), (2, 0))
     g2, _, etype = hetero_power_law(type_sizes=sizes, relations=rels, device="cuda")
     g2, etype = relation_major(g2, etype)
     g2 = graph_preprocess(g2)
     rg = relation_graphs(g2, etype, rels, sizes)
+    n = g2.num_nodes()
+    xh = torch.randn(n, 256, device="cuda")
+    lh = torch.randint(0, 16, (n,), device="cuda")
     layers = torch.nn.ModuleList([HeteroHGTLayer(256, 256, 4, sizes, rg) for _ in range(2)]).cuda()
     proj = torch.nn.Linear(256, 16).cuda()
     opt2 = torch.optim.Adam(list(layers.parameters()) + list(proj.parameters()), lr=1e-3, fused=True)
@@ -328,8 +346,7 @@ def _hgt_step(K, torch, iters, warm):
             h = layer(g2, h)
         cross_entropy(proj(h), lh).backward()
         opt2.step()
-    out["hetero_hgt2_step_170000n_8.17Me_ms"] = round(time_op(hetero_step, iters=iters, warm=warm), 3)
-    return out
+    return {"hetero_hgt2_step_170000n_8.17Me_ms": round(time_op(hetero_step, iters=iters, warm=warm), 3)}
 
 
 def cpu_baseline(g, X, W1, W2, frac, reps=3):
@@ -444,7 +461,7 @@ def main():
         torch.cuda.synchronize()
         print(json.dumps({"profile_mode": "copy", "bytes_read": src.numel() * 4, "bytes_written": src.numel() * 4}))
         return
-    if args.profile_mode in ("gat", "hgt"):  # one training step of the attention models, for kernel traces
+    if args.profile_mode in ("gat", "arxiv", "hgt", "hetero"):  # one training step of the attention models, for kernel traces
         out = model_steps(K, torch, which=(args.profile_mode,), iters=args.steps, warm=args.warmup)
         print(json.dumps(dict(out, profile_mode=args.profile_mode)))
         return
@@ -459,15 +476,33 @@ def main():
         print(json.dumps({"profile_mode": "qlinear", "M": M, "K": Kd, "N": N, "avg_ms": round(ms, 4),
                           "ops": 2 * M * N * Kd, "algorithmic_bytes": 5 * (M * Kd + N * Kd) + 4 * M * N + 4 * N}))
         return
-    if args.profile_mode == "gradx":  # gradX of the epoch's second layer: int8 dY [M, 41] -> fp32 dX [M, 256]
-        M, Kd, N = args.nodes, 256, 41
+    if args.profile_mode in ("gradx", "gradw"):
+        # gradX: int8 dY [M, N] -> fp32 dX [M, K] (default shape: the epoch's second layer);
+        # gradW: int8 dY [M, N] and int8 X [M, K] -> fp32 dW [N, K]
+        Kd, N = (int(v) for v in args.gemm_shape.split(","))
+        M = args.nodes
         dY, s_dY = K.quantize_padded(torch.randn(M, N, device="cuda"))
         Wq, sW = K.quantize(torch.randn(N, Kd, device="cuda") * 0.05)
-        Xq = torch.empty((M, Kd), dtype=torch.int8, device="cuda")
+        ld = (Kd + 15) // 16 * 16
+        Xq = torch.randint(-127, 128, (M, ld), dtype=torch.int8, device="cuda")[:, :Kd]
         sX = torch.ones(1, device="cuda")
-        ms = time_op(lambda: K.QGEMM_backward(dY, Xq, Wq, s_dY, sX, sW, True, False), iters=args.steps, warm=args.warmup)
-        print(json.dumps({"profile_mode": "gradx", "M": M, "K": Kd, "N": N, "avg_ms": round(ms, 4),
-                          "ops": 2 * M * N * Kd, "algorithmic_bytes": M * N + N * Kd + 4 * M * Kd}))
+        dx = args.profile_mode == "gradx"
+        ms = time_op(lambda: K.QGEMM_backward(dY, Xq, Wq, s_dY, sX, sW, dx, not dx), iters=args.steps, warm=args.warmup)
+        byt = M * N + N * Kd + 4 * M * Kd if dx else M * (N + Kd) + 4 * N * Kd
+        print(json.dumps({"profile_mode": args.profile_mode, "M": M, "K": Kd, "N": N, "avg_ms": round(ms, 4),
+                          "ops": 2 * M * N * Kd, "algorithmic_bytes": byt}))
+        return
+    if args.profile_mode == "softmax":  # edge softmax forward / backward, 8 heads, on the 169,343-node graph
+        g4 = graph_preprocess(chung_lu(169343, 1166243, 2.2, seed=4, device="cuda").reorder_edges_by_dst())
+        E, H = g4.num_edges(), 8
+        e = torch.randn(E, H, 1, device="cuda")
+        ip, _, eid = g4.adj_csc
+        ms_f = time_op(lambda: K.cuda_kernels.edge_softmax_forward(e, ip, eid, 0.2), iters=args.steps, warm=args.warmup)
+        a = K.cuda_kernels.edge_softmax_forward(e, ip, eid, 0.2)
+        da = torch.randn_like(a)
+        ms_b = time_op(lambda: K.cuda_kernels.edge_softmax_backward(a, da, e, ip, eid, 0.2), iters=args.steps, warm=args.warmup)
+        print(json.dumps({"profile_mode": "softmax", "edges": E, "H": H, "fwd_ms": round(ms_f, 4), "bwd_ms": round(ms_b, 4),
+                          "fwd_bytes": E * (8 * H + 8), "bwd_bytes": E * (16 * H + 8)}))
         return
     if args.profile_mode == "quantize":
         X = torch.randn(args.nodes, 602, device="cuda")

@@ -126,7 +126,10 @@ int tango_transpose_quant_f32_i8(const float* x, int64_t nrow, int64_t ncol, con
 
 /* All GEMM entry points take a caller-provided workspace (device memory,
    16-byte aligned) whose size the matching *_workspace() query returns; the
-   library uses it to re-pack the small operand into aligned, zero-padded rows. */
+   library uses it to re-pack the small operand into aligned, zero-padded rows.
+   A row stride of an fp32 output that exceeds its column count is padding, not a
+   view into a wider matrix: the kernels may store zeros into the columns between
+   the last one and the next multiple of 16 (never at or past the stride). */
 
 /* QGEMM_forward (cuda/src/cuda.cpp:11-17 -> QGEMM_forward_impl,
    QGEMM_forward.cu:125-157): quantizes X[M,K] and W[N,K] with scaleX / scaleW

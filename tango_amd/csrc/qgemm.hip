@@ -422,6 +422,152 @@ __global__ __launch_bounds__(64 * WAVES) void gemm_nts_kernel(const NtParams p, 
     if (p.absmax_out) block_absmax_to_global(m / 127.0f, p.absmax_out);
 }
 
+// NT kernel with the small operand stationary in registers, for wide fp32 outputs (257 to 960 columns) and
+// reductions of at most 64 KS.  The workgroup's waves share one 16-row tile of A at a time and split its output
+// row into pieces of 64 columns: wave w holds the B fragments of column tiles 4 w .. 4 w + 3 for the whole launch
+// (16 KS registers), reads the A tile from LDS, runs its 4 KS MFMAs and stores a 16 x 64 piece.  A tile's rows
+// leave the compute unit together, so the launch writes one compact window that moves through C front to back;
+// with a wave per tile (gemm_nts_kernel) some three thousand separate rows of C are open at once, and a
+// store-only kernel of that shape sustains 5.0 TB/s on outputs beyond the Infinity Cache against 6.0 TB/s for
+// this one.
+// The last wave of the workgroup only fetches: it reads the next tiles of A in whole rows (a quarter-wave per
+// 256-byte row; loading fragments directly costs a cache line look-up per lane, which a dozen waves asking for
+// the same tile cannot afford) and writes them to a two-slot LDS ring, rotated per row so that the fragment
+// reads of a quarter-wave (one 16-byte chunk of sixteen rows) fall on sixteen different bank groups.  Memory
+// operations of a wave complete in order; because the fetching wave stores nothing and the storing waves load
+// nothing, no wave ever waits for a store.  One barrier per tile hands a slot over.
+// Epilogue: dequantization, the optional row scale and absmax only; C must be 16-byte aligned with a pitch that
+// is a multiple of 4 floats; rows of A must be readable in aligned 16-byte pieces.
+template <int KS>
+__global__ __launch_bounds__(1024) void gemm_ntr_kernel(const NtParams p, int ntiles) {
+    constexpr int CT = 4;
+    constexpr int CH = 4 * KS;            // 16-byte chunks of a tile row
+    constexpr int SLOT = 16 * CH * 16 + 64;  // bytes of a ring slot: the tile, then sixteen row scales
+    __shared__ __attribute__((aligned(16))) int8_t ring[2 * SLOT];
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(static_cast<int>(threadIdx.x >> 6));
+    const int consumers = static_cast<int>(blockDim.x >> 6) - 1;
+    const int g = lane >> 4, r16 = lane & 15;
+    const int stride = static_cast<int>(gridDim.x);
+    const int t0 = static_cast<int>(blockIdx.x);
+    const int rounds = t0 < ntiles ? (ntiles - t0 + stride - 1) / stride : 0;  // the same for every wave
+    // chunk c of row r lives at 16-byte position CH r + (c + r / (16 / CH)) mod CH of its slot
+    auto position = [](int r, int c) { return CH * r + ((c + r / (16 / CH)) & (CH - 1)); };
+    auto hand_over = [] { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); };
+
+    if (wave == consumers) {  // the fetching wave
+        constexpr int NI = CH / 4;  // 16-byte loads per lane and tile: 64 lanes x NI chunks = 16 rows x CH chunks
+        int8_t* dst[NI];
+        int64_t off[NI];  // byte offset of the lane's chunk inside a row of A; negative: not readable
+        int rr[NI];
+#pragma unroll
+        for (int i = 0; i < NI; ++i) {
+            const int pos = 64 * i + lane;  // lanes cover positions in order: a run of CH lanes is one whole row
+            const int r = pos / CH;
+            const int c = ((pos & (CH - 1)) - r / (16 / CH)) & (CH - 1);
+            rr[i] = r;
+            off[i] = 16 * c < p.a_row_bytes ? 16 * c : -1;
+            dst[i] = ring + pos * 16;
+        }
+        auto fetch = [&](i32x4* v, float& rs, int t) {
+#pragma unroll
+            for (int i = 0; i < NI; ++i) {
+                int64_t row = static_cast<int64_t>(t) * 16 + rr[i];
+                if (row >= p.M) row = p.M - 1;  // rows past the end (last tile) are computed and not stored
+                v[i] = i32x4{0, 0, 0, 0};
+                if (off[i] >= 0) v[i] = *reinterpret_cast<const i32x4*>(p.A + row * p.lda + off[i]);
+            }
+            int64_t row = static_cast<int64_t>(t) * 16 + r16;
+            if (row >= p.M) row = p.M - 1;
+            rs = p.row_scale ? p.row_scale[row] : 1.0f;
+        };
+        auto put = [&](const i32x4* v, float rs, int slot) {
+#pragma unroll
+            for (int i = 0; i < NI; ++i) *reinterpret_cast<i32x4*>(dst[i] + slot * SLOT) = v[i];
+            if (lane < 16) *reinterpret_cast<float*>(ring + slot * SLOT + 16 * CH * 16 + 4 * lane) = rs;
+        };
+        // tiles are requested four rounds ahead (one round lasts less than a trip to memory); the four register
+        // sets take turns by unrolling, so that no set is copied while its load is in flight
+        i32x4 v[4][NI];
+        float rs[4] = {1.0f, 1.0f, 1.0f, 1.0f};
+#pragma unroll
+        for (int u = 0; u < 4; ++u)
+            if (u < rounds) fetch(v[u], rs[u], t0 + u * stride);
+        if (rounds > 0) put(v[0], rs[0], 0);
+        if (4 < rounds) fetch(v[0], rs[0], t0 + 4 * stride);
+        hand_over();  // slot 0 holds round 0
+        // round k: the tile of round k + 1 goes to slot (k + 1) % 2 while the other waves read slot k % 2
+        for (int kb = 0; kb < rounds; kb += 4) {
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                const int k = kb + u;
+                if (k >= rounds) break;
+                const int set = (u + 1) & 3;
+                if (k + 1 < rounds) put(v[set], rs[set], (k + 1) & 1);
+                if (k + 5 < rounds) fetch(v[set], rs[set], t0 + (k + 5) * stride);
+                hand_over();
+            }
+        }
+        if (p.absmax_out) block_absmax_to_global(0.0f, p.absmax_out);
+        return;
+    }
+
+    i32x4 b[CT][KS];
+#pragma unroll
+    for (int j = 0; j < CT; ++j) {
+        const int64_t n = 16 * static_cast<int64_t>(CT * wave + j) + r16;
+#pragma unroll
+        for (int st = 0; st < KS; ++st) {
+            // zero rows past the last column, zero fill of the packed rows past the reduction length: whatever
+            // the ring holds at those places does not count
+            b[j][st] = i32x4{0, 0, 0, 0};
+            if (n < p.N && st * 64 < p.Kr) b[j][st] = *reinterpret_cast<const i32x4*>(p.B + n * p.ldb + st * 64 + g * 16);
+        }
+    }
+    const float s = p.sA[0] * p.sB[0];
+    const bool want_max = p.absmax_out != nullptr;
+    const int col0 = 64 * wave + 4 * g;  // first of the lane's four columns in tile j = 0
+    // columns that may be written: a row's padding, up to the next multiple of 16 columns, takes the zeros of the
+    // zero-filled rows of B
+    const int n16c = static_cast<int>((p.N + 15) >> 4) * 16;
+    const int wcols = p.ldc < n16c ? static_cast<int>(p.ldc) : n16c;
+    int frag[KS];  // byte offset of the lane's fragment of k-step st inside a slot
+#pragma unroll
+    for (int st = 0; st < KS; ++st) frag[st] = position(r16, 4 * st + g) * 16;
+    float m = 0.0f;
+    hand_over();
+    for (int k = 0; k < rounds; ++k) {
+        const int8_t* slot = ring + (k & 1) * SLOT;
+        i32x4 a[KS];
+#pragma unroll
+        for (int st = 0; st < KS; ++st) a[st] = *reinterpret_cast<const i32x4*>(slot + frag[st]);
+        const float rsc = *reinterpret_cast<const float*>(slot + 16 * CH * 16 + 4 * r16);
+        i32x4 acc[CT];
+#pragma unroll
+        for (int j = 0; j < CT; ++j) acc[j] = i32x4{0, 0, 0, 0};
+#pragma unroll
+        for (int st = 0; st < KS; ++st)
+#pragma unroll
+            for (int j = 0; j < CT; ++j)
+                acc[j] = mfma_16x16x64(b[j][st], a[st], acc[j]);  // operands swapped, see gemm_nt_kernel
+        const int64_t row = static_cast<int64_t>(t0 + k * stride) * 16 + r16;
+        if (row < p.M) {
+            float* crow = p.C + row * p.ldc + col0;
+#pragma unroll
+            for (int j = 0; j < CT; ++j) {
+                if (col0 + 16 * j + 4 <= wcols) {
+                    const f32x4 y{(s * static_cast<float>(acc[j][0])) * rsc, (s * static_cast<float>(acc[j][1])) * rsc,
+                                  (s * static_cast<float>(acc[j][2])) * rsc, (s * static_cast<float>(acc[j][3])) * rsc};
+                    if (want_max) m = fmaxf(fmaxf(m, fmaxf(fabsf(y[0]), fabsf(y[1]))), fmaxf(fabsf(y[2]), fabsf(y[3])));
+                    *reinterpret_cast<f32x4*>(crow + 16 * j) = y;
+                }
+            }
+        }
+        hand_over();  // the slot just read may be refilled, the other one is complete
+    }
+    if (p.absmax_out) block_absmax_to_global(m / 127.0f, p.absmax_out);
+}
+
 // ------------------------------------ forward GEMM with the quantize fused in
 // Workgroup = 4 waves = 64 rows of X.  Phase A: the waves stream their rows of the
 // fp32 X from HBM (each lane 4 consecutive floats per step, a wavefront 1 KiB of one
@@ -1118,10 +1264,33 @@ static bool launch_nts(const NtParams& p, hipStream_t s) {
 #undef TANGO_NTS
 }
 
+// The register-stationary form: fp32 output of 257 .. 960 columns (at most fifteen computing waves and the
+// fetching one) with the plain epilogue, reduction <= 256, and
+// enough row tiles to keep every compute unit busy for many rounds.
+static bool launch_ntr(const NtParams& p, hipStream_t s) {
+    const int64_t n16 = ceil_div(p.N, 16);
+    const int64_t ntiles = ceil_div(p.M, 16);
+    const uintptr_t ca = reinterpret_cast<uintptr_t>(p.C);
+    if (n16 <= 16 || n16 > 60 || p.Kr > 256 || p.bias || p.accumulate || (ca & 15) != 0 || (p.ldc & 3) != 0 ||
+        ntiles < 8 * compute_units() || ntiles > INT32_MAX)
+        return false;
+    // One workgroup per compute unit, the whole output row in it: cutting the columns over two to four workgroups
+    // (more, smaller barrier groups per compute unit) was measured at 0.18 to 0.21 ms against 0.16 ms at
+    // 232,965 x 256 -> 602, because the pieces of a row then reach memory at different times.
+    const int waves = static_cast<int>(ceil_div(n16, 4)) + 1;  // the last one fetches
+    const int gx = compute_units();
+    if (p.Kr <= 128)
+        hipLaunchKernelGGL((gemm_ntr_kernel<2>), dim3(gx), dim3(64 * waves), 0, s, p, static_cast<int>(ntiles));
+    else
+        hipLaunchKernelGGL((gemm_ntr_kernel<4>), dim3(gx), dim3(64 * waves), 0, s, p, static_cast<int>(ntiles));
+    return true;
+}
+
 template <int VEC>
 static void launch_nt_vec(const NtParams& p, hipStream_t s) {
     const int64_t n16 = ceil_div(p.N, 16);
     const unsigned gx = static_cast<unsigned>(ceil_div(p.M, 128));
+    if (VEC == 16 && launch_ntr(p, s)) return;  // A rows in aligned 16-byte pieces
 #define TANGO_NT(NT_)                                                                             \
     hipLaunchKernelGGL((gemm_nt_kernel<NT_, VEC>), dim3(gx, static_cast<unsigned>(ceil_div(n16, NT_))), \
                        dim3(256), 0, s, p)

@@ -181,6 +181,36 @@ def test_qgemm_i8_small_operand_stationary(K, orc, M, N, Kd):
     assert np.array_equal(host(Y), want) and host(sY)[0] == orc.absmax_scale(want)
 
 
+@pytest.mark.parametrize("M,N,Kd,pitch,rows", [(40000, 602, 256, 608, False), (36005, 330, 100, 332, True),
+                                               (33000, 960, 64, 960, False), (34003, 264, 200, 264, True)])
+def test_nt_small_operand_in_registers(K, orc, M, N, Kd, pitch, rows):
+    """The NT form for outputs of 257 to 960 columns and many row tiles (the small operand's fragments stay in
+    registers, one wave fetches the A tiles for the others): output pitches that are and are not multiples of 16,
+    reductions of one, two and four k-steps, a last tile with fewer than 16 rows, the row multiplier, the output
+    scale; padding columns of the output beyond the next multiple of 16 must stay untouched."""
+    rng = np.random.default_rng(M + N + Kd)
+    A = rng.integers(-127, 128, (M, Kd)).astype(np.int8)
+    B = rng.integers(-127, 128, (Kd, N)).astype(np.int8)
+    ld = (Kd + 15) // 16 * 16
+    Abuf = torch.full((M, ld), 77, dtype=torch.int8, device="cuda")
+    Abuf[:, :Kd] = dev(A)
+    rs = dev(rng.random(M).astype(np.float32) + 0.5) if rows else None
+    acc = (A.astype(np.float64) @ B.astype(np.float64)).astype(np.float32) * np.float32(0.0625)
+    if rows:
+        acc = acc * host(rs)[:, None]
+    out = torch.full((M, pitch), -3.0, dtype=torch.float32, device="cuda")
+    K.cuda_kernels.QGEMM_backward_gradX(out[:, :N], Abuf[:, :Kd], dev(B), sc(0.5), sc(0.125), row_scale=rs)
+    assert np.array_equal(host(out[:, :N]), acc)
+    n16 = (N + 15) // 16 * 16
+    if pitch > n16:
+        assert bool((out[:, n16:] == -3.0).all())
+    if not rows:
+        Y = torch.empty((M, pitch), dtype=torch.float32, device="cuda")[:, :N]
+        sY = torch.empty(1, dtype=torch.float32, device="cuda")
+        K.cuda_kernels.QGEMM_i8(Y, Abuf[:, :Kd], dev(np.ascontiguousarray(B.T)), None, sY, sc(0.5), sc(0.125))
+        assert np.array_equal(host(Y), acc) and host(sY)[0] == orc.absmax_scale(acc)
+
+
 @pytest.mark.parametrize("M,N,Kd,rows", [(5000, 256, 256, False), (3001, 300, 41, True), (777, 64, 130, False)])
 def test_gradx_accumulates_into_its_output(K, M, N, Kd, rows):
     """gradX added to what dX holds == dX + the gradX written on its own, bit for bit (one fp32 addition per
