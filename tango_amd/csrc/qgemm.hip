@@ -590,6 +590,7 @@ struct FqParams {
     int64_t ldx, ldxq, ldb, ldc;
     int kp;               // K rounded up to 64
     int pitch;            // bytes between rows of the LDS block (fq_pitch)
+    int b_frag;           // B is in fragment order (see quantize_pack_w_kernel), rows zero-filled to a multiple of 16
 };
 
 // TPW = 16-column tiles per wave (the workgroup covers 64 * TPW columns), XV = floats per load,
@@ -706,18 +707,26 @@ __global__ __launch_bounds__(256, 2) void gemm_fq_kernel(const FqParams p) {
     if (n0 < p.N) {  // wave-uniform: waves whose columns lie beyond N only take part in phase A
         const int8_t* pb[TPW];
         bool bok[TPW];
+        // row-major B: a lane reads its 16 bytes from its own row (a cache line look-up per lane); fragment
+        // order: the wave reads one contiguous KB per fragment
+        const int64_t bstep = p.b_frag ? 1024 : 64;
 #pragma unroll
         for (int j = 0; j < TPW; ++j) {
             const int64_t n = n0 + j * 16 + r16;
             bok[j] = n < p.N;
-            pb[j] = p.B + (bok[j] ? n : 0) * p.ldb + g * 16;
+            if (p.b_frag) {
+                const int64_t tile = n0 + j * 16 < p.N ? (n0 >> 4) + j : 0;
+                pb[j] = p.B + ((tile * ksteps) << 10) + lane * 16;
+            } else {
+                pb[j] = p.B + (bok[j] ? n : 0) * p.ldb + g * 16;
+            }
         }
         // B fragments run two k-steps ahead of the MFMAs that consume them
         i32x4 b0[TPW], b1[TPW], b2[TPW];
         auto load_bfrag = [&](i32x4* dst, int step) {
             const int sc = step < ksteps ? step : ksteps - 1;
 #pragma unroll
-            for (int j = 0; j < TPW; ++j) dst[j] = *reinterpret_cast<const i32x4*>(pb[j] + static_cast<int64_t>(sc) * 64);
+            for (int j = 0; j < TPW; ++j) dst[j] = *reinterpret_cast<const i32x4*>(pb[j] + static_cast<int64_t>(sc) * bstep);
         };
         auto mma_step = [&](const i32x4* bf, int step) {
 #pragma unroll
@@ -796,6 +805,212 @@ __global__ __launch_bounds__(256, 2) void gemm_fq_kernel(const FqParams p) {
                 }
             }
         }
+    }
+    if (p.absmax_out) block_absmax_to_global(m / 127.0f, p.absmax_out);
+}
+
+// Forward GEMM with the quantize fused in, for tall X, 129 to 256 output columns and K <= 64 KSTEPS: one
+// persistent workgroup of sixteen waves per compute unit walks the 16-row tiles of X.  Waves 8..15 only stream:
+// each owns two rows of every tile, requests them three tiles ahead, quantizes them in registers and writes the
+// bytes to Xq and to a two-slot LDS ring.  Waves 0..7 only multiply and store: each keeps the B fragments of two
+// column tiles in registers for the whole launch (fragment-order packing: one contiguous KB per fragment), reads
+// the A fragments of the tile from the ring and stores a 16 x 32 piece of Y.  gemm_fq_kernel runs these phases
+// one after the other inside a workgroup of four waves; here the stream of X never pauses for the MFMAs or the
+// Y stores, and the sixteen rows of a tile reach Y (and Xq) together.  One barrier per tile hands a slot over.
+template <int KSTEPS, int XV, int MODE>
+__global__ __launch_bounds__(1024) void gemm_fqr_kernel(const FqParams p, int ntiles) {
+    constexpr int IT = (KSTEPS * 64 + 255) / 256;  // 256-column chunks of a row a lane loads from
+    constexpr int D = 3;                           // tiles in flight per streaming wave
+    extern __shared__ __attribute__((aligned(16))) int8_t ring[];  // 2 x ([16][pitch] + 64), then 256 floats of bias
+    const int pitch = p.pitch;
+    const int slot_bytes = 16 * pitch + 64;
+    float* bias_lds = reinterpret_cast<float*>(ring + 2 * slot_bytes);
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(static_cast<int>(threadIdx.x >> 6));
+    const int stride = static_cast<int>(gridDim.x);
+    const int t0 = static_cast<int>(blockIdx.x);
+    const int rounds = t0 < ntiles ? (ntiles - t0 + stride - 1) / stride : 0;  // the same for every wave
+    auto hand_over = [] { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); };
+    if (threadIdx.x < 256) bias_lds[threadIdx.x] = (p.bias && threadIdx.x < p.N) ? p.bias[threadIdx.x] : 0.0f;
+
+    if (wave >= 8) {  // ---- streaming waves: rows 2 (wave - 8) and 2 (wave - 8) + 1 of every tile
+        const int lr0 = 2 * (wave - 8);
+        const float rs = rscale_of(p.sA[0]);
+        // lane owns columns 4 (lane + 64 it) .. + 3 of its rows, read in pieces of XV floats; K is a multiple of XV
+        // (host), so a piece is either inside a row or past its end
+        bool in[IT][4 / XV];
+#pragma unroll
+        for (int it = 0; it < IT; ++it)
+#pragma unroll
+            for (int h = 0; h < 4 / XV; ++h) in[it][h] = ((lane + 64 * it) << 2) + XV * h < p.K;
+        // Every load is issued unconditionally (a piece past the end of a row reads the row's first floats, a row
+        // past the end of X reads the last row, a tile past the last one reads the last one again) and what must
+        // not count is replaced afterwards: the number of loads between a request and its use is then fixed, and
+        // the wait for a register set waits for that set only, not for the younger requests
+        const int t_last = t0 + (rounds - 1) * stride;
+        auto fetch = [&](float (*f)[IT][4], float* rm, int t) {
+            if (t > t_last) t = t_last;
+#pragma unroll
+            for (int b = 0; b < 2; ++b) {
+                int64_t row = static_cast<int64_t>(t) * 16 + lr0 + b;
+                if (row >= p.M) row = p.M - 1;  // last tile only; these rows are not stored
+                const float* xr = p.X + row * p.ldx;
+                const float* rp = p.x_row_mul ? p.x_row_mul + row : p.sA;
+                rm[b] = *rp;
+#pragma unroll
+                for (int it = 0; it < IT; ++it) {
+                    if (XV == 4) {
+                        const f32x4 v = __builtin_nontemporal_load(
+                            reinterpret_cast<const f32x4*>(xr + (in[it][0] ? (lane << 2) + 256 * it : 0)));
+                        f[b][it][0] = v.x; f[b][it][1] = v.y; f[b][it][2] = v.z; f[b][it][3] = v.w;
+                    } else {
+                        typedef float f32x2 __attribute__((ext_vector_type(2)));
+#pragma unroll
+                        for (int h = 0; h < 2; ++h) {
+                            const f32x2 v = __builtin_nontemporal_load(
+                                reinterpret_cast<const f32x2*>(xr + (in[it][h] ? (lane << 2) + 256 * it + 2 * h : 0)));
+                            f[b][it][2 * h] = v.x;
+                            f[b][it][2 * h + 1] = v.y;
+                        }
+                    }
+                }
+            }
+        };
+        auto emit = [&](float (*f)[IT][4], const float* rm, int slot) {
+#pragma unroll
+            for (int b = 0; b < 2; ++b) {
+                int8_t* dst = ring + slot * slot_bytes + (lr0 + b) * pitch + (lane << 2);
+#pragma unroll
+                for (int it = 0; it < IT; ++it) {
+                    const int c0 = (lane + 64 * it) << 2;
+                    if (c0 < pitch) {  // the columns between K and the pitch take zeros
+                        constexpr int H = 4 / XV;  // pieces per four floats
+                        float x0 = f[b][it][0], x1 = f[b][it][1], x2 = f[b][it][2], x3 = f[b][it][3];
+                        if (it == IT - 1) {  // K > 256 (IT - 1) (host): only the last chunk can reach past the row
+                            x0 = in[it][0] ? x0 : 0.0f; x1 = in[it][0] ? x1 : 0.0f;
+                            x2 = in[it][H - 1] ? x2 : 0.0f; x3 = in[it][H - 1] ? x3 : 0.0f;
+                        }
+                        if (p.x_row_mul) { x0 = x0 * rm[b]; x1 = x1 * rm[b]; x2 = x2 * rm[b]; x3 = x3 * rm[b]; }
+                        *reinterpret_cast<uint32_t*>(dst + 256 * it) =
+                            pack4(quant_one<MODE>(x0, rs, 0.f), quant_one<MODE>(x1, rs, 0.f),
+                                  quant_one<MODE>(x2, rs, 0.f), quant_one<MODE>(x3, rs, 0.f));
+                    }
+                }
+            }
+        };
+        // the register sets take turns by unrolling, so that no set is copied while its loads are in flight
+        float f[D][2][IT][4];
+        float rm[D][2];
+#pragma unroll
+        for (int u = 0; u < D; ++u) fetch(f[u], rm[u], t0 + u * stride);  // rounds >= 1 (host)
+        emit(f[0], rm[0], 0);
+        fetch(f[0], rm[0], t0 + D * stride);
+        hand_over();  // slot 0 holds round 0
+        // round k: the tile of round k + 1 goes to slot (k + 1) % 2 while waves 0..7 read slot k % 2
+        for (int kb = 0; kb < rounds; kb += D) {
+#pragma unroll
+            for (int u = 0; u < D; ++u) {
+                const int k = kb + u;
+                if (k >= rounds) break;
+                const int set = (u + 1) % D;
+                emit(f[set], rm[set], (k + 1) & 1);  // past the last round: the last tile again, read by nobody
+                fetch(f[set], rm[set], t0 + (k + 1 + D) * stride);
+                hand_over();
+            }
+        }
+        if (p.absmax_out) block_absmax_to_global(0.0f, p.absmax_out);
+        return;
+    }
+
+    // ---- multiplying waves: column tiles 2 wave and 2 wave + 1
+    const int g = lane >> 4, r16 = lane & 15;
+    const int n0 = 32 * wave;
+    i32x4 b[2][KSTEPS];
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+        const bool tile_ok = n0 + 16 * j < p.N;  // tiles past the last column multiply zeros and store nothing
+        const int8_t* pb = p.B + ((static_cast<int64_t>(tile_ok ? 2 * wave + j : 0) * KSTEPS) << 10) + lane * 16;
+#pragma unroll
+        for (int st = 0; st < KSTEPS; ++st) {
+            b[j][st] = i32x4{0, 0, 0, 0};
+            if (tile_ok) b[j][st] = *reinterpret_cast<const i32x4*>(pb + (st << 10));
+        }
+    }
+    const float s = p.sA[0] * p.sB[0];
+    const uintptr_t ca = reinterpret_cast<uintptr_t>(p.C);
+    const int wide = ((ca & 15) == 0 && (p.ldc & 3) == 0) ? 4 : ((ca & 7) == 0 && (p.ldc & 1) == 0) ? 2 : 1;
+    const int frag0 = r16 * pitch + g * 16;
+    const bool plain = !p.bias && wide == 4 && n0 + 32 <= p.N;
+    // Xq leaves through these waves too, 16 bytes per lane straight from the ring (a row of Xq is ldxq / 16 <= pitch / 16
+    // pieces; the bytes past K are the zeros the streaming waves wrote): the streaming waves hold 4 bytes per lane
+    // and row, and a store of 256 bytes per instruction costs as much issue time as one of 1 KB
+    const int cpr = static_cast<int>(p.ldxq >> 4);
+    int q_lds[2], q_row[2];
+    int64_t q_glb[2];
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+        const int id = i * 512 + wave * 64 + lane;
+        const int r = id / cpr, c = id - r * cpr;
+        q_row[i] = r < 16 ? r : -1;
+        q_lds[i] = r * pitch + c * 16;
+        q_glb[i] = static_cast<int64_t>(r) * p.ldxq + c * 16;
+    }
+    float m = 0.0f;
+    hand_over();
+    for (int k = 0; k < rounds; ++k) {
+        const int8_t* slot = ring + (k & 1) * slot_bytes + frag0;
+        i32x4 acc[2] = {i32x4{0, 0, 0, 0}, i32x4{0, 0, 0, 0}};
+#pragma unroll
+        for (int st = 0; st < KSTEPS; ++st) {
+            const i32x4 a = *reinterpret_cast<const i32x4*>(slot + st * 64);
+            acc[0] = mfma_16x16x64(b[0][st], a, acc[0]);  // operands swapped, see gemm_nt_kernel
+            acc[1] = mfma_16x16x64(b[1][st], a, acc[1]);
+        }
+        const int64_t row0 = static_cast<int64_t>(t0 + k * stride) * 16;
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+            if (q_row[i] >= 0 && row0 + q_row[i] < p.M)
+                *reinterpret_cast<i32x4*>(p.Xq + row0 * p.ldxq + q_glb[i]) =
+                    *reinterpret_cast<const i32x4*>(ring + (k & 1) * slot_bytes + q_lds[i]);
+        }
+        const int64_t row = row0 + r16;
+        if (row < p.M && plain) {  // whole tiles, 16-byte stores, no bias: nothing to test per tile
+            f32x4* cp = reinterpret_cast<f32x4*>(p.C + row * p.ldc + n0 + 4 * g);
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+                const f32x4 y{s * static_cast<float>(acc[j][0]), s * static_cast<float>(acc[j][1]),
+                              s * static_cast<float>(acc[j][2]), s * static_cast<float>(acc[j][3])};
+                m = fmaxf(fmaxf(m, fmaxf(fabsf(y[0]), fabsf(y[1]))), fmaxf(fabsf(y[2]), fabsf(y[3])));
+                cp[4 * j] = y;
+            }
+        } else if (row < p.M) {
+            float* crow = p.C + row * p.ldc;
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+                const int col = n0 + 16 * j + 4 * g;
+                if (col >= p.N) continue;
+                float y[4];
+                const f32x4 bv = *reinterpret_cast<const f32x4*>(bias_lds + col);
+#pragma unroll
+                for (int v = 0; v < 4; ++v) {
+                    y[v] = s * static_cast<float>(acc[j][v]);
+                    if (p.bias) y[v] = bv[v] + y[v];
+                    if (col + v < p.N) m = fmaxf(m, fabsf(y[v]));
+                }
+                if (col + 4 <= p.N && wide == 4) {
+                    *reinterpret_cast<f32x4*>(crow + col) = f32x4{y[0], y[1], y[2], y[3]};
+                } else if (col + 4 <= p.N && wide == 2) {
+                    typedef float f32x2 __attribute__((ext_vector_type(2)));
+                    *reinterpret_cast<f32x2*>(crow + col) = f32x2{y[0], y[1]};
+                    *reinterpret_cast<f32x2*>(crow + col + 2) = f32x2{y[2], y[3]};
+                } else {
+#pragma unroll
+                    for (int v = 0; v < 4; ++v)
+                        if (col + v < p.N) crow[col + v] = y[v];
+                }
+            }
+        }
+        hand_over();  // the slot just read may be refilled, the other one is complete
     }
     if (p.absmax_out) block_absmax_to_global(m / 127.0f, p.absmax_out);
 }
@@ -998,19 +1213,26 @@ __global__ __launch_bounds__(256) void quantize_pack_w_kernel(const float* __res
                                                               const float* __restrict__ scale,
                                                               int8_t* __restrict__ Wq, int8_t* __restrict__ packed,
                                                               int64_t ldp, int64_t N, int64_t K,
-                                                              float* __restrict__ zero_slot) {
+                                                              float* __restrict__ zero_slot, int frag) {
     if (zero_slot && blockIdx.x == 0 && threadIdx.x == 0) zero_slot[0] = 0.0f;
     const float r = rscale_of(scale[0]);
-    const int64_t total = N * ldp;
+    // frag: the packed copy is laid out in MFMA fragment order instead of rows (ldp is a multiple of 64): the 16
+    // bytes that lane 16 g + r feeds the MFMA of column tile j at k-step st (row 16 j + r, columns 64 st + 16 g ..)
+    // stand at ((j ldp / 64 + st) 64 + 16 g + r) 16, so that a wave fetches a fragment as one contiguous KB; rows
+    // up to the next multiple of 16 are zero-filled
+    const int64_t rows = frag ? (N + 15) / 16 * 16 : N;
+    const int64_t total = rows * ldp;
     const int64_t nthr = static_cast<int64_t>(gridDim.x) * blockDim.x;
     for (int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < total; i += nthr) {
         const int64_t n = i / ldp, k = i - n * ldp;
         int8_t q = 0;
-        if (k < K) {
+        if (k < K && n < N) {
             q = static_cast<int8_t>(quant_one<MODE>(W[n * ldw + k], r, 0.0f));
             Wq[n * K + k] = q;
         }
-        packed[i] = q;
+        int64_t at = i;
+        if (frag) at = ((((n >> 4) * (ldp >> 6) + (k >> 6)) << 6) + (((k >> 4) & 3) << 4) + (n & 15)) * 16 + (k & 15);
+        packed[at] = q;
     }
 }
 
@@ -1358,9 +1580,13 @@ static bool launch_ws_nt(const FqParams& p, hipStream_t s) {
 // outputs were measured with this kernel too, eight or twelve waves per compute unit and 4 NT accumulator
 // registers per lane: 232,965 x 602 x 256 0.336 ms against 0.29 ms for gemm_fq_kernel, x 256 x 41 0.098 against
 // 0.080 ms.)
+static bool ws_shape(int64_t M, int64_t N) {
+    return N <= 32 && ceil_div(M, 16) >= 12LL * compute_units() && ceil_div(M, 16) <= INT32_MAX;
+}
+
 template <int XV, int MODE>
 static bool launch_ws(const FqParams& p, hipStream_t s) {
-    if (p.N > 32 || ceil_div(p.M, 16) < 12LL * compute_units() || ceil_div(p.M, 16) > INT32_MAX) return false;
+    if (!ws_shape(p.M, p.N)) return false;
     if (p.N <= 16) return launch_ws_nt<1, XV, MODE, 768>(p, s);
     return launch_ws_nt<2, XV, MODE, 768>(p, s);
 }
@@ -1377,7 +1603,22 @@ static int fq_pitch(int64_t K) {
 template <int XV, int MODE>
 static void launch_fq_mode(const FqParams& p, hipStream_t s) {
     constexpr int RT = 4;  // 64 rows per workgroup measured faster than 32 at every benchmark shape
-    if (launch_ws<XV, MODE>(p, s)) return;
+    if (!p.b_frag && launch_ws<XV, MODE>(p, s)) return;
+    if (p.b_frag && p.N > 128 && p.N <= 256 && (p.kp == 640 || p.kp == 256) && p.ldxq <= p.pitch && p.K % 2 == 0 &&
+        p.K > (p.kp == 640 ? 512 : 0) && ceil_div(p.M, 16) >= 8LL * compute_units() && ceil_div(p.M, 16) <= INT32_MAX) {
+        const size_t lds = 2 * (static_cast<size_t>(16) * p.pitch + 64) + 256 * sizeof(float);
+        const int nt = static_cast<int>(ceil_div(p.M, 16));
+        const bool v4 = XV == 4 && p.K % 4 == 0;
+#define TANGO_FQR(KS_)                                                                                              \
+    do {                                                                                                            \
+        if (v4) hipLaunchKernelGGL((gemm_fqr_kernel<KS_, 4, MODE>), dim3(compute_units()), dim3(1024), lds, s, p, nt); \
+        else hipLaunchKernelGGL((gemm_fqr_kernel<KS_, 2, MODE>), dim3(compute_units()), dim3(1024), lds, s, p, nt);  \
+    } while (0)
+        if (p.kp == 640) TANGO_FQR(10);
+        else TANGO_FQR(4);
+#undef TANGO_FQR
+        return;
+    }
     const size_t lds = static_cast<size_t>(16 * RT) * p.pitch + 64 + 256 * sizeof(float);
     const unsigned gx = static_cast<unsigned>(ceil_div(p.M, 16 * RT));
 #define TANGO_FQ_IT(TPW_, IT_)                                                                   \
@@ -1427,7 +1668,7 @@ extern "C" {
 size_t tango_qgemm_fwd_workspace(int64_t M, int64_t N, int64_t K) {
     (void)M;
     if (N <= 0 || K <= 0) return 0;
-    return static_cast<size_t>(N * round_up(K, 64));
+    return static_cast<size_t>(round_up(N, 16) * round_up(K, 64));  // rows to a multiple of 16: the fragment-order form
 }
 
 int tango_qgemm_fwd_ex(float* Y, int64_t ldy, const float* X, int64_t ldx, const float* x_row_mul, int8_t* Xq, int64_t ldxq,
@@ -1457,14 +1698,17 @@ int tango_qgemm_fwd_ex(float* Y, int64_t ldy, const float* X, int64_t ldx, const
     }
     int8_t* Bp = static_cast<int8_t*>(workspace);
     const int64_t ldb = round_up(K, 64);
+    // the fused kernel reads the small operand fragment by fragment; the W-stationary one (narrow outputs) and the
+    // kernels for an int8 X stage its rows through LDS
+    const int frag = fused && !ws_shape(M, N);
     if (N > 0 && K > 0) {  // W -> Wq and its packed copy, and the zeroing of scaleY, in one launch
-        const dim3 wgrid(grid_for(N * ldb, 256));
+        const dim3 wgrid(grid_for(round_up(N, 16) * ldb, 256));
         if (round_mode == TANGO_ROUND_RNE)
             hipLaunchKernelGGL(quantize_pack_w_kernel<TANGO_ROUND_RNE>, wgrid, dim3(256), 0, s, W, ldw, scaleW, Wq, Bp,
-                               ldb, N, K, scaleY);
+                               ldb, N, K, scaleY, frag);
         else
             hipLaunchKernelGGL(quantize_pack_w_kernel<TANGO_ROUND_TRUNC>, wgrid, dim3(256), 0, s, W, ldw, scaleW, Wq, Bp,
-                               ldb, N, K, scaleY);
+                               ldb, N, K, scaleY, frag);
     } else if (scaleY) {
         fill_u32(scaleY, 0u, 1, s);
     }
@@ -1473,7 +1717,7 @@ int tango_qgemm_fwd_ex(float* Y, int64_t ldy, const float* X, int64_t ldx, const
         FqParams q{};
         q.C = Y; q.X = X; q.Xq = Xq; q.B = Bp; q.bias = bias; q.x_row_mul = x_row_mul; q.absmax_out = scaleY;
         q.sA = scaleX; q.sB = scaleW; q.M = M; q.N = N; q.K = K; q.ldx = ldx; q.ldxq = ldxq; q.ldb = ldb;
-        q.ldc = ldy; q.kp = static_cast<int>(ldb); q.pitch = fq_pitch(K);
+        q.ldc = ldy; q.kp = static_cast<int>(ldb); q.pitch = fq_pitch(K); q.b_frag = frag;
         return launch_fq(q, round_mode, s, true);
     }
     NtParams p{};
@@ -1503,10 +1747,10 @@ int tango_qgemm_fwd_q8(int8_t* Yq, int64_t ldyq, float* scaleY, const int8_t* Xq
         const dim3 wgrid(grid_for(N * ldb, 256));
         if (round_mode == TANGO_ROUND_RNE)
             hipLaunchKernelGGL(quantize_pack_w_kernel<TANGO_ROUND_RNE>, wgrid, dim3(256), 0, s, W, ldw, scaleW, Wq, Bp,
-                               ldb, N, K, scaleY);
+                               ldb, N, K, scaleY, 0);
         else
             hipLaunchKernelGGL(quantize_pack_w_kernel<TANGO_ROUND_TRUNC>, wgrid, dim3(256), 0, s, W, ldw, scaleW, Wq, Bp,
-                               ldb, N, K, scaleY);
+                               ldb, N, K, scaleY, 0);
     } else {
         fill_u32(scaleY, 0u, 1, s);
     }

@@ -65,6 +65,36 @@ def test_forward(K, orc, M, N, Kd, padded):
     assert orc.overflow_count() == 0
 
 
+@pytest.mark.parametrize("M,N,Kd,mode,rowmul", [(33003, 256, 602, "trunc", False), (33000, 200, 580, "rne", True),
+                                                  (34001, 130, 256, "trunc", True), (33500, 256, 200, "rne", False),
+                                                  (33100, 256, 604, "trunc", False)])
+def test_forward_persistent_form(K, orc, M, N, Kd, mode, rowmul):
+    """The forward kernel for tall X and 129..256 output columns (a persistent workgroup per compute unit; half of
+    its waves stream and quantize X, the other half multiply and store): reductions of ten and of four k-steps,
+    rows read in 8- and in 16-byte pieces, a last tile with fewer than 16 rows, output columns that do not fill the
+    last column tile, bias, the row multiplier, both rounding modes; Xq, its zero padding, Wq, Y and the output
+    scale are compared."""
+    rng = np.random.default_rng(M + N + Kd)
+    X = rng.standard_normal((M, Kd)).astype(np.float32)
+    W = glorot(rng, N, Kd)
+    bias = rng.standard_normal(N).astype(np.float32) if N != 256 else None
+    rm = (rng.random(M).astype(np.float32) + 0.5) if rowmul else None
+    Xs = X * rm[:, None] if rowmul else X
+    Xd, Wd = dev(X), dev(W)
+    sX = dev(np.array([orc.absmax_scale(Xs)], np.float32))
+    sW = K.cuda_kernels.get_scale(Wd)
+    ld = (Kd + 15) // 16 * 16
+    Xbuf = torch.full((M, ld), 99, dtype=torch.int8, device="cuda")
+    Wq = torch.empty((N, Kd), dtype=torch.int8, device="cuda")
+    Y, sY = K.QGEMM_forward(Xd, Xbuf[:, :Kd], sX, Wd, Wq, sW, None if bias is None else dev(bias), True,
+                            round_mode=mode, x_row_mul=None if rm is None else dev(rm))
+    oY, oXq, oWq, _, _, osY = orc.qgemm_fwd(Xs, W, bias=bias, reduce=True, mode=orc.RNE if mode == "rne" else orc.TRUNC,
+                                            sX=host(sX)[0])
+    assert np.array_equal(host(Xbuf[:, :Kd]), oXq) and not host(Xbuf[:, Kd:]).any()
+    assert np.array_equal(host(Wq), oWq)
+    assert np.array_equal(host(Y), oY) and host(sY)[0] == osY
+
+
 def test_forward_rne_mode_and_lcg_pattern(K, orc):
     rng = np.random.default_rng(0)
     X = rng.standard_normal((200, 72)).astype(np.float32)
