@@ -357,8 +357,8 @@ int tango_edge_softmax_fwd(float* a, const float* e, const int64_t* indptr,
    in a fixed array of TANGO_EDGE_SOFTMAX_STATIC_BYTES inside the library's device image (one copy
    per GPU, held until the process ends) and no memory is allocated or freed by the call.
    Inputs with tango_edge_softmax_workspace(num_edges, H) > TANGO_EDGE_SOFTMAX_STATIC_BYTES are
-   rejected with TANGO_ERR_STATIC_LIMIT before anything is launched (at H = 8 the limit is about
-   3.5 million edges).  All calls on one GPU share the array: calls that overlap on one GPU
+   rejected with TANGO_ERR_STATIC_LIMIT before anything is launched (at H = 8 a span of 128 slots
+   takes 160 bytes: the limit is about 3.3 million edges).  All calls on one GPU share the array: calls that overlap on one GPU
    (different streams or threads) race; calls on one stream are ordered and safe. */
 #define TANGO_EDGE_SOFTMAX_STATIC_BYTES (4u << 20)
 int tango_edge_softmax_fwd_static(float* a, const float* e, const int64_t* indptr,
