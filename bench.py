@@ -54,8 +54,11 @@ def parse():
                     help="--profile-mode spmm on the benchmark graph with its node ids randomly permuted")
     ap.add_argument("--gemm-shape", default="256,41", metavar="K,N",
                     help="layer shape of --profile-mode gradx / gradw (dY [nodes, N] int8, X [nodes, K])")
+    ap.add_argument("--attn-graph", choices=["gat", "hgt"], default="gat",
+                    help="graph of --profile-mode umule / sddmm-dot: the 169,343-node GAT graph (8 heads x 16) or the "
+                         "170,000-node / 8.17 M-edge homogenised heterogeneous graph (4 heads x 64)")
     ap.add_argument("--profile-mode", default=None,
-                    choices=["spmm", "copy", "qlinear", "gradx", "gradw", "sddmm", "quantize", "softmax",
+                    choices=["spmm", "copy", "qlinear", "gradx", "gradw", "sddmm", "quantize", "softmax", "umule",
                              "gat", "arxiv", "hgt", "hetero"],
                     help="run only the dominant kernel (spmm: copy_u F=256 on the benchmark graph) or a "
                          "1 GiB device copy (counter calibration), for rocprofv3 --pmc passes")
@@ -491,6 +494,26 @@ def main():
         byt = M * N + N * Kd + 4 * M * Kd if dx else M * (N + Kd) + 4 * N * Kd
         print(json.dumps({"profile_mode": args.profile_mode, "M": M, "K": Kd, "N": N, "avg_ms": round(ms, 4),
                           "ops": 2 * M * N * Kd, "algorithmic_bytes": byt}))
+        return
+    if args.profile_mode == "umule":  # the attention layers' aggregation (u_mul_e, edge-major int8 edge values) and SDDMM dot
+        from tango_amd.graph import hetero_power_law
+        if args.attn_graph == "gat":
+            g4, H, D = chung_lu(169343, 1166243, 2.2, seed=4, device="cuda"), 8, 16
+        else:
+            g4, H, D = hetero_power_law(device="cuda")[0], 4, 64
+        g4 = graph_preprocess(g4.reorder_edges_by_dst())
+        n4, E = g4.num_nodes(), g4.num_edges()
+        feat = torch.randint(-127, 128, (n4, H, D), dtype=torch.int8, device="cuda")
+        ev = torch.randint(-127, 128, (E, H, 1), dtype=torch.int8, device="cuda")
+        one = torch.full((1,), 0.01, device="cuda")
+        ms = time_op(lambda: K.multi_cusparse_SPMM(g4, feat, ev, one, edge_major=True), iters=args.steps, warm=args.warmup)
+        ms_d = time_op(lambda: K.mySDDMM_int8(g4, "dot", feat, feat, one, one, False), iters=args.steps, warm=args.warmup)
+        print(json.dumps({"profile_mode": "umule", "graph": args.attn_graph, "nodes": n4, "edges": E, "H": H, "D": D,
+                          "u_mul_e_ms": round(ms, 4), "sddmm_dot_ms": round(ms_d, 4),
+                          "u_mul_e_gather_model_bytes": E * (H * D + H + 2 * IDX_BYTES) + n4 * (4 * H * D + 8),
+                          "u_mul_e_compulsory_bytes": E * (H + 2 * IDX_BYTES) + n4 * (5 * H * D + 8),
+                          "sddmm_gather_model_bytes": E * (16 + 2 * H * D + 4 * H),
+                          "sddmm_compulsory_bytes": E * 16 + 2 * n4 * H * D + 4 * E * H}))
         return
     if args.profile_mode == "softmax":  # edge softmax forward / backward, 8 heads, on the 169,343-node graph
         g4 = graph_preprocess(chung_lu(169343, 1166243, 2.2, seed=4, device="cuda").reorder_edges_by_dst())

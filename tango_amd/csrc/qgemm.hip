@@ -495,7 +495,7 @@ __global__ __launch_bounds__(1024) void gemm_ntr_kernel(const NtParams p, int nt
             if (u < rounds) fetch(v[u], rs[u], t0 + u * stride);
         if (rounds > 0) put(v[0], rs[0], 0);
         if (4 < rounds) fetch(v[0], rs[0], t0 + 4 * stride);
-        hand_over();  // slot 0 holds round 0
+        hand_over();  // slot 0 holds the first tile
         // round k: the tile of round k + 1 goes to slot (k + 1) % 2 while the other waves read slot k % 2
         for (int kb = 0; kb < rounds; kb += 4) {
 #pragma unroll
@@ -843,7 +843,9 @@ __global__ __launch_bounds__(1024) void gemm_fqr_kernel(const FqParams p, int nt
         for (int it = 0; it < IT; ++it)
 #pragma unroll
             for (int h = 0; h < 4 / XV; ++h) in[it][h] = ((lane + 64 * it) << 2) + XV * h < p.K;
-        // Every load is issued unconditionally (a piece past the end of a row reads the row's first floats, a row
+        const int last_piece = static_cast<int>(p.K) - XV;  // where the pieces past a row's end read instead
+        // Every load is issued unconditionally (a piece past the end of a row reads the row's last piece again:
+        // the same 64 bytes as its neighbour lanes in the same instruction, so no request is added; a row
         // past the end of X reads the last row, a tile past the last one reads the last one again) and what must
         // not count is replaced afterwards: the number of loads between a request and its use is then fixed, and
         // the wait for a register set waits for that set only, not for the younger requests
@@ -861,14 +863,14 @@ __global__ __launch_bounds__(1024) void gemm_fqr_kernel(const FqParams p, int nt
                 for (int it = 0; it < IT; ++it) {
                     if (XV == 4) {
                         const f32x4 v = __builtin_nontemporal_load(
-                            reinterpret_cast<const f32x4*>(xr + (in[it][0] ? (lane << 2) + 256 * it : 0)));
+                            reinterpret_cast<const f32x4*>(xr + (in[it][0] ? (lane << 2) + 256 * it : last_piece)));
                         f[b][it][0] = v.x; f[b][it][1] = v.y; f[b][it][2] = v.z; f[b][it][3] = v.w;
                     } else {
                         typedef float f32x2 __attribute__((ext_vector_type(2)));
 #pragma unroll
                         for (int h = 0; h < 2; ++h) {
                             const f32x2 v = __builtin_nontemporal_load(
-                                reinterpret_cast<const f32x2*>(xr + (in[it][h] ? (lane << 2) + 256 * it + 2 * h : 0)));
+                                reinterpret_cast<const f32x2*>(xr + (in[it][h] ? (lane << 2) + 256 * it + 2 * h : last_piece)));
                             f[b][it][2 * h] = v.x;
                             f[b][it][2 * h + 1] = v.y;
                         }
@@ -905,7 +907,7 @@ __global__ __launch_bounds__(1024) void gemm_fqr_kernel(const FqParams p, int nt
         for (int u = 0; u < D; ++u) fetch(f[u], rm[u], t0 + u * stride);  // rounds >= 1 (host)
         emit(f[0], rm[0], 0);
         fetch(f[0], rm[0], t0 + D * stride);
-        hand_over();  // slot 0 holds round 0
+        hand_over();  // slot 0 holds the first tile
         // round k: the tile of round k + 1 goes to slot (k + 1) % 2 while waves 0..7 read slot k % 2
         for (int kb = 0; kb < rounds; kb += D) {
 #pragma unroll

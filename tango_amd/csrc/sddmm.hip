@@ -50,6 +50,63 @@ __global__ __launch_bounds__(256) void sddmm_dot_kernel(
     if (REDUCE) block_absmax_to_global(m / 127.0f, scale_out);
 }
 
+// The dot product when an edge's H * D bytes are a power of two of at most 1 KB (D = 16 * LPH): the 64 lanes of a
+// wavefront hold 64 / (H * LPH) whole edges, a lane's place inside its edge never changes, and the edge index is
+// wave-uniform arithmetic, so the loop carries no division (the kernels below divide a 64-bit index by a run-time
+// value per element, which costs more instructions than the dot product itself).  Four groups of edges per
+// iteration: the index loads of all four, then the eight row loads, are in flight together.  Every load is
+// unconditional (edges past the end read the last edge again and store nothing).
+template <int LPH, bool REDUCE>
+__global__ __launch_bounds__(256) void sddmm_dot_wave_kernel(
+    float* __restrict__ out, float* __restrict__ scale_out, const int64_t* __restrict__ src,
+    const int64_t* __restrict__ dst, const int8_t* __restrict__ U, const int8_t* __restrict__ V,
+    const float* __restrict__ sU, const float* __restrict__ sV, int64_t E, int H, int shift) {
+    constexpr int UNR = 8;
+    const float s = sU[0] * sV[0];
+    const int lane = threadIdx.x & (kWave - 1);
+    const int per = 1 << shift;            // lanes per edge = H * LPH
+    const int epw = kWave >> shift;        // edges per wavefront and group
+    const int sub = lane >> shift;         // the lane's edge inside a group
+    const int r = lane & (per - 1);        // the lane's 16-byte piece of the edge's row
+    const bool writer = (r & (LPH - 1)) == 0;
+    const int head = r / LPH;
+    const int64_t wave = (static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x) >> 6;
+    const int64_t waves = (static_cast<int64_t>(gridDim.x) * blockDim.x) >> 6;
+    const int64_t step = static_cast<int64_t>(epw) * UNR;
+    float m = 0.0f;
+    for (int64_t base = wave * step; base < E; base += waves * step) {
+        int64_t e[UNR], su[UNR], dv[UNR];
+#pragma unroll
+        for (int u = 0; u < UNR; ++u) {
+            e[u] = base + u * epw + sub;
+            const int64_t ec = e[u] < E ? e[u] : E - 1;
+            su[u] = src[ec];
+            dv[u] = dst[ec];
+        }
+        u32x4 a[UNR], b[UNR];
+#pragma unroll
+        for (int u = 0; u < UNR; ++u) {
+            a[u] = *reinterpret_cast<const u32x4*>(U + (((su[u] << shift) + r) << 4));
+            b[u] = *reinterpret_cast<const u32x4*>(V + (((dv[u] << shift) + r) << 4));
+        }
+#pragma unroll
+        for (int u = 0; u < UNR; ++u) {
+            int acc = __builtin_amdgcn_sdot4(a[u].x, b[u].x, 0, false);
+            acc = __builtin_amdgcn_sdot4(a[u].y, b[u].y, acc, false);
+            acc = __builtin_amdgcn_sdot4(a[u].z, b[u].z, acc, false);
+            acc = __builtin_amdgcn_sdot4(a[u].w, b[u].w, acc, false);
+#pragma unroll
+            for (int off = 1; off < LPH; off <<= 1) acc += __shfl_xor(acc, off, kWave);
+            if (writer && e[u] < E) {
+                const float y = static_cast<float>(acc) * s;
+                __builtin_nontemporal_store(y, out + e[u] * H + head);
+                if (REDUCE) m = fmaxf(m, fabsf(y));
+            }
+        }
+    }
+    if (REDUCE) block_absmax_to_global(m / 127.0f, scale_out);
+}
+
 // Heads wider than 16 bytes (D = 16 * LPH, LPH a power of two): LPH consecutive lanes share one
 // (edge, head) pair, each with 16 bytes of it, so the lanes of an edge read its two rows as
 // contiguous runs; the partial dot products meet with xor-shuffles.  (With one lane per head and
@@ -190,6 +247,30 @@ int tango_sddmm_dot_i8(float* out, float* scale_out, const int64_t* src, const i
     const uintptr_t al = reinterpret_cast<uintptr_t>(U) | reinterpret_cast<uintptr_t>(V);
     const int vec = ((D & 15) == 0 && (al & 15) == 0) ? 16 : ((D & 3) == 0 && (al & 3) == 0) ? 4 : 1;
     const int64_t lph = D / 16;
+    const int64_t per = H * lph;  // lanes per edge with 16 bytes per lane
+    if (vec == 16 && lph >= 1 && lph <= 16 && (lph & (lph - 1)) == 0 && per <= 64 && (per & (per - 1)) == 0 &&
+        D == 16 * lph) {
+        int shift = 0;
+        while ((1 << shift) < per) ++shift;
+        const int64_t groups = ceil_div(num_edges, (64 / per) * 8);  // wavefront iterations of four edge groups
+        const dim3 wgrid(grid_for(groups * 64, 256, 16)), wblock(256);
+#define TANGO_DOT_WAVE(L_)                                                                                    \
+    do {                                                                                                      \
+        if (scale_out)                                                                                        \
+            hipLaunchKernelGGL((sddmm_dot_wave_kernel<L_, true>), wgrid, wblock, 0, s, out, scale_out, src,   \
+                               dst, U, V, sU, sV, num_edges, static_cast<int>(H), shift);                     \
+        else                                                                                                  \
+            hipLaunchKernelGGL((sddmm_dot_wave_kernel<L_, false>), wgrid, wblock, 0, s, out, scale_out, src,  \
+                               dst, U, V, sU, sV, num_edges, static_cast<int>(H), shift);                     \
+    } while (0)
+        if (lph == 1) TANGO_DOT_WAVE(1);
+        else if (lph == 2) TANGO_DOT_WAVE(2);
+        else if (lph == 4) TANGO_DOT_WAVE(4);
+        else if (lph == 8) TANGO_DOT_WAVE(8);
+        else TANGO_DOT_WAVE(16);
+#undef TANGO_DOT_WAVE
+        return launch_status();
+    }
     if (vec == 16 && lph >= 2 && lph <= 16 && (lph & (lph - 1)) == 0) {
         const dim3 sgrid(grid_for(total * lph, 256, 16)), sblock(256);
 #define TANGO_DOT_SPLIT(L_)                                                                                   \
