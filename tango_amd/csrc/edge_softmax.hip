@@ -378,7 +378,7 @@ __global__ __launch_bounds__(256) void span_kernel(
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-    const unsigned sub = (maskw[(g * K) >> 5] >> ((g * K) & 31)) & ((1u << K) - 1u);
+    const unsigned sub = (maskw[(g * K) >> 5] >> ((g * K) & 31)) & (K == 32 ? 0xFFFFFFFFu : (1u << (K & 31)) - 1u);
     const bool last_open = (maskw[8] & 1u) == 0u;  // the row of the last slot runs on into the next span
     const bool head = (maskw[0] & 1u) == 0u;       // the row of the first slot began before the span
     const uint64_t bm = __ballot(sub != 0u);       // lanes of groups that hold a row start
