@@ -67,7 +67,10 @@ struct SpmmParams {
     size_t span_ws_bytes;
 };
 
-enum { KIND_COPY = 0, KIND_WEIGHTED = 1, KIND_COO = 2 };
+enum { KIND_COPY = 0, KIND_WEIGHTED = 1, KIND_COO = 2, KIND_WEIGHTED_F32 = 3 };
+// weighted kinds: int8 edge values, or fp32 edge values rounded as they are loaded (a kind of its own, so that the
+// int8 path carries no test for it: on 8-byte rows a uniform branch per slot cost 16 % of the launch)
+__host__ __device__ constexpr bool weighted(int kind) { return kind == KIND_WEIGHTED || kind == KIND_WEIGHTED_F32; }
 
 // Byte offset of gathered row j: a shift when the row pitch allows (64-bit multiplies are quarter rate).
 __device__ __forceinline__ int64_t row_offset(int j, const SpmmParams& p) {
@@ -161,8 +164,9 @@ struct LaneCols {
 };
 
 // The int8 edge value at position pos (in units of ev_se) as the multiplier byte of a v_dot4.
+template <int KIND>
 __device__ __forceinline__ uint32_t edge_value(const SpmmParams& p, const LaneCols& c, int64_t pos) {
-    if (p.evals_f32)  // uniform
+    if (KIND == KIND_WEIGHTED_F32)
         return static_cast<uint32_t>(quant_one<TANGO_ROUND_RNE>(c.wbase_f[pos * p.ev_se], c.ev_r, 0.0f)) & 0xffu;
     return static_cast<uint32_t>(static_cast<uint8_t>(c.wbase[pos * p.ev_se]));
 }
@@ -183,11 +187,11 @@ __device__ __forceinline__ LaneCols lane_cols(const SpmmParams& p, int lane) {
     c.wbase = p.evals;
     c.wbase_f = p.evals_f32;
     c.ev_r = 0.0f;
-    if (KIND == KIND_WEIGHTED && c.col_ok) {
+    if (weighted(KIND) && c.col_ok) {
         const int64_t h = c.col / p.F;
         const int64_t d = (p.D == 1) ? 0 : (c.col - h * p.F);
         c.wbase = p.evals + h * p.ev_sh + d * p.ev_sd;
-        if (p.evals_f32) {
+        if (KIND == KIND_WEIGHTED_F32) {
             c.wbase_f = p.evals_f32 + h * p.ev_sh + d * p.ev_sd;
             c.ev_r = rscale_of(p.scale2[0]);
         }
@@ -218,7 +222,7 @@ __device__ __forceinline__ void wave_row_sum(const SpmmParams& p, const LaneCols
             const int v = load_index<true>(p, p.indices, qc);
             my[r] = q < end ? v : -1;
             my_e[r] = 0;
-            if (KIND == KIND_WEIGHTED && p.edge_ids)
+            if (weighted(KIND) && p.edge_ids)
                 my_e[r] = load_index<true>(p, p.edge_ids, qc);
         }
         // The 256 slots are walked as one flat sequence of steps (64 / lpe slots each), always
@@ -236,7 +240,7 @@ __device__ __forceinline__ void wave_row_sum(const SpmmParams& p, const LaneCols
                 const int reg = r == 0 ? my[0] : r == 1 ? my[1] : r == 2 ? my[2] : my[3];
                 j[u] = __shfl(reg, slot, kWave);
                 sl[u] = 0;
-                if (KIND == KIND_WEIGHTED) {
+                if (weighted(KIND)) {
                     const int rege = r == 0 ? my_e[0] : r == 1 ? my_e[1] : r == 2 ? my_e[2] : my_e[3];
                     // position of this slot's edge value: permuted id, or the CSR slot itself
                     sl[u] = p.edge_ids ? static_cast<int64_t>(__shfl(rege, slot, kWave)) : base + r * kWave + slot;
@@ -250,8 +254,8 @@ __device__ __forceinline__ void wave_row_sum(const SpmmParams& p, const LaneCols
                 // invalid slots read row 0 with multiplier 0: no branch around the load
                 d[u] = Gather<VEC>::load(c.fcol + row_offset(ok ? j[u] : 0, p));
                 uint32_t w = 1u;
-                if (KIND == KIND_WEIGHTED)
-                    w = edge_value(p, c, ok ? sl[u] : 0);
+                if (weighted(KIND))
+                    w = edge_value<KIND>(p, c, ok ? sl[u] : 0);
                 m |= (ok ? w : 0u) << (8 * u);
             }
             accumulate4<VEC>(acc, d, m);
@@ -404,7 +408,7 @@ __global__ __launch_bounds__(256) void spmm_group_kernel(const SpmmParams p) {
     // a wave's groups stage their rows' column indices (and edge ids) here, so that the gather loop
     // holds no dependent index load; used when a wave has at most 16 groups
     __shared__ int sidx[4][16 * kGroupRow];
-    __shared__ int seid[KIND == KIND_WEIGHTED ? 4 : 1][KIND == KIND_WEIGHTED ? 16 * kGroupRow : 1];
+    __shared__ int seid[weighted(KIND) ? 4 : 1][weighted(KIND) ? 16 * kGroupRow : 1];
     const int lane = lane_id();
     const int wave = __builtin_amdgcn_readfirstlane(static_cast<int>(threadIdx.x) >> 6);
     const LaneCols c = lane_cols<VEC, KIND>(p, lane);
@@ -417,11 +421,11 @@ __global__ __launch_bounds__(256) void spmm_group_kernel(const SpmmParams p) {
     const bool mine = row < p.rows && end - start <= kGroupRow;
     const int deg = mine ? static_cast<int>(end - start) : 0;
     const bool staged = p.lpe_log2 >= 2;
-    const bool permuted = KIND == KIND_WEIGHTED && p.edge_ids;
+    const bool permuted = weighted(KIND) && p.edge_ids;
     if (staged) {
         for (int k = c.sub; k < deg; k += c.lpe) {
             sidx[wave][(c.grp << 5) + k] = load_index<false>(p, p.indices, start + k);
-            if (permuted) seid[KIND == KIND_WEIGHTED ? wave : 0][(c.grp << 5) + k] = load_index<false>(p, p.edge_ids, start + k);
+            if (permuted) seid[weighted(KIND) ? wave : 0][(c.grp << 5) + k] = load_index<false>(p, p.edge_ids, start + k);
         }
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
@@ -440,12 +444,12 @@ __global__ __launch_bounds__(256) void spmm_group_kernel(const SpmmParams p) {
             const int j = staged ? sidx[wave][(c.grp << 5) + slot] : load_index<false>(p, p.indices, start + slot);
             d[u] = Gather<VEC>::load(c.fcol + row_offset(j, p));
             uint32_t w = 1u;
-            if (KIND == KIND_WEIGHTED) {
+            if (weighted(KIND)) {
                 int64_t pos = start + slot;
                 if (permuted)
-                    pos = staged ? seid[KIND == KIND_WEIGHTED ? wave : 0][(c.grp << 5) + slot]
+                    pos = staged ? seid[weighted(KIND) ? wave : 0][(c.grp << 5) + slot]
                                  : load_index<false>(p, p.edge_ids, start + slot);
-                w = edge_value(p, c, pos);
+                w = edge_value<KIND>(p, c, pos);
             }
             m |= (ok ? w : 0u) << (8 * u);
         }
@@ -723,7 +727,7 @@ __global__ __launch_bounds__(256) void spmm_span_kernel(const SpmmParams p) {
     constexpr int U = 4;
     extern __shared__ __align__(16) int dyn_lds[];
     __shared__ int sidx_all[4][kSpanSlots];
-    __shared__ int seid_all[KIND == KIND_WEIGHTED ? 4 : 1][KIND == KIND_WEIGHTED ? kSpanSlots : 1];
+    __shared__ int seid_all[weighted(KIND) ? 4 : 1][weighted(KIND) ? kSpanSlots : 1];
     __shared__ int rowof_all[4][kSpanSlots];
     __shared__ unsigned maskw_all[4][12];
     const int lane = lane_id();
@@ -736,10 +740,10 @@ __global__ __launch_bounds__(256) void spmm_span_kernel(const SpmmParams p) {
     int* accbuf = dyn_lds + wave * span_wave_ints(p.lpe_log2, VEC);
     int64_t* win = reinterpret_cast<int64_t*>(accbuf);  // only while the row structure is built
     int* sidx = sidx_all[wave];
-    int* seid = seid_all[KIND == KIND_WEIGHTED ? wave : 0];
+    int* seid = seid_all[weighted(KIND) ? wave : 0];
     int* rowof = rowof_all[wave];
     unsigned* maskw = maskw_all[wave];
-    const bool permuted = KIND == KIND_WEIGHTED && p.edge_ids;
+    const bool permuted = weighted(KIND) && p.edge_ids;
     const int64_t base = w * kSpanSlots;
     const int endl = static_cast<int>(p.nnz - base < kSpanSlots ? p.nnz - base : kSpanSlots);
     const int64_t end = base + endl;
@@ -901,9 +905,9 @@ __global__ __launch_bounds__(256) void spmm_span_kernel(const SpmmParams p) {
             const int sl = ok ? slot : 0;  // slot 0 exists; its multiplier is 0 here
             d[u] = Gather<VEC>::load(c.fcol + row_offset(sidx[sl], p));
             uint32_t wv = 1u;
-            if (KIND == KIND_WEIGHTED) {
+            if (weighted(KIND)) {
                 const int64_t pos = permuted ? static_cast<int64_t>(seid[sl]) : base + sl;
-                wv = edge_value(p, c, pos);
+                wv = edge_value<KIND>(p, c, pos);
             }
             m |= (ok ? wv : 0u) << (8 * u);
         }
@@ -1246,6 +1250,7 @@ static int spmm_u_mul_e_common(float* out, const int64_t* indptr, const void* in
         if ((F & 15) == 0 && (a & 15) == 0) vec = 16;
         else if ((F & 3) == 0 && (a & 3) == 0) vec = 4;
     }
+    if (evals_f32) return launch_spmm<KIND_WEIGHTED_F32>(p, vec, as_stream(stream));
     return launch_spmm<KIND_WEIGHTED>(p, vec, as_stream(stream));
 }
 
