@@ -101,12 +101,12 @@ __global__ __launch_bounds__(256) void absmax_rowmul_dense_kernel(const float* _
         if (col >= cols) { col -= cols; ++row; }
     };
     int64_t i = tid;
-    for (; i + 3 * nthr < n4; i += 4 * nthr) {
-        const f32x4 a = __builtin_nontemporal_load(x4 + i);
-        const f32x4 b = __builtin_nontemporal_load(x4 + i + nthr);
-        const f32x4 c = __builtin_nontemporal_load(x4 + i + 2 * nthr);
-        const f32x4 d = __builtin_nontemporal_load(x4 + i + 3 * nthr);
-        take(a); take(b); take(c); take(d);
+    for (; i + 7 * nthr < n4; i += 8 * nthr) {  // eight 16-byte loads in flight per lane
+        f32x4 v[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) v[u] = __builtin_nontemporal_load(x4 + i + u * nthr);
+#pragma unroll
+        for (int u = 0; u < 8; ++u) take(v[u]);
     }
     for (; i < n4; i += nthr) take(__builtin_nontemporal_load(x4 + i));
     const int64_t t = (n4 << 2) + tid;  // at most two elements remain, in the last row
