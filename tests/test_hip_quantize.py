@@ -105,6 +105,31 @@ def test_quantize_rows_padded(K, orc):
         assert np.array_equal(host(out), orc.quantize_rows(x, s, False, ldq=ld, mode=orc.STOCHASTIC, seed=5, offset=8))
 
 
+@pytest.mark.parametrize("rows,cols", [(3001, 41), (2000, 602), (70001, 3), (1601, 41)])
+@pytest.mark.parametrize("rowmul", [False, True])
+def test_quantize_dense_rows_of_odd_width(K, orc, rows, cols, rowmul):
+    """Dense inputs whose rows do not hold a multiple of four columns, quantized into padded rows: the flat walk
+    (16-byte loads, a lane's four elements in up to two rows, one Philox block per lane) for inputs of at least
+    65,536 elements, the row-strided kernel below that; every rounding mode, the random stream at an aligned and
+    at an unaligned offset, injected noise, the row multiplier; the padding must come back as zeros."""
+    rng = np.random.default_rng(rows + cols)
+    x = (rng.standard_normal((rows, cols)) * 3).astype(np.float32)
+    rm = (rng.random(rows).astype(np.float32) + 0.5) if rowmul else None
+    s = orc.absmax_ex(x, row_mul=rm)[0] if rowmul else orc.absmax_scale(x)
+    ld = (cols + 15) // 16 * 16
+    noise = rng.random((rows, cols)).astype(np.float32)
+    cases = [("rne", {}, dict(mode=orc.RNE)), ("trunc", {}, dict(mode=orc.TRUNC)),
+             ("stochastic", dict(seed=7, offset=0), dict(mode=orc.STOCHASTIC, seed=7, offset=0)),
+             ("stochastic", dict(seed=7, offset=4 * 10 ** 6 + 5), dict(mode=orc.STOCHASTIC, seed=7, offset=4 * 10 ** 6 + 5)),
+             ("stochastic", dict(noise=dev(noise)), dict(mode=orc.STOCHASTIC, noise=noise))]
+    for mode, kw, okw in cases:
+        q, _ = K.quantize_padded(dev(x), sc(s), round_mode=mode, row_mul=None if rm is None else dev(rm), **kw)
+        want = orc.quantize_rows_ex(x, s, row_mul=rm, ldq=ld, **okw)
+        full = host(q._base) if q._base is not None else host(q)
+        assert np.array_equal(full[:, :cols], want[:, :cols]), (mode, kw.keys())
+        assert not full[:, cols:].any()
+
+
 @pytest.mark.parametrize("shape", [(1335586, 8, 1), (1001, 4, 1), (77, 2, 3), (4096, 1, 1), (5, 64, 4)])
 def test_transpose_quant(K, orc, shape):
     rng = np.random.default_rng(6)
