@@ -425,6 +425,33 @@ int tango_softmax_xent_f32(const float* logits, int64_t ld, const int64_t* label
                            int64_t classes, float* loss_out, float* grad_out, int64_t ldg,
                            void* workspace, size_t workspace_bytes, tango_stream_t stream);
 
+/* ------------------------------------------------------- batch normalisation */
+
+/* Training-mode batch normalisation over the rows of x [rows, cols] fp32 (row stride
+   cols), with the ReLU that follows it folded in (no counterpart in the reference's
+   native code: its arxiv drivers call torch.nn.BatchNorm1d and then the activation,
+   evaluation/arxiv_gat.py:376-448, evaluation/arxiv_gcn.py:156-209).
+     mean[c] = mean_r x[r, c], var[c] = mean_r (x[r, c] - mean[c])^2 (biased),
+     rstd[c] = 1 / sqrt(var[c] + eps),
+     y[r, c] = (x[r, c] - mean[c]) * (rstd[c] * gamma[c]) + beta[c], max(., 0) if relu != 0.
+   scale_y (may be NULL) receives max|y| / 127.  The backward takes the incoming gradient
+   through the ReLU (the forward's sign, recomputed from x) and returns
+     dbeta[c] = sum_r dy'[r, c], dgamma[c] = sum_r dy'[r, c] * xhat[r, c],
+     dx[r, c] = rstd[c] * gamma[c] * (dy'[r, c] - dbeta[c] / rows - xhat[r, c] * dgamma[c] / rows),
+   xhat = (x - mean) * rstd.  cols must be a multiple of 4 and at most 1024, x / y / dy / dx
+   16-byte aligned (TANGO_ERR_UNSUPPORTED otherwise).  All sums run in a fixed order.
+   workspace: tango_batchnorm_workspace(rows, cols) bytes, the same for both calls. */
+size_t tango_batchnorm_workspace(int64_t rows, int64_t cols);
+int tango_batchnorm_fwd_f32(float* y, float* mean, float* var, float* rstd, float* scale_y,
+                            const float* x, const float* gamma, const float* beta, int64_t rows,
+                            int64_t cols, float eps, int relu, void* workspace,
+                            size_t workspace_bytes, tango_stream_t stream);
+int tango_batchnorm_bwd_f32(float* dx, float* dgamma, float* dbeta, const float* dy,
+                            const float* x, const float* mean, const float* rstd,
+                            const float* gamma, const float* beta, int64_t rows, int64_t cols,
+                            int relu, void* workspace, size_t workspace_bytes,
+                            tango_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -58,6 +58,9 @@ SIGNATURES = {
     "tango_sddmm_ewise_f32q": (I, [I, P, P, P, P, P, P, P, I64, I64, I, P]),
     "tango_softmax_xent_workspace": (SZ, [I64]),
     "tango_softmax_xent_f32": (I, [P, I64, P, I64, I64, P, P, I64, P, SZ, P]),
+    "tango_batchnorm_workspace": (SZ, [I64, I64]),
+    "tango_batchnorm_fwd_f32": (I, [P, P, P, P, P, P, P, P, I64, I64, F, I, P, SZ, P]),
+    "tango_batchnorm_bwd_f32": (I, [P, P, P, P, P, P, P, P, P, I64, I64, I, P, SZ, P]),
     "tango_edge_softmax_workspace": (SZ, [I64, I64]),
     "tango_edge_softmax_fwd": (I, [P, P, P, P, I64, I64, I64, F, P, SZ, P]),
     "tango_edge_softmax_fwd_static": (I, [P, P, P, P, I64, I64, I64, F, P]),

@@ -1,0 +1,271 @@
+// Batch normalisation over the rows of a dense fp32 matrix [rows, C] (training mode: statistics of the batch),
+// with the ReLU that follows it and the scale of the result for the next quantized layer folded in.
+//
+// Not part of the reference's primitive layer: its arxiv drivers use torch.nn.BatchNorm1d followed by the
+// activation between the graph layers (evaluation/arxiv_gat.py:376-448, evaluation/arxiv_gcn.py:156-209).  On
+// [169343, 128] torch's training-mode kernels take 0.42 ms per layer and step (statistics 0.15, transform 0.03,
+// backward reduction 0.20, backward element-wise 0.04); the passes here are bound by HBM: forward = one read
+// for the statistics, one read + one write for the result; backward = two reads for the column sums, three
+// reads + one write for the input gradient.  Every reduction runs in a fixed order (register sums over a
+// thread's rows -> LDS over the workgroup's row lanes -> one partial per workgroup -> a finishing kernel), so
+// results do not depend on scheduling.
+//
+// Variance: sums of (x - k) and (x - k)^2 with k = the column's first element (the shifted-data form; the
+// plain sum of squares cancels when |mean| >> std).
+#include "common.hpp"
+
+namespace tango {
+
+constexpr int kBnMaxGroups = 512;  // workgroups (partials) of the column reductions
+
+// Thread t of 256 owns column quad t % cq and row lane t / cq (row lanes = 256 / cq; threads beyond are idle).
+// DYNAMIC LDS: 2 * row_lanes * C floats.
+// MODE 0: s1 = sum(x - k), s2 = sum((x - k)^2).
+// MODE 1: s1 = sum(dy'), s2 = sum(dy' * xhat), dy' = dy where the forward output was positive (relu) else 0.
+template <int MODE>
+__global__ __launch_bounds__(256) void bn_reduce_kernel(const float* __restrict__ x, const float* __restrict__ dy,
+                                                        const float* __restrict__ mean, const float* __restrict__ rstd,
+                                                        const float* __restrict__ gamma, const float* __restrict__ beta,
+                                                        int64_t rows, int C, int relu, float* __restrict__ partial) {
+    extern __shared__ float red[];  // [2][row_lanes][C]
+    const int cq = C >> 2;
+    const int row_lanes = 256 / cq;
+    const int quad = threadIdx.x % cq, rl = threadIdx.x / cq;
+    const bool active = rl < row_lanes;
+    const int c0 = quad << 2;
+    float k[4] = {0.f, 0.f, 0.f, 0.f}, a[4] = {0.f, 0.f, 0.f, 0.f}, b[4] = {0.f, 0.f, 0.f, 0.f}, mu[4] = {0.f, 0.f, 0.f, 0.f},
+          rs[4] = {0.f, 0.f, 0.f, 0.f};
+    if (MODE == 0) {
+        const f32x4 v = *reinterpret_cast<const f32x4*>(x + c0);
+        k[0] = v.x; k[1] = v.y; k[2] = v.z; k[3] = v.w;
+    } else {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            mu[i] = mean[c0 + i];
+            rs[i] = rstd[c0 + i];
+            a[i] = rs[i] * gamma[c0 + i];
+            b[i] = beta[c0 + i];
+        }
+    }
+    float s1[4] = {0.f, 0.f, 0.f, 0.f}, s2[4] = {0.f, 0.f, 0.f, 0.f};
+    const int64_t step = static_cast<int64_t>(gridDim.x) * row_lanes;
+    auto take = [&](const f32x4 xv, const f32x4 dv) {
+        const float xs[4] = {xv.x, xv.y, xv.z, xv.w}, ds[4] = {dv.x, dv.y, dv.z, dv.w};
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            if (MODE == 0) {
+                const float d = xs[i] - k[i];
+                s1[i] += d;
+                s2[i] += d * d;
+            } else {
+                const float c = xs[i] - mu[i];
+                float g = ds[i];
+                if (relu && !(c * a[i] + b[i] > 0.0f)) g = 0.0f;  // the forward's own arithmetic: same sign
+                s1[i] += g;
+                s2[i] += g * (c * rs[i]);
+            }
+        }
+    };
+    if (active) {
+        int64_t r = static_cast<int64_t>(blockIdx.x) * row_lanes + rl;
+        for (; r + 3 * step < rows; r += 4 * step) {  // four rows in flight per thread
+            f32x4 xv[4], dv[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                xv[u] = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(x + (r + u * step) * C + c0));
+                dv[u] = MODE == 1 ? __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(dy + (r + u * step) * C + c0))
+                                  : f32x4{0.f, 0.f, 0.f, 0.f};
+            }
+#pragma unroll
+            for (int u = 0; u < 4; ++u) take(xv[u], dv[u]);
+        }
+        for (; r < rows; r += step) {
+            const f32x4 xv = *reinterpret_cast<const f32x4*>(x + r * C + c0);
+            const f32x4 dv = MODE == 1 ? *reinterpret_cast<const f32x4*>(dy + r * C + c0) : f32x4{0.f, 0.f, 0.f, 0.f};
+            take(xv, dv);
+        }
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            red[rl * C + c0 + i] = s1[i];
+            red[(row_lanes + rl) * C + c0 + i] = s2[i];
+        }
+    }
+    __syncthreads();
+    for (int j = threadIdx.x; j < 2 * C; j += 256) {  // column j of s1 (j < C) or s2: the row lanes in order
+        const int which = j / C, c = j - which * C;
+        float t = 0.0f;
+        for (int l = 0; l < row_lanes; ++l) t += red[(which * row_lanes + l) * C + c];
+        partial[static_cast<int64_t>(blockIdx.x) * 2 * C + j] = t;
+    }
+}
+
+// Sums the partials of 16 columns (64 partial lanes each, fixed order) and finishes the statistics.
+// MODE 0: mean, biased variance, 1 / sqrt(var + eps).  MODE 1: out1 = s1 (dbeta), out2 = s2 (dgamma).
+template <int MODE>
+__global__ __launch_bounds__(1024) void bn_finish_kernel(const float* __restrict__ partial, int groups, int C, int64_t rows,
+                                                        float eps, const float* __restrict__ x, float* __restrict__ out1,
+                                                        float* __restrict__ out2, float* __restrict__ out3) {
+    __shared__ float red[2][64][16];
+    const int e = threadIdx.x & 15, sl = threadIdx.x >> 4;
+    const int c = blockIdx.x * 16 + e;
+    float t1 = 0.0f, t2 = 0.0f;
+    if (c < C)
+        for (int g = sl; g < groups; g += 64) {
+            t1 += partial[static_cast<int64_t>(g) * 2 * C + c];
+            t2 += partial[static_cast<int64_t>(g) * 2 * C + C + c];
+        }
+    red[0][sl][e] = t1;
+    red[1][sl][e] = t2;
+    __syncthreads();
+    if (sl == 0 && c < C) {
+        float s1 = 0.0f, s2 = 0.0f;
+#pragma unroll
+        for (int w = 0; w < 64; ++w) {
+            s1 += red[0][w][e];
+            s2 += red[1][w][e];
+        }
+        if (MODE == 0) {
+            const float n = static_cast<float>(rows);
+            const float m1 = s1 / n;           // mean of x - k
+            float var = s2 / n - m1 * m1;      // biased variance
+            var = var > 0.0f ? var : 0.0f;
+            out1[c] = x[c] + m1;               // k = x[0, c]
+            out2[c] = var;
+            out3[c] = 1.0f / sqrtf(var + eps);
+        } else {
+            out1[c] = s1;
+            out2[c] = s2;
+        }
+    }
+}
+
+// y = (x - mean) * (rstd * gamma) + beta, ReLU if asked; optionally max|y| / 127 into scale_out (pre-zeroed).
+// Backward (BWD): dx = (rstd * gamma) * (dy' - dbeta / n - xhat * dgamma / n).
+template <bool BWD>
+__global__ __launch_bounds__(256) void bn_apply_kernel(float* __restrict__ out, const float* __restrict__ x,
+                                                       const float* __restrict__ dy, const float* __restrict__ mean,
+                                                       const float* __restrict__ rstd, const float* __restrict__ gamma,
+                                                       const float* __restrict__ beta, const float* __restrict__ dbeta,
+                                                       const float* __restrict__ dgamma, int64_t rows, int C, int relu,
+                                                       float* __restrict__ scale_out) {
+    extern __shared__ float par[];  // [6][C]: mean, rstd, a = rstd * gamma, beta, dbeta / n, dgamma / n
+    const float inv_n = 1.0f / static_cast<float>(rows);
+    for (int c = threadIdx.x; c < C; c += 256) {
+        par[c] = mean[c];
+        par[C + c] = rstd[c];
+        par[2 * C + c] = rstd[c] * gamma[c];
+        par[3 * C + c] = beta[c];
+        par[4 * C + c] = BWD ? dbeta[c] * inv_n : 0.0f;
+        par[5 * C + c] = BWD ? dgamma[c] * inv_n : 0.0f;
+    }
+    __syncthreads();
+    const int cq = C >> 2;
+    const int64_t n4 = rows * cq;
+    const int64_t tid = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    const int64_t nthr = static_cast<int64_t>(gridDim.x) * blockDim.x;
+    int quad = static_cast<int>(tid % cq);
+    const int qstep = static_cast<int>(nthr % cq);
+    float m = 0.0f;
+    for (int64_t i = tid; i < n4; i += nthr) {
+        const int c0 = quad << 2;
+        const f32x4 xv = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(x) + i);
+        const float xs[4] = {xv.x, xv.y, xv.z, xv.w};
+        float o[4];
+        if (!BWD) {
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+                float y = (xs[k] - par[c0 + k]) * par[2 * C + c0 + k] + par[3 * C + c0 + k];
+                if (relu && !(y > 0.0f)) y = 0.0f;
+                o[k] = y;
+                m = fmaxf(m, fabsf(y));
+            }
+        } else {
+            const f32x4 dv = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(dy) + i);
+            const float ds[4] = {dv.x, dv.y, dv.z, dv.w};
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+                const float c = xs[k] - par[c0 + k];
+                float g = ds[k];
+                if (relu && !(c * par[2 * C + c0 + k] + par[3 * C + c0 + k] > 0.0f)) g = 0.0f;
+                o[k] = par[2 * C + c0 + k] * (g - par[4 * C + c0 + k] - (c * par[C + c0 + k]) * par[5 * C + c0 + k]);
+            }
+        }
+        __builtin_nontemporal_store(f32x4{o[0], o[1], o[2], o[3]}, reinterpret_cast<f32x4*>(out) + i);
+        quad += qstep;
+        if (quad >= cq) quad -= cq;
+    }
+    if (!BWD && scale_out) block_absmax_to_global(m / 127.0f, scale_out);
+}
+
+static int bn_groups(int64_t rows, int64_t C) {
+    const int64_t row_lanes = 256 / (C >> 2);
+    const int64_t g = ceil_div(rows, row_lanes * 8);  // at least eight rows per thread
+    return static_cast<int>(g < 1 ? 1 : (g < kBnMaxGroups ? g : kBnMaxGroups));
+}
+
+static bool bn_shape_ok(int64_t rows, int64_t C) { return rows > 0 && C >= 4 && C <= 1024 && (C & 3) == 0; }
+
+}  // namespace tango
+
+using namespace tango;
+
+extern "C" {
+
+size_t tango_batchnorm_workspace(int64_t rows, int64_t cols) {
+    if (!bn_shape_ok(rows, cols)) return 0;
+    return static_cast<size_t>(bn_groups(rows, cols)) * 2 * cols * sizeof(float);
+}
+
+int tango_batchnorm_fwd_f32(float* y, float* mean, float* var, float* rstd, float* scale_y, const float* x,
+                            const float* gamma, const float* beta, int64_t rows, int64_t cols, float eps, int relu,
+                            void* workspace, size_t workspace_bytes, tango_stream_t stream) {
+    if (rows < 0 || cols < 0) return TANGO_ERR_INVALID_ARG;
+    if (rows == 0 || cols == 0) return TANGO_OK;
+    if (!bn_shape_ok(rows, cols)) return TANGO_ERR_UNSUPPORTED;
+    if (!y || !mean || !var || !rstd || !x || !gamma || !beta) return TANGO_ERR_INVALID_ARG;
+    if (((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(y)) & 15) != 0) return TANGO_ERR_UNSUPPORTED;
+    const size_t need = tango_batchnorm_workspace(rows, cols);
+    if (!workspace || workspace_bytes < need || (reinterpret_cast<uintptr_t>(workspace) & 15) != 0)
+        return TANGO_ERR_WORKSPACE;
+    hipStream_t s = as_stream(stream);
+    const int C = static_cast<int>(cols);
+    const int groups = bn_groups(rows, cols);
+    const int row_lanes = 256 / (C >> 2);
+    float* partial = static_cast<float*>(workspace);
+    if (scale_y) fill_u32(scale_y, 0u, 1, s);
+    hipLaunchKernelGGL(bn_reduce_kernel<0>, dim3(groups), dim3(256), sizeof(float) * 2 * row_lanes * C, s, x, nullptr,
+                       nullptr, nullptr, nullptr, nullptr, rows, C, 0, partial);
+    hipLaunchKernelGGL(bn_finish_kernel<0>, dim3((C + 15) / 16), dim3(1024), 0, s, partial, groups, C, rows, eps, x, mean,
+                       var, rstd);
+    hipLaunchKernelGGL(bn_apply_kernel<false>, dim3(grid_for(rows * (cols >> 2), 256)), dim3(256), sizeof(float) * 6 * C, s,
+                       y, x, nullptr, mean, rstd, gamma, beta, nullptr, nullptr, rows, C, relu, scale_y);
+    return launch_status();
+}
+
+int tango_batchnorm_bwd_f32(float* dx, float* dgamma, float* dbeta, const float* dy, const float* x,
+                            const float* mean, const float* rstd, const float* gamma, const float* beta, int64_t rows,
+                            int64_t cols, int relu, void* workspace, size_t workspace_bytes, tango_stream_t stream) {
+    if (rows < 0 || cols < 0) return TANGO_ERR_INVALID_ARG;
+    if (rows == 0 || cols == 0) return TANGO_OK;
+    if (!bn_shape_ok(rows, cols)) return TANGO_ERR_UNSUPPORTED;
+    if (!dx || !dgamma || !dbeta || !dy || !x || !mean || !rstd || !gamma || !beta) return TANGO_ERR_INVALID_ARG;
+    if (((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(dy) | reinterpret_cast<uintptr_t>(dx)) & 15) != 0)
+        return TANGO_ERR_UNSUPPORTED;
+    const size_t need = tango_batchnorm_workspace(rows, cols);
+    if (!workspace || workspace_bytes < need || (reinterpret_cast<uintptr_t>(workspace) & 15) != 0)
+        return TANGO_ERR_WORKSPACE;
+    hipStream_t s = as_stream(stream);
+    const int C = static_cast<int>(cols);
+    const int groups = bn_groups(rows, cols);
+    const int row_lanes = 256 / (C >> 2);
+    float* partial = static_cast<float*>(workspace);
+    hipLaunchKernelGGL(bn_reduce_kernel<1>, dim3(groups), dim3(256), sizeof(float) * 2 * row_lanes * C, s, x, dy, mean,
+                       rstd, gamma, beta, rows, C, relu, partial);
+    hipLaunchKernelGGL(bn_finish_kernel<1>, dim3((C + 15) / 16), dim3(1024), 0, s, partial, groups, C, rows, 0.0f, x,
+                       dbeta, dgamma, nullptr);
+    hipLaunchKernelGGL(bn_apply_kernel<true>, dim3(grid_for(rows * (cols >> 2), 256)), dim3(256), sizeof(float) * 6 * C, s,
+                       dx, x, dy, mean, rstd, gamma, beta, dbeta, dgamma, rows, C, relu, nullptr);
+    return launch_status();
+}
+
+}  // extern "C"

@@ -10,6 +10,7 @@ import torch.nn.functional as F
 from torch.autograd.function import Function, once_differentiable
 
 from .QLinear import QLinear, Qlinear_func_reduce, shared_input_linears
+from .batchnorm import BatchNorm1dAct
 from .kernels import cuda_kernels, refuse_capture
 from .SDDMM import sddmm_u_add_v, sddmm_u_dot_v
 from .SPMM import spmm_u_mul_e
@@ -92,7 +93,13 @@ class QGATConv(nn.Module):
                 raise Exception("There are 0-in-degree nodes in the graph.")
         n = feat.size(0)
         h = self.feat_drop(feat).contiguous()
-        feat_src, s_feat = self.fc(h)
+        res = None
+        if isinstance(self.res_fc, QLinear) and h.dim() == 2:
+            # the projection and the residual projection read the same input: quantized once, and their two
+            # input gradients land in one tensor
+            (feat_src, s_feat), (res, _) = shared_input_linears(h, [self.fc, self.res_fc])
+        else:
+            feat_src, s_feat = self.fc(h)
         feat_src = feat_src.view(n, self._num_heads, self._out_feats)
         el, er, s_el, s_er = attn_scores.apply(feat_src, self.attn_l, self.attn_r)  # test_gat.py:135-137
         s_a = None
@@ -113,7 +120,7 @@ class QGATConv(nn.Module):
             fold_act = "elu" if self.activation is F.elu else "relu" if self.activation in (F.relu, torch.relu) else None
         rst = spmm_u_mul_e.apply(graph, feat_src, a, self.bias if fold_bias else None, s_feat, fold_act, s_a)  # :151
         if self.res_fc is not None:
-            rst = rst + self.res_fc(h).view(n, -1, self._out_feats)
+            rst = rst + (self.res_fc(h) if res is None else res).view(n, -1, self._out_feats)
         if self.bias is not None and not fold_bias:
             rst = rst + self.bias.view(1, self._num_heads, self._out_feats)
         if self.activation and fold_act is None:
@@ -229,12 +236,18 @@ class ArxivGATConv(nn.Module):
             assert not zero_in
         n = feat.size(0)
         h = self.feat_drop(feat).contiguous()
+        res = None
         if self._use_symmetric_norm:  # :158-163; the product is a new tensor, so the epilogue's scale does not apply
             self.fc.isReduce = False
             feat_src = self.fc(h).view(n, self._num_heads, self._out_feats)
             self.fc.isReduce = True
             s_feat = None
             feat_src = feat_src * graph.out_degrees().float().clamp(min=1).pow(-0.5).view(n, 1, 1)
+        elif self.res_fc is not None and h.dim() == 2:
+            # the projection and the residual projection read the same input: quantized once, and their two
+            # input gradients land in one tensor
+            (feat_src, s_feat), (res, _) = shared_input_linears(h, [self.fc, self.res_fc])
+            feat_src = feat_src.view(n, self._num_heads, self._out_feats)
         else:
             feat_src, s_feat = self.fc(h)
             feat_src = feat_src.view(n, self._num_heads, self._out_feats)
@@ -254,7 +267,7 @@ class ArxivGATConv(nn.Module):
         if self._use_symmetric_norm:  # :203-208
             rst = rst * graph.in_degrees().float().clamp(min=1).pow(0.5).view(n, 1, 1)
         if self.res_fc is not None:  # :211-214
-            rst = rst + self.res_fc(h).view(n, -1, self._out_feats)
+            rst = rst + (self.res_fc(h) if res is None else res).view(n, -1, self._out_feats)
         if self._activation is not None:
             rst = self._activation(rst)
         return rst
@@ -278,7 +291,7 @@ class ArxivGAT(nn.Module):
                                            edge_drop=edge_drop, use_attn_dst=use_attn_dst,
                                            use_symmetric_norm=use_symmetric_norm, residual=True))
             if i < n_layers - 1:
-                self.norms.append(nn.BatchNorm1d(n_heads * out_hidden))
+                self.norms.append(BatchNorm1dAct(n_heads * out_hidden, activation=activation))
         self.bias_last = nn.Parameter(torch.zeros(n_classes))  # ElementWiseLinear(weight=False, bias=True), :28-58
         self.input_drop, self.dropout = nn.Dropout(input_drop), nn.Dropout(dropout)
         self.activation = activation
@@ -288,7 +301,7 @@ class ArxivGAT(nn.Module):
         for i in range(self.n_layers):
             h = self.convs[i](graph, h)
             if i < self.n_layers - 1:
-                h = self.dropout(self.activation(self.norms[i](h.flatten(1))))
+                h = self.dropout(self.norms[i](h.flatten(1)))  # normalisation + activation in one module
         return h.mean(1) + self.bias_last
 
 

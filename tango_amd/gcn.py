@@ -5,6 +5,7 @@ import torch
 import torch.nn as nn
 
 from .QLinear import Qlinear_func, Qlinear_func_reduce
+from .batchnorm import BatchNorm1dAct
 from .SPMM import spmm_copy_u
 
 
@@ -104,7 +105,7 @@ class ArxivGCN(nn.Module):
             if use_linear:
                 self.linear.append(QLinear(in_hidden, out_hidden, bias=False))
             if i < n_layers - 1:
-                self.norms.append(nn.BatchNorm1d(out_hidden))
+                self.norms.append(BatchNorm1dAct(out_hidden, activation=activation))
         self.input_drop, self.dropout = nn.Dropout(min(0.1, dropout)), nn.Dropout(dropout)
         self.activation = activation
 
@@ -115,5 +116,5 @@ class ArxivGCN(nn.Module):
             conv = self.convs[i](graph, h, norms)
             h = conv + self.linear[i](h) if self.use_linear else conv
             if i < self.n_layers - 1:
-                h = self.dropout(self.activation(self.norms[i](h)))
+                h = self.dropout(self.norms[i](h))  # normalisation + activation in one module
         return h

@@ -460,3 +460,122 @@ def test_shared_input_linears_with_a_second_layer(M, Kd, N, N2):
     assert torch.equal(x.grad, want_dx)
     for p in params:
         assert torch.equal(p.grad, want_dp[id(p)])
+
+
+def _bn_f64(x, gamma, beta, eps, relu, dy=None, mask=None):
+    """Training-mode batch normalisation (+ ReLU) and its gradients in float64: the textbook formulas.  ``mask``:
+    which outputs the ReLU let through, when the caller wants the gradients for a given forward result."""
+    x, gamma, beta = x.astype(np.float64), gamma.astype(np.float64), beta.astype(np.float64)
+    n = x.shape[0]
+    mean, var = x.mean(0), x.var(0)
+    rstd = 1.0 / np.sqrt(var + eps)
+    xhat = (x - mean) * rstd
+    y = xhat * gamma + beta
+    out = {"mean": mean, "var": var, "y": np.maximum(y, 0) if relu else y}
+    if dy is not None:
+        g = dy.astype(np.float64) * (((y > 0) if mask is None else mask) if relu else 1.0)
+        out["dbeta"], out["dgamma"] = g.sum(0), (g * xhat).sum(0)
+        out["dx"] = rstd * gamma * (g - out["dbeta"] / n - xhat * out["dgamma"] / n)
+    return out
+
+
+@pytest.mark.parametrize("rows,cols,relu", [(5000, 128, True), (169343, 128, True), (777, 768, False), (33, 4, True),
+                                            (2, 1024, True), (1001, 40, False), (4096, 256, True)])
+def test_batchnorm_act_c_abi(K, rows, cols, relu):
+    """The two entry points against float64 formulas (means far from zero, so a variance from a plain sum of
+    squares would fail), and the scale of the result against the result's own maximum."""
+    import ctypes
+    L = K._L
+    rng = np.random.default_rng(rows + cols)
+    x = (rng.standard_normal((rows, cols)) * rng.uniform(0.1, 3.0, cols) + rng.uniform(-50, 50, cols)).astype(np.float32)
+    gamma, beta = rng.uniform(0.5, 1.5, cols).astype(np.float32), rng.uniform(-0.5, 0.5, cols).astype(np.float32)
+    dy = rng.standard_normal((rows, cols)).astype(np.float32)
+    ref = _bn_f64(x, gamma, beta, 1e-5, relu, dy)
+    X, G, B, DY = dev(x), dev(gamma), dev(beta), dev(dy)
+    Y, DX = torch.empty_like(X), torch.empty_like(X)
+    st = torch.empty(3, cols, device="cuda")
+    dgb = torch.empty(2, cols, device="cuda")
+    scale = torch.full((1,), 7.0, device="cuda")
+    wsb = L.tango_batchnorm_workspace(rows, cols)
+    ws = torch.empty(wsb, dtype=torch.uint8, device="cuda")
+    stream = torch.cuda.current_stream().cuda_stream
+    assert L.tango_batchnorm_fwd_f32(Y.data_ptr(), st[0].data_ptr(), st[1].data_ptr(), st[2].data_ptr(), scale.data_ptr(),
+                                     X.data_ptr(), G.data_ptr(), B.data_ptr(), rows, cols, ctypes.c_float(1e-5), int(relu),
+                                     ws.data_ptr(), wsb, stream) == 0
+    assert L.tango_batchnorm_bwd_f32(DX.data_ptr(), dgb[0].data_ptr(), dgb[1].data_ptr(), DY.data_ptr(), X.data_ptr(),
+                                     st[0].data_ptr(), st[2].data_ptr(), G.data_ptr(), B.data_ptr(), rows, cols, int(relu),
+                                     ws.data_ptr(), wsb, stream) == 0
+    np.testing.assert_allclose(host(st[0]), ref["mean"], rtol=1e-6, atol=1e-6)
+    np.testing.assert_allclose(host(st[1]), ref["var"], rtol=2e-5, atol=1e-7)
+    # fp32 rounds the mean to its own grid: x - mean carries an absolute error of about an ulp of |x|, which the
+    # normalisation magnifies by rstd (columns whose spread is tiny beside their mean, two-row batches)
+    rstd64 = 1.0 / np.sqrt(ref["var"] + 1e-5)
+    eps_hat = 2.0 ** -22 * (np.abs(ref["mean"]) + np.abs(x).max(0)) * rstd64  # error of xhat per column
+
+    def close(actual, desired, rtol, atol):
+        bad = np.abs(actual - desired) > atol + rtol * np.abs(desired)
+        assert not bad.any(), (int(bad.sum()), float(np.abs(actual - desired).max()))
+
+    close(host(Y), ref["y"], 1e-5, 1e-5 + eps_hat * gamma)
+    assert scale.item() == (Y.abs().max() / 127.0).item()
+    # gradients: through the fp32 result's own ReLU mask (the few elements at y ~ 0 differ from float64's)
+    if relu:
+        assert ((host(Y) > 0) == (ref["y"] > 0)).mean() > 0.999
+        ref = _bn_f64(x, gamma, beta, 1e-5, relu, dy, mask=host(Y) > 0)
+    close(host(dgb[1]), ref["dbeta"], 1e-4, 1e-4 * np.sqrt(rows))
+    close(host(dgb[0]), ref["dgamma"], 1e-4, 1e-4 * np.sqrt(rows) + 3 * rows * eps_hat)
+    close(host(DX), ref["dx"], 1e-4, 1e-5 + rstd64 * gamma * (1e-5 + 4 * eps_hat * (np.abs(ref["dgamma"]) / rows + 1)))
+    # a second call gives the same bits (fixed summation order)
+    Y2, st2 = torch.empty_like(Y), torch.empty_like(st)
+    assert L.tango_batchnorm_fwd_f32(Y2.data_ptr(), st2[0].data_ptr(), st2[1].data_ptr(), st2[2].data_ptr(), None,
+                                     X.data_ptr(), G.data_ptr(), B.data_ptr(), rows, cols, ctypes.c_float(1e-5), int(relu),
+                                     ws.data_ptr(), wsb, stream) == 0
+    assert torch.equal(Y, Y2) and torch.equal(st, st2)
+
+
+@pytest.mark.parametrize("rows,cols,act", [(3000, 128, "relu"), (500, 64, None), (700, 36, "relu"), (900, 128, "elu"),
+                                           (400, 30, "relu")])
+def test_batchnorm_module_matches_torch(rows, cols, act):
+    """The module against torch.nn.BatchNorm1d + activation: outputs, gradients, running statistics over two
+    training steps, the evaluation-mode pass and the state dict."""
+    from tango_amd.batchnorm import BatchNorm1dAct
+    fn = {"relu": torch.relu, "elu": torch.nn.functional.elu, None: None}[act]
+    torch.manual_seed(rows)
+    a = BatchNorm1dAct(cols, activation=fn).cuda()
+    b = torch.nn.BatchNorm1d(cols).cuda()
+    with torch.no_grad():
+        a.weight.uniform_(0.5, 1.5)
+        a.bias.uniform_(-0.5, 0.5)
+    b.load_state_dict(a.state_dict())
+    for step in range(2):
+        x = torch.randn(rows, cols, device="cuda") * 2 + 1
+        xa, xb = x.clone().requires_grad_(True), x.clone().requires_grad_(True)
+        ya = a(xa)
+        yb = b(xb) if fn is None else fn(b(xb))
+        assert torch.allclose(ya, yb, rtol=1e-5, atol=1e-5)
+        w = torch.randn_like(ya)
+        (ya * w).sum().backward()
+        (yb * w).sum().backward()
+        assert torch.allclose(xa.grad, xb.grad, rtol=1e-4, atol=1e-5)
+        assert torch.allclose(a.weight.grad, b.weight.grad, rtol=1e-4, atol=1e-3)
+        assert torch.allclose(a.bias.grad, b.bias.grad, rtol=1e-4, atol=1e-3)
+        assert torch.allclose(a.running_mean, b.running_mean, rtol=1e-5, atol=1e-6)
+        assert torch.allclose(a.running_var, b.running_var, rtol=1e-5, atol=1e-6)
+        assert int(a.num_batches_tracked) == int(b.num_batches_tracked) == step + 1
+        a.zero_grad(), b.zero_grad()
+    a.eval(), b.eval()
+    x = torch.randn(50, cols, device="cuda")
+    yb = b(x) if fn is None else fn(b(x))
+    assert torch.allclose(a(x), yb, rtol=1e-6, atol=1e-6)
+    assert a.state_dict().keys() == b.state_dict().keys()
+
+
+def test_batchnorm_rejects_unsupported_shapes(K):
+    L = K._L
+    assert L.tango_batchnorm_workspace(100, 6) == 0 and L.tango_batchnorm_workspace(100, 2048) == 0
+    x = torch.zeros(100, 6, device="cuda")
+    p = x.data_ptr()
+    import ctypes
+    assert L.tango_batchnorm_fwd_f32(p, p, p, p, None, p, p, p, 100, 6, ctypes.c_float(1e-5), 1, p, 1 << 20, None) == -2
+    assert L.tango_batchnorm_fwd_f32(p, p, p, p, None, p, p, p, 100, 8, ctypes.c_float(1e-5), 1, None, 0, None) == -4
+    assert L.tango_batchnorm_fwd_f32(p, p, p, p, None, p, p, p, 0, 8, ctypes.c_float(1e-5), 1, None, 0, None) == 0
