@@ -336,35 +336,58 @@ class HeteroHGTLayer(nn.Module):
         return torch.cat([layers[t](h[self.bounds[t]:self.bounds[t + 1]]) for t in range(len(layers))])
 
     def forward(self, g, h):
-        n, H, dk = h.size(0), self.n_heads, self.d_k
-        k, q, v = self._typed(self.k_linear, h), self._typed(self.q_linear, h), self._typed(self.v_linear, h)
-        q = q.view(n, H, dk)
-        contiguous = all(getattr(gr, "edge_range", None) is not None for gr in self.rels)
-        t = None if contiguous else h.new_zeros((g.num_edges(), H, 1))
-        vr, parts = [], []
-        for r, gr in enumerate(self.rels):
-            lo, hi = (0, n) if gr.src_type is None else (self.bounds[gr.src_type], self.bounds[gr.src_type + 1])
-            # relation-specific key and message of the relation's source type; other rows stay zero (no edge of
-            # this relation starts there)
-            kr = torch.zeros_like(k)
-            kr[lo:hi] = self.attn_linear[r](k[lo:hi])
-            vv = torch.zeros_like(v)
-            vv[lo:hi] = self.msg_linear[r](v[lo:hi])
-            vr.append(vv.view(n, H, dk))
-            tr = sddmm_u_dot_v.apply(gr, kr.view(n, H, dk), q, None, None, 1.0 / self.sqrt_dk)
-            if contiguous:
-                parts.append(tr)
-            else:
-                t = t.index_copy(0, gr.eids, tr)
-        if contiguous:  # relations own consecutive edge-id ranges, in order: the scores are their concatenation
-            t = torch.cat(parts)
-        attn = edge_softmax(g, t)  # over every in-edge of a destination, all relations together
-        out = None
-        for r, gr in enumerate(self.rels):
-            ar = attn[gr.edge_range[0]:gr.edge_range[1]] if contiguous else attn[gr.eids]
-            o = spmm_u_mul_e.apply(gr, vr[r], ar)
-            out = o if out is None else out + o
-        return self._typed(self.a_linear, out.reshape(n, self.out_dim))
+        H, dk, nt = self.n_heads, self.d_k, len(self.bounds) - 1
+        # k / v / q per node type: the type's rows are quantized once for the three projections, whose input
+        # gradients land in one tensor
+        k, v, q = [], [], []
+        for t in range(nt):
+            kt, vt, qt = shared_input_linears(h[self.bounds[t]:self.bounds[t + 1]],
+                                              (self.k_linear[t], self.v_linear[t], self.q_linear[t]))
+            k.append(kt), v.append(vt), q.append(qt)
+        # every relation runs on its own bipartite graph(s), each endpoint numbered inside its node type: no
+        # tensor here has rows for nodes the relation does not touch
+        units = [(r, part) for r, gr in enumerate(self.rels) for part in gr.parts]
+        # relation-specific keys and messages; the relations that start at one node type share that type's
+        # k (v) quantized once
+        kr, vr = {}, {}
+        for t in range(nt):
+            rs = sorted({r for r, part in units if part.src_type == t})
+            if not rs:
+                continue
+            for r, pair in zip(rs, shared_input_linears(k[t][0], [self.attn_linear[r] for r in rs], k[t][1])):
+                kr[t, r] = pair
+            for r, pair in zip(rs, shared_input_linears(v[t][0], [self.msg_linear[r] for r in rs], v[t][1])):
+                vr[t, r] = pair
+        scores = []
+        for r, part in units:
+            (U, sU), (V, sV) = kr[part.src_type, r], q[part.dst_type]
+            scores.append(sddmm_u_dot_v.apply(part, U.view(-1, H, dk), V.view(-1, H, dk), sU, sV, 1.0 / self.sqrt_dk))
+        ranges = [part.edge_range for _, part in units]
+        contiguous = all(rg is not None for rg in ranges)
+        if contiguous:
+            order = sorted(range(len(units)), key=lambda i: ranges[i][0])
+            ends = [0] + [ranges[i][1] for i in order]
+            contiguous = all(ranges[i][0] == e for i, e in zip(order, ends)) and ends[-1] == g.num_edges()
+        if contiguous:  # the parts own consecutive edge-id ranges: the scores are their concatenation
+            t = torch.cat([scores[i] for i in order])
+        else:
+            t = h.new_zeros((g.num_edges(), H, 1))
+            for (_, part), tr in zip(units, scores):
+                t = t.index_copy(0, part.eids, tr)
+        # over every in-edge of a destination, all relations together; the kernel also finds max(attn) / 127
+        attn, s_attn = edge_softmax(g, t, want_scale=True)
+        out = [None] * nt
+        for r, part in units:
+            ar = attn[part.edge_range[0]:part.edge_range[1]] if contiguous else attn[part.eids]
+            M, sM = vr[part.src_type, r]
+            o = spmm_u_mul_e.apply(part, M.view(-1, H, dk), ar, None, sM, None, s_attn)
+            out[part.dst_type] = o if out[part.dst_type] is None else out[part.dst_type] + o
+        res = []
+        for t in range(nt):
+            m = self.bounds[t + 1] - self.bounds[t]
+            o = h.new_zeros((m, self.out_dim)) if out[t] is None else out[t].reshape(m, self.out_dim)
+            res.append(self.a_linear[t](o))
+        return torch.cat(res)
 
 
 def relation_major(g, edge_type):
@@ -383,26 +406,46 @@ def relation_graphs(g, edge_type, relations, type_sizes):
     """Per relation id in ``edge_type`` ([E], ids 0 .. len(relations) where the last id marks self loops) a
     preprocessed Graph over all nodes of ``g`` with that relation's edges, ``eids`` (their ids in ``g``),
     ``edge_range`` ((first, last + 1) when those ids are consecutive and the relations come in order, as after
-    ``relation_major``; else None) and ``src_type`` attached."""
+    ``relation_major``; else None), ``src_type`` and ``parts`` attached.  ``parts``: the same edges as bipartite
+    graphs, one per (source type, destination type) pair that occurs, each endpoint numbered inside its node
+    type, with ``src_type``, ``dst_type``, ``eids`` and ``edge_range`` of their own: what the layer runs on."""
     from .graph import Graph
     from .util import graph_preprocess
     src, dst = g.edges()
+    bounds = [0]
+    for m in type_sizes:
+        bounds.append(bounds[-1] + m)
+    edges_of = torch.tensor(bounds[1:], device=src.device)
     out, nxt, in_order = [], 0, True
     for r in range(len(relations) + 1):
         eids = torch.nonzero(edge_type == r).flatten()
         if eids.numel() == 0:
             continue
-        gr = graph_preprocess(Graph(src[eids], dst[eids], g.num_nodes()))
+        rs, rd = src[eids], dst[eids]
+        gr = graph_preprocess(Graph(rs, rd, g.num_nodes()))
         gr.eids = eids
         lo, hi = int(eids[0]), int(eids[-1]) + 1
         in_order = in_order and lo == nxt and hi - lo == eids.numel()
         gr.edge_range = (lo, hi)
         nxt = hi
         gr.src_type = relations[r][0] if r < len(relations) else None  # self loops start at every type
+        ts, td = torch.bucketize(rs, edges_of, right=True), torch.bucketize(rd, edges_of, right=True)
+        pair = ts * len(type_sizes) + td
+        gr.parts = []
+        for code in torch.unique(pair).tolist():
+            a, b = divmod(code, len(type_sizes))
+            sub = torch.nonzero(pair == code).flatten()
+            part = graph_preprocess(Graph(rs[sub] - bounds[a], rd[sub] - bounds[b], type_sizes[a], type_sizes[b]))
+            part.src_type, part.dst_type, part.eids = a, b, eids[sub]
+            plo, phi = int(part.eids[0]), int(part.eids[-1]) + 1
+            part.edge_range = (plo, phi) if phi - plo == sub.numel() else None
+            gr.parts.append(part)
         out.append(gr)
     if not in_order or nxt != g.num_edges():
         for gr in out:
             gr.edge_range = None
+            for part in gr.parts:
+                part.edge_range = None
     return out
 
 

@@ -22,14 +22,17 @@ def _compress(rows, cols, num_nodes):
 
 
 class Graph:
-    """Homogeneous directed multigraph on ``num_nodes`` nodes; edge e is (src[e], dst[e])."""
+    """Homogeneous directed multigraph on ``num_nodes`` nodes; edge e is (src[e], dst[e]).  With ``num_dst``
+    the graph is bipartite: sources are numbered 0 .. num_nodes - 1, destinations 0 .. num_dst - 1 in a space
+    of their own (one relation of a heterogeneous graph, each endpoint numbered inside its node type)."""
 
     is_block = False
 
-    def __init__(self, src, dst, num_nodes):
+    def __init__(self, src, dst, num_nodes, num_dst=None):
         self._src = src.to(torch.int64).contiguous()
         self._dst = dst.to(torch.int64).contiguous()
         self._n = int(num_nodes)
+        self._n_dst = self._n if num_dst is None else int(num_dst)
         self.ndata, self.edata = {}, {}
         self.srcdata = self.dstdata = self.ndata
         self._csr = self._csc = None
@@ -41,14 +44,23 @@ class Graph:
         return self._src.device
 
     def to(self, device):
-        g = Graph(self._src.to(device), self._dst.to(device), self._n)
+        g = Graph(self._src.to(device), self._dst.to(device), self._n, self._n_dst)
         return g
 
     def num_nodes(self):
+        if self._n_dst != self._n:
+            raise ValueError("bipartite graph: ask for num_src_nodes() or num_dst_nodes()")
         return self._n
 
+    def num_src_nodes(self):
+        return self._n
+
+    def num_dst_nodes(self):
+        return self._n_dst
+
     number_of_nodes = num_nodes
-    number_of_dst_nodes = num_nodes
+    number_of_src_nodes = num_src_nodes
+    number_of_dst_nodes = num_dst_nodes
 
     def num_edges(self):
         return self._src.numel()
@@ -66,7 +78,7 @@ class Graph:
             return self._csr
         if fmt == "csc":
             if self._csc is None:
-                self._csc = _compress(self._dst, self._src, self._n)
+                self._csc = _compress(self._dst, self._src, self._n_dst)
             return self._csc
         raise ValueError("format must be 'csr' or 'csc'")
 
@@ -108,7 +120,7 @@ class Graph:
         per-edge input (GAT, HGT) give the same node outputs on either numbering; per-edge inputs
         must be permuted with ``edge_order`` first."""
         order = self.adj_sparse("csc")[2]
-        g = Graph(self._src[order], self._dst[order], self._n)
+        g = Graph(self._src[order], self._dst[order], self._n, self._n_dst)
         g.edge_order = order
         return g
 

@@ -89,3 +89,41 @@ def test_backward_passes_refuse_graph_capture(monkeypatch):
                       (spmm_copy_u, 1), (spmm_u_mul_e, 1), (_EdgeSoftmax, 1), (attn_scores, 2), (_SoftmaxXent, 1)):
         with pytest.raises(RuntimeError, match="HIP graph"):
             fn.backward(object(), *([None] * nargs))  # refuses before it looks at its context
+
+
+def test_bipartite_graph_formats():
+    """A bipartite Graph (sources and destinations numbered in spaces of their own): its compressed formats are
+    those of the square graph on max(n_src, n_dst) nodes cut to their own row counts, and the relation parts of
+    a heterogeneous graph put every edge in exactly one part with endpoints inside the part's node types.
+    Host tensors only."""
+    import numpy as np
+    import torch
+    from tango_amd.graph import Graph, hetero_power_law
+    rng = np.random.default_rng(4)
+    ns, nd, E = 7, 19, 60
+    src, dst = rng.integers(0, ns, E), rng.integers(0, nd, E)
+    g = Graph(torch.from_numpy(src), torch.from_numpy(dst), ns, nd)
+    sq = Graph(torch.from_numpy(src), torch.from_numpy(dst), nd)
+    assert (g.num_src_nodes(), g.num_dst_nodes(), g.num_edges()) == (ns, nd, E)
+    import pytest
+    with pytest.raises(ValueError):
+        g.num_nodes()
+    ip, ix, eid = g.adj_sparse("csr")
+    sip, six, seid = sq.adj_sparse("csr")
+    assert ip.numel() == ns + 1 and torch.equal(ip, sip[:ns + 1]) and torch.equal(ix, six) and torch.equal(eid, seid)
+    ip, ix, eid = g.adj_sparse("csc")
+    assert ip.numel() == nd + 1 and all(torch.equal(a, b) for a, b in zip((ip, ix, eid), sq.adj_sparse("csc")))
+    assert torch.equal(g.in_degrees(), torch.bincount(torch.from_numpy(dst), minlength=nd))
+    assert torch.equal(g.out_degrees(), torch.bincount(torch.from_numpy(src), minlength=ns))
+    g2 = g.reorder_edges_by_dst()
+    assert g2.num_dst_nodes() == nd and bool((g2.edges()[1][1:] >= g2.edges()[1][:-1]).all())
+    # the generator's heterogeneous graph, cut into parts the way relation_graphs does (that function itself
+    # builds the device-side formats and needs the library)
+    sizes, rels = (30, 20, 10), ((0, 1), (1, 0), (1, 2), (2, 0))
+    hg, node_type, edge_type = hetero_power_law(type_sizes=sizes, relations=rels, edges_per_relation=100)
+    bounds = np.cumsum((0,) + sizes)
+    s, d = (t.numpy() for t in hg.edges())
+    for r, (a, b) in enumerate(rels):
+        m = edge_type.numpy() == r
+        assert (node_type.numpy()[s[m]] == a).all() and (node_type.numpy()[d[m]] == b).all()
+        assert s[m].min() >= bounds[a] and s[m].max() < bounds[a + 1] and d[m].max() < bounds[b + 1]

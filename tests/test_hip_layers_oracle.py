@@ -270,7 +270,27 @@ def _fp32_hetero_hgt(layer, g, h):
     return typed(layer.a_linear, agg.reshape(n, H * dk))
 
 
-def test_hetero_hgt_layer_tracks_fp32_and_trains():
+def _bipartite_primitives_match_oracle(part, orc):
+    """SDDMM dot and the u_mul_e aggregation in both directions on a bipartite graph, against the oracle."""
+    from tango_amd import kernels as K
+    from gpu_util import dev, host, sc
+    ns, nd, E, H, D = part.num_src_nodes(), part.num_dst_nodes(), part.num_edges(), 4, 16
+    rng = np.random.default_rng(21)
+    U, V = (rng.integers(-127, 128, (m, H, D)).astype(np.int8) for m in (ns, nd))
+    src, dst = host(part.coo[0]), host(part.coo[1])
+    t, _ = K.mySDDMM_int8(part, "dot", dev(U), dev(V), sc(3e-3), sc(2e-3), False)
+    want, _ = orc.sddmm_dot(src, dst, U, V, 3e-3, 2e-3)
+    assert np.array_equal(host(t).reshape(E, H), want)
+    a = rng.integers(0, 128, (E, H, 1)).astype(np.int8)
+    for reverse, feat, rows in ((False, U, nd), (True, V, ns)):
+        agg = K.multi_cusparse_SPMM(part, dev(feat), dev(a), sc(1e-3), reverse, edge_major=True, scale2=sc(0.5))
+        assert agg.shape == (rows, H, D)
+        ip, ix, eid = (host(x) for x in (part.adj_csr if reverse else part.adj_csc))
+        want = orc.spmm_csr_u_mul_e_ex(ip, ix, eid, feat, a, 1e-3, scale2=0.5, edge_major=True)
+        assert np.array_equal(host(agg), want), reverse
+
+
+def test_hetero_hgt_layer_tracks_fp32_and_trains(orc):
     """Weights per node type and per relation: the quantized layer stays within int8 noise of the same math in
     fp32, every typed and relation-specific parameter receives a gradient, and a relation's weights do not
     influence destinations that relation does not reach."""
@@ -291,6 +311,16 @@ def test_hetero_hgt_layer_tracks_fp32_and_trains():
     rg = relation_graphs(g, edge_type, rels, sizes)
     assert len(rg) == 5 and sum(r.num_edges() for r in rg) == g.num_edges()
     assert all(r.edge_range is not None and r.csc_slots_are_edge_ids for r in rg)
+    # what the layer runs on: bipartite parts, endpoints numbered inside their node types
+    assert [len(r.parts) for r in rg] == [1, 1, 1, 1, 3]
+    assert [(p.src_type, p.dst_type) for r in rg for p in r.parts] == list(rels) + [(0, 0), (1, 1), (2, 2)]
+    assert sum(p.num_edges() for r in rg for p in r.parts) == g.num_edges()
+    assert all(p.edge_range is not None and p.csc_slots_are_edge_ids for r in rg for p in r.parts)
+    assert all(p.edge_range is None for r in rg_any for p in r.parts)
+    part = rg[3].parts[0]  # type 2 -> type 0: 600 sources, 3000 destinations
+    assert (part.num_src_nodes(), part.num_dst_nodes()) == (sizes[2], sizes[0])
+    assert torch.equal(part.coo[0] + sizes[0] + sizes[1], rg[3].coo[0]) and torch.equal(part.coo[1], rg[3].coo[1])
+    _bipartite_primitives_match_oracle(part, orc)
     torch.manual_seed(9)
     layer = HeteroHGTLayer(64, 64, 4, sizes, rg).cuda()
     h = torch.randn(g.num_nodes(), 64, device="cuda", requires_grad=True)
@@ -308,6 +338,14 @@ def test_hetero_hgt_layer_tracks_fp32_and_trains():
     assert bool(torch.isfinite(h.grad).all())
     for name, p in layer.named_parameters():
         assert p.grad is not None and float(p.grad.abs().sum()) > 0, name
+    # the gradients track those of the fp32 math (int8 noise of the gradient quantizers on top of the forward's)
+    h2 = h.detach().clone().requires_grad_(True)
+    names, params = zip(*layer.named_parameters())
+    want = torch.autograd.grad(_fp32_hetero_hgt(layer, g, h2).square().mean(), (h2,) + params)
+    rel = lambda a, b: ((a - b).norm() / b.norm()).item()
+    assert rel(h.grad, want[0]) < 0.15, rel(h.grad, want[0])
+    for name, p, w in zip(names, params, want[1:]):
+        assert rel(p.grad, w) < 0.25, (name, rel(p.grad, w))
     # relation 2 goes from type 1 to type 2: changing its message weights moves type-2 rows only
     with torch.no_grad():
         layer.msg_linear[2].weight.mul_(1.5)
