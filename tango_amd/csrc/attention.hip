@@ -133,6 +133,68 @@ __global__ __launch_bounds__(256) void attn_scores_bwd_kernel(
     }
 }
 
+// The same sums and products with the rows read the way they lie in memory: thread t owns VEC consecutive
+// columns (of the H * D of a row; VEC = 4 needs D % 4 == 0 so that they share a head) and row lane t / cg of
+// blockDim.x / cg, cg = H * D / VEC column groups: a wavefront's loads and stores cover consecutive bytes,
+// where a thread per (row, head) reads D floats at a stride of D floats.  Same partials layout.
+// DYNAMIC LDS: 2 * row_lanes * H * D floats.
+template <int VEC>
+__global__ __launch_bounds__(256) void attn_scores_bwd_rows_kernel(
+    float* __restrict__ dfeat, float* __restrict__ part, const float* __restrict__ del,
+    const float* __restrict__ der, const float* __restrict__ feat, const float* __restrict__ al,
+    const float* __restrict__ ar, int64_t n, int H, int D) {
+    extern __shared__ float red_rows[];  // [2][row_lanes][C]
+    const int C = H * D;
+    const int cg = C / VEC;
+    const int row_lanes = 256 / cg;
+    const int grp = threadIdx.x % cg, rl = threadIdx.x / cg;
+    const int c0 = grp * VEC;
+    const int h = c0 / D;
+    float wl[VEC], wr[VEC], accl[VEC], accr[VEC];
+#pragma unroll
+    for (int k = 0; k < VEC; ++k) {
+        wl[k] = al[c0 + k];
+        wr[k] = ar[c0 + k];
+        accl[k] = accr[k] = 0.0f;
+    }
+    if (rl < row_lanes) {
+        const int64_t step = static_cast<int64_t>(gridDim.x) * row_lanes;
+        for (int64_t r = static_cast<int64_t>(blockIdx.x) * row_lanes + rl; r < n; r += step) {
+            const float gl = del[r * H + h], gr = der[r * H + h];
+            float x[VEC], y[VEC];
+            if (VEC == 4) {
+                const f32x4 v = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(feat + r * C + c0));
+                x[0] = v.x; x[1] = v.y; x[2] = v.z; x[3] = v.w;
+            } else {
+                x[0] = feat[r * C + c0];
+            }
+#pragma unroll
+            for (int k = 0; k < VEC; ++k) {
+                y[k] = gl * wl[k] + gr * wr[k];
+                accl[k] += gl * x[k];
+                accr[k] += gr * x[k];
+            }
+            if (VEC == 4) {
+                *reinterpret_cast<f32x4*>(dfeat + r * C + c0) = f32x4{y[0], y[VEC > 1 ? 1 : 0], y[VEC > 2 ? 2 : 0], y[VEC > 3 ? 3 : 0]};
+            } else {
+                dfeat[r * C + c0] = y[0];
+            }
+        }
+#pragma unroll
+        for (int k = 0; k < VEC; ++k) {
+            red_rows[rl * C + c0 + k] = accl[k];
+            red_rows[(row_lanes + rl) * C + c0 + k] = accr[k];
+        }
+    }
+    __syncthreads();
+    for (int j = threadIdx.x; j < 2 * C; j += 256) {  // (which, column): the row lanes in order
+        const int which = j / C, c = j - which * C;
+        float t = 0.0f;
+        for (int l = 0; l < row_lanes; ++l) t += red_rows[(which * row_lanes + l) * C + c];
+        part[static_cast<int64_t>(blockIdx.x) * 2 * C + j] = t;
+    }
+}
+
 // out[0 .. 2 H D) = sum over slabs, sixteen slab lanes per element, fixed order.
 __global__ __launch_bounds__(256) void attn_scores_finish_kernel(float* __restrict__ dal, float* __restrict__ dar,
                                                                  const float* __restrict__ part, int slabs,
@@ -214,13 +276,28 @@ int tango_attn_scores_bwd(float* dfeat, float* dattn_l, float* dattn_r, const fl
         if (!workspace || workspace_bytes < need) return TANGO_ERR_WORKSPACE;
         if ((reinterpret_cast<uintptr_t>(workspace) & 3) != 0) return TANGO_ERR_INVALID_ARG;
         groups = bwd_groups(n, H);
-        const int tpb = static_cast<int>((256 / H) * H);
         const uintptr_t bits = reinterpret_cast<uintptr_t>(feat) | reinterpret_cast<uintptr_t>(dfeat);
-        const int vec4 = (D % kDChunk == 0) && (bits & 15) == 0;
-        hipLaunchKernelGGL(attn_scores_bwd_kernel,
-                           dim3(static_cast<unsigned>(groups), static_cast<unsigned>(ceil_div(D, kDChunk))),
-                           dim3(tpb), 0, s, dfeat, part, del, der, feat, attn_l, attn_r, n, static_cast<int>(H),
-                           static_cast<int>(D), vec4);
+        const int64_t C = H * D;
+        const bool quads = D % 4 == 0 && C <= 1024 && (bits & 15) == 0;
+        if (quads || C <= 256) {  // rows read the way they lie in memory
+            const int row_lanes = static_cast<int>(256 / (quads ? C / 4 : C));
+            const int64_t want = ceil_div(n, static_cast<int64_t>(row_lanes) * 8);  // eight rows per thread or more
+            groups = static_cast<int>(want < groups ? (want < 1 ? 1 : want) : groups);
+            const size_t lds = sizeof(float) * 2 * row_lanes * C;
+            if (quads)
+                hipLaunchKernelGGL(attn_scores_bwd_rows_kernel<4>, dim3(static_cast<unsigned>(groups)), dim3(256), lds, s,
+                                   dfeat, part, del, der, feat, attn_l, attn_r, n, static_cast<int>(H), static_cast<int>(D));
+            else
+                hipLaunchKernelGGL(attn_scores_bwd_rows_kernel<1>, dim3(static_cast<unsigned>(groups)), dim3(256), lds, s,
+                                   dfeat, part, del, der, feat, attn_l, attn_r, n, static_cast<int>(H), static_cast<int>(D));
+        } else {
+            const int tpb = static_cast<int>((256 / H) * H);
+            const int vec4 = (D % kDChunk == 0) && (bits & 15) == 0;
+            hipLaunchKernelGGL(attn_scores_bwd_kernel,
+                               dim3(static_cast<unsigned>(groups), static_cast<unsigned>(ceil_div(D, kDChunk))),
+                               dim3(tpb), 0, s, dfeat, part, del, der, feat, attn_l, attn_r, n, static_cast<int>(H),
+                               static_cast<int>(D), vec4);
+        }
     }
     hipLaunchKernelGGL(attn_scores_finish_kernel, dim3(static_cast<unsigned>(ceil_div(2 * H * D, 16))), dim3(256), 0,
                        s, dattn_l, dattn_r, part, groups, H * D);
