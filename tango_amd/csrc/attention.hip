@@ -195,22 +195,22 @@ __global__ __launch_bounds__(256) void attn_scores_bwd_rows_kernel(
     }
 }
 
-// out[0 .. 2 H D) = sum over slabs, sixteen slab lanes per element, fixed order.
-__global__ __launch_bounds__(256) void attn_scores_finish_kernel(float* __restrict__ dal, float* __restrict__ dar,
-                                                                 const float* __restrict__ part, int slabs,
-                                                                 int64_t hd) {
-    __shared__ float red[16][16];
+// out[0 .. 2 H D) = sum over slabs, 64 slab lanes per element, fixed order.
+__global__ __launch_bounds__(1024) void attn_scores_finish_kernel(float* __restrict__ dal, float* __restrict__ dar,
+                                                                  const float* __restrict__ part, int slabs,
+                                                                  int64_t hd) {
+    __shared__ float red[64][16];
     const int e = threadIdx.x & 15, sl = threadIdx.x >> 4;
     const int64_t idx = static_cast<int64_t>(blockIdx.x) * 16 + e;
     float s = 0.0f;
     if (idx < 2 * hd)
-        for (int b = sl; b < slabs; b += 16) s += part[static_cast<int64_t>(b) * 2 * hd + idx];
+        for (int b = sl; b < slabs; b += 64) s += part[static_cast<int64_t>(b) * 2 * hd + idx];
     red[sl][e] = s;
     __syncthreads();
     if (sl == 0 && idx < 2 * hd) {
         float tot = 0.0f;
 #pragma unroll
-        for (int w = 0; w < 16; ++w) tot += red[w][e];
+        for (int w = 0; w < 64; ++w) tot += red[w][e];
         if (idx < hd) dal[idx] = tot; else dar[idx - hd] = tot;
     }
 }
@@ -281,7 +281,8 @@ int tango_attn_scores_bwd(float* dfeat, float* dattn_l, float* dattn_r, const fl
         const bool quads = D % 4 == 0 && C <= 1024 && (bits & 15) == 0;
         if (quads || C <= 256) {  // rows read the way they lie in memory
             const int row_lanes = static_cast<int>(256 / (quads ? C / 4 : C));
-            const int64_t want = ceil_div(n, static_cast<int64_t>(row_lanes) * 8);  // eight rows per thread or more
+            int64_t want = ceil_div(n, static_cast<int64_t>(row_lanes) * 8);  // eight rows per thread or more,
+            if (want > 512) want = 512;                                          // two workgroups per compute unit at most
             groups = static_cast<int>(want < groups ? (want < 1 ? 1 : want) : groups);
             const size_t lds = sizeof(float) * 2 * row_lanes * C;
             if (quads)
@@ -299,7 +300,7 @@ int tango_attn_scores_bwd(float* dfeat, float* dattn_l, float* dattn_r, const fl
                                static_cast<int>(D), vec4);
         }
     }
-    hipLaunchKernelGGL(attn_scores_finish_kernel, dim3(static_cast<unsigned>(ceil_div(2 * H * D, 16))), dim3(256), 0,
+    hipLaunchKernelGGL(attn_scores_finish_kernel, dim3(static_cast<unsigned>(ceil_div(2 * H * D, 16))), dim3(1024), 0,
                        s, dattn_l, dattn_r, part, groups, H * D);
     return launch_status();
 }
