@@ -10,17 +10,35 @@
 // thread's rows -> LDS over the workgroup's row lanes -> one partial per workgroup -> a finishing kernel), so
 // results do not depend on scheduling.
 //
-// Variance: sums of (x - k) and (x - k)^2 with k = the column's first element (the shifted-data form; the
-// plain sum of squares cancels when |mean| >> std).
+// Variance: every workgroup forms sums of (x - k) and (x - k)^2 over its rows with k = the median of the column's
+// elements in the workgroup's first three rows (the shifted-data form; the plain sum of squares cancels when |mean| >> std), turns them
+// into (mean, sum of squared deviations) of its rows, and the finishing kernel merges the workgroups' pairs with
+// the pairwise update of Chan et al. (mean += d n_b / n, M2 += M2_b + d^2 n_a n_b / n): a shift that happens to be an
+// unlucky value then costs precision in one workgroup's few hundred rows only.
 #include "common.hpp"
 
 namespace tango {
 
 constexpr int kBnMaxGroups = 512;  // workgroups (partials) of the column reductions
 
+// Rows that workgroup b of `groups` reduces: row r belongs to workgroup (r / row_lanes) % groups.
+__host__ __device__ inline int64_t bn_group_rows(int64_t rows, int row_lanes, int groups, int b) {
+    const int64_t period = static_cast<int64_t>(groups) * row_lanes;
+    const int64_t rem = rows % period - static_cast<int64_t>(b) * row_lanes;
+    return rows / period * row_lanes + (rem < 0 ? 0 : (rem > row_lanes ? row_lanes : rem));
+}
+
+// The shift of a workgroup's sums in column c: the median of the column's elements in the workgroup's first three
+// rows (one outlier among them is not taken).
+__device__ __forceinline__ float bn_shift(const float* __restrict__ x, int64_t first_row, int64_t rows, int C, int c) {
+    const int64_t r1 = first_row + 1 < rows ? first_row + 1 : first_row, r2 = first_row + 2 < rows ? first_row + 2 : first_row;
+    const float a = x[first_row * C + c], b = x[r1 * C + c], d = x[r2 * C + c];
+    return fmaxf(fminf(a, b), fminf(fmaxf(a, b), d));
+}
+
 // Thread t of 256 owns column quad t % cq and row lane t / cq (row lanes = 256 / cq; threads beyond are idle).
 // DYNAMIC LDS: 2 * row_lanes * C floats.
-// MODE 0: s1 = sum(x - k), s2 = sum((x - k)^2).
+// MODE 0: partial = (mean, sum of squared deviations) of the workgroup's rows, from s1 = sum(x - k), s2 = sum((x - k)^2).
 // MODE 1: s1 = sum(dy'), s2 = sum(dy' * xhat), dy' = dy where the forward output was positive (relu) else 0.
 template <int MODE>
 __global__ __launch_bounds__(256) void bn_reduce_kernel(const float* __restrict__ x, const float* __restrict__ dy,
@@ -35,9 +53,10 @@ __global__ __launch_bounds__(256) void bn_reduce_kernel(const float* __restrict_
     const int c0 = quad << 2;
     float k[4] = {0.f, 0.f, 0.f, 0.f}, a[4] = {0.f, 0.f, 0.f, 0.f}, b[4] = {0.f, 0.f, 0.f, 0.f}, mu[4] = {0.f, 0.f, 0.f, 0.f},
           rs[4] = {0.f, 0.f, 0.f, 0.f};
+    const int64_t first_row = static_cast<int64_t>(blockIdx.x) * row_lanes;  // < rows (host: eight rows per thread or more)
     if (MODE == 0) {
-        const f32x4 v = *reinterpret_cast<const f32x4*>(x + c0);
-        k[0] = v.x; k[1] = v.y; k[2] = v.z; k[3] = v.w;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) k[i] = bn_shift(x, first_row, rows, C, c0 + i);
     } else {
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
@@ -91,6 +110,22 @@ __global__ __launch_bounds__(256) void bn_reduce_kernel(const float* __restrict_
         }
     }
     __syncthreads();
+    if (MODE == 0) {
+        // rows of this workgroup: those whose index modulo (gridDim.x row_lanes) lies in its row_lanes-wide window
+        const int64_t nb = bn_group_rows(rows, row_lanes, gridDim.x, blockIdx.x);
+        for (int c = threadIdx.x; c < C; c += 256) {  // the row lanes in order
+            float t1 = 0.0f, t2 = 0.0f;
+            for (int l = 0; l < row_lanes; ++l) {
+                t1 += red[l * C + c];
+                t2 += red[(row_lanes + l) * C + c];
+            }
+            const float n = static_cast<float>(nb);
+            const float m2 = t2 - t1 * (t1 / n);
+            partial[static_cast<int64_t>(blockIdx.x) * 2 * C + c] = bn_shift(x, first_row, rows, C, c) + t1 / n;
+            partial[static_cast<int64_t>(blockIdx.x) * 2 * C + C + c] = m2 > 0.0f ? m2 : 0.0f;
+        }
+        return;
+    }
     for (int j = threadIdx.x; j < 2 * C; j += 256) {  // column j of s1 (j < C) or s2: the row lanes in order
         const int which = j / C, c = j - which * C;
         float t = 0.0f;
@@ -99,42 +134,59 @@ __global__ __launch_bounds__(256) void bn_reduce_kernel(const float* __restrict_
     }
 }
 
-// Sums the partials of 16 columns (64 partial lanes each, fixed order) and finishes the statistics.
-// MODE 0: mean, biased variance, 1 / sqrt(var + eps).  MODE 1: out1 = s1 (dbeta), out2 = s2 (dgamma).
+// Merges the partials of 16 columns (64 partial lanes each, fixed order) and finishes the statistics.
+// MODE 0: the workgroups' (mean, M2) pairs -> mean, biased variance, 1 / sqrt(var + eps).
+// MODE 1: out1 = sum of the first partials (dbeta), out2 = sum of the second (dgamma).
 template <int MODE>
 __global__ __launch_bounds__(1024) void bn_finish_kernel(const float* __restrict__ partial, int groups, int C, int64_t rows,
-                                                        float eps, const float* __restrict__ x, float* __restrict__ out1,
-                                                        float* __restrict__ out2, float* __restrict__ out3) {
-    __shared__ float red[2][64][16];
+                                                         int row_lanes, float eps, float* __restrict__ out1,
+                                                         float* __restrict__ out2, float* __restrict__ out3) {
+    __shared__ float red[3][64][16];
     const int e = threadIdx.x & 15, sl = threadIdx.x >> 4;
     const int c = blockIdx.x * 16 + e;
-    float t1 = 0.0f, t2 = 0.0f;
+    // MODE 0: (n, mean, M2) of the rows merged so far; MODE 1: t1, t2 = plain sums
+    float n = 0.0f, t1 = 0.0f, t2 = 0.0f;
+    auto merge = [&](float nb, float mb, float m2b) {
+        if (nb <= 0.0f) return;
+        const float tot = n + nb, d = mb - t1;
+        t1 = t1 + d * (nb / tot);
+        t2 = t2 + m2b + d * d * (n * (nb / tot));
+        n = tot;
+    };
     if (c < C)
         for (int g = sl; g < groups; g += 64) {
-            t1 += partial[static_cast<int64_t>(g) * 2 * C + c];
-            t2 += partial[static_cast<int64_t>(g) * 2 * C + C + c];
+            const float p1 = partial[static_cast<int64_t>(g) * 2 * C + c];
+            const float p2 = partial[static_cast<int64_t>(g) * 2 * C + C + c];
+            if (MODE == 0) {
+                merge(static_cast<float>(bn_group_rows(rows, row_lanes, groups, g)), p1, p2);
+            } else {
+                t1 += p1;
+                t2 += p2;
+            }
         }
-    red[0][sl][e] = t1;
-    red[1][sl][e] = t2;
+    red[0][sl][e] = n;
+    red[1][sl][e] = t1;
+    red[2][sl][e] = t2;
     __syncthreads();
     if (sl == 0 && c < C) {
-        float s1 = 0.0f, s2 = 0.0f;
-#pragma unroll
+        n = t1 = t2 = 0.0f;
+#pragma unroll 4
         for (int w = 0; w < 64; ++w) {
-            s1 += red[0][w][e];
-            s2 += red[1][w][e];
+            if (MODE == 0) {
+                merge(red[0][w][e], red[1][w][e], red[2][w][e]);
+            } else {
+                t1 += red[1][w][e];
+                t2 += red[2][w][e];
+            }
         }
         if (MODE == 0) {
-            const float n = static_cast<float>(rows);
-            const float m1 = s1 / n;           // mean of x - k
-            float var = s2 / n - m1 * m1;      // biased variance
-            var = var > 0.0f ? var : 0.0f;
-            out1[c] = x[c] + m1;               // k = x[0, c]
+            const float var = t2 / n;  // biased variance
+            out1[c] = t1;
             out2[c] = var;
             out3[c] = 1.0f / sqrtf(var + eps);
         } else {
-            out1[c] = s1;
-            out2[c] = s2;
+            out1[c] = t1;
+            out2[c] = t2;
         }
     }
 }
@@ -235,8 +287,8 @@ int tango_batchnorm_fwd_f32(float* y, float* mean, float* var, float* rstd, floa
     if (scale_y) fill_u32(scale_y, 0u, 1, s);
     hipLaunchKernelGGL(bn_reduce_kernel<0>, dim3(groups), dim3(256), sizeof(float) * 2 * row_lanes * C, s, x, nullptr,
                        nullptr, nullptr, nullptr, nullptr, rows, C, 0, partial);
-    hipLaunchKernelGGL(bn_finish_kernel<0>, dim3((C + 15) / 16), dim3(1024), 0, s, partial, groups, C, rows, eps, x, mean,
-                       var, rstd);
+    hipLaunchKernelGGL(bn_finish_kernel<0>, dim3((C + 15) / 16), dim3(1024), 0, s, partial, groups, C, rows, row_lanes, eps,
+                       mean, var, rstd);
     hipLaunchKernelGGL(bn_apply_kernel<false>, dim3(grid_for(rows * (cols >> 2), 256)), dim3(256), sizeof(float) * 6 * C, s,
                        y, x, nullptr, mean, rstd, gamma, beta, nullptr, nullptr, rows, C, relu, scale_y);
     return launch_status();
@@ -261,7 +313,7 @@ int tango_batchnorm_bwd_f32(float* dx, float* dgamma, float* dbeta, const float*
     float* partial = static_cast<float*>(workspace);
     hipLaunchKernelGGL(bn_reduce_kernel<1>, dim3(groups), dim3(256), sizeof(float) * 2 * row_lanes * C, s, x, dy, mean,
                        rstd, gamma, beta, rows, C, relu, partial);
-    hipLaunchKernelGGL(bn_finish_kernel<1>, dim3((C + 15) / 16), dim3(1024), 0, s, partial, groups, C, rows, 0.0f, x,
+    hipLaunchKernelGGL(bn_finish_kernel<1>, dim3((C + 15) / 16), dim3(1024), 0, s, partial, groups, C, rows, row_lanes, 0.0f,
                        dbeta, dgamma, nullptr);
     hipLaunchKernelGGL(bn_apply_kernel<true>, dim3(grid_for(rows * (cols >> 2), 256)), dim3(256), sizeof(float) * 6 * C, s,
                        dx, x, dy, mean, rstd, gamma, beta, dbeta, dgamma, rows, C, relu, nullptr);
