@@ -153,12 +153,16 @@ __global__ __launch_bounds__(1024) void bn_finish_kernel(const float* __restrict
         t2 = t2 + m2b + d * d * (n * (nb / tot));
         n = tot;
     };
+    // rows of workgroup g (bn_group_rows): whole periods, plus its window of the last, partial one
+    const int64_t period = static_cast<int64_t>(groups) * row_lanes;
+    const int64_t whole = rows / period * row_lanes, tail = rows % period;
     if (c < C)
         for (int g = sl; g < groups; g += 64) {
             const float p1 = partial[static_cast<int64_t>(g) * 2 * C + c];
             const float p2 = partial[static_cast<int64_t>(g) * 2 * C + C + c];
             if (MODE == 0) {
-                merge(static_cast<float>(bn_group_rows(rows, row_lanes, groups, g)), p1, p2);
+                const int64_t rem = tail - static_cast<int64_t>(g) * row_lanes;
+                merge(static_cast<float>(whole + (rem < 0 ? 0 : (rem > row_lanes ? row_lanes : rem))), p1, p2);
             } else {
                 t1 += p1;
                 t2 += p2;
@@ -168,17 +172,22 @@ __global__ __launch_bounds__(1024) void bn_finish_kernel(const float* __restrict
     red[1][sl][e] = t1;
     red[2][sl][e] = t2;
     __syncthreads();
-    if (sl == 0 && c < C) {
-        n = t1 = t2 = 0.0f;
-#pragma unroll 4
-        for (int w = 0; w < 64; ++w) {
+    // the 64 partial lanes of a column fold pairwise: lane sl takes in lane sl + half (a fixed tree)
+    for (int half = 32; half >= 1; half >>= 1) {
+        if (sl < half) {
             if (MODE == 0) {
-                merge(red[0][w][e], red[1][w][e], red[2][w][e]);
+                merge(red[0][sl + half][e], red[1][sl + half][e], red[2][sl + half][e]);
             } else {
-                t1 += red[1][w][e];
-                t2 += red[2][w][e];
+                t1 += red[1][sl + half][e];
+                t2 += red[2][sl + half][e];
             }
+            red[0][sl][e] = n;
+            red[1][sl][e] = t1;
+            red[2][sl][e] = t2;
         }
+        __syncthreads();
+    }
+    if (sl == 0 && c < C) {
         if (MODE == 0) {
             const float var = t2 / n;  // biased variance
             out1[c] = t1;
