@@ -59,7 +59,7 @@ def parse():
                          "170,000-node / 8.17 M-edge homogenised heterogeneous graph (4 heads x 64)")
     ap.add_argument("--profile-mode", default=None,
                     choices=["spmm", "copy", "qlinear", "gradx", "gradw", "sddmm", "quantize", "softmax", "umule",
-                             "gat", "arxiv", "hgt", "hetero"],
+                             "gat", "arxiv", "arxiv-gcn", "hgt", "hetero"],
                     help="run only the dominant kernel (spmm: copy_u F=256 on the benchmark graph) or a "
                          "1 GiB device copy (counter calibration), for rocprofv3 --pmc passes")
     return ap.parse_args()
@@ -248,13 +248,14 @@ def sddmm_primitives(K, torch):
     return out
 
 
-def model_steps(K, torch, which=("gat", "arxiv", "hgt", "hetero"), iters=10, warm=3):
+def model_steps(K, torch, which=("gat", "arxiv", "arxiv-gcn", "hgt", "hetero"), iters=10, warm=3):
     """The other model configurations, one training step each (forward + loss + backward + Adam):
     the 3-layer GAT (hidden 16 x 8 heads, evaluation/test_gat.py:170-214) on the 169,343-node graph
     and two HGT layers (256-d, 4 heads) on the homogenised 3-type / 4-relation graph."""
     out = {}
     torch.manual_seed(4)
-    for name, fn in (("gat", _gat_step), ("arxiv", _arxiv_step), ("hgt", _hgt_step), ("hetero", _hetero_step)):
+    for name, fn in (("gat", _gat_step), ("arxiv", _arxiv_step), ("arxiv-gcn", _arxiv_gcn_step), ("hgt", _hgt_step),
+                     ("hetero", _hetero_step)):
         if name in which:
             out.update(fn(K, torch, iters, warm))
     return out
@@ -301,6 +302,24 @@ def _arxiv_step(K, torch, iters, warm):
         arxiv_loss(am(g, x), al).backward()
         aopt.step()
     return {"arxiv_gat3_step_169343n_1.34Me_ms": round(time_op(arxiv_step, iters=iters, warm=warm), 3)}
+
+
+def _arxiv_gcn_step(K, torch, iters, warm):
+    # evaluation/arxiv_gcn.py:156-209 on the same graph: three graph convolutions (hidden 256) with a quantized linear
+    # skip branch each, batch norm + ReLU between them; dropout off
+    from tango_amd.evaluation import arxiv_loss
+    from tango_amd.gcn import ArxivGCN
+    g, x = _gat_graph(torch)
+    n = g.num_nodes()
+    gm = ArxivGCN(128, 256, 40, 3, torch.relu, 0.0, True).cuda()
+    gl = torch.randint(0, 40, (n,), device="cuda")
+    gopt = torch.optim.Adam(gm.parameters(), lr=5e-3, fused=True)
+
+    def arxiv_gcn_step():
+        gopt.zero_grad(set_to_none=True)
+        arxiv_loss(gm(g, x), gl).backward()
+        gopt.step()
+    return {"arxiv_gcn3_step_169343n_1.34Me_ms": round(time_op(arxiv_gcn_step, iters=iters, warm=warm), 3)}
 
 
 def _hgt_step(K, torch, iters, warm):
@@ -464,7 +483,7 @@ def main():
         torch.cuda.synchronize()
         print(json.dumps({"profile_mode": "copy", "bytes_read": src.numel() * 4, "bytes_written": src.numel() * 4}))
         return
-    if args.profile_mode in ("gat", "arxiv", "hgt", "hetero"):  # one training step of the attention models, for kernel traces
+    if args.profile_mode in ("gat", "arxiv", "arxiv-gcn", "hgt", "hetero"):  # one training step of the attention models, for kernel traces
         out = model_steps(K, torch, which=(args.profile_mode,), iters=args.steps, warm=args.warmup)
         print(json.dumps(dict(out, profile_mode=args.profile_mode)))
         return

@@ -33,16 +33,22 @@ class spmm_copy_u(Function):
     ``row_scale`` [n], ``bias`` [F] and ``relu`` fold the glue that follows the
     aggregation in a GCN layer (evaluation/test_gcn.py:123-137: ``* in_deg^-1/2``,
     ``+ bias``, activation) into the kernel's epilogue; the backward then masks,
-    sums the bias gradient, scales rows and quantizes in two reads of dOut."""
+    sums the bias gradient, scales rows and quantizes in two reads of dOut.
+    ``src_row_mul`` [n] folds the ``feat * out_deg^-1/2`` in front of the aggregation (evaluation/test_gcn.py:86-94)
+    into the pass that quantizes N, and its backward into the epilogue of the reverse aggregation; same roundings
+    as the separate multiplications."""
 
     @staticmethod
-    def forward(ctx, g, N, scaleN=None, row_scale=None, bias=None, relu=False):
+    def forward(ctx, g, N, scaleN=None, row_scale=None, bias=None, relu=False, src_row_mul=None):
         N = N if N.is_contiguous() else N.contiguous()
-        fused = row_scale is not None or bias is not None or relu
+        fused = row_scale is not None or bias is not None or relu or src_row_mul is not None
         if fused and N.dim() != 2:
-            raise RuntimeError("spmm_copy_u: the fused epilogue needs 2-D features")
+            raise RuntimeError("spmm_copy_u: the fused prologue / epilogue needs 2-D features")
+        if src_row_mul is not None and scaleN is not None:
+            raise RuntimeError("spmm_copy_u: a precomputed scale cannot be combined with src_row_mul")
+        ctx.src_row_mul = src_row_mul
         if N.dim() == 2:
-            N_, scaleN = quantize_padded(N, scaleN, align=_gather_align(N.size(1)))
+            N_, scaleN = quantize_padded(N, scaleN, align=_gather_align(N.size(1)), row_mul=src_row_mul)
         else:
             N_, scaleN = quantize(N, scaleN)
         # the backward pass needs only the sign of the ReLU's output: sixteen columns per 16-bit word, written
@@ -70,8 +76,8 @@ class spmm_copy_u(Function):
         if row_scale is None and not has_bias and mask is None:
             if ctx.needs_input_grad[1]:
                 dZ_, scaledZ = _quantize_grad(dOut, True)
-                dN = csr_SPMM(g, dZ_, scaledZ, True)
-            return None, dN, None, None, None, None
+                dN = csr_SPMM(g, dZ_, scaledZ, True, row_scale=ctx.src_row_mul)
+            return None, dN, None, None, None, None, None
         dOut = dOut if dOut.is_contiguous() else dOut.contiguous()
         want_bias = has_bias and ctx.needs_input_grad[4]
         # dZ = (dOut where out > 0) * row_scale; its scale and the bias gradient come from one pass
@@ -83,8 +89,8 @@ class spmm_copy_u(Function):
                 kw.update(config.stochastic_args(dOut.device))
             dZ_, _ = quantize_padded(dOut, scaledZ, row_mul=row_scale, mask=mask, mask_mode=mode,
                                      align=_gather_align(dOut.size(1)), **kw)
-            dN = csr_SPMM(g, dZ_, scaledZ, True)
-        return None, dN, None, None, dbias, None
+            dN = csr_SPMM(g, dZ_, scaledZ, True, row_scale=ctx.src_row_mul)
+        return None, dN, None, None, dbias, None, None
 
 
 def _need_reduce_last_dim(ufeat, efeat):

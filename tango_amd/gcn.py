@@ -45,7 +45,7 @@ class QGraphConv(nn.Module):
                 if self._activation is not None and not relu:
                     rst = self._activation(rst)
                 return rst
-            rst = spmm_copy_u.apply(graph, feat * norm_src.unsqueeze(1))
+            rst = spmm_copy_u.apply(graph, feat, None, None, None, False, norm_src)  # "feat * norm_src" in the quantize pass
             rst = Qlinear_func.apply(rst, self.weight) * norm_dst.unsqueeze(1)
         else:
             feat_src = feat * norm_src.unsqueeze(1)

@@ -135,7 +135,7 @@ def test_gemm_row_scale_prologue_and_gradx_epilogue(K, orc):
     assert np.array_equal(host(dX), want)
 
 
-@pytest.mark.parametrize("dims", [(100, 32, 7), (64, 16, 16)])
+@pytest.mark.parametrize("dims", [(100, 32, 7), (64, 16, 16), (16, 48, 64), (41, 128, 128)])
 def test_fused_gcn_matches_unfused(dims):
     from tango_amd.gcn import GCN
     from tango_amd.graph import chung_lu
