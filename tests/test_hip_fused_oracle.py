@@ -101,3 +101,35 @@ def test_shared_input_linears_match_oracle(orc, M, Kd, N1, N2):
         np.testing.assert_allclose(host(lin.bias.grad), dY.astype(np.float64).sum(0), rtol=1e-4, atol=2e-3)
         dX = orc.qgemm_bwd_dx_ex(dq, Wq, s_d, sW, accumulate_into=dX)
     assert np.array_equal(host(X.grad), dX)
+
+
+@pytest.mark.parametrize("n,e,F", [(900, 20000, 128), (400, 6000, 41), (1500, 30000, 256)])
+def test_copy_u_with_source_multiplier_matches_oracle(orc, n, e, F):
+    """The aggregate-first graph convolution's "feat * out_deg^-1/2" folded into the aggregation: the multiplier
+    rides in the pass that quantizes the input (forward) and in the reverse aggregation's epilogue (backward)."""
+    from tango_amd import config
+    from tango_amd.SPMM import spmm_copy_u
+    rng = np.random.default_rng(n)
+    src, dst = rand_graph(rng, n, e)
+    g = make_graph(src, dst, n)
+    N = rng.standard_normal((n, F)).astype(np.float32)
+    mul = (rng.random(n) + 0.2).astype(np.float32)
+    dZ = rng.standard_normal((n, F)).astype(np.float32)
+    old = config.grad_round_mode
+    config.grad_round_mode = "rne"
+    try:
+        tN = dev(N).requires_grad_()
+        out = spmm_copy_u.apply(g, tN, None, None, None, False, dev(mul))
+        out.backward(dev(dZ))
+    finally:
+        config.grad_round_mode = old
+    sN, _ = orc.absmax_ex(N, row_mul=mul)
+    Nq = orc.quantize_rows_ex(N, sN, row_mul=mul)
+    cip, cix, _ = (host(t) for t in g.adj_csc)
+    assert np.array_equal(host(out), orc.spmm_csr_copy_u_ex(cip, cix, Nq, sN))
+    # the same bits as multiplying first
+    assert torch.equal(out, spmm_copy_u.apply(g, dev(N) * dev(mul).unsqueeze(1)))
+    s_dZ = orc.absmax_scale(dZ)
+    dZq = orc.quantize(dZ, s_dZ)
+    rip, rix, _ = (host(t) for t in g.adj_csr)
+    assert np.array_equal(host(tN.grad), orc.spmm_csr_copy_u_ex(rip, rix, dZq, s_dZ, row_scale=mul))
