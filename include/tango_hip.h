@@ -438,8 +438,8 @@ int tango_softmax_xent_f32(const float* logits, int64_t ld, const int64_t* label
    through the ReLU (the forward's sign, recomputed from x) and returns
      dbeta[c] = sum_r dy'[r, c], dgamma[c] = sum_r dy'[r, c] * xhat[r, c],
      dx[r, c] = rstd[c] * gamma[c] * (dy'[r, c] - dbeta[c] / rows - xhat[r, c] * dgamma[c] / rows),
-   xhat = (x - mean) * rstd.  cols must be a multiple of 4 and at most 1024, x / y / dy / dx
-   16-byte aligned (TANGO_ERR_UNSUPPORTED otherwise).  All sums run in a fixed order.
+   xhat = (x - mean) * rstd.  cols <= 2048 (TANGO_ERR_UNSUPPORTED otherwise); rows are read 16, 8 or 4 bytes
+   per lane, the widest that cols and the alignment of x / y / dy / dx allow.  All sums run in a fixed order.
    workspace: tango_batchnorm_workspace(rows, cols) bytes, the same for both calls. */
 size_t tango_batchnorm_workspace(int64_t rows, int64_t cols);
 int tango_batchnorm_fwd_f32(float* y, float* mean, float* var, float* rstd, float* scale_y,

@@ -5,7 +5,7 @@ from torch.autograd.function import Function, once_differentiable
 
 from . import config
 from .kernels import (cuda_kernels, incidence_SPMM, multi_cusparse_SPMM, mySDDMM_int8, mySDDMM_quantize_on_load,
-                      quantize, refuse_capture)
+                      quantize, quantize_heads, refuse_capture, unpad_heads)
 
 
 def _quantize_grad(t):
@@ -58,8 +58,10 @@ class sddmm_u_dot_v(Function):
 
     @staticmethod
     def forward(ctx, g, U, V, scaleU_=None, scaleV_=None, out_scale=None):
-        U_, scaleU = quantize(U if U.is_contiguous() else U.contiguous(), scaleU_)
-        V_, scaleV = quantize(V if V.is_contiguous() else V.contiguous(), scaleV_)
+        # heads whose width would leave the int8 rows unaligned are zero-padded (kernels.pad_heads): same dot products
+        U_, scaleU = quantize_heads(U if U.is_contiguous() else U.contiguous(), scaleU_)
+        V_, scaleV = quantize_heads(V if V.is_contiguous() else V.contiguous(), scaleV_)
+        ctx.width = U.size(-1)
         if out_scale is not None:
             # 1-element products: the forward dequantizes with sU * (sV c), the backward passes with
             # s_dZ * (sV c) and s_dZ * (sU c)
@@ -83,7 +85,9 @@ class sddmm_u_dot_v(Function):
         dZ_, scaledZ = _quantize_grad(dZ3)  # [E, H, 1], edge-major edge values
         dU = dV = None
         if ctx.needs_input_grad[1]:
-            dU = multi_cusparse_SPMM(g, V3, dZ_, scaledZ, True, edge_major=True, scale2=scaleV).reshape(U_.shape)
+            dU = unpad_heads(multi_cusparse_SPMM(g, V3, dZ_, scaledZ, True, edge_major=True, scale2=scaleV).reshape(U_.shape),
+                             ctx.width)
         if ctx.needs_input_grad[2]:
-            dV = multi_cusparse_SPMM(g, U3, dZ_, scaledZ, edge_major=True, scale2=scaleU).reshape(V_.shape)
+            dV = unpad_heads(multi_cusparse_SPMM(g, U3, dZ_, scaledZ, edge_major=True, scale2=scaleU).reshape(V_.shape),
+                             ctx.width)
         return None, dU, dV, None, None, None

@@ -3,8 +3,8 @@ import torch
 from torch.autograd.function import Function, once_differentiable
 
 from . import config
-from .kernels import (cuda_kernels, csr_SPMM, multi_cusparse_SPMM, mySDDMM_int8, quantize, quantize_padded,
-                      refuse_capture)
+from .kernels import (cuda_kernels, csr_SPMM, multi_cusparse_SPMM, mySDDMM_int8, pad_heads, quantize, quantize_heads,
+                      quantize_padded, refuse_capture, unpad_heads)
 
 
 def _gather_align(width):
@@ -129,10 +129,16 @@ class spmm_u_mul_e(Function):
             E_T_, _ = quantize(E, scaleE)  # no pass that looks for the scale
         else:
             E_T_, scaleE = quantize(E)
-        N_, scaleN = quantize(N, scaleN)  # one absmax pass (the reference runs two, cuda/SPMM.py:39,43)
+        # one absmax pass (the reference runs two, cuda/SPMM.py:39,43).  Broadcast edge values, no epilogue: heads whose
+        # width would leave the int8 rows unaligned are zero-padded (kernels.pad_heads); the padding columns of the
+        # result are dropped again
+        padded = N.dim() == 3 and E.size(-1) == 1 and bias is None and act is None and pad_heads(N.size(2)) != N.size(2)
+        N_, scaleN = quantize_heads(N, scaleN) if padded else quantize(N, scaleN)
         # dequantized with scaleN * scaleE (cuda/SPMM.py:44); the kernel multiplies the two itself
         out = multi_cusparse_SPMM(g, N_, E_T_, scaleN, edge_major=True, bias=bias, scale2=scaleE, act=act)
+        out = unpad_heads(out, N.size(-1))
         reduce_last = _need_reduce_last_dim(N, E)
+        ctx.padded = padded
         ctx.backward_cache = g, N_, scaleN, E_T_, scaleE, reduce_last, E.shape, bias is not None, act
         if act is not None:
             ctx.save_for_backward(out)  # not an attribute: that would tie the output to its own grad_fn
@@ -164,6 +170,12 @@ class spmm_u_mul_e(Function):
             if config.grad_round_mode == "stochastic":
                 kw.update(config.stochastic_args(dZ.device))
             dZ_, _ = quantize(dZ, scaledZ, **kw)
+        elif ctx.padded:
+            dZ = dZ if dZ.is_contiguous() else dZ.contiguous()
+            kw = {"round_mode": config.grad_round_mode}
+            if config.grad_round_mode == "stochastic":
+                kw.update(config.stochastic_args(dZ.device))
+            dZ_, scaledZ = quantize_heads(dZ, **kw)
         else:
             dZ_, scaledZ = _quantize_grad(dZ, False)
         dN = dE = None
@@ -171,7 +183,7 @@ class spmm_u_mul_e(Function):
             # dN = A^T (E * dZ): the dequantization scale is s_dZ * s_E.  The reference passes
             # the forward scale s_N * s_E here (cuda/SPMM.py:56); ref_compat reproduces that.
             first = scaleN if config.ref_compat else scaledZ
-            dN = multi_cusparse_SPMM(g, dZ_, E_T_, first, True, edge_major=True, scale2=scaleE)
+            dN = unpad_heads(multi_cusparse_SPMM(g, dZ_, E_T_, first, True, edge_major=True, scale2=scaleE), dZ.size(-1))
         if ctx.needs_input_grad[2]:
             op = "dot" if reduce_last else "mul"
             dE, _ = mySDDMM_int8(g, op, N_, dZ_, scaleN, scaledZ, False)

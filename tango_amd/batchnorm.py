@@ -14,8 +14,7 @@ from .kernels import _L, _ptr, _stream, _workspace, check, refuse_capture
 
 
 def _fusable(x, cols):
-    return x.is_cuda and x.dim() == 2 and x.dtype == torch.float32 and cols % 4 == 0 and 4 <= cols <= 1024 \
-        and x.size(0) > 1
+    return x.is_cuda and x.dim() == 2 and x.dtype == torch.float32 and 1 <= cols <= 2048 and x.size(0) > 1
 
 
 class _BatchNormAct(Function):

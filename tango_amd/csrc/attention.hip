@@ -15,7 +15,6 @@
 
 namespace tango {
 
-constexpr int kDChunk = 16;       // columns of one head a backward thread keeps in registers
 constexpr int kBwdGroups = 1024;  // workgroups (slabs) of the backward reduction
 
 // One (node, head) item per thread and loop step.  SCALES: the launch is a fixed number of large workgroups
@@ -65,90 +64,28 @@ __global__ __launch_bounds__(SCALES ? 1024 : 256) void attn_scores_fwd_kernel(
     }
 }
 
-// blockDim.x = tpb, a multiple of H: thread t is head t % H of row slot t / H.  gridDim.y tiles D
-// in chunks of kDChunk.  part[b][2][H][D]: workgroup b's sums of del * feat and der * feat.
-__global__ __launch_bounds__(256) void attn_scores_bwd_kernel(
-    float* __restrict__ dfeat, float* __restrict__ part, const float* __restrict__ del,
-    const float* __restrict__ der, const float* __restrict__ feat, const float* __restrict__ al,
-    const float* __restrict__ ar, int64_t n, int H, int D, int vec4) {
-    __shared__ float red[256][2 * kDChunk + 1];
-    const int t = threadIdx.x;
-    const int tpb = blockDim.x;
-    const int h = t % H;
-    const int slots = tpb / H;
-    const int d0 = blockIdx.y * kDChunk;
-    const int dn = (D - d0) < kDChunk ? (D - d0) : kDChunk;
-    float wl[kDChunk], wr[kDChunk], accl[kDChunk], accr[kDChunk];
-#pragma unroll
-    for (int k = 0; k < kDChunk; ++k) {
-        wl[k] = k < dn ? al[static_cast<int64_t>(h) * D + d0 + k] : 0.0f;
-        wr[k] = k < dn ? ar[static_cast<int64_t>(h) * D + d0 + k] : 0.0f;
-        accl[k] = accr[k] = 0.0f;
-    }
-    const int64_t step = static_cast<int64_t>(gridDim.x) * slots;
-    for (int64_t r = static_cast<int64_t>(blockIdx.x) * slots + t / H; r < n; r += step) {
-        const int64_t i = r * H + h;
-        const float gl = del[i], gr = der[i];
-        const float* f = feat + i * D + d0;
-        float* o = dfeat + i * D + d0;
-        if (vec4) {  // whole chunks, 16-byte aligned
-#pragma unroll
-            for (int q = 0; q < kDChunk / 4; ++q) {
-                const f32x4 x = *reinterpret_cast<const f32x4*>(f + 4 * q);
-                f32x4 y;
-#pragma unroll
-                for (int k = 0; k < 4; ++k) {
-                    y[k] = gl * wl[4 * q + k] + gr * wr[4 * q + k];
-                    accl[4 * q + k] += gl * x[k];
-                    accr[4 * q + k] += gr * x[k];
-                }
-                *reinterpret_cast<f32x4*>(o + 4 * q) = y;
-            }
-            continue;
-        }
-#pragma unroll
-        for (int k = 0; k < kDChunk; ++k) {
-            if (k < dn) {
-                const float x = f[k];
-                o[k] = gl * wl[k] + gr * wr[k];
-                accl[k] += gl * x;
-                accr[k] += gr * x;
-            }
-        }
-    }
-#pragma unroll
-    for (int k = 0; k < kDChunk; ++k) {
-        red[t][k] = accl[k];
-        red[t][kDChunk + k] = accr[k];
-    }
-    __syncthreads();
-    // (which, head, column) sums over the workgroup's row slots, in slot order
-    for (int idx = t; idx < 2 * H * dn; idx += tpb) {
-        const int which = idx / (H * dn);
-        const int rem = idx - which * H * dn;
-        const int hh = rem / dn, k = rem - hh * dn;
-        float s = 0.0f;
-        for (int sl = 0; sl < slots; ++sl) s += red[sl * H + hh][which * kDChunk + k];
-        part[((static_cast<int64_t>(blockIdx.x) * 2 + which) * H + hh) * D + d0 + k] = s;
-    }
-}
-
-// The same sums and products with the rows read the way they lie in memory: thread t owns VEC consecutive
-// columns (of the H * D of a row; VEC = 4 needs D % 4 == 0 so that they share a head) and row lane t / cg of
-// blockDim.x / cg, cg = H * D / VEC column groups: a wavefront's loads and stores cover consecutive bytes,
-// where a thread per (row, head) reads D floats at a stride of D floats.  Same partials layout.
-// DYNAMIC LDS: 2 * row_lanes * H * D floats.
+// d_feat = del * attn_l + der * attn_r and the two [H, D] parameter gradients (sums over the rows of del * feat and
+// der * feat), with the rows read the way they lie in memory: a thread owns VEC consecutive columns
+// (of the H * D of a row; VEC = 4 or 2 needs D % VEC == 0 so that they share a head) of one of the row lanes of its
+// workgroup: a wavefront's loads and stores cover consecutive bytes (a thread per (row, head) would read D floats
+// at a stride of D floats).  part[b][2][H][D]: workgroup b's sums.  gridDim.y cuts the H * D / VEC column groups into chunks of at most 256; a workgroup
+// has 256 / (groups of its chunk) row lanes.
+// DYNAMIC LDS: 2 * 256 * VEC floats at most (2 * row_lanes * columns of the chunk).
 template <int VEC>
 __global__ __launch_bounds__(256) void attn_scores_bwd_rows_kernel(
     float* __restrict__ dfeat, float* __restrict__ part, const float* __restrict__ del,
     const float* __restrict__ der, const float* __restrict__ feat, const float* __restrict__ al,
     const float* __restrict__ ar, int64_t n, int H, int D) {
-    extern __shared__ float red_rows[];  // [2][row_lanes][C]
+    extern __shared__ float red_rows[];  // [2][row_lanes][cw]
+    typedef float fvec __attribute__((ext_vector_type(VEC == 1 ? 2 : VEC)));  // (unused for VEC == 1)
     const int C = H * D;
-    const int cg = C / VEC;
+    const int cg_all = C / VEC;
+    const int g0 = blockIdx.y * 256;                               // first column group of this chunk
+    const int cg = cg_all - g0 < 256 ? cg_all - g0 : 256;          // column groups of this chunk
+    const int cw = cg * VEC;                                       // its columns
     const int row_lanes = 256 / cg;
     const int grp = threadIdx.x % cg, rl = threadIdx.x / cg;
-    const int c0 = grp * VEC;
+    const int c0 = (g0 + grp) * VEC;
     const int h = c0 / D;
     float wl[VEC], wr[VEC], accl[VEC], accr[VEC];
 #pragma unroll
@@ -162,9 +99,10 @@ __global__ __launch_bounds__(256) void attn_scores_bwd_rows_kernel(
         for (int64_t r = static_cast<int64_t>(blockIdx.x) * row_lanes + rl; r < n; r += step) {
             const float gl = del[r * H + h], gr = der[r * H + h];
             float x[VEC], y[VEC];
-            if (VEC == 4) {
-                const f32x4 v = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(feat + r * C + c0));
-                x[0] = v.x; x[1] = v.y; x[2] = v.z; x[3] = v.w;
+            if (VEC > 1) {
+                const fvec v = __builtin_nontemporal_load(reinterpret_cast<const fvec*>(feat + r * C + c0));
+#pragma unroll
+                for (int k = 0; k < VEC; ++k) x[k] = v[k];
             } else {
                 x[0] = feat[r * C + c0];
             }
@@ -174,24 +112,27 @@ __global__ __launch_bounds__(256) void attn_scores_bwd_rows_kernel(
                 accl[k] += gl * x[k];
                 accr[k] += gr * x[k];
             }
-            if (VEC == 4) {
-                *reinterpret_cast<f32x4*>(dfeat + r * C + c0) = f32x4{y[0], y[VEC > 1 ? 1 : 0], y[VEC > 2 ? 2 : 0], y[VEC > 3 ? 3 : 0]};
+            if (VEC > 1) {
+                fvec o;
+#pragma unroll
+                for (int k = 0; k < VEC; ++k) o[k] = y[k];
+                *reinterpret_cast<fvec*>(dfeat + r * C + c0) = o;
             } else {
                 dfeat[r * C + c0] = y[0];
             }
         }
 #pragma unroll
         for (int k = 0; k < VEC; ++k) {
-            red_rows[rl * C + c0 + k] = accl[k];
-            red_rows[(row_lanes + rl) * C + c0 + k] = accr[k];
+            red_rows[rl * cw + grp * VEC + k] = accl[k];
+            red_rows[(row_lanes + rl) * cw + grp * VEC + k] = accr[k];
         }
     }
     __syncthreads();
-    for (int j = threadIdx.x; j < 2 * C; j += 256) {  // (which, column): the row lanes in order
-        const int which = j / C, c = j - which * C;
+    for (int j = threadIdx.x; j < 2 * cw; j += 256) {  // (which, column of the chunk): the row lanes in order
+        const int which = j / cw, c = j - which * cw;
         float t = 0.0f;
-        for (int l = 0; l < row_lanes; ++l) t += red_rows[(which * row_lanes + l) * C + c];
-        part[static_cast<int64_t>(blockIdx.x) * 2 * C + j] = t;
+        for (int l = 0; l < row_lanes; ++l) t += red_rows[(which * row_lanes + l) * cw + c];
+        part[(static_cast<int64_t>(blockIdx.x) * 2 + which) * C + g0 * VEC + c] = t;
     }
 }
 
@@ -265,7 +206,7 @@ int tango_attn_scores_bwd(float* dfeat, float* dattn_l, float* dattn_r, const fl
                           size_t workspace_bytes, tango_stream_t stream) {
     if (n < 0 || H < 0 || D < 0) return TANGO_ERR_INVALID_ARG;
     if (H * D == 0) return TANGO_OK;
-    if (H > 256 || D >= (1LL << 31) || ceil_div(D, kDChunk) > 65535) return TANGO_ERR_UNSUPPORTED;
+    if (H > 256 || D >= (1LL << 31) || H * D > (1LL << 23)) return TANGO_ERR_UNSUPPORTED;
     if (!dattn_l || !dattn_r || !attn_l || !attn_r || (n > 0 && (!dfeat || !del || !der || !feat)))
         return TANGO_ERR_INVALID_ARG;
     hipStream_t s = as_stream(stream);
@@ -278,26 +219,24 @@ int tango_attn_scores_bwd(float* dfeat, float* dattn_l, float* dattn_r, const fl
         groups = bwd_groups(n, H);
         const uintptr_t bits = reinterpret_cast<uintptr_t>(feat) | reinterpret_cast<uintptr_t>(dfeat);
         const int64_t C = H * D;
-        const bool quads = D % 4 == 0 && C <= 1024 && (bits & 15) == 0;
-        if (quads || C <= 256) {  // rows read the way they lie in memory
-            const int row_lanes = static_cast<int>(256 / (quads ? C / 4 : C));
+        const int vec = (D % 4 == 0 && (bits & 15) == 0) ? 4 : (D % 2 == 0 && (bits & 7) == 0) ? 2 : 1;
+        const int64_t cg_all = C / vec, chunks = ceil_div(cg_all, 256);
+        {
+            const int row_lanes = static_cast<int>(256 / (cg_all < 256 ? cg_all : 256));
             int64_t want = ceil_div(n, static_cast<int64_t>(row_lanes) * 8);  // eight rows per thread or more,
             if (want > 512) want = 512;                                          // two workgroups per compute unit at most
             groups = static_cast<int>(want < groups ? (want < 1 ? 1 : want) : groups);
-            const size_t lds = sizeof(float) * 2 * row_lanes * C;
-            if (quads)
-                hipLaunchKernelGGL(attn_scores_bwd_rows_kernel<4>, dim3(static_cast<unsigned>(groups)), dim3(256), lds, s,
-                                   dfeat, part, del, der, feat, attn_l, attn_r, n, static_cast<int>(H), static_cast<int>(D));
+            const size_t lds = sizeof(float) * 2 * 256 * vec;
+            const dim3 grid(static_cast<unsigned>(groups), static_cast<unsigned>(chunks));
+            if (vec == 4)
+                hipLaunchKernelGGL(attn_scores_bwd_rows_kernel<4>, grid, dim3(256), lds, s, dfeat, part, del, der, feat,
+                                   attn_l, attn_r, n, static_cast<int>(H), static_cast<int>(D));
+            else if (vec == 2)
+                hipLaunchKernelGGL(attn_scores_bwd_rows_kernel<2>, grid, dim3(256), lds, s, dfeat, part, del, der, feat,
+                                   attn_l, attn_r, n, static_cast<int>(H), static_cast<int>(D));
             else
-                hipLaunchKernelGGL(attn_scores_bwd_rows_kernel<1>, dim3(static_cast<unsigned>(groups)), dim3(256), lds, s,
-                                   dfeat, part, del, der, feat, attn_l, attn_r, n, static_cast<int>(H), static_cast<int>(D));
-        } else {
-            const int tpb = static_cast<int>((256 / H) * H);
-            const int vec4 = (D % kDChunk == 0) && (bits & 15) == 0;
-            hipLaunchKernelGGL(attn_scores_bwd_kernel,
-                               dim3(static_cast<unsigned>(groups), static_cast<unsigned>(ceil_div(D, kDChunk))),
-                               dim3(tpb), 0, s, dfeat, part, del, der, feat, attn_l, attn_r, n, static_cast<int>(H),
-                               static_cast<int>(D), vec4);
+                hipLaunchKernelGGL(attn_scores_bwd_rows_kernel<1>, grid, dim3(256), lds, s, dfeat, part, del, der, feat,
+                                   attn_l, attn_r, n, static_cast<int>(H), static_cast<int>(D));
         }
     }
     hipLaunchKernelGGL(attn_scores_finish_kernel, dim3(static_cast<unsigned>(ceil_div(2 * H * D, 16))), dim3(1024), 0,

@@ -36,42 +36,78 @@ __device__ __forceinline__ float bn_shift(const float* __restrict__ x, int64_t f
     return fmaxf(fminf(a, b), fminf(fmaxf(a, b), d));
 }
 
-// Thread t of 256 owns column quad t % cq and row lane t / cq (row lanes = 256 / cq; threads beyond are idle).
-// DYNAMIC LDS: 2 * row_lanes * C floats.
+// Column layout of the reductions: a thread owns VEC consecutive columns (VEC = 4, 2 or 1: the widest that divides C
+// and keeps the loads aligned) of one row lane.  gridDim.y cuts the C / VEC column groups into chunks of at most
+// 256; a workgroup has 256 / (groups of its chunk) row lanes (threads beyond are idle).
+struct BnChunk {
+    int g0, cg, cw, row_lanes;  // first column group, groups and columns of the chunk, row lanes of its workgroups
+};
+__host__ __device__ inline BnChunk bn_chunk(int C, int vec, int chunk) {
+    const int cg_all = C / vec;
+    BnChunk k;
+    k.g0 = chunk * 256;
+    k.cg = cg_all - k.g0 < 256 ? cg_all - k.g0 : 256;
+    k.cw = k.cg * vec;
+    k.row_lanes = 256 / k.cg;
+    return k;
+}
+
+template <int VEC>
+struct BnVec {
+    typedef float T __attribute__((ext_vector_type(VEC)));
+    static __device__ __forceinline__ void load(const float* p, float* v) {
+        const T t = __builtin_nontemporal_load(reinterpret_cast<const T*>(p));
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) v[i] = t[i];
+    }
+    static __device__ __forceinline__ void store(float* p, const float* v) {
+        T t;
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) t[i] = v[i];
+        __builtin_nontemporal_store(t, reinterpret_cast<T*>(p));
+    }
+};
+template <>
+struct BnVec<1> {
+    static __device__ __forceinline__ void load(const float* p, float* v) { v[0] = __builtin_nontemporal_load(p); }
+    static __device__ __forceinline__ void store(float* p, const float* v) { __builtin_nontemporal_store(v[0], p); }
+};
+
+// DYNAMIC LDS: 2 * 256 * VEC floats (2 * row_lanes * columns of the chunk at most).
 // MODE 0: partial = (mean, sum of squared deviations) of the workgroup's rows, from s1 = sum(x - k), s2 = sum((x - k)^2).
 // MODE 1: s1 = sum(dy'), s2 = sum(dy' * xhat), dy' = dy where the forward output was positive (relu) else 0.
-template <int MODE>
+template <int MODE, int VEC>
 __global__ __launch_bounds__(256) void bn_reduce_kernel(const float* __restrict__ x, const float* __restrict__ dy,
                                                         const float* __restrict__ mean, const float* __restrict__ rstd,
                                                         const float* __restrict__ gamma, const float* __restrict__ beta,
                                                         int64_t rows, int C, int relu, float* __restrict__ partial) {
-    extern __shared__ float red[];  // [2][row_lanes][C]
-    const int cq = C >> 2;
-    const int row_lanes = 256 / cq;
-    const int quad = threadIdx.x % cq, rl = threadIdx.x / cq;
+    extern __shared__ float red[];  // [2][row_lanes][cw]
+    const BnChunk ck = bn_chunk(C, VEC, blockIdx.y);
+    const int row_lanes = ck.row_lanes, cw = ck.cw;
+    const int grp = threadIdx.x % ck.cg, rl = threadIdx.x / ck.cg;
     const bool active = rl < row_lanes;
-    const int c0 = quad << 2;
-    float k[4] = {0.f, 0.f, 0.f, 0.f}, a[4] = {0.f, 0.f, 0.f, 0.f}, b[4] = {0.f, 0.f, 0.f, 0.f}, mu[4] = {0.f, 0.f, 0.f, 0.f},
-          rs[4] = {0.f, 0.f, 0.f, 0.f};
-    const int64_t first_row = static_cast<int64_t>(blockIdx.x) * row_lanes;  // < rows (host: eight rows per thread or more)
-    if (MODE == 0) {
+    const int c0 = (ck.g0 + grp) * VEC;
+    float k[VEC], a[VEC], b[VEC], mu[VEC], rs[VEC], s1[VEC], s2[VEC];
+    // The number of workgroups comes from the chunk with the fewest row lanes; in a narrower chunk (more row lanes)
+    // the last workgroups may have no row at all: they read nothing and hand in an empty partial.
+    const int64_t first_row = static_cast<int64_t>(blockIdx.x) * row_lanes;
+    const bool has_rows = first_row < rows;
 #pragma unroll
-        for (int i = 0; i < 4; ++i) k[i] = bn_shift(x, first_row, rows, C, c0 + i);
-    } else {
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
+    for (int i = 0; i < VEC; ++i) {
+        k[i] = a[i] = b[i] = mu[i] = rs[i] = s1[i] = s2[i] = 0.0f;
+        if (MODE == 0) {
+            if (has_rows) k[i] = bn_shift(x, first_row, rows, C, c0 + i);
+        } else {
             mu[i] = mean[c0 + i];
             rs[i] = rstd[c0 + i];
             a[i] = rs[i] * gamma[c0 + i];
             b[i] = beta[c0 + i];
         }
     }
-    float s1[4] = {0.f, 0.f, 0.f, 0.f}, s2[4] = {0.f, 0.f, 0.f, 0.f};
     const int64_t step = static_cast<int64_t>(gridDim.x) * row_lanes;
-    auto take = [&](const f32x4 xv, const f32x4 dv) {
-        const float xs[4] = {xv.x, xv.y, xv.z, xv.w}, ds[4] = {dv.x, dv.y, dv.z, dv.w};
+    auto take = [&](const float* xs, const float* ds) {
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
+        for (int i = 0; i < VEC; ++i) {
             if (MODE == 0) {
                 const float d = xs[i] - k[i];
                 s1[i] += d;
@@ -88,49 +124,54 @@ __global__ __launch_bounds__(256) void bn_reduce_kernel(const float* __restrict_
     if (active) {
         int64_t r = static_cast<int64_t>(blockIdx.x) * row_lanes + rl;
         for (; r + 3 * step < rows; r += 4 * step) {  // four rows in flight per thread
-            f32x4 xv[4], dv[4];
+            float xv[4][VEC], dv[4][VEC];
 #pragma unroll
             for (int u = 0; u < 4; ++u) {
-                xv[u] = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(x + (r + u * step) * C + c0));
-                dv[u] = MODE == 1 ? __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(dy + (r + u * step) * C + c0))
-                                  : f32x4{0.f, 0.f, 0.f, 0.f};
+                BnVec<VEC>::load(x + (r + u * step) * C + c0, xv[u]);
+                if (MODE == 1) BnVec<VEC>::load(dy + (r + u * step) * C + c0, dv[u]);
             }
 #pragma unroll
             for (int u = 0; u < 4; ++u) take(xv[u], dv[u]);
         }
         for (; r < rows; r += step) {
-            const f32x4 xv = *reinterpret_cast<const f32x4*>(x + r * C + c0);
-            const f32x4 dv = MODE == 1 ? *reinterpret_cast<const f32x4*>(dy + r * C + c0) : f32x4{0.f, 0.f, 0.f, 0.f};
+            float xv[VEC], dv[VEC];
+            BnVec<VEC>::load(x + r * C + c0, xv);
+            if (MODE == 1) BnVec<VEC>::load(dy + r * C + c0, dv);
             take(xv, dv);
         }
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            red[rl * C + c0 + i] = s1[i];
-            red[(row_lanes + rl) * C + c0 + i] = s2[i];
+        for (int i = 0; i < VEC; ++i) {
+            red[rl * cw + grp * VEC + i] = s1[i];
+            red[(row_lanes + rl) * cw + grp * VEC + i] = s2[i];
         }
     }
     __syncthreads();
+    float* mine = partial + static_cast<int64_t>(blockIdx.x) * 2 * C + ck.g0 * VEC;  // this chunk's columns of slab b
     if (MODE == 0) {
-        // rows of this workgroup: those whose index modulo (gridDim.x row_lanes) lies in its row_lanes-wide window
         const int64_t nb = bn_group_rows(rows, row_lanes, gridDim.x, blockIdx.x);
-        for (int c = threadIdx.x; c < C; c += 256) {  // the row lanes in order
+        for (int c = threadIdx.x; c < cw; c += 256) {  // the row lanes in order
             float t1 = 0.0f, t2 = 0.0f;
             for (int l = 0; l < row_lanes; ++l) {
-                t1 += red[l * C + c];
-                t2 += red[(row_lanes + l) * C + c];
+                t1 += red[l * cw + c];
+                t2 += red[(row_lanes + l) * cw + c];
+            }
+            if (!has_rows) {  // nb == 0: skipped by the merge
+                mine[c] = 0.0f;
+                mine[C + c] = 0.0f;
+                continue;
             }
             const float n = static_cast<float>(nb);
             const float m2 = t2 - t1 * (t1 / n);
-            partial[static_cast<int64_t>(blockIdx.x) * 2 * C + c] = bn_shift(x, first_row, rows, C, c) + t1 / n;
-            partial[static_cast<int64_t>(blockIdx.x) * 2 * C + C + c] = m2 > 0.0f ? m2 : 0.0f;
+            mine[c] = bn_shift(x, first_row, rows, C, ck.g0 * VEC + c) + t1 / n;
+            mine[C + c] = m2 > 0.0f ? m2 : 0.0f;
         }
         return;
     }
-    for (int j = threadIdx.x; j < 2 * C; j += 256) {  // column j of s1 (j < C) or s2: the row lanes in order
-        const int which = j / C, c = j - which * C;
+    for (int j = threadIdx.x; j < 2 * cw; j += 256) {  // (which, column of the chunk): the row lanes in order
+        const int which = j / cw, c = j - which * cw;
         float t = 0.0f;
-        for (int l = 0; l < row_lanes; ++l) t += red[(which * row_lanes + l) * C + c];
-        partial[static_cast<int64_t>(blockIdx.x) * 2 * C + j] = t;
+        for (int l = 0; l < row_lanes; ++l) t += red[(which * row_lanes + l) * cw + c];
+        mine[which * C + c] = t;
     }
 }
 
@@ -139,7 +180,7 @@ __global__ __launch_bounds__(256) void bn_reduce_kernel(const float* __restrict_
 // MODE 1: out1 = sum of the first partials (dbeta), out2 = sum of the second (dgamma).
 template <int MODE>
 __global__ __launch_bounds__(1024) void bn_finish_kernel(const float* __restrict__ partial, int groups, int C, int64_t rows,
-                                                         int row_lanes, float eps, float* __restrict__ out1,
+                                                         int vec, float eps, float* __restrict__ out1,
                                                          float* __restrict__ out2, float* __restrict__ out3) {
     __shared__ float red[3][64][16];
     const int e = threadIdx.x & 15, sl = threadIdx.x >> 4;
@@ -153,7 +194,9 @@ __global__ __launch_bounds__(1024) void bn_finish_kernel(const float* __restrict
         t2 = t2 + m2b + d * d * (n * (nb / tot));
         n = tot;
     };
-    // rows of workgroup g (bn_group_rows): whole periods, plus its window of the last, partial one
+    // rows of workgroup g (bn_group_rows, with the row lanes of this column's chunk): whole periods, plus its window
+    // of the last, partial one
+    const int row_lanes = bn_chunk(C, vec, (c < C ? c : 0) / vec / 256).row_lanes;
     const int64_t period = static_cast<int64_t>(groups) * row_lanes;
     const int64_t whole = rows / period * row_lanes, tail = rows % period;
     if (c < C)
@@ -202,7 +245,7 @@ __global__ __launch_bounds__(1024) void bn_finish_kernel(const float* __restrict
 
 // y = (x - mean) * (rstd * gamma) + beta, ReLU if asked; optionally max|y| / 127 into scale_out (pre-zeroed).
 // Backward (BWD): dx = (rstd * gamma) * (dy' - dbeta / n - xhat * dgamma / n).
-template <bool BWD>
+template <bool BWD, int VEC>
 __global__ __launch_bounds__(256) void bn_apply_kernel(float* __restrict__ out, const float* __restrict__ x,
                                                        const float* __restrict__ dy, const float* __restrict__ mean,
                                                        const float* __restrict__ rstd, const float* __restrict__ gamma,
@@ -220,51 +263,85 @@ __global__ __launch_bounds__(256) void bn_apply_kernel(float* __restrict__ out, 
         par[5 * C + c] = BWD ? dgamma[c] * inv_n : 0.0f;
     }
     __syncthreads();
-    const int cq = C >> 2;
-    const int64_t n4 = rows * cq;
+    const int cg = C / VEC;
+    const int64_t nv = rows * cg;
     const int64_t tid = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
     const int64_t nthr = static_cast<int64_t>(gridDim.x) * blockDim.x;
-    int quad = static_cast<int>(tid % cq);
-    const int qstep = static_cast<int>(nthr % cq);
+    int grp = static_cast<int>(tid % cg);
+    const int gstep = static_cast<int>(nthr % cg);
     float m = 0.0f;
-    for (int64_t i = tid; i < n4; i += nthr) {
-        const int c0 = quad << 2;
-        const f32x4 xv = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(x) + i);
-        const float xs[4] = {xv.x, xv.y, xv.z, xv.w};
-        float o[4];
+    for (int64_t i = tid; i < nv; i += nthr) {
+        const int c0 = grp * VEC;
+        float xs[VEC], ds[VEC], o[VEC];
+        BnVec<VEC>::load(x + i * VEC, xs);
         if (!BWD) {
 #pragma unroll
-            for (int k = 0; k < 4; ++k) {
+            for (int k = 0; k < VEC; ++k) {
                 float y = (xs[k] - par[c0 + k]) * par[2 * C + c0 + k] + par[3 * C + c0 + k];
                 if (relu && !(y > 0.0f)) y = 0.0f;
                 o[k] = y;
                 m = fmaxf(m, fabsf(y));
             }
         } else {
-            const f32x4 dv = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(dy) + i);
-            const float ds[4] = {dv.x, dv.y, dv.z, dv.w};
+            BnVec<VEC>::load(dy + i * VEC, ds);
 #pragma unroll
-            for (int k = 0; k < 4; ++k) {
+            for (int k = 0; k < VEC; ++k) {
                 const float c = xs[k] - par[c0 + k];
                 float g = ds[k];
                 if (relu && !(c * par[2 * C + c0 + k] + par[3 * C + c0 + k] > 0.0f)) g = 0.0f;
                 o[k] = par[2 * C + c0 + k] * (g - par[4 * C + c0 + k] - (c * par[C + c0 + k]) * par[5 * C + c0 + k]);
             }
         }
-        __builtin_nontemporal_store(f32x4{o[0], o[1], o[2], o[3]}, reinterpret_cast<f32x4*>(out) + i);
-        quad += qstep;
-        if (quad >= cq) quad -= cq;
+        BnVec<VEC>::store(out + i * VEC, o);
+        grp += gstep;
+        if (grp >= cg) grp -= cg;
     }
     if (!BWD && scale_out) block_absmax_to_global(m / 127.0f, scale_out);
 }
 
-static int bn_groups(int64_t rows, int64_t C) {
-    const int64_t row_lanes = 256 / (C >> 2);
+constexpr int kBnMaxCols = 2048;
+
+// the widest vector that divides the row length and keeps every row's loads aligned
+static int bn_vec(int64_t C, uintptr_t addr_bits) {
+    return (C % 4 == 0 && (addr_bits & 15) == 0) ? 4 : (C % 2 == 0 && (addr_bits & 7) == 0) ? 2 : 1;
+}
+
+// Workgroups of the reductions; sized for the narrowest vector so that the workspace does not depend on alignment
+static int bn_groups(int64_t rows, int64_t C, int vec) {
+    const int64_t cg = C / vec;
+    const int64_t row_lanes = 256 / (cg < 256 ? cg : 256);
     const int64_t g = ceil_div(rows, row_lanes * 8);  // at least eight rows per thread
     return static_cast<int>(g < 1 ? 1 : (g < kBnMaxGroups ? g : kBnMaxGroups));
 }
 
-static bool bn_shape_ok(int64_t rows, int64_t C) { return rows > 0 && C >= 4 && C <= 1024 && (C & 3) == 0; }
+static bool bn_shape_ok(int64_t rows, int64_t C) { return rows > 0 && C >= 1 && C <= kBnMaxCols; }
+
+template <int MODE>
+static void bn_launch_reduce(int vec, dim3 grid, hipStream_t s, const float* x, const float* dy, const float* mean,
+                             const float* rstd, const float* gamma, const float* beta, int64_t rows, int C, int relu,
+                             float* partial) {
+    const size_t lds = sizeof(float) * 2 * 256 * vec;
+    if (vec == 4)
+        hipLaunchKernelGGL((bn_reduce_kernel<MODE, 4>), grid, dim3(256), lds, s, x, dy, mean, rstd, gamma, beta, rows, C, relu, partial);
+    else if (vec == 2)
+        hipLaunchKernelGGL((bn_reduce_kernel<MODE, 2>), grid, dim3(256), lds, s, x, dy, mean, rstd, gamma, beta, rows, C, relu, partial);
+    else
+        hipLaunchKernelGGL((bn_reduce_kernel<MODE, 1>), grid, dim3(256), lds, s, x, dy, mean, rstd, gamma, beta, rows, C, relu, partial);
+}
+
+template <bool BWD>
+static void bn_launch_apply(int vec, hipStream_t s, float* out, const float* x, const float* dy, const float* mean,
+                            const float* rstd, const float* gamma, const float* beta, const float* dbeta,
+                            const float* dgamma, int64_t rows, int C, int relu, float* scale_out) {
+    const dim3 grid(grid_for(rows * (C / vec), 256));
+    const size_t lds = sizeof(float) * 6 * C;
+    if (vec == 4)
+        hipLaunchKernelGGL((bn_apply_kernel<BWD, 4>), grid, dim3(256), lds, s, out, x, dy, mean, rstd, gamma, beta, dbeta, dgamma, rows, C, relu, scale_out);
+    else if (vec == 2)
+        hipLaunchKernelGGL((bn_apply_kernel<BWD, 2>), grid, dim3(256), lds, s, out, x, dy, mean, rstd, gamma, beta, dbeta, dgamma, rows, C, relu, scale_out);
+    else
+        hipLaunchKernelGGL((bn_apply_kernel<BWD, 1>), grid, dim3(256), lds, s, out, x, dy, mean, rstd, gamma, beta, dbeta, dgamma, rows, C, relu, scale_out);
+}
 
 }  // namespace tango
 
@@ -274,7 +351,7 @@ extern "C" {
 
 size_t tango_batchnorm_workspace(int64_t rows, int64_t cols) {
     if (!bn_shape_ok(rows, cols)) return 0;
-    return static_cast<size_t>(bn_groups(rows, cols)) * 2 * cols * sizeof(float);
+    return static_cast<size_t>(kBnMaxGroups) * 2 * cols * sizeof(float);
 }
 
 int tango_batchnorm_fwd_f32(float* y, float* mean, float* var, float* rstd, float* scale_y, const float* x,
@@ -284,22 +361,21 @@ int tango_batchnorm_fwd_f32(float* y, float* mean, float* var, float* rstd, floa
     if (rows == 0 || cols == 0) return TANGO_OK;
     if (!bn_shape_ok(rows, cols)) return TANGO_ERR_UNSUPPORTED;
     if (!y || !mean || !var || !rstd || !x || !gamma || !beta) return TANGO_ERR_INVALID_ARG;
-    if (((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(y)) & 15) != 0) return TANGO_ERR_UNSUPPORTED;
+    if (((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(y)) & 3) != 0) return TANGO_ERR_INVALID_ARG;
     const size_t need = tango_batchnorm_workspace(rows, cols);
     if (!workspace || workspace_bytes < need || (reinterpret_cast<uintptr_t>(workspace) & 15) != 0)
         return TANGO_ERR_WORKSPACE;
     hipStream_t s = as_stream(stream);
     const int C = static_cast<int>(cols);
-    const int groups = bn_groups(rows, cols);
-    const int row_lanes = 256 / (C >> 2);
+    const int vec = bn_vec(cols, reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(y));
+    const int groups = bn_groups(rows, cols, vec);
+    const dim3 rgrid(groups, static_cast<unsigned>(ceil_div(cols / vec, 256)));
     float* partial = static_cast<float*>(workspace);
     if (scale_y) fill_u32(scale_y, 0u, 1, s);
-    hipLaunchKernelGGL(bn_reduce_kernel<0>, dim3(groups), dim3(256), sizeof(float) * 2 * row_lanes * C, s, x, nullptr,
-                       nullptr, nullptr, nullptr, nullptr, rows, C, 0, partial);
-    hipLaunchKernelGGL(bn_finish_kernel<0>, dim3((C + 15) / 16), dim3(1024), 0, s, partial, groups, C, rows, row_lanes, eps,
-                       mean, var, rstd);
-    hipLaunchKernelGGL(bn_apply_kernel<false>, dim3(grid_for(rows * (cols >> 2), 256)), dim3(256), sizeof(float) * 6 * C, s,
-                       y, x, nullptr, mean, rstd, gamma, beta, nullptr, nullptr, rows, C, relu, scale_y);
+    bn_launch_reduce<0>(vec, rgrid, s, x, nullptr, nullptr, nullptr, nullptr, nullptr, rows, C, 0, partial);
+    hipLaunchKernelGGL(bn_finish_kernel<0>, dim3((C + 15) / 16), dim3(1024), 0, s, partial, groups, C, rows, vec, eps, mean, var,
+                       rstd);
+    bn_launch_apply<false>(vec, s, y, x, nullptr, mean, rstd, gamma, beta, nullptr, nullptr, rows, C, relu, scale_y);
     return launch_status();
 }
 
@@ -310,22 +386,21 @@ int tango_batchnorm_bwd_f32(float* dx, float* dgamma, float* dbeta, const float*
     if (rows == 0 || cols == 0) return TANGO_OK;
     if (!bn_shape_ok(rows, cols)) return TANGO_ERR_UNSUPPORTED;
     if (!dx || !dgamma || !dbeta || !dy || !x || !mean || !rstd || !gamma || !beta) return TANGO_ERR_INVALID_ARG;
-    if (((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(dy) | reinterpret_cast<uintptr_t>(dx)) & 15) != 0)
-        return TANGO_ERR_UNSUPPORTED;
+    const uintptr_t bits = reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(dy) | reinterpret_cast<uintptr_t>(dx);
+    if ((bits & 3) != 0) return TANGO_ERR_INVALID_ARG;
     const size_t need = tango_batchnorm_workspace(rows, cols);
     if (!workspace || workspace_bytes < need || (reinterpret_cast<uintptr_t>(workspace) & 15) != 0)
         return TANGO_ERR_WORKSPACE;
     hipStream_t s = as_stream(stream);
     const int C = static_cast<int>(cols);
-    const int groups = bn_groups(rows, cols);
-    const int row_lanes = 256 / (C >> 2);
+    const int vec = bn_vec(cols, bits);
+    const int groups = bn_groups(rows, cols, vec);
+    const dim3 rgrid(groups, static_cast<unsigned>(ceil_div(cols / vec, 256)));
     float* partial = static_cast<float*>(workspace);
-    hipLaunchKernelGGL(bn_reduce_kernel<1>, dim3(groups), dim3(256), sizeof(float) * 2 * row_lanes * C, s, x, dy, mean,
-                       rstd, gamma, beta, rows, C, relu, partial);
-    hipLaunchKernelGGL(bn_finish_kernel<1>, dim3((C + 15) / 16), dim3(1024), 0, s, partial, groups, C, rows, row_lanes, 0.0f,
-                       dbeta, dgamma, nullptr);
-    hipLaunchKernelGGL(bn_apply_kernel<true>, dim3(grid_for(rows * (cols >> 2), 256)), dim3(256), sizeof(float) * 6 * C, s,
-                       dx, x, dy, mean, rstd, gamma, beta, dbeta, dgamma, rows, C, relu, nullptr);
+    bn_launch_reduce<1>(vec, rgrid, s, x, dy, mean, rstd, gamma, beta, rows, C, relu, partial);
+    hipLaunchKernelGGL(bn_finish_kernel<1>, dim3((C + 15) / 16), dim3(1024), 0, s, partial, groups, C, rows, vec, 0.0f, dbeta,
+                       dgamma, nullptr);
+    bn_launch_apply<true>(vec, s, dx, x, dy, mean, rstd, gamma, beta, dbeta, dgamma, rows, C, relu, nullptr);
     return launch_status();
 }
 

@@ -798,6 +798,32 @@ def quantize_padded(t, scale=None, round_mode=ROUND_RNE, noise=None, seed=0, off
     return buf[:, :cols], scale
 
 
+def pad_heads(D):
+    """Columns per head of the int8 copy of an [n, H, D] tensor: D itself, or the next multiple of 16 when heads
+    of at least 24 columns would otherwise leave the rows without 16-byte alignment (250 -> 256): the gathers of
+    the aggregation and of the SDDMM then run on aligned 16-byte pieces instead of single bytes."""
+    return (D + 15) // 16 * 16 if D >= 24 and D % 16 != 0 else D
+
+
+def quantize_heads(t, scale=None, **kw):
+    """``quantize`` for a 3-D [n, H, D] tensor with every head zero-padded to ``pad_heads(D)`` columns: returns
+    (int8 [n, H, pad_heads(D)], scale).  The zeros add nothing to a dot product or an aggregation."""
+    if t.dim() != 3 or pad_heads(t.size(2)) == t.size(2):
+        return quantize(t, scale, **kw)
+    n, H, D = t.shape
+    Dp = pad_heads(D)
+    t = t if t.is_contiguous() else t.contiguous()
+    if scale is None:
+        scale = cuda_kernels.get_scale(t)
+    q, scale = quantize_padded(t.view(n * H, D), scale, align=16, **kw)  # the [n H, D] view of an [n H, Dp] buffer
+    return q.as_strided((n, H, Dp), (H * Dp, Dp, 1)), scale
+
+
+def unpad_heads(t, D):
+    """[n, H, D] contiguous from a result computed on head-padded operands."""
+    return t if t.size(-1) == D else t[..., :D].contiguous()
+
+
 def mySDDMM_int8(g, op, U, V, scaleU, scaleV, isReduce, reverse=False):
     """cuda/kernels.py:33-59."""
     if reverse:

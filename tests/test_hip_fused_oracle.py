@@ -133,3 +133,57 @@ def test_copy_u_with_source_multiplier_matches_oracle(orc, n, e, F):
     dZq = orc.quantize(dZ, s_dZ)
     rip, rix, _ = (host(t) for t in g.adj_csr)
     assert np.array_equal(host(tN.grad), orc.spmm_csr_copy_u_ex(rip, rix, dZq, s_dZ, row_scale=mul))
+
+
+@pytest.mark.parametrize("n,e,H,D", [(500, 8000, 3, 250), (300, 5000, 2, 40), (400, 6000, 4, 24)])
+def test_unaligned_head_widths_run_on_padded_heads(orc, n, e, H, D):
+    """Head widths that are not multiples of 16 (the reference's arxiv GAT trains with 3 heads of 250): the int8
+    copies are zero-padded per head, the SDDMM dot and the u_mul_e aggregation run on aligned rows, and every
+    result equals the oracle's on the unpadded operands, forward and backward."""
+    from tango_amd import config
+    from tango_amd.SDDMM import sddmm_u_dot_v
+    from tango_amd.SPMM import spmm_u_mul_e
+    from tango_amd.kernels import pad_heads, quantize_heads
+    assert pad_heads(D) % 16 == 0 and pad_heads(D) != D and pad_heads(16) == 16 and pad_heads(5) == 5
+    rng = np.random.default_rng(D)
+    src, dst = rand_graph(rng, n, e)
+    g = make_graph(src, dst, n)
+    U, V = (rng.standard_normal((n, H, D)).astype(np.float32) for _ in range(2))
+    q, s = quantize_heads(dev(U))
+    assert q.shape == (n, H, pad_heads(D)) and np.array_equal(host(q)[..., :D], orc.quantize(U, orc.absmax_scale(U)))
+    assert not host(q)[..., D:].any()
+    old = config.grad_round_mode
+    config.grad_round_mode = "rne"
+    try:
+        # SDDMM dot: forward, and both backward aggregations with dZ as edge values
+        tU, tV = dev(U).requires_grad_(), dev(V).requires_grad_()
+        out = sddmm_u_dot_v.apply(g, tU, tV)
+        dZ = rng.standard_normal((e, H, 1)).astype(np.float32)
+        out.backward(dev(dZ))
+        sU, sV = orc.absmax_scale(U), orc.absmax_scale(V)
+        Uq, Vq = orc.quantize(U, sU), orc.quantize(V, sV)
+        want, _ = orc.sddmm_dot(src, dst, Uq, Vq, sU, sV)
+        assert np.array_equal(host(out).reshape(e, H), want)
+        s_dZ = orc.absmax_scale(dZ)
+        dZq = orc.quantize(dZ, s_dZ)
+        cip, cix, ceid = (host(t) for t in g.adj_csc)
+        rip, rix, reid = (host(t) for t in g.adj_csr)
+        assert np.array_equal(host(tV.grad), orc.spmm_csr_u_mul_e_ex(cip, cix, ceid, Uq, dZq, s_dZ, scale2=sU, edge_major=True))
+        assert np.array_equal(host(tU.grad), orc.spmm_csr_u_mul_e_ex(rip, rix, reid, Vq, dZq, s_dZ, scale2=sV, edge_major=True))
+        # u_mul_e: forward, dN (reverse aggregation) and dE (dot of the features with dOut)
+        E = rng.random((e, H, 1)).astype(np.float32)
+        tN, tE = dev(U).requires_grad_(), dev(E).requires_grad_()
+        agg = spmm_u_mul_e.apply(g, tN, tE)
+        dOut = rng.standard_normal((n, H, D)).astype(np.float32)
+        agg.backward(dev(dOut))
+        sE = orc.absmax_scale(E)
+        Eq = orc.quantize(E, sE)
+        assert agg.shape == (n, H, D) and agg.is_contiguous()
+        assert np.array_equal(host(agg), orc.spmm_csr_u_mul_e_ex(cip, cix, ceid, Uq, Eq, sU, scale2=sE, edge_major=True))
+        s_dO = orc.absmax_scale(dOut)
+        dOq = orc.quantize(dOut, s_dO)
+        assert np.array_equal(host(tN.grad), orc.spmm_csr_u_mul_e_ex(rip, rix, reid, dOq, Eq, s_dO, scale2=sE, edge_major=True))
+        wantE, _ = orc.sddmm_dot(src, dst, Uq, dOq, sU, s_dO)
+        assert np.array_equal(host(tE.grad).reshape(e, H), wantE)
+    finally:
+        config.grad_round_mode = old

@@ -183,13 +183,14 @@ def test_cross_entropy_matches_torch(rows, classes):
 
 
 @pytest.mark.parametrize("n,H,D", [(1000, 8, 16), (333, 3, 5), (50, 1, 64), (2049, 12, 20), (7, 70, 4),
-                                   (70000, 8, 16), (169343, 1, 40), (3001, 1, 41), (500, 3, 101), (300, 2, 640)])
+                                   (70000, 8, 16), (169343, 1, 40), (3001, 1, 41), (500, 3, 101), (300, 2, 640), (2000, 3, 250)])
 def test_attn_scores_match_torch(K, n, H, D):
     """fp32 kernel against the torch expression it replaces; only the summation order differs.  The form that
     also hands out the scales (a few large workgroups walking the items with a grid stride; the last case has
     more items than threads in that launch) writes the same el / er bit for bit, and its scales are
     max|.| / 127 of what it wrote.  The backward reads rows the way they lie in memory (column quads when D is a
-    multiple of 4, single columns for rows of at most 256 floats); the last two cases run its thread-per-head form."""
+    multiple of 4, pairs when it is even, else single columns; rows of more than 256 such groups are cut into
+    column chunks: the last three cases)."""
     g = torch.Generator().manual_seed(n + H)
     feat = torch.randn(n, H, D, generator=g).cuda()
     al = torch.randn(1, H, D, generator=g).cuda()
@@ -482,7 +483,8 @@ def _bn_f64(x, gamma, beta, eps, relu, dy=None, mask=None):
 
 
 @pytest.mark.parametrize("rows,cols,relu", [(5000, 128, True), (169343, 128, True), (777, 768, False), (33, 4, True),
-                                            (2, 1024, True), (1001, 40, False), (4096, 256, True), (20000, 64, True)])
+                                            (2, 1024, True), (1001, 40, False), (4096, 256, True), (20000, 64, True),
+                                            (3000, 750, True), (999, 7, False), (640, 1538, True), (500, 2048, True)])
 def test_batchnorm_act_c_abi(K, rows, cols, relu):
     """The two entry points against float64 formulas (means far from zero, so a variance from a plain sum of
     squares would fail; one case with outliers in the rows the shifted sums take their shifts from), and the scale
@@ -539,7 +541,7 @@ def test_batchnorm_act_c_abi(K, rows, cols, relu):
 
 
 @pytest.mark.parametrize("rows,cols,act", [(3000, 128, "relu"), (500, 64, None), (700, 36, "relu"), (900, 128, "elu"),
-                                           (400, 30, "relu")])
+                                           (400, 30, "relu"), (600, 750, "relu"), (300, 5, None)])
 def test_batchnorm_module_matches_torch(rows, cols, act):
     """The module against torch.nn.BatchNorm1d + activation: outputs, gradients, running statistics over two
     training steps, the evaluation-mode pass and the state dict."""
@@ -577,10 +579,10 @@ def test_batchnorm_module_matches_torch(rows, cols, act):
 
 def test_batchnorm_rejects_unsupported_shapes(K):
     L = K._L
-    assert L.tango_batchnorm_workspace(100, 6) == 0 and L.tango_batchnorm_workspace(100, 2048) == 0
-    x = torch.zeros(100, 6, device="cuda")
+    assert L.tango_batchnorm_workspace(100, 6) > 0 and L.tango_batchnorm_workspace(100, 4096) == 0
+    x = torch.zeros(100, 8, device="cuda")
     p = x.data_ptr()
     import ctypes
-    assert L.tango_batchnorm_fwd_f32(p, p, p, p, None, p, p, p, 100, 6, ctypes.c_float(1e-5), 1, p, 1 << 20, None) == -2
+    assert L.tango_batchnorm_fwd_f32(p, p, p, p, None, p, p, p, 100, 4096, ctypes.c_float(1e-5), 1, p, 1 << 30, None) == -2
     assert L.tango_batchnorm_fwd_f32(p, p, p, p, None, p, p, p, 100, 8, ctypes.c_float(1e-5), 1, None, 0, None) == -4
     assert L.tango_batchnorm_fwd_f32(p, p, p, p, None, p, p, p, 0, 8, ctypes.c_float(1e-5), 1, None, 0, None) == 0
