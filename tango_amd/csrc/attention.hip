@@ -64,6 +64,60 @@ __global__ __launch_bounds__(SCALES ? 1024 : 256) void attn_scores_fwd_kernel(
     }
 }
 
+// Wide heads (D >= 128): one wavefront per (node, head) item, its lanes striding over the head's columns VEC floats
+// at a time (consecutive bytes per load instruction, where a thread per item reads D floats at a stride of D floats),
+// then a butterfly over the lanes: a fixed order.  Launched like attn_scores_fwd_kernel.
+template <bool SCALES, int VEC>
+__global__ __launch_bounds__(SCALES ? 1024 : 256) void attn_scores_fwd_wide_kernel(
+    float* __restrict__ el, float* __restrict__ er, float* __restrict__ scale_el, float* __restrict__ scale_er,
+    const float* __restrict__ feat, const float* __restrict__ al, const float* __restrict__ ar, int64_t total,
+    int H, int D) {
+    typedef float fvec __attribute__((ext_vector_type(VEC == 1 ? 2 : VEC)));  // (unused for VEC == 1)
+    const int lane = threadIdx.x & 63;
+    const int64_t nwaves = static_cast<int64_t>(gridDim.x) * (blockDim.x >> 6);
+    float ml = 0.0f, mr = 0.0f;
+    for (int64_t i = static_cast<int64_t>(blockIdx.x) * (blockDim.x >> 6) + (threadIdx.x >> 6); i < total; i += nwaves) {
+        const int h = static_cast<int>(i % H);
+        const float* f = feat + i * D;
+        const float* a = al + static_cast<int64_t>(h) * D;
+        const float* b = ar + static_cast<int64_t>(h) * D;
+        float sl = 0.0f, sr = 0.0f;
+        for (int d = lane * VEC; d < D; d += 64 * VEC) {
+            if (VEC > 1) {
+                const fvec x = __builtin_nontemporal_load(reinterpret_cast<const fvec*>(f + d));
+                const fvec u = *reinterpret_cast<const fvec*>(a + d);
+                const fvec v = *reinterpret_cast<const fvec*>(b + d);
+#pragma unroll
+                for (int k = 0; k < VEC; ++k) {
+                    sl += x[k] * u[k];
+                    sr += x[k] * v[k];
+                }
+            } else {
+                sl += f[d] * a[d];
+                sr += f[d] * b[d];
+            }
+        }
+#pragma unroll
+        for (int off = 32; off >= 1; off >>= 1) {
+            sl += __shfl_xor(sl, off, 64);
+            sr += __shfl_xor(sr, off, 64);
+        }
+        if (lane == 0) {
+            el[i] = sl;
+            er[i] = sr;
+        }
+        if (SCALES) {
+            ml = fmaxf(ml, fabsf(sl));
+            mr = fmaxf(mr, fabsf(sr));
+        }
+    }
+    if (SCALES) {
+        block_absmax_to_global(ml / 127.0f, scale_el);
+        __syncthreads();  // the helper's staging array is reused by the second call
+        block_absmax_to_global(mr / 127.0f, scale_er);
+    }
+}
+
 // d_feat = del * attn_l + der * attn_r and the two [H, D] parameter gradients (sums over the rows of del * feat and
 // der * feat), with the rows read the way they lie in memory: a thread owns VEC consecutive columns
 // (of the H * D of a row; VEC = 4 or 2 needs D % VEC == 0 so that they share a head) of one of the row lanes of its
@@ -180,6 +234,24 @@ int tango_attn_scores_fwd(float* el, float* er, float* scale_el, float* scale_er
     const uintptr_t bits = reinterpret_cast<uintptr_t>(feat) | reinterpret_cast<uintptr_t>(attn_l) |
                            reinterpret_cast<uintptr_t>(attn_r);
     const int vec4 = (D % 4 == 0) && (bits & 15) == 0;
+    if (D >= 128) {  // a wavefront per item
+        const int vec = vec4 ? 4 : (D % 2 == 0 && (bits & 7) == 0) ? 2 : 1;
+        const int64_t want = ceil_div(total, scale_el ? 16 : 4);  // items per workgroup = its wavefronts
+        const hipStream_t s = as_stream(stream);
+        const int Hi = static_cast<int>(H), Di = static_cast<int>(D);
+        if (scale_el) {
+            const dim3 grid(static_cast<unsigned>(want < 512 ? want : 512));
+            if (vec == 4) hipLaunchKernelGGL((attn_scores_fwd_wide_kernel<true, 4>), grid, dim3(1024), 0, s, el, er, scale_el, scale_er, feat, attn_l, attn_r, total, Hi, Di);
+            else if (vec == 2) hipLaunchKernelGGL((attn_scores_fwd_wide_kernel<true, 2>), grid, dim3(1024), 0, s, el, er, scale_el, scale_er, feat, attn_l, attn_r, total, Hi, Di);
+            else hipLaunchKernelGGL((attn_scores_fwd_wide_kernel<true, 1>), grid, dim3(1024), 0, s, el, er, scale_el, scale_er, feat, attn_l, attn_r, total, Hi, Di);
+        } else {
+            const dim3 grid(static_cast<unsigned>(want < 8192 ? want : 8192));
+            if (vec == 4) hipLaunchKernelGGL((attn_scores_fwd_wide_kernel<false, 4>), grid, dim3(256), 0, s, el, er, scale_el, scale_er, feat, attn_l, attn_r, total, Hi, Di);
+            else if (vec == 2) hipLaunchKernelGGL((attn_scores_fwd_wide_kernel<false, 2>), grid, dim3(256), 0, s, el, er, scale_el, scale_er, feat, attn_l, attn_r, total, Hi, Di);
+            else hipLaunchKernelGGL((attn_scores_fwd_wide_kernel<false, 1>), grid, dim3(256), 0, s, el, er, scale_el, scale_er, feat, attn_l, attn_r, total, Hi, Di);
+        }
+        return launch_status();
+    }
     if (scale_el) {
         // one 16-wave workgroup per compute unit at most: a few hundred atomics per slot in all
         const int64_t want = ceil_div(total, 1024);
