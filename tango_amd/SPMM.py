@@ -132,7 +132,7 @@ class spmm_u_mul_e(Function):
         # one absmax pass (the reference runs two, cuda/SPMM.py:39,43).  Broadcast edge values, no epilogue: heads whose
         # width would leave the int8 rows unaligned are zero-padded (kernels.pad_heads); the padding columns of the
         # result are dropped again
-        padded = N.dim() == 3 and E.size(-1) == 1 and bias is None and act is None and pad_heads(N.size(2)) != N.size(2)
+        padded = N.dim() == 3 and E.size(-1) == 1 and bias is None and act is None and pad_heads(N.size(2), N.size(1)) != N.size(2)
         N_, scaleN = quantize_heads(N, scaleN) if padded else quantize(N, scaleN)
         # dequantized with scaleN * scaleE (cuda/SPMM.py:44); the kernel multiplies the two itself
         out = multi_cusparse_SPMM(g, N_, E_T_, scaleN, edge_major=True, bias=bias, scale2=scaleE, act=act)

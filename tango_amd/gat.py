@@ -114,7 +114,7 @@ class QGATConv(nn.Module):
             a, s_a = self.attn_drop(a), None  # the dropped-out tensor has another maximum
         # without a residual branch the bias add (:160-162) rides in the aggregation's epilogue
         # (not for head widths whose int8 copies are zero-padded per head: that form of the aggregation has no epilogue)
-        aligned = pad_heads(self._out_feats) == self._out_feats
+        aligned = pad_heads(self._out_feats, self._num_heads) == self._out_feats
         fold_bias = self.bias is not None and self.res_fc is None and aligned
         # and so does the activation (:164-165) when nothing else is added between the two
         fold_act = None

@@ -798,20 +798,23 @@ def quantize_padded(t, scale=None, round_mode=ROUND_RNE, noise=None, seed=0, off
     return buf[:, :cols], scale
 
 
-def pad_heads(D):
-    """Columns per head of the int8 copy of an [n, H, D] tensor: D itself, or the next multiple of 16 when heads
-    of at least 24 columns would otherwise leave the rows without 16-byte alignment (250 -> 256): the gathers of
-    the aggregation and of the SDDMM then run on aligned 16-byte pieces instead of single bytes."""
-    return (D + 15) // 16 * 16 if D >= 24 and D % 16 != 0 else D
+def pad_heads(D, H=1):
+    """Columns per head of the int8 copy of an [n, H, D] tensor: D itself, or the next multiple of 16 when the rows
+    of H * D bytes could only be gathered byte by byte (H * D not a multiple of 4: 3 x 250, 1 x 41) or when heads
+    of 128 columns or more are not whole 16-byte pieces (3 x 248): the gathers of the aggregation and of the SDDMM
+    then run on aligned 16-byte pieces."""
+    if D % 16 != 0 and D >= 24 and ((H * D) % 4 != 0 or D >= 128):
+        return (D + 15) // 16 * 16
+    return D
 
 
 def quantize_heads(t, scale=None, **kw):
     """``quantize`` for a 3-D [n, H, D] tensor with every head zero-padded to ``pad_heads(D)`` columns: returns
     (int8 [n, H, pad_heads(D)], scale).  The zeros add nothing to a dot product or an aggregation."""
-    if t.dim() != 3 or pad_heads(t.size(2)) == t.size(2):
+    if t.dim() != 3 or pad_heads(t.size(2), t.size(1)) == t.size(2):
         return quantize(t, scale, **kw)
     n, H, D = t.shape
-    Dp = pad_heads(D)
+    Dp = pad_heads(D, H)
     t = t if t.is_contiguous() else t.contiguous()
     if scale is None:
         scale = cuda_kernels.get_scale(t)

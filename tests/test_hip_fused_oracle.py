@@ -135,7 +135,7 @@ def test_copy_u_with_source_multiplier_matches_oracle(orc, n, e, F):
     assert np.array_equal(host(tN.grad), orc.spmm_csr_copy_u_ex(rip, rix, dZq, s_dZ, row_scale=mul))
 
 
-@pytest.mark.parametrize("n,e,H,D", [(500, 8000, 3, 250), (300, 5000, 2, 40), (400, 6000, 4, 24)])
+@pytest.mark.parametrize("n,e,H,D", [(500, 8000, 3, 250), (300, 5000, 1, 41), (400, 6000, 3, 248), (350, 4000, 5, 25)])
 def test_unaligned_head_widths_run_on_padded_heads(orc, n, e, H, D):
     """Head widths that are not multiples of 16 (the reference's arxiv GAT trains with 3 heads of 250): the int8
     copies are zero-padded per head, the SDDMM dot and the u_mul_e aggregation run on aligned rows, and every
@@ -144,13 +144,14 @@ def test_unaligned_head_widths_run_on_padded_heads(orc, n, e, H, D):
     from tango_amd.SDDMM import sddmm_u_dot_v
     from tango_amd.SPMM import spmm_u_mul_e
     from tango_amd.kernels import pad_heads, quantize_heads
-    assert pad_heads(D) % 16 == 0 and pad_heads(D) != D and pad_heads(16) == 16 and pad_heads(5) == 5
+    assert pad_heads(D, H) % 16 == 0 and pad_heads(D, H) != D and pad_heads(16, 8) == 16 and pad_heads(5, 3) == 5
+    assert pad_heads(40, 1) == 40 and pad_heads(40, 8) == 40  # rows of whole 4-byte pieces stay as they are
     rng = np.random.default_rng(D)
     src, dst = rand_graph(rng, n, e)
     g = make_graph(src, dst, n)
     U, V = (rng.standard_normal((n, H, D)).astype(np.float32) for _ in range(2))
     q, s = quantize_heads(dev(U))
-    assert q.shape == (n, H, pad_heads(D)) and np.array_equal(host(q)[..., :D], orc.quantize(U, orc.absmax_scale(U)))
+    assert q.shape == (n, H, pad_heads(D, H)) and np.array_equal(host(q)[..., :D], orc.quantize(U, orc.absmax_scale(U)))
     assert not host(q)[..., D:].any()
     old = config.grad_round_mode
     config.grad_round_mode = "rne"
