@@ -129,13 +129,17 @@ class spmm_u_mul_e(Function):
             E_T_, _ = quantize(E, scaleE)  # no pass that looks for the scale
         else:
             E_T_, scaleE = quantize(E)
-        # one absmax pass (the reference runs two, cuda/SPMM.py:39,43).  Broadcast edge values, no epilogue: heads whose
-        # width would leave the int8 rows unaligned are zero-padded (kernels.pad_heads); the padding columns of the
-        # result are dropped again
-        padded = N.dim() == 3 and E.size(-1) == 1 and bias is None and act is None and pad_heads(N.size(2), N.size(1)) != N.size(2)
+        # one absmax pass (the reference runs two, cuda/SPMM.py:39,43).  Broadcast edge values: heads whose width would
+        # leave the int8 rows unaligned are zero-padded (kernels.pad_heads), the bias with them; the padding columns of
+        # the result are dropped again
+        padded = N.dim() == 3 and E.size(-1) == 1 and pad_heads(N.size(2), N.size(1)) != N.size(2)
         N_, scaleN = quantize_heads(N, scaleN) if padded else quantize(N, scaleN)
+        kbias = bias
+        if padded and bias is not None:
+            H, D = N.size(1), N.size(2)
+            kbias = torch.nn.functional.pad(bias.detach().view(H, D), (0, N_.size(2) - D)).reshape(-1)
         # dequantized with scaleN * scaleE (cuda/SPMM.py:44); the kernel multiplies the two itself
-        out = multi_cusparse_SPMM(g, N_, E_T_, scaleN, edge_major=True, bias=bias, scale2=scaleE, act=act)
+        out = multi_cusparse_SPMM(g, N_, E_T_, scaleN, edge_major=True, bias=kbias, scale2=scaleE, act=act)
         out = unpad_heads(out, N.size(-1))
         reduce_last = _need_reduce_last_dim(N, E)
         ctx.padded = padded
@@ -160,8 +164,11 @@ class spmm_u_mul_e(Function):
             kw = {"round_mode": config.grad_round_mode}
             if config.grad_round_mode == "stochastic":
                 kw.update(config.stochastic_args(dZ.device))
-            dZ_, _ = quantize_padded(dZ2, scaledZ, mask=out2, mask_mode=act, align=1, **kw)
-            dZ_ = dZ_.view(dZ.shape)
+            if ctx.padded:
+                dZ_, _ = quantize_heads(dZ, scaledZ, mask=out2, mask_mode=act, **kw)
+            else:
+                dZ_, _ = quantize_padded(dZ2, scaledZ, mask=out2, mask_mode=act, align=1, **kw)
+                dZ_ = dZ_.view(dZ.shape)
         elif has_bias and ctx.needs_input_grad[3]:
             # the scale of dZ and the bias gradient (column sums) in one read
             dZ = dZ if dZ.is_contiguous() else dZ.contiguous()
@@ -169,7 +176,7 @@ class spmm_u_mul_e(Function):
             kw = {"round_mode": config.grad_round_mode}
             if config.grad_round_mode == "stochastic":
                 kw.update(config.stochastic_args(dZ.device))
-            dZ_, _ = quantize(dZ, scaledZ, **kw)
+            dZ_, _ = quantize_heads(dZ, scaledZ, **kw) if ctx.padded else quantize(dZ, scaledZ, **kw)
         elif ctx.padded:
             dZ = dZ if dZ.is_contiguous() else dZ.contiguous()
             kw = {"round_mode": config.grad_round_mode}

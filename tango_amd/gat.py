@@ -11,7 +11,7 @@ from torch.autograd.function import Function, once_differentiable
 
 from .QLinear import QLinear, Qlinear_func_reduce, shared_input_linears
 from .batchnorm import BatchNorm1dAct
-from .kernels import cuda_kernels, pad_heads, refuse_capture
+from .kernels import cuda_kernels, refuse_capture
 from .SDDMM import sddmm_u_add_v, sddmm_u_dot_v
 from .SPMM import spmm_u_mul_e
 from .edge_softmax import edge_softmax, gat_edge_attention
@@ -113,12 +113,10 @@ class QGATConv(nn.Module):
         if self.attn_drop.p > 0 and self.training:
             a, s_a = self.attn_drop(a), None  # the dropped-out tensor has another maximum
         # without a residual branch the bias add (:160-162) rides in the aggregation's epilogue
-        # (not for head widths whose int8 copies are zero-padded per head: that form of the aggregation has no epilogue)
-        aligned = pad_heads(self._out_feats, self._num_heads) == self._out_feats
-        fold_bias = self.bias is not None and self.res_fc is None and aligned
+        fold_bias = self.bias is not None and self.res_fc is None
         # and so does the activation (:164-165) when nothing else is added between the two
         fold_act = None
-        if self.res_fc is None and aligned and (fold_bias or self.bias is None):
+        if self.res_fc is None and (fold_bias or self.bias is None):
             fold_act = "elu" if self.activation is F.elu else "relu" if self.activation in (F.relu, torch.relu) else None
         rst = spmm_u_mul_e.apply(graph, feat_src, a, self.bias if fold_bias else None, s_feat, fold_act, s_a)  # :151
         if self.res_fc is not None:

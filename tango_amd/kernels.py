@@ -818,6 +818,8 @@ def quantize_heads(t, scale=None, **kw):
     t = t if t.is_contiguous() else t.contiguous()
     if scale is None:
         scale = cuda_kernels.get_scale(t)
+    if kw.get("mask") is not None:  # an [n, H D] activation output: the same rows as t
+        kw["mask"] = kw["mask"].reshape(n * H, D)
     q, scale = quantize_padded(t.view(n * H, D), scale, align=16, **kw)  # the [n H, D] view of an [n H, Dp] buffer
     return q.as_strided((n, H, Dp), (H * Dp, Dp, 1)), scale
 

@@ -18,7 +18,8 @@ def make_graph(src, dst, n):
 
 @pytest.mark.parametrize("act", [None, "relu", "elu"])
 @pytest.mark.parametrize("with_bias", [True, False])
-@pytest.mark.parametrize("n,e,H,F", [(700, 9000, 4, 16), (300, 40000, 3, 5)])
+@pytest.mark.parametrize("n,e,H,F", [(700, 9000, 4, 16), (300, 40000, 3, 5), (500, 8000, 3, 25), (300, 5000, 1, 41),
+                                     (200, 3000, 2, 250)])
 def test_u_mul_e_fused_forward_and_backward_match_oracle(orc, act, with_bias, n, e, H, F):
     from tango_amd.SPMM import spmm_u_mul_e
     rng = np.random.default_rng(31)
