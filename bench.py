@@ -252,6 +252,8 @@ def model_steps(K, torch, which=("gat", "arxiv", "arxiv-gcn", "hgt", "hetero"), 
     """The other model configurations, one training step each (forward + loss + backward + Adam):
     the 3-layer GAT (hidden 16 x 8 heads, evaluation/test_gat.py:170-214) on the 169,343-node graph
     and two HGT layers (256-d, 4 heads) on the homogenised 3-type / 4-relation graph."""
+    from tango_amd import config
+    config.grad_round_mode = "stochastic"  # as in the epoch: gradients are rounded stochastically (Philox on the device)
     out = {}
     torch.manual_seed(4)
     for name, fn in (("gat", _gat_step), ("arxiv", _arxiv_step), ("arxiv-gcn", _arxiv_gcn_step), ("hgt", _hgt_step),

@@ -92,11 +92,18 @@ __global__ __launch_bounds__(256) void bn_reduce_kernel(const float* __restrict_
     // the last workgroups may have no row at all: they read nothing and hand in an empty partial.
     const int64_t first_row = static_cast<int64_t>(blockIdx.x) * row_lanes;
     const bool has_rows = first_row < rows;
+    float sh[3][VEC];
+    if (MODE == 0 && has_rows) {  // the three rows of bn_shift, one load each
+        const int64_t r1 = first_row + 1 < rows ? first_row + 1 : first_row, r2 = first_row + 2 < rows ? first_row + 2 : first_row;
+        BnVec<VEC>::load(x + first_row * C + c0, sh[0]);
+        BnVec<VEC>::load(x + r1 * C + c0, sh[1]);
+        BnVec<VEC>::load(x + r2 * C + c0, sh[2]);
+    }
 #pragma unroll
     for (int i = 0; i < VEC; ++i) {
         k[i] = a[i] = b[i] = mu[i] = rs[i] = s1[i] = s2[i] = 0.0f;
         if (MODE == 0) {
-            if (has_rows) k[i] = bn_shift(x, first_row, rows, C, c0 + i);
+            if (has_rows) k[i] = fmaxf(fminf(sh[0][i], sh[1][i]), fminf(fmaxf(sh[0][i], sh[1][i]), sh[2][i]));
         } else {
             mu[i] = mean[c0 + i];
             rs[i] = rstd[c0 + i];
