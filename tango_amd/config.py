@@ -36,8 +36,8 @@ def next_offset():
 
 def device_offset(device):
     """The position in the stream as one int64 word in ``device``'s memory.  The quantize kernels add it to their
-    offset when they start and the call that used it advances it by WINDOW with a one-thread kernel on the same
-    stream, so the position moves with the work itself: a captured graph that is replayed draws a fresh window
+    offset when they start and a one-thread kernel on the same stream advances it (see ``stochastic_args`` for
+    when), so the position moves with the work itself: a captured graph that is replayed draws a fresh window
     per replay, where a host-side counter would be frozen into the captured launch."""
     import torch
     key = torch.device(device)
@@ -53,10 +53,26 @@ def reset_offsets():
     """Back to the start of the stream (tests that compare with a host-side replay of the same draws)."""
     global _calls
     _calls = itertools.count()
+    _pending.clear()
     for c in _counters.values():
         c.zero_()
 
 
+# Calls since a device's counter last moved.  Outside a stream capture the position of a call is
+# (device counter) + (pending calls) * WINDOW with the second term passed by value, and the counter moves once per
+# BATCH calls: one one-thread launch per BATCH quantize launches instead of one each.  Under capture every call
+# moves the counter itself (first by whatever is pending), so that a replayed graph draws fresh windows.
+BATCH = 64
+_pending = {}
+
+
 def stochastic_args(device):
     """Keyword arguments of a stochastically rounding quantize call."""
-    return {"seed": seed, "offset": device_offset(device), "advance": WINDOW}
+    import torch
+    c = device_offset(device)
+    k = _pending.get(c, 0)
+    if torch.cuda.is_current_stream_capturing() or k + 1 >= BATCH:
+        _pending[c] = 0
+        return {"seed": seed, "offset": (k * WINDOW, c), "advance": (k + 1) * WINDOW}
+    _pending[c] = k + 1
+    return {"seed": seed, "offset": (k * WINDOW, c), "advance": 0}

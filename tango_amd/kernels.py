@@ -139,7 +139,11 @@ def refuse_capture(what):
 
 
 def _split_offset(offset):
-    """(host offset, device counter or None) of an ``offset`` argument that is a number or an int64 device tensor."""
+    """(host offset, device counter or None) of an ``offset`` argument that is a number, an int64 device tensor, or
+    a pair of both (the kernel adds the two)."""
+    if isinstance(offset, tuple):
+        host, dev = offset
+        return int(host) + _split_offset(dev)[0], _split_offset(dev)[1]
     if torch.is_tensor(offset):
         if offset.dtype != torch.int64 or offset.numel() != 1 or not offset.is_cuda:
             raise RuntimeError("quantize: a device offset must be a 1-element int64 GPU tensor")

@@ -203,3 +203,28 @@ def test_device_resident_stream_position_advances_on_graph_replay(K, orc):
     out2 = torch.empty_like(out)
     K.cuda_kernels.quantize(out2, x, s, round_mode="stochastic", seed=9, offset=8)
     assert torch.equal(out, out2) and int(counter) == 8
+
+
+def test_stochastic_positions_with_batched_counter_moves(K, orc):
+    """config.stochastic_args outside a capture: call k of a device draws window k of the stream whether the
+    position is carried by the device counter or by the pending count passed by value, and the counter moves once
+    per config.BATCH calls."""
+    from tango_amd import config
+    old_seed = config.seed
+    config.seed = 77
+    config.reset_offsets()
+    try:
+        n = 4099
+        x = torch.randn(n, device="cuda")
+        s = K.cuda_kernels.get_scale(x)
+        counter = config.device_offset(x.device)
+        for k in range(config.BATCH + 3):
+            q, _ = K.quantize(x, s, round_mode="stochastic", **config.stochastic_args(x.device))
+            if k in (0, 1, config.BATCH - 2, config.BATCH - 1, config.BATCH, config.BATCH + 2):
+                want = orc.quantize(host(x), host(s)[0], orc.STOCHASTIC, seed=77, offset=k * config.WINDOW)
+                assert np.array_equal(host(q), want), k
+            moved = (k + 1) // config.BATCH * config.BATCH
+            assert int(counter) == moved * config.WINDOW, k
+    finally:
+        config.seed = old_seed
+        config.reset_offsets()
