@@ -127,3 +127,13 @@ def test_bipartite_graph_formats():
         m = edge_type.numpy() == r
         assert (node_type.numpy()[s[m]] == a).all() and (node_type.numpy()[d[m]] == b).all()
         assert s[m].min() >= bounds[a] and s[m].max() < bounds[a + 1] and d[m].max() < bounds[b + 1]
+
+
+def test_bench_refuses_more_than_one_gpu():
+    """bench.py measures one GPU; asking for more exits with a message before anything touches a device."""
+    import os
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    res = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--gpus", "2"], capture_output=True, text=True)
+    assert res.returncode != 0 and "one GPU" in (res.stderr + res.stdout)
