@@ -608,6 +608,9 @@ def main():
     raw_spmm = K.cuda_kernels.csr_SPMM
     K.cuda_kernels.csr_SPMM = staticmethod(timer.wrap(
         raw_spmm, lambda out, *a, **kw: "spmm_F%d" % (out.size(1))))
+    raw_dense = K.cuda_kernels.csr_SPMM_dense
+    K.cuda_kernels.csr_SPMM_dense = staticmethod(timer.wrap(
+        raw_dense, lambda out, *a, **kw: "spmm_F%d" % (out.size(1))))
 
     def step():
         loss = cross_entropy(model(X), labels)
@@ -626,6 +629,7 @@ def main():
     torch.cuda.synchronize()
     ms_per_step = (time.perf_counter() - t1) * 1000.0 / args.steps
     K.cuda_kernels.csr_SPMM = staticmethod(raw_spmm)
+    K.cuda_kernels.csr_SPMM_dense = staticmethod(raw_dense)
 
     # Dominant kernel: the 256-wide copy_u aggregation (forward and reverse launches of the same kernel).
     # What binds it is the caches, not HBM: a gathered 128-byte row piece is one L2 -> L1 line transfer, and

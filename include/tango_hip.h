@@ -260,6 +260,71 @@ int tango_spmm_csr_copy_u_ex(float* out, const int64_t* indptr, const void* indi
                              int64_t rows, int64_t num_src, int64_t nnz, int64_t F, int64_t max_row_nnz,
                              void* workspace, size_t workspace_bytes, tango_stream_t stream);
 
+/* csr_SPMM (cuda/src/cuda.cpp:110-117 -> SPMM.cu:23-68) on a graph whose heavy rows and heavy columns
+   form nearly dense blocks (power-law graphs): the adjacency is split once per graph into
+     - bit blocks: with rows and columns ranked by falling slot count, row block b (256 consecutive row
+       ranks) owns the cells (row, column rank < extent[b]), extent a multiple of 256; a set bit is one
+       edge.  These are multiplied with the int8 features on the matrix cores (0/1 bytes x int8 -> int32);
+     - the rest: an ordinary CSR (res_indptr, res_indices) holding every slot not represented by a bit
+       (outside the blocks, or a repeated edge whose bit was already set), gathered as in
+       tango_spmm_csr_copy_u_ex, whose epilogue adds the blocks' int32 partial sums.
+   Integer sums are exact in any order, so out equals tango_spmm_csr_copy_u_ex on the whole CSR bit for bit.
+   All arrays are device memory and belong to the caller.
+   mask layout: row block b starts at dword mask_off[b]; unit u (columns 256 u .. 256 u + 255 by rank), row
+   group g (64 rows), half q (k-steps 4 q .. 4 q + 3 of 32 columns each), lane l, k-step s4 is dword
+   (((u * 4 + g) * 2 + q) * 64 + l) * 4 + s4; its bit 8 b + 4 h + w is the cell (row 64 g + 32 h + l % 32 of
+   the block, column 256 u + 32 (4 q + s4) + 16 (l / 32) + 4 w + b).
+   segs: num_segments x 4 int32 (row block, first unit, units, 1 if other segments add into the same
+   row block); workgroup i of num_groups processes segments seg_ptr[i] .. seg_ptr[i + 1] - 1.  Two such
+   tables, each covering every unit of every row block once: (num_groups, seg_ptr, segs) for features wider
+   than 128 columns, where two workgroups share a group's segments (one half of the columns each), and
+   (num_groups2, seg_ptr2, segs2), usually twice as many groups, for narrower features.
+   shared_blocks lists the row blocks with shared segments in either table (zeroed before the product). */
+typedef struct tango_spmm_dense_plan {
+    int64_t rows;        /* output rows of the adjacency */
+    int64_t num_src;     /* rows of the gathered matrix */
+    int64_t dense_rows;  /* rows covered by row blocks: 256 * row_blocks */
+    int64_t dense_cols;  /* widest extent, a multiple of 256 */
+    int64_t row_blocks;
+    int64_t num_groups;
+    int64_t num_groups2;
+    int64_t num_shared;
+    const int32_t* col_ids;        /* [dense_cols] column rank -> row of the gathered matrix, -1 = none */
+    const int32_t* row_slot;       /* [rows] output row -> its row rank if below dense_rows, else -1 */
+    const int64_t* mask_off;       /* [row_blocks] */
+    const uint32_t* mask;
+    const int32_t* seg_ptr;        /* [num_groups + 1] */
+    const int32_t* segs;           /* [seg_ptr[num_groups]][4] */
+    const int32_t* seg_ptr2;       /* [num_groups2 + 1] */
+    const int32_t* segs2;          /* [seg_ptr2[num_groups2]][4] */
+    const int32_t* shared_blocks;  /* [num_shared] */
+    const int64_t* res_indptr;     /* [rows + 1] */
+    const int32_t* res_indices;    /* [res_nnz] */
+    int64_t res_nnz;
+    int64_t res_max_row;           /* longest row of the rest, 0 if unknown */
+} tango_spmm_dense_plan;
+
+/* Sets the bits of a plan's mask (which the caller has zeroed) from the adjacency (indptr, indices;
+   idx_bits 32 or 64) and says which slots remain for the rest: keep[p] = 0 when slot p is now a bit of
+   the mask, 1 when it stays (outside the blocks, or its bit was already set by an equal edge);
+   kept[r] = number of kept slots of row r.  row_rank / col_rank: rank of every row / gathered row
+   (int32); extent_cols[b]: extent of row block b in columns.  One-time graph preprocessing
+   (extends cuda/util.py:5-11). */
+int tango_spmm_dense_mask_build(const int64_t* indptr, const void* indices, int idx_bits, int64_t rows,
+                                const int32_t* row_rank, const int32_t* col_rank,
+                                const int32_t* extent_cols, const int64_t* mask_off, int64_t row_blocks,
+                                uint32_t* mask, uint8_t* keep, int32_t* kept, tango_stream_t stream);
+
+/* out as tango_spmm_csr_copy_u_ex computes it on the whole adjacency (same epilogue arguments).
+   Needs 16-byte aligned feat rows (ldf % 16 == 0, ceil16(F) <= ldf) and F <= 256, else
+   TANGO_ERR_UNSUPPORTED (callers then use tango_spmm_csr_copy_u_ex on the whole CSR).
+   workspace: tango_spmm_dense_workspace(plan, F) bytes, 256-byte aligned. */
+size_t tango_spmm_dense_workspace(const tango_spmm_dense_plan* plan, int64_t F);
+int tango_spmm_csr_copy_u_dense(float* out, const tango_spmm_dense_plan* plan, const int8_t* feat,
+                                int64_t ldf, const float* scale, const float* row_scale,
+                                const float* bias, int relu, uint16_t* sign_bits, int64_t F,
+                                void* workspace, size_t workspace_bytes, tango_stream_t stream);
+
 /* multi_cusparse_SPMM (cuda/src/cuda.cpp:119-158 -> SPMM.cu:70-194):
    out[r,h,f] = scale[0] * float(sum_p evals[h, d, e(p)] * feat[indices[p], h, f]),
    d = 0 when D == 1 (broadcast edge value) else d = f (D == F, element-wise).

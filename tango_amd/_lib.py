@@ -46,6 +46,9 @@ SIGNATURES = {
     "tango_spmm_csr_copy_u": (I, [P, P, P, P, I64, P, I64, I64, I64, I64, P]),
     "tango_spmm_workspace": (SZ, [I64, I64, I64]),
     "tango_spmm_csr_copy_u_ex": (I, [P, P, P, I, P, I64, P, P, P, I, P, I64, I64, I64, I64, I64, P, SZ, P]),
+    "tango_spmm_dense_mask_build": (I, [P, P, I, I64, P, P, P, P, I64, P, P, P, P]),
+    "tango_spmm_dense_workspace": (SZ, [P, I64]),
+    "tango_spmm_csr_copy_u_dense": (I, [P, P, P, I64, P, P, P, I, P, I64, P, SZ, P]),
     "tango_spmm_csr_u_mul_e": (I, [P, P, P, P, P, P, P, I64, I64, I64, I64, I64, I64, P]),
     "tango_spmm_csr_u_mul_e_ex": (I, [P, P, P, P, I, P, P, I, P, P, P, I, I64, I64, I64, I64, I64, I64, I64, P, SZ, P]),
     "tango_spmm_csr_u_mul_e_f32e": (I, [P, P, P, P, I, P, P, I, P, P, P, I, I64, I64, I64, I64, I64, I64, I64, P, SZ, P]),
@@ -68,6 +71,17 @@ SIGNATURES = {
     "tango_edge_softmax_bwd_ex": (I, [P, P, P, P, P, P, P, P, I64, I64, I64, F, P, SZ, P]),
     "tango_edge_softmax_bwd": (I, [P, P, P, P, P, P, I64, I64, I64, F, P, SZ, P]),
 }
+
+
+
+class DensePlan(C.Structure):
+    """tango_spmm_dense_plan of include/tango_hip.h."""
+    _fields_ = [(n, I64) for n in ("rows", "num_src", "dense_rows", "dense_cols", "row_blocks", "num_groups",
+                                   "num_groups2", "num_shared")] + \
+               [(n, P) for n in ("col_ids", "row_slot", "mask_off", "mask", "seg_ptr", "segs", "seg_ptr2", "segs2", "shared_blocks",
+                                 "res_indptr", "res_indices")] + \
+               [("res_nnz", I64), ("res_max_row", I64)]
+
 
 ROUND_RNE, ROUND_TRUNC, ROUND_STOCHASTIC = 0, 1, 2
 ROUND_MODES = {"rne": ROUND_RNE, "trunc": ROUND_TRUNC, "stochastic": ROUND_STOCHASTIC}

@@ -12,7 +12,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB_DIR = os.path.join(HERE, "lib")
 LIB_PATH = os.path.join(LIB_DIR, "libtango_hip.so")
-SOURCES = ["quantize.hip", "spmm.hip", "sddmm.hip", "edge_softmax.hip", "qgemm.hip", "loss.hip", "attention.hip", "batchnorm.hip"]
+SOURCES = ["quantize.hip", "spmm.hip", "spmm_dense.hip", "sddmm.hip", "edge_softmax.hip", "qgemm.hip", "loss.hip", "attention.hip", "batchnorm.hip"]
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = [

@@ -706,7 +706,7 @@ const char* tango_status_string(int status) {
     }
 }
 
-int tango_abi_version(void) { return 2; }
+int tango_abi_version(void) { return 3; }
 
 int tango_absmax_f32(const float* x, int64_t n, float* scale_out, tango_stream_t stream) {
     if (!scale_out || n < 0 || (n > 0 && !x)) return TANGO_ERR_INVALID_ARG;

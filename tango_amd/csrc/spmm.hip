@@ -25,6 +25,7 @@
 //   * the lane groups are folded with ds_bpermute shuffles, the waves of a
 //     workgroup through LDS, and the row leaves as fp32 = scale * float(sum).
 #include "common.hpp"
+#include "spmm_dense.hpp"
 
 namespace tango {
 
@@ -65,6 +66,9 @@ struct SpmmParams {
     void* span_ws;     // sparse graphs: caller's workspace for the slot-span path, or null
     int64_t span_wp;   // padded row width (int32 entries) of a partial row in span_ws
     size_t span_ws_bytes;
+    const int* part;       // optional int32 partial sums added to a row's sum before dequantization (the dense
+    const int* part_slot;  // blocks of spmm_dense.hip): row r owns row part_slot[r] of part (stride part_ld ints)
+    int part_ld;           // when that is not negative
 };
 
 enum { KIND_COPY = 0, KIND_WEIGHTED = 1, KIND_COO = 2, KIND_WEIGHTED_F32 = 3 };
@@ -294,11 +298,30 @@ __device__ __forceinline__ void store_row(const SpmmParams& p, const LaneCols& c
     const float s = p.scale2 ? p.scale[0] * p.scale2[0] : p.scale[0];
     const float rs = p.row_scale ? p.row_scale[row] : 1.0f;
     float* o = p.out + row * p.W + c.col;
+    int extra[VEC];
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) extra[i] = 0;
+    if (p.part) {  // uniform
+        const int slot = p.part_slot[row];
+        if (slot >= 0) {
+            const int* pr = p.part + static_cast<int64_t>(slot) * p.part_ld + c.col;  // rows padded: no column guard
+            if (VEC == 16) {
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const i32x4 v = reinterpret_cast<const i32x4*>(pr)[i];
+                    extra[4 * i] = v[0]; extra[4 * i + 1] = v[1]; extra[4 * i + 2] = v[2]; extra[4 * i + 3] = v[3];
+                }
+            } else {
+#pragma unroll
+                for (int i = 0; i < VEC; ++i) extra[i] = pr[i];
+            }
+        }
+    }
     float y[VEC];
 #pragma unroll
     for (int i = 0; i < VEC; ++i) {
         // same sequence of roundings as dequantize, then "* norm", "+ bias", relu as separate passes
-        y[i] = s * static_cast<float>(acc[i]);
+        y[i] = s * static_cast<float>(acc[i] + extra[i]);
         if (p.row_scale) y[i] = y[i] * rs;
         if (p.bias && c.col + i < p.W) y[i] = y[i] + p.bias[c.col + i];
     }
@@ -1102,7 +1125,7 @@ static int launch_spmm(SpmmParams p, int vec, hipStream_t s) {
     const int64_t nspans_all = ceil_div(p.nnz, kSpanSlots);
     const bool span_fits = span_parts_offset(nspans_all) + sizeof(int) * 2 * static_cast<size_t>(nspans_all) *
                                static_cast<size_t>(ychunks * p.tile) <= p.span_ws_bytes;
-    if (KIND != KIND_COO && p.span_ws && span_fits && span_graph(p.rows, p.nnz)) {  // sparse graph: slot spans, two launches
+    if (KIND != KIND_COO && p.span_ws && span_fits && span_graph(p.rows, p.nnz) && !p.part) {  // sparse graph: slot spans, two launches
         const int64_t nspans = nspans_all;
         p.span_wp = ychunks * p.tile;
         const dim3 spgrid(static_cast<unsigned>(ceil_div(nspans > 0 ? nspans : 1, 4)), static_cast<unsigned>(ychunks));
@@ -1125,7 +1148,7 @@ static int launch_spmm(SpmmParams p, int vec, hipStream_t s) {
     }
 #undef TANGO_SPMM_LONG
     // Sparse graph: lane groups own the short rows, single waves the rest up to long_row.
-    if (KIND != KIND_COO && p.nnz < 64 * p.rows && p.lpe_log2 < 6) {
+    if (KIND != KIND_COO && p.nnz < 64 * p.rows && p.lpe_log2 < 6 && !p.part) {
         p.group_row = kGroupRow;
         const int64_t rows_per_block = 4LL << (6 - p.lpe_log2);
         const dim3 ggrid(static_cast<unsigned>(ceil_div(p.rows, rows_per_block)), static_cast<unsigned>(ychunks));
@@ -1283,6 +1306,44 @@ int tango_spmm_csr_u_mul_e(float* out, const int64_t* indptr, const int64_t* ind
                            int64_t F, int64_t D, int64_t nnz, tango_stream_t stream) {
     return tango_spmm_csr_u_mul_e_ex(out, indptr, indices, edge_ids, 64, feat, evals, 0, scale, nullptr, nullptr, 0, rows, num_src,
                                      H, F, D, nnz, 0, nullptr, 0, stream);
+}
+
+size_t tango_spmm_dense_workspace(const tango_spmm_dense_plan* plan, int64_t F) {
+    if (!plan || F < 0) return 0;
+    const size_t dense = dense_workspace_bytes(*plan, F);
+    if (!dense) return 0;
+    // the gather kernels' own workspace for hub rows of the rest follows the dense part
+    return dense + ((64 + sizeof(int64_t) * static_cast<size_t>(plan->res_nnz / kHubRowMin + 2) + 255) & ~static_cast<size_t>(255));
+}
+
+int tango_spmm_csr_copy_u_dense(float* out, const tango_spmm_dense_plan* plan, const int8_t* feat,
+                                int64_t ldf, const float* scale, const float* row_scale,
+                                const float* bias, int relu, uint16_t* sign_bits, int64_t F,
+                                void* workspace, size_t workspace_bytes, tango_stream_t stream) {
+    if (!plan || F < 0 || !scale || ldf < F || !feat || plan->rows < 0 || plan->res_nnz < 0 || !plan->res_indptr ||
+        !plan->row_slot || (plan->rows * F > 0 && !out) || (plan->res_nnz > 0 && !plan->res_indices))
+        return TANGO_ERR_INVALID_ARG;
+    if (plan->num_src >= (1LL << 31) || plan->res_nnz >= (1LL << 31) || relu < 0 || relu > 2) return TANGO_ERR_UNSUPPORTED;
+    if (sign_bits && (F & 15) != 0) return TANGO_ERR_UNSUPPORTED;
+    if (plan->rows == 0 || F == 0) return TANGO_OK;
+    const size_t need = tango_spmm_dense_workspace(plan, F);
+    if (!need) return TANGO_ERR_UNSUPPORTED;
+    if (!workspace || workspace_bytes < need) return TANGO_ERR_WORKSPACE;
+    SpmmParams p{};
+    if (plan->row_blocks > 0) {
+        const int st = launch_dense_block(*plan, feat, ldf, F, workspace, workspace_bytes, &p.part, &p.part_ld,
+                                          as_stream(stream));
+        if (st != TANGO_OK) return st;
+        p.part_slot = plan->row_slot;
+    } else if (pick_vec(feat, ldf, F) != 16) {
+        return TANGO_ERR_UNSUPPORTED;
+    }
+    p.out = out; p.indptr = plan->res_indptr; p.indices = reinterpret_cast<const int64_t*>(plan->res_indices); p.idx32 = 1;
+    p.feat = feat; p.scale = scale;
+    p.row_scale = row_scale; p.bias = bias; p.relu = relu; p.sign_bits = sign_bits; p.max_row = plan->res_max_row;
+    p.hub_ws = static_cast<char*>(workspace) + dense_workspace_bytes(*plan, F);
+    p.rows = plan->rows; p.num_src = plan->num_src; p.ldf = ldf; p.W = F; p.F = F; p.D = 1; p.nnz = plan->res_nnz;
+    return launch_spmm<KIND_COPY>(p, 16, as_stream(stream));
 }
 
 int tango_spmm_incidence(float* out, const int64_t* node_ids, const int64_t* edge_ids,

@@ -1,0 +1,160 @@
+"""Per-graph split of an adjacency into dense bit blocks and a sparse rest (graph preprocessing,
+an extension of cuda/util.py:5-11 of the reference, which caches CSR / CSC / COO once per graph).
+
+On power-law graphs the cells (row i, column j) with expected density deg(i) * cnt(j) / nnz above a
+few per cent hold a large part of all edges.  With rows and columns ranked by falling slot count that
+region is a staircase: row block b (256 consecutive row ranks) gets the columns of rank below
+``extent[b]``.  Inside it an edge is one bit and the copy_u aggregation a 0/1 x int8 matrix product
+(tango_spmm_csr_copy_u_dense); everything else stays a CSR.  The split changes no result: integer
+sums are exact in any order.
+"""
+import ctypes
+import heapq
+import os
+
+import numpy as np
+import torch
+
+from . import _lib
+from ._lib import check
+
+ROWS = 256   # rows of a row block
+UNIT = 256   # mask columns of a unit
+
+
+def default_tau():
+    """Density above which a cell is worth a bit (the matrix product costs about this fraction of a
+    gathered row per cell); TANGO_DENSE_TAU overrides, 0 switches the dense blocks off."""
+    return float(os.environ.get("TANGO_DENSE_TAU", "0.02"))
+
+
+class DensePlan:
+    """Device tensors of one orientation's split plus the C struct that points at them."""
+
+    def __init__(self, **kw):
+        self.__dict__.update(kw)
+        s = _lib.DensePlan()
+        s.rows, s.num_src = self.rows, self.num_src
+        s.dense_rows, s.dense_cols = self.row_blocks * ROWS, self.dense_cols
+        s.row_blocks, s.num_groups = self.row_blocks, self.seg_ptr.numel() - 1
+        s.num_groups2, s.num_shared = self.seg_ptr2.numel() - 1, self.shared_blocks.numel()
+        for name in ("col_ids", "row_slot", "mask_off", "mask", "seg_ptr", "segs", "seg_ptr2", "segs2", "shared_blocks",
+                     "res_indptr", "res_indices"):
+            t = getattr(self, name)
+            setattr(s, name, t.data_ptr() if t.numel() else None)
+        s.res_nnz, s.res_max_row = self.res_indices.numel(), self.res_max_row
+        self.struct = s
+        self.ref = ctypes.byref(s)
+
+
+def _segments(units, groups):
+    """Deals the units of every row block over ``groups`` workgroups: blocks much longer than a fair share
+    are cut into pieces (several workgroups then add into the block's partial sums), the others stay whole;
+    longest piece first to the least loaded workgroup.  Returns (seg_ptr, segs, shared_blocks) as numpy."""
+    total = int(units.sum())
+    groups = max(1, min(groups, total))
+    fair = total / groups
+    items = []  # (units, row block, first unit, shared)
+    shared = []
+    for b, n in enumerate(units.tolist()):
+        if n > 1.5 * fair:
+            pieces = int(np.ceil(n / fair))
+            cuts = np.linspace(0, n, pieces + 1).round().astype(np.int64)
+            shared.append(b)
+            for a, e in zip(cuts[:-1], cuts[1:]):
+                if e > a:
+                    items.append((int(e - a), b, int(a), 1))
+        elif n > 0:
+            items.append((n, b, 0, 0))
+    items.sort(key=lambda it: -it[0])
+    heap = [(0, g) for g in range(groups)]
+    per_group = [[] for _ in range(groups)]
+    for n, b, a, sh in items:
+        load, g = heapq.heappop(heap)
+        per_group[g].append((b, a, n, sh))
+        heapq.heappush(heap, (load + n, g))
+    seg_ptr = np.zeros(groups + 1, dtype=np.int32)
+    segs = []
+    for g, lst in enumerate(per_group):
+        segs.extend(lst)
+        seg_ptr[g + 1] = len(segs)
+    return seg_ptr, np.asarray(segs, dtype=np.int32).reshape(-1, 4), np.asarray(shared, dtype=np.int32)
+
+
+def build_dense_plan(indptr, indices, num_src, tau=None, groups=256, sort_rest=True, min_share=0.05, min_extent=None):
+    """Splits the CSR (indptr int64 [rows + 1], indices int32 / int64 [nnz], gathered rows < num_src).
+    Returns a DensePlan, or None when fewer than ``min_share`` of the slots would become bits."""
+    tau = default_tau() if tau is None else float(tau)
+    min_extent = int(os.environ.get("TANGO_DENSE_MIN_EXTENT", "2048")) if min_extent is None else int(min_extent)
+    min_extent = max(min_extent, UNIT)
+    rows = indptr.numel() - 1
+    nnz = indices.numel()
+    if tau <= 0 or rows <= 0 or nnz == 0:
+        return None
+    dev = indptr.device
+    row_deg = torch.diff(indptr)
+    col_cnt = torch.bincount(indices, minlength=num_src)
+    row_order = torch.argsort(row_deg, descending=True, stable=True)
+    col_order = torch.argsort(col_cnt, descending=True, stable=True)
+    rd = row_deg[row_order].cpu().numpy().astype(np.float64)
+    cc = col_cnt[col_order].cpu().numpy().astype(np.float64)
+    extents = []
+    for b in range((rows + ROWS - 1) // ROWS):
+        mean_deg = rd[b * ROWS:(b + 1) * ROWS].mean()
+        if mean_deg <= 0:
+            break
+        cols = int(np.searchsorted(-cc, -(tau * nnz / mean_deg), side="left"))  # columns with cnt * deg / nnz > tau
+        ext = cols // UNIT * UNIT
+        if ext < min_extent:  # a block's partial sums cost a write and a read of 256 rows whatever its extent
+            break
+        extents.append(ext)
+    if not extents:
+        return None
+    extents = np.asarray(extents, dtype=np.int64)
+    # expected number of slots inside the blocks under the density model
+    covered = sum(np.minimum(1.0, rd[b * ROWS:(b + 1) * ROWS].mean() * cc[:e] / nnz).sum() * ROWS for b, e in enumerate(extents))
+    if covered < min_share * nnz:
+        return None
+    row_blocks = len(extents)
+    row_rank = torch.empty(rows, dtype=torch.int32, device=dev)
+    row_rank[row_order] = torch.arange(rows, dtype=torch.int32, device=dev)
+    col_rank = torch.empty(num_src, dtype=torch.int32, device=dev)
+    col_rank[col_order] = torch.arange(num_src, dtype=torch.int32, device=dev)
+    mask_words = extents * (ROWS // 32)
+    mask_off = np.concatenate([[0], np.cumsum(mask_words)[:-1]]).astype(np.int64)
+    mask = torch.zeros(int(mask_words.sum()), dtype=torch.int32, device=dev)
+    mask_off_t = torch.from_numpy(mask_off).to(dev)
+    extent_t = torch.from_numpy(extents.astype(np.int32)).to(dev)
+    keep = torch.empty(nnz, dtype=torch.uint8, device=dev)
+    kept = torch.empty(rows, dtype=torch.int32, device=dev)
+    idx_bits = 32 if indices.dtype == torch.int32 else 64
+    stream = torch.cuda.current_stream(dev).cuda_stream
+    check(_lib.lib().tango_spmm_dense_mask_build(indptr.data_ptr(), indices.data_ptr(), idx_bits, rows,
+                                                 row_rank.data_ptr(), col_rank.data_ptr(), extent_t.data_ptr(),
+                                                 mask_off_t.data_ptr(), row_blocks, mask.data_ptr(), keep.data_ptr(),
+                                                 kept.data_ptr(), stream), "dense_mask_build")
+    res_indices = indices[keep.bool()].to(torch.int32)
+    res_indptr = torch.zeros(rows + 1, dtype=torch.int64, device=dev)
+    torch.cumsum(kept, 0, out=res_indptr[1:])
+    if sort_rest and res_indices.numel():
+        # inside a row, popular sources first: rows walked at the same time then ask for the same lines
+        row_of = torch.repeat_interleave(torch.arange(rows, device=dev), kept.long())
+        key = row_of * num_src + col_rank[res_indices.long()].long()
+        del row_of
+        res_indices = res_indices[torch.argsort(key)]
+        del key
+    del keep
+    seg_ptr, segs, shared = _segments(extents // UNIT, groups)
+    seg_ptr2, segs2, shared2 = _segments(extents // UNIT, 2 * groups)
+    shared = np.union1d(shared, shared2).astype(np.int32)
+    row_slot = torch.where(row_rank < row_blocks * ROWS, row_rank, torch.full_like(row_rank, -1))
+    return DensePlan(
+        rows=rows, num_src=int(num_src), row_blocks=row_blocks, dense_cols=int(extents.max()),
+        tau=tau, nnz=nnz,
+        col_ids=col_order[:int(extents.max())].to(torch.int32).contiguous(), row_slot=row_slot.contiguous(),
+        mask_off=mask_off_t, mask=mask, seg_ptr=torch.from_numpy(seg_ptr).to(dev),
+        segs=torch.from_numpy(segs).to(dev).contiguous(), seg_ptr2=torch.from_numpy(seg_ptr2).to(dev),
+        segs2=torch.from_numpy(segs2).to(dev).contiguous(), shared_blocks=torch.from_numpy(shared).to(dev),
+        res_indptr=res_indptr, res_indices=res_indices.contiguous(),
+        res_max_row=int(kept.max().item()) if rows else 0,
+        cells=int((extents * ROWS).sum()))

@@ -521,6 +521,43 @@ class cuda_kernels:
                                           _stream()), "csr_SPMM")
 
     @staticmethod
+    def csr_SPMM_dense(out, plan, U, scaleU, ldf=None, F=None, row_scale=None, bias=None, relu=False, sign_bits=None):
+        """csr_SPMM on an adjacency split by ``dense_plan.build_dense_plan`` into bit blocks (multiplied with
+        U on the matrix cores) and a sparse rest; same result as csr_SPMM on the whole CSR, bit for bit.
+        Returns False (nothing launched) when U's layout rules the dense path out."""
+        _need(out, torch.float32, "out")
+        _need(U, torch.int8, "U")
+        _need(scaleU, torch.float32, "scaleU")
+        width = math.prod(U.shape[1:])
+        ldf = width if ldf is None else ldf
+        F = width if F is None else F
+        if F > 256 or ldf % 16 or (F + 15) // 16 * 16 > ldf or U.data_ptr() % 16 or U.size(0) != plan.num_src:
+            return False
+        if out.numel() != plan.rows * F:
+            raise RuntimeError("csr_SPMM_dense: out must be [%d, %d]" % (plan.rows, F))
+        if sign_bits is not None:
+            _need(sign_bits, torch.int16, "sign_bits")
+            if F % 16 or tuple(sign_bits.shape) != (plan.rows, F // 16):
+                raise RuntimeError("csr_SPMM_dense: sign_bits must be int16 [rows, F / 16], F a multiple of 16")
+        if row_scale is not None:
+            _need(row_scale, torch.float32, "row_scale")
+            if row_scale.numel() != plan.rows:
+                raise RuntimeError("csr_SPMM_dense: row_scale must have one entry per output row")
+        if bias is not None:
+            _need(bias, torch.float32, "bias")
+            if bias.numel() != F:
+                raise RuntimeError("csr_SPMM_dense: bias must have F entries")
+        key = ("dense", id(plan), F)
+        ws_bytes = _WS_SIZES.get(key)
+        if ws_bytes is None:
+            ws_bytes = _WS_SIZES[key] = _L.tango_spmm_dense_workspace(plan.ref, F)
+        ws = _workspace(ws_bytes, U.device)
+        check(_L.tango_spmm_csr_copy_u_dense(_ptr(out), plan.ref, _ptr(U), ldf, scaleU.data_ptr(), _ptr(row_scale),
+                                             _ptr(bias), int(bool(relu)), _ptr(sign_bits), F, _ptr(ws), ws_bytes,
+                                             _stream()), "csr_SPMM_dense")
+        return True
+
+    @staticmethod
     def multi_cusparse_SPMM(indptr, indices, N, E_T, scale, edge_ids=None, edge_major=False, bias=None, max_row=0,
                             scale2=None, act=None):
         """E_T is [H, D, nnz] in CSR slot order, or in edge-id order when the
@@ -979,11 +1016,18 @@ def csr_SPMM(g, N, scaleN, reverse=False, row_scale=None, bias=None, relu=False,
     out_shape = (g.num_nodes(),) + feat_shape
     dim = math.prod(N.shape[1:])
     out = torch.empty((g.num_nodes(), dim), dtype=torch.float32, device=N.device)
+    plan = getattr(g, "dense_csr" if reverse else "dense_csc", None)
     if N.dim() == 2 and not N.is_contiguous():
         ld = _rows_view(N, "N")
         base = N.as_strided((N.size(0), ld), (ld, 1))
+        if plan is not None and cuda_kernels.csr_SPMM_dense(out, plan, base, scaleN, ldf=ld, F=dim, row_scale=row_scale,
+                                                            bias=bias, relu=relu, sign_bits=sign_bits):
+            return out.view(out_shape)
         cuda_kernels.csr_SPMM(out, indptr, indices, base, scaleN, ldf=ld, F=dim, row_scale=row_scale, bias=bias,
                               relu=relu, max_row=longest, sign_bits=sign_bits)
+    elif plan is not None and cuda_kernels.csr_SPMM_dense(out, plan, N.reshape(N.size(0), dim), scaleN, row_scale=row_scale,
+                                                          bias=bias, relu=relu, sign_bits=sign_bits):
+        pass
     else:
         cuda_kernels.csr_SPMM(out, indptr, indices, N, scaleN, row_scale=row_scale, bias=bias, relu=relu,
                               max_row=longest, sign_bits=sign_bits)

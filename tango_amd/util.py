@@ -4,10 +4,12 @@ import torch
 from .graph import Graph
 
 
-def graph_preprocess(graph):
+def graph_preprocess(graph, dense_blocks=True):
     """Materialise CSR/CSC/COO/incidence once and cache them on the graph
     (cuda/util.py:5-11).  Accepts a ``tango_amd.graph.Graph`` or any object
-    with DGL's ``inc`` / ``adj_sparse`` / ``edges`` methods."""
+    with DGL's ``inc`` / ``adj_sparse`` / ``edges`` methods.  ``dense_blocks``: on graphs
+    averaging 64 or more edges per node also split both orientations into dense bit blocks and
+    a sparse rest (``dense_plan.build_dense_plan``), which the copy_u aggregation then uses."""
     if isinstance(graph, Graph):
         graph.inc_in = graph.incidence("in")
         graph.inc_out = graph.incidence("out")
@@ -33,4 +35,14 @@ def graph_preprocess(graph):
     # kernels whether the launches that exist for hub rows are needed at all
     graph.max_out_degree = int(torch.diff(graph.adj_csr[0]).max().item()) if graph.adj_csr[0].numel() > 1 else 0
     graph.max_in_degree = int(torch.diff(graph.adj_csc[0]).max().item()) if graph.adj_csc[0].numel() > 1 else 0
+    graph.dense_csr = graph.dense_csc = None
+    nnz = graph.adj_csr[1].numel()
+    if dense_blocks and nnz >= (1 << 22):
+        from .dense_plan import build_dense_plan
+        for name, (indptr, _, _), narrow in (("dense_csr", graph.adj_csr, graph.adj_csr32),
+                                             ("dense_csc", graph.adj_csc, graph.adj_csc32)):
+            rows = indptr.numel() - 1
+            if nnz >= 64 * rows:
+                num_src = graph.num_dst_nodes() if name == "dense_csr" else graph.num_src_nodes()
+                setattr(graph, name, build_dense_plan(indptr, narrow[0], num_src))
     return graph
