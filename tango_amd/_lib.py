@@ -78,7 +78,7 @@ class DensePlan(C.Structure):
     """tango_spmm_dense_plan of include/tango_hip.h."""
     _fields_ = [(n, I64) for n in ("rows", "num_src", "dense_rows", "dense_cols", "row_blocks", "num_groups",
                                    "num_groups2", "num_shared")] + \
-               [(n, P) for n in ("col_ids", "row_slot", "mask_off", "mask", "seg_ptr", "segs", "seg_ptr2", "segs2", "shared_blocks",
+               [(n, P) for n in ("col_ids", "row_slot", "row_order", "mask_off", "mask", "seg_ptr", "segs", "seg_ptr2", "segs2", "shared_blocks",
                                  "res_indptr", "res_indices")] + \
                [("res_nnz", I64), ("res_max_row", I64)]
 

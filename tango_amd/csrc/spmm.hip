@@ -69,6 +69,8 @@ struct SpmmParams {
     const int* part;       // optional int32 partial sums added to a row's sum before dequantization (the dense
     const int* part_slot;  // blocks of spmm_dense.hip): row r owns row part_slot[r] of part (stride part_ld ints)
     int part_ld;           // when that is not negative
+    const int* row_order;  // optional: workgroups take rows in this order (rows of similar length side by side,
+                           // whatever the numbering of the nodes) instead of by row number
 };
 
 enum { KIND_COPY = 0, KIND_WEIGHTED = 1, KIND_COO = 2, KIND_WEIGHTED_F32 = 3 };
@@ -378,10 +380,11 @@ template <int VEC, int WPR, int KIND>
 __global__ __launch_bounds__(256) void spmm_kernel(const SpmmParams p) {
     const int lane = lane_id();
     const int wave = __builtin_amdgcn_readfirstlane(static_cast<int>(threadIdx.x) >> 6);
-    const int64_t row = (WPR == 4) ? static_cast<int64_t>(blockIdx.x)
-                                   : static_cast<int64_t>(blockIdx.x) * 4 + wave;
+    int64_t row = (WPR == 4) ? static_cast<int64_t>(blockIdx.x)
+                             : static_cast<int64_t>(blockIdx.x) * 4 + wave;
     __shared__ int part[(WPR == 4) ? 3 * 64 * VEC : 1];
     if (WPR == 1 && row >= p.rows) return;  // whole wave leaves; no barrier follows for WPR == 1
+    if (p.row_order) row = p.row_order[row];
 
     int64_t start, end;
     if (KIND == KIND_COO) {
@@ -1341,6 +1344,7 @@ int tango_spmm_csr_copy_u_dense(float* out, const tango_spmm_dense_plan* plan, c
     p.out = out; p.indptr = plan->res_indptr; p.indices = reinterpret_cast<const int64_t*>(plan->res_indices); p.idx32 = 1;
     p.feat = feat; p.scale = scale;
     p.row_scale = row_scale; p.bias = bias; p.relu = relu; p.sign_bits = sign_bits; p.max_row = plan->res_max_row;
+    p.row_order = plan->row_order;
     p.hub_ws = static_cast<char*>(workspace) + dense_workspace_bytes(*plan, F);
     p.rows = plan->rows; p.num_src = plan->num_src; p.ldf = ldf; p.W = F; p.F = F; p.D = 1; p.nnz = plan->res_nnz;
     return launch_spmm<KIND_COPY>(p, 16, as_stream(stream));

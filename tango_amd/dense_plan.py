@@ -38,10 +38,10 @@ class DensePlan:
         s.dense_rows, s.dense_cols = self.row_blocks * ROWS, self.dense_cols
         s.row_blocks, s.num_groups = self.row_blocks, self.seg_ptr.numel() - 1
         s.num_groups2, s.num_shared = self.seg_ptr2.numel() - 1, self.shared_blocks.numel()
-        for name in ("col_ids", "row_slot", "mask_off", "mask", "seg_ptr", "segs", "seg_ptr2", "segs2", "shared_blocks",
+        for name in ("col_ids", "row_slot", "row_order", "mask_off", "mask", "seg_ptr", "segs", "seg_ptr2", "segs2", "shared_blocks",
                      "res_indptr", "res_indices"):
             t = getattr(self, name)
-            setattr(s, name, t.data_ptr() if t.numel() else None)
+            setattr(s, name, t.data_ptr() if t is not None and t.numel() else None)
         s.res_nnz, s.res_max_row = self.res_indices.numel(), self.res_max_row
         self.struct = s
         self.ref = ctypes.byref(s)
@@ -148,7 +148,9 @@ def build_dense_plan(indptr, indices, num_src, tau=None, groups=256, sort_rest=T
     seg_ptr2, segs2, shared2 = _segments(extents // UNIT, 2 * groups)
     shared = np.union1d(shared, shared2).astype(np.int32)
     row_slot = torch.where(row_rank < row_blocks * ROWS, row_rank, torch.full_like(row_rank, -1))
+    identity = bool(torch.equal(row_order, torch.arange(rows, device=dev)))
     return DensePlan(
+        row_order=None if identity else row_order.to(torch.int32).contiguous(),
         rows=rows, num_src=int(num_src), row_blocks=row_blocks, dense_cols=int(extents.max()),
         tau=tau, nnz=nnz,
         col_ids=col_order[:int(extents.max())].to(torch.int32).contiguous(), row_slot=row_slot.contiguous(),
