@@ -252,12 +252,18 @@ int tango_spmm_csr_copy_u(float* out, const int64_t* indptr, const int64_t* indi
    W in the size query: bytes summed per gathered row (F here, H * F for u_mul_e).
    sign_bits (or NULL; needs F % 16 == 0 and 16-byte aligned feat rows): [rows, F / 16] 16-bit words that
    receive bit c % 16 of word [r, c / 16] = (out[r, c] > 0), the mask the backward pass of the ReLU needs,
-   in 1/32 of the bytes of out (mask_mode 2 of tango_absmax_ex_f32 / tango_quantize_rows_ex_f32_i8). */
+   in 1/32 of the bytes of out (mask_mode 2 of tango_absmax_ex_f32 / tango_quantize_rows_ex_f32_i8).
+   scale_out (or NULL; needs the workspace): must hold 0 (or an earlier partial maximum) on entry and receives
+   max(scale_out[0], max |out[r, c] * absmax_row_mul[r]| / 127) (absmax_row_mul NULL: no multiplier): the scale the
+   quantizer of the next op needs, formed where out is produced instead of by a pass over out (the reference's only
+   fused reduction of this kind sits in its GEMM epilogue, cuda/src/epilogue.h:105-626).  The value equals
+   tango_absmax_ex_f32(out, row_mul = absmax_row_mul) bit for bit. */
 size_t tango_spmm_workspace(int64_t rows, int64_t nnz, int64_t W);
 int tango_spmm_csr_copy_u_ex(float* out, const int64_t* indptr, const void* indices, int idx_bits,
                              const int8_t* feat, int64_t ldf, const float* scale,
                              const float* row_scale, const float* bias, int relu, uint16_t* sign_bits,
                              int64_t rows, int64_t num_src, int64_t nnz, int64_t F, int64_t max_row_nnz,
+                             const float* absmax_row_mul, float* scale_out,
                              void* workspace, size_t workspace_bytes, tango_stream_t stream);
 
 /* csr_SPMM (cuda/src/cuda.cpp:110-117 -> SPMM.cu:23-68) on a graph whose heavy rows and heavy columns
@@ -318,7 +324,7 @@ int tango_spmm_dense_mask_build(const int64_t* indptr, const void* indices, int 
                                 const int32_t* extent_cols, const int64_t* mask_off, int64_t row_blocks,
                                 uint32_t* mask, uint8_t* keep, int32_t* kept, tango_stream_t stream);
 
-/* out as tango_spmm_csr_copy_u_ex computes it on the whole adjacency (same epilogue arguments).
+/* out as tango_spmm_csr_copy_u_ex computes it on the whole adjacency (same epilogue arguments, same scale output).
    Needs 16-byte aligned feat rows (ldf % 16 == 0, ceil16(F) <= ldf) and F <= 256, else
    TANGO_ERR_UNSUPPORTED (callers then use tango_spmm_csr_copy_u_ex on the whole CSR).
    workspace: tango_spmm_dense_workspace(plan, F) bytes, 256-byte aligned. */
@@ -326,6 +332,7 @@ size_t tango_spmm_dense_workspace(const tango_spmm_dense_plan* plan, int64_t F);
 int tango_spmm_csr_copy_u_dense(float* out, const tango_spmm_dense_plan* plan, const int8_t* feat,
                                 int64_t ldf, const float* scale, const float* row_scale,
                                 const float* bias, int relu, uint16_t* sign_bits, int64_t F,
+                                const float* absmax_row_mul, float* scale_out,
                                 void* workspace, size_t workspace_bytes, tango_stream_t stream);
 
 /* multi_cusparse_SPMM (cuda/src/cuda.cpp:119-158 -> SPMM.cu:70-194):

@@ -22,9 +22,12 @@ def _padded_i8(rows, cols, device):
 def _quantize_grad(dY, want_colsum=False):
     """Quantize a gradient (cuda/QLinear.py:42) with the configured rounding.  Returns
     (int8, scale, column sums or None): the bias gradient dY.sum(0) (cuda/QLinear.py:46)
-    comes out of the same read of dY that finds its scale."""
+    comes out of the same read of dY that finds its scale; a scale that the producer of dY left on it
+    (an aggregation's epilogue) is taken instead of a pass over dY."""
+    from .SPMM import grad_scale_hint
+    scale = grad_scale_hint(dY) if dY.is_contiguous() else None
     dY = dY if dY.is_contiguous() else dY.contiguous()
-    scale = colsum = None
+    colsum = None
     if want_colsum:
         scale, colsum = kernels.cuda_kernels.absmax_ex(dY, want_colsum=True)
     kw = {"round_mode": config.grad_round_mode}
@@ -76,8 +79,7 @@ def _forward(ctx, X, W, b, reduce, row_scale=None, scaleX=None, Xq=None):
         ctx.backward_cache = Xq, scaleX, W_, scaleW, b, None
         return res
     if scaleX is not None:
-        if row_scale is not None:
-            raise RuntimeError("QLinear: a precomputed input scale cannot be combined with row_scale")
+        pass  # with row_scale: the scale of X * row_scale[:, None], as its producer found it
     elif row_scale is not None:
         # the layer's "X * row_scale[:, None]" is folded into the quantize pass (no fp32 copy of X)
         scaleX, _ = kernels.cuda_kernels.absmax_ex(X, row_mul=row_scale)
@@ -105,8 +107,9 @@ def _backward(ctx, grad_output):
 class Qlinear_func(Function):
     """cuda/QLinear.py:26-47.  ``row_scale`` (optional, [M]) multiplies the rows of X before
     quantization, fused into the quantize pass and, in backward, into gradX's epilogue.
-    ``scaleX`` (optional, [1]) is max|X| / 127 when the producer of X already knows it
-    (a preceding Qlinear_func_reduce): no absmax pass over X runs then.  ``Xq`` (optional, with
+    ``scaleX`` (optional, [1]) is max|X| / 127 (of X * row_scale[:, None] when ``row_scale`` is given) when
+    the producer of X already knows it (a preceding Qlinear_func_reduce, an aggregation's epilogue): no absmax
+    pass over X runs then.  ``Xq`` (optional, with
     ``scaleX``): X already quantized (``quantize_input``), shared by several layers."""
 
     @staticmethod

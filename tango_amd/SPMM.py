@@ -16,6 +16,24 @@ def _gather_align(width):
     return 128
 
 
+def _dense_enough(g, reverse=False):
+    """Whether the aggregation of this orientation runs the row kernels, whose epilogue can return the scale of
+    its output (graphs averaging fewer than 64 slots per row take the slot-span kernels, which cannot)."""
+    if not config.scale_from_aggregation:
+        return False
+    indptr, indices = (g.adj_csr if reverse else g.adj_csc)[:2]
+    return indices.numel() >= 64 * (indptr.numel() - 1)
+
+
+def grad_scale_hint(t):
+    """max|t| / 127 if the kernel that produced the gradient ``t`` left it on the tensor and nothing has written
+    to ``t`` since (autograd may add another gradient into it in place), else None."""
+    hint = getattr(t, "_tango_scale", None)
+    if hint is not None and hint[1] == t._version and hint[2] == t.data_ptr():
+        return hint[0]
+    return None
+
+
 def _quantize_grad(t, padded):
     t = t if t.is_contiguous() else t.contiguous()
     kw = {"round_mode": config.grad_round_mode}
@@ -39,7 +57,11 @@ class spmm_copy_u(Function):
     as the separate multiplications."""
 
     @staticmethod
-    def forward(ctx, g, N, scaleN=None, row_scale=None, bias=None, relu=False, src_row_mul=None):
+    def forward(ctx, g, N, scaleN=None, row_scale=None, bias=None, relu=False, src_row_mul=None, want_scale=False,
+                scale_mul=None):
+        """``want_scale``: returns (out, max|out * scale_mul[:, None]| / 127) (``scale_mul`` optional): the scale the
+        next op's quantizer needs, from the aggregation's epilogue where the graph is dense enough for the row
+        kernels, else from a pass over out."""
         N = N if N.is_contiguous() else N.contiguous()
         fused = row_scale is not None or bias is not None or relu or src_row_mul is not None
         if fused and N.dim() != 2:
@@ -56,19 +78,42 @@ class spmm_copy_u(Function):
         bits = None
         if relu and N.dim() == 2 and N.size(1) % 16 == 0:
             bits = torch.empty((g.num_nodes(), N.size(1) // 16), dtype=torch.int16, device=N.device)
-        out = csr_SPMM(g, N_, scaleN, row_scale=row_scale, bias=bias, relu=relu, sign_bits=bits)
+        scale_out = None
+        if want_scale and N.dim() == 2 and _dense_enough(g):
+            out, scale_out = csr_SPMM(g, N_, scaleN, row_scale=row_scale, bias=bias, relu=relu, sign_bits=bits,
+                                      want_scale=True, scale_mul=scale_mul)
+        else:
+            out = csr_SPMM(g, N_, scaleN, row_scale=row_scale, bias=bias, relu=relu, sign_bits=bits)
+            if want_scale:
+                scale_out, _ = cuda_kernels.absmax_ex(out.reshape(out.size(0), -1), row_mul=scale_mul)
         # the op's own output goes through save_for_backward (autograd then holds it without the
         # output -> grad_fn -> ctx -> output cycle a plain attribute would form); everything else is an input
         # or an auxiliary tensor, kept as the reference keeps its cache (cuda/SPMM.py:13)
         ctx.backward_cache = g, row_scale, bias is not None, bits, relu
         if relu and bits is None:
             ctx.save_for_backward(out)
+        if want_scale:
+            ctx.mark_non_differentiable(scale_out)
+            ctx.set_materialize_grads(False)
+            return out, scale_out
         return out
 
     @staticmethod
+    def _reverse(ctx, g, dZ_, scaledZ):
+        """The reverse aggregation; on dense graphs its epilogue also finds max|dN| / 127, left on the result for
+        the op that quantizes this gradient next (``grad_scale_hint``)."""
+        if dZ_.dim() == 2 and _dense_enough(g, True):
+            dN, s = csr_SPMM(g, dZ_, scaledZ, True, row_scale=ctx.src_row_mul, want_scale=True)
+            dN._tango_scale = (s, dN._version, dN.data_ptr())
+            return dN
+        return csr_SPMM(g, dZ_, scaledZ, True, row_scale=ctx.src_row_mul)
+
+    @staticmethod
     @once_differentiable
-    def backward(ctx, dOut):
+    def backward(ctx, dOut, dscale=None):
         refuse_capture("spmm_copy_u.backward")
+        if dOut is None:
+            return (None,) * 9
         g, row_scale, has_bias, mask, relu = ctx.backward_cache
         if relu and mask is None:
             mask, = ctx.saved_tensors
@@ -76,8 +121,8 @@ class spmm_copy_u(Function):
         if row_scale is None and not has_bias and mask is None:
             if ctx.needs_input_grad[1]:
                 dZ_, scaledZ = _quantize_grad(dOut, True)
-                dN = csr_SPMM(g, dZ_, scaledZ, True, row_scale=ctx.src_row_mul)
-            return None, dN, None, None, None, None, None
+                dN = spmm_copy_u._reverse(ctx, g, dZ_, scaledZ)
+            return None, dN, None, None, None, None, None, None, None
         dOut = dOut if dOut.is_contiguous() else dOut.contiguous()
         want_bias = has_bias and ctx.needs_input_grad[4]
         # dZ = (dOut where out > 0) * row_scale; its scale and the bias gradient come from one pass
@@ -89,8 +134,8 @@ class spmm_copy_u(Function):
                 kw.update(config.stochastic_args(dOut.device))
             dZ_, _ = quantize_padded(dOut, scaledZ, row_mul=row_scale, mask=mask, mask_mode=mode,
                                      align=_gather_align(dOut.size(1)), **kw)
-            dN = csr_SPMM(g, dZ_, scaledZ, True, row_scale=ctx.src_row_mul)
-        return None, dN, None, None, dbias, None, None
+            dN = spmm_copy_u._reverse(ctx, g, dZ_, scaledZ)
+        return None, dN, None, None, dbias, None, None, None, None
 
 
 def _need_reduce_last_dim(ufeat, efeat):

@@ -21,6 +21,13 @@ edge_values_on_load = os.environ.get("TANGO_EDGE_ON_LOAD", "0") == "1"
 # per slot lengthen the softmax kernel's latency chain by more than the stored tensor costs), hence off.
 attention_logits_on_the_fly = os.environ.get("TANGO_ATTN_ON_THE_FLY", "0") == "1"
 
+# spmm_copy_u on dense graphs: let the aggregation's epilogue return the scale of its output (forward: to the next
+# layer's GEMM; backward: to the quantizer of the gradient it produces) instead of a pass over that output.  Same
+# values.  Measured on the 114.8 M-edge benchmark epoch: the three passes it removes take 100 us, but the few
+# registers the epilogue needs for it cost the gather kernel one of its eight waves per SIMD (65 instead of 64
+# VGPRs) and with it 50 us per launch: 5.66 against 5.61 ms per epoch, hence off.
+scale_from_aggregation = os.environ.get("TANGO_SCALE_FROM_AGGREGATION", "0") == "1"
+
 # Seed of the counter-based RNG for stochastic rounding; every quantize call
 # draws a fresh 2^40-element window of the stream.
 seed = int(os.environ.get("TANGO_SEED", "0"))

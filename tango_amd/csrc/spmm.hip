@@ -69,6 +69,10 @@ struct SpmmParams {
     const int* part;       // optional int32 partial sums added to a row's sum before dequantization (the dense
     const int* part_slot;  // blocks of spmm_dense.hip): row r owns row part_slot[r] of part (stride part_ld ints)
     int part_ld;           // when that is not negative
+    float* amax_part;      // optional: [rows][amax_tiles] receives max |out * amax_mul[row]| of every row piece stored
+    const float* amax_mul; // (amax_mul optional), from which amax_reduce_kernel forms the scale of the output
+    int amax_tiles;
+    float* amax_scale;     // where amax_reduce_kernel maxes the scale into (holds 0 or a partial result on entry)
     const int* row_order;  // optional: workgroups take rows in this order (rows of similar length side by side,
                            // whatever the numbering of the nodes) instead of by row number
 };
@@ -293,10 +297,9 @@ __device__ __forceinline__ void store_sign_bits(const SpmmParams& p, int64_t row
     p.sign_bits[row * (p.W >> 4) + (col >> 4)] = static_cast<uint16_t>(b);
 }
 
-// Dequantize and store one output row's tile; called by the lanes with grp == 0.
-template <int VEC>
-__device__ __forceinline__ void store_row(const SpmmParams& p, const LaneCols& c, int64_t row, const int* acc) {
-    if (!c.col_ok) return;
+// Dequantize and store one output row's tile; called by all lanes of one lane group (grp == 0 in the row kernels).
+template <int VEC, bool AMAX>
+__device__ __forceinline__ float store_row_piece(const SpmmParams& p, const LaneCols& c, int64_t row, const int* acc) {
     const float s = p.scale2 ? p.scale[0] * p.scale2[0] : p.scale[0];
     const float rs = p.row_scale ? p.row_scale[row] : 1.0f;
     float* o = p.out + row * p.W + c.col;
@@ -331,6 +334,13 @@ __device__ __forceinline__ void store_row(const SpmmParams& p, const LaneCols& c
 #pragma unroll
         for (int i = 0; i < VEC; ++i) y[i] = activate(y[i], p.relu);
     }
+    float m = 0.0f;
+    if (AMAX) {
+        const float mul = p.amax_mul ? p.amax_mul[row] : 1.0f;
+#pragma unroll
+        for (int i = 0; i < VEC; ++i)
+            if (c.col + i < p.W) m = fmaxf(m, fabsf(y[i] * mul));  // * 1.0f is exact
+    }
     if (VEC == 16 && p.out_vec && c.col + 16 <= p.W) {
         f32x4* o4 = reinterpret_cast<f32x4*>(o);
 #pragma unroll
@@ -343,6 +353,35 @@ __device__ __forceinline__ void store_row(const SpmmParams& p, const LaneCols& c
     }
     // after the row's own stores, so that the sixteen values need not all be live at once
     if (VEC == 16 && p.sign_bits) store_sign_bits<VEC>(p, row, c.col, y);
+    return m;
+}
+
+// AMAX: also leave max |out * amax_mul[row]| of the piece in p.amax_part.  A variant of its own: the few registers
+// it takes cost the row kernel one of its eight waves per SIMD, so kernels are built with it only where asked.
+template <int VEC, bool AMAX = false>
+__device__ __forceinline__ void store_row(const SpmmParams& p, const LaneCols& c, int64_t row, const int* acc) {
+    float m = 0.0f;
+    if (c.col_ok) m = store_row_piece<VEC, AMAX>(p, c, row, acc);
+    if (AMAX) {  // the lanes of the piece are all here, also those past the row's width
+        for (int off = c.lpe >> 1; off > 0; off >>= 1) m = fmaxf(m, __shfl_xor(m, off, kWave));
+        if (c.sub == 0) p.amax_part[row * p.amax_tiles + blockIdx.y] = m;
+    }
+}
+
+// scale[0] = max(scale[0], max(part[0 .. n)) / 127): scale must hold 0 (or an earlier partial result) on entry.
+// x -> fl(x / 127) is monotone, so the maximum of the workgroups' quotients is the quotient of the maximum.
+__global__ __launch_bounds__(256) void amax_reduce_kernel(const float* __restrict__ part, int64_t n, float* scale) {
+    float m = 0.0f;
+    for (int64_t i = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x; i < n; i += static_cast<int64_t>(gridDim.x) * 256)
+        m = fmaxf(m, part[i]);
+    __shared__ float w[4];
+    m = wave_max(m);
+    if ((threadIdx.x & 63) == 0) w[threadIdx.x >> 6] = m;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        m = fmaxf(fmaxf(w[0], w[1]), fmaxf(w[2], w[3]));
+        atomicMax(reinterpret_cast<int*>(scale), __float_as_int(m / 127.0f));
+    }
 }
 
 template <int KIND>
@@ -376,7 +415,7 @@ __device__ __forceinline__ int64_t lower_bound_wave(const int64_t* a, int64_t n,
 // blockDim.x = 256.  WPR = waves that share one output row (1 or 4).
 // gridDim.y tiles the columns in chunks of p.tile bytes.
 // Rows with more than p.long_row slots are left to spmm_long_kernel.
-template <int VEC, int WPR, int KIND>
+template <int VEC, int WPR, int KIND, bool AMAX = false>
 __global__ __launch_bounds__(256) void spmm_kernel(const SpmmParams p) {
     const int lane = lane_id();
     const int wave = __builtin_amdgcn_readfirstlane(static_cast<int>(threadIdx.x) >> 6);
@@ -419,7 +458,7 @@ __global__ __launch_bounds__(256) void spmm_kernel(const SpmmParams p) {
                 acc[i] += part[i * 64 + c.sub] + part[64 * VEC + i * 64 + c.sub] + part[2 * 64 * VEC + i * 64 + c.sub];
         }
     }
-    if (c.grp == 0) store_row<VEC>(p, c, row, acc);
+    if (c.grp == 0) store_row<VEC, AMAX>(p, c, row, acc);
 }
 
 // Sparse graphs (a handful of neighbours per row): a wavefront that owns one row would leave most
@@ -598,7 +637,8 @@ __global__ __launch_bounds__(1024) void spmm_long_kernel(const SpmmParams p) {
                     acc[i] = part[i * 64 + c.sub];
                     part[i * 64 + c.sub] = 0;
                 }
-                store_row<VEC>(p, c, row, acc);
+                if (p.amax_part) store_row<VEC, true>(p, c, row, acc);  // uniform
+                else store_row<VEC>(p, c, row, acc);
             }
             __syncthreads();
         }
@@ -699,12 +739,13 @@ __global__ __launch_bounds__(256) void spmm_hub_store_kernel(const SpmmParams p)
     const int64_t* hubs = hub_list(p.hub_ws);
     for (int h = blockIdx.x * 4 + wave; h < nhub; h += gridDim.x * 4) {
         const int64_t row = hubs[h];
-        if (c.grp == 0 && c.col_ok) {
+        if (c.grp == 0) {
             const int* orow = reinterpret_cast<const int*>(p.out) + row * p.W + c.col;
             int acc[VEC];
 #pragma unroll
-            for (int i = 0; i < VEC; ++i) acc[i] = (c.col + i < p.W) ? orow[i] : 0;
-            store_row<VEC>(p, c, row, acc);
+            for (int i = 0; i < VEC; ++i) acc[i] = (c.col_ok && c.col + i < p.W) ? orow[i] : 0;
+            if (p.amax_part) store_row<VEC, true>(p, c, row, acc);  // uniform
+            else store_row<VEC>(p, c, row, acc);
         }
     }
 }
@@ -1093,6 +1134,7 @@ static int launch_spmm(SpmmParams p, int vec, hipStream_t s) {
         while ((1LL << p.ldf_shift) < p.ldf) ++p.ldf_shift;
     }
     const int64_t ychunks = ceil_div(p.W, p.tile);
+    p.amax_tiles = static_cast<int>(ychunks);
     if (ychunks > 65535) return TANGO_ERR_UNSUPPORTED;
     // four waves split each row when rows are long AND wide (few neighbours per load instruction);
     // otherwise one wave per row, which amortises the per-row latencies over more edges
@@ -1128,7 +1170,7 @@ static int launch_spmm(SpmmParams p, int vec, hipStream_t s) {
     const int64_t nspans_all = ceil_div(p.nnz, kSpanSlots);
     const bool span_fits = span_parts_offset(nspans_all) + sizeof(int) * 2 * static_cast<size_t>(nspans_all) *
                                static_cast<size_t>(ychunks * p.tile) <= p.span_ws_bytes;
-    if (KIND != KIND_COO && p.span_ws && span_fits && span_graph(p.rows, p.nnz) && !p.part) {  // sparse graph: slot spans, two launches
+    if (KIND != KIND_COO && p.span_ws && span_fits && span_graph(p.rows, p.nnz) && !p.part && !p.amax_part) {  // sparse graph: slot spans, two launches
         const int64_t nspans = nspans_all;
         p.span_wp = ychunks * p.tile;
         const dim3 spgrid(static_cast<unsigned>(ceil_div(nspans > 0 ? nspans : 1, 4)), static_cast<unsigned>(ychunks));
@@ -1151,7 +1193,7 @@ static int launch_spmm(SpmmParams p, int vec, hipStream_t s) {
     }
 #undef TANGO_SPMM_LONG
     // Sparse graph: lane groups own the short rows, single waves the rest up to long_row.
-    if (KIND != KIND_COO && p.nnz < 64 * p.rows && p.lpe_log2 < 6 && !p.part) {
+    if (KIND != KIND_COO && p.nnz < 64 * p.rows && p.lpe_log2 < 6 && !p.part && !p.amax_part) {
         p.group_row = kGroupRow;
         const int64_t rows_per_block = 4LL << (6 - p.lpe_log2);
         const dim3 ggrid(static_cast<unsigned>(ceil_div(p.rows, rows_per_block)), static_cast<unsigned>(ychunks));
@@ -1169,7 +1211,11 @@ static int launch_spmm(SpmmParams p, int vec, hipStream_t s) {
     }
 #define TANGO_SPMM_LAUNCH(V, WPR) \
     hipLaunchKernelGGL((spmm_kernel<V, WPR, KIND>), grid, dim3(256), 0, s, p)
-    if (vec == 16) {
+    if (p.amax_part) {  // copy_u only (the entry points see to that)
+        if (vec != 16 || KIND != KIND_COPY) return TANGO_ERR_UNSUPPORTED;
+        if (wide) hipLaunchKernelGGL((spmm_kernel<16, 4, KIND_COPY, true>), grid, dim3(256), 0, s, p);
+        else hipLaunchKernelGGL((spmm_kernel<16, 1, KIND_COPY, true>), grid, dim3(256), 0, s, p);
+    } else if (vec == 16) {
         if (wide) TANGO_SPMM_LAUNCH(16, 4); else TANGO_SPMM_LAUNCH(16, 1);
     } else if (vec == 4) {
         if (wide) TANGO_SPMM_LAUNCH(4, 4); else TANGO_SPMM_LAUNCH(4, 1);
@@ -1177,6 +1223,11 @@ static int launch_spmm(SpmmParams p, int vec, hipStream_t s) {
         if (wide) TANGO_SPMM_LAUNCH(1, 4); else TANGO_SPMM_LAUNCH(1, 1);
     }
 #undef TANGO_SPMM_LAUNCH
+    if (p.amax_part) {
+        const int64_t n = p.rows * ychunks;
+        hipLaunchKernelGGL(amax_reduce_kernel, dim3(static_cast<unsigned>(n < 65536 ? ceil_div(n, 256) : 256)), dim3(256),
+                           0, s, p.amax_part, n, p.amax_scale);
+    }
     return launch_status();
 }
 
@@ -1195,8 +1246,10 @@ using namespace tango;
 
 extern "C" {
 
-size_t tango_spmm_workspace(int64_t rows, int64_t nnz, int64_t W) {
-    if (rows < 0 || nnz < 0 || W < 0) return 0;
+// floats of per-row-piece maxima an aggregation with a scale output writes: a row has at most W / 64 + 1 pieces
+static size_t amax_floats(int64_t rows, int64_t W) { return static_cast<size_t>(rows) * static_cast<size_t>(W / 64 + 2); }
+
+static size_t spmm_base_workspace(int64_t rows, int64_t nnz, int64_t W) {
     if (span_graph(rows, nnz)) {
         // two int32 partial rows per span.  Their padded width is column tiles x tile: below 2 W + 16 while the
         // lanes of a row piece fit a wavefront (tile = vec x the lane count rounded up to a power of two), and
@@ -1205,6 +1258,11 @@ size_t tango_spmm_workspace(int64_t rows, int64_t nnz, int64_t W) {
         return span_parts_offset(nspans) + sizeof(int) * 2 * static_cast<size_t>(nspans) * static_cast<size_t>(2 * W + 16);
     }
     return 64 + sizeof(int64_t) * static_cast<size_t>(nnz / kHubRowMin + 2);
+}
+
+size_t tango_spmm_workspace(int64_t rows, int64_t nnz, int64_t W) {
+    if (rows < 0 || nnz < 0 || W < 0) return 0;
+    return ((spmm_base_workspace(rows, nnz, W) + 255) & ~static_cast<size_t>(255)) + sizeof(float) * amax_floats(rows, W);
 }
 
 int tango_spmm_csr_copy_u(float* out, const int64_t* indptr, const int64_t* indices,
@@ -1224,9 +1282,11 @@ int tango_spmm_csr_copy_u_ex(float* out, const int64_t* indptr, const void* indi
                              const int8_t* feat, int64_t ldf, const float* scale,
                              const float* row_scale, const float* bias, int relu, uint16_t* sign_bits,
                              int64_t rows, int64_t num_src, int64_t nnz, int64_t F, int64_t max_row_nnz,
+                             const float* absmax_row_mul, float* scale_out,
                              void* workspace, size_t workspace_bytes, tango_stream_t stream) {
     if (rows < 0 || F < 0 || nnz < 0 || num_src < 0 || ldf < F || !scale || !indptr || max_row_nnz < 0 ||
-        (rows * F > 0 && !out) || (nnz > 0 && (!indices || !feat)) || (idx_bits != 32 && idx_bits != 64))
+        (rows * F > 0 && !out) || (nnz > 0 && (!indices || !feat)) || (idx_bits != 32 && idx_bits != 64) ||
+        (scale_out && !workspace))
         return TANGO_ERR_INVALID_ARG;
     if (workspace && (workspace_bytes < tango_spmm_workspace(rows, nnz, F) || (reinterpret_cast<uintptr_t>(workspace) & 15)))
         return TANGO_ERR_WORKSPACE;
@@ -1237,7 +1297,11 @@ int tango_spmm_csr_copy_u_ex(float* out, const int64_t* indptr, const void* indi
     const int vec = pick_vec(feat, ldf, F);
     if (sign_bits && (vec != 16 || (F & 15) != 0)) return TANGO_ERR_UNSUPPORTED;
     p.row_scale = row_scale; p.bias = bias; p.relu = relu; p.sign_bits = sign_bits; p.max_row = max_row_nnz; p.hub_ws = workspace;
-    p.span_ws = workspace; p.span_ws_bytes = workspace_bytes;
+    p.span_ws = workspace; p.span_ws_bytes = workspace ? (spmm_base_workspace(rows, nnz, F) + 255) & ~static_cast<size_t>(255) : 0;
+    if (scale_out && rows * F > 0) {
+        p.amax_part = reinterpret_cast<float*>(static_cast<char*>(workspace) + p.span_ws_bytes);
+        p.amax_mul = absmax_row_mul; p.amax_scale = scale_out;
+    }
     p.rows = rows; p.num_src = num_src; p.ldf = ldf; p.W = F; p.F = F; p.D = 1; p.nnz = nnz;
     return launch_spmm<KIND_COPY>(p, pick_vec(feat, ldf, F), as_stream(stream));
 }
@@ -1316,12 +1380,14 @@ size_t tango_spmm_dense_workspace(const tango_spmm_dense_plan* plan, int64_t F) 
     const size_t dense = dense_workspace_bytes(*plan, F);
     if (!dense) return 0;
     // the gather kernels' own workspace for hub rows of the rest follows the dense part
-    return dense + ((64 + sizeof(int64_t) * static_cast<size_t>(plan->res_nnz / kHubRowMin + 2) + 255) & ~static_cast<size_t>(255));
+    return dense + ((64 + sizeof(int64_t) * static_cast<size_t>(plan->res_nnz / kHubRowMin + 2) + 255) & ~static_cast<size_t>(255)) +
+           sizeof(float) * amax_floats(plan->rows, F);
 }
 
 int tango_spmm_csr_copy_u_dense(float* out, const tango_spmm_dense_plan* plan, const int8_t* feat,
                                 int64_t ldf, const float* scale, const float* row_scale,
                                 const float* bias, int relu, uint16_t* sign_bits, int64_t F,
+                                const float* absmax_row_mul, float* scale_out,
                                 void* workspace, size_t workspace_bytes, tango_stream_t stream) {
     if (!plan || F < 0 || !scale || ldf < F || !feat || plan->rows < 0 || plan->res_nnz < 0 || !plan->res_indptr ||
         !plan->row_slot || (plan->rows * F > 0 && !out) || (plan->res_nnz > 0 && !plan->res_indices))
@@ -1346,6 +1412,11 @@ int tango_spmm_csr_copy_u_dense(float* out, const tango_spmm_dense_plan* plan, c
     p.row_scale = row_scale; p.bias = bias; p.relu = relu; p.sign_bits = sign_bits; p.max_row = plan->res_max_row;
     p.row_order = plan->row_order;
     p.hub_ws = static_cast<char*>(workspace) + dense_workspace_bytes(*plan, F);
+    if (scale_out) {
+        p.amax_part = reinterpret_cast<float*>(static_cast<char*>(p.hub_ws) +
+                                               ((64 + sizeof(int64_t) * static_cast<size_t>(plan->res_nnz / kHubRowMin + 2) + 255) & ~static_cast<size_t>(255)));
+        p.amax_mul = absmax_row_mul; p.amax_scale = scale_out;
+    }
     p.rows = plan->rows; p.num_src = plan->num_src; p.ldf = ldf; p.W = F; p.F = F; p.D = 1; p.nnz = plan->res_nnz;
     return launch_spmm<KIND_COPY>(p, 16, as_stream(stream));
 }

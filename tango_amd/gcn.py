@@ -30,9 +30,11 @@ class QGraphConv(nn.Module):
         if self.bias is not None:
             nn.init.zeros_(self.bias)
 
-    def forward(self, graph, feat, norms=None):
+    def forward(self, graph, feat, norms=None, feat_scale=None, want_scale=False):
         """``norms``: (out_deg^-1/2, in_deg^-1/2) from ``degree_norms`` when the caller computes them once
-        for several layers of one forward pass; the reference's layer computes them itself every time."""
+        for several layers of one forward pass; the reference's layer computes them itself every time.
+        ``want_scale`` (fused layers that multiply first): also returns max|out * out_deg^-1/2| / 127, which the
+        next such layer takes as ``feat_scale`` instead of scanning its input."""
         norm_src, norm_dst = degree_norms(graph) if norms is None else norms
         relu = self._activation is torch.relu
         if self.fused:
@@ -40,11 +42,13 @@ class QGraphConv(nn.Module):
             # "* norm_src" into the quantize of the GEMM / aggregation input, "* norm_dst, + bias,
             # relu" into the aggregation's epilogue (or "* norm_dst" into nothing when the GEMM is last)
             if self._in_feats > self._out_feats:
-                y, sy = Qlinear_func_reduce.apply(feat, self.weight, None, norm_src)
-                rst = spmm_copy_u.apply(graph, y, sy, norm_dst, self.bias, relu)
+                y, sy = Qlinear_func_reduce.apply(feat, self.weight, None, norm_src, feat_scale)
+                emit = want_scale and (self._activation is None or relu)
+                rst = spmm_copy_u.apply(graph, y, sy, norm_dst, self.bias, relu, None, emit, norm_src if emit else None)
+                rst, scale = rst if emit else (rst, None)
                 if self._activation is not None and not relu:
                     rst = self._activation(rst)
-                return rst
+                return (rst, scale) if want_scale else rst
             rst = spmm_copy_u.apply(graph, feat, None, None, None, False, norm_src)  # "feat * norm_src" in the quantize pass
             rst = Qlinear_func.apply(rst, self.weight) * norm_dst.unsqueeze(1)
         else:
@@ -61,7 +65,7 @@ class QGraphConv(nn.Module):
             rst = rst + self.bias
         if self._activation is not None:
             rst = self._activation(rst)
-        return rst
+        return (rst, None) if want_scale else rst
 
 
 class GCN(nn.Module):
@@ -80,10 +84,18 @@ class GCN(nn.Module):
     def forward(self, features):
         h = features
         norms = degree_norms(self.g)  # once per forward pass, shared by the layers
+        scale = None
+        last = len(self.layers) - 1
         for i, layer in enumerate(self.layers):
             if i != 0:
                 h = self.dropout(h)
-            h = layer(self.g, h, norms)
+            # a layer's aggregation hands max|h * out_deg^-1/2| / 127 to the next layer's GEMM, unless dropout
+            # changes h in between
+            hand_on = i < last and (self.dropout.p == 0.0 or not self.training)
+            if hand_on:
+                h, scale = layer(self.g, h, norms, scale, True)
+            else:
+                h, scale = layer(self.g, h, norms, scale), None
         return h
 
 

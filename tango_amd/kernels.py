@@ -482,9 +482,11 @@ class cuda_kernels:
     # ------------------------------------------------------------------ SpMM
     @staticmethod
     def csr_SPMM(out, indptr, indices, U, scaleU, ldf=None, F=None, row_scale=None, bias=None, relu=False,
-                 max_row=0, sign_bits=None):
+                 max_row=0, sign_bits=None, scale_out=None, scale_mul=None):
         """``sign_bits`` (int16 [rows, F / 16], F a multiple of 16): receives one bit per output element,
-        set where it is positive: all a backward pass needs of a ReLU's output."""
+        set where it is positive: all a backward pass needs of a ReLU's output.
+        ``scale_out`` (1-element fp32 holding 0): receives max|out * scale_mul[:, None]| / 127 (``scale_mul``
+        optional, one fp32 per row), formed in the kernel's epilogue."""
         _need(out, torch.float32, "out")
         _need(indptr, torch.int64, "indptr")
         idx_bits = _need_index(indices, "indices")
@@ -500,7 +502,8 @@ class cuda_kernels:
             _need(sign_bits, torch.int16, "sign_bits")
             if F % 16 or tuple(sign_bits.shape) != (rows, F // 16):
                 raise RuntimeError("csr_SPMM: sign_bits must be int16 [rows, F / 16], F a multiple of 16")
-        if row_scale is None and bias is None and not relu and idx_bits == 64 and not max_row and sign_bits is None:
+        if (row_scale is None and bias is None and not relu and idx_bits == 64 and not max_row and sign_bits is None
+                and scale_out is None):
             check(_L.tango_spmm_csr_copy_u(_ptr(out), indptr.data_ptr(), _ptr(indices), _ptr(U), ldf,
                                            scaleU.data_ptr(), rows, U.size(0), indices.numel(), F,
                                            _stream()), "csr_SPMM")
@@ -513,15 +516,21 @@ class cuda_kernels:
             _need(bias, torch.float32, "bias")
             if bias.numel() != F:
                 raise RuntimeError("csr_SPMM: bias must have F entries")
+        if scale_mul is not None:
+            _need(scale_mul, torch.float32, "scale_mul")
+            if scale_mul.numel() != rows or scale_out is None:
+                raise RuntimeError("csr_SPMM: scale_mul needs one entry per output row and a scale_out")
         ws_bytes = _ws_bytes("tango_spmm_workspace", rows, indices.numel(), F)
         ws = _workspace(ws_bytes, U.device)
         check(_L.tango_spmm_csr_copy_u_ex(_ptr(out), indptr.data_ptr(), _ptr(indices), idx_bits, _ptr(U), ldf,
                                           scaleU.data_ptr(), _ptr(row_scale), _ptr(bias), int(bool(relu)),
-                                          _ptr(sign_bits), rows, U.size(0), indices.numel(), F, int(max_row), _ptr(ws), ws_bytes,
+                                          _ptr(sign_bits), rows, U.size(0), indices.numel(), F, int(max_row),
+                                          _ptr(scale_mul), _ptr(scale_out), _ptr(ws), ws_bytes,
                                           _stream()), "csr_SPMM")
 
     @staticmethod
-    def csr_SPMM_dense(out, plan, U, scaleU, ldf=None, F=None, row_scale=None, bias=None, relu=False, sign_bits=None):
+    def csr_SPMM_dense(out, plan, U, scaleU, ldf=None, F=None, row_scale=None, bias=None, relu=False, sign_bits=None,
+                       scale_out=None, scale_mul=None):
         """csr_SPMM on an adjacency split by ``dense_plan.build_dense_plan`` into bit blocks (multiplied with
         U on the matrix cores) and a sparse rest; same result as csr_SPMM on the whole CSR, bit for bit.
         Returns False (nothing launched) when U's layout rules the dense path out."""
@@ -547,14 +556,18 @@ class cuda_kernels:
             _need(bias, torch.float32, "bias")
             if bias.numel() != F:
                 raise RuntimeError("csr_SPMM_dense: bias must have F entries")
+        if scale_mul is not None:
+            _need(scale_mul, torch.float32, "scale_mul")
+            if scale_mul.numel() != plan.rows or scale_out is None:
+                raise RuntimeError("csr_SPMM_dense: scale_mul needs one entry per output row and a scale_out")
         key = ("dense", id(plan), F)
         ws_bytes = _WS_SIZES.get(key)
         if ws_bytes is None:
             ws_bytes = _WS_SIZES[key] = _L.tango_spmm_dense_workspace(plan.ref, F)
         ws = _workspace(ws_bytes, U.device)
         check(_L.tango_spmm_csr_copy_u_dense(_ptr(out), plan.ref, _ptr(U), ldf, scaleU.data_ptr(), _ptr(row_scale),
-                                             _ptr(bias), int(bool(relu)), _ptr(sign_bits), F, _ptr(ws), ws_bytes,
-                                             _stream()), "csr_SPMM_dense")
+                                             _ptr(bias), int(bool(relu)), _ptr(sign_bits), F, _ptr(scale_mul),
+                                             _ptr(scale_out), _ptr(ws), ws_bytes, _stream()), "csr_SPMM_dense")
         return True
 
     @staticmethod
@@ -1007,31 +1020,33 @@ def incidence_SPMM(g, E, scaleE, reverse=False):
     return out.view(out_shape)
 
 
-def csr_SPMM(g, N, scaleN, reverse=False, row_scale=None, bias=None, relu=False, sign_bits=None):
+def csr_SPMM(g, N, scaleN, reverse=False, row_scale=None, bias=None, relu=False, sign_bits=None, want_scale=False,
+             scale_mul=None):
     """cuda/kernels.py:154-165.  N may be a 2-D view of a row-padded buffer.  ``row_scale`` / ``bias`` /
     ``relu`` fold "* norm, + bias, activation" (evaluation/test_gcn.py:123-137) into the kernel's epilogue;
-    ``sign_bits`` (int16 [n, F / 16]) receives the signs of the output."""
+    ``sign_bits`` (int16 [n, F / 16]) receives the signs of the output.  ``want_scale``: also returns
+    max|out * scale_mul[:, None]| / 127 (``scale_mul`` optional), found in the epilogue: (out, scale)."""
     indptr, indices, _, longest = _csr_of(g, reverse)
     feat_shape = N.shape[1:]
     out_shape = (g.num_nodes(),) + feat_shape
     dim = math.prod(N.shape[1:])
     out = torch.empty((g.num_nodes(), dim), dtype=torch.float32, device=N.device)
+    scale_out = None
+    if want_scale:
+        scale_out = _zero_slot(N.device)
+        if scale_out is None:
+            scale_out = torch.zeros(1, dtype=torch.float32, device=N.device)
+    extra = dict(row_scale=row_scale, bias=bias, relu=relu, sign_bits=sign_bits, scale_out=scale_out, scale_mul=scale_mul)
     plan = getattr(g, "dense_csr" if reverse else "dense_csc", None)
     if N.dim() == 2 and not N.is_contiguous():
         ld = _rows_view(N, "N")
         base = N.as_strided((N.size(0), ld), (ld, 1))
-        if plan is not None and cuda_kernels.csr_SPMM_dense(out, plan, base, scaleN, ldf=ld, F=dim, row_scale=row_scale,
-                                                            bias=bias, relu=relu, sign_bits=sign_bits):
-            return out.view(out_shape)
-        cuda_kernels.csr_SPMM(out, indptr, indices, base, scaleN, ldf=ld, F=dim, row_scale=row_scale, bias=bias,
-                              relu=relu, max_row=longest, sign_bits=sign_bits)
-    elif plan is not None and cuda_kernels.csr_SPMM_dense(out, plan, N.reshape(N.size(0), dim), scaleN, row_scale=row_scale,
-                                                          bias=bias, relu=relu, sign_bits=sign_bits):
-        pass
-    else:
-        cuda_kernels.csr_SPMM(out, indptr, indices, N, scaleN, row_scale=row_scale, bias=bias, relu=relu,
-                              max_row=longest, sign_bits=sign_bits)
-    return out.view(out_shape)
+        if not (plan is not None and cuda_kernels.csr_SPMM_dense(out, plan, base, scaleN, ldf=ld, F=dim, **extra)):
+            cuda_kernels.csr_SPMM(out, indptr, indices, base, scaleN, ldf=ld, F=dim, max_row=longest, **extra)
+    elif not (plan is not None and cuda_kernels.csr_SPMM_dense(out, plan, N.reshape(N.size(0), dim), scaleN, **extra)):
+        cuda_kernels.csr_SPMM(out, indptr, indices, N, scaleN, max_row=longest, **extra)
+    out = out.view(out_shape)
+    return (out, scale_out) if want_scale else out
 
 
 def multi_cusparse_SPMV(g, N_T, E_T, scale, reverse=False):

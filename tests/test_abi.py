@@ -44,7 +44,7 @@ def test_argument_validation_needs_no_gpu():
     assert L.tango_sddmm_ewise_i8(7, 1, None, 1, 1, 1, 1, 1, 1, 4, 4, None) == -2  # unknown op
     assert L.tango_spmm_csr_copy_u(1, 1, 1, 1, 8, 1, 4, 1 << 31, 10, 8, None) == -2  # node ids must fit 31 bits
     # the dense-block aggregation: a plan is required, and features wider than 256 columns have no workspace size
-    assert L.tango_spmm_csr_copy_u_dense(1, None, 1, 64, 1, None, None, 0, None, 64, None, 0, None) == -1
+    assert L.tango_spmm_csr_copy_u_dense(1, None, 1, 64, 1, None, None, 0, None, 64, None, None, None, 0, None) == -1
     plan = _lib.DensePlan()
     plan.rows, plan.num_src, plan.row_blocks, plan.dense_rows, plan.dense_cols = 512, 512, 1, 256, 256
     assert L.tango_spmm_dense_workspace(ctypes.byref(plan), 300) == 0

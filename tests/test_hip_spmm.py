@@ -198,5 +198,5 @@ def test_spmm_without_workspace(K, orc, kind, n, e, F):
     s = sc(0.25)
     st = torch.cuda.current_stream().cuda_stream
     assert _lib.lib().tango_spmm_csr_copy_u_ex(out.data_ptr(), ip.data_ptr(), ix.data_ptr(), 64, feat.data_ptr(), F,
-                                               s.data_ptr(), None, None, 0, None, n, n, e, F, 0, None, 0, st) == 0
+                                               s.data_ptr(), None, None, 0, None, n, n, e, F, 0, None, None, None, 0, st) == 0
     assert np.array_equal(host(out), orc.spmm_csr_copy_u(o["adj_csc"][0], o["adj_csc"][1], host(feat), 0.25))

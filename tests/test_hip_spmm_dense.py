@@ -179,3 +179,77 @@ def test_graph_level_wrapper_uses_the_plan(K, orc):
     for reverse, fmt in ((False, "adj_csc"), (True, "adj_csr")):
         got = K.csr_SPMM(g, dev(feat), sc(0.01), reverse=reverse)
         assert np.array_equal(host(got), orc.spmm_csr_copy_u(o[fmt][0], o[fmt][1], feat, np.float32(0.01)))
+
+
+@pytest.mark.parametrize("with_plan", [False, True])
+@pytest.mark.parametrize("F,use_mul", [(256, True), (41, False), (64, True)])
+def test_aggregation_returns_the_scale_of_its_output(K, orc, F, use_mul, with_plan):
+    """The scale an aggregation's epilogue finds for its own output is max|out * mul| / 127 of the stored values."""
+    from tango_amd.dense_plan import build_dense_plan
+    from tango_amd.graph import Graph
+    from tango_amd.util import graph_preprocess
+    rng = np.random.default_rng(F)
+    n = 2200
+    s, d = heavy_graph(rng, n, 220_000, symmetric=False)
+    g = graph_preprocess(Graph(dev(s), dev(d), n))
+    if with_plan:
+        g.dense_csc = build_dense_plan(g.adj_csc[0], g.adj_csc32[0], n, tau=0.02, groups=4, min_extent=256)
+        assert g.dense_csc is not None
+    ld = (F + 15) // 16 * 16
+    feat = np.zeros((n, ld), np.int8)
+    feat[:, :F] = rng.integers(-127, 128, (n, F))
+    row_scale = rng.random(n).astype(np.float32)
+    bias = rng.standard_normal(F).astype(np.float32)
+    mul = (rng.random(n).astype(np.float32) + 0.5) if use_mul else None
+    fd = dev(feat)[:, :F]
+    out, scale = K.csr_SPMM(g, fd, sc(0.02), row_scale=dev(row_scale), bias=dev(bias), relu=True, want_scale=True,
+                            scale_mul=None if mul is None else dev(mul))
+    o = orc.graph_formats(s, d, n)
+    want = orc.spmm_csr_copy_u_ex(o["adj_csc"][0], o["adj_csc"][1], np.ascontiguousarray(feat[:, :F]), np.float32(0.02),
+                                  row_scale=row_scale, bias=bias, act=1)
+    assert np.array_equal(host(out), want)
+    want_scale, _ = orc.absmax_ex(want, row_mul=mul)
+    assert host(scale)[0] == want_scale and want_scale > 0
+
+
+def test_gcn_scale_hand_off_changes_nothing(K, monkeypatch):
+    """A 2-layer GCN step on a dense graph with the scales handed from the aggregations' epilogues to the next
+    quantizers (forward and backward) gives the same logits and gradients, bit for bit, as with the separate
+    absmax passes."""
+    from tango_amd import SPMM, config
+    from tango_amd.gcn import GCN
+    from tango_amd.graph import Graph
+    from tango_amd.loss import cross_entropy
+    from tango_amd.util import graph_preprocess
+    rng = np.random.default_rng(3)
+    n = 2048
+    s, d = heavy_graph(rng, n, 150_000)
+    g = graph_preprocess(Graph(dev(s), dev(d), n))
+    X = torch.randn(n, 96, device="cuda")
+    labels = torch.randint(0, 7, (n,), device="cuda")
+    saved = config.grad_round_mode
+    config.grad_round_mode = "rne"
+    monkeypatch.setattr(config, "scale_from_aggregation", True)
+    calls = []
+    for name in ("get_scale", "absmax_ex"):
+        raw = getattr(K.cuda_kernels, name)
+        monkeypatch.setattr(K.cuda_kernels, name, staticmethod(
+            lambda *a, _raw=raw, _n=name, **kw: (calls.append((_n, tuple(a[0].shape))), _raw(*a, **kw))[1]))
+    try:
+        res, passes = [], []
+        for fused in (True, False):
+            if not fused:
+                monkeypatch.setattr(SPMM, "_dense_enough", lambda g, reverse=False: False)
+            torch.manual_seed(0)
+            model = GCN(g, 96, 32, 7, 1, torch.relu, 0.0).cuda()
+            del calls[:]
+            logits = model(X)
+            cross_entropy(logits, labels).backward()
+            passes.append([c for c in calls if c[1][0] == n])  # scans of node tensors (not of the weights)
+            res.append([logits.detach().clone()] + [p.grad.clone() for p in model.parameters()])
+        for a, b in zip(*res):
+            assert torch.equal(a, b)
+        # gone with the hand-off: the scan of layer 2's input and of the two reverse aggregations' outputs
+        assert len(passes[1]) - len(passes[0]) == 3, (passes[0], passes[1])
+    finally:
+        config.grad_round_mode = saved
