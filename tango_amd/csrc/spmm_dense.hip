@@ -135,9 +135,11 @@ __global__ __launch_bounds__(256, 2) void dense_block_kernel(const DenseParams p
         }
         for (int k = 0; k < nu; ++k) {
             const int8_t* buf = ring + (k & 1) * CHUNK;
-            const bool more = k + 1 < nu;  // uniform
-            if (more) {
-                const int64_t un = u0 + k + 1;
+            // the next unit's chunk and mask words (the last unit asks for itself again: every load is
+            // unconditional, so that the compiler waits for them where they are used, after the products,
+            // and not at a join in front of them)
+            const int64_t un = u0 + (k + 1 < nu ? k + 1 : k);
+            {
                 const u32x4* x = xsrc + un * (CHUNK / 16);
 #pragma unroll
                 for (int i = 0; i < PASSES; ++i) xnext[i] = x[i * 256];
@@ -146,6 +148,7 @@ __global__ __launch_bounds__(256, 2) void dense_block_kernel(const DenseParams p
 #pragma unroll
                     for (int hf = 0; hf < 2; ++hf) mnext[g][hf] = mrow[un * 512 + g * 128 + hf * 64];
             }
+            __builtin_amdgcn_sched_barrier(0);  // the loads stay in front of the products, their use behind them
 #pragma unroll
             for (int s = 0; s < 8; ++s) {
                 i32x4 mf[RW];
@@ -166,7 +169,8 @@ __global__ __launch_bounds__(256, 2) void dense_block_kernel(const DenseParams p
                         acc[c][h] = __builtin_amdgcn_mfma_i32_32x32x32_i8(mf[h], ff, acc[c][h], 0, 0, 0);
                 }
             }
-            if (more) {
+            __builtin_amdgcn_sched_barrier(0);
+            {
                 int8_t* nbuf = ring + ((k + 1) & 1) * CHUNK;
 #pragma unroll
                 for (int i = 0; i < PASSES; ++i) *reinterpret_cast<u32x4*>(nbuf + (i * 256 + t) * 16) = xnext[i];
