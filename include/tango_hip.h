@@ -47,6 +47,12 @@ const char* tango_status_string(int status);
 /* ABI version; bumped when a signature changes. */
 int tango_abi_version(void);
 
+/* Measurement probe (no counterpart in the reference): `blocks` workgroups of four wavefronts each run
+   `iters` rounds of eight independent chains of one int8 matrix instruction out of registers; shape 0:
+   16x16x64 (2 * 16 * 16 * 64 operations each), shape 1: 32x32x32 (2 * 32 * 32 * 32).  The rate of such a launch
+   is what the matrix cores of the device sustain; sink: one int of device memory, never written in practice. */
+int tango_probe_mfma_i8(int shape, int iters, int blocks, int* sink, tango_stream_t stream);
+
 /* ------------------------------------------------------------ quantization */
 
 /* get_scale (cuda/src/cuda.cpp:24-25 -> get_scale_impl, quantization.cu:79-93):
@@ -329,6 +335,10 @@ int tango_spmm_dense_mask_build(const int64_t* indptr, const void* indices, int 
    TANGO_ERR_UNSUPPORTED (callers then use tango_spmm_csr_copy_u_ex on the whole CSR).
    workspace: tango_spmm_dense_workspace(plan, F) bytes, 256-byte aligned. */
 size_t tango_spmm_dense_workspace(const tango_spmm_dense_plan* plan, int64_t F);
+/* The first part of tango_spmm_csr_copy_u_dense alone (staging, zeroing, the matrix product of the bit blocks into
+   the workspace), for measurements: its time subtracted from the whole call's is the gather kernel's. */
+int tango_spmm_dense_partial(const tango_spmm_dense_plan* plan, const int8_t* feat, int64_t ldf, int64_t F,
+                             void* workspace, size_t workspace_bytes, tango_stream_t stream);
 int tango_spmm_csr_copy_u_dense(float* out, const tango_spmm_dense_plan* plan, const int8_t* feat,
                                 int64_t ldf, const float* scale, const float* row_scale,
                                 const float* bias, int relu, uint16_t* sign_bits, int64_t F,

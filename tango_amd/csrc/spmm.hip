@@ -1384,6 +1384,18 @@ size_t tango_spmm_dense_workspace(const tango_spmm_dense_plan* plan, int64_t F) 
            sizeof(float) * amax_floats(plan->rows, F);
 }
 
+int tango_spmm_dense_partial(const tango_spmm_dense_plan* plan, const int8_t* feat, int64_t ldf, int64_t F,
+                             void* workspace, size_t workspace_bytes, tango_stream_t stream) {
+    if (!plan || F <= 0 || ldf < F || !feat) return TANGO_ERR_INVALID_ARG;
+    if (plan->row_blocks <= 0) return TANGO_OK;
+    const size_t need = tango_spmm_dense_workspace(plan, F);
+    if (!need) return TANGO_ERR_UNSUPPORTED;
+    if (!workspace || workspace_bytes < need) return TANGO_ERR_WORKSPACE;
+    const int* part;
+    int ld;
+    return launch_dense_block(*plan, feat, ldf, F, workspace, workspace_bytes, &part, &ld, as_stream(stream));
+}
+
 int tango_spmm_csr_copy_u_dense(float* out, const tango_spmm_dense_plan* plan, const int8_t* feat,
                                 int64_t ldf, const float* scale, const float* row_scale,
                                 const float* bias, int relu, uint16_t* sign_bits, int64_t F,

@@ -239,6 +239,41 @@ __global__ __launch_bounds__(256) void dense_mask_build_kernel(const int64_t* in
     if (lane == 0) kept[row] = cnt;
 }
 
+// Rate probe of the int8 matrix instructions: every wavefront runs `iters` rounds of eight independent
+// accumulator chains out of registers (no memory traffic); blockDim.x = 256.
+template <int SHAPE>
+__global__ __launch_bounds__(256) void mfma_probe_kernel(int iters, int* sink) {
+    const int lane = lane_id();
+    i32x4 a{lane, lane + 1, lane + 2, lane + 3}, b{3 * lane, 5 * lane, 7 * lane, 11 * lane};
+    int total = 0;
+    if (SHAPE == 0) {
+        i32x4 acc[8];
+#pragma unroll
+        for (int c = 0; c < 8; ++c) acc[c] = i32x4{c, 0, 0, 0};
+        for (int it = 0; it < iters; ++it) {
+#pragma unroll
+            for (int c = 0; c < 8; ++c) acc[c] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, b, acc[c], 0, 0, 0);
+        }
+#pragma unroll
+        for (int c = 0; c < 8; ++c) total += acc[c][0] + acc[c][1] + acc[c][2] + acc[c][3];
+    } else {
+        i32x16v acc[8];
+#pragma unroll
+        for (int c = 0; c < 8; ++c)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) acc[c][v] = c + v;
+        for (int it = 0; it < iters; ++it) {
+#pragma unroll
+            for (int c = 0; c < 8; ++c) acc[c] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, b, acc[c], 0, 0, 0);
+        }
+#pragma unroll
+        for (int c = 0; c < 8; ++c)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) total += acc[c][v];
+    }
+    if (total == 0x7fffffff) sink[0] = total;  // keeps the chains alive; practically never taken
+}
+
 static size_t align256(size_t v) { return (v + 255) & ~static_cast<size_t>(255); }
 
 size_t dense_workspace_bytes(const tango_spmm_dense_plan& plan, int64_t F) {
@@ -295,6 +330,13 @@ int launch_dense_block(const tango_spmm_dense_plan& plan, const int8_t* feat, in
 using namespace tango;
 
 extern "C" {
+
+int tango_probe_mfma_i8(int shape, int iters, int blocks, int* sink, tango_stream_t stream) {
+    if ((shape != 0 && shape != 1) || iters < 0 || blocks <= 0 || !sink) return TANGO_ERR_INVALID_ARG;
+    if (shape == 0) hipLaunchKernelGGL(mfma_probe_kernel<0>, dim3(blocks), dim3(256), 0, as_stream(stream), iters, sink);
+    else hipLaunchKernelGGL(mfma_probe_kernel<1>, dim3(blocks), dim3(256), 0, as_stream(stream), iters, sink);
+    return launch_status();
+}
 
 int tango_spmm_dense_mask_build(const int64_t* indptr, const void* indices, int idx_bits, int64_t rows,
                                 const int32_t* row_rank, const int32_t* col_rank,
