@@ -430,3 +430,56 @@ def test_gcn_config1_layer_matches_oracle(orc):
     assert np.array_equal(host(Y), Yo) and sY.item() == sYo
     ip, ix, _ = g.adj_csc
     assert np.array_equal(host(out), orc.spmm_csr_copy_u(host(ip), host(ix), orc.quantize(Yo, sYo), sYo))
+
+
+def test_gat_backward_primitives_full(K, orc):
+    """The backward halves of the GAT block at the benchmark size (169,343 nodes / 1,335,586 edges, 8 heads x 16):
+    edge softmax backward, the attention logits' backward and both gradients of the attention-weighted
+    aggregation, against the oracle (closed forms in float64 for the logits, which have no oracle function)."""
+    from tango_amd import config
+    from tango_amd.SPMM import spmm_u_mul_e
+    from tango_amd.graph import chung_lu
+    from tango_amd.util import graph_preprocess
+    g = graph_preprocess(chung_lu(169343, 1166243, 2.2, seed=4, device="cuda"))
+    n, E, H, D = g.num_nodes(), g.num_edges(), 8, 16
+    rng = np.random.default_rng(40)
+    ip, ix, eid = g.adj_csc
+    # edge softmax backward (LeakyReLU 0.2 folded in)
+    e = rng.standard_normal((E, H)).astype(np.float32)
+    da = rng.standard_normal((E, H)).astype(np.float32)
+    e_d, da_d = dev(e).view(E, H, 1), dev(da).view(E, H, 1)
+    a = K.cuda_kernels.edge_softmax_forward(e_d, ip, eid, 0.2)
+    de = K.cuda_kernels.edge_softmax_backward(a, da_d, e_d, ip, eid, 0.2)
+    want_de = orc.edge_softmax_bwd(host(a).reshape(E, H), da, e, host(ip), host(eid), 0.2)
+    assert np.allclose(host(de).reshape(E, H), want_de, rtol=1e-5, atol=1e-6)
+    # attention logits backward: dfeat = del * attn_l + der * attn_r, dattn = sum over nodes of d * feat
+    feat = rng.standard_normal((n, H, D)).astype(np.float32)
+    al, ar = rng.standard_normal((H, D)).astype(np.float32), rng.standard_normal((H, D)).astype(np.float32)
+    dl, dr = rng.standard_normal((n, H)).astype(np.float32), rng.standard_normal((n, H)).astype(np.float32)
+    dfeat, dal, dar = K.cuda_kernels.attn_scores_backward(dev(dl), dev(dr), dev(feat), dev(al), dev(ar))
+    f64 = feat.astype(np.float64)
+    want_dfeat = dl[:, :, None].astype(np.float64) * al + dr[:, :, None].astype(np.float64) * ar
+    np.testing.assert_allclose(host(dfeat), want_dfeat, rtol=1e-5, atol=1e-5)
+    np.testing.assert_allclose(host(dal), (dl[:, :, None] * f64).sum(0), rtol=1e-4, atol=1e-2)  # sums of 169,343 terms
+    np.testing.assert_allclose(host(dar), (dr[:, :, None] * f64).sum(0), rtol=1e-4, atol=1e-2)
+    # u_mul_e backward: dN = reverse aggregation of the quantized dZ with the edge values, dE = SDDMM dot
+    saved = config.grad_round_mode
+    config.grad_round_mode = "rne"
+    try:
+        N = torch.randn(n, H, D, device="cuda", requires_grad=True)
+        Ev = a.detach().clone().requires_grad_(True)
+        out = spmm_u_mul_e.apply(g, N, Ev)
+        dZ = torch.randn(n, H, D, device="cuda")
+        out.backward(dZ)
+    finally:
+        config.grad_round_mode = saved
+    Nn, En, dZn = host(N.detach()), host(Ev.detach()), host(dZ)
+    sN, sE, sdZ = orc.absmax_scale(Nn), orc.absmax_scale(En), orc.absmax_scale(dZn)
+    Nq, Eq, dZq = orc.quantize(Nn, sN), orc.quantize(En, sE), orc.quantize(dZn, sdZ)
+    want_out = orc.spmm_csr_u_mul_e_ex(host(ip), host(ix), host(eid), Nq, Eq, sN, scale2=sE, edge_major=True)
+    assert np.array_equal(host(out.detach()), want_out)
+    rp, rx, reid = (host(t) for t in g.adj_csr)
+    want_dN = orc.spmm_csr_u_mul_e_ex(rp, rx, reid, dZq, Eq, sdZ, scale2=sE, edge_major=True)
+    assert np.array_equal(host(N.grad), want_dN)
+    want_dE, _ = orc.sddmm_dot(host(g.coo[0]), host(g.coo[1]), Nq, dZq, sN, sdZ)
+    assert np.array_equal(host(Ev.grad).reshape(E, H), want_dE)
