@@ -13,8 +13,13 @@ from torch.autograd.function import Function, once_differentiable
 from .kernels import _L, _ptr, _stream, _workspace, check, refuse_capture
 
 
-def _fusable(x, cols):
-    return x.is_cuda and x.dim() == 2 and x.dtype == torch.float32 and 1 <= cols <= 2048 and x.size(0) > 1
+def _fusable(x, cols, weight, bias):
+    """The kernels read x, weight and bias as contiguous fp32 on x's device and merge per-workgroup row counts held
+    as floats (exact below 2^24 rows); anything else takes torch's batch normalisation."""
+    def ok(t):
+        return t is not None and t.dtype == torch.float32 and t.device == x.device and t.is_contiguous()
+    return (x.is_cuda and x.dim() == 2 and x.dtype == torch.float32 and 1 <= cols <= 2048
+            and 1 < x.size(0) < (1 << 24) and ok(weight) and ok(bias))
 
 
 class _BatchNormAct(Function):
@@ -61,7 +66,8 @@ class BatchNorm1dAct(nn.BatchNorm1d):
 
     def forward(self, x):
         relu = self.activation in (torch.relu, F.relu) or isinstance(self.activation, nn.ReLU)
-        if not (self.training and self.affine and (relu or self.activation is None) and _fusable(x, self.num_features)):
+        if not (self.training and self.affine and (relu or self.activation is None)
+                and _fusable(x, self.num_features, self.weight, self.bias)):
             y = super().forward(x)
             return y if self.activation is None else self.activation(y)
         stats_out = []

@@ -67,9 +67,13 @@ def reset_offsets():
 
 # Calls since a device's counter last moved.  Outside a stream capture the position of a call is
 # (device counter) + (pending calls) * WINDOW with the second term passed by value, and the counter moves once per
-# BATCH calls: one one-thread launch per BATCH quantize launches instead of one each.  Under capture every call
-# moves the counter itself (first by whatever is pending), so that a replayed graph draws fresh windows.
+# BATCH calls: one one-thread launch per BATCH quantize launches instead of one each.  A call recorded into a HIP
+# graph draws from a part of the stream of its own (CAPTURE_BASE set in its offset) at the device counter's value
+# when the graph runs, and moves the counter by one window itself, so that every replay draws fresh windows; the
+# host-side count of pending eager calls is left alone (a capture only records kernels: the counter does not move
+# at capture time, and eager calls made afterwards must not start again at the counter's own value).
 BATCH = 64
+CAPTURE_BASE = 1 << 62
 _pending = {}
 
 
@@ -77,8 +81,10 @@ def stochastic_args(device):
     """Keyword arguments of a stochastically rounding quantize call."""
     import torch
     c = device_offset(device)
+    if torch.cuda.is_current_stream_capturing():
+        return {"seed": seed, "offset": (CAPTURE_BASE, c), "advance": WINDOW}
     k = _pending.get(c, 0)
-    if torch.cuda.is_current_stream_capturing() or k + 1 >= BATCH:
+    if k + 1 >= BATCH:
         _pending[c] = 0
         return {"seed": seed, "offset": (k * WINDOW, c), "advance": (k + 1) * WINDOW}
     _pending[c] = k + 1

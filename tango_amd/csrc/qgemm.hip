@@ -292,7 +292,9 @@ __global__ __launch_bounds__(64 * WAVES) void gemm_nts_kernel(const NtParams p, 
     // columns of this block, as a 32-bit count: the bounds tests of the epilogue are 32-bit compares
     const int ncols = static_cast<int>(p.N - n0 < 16 * TT ? p.N - n0 : 16 * TT);
     // columns that may be written: a row's padding up to its pitch takes the zeros of the zero-filled rows of B
-    const int wcols = EPI == 0 ? static_cast<int>(p.ldc - n0 < 16 * TT ? p.ldc - n0 : 16 * TT) : ncols;
+    // (never past the next multiple of 16 columns: what lies beyond may belong to the caller)
+    const int64_t wlim = ((p.N + 15) & ~static_cast<int64_t>(15)) < p.ldc ? ((p.N + 15) & ~static_cast<int64_t>(15)) : p.ldc;
+    const int wcols = EPI == 0 ? static_cast<int>(wlim - n0 < 16 * TT ? wlim - n0 : 16 * TT) : ncols;
     for (; t < ntiles; t += stride) {
         load_tile(nxt, rsc_nxt, t + stride);
         const int64_t row = static_cast<int64_t>(t) * 16 + r16;

@@ -9,7 +9,7 @@ import torch.nn.functional as F
 
 from torch.autograd.function import Function, once_differentiable
 
-from .QLinear import QLinear, Qlinear_func_reduce, shared_input_linears
+from .QLinear import QLinear, Qlinear_func, Qlinear_func_reduce, shared_input_linears
 from .batchnorm import BatchNorm1dAct
 from .kernels import cuda_kernels, refuse_capture
 from .SDDMM import sddmm_u_add_v, sddmm_u_dot_v
@@ -238,9 +238,9 @@ class ArxivGATConv(nn.Module):
         h = self.feat_drop(feat).contiguous()
         res = None
         if self._use_symmetric_norm:  # :158-163; the product is a new tensor, so the epilogue's scale does not apply
-            self.fc.isReduce = False
-            feat_src = self.fc(h).view(n, self._num_heads, self._out_feats)
-            self.fc.isReduce = True
+            # the plain (no output scale) functional form of self.fc: no state of the module is touched
+            feat_src = Qlinear_func.apply(h.reshape(-1, h.size(-1)), self.fc.weight, self.fc.bias)
+            feat_src = feat_src.view(n, self._num_heads, self._out_feats)
             s_feat = None
             feat_src = feat_src * graph.out_degrees().float().clamp(min=1).pow(-0.5).view(n, 1, 1)
         elif self.res_fc is not None and h.dim() == 2:
@@ -325,7 +325,11 @@ class HeteroHGTLayer(nn.Module):
         for m in type_sizes:
             self.bounds.append(self.bounds[-1] + m)
         self.rels = list(relation_graphs)
-        nt, nr = len(type_sizes), len(self.rels)
+        # per-relation layers are indexed by the relation's id, not by its place in the list, so that the parameter
+        # layout does not depend on which relations happen to have edges in this graph
+        self.rel_ids = [getattr(gr, "rel_id", i) for i, gr in enumerate(self.rels)]
+        nt = len(type_sizes)
+        nr = max([getattr(gr, "num_relations", 0) for gr in self.rels] + [max(self.rel_ids, default=-1) + 1])
         mk = lambda i, o, k: nn.ModuleList(QLinear(i, o) for _ in range(k))
         self.k_linear, self.q_linear, self.v_linear = mk(in_dim, out_dim, nt), mk(in_dim, out_dim, nt), mk(in_dim, out_dim, nt)
         self.a_linear = mk(out_dim, out_dim, nt)
@@ -346,7 +350,7 @@ class HeteroHGTLayer(nn.Module):
             k.append(kt), v.append(vt), q.append(qt)
         # every relation runs on its own bipartite graph(s), each endpoint numbered inside its node type: no
         # tensor here has rows for nodes the relation does not touch
-        units = [(r, part) for r, gr in enumerate(self.rels) for part in gr.parts]
+        units = [(r, part) for r, gr in zip(self.rel_ids, self.rels) for part in gr.parts]
         # relation-specific keys and messages; the relations that start at one node type share that type's
         # k (v) quantized once
         kr, vr = {}, {}
@@ -432,6 +436,7 @@ def relation_graphs(g, edge_type, relations, type_sizes):
         gr.edge_range = (lo, hi)
         nxt = hi
         gr.src_type = relations[r][0] if r < len(relations) else None  # self loops start at every type
+        gr.rel_id, gr.num_relations = r, len(relations) + 1  # what the layer keys its per-relation weights by
         ts, td = torch.bucketize(rs, edges_of, right=True), torch.bucketize(rd, edges_of, right=True)
         pair = ts * len(type_sizes) + td
         gr.parts = []

@@ -941,7 +941,10 @@ def mySDDMM_quantize_on_load(g, op, U, V, scaleU, scaleV, round_mode=ROUND_RNE):
 
 def QGEMM_backward(dY, X, W, scaledY, scaleX, scaleW, X_need=True, W_need=True, x_row_scale=None, dX_acc=None):
     """cuda/kernels.py:97-111.  ``dX_acc``: a gradient of X from another consumer; the input gradient is
-    added to it in place (and it is returned) instead of going to a new tensor."""
+    added to it in place (and it is returned) instead of going to a new tensor.
+    When K is not a multiple of 32 (and above 32) the returned dX is the [M, K] view of a buffer whose rows are
+    padded to 32 floats: not contiguous, and as a leaf's ``.grad`` it keeps the padded allocation alive; callers
+    that need dense storage call ``.contiguous()`` on it (one [M, K] copy)."""
     assert scaledY.is_cuda, "scaledY must be on GPU"
     assert dY.is_cuda, "dY must be on GPU"
     dX, dW = None, None

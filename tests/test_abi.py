@@ -144,3 +144,39 @@ def test_bench_refuses_more_than_one_gpu():
     root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
     res = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--gpus", "2"], capture_output=True, text=True)
     assert res.returncode != 0 and "one GPU" in (res.stderr + res.stdout)
+
+
+def test_stochastic_windows_are_never_handed_out_twice(monkeypatch):
+    """Eager stochastic quantize calls interleaved with the capture and replays of a graph: replaying the
+    (host offset, advance) pairs against a stand-in for the device counter, no window of the random stream is used
+    twice, and captured calls draw from a part of the stream of their own.  Host only: the capture state is stubbed."""
+    import torch
+    from tango_amd import config
+    capturing = [False]
+    monkeypatch.setattr(torch.cuda, "is_current_stream_capturing", lambda: capturing[0])
+    key = object()
+    monkeypatch.setattr(config, "device_offset", lambda device: key)
+    monkeypatch.setattr(config, "_pending", {})
+    counter = [0]
+    used = []
+
+    def run(args):  # what the kernels do: draw at counter + offset, then the one-thread kernel moves the counter
+        used.append(counter[0] + args["offset"][0])
+        counter[0] += args["advance"]
+
+    def eager(k):
+        for _ in range(k):
+            run(config.stochastic_args(None))
+
+    eager(5)
+    capturing[0] = True
+    graph = [config.stochastic_args(None) for _ in range(3)]  # recorded, not run: the counter stays put
+    capturing[0] = False
+    eager(4)                      # after the capture, before any replay
+    for _ in range(2):
+        for args in graph:        # a replay
+            run(args)
+        eager(70)                 # crosses a batch boundary of the eager calls
+    assert len(set(used)) == len(used)
+    assert all(a["offset"][0] == config.CAPTURE_BASE and a["advance"] == config.WINDOW for a in graph)
+    assert all(u % config.WINDOW == 0 for u in used)
