@@ -443,8 +443,12 @@ int tango_edge_softmax_fwd(float* a, const float* e, const int64_t* indptr,
    per GPU, held until the process ends) and no memory is allocated or freed by the call.
    Inputs with tango_edge_softmax_workspace(num_edges, H) > TANGO_EDGE_SOFTMAX_STATIC_BYTES are
    rejected with TANGO_ERR_STATIC_LIMIT before anything is launched (at H = 8 a span of 128 slots
-   takes 160 bytes: the limit is about 3.3 million edges).  All calls on one GPU share the array: calls that overlap on one GPU
-   (different streams or threads) race; calls on one stream are ordered and safe. */
+   takes 160 bytes: the limit is about 3.3 million edges).  All calls on one GPU share the array.  Calls on
+   one stream are ordered by the stream; a call on another stream than the previous call's first waits
+   (hipStreamWaitEvent on an event created once per GPU at the first call) for the previous call's kernels, so eager
+   calls from several streams or threads are serialised on the GPU rather than racing.  Under stream capture no event
+   is used: graphs that contain this call and replay at the same time on one GPU still race, which is the
+   caller's to order. */
 #define TANGO_EDGE_SOFTMAX_STATIC_BYTES (4u << 20)
 int tango_edge_softmax_fwd_static(float* a, const float* e, const int64_t* indptr,
                                   const int64_t* edge_ids, int64_t rows, int64_t num_edges, int64_t H,

@@ -23,22 +23,35 @@ static __device__ __align__(256) unsigned char scratch[TANGO_EDGE_SOFTMAX_STATIC
 
 constexpr int kMaxDevices = 64;
 static std::mutex scratch_mutex;
-static void* scratch_address[kMaxDevices];  // device address of `scratch` on each device, once looked up
+// Per device: the device address of `scratch` (looked up once), and what orders calls that arrive on different
+// streams: the stream of the last call and an event recorded behind its kernels.  A call on another stream waits
+// for that event first, so that it does not overwrite records the earlier call's kernels still read.
+struct StaticScratch {
+    void* address;
+    hipEvent_t done;
+    hipStream_t last_stream;
+    bool recorded;
+};
+static StaticScratch static_scratch[kMaxDevices];
 
-// Device address of `scratch` on the current device (looked up once per device), or nullptr.
-static void* scratch_of_current_device() {
+// Set-up of the current device's entry (address of `scratch`, the event), once per device; nullptr on failure.
+// Call with scratch_mutex held.
+static StaticScratch* scratch_of_current_device() {
     int dev = -1;
     if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return nullptr;
-    std::lock_guard<std::mutex> lock(scratch_mutex);
-    if (!scratch_address[dev]) {
+    StaticScratch& sc = static_scratch[dev];
+    if (!sc.address) {
         void* p = nullptr;
-        if (hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)) != hipSuccess) {
+        hipEvent_t ev = nullptr;
+        if (hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)) != hipSuccess ||
+            hipEventCreateWithFlags(&ev, hipEventDisableTiming) != hipSuccess) {
             (void)hipGetLastError();
             return nullptr;
         }
-        scratch_address[dev] = p;
+        sc.done = ev;
+        sc.address = p;
     }
-    return scratch_address[dev];
+    return &sc;
 }
 
 __device__ __forceinline__ float leaky(float v, float slope) { return v > 0.0f ? v : v * slope; }
@@ -690,12 +703,35 @@ int tango_edge_softmax_fwd_static(float* a, const float* e, const int64_t* indpt
     if (!a || !e) return TANGO_ERR_INVALID_ARG;
     if (ceil_div(nnz, 4 * 128) > INT32_MAX || ceil_div(H, 8) > 65535) return TANGO_ERR_UNSUPPORTED;
     if (span_workspace_bytes(nnz, H) > TANGO_EDGE_SOFTMAX_STATIC_BYTES) return TANGO_ERR_STATIC_LIMIT;
-    void* ws = scratch_of_current_device();
-    if (!ws) return TANGO_ERR_LAUNCH;
+    hipStream_t s = as_stream(stream);
+    std::lock_guard<std::mutex> lock(scratch_mutex);
+    StaticScratch* sc = scratch_of_current_device();
+    if (!sc) return TANGO_ERR_LAUNCH;
+    // Calls on one stream are ordered by the stream.  A call on another stream than the last one first waits for
+    // the last call's kernels.  Not under stream capture: there the graph's own dependencies order the nodes, and
+    // an event recorded outside the capture must not be waited for inside it.
+    hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(s, &capture) != hipSuccess) {
+        (void)hipGetLastError();
+        capture = hipStreamCaptureStatusActive;  // the legacy stream while another stream captures: no event calls
+    }
+    const bool eager = capture == hipStreamCaptureStatusNone;
+    if (eager && sc->recorded && sc->last_stream != s && hipStreamWaitEvent(s, sc->done, 0) != hipSuccess) {
+        (void)hipGetLastError();
+        return TANGO_ERR_LAUNCH;
+    }
     // The span kernels write every record of the scratch they later read, so nothing has to be cleared.
-    launch_spans<true>(a, nullptr, nullptr, e, indptr, edge_ids, rows, nnz, static_cast<int>(H), slope, ws,
-                       as_stream(stream));
-    return launch_status();
+    launch_spans<true>(a, nullptr, nullptr, e, indptr, edge_ids, rows, nnz, static_cast<int>(H), slope, sc->address, s);
+    const int rc = launch_status();
+    if (eager && rc == TANGO_OK) {
+        if (hipEventRecord(sc->done, s) != hipSuccess) {
+            (void)hipGetLastError();
+            return TANGO_ERR_LAUNCH;
+        }
+        sc->last_stream = s;
+        sc->recorded = true;
+    }
+    return rc;
 }
 
 int tango_edge_softmax_fwd_ex(float* a, float* scale_a, uint8_t* sign_out, const float* e, const float* el,

@@ -92,23 +92,37 @@ __global__ __launch_bounds__(256) void absmax_rowmul_dense_kernel(const float* _
     int64_t row = (4 * tid) / cols, col = (4 * tid) % cols;
     const int64_t srow = (4 * nthr) / cols, scol = (4 * nthr) % cols;
     float m = 0.0f;
-    auto take = [&](const f32x4 v) {
-        const float r0 = row_mul[row];
-        const float r1 = (col + 2 >= cols) ? row_mul[row + 1] : r0;
-        m = fmaxf(m, fmaxf(fmaxf(fabsf(v.x * r0), fabsf(v.y * r0)), fmaxf(fabsf(v.z * r1), fabsf(v.w * r1))));
+    // the two multipliers of a vector, then the step to the lane's next vector: index arithmetic and selects only,
+    // so that the multiplier loads of a whole batch are in flight together with its vector loads
+    auto multipliers = [&](float& r0, float& r1) {
+        r0 = row_mul[row];
+        r1 = row_mul[row + (col + 2 >= cols ? 1 : 0)];  // a vector whose second half is in the next row never ends the matrix
         row += srow;
         col += scol;
-        if (col >= cols) { col -= cols; ++row; }
+        const bool wrap = col >= cols;
+        col -= wrap ? cols : 0;
+        row += wrap ? 1 : 0;
+    };
+    auto take = [&](const f32x4 v, float r0, float r1) {
+        m = fmaxf(m, fmaxf(fmaxf(fabsf(v.x * r0), fabsf(v.y * r0)), fmaxf(fabsf(v.z * r1), fabsf(v.w * r1))));
     };
     int64_t i = tid;
     for (; i + 7 * nthr < n4; i += 8 * nthr) {  // eight 16-byte loads in flight per lane
         f32x4 v[8];
+        float r0[8], r1[8];
 #pragma unroll
         for (int u = 0; u < 8; ++u) v[u] = __builtin_nontemporal_load(x4 + i + u * nthr);
 #pragma unroll
-        for (int u = 0; u < 8; ++u) take(v[u]);
+        for (int u = 0; u < 8; ++u) multipliers(r0[u], r1[u]);
+#pragma unroll
+        for (int u = 0; u < 8; ++u) take(v[u], r0[u], r1[u]);
     }
-    for (; i < n4; i += nthr) take(__builtin_nontemporal_load(x4 + i));
+    for (; i < n4; i += nthr) {
+        const f32x4 v = __builtin_nontemporal_load(x4 + i);
+        float r0, r1;
+        multipliers(r0, r1);
+        take(v, r0, r1);
+    }
     const int64_t t = (n4 << 2) + tid;  // at most two elements remain, in the last row
     if (t < n) m = fmaxf(m, fabsf(x[t] * row_mul[t / cols]));
     block_absmax_to_global(m / 127.0f, out);

@@ -1,6 +1,7 @@
 """Edge softmax over the in-edges of each destination node, optionally with the
 LeakyReLU that precedes it in GAT fused in (evaluation/test_gat.py:144-146;
 the reference calls DGL's fp32 edge_softmax, which is not part of its tree)."""
+import torch
 from torch.autograd.function import Function, once_differentiable
 
 from .kernels import cuda_kernels, refuse_capture
@@ -43,10 +44,23 @@ class _EdgeSoftmax(Function):
         return None, cuda_kernels.edge_softmax_backward(a, da, None if slope == 1.0 else e, indptr, eids, slope), None, None
 
 
-def edge_softmax(g, e, negative_slope=None, want_scale=False):
+def edge_softmax(g, e, negative_slope=None, want_scale=False, eids=None):
     """softmax_dst(e) if ``negative_slope`` is None, else softmax_dst(leaky_relu(e)).  ``want_scale``: returns
-    (a, max(a) / 127), the second found by the kernel that writes a (hand it to spmm_u_mul_e as ``scaleE``)."""
-    return _EdgeSoftmax.apply(g, e, 1.0 if negative_slope is None else float(negative_slope), want_scale)
+    (a, max(a) / 127), the second found by the kernel that writes a (hand it to spmm_u_mul_e as ``scaleE``).
+    ``eids`` (int64 [k], distinct): the softmax runs over these edges only, as DGL's ``edge_softmax(graph, e, eids=eids)``
+    does (evaluation/arxiv_gat.py:186-192, edge dropping); ``e`` then holds the logits of those k edges and so does
+    the result.  The other edges take part with a logit of -FLT_MAX, whose exponential is an exact zero, so a
+    destination's kept edges get the sums of the kept edges alone."""
+    slope = 1.0 if negative_slope is None else float(negative_slope)
+    if eids is None:
+        return _EdgeSoftmax.apply(g, e, slope, want_scale)
+    if want_scale:
+        raise RuntimeError("edge_softmax: want_scale is not available with eids")
+    if e.size(0) != eids.numel():
+        raise RuntimeError("edge_softmax: e must hold one row per entry of eids")
+    full = e.new_full((g.num_edges(),) + tuple(e.shape[1:]), -torch.finfo(e.dtype).max)
+    full = full.index_copy(0, eids, e)
+    return _EdgeSoftmax.apply(g, full, slope, False).index_select(0, eids)
 
 
 class gat_edge_attention(Function):

@@ -201,15 +201,16 @@ class ArxivGATConv(nn.Module):
     """The attention layer of evaluation/arxiv_gat.py:63-218 on a homogeneous graph: no bias (the model adds
     one after its last layer), a quantized residual projection of the layer's input, an optional attention
     term for the destination (``use_attn_dst``) and the optional symmetric degree normalisation.
-    ``edge_drop`` must be 0: dropping edges needs the ``eids=`` form of the edge softmax
-    (arxiv_gat.py:191-194), which this package does not carry."""
+    ``edge_drop`` > 0 (training mode): a random share of the edges takes no part in the softmax and aggregates
+    nothing (arxiv_gat.py:186-194, the ``eids=`` form of the edge softmax); that path runs the unfused ops."""
 
     def __init__(self, in_feats, out_feats, num_heads=1, feat_drop=0.0, attn_drop=0.0, edge_drop=0.0,
                  negative_slope=0.2, use_attn_dst=True, residual=False, activation=None,
                  allow_zero_in_degree=False, use_symmetric_norm=False):
         super().__init__()
-        if edge_drop != 0.0:
-            raise NotImplementedError("ArxivGATConv: edge_drop needs an edge softmax over a subset of the edges")
+        if not 0.0 <= edge_drop < 1.0:
+            raise ValueError("ArxivGATConv: edge_drop must be in [0, 1)")
+        self.edge_drop = edge_drop
         self._num_heads, self._out_feats = num_heads, out_feats
         self._allow_zero_in_degree, self._use_symmetric_norm = allow_zero_in_degree, use_symmetric_norm
         self.fc = QLinear(in_feats, out_feats * num_heads, bias=False)
@@ -252,7 +253,17 @@ class ArxivGATConv(nn.Module):
             feat_src, s_feat = self.fc(h)
             feat_src = feat_src.view(n, self._num_heads, self._out_feats)
         s_a = None
-        if self.attn_r is not None:  # :176-184
+        if self.training and self.edge_drop > 0:  # :186-194
+            if self.attn_r is not None:
+                el, er, s_el, s_er = attn_scores.apply(feat_src, self.attn_l, self.attn_r)
+                e = sddmm_u_add_v.apply(graph, el, er, s_el, s_er)
+            else:
+                e = (feat_src * self.attn_l).sum(-1, keepdim=True)[graph.coo[0]]
+            perm = torch.randperm(graph.num_edges(), device=e.device)
+            eids = perm[int(graph.num_edges() * self.edge_drop):]
+            kept = self.attn_drop(edge_softmax(graph, e[eids], negative_slope=self.negative_slope, eids=eids))
+            a = torch.zeros_like(e).index_copy(0, eids, kept)
+        elif self.attn_r is not None:  # :176-184
             el, er, s_el, s_er = attn_scores.apply(feat_src, self.attn_l, self.attn_r)
             if s_el is not None and fused_attention:
                 a, s_a = gat_edge_attention.apply(graph, el, er, s_el, s_er, self.negative_slope)  # :184, :187, :196
@@ -261,7 +272,7 @@ class ArxivGATConv(nn.Module):
         else:  # copy_u of el (:186)
             e = (feat_src * self.attn_l).sum(-1, keepdim=True)[graph.coo[0]]
             a, s_a = edge_softmax(graph, e, negative_slope=self.negative_slope, want_scale=True)  # :187, :196
-        if self.attn_drop.p > 0 and self.training:
+        if self.attn_drop.p > 0 and self.training and not self.edge_drop > 0:
             a, s_a = self.attn_drop(a), None
         rst = spmm_u_mul_e.apply(graph, feat_src, a, None, s_feat, None, s_a)  # :201
         if self._use_symmetric_norm:  # :203-208

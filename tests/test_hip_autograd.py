@@ -206,6 +206,64 @@ def test_edge_softmax_autograd():
     assert torch.allclose(x.grad, xr.grad, rtol=1e-4, atol=1e-6)
 
 
+def test_edge_softmax_over_a_subset_of_edges():
+    """``eids=``: the softmax of the kept edges alone (DGL's form, evaluation/arxiv_gat.py:186-192), against the
+    plain softmax on a graph built from the kept edges only; some destinations lose every edge."""
+    from tango_amd.edge_softmax import edge_softmax
+    rng = np.random.default_rng(11)
+    n, e, H = 60, 700, 4
+    src, dst = rand_graph(rng, n, e)
+    g = make_graph(src, dst, n)
+    keep = np.sort(rng.permutation(e)[: e // 3])
+    keep = keep[dst[keep] % 5 != 0]  # destinations 0, 5, 10, ... keep nothing
+    sub = make_graph(src[keep], dst[keep], n)
+    xs = rng.standard_normal((keep.size, H, 1)).astype(np.float32)
+    w = dev(rng.standard_normal((keep.size, H, 1)).astype(np.float32))
+    for slope in (None, 0.2):
+        x = dev(xs).requires_grad_(True)
+        a = edge_softmax(g, x, negative_slope=slope, eids=dev(keep))
+        xr = dev(xs).requires_grad_(True)
+        ref = edge_softmax(sub, xr, negative_slope=slope)
+        a.backward(w)
+        ref.backward(w)
+        assert a.shape == ref.shape and torch.isfinite(a).all()
+        assert torch.allclose(a, ref, rtol=1e-5, atol=1e-7)
+        assert torch.allclose(x.grad, xr.grad, rtol=1e-4, atol=1e-6)
+    with pytest.raises(RuntimeError):
+        edge_softmax(g, dev(xs)[:-1], eids=dev(keep))
+
+
+def test_arxiv_gat_layer_with_edge_drop():
+    """Training-mode edge dropping: the layer on the full graph with a share of the edges dropped equals the layer
+    on the graph of the kept edges (same draw of the permutation), to the rounding of the int8 attention values."""
+    from tango_amd.gat import ArxivGATConv
+    rng = np.random.default_rng(12)
+    n, e, H, D = 300, 6000, 2, 16
+    src, dst = rand_graph(rng, n, e)
+    src, dst = np.concatenate([src, np.arange(n)]), np.concatenate([dst, np.arange(n)])
+    g = make_graph(src, dst, n)
+    torch.manual_seed(5)
+    layer = ArxivGATConv(32, D, num_heads=H, edge_drop=0.4, residual=True, allow_zero_in_degree=True).cuda().train()
+    x = dev(rng.standard_normal((n, 32)).astype(np.float32))
+    torch.manual_seed(99)
+    out = layer(g, x)
+    torch.manual_seed(99)
+    perm = torch.randperm(g.num_edges(), device="cuda")
+    kept = perm[int(g.num_edges() * 0.4):].sort().values.cpu().numpy()
+    sub = make_graph(src[kept], dst[kept], n)
+    layer.edge_drop = 0.0
+    ref = layer(sub, x)
+    assert out.shape == ref.shape == (n, H, D)
+    assert rel_err(out.detach(), ref.detach()) < 0.02
+    layer.edge_drop = 0.4
+    out.square().mean().backward()
+    assert all(p.grad is not None and torch.isfinite(p.grad).all() for p in layer.parameters())
+    layer.eval()  # no dropping outside training
+    assert torch.equal(layer(g, x), ArxivGATConv.forward(layer, g, x))
+    with pytest.raises(ValueError):
+        ArxivGATConv(32, D, edge_drop=1.0)
+
+
 def test_stochastic_gradient_rounding_switch():
     from tango_amd import config
     from tango_amd.QLinear import QLinear

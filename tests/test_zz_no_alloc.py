@@ -54,3 +54,27 @@ def test_static_scratch_matches_workspace_form_twice(orc):
         assert np.array_equal(got, want)
         ref = orc.edge_softmax_fwd(e, indptr, eids, slope)
         np.testing.assert_allclose(got, ref, rtol=1e-5, atol=1e-6)
+
+
+def test_static_scratch_calls_on_two_streams_are_ordered(orc):
+    """Two calls that share the device array, issued back to back on different streams without any host-side
+    ordering: the second waits for the first on the GPU, so both results are right."""
+    from tango_amd import _lib
+    from tango_amd._lib import check
+    L = _lib.lib()
+    rng = np.random.default_rng(72)
+    cases = []
+    for n, E, H in ((5000, 300000, 8), (4000, 250000, 4)):
+        src, dst = powerlaw_graph(rng, n, E)
+        indptr, eids = _dst_major(src, dst, n)
+        e = rng.standard_normal((E, H)).astype(np.float32) * 3
+        cases.append((n, E, H, e, indptr, eids, dev(e), dev(indptr), dev(eids), torch.full((E, H), float("nan"), device="cuda")))
+    torch.cuda.synchronize()
+    streams = [torch.cuda.Stream(), torch.cuda.Stream()]
+    for rep in range(3):
+        for (n, E, H, _, _, _, e_d, ip_d, id_d, out), st in zip(cases, streams):
+            check(L.tango_edge_softmax_fwd_static(out.data_ptr(), e_d.data_ptr(), ip_d.data_ptr(), id_d.data_ptr(), n, E, H,
+                                                  0.2, st.cuda_stream), "edge_softmax_fwd_static")
+    torch.cuda.synchronize()
+    for n, E, H, e, indptr, eids, _, _, _, out in cases:
+        np.testing.assert_allclose(host(out), orc.edge_softmax_fwd(e, indptr, eids, 0.2), rtol=1e-5, atol=1e-6)
