@@ -138,10 +138,19 @@ def mfma_probe(torch, iters=4000):
     cus = torch.cuda.get_device_properties(0).multi_processor_count
     blocks = cus * 8
     out = {}
-    for shape, name, ops in ((0, "16x16x64", 2 * 16 * 16 * 64), (1, "32x32x32", 2 * 32 * 32 * 32)):
-        ms = time_op(lambda: _lib.check(L.tango_probe_mfma_i8(shape, iters, blocks, sink.data_ptr(), st), "probe"),
+    shapes = ((0, "16x16x64", 2 * 16 * 16 * 64), (1, "32x32x32", 2 * 32 * 32 * 32),
+              # the same instruction with its first operand expanded from bits in front of every 1, 2, 4 of them
+              (2, "32x32x32_8valu", 2 * 32 * 32 * 32), (3, "32x32x32_4valu", 2 * 32 * 32 * 32),
+              (4, "32x32x32_2valu", 2 * 32 * 32 * 32),
+              # the bit-block kernel's inner loop without global loads (64 instructions per round), without / with
+              # the LDS writes and the barrier that end a unit; two workgroups per CU
+              (5, "32x32x32_loop", 2 * 32 * 32 * 32), (6, "32x32x32_loop_write_barrier", 2 * 32 * 32 * 32),
+              (7, "32x32x32_loop_barrier", 2 * 32 * 32 * 32))
+    for shape, name, ops in shapes:
+        nb, it, per = (blocks, iters, 8) if shape < 5 else (cus * 2, iters // 8, 64)
+        ms = time_op(lambda: _lib.check(L.tango_probe_mfma_i8(shape, it, nb, sink.data_ptr(), st), "probe"),
                      iters=5, warm=2)
-        out["i8_%s_TOPS" % name] = round(blocks * 4 * iters * 8 * ops / ms / 1e9, 1)
+        out["i8_%s_TOPS" % name] = round(nb * 4 * it * per * ops / ms / 1e9, 1)
     return out
 
 

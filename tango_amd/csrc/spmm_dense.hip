@@ -7,11 +7,12 @@
 //   dense_stage_kernel   gathers the ranked columns' feature rows and writes them transposed, in the
 //                        order the matrix instruction's second operand wants them (one KB per fragment);
 //   dense_zero_kernel    zeroes the partial sums of row blocks that several workgroups add into;
-//   dense_block_kernel   one persistent 8-wave workgroup per CU walks its segments (row block, range of
-//                        256-column units): a unit's staged features go through a two-buffer LDS ring,
-//                        the mask bits come straight from memory (one dword per lane and k-step = two
-//                        operand fragments after a shift and an AND per dword), a wave owns 64 rows x half
-//                        the columns in accumulator registers and leaves them as int32 partial sums.
+//   dense_block_kernel   two persistent 4-wave workgroups per CU walk their segments (row block, range of
+//                        256-column units): a unit's staged features go from global memory straight into one
+//                        of two LDS chunks, the mask bits come straight from memory (one dword per lane and
+//                        k-step = two operand fragments after a shift and an AND per dword), a wave owns a
+//                        128 x 64 (narrow features: 64 x 64) tile in accumulator registers and leaves it as
+//                        int32 partial sums.
 // The gather kernels of spmm.hip then add those partial sums in their epilogue.  Integer arithmetic
 // throughout: the result does not depend on how the adjacency was split.
 #include "spmm_dense.hpp"
@@ -99,14 +100,34 @@ __global__ __launch_bounds__(256, 2) void dense_block_kernel(const DenseParams p
     constexpr int PASSES = CHUNK / (256 * 16);
     constexpr int CT = NCTW * 2 / RW;  // column tiles of a wave
     constexpr int RG = RW / 2;         // 64-row groups of a wave
-    extern __shared__ __attribute__((aligned(16))) int8_t ring[];
+    // Two chunks, as two objects: the compiler then knows that the loads that fill one do not touch the one
+    // the fragment reads come from, and does not make those reads wait for the loads.
+    __shared__ __attribute__((aligned(16))) int8_t chunk_a[CHUNK];
+    __shared__ __attribute__((aligned(16))) int8_t chunk_b[CHUNK];
     const int t = threadIdx.x;
     const int lane = t & 63;
     const int wave = __builtin_amdgcn_readfirstlane(t >> 6);
     const int rgrp = RW == 4 ? wave >> 1 : wave, cgrp = RW == 4 ? wave & 1 : 0;
-    const int q = blockIdx.y;  // column split
-    const int sg0 = p.seg_ptr[blockIdx.x], sg1 = p.seg_ptr[blockIdx.x + 1];
+    // Workgroups go to the eight XCDs round-robin by their linear id.  A column split is bound to 8 / SPLIT of them, so
+    // that an XCD's L2 only has to hold that split's share of the staged features (every row block reads all of it).
+    int q = blockIdx.y, grp = blockIdx.x;  // column split, group of segments
+    if (SPLIT > 1 && (gridDim.x & 7) == 0) {
+        constexpr int PER = 8 / SPLIT;
+        const int lin = blockIdx.y * gridDim.x + blockIdx.x, xcd = lin & 7;
+        q = xcd / PER;
+        grp = (lin >> 3) * PER + xcd % PER;
+    }
+    const int sg0 = p.seg_ptr[grp], sg1 = p.seg_ptr[grp + 1];
     const u32x4* xsrc = reinterpret_cast<const u32x4*>(p.xt + static_cast<int64_t>(q) * p.units * CHUNK) + t;
+    // The staged chunk of unit u goes from global memory straight into LDS (no registers, no LDS store instructions,
+    // which cost this loop a third of its rate): each wave instruction lands 64 lanes x 16 bytes at a wave-uniform
+    // LDS address, in the order they sit in global memory.
+    auto stage = [&](int8_t* chunk, int64_t u) {
+        const u32x4* x = xsrc + u * (CHUNK / 16);
+#pragma unroll
+        for (int i = 0; i < PASSES; ++i)
+            __builtin_amdgcn_global_load_lds(x + i * 256, reinterpret_cast<u32x4*>(chunk) + i * 256 + wave * 64, 16, 0, 0);
+    };
     for (int sg = sg0; sg < sg1; ++sg) {
         const int rb = p.segs[4 * sg], u0 = p.segs[4 * sg + 1], nu = p.segs[4 * sg + 2], shared = p.segs[4 * sg + 3];
         i32x16v acc[CT][RW];
@@ -118,36 +139,26 @@ __global__ __launch_bounds__(256, 2) void dense_block_kernel(const DenseParams p
                 for (int v = 0; v < 16; ++v) acc[c][h][v] = 0;
         // this wave's mask words of unit u: two row groups of 64 rows, two 16-byte loads per lane each
         const u32x4* mrow = reinterpret_cast<const u32x4*>(p.mask + p.mask_off[rb]) + rgrp * (128 * RG) + lane;
-        u32x4 mw[RG][2], mnext[RG][2], xnext[PASSES];
-        {   // first unit of the segment: straight into buffer 0.  The mask words are asked for first, so that
-            // nothing is in flight when the loop is entered (the compiler would otherwise wait for every load
-            // at the top of each iteration instead of at its end)
+        u32x4 mw[RG][2], mnext[RG][2];
+        // first unit of the segment: every wave is past the barrier that ended the previous segment's last unit,
+        // so nobody reads either chunk any more
+        stage(chunk_a, u0);
+#pragma unroll
+        for (int g = 0; g < RG; ++g)
+#pragma unroll
+            for (int hf = 0; hf < 2; ++hf) mw[g][hf] = mrow[static_cast<int64_t>(u0) * 512 + g * 128 + hf * 64];
+        __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): the chunk has landed in LDS
+        __syncthreads();
+        // One unit: ask for the next unit's chunk (into the chunk nobody reads now) and mask words, multiply this
+        // one, wait for what was asked for (long since there), barrier.  The last unit asks for itself again: every
+        // load is unconditional, so that the compiler waits for them behind the products and not at a join in front.
+        auto unit = [&](const int8_t* cur, int8_t* nxt, int k) {
+            const int64_t un = u0 + (k + 1 < nu ? k + 1 : k);
+            stage(nxt, un);
 #pragma unroll
             for (int g = 0; g < RG; ++g)
 #pragma unroll
-                for (int hf = 0; hf < 2; ++hf) mw[g][hf] = mrow[static_cast<int64_t>(u0) * 512 + g * 128 + hf * 64];
-            const u32x4* x = xsrc + static_cast<int64_t>(u0) * (CHUNK / 16);
-#pragma unroll
-            for (int i = 0; i < PASSES; ++i) xnext[i] = x[i * 256];
-#pragma unroll
-            for (int i = 0; i < PASSES; ++i) *reinterpret_cast<u32x4*>(ring + (i * 256 + t) * 16) = xnext[i];
-            __syncthreads();
-        }
-        for (int k = 0; k < nu; ++k) {
-            const int8_t* buf = ring + (k & 1) * CHUNK;
-            // the next unit's chunk and mask words (the last unit asks for itself again: every load is
-            // unconditional, so that the compiler waits for them where they are used, after the products,
-            // and not at a join in front of them)
-            const int64_t un = u0 + (k + 1 < nu ? k + 1 : k);
-            {
-                const u32x4* x = xsrc + un * (CHUNK / 16);
-#pragma unroll
-                for (int i = 0; i < PASSES; ++i) xnext[i] = x[i * 256];
-#pragma unroll
-                for (int g = 0; g < RG; ++g)
-#pragma unroll
-                    for (int hf = 0; hf < 2; ++hf) mnext[g][hf] = mrow[un * 512 + g * 128 + hf * 64];
-            }
+                for (int hf = 0; hf < 2; ++hf) mnext[g][hf] = mrow[un * 512 + g * 128 + hf * 64];
             __builtin_amdgcn_sched_barrier(0);  // the loads stay in front of the products, their use behind them
 #pragma unroll
             for (int s = 0; s < 8; ++s) {
@@ -163,23 +174,23 @@ __global__ __launch_bounds__(256, 2) void dense_block_kernel(const DenseParams p
                 }
 #pragma unroll
                 for (int c = 0; c < CT; ++c) {
-                    const i32x4 ff = *reinterpret_cast<const i32x4*>(buf + ((s * NCTW + cgrp * CT + c) * 64 + lane) * 16);
+                    const i32x4 ff = *reinterpret_cast<const i32x4*>(cur + ((s * NCTW + cgrp * CT + c) * 64 + lane) * 16);
 #pragma unroll
                     for (int h = 0; h < RW; ++h)
                         acc[c][h] = __builtin_amdgcn_mfma_i32_32x32x32_i8(mf[h], ff, acc[c][h], 0, 0, 0);
                 }
             }
             __builtin_amdgcn_sched_barrier(0);
-            {
-                int8_t* nbuf = ring + ((k + 1) & 1) * CHUNK;
+            __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
 #pragma unroll
-                for (int i = 0; i < PASSES; ++i) *reinterpret_cast<u32x4*>(nbuf + (i * 256 + t) * 16) = xnext[i];
+            for (int g = 0; g < RG; ++g)
 #pragma unroll
-                for (int g = 0; g < RG; ++g)
-#pragma unroll
-                    for (int hf = 0; hf < 2; ++hf) mw[g][hf] = mnext[g][hf];
-            }
+                for (int hf = 0; hf < 2; ++hf) mw[g][hf] = mnext[g][hf];
             __syncthreads();  // the next chunk is in place and nobody reads the current one any more
+        };
+        for (int k = 0; k < nu; k += 2) {
+            unit(chunk_a, chunk_b, k);
+            if (k + 1 < nu) unit(chunk_b, chunk_a, k + 1);
         }
         // the mask is the instruction's first operand, so accumulator v of tile (c, h) is row
         // 8 (v / 4) + 4 (lane / 32) + v % 4, column lane % 32 of the tile: a store covers 128 bytes of two rows
@@ -262,9 +273,20 @@ __global__ __launch_bounds__(256) void mfma_probe_kernel(int iters, int* sink) {
         for (int c = 0; c < 8; ++c)
 #pragma unroll
             for (int v = 0; v < 16; ++v) acc[c][v] = c + v;
+        // SHAPE 2, 3, 4: the first operand is expanded from a word of bits (a shift and an and per register, as the
+        // bit-block kernel does) once per 1, 2, 4 matrix instructions: what the matrix pipes sustain beside that work
+        constexpr int PER = SHAPE <= 1 ? 0 : 1 << (SHAPE - 2);
+        uint32_t word = 0x9e3779b9u * static_cast<uint32_t>(lane + 1);
         for (int it = 0; it < iters; ++it) {
+            if (PER) word += 0x01000193u;
 #pragma unroll
-            for (int c = 0; c < 8; ++c) acc[c] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, b, acc[c], 0, 0, 0);
+            for (int c = 0; c < 8; ++c) {
+                if (PER && c % PER == 0) {
+#pragma unroll
+                    for (int w = 0; w < 4; ++w) a[w] = static_cast<int>((word >> ((c + w) & 7)) & 0x01010101u);
+                }
+                acc[c] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, b, acc[c], 0, 0, 0);
+            }
         }
 #pragma unroll
         for (int c = 0; c < 8; ++c)
@@ -272,6 +294,64 @@ __global__ __launch_bounds__(256) void mfma_probe_kernel(int iters, int* sink) {
             for (int v = 0; v < 16; ++v) total += acc[c][v];
     }
     if (total == 0x7fffffff) sink[0] = total;  // keeps the chains alive; practically never taken
+}
+
+// The inner loop of the bit-block kernel without its global loads (timing experiments): per round eight k-steps of
+// (two fragment reads from LDS, four operand expansions, eight matrix instructions); LEVEL 1 adds the LDS writes
+// and the workgroup barrier that end a unit.  blockDim.x = 256, dynamic LDS 64 KB.
+template <int LEVEL>
+__global__ __launch_bounds__(256, 2) void mfma_loop_probe_kernel(int iters, int* sink) {
+    extern __shared__ __attribute__((aligned(16))) int8_t ring[];
+    const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
+    for (int i = t; i < 4096; i += 256) reinterpret_cast<i32x4*>(ring)[i] = i32x4{i, i + 1, i + 2, i + 3};
+    __syncthreads();
+    i32x16v acc[2][4];
+#pragma unroll
+    for (int c = 0; c < 2; ++c)
+#pragma unroll
+        for (int h = 0; h < 4; ++h)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) acc[c][h][v] = 0;
+    u32x4 mw[2][2];
+#pragma unroll
+    for (int g = 0; g < 2; ++g)
+#pragma unroll
+        for (int hf = 0; hf < 2; ++hf) mw[g][hf] = u32x4{0x9e3779b9u * (lane + 1), 0x85ebca6bu * (lane + 3), 0xc2b2ae35u * (lane + 5), 0x27d4eb2fu * (lane + 7)};
+    for (int k = 0; k < iters; ++k) {
+        const int8_t* buf = ring + (k & 1) * 32768;
+#pragma unroll
+        for (int s = 0; s < 8; ++s) {
+            i32x4 mf[4];
+#pragma unroll
+            for (int g = 0; g < 2; ++g) {
+                const uint32_t word = mw[g][s >> 2][s & 3] + k;
+#pragma unroll
+                for (int h = 0; h < 2; ++h)
+#pragma unroll
+                    for (int w = 0; w < 4; ++w) mf[2 * g + h][w] = static_cast<int>((word >> (4 * h + w)) & 0x01010101u);
+            }
+#pragma unroll
+            for (int c = 0; c < 2; ++c) {
+                const i32x4 ff = *reinterpret_cast<const i32x4*>(buf + ((s * 4 + (wave & 1) * 2 + c) * 64 + lane) * 16);
+#pragma unroll
+                for (int h = 0; h < 4; ++h) acc[c][h] = __builtin_amdgcn_mfma_i32_32x32x32_i8(mf[h], ff, acc[c][h], 0, 0, 0);
+            }
+        }
+        if (LEVEL == 1) {
+            int8_t* nbuf = ring + ((k + 1) & 1) * 32768;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) *reinterpret_cast<u32x4*>(nbuf + (i * 256 + t) * 16) = mw[i & 1][(i >> 1) & 1];
+        }
+        if (LEVEL >= 1) __syncthreads();
+    }
+    int total = 0;
+#pragma unroll
+    for (int c = 0; c < 2; ++c)
+#pragma unroll
+        for (int h = 0; h < 4; ++h)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) total += acc[c][h][v];
+    if (total == 0x7fffffff) sink[0] = total;
 }
 
 static size_t align256(size_t v) { return (v + 255) & ~static_cast<size_t>(255); }
@@ -307,7 +387,6 @@ int launch_dense_block(const tango_spmm_dense_plan& plan, const int8_t* feat, in
     const dim3 sgrid(static_cast<unsigned>(plan.dense_cols / 64));
 #define TANGO_DENSE(NPAD, NCTW, RW)                                                                              \
     do {                                                                                                     \
-        constexpr int LDS = 2 * 8 * NCTW * 1024;                                                             \
         constexpr int SPLIT = NPAD / (32 * NCTW);                                                            \
         if (SPLIT == 1) {                                                                                    \
             p.seg_ptr = plan.seg_ptr2; p.segs = plan.segs2;                                                  \
@@ -316,10 +395,10 @@ int launch_dense_block(const tango_spmm_dense_plan& plan, const int8_t* feat, in
         hipLaunchKernelGGL((dense_stage_kernel<NPAD, NCTW>), sgrid, dim3(256), 0, s, p);                     \
         if (plan.num_shared > 0)                                                                             \
             hipLaunchKernelGGL(dense_zero_kernel, dim3(static_cast<unsigned>(plan.num_shared)), dim3(256), 0, s, p); \
-        hipLaunchKernelGGL((dense_block_kernel<NCTW, SPLIT, RW>), bgrid, dim3(256), LDS, s, p);                           \
+        hipLaunchKernelGGL((dense_block_kernel<NCTW, SPLIT, RW>), bgrid, dim3(256), 0, s, p);                             \
     } while (0)
     if (npad == 64) TANGO_DENSE(64, 2, 2);
-    else if (npad == 128) TANGO_DENSE(128, 4, 4);
+    else if (npad == 128) TANGO_DENSE(128, 2, 2);
     else TANGO_DENSE(256, 4, 4);
 #undef TANGO_DENSE
     return launch_status();
@@ -332,9 +411,18 @@ using namespace tango;
 extern "C" {
 
 int tango_probe_mfma_i8(int shape, int iters, int blocks, int* sink, tango_stream_t stream) {
-    if ((shape != 0 && shape != 1) || iters < 0 || blocks <= 0 || !sink) return TANGO_ERR_INVALID_ARG;
-    if (shape == 0) hipLaunchKernelGGL(mfma_probe_kernel<0>, dim3(blocks), dim3(256), 0, as_stream(stream), iters, sink);
-    else hipLaunchKernelGGL(mfma_probe_kernel<1>, dim3(blocks), dim3(256), 0, as_stream(stream), iters, sink);
+    if (shape < 0 || shape > 7 || iters < 0 || blocks <= 0 || !sink) return TANGO_ERR_INVALID_ARG;
+    hipStream_t s = as_stream(stream);
+    switch (shape) {
+        case 0: hipLaunchKernelGGL(mfma_probe_kernel<0>, dim3(blocks), dim3(256), 0, s, iters, sink); break;
+        case 1: hipLaunchKernelGGL(mfma_probe_kernel<1>, dim3(blocks), dim3(256), 0, s, iters, sink); break;
+        case 2: hipLaunchKernelGGL(mfma_probe_kernel<2>, dim3(blocks), dim3(256), 0, s, iters, sink); break;
+        case 3: hipLaunchKernelGGL(mfma_probe_kernel<3>, dim3(blocks), dim3(256), 0, s, iters, sink); break;
+        case 4: hipLaunchKernelGGL(mfma_probe_kernel<4>, dim3(blocks), dim3(256), 0, s, iters, sink); break;
+        case 5: hipLaunchKernelGGL(mfma_loop_probe_kernel<0>, dim3(blocks), dim3(256), 65536, s, iters, sink); break;
+        case 6: hipLaunchKernelGGL(mfma_loop_probe_kernel<1>, dim3(blocks), dim3(256), 65536, s, iters, sink); break;
+        default: hipLaunchKernelGGL(mfma_loop_probe_kernel<2>, dim3(blocks), dim3(256), 65536, s, iters, sink); break;
+    }
     return launch_status();
 }
 

@@ -47,36 +47,74 @@ class DensePlan:
         self.ref = ctypes.byref(s)
 
 
-def _segments(units, groups):
-    """Deals the units of every row block over ``groups`` workgroups: blocks much longer than a fair share
-    are cut into pieces (several workgroups then add into the block's partial sums), the others stay whole;
-    longest piece first to the least loaded workgroup.  Returns (seg_ptr, segs, shared_blocks) as numpy."""
+# what a segment costs beside its units, in units of work: its prologue and flush; the atomic flush of a shared block
+SEGMENT_COST = 1.8
+SHARED_COST = 1.3
+
+
+def _segments(units, groups, min_piece=4):
+    """Deals the units of every row block over ``groups`` workgroups so that all finish together (a launch lasts
+    as long as its slowest workgroup).  Blocks of less than 0.8 of a fair share stay whole and go, heaviest first,
+    to the least loaded workgroup; the longer blocks are then poured into what room is left below a common level,
+    cut where a workgroup is full (several workgroups then add into such a block's partial sums).  Returns (seg_ptr, segs [(row block, first unit, units, shared)], shared_blocks)
+    as numpy."""
     total = int(units.sum())
     groups = max(1, min(groups, total))
     fair = total / groups
-    items = []  # (units, row block, first unit, shared)
-    shared = []
-    for b, n in enumerate(units.tolist()):
-        if n > 1.5 * fair:
-            pieces = int(np.ceil(n / fair))
-            cuts = np.linspace(0, n, pieces + 1).round().astype(np.int64)
-            shared.append(b)
-            for a, e in zip(cuts[:-1], cuts[1:]):
-                if e > a:
-                    items.append((int(e - a), b, int(a), 1))
-        elif n > 0:
-            items.append((n, b, 0, 0))
-    items.sort(key=lambda it: -it[0])
-    heap = [(0, g) for g in range(groups)]
+    whole = sorted(((n, b) for b, n in enumerate(units.tolist()) if 0 < n <= 0.8 * fair), reverse=True)
+    cut = sorted(((n, b) for b, n in enumerate(units.tolist()) if n > 0.8 * fair), reverse=True)
+    load = np.zeros(groups)
     per_group = [[] for _ in range(groups)]
-    for n, b, a, sh in items:
-        load, g = heapq.heappop(heap)
-        per_group[g].append((b, a, n, sh))
-        heapq.heappush(heap, (load + n, g))
+    for n, b in whole:
+        g = int(np.argmin(load))
+        per_group[g].append((b, 0, n, 0))
+        load[g] += n + SEGMENT_COST
+    piece_cost = SEGMENT_COST + SHARED_COST
+    need = sum(n for n, _ in cut)
+
+    def room(level):
+        r = np.floor(level - load - piece_cost)
+        r[r < min_piece] = 0
+        return r
+
+    lo, hi = 0.0, float(load.max() + need + piece_cost + min_piece)
+    for _ in range(60):
+        mid = 0.5 * (lo + hi)
+        if room(mid).sum() >= need:
+            hi = mid
+        else:
+            lo = mid
+    left = room(hi).astype(np.int64)
+    order = [int(g) for g in np.argsort(-left, kind="stable") if left[g] > 0]
+    gi = 0
+    for n, b in cut:
+        a = 0
+        while n > 0:
+            if gi < len(order):
+                g = order[gi]
+                take = int(min(n, left[g]))
+                if 0 < n - take < min_piece:  # no sliver of a block: this workgroup takes it too
+                    take = n
+                left[g] -= take
+                if left[g] < min_piece:
+                    gi += 1
+            else:  # rounding leftovers
+                g = int(np.argmin(load))
+                take = n
+            per_group[g].append((b, a, take, 1))
+            load[g] += take + piece_cost
+            a += take
+            n -= take
+    pieces = {}
+    for lst in per_group:
+        for b, _, _, _ in lst:
+            pieces[b] = pieces.get(b, 0) + 1
+    shared = sorted(b for b, k in pieces.items() if k > 1)
     seg_ptr = np.zeros(groups + 1, dtype=np.int32)
     segs = []
     for g, lst in enumerate(per_group):
-        segs.extend(lst)
+        lst.sort(key=lambda it: -it[2])  # the longest piece first
+        segs.extend((b, a, n, 1 if pieces[b] > 1 else 0) for b, a, n, _ in lst)
         seg_ptr[g + 1] = len(segs)
     return seg_ptr, np.asarray(segs, dtype=np.int32).reshape(-1, 4), np.asarray(shared, dtype=np.int32)
 
