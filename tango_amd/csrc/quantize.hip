@@ -641,6 +641,17 @@ __global__ __launch_bounds__(256) void absmax_ex_kernel(
         float v[RU][T][4];
         float mk[MK == 1 ? RU : 1][T][4];  // fp32 mask values
         unsigned wb[MK == 2 ? RU : 1][T];  // the four sign bits of the lane's columns (bit set = keep)
+        // the rows' multipliers, asked for with the rows themselves (without a multiplier: some valid address, and
+        // the value is not used); a load in the loop that consumes the rows would wait for each row in turn
+        float rmv[RU];
+        {
+            const float* rmp = row_mul ? row_mul : x;
+#pragma unroll
+            for (int u = 0; u < RU; ++u) {
+                const int64_t row = row0 + u * row_step;
+                rmv[u] = rmp[row_mul ? (row < rows ? row : rows - 1) : 0];
+            }
+        }
         if (XV == 4 && whole_quads && (MK != 1 || mask_vec)) {
             // No lane has a partial quad: every load is issued unconditionally from a clamped address and the
             // lanes outside the matrix discard theirs.  Without branches between them the loads of all RU rows
@@ -669,32 +680,58 @@ __global__ __launch_bounds__(256) void absmax_ex_kernel(
                 }
             }
         } else {
+            // Rows with a partial last quad, or without 16-byte alignment: the same unconditional loads from
+            // clamped addresses, as wide as the layout allows (a quad of a padded row lies inside its pitch).
 #pragma unroll
-        for (int u = 0; u < RU; ++u) {
-            const int64_t row = row0 + u * row_step;
+            for (int u = 0; u < RU; ++u) {
+                const int64_t row = row0 + u * row_step;
+                const int64_t rr = row < rows ? row : rows - 1;
+                const float* xr = x + rr * ldx;
 #pragma unroll
-            for (int t = 0; t < T; ++t) {
-                const int64_t c0 = (static_cast<int64_t>(gl) + 64 * t) << 2;
+                for (int t = 0; t < T; ++t) {
+                    const int64_t c0 = (static_cast<int64_t>(gl) + 64 * t) << 2;
+                    const bool in0 = row < rows && c0 < cols;
+                    if (XV == 4) {
+                        const int64_t cc = c0 < cols ? c0 : ((cols - 1) & ~static_cast<int64_t>(3));
+                        const f32x4 a = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(xr + cc));
 #pragma unroll
-                for (int k = 0; k < 4; ++k) {
-                    v[u][t][k] = 0.0f;
-                    if (MK == 1) mk[u][t][k] = 1.0f;
-                }
-                if (MK == 2) wb[u][t] = 0xFu;
-                if (row < rows && c0 < cols) {
-                    load4<XV>(v[u][t], x + row * ldx, c0, cols);
-                    if (MK == 2)
-                        wb[u][t] = static_cast<unsigned>((reinterpret_cast<const uint16_t*>(mask) + row * ldm)[c0 >> 4]) >> (c0 & 15);
-                    else if (MK == 1 && mask_vec) load4<XV>(mk[u][t], mask + row * ldm, c0, cols);
-                    else if (MK == 1) load4<1>(mk[u][t], mask + row * ldm, c0, cols);
+                        for (int k = 0; k < 4; ++k) v[u][t][k] = (in0 && c0 + k < cols) ? a[k] : 0.0f;
+                    } else if (XV == 2) {  // even columns and pitch: a pair lies inside the row or outside
+                        typedef float f32x2 __attribute__((ext_vector_type(2)));
+#pragma unroll
+                        for (int h = 0; h < 2; ++h) {
+                            const int64_t c = c0 + 2 * h;
+                            const f32x2 a = __builtin_nontemporal_load(reinterpret_cast<const f32x2*>(xr + (c < cols ? c : cols - 2)));
+                            v[u][t][2 * h] = (row < rows && c < cols) ? a[0] : 0.0f;
+                            v[u][t][2 * h + 1] = (row < rows && c + 1 < cols) ? a[1] : 0.0f;
+                        }
+                    } else {
+#pragma unroll
+                        for (int k = 0; k < 4; ++k) {
+                            const int64_t c = c0 + k;
+                            const float a = xr[c < cols ? c : cols - 1];
+                            v[u][t][k] = (row < rows && c < cols) ? a : 0.0f;
+                        }
+                    }
+                    if (MK == 1) {
+#pragma unroll
+                        for (int k = 0; k < 4; ++k) {
+                            const int64_t c = c0 + k;
+                            const float b = mask[rr * ldm + (c < cols ? c : cols - 1)];
+                            mk[u][t][k] = (row < rows && c < cols) ? b : 1.0f;
+                        }
+                    }
+                    if (MK == 2) {  // cols is a multiple of 16 here (checked by the caller)
+                        const int64_t cc = c0 < cols ? c0 : cols - 4;
+                        const unsigned w = (reinterpret_cast<const uint16_t*>(mask) + rr * ldm)[cc >> 4];
+                        wb[u][t] = in0 ? (w >> (cc & 15)) : 0xFu;
+                    }
                 }
             }
         }
-        }
 #pragma unroll
         for (int u = 0; u < RU; ++u) {  // rows are added in the order a one-row-at-a-time loop would take them
-            const int64_t row = row0 + u * row_step;
-            const float rm = (row_mul && row < rows) ? row_mul[row] : 1.0f;
+            const float rm = rmv[u];
 #pragma unroll
             for (int t = 0; t < T; ++t)
 #pragma unroll
