@@ -122,6 +122,20 @@ int tango_quantize_rows_ex_f32_i8(const float* x, int64_t rows, int64_t cols, in
                                   int round_mode, const float* noise, uint64_t seed,
                                   uint64_t offset, const uint64_t* offset_dev, tango_stream_t stream);
 
+/* tango_quantize_rows_ex_f32_i8 on a dense matrix (no padding in x, q or the mask) that also returns the column
+   sums of the masked input before the row multiplier, colsum_out[c] = sum_r masked(x[r, c]): the bias gradient of a
+   fused "mask, sum, scale rows, quantize" backward step (cuda/QLinear.py:46 with the glue of
+   evaluation/test_gcn.py:123-137) out of the pass that quantizes, for callers that already hold the scale.  Added in
+   a fixed order.  Only for cols a multiple of 4 with 256 % (cols / 4) == 0 (a multiple of 16 with sign-word masks),
+   x 16-byte and q 4-byte aligned: TANGO_ERR_UNSUPPORTED otherwise, before anything is launched.
+   workspace: tango_quantize_rows_colsum_workspace(rows, cols) bytes. */
+size_t tango_quantize_rows_colsum_workspace(int64_t rows, int64_t cols);
+int tango_quantize_rows_colsum_f32_i8(const float* x, int64_t rows, int64_t cols, const float* row_mul,
+                                      const void* mask, int mask_mode, const float* scale, int8_t* q,
+                                      int round_mode, const float* noise, uint64_t seed, uint64_t offset,
+                                      const uint64_t* offset_dev, float* colsum_out, void* workspace,
+                                      size_t workspace_bytes, tango_stream_t stream);
+
 /* transpose_quant (cuda/src/cuda.cpp:27-33 -> transpose_quant_impl,
    quantization.cu:95-167): x[nrow, ncol] fp32 -> out[ncol, nrow] int8,
    half-to-even, clamped to +-127. */
@@ -207,6 +221,20 @@ int tango_qgemm_bwd_dx_ex(float* dX, int64_t lddx, const int8_t* dYq, int64_t ld
                           const int8_t* Wq, int64_t ldw, const float* s_dY, const float* s_W,
                           const float* row_scale, int accumulate, int64_t M, int64_t N, int64_t K,
                           void* workspace, size_t workspace_bytes, tango_stream_t stream);
+
+/* tango_qgemm_bwd_dx_ex that also finds the scale its consumer needs when that consumer takes dX back through
+   a ReLU and multiplies its rows (the aggregation in front of this layer, cuda/SPMM.py:15-24 with the layer glue of
+   evaluation/test_gcn.py:123-137 folded in): masked_scale_out[0] = max |dX[m, k] * mask_mul[m]| / 127 over the
+   elements whose sign bit is set (bit k % 16 of the 16-bit word mask_bits[m * ldmask + k / 16]; mask_mul may be
+   NULL), from the epilogue that stores dX instead of a pass over it.  Only for K (columns of dX) in {32, 64, 128,
+   256}, N <= 256, dX rows 16-byte aligned, dYq rows readable in 4-byte pieces, ldmask even and mask_bits 4-byte
+   aligned: TANGO_ERR_UNSUPPORTED otherwise, before anything is launched (call tango_qgemm_bwd_dx_ex and
+   tango_absmax_ex_f32 then). */
+int tango_qgemm_bwd_dx_masked(float* dX, int64_t lddx, const int8_t* dYq, int64_t lddy, const int8_t* Wq,
+                              int64_t ldw, const float* s_dY, const float* s_W, const float* row_scale,
+                              const uint16_t* mask_bits, int64_t ldmask, const float* mask_mul,
+                              float* masked_scale_out, int64_t M, int64_t N, int64_t K, void* workspace,
+                              size_t workspace_bytes, tango_stream_t stream);
 
 /* QGEMM_backward_gradW (cuda/src/cuda.cpp:100-108 -> QGEMM_backward.cu:50-113):
    dW[N,K] = (s_dY*s_X) * float(sum_m dYq[m,n] * Xq[m,k]), int32 accumulation.

@@ -67,6 +67,9 @@ def quantize_input(X, scaleX=None):
 
 
 def _forward(ctx, X, W, b, reduce, row_scale=None, scaleX=None, Xq=None):
+    from .SPMM import relu_mask_of
+    # X straight out of an aggregation's fused ReLU: the backward pass can hand that op the scale it needs
+    ctx.dx_masked = relu_mask_of(X) if X.dim() == 2 and X.is_contiguous() else None
     X = X if X.is_contiguous() else X.contiguous()
     if Xq is not None:
         if scaleX is None or row_scale is not None:
@@ -100,7 +103,7 @@ def _backward(ctx, grad_output):
     dY_, scaledY, grad_bias = _quantize_grad(grad_output, want_bias)
     grad_input, grad_weight = kernels.QGEMM_backward(
         dY_, X_, W_, scaledY, scaleX, scaleW, ctx.needs_input_grad[0], ctx.needs_input_grad[1],
-        x_row_scale=row_scale)
+        x_row_scale=row_scale, dx_masked=getattr(ctx, "dx_masked", None))
     return grad_input, grad_weight, grad_bias, None
 
 

@@ -34,6 +34,26 @@ def grad_scale_hint(t):
     return None
 
 
+def masked_scale_hint(t, bits, row_mul):
+    """max|t' * row_mul| / 127 (t' = t where its sign bit in ``bits`` is set) if the GEMM that produced the gradient
+    ``t`` found it in its epilogue for exactly this mask and multiplier and nothing has written to ``t`` since."""
+    hint = getattr(t, "_tango_masked_scale", None)
+    if hint is None or hint[3] != t._version or hint[4] != t.data_ptr() or hint[1] is not bits:
+        return None
+    if (hint[2] is None) != (row_mul is None) or (row_mul is not None and hint[2].data_ptr() != row_mul.data_ptr()):
+        return None
+    return hint[0]
+
+
+def relu_mask_of(t):
+    """(sign words, row multiplier) of the fused ReLU epilogue that produced the activation ``t``, if ``t`` is still
+    that tensor: what the backward pass of ``t``'s producer will apply to the gradient of ``t``."""
+    tag = getattr(t, "_tango_relu", None)
+    if tag is not None and tag[2] == t._version and tag[3] == t.data_ptr():
+        return tag[0], tag[1]
+    return None
+
+
 def _quantize_grad(t, padded):
     t = t if t.is_contiguous() else t.contiguous()
     kw = {"round_mode": config.grad_round_mode}
@@ -92,6 +112,10 @@ class spmm_copy_u(Function):
         ctx.backward_cache = g, row_scale, bias is not None, bits, relu
         if relu and bits is None:
             ctx.save_for_backward(out)
+        if bits is not None:
+            # for a quantized linear layer that consumes out: its backward can then find the scale of the masked,
+            # row-scaled gradient in the epilogue that writes the gradient (relu_mask_of)
+            out._tango_relu = (bits, row_scale, out._version, out.data_ptr())
         if want_scale:
             ctx.mark_non_differentiable(scale_out)
             ctx.set_materialize_grads(False)
@@ -127,9 +151,30 @@ class spmm_copy_u(Function):
         want_bias = has_bias and ctx.needs_input_grad[4]
         # dZ = (dOut where out > 0) * row_scale; its scale and the bias gradient come from one pass
         mode = "bits" if mask is not None and mask.dtype == torch.int16 else "relu"
+        kw = {"round_mode": config.grad_round_mode}
+        # the GEMM that wrote dOut may already have found the scale (of exactly this mask and multiplier)
+        scaledZ = masked_scale_hint(dOut, mask, row_scale) if mode == "bits" and ctx.needs_input_grad[1] else None
+        if scaledZ is not None:
+            if config.grad_round_mode == "stochastic":
+                kw.update(config.stochastic_args(dOut.device))
+            cols = dOut.size(1)
+            dZ_ = None
+            if want_bias and _gather_align(cols) <= cols and cols % _gather_align(cols) == 0:
+                # the bias gradient out of the pass that quantizes: no pass over dOut is left that only reduces
+                dZ_ = torch.empty(dOut.shape, dtype=torch.int8, device=dOut.device)
+                dbias = cuda_kernels.quantize_rows_colsum(dZ_, dOut, scaledZ, row_mul=row_scale, mask=mask,
+                                                          mask_mode=mode, **kw)
+                if dbias is None:
+                    dZ_ = None
+            if dZ_ is None:
+                if want_bias:
+                    _, dbias = cuda_kernels.absmax_ex(dOut, row_mul=row_scale, mask=mask, want_colsum=True, mask_mode=mode)
+                dZ_, _ = quantize_padded(dOut, scaledZ, row_mul=row_scale, mask=mask, mask_mode=mode,
+                                         align=_gather_align(cols), **kw)
+            dN = spmm_copy_u._reverse(ctx, g, dZ_, scaledZ)
+            return None, dN, None, None, dbias, None, None, None, None
         scaledZ, dbias = cuda_kernels.absmax_ex(dOut, row_mul=row_scale, mask=mask, want_colsum=want_bias, mask_mode=mode)
         if ctx.needs_input_grad[1]:
-            kw = {"round_mode": config.grad_round_mode}
             if config.grad_round_mode == "stochastic":
                 kw.update(config.stochastic_args(dOut.device))
             dZ_, _ = quantize_padded(dOut, scaledZ, row_mul=row_scale, mask=mask, mask_mode=mode,

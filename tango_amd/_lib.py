@@ -29,6 +29,8 @@ SIGNATURES = {
     "tango_absmax_ex_workspace": (SZ, [I64, I64, I]),
     "tango_absmax_ex_f32": (I, [P, I64, I64, I64, P, P, I64, I, P, I, P, P, SZ, P]),
     "tango_quantize_rows_ex_f32_i8": (I, [P, I64, I64, I64, P, P, I64, I, P, I, P, I64, I, P, U64, U64, P, P]),
+    "tango_quantize_rows_colsum_workspace": (SZ, [I64, I64]),
+    "tango_quantize_rows_colsum_f32_i8": (I, [P, I64, I64, P, P, I, P, P, I, P, U64, U64, P, P, P, SZ, P]),
     "tango_transpose_quant_f32_i8": (I, [P, I64, I64, P, P, P]),
     "tango_qgemm_fwd_workspace": (SZ, [I64, I64, I64]),
     "tango_qgemm_fwd": (I, [P, I64, P, I64, P, I64, P, I64, P, P, P, P, P, I64, I64, I64, I, P, SZ, P]),
@@ -39,6 +41,7 @@ SIGNATURES = {
     "tango_qgemm_bwd_dx": (I, [P, I64, P, I64, P, I64, P, P, I64, I64, I64, P, SZ, P]),
     "tango_qgemm_fwd_q8": (I, [P, I64, P, P, I64, P, I64, P, P, P, P, I64, I64, I64, I, P, SZ, P]),
     "tango_qgemm_bwd_dx_ex": (I, [P, I64, P, I64, P, I64, P, P, P, I, I64, I64, I64, P, SZ, P]),
+    "tango_qgemm_bwd_dx_masked": (I, [P, I64, P, I64, P, I64, P, P, P, P, I64, P, P, I64, I64, I64, P, SZ, P]),
     "tango_qgemm_bwd_dw_workspace": (SZ, [I64, I64, I64]),
     "tango_qgemm_bwd_dw": (I, [P, I64, P, I64, P, I64, P, P, I64, I64, I64, P, SZ, P]),
     "tango_qgemm_legacy_workspace": (SZ, [I64, I64, I64]),

@@ -65,6 +65,13 @@ struct NtParams {
     int64_t ldcq;
     const float* q_scale;  // the scale Cq is rounded with
     int q_mode;          // TANGO_ROUND_RNE or TANGO_ROUND_TRUNC
+    // stationary form, fp32 output: also max |C[m, n] * mask_mul[m]| / 127 over the elements whose sign bit is set
+    // (bit n % 16 of word mask_bits[m * ldmask + n / 16]): the scale the consumer of a gradient needs when it takes
+    // the gradient back through a ReLU and multiplies its rows (pre-zeroed; mask_mul may be null)
+    const uint16_t* mask_bits;
+    int64_t ldmask;
+    const float* mask_mul;
+    float* masked_absmax_out;
 };
 
 // Workgroup = 4 waves = 128 rows x (16 * NT) columns.  gridDim = (ceil(M/128), ceil(N/(16 NT))).
@@ -221,6 +228,7 @@ __global__ __launch_bounds__(256, 2) void gemm_nt_kernel(const NtParams p) {
 // 1 then 2 store exactly what a quantize pass over the fp32 output of 0 would).
 template <int NT, int VEC, int WAVES, int EPI = 0, int PASSES = 1>
 __global__ __launch_bounds__(64 * WAVES) void gemm_nts_kernel(const NtParams p, int ntiles) {
+    constexpr bool F32OUT = EPI == 0 || EPI == 3;  // EPI 3: EPI 0 that also finds the masked maximum
     // B in fragment order: block (j, st) of 1 KB holds, at 16 lane bytes, the 16 bytes lane `lane` feeds the MFMA
     // of column tile j at k-step st, so a fragment read is one linear 1 KB sweep (no bank conflicts by construction)
     extern __shared__ __attribute__((aligned(16))) int8_t b_lds[];  // [PASSES NT][ksteps][64 lanes][16]
@@ -267,11 +275,20 @@ __global__ __launch_bounds__(64 * WAVES) void gemm_nts_kernel(const NtParams p, 
     const float qr = EPI == 2 ? rscale_of(p.q_scale[0]) : 0.0f;
     const bool qwide = EPI == 2 && (reinterpret_cast<uintptr_t>(p.Cq) & 3) == 0 && (p.ldcq & 3) == 0;
     const bool q16 = EPI == 2 && (reinterpret_cast<uintptr_t>(p.Cq) & 15) == 0 && (p.ldcq & 15) == 0;
-    float m = 0.0f;
-    auto load_tile = [&](i32x4* a, float& rsc, int t) {
+    float m = 0.0f, m2 = 0.0f;
+    // the masked maximum: only with the plain fp32 epilogue over whole blocks of NT tiles (checked by the host)
+    constexpr bool want_masked = EPI == 3 && PASSES == 1 && NT % 2 == 0;
+    constexpr int BW = want_masked ? NT / 2 : 1;
+    auto load_tile = [&](i32x4* a, float& rsc, float& mmul, uint32_t* bw, int t) {
         const int64_t row = static_cast<int64_t>(t) * 16 + r16;
         const bool ok = t < ntiles && row < p.M;
         rsc = (p.row_scale && ok) ? p.row_scale[row] : 1.0f;  // requested with the tile, not in the epilogue
+        if (want_masked) {  // uniform: the row's sign words of this block's columns, two per register
+            const uint32_t* w = reinterpret_cast<const uint32_t*>(p.mask_bits + (ok ? row : 0) * p.ldmask + (n0 >> 4));
+#pragma unroll
+            for (int j = 0; j < BW; ++j) bw[j] = w[j];
+            mmul = (p.mask_mul && ok) ? p.mask_mul[row] : 1.0f;
+        }
         const int8_t* pa = p.A + (ok ? row : 0) * p.lda + g * 16;
 #pragma unroll
         for (int st = 0; st < KS; ++st) {
@@ -282,21 +299,22 @@ __global__ __launch_bounds__(64 * WAVES) void gemm_nts_kernel(const NtParams p, 
     };
     const int stride = static_cast<int>(gridDim.x) * WAVES;
     i32x4 cur[KS], nxt[KS];
-    float rsc, rsc_nxt;
+    float rsc, rsc_nxt, mmul = 1.0f, mmul_nxt = 1.0f;
+    uint32_t bw[BW], bw_nxt[BW];
     int t = static_cast<int>(blockIdx.x) * WAVES + wave;
-    load_tile(cur, rsc, t);
+    load_tile(cur, rsc, mmul, bw, t);
     // fp32 output with nothing but the dequantization (and the optional row scale) in the epilogue: the common case
     // gets a loop without a branch per tile (the general loop below tests six uniform conditions per column tile)
-    const bool plain = EPI == 0 && !p.bias && !p.accumulate && wide == 4;
-    const bool want_max = EPI == 1 || (EPI == 0 && p.absmax_out != nullptr);
+    const bool plain = F32OUT && !p.bias && !p.accumulate && wide == 4;
+    const bool want_max = EPI == 1 || (F32OUT && p.absmax_out != nullptr);
     // columns of this block, as a 32-bit count: the bounds tests of the epilogue are 32-bit compares
     const int ncols = static_cast<int>(p.N - n0 < 16 * TT ? p.N - n0 : 16 * TT);
     // columns that may be written: a row's padding up to its pitch takes the zeros of the zero-filled rows of B
     // (never past the next multiple of 16 columns: what lies beyond may belong to the caller)
     const int64_t wlim = ((p.N + 15) & ~static_cast<int64_t>(15)) < p.ldc ? ((p.N + 15) & ~static_cast<int64_t>(15)) : p.ldc;
-    const int wcols = EPI == 0 ? static_cast<int>(wlim - n0 < 16 * TT ? wlim - n0 : 16 * TT) : ncols;
+    const int wcols = F32OUT ? static_cast<int>(wlim - n0 < 16 * TT ? wlim - n0 : 16 * TT) : ncols;
     for (; t < ntiles; t += stride) {
-        load_tile(nxt, rsc_nxt, t + stride);
+        load_tile(nxt, rsc_nxt, mmul_nxt, bw_nxt, t + stride);
         const int64_t row = static_cast<int64_t>(t) * 16 + r16;
         float* crow = p.C + row * p.ldc + n0;
 #pragma unroll
@@ -319,7 +337,21 @@ __global__ __launch_bounds__(64 * WAVES) void gemm_nts_kernel(const NtParams p, 
             const int c0 = ps * 16 * NT;  // first column of this pass inside the block
             if (plain && c0 + 16 * NT <= wcols) {
                 f32x4* cp = reinterpret_cast<f32x4*>(crow + c0 + 4 * g);
-                if (want_max) {
+                if (want_masked) {
+#pragma unroll
+                    for (int j = 0; j < NT; ++j) {
+                        const f32x4 y{(s * static_cast<float>(acc[j][0])) * rsc, (s * static_cast<float>(acc[j][1])) * rsc,
+                                      (s * static_cast<float>(acc[j][2])) * rsc, (s * static_cast<float>(acc[j][3])) * rsc};
+                        const uint32_t keep = bw[(j >> 1) % BW] >> (16 * (j & 1) + 4 * g);  // bits of columns 16 j + 4 g ..
+#pragma unroll
+                        for (int v = 0; v < 4; ++v) {
+                            const float e = ((keep >> v) & 1u) ? y[v] : 0.0f;
+                            m2 = fmaxf(m2, fabsf(p.mask_mul ? e * mmul : e));
+                        }
+                        if (want_max) m = fmaxf(fmaxf(m, fmaxf(fabsf(y[0]), fabsf(y[1]))), fmaxf(fabsf(y[2]), fabsf(y[3])));
+                        cp[4 * j] = y;
+                    }
+                } else if (want_max) {
 #pragma unroll
                     for (int j = 0; j < NT; ++j) {
                         const f32x4 y{(s * static_cast<float>(acc[j][0])) * rsc, (s * static_cast<float>(acc[j][1])) * rsc,
@@ -420,8 +452,17 @@ __global__ __launch_bounds__(64 * WAVES) void gemm_nts_kernel(const NtParams p, 
 #pragma unroll
         for (int st = 0; st < KS; ++st) cur[st] = nxt[st];
         rsc = rsc_nxt;
+        if (want_masked) {
+            mmul = mmul_nxt;
+#pragma unroll
+            for (int j = 0; j < BW; ++j) bw[j] = bw_nxt[j];
+        }
     }
     if (p.absmax_out) block_absmax_to_global(m / 127.0f, p.absmax_out);
+    if (want_masked) {
+        __syncthreads();  // the reduction above and this one share their LDS words
+        block_absmax_to_global(m2 / 127.0f, p.masked_absmax_out);
+    }
 }
 
 // NT kernel with the small operand stationary in registers, for wide fp32 outputs (257 to 960 columns) and
@@ -1477,6 +1518,14 @@ static bool launch_nts(const NtParams& p, hipStream_t s) {
                            static_cast<size_t>(NT_ * PASSES_) * (ksteps * 1024 + 64), s, p, ntiles);           \
         return true;                                                                                            \
     } while (0)
+    if constexpr (EPI == 3) {  // whole blocks of an even number of tiles only (the entry point admits no other shape)
+        if (two_rounds || ny != 1) return false;
+        if (nt == 2) TANGO_NTS(2, 1);
+        else if (nt == 4) TANGO_NTS(4, 1);
+        else if (nt == 8) TANGO_NTS(8, 1);
+        else if (nt == 16) TANGO_NTS(16, 1);
+        return false;
+    } else {
     if (two_rounds) {
         if (nt <= 24) TANGO_NTS(12, (EPI == 0 ? 2 : 1));
         else if (nt <= 32) TANGO_NTS(16, (EPI == 0 ? 2 : 1));
@@ -1487,6 +1536,7 @@ static bool launch_nts(const NtParams& p, hipStream_t s) {
     else if (nt <= 8) TANGO_NTS(8, 1);
     else if (nt <= 13) TANGO_NTS(13, 1);
     else TANGO_NTS(16, 1);
+    }
 #undef TANGO_NTS
 }
 
@@ -1512,16 +1562,18 @@ static bool launch_ntr(const NtParams& p, hipStream_t s) {
     return true;
 }
 
+// False when the masked maximum was asked for and the stationary kernel, the only one that finds it, could not run.
 template <int VEC>
-static void launch_nt_vec(const NtParams& p, hipStream_t s) {
+static bool launch_nt_vec(const NtParams& p, hipStream_t s) {
     const int64_t n16 = ceil_div(p.N, 16);
     const unsigned gx = static_cast<unsigned>(ceil_div(p.M, 128));
-    if (VEC == 16 && launch_ntr(p, s)) return;  // A rows in aligned 16-byte pieces
+    if (p.masked_absmax_out) return p.Kr <= 256 && VEC != 1 && launch_nts<VEC == 1 ? 4 : VEC, 3>(p, s);
+    if (VEC == 16 && launch_ntr(p, s)) return true;  // A rows in aligned 16-byte pieces
 #define TANGO_NT(NT_)                                                                             \
     hipLaunchKernelGGL((gemm_nt_kernel<NT_, VEC>), dim3(gx, static_cast<unsigned>(ceil_div(n16, NT_))), \
                        dim3(256), 0, s, p)
     if (p.Kr <= 256 && VEC != 1) {  // the small operand fits LDS: the stationary form
-        if (launch_nts<VEC == 1 ? 4 : VEC, 0>(p, s)) return;
+        if (launch_nts<VEC == 1 ? 4 : VEC, 0>(p, s)) return true;
     }
     if (n16 <= 1) TANGO_NT(1);
     else if (n16 <= 2) TANGO_NT(2);
@@ -1530,6 +1582,7 @@ static void launch_nt_vec(const NtParams& p, hipStream_t s) {
     else if (n16 <= 8) TANGO_NT(8);
     else TANGO_NT(16);
 #undef TANGO_NT
+    return true;
 }
 
 // B must already be packed (16-byte aligned rows, zero-filled to a multiple of 64 columns).
@@ -1541,10 +1594,8 @@ static int launch_nt(NtParams p, hipStream_t s, bool slot_zeroed = false) {
     int64_t readable = 0;
     const int vec = row_vec(p.A, p.lda, p.Kr, &readable);
     p.a_row_bytes = readable;
-    if (vec == 16) launch_nt_vec<16>(p, s);
-    else if (vec == 4) launch_nt_vec<4>(p, s);
-    else launch_nt_vec<1>(p, s);
-    return launch_status();
+    const bool done = vec == 16 ? launch_nt_vec<16>(p, s) : vec == 4 ? launch_nt_vec<4>(p, s) : launch_nt_vec<1>(p, s);
+    return done ? launch_status() : TANGO_ERR_LAUNCH;
 }
 
 // The fused forward needs: a deterministic rounding mode, K <= 768 (the 64 x K int8 block and
@@ -1834,6 +1885,36 @@ int tango_qgemm_bwd_dx_ex(float* dX, int64_t lddx, const int8_t* dYq, int64_t ld
     NtParams p{};
     p.C = dX; p.A = dYq; p.B = Wt; p.sA = s_dY; p.sB = s_W; p.row_scale = row_scale; p.accumulate = accumulate;
     p.M = M; p.N = K; p.Kr = N; p.lda = lddy; p.ldb = ldt; p.ldc = lddx;
+    return launch_nt(p, s);
+}
+
+int tango_qgemm_bwd_dx_masked(float* dX, int64_t lddx, const int8_t* dYq, int64_t lddy, const int8_t* Wq,
+                              int64_t ldw, const float* s_dY, const float* s_W, const float* row_scale,
+                              const uint16_t* mask_bits, int64_t ldmask, const float* mask_mul,
+                              float* masked_scale_out, int64_t M, int64_t N, int64_t K, void* workspace,
+                              size_t workspace_bytes, tango_stream_t stream) {
+    if (M < 0 || N < 0 || K < 0 || !s_dY || !s_W || lddx < K || lddy < N || ldw < K || !mask_bits ||
+        !masked_scale_out || ldmask < K / 16)
+        return TANGO_ERR_INVALID_ARG;
+    if ((M * K > 0 && !dX) || (M * N > 0 && !dYq) || (N * K > 0 && !Wq)) return TANGO_ERR_INVALID_ARG;
+    // the shapes whose launch is the stationary kernel over whole blocks of an even number of 16-column tiles
+    int64_t readable = 0;
+    const bool ok = (K == 32 || K == 64 || K == 128 || K == 256) && N >= 1 && N <= 256 && M > 0 &&
+                    row_vec(dYq, lddy, N, &readable) != 1 && (reinterpret_cast<uintptr_t>(dX) & 15) == 0 &&
+                    (lddx & 3) == 0 && (ldmask & 1) == 0 && (reinterpret_cast<uintptr_t>(mask_bits) & 3) == 0;
+    if (!ok) return TANGO_ERR_UNSUPPORTED;
+    const size_t need = tango_qgemm_bwd_dx_workspace(M, N, K);
+    if (need > 0 && (!workspace || workspace_bytes < need)) return TANGO_ERR_WORKSPACE;
+    if ((reinterpret_cast<uintptr_t>(workspace) & 15) != 0) return TANGO_ERR_INVALID_ARG;
+    hipStream_t s = as_stream(stream);
+    int8_t* Wt = static_cast<int8_t*>(workspace);
+    const int64_t ldt = round_up(N, 64);
+    hipLaunchKernelGGL(transpose_pack_i8_kernel, dim3(grid_for(K * ldt, 256)), dim3(256), 0, s, Wt, ldt, Wq, ldw, N, K);
+    fill_u32(masked_scale_out, 0u, 1, s);
+    NtParams p{};
+    p.C = dX; p.A = dYq; p.B = Wt; p.sA = s_dY; p.sB = s_W; p.row_scale = row_scale;
+    p.M = M; p.N = K; p.Kr = N; p.lda = lddy; p.ldb = ldt; p.ldc = lddx;
+    p.mask_bits = mask_bits; p.ldmask = ldmask; p.mask_mul = mask_mul; p.masked_absmax_out = masked_scale_out;
     return launch_nt(p, s);
 }
 

@@ -249,12 +249,13 @@ __device__ __forceinline__ void mask_bits4(float* mk, const uint16_t* __restrict
 // quantize_rows_kernel's job on dense matrices whose rows hold a multiple of four columns (x, q and the
 // mask all [rows, cols] without padding): the flat walk of quantize_vec_kernel, a lane's four elements
 // never straddle a row, and the row index (for row_mul) advances by a fixed step per iteration.
-template <int MODE>
+template <int MODE, bool COLSUM = false>
 __global__ __launch_bounds__(256) void quantize_dense_ex_kernel(
     const float* __restrict__ x, int64_t n4, int64_t cols, const float* __restrict__ scale,
     int8_t* __restrict__ q, const float* __restrict__ noise, uint64_t seed, uint64_t offset_host,
     const uint64_t* __restrict__ offset_dev,
-    const float* __restrict__ row_mul, const float* __restrict__ mask, int mask_mode) {
+    const float* __restrict__ row_mul, const float* __restrict__ mask, int mask_mode,
+    float* __restrict__ colsum_partial /* null, or [gridDim.x, cols]: needs 256 % (cols / 4) == 0 */) {
     const uint64_t offset = offset_host + (offset_dev ? offset_dev[0] : 0);
     const int64_t tid = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
     const int64_t nthr = static_cast<int64_t>(gridDim.x) * blockDim.x;
@@ -265,26 +266,41 @@ __global__ __launch_bounds__(256) void quantize_dense_ex_kernel(
     const bool shared_block = (offset & 3) == 0;
     int64_t row = (4 * tid) / cols, col = (4 * tid) % cols;
     const int64_t srow = (4 * nthr) / cols, scol = (4 * nthr) % cols;
+    // column sums of the masked input (before the row multiplier): with a number of threads that is a multiple of
+    // cols / 4 a lane meets the same four columns in every iteration
+    float cs[4] = {0.f, 0.f, 0.f, 0.f};
+    // The sign word and the row multiplier of a vector are asked for together with the vector, without a branch
+    // around the loads (absent operands: some valid address, value unused): one memory round trip per iteration
+    // instead of three in a row.
+    const bool bits_mode = mask && mask_mode == 2;
+    const uint16_t* words = bits_mode ? reinterpret_cast<const uint16_t*>(mask) : reinterpret_cast<const uint16_t*>(x);
+    const float* rmp = row_mul ? row_mul : x;
     for (int64_t i = tid; i < n4; i += nthr) {
         const f32x4 v = __builtin_nontemporal_load(x4 + i);
+        const unsigned word = words[(4 * i) >> 4];  // dense rows of a multiple of 16 columns: element e lies in word e / 16
+        const float rm = rmp[row_mul ? row : 0];
         float f[4] = {v.x, v.y, v.z, v.w};
-        if (mask && mask_mode == 2) {  // dense rows of a multiple of 16 columns: element e lies in word e / 16
-            float mk[4];
-            mask_bits4(mk, reinterpret_cast<const uint16_t*>(mask), 4 * i);
+        if (bits_mode) {
+            const unsigned w = word >> ((4 * i) & 15);
 #pragma unroll
-            for (int k = 0; k < 4; ++k) f[k] = masked(f[k], mk[k], mask_mode);
+            for (int k = 0; k < 4; ++k) f[k] = ((w >> k) & 1u) ? f[k] : 0.0f;
         } else if (mask) {
             const f32x4 mk = __builtin_nontemporal_load(m4 + i);
             f[0] = masked(f[0], mk.x, mask_mode); f[1] = masked(f[1], mk.y, mask_mode);
             f[2] = masked(f[2], mk.z, mask_mode); f[3] = masked(f[3], mk.w, mask_mode);
         }
+        if (COLSUM) {
+#pragma unroll
+            for (int k = 0; k < 4; ++k) cs[k] += f[k];
+        }
         if (row_mul) {
-            const float rm = row_mul[row];
 #pragma unroll
             for (int k = 0; k < 4; ++k) f[k] = f[k] * rm;
             row += srow;
             col += scol;
-            if (col >= cols) { col -= cols; ++row; }
+            const bool wrap = col >= cols;
+            col -= wrap ? cols : 0;
+            row += wrap ? 1 : 0;
         }
         float u[4] = {0.f, 0.f, 0.f, 0.f};
         if (MODE == TANGO_ROUND_STOCHASTIC) {
@@ -305,6 +321,22 @@ __global__ __launch_bounds__(256) void quantize_dense_ex_kernel(
         }
         __builtin_nontemporal_store(pack4(quant_one<MODE>(f[0], r, u[0]), quant_one<MODE>(f[1], r, u[1]),
                                           quant_one<MODE>(f[2], r, u[2]), quant_one<MODE>(f[3], r, u[3])), q4 + i);
+    }
+    if (COLSUM) {  // the lanes of a column quad are threadIdx.x = quad, quad + cols / 4, ...: added in that order
+        __shared__ float red[256][4];
+#pragma unroll
+        for (int k = 0; k < 4; ++k) red[threadIdx.x][k] = cs[k];
+        __syncthreads();
+        const int quads = static_cast<int>(cols >> 2);
+        if (static_cast<int>(threadIdx.x) < quads) {
+            float a[4] = {0.f, 0.f, 0.f, 0.f};
+            for (int t = threadIdx.x; t < 256; t += quads)
+#pragma unroll
+                for (int k = 0; k < 4; ++k) a[k] += red[t][k];
+            float* prow = colsum_partial + static_cast<int64_t>(blockIdx.x) * cols + 4 * threadIdx.x;
+#pragma unroll
+            for (int k = 0; k < 4; ++k) prow[k] = a[k];
+        }
     }
 }
 
@@ -776,30 +808,32 @@ __global__ __launch_bounds__(256) void absmax_ex_kernel(
     block_absmax_to_global(m / 127.0f, scale_out);
 }
 
-// blockDim = (16, 16): 16 columns per block; thread (x, y) sums partial rows y, y + 16, ... with
-// four loads in flight; the sixteen sums of a column are then added in a fixed order.
-__global__ __launch_bounds__(256) void colsum_finish_kernel(const float* __restrict__ partial,
-                                                            int64_t nrows, int64_t cols,
-                                                            float* __restrict__ out) {
-    __shared__ float red[16][16];
+// blockDim = (16, 64): 16 columns per block; thread (x, y) sums partial rows y, y + 64, ... with four loads in
+// flight (a thousand lanes per block: the partial rows are few, and each step is one memory round trip); the
+// sixty-four sums of a column are then added in a fixed order.
+__global__ __launch_bounds__(1024) void colsum_finish_kernel(const float* __restrict__ partial,
+                                                             int64_t nrows, int64_t cols,
+                                                             float* __restrict__ out) {
+    constexpr int RY = 64;
+    __shared__ float red[RY][16];
     const int64_t c = static_cast<int64_t>(blockIdx.x) * 16 + threadIdx.x;
     float a0 = 0.0f, a1 = 0.0f, a2 = 0.0f, a3 = 0.0f;
     if (c < cols) {
         int64_t r = threadIdx.y;
-        for (; r + 48 < nrows; r += 64) {
+        for (; r + 3 * RY < nrows; r += 4 * RY) {
             a0 += partial[r * cols + c];
-            a1 += partial[(r + 16) * cols + c];
-            a2 += partial[(r + 32) * cols + c];
-            a3 += partial[(r + 48) * cols + c];
+            a1 += partial[(r + RY) * cols + c];
+            a2 += partial[(r + 2 * RY) * cols + c];
+            a3 += partial[(r + 3 * RY) * cols + c];
         }
-        for (; r < nrows; r += 16) a0 += partial[r * cols + c];
+        for (; r < nrows; r += RY) a0 += partial[r * cols + c];
     }
     red[threadIdx.y][threadIdx.x] = (a0 + a1) + (a2 + a3);
     __syncthreads();
     if (threadIdx.y == 0 && c < cols) {
         float s = 0.0f;
 #pragma unroll
-        for (int y = 0; y < 16; ++y) s += red[y][threadIdx.x];
+        for (int y = 0; y < RY; ++y) s += red[y][threadIdx.x];
         out[c] = s;
     }
 }
@@ -937,7 +971,7 @@ int tango_absmax_ex_f32(const float* x, int64_t rows, int64_t cols, int64_t ldx,
 #undef TANGO_AEX
 #undef TANGO_AEX_M
     if (colsum_out)
-        hipLaunchKernelGGL(colsum_finish_kernel, dim3(static_cast<unsigned>(ceil_div(cols, 16))), dim3(16, 16), 0,
+        hipLaunchKernelGGL(colsum_finish_kernel, dim3(static_cast<unsigned>(ceil_div(cols, 16))), dim3(16, 64), 0,
                            s, partial, static_cast<int64_t>(grid), cols, colsum_out);
     return launch_status();
 }
@@ -1000,7 +1034,7 @@ int tango_quantize_rows_ex_f32_i8(const float* x, int64_t rows, int64_t cols, in
         int rc = dispatch_mode(round_mode, [&](auto mode) {
             constexpr int M = decltype(mode)::value;
             hipLaunchKernelGGL(quantize_dense_ex_kernel<M>, dim3(grid_for(n4, 256)), dim3(256), 0, s, x, n4, cols, scale,
-                               q, noise, seed, offset, offset_dev, row_mul, mask, mask_mode);
+                               q, noise, seed, offset, offset_dev, row_mul, mask, mask_mode, static_cast<float*>(nullptr));
         });
         return rc != TANGO_OK ? rc : launch_status();
     }
@@ -1047,6 +1081,42 @@ int tango_quantize_rows_ex_f32_i8(const float* x, int64_t rows, int64_t cols, in
                                per_row, q, ldq, noise, seed, offset, offset_dev, row_mul, mask, ldm, gpr_log2, mask_mode);
     });
     return rc != TANGO_OK ? rc : launch_status();
+}
+
+size_t tango_quantize_rows_colsum_workspace(int64_t rows, int64_t cols) {
+    if (rows <= 0 || cols <= 0) return 0;
+    return static_cast<size_t>(grid_for(rows * (cols >> 2), 256)) * static_cast<size_t>(cols) * sizeof(float);
+}
+
+int tango_quantize_rows_colsum_f32_i8(const float* x, int64_t rows, int64_t cols, const float* row_mul,
+                                      const void* mask_, int mask_mode, const float* scale, int8_t* q,
+                                      int round_mode, const float* noise, uint64_t seed, uint64_t offset,
+                                      const uint64_t* offset_dev, float* colsum_out, void* workspace,
+                                      size_t workspace_bytes, tango_stream_t stream) {
+    const float* mask = static_cast<const float*>(mask_);  // 16-bit words in mode 2
+    if (rows < 0 || cols < 0 || !scale || !colsum_out || (rows * cols > 0 && (!x || !q))) return TANGO_ERR_INVALID_ARG;
+    if (mask_mode < 0 || mask_mode > 2 || round_mode < 0 || round_mode > 2) return TANGO_ERR_UNSUPPORTED;
+    // dense rows of 4, 8, ..., 1024 columns whose quads divide a workgroup's 256 lanes; sign words need whole words
+    const int64_t quads = cols >> 2;
+    if (rows == 0 || cols == 0 || (cols & 3) != 0 || quads > 256 || 256 % quads != 0 ||
+        (mask && mask_mode == 2 && (cols & 15) != 0) || (reinterpret_cast<uintptr_t>(x) & 15) != 0 ||
+        (reinterpret_cast<uintptr_t>(mask) & (mask_mode == 2 ? 1 : 15)) != 0 || (reinterpret_cast<uintptr_t>(q) & 3) != 0)
+        return TANGO_ERR_UNSUPPORTED;
+    const size_t need = tango_quantize_rows_colsum_workspace(rows, cols);
+    if (!workspace || workspace_bytes < need || (reinterpret_cast<uintptr_t>(workspace) & 3) != 0) return TANGO_ERR_WORKSPACE;
+    hipStream_t s = as_stream(stream);
+    const int64_t n4 = rows * quads;
+    const int grid = grid_for(n4, 256);
+    float* partial = static_cast<float*>(workspace);
+    int rc = dispatch_mode(round_mode, [&](auto mode) {
+        constexpr int M = decltype(mode)::value;
+        hipLaunchKernelGGL((quantize_dense_ex_kernel<M, true>), dim3(grid), dim3(256), 0, s, x, n4, cols, scale, q, noise,
+                           seed, offset, offset_dev, row_mul, mask, mask_mode, partial);
+    });
+    if (rc != TANGO_OK) return rc;
+    hipLaunchKernelGGL(colsum_finish_kernel, dim3(static_cast<unsigned>(ceil_div(cols, 16))), dim3(16, 64), 0, s,
+                       partial, static_cast<int64_t>(grid), cols, colsum_out);
+    return launch_status();
 }
 
 int tango_transpose_quant_f32_i8(const float* x, int64_t nrow, int64_t ncol, const float* scale,

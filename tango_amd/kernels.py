@@ -280,6 +280,38 @@ class cuda_kernels:
         _advance(offset_dev, advance)
 
     @staticmethod
+    def quantize_rows_colsum(out, inp, scale, round_mode=ROUND_RNE, noise=None, seed=0, offset=0, row_mul=None,
+                             mask=None, mask_mode="relu", advance=0):
+        """``quantize_rows`` on dense 2-D tensors that also returns the column sums of the masked input (before
+        ``row_mul``) from the same pass: the bias gradient of a caller that already holds the scale.  Returns the
+        sums, or None when the layout is not one the kernel takes (nothing has run then)."""
+        _need(out, torch.int8, "out")
+        _need(inp, torch.float32, "in")
+        _need(scale, torch.float32, "scale")
+        rows, cols = inp.shape
+        if tuple(out.shape) != (rows, cols) or cols % 4 or cols > 1024 or 256 % max(cols // 4, 1):
+            return None
+        if mask is not None:
+            if cuda_kernels._mask_ld(mask, mask_mode, inp, "quantize_rows_colsum") != (cols // 16 if mask_mode == "bits" else cols):
+                return None
+        if row_mul is not None:
+            _need(row_mul, torch.float32, "row_mul")
+        if noise is not None:
+            _need(noise, torch.float32, "noise")
+        colsum = torch.empty(cols, dtype=torch.float32, device=inp.device)
+        ws_bytes = _ws_bytes("tango_quantize_rows_colsum_workspace", rows, cols)
+        ws = _workspace(ws_bytes, inp.device)
+        offset, offset_dev = _split_offset(offset)
+        rc = _L.tango_quantize_rows_colsum_f32_i8(_ptr(inp), rows, cols, _ptr(row_mul), _ptr(mask), _MASK_MODES[mask_mode],
+                                                  scale.data_ptr(), _ptr(out), _mode(round_mode), _ptr(noise), int(seed),
+                                                  offset, _ptr(offset_dev), _ptr(colsum), _ptr(ws), ws_bytes, _stream())
+        if rc == -2:  # unsupported layout
+            return None
+        check(rc, "quantize_rows_colsum")
+        _advance(offset_dev, advance)
+        return colsum
+
+    @staticmethod
     def absmax_ex(inp, row_mul=None, mask=None, want_colsum=False, mask_mode="relu"):
         """(max|inp' * row_mul| / 127, column sums of inp' or None) in one read of a 2-D tensor (not in
         the reference); inp' = inp passed backwards through the activation whose output is ``mask``
@@ -413,8 +445,10 @@ class cuda_kernels:
                                    scaleB.data_ptr(), M, N, K, _ptr(ws), ws_bytes, _stream()), "QGEMM_i8")
 
     @staticmethod
-    def QGEMM_backward_gradX(dX, dY, W, scaledY, scaleW, row_scale=None, accumulate=False):
-        """``accumulate``: add the product to what dX holds instead of overwriting it."""
+    def QGEMM_backward_gradX(dX, dY, W, scaledY, scaleW, row_scale=None, accumulate=False, masked=None):
+        """``accumulate``: add the product to what dX holds instead of overwriting it.  ``masked`` = (sign words int16
+        [M, K / 16], row multiplier [M] or None): returns max|dX' * multiplier| / 127 with dX' = dX where its sign bit
+        is set, else 0 (None when the shape is not one the epilogue takes, and otherwise)."""
         _need(dX, torch.float32, "dX", contiguous=False)
         _need(dY, torch.int8, "dY", contiguous=False)
         _need(W, torch.int8, "W", contiguous=False)
@@ -428,6 +462,22 @@ class cuda_kernels:
         ws = _workspace(ws_bytes, dY.device)
         if row_scale is not None:
             _need(row_scale, torch.float32, "row_scale")
+        if masked is not None:
+            # also the scale of dX taken back through a ReLU (sign words) and multiplied row by row, from the epilogue
+            bits, mul = masked
+            _need(bits, torch.int16, "mask bits")
+            if mul is not None:
+                _need(mul, torch.float32, "mask multiplier")
+            if accumulate or K % 16 or tuple(bits.shape) != (M, K // 16) or (mul is not None and mul.numel() != M):
+                raise RuntimeError("QGEMM_backward_gradX: the mask must be int16 [M, K / 16] and excludes accumulate")
+            scale = torch.empty(1, dtype=torch.float32, device=dX.device)
+            rc = _L.tango_qgemm_bwd_dx_masked(_ptr(dX), _rows_view(dX, "dX"), _ptr(dY), _rows_view(dY, "dY"), _ptr(W),
+                                              _rows_view(W, "W"), scaledY.data_ptr(), scaleW.data_ptr(), _ptr(row_scale),
+                                              _ptr(bits), K // 16, _ptr(mul), scale.data_ptr(), M, N, K, _ptr(ws),
+                                              ws_bytes, _stream())
+            if rc != -2:  # -2: not a shape the masked epilogue takes; the plain call below runs instead
+                check(rc, "QGEMM_backward_gradX")
+                return scale
         check(_L.tango_qgemm_bwd_dx_ex(_ptr(dX), _rows_view(dX, "dX"), _ptr(dY), _rows_view(dY, "dY"),
                                        _ptr(W), _rows_view(W, "W"), scaledY.data_ptr(), scaleW.data_ptr(),
                                        _ptr(row_scale), int(bool(accumulate)), M, N, K, _ptr(ws), ws_bytes,
@@ -939,12 +989,15 @@ def mySDDMM_quantize_on_load(g, op, U, V, scaleU, scaleV, round_mode=ROUND_RNE):
     return out.squeeze(1) if U3 is not U else out
 
 
-def QGEMM_backward(dY, X, W, scaledY, scaleX, scaleW, X_need=True, W_need=True, x_row_scale=None, dX_acc=None):
+def QGEMM_backward(dY, X, W, scaledY, scaleX, scaleW, X_need=True, W_need=True, x_row_scale=None, dX_acc=None,
+                   dx_masked=None):
     """cuda/kernels.py:97-111.  ``dX_acc``: a gradient of X from another consumer; the input gradient is
     added to it in place (and it is returned) instead of going to a new tensor.
     When K is not a multiple of 32 (and above 32) the returned dX is the [M, K] view of a buffer whose rows are
     padded to 32 floats: not contiguous, and as a leaf's ``.grad`` it keeps the padded allocation alive; callers
-    that need dense storage call ``.contiguous()`` on it (one [M, K] copy)."""
+    that need dense storage call ``.contiguous()`` on it (one [M, K] copy).
+    ``dx_masked`` = (sign words, row multiplier or None) of the ReLU and row scaling that the consumer of dX will
+    apply to it: gradX's epilogue then also finds the scale of that product and leaves it on dX."""
     assert scaledY.is_cuda, "scaledY must be on GPU"
     assert dY.is_cuda, "dY must be on GPU"
     dX, dW = None, None
@@ -960,8 +1013,12 @@ def QGEMM_backward(dY, X, W, scaledY, scaleX, scaleW, X_need=True, W_need=True, 
             dX = torch.empty((X.size(0), ld), dtype=torch.float32, device=X.device)[:, :X.size(1)]
         else:
             dX = torch.empty(X.shape, dtype=torch.float32, device=X.device)
-        cuda_kernels.QGEMM_backward_gradX(dX, dY, W, scaledY, scaleW, row_scale=x_row_scale,
-                                          accumulate=dX_acc is not None)
+        masked_scale = cuda_kernels.QGEMM_backward_gradX(dX, dY, W, scaledY, scaleW, row_scale=x_row_scale,
+                                                         accumulate=dX_acc is not None,
+                                                         masked=dx_masked if dX_acc is None else None)
+        if masked_scale is not None:
+            # for the consumer that takes dX back through that ReLU (SPMM.masked_scale_hint)
+            dX._tango_masked_scale = (masked_scale, dx_masked[0], dx_masked[1], dX._version, dX.data_ptr())
     if W_need:
         assert X.is_cuda, "X must be on GPU"
         assert scaleX.is_cuda, "scaleX must be on GPU"

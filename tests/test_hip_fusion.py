@@ -586,3 +586,115 @@ def test_batchnorm_rejects_unsupported_shapes(K):
     assert L.tango_batchnorm_fwd_f32(p, p, p, p, None, p, p, p, 100, 4096, ctypes.c_float(1e-5), 1, p, 1 << 30, None) == -2
     assert L.tango_batchnorm_fwd_f32(p, p, p, p, None, p, p, p, 100, 8, ctypes.c_float(1e-5), 1, None, 0, None) == -4
     assert L.tango_batchnorm_fwd_f32(p, p, p, p, None, p, p, p, 0, 8, ctypes.c_float(1e-5), 1, None, 0, None) == 0
+
+
+
+def _sign_words(keep):
+    rows, cols = keep.shape
+    return np.ascontiguousarray(np.packbits(keep.reshape(rows, cols // 16, 16), axis=-1, bitorder="little").view(np.int16).reshape(rows, cols // 16))
+
+
+@pytest.mark.parametrize("M,N,Kc", [(3001, 41, 256), (1000, 64, 128), (517, 200, 64), (77, 16, 32), (300, 41, 48)])
+@pytest.mark.parametrize("with_mul", [True, False])
+def test_gradx_epilogue_finds_the_masked_scale(K, orc, M, N, Kc, with_mul):
+    """gradX whose epilogue also returns max|dX' * multiplier| / 127 (dX' = dX where its sign bit is set): the stored
+    dX is the oracle's, and the scale is the oracle's absmax over that dX with the mask and multiplier: what the
+    separate pass finds.  48 columns: not a width the epilogue takes, the wrapper falls back and returns None."""
+    rng = np.random.default_rng(M + N + Kc)
+    dYq = rng.integers(-127, 128, (M, N), dtype=np.int8)
+    Wq = rng.integers(-127, 128, (N, Kc), dtype=np.int8)
+    rs = (rng.random(M).astype(np.float32) + 0.5)
+    mul = (rng.random(M).astype(np.float32) + 0.25) if with_mul else None
+    keep = rng.random((M, Kc)) < 0.5
+    bits = _sign_words(keep)
+    s_dY, s_W = np.float32(0.013), np.float32(0.0021)
+    dq = torch.zeros((M, (N + 15) // 16 * 16), dtype=torch.int8, device="cuda")[:, :N]
+    dq.copy_(dev(dYq))
+    dX = torch.full((M, Kc), float("nan"), device="cuda")
+    got = K.cuda_kernels.QGEMM_backward_gradX(dX, dq, dev(Wq), sc(s_dY), sc(s_W), row_scale=dev(rs),
+                                              masked=(dev(bits), None if mul is None else dev(mul)))
+    want = orc.qgemm_bwd_dx_ex(dYq, Wq, s_dY, s_W, row_scale=rs)
+    assert np.array_equal(host(dX), want)
+    if Kc == 48:
+        assert got is None
+        return
+    s_want, _ = orc.absmax_ex(want, row_mul=mul, mask=bits, mask_mode="bits")
+    assert host(got)[0] == s_want
+    # the pass it replaces agrees
+    s_pass, _ = K.cuda_kernels.absmax_ex(dX, row_mul=None if mul is None else dev(mul), mask=dev(bits), mask_mode="bits")
+    assert torch.equal(got, s_pass)
+
+
+@pytest.mark.parametrize("rows,cols", [(3001, 256), (999, 64), (70, 16), (2000, 1024), (500, 48)])
+def test_quantize_pass_returns_the_column_sums(K, orc, rows, cols):
+    """The dense quantize pass that also sums the masked input per column: same bytes as the plain pass (every rounding
+    mode, sign-word and fp32 masks, with and without the row multiplier), sums against float64; 48 columns: not a width
+    it takes (returns None, nothing written)."""
+    rng = np.random.default_rng(rows + cols)
+    x = (rng.standard_normal((rows, cols)) * 2).astype(np.float32)
+    rm = rng.random(rows).astype(np.float32) + 0.5
+    keep = rng.random((rows, cols)) < 0.6
+    bits = _sign_words(keep)
+    fmask = np.where(keep, 1.0, -1.0).astype(np.float32)
+    masked = np.where(keep, x, 0).astype(np.float32)
+    s, _ = orc.absmax_ex(x, row_mul=rm, mask=bits, mask_mode="bits")
+    for mask_d, mode_name in ((dev(bits), "bits"), (dev(fmask), "relu"), (None, "relu")):
+        ref = masked if mask_d is not None else x
+        for rmul in (dev(rm), None):
+            for kw, okw in (({}, dict(mode=orc.RNE)), ({"round_mode": "trunc"}, dict(mode=orc.TRUNC)),
+                            ({"round_mode": "stochastic", "seed": 9, "offset": 128}, dict(mode=orc.STOCHASTIC, seed=9, offset=128)),
+                            ({"round_mode": "stochastic", "seed": 9, "offset": 131}, dict(mode=orc.STOCHASTIC, seed=9, offset=131))):
+                out = torch.full((rows, cols), 77, dtype=torch.int8, device="cuda")
+                cs = K.cuda_kernels.quantize_rows_colsum(out, dev(x), sc(s), row_mul=rmul, mask=mask_d, mask_mode=mode_name, **kw)
+                if cols == 48:
+                    assert cs is None and bool((out == 77).all())
+                    continue
+                want = orc.quantize_rows_ex(x, s, row_mul=None if rmul is None else rm, mask=None if mask_d is None else bits,
+                                            mask_mode="bits", **okw)
+                assert np.array_equal(host(out), want), (mode_name, kw)
+                assert np.allclose(host(cs), ref.astype(np.float64).sum(0), rtol=1e-5, atol=2e-3)
+    if cols != 48:
+        a = K.cuda_kernels.quantize_rows_colsum(torch.empty((rows, cols), dtype=torch.int8, device="cuda"), dev(x), sc(s))
+        b = K.cuda_kernels.quantize_rows_colsum(torch.empty((rows, cols), dtype=torch.int8, device="cuda"), dev(x), sc(s))
+        assert torch.equal(a, b)  # a fixed order of additions
+
+
+def test_gcn_backward_takes_the_scale_from_gradx(monkeypatch):
+    """Two fused GCN layers: the second layer's gradX hands the first layer's aggregation the scale of the masked,
+    row-scaled gradient, and the bias gradient comes out of the quantize pass: no reducing pass over that gradient
+    runs, and every gradient is the same as without the hand-off, bit for bit."""
+    from tango_amd import SPMM, config, kernels
+    from tango_amd.gcn import GCN
+    from tango_amd.graph import Graph
+    from tango_amd.util import graph_preprocess
+    rng = np.random.default_rng(31)
+    n, e = 3000, 40000
+    src, dst = rand_graph(rng, n, e)
+    g = graph_preprocess(Graph(dev(np.concatenate([src, np.arange(n)])), dev(np.concatenate([dst, np.arange(n)])), n))
+    x = dev(rng.standard_normal((n, 96)).astype(np.float32))
+    labels = dev(rng.integers(0, 7, n))
+    torch.manual_seed(3)
+    model = GCN(g, 96, 64, 7, 1, torch.relu, 0.0).cuda()
+    config.grad_round_mode = "rne"
+    calls = []
+    real = kernels.cuda_kernels.absmax_ex
+    monkeypatch.setattr(kernels.cuda_kernels, "absmax_ex",
+                        staticmethod(lambda *a, **k: (calls.append(k.get("mask") is not None), real(*a, **k))[1]))
+
+    def grads(hand_off):
+        calls.clear()
+        if not hand_off:
+            monkeypatch.setattr(SPMM, "relu_mask_of", lambda t: None)
+        model.zero_grad()
+        torch.nn.functional.cross_entropy(model(x), labels).backward()
+        return [p.grad.clone() for p in model.parameters()], sum(calls)
+
+    with_, masked_passes = grads(True)
+    assert masked_passes == 0
+    without, masked_passes = grads(False)
+    assert masked_passes == 1
+    for a, b in zip(with_, without):
+        if a.dim() == 1:  # bias gradients: the two passes add the rows in different orders
+            assert torch.allclose(a, b, rtol=1e-5, atol=1e-6)
+        else:
+            assert torch.equal(a, b)
