@@ -1412,6 +1412,194 @@ __global__ __launch_bounds__(256, 2) void gemm_tn_kernel(const TnParams p) {
         }
 }
 
+// The same tile and slab layout with the operands staged by global-to-LDS loads into a ring of four steps (rows
+// readable in aligned 16-byte chunks only).  The loop above pays one memory round trip per 64-row step: its loads
+// are asked for one step ahead, land in registers and go through LDS store instructions and a second barrier.  Here
+// a step's 16 KB are asked for three steps ahead, land in LDS by themselves, and a step is: wait for the oldest
+// loads (s_waitcnt vmcnt(8): two younger steps stay in flight), one barrier, ask for step s + 3 into the stage that
+// step s - 1 just left, fragments, matrix instructions.  Each stage is an LDS object of its own, so that the
+// compiler does not make the fragment reads of one wait for the loads into another.
+// LDS rows have a pitch of exactly 128 bytes (a wave's load instruction lands 64 x 16 bytes back to back); what the
+// odd pitch of the loop above does for the banks, an XOR of the 16-byte chunk index with 4 * (row / 16 % 2) does
+// here: lane L of a load instruction fills LDS chunk L, so it asks global memory for the chunk that belongs there.
+// 64 lanes x 16 bytes from the lanes' global addresses to 1 KB of LDS starting at a wave-uniform address.  As
+// assembly, not as the compiler's builtin: the compiler makes every later LDS read of the kernel wait for all such
+// loads in flight at some joins of the loop (it cannot tell the ring's stages apart there), which would undo the
+// ring; the kernel's own s_waitcnt instructions order these loads instead.  M0 carries the LDS address and is not
+// used by anything else in the kernel.
+__device__ __forceinline__ void load_to_lds_16(const void* gptr, void* lds_wave_base) {
+    const unsigned lds = static_cast<unsigned>(
+        reinterpret_cast<uintptr_t>((__attribute__((address_space(3))) void*)lds_wave_base));  // generic -> LDS offset
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(lds), "v"(gptr) : "memory");
+}
+
+__global__ __launch_bounds__(256, 2) void gemm_tn_dma_kernel(const TnParams p) {
+    // a stage: the A tile, then the B tile, [64 rows][32 dwords] each
+    __shared__ uint32_t st0[4096], st1[4096], st2[4096], st3[4096];
+    uint32_t* const sA0 = st0; uint32_t* const sB0 = st0 + 2048;
+    uint32_t* const sA1 = st1; uint32_t* const sB1 = st1 + 2048;
+    uint32_t* const sA2 = st2; uint32_t* const sB2 = st2 + 2048;
+    uint32_t* const sA3 = st3; uint32_t* const sB3 = st3 + 2048;
+
+    const int nblk = gridDim.x;
+    int bid = blockIdx.x;
+    if ((nblk & 7) == 0) bid = (bid & 7) * (nblk >> 3) + (bid >> 3);  // tiles that share an M-chunk on one XCD
+    const int tiles = p.tiles_n * p.tiles_k;
+    const int split = bid / tiles;
+    const int tile = bid - split * tiles;
+    const int tn = tile / p.tiles_k, tk = tile - tn * p.tiles_k;
+    const int64_t n0 = static_cast<int64_t>(tn) * 128, k0 = static_cast<int64_t>(tk) * 128;
+    const int64_t m_begin = static_cast<int64_t>(split) * p.chunk;
+    const int64_t m_end = (m_begin + p.chunk < p.M) ? m_begin + p.chunk : p.M;
+    const int64_t steps = (m_end - m_begin) >> 6;  // whole 64-row steps; a last partial one goes through registers
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wn = wave >> 1, wk = wave & 1;
+    const int g = lane >> 4, r16 = lane & 15;
+
+    // this lane's two chunks per operand and step: LDS chunk P = tid + 256 i holds row P / 8, logical chunk
+    // (P % 8) ^ swizzle; columns beyond the readable row bytes re-read the row's last chunk (they only reach outputs
+    // that are not stored)
+    int64_t a_off[2], b_off[2];
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+        const int P = tid + 256 * i, row = P >> 3;
+        const int lc = (P & 7) ^ (4 * ((row >> 4) & 1));
+        int64_t ca = n0 + 16 * lc, cb = k0 + 16 * lc;
+        if (ca > p.a_row_bytes - 16) ca = p.a_row_bytes - 16;
+        if (cb > p.b_row_bytes - 16) cb = p.b_row_bytes - 16;
+        a_off[i] = row * p.lda + ca;
+        b_off[i] = row * p.ldb + cb;
+    }
+    auto issue = [&](uint32_t* dA, uint32_t* dB, int64_t step) {
+        const int64_t m0 = m_begin + (step < steps ? step : steps - 1) * 64;  // past the end: some valid rows, never read
+        const int8_t* ga = p.A + m0 * p.lda;
+        const int8_t* gb = p.B + m0 * p.ldb;
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+            load_to_lds_16(ga + a_off[i], dA + (i * 256 + wave * 64) * 4);
+            load_to_lds_16(gb + b_off[i], dB + (i * 256 + wave * 64) * 4);
+        }
+    };
+
+    i32x4 acc[4][4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[i][j] = i32x4{0, 0, 0, 0};
+
+    // A step's fragments are read from LDS one step ahead, as the raw dwords of sixteen rows per operand, while
+    // the matrix instructions of the current step run; the byte transposes that turn them into fragments follow
+    // those instructions.  (With the reads, the transposes and the matrix instructions of one step in a row, a
+    // wave spends a step waiting for each in turn, and two waves per SIMD do not cover that.)
+    uint32_t rawA[16], rawB[16];
+    i32x4 fa[4], fb[4];
+    const int cA = (wn * 16 + r16) ^ (16 * (g & 1));  // rows 16 g .. 16 g + 15 sit behind the swizzle of row / 16 % 2
+    const int cB = (wk * 16 + r16) ^ (16 * (g & 1));
+    auto read_raw = [&](const uint32_t* la, const uint32_t* lb) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            rawA[r] = la[(g * 16 + r) * 32 + cA];
+            rawB[r] = lb[(g * 16 + r) * 32 + cB];
+        }
+    };
+    // four fragments (sub-tiles j = 0..3) of the wave's 64 columns per operand (see gemm_tn_kernel)
+    auto transpose_raw = [&]() {
+        uint32_t col[4][4];
+#pragma unroll
+        for (int mb = 0; mb < 4; ++mb) transpose4x4(rawA[4 * mb], rawA[4 * mb + 1], rawA[4 * mb + 2], rawA[4 * mb + 3], col[mb]);
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+            fa[j] = i32x4{static_cast<int>(col[0][j]), static_cast<int>(col[1][j]),
+                          static_cast<int>(col[2][j]), static_cast<int>(col[3][j])};
+#pragma unroll
+        for (int mb = 0; mb < 4; ++mb) transpose4x4(rawB[4 * mb], rawB[4 * mb + 1], rawB[4 * mb + 2], rawB[4 * mb + 3], col[mb]);
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+            fb[j] = i32x4{static_cast<int>(col[0][j]), static_cast<int>(col[1][j]),
+                          static_cast<int>(col[2][j]), static_cast<int>(col[3][j])};
+    };
+    auto multiply = [&]() {
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+#pragma unroll
+            for (int j = 0; j < 4; ++j) acc[i][j] = mfma_16x16x64(fa[i], fb[j], acc[i][j]);
+    };
+
+    if (steps > 0) {
+        issue(sA0, sB0, 0);
+        issue(sA1, sB1, 1);
+        issue(sA2, sB2, 2);
+        // step 0's fragments
+        __builtin_amdgcn_s_waitcnt(0x0F78);  // vmcnt(8): step 0 has landed
+        __builtin_amdgcn_s_barrier();
+        asm volatile("" ::: "memory");
+        read_raw(sA0, sB0);
+        transpose_raw();
+// Step s_ (fragments in registers): steps s_ and s_ + 1 have landed when four younger loads remain (vmcnt(4)); after
+// the barrier every wave's have, and every wave is done reading stage s_ - 1.  Ask for step s_ + 3 into that stage,
+// read step s_ + 1's raw rows (NA, NB: the next stage), multiply step s_, then transpose for the next step.
+// (A bare barrier: __syncthreads() carries a release fence that waits for every load in flight, which is exactly
+// what the ring is there to avoid.)  The last step reads a stage that holds rows of an earlier step: not used.
+#define TANGO_TN_STEP(NA, NB, FA, FB, s_)          \
+        asm volatile("" ::: "memory");             \
+        __builtin_amdgcn_s_waitcnt(0x0F74);        \
+        __builtin_amdgcn_s_barrier();              \
+        asm volatile("" ::: "memory");             \
+        issue(FA, FB, (s_) + 3);                   \
+        read_raw(NA, NB);                          \
+        multiply();                                \
+        transpose_raw()
+        for (int64_t s = 0; s < steps; s += 4) {
+            TANGO_TN_STEP(sA1, sB1, sA3, sB3, s);
+            if (s + 1 >= steps) break;
+            TANGO_TN_STEP(sA2, sB2, sA0, sB0, s + 1);
+            if (s + 2 >= steps) break;
+            TANGO_TN_STEP(sA3, sB3, sA1, sB1, s + 2);
+            if (s + 3 >= steps) break;
+            TANGO_TN_STEP(sA0, sB0, sA2, sB2, s + 3);
+        }
+#undef TANGO_TN_STEP
+        __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): nothing lands in LDS behind this point
+        __syncthreads();
+    }
+    const int64_t m_tail = m_begin + steps * 64;
+    if (m_tail < m_end) {  // the rows of a last partial step, through registers, zeros beyond the end
+        const int srow = tid >> 3, scol = tid & 7;
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            const int row = srow + 32 * h;
+            const int64_t m = m_tail + row;
+            const bool mok = m < m_end;
+            const int64_t ca = n0 + scol * 16, cb = k0 + scol * 16;
+            const i32x4 ra = load16<16>(p.A + m * p.lda + ca, (mok && ca < p.N) ? p.a_row_bytes - ca : 0);
+            const i32x4 rb = load16<16>(p.B + m * p.ldb + cb, (mok && cb < p.K) ? p.b_row_bytes - cb : 0);
+            const int pc = scol ^ (4 * ((row >> 4) & 1));
+            *reinterpret_cast<i32x4*>(sA0 + row * 32 + pc * 4) = ra;
+            *reinterpret_cast<i32x4*>(sB0 + row * 32 + pc * 4) = rb;
+        }
+        __syncthreads();
+        read_raw(sA0, sB0);
+        transpose_raw();
+        multiply();
+    }
+
+    // acc[i][j][v] at lane (g, r16): n = n0 + 64 wn + 4 (4 g + v) + i, k = k0 + 64 wk + 4 r16 + j (see gemm_tn_kernel)
+    int* slab = p.acc + static_cast<int64_t>(split) * p.N * p.Kp;
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int v = 0; v < 4; ++v) {
+            const int64_t n = n0 + wn * 64 + 4 * (4 * g + v) + i;
+            const int64_t k = k0 + wk * 64 + 4 * r16;
+            if (n < p.N && k < p.Kp)
+                *reinterpret_cast<i32x4*>(slab + n * p.Kp + k) =
+                    i32x4{acc[i][0][v], acc[i][1][v], acc[i][2][v], acc[i][3][v]};
+        }
+}
+
 // dW[n, k] = (sA * sB) * float(sum over splits of part[split][n][k]).  A workgroup is 16 column
 // quads x 16 split lanes: the split lanes add every 16th slab, LDS adds the sixteen.
 __global__ __launch_bounds__(256) void tn_reduce_kernel(float* __restrict__ out, int64_t ldo,
@@ -1932,20 +2120,28 @@ struct TnPlan {
     int64_t splits, chunk, Kp;
 };
 
-static TnPlan tn_plan(int64_t M, int64_t N, int64_t K) {
+static TnPlan tn_plan(int64_t M, int64_t N, int64_t K, int64_t workgroups = 768) {
     TnPlan t{};
     t.tiles_n = static_cast<int>(ceil_div(N, 128));
     t.tiles_k = static_cast<int>(ceil_div(K, 128));
     t.Kp = round_up(K, 4);
     const int64_t tiles = static_cast<int64_t>(t.tiles_n) * t.tiles_k;
-    // enough workgroups for ~3 per CU, each with at least 4 reduction steps ...
-    int64_t splits = ceil_div(768, tiles);
+    // enough workgroups for `workgroups` / 256 per CU, each with at least 4 reduction steps ...
+    int64_t splits = workgroups == 768 ? ceil_div(workgroups, tiles) : workgroups / tiles;  // the ring kernel: no partial second round
     const int64_t max_splits = ceil_div(M, 256);
     if (splits > max_splits) splits = max_splits;
     // ... but the slabs (written once, read once, 4 bytes each way) stay below the operand bytes
     const int64_t by_traffic = M * (N + K) / (8 * N * t.Kp);
     if (splits > by_traffic) splits = by_traffic;
     if (splits < 1) splits = 1;
+    if (workgroups != 768) {
+        // A number of workgroups that is a multiple of eight: the kernel then gives each XCD a contiguous range of
+        // them, so that the tiles that share a chunk of rows meet in one L2 (232,965 x 256 x 602: 71 us with 480
+        // workgroups, 128 us with 510)
+        int64_t s8 = splits;
+        while (s8 > 1 && (s8 * tiles) % 8 != 0) --s8;
+        if ((s8 * tiles) % 8 == 0) splits = s8;
+    }
     t.chunk = round_up(ceil_div(M, splits), 64);
     t.splits = M > 0 ? ceil_div(M, t.chunk) : 0;
     return t;
@@ -1970,7 +2166,12 @@ int tango_qgemm_bwd_dw(float* dW, int64_t lddw, const int8_t* dYq, int64_t lddy,
     if ((reinterpret_cast<uintptr_t>(workspace) & 15) != 0) return TANGO_ERR_INVALID_ARG;
     hipStream_t s = as_stream(stream);
     int* acc = static_cast<int*>(workspace);
-    const TnPlan t = tn_plan(M, N, K);
+    int64_t ra = 0, rb = 0;
+    const int va = row_vec(dYq, lddy, N, &ra), vb = row_vec(Xq, ldx, K, &rb);
+    const int vec = va < vb ? va : vb;
+    // the ring kernel holds 64 KB of LDS per workgroup, two per CU: fewer, longer splits than the workspace was
+    // sized for (never more)
+    const TnPlan t = vec == 16 ? tn_plan(M, N, K, 512) : tn_plan(M, N, K);
     if (M > 0) {
         TnParams p{};
         p.acc = acc; p.Kp = t.Kp; p.A = dYq; p.B = Xq; p.M = M; p.N = N; p.K = K; p.lda = lddy; p.ldb = ldx;
@@ -1980,13 +2181,10 @@ int tango_qgemm_bwd_dw(float* dW, int64_t lddw, const int8_t* dYq, int64_t lddy,
         p.chunk = t.chunk;
         p.splits = static_cast<int>(t.splits);
         if (tiles * t.splits > INT32_MAX) return TANGO_ERR_UNSUPPORTED;
-        int64_t ra = 0, rb = 0;
-        const int va = row_vec(dYq, lddy, N, &ra), vb = row_vec(Xq, ldx, K, &rb);
-        const int vec = va < vb ? va : vb;
         p.a_row_bytes = (vec == 16) ? round_up(N, 16) : (vec == 4 ? round_up(N, 4) : N);
         p.b_row_bytes = (vec == 16) ? round_up(K, 16) : (vec == 4 ? round_up(K, 4) : K);
         const dim3 grid(static_cast<unsigned>(tiles * t.splits));
-        if (vec == 16) hipLaunchKernelGGL(gemm_tn_kernel<16>, grid, dim3(256), 0, s, p);
+        if (vec == 16) hipLaunchKernelGGL(gemm_tn_dma_kernel, grid, dim3(256), 0, s, p);
         else if (vec == 4) hipLaunchKernelGGL(gemm_tn_kernel<4>, grid, dim3(256), 0, s, p);
         else hipLaunchKernelGGL(gemm_tn_kernel<1>, grid, dim3(256), 0, s, p);
     }
