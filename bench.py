@@ -133,7 +133,7 @@ def mfma_probe(torch, iters=4000):
     """Sustained rate of the int8 matrix instructions (register-resident chains, 32 wavefronts per CU)."""
     from tango_amd import _lib
     L = _lib.lib()
-    sink = torch.zeros(1, dtype=torch.int32, device="cuda")
+    sink = torch.zeros(64 + 65536, dtype=torch.int32, device="cuda")  # the result word, then a source for the staged probe
     st = torch.cuda.current_stream().cuda_stream
     cus = torch.cuda.get_device_properties(0).multi_processor_count
     blocks = cus * 8
@@ -145,7 +145,9 @@ def mfma_probe(torch, iters=4000):
               # the bit-block kernel's inner loop without global loads (64 instructions per round), without / with
               # the LDS writes and the barrier that end a unit; two workgroups per CU
               (5, "32x32x32_loop", 2 * 32 * 32 * 32), (6, "32x32x32_loop_write_barrier", 2 * 32 * 32 * 32),
-              (7, "32x32x32_loop_barrier", 2 * 32 * 32 * 32))
+              (7, "32x32x32_loop_barrier", 2 * 32 * 32 * 32),
+              # ... and with the next chunk staged by global-to-LDS loads from a cached buffer (sink: 256 B + 256 KB)
+              (8, "32x32x32_loop_lds_loads_barrier", 2 * 32 * 32 * 32))
     for shape, name, ops in shapes:
         nb, it, per = (blocks, iters, 8) if shape < 5 else (cus * 2, iters // 8, 64)
         ms = time_op(lambda: _lib.check(L.tango_probe_mfma_i8(shape, it, nb, sink.data_ptr(), st), "probe"),

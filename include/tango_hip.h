@@ -47,10 +47,15 @@ const char* tango_status_string(int status);
 /* ABI version; bumped when a signature changes. */
 int tango_abi_version(void);
 
-/* Measurement probe (no counterpart in the reference): `blocks` workgroups of four wavefronts each run
-   `iters` rounds of eight independent chains of one int8 matrix instruction out of registers; shape 0:
-   16x16x64 (2 * 16 * 16 * 64 operations each), shape 1: 32x32x32 (2 * 32 * 32 * 32).  The rate of such a launch
-   is what the matrix cores of the device sustain; sink: one int of device memory, never written in practice. */
+/* Measurement probes (no counterpart in the reference): `blocks` workgroups of four wavefronts.  Shapes 0 and 1:
+   `iters` rounds of eight independent chains of one int8 matrix instruction out of registers, 16x16x64
+   (2 * 16 * 16 * 64 operations each) and 32x32x32 (2 * 32 * 32 * 32): what the matrix cores of the device sustain.
+   Shapes 2, 3, 4: 32x32x32 with the first operand expanded from a word of bits (a shift and a mask per register)
+   in front of every 1, 2, 4 instructions.  Shapes 5 .. 8: `iters` rounds of the bit-block kernel's inner loop (64
+   instructions of 32x32x32 per wavefront and round, fragments read from 64 KB of LDS): 5 as is, 6 with the LDS store
+   instructions of a register-staged chunk and a barrier per round, 7 with the barrier alone, 8 with the chunk
+   staged by global-to-LDS loads and the barrier.  sink: device memory, one int (never written in practice); shape 8
+   reads the 256 KB that follow its first 256 bytes. */
 int tango_probe_mfma_i8(int shape, int iters, int blocks, int* sink, tango_stream_t stream);
 
 /* ------------------------------------------------------------ quantization */

@@ -1,7 +1,7 @@
 // Dense blocks of a power-law adjacency on the CDNA4 matrix cores (v_mfma_i32_32x32x32_i8).
 //
 // With rows and columns ranked by falling slot count, the cells (row rank i, column rank j) whose
-// expected density deg(i) * cnt(j) / nnz is above a few per cent form a staircase in the corner of the
+// expected density deg(i) * cnt(j) / nnz is above about one per cent form a staircase in the corner of the
 // adjacency that holds a third to a half of all edges of such a graph.  There one bit per cell and a
 // 0/1-byte x int8 matrix product cost less than one gathered 128-byte line per edge.  Per launch:
 //   dense_stage_kernel   gathers the ranked columns' feature rows and writes them transposed, in the
@@ -300,7 +300,7 @@ __global__ __launch_bounds__(256) void mfma_probe_kernel(int iters, int* sink) {
 // (two fragment reads from LDS, four operand expansions, eight matrix instructions); LEVEL 1 adds the LDS writes
 // and the workgroup barrier that end a unit.  blockDim.x = 256, dynamic LDS 64 KB.
 template <int LEVEL>
-__global__ __launch_bounds__(256, 2) void mfma_loop_probe_kernel(int iters, int* sink) {
+__global__ __launch_bounds__(256, 2) void mfma_loop_probe_kernel(int iters, int* sink, const int8_t* src = nullptr) {
     extern __shared__ __attribute__((aligned(16))) int8_t ring[];
     const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
     for (int i = t; i < 4096; i += 256) reinterpret_cast<i32x4*>(ring)[i] = i32x4{i, i + 1, i + 2, i + 3};
@@ -341,6 +341,14 @@ __global__ __launch_bounds__(256, 2) void mfma_loop_probe_kernel(int iters, int*
             int8_t* nbuf = ring + ((k + 1) & 1) * 32768;
 #pragma unroll
             for (int i = 0; i < 8; ++i) *reinterpret_cast<u32x4*>(nbuf + (i * 256 + t) * 16) = mw[i & 1][(i >> 1) & 1];
+        }
+        if (LEVEL == 3) {  // the next chunk by global-to-LDS loads from a small (cached) buffer, as the block kernel stages
+            int8_t* nbuf = ring + ((k + 1) & 1) * 32768;
+            const u32x4* x = reinterpret_cast<const u32x4*>(src) + ((k & 7) * 2048 + t);
+#pragma unroll
+            for (int i = 0; i < 8; ++i)
+                __builtin_amdgcn_global_load_lds(x + i * 256, reinterpret_cast<u32x4*>(nbuf) + i * 256 + (t >> 6) * 64, 16, 0, 0);
+            __builtin_amdgcn_s_waitcnt(0x0F70);
         }
         if (LEVEL >= 1) __syncthreads();
     }
@@ -411,7 +419,7 @@ using namespace tango;
 extern "C" {
 
 int tango_probe_mfma_i8(int shape, int iters, int blocks, int* sink, tango_stream_t stream) {
-    if (shape < 0 || shape > 7 || iters < 0 || blocks <= 0 || !sink) return TANGO_ERR_INVALID_ARG;
+    if (shape < 0 || shape > 8 || iters < 0 || blocks <= 0 || !sink) return TANGO_ERR_INVALID_ARG;
     hipStream_t s = as_stream(stream);
     switch (shape) {
         case 0: hipLaunchKernelGGL(mfma_probe_kernel<0>, dim3(blocks), dim3(256), 0, s, iters, sink); break;
@@ -419,9 +427,11 @@ int tango_probe_mfma_i8(int shape, int iters, int blocks, int* sink, tango_strea
         case 2: hipLaunchKernelGGL(mfma_probe_kernel<2>, dim3(blocks), dim3(256), 0, s, iters, sink); break;
         case 3: hipLaunchKernelGGL(mfma_probe_kernel<3>, dim3(blocks), dim3(256), 0, s, iters, sink); break;
         case 4: hipLaunchKernelGGL(mfma_probe_kernel<4>, dim3(blocks), dim3(256), 0, s, iters, sink); break;
-        case 5: hipLaunchKernelGGL(mfma_loop_probe_kernel<0>, dim3(blocks), dim3(256), 65536, s, iters, sink); break;
-        case 6: hipLaunchKernelGGL(mfma_loop_probe_kernel<1>, dim3(blocks), dim3(256), 65536, s, iters, sink); break;
-        default: hipLaunchKernelGGL(mfma_loop_probe_kernel<2>, dim3(blocks), dim3(256), 65536, s, iters, sink); break;
+        case 5: hipLaunchKernelGGL(mfma_loop_probe_kernel<0>, dim3(blocks), dim3(256), 65536, s, iters, sink, nullptr); break;
+        case 6: hipLaunchKernelGGL(mfma_loop_probe_kernel<1>, dim3(blocks), dim3(256), 65536, s, iters, sink, nullptr); break;
+        case 7: hipLaunchKernelGGL(mfma_loop_probe_kernel<2>, dim3(blocks), dim3(256), 65536, s, iters, sink, nullptr); break;
+        default: hipLaunchKernelGGL(mfma_loop_probe_kernel<3>, dim3(blocks), dim3(256), 65536, s, iters, sink,
+                                    reinterpret_cast<const int8_t*>(sink) + 256); break;
     }
     return launch_status();
 }

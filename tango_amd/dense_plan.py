@@ -2,14 +2,13 @@
 an extension of cuda/util.py:5-11 of the reference, which caches CSR / CSC / COO once per graph).
 
 On power-law graphs the cells (row i, column j) with expected density deg(i) * cnt(j) / nnz above a
-few per cent hold a large part of all edges.  With rows and columns ranked by falling slot count that
+percent or so hold a large part of all edges.  With rows and columns ranked by falling slot count that
 region is a staircase: row block b (256 consecutive row ranks) gets the columns of rank below
 ``extent[b]``.  Inside it an edge is one bit and the copy_u aggregation a 0/1 x int8 matrix product
 (tango_spmm_csr_copy_u_dense); everything else stays a CSR.  The split changes no result: integer
 sums are exact in any order.
 """
 import ctypes
-import heapq
 import os
 
 import numpy as np
@@ -23,9 +22,10 @@ UNIT = 256   # mask columns of a unit
 
 
 def default_tau():
-    """Density above which a cell is worth a bit (the matrix product costs about this fraction of a
-    gathered row per cell); TANGO_DENSE_TAU overrides, 0 switches the dense blocks off."""
-    return float(os.environ.get("TANGO_DENSE_TAU", "0.02"))
+    """Density above which a cell is worth a bit: a cell costs the matrix cores about 0.7 % of what a gathered
+    edge costs the gather kernel, at 64 columns as at 256 (measured on the 114.8 M-edge benchmark graph, where
+    0.007 .. 0.009 give the shortest epochs); TANGO_DENSE_TAU overrides, 0 switches the dense blocks off."""
+    return float(os.environ.get("TANGO_DENSE_TAU", "0.008"))
 
 
 class DensePlan:
@@ -123,7 +123,7 @@ def build_dense_plan(indptr, indices, num_src, tau=None, groups=256, sort_rest=T
     """Splits the CSR (indptr int64 [rows + 1], indices int32 / int64 [nnz], gathered rows < num_src).
     Returns a DensePlan, or None when fewer than ``min_share`` of the slots would become bits."""
     tau = default_tau() if tau is None else float(tau)
-    min_extent = int(os.environ.get("TANGO_DENSE_MIN_EXTENT", "2048")) if min_extent is None else int(min_extent)
+    min_extent = int(os.environ.get("TANGO_DENSE_MIN_EXTENT", "4096")) if min_extent is None else int(min_extent)
     min_extent = max(min_extent, UNIT)
     rows = indptr.numel() - 1
     nnz = indices.numel()
