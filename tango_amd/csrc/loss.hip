@@ -24,34 +24,48 @@ __global__ __launch_bounds__(256) void softmax_xent_kernel(
     const float inv_rows = 1.0f / static_cast<float>(rows);
     float loss = 0.0f;
     const int64_t step = static_cast<int64_t>(gridDim.x) * 4 * rpw;
-    for (int64_t row = (static_cast<int64_t>(blockIdx.x) * 4 + wave) * rpw + sub; row < rows; row += step) {
-        const float* x = logits + row * ld;
-        float v[4];
-        float mx = -INFINITY;
+    // Two rows per lane group in flight: the loads of both (and their labels) are asked for before either is used, from
+    // clamped addresses without a branch around them (a guarded load makes the wave wait at the join behind it).
+    constexpr int RU = 2;
+    for (int64_t row0 = (static_cast<int64_t>(blockIdx.x) * 4 + wave) * rpw + sub; row0 < rows; row0 += RU * step) {
+        float v[RU][4];
+        int64_t lab[RU];
 #pragma unroll
-        for (int k = 0; k < 4; ++k) {
-            const int c = l * 4 + k;
-            v[k] = c < C ? x[c] : -INFINITY;
-            mx = fmaxf(mx, v[k]);
+        for (int u = 0; u < RU; ++u) {
+            const int64_t row = row0 + u * step;
+            const int64_t rr = row < rows ? row : rows - 1;
+            const float* x = logits + rr * ld;
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+                const int c = l * 4 + k;
+                const float a = x[c < C ? c : C - 1];
+                v[u][k] = c < C ? a : -INFINITY;
+            }
+            lab[u] = labels[rr];
         }
-        for (int off = 1; off < gl; off <<= 1) mx = fmaxf(mx, __shfl_xor(mx, off, kWave));
-        float e[4], s = 0.0f;
 #pragma unroll
-        for (int k = 0; k < 4; ++k) {
-            e[k] = (l * 4 + k < C) ? expf(v[k] - mx) : 0.0f;
-            s += e[k];
-        }
-        for (int off = 1; off < gl; off <<= 1) s += __shfl_xor(s, off, kWave);
-        const int64_t lab = labels[row];
-        const float inv = 1.0f / s;
-        float* g = grad + row * ldg;
+        for (int u = 0; u < RU; ++u) {
+            const int64_t row = row0 + u * step;
+            float mx = fmaxf(fmaxf(v[u][0], v[u][1]), fmaxf(v[u][2], v[u][3]));
+            for (int off = 1; off < gl; off <<= 1) mx = fmaxf(mx, __shfl_xor(mx, off, kWave));
+            float e[4], s = 0.0f;
 #pragma unroll
-        for (int k = 0; k < 4; ++k) {
-            const int c = l * 4 + k;
-            if (c < C) {
-                const float p = e[k] * inv;
-                g[c] = (p - (c == lab ? 1.0f : 0.0f)) * inv_rows;
-                if (c == lab) loss += (logf(s) + mx) - v[k];  // -log softmax[label]
+            for (int k = 0; k < 4; ++k) {
+                e[k] = (l * 4 + k < C) ? expf(v[u][k] - mx) : 0.0f;
+                s += e[k];
+            }
+            for (int off = 1; off < gl; off <<= 1) s += __shfl_xor(s, off, kWave);
+            if (row >= rows) continue;  // after the shuffles: every lane of the wave takes part in them
+            const float inv = 1.0f / s;
+            float* g = grad + row * ldg;
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+                const int c = l * 4 + k;
+                if (c < C) {
+                    const float p = e[k] * inv;
+                    g[c] = (p - (c == lab[u] ? 1.0f : 0.0f)) * inv_rows;
+                    if (c == lab[u]) loss += (logf(s) + mx) - v[u][k];  // -log softmax[label]
+                }
             }
         }
     }

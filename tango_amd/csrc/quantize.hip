@@ -738,11 +738,13 @@ __global__ __launch_bounds__(256) void absmax_ex_kernel(
                             v[u][t][2 * h + 1] = (row < rows && c + 1 < cols) ? a[1] : 0.0f;
                         }
                     } else {
+                        const int cl = static_cast<int>(cols), cb = static_cast<int>(c0);  // cols <= 1024: 32-bit column math
+                        const bool rin = row < rows;
 #pragma unroll
                         for (int k = 0; k < 4; ++k) {
-                            const int64_t c = c0 + k;
-                            const float a = xr[c < cols ? c : cols - 1];
-                            v[u][t][k] = (row < rows && c < cols) ? a : 0.0f;
+                            const int c = cb + k;
+                            const float a = xr[c < cl ? c : cl - 1];
+                            v[u][t][k] = (rin && c < cl) ? a : 0.0f;
                         }
                     }
                     if (MK == 1) {
