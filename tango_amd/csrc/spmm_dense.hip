@@ -6,7 +6,7 @@
 // 0/1-byte x int8 matrix product cost less than one gathered 128-byte line per edge.  Per launch:
 //   dense_stage_kernel   gathers the ranked columns' feature rows and writes them transposed, in the
 //                        order the matrix instruction's second operand wants them (one KB per fragment);
-//   dense_zero_kernel    zeroes the partial sums of row blocks that several workgroups add into;
+//                        its last workgroups zero the partial sums of row blocks that several workgroups add into;
 //   dense_block_kernel   two persistent 4-wave workgroups per CU walk their segments (row block, range of
 //                        256-column units): a unit's staged features go from global memory straight into one
 //                        of two LDS chunks, the mask bits come straight from memory (one dword per lane and
@@ -35,6 +35,7 @@ struct DenseParams {
     int* part;       // [dense_rows][npad]
     int npad;
     int64_t units;   // dense_cols / 256
+    int64_t stage_groups;  // workgroups of the staging kernel that stage (64 columns each); the rest zero
 };
 
 // blockDim.x = 256; workgroup b stages mask columns 64 b .. 64 b + 63 (two k-steps of 32).
@@ -46,8 +47,17 @@ __global__ __launch_bounds__(256) void dense_stage_kernel(const DenseParams p) {
     constexpr int CPR = NPAD / 16;  // 16-byte chunks per staged row
     __shared__ __attribute__((aligned(16))) uint32_t tile[64 * (NPAD / 4)];
     const int t = threadIdx.x;
+    if (static_cast<int64_t>(blockIdx.x) >= p.stage_groups) {
+        // the workgroups behind the staging ones zero the partial sums of the row blocks that several workgroups
+        // of the block kernel add into (one launch less than a kernel of their own)
+        const int64_t rb = p.shared_blocks[blockIdx.x - p.stage_groups];
+        i32x4* dst = reinterpret_cast<i32x4*>(p.part + rb * kDenseRows * p.npad);
+        const int n = kDenseRows * p.npad / 4;
+        for (int i = t; i < n; i += 256) dst[i] = i32x4{0, 0, 0, 0};
+        return;
+    }
     const int64_t j0 = static_cast<int64_t>(blockIdx.x) * 64;
-    const int64_t ksteps = static_cast<int64_t>(gridDim.x) * 2;
+    const int64_t ksteps = p.stage_groups * 2;
     for (int c = t; c < 64 * CPR; c += 256) {
         const int r = c / CPR, cc = c - r * CPR;
         const int id = p.col_ids[j0 + r];
@@ -77,14 +87,6 @@ __global__ __launch_bounds__(256) void dense_stage_kernel(const DenseParams p) {
             *reinterpret_cast<u32x4*>(dst) = u32x4{c[0][i], c[1][i], c[2][i], c[3][i]};
         }
     }
-}
-
-// grid = shared row blocks; blockDim.x = 256.
-__global__ __launch_bounds__(256) void dense_zero_kernel(const DenseParams p) {
-    const int64_t rb = p.shared_blocks[blockIdx.x];
-    i32x4* dst = reinterpret_cast<i32x4*>(p.part + rb * kDenseRows * p.npad);
-    const int n = kDenseRows * p.npad / 4;
-    for (int i = threadIdx.x; i < n; i += 256) dst[i] = i32x4{0, 0, 0, 0};
 }
 
 // blockDim.x = 256 (4 waves), grid (groups, SPLIT): with one split the plan's finer table of segments is used
@@ -392,7 +394,8 @@ int launch_dense_block(const tango_spmm_dense_plan& plan, const int8_t* feat, in
     *part = p.part;
     *npad_out = npad;
     p.units = plan.dense_cols / kDenseUnit;
-    const dim3 sgrid(static_cast<unsigned>(plan.dense_cols / 64));
+    p.stage_groups = plan.dense_cols / 64;
+    const dim3 sgrid(static_cast<unsigned>(p.stage_groups + plan.num_shared));  // staging, then zeroing workgroups
 #define TANGO_DENSE(NPAD, NCTW, RW)                                                                              \
     do {                                                                                                     \
         constexpr int SPLIT = NPAD / (32 * NCTW);                                                            \
@@ -401,8 +404,6 @@ int launch_dense_block(const tango_spmm_dense_plan& plan, const int8_t* feat, in
         }                                                                                                    \
         const dim3 bgrid(static_cast<unsigned>(SPLIT == 1 ? plan.num_groups2 : plan.num_groups), SPLIT);     \
         hipLaunchKernelGGL((dense_stage_kernel<NPAD, NCTW>), sgrid, dim3(256), 0, s, p);                     \
-        if (plan.num_shared > 0)                                                                             \
-            hipLaunchKernelGGL(dense_zero_kernel, dim3(static_cast<unsigned>(plan.num_shared)), dim3(256), 0, s, p); \
         hipLaunchKernelGGL((dense_block_kernel<NCTW, SPLIT, RW>), bgrid, dim3(256), 0, s, p);                             \
     } while (0)
     if (npad == 64) TANGO_DENSE(64, 2, 2);
