@@ -1412,16 +1412,6 @@ __global__ __launch_bounds__(256, 2) void gemm_tn_kernel(const TnParams p) {
         }
 }
 
-// The same tile and slab layout with the operands staged by global-to-LDS loads into a ring of four steps (rows
-// readable in aligned 16-byte chunks only).  The loop above pays one memory round trip per 64-row step: its loads
-// are asked for one step ahead, land in registers and go through LDS store instructions and a second barrier.  Here
-// a step's 16 KB are asked for three steps ahead, land in LDS by themselves, and a step is: wait for the oldest
-// loads (s_waitcnt vmcnt(8): two younger steps stay in flight), one barrier, ask for step s + 3 into the stage that
-// step s - 1 just left, fragments, matrix instructions.  Each stage is an LDS object of its own, so that the
-// compiler does not make the fragment reads of one wait for the loads into another.
-// LDS rows have a pitch of exactly 128 bytes (a wave's load instruction lands 64 x 16 bytes back to back); what the
-// odd pitch of the loop above does for the banks, an XOR of the 16-byte chunk index with 4 * (row / 16 % 2) does
-// here: lane L of a load instruction fills LDS chunk L, so it asks global memory for the chunk that belongs there.
 // 64 lanes x 16 bytes from the lanes' global addresses to 1 KB of LDS starting at a wave-uniform address.  As
 // assembly, not as the compiler's builtin: the compiler makes every later LDS read of the kernel wait for all such
 // loads in flight at some joins of the loop (it cannot tell the ring's stages apart there), which would undo the
@@ -1433,8 +1423,29 @@ __device__ __forceinline__ void load_to_lds_16(const void* gptr, void* lds_wave_
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(lds), "v"(gptr) : "memory");
 }
 
-__global__ __launch_bounds__(256, 2) void gemm_tn_dma_kernel(const TnParams p) {
-    // a stage: the A tile, then the B tile, [64 rows][32 dwords] each
+// The same tile and slab layout as gemm_tn_kernel for rows readable in aligned 16-byte chunks, built around three
+// things that kernel lacks.  (1) The operands are staged by global-to-LDS loads into a ring of four 64-row steps:
+// gemm_tn_kernel pays one memory round trip per step (its loads are asked for one step ahead, land in registers
+// and go through LDS store instructions and a second barrier); here a step's 16 KB are asked for three steps ahead
+// and land in LDS by themselves, and a step is: wait for the loads of steps s and s + 1 (s_waitcnt vmcnt(4): the
+// youngest step stays in flight), one bare barrier (__syncthreads() carries a release fence that waits for every
+// load in flight, which is exactly what the ring is there to avoid), ask for step s + 3 into the stage that step
+// s - 1 left, read the operands of step s + 1, multiply step s.  Each stage is an LDS object of its own.
+// (2) The operands are read by the transposing LDS read, no byte transposes in registers.  ds_read_b64_tr_b8: within
+// sixteen lanes, lane j gives the address of an 8-byte block and lane i receives byte i % 8 of the blocks of lanes
+// i / 8, i / 8 + 2, ..., i / 8 + 14; with lane j pointing at row j / 2, bytes 8 (j % 2) .. of a 16-column strip, lane i
+// gets column i of eight consecutive rows: eight consecutive m of one n (or k), which is what a matrix operand
+// wants of a tile stored [m][n].  Two such reads are a lane's sixteen bytes of an operand of
+// (3) v_mfma_i32_32x32x32_i8 (lane l: row l % 32, reduction indices 16 (l / 32) .. + 15), which runs at 1.7 times the
+// rate of the 16 x 16 x 64 instruction on this device.
+// LDS rows have a pitch of exactly 128 bytes (a wave's load instruction lands 64 x 16 bytes back to back); the
+// 16-byte chunk index is XORed with row % 8, so that the eight rows of a transposing read sit in eight different
+// chunks (all 32 banks): lane L of a load instruction fills LDS chunk L, so it asks global memory for the chunk that
+// belongs there.  232,965 x 256 x 602: 48 us (gemm_tn_kernel 69, the ring with byte transposes and 16 x 16 x 64: 64).
+__global__ __launch_bounds__(256, 2) void gemm_tn_tr_kernel(const TnParams p) {
+    typedef int v2i32 __attribute__((ext_vector_type(2)));
+    typedef int i32x16t __attribute__((ext_vector_type(16)));
+    // a stage: the A tile, then the B tile, [64 rows][128 bytes] each
     __shared__ uint32_t st0[4096], st1[4096], st2[4096], st3[4096];
     uint32_t* const sA0 = st0; uint32_t* const sB0 = st0 + 2048;
     uint32_t* const sA1 = st1; uint32_t* const sB1 = st1 + 2048;
@@ -1451,22 +1462,18 @@ __global__ __launch_bounds__(256, 2) void gemm_tn_dma_kernel(const TnParams p) {
     const int64_t n0 = static_cast<int64_t>(tn) * 128, k0 = static_cast<int64_t>(tk) * 128;
     const int64_t m_begin = static_cast<int64_t>(split) * p.chunk;
     const int64_t m_end = (m_begin + p.chunk < p.M) ? m_begin + p.chunk : p.M;
-    const int64_t steps = (m_end - m_begin) >> 6;  // whole 64-row steps; a last partial one goes through registers
+    const int64_t steps = (m_end - m_begin) >> 6;
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wn = wave >> 1, wk = wave & 1;
-    const int g = lane >> 4, r16 = lane & 15;
 
-    // this lane's two chunks per operand and step: LDS chunk P = tid + 256 i holds row P / 8, logical chunk
-    // (P % 8) ^ swizzle; columns beyond the readable row bytes re-read the row's last chunk (they only reach outputs
-    // that are not stored)
     int64_t a_off[2], b_off[2];
 #pragma unroll
     for (int i = 0; i < 2; ++i) {
         const int P = tid + 256 * i, row = P >> 3;
-        const int lc = (P & 7) ^ (4 * ((row >> 4) & 1));
+        const int lc = (P & 7) ^ (row & 7);
         int64_t ca = n0 + 16 * lc, cb = k0 + 16 * lc;
         if (ca > p.a_row_bytes - 16) ca = p.a_row_bytes - 16;
         if (cb > p.b_row_bytes - 16) cb = p.b_row_bytes - 16;
@@ -1474,7 +1481,7 @@ __global__ __launch_bounds__(256, 2) void gemm_tn_dma_kernel(const TnParams p) {
         b_off[i] = row * p.ldb + cb;
     }
     auto issue = [&](uint32_t* dA, uint32_t* dB, int64_t step) {
-        const int64_t m0 = m_begin + (step < steps ? step : steps - 1) * 64;  // past the end: some valid rows, never read
+        const int64_t m0 = m_begin + (step < steps ? step : steps - 1) * 64;
         const int8_t* ga = p.A + m0 * p.lda;
         const int8_t* gb = p.B + m0 * p.ldb;
 #pragma unroll
@@ -1484,74 +1491,76 @@ __global__ __launch_bounds__(256, 2) void gemm_tn_dma_kernel(const TnParams p) {
         }
     };
 
-    i32x4 acc[4][4];
+    i32x16t acc[2][2];
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
+    for (int i = 0; i < 2; ++i)
 #pragma unroll
-        for (int j = 0; j < 4; ++j) acc[i][j] = i32x4{0, 0, 0, 0};
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) acc[i][j][v] = 0;
 
-    // A step's fragments are read from LDS one step ahead, as the raw dwords of sixteen rows per operand, while
-    // the matrix instructions of the current step run; the byte transposes that turn them into fragments follow
-    // those instructions.  (With the reads, the transposes and the matrix instructions of one step in a row, a
-    // wave spends a step waiting for each in turn, and two waves per SIMD do not cover that.)
-    uint32_t rawA[16], rawB[16];
-    i32x4 fa[4], fb[4];
-    const int cA = (wn * 16 + r16) ^ (16 * (g & 1));  // rows 16 g .. 16 g + 15 sit behind the swizzle of row / 16 % 2
-    const int cB = (wk * 16 + r16) ^ (16 * (g & 1));
-    auto read_raw = [&](const uint32_t* la, const uint32_t* lb) {
+    // this lane's part of the reads: group q = lane / 16 takes column strip q % 2 of a 32-column tile and the reduction
+    // half q / 2; inside the group lane j points at row j / 2 and the 8-byte half j % 2 of the strip
+    const int q = lane >> 4, j16 = lane & 15;
+    const int rsub = j16 >> 1, hb = j16 & 1;
+    // operand (tile t, half hm): rows 32 hm + 16 (q / 2) + 8 u + rsub for u = 0, 1; logical chunk base + 2 t + q % 2
+    auto read_ops = [&](const uint32_t* lds, int chunk_base, i32x4 (*op)[2]) {
+        const int8_t* base = reinterpret_cast<const int8_t*>(lds);
 #pragma unroll
-        for (int r = 0; r < 16; ++r) {
-            rawA[r] = la[(g * 16 + r) * 32 + cA];
-            rawB[r] = lb[(g * 16 + r) * 32 + cB];
-        }
+        for (int t = 0; t < 2; ++t)
+#pragma unroll
+            for (int hm = 0; hm < 2; ++hm) {
+                v2i32 r[2];
+#pragma unroll
+                for (int u = 0; u < 2; ++u) {
+                    const int row = 32 * hm + 16 * (q >> 1) + 8 * u + rsub;
+                    const int pc = (chunk_base + 2 * t + (q & 1)) ^ (row & 7);
+                    r[u] = __builtin_amdgcn_ds_read_tr8_b64_v2i32(
+                        (__attribute__((address_space(3))) v2i32*)(base + row * 128 + pc * 16 + 8 * hb));
+                }
+                op[t][hm] = i32x4{r[0][0], r[0][1], r[1][0], r[1][1]};
+            }
     };
-    // four fragments (sub-tiles j = 0..3) of the wave's 64 columns per operand (see gemm_tn_kernel)
-    auto transpose_raw = [&]() {
-        uint32_t col[4][4];
-#pragma unroll
-        for (int mb = 0; mb < 4; ++mb) transpose4x4(rawA[4 * mb], rawA[4 * mb + 1], rawA[4 * mb + 2], rawA[4 * mb + 3], col[mb]);
-#pragma unroll
-        for (int j = 0; j < 4; ++j)
-            fa[j] = i32x4{static_cast<int>(col[0][j]), static_cast<int>(col[1][j]),
-                          static_cast<int>(col[2][j]), static_cast<int>(col[3][j])};
-#pragma unroll
-        for (int mb = 0; mb < 4; ++mb) transpose4x4(rawB[4 * mb], rawB[4 * mb + 1], rawB[4 * mb + 2], rawB[4 * mb + 3], col[mb]);
-#pragma unroll
-        for (int j = 0; j < 4; ++j)
-            fb[j] = i32x4{static_cast<int>(col[0][j]), static_cast<int>(col[1][j]),
-                          static_cast<int>(col[2][j]), static_cast<int>(col[3][j])};
-    };
+    i32x4 opA[2][2], opB[2][2], nxA[2][2], nxB[2][2];
     auto multiply = [&]() {
 #pragma unroll
-        for (int i = 0; i < 4; ++i)
+        for (int hm = 0; hm < 2; ++hm)
 #pragma unroll
-            for (int j = 0; j < 4; ++j) acc[i][j] = mfma_16x16x64(fa[i], fb[j], acc[i][j]);
+            for (int i = 0; i < 2; ++i)
+#pragma unroll
+                for (int j = 0; j < 2; ++j)
+                    acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(opA[i][hm], opB[j][hm], acc[i][j], 0, 0, 0);
+    };
+    auto advance = [&]() {
+#pragma unroll
+        for (int t = 0; t < 2; ++t)
+#pragma unroll
+            for (int hm = 0; hm < 2; ++hm) {
+                opA[t][hm] = nxA[t][hm];
+                opB[t][hm] = nxB[t][hm];
+            }
     };
 
     if (steps > 0) {
         issue(sA0, sB0, 0);
         issue(sA1, sB1, 1);
         issue(sA2, sB2, 2);
-        // step 0's fragments
         __builtin_amdgcn_s_waitcnt(0x0F78);  // vmcnt(8): step 0 has landed
         __builtin_amdgcn_s_barrier();
         asm volatile("" ::: "memory");
-        read_raw(sA0, sB0);
-        transpose_raw();
-// Step s_ (fragments in registers): steps s_ and s_ + 1 have landed when four younger loads remain (vmcnt(4)); after
-// the barrier every wave's have, and every wave is done reading stage s_ - 1.  Ask for step s_ + 3 into that stage,
-// read step s_ + 1's raw rows (NA, NB: the next stage), multiply step s_, then transpose for the next step.
-// (A bare barrier: __syncthreads() carries a release fence that waits for every load in flight, which is exactly
-// what the ring is there to avoid.)  The last step reads a stage that holds rows of an earlier step: not used.
+        read_ops(sA0, wn * 4, opA);
+        read_ops(sB0, wk * 4, opB);
+// steps s_ and s_ + 1 have landed at vmcnt(4); ask for s_ + 3 (FA, FB: the stage step s_ - 1 left), read s_ + 1, multiply s_
 #define TANGO_TN_STEP(NA, NB, FA, FB, s_)          \
         asm volatile("" ::: "memory");             \
         __builtin_amdgcn_s_waitcnt(0x0F74);        \
         __builtin_amdgcn_s_barrier();              \
         asm volatile("" ::: "memory");             \
         issue(FA, FB, (s_) + 3);                   \
-        read_raw(NA, NB);                          \
+        read_ops(NA, wn * 4, nxA);                 \
+        read_ops(NB, wk * 4, nxB);                 \
         multiply();                                \
-        transpose_raw()
+        advance()
         for (int64_t s = 0; s < steps; s += 4) {
             TANGO_TN_STEP(sA1, sB1, sA3, sB3, s);
             if (s + 1 >= steps) break;
@@ -1562,7 +1571,7 @@ __global__ __launch_bounds__(256, 2) void gemm_tn_dma_kernel(const TnParams p) {
             TANGO_TN_STEP(sA0, sB0, sA2, sB2, s + 3);
         }
 #undef TANGO_TN_STEP
-        __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): nothing lands in LDS behind this point
+        __builtin_amdgcn_s_waitcnt(0x0F70);
         __syncthreads();
     }
     const int64_t m_tail = m_begin + steps * 64;
@@ -1576,27 +1585,29 @@ __global__ __launch_bounds__(256, 2) void gemm_tn_dma_kernel(const TnParams p) {
             const int64_t ca = n0 + scol * 16, cb = k0 + scol * 16;
             const i32x4 ra = load16<16>(p.A + m * p.lda + ca, (mok && ca < p.N) ? p.a_row_bytes - ca : 0);
             const i32x4 rb = load16<16>(p.B + m * p.ldb + cb, (mok && cb < p.K) ? p.b_row_bytes - cb : 0);
-            const int pc = scol ^ (4 * ((row >> 4) & 1));
+            const int pc = scol ^ (row & 7);
             *reinterpret_cast<i32x4*>(sA0 + row * 32 + pc * 4) = ra;
             *reinterpret_cast<i32x4*>(sB0 + row * 32 + pc * 4) = rb;
         }
         __syncthreads();
-        read_raw(sA0, sB0);
-        transpose_raw();
+        read_ops(sA0, wn * 4, opA);
+        read_ops(sB0, wk * 4, opB);
         multiply();
     }
 
-    // acc[i][j][v] at lane (g, r16): n = n0 + 64 wn + 4 (4 g + v) + i, k = k0 + 64 wk + 4 r16 + j (see gemm_tn_kernel)
+    // tile (i, j), register v, lane l: n = n0 + 64 wn + 32 i + 8 (v / 4) + 4 (l / 32) + v % 4, k = k0 + 64 wk + 32 j + l % 32:
+    // a store instruction writes 128 contiguous bytes of two rows of the slab
     int* slab = p.acc + static_cast<int64_t>(split) * p.N * p.Kp;
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
+    for (int i = 0; i < 2; ++i)
 #pragma unroll
-        for (int v = 0; v < 4; ++v) {
-            const int64_t n = n0 + wn * 64 + 4 * (4 * g + v) + i;
-            const int64_t k = k0 + wk * 64 + 4 * r16;
-            if (n < p.N && k < p.Kp)
-                *reinterpret_cast<i32x4*>(slab + n * p.Kp + k) =
-                    i32x4{acc[i][0][v], acc[i][1][v], acc[i][2][v], acc[i][3][v]};
+        for (int j = 0; j < 2; ++j) {
+            const int64_t k = k0 + wk * 64 + 32 * j + (lane & 31);
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+                const int64_t n = n0 + wn * 64 + 32 * i + 8 * (v >> 2) + 4 * (lane >> 5) + (v & 3);
+                if (n < p.N && k < p.Kp) slab[n * p.Kp + k] = acc[i][j][v];
+            }
         }
 }
 
@@ -2184,7 +2195,7 @@ int tango_qgemm_bwd_dw(float* dW, int64_t lddw, const int8_t* dYq, int64_t lddy,
         p.a_row_bytes = (vec == 16) ? round_up(N, 16) : (vec == 4 ? round_up(N, 4) : N);
         p.b_row_bytes = (vec == 16) ? round_up(K, 16) : (vec == 4 ? round_up(K, 4) : K);
         const dim3 grid(static_cast<unsigned>(tiles * t.splits));
-        if (vec == 16) hipLaunchKernelGGL(gemm_tn_dma_kernel, grid, dim3(256), 0, s, p);
+        if (vec == 16) hipLaunchKernelGGL(gemm_tn_tr_kernel, grid, dim3(256), 0, s, p);
         else if (vec == 4) hipLaunchKernelGGL(gemm_tn_kernel<4>, grid, dim3(256), 0, s, p);
         else hipLaunchKernelGGL(gemm_tn_kernel<1>, grid, dim3(256), 0, s, p);
     }
