@@ -534,6 +534,17 @@ int tango_attn_scores_bwd(float* dfeat, float* dattn_l, float* dattn_r, const fl
                           const float* attn_r, int64_t n, int64_t H, int64_t D, void* workspace,
                           size_t workspace_bytes, tango_stream_t stream);
 
+/* The same with the gradient feat receives from its other consumer folded in: feat feeds both the logits and
+   the aggregation (evaluation/test_gat.py:135-137 and :151), so autograd adds the two gradients of feat in a
+   pass of its own and the layer that produced feat then scans the sum for its scale (cuda/QLinear.py:37-39,
+   cuda/kernels.py:26-27).  Here dfeat = addend + (del*attn_l + der*attn_r), the very sum of that addition
+   (same operands, one rounding), and *scale_out (a slot holding 0) receives max|dfeat| / 127.  addend
+   [n, H, D] must not overlap dfeat.  Same workspace as tango_attn_scores_bwd. */
+int tango_attn_scores_bwd_acc(float* dfeat, float* dattn_l, float* dattn_r, float* scale_out, const float* addend,
+                              const float* del, const float* der, const float* feat, const float* attn_l,
+                              const float* attn_r, int64_t n, int64_t H, int64_t D, void* workspace,
+                              size_t workspace_bytes, tango_stream_t stream);
+
 /* -------------------------------------------------------------------- loss */
 
 /* Softmax cross-entropy with mean reduction and its gradient in one pass (no

@@ -60,6 +60,7 @@ SIGNATURES = {
     "tango_attn_scores_fwd": (I, [P, P, P, P, P, P, P, I64, I64, I64, P]),
     "tango_attn_scores_bwd_workspace": (SZ, [I64, I64, I64]),
     "tango_attn_scores_bwd": (I, [P, P, P, P, P, P, P, P, I64, I64, I64, P, SZ, P]),
+    "tango_attn_scores_bwd_acc": (I, [P, P, P, P, P, P, P, P, P, P, I64, I64, I64, P, SZ, P]),
     "tango_spmm_incidence": (I, [P, P, P, P, P, I64, I64, I64, I64, P]),
     "tango_sddmm_dot_i8": (I, [P, P, P, P, P, P, P, P, I64, I64, I64, P]),
     "tango_sddmm_ewise_i8": (I, [I, P, P, P, P, P, P, P, P, I64, I64, P]),

@@ -124,12 +124,15 @@ __global__ __launch_bounds__(SCALES ? 1024 : 256) void attn_scores_fwd_wide_kern
 // workgroup: a wavefront's loads and stores cover consecutive bytes (a thread per (row, head) would read D floats
 // at a stride of D floats).  part[b][2][H][D]: workgroup b's sums.  gridDim.y cuts the H * D / VEC column groups into chunks of at most 256; a workgroup
 // has 256 / (groups of its chunk) row lanes.
+// ACC: d_feat = addend + (del * attn_l + der * attn_r), the sum autograd would form in a pass of its own when feat
+// has a second consumer whose gradient is ``addend``, and max|d_feat| / 127 goes to *scale_out (which holds 0).
 // DYNAMIC LDS: 2 * 256 * VEC floats at most (2 * row_lanes * columns of the chunk).
-template <int VEC>
+template <int VEC, bool ACC>
 __global__ __launch_bounds__(256) void attn_scores_bwd_rows_kernel(
     float* __restrict__ dfeat, float* __restrict__ part, const float* __restrict__ del,
     const float* __restrict__ der, const float* __restrict__ feat, const float* __restrict__ al,
-    const float* __restrict__ ar, int64_t n, int H, int D) {
+    const float* __restrict__ ar, const float* __restrict__ addend, float* __restrict__ scale_out, int64_t n, int H,
+    int D) {
     extern __shared__ float red_rows[];  // [2][row_lanes][cw]
     typedef float fvec __attribute__((ext_vector_type(VEC == 1 ? 2 : VEC)));  // (unused for VEC == 1)
     const int C = H * D;
@@ -148,21 +151,32 @@ __global__ __launch_bounds__(256) void attn_scores_bwd_rows_kernel(
         wr[k] = ar[c0 + k];
         accl[k] = accr[k] = 0.0f;
     }
+    float m = 0.0f;
     if (rl < row_lanes) {
         const int64_t step = static_cast<int64_t>(gridDim.x) * row_lanes;
         for (int64_t r = static_cast<int64_t>(blockIdx.x) * row_lanes + rl; r < n; r += step) {
             const float gl = del[r * H + h], gr = der[r * H + h];
-            float x[VEC], y[VEC];
+            float x[VEC], y[VEC], a[VEC];
             if (VEC > 1) {
                 const fvec v = __builtin_nontemporal_load(reinterpret_cast<const fvec*>(feat + r * C + c0));
+                fvec u = v;
+                if (ACC) u = __builtin_nontemporal_load(reinterpret_cast<const fvec*>(addend + r * C + c0));
 #pragma unroll
-                for (int k = 0; k < VEC; ++k) x[k] = v[k];
+                for (int k = 0; k < VEC; ++k) {
+                    x[k] = v[k];
+                    a[k] = u[k];
+                }
             } else {
                 x[0] = feat[r * C + c0];
+                a[0] = ACC ? addend[r * C + c0] : 0.0f;
             }
 #pragma unroll
             for (int k = 0; k < VEC; ++k) {
                 y[k] = gl * wl[k] + gr * wr[k];
+                if (ACC) {
+                    y[k] = a[k] + y[k];
+                    m = fmaxf(m, fabsf(y[k]));
+                }
                 accl[k] += gl * x[k];
                 accr[k] += gr * x[k];
             }
@@ -188,6 +202,7 @@ __global__ __launch_bounds__(256) void attn_scores_bwd_rows_kernel(
         for (int l = 0; l < row_lanes; ++l) t += red_rows[(which * row_lanes + l) * cw + c];
         part[(static_cast<int64_t>(blockIdx.x) * 2 + which) * C + g0 * VEC + c] = t;
     }
+    if (ACC) block_absmax_to_global(m / 127.0f, scale_out);
 }
 
 // out[0 .. 2 H D) = sum over slabs, 64 slab lanes per element, fixed order.
@@ -272,10 +287,10 @@ size_t tango_attn_scores_bwd_workspace(int64_t n, int64_t H, int64_t D) {
     return static_cast<size_t>(bwd_groups(n, H)) * 2 * H * D * sizeof(float);
 }
 
-int tango_attn_scores_bwd(float* dfeat, float* dattn_l, float* dattn_r, const float* del,
-                          const float* der, const float* feat, const float* attn_l,
-                          const float* attn_r, int64_t n, int64_t H, int64_t D, void* workspace,
-                          size_t workspace_bytes, tango_stream_t stream) {
+static int attn_scores_bwd_impl(float* dfeat, float* dattn_l, float* dattn_r, const float* del, const float* der,
+                               const float* feat, const float* attn_l, const float* attn_r, const float* addend,
+                               float* scale_out, int64_t n, int64_t H, int64_t D, void* workspace,
+                               size_t workspace_bytes, tango_stream_t stream) {
     if (n < 0 || H < 0 || D < 0) return TANGO_ERR_INVALID_ARG;
     if (H * D == 0) return TANGO_OK;
     if (H > 256 || D >= (1LL << 31) || H * D > (1LL << 23)) return TANGO_ERR_UNSUPPORTED;
@@ -289,7 +304,8 @@ int tango_attn_scores_bwd(float* dfeat, float* dattn_l, float* dattn_r, const fl
         if (!workspace || workspace_bytes < need) return TANGO_ERR_WORKSPACE;
         if ((reinterpret_cast<uintptr_t>(workspace) & 3) != 0) return TANGO_ERR_INVALID_ARG;
         groups = bwd_groups(n, H);
-        const uintptr_t bits = reinterpret_cast<uintptr_t>(feat) | reinterpret_cast<uintptr_t>(dfeat);
+        const uintptr_t bits = reinterpret_cast<uintptr_t>(feat) | reinterpret_cast<uintptr_t>(dfeat) |
+                               reinterpret_cast<uintptr_t>(addend);
         const int64_t C = H * D;
         const int vec = (D % 4 == 0 && (bits & 15) == 0) ? 4 : (D % 2 == 0 && (bits & 7) == 0) ? 2 : 1;
         const int64_t cg_all = C / vec, chunks = ceil_div(cg_all, 256);
@@ -300,20 +316,42 @@ int tango_attn_scores_bwd(float* dfeat, float* dattn_l, float* dattn_r, const fl
             groups = static_cast<int>(want < groups ? (want < 1 ? 1 : want) : groups);
             const size_t lds = sizeof(float) * 2 * 256 * vec;
             const dim3 grid(static_cast<unsigned>(groups), static_cast<unsigned>(chunks));
-            if (vec == 4)
-                hipLaunchKernelGGL(attn_scores_bwd_rows_kernel<4>, grid, dim3(256), lds, s, dfeat, part, del, der, feat,
-                                   attn_l, attn_r, n, static_cast<int>(H), static_cast<int>(D));
-            else if (vec == 2)
-                hipLaunchKernelGGL(attn_scores_bwd_rows_kernel<2>, grid, dim3(256), lds, s, dfeat, part, del, der, feat,
-                                   attn_l, attn_r, n, static_cast<int>(H), static_cast<int>(D));
-            else
-                hipLaunchKernelGGL(attn_scores_bwd_rows_kernel<1>, grid, dim3(256), lds, s, dfeat, part, del, der, feat,
-                                   attn_l, attn_r, n, static_cast<int>(H), static_cast<int>(D));
+#define TANGO_ATTN_BWD(V, A)                                                                                    \
+    hipLaunchKernelGGL((attn_scores_bwd_rows_kernel<V, A>), grid, dim3(256), lds, s, dfeat, part, del, der, feat,   \
+                       attn_l, attn_r, addend, scale_out, n, static_cast<int>(H), static_cast<int>(D))
+            if (addend) {
+                if (vec == 4) TANGO_ATTN_BWD(4, true);
+                else if (vec == 2) TANGO_ATTN_BWD(2, true);
+                else TANGO_ATTN_BWD(1, true);
+            } else {
+                if (vec == 4) TANGO_ATTN_BWD(4, false);
+                else if (vec == 2) TANGO_ATTN_BWD(2, false);
+                else TANGO_ATTN_BWD(1, false);
+            }
+#undef TANGO_ATTN_BWD
         }
     }
     hipLaunchKernelGGL(attn_scores_finish_kernel, dim3(static_cast<unsigned>(ceil_div(2 * H * D, 16))), dim3(1024), 0,
                        s, dattn_l, dattn_r, part, groups, H * D);
     return launch_status();
+}
+
+int tango_attn_scores_bwd(float* dfeat, float* dattn_l, float* dattn_r, const float* del,
+                          const float* der, const float* feat, const float* attn_l,
+                          const float* attn_r, int64_t n, int64_t H, int64_t D, void* workspace,
+                          size_t workspace_bytes, tango_stream_t stream) {
+    return attn_scores_bwd_impl(dfeat, dattn_l, dattn_r, del, der, feat, attn_l, attn_r, nullptr, nullptr, n, H, D,
+                                workspace, workspace_bytes, stream);
+}
+
+int tango_attn_scores_bwd_acc(float* dfeat, float* dattn_l, float* dattn_r, float* scale_out, const float* addend,
+                              const float* del, const float* der, const float* feat, const float* attn_l,
+                              const float* attn_r, int64_t n, int64_t H, int64_t D, void* workspace,
+                              size_t workspace_bytes, tango_stream_t stream) {
+    if (!scale_out || (n > 0 && H * D > 0 && !addend)) return TANGO_ERR_INVALID_ARG;
+    if (addend == dfeat && n > 0 && H * D > 0) return TANGO_ERR_INVALID_ARG;  // the kernel's pointers do not alias
+    return attn_scores_bwd_impl(dfeat, dattn_l, dattn_r, del, der, feat, attn_l, attn_r, addend, scale_out, n, H, D,
+                                workspace, workspace_bytes, stream);
 }
 
 }  // extern "C"

@@ -26,30 +26,44 @@ class attn_scores(Function):
     """el = (feat * attn_l).sum(-1), er = (feat * attn_r).sum(-1) for feat [n, H, D] and
     attn_l, attn_r [1, H, D] (evaluation/test_gat.py:135-137), forward and backward each in
     one pass over feat.  Returns el, er as [n, H, 1] and their quantization scales max|.| / 127
-    (None while a graph is being captured), which the same kernel finds."""
+    (None while a graph is being captured), which the same kernel finds.
+
+    ``through=True`` returns feat itself as a fifth result, for the layer's other reader of feat (the
+    aggregation, evaluation/test_gat.py:151) to take instead of feat: both gradients of feat then arrive at
+    this node, whose backward kernel adds the aggregation's to its own as it writes and finds max|sum| / 127
+    for the linear layer below (left on the gradient, ``grad_scale_hint``), where autograd would add the two in
+    a pass of its own and that layer scan the sum in another.  Same sum, same bits."""
 
     @staticmethod
-    def forward(ctx, feat, attn_l, attn_r):
+    def forward(ctx, feat, attn_l, attn_r, through=False):
         feat = feat if feat.is_contiguous() else feat.contiguous()
         al, ar = attn_l.contiguous(), attn_r.contiguous()
         el, er, s_el, s_er = cuda_kernels.attn_scores_forward(feat, al, ar, want_scales=True)
-        ctx.backward_cache = feat, al, ar, attn_l.shape
+        ctx.backward_cache = feat, al, ar, attn_l.shape, through
         ctx.set_materialize_grads(False)  # no zero tensors (a fill launch each) for the scales' absent gradients
         if s_el is not None:
             ctx.mark_non_differentiable(s_el, s_er)
-        return el.unsqueeze(-1), er.unsqueeze(-1), s_el, s_er
+        out = el.unsqueeze(-1), er.unsqueeze(-1), s_el, s_er
+        return (out + (feat.view_as(feat),)) if through else out
 
     @staticmethod
     @once_differentiable
-    def backward(ctx, del_, der, _ds_el=None, _ds_er=None):
+    def backward(ctx, *grads):
         refuse_capture("attn_scores.backward")
-        feat, al, ar, shape = ctx.backward_cache
+        feat, al, ar, shape, through = ctx.backward_cache
+        del_, der = grads[0], grads[1]
+        dthrough = grads[4] if through else None
         if del_ is None and der is None:
-            return None, None, None
+            return dthrough, None, None, None
         del_ = torch.zeros_like(der) if del_ is None else del_
         der = torch.zeros_like(del_) if der is None else der
-        dfeat, dal, dar = cuda_kernels.attn_scores_backward(del_.contiguous(), der.contiguous(), feat, al, ar)
-        return dfeat, dal.view(shape), dar.view(shape)
+        if dthrough is None:
+            dfeat, dal, dar = cuda_kernels.attn_scores_backward(del_.contiguous(), der.contiguous(), feat, al, ar)
+        else:
+            dfeat, dal, dar, s = cuda_kernels.attn_scores_backward(del_.contiguous(), der.contiguous(), feat, al, ar,
+                                                                   addend=dthrough.contiguous())
+            dfeat._tango_scale = (s, dfeat._version, dfeat.data_ptr())
+        return dfeat, dal.view(shape), dar.view(shape), None
 
 
 class QGATConv(nn.Module):
@@ -101,7 +115,7 @@ class QGATConv(nn.Module):
         else:
             feat_src, s_feat = self.fc(h)
         feat_src = feat_src.view(n, self._num_heads, self._out_feats)
-        el, er, s_el, s_er = attn_scores.apply(feat_src, self.attn_l, self.attn_r)  # test_gat.py:135-137
+        el, er, s_el, s_er, feat_src = attn_scores.apply(feat_src, self.attn_l, self.attn_r, True)  # test_gat.py:135-137
         s_a = None
         if s_el is not None and fused_attention:
             # u_add_v :141, LeakyReLU :144 and the softmax :146 as one op that also hands the aggregation
@@ -264,7 +278,7 @@ class ArxivGATConv(nn.Module):
             kept = self.attn_drop(edge_softmax(graph, e[eids], negative_slope=self.negative_slope, eids=eids))
             a = torch.zeros_like(e).index_copy(0, eids, kept)
         elif self.attn_r is not None:  # :176-184
-            el, er, s_el, s_er = attn_scores.apply(feat_src, self.attn_l, self.attn_r)
+            el, er, s_el, s_er, feat_src = attn_scores.apply(feat_src, self.attn_l, self.attn_r, True)
             if s_el is not None and fused_attention:
                 a, s_a = gat_edge_attention.apply(graph, el, er, s_el, s_er, self.negative_slope)  # :184, :187, :196
             else:

@@ -847,8 +847,10 @@ class cuda_kernels:
         return (el, er, s_el, s_er) if want_scales else (el, er)
 
     @staticmethod
-    def attn_scores_backward(del_, der, feat, attn_l, attn_r):
-        """(dfeat [n, H, D], dattn_l [H, D], dattn_r [H, D])."""
+    def attn_scores_backward(del_, der, feat, attn_l, attn_r, addend=None):
+        """(dfeat [n, H, D], dattn_l [H, D], dattn_r [H, D]).  ``addend`` (fp32, feat's shape): the gradient feat
+        receives from another consumer; dfeat is then the sum of the two and a fourth result is max|dfeat| / 127,
+        found by the same kernel."""
         for t, nm in ((del_, "del"), (der, "der"), (feat, "feat"), (attn_l, "attn_l"), (attn_r, "attn_r")):
             _need(t, torch.float32, nm)
         n, H, D = feat.shape
@@ -859,6 +861,15 @@ class cuda_kernels:
         dar = torch.empty((H, D), dtype=torch.float32, device=feat.device)
         ws_bytes = _ws_bytes("tango_attn_scores_bwd_workspace", n, H, D)
         ws = _workspace(ws_bytes, feat.device)
+        if addend is not None:
+            _need(addend, torch.float32, "addend")
+            if addend.numel() != feat.numel():
+                raise RuntimeError("attn_scores_backward: addend must have feat's size")
+            scale = _zero_slot(feat.device)
+            check(_L.tango_attn_scores_bwd_acc(_ptr(dfeat), _ptr(dal), _ptr(dar), _ptr(scale), _ptr(addend), _ptr(del_),
+                                               _ptr(der), _ptr(feat), _ptr(attn_l), _ptr(attn_r), n, H, D, _ptr(ws),
+                                               ws_bytes, _stream()), "attn_scores_backward")
+            return dfeat, dal, dar, scale
         check(_L.tango_attn_scores_bwd(_ptr(dfeat), _ptr(dal), _ptr(dar), _ptr(del_), _ptr(der), _ptr(feat),
                                        _ptr(attn_l), _ptr(attn_r), n, H, D, _ptr(ws), ws_bytes, _stream()),
               "attn_scores_backward")

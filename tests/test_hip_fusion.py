@@ -211,6 +211,50 @@ def test_attn_scores_match_torch(K, n, H, D):
     atol = 1e-4 * max(1.0, n / 2000)  # fp32 sums over n terms
     assert torch.allclose(dal.double(), (dl.double().unsqueeze(-1) * f64).sum(0), rtol=1e-5, atol=atol)
     assert torch.allclose(dar.double(), (dr.double().unsqueeze(-1) * f64).sum(0), rtol=1e-5, atol=atol)
+    # with the gradient of feat's other consumer folded in: the sum autograd would form, and its scale
+    other = torch.randn(n, H, D, generator=g).cuda() * 0.7
+    dsum, dal2, dar2, s = K.cuda_kernels.attn_scores_backward(dl, dr, feat, al.contiguous(), ar.contiguous(), addend=other)
+    assert torch.equal(dsum, other + dfeat)
+    assert torch.equal(dal2, dal) and torch.equal(dar2, dar)
+    assert torch.equal(s, K.cuda_kernels.get_scale(dsum))
+
+
+def test_attn_scores_pass_through_collects_both_gradients():
+    """feat read by the logits and, through the node's fifth result, by a second consumer: the gradient that reaches
+    feat is the sum autograd forms when the two read feat directly, bit for bit, and it carries its scale."""
+    from tango_amd.SPMM import grad_scale_hint
+    from tango_amd.gat import attn_scores
+    g = torch.Generator().manual_seed(6)
+    n, H, D = 5000, 8, 16
+    base = torch.randn(n, H, D, generator=g).cuda()
+    al = torch.randn(1, H, D, generator=g).cuda().requires_grad_()
+    ar = torch.randn(1, H, D, generator=g).cuda().requires_grad_()
+    w1, w2 = torch.randn(n, H, 1, generator=g).cuda(), torch.randn(n, H, 1, generator=g).cuda()
+    w3 = torch.randn(n, H, D, generator=g).cuda()
+    grads, seen = [], []
+    for through in (False, True):
+        feat = base.clone().requires_grad_()
+        feat2 = feat * 1.0  # a non-leaf, so that a hook sees the gradient tensor the node returns
+        feat2.register_hook(lambda t: seen.append((t, grad_scale_hint(t))))
+        out = attn_scores.apply(feat2, al, ar, through)
+        second = out[4] if through else feat2
+        ((out[0] * w1).sum() + (out[1] * w2).sum() + (second * second * w3).sum()).backward()
+        grads.append([t.grad.clone() for t in (feat, al, ar)])
+        al.grad = ar.grad = None
+    for a, b in zip(*grads):
+        assert torch.equal(a, b)
+    assert seen[0][1] is None  # autograd's own sum carries no scale
+    t, s = seen[1]
+    assert s is not None and torch.equal(s, t.abs().max().reshape(1) / 127)
+    # one consumer only: nothing to add, the plain kernel runs
+    feat = base.clone().requires_grad_()
+    out = attn_scores.apply(feat, al, ar, True)
+    ((out[0] * w1).sum() + (out[1] * w2).sum()).backward()
+    assert torch.equal(feat.grad, w1 * al.detach() + w2 * ar.detach())
+    feat.grad = None
+    out = attn_scores.apply(feat, al, ar, True)
+    (out[4] * w3).sum().backward()  # the logits unused: the second consumer's gradient passes through
+    assert torch.equal(feat.grad, w3)
 
 
 def test_attn_scores_autograd_matches_torch():

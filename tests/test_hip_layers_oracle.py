@@ -61,7 +61,7 @@ def test_arxiv_gat_layer_matches_oracle_stage_by_stage(orc, recorded, monkeypatc
     feat, _, _, _, _, s_feat = orc.qgemm_fwd(host(x), W, reduce=True)
     (args, res), = recorded["attn_scores"].calls
     assert np.array_equal(host(args[0]).reshape(n, H * D), feat)
-    el, er, s_el, s_er = res
+    el, er, s_el, s_er = res[:4]
     al, ar = host(layer.attn_l).reshape(H, D), host(layer.attn_r).reshape(H, D)
     f3 = feat.reshape(n, H, D).astype(np.float64)
     np.testing.assert_allclose(host(el).reshape(n, H), (f3 * al).sum(-1), rtol=1e-5, atol=1e-5)
