@@ -23,9 +23,10 @@ attention_logits_on_the_fly = os.environ.get("TANGO_ATTN_ON_THE_FLY", "0") == "1
 
 # spmm_copy_u on dense graphs: let the aggregation's epilogue return the scale of its output (forward: to the next
 # layer's GEMM; backward: to the quantizer of the gradient it produces) instead of a pass over that output.  Same
-# values.  Measured on the 114.8 M-edge benchmark epoch: the three passes it removes take 100 us, but the few
-# registers the epilogue needs for it cost the gather kernel one of its eight waves per SIMD (65 instead of 64
-# VGPRs) and with it 50 us per launch: 5.66 against 5.61 ms per epoch, hence off.
+# values.  Measured on the 114.8 M-edge benchmark epoch: the passes it removes take 100 us and the reduction over
+# the per-row maxima adds 17, but the gather launches that carry the epilogue take 130 us longer in all (57 us each
+# at 256 columns): 5.22 against 5.17 ms per epoch, hence off.  The epilogue needs 65 instead of 64 VGPRs (seven
+# instead of eight waves per SIMD); held at 64 by a launch bound (two dwords spilled in the epilogue) it costs the same.
 scale_from_aggregation = os.environ.get("TANGO_SCALE_FROM_AGGREGATION", "0") == "1"
 
 # Seed of the counter-based RNG for stochastic rounding; every quantize call
