@@ -9,10 +9,11 @@ from .kernels import (cuda_kernels, incidence_SPMM, multi_cusparse_SPMM, mySDDMM
 
 
 def _quantize_grad(t):
+    from .SPMM import grad_scale
     t = t if t.is_contiguous() else t.contiguous()
     if config.grad_round_mode == "stochastic":
-        return quantize(t, round_mode="stochastic", **config.stochastic_args(t.device))
-    return quantize(t, round_mode=config.grad_round_mode)
+        return quantize(t, grad_scale(t), round_mode="stochastic", **config.stochastic_args(t.device))
+    return quantize(t, grad_scale(t), round_mode=config.grad_round_mode)
 
 
 class sddmm_u_add_v(Function):

@@ -34,6 +34,17 @@ def grad_scale_hint(t):
     return None
 
 
+def grad_scale(t):
+    """max|t| / 127 of the contiguous gradient ``t``: the value its producer left on it, else one absmax pass whose
+    result stays on the tensor, so that a gradient autograd hands to several nodes (the sum of the per-relation
+    aggregates of a heterogeneous layer) is scanned by the first of them only."""
+    s = grad_scale_hint(t)
+    if s is None:
+        s = cuda_kernels.get_scale(t)
+        t._tango_scale = (s, t._version, t.data_ptr())
+    return s
+
+
 def masked_scale_hint(t, bits, row_mul):
     """max|t' * row_mul| / 127 (t' = t where its sign bit in ``bits`` is set) if the GEMM that produced the gradient
     ``t`` found it in its epilogue for exactly this mask and multiplier and nothing has written to ``t`` since."""
@@ -60,8 +71,8 @@ def _quantize_grad(t, padded):
     if config.grad_round_mode == "stochastic":
         kw.update(config.stochastic_args(t.device))
     if padded and t.dim() == 2:
-        return quantize_padded(t, align=_gather_align(t.size(1)), **kw)
-    return quantize(t, **kw)
+        return quantize_padded(t, grad_scale(t), align=_gather_align(t.size(1)), **kw)
+    return quantize(t, grad_scale(t), **kw)
 
 
 class spmm_copy_u(Function):

@@ -742,3 +742,41 @@ def test_gcn_backward_takes_the_scale_from_gradx(monkeypatch):
             assert torch.allclose(a, b, rtol=1e-5, atol=1e-6)
         else:
             assert torch.equal(a, b)
+
+
+def test_gradient_with_two_consumers_is_scanned_once(monkeypatch):
+    """The sum of two aggregations: autograd hands both nodes the same gradient tensor, the first leaves its scale
+    on it and the second takes it from there.  Same gradients as with a scan each."""
+    from tango_amd import SPMM, config, kernels
+    from tango_amd.SPMM import spmm_copy_u
+    from tango_amd.graph import Graph
+    from tango_amd.util import graph_preprocess
+    rng = np.random.default_rng(41)
+    n = 2000
+    graphs = []
+    for e in (15000, 9000):
+        src, dst = rand_graph(rng, n, e)
+        graphs.append(graph_preprocess(Graph(dev(src), dev(dst), n)))
+    config.grad_round_mode = "rne"
+    xs = [dev(rng.standard_normal((n, 64)).astype(np.float32)).requires_grad_() for _ in graphs]
+    w = dev(rng.standard_normal((n, 64)).astype(np.float32))
+    scans = []
+    real = kernels.cuda_kernels.get_scale
+    monkeypatch.setattr(kernels.cuda_kernels, "get_scale",
+                        staticmethod(lambda t: (scans.append(t.requires_grad), real(t))[1]))
+
+    def grads():
+        scans.clear()
+        for x in xs:
+            x.grad = None
+        out = spmm_copy_u.apply(graphs[0], xs[0]) + spmm_copy_u.apply(graphs[1], xs[1])
+        fwd = len(scans)
+        (out * w).sum().backward()
+        return [x.grad.clone() for x in xs], len(scans) - fwd
+
+    shared, n_shared = grads()
+    monkeypatch.setattr(SPMM, "grad_scale_hint", lambda t: None)
+    apart, n_apart = grads()
+    assert n_shared == 1 and n_apart == 2
+    for a, b in zip(shared, apart):
+        assert torch.equal(a, b)
