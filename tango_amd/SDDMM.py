@@ -1,6 +1,7 @@
 """Quantized per-edge ops: mirrors cuda/SDDMM.py of the reference, plus the
 ``sddmm_u_dot_v`` op that the reference's drivers call but its tree does not
 define (evaluation/test_HGT.py:58, evaluation/link_pred_gcn.py:145)."""
+import torch
 from torch.autograd.function import Function, once_differentiable
 
 from . import config
@@ -55,13 +56,20 @@ class sddmm_u_dot_v(Function):
     ``out_scale`` (a Python float) multiplies the result, e.g. the 1 / sqrt(d_k) of an attention
     score (evaluation/test_HGT.py:58): it is folded into the dequantization scales of the forward
     and of both backward aggregations, so no pass over the [E, H] tensor runs for it (bit-identical
-    to multiplying afterwards when it is a power of two, else within an ulp or two)."""
+    to multiplying afterwards when it is a power of two, else within an ulp or two).
+    ``Vq``: (int8 V, scale) as ``kernels.quantize_heads(V, scaleV_)`` returns them, when several calls share one V
+    (the queries of a node type that several relations end at): V is then quantized once, by the caller."""
 
     @staticmethod
-    def forward(ctx, g, U, V, scaleU_=None, scaleV_=None, out_scale=None):
+    def forward(ctx, g, U, V, scaleU_=None, scaleV_=None, out_scale=None, Vq=None):
         # heads whose width would leave the int8 rows unaligned are zero-padded (kernels.pad_heads): same dot products
         U_, scaleU = quantize_heads(U if U.is_contiguous() else U.contiguous(), scaleU_)
-        V_, scaleV = quantize_heads(V if V.is_contiguous() else V.contiguous(), scaleV_)
+        if Vq is not None:
+            V_, scaleV = Vq
+            if V_.dtype != torch.int8 or V_.shape[:-1] != V.shape[:-1] or V_.size(-1) < V.size(-1):
+                raise RuntimeError("sddmm_u_dot_v: Vq must be the int8 copy of V")
+        else:
+            V_, scaleV = quantize_heads(V if V.is_contiguous() else V.contiguous(), scaleV_)
         ctx.width = U.size(-1)
         if out_scale is not None:
             # 1-element products: the forward dequantizes with sU * (sV c), the backward passes with
@@ -91,4 +99,4 @@ class sddmm_u_dot_v(Function):
         if ctx.needs_input_grad[2]:
             dV = unpad_heads(multi_cusparse_SPMM(g, U3, dZ_, scaledZ, edge_major=True, scale2=scaleU).reshape(V_.shape),
                              ctx.width)
-        return None, dU, dV, None, None, None
+        return None, dU, dV, None, None, None, None

@@ -11,7 +11,7 @@ from torch.autograd.function import Function, once_differentiable
 
 from .QLinear import QLinear, Qlinear_func, Qlinear_func_reduce, shared_input_linears
 from .batchnorm import BatchNorm1dAct
-from .kernels import cuda_kernels, refuse_capture
+from .kernels import cuda_kernels, quantize_heads, refuse_capture
 from .SDDMM import sddmm_u_add_v, sddmm_u_dot_v
 from .SPMM import spmm_u_mul_e
 from .edge_softmax import edge_softmax, gat_edge_attention
@@ -388,9 +388,13 @@ class HeteroHGTLayer(nn.Module):
             for r, pair in zip(rs, shared_input_linears(v[t][0], [self.msg_linear[r] for r in rs], v[t][1])):
                 vr[t, r] = pair
         scores = []
+        q8 = {}  # the queries of a node type in int8, shared by the relations that end there
         for r, part in units:
             (U, sU), (V, sV) = kr[part.src_type, r], q[part.dst_type]
-            scores.append(sddmm_u_dot_v.apply(part, U.view(-1, H, dk), V.view(-1, H, dk), sU, sV, 1.0 / self.sqrt_dk))
+            V = V.view(-1, H, dk)
+            if part.dst_type not in q8:
+                q8[part.dst_type] = quantize_heads(V if V.is_contiguous() else V.contiguous(), sV)
+            scores.append(sddmm_u_dot_v.apply(part, U.view(-1, H, dk), V, sU, sV, 1.0 / self.sqrt_dk, q8[part.dst_type]))
         ranges = [part.edge_range for _, part in units]
         contiguous = all(rg is not None for rg in ranges)
         if contiguous:
