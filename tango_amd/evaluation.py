@@ -70,38 +70,77 @@ def arxiv_loss(x, labels):
     return torch.mean(torch.log(ARXIV_EPSILON + y) - math.log(ARXIV_EPSILON))
 
 
+def add_labels(feat, labels, idx, n_classes):
+    """``feat`` widened by ``n_classes`` columns that hold the one-hot labels of the nodes ``idx`` and zeros for all
+    others: the label-reuse input of evaluation/arxiv_gat.py:534-537 and arxiv_gcn.py:234-237."""
+    onehot = feat.new_zeros(feat.size(0), n_classes)
+    onehot[idx, labels[idx]] = 1
+    return torch.cat([feat, onehot], dim=-1)
+
+
+def warm_up_lr(optimizer, lr, epoch, span=50):
+    """The learning rate of epoch 1, 2, ... climbs linearly to ``lr`` over the first ``span`` epochs
+    (evaluation/arxiv_gat.py:540-543, called at the top of every epoch, :655)."""
+    if epoch <= span:
+        for group in optimizer.param_groups:
+            group["lr"] = lr * epoch / span
+
+
 def train_arxiv(model_name="gat", epochs=20, n_hidden=None, n_layers=3, n_heads=3, lr=2e-3, dropout=0.75,
-                input_drop=0.1, attn_drop=0.05, use_linear=True, dataset="ogbn-arxiv", quiet=False):
-    """evaluation/arxiv_gat.py:536-560 / arxiv_gcn.py:246-281 (``train``) on the synthetic stand-in of
-    ogbn-arxiv: the GAT or GCN stack of those scripts, the smoothed loss on the training nodes, RMSprop for the
-    GAT (arxiv_gat.py:603) and AdamW for the GCN (arxiv_gcn.py:311).  The scripts' label-reuse trick
-    (``--use-labels``) and their learning-rate warm-up are left to the caller.  Returns (mean ms per epoch
-    after the first three, final loss)."""
+                input_drop=0.1, attn_drop=0.05, edge_drop=0.0, use_linear=True, dataset="ogbn-arxiv", quiet=False,
+                use_labels=False, mask_rate=0.5, n_label_iters=0, warm_up=True):
+    """evaluation/arxiv_gat.py:546-590 / arxiv_gcn.py:246-281 (``train``) on the synthetic stand-in of
+    ogbn-arxiv: the GAT or GCN stack of those scripts, the smoothed loss, RMSprop for the GAT (arxiv_gat.py:603)
+    and AdamW for the GCN (arxiv_gcn.py:311), the learning-rate warm-up of the scripts' epoch loops, and their
+    per-epoch random split of the training nodes: with ``use_labels`` the nodes drawn with probability ``mask_rate``
+    feed their labels in as extra input columns and the loss is taken on the others, without it the loss is
+    taken on the drawn nodes.  ``n_label_iters`` (needs ``use_labels``, arxiv_gat.py:794-796) repeats the forward
+    pass that many times with the softmax of the previous prediction written into the label columns of every
+    node whose label is not an input (arxiv_gat.py:572-578); only the last pass is differentiated.  Returns
+    (mean ms per epoch after the first three, final loss)."""
+    if n_label_iters > 0 and not use_labels:
+        raise ValueError("n_label_iters > 0 needs use_labels")
     g = load_graph_train(dataset)
-    feats, labels, train_mask = g.ndata["feat"], g.ndata["label"], g.ndata["train_mask"]
+    feats, labels = g.ndata["feat"], g.ndata["label"]
+    train_idx = g.ndata["train_mask"].nonzero().squeeze(1)
+    rest_idx = (~g.ndata["train_mask"]).nonzero().squeeze(1)  # the scripts' validation and test nodes
+    classes = g.n_classes
+    width = feats.size(1) + (classes if use_labels else 0)
     if model_name == "gat":
-        model = ArxivGAT(feats.size(1), g.n_classes, n_hidden or 250, n_layers, n_heads, F.relu, dropout=dropout,
-                         input_drop=input_drop, attn_drop=attn_drop).cuda()
+        model = ArxivGAT(width, classes, n_hidden or 250, n_layers, n_heads, F.relu, dropout=dropout,
+                         input_drop=input_drop, attn_drop=attn_drop, edge_drop=edge_drop).cuda()
         opt = torch.optim.RMSprop(model.parameters(), lr=lr, weight_decay=0)
     elif model_name == "gcn":
-        model = ArxivGCN(feats.size(1), n_hidden or 256, g.n_classes, n_layers, F.relu, min(dropout, 0.5),
-                         use_linear).cuda()
+        model = ArxivGCN(width, n_hidden or 256, classes, n_layers, F.relu, min(dropout, 0.5), use_linear).cuda()
         opt = torch.optim.AdamW(model.parameters(), lr=lr, weight_decay=0)
     else:
         raise ValueError("model must be gat or gcn")
     dur, loss = [], None
-    for epoch in range(epochs):
+    for epoch in range(1, epochs + 1):
+        if warm_up:
+            warm_up_lr(opt, lr, epoch)
         model.train()
+        drawn = torch.rand(train_idx.shape, device=train_idx.device) < mask_rate
+        if use_labels:
+            x, pred_idx = add_labels(feats, labels, train_idx[drawn], classes), train_idx[~drawn]
+        else:
+            x, pred_idx = feats, train_idx[drawn]
+        opt.zero_grad()
         start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         start.record()
-        pred = model(g, feats)
-        loss = arxiv_loss(pred[train_mask], labels[train_mask])
-        opt.zero_grad()
+        pred = model(g, x)
+        if n_label_iters > 0:
+            unlabelled = torch.cat([pred_idx, rest_idx])
+            for _ in range(n_label_iters):
+                pred = pred.detach()
+                x[unlabelled, -classes:] = F.softmax(pred[unlabelled], dim=-1)
+                pred = model(g, x)
+        loss = arxiv_loss(pred[pred_idx], labels[pred_idx])
         loss.backward()
         stop.record()
         torch.cuda.synchronize()
         opt.step()
-        if epoch >= 3:
+        if epoch > 3:
             dur.append(start.elapsed_time(stop))
         if not quiet:
             print("Epoch {:05d} | Time(ms) {:.4f} | Loss {:.4f}".format(epoch, np.mean(dur) if dur else float("nan"),

@@ -136,6 +136,24 @@ def test_bipartite_graph_formats():
         assert s[m].min() >= bounds[a] and s[m].max() < bounds[a + 1] and d[m].max() < bounds[b + 1]
 
 
+def test_label_reuse_input_and_warm_up_schedule():
+    """evaluation/arxiv_gat.py:534-543 on host tensors: one-hot label columns for the chosen nodes only, and a
+    learning rate that climbs linearly over the first 50 epochs and is left alone afterwards."""
+    import torch
+    from tango_amd.evaluation import add_labels, warm_up_lr
+    feat = torch.arange(12.0).reshape(4, 3)
+    labels = torch.tensor([2, 0, 1, 2])
+    out = add_labels(feat, labels, torch.tensor([0, 2]), 3)
+    assert out.shape == (4, 6) and torch.equal(out[:, :3], feat)
+    assert torch.equal(out[:, 3:], torch.tensor([[0.0, 0, 1], [0, 0, 0], [0, 1, 0], [0, 0, 0]]))
+    opt = torch.optim.SGD([torch.zeros(1, requires_grad=True)], lr=0.5)
+    seen = []
+    for epoch in (1, 25, 50, 51):
+        warm_up_lr(opt, 0.2, epoch)
+        seen.append(opt.param_groups[0]["lr"])
+    assert seen == [0.2 / 50, 0.1, 0.2, 0.2]
+
+
 def test_bench_refuses_more_than_one_gpu():
     """bench.py measures one GPU; asking for more exits with a message before anything touches a device."""
     import os

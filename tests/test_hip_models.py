@@ -200,6 +200,24 @@ def test_evaluation_drivers_train_on_the_pubmed_stand_in(model):
     assert np.isfinite(ms) and ms > 0 and np.isfinite(loss) and loss < first_loss
 
 
+@pytest.mark.parametrize("model,kw", [("gat", {"use_labels": True, "n_label_iters": 1, "mask_rate": 0.5}),
+                                      ("gat", {"edge_drop": 0.2}), ("gcn", {"use_labels": True}), ("gcn", {})])
+def test_arxiv_drivers_train_with_label_reuse_and_warm_up(model, kw):
+    """tango_amd.evaluation.train_arxiv: the loops of evaluation/arxiv_gat.py:546-590 and arxiv_gcn.py:246-281 with
+    their learning-rate warm-up, the per-epoch split of the training nodes, labels fed back in as input columns
+    and one refinement pass over the unlabelled nodes, on the small stand-in graph."""
+    from tango_amd import evaluation
+    common = dict(dataset="pubmed", n_hidden=32, n_layers=2, n_heads=2, dropout=0.1, input_drop=0.0, attn_drop=0.0,
+                  quiet=True, lr=2e-2)
+    torch.manual_seed(17)
+    _, first = evaluation.train_arxiv(model, epochs=1, warm_up=False, **common, **kw)
+    torch.manual_seed(17)
+    ms, loss = evaluation.train_arxiv(model, epochs=25, **common, **kw)
+    assert np.isfinite(ms) and ms > 0 and np.isfinite(loss) and loss < first
+    with pytest.raises(ValueError):
+        evaluation.train_arxiv(model, epochs=1, n_label_iters=1, **common)
+
+
 def test_link_prediction_driver_trains_on_the_pubmed_stand_in():
     """tango_amd.evaluation.train_link_pred: the reference's evaluation/link_pred_gcn.py loop (GCN embeddings,
     sddmm_u_dot_v scores of edges and of k sampled non-edges, a negative graph built on the device per epoch)."""
