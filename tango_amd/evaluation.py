@@ -342,6 +342,10 @@ def main():
     ap.add_argument("--num-heads", type=int, default=8)
     ap.add_argument("--lr", type=float, default=1e-2)
     ap.add_argument("--weight-decay", type=float, default=5e-4)
+    ap.add_argument("--use-labels", action="store_true", help="arxiv models: feed training labels in as input columns")
+    ap.add_argument("--n-label-iters", type=int, default=0, help="arxiv models: refinement passes (needs --use-labels)")
+    ap.add_argument("--mask-rate", type=float, default=0.5, help="arxiv models: share of training nodes drawn per epoch")
+    ap.add_argument("--edge-drop", type=float, default=0.0, help="arxiv-gat: share of edges dropped per layer and epoch")
     args = ap.parse_args()
     if args.model.startswith("linkpred"):
         which = args.model.partition("-")[2] or "gcn"
@@ -349,7 +353,9 @@ def main():
                                    args.n_layers or (4 if which == "gcn" else 2), args.k, args.lr, args.weight_decay,
                                    model_name=which, heads=min(args.num_heads, 4))
     elif args.model.startswith("arxiv"):
-        ms, loss = train_arxiv(args.model.partition("-")[2], args.epochs, args.n_hidden, args.n_layers or 3)
+        ms, loss = train_arxiv(args.model.partition("-")[2], args.epochs, args.n_hidden, args.n_layers or 3,
+                               edge_drop=args.edge_drop, use_labels=args.use_labels, mask_rate=args.mask_rate,
+                               n_label_iters=args.n_label_iters)
     elif args.model == "hetero-hgt":
         ms, loss = train_hetero_hgt(args.epochs, args.n_hidden or 256, min(args.num_heads, 4))
     else:
