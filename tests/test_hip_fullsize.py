@@ -140,6 +140,51 @@ def test_qlinear_backward_full_closed_forms(K, orc, M, Kd, N):
     assert np.array_equal(host(dW2), orc.qgemm_bwd_dw(host(dYr[:Ms]), host(Xq[:Ms]), 0.01, 0.03))
 
 
+def test_hidden_gradient_hand_off_full(K, orc):
+    """The benchmark epoch's hand-off at its own shapes (232,965 rows, 41 -> 256 columns): gradX with the masked-scale
+    epilogue stores the dX of the plain kernel (sampled rows: the oracle's), its scale is max|dX' * mul| / 127 formed
+    with torch's exact elementwise ops and agrees with the separate masked pass, and the quantize pass that also
+    sums the columns writes the bytes of the plain pass (sampled rows: the oracle's) with column sums matching a
+    float64 sum."""
+    M, N, Kc = N_NODES, 41, 256
+    gen = torch.Generator("cuda").manual_seed(5)
+    dYq = torch.zeros((M, 48), dtype=torch.int8, device="cuda")[:, :N]
+    dYq.copy_(torch.randint(-127, 128, (M, N), dtype=torch.int8, device="cuda", generator=gen))
+    Wq = torch.randint(-127, 128, (N, Kc), dtype=torch.int8, device="cuda", generator=gen)
+    rs = torch.rand(M, device="cuda", generator=gen) + 0.5
+    mul = torch.rand(M, device="cuda", generator=gen) + 0.25
+    keep = torch.rand((M, Kc), device="cuda", generator=gen) < 0.5
+    weights = (1 << torch.arange(16, device="cuda", dtype=torch.int32))
+    bits = (keep.view(M, Kc // 16, 16).int() * weights).sum(-1).to(torch.int16).contiguous()  # one bit per column
+    s_dY, s_W = sc(0.013), sc(0.0021)
+    dX = torch.full((M, Kc), float("nan"), device="cuda")
+    got = K.cuda_kernels.QGEMM_backward_gradX(dX, dYq, Wq, s_dY, s_W, row_scale=rs, masked=(bits, mul))
+    assert got is not None
+    plain = torch.empty_like(dX)
+    K.cuda_kernels.QGEMM_backward_gradX(plain, dYq, Wq, s_dY, s_W, row_scale=rs)
+    assert torch.equal(dX, plain)
+    rows = np.sort(np.random.default_rng(4).choice(M, 1500, replace=False))
+    want = orc.qgemm_bwd_dx_ex(host(dYq)[rows], host(Wq), np.float32(0.013), np.float32(0.0021), row_scale=host(rs)[rows])
+    assert np.array_equal(host(dX)[rows], want)
+    masked = torch.where(keep, dX, torch.zeros((), device="cuda"))
+    assert torch.equal(got, ((masked * mul.unsqueeze(1)).abs().max() / 127).reshape(1))
+    s_pass, _ = K.cuda_kernels.absmax_ex(dX, row_mul=mul, mask=bits, mask_mode="bits")
+    assert torch.equal(got, s_pass)
+    # the quantize pass of that gradient, stochastic as in the epoch, with the bias gradient
+    kw = dict(row_mul=mul, mask=bits, mask_mode="bits", round_mode="stochastic", seed=9, offset=1 << 20)
+    q = torch.full((M, Kc), 77, dtype=torch.int8, device="cuda")
+    cs = K.cuda_kernels.quantize_rows_colsum(q, dX, got, **kw)
+    q_plain, _ = K.quantize_padded(dX, got, align=16, **kw)
+    assert torch.equal(q, q_plain)
+    assert torch.allclose(cs.double(), masked.double().sum(0), rtol=1e-5, atol=1e-3)
+    # a block of rows' bytes depend on its own values and on its position in the random stream only
+    for r0 in (0, 117_003, M - 600):
+        blk = slice(r0, r0 + 600)
+        want_q = orc.quantize_rows_ex(host(dX[blk]), host(got)[0], row_mul=host(mul[blk]), mask=host(bits[blk]),
+                                      mask_mode="bits", mode=orc.STOCHASTIC, seed=9, offset=(1 << 20) + r0 * Kc)
+        assert np.array_equal(host(q[blk]), want_q)
+
+
 def _row_sample_csr(g, count, seed, reverse=False):
     """Sub-CSR of `count` sampled destination rows (hubs included): indptr, column ids and slot
     numbers, as host arrays plus the slots as a device tensor."""
