@@ -461,20 +461,23 @@ __global__ __launch_bounds__(256) void spmm_kernel(const SpmmParams p) {
     if (c.grp == 0) store_row<VEC, AMAX>(p, c, row, acc);
 }
 
-// copy_u on narrow column tiles (a slot's piece of a gathered row is at most 64 bytes: 1, 2 or 4 lanes) when the rows
-// come ordered by length (p.row_order of a dense-block plan): a wavefront that owns one row then spends more
-// instructions on what a row costs whatever its length (index round trip, the fold over its sixteen or more slot
-// groups, the epilogue) than on the slots themselves, and the launch is bound by instruction issue.  Here sixteen
-// lanes own a row, four rows to a wavefront: a gather instruction serves 16 / lpe slots of each of the four rows,
-// the fold has log2(16 / lpe) stages, and prologue and epilogue run once for the four.  Neighbouring rows in that
-// order are about equally long, so the four finish together.  Rows above p.long_row are left to spmm_long_kernel,
-// as in spmm_kernel.  RL = log2 of the lanes that own a row: 4 (measured on 232,965 rows of 72 .. 777 slots, 41
-// columns: 0.533 ms per call against 0.563 with a wavefront per row; 8 lanes per row 0.556, 32 lanes 0.565; held
-// to eight waves per SIMD by a launch bound, which spills, 0.550).  blockDim.x = 256;
-// gridDim.x = ceil(rows / (4 * (64 >> RL))); gridDim.y tiles the columns.
-template <int RL>
+// copy_u on column tiles of at most 128 bytes (a slot's piece of a gathered row takes 1 .. 8 lanes) when the rows come
+// ordered by length (p.row_order of a dense-block plan): a wavefront that owns one row spends about as many
+// instructions on what a row costs whatever its length (index round trip, the fold over its eight or more slot
+// groups, the epilogue) as on the slots themselves.  Here 2^RL lanes own a row, 64 >> RL rows to a wavefront: a
+// gather instruction serves (1 << RL) / lpe slots of each of those rows, the fold has RL - log2(lpe) stages, and
+// prologue and epilogue run once for all of them.  Neighbouring rows in that order are about equally long, so they
+// finish together.  Rows above p.long_row are left to spmm_long_kernel, as in spmm_kernel.  U gathers in flight per
+// lane.  Measured on the rest of the 114.8 M-edge benchmark graph (232,965 rows of 72 .. 777 slots), per
+// aggregation call, against a wavefront per row: RL = 4 (sixteen lanes, four rows) 256 columns 1.467 -> 1.378 ms,
+// 128 columns 0.770 -> 0.719, 41 columns 0.563 -> 0.533; RL = 5 1.393 / 0.727; RL = 3 1.48 / 0.75 (41 columns:
+// 0.556); RL = 6 (this kernel with a row per wavefront) as spmm_kernel.  With RL = 4: U = 8 +20 us at 256 columns;
+// the next batch's indices fetched a batch ahead +25 us; held to eight waves per SIMD by a launch bound (66 VGPRs
+// otherwise: seven) +17 us at 41 columns (spills).  blockDim.x = 256; gridDim.x = ceil(rows / (4 * (64 >> RL)));
+// gridDim.y tiles the columns.
+template <int RL, int U = 4>
 __global__ __launch_bounds__(256) void spmm_quad_kernel(const SpmmParams p) {
-    constexpr int VEC = 16, U = 4, SEGL = 1 << RL;  // SEGL lanes own a row
+    constexpr int VEC = 16, SEGL = 1 << RL;  // SEGL lanes own a row
     const int lane = lane_id();
     const int wave = static_cast<int>(threadIdx.x) >> 6;
     const int seg = lane >> RL, sl = lane & (SEGL - 1);
@@ -512,8 +515,7 @@ __global__ __launch_bounds__(256) void spmm_quad_kernel(const SpmmParams p) {
 #pragma unroll
     for (int i = 0; i < VEC; ++i) acc[i] = 0;
     // indices: 4 SEGL slots of every row at a time, four coalesced loads per lane (lane sl of load r holds slot SEGL r + sl)
-    for (int base = 0; base < nmax; base += 4 * SEGL) {
-        int my[4];
+    auto fetch = [&](int base, int* dst) {
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
             const int q = base + r * SEGL + sl;
@@ -521,8 +523,12 @@ __global__ __launch_bounds__(256) void spmm_quad_kernel(const SpmmParams p) {
             // clamped: the load is unconditional (a row without slots reads the array's first entry)
             const int64_t qc = ok ? start + q : (n > 0 ? start + n - 1 : 0);
             const int v = load_index<true>(p, p.indices, qc);
-            my[r] = ok ? v : -1;
+            dst[r] = ok ? v : -1;
         }
+    };
+    for (int base = 0; base < nmax; base += 4 * SEGL) {
+        int my[4];
+        fetch(base, my);
         const int cnt = nmax - base < 4 * SEGL ? nmax - base : 4 * SEGL;
         const int total = (cnt + c.epi - 1) >> sh;  // steps of this batch
         for (int t = 0; t < total; t += U) {
@@ -535,14 +541,17 @@ __global__ __launch_bounds__(256) void spmm_quad_kernel(const SpmmParams p) {
                 j[u] = __shfl(reg, (seg << RL) | (k & (SEGL - 1)), kWave);
             }
             typename Gather<VEC>::T d[U];
-            uint32_t m = 0u;  // byte u: 1 where neighbour u counts
+            uint32_t m[U / 4];  // byte u: 1 where neighbour u counts
+#pragma unroll
+            for (int v = 0; v < U / 4; ++v) m[v] = 0u;
 #pragma unroll
             for (int u = 0; u < U; ++u) {
                 const bool ok = (t + u) < total && j[u] >= 0;
                 d[u] = Gather<VEC>::load(c.fcol + row_offset(ok ? j[u] : 0, p));  // row 0 with multiplier 0: no branch
-                m |= (ok ? 1u : 0u) << (8 * u);
+                m[u >> 2] |= (ok ? 1u : 0u) << (8 * (u & 3));
             }
-            accumulate4<VEC>(acc, d, m);
+#pragma unroll
+            for (int v = 0; v < U / 4; ++v) accumulate4<VEC>(acc, d + 4 * v, m[v]);
         }
     }
     // fold the row's slot groups: afterwards its lanes [0, lpe) hold the column sums
@@ -1303,10 +1312,10 @@ static int launch_spmm(SpmmParams p, int vec, hipStream_t s) {
     }
 #define TANGO_SPMM_LAUNCH(V, WPR) \
     hipLaunchKernelGGL((spmm_kernel<V, WPR, KIND>), grid, dim3(256), 0, s, p)
-    if (KIND == KIND_COPY && vec == 16 && p.lpe_log2 <= 2 && p.row_order && !p.amax_part && p.nnz > 0) {
-        // narrow tiles, rows ordered by length: four rows to a wavefront
+    if (KIND == KIND_COPY && vec == 16 && p.lpe_log2 <= 3 && p.row_order && !p.amax_part && p.nnz > 0) {
+        // tiles of at most 128 bytes, rows ordered by length: four rows to a wavefront
         const dim3 qgrid(static_cast<unsigned>(ceil_div(p.rows, 16)), static_cast<unsigned>(ychunks));
-        hipLaunchKernelGGL(spmm_quad_kernel<4>, qgrid, dim3(256), 0, s, p);
+        hipLaunchKernelGGL((spmm_quad_kernel<4, 4>), qgrid, dim3(256), 0, s, p);
         return launch_status();
     }
     if (p.amax_part) {  // copy_u only (the entry points see to that)
