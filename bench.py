@@ -795,7 +795,7 @@ def main():
     floor_ms = folded_ms * rest / nnz if folded_ms else None
     achieved = traffic / k_ms / 1e6 if traffic else None
     probe = mfma_probe(torch)
-    roofline = {"kernel": consts.get("kernel", "spmm_kernel<16,1,copy_u> on the rest of the adjacency, F=256"),
+    roofline = {"kernel": consts.get("kernel", "spmm_quad_kernel<4> on the rest of the adjacency, F=256"),
                 "bound": "hbm", "served_from": "infinity cache (the L2 misses are refilled over the fabric, not from HBM)",
                 "achieved": round(achieved, 1) if achieved else None, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                 "frac": round(achieved / HBM_PEAK_GBPS, 4) if achieved else None, "traffic": traffic,
