@@ -377,6 +377,14 @@ int tango_spmm_csr_copy_u_dense(float* out, const tango_spmm_dense_plan* plan, c
                                 const float* bias, int relu, uint16_t* sign_bits, int64_t F,
                                 const float* absmax_row_mul, float* scale_out,
                                 void* workspace, size_t workspace_bytes, tango_stream_t stream);
+/* The second part alone: the gather kernel on the rest of the adjacency, whose epilogue adds the partial sums that a
+   preceding tango_spmm_dense_partial (same plan, feat, F and workspace) left in the workspace.  The two calls in
+   a row give what tango_spmm_csr_copy_u_dense gives; for measurements (this launch is the dominant kernel of the
+   benchmark epoch and can be timed by itself).  No counterpart in the reference. */
+int tango_spmm_dense_rest(float* out, const tango_spmm_dense_plan* plan, const int8_t* feat,
+                          int64_t ldf, const float* scale, const float* row_scale,
+                          const float* bias, int relu, uint16_t* sign_bits, int64_t F,
+                          void* workspace, size_t workspace_bytes, tango_stream_t stream);
 
 /* multi_cusparse_SPMM (cuda/src/cuda.cpp:119-158 -> SPMM.cu:70-194):
    out[r,h,f] = scale[0] * float(sum_p evals[h, d, e(p)] * feat[indices[p], h, f]),

@@ -54,6 +54,7 @@ SIGNATURES = {
     "tango_spmm_dense_partial": (I, [P, P, I64, I64, P, SZ, P]),
     "tango_probe_mfma_i8": (I, [I, I, I, P, P]),
     "tango_spmm_csr_copy_u_dense": (I, [P, P, P, I64, P, P, P, I, P, I64, P, P, P, SZ, P]),
+    "tango_spmm_dense_rest": (I, [P, P, P, I64, P, P, P, I, P, I64, P, SZ, P]),
     "tango_spmm_csr_u_mul_e": (I, [P, P, P, P, P, P, P, I64, I64, I64, I64, I64, I64, P]),
     "tango_spmm_csr_u_mul_e_ex": (I, [P, P, P, P, I, P, P, I, P, P, P, I, I64, I64, I64, I64, I64, I64, I64, P, SZ, P]),
     "tango_spmm_csr_u_mul_e_f32e": (I, [P, P, P, P, I, P, P, I, P, P, P, I, I64, I64, I64, I64, I64, I64, I64, P, SZ, P]),

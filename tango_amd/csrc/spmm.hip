@@ -1503,11 +1503,12 @@ int tango_spmm_dense_partial(const tango_spmm_dense_plan* plan, const int8_t* fe
     return launch_dense_block(*plan, feat, ldf, F, workspace, workspace_bytes, &part, &ld, as_stream(stream));
 }
 
-int tango_spmm_csr_copy_u_dense(float* out, const tango_spmm_dense_plan* plan, const int8_t* feat,
-                                int64_t ldf, const float* scale, const float* row_scale,
-                                const float* bias, int relu, uint16_t* sign_bits, int64_t F,
-                                const float* absmax_row_mul, float* scale_out,
-                                void* workspace, size_t workspace_bytes, tango_stream_t stream) {
+// ``run_dense``: stage and multiply the bit blocks first; without it the gather kernel adds whatever partial sums a
+// preceding tango_spmm_dense_partial call (same plan, F and workspace) left in the workspace.
+static int copy_u_dense_impl(float* out, const tango_spmm_dense_plan* plan, const int8_t* feat, int64_t ldf,
+                             const float* scale, const float* row_scale, const float* bias, int relu,
+                             uint16_t* sign_bits, int64_t F, const float* absmax_row_mul, float* scale_out,
+                             void* workspace, size_t workspace_bytes, tango_stream_t stream, bool run_dense) {
     if (!plan || F < 0 || !scale || ldf < F || !feat || plan->rows < 0 || plan->res_nnz < 0 || !plan->res_indptr ||
         !plan->row_slot || (plan->rows * F > 0 && !out) || (plan->res_nnz > 0 && !plan->res_indices))
         return TANGO_ERR_INVALID_ARG;
@@ -1519,9 +1520,14 @@ int tango_spmm_csr_copy_u_dense(float* out, const tango_spmm_dense_plan* plan, c
     if (!workspace || workspace_bytes < need) return TANGO_ERR_WORKSPACE;
     SpmmParams p{};
     if (plan->row_blocks > 0) {
-        const int st = launch_dense_block(*plan, feat, ldf, F, workspace, workspace_bytes, &p.part, &p.part_ld,
-                                          as_stream(stream));
-        if (st != TANGO_OK) return st;
+        if (run_dense) {
+            const int st = launch_dense_block(*plan, feat, ldf, F, workspace, workspace_bytes, &p.part, &p.part_ld,
+                                              as_stream(stream));
+            if (st != TANGO_OK) return st;
+        } else {
+            const int st = dense_partial_sums(*plan, feat, ldf, F, workspace, workspace_bytes, &p.part, &p.part_ld);
+            if (st != TANGO_OK) return st;
+        }
         p.part_slot = plan->row_slot;
     } else if (pick_vec(feat, ldf, F) != 16) {
         return TANGO_ERR_UNSUPPORTED;
@@ -1538,6 +1544,23 @@ int tango_spmm_csr_copy_u_dense(float* out, const tango_spmm_dense_plan* plan, c
     }
     p.rows = plan->rows; p.num_src = plan->num_src; p.ldf = ldf; p.W = F; p.F = F; p.D = 1; p.nnz = plan->res_nnz;
     return launch_spmm<KIND_COPY>(p, 16, as_stream(stream));
+}
+
+int tango_spmm_csr_copy_u_dense(float* out, const tango_spmm_dense_plan* plan, const int8_t* feat,
+                                int64_t ldf, const float* scale, const float* row_scale,
+                                const float* bias, int relu, uint16_t* sign_bits, int64_t F,
+                                const float* absmax_row_mul, float* scale_out,
+                                void* workspace, size_t workspace_bytes, tango_stream_t stream) {
+    return copy_u_dense_impl(out, plan, feat, ldf, scale, row_scale, bias, relu, sign_bits, F, absmax_row_mul, scale_out,
+                             workspace, workspace_bytes, stream, true);
+}
+
+int tango_spmm_dense_rest(float* out, const tango_spmm_dense_plan* plan, const int8_t* feat,
+                          int64_t ldf, const float* scale, const float* row_scale,
+                          const float* bias, int relu, uint16_t* sign_bits, int64_t F,
+                          void* workspace, size_t workspace_bytes, tango_stream_t stream) {
+    return copy_u_dense_impl(out, plan, feat, ldf, scale, row_scale, bias, relu, sign_bits, F, nullptr, nullptr,
+                             workspace, workspace_bytes, stream, false);
 }
 
 int tango_spmm_incidence(float* out, const int64_t* node_ids, const int64_t* edge_ids,

@@ -373,8 +373,8 @@ size_t dense_workspace_bytes(const tango_spmm_dense_plan& plan, int64_t F) {
            align256(static_cast<size_t>(plan.dense_rows) * npad * sizeof(int));
 }
 
-int launch_dense_block(const tango_spmm_dense_plan& plan, const int8_t* feat, int64_t ldf, int64_t F,
-                       void* workspace, size_t workspace_bytes, const int** part, int* npad_out, hipStream_t s) {
+int dense_partial_sums(const tango_spmm_dense_plan& plan, const int8_t* feat, int64_t ldf, int64_t F,
+                       void* workspace, size_t workspace_bytes, const int** part, int* npad_out) {
     const int npad = dense_npad(F);
     if (!npad) return TANGO_ERR_UNSUPPORTED;
     if ((reinterpret_cast<uintptr_t>(feat) & 15) || (ldf & 15) || ((F + 15) & ~15LL) > ldf) return TANGO_ERR_UNSUPPORTED;
@@ -384,15 +384,23 @@ int launch_dense_block(const tango_spmm_dense_plan& plan, const int8_t* feat, in
         plan.num_groups > 65535 || plan.num_groups2 <= 0 || plan.num_groups2 > 65535 || !plan.seg_ptr2 || !plan.segs2 || !plan.col_ids || !plan.mask || !plan.mask_off || !plan.seg_ptr || !plan.segs ||
         (plan.num_shared > 0 && !plan.shared_blocks))
         return TANGO_ERR_INVALID_ARG;
+    *part = reinterpret_cast<const int*>(static_cast<char*>(workspace) + align256(static_cast<size_t>(plan.dense_cols) * npad));
+    *npad_out = npad;
+    return TANGO_OK;
+}
+
+int launch_dense_block(const tango_spmm_dense_plan& plan, const int8_t* feat, int64_t ldf, int64_t F,
+                       void* workspace, size_t workspace_bytes, const int** part, int* npad_out, hipStream_t s) {
+    const int checked = dense_partial_sums(plan, feat, ldf, F, workspace, workspace_bytes, part, npad_out);
+    if (checked != TANGO_OK) return checked;
+    const int npad = *npad_out;
     DenseParams p{};
     p.mask = plan.mask; p.mask_off = plan.mask_off; p.seg_ptr = plan.seg_ptr; p.segs = plan.segs;
     p.shared_blocks = plan.shared_blocks; p.col_ids = plan.col_ids; p.feat = feat; p.ldf = ldf;
     p.fbytes = (F + 15) & ~15LL;
     p.xt = static_cast<int8_t*>(workspace);
-    p.part = reinterpret_cast<int*>(static_cast<char*>(workspace) + align256(static_cast<size_t>(plan.dense_cols) * npad));
+    p.part = const_cast<int*>(*part);
     p.npad = npad;
-    *part = p.part;
-    *npad_out = npad;
     p.units = plan.dense_cols / kDenseUnit;
     p.stage_groups = plan.dense_cols / 64;
     const dim3 sgrid(static_cast<unsigned>(p.stage_groups + plan.num_shared));  // staging, then zeroing workgroups

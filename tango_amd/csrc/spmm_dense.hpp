@@ -19,4 +19,9 @@ size_t dense_workspace_bytes(const tango_spmm_dense_plan& plan, int64_t F);
 int launch_dense_block(const tango_spmm_dense_plan& plan, const int8_t* feat, int64_t ldf, int64_t F,
                        void* workspace, size_t workspace_bytes, const int** part, int* npad, hipStream_t s);
 
+// Where launch_dense_block leaves its partial sums for this plan, width and workspace, with its argument checks and
+// no launch.
+int dense_partial_sums(const tango_spmm_dense_plan& plan, const int8_t* feat, int64_t ldf, int64_t F,
+                       void* workspace, size_t workspace_bytes, const int** part, int* npad);
+
 }  // namespace tango

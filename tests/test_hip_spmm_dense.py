@@ -142,6 +142,36 @@ def test_dense_copy_u_epilogue_matches_oracle(K, orc, F):
         assert np.array_equal(host(sign).view(np.uint16), bits)
 
 
+@pytest.mark.parametrize("F", [41, 256])
+def test_dense_part_then_rest_is_the_whole_call(K, F):
+    """tango_spmm_dense_partial followed by tango_spmm_dense_rest on the same workspace: the output of
+    tango_spmm_csr_copy_u_dense, bit for bit, epilogue included."""
+    from tango_amd import _lib
+    L = _lib.lib()
+    rng = np.random.default_rng(F + 1)
+    n = 2300
+    s, d = heavy_graph(rng, n, 280_000)
+    indptr, indices = csr_of(d, s, n)
+    plan = plan_for(indptr, indices, n, tau=0.03, groups=6, min_extent=256)
+    ld = (F + 15) // 16 * 16
+    feat = dev(rng.integers(-127, 128, (n, ld)).astype(np.int8))
+    scale, row_scale = sc(0.0021), dev(rng.random(n).astype(np.float32))
+    bias = dev(rng.standard_normal(F).astype(np.float32))
+    whole = torch.empty((n, F), dtype=torch.float32, device="cuda")
+    assert K.cuda_kernels.csr_SPMM_dense(whole, plan, feat, scale, ldf=ld, F=F, row_scale=row_scale, bias=bias, relu=True)
+    nbytes = L.tango_spmm_dense_workspace(plan.ref, F)
+    ws = torch.empty(nbytes, dtype=torch.uint8, device="cuda")
+    st = torch.cuda.current_stream().cuda_stream
+    parts = torch.full((n, F), float("nan"), device="cuda")
+    _lib.check(L.tango_spmm_dense_partial(plan.ref, feat.data_ptr(), ld, F, ws.data_ptr(), nbytes, st), "partial")
+    for _ in range(2):  # the partial sums stay in the workspace: the second part can run again
+        _lib.check(L.tango_spmm_dense_rest(parts.data_ptr(), plan.ref, feat.data_ptr(), ld, scale.data_ptr(),
+                                           row_scale.data_ptr(), bias.data_ptr(), 1, None, F, ws.data_ptr(), nbytes, st), "rest")
+        assert torch.equal(parts, whole)
+    assert L.tango_spmm_dense_rest(parts.data_ptr(), plan.ref, feat.data_ptr(), ld, scale.data_ptr(), None, None, 0, None, F,
+                                   ws.data_ptr(), 16, st) != 0  # workspace too small: refused
+
+
 def test_dense_copy_u_bipartite_and_repeated_edges(K, orc):
     rng = np.random.default_rng(11)
     n_dst, n_src = 1500, 4000
