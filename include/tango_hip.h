@@ -336,9 +336,10 @@ typedef struct tango_spmm_dense_plan {
     int64_t num_shared;
     const int32_t* col_ids;        /* [dense_cols] column rank -> row of the gathered matrix, -1 = none */
     const int32_t* row_slot;       /* [rows] output row -> its row rank if below dense_rows, else -1 */
-    const int32_t* row_order;      /* [rows] rank -> output row, or NULL when that is the identity: the order the
-                                      gather kernel takes rows in (rows of similar length run side by side and
-                                      ask for the same sources, whatever the numbering of the nodes) */
+    const int32_t* row_order;      /* [rows] a permutation of the output rows, or NULL for the identity: the order the
+                                      gather kernel takes rows in, by falling slot count (the rows that share a
+                                      wavefront are about equally long, whatever the numbering of the nodes; with
+                                      NULL the kernel gives every row a wavefront of its own) */
     const int64_t* mask_off;       /* [row_blocks] */
     const uint32_t* mask;
     const int32_t* seg_ptr;        /* [num_groups + 1] */

@@ -186,9 +186,10 @@ def build_dense_plan(indptr, indices, num_src, tau=None, groups=256, sort_rest=T
     seg_ptr2, segs2, shared2 = _segments(extents // UNIT, 2 * groups)
     shared = np.union1d(shared, shared2).astype(np.int32)
     row_slot = torch.where(row_rank < row_blocks * ROWS, row_rank, torch.full_like(row_rank, -1))
-    identity = bool(torch.equal(row_order, torch.arange(rows, device=dev)))
+    # the gather kernel takes the rows in rank order: the rows that share a wavefront are then about equally long
+    # (ordering by the number of slots left to it instead was measured: the same times)
     return DensePlan(
-        row_order=None if identity else row_order.to(torch.int32).contiguous(),
+        row_order=row_order.to(torch.int32).contiguous(),
         rows=rows, num_src=int(num_src), row_blocks=row_blocks, dense_cols=int(extents.max()),
         tau=tau, nnz=nnz,
         col_ids=col_order[:int(extents.max())].to(torch.int32).contiguous(), row_slot=row_slot.contiguous(),
