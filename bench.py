@@ -822,7 +822,7 @@ def main():
                 "frac": round(achieved / HBM_PEAK_GBPS, 4) if achieved else None, "traffic": traffic,
                 "achieved_basis": "measured bytes beyond L2 per launch (FETCH_SIZE + WRITE_SIZE of the gather kernel, "
                                   "profiles/spmm_copy_u_F256_counters.md) / avg_launch_ms",
-                "binding_limit": "refills of the L2 misses over the fabric (49 % of the gathers hit the 4 MB L2s); "
+                "binding_limit": "refills of the L2 misses over the fabric (half of the gathers hit the 4 MB L2s); "
                                  "with every gather hitting, the L2 request rate (one 128-byte line per gathered row piece)",
                 "avg_launch_ms": round(k_ms, 4), "launches_timed": 20 if plan is not None else len(timer.spans.get("spmm_F256", [])),
                 "avg_launch_basis": "HIP events around tango_spmm_dense_rest (this kernel alone, the blocks' sums already in the workspace)",

@@ -22,10 +22,11 @@ UNIT = 256   # mask columns of a unit
 
 
 def default_tau():
-    """Density above which a cell is worth a bit: a cell costs the matrix cores about 0.7 % of what a gathered
+    """Density above which a cell is worth a bit: a cell costs the matrix cores about 0.9 % of what a gathered
     edge costs the gather kernel, at 64 columns as at 256 (measured on the 114.8 M-edge benchmark graph, where
-    0.007 .. 0.009 give the shortest epochs); TANGO_DENSE_TAU overrides, 0 switches the dense blocks off."""
-    return float(os.environ.get("TANGO_DENSE_TAU", "0.008"))
+    0.009 .. 0.011 give the shortest epochs: 4.83 / 4.81 / 4.80 / 4.82 ms at 0.008 / 0.009 / 0.010 / 0.011);
+    TANGO_DENSE_TAU overrides, 0 switches the dense blocks off."""
+    return float(os.environ.get("TANGO_DENSE_TAU", "0.010"))
 
 
 class DensePlan:
