@@ -475,26 +475,36 @@ __global__ __launch_bounds__(256) void spmm_kernel(const SpmmParams p) {
 // the next batch's indices fetched a batch ahead +25 us; held to eight waves per SIMD by a launch bound (66 VGPRs
 // otherwise: seven) +17 us at 41 columns (spills).  blockDim.x = 256; gridDim.x = ceil(rows / (4 * (64 >> RL)));
 // gridDim.y tiles the columns.
-template <int RL, int U = 4>
+// LPL = log2 of the lanes per slot, fixed at compile time for tiles of at most 64 bytes (the slot -> index register
+// mapping and the fold then are too), or -1: read from p, the form the 128-byte tiles run (their launch moves its
+// misses at the fabric's rate, and the leaner instruction stream of a fixed LPL = 3 was measured slower there:
+// 1.43 against 1.37 ms per 256-column call; 41 columns with LPL = 2: 0.509 against 0.536).  SHIFT (with LPL >= 0):
+// the rows of the gathered matrix are a power of two bytes apart and the whole matrix below 2 GiB
+// (p.ldf_shift >= 0), which makes a gather's address a 32-bit offset from one base for the whole wavefront.
+template <int RL, int LPL, bool SHIFT>
 __global__ __launch_bounds__(256) void spmm_quad_kernel(const SpmmParams p) {
-    constexpr int VEC = 16, SEGL = 1 << RL;  // SEGL lanes own a row
+    constexpr int VEC = 16, U = 4, SEGL = 1 << RL;  // SEGL lanes own a row
+    const int lpl = LPL >= 0 ? LPL : p.lpe_log2;
+    const int sh = RL - lpl;   // log2 of the slots a row advances per step
+    const int lpe = 1 << lpl;  // lanes per slot
     const int lane = lane_id();
     const int wave = static_cast<int>(threadIdx.x) >> 6;
     const int seg = lane >> RL, sl = lane & (SEGL - 1);
-    const int lpe = 1 << p.lpe_log2;  // lanes per slot
-    const int sh = RL - p.lpe_log2;   // log2 of the slots a row advances per step
     LaneCols c;
     c.lpe = lpe;
     c.epi = 1 << sh;
     c.sub = sl & (lpe - 1);
-    c.grp = sl >> p.lpe_log2;         // slot group inside the row's sixteen lanes
+    c.grp = sl >> lpl;  // slot group inside the row's lanes
     c.sh = sh;
     c.col = static_cast<int64_t>(blockIdx.y) * p.tile + static_cast<int64_t>(c.sub) * VEC;
     c.col_ok = c.col < p.W;
-    c.fcol = p.feat + (c.col_ok ? c.col : 0);
+    c.fcol = p.feat + (c.col_ok ? c.col : 0);  // lanes past the row's width read a valid piece and never store
     c.wbase = nullptr;
     c.wbase_f = nullptr;
     c.ev_r = 0.0f;
+    // SHIFT: address = tile base (the same for all lanes) + a 32-bit lane offset
+    const int8_t* tile_base = p.feat + static_cast<int64_t>(blockIdx.y) * p.tile;
+    const uint32_t lane_off = c.col_ok ? static_cast<uint32_t>(c.sub) * VEC : 0u;  // (past the width: the tile's first piece)
 
     const int64_t pos = (static_cast<int64_t>(blockIdx.x) * 4 + wave) * (kWave >> RL) + seg;
     const bool live = pos < p.rows;
@@ -505,17 +515,20 @@ __global__ __launch_bounds__(256) void spmm_quad_kernel(const SpmmParams p) {
     const bool mine = live && len <= p.long_row;
     if (!mine) len = 0;
     const int n = static_cast<int>(len);
-    int nmax = n;  // the longest of the wavefront's four rows
+    int nmax = n;  // the longest of the wavefront's rows
     for (int off = SEGL; off < kWave; off <<= 1) {
         const int other = __shfl_xor(nmax, off, kWave);
         nmax = other > nmax ? other : nmax;
     }
+    const int src_lane = (seg << RL) | c.grp;  // lane that holds the index of this lane group's slot of step 0
 
     int acc[VEC];
 #pragma unroll
     for (int i = 0; i < VEC; ++i) acc[i] = 0;
-    // indices: 4 SEGL slots of every row at a time, four coalesced loads per lane (lane sl of load r holds slot SEGL r + sl)
-    auto fetch = [&](int base, int* dst) {
+    // indices: 4 SEGL slots of every row at a time, four coalesced loads per lane (lane sl of load r holds slot
+    // SEGL r + sl); slots past the row's end hold -1
+    for (int base = 0; base < nmax; base += 4 * SEGL) {
+        int my[4];
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
             const int q = base + r * SEGL + sl;
@@ -523,35 +536,42 @@ __global__ __launch_bounds__(256) void spmm_quad_kernel(const SpmmParams p) {
             // clamped: the load is unconditional (a row without slots reads the array's first entry)
             const int64_t qc = ok ? start + q : (n > 0 ? start + n - 1 : 0);
             const int v = load_index<true>(p, p.indices, qc);
-            dst[r] = ok ? v : -1;
+            my[r] = ok ? v : -1;
         }
-    };
-    for (int base = 0; base < nmax; base += 4 * SEGL) {
-        int my[4];
-        fetch(base, my);
         const int cnt = nmax - base < 4 * SEGL ? nmax - base : 4 * SEGL;
-        const int total = (cnt + c.epi - 1) >> sh;  // steps of this batch
+        const int total = (cnt + c.epi - 1) >> sh;  // steps of this batch; a step past it finds -1 everywhere
         for (int t = 0; t < total; t += U) {
             int j[U];
-#pragma unroll
-            for (int u = 0; u < U; ++u) {
-                const int k = ((t + u) << sh) + c.grp;  // slot of the batch this lane group gathers
-                const int r = ((t + u) << sh) >> RL;    // its index register (wave-uniform: grp < SEGL >> lpe_log2)
+            if (LPL >= 2) {
+                // the four steps of a round take their slots from one index register
+                const int r = (t << sh) >> RL;  // wave-uniform
                 const int reg = r == 0 ? my[0] : r == 1 ? my[1] : r == 2 ? my[2] : my[3];
-                j[u] = __shfl(reg, (seg << RL) | (k & (SEGL - 1)), kWave);
+#pragma unroll
+                for (int u = 0; u < U; ++u)
+                    j[u] = __shfl(reg, src_lane + (((t + u) << sh) & (SEGL - 1)), kWave);
+            } else {
+#pragma unroll
+                for (int u = 0; u < U; ++u) {
+                    const int r = ((t + u) << sh) >> RL;  // wave-uniform
+                    const int reg = r == 0 ? my[0] : r == 1 ? my[1] : r == 2 ? my[2] : my[3];
+                    j[u] = __shfl(reg, src_lane + (((t + u) << sh) & (SEGL - 1)), kWave);
+                }
             }
             typename Gather<VEC>::T d[U];
-            uint32_t m[U / 4];  // byte u: 1 where neighbour u counts
-#pragma unroll
-            for (int v = 0; v < U / 4; ++v) m[v] = 0u;
+            uint32_t m = 0u;  // byte u: 1 where neighbour u counts
 #pragma unroll
             for (int u = 0; u < U; ++u) {
-                const bool ok = (t + u) < total && j[u] >= 0;
-                d[u] = Gather<VEC>::load(c.fcol + row_offset(ok ? j[u] : 0, p));  // row 0 with multiplier 0: no branch
-                m[u >> 2] |= (ok ? 1u : 0u) << (8 * (u & 3));
+                const bool ok = LPL >= 0 ? j[u] >= 0 : ((t + u) < total && j[u] >= 0);
+                const int jj = ok ? j[u] : 0;  // row 0 with multiplier 0: no branch around the load
+                if (LPL >= 0 && SHIFT)
+                    d[u] = Gather<VEC>::load(tile_base + ((static_cast<uint32_t>(jj) << p.ldf_shift) + lane_off));
+                else if (LPL >= 0)
+                    d[u] = Gather<VEC>::load(c.fcol + static_cast<int64_t>(jj) * p.ldf);
+                else
+                    d[u] = Gather<VEC>::load(c.fcol + row_offset(jj, p));
+                m |= (ok ? 1u : 0u) << (8 * u);
             }
-#pragma unroll
-            for (int v = 0; v < U / 4; ++v) accumulate4<VEC>(acc, d + 4 * v, m[v]);
+            accumulate4<VEC>(acc, d, m);
         }
     }
     // fold the row's slot groups: afterwards its lanes [0, lpe) hold the column sums
@@ -1315,7 +1335,16 @@ static int launch_spmm(SpmmParams p, int vec, hipStream_t s) {
     if (KIND == KIND_COPY && vec == 16 && p.lpe_log2 <= 3 && p.row_order && !p.amax_part && p.nnz > 0) {
         // tiles of at most 128 bytes, rows ordered by length: four rows to a wavefront
         const dim3 qgrid(static_cast<unsigned>(ceil_div(p.rows, 16)), static_cast<unsigned>(ychunks));
-        hipLaunchKernelGGL((spmm_quad_kernel<4, 4>), qgrid, dim3(256), 0, s, p);
+#define TANGO_SPMM_QUAD(LPL)                                                                              \
+    do {                                                                                                 \
+        if (p.ldf_shift >= 0) hipLaunchKernelGGL((spmm_quad_kernel<4, LPL, true>), qgrid, dim3(256), 0, s, p);  \
+        else hipLaunchKernelGGL((spmm_quad_kernel<4, LPL, false>), qgrid, dim3(256), 0, s, p);                \
+    } while (0)
+        if (p.lpe_log2 == 3) hipLaunchKernelGGL((spmm_quad_kernel<4, -1, false>), qgrid, dim3(256), 0, s, p);
+        else if (p.lpe_log2 == 2) TANGO_SPMM_QUAD(2);
+        else if (p.lpe_log2 == 1) TANGO_SPMM_QUAD(1);
+        else TANGO_SPMM_QUAD(0);
+#undef TANGO_SPMM_QUAD
         return launch_status();
     }
     if (p.amax_part) {  // copy_u only (the entry points see to that)
