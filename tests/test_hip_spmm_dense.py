@@ -94,7 +94,8 @@ def test_plan_holds_every_edge_once():
         assert np.all(np.diff(c) <= 0)
 
 
-@pytest.mark.parametrize("F,ld", [(16, 16), (41, 48), (41, 64), (64, 64), (100, 112), (128, 128), (200, 208), (256, 256)])
+@pytest.mark.parametrize("F,ld", [(16, 16), (24, 32), (20, 48), (32, 32), (41, 48), (41, 64), (64, 64), (100, 112), (128, 128), (200, 208),
+                                  (256, 256)])
 def test_dense_copy_u_matches_oracle(K, orc, F, ld):
     rng = np.random.default_rng(F + ld)
     n = 2500
