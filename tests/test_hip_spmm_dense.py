@@ -173,6 +173,27 @@ def test_dense_part_then_rest_is_the_whole_call(K, F):
                                    ws.data_ptr(), 16, st) != 0  # workspace too small: refused
 
 
+@pytest.mark.parametrize("F", [41, 256])
+def test_dense_plan_whose_hub_rows_keep_long_rests(K, orc, F):
+    """A high threshold leaves the hub rows thousands of slots outside the blocks: the rows-per-wavefront kernel
+    passes them over and the kernel for long rows sums them; the result is the oracle's all the same."""
+    rng = np.random.default_rng(F + 3)
+    n = 2600
+    s, d = heavy_graph(rng, n, 320_000)
+    perm = rng.permutation(n)
+    s, d = perm[s], perm[d]
+    indptr, indices = csr_of(d, s, n)
+    plan = plan_for(indptr, indices, n, tau=0.45, groups=4, min_extent=256, min_share=0.0)
+    assert plan.res_max_row > 4096
+    ld = (F + 15) // 16 * 16
+    feat = rng.integers(-127, 128, (n, ld)).astype(np.int8)
+    scale = np.float32(0.0007)
+    want = orc.spmm_csr_copy_u(indptr, indices, np.ascontiguousarray(feat[:, :F]), scale)
+    out = torch.empty((n, F), dtype=torch.float32, device="cuda")
+    assert K.cuda_kernels.csr_SPMM_dense(out, plan, dev(feat), sc(scale), ldf=ld, F=F)
+    assert np.array_equal(host(out), want)
+
+
 def test_dense_copy_u_bipartite_and_repeated_edges(K, orc):
     rng = np.random.default_rng(11)
     n_dst, n_src = 1500, 4000
